@@ -1,0 +1,172 @@
+/*
+ * tfjs_hip.h — C ABI of libtfjs_hip.so, the MI355X (gfx950) device library behind the
+ * `hip` backend for tfjs-core's KernelBackend plugin API.
+ *
+ * Everything the JavaScript backend class (through the N-API addon), the Python ctypes
+ * driver and any C/C++ caller needs goes through these entry points: plain pointers,
+ * integers and sizes only.  The shape of the interface follows the reference's own
+ * native precedent, the WASM backend, which keys device tensors by an integer data id
+ * chosen by the host (tfjs-backend-wasm/src/lib.cc:55-134, backend_wasm.ts:35-51,166-187)
+ * and passes ids of pre-registered outputs to each kernel call (lib.cc:102-124).
+ *
+ * Conventions
+ *  - Every call returns 0 on success or a TFHIP_E* code; tfhip_last_error() then holds a
+ *    message.  The JS shim turns non-zero into `throw new Error(msg)`, which is how
+ *    backend_cpu reports errors (backend_cpu.ts:119-127).
+ *  - All device work is queued on the context's single in-order stream and returns
+ *    immediately; only tfhip_read / tfhip_sync / tfhip_time_end wait for the device.
+ *  - A data id owns one device buffer whose element type was fixed at register time.
+ *    Several tensors may alias one id (reshape and widening casts do,
+ *    backends/backend_util.ts:34-82), so kernels convert from the *stored* dtype.
+ *  - Tensors are dense row-major; images are NHWC, filters HWIO.
+ */
+#ifndef TFJS_HIP_H_
+#define TFJS_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tfhip_ctx tfhip_ctx;
+
+/* dtype codes 0..2 are the reference's (tfjs-backend-wasm/src/lib.cc:26-30);
+ * UINT8Q holds affine-quantised weights (io/types.ts:100-107) kept as bytes in HBM. */
+enum { TFHIP_FLOAT32 = 0, TFHIP_INT32 = 1, TFHIP_BOOL = 2, TFHIP_UINT8Q = 3 };
+
+enum {
+  TFHIP_OK = 0,
+  TFHIP_EINVAL = 1,   /* bad argument / shape mismatch */
+  TFHIP_ENOENT = 2,   /* unknown data id */
+  TFHIP_EEXIST = 3,   /* data id registered twice (backend_cpu.ts:119-121) */
+  TFHIP_EDEVICE = 4,  /* HIP runtime error */
+  TFHIP_ENOTSUP = 5   /* legal in the reference but not built here */
+};
+
+/* Activation applied in the epilogue of the dense kernels.  LINEAR/RELU/PRELU are the
+ * reference's Activation type (ops/fused_util.ts:19); RELU6 is clip(x,0,6)
+ * (backend_cpu.ts:1265-1275) folded into the same epilogue. */
+enum { TFHIP_ACT_LINEAR = 0, TFHIP_ACT_RELU = 1, TFHIP_ACT_PRELU = 2, TFHIP_ACT_RELU6 = 3 };
+
+/* Mirrors Conv2DInfo (ops/conv_util.ts:43-64), channelsLast only. */
+typedef struct tfhip_conv2d_info {
+  int32_t batch;
+  int32_t in_h, in_w, in_c;
+  int32_t out_h, out_w, out_c;
+  int32_t stride_h, stride_w;
+  int32_t dilation_h, dilation_w;
+  int32_t filter_h, filter_w;
+  int32_t pad_top, pad_left, pad_bottom, pad_right;
+} tfhip_conv2d_info;
+
+/* Affine dequantisation of a TFHIP_UINT8Q operand: w = q*scale + min evaluated in double
+ * and rounded once to float32, as decodeWeights does (io/io_utils.ts:133-136). */
+typedef struct tfhip_qparams {
+  double scale;
+  double min;
+} tfhip_qparams;
+
+/* ---- context --------------------------------------------------------------------- */
+/* Factory of the backend (engine.ts:261-307 calls it): picks the device, creates the
+ * stream and the buffer pool. */
+int tfhip_init(int device, tfhip_ctx** out);
+/* KernelBackend.dispose (backend.ts:646): frees every buffer and the stream. */
+void tfhip_destroy(tfhip_ctx* ctx);
+/* Message of the last failed call on this context (ctx may be NULL after a failed init). */
+const char* tfhip_last_error(tfhip_ctx* ctx);
+
+/* ---- storage (KernelBackend.register/write/read/readSync/disposeData/memory,
+ *      backend.ts:92-126; CPU implementation backend_cpu.ts:102-129,199-254) ---------- */
+int tfhip_register(tfhip_ctx* ctx, int64_t id, const int32_t* shape, int rank, int dtype);
+int tfhip_write(tfhip_ctx* ctx, int64_t id, const void* host, size_t nbytes);
+int tfhip_read(tfhip_ctx* ctx, int64_t id, void* host, size_t nbytes);
+int tfhip_dispose(tfhip_ctx* ctx, int64_t id);
+/* bytes held by live ids / bytes parked in the pool / number of live ids */
+int tfhip_mem_info(tfhip_ctx* ctx, size_t* in_use, size_t* pooled, size_t* num_ids);
+int tfhip_sync(tfhip_ctx* ctx);
+/* KernelBackend.time (backend.ts:92, backend_cpu.ts:239-244): event pair on the stream. */
+int tfhip_time_begin(tfhip_ctx* ctx);
+int tfhip_time_end(tfhip_ctx* ctx, float* ms);
+/* Raw device address of an id's buffer (for callers that share the device, e.g. a
+ * harness that generates inputs in HBM).  Not part of the reference interface. */
+int tfhip_device_ptr(tfhip_ctx* ctx, int64_t id, void** ptr, size_t* nbytes);
+
+/* ---- dense contractions ------------------------------------------------------------ */
+/* batchMatMul / fusedBatchMatMul (backend.ts:128-138; backend_cpu.ts:491-555).
+ * a: [batch,M,K] (or [batch,K,M] when transpose_a), b: [batch,K,N] (or [batch,N,K]),
+ * out: [batch,M,N] float32.  bias / prelu: data id or -1; each must hold 1, N or
+ * batch*M*N elements (scalar, per-column, full).  q: non-NULL iff b is TFHIP_UINT8Q. */
+int tfhip_matmul(tfhip_ctx* ctx, int64_t a, int64_t b, int64_t out, int batch, int m, int n,
+                 int k, int transpose_a, int transpose_b, int64_t bias, int act,
+                 int64_t prelu, const tfhip_qparams* q);
+/* conv2d / fusedConv2d (backend.ts:414-421; backend_cpu.ts:1536-1616): x NHWC,
+ * filter [fh,fw,in_c,out_c], out NHWC float32.  bias/prelu/q as for tfhip_matmul with
+ * N = out_c. */
+int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t out,
+                 const tfhip_conv2d_info* info, int64_t bias, int act, int64_t prelu,
+                 const tfhip_qparams* q);
+
+/* ---- memory-bound image kernels ------------------------------------------------------ */
+/* depthwiseConv2D (backend.ts:431-434; backend_cpu.ts:1979-2035): filter
+ * [fh,fw,in_c,ch_mul], out_c = in_c*ch_mul.  bias (-1 or out_c elements) and act
+ * (LINEAR/RELU/RELU6) fold the add + clip that follow it in MobileNet into the same pass;
+ * the reference issues them as separate add/clip calls.  q: filter may be UINT8Q. */
+int tfhip_depthwise_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t out,
+                           const tfhip_conv2d_info* info, int64_t bias, int act,
+                           const tfhip_qparams* q);
+/* avgPool / maxPool (backend.ts:453-462; backend_cpu.ts:2273-2345, 2869-2873). */
+enum { TFHIP_POOL_AVG = 0, TFHIP_POOL_MAX = 1 };
+int tfhip_pool2d(tfhip_ctx* ctx, int64_t x, int64_t out, const tfhip_conv2d_info* info,
+                 int kind);
+
+/* ---- elementwise ------------------------------------------------------------------- */
+/* add/subtract/multiply/realDivide/prelu/maximum/minimum (backend.ts:164-177, 247, 258, 328;
+ * backend_cpu.ts:440-481,557-580,1203-1209,3515-3549) with N-d broadcasting
+ * (ops/broadcast_util.ts:27-87).  Shapes are right-aligned, rank <= 6. */
+enum {
+  TFHIP_ADD = 0, TFHIP_SUB = 1, TFHIP_MUL = 2, TFHIP_DIV = 3, TFHIP_PRELU = 4,
+  TFHIP_MAXIMUM = 5, TFHIP_MINIMUM = 6
+};
+int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_shape, int a_rank,
+                 int64_t b, const int32_t* b_shape, int b_rank, int64_t out);
+/* relu/clip/exp/log/neg/abs/sigmoid/sqrt/square/tanh/rsqrt
+ * (backend.ts:160, 300-357, 392; backend_cpu.ts:1094-1126,1191-1201,1265-1275).  p0,p1: clip min,max. */
+enum {
+  TFHIP_RELU = 0, TFHIP_CLIP = 1, TFHIP_EXP = 2, TFHIP_LOG = 3, TFHIP_NEG = 4,
+  TFHIP_ABS = 5, TFHIP_SIGMOID = 6, TFHIP_SQRT = 7, TFHIP_SQUARE = 8, TFHIP_TANH = 9,
+  TFHIP_RSQRT = 10
+};
+int tfhip_unary(tfhip_ctx* ctx, int op, int64_t x, int64_t out, float p0, float p1);
+/* cast / int (backend.ts:340, 484; backend_cpu.ts:1299-1308, 2861-2863; backends/backend_util.ts:34-71):
+ * converts from x's stored dtype to out's stored dtype (float->int32 truncates,
+ * ->bool is x != 0). */
+int tfhip_cast(tfhip_ctx* ctx, int64_t x, int64_t out);
+/* fill/zerosLike/onesLike (backend.ts:629-640; backend_cpu.ts:3816-3836). */
+int tfhip_fill(tfhip_ctx* ctx, int64_t out, double value);
+
+/* ---- reductions over the innermost axis ---------------------------------------------- */
+/* sum/max/min/argMax/argMin (backend.ts:183, 195-200, 244, 255; backend_cpu.ts:590-611,686-712,906-929):
+ * x viewed as [outer, inner]; out has `outer` elements (int32 for ARG*). */
+enum { TFHIP_SUM = 0, TFHIP_MAX = 1, TFHIP_MIN = 2, TFHIP_ARGMAX = 3, TFHIP_ARGMIN = 4 };
+int tfhip_reduce(tfhip_ctx* ctx, int op, int64_t x, int64_t out, int64_t outer, int64_t inner);
+/* One-pass row softmax; same result as the reference's 10-call composite
+ * (ops/softmax.ts:45-79, ops/reduction_ops.ts:56-74) within float32 tolerance. */
+int tfhip_softmax_rows(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t rows, int64_t cols);
+
+/* ---- data movement ------------------------------------------------------------------- */
+/* gather (backend.ts:501; backend_cpu.ts:2204-2223): x viewed as
+ * [outer, axis_dim, inner]; out [outer, n_indices, inner]; indices int32. */
+int tfhip_gather(tfhip_ctx* ctx, int64_t x, int64_t indices, int64_t out, int64_t outer,
+                 int64_t axis_dim, int64_t inner, int64_t n_indices);
+/* transpose (backend.ts:497; backend_cpu.ts:2166-2202), rank <= 6. */
+int tfhip_transpose(tfhip_ctx* ctx, int64_t x, const int32_t* x_shape, int rank,
+                    const int32_t* perm, int64_t out);
+/* Device-to-device copy between ids of equal byte size (identity / clone). */
+int tfhip_copy(tfhip_ctx* ctx, int64_t x, int64_t out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TFJS_HIP_H_ */

@@ -1,0 +1,375 @@
+/*
+ * cpu_ref.c — TEST INFRASTRUCTURE, not product code.
+ *
+ * A plain-C restatement of the loops of tfjs-core's backend_cpu that sit on the hip
+ * backend's hot path.  It exists only to check the HIP kernels (tests, smoke) and to be
+ * timed as the CPU baseline; nothing in the product path may call it.
+ *
+ * backend_cpu computes in JavaScript numbers (IEEE double) and stores into Float32Array /
+ * Int32Array, so every function below does its arithmetic in double and rounds to float
+ * exactly where the reference stores to a typed array.  Each function cites the reference
+ * lines it follows (paths relative to tfjs-core/src/).
+ *
+ * Parity pins (see tests/test_oracle_*.py): every function is checked against the
+ * known-answer vectors of the reference's own *_test.ts files transcribed under
+ * tests/golden/, plus float64 brute-force / closed-form checks.  One behaviour is
+ * PARITY UNPINNED: depthwise convolution with asymmetric padding on non-square inputs,
+ * where backend_cpu swaps padLeft/padTop (backends/cpu/backend_cpu.ts:2000,2010); no
+ * reference vector covers it.  `pad_quirk` selects the backend_cpu behaviour; 0 selects
+ * the TensorFlow / WebGL semantics that the hip backend implements.
+ *
+ * Build: gcc -O2 -fPIC -shared (see Makefile).  -ffast-math must NOT be used: the
+ * float/double rounding points are the whole point.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+typedef struct ref_conv2d_info { /* same field order as tfhip_conv2d_info */
+  int32_t batch;
+  int32_t in_h, in_w, in_c;
+  int32_t out_h, out_w, out_c;
+  int32_t stride_h, stride_w;
+  int32_t dilation_h, dilation_w;
+  int32_t filter_h, filter_w;
+  int32_t pad_top, pad_left, pad_bottom, pad_right;
+} ref_conv2d_info;
+
+/* backends/cpu/backend_cpu.ts:491-540 — 48-wide blocking (blockSize, :83); products and
+ * the per-block sum are doubles, `resVals[...] += sum` rounds to float once per k-block. */
+void ref_batch_matmul(const float* a, const float* b, float* out, int batch, int m, int n,
+                      int k, int transpose_a, int transpose_b) {
+  const int bs = 48;
+  const int64_t a_batch = (int64_t)m * k, b_batch = (int64_t)k * n;
+  const int64_t a_outer = transpose_a ? 1 : k, a_inner = transpose_a ? m : 1;
+  const int64_t b_inner = transpose_b ? 1 : n, b_outer = transpose_b ? k : 1;
+  const int64_t size = (int64_t)m * n;
+  memset(out, 0, sizeof(float) * (size_t)(batch * size));
+  for (int bi = 0; bi < batch; bi++)
+    for (int i0 = 0; i0 < m; i0 += bs)
+      for (int j0 = 0; j0 < n; j0 += bs)
+        for (int k0 = 0; k0 < k; k0 += bs) {
+          const int i1 = i0 + bs < m ? i0 + bs : m;
+          const int j1 = j0 + bs < n ? j0 + bs : n;
+          const int k1 = k0 + bs < k ? k0 + bs : k;
+          for (int i = i0; i < i1; i++)
+            for (int j = j0; j < j1; j++) {
+              double sum = 0.0;
+              for (int kk = k0; kk < k1; kk++)
+                sum += (double)a[bi * a_batch + i * a_outer + kk * a_inner] *
+                       (double)b[kk * b_inner + j * b_outer + bi * b_batch];
+              float* r = &out[bi * size + (int64_t)i * n + j];
+              *r = (float)((double)*r + sum);
+            }
+        }
+}
+
+/* backends/cpu/backend_cpu.ts:1552-1616, channelsLast strides; out-of-bounds taps are
+ * skipped (:1586,:1596); `yVals[...] += xVal * w` rounds to float after every MAC. */
+void ref_conv2d(const float* x, const float* w, float* y, const ref_conv2d_info* ci) {
+  const int64_t x_row = (int64_t)ci->in_w * ci->in_c, x_b = x_row * ci->in_h;
+  const int64_t y_row = (int64_t)ci->out_w * ci->out_c, y_b = y_row * ci->out_h;
+  const int64_t w_s0 = (int64_t)ci->filter_w * ci->in_c * ci->out_c;
+  const int64_t w_s1 = (int64_t)ci->in_c * ci->out_c;
+  const int oc = ci->out_c;
+  memset(y, 0, sizeof(float) * (size_t)(y_b * ci->batch));
+  for (int b = 0; b < ci->batch; ++b)
+    for (int yr = 0; yr < ci->out_h; ++yr) {
+      const int xr_corner = yr * ci->stride_h - ci->pad_top;
+      for (int wr = 0; wr < ci->filter_h; ++wr) {
+        const int xr = xr_corner + wr * ci->dilation_h;
+        if (xr < 0 || xr >= ci->in_h) continue;
+        for (int yc = 0; yc < ci->out_w; ++yc) {
+          float* yp = y + b * y_b + yr * y_row + (int64_t)yc * oc;
+          const int xc_corner = yc * ci->stride_w - ci->pad_left;
+          for (int wc = 0; wc < ci->filter_w; ++wc) {
+            const int xc = xc_corner + wc * ci->dilation_w;
+            if (xc < 0 || xc >= ci->in_w) continue;
+            const float* xp = x + b * x_b + xr * x_row + (int64_t)xc * ci->in_c;
+            const float* wp = w + wr * w_s0 + wc * w_s1;
+            for (int d1 = 0; d1 < ci->in_c; ++d1) {
+              const double xv = (double)xp[d1];
+              for (int d2 = 0; d2 < oc; ++d2)
+                yp[d2] = (float)((double)yp[d2] + xv * (double)wp[d2]);
+              wp += oc;
+            }
+          }
+        }
+      }
+    }
+}
+
+/* backends/cpu/backend_cpu.ts:1979-2035.  pad_quirk != 0 reproduces :2000 (rows offset by
+ * padLeft) and :2010 (columns offset by padTop); 0 uses top for rows, left for columns. */
+void ref_depthwise_conv2d(const float* x, const float* w, float* y, const ref_conv2d_info* ci,
+                          int pad_quirk) {
+  const int ch_mul = ci->out_c / ci->in_c;
+  const int64_t x_row = (int64_t)ci->in_w * ci->in_c, x_b = x_row * ci->in_h;
+  const int64_t y_row = (int64_t)ci->out_w * ci->out_c, y_b = y_row * ci->out_h;
+  const int64_t w_s0 = (int64_t)ci->filter_w * ci->in_c * ch_mul;
+  const int64_t w_s1 = (int64_t)ci->in_c * ch_mul;
+  const int row_pad = pad_quirk ? ci->pad_left : ci->pad_top;
+  const int col_pad = pad_quirk ? ci->pad_top : ci->pad_left;
+  memset(y, 0, sizeof(float) * (size_t)(y_b * ci->batch));
+  for (int b = 0; b < ci->batch; ++b)
+    for (int yr = 0; yr < ci->out_h; ++yr) {
+      const int xr_corner = yr * ci->stride_h - row_pad;
+      for (int wr = 0; wr < ci->filter_h; ++wr) {
+        const int xr = xr_corner + wr * ci->dilation_h;
+        if (xr < 0 || xr >= ci->in_h) continue;
+        for (int yc = 0; yc < ci->out_w; ++yc) {
+          const int xc_corner = yc * ci->stride_w - col_pad;
+          for (int wc = 0; wc < ci->filter_w; ++wc) {
+            const int xc = xc_corner + wc * ci->dilation_w;
+            if (xc < 0 || xc >= ci->in_w) continue;
+            const float* xp = x + b * x_b + xr * x_row + (int64_t)xc * ci->in_c;
+            const float* wp = w + wr * w_s0 + wc * w_s1;
+            float* yp = y + b * y_b + yr * y_row + (int64_t)yc * ci->out_c;
+            for (int d1 = 0; d1 < ci->in_c; ++d1) {
+              const double xv = (double)xp[d1];
+              for (int q = 0; q < ch_mul; ++q)
+                yp[q] = (float)((double)yp[q] + xv * (double)wp[q]);
+              yp += ch_mul;
+              wp += ch_mul;
+            }
+          }
+        }
+      }
+    }
+}
+
+/* backends/cpu/backend_cpu.ts:2273-2341 (avgPool :2869-2873, maxPool :2343-2345).
+ * kind 0 = avg: double window sum over in-bounds pixels only, divided by their count.
+ * kind 1 = max: starts at -inf, `pixel > max` so NaN never replaces a number; the
+ * isNaN(minMaxValue) early exit (:2329) can never fire for max, kept for fidelity. */
+void ref_pool2d(const float* x, float* y, const ref_conv2d_info* ci, int kind) {
+  const int eff_h = ci->filter_h + (ci->filter_h - 1) * (ci->dilation_h - 1);
+  const int eff_w = ci->filter_w + (ci->filter_w - 1) * (ci->dilation_w - 1);
+  const int64_t x_row = (int64_t)ci->in_w * ci->in_c, x_b = x_row * ci->in_h;
+  const int64_t y_row = (int64_t)ci->out_w * ci->out_c, y_b = y_row * ci->out_h;
+  for (int b = 0; b < ci->batch; ++b)
+    for (int d = 0; d < ci->in_c; ++d)
+      for (int yr = 0; yr < ci->out_h; ++yr) {
+        const int xr_corner = yr * ci->stride_h - ci->pad_top;
+        const int xr_min = xr_corner > 0 ? xr_corner : 0;
+        const int xr_max = ci->in_h < eff_h + xr_corner ? ci->in_h : eff_h + xr_corner;
+        for (int yc = 0; yc < ci->out_w; ++yc) {
+          const int xc_corner = yc * ci->stride_w - ci->pad_left;
+          const int xc_min = xc_corner > 0 ? xc_corner : 0;
+          const int xc_max = ci->in_w < eff_w + xc_corner ? ci->in_w : eff_w + xc_corner;
+          double mm = -INFINITY, avg = 0.0;
+          int count = 0;
+          for (int xr = xr_min; xr < xr_max; xr += ci->dilation_h) {
+            for (int xc = xc_min; xc < xc_max; xc += ci->dilation_w) {
+              const double pixel = (double)x[b * x_b + xr * x_row + (int64_t)xc * ci->in_c + d];
+              if (kind == 1) {
+                if (pixel > mm) mm = pixel;
+              } else {
+                avg += pixel;
+                count++;
+              }
+            }
+            if (isnan(mm)) break;
+          }
+          y[b * y_b + yr * y_row + (int64_t)yc * ci->out_c + d] =
+              kind == 0 ? (float)(avg / (double)count) : (float)mm;
+        }
+      }
+}
+
+/* ---- elementwise ------------------------------------------------------------------- */
+enum { REF_ADD = 0, REF_SUB, REF_MUL, REF_DIV, REF_PRELU, REF_MAXIMUM, REF_MINIMUM };
+
+static double binary_eval(int op, double a, double b) {
+  switch (op) {
+    case REF_ADD: return a + b;                       /* backend_cpu.ts:440-452 */
+    case REF_SUB: return a - b;                       /* :469-481 */
+    case REF_MUL: return a * b;                       /* :557-572 */
+    case REF_DIV: return a / b;                       /* :574-580 */
+    case REF_PRELU: return a < 0 ? b * a : a;         /* :1203-1209 */
+    case REF_MAXIMUM: return (isnan(a) || isnan(b)) ? NAN : (a > b ? a : b); /* Math.max :931-936 */
+    case REF_MINIMUM: return (isnan(a) || isnan(b)) ? NAN : (a < b ? a : b); /* Math.min :886-891 */
+  }
+  return NAN;
+}
+
+/* backends/cpu/backend_cpu.ts:3515-3549 with ops/broadcast_util.ts:27-87.  Operands and
+ * result are doubles here; the Python wrapper converts from / rounds to the stored dtype
+ * (float32 store rounds, Int32Array store truncates).  Shapes are right-aligned. */
+int ref_binary(int op, const double* a, const int32_t* a_shape, int a_rank, const double* b,
+               const int32_t* b_shape, int b_rank, double* out, const int32_t* out_shape,
+               int out_rank) {
+  int64_t n = 1, a_len = 1, b_len = 1;
+  for (int i = 0; i < out_rank; i++) n *= out_shape[i];
+  for (int i = 0; i < a_rank; i++) a_len *= a_shape[i];
+  for (int i = 0; i < b_rank; i++) b_len *= b_shape[i];
+  /* getBroadcastDims (:27-42): dims of the operand that are 1 where the result is > 1 */
+  int a_bc = 0, b_bc = 0;
+  for (int i = 0; i < a_rank; i++) {
+    const int dim = a_rank - 1 - i, od = out_rank - 1 - i;
+    if (a_shape[dim] == 1 && out_shape[od] > 1) a_bc++;
+  }
+  for (int i = 0; i < b_rank; i++) {
+    const int dim = b_rank - 1 - i, od = out_rank - 1 - i;
+    if (b_shape[dim] == 1 && out_shape[od] > 1) b_bc++;
+  }
+  if (a_bc + b_bc == 0) { /* fast path :3526-3530 (what a [C] bias on [...,C] hits) */
+    for (int64_t i = 0; i < n; i++) out[i] = binary_eval(op, a[i % a_len], b[i % b_len]);
+    return 0;
+  }
+  int32_t loc[8];
+  if (out_rank > 8) return 1;
+  for (int64_t i = 0; i < n; i++) {
+    int64_t rem = i;
+    for (int d = out_rank - 1; d >= 0; d--) {
+      loc[d] = (int32_t)(rem % out_shape[d]);
+      rem /= out_shape[d];
+    }
+    int64_t ai = 0, bi = 0, stride = 1;
+    for (int d = a_rank - 1; d >= 0; d--) {
+      const int od = out_rank - a_rank + d;
+      const int32_t c = (a_shape[d] == 1 && out_shape[od] > 1) ? 0 : loc[od];
+      ai += c * stride;
+      stride *= a_shape[d];
+    }
+    stride = 1;
+    for (int d = b_rank - 1; d >= 0; d--) {
+      const int od = out_rank - b_rank + d;
+      const int32_t c = (b_shape[d] == 1 && out_shape[od] > 1) ? 0 : loc[od];
+      bi += c * stride;
+      stride *= b_shape[d];
+    }
+    out[i] = binary_eval(op, a[ai], b[bi]);
+  }
+  return 0;
+}
+
+enum {
+  REF_RELU = 0, REF_CLIP, REF_EXP, REF_LOG, REF_NEG, REF_ABS, REF_SIGMOID, REF_SQRT,
+  REF_SQUARE, REF_TANH, REF_RSQRT
+};
+
+/* backends/cpu/backend_cpu.ts: relu :1191-1201 (Math.max(0,x), NaN-propagating), clip
+ * :1265-1275, exp :1094-1103, log :1116-1126, neg :434-438 (multiply by -1), abs
+ * :1277-1285, sigmoid :1310-1318, sqrt :1140-1150, square :1164-1174, tanh (util.tanh)
+ * :1455-1465, rsqrt :1152-1162.  double libm, one rounding to float at the store. */
+void ref_unary(int op, const float* x, float* out, int64_t n, float p0, float p1) {
+  for (int64_t i = 0; i < n; i++) {
+    const double v = (double)x[i];
+    double r;
+    switch (op) {
+      case REF_RELU: r = isnan(v) ? NAN : (v > 0 ? v : 0); break;
+      case REF_CLIP: r = v > (double)p1 ? (double)p1 : (v < (double)p0 ? (double)p0 : v); break;
+      case REF_EXP: r = exp(v); break;
+      case REF_LOG: r = log(v); break;
+      case REF_NEG: r = -v; break;
+      case REF_ABS: r = fabs(v); break;
+      case REF_SIGMOID: r = 1.0 / (1.0 + exp(-v)); break;
+      case REF_SQRT: r = sqrt(v); break;
+      case REF_SQUARE: r = v * v; break;
+      case REF_TANH: r = tanh(v); break;
+      case REF_RSQRT: r = 1.0 / sqrt(v); break;
+      default: r = NAN;
+    }
+    out[i] = (float)r;
+  }
+}
+
+/* ---- reductions over the innermost axis ---------------------------------------------- */
+enum { REF_SUM = 0, REF_MAX, REF_MIN, REF_ARGMAX, REF_ARGMIN };
+
+/* sum backend_cpu.ts:590-611 (double accumulator, one rounding); max :906-929 and min
+ * :861-884 (seeded with element 0, strict compare, so a NaN only survives in slot 0);
+ * argMax :686-712 / argMin :658-684 (first index of the strict extremum).  x is read as
+ * doubles; out is double (values) — the wrapper rounds / converts. */
+void ref_reduce(int op, const double* x, double* out, int64_t outer, int64_t inner) {
+  for (int64_t i = 0; i < outer; i++) {
+    const double* row = x + i * inner;
+    double acc = (op == REF_SUM) ? 0.0 : row[0];
+    int64_t idx = 0;
+    for (int64_t j = 0; j < inner; j++) {
+      const double v = row[j];
+      switch (op) {
+        case REF_SUM: acc += v; break;
+        case REF_MAX: if (v > acc) acc = v; break;
+        case REF_MIN: if (v < acc) acc = v; break;
+        case REF_ARGMAX: if (v > acc) { acc = v; idx = j; } break;
+        case REF_ARGMIN: if (v < acc) { acc = v; idx = j; } break;
+      }
+    }
+    out[i] = (op == REF_ARGMAX || op == REF_ARGMIN) ? (double)idx : acc;
+  }
+}
+
+/* ops/softmax.ts:45-79 + ops/reduction_ops.ts:56-74 as backend_cpu executes them:
+ * max -> sub -> exp -> sum -> log -> add -> sub -> exp, every intermediate stored as
+ * float32 (the sum accumulates in double and rounds once). */
+void ref_softmax_rows(const float* x, float* out, int64_t rows, int64_t cols) {
+  float* tmp = (float*)malloc(sizeof(float) * (size_t)(cols > 0 ? cols : 1));
+  for (int64_t r = 0; r < rows; r++) {
+    const float* row = x + r * cols;
+    float mx = row[0];
+    for (int64_t j = 0; j < cols; j++) if (row[j] > mx) mx = row[j];
+    double s = 0.0;
+    for (int64_t j = 0; j < cols; j++) {
+      const float a = (float)((double)row[j] - (double)mx);
+      tmp[j] = (float)exp((double)a);
+      s += (double)tmp[j];
+    }
+    const float c = (float)s;
+    const float d = (float)log((double)c);
+    const float lse = (float)((double)mx + (double)d);
+    for (int64_t j = 0; j < cols; j++) {
+      const float lr = (float)((double)row[j] - (double)lse);
+      out[r * cols + j] = (float)exp((double)lr);
+    }
+  }
+  free(tmp);
+}
+
+/* ---- data movement ------------------------------------------------------------------- */
+/* backends/cpu/backend_cpu.ts:2204-2223 with x viewed as [outer, axis_dim, inner];
+ * 4-byte elements copied verbatim. */
+void ref_gather(const int32_t* x, const int32_t* indices, int32_t* out, int64_t outer,
+                int64_t axis_dim, int64_t inner, int64_t n_idx) {
+  for (int64_t o = 0; o < outer; o++)
+    for (int64_t i = 0; i < n_idx; i++)
+      memcpy(out + (o * n_idx + i) * inner, x + (o * axis_dim + indices[i]) * inner,
+             sizeof(int32_t) * (size_t)inner);
+}
+
+/* backends/cpu/backend_cpu.ts:2178-2200: newLoc[i] = loc[perm[i]]. */
+int ref_transpose(const int32_t* x, const int32_t* shape, int rank, const int32_t* perm,
+                  int32_t* out) {
+  int32_t new_shape[8], loc[8];
+  if (rank > 8) return 1;
+  int64_t n = 1;
+  for (int i = 0; i < rank; i++) { new_shape[i] = shape[perm[i]]; n *= shape[i]; }
+  for (int64_t i = 0; i < n; i++) {
+    int64_t rem = i;
+    for (int d = rank - 1; d >= 0; d--) { loc[d] = (int32_t)(rem % shape[d]); rem /= shape[d]; }
+    int64_t ni = 0;
+    for (int d = 0; d < rank; d++) ni = ni * new_shape[d] + loc[perm[d]];
+    out[ni] = x[i];
+  }
+  return 0;
+}
+
+/* io/io_utils.ts:122-147, float32 branch: v*scale + min in double, one rounding. */
+void ref_dequantize_u8(const uint8_t* q, float* out, int64_t n, double scale, double min) {
+  for (int64_t i = 0; i < n; i++) out[i] = (float)((double)q[i] * scale + min);
+}
+
+/* backends/cpu/backend_cpu.ts:1299-1308: Int32Array store of a float = ToInt32 (truncate
+ * toward zero, NaN/inf -> 0, wrap modulo 2^32). */
+void ref_float_to_int(const float* x, int32_t* out, int64_t n) {
+  for (int64_t i = 0; i < n; i++) {
+    const double v = (double)x[i];
+    if (isnan(v) || isinf(v)) { out[i] = 0; continue; }
+    const double t = trunc(v);
+    const double m = fmod(t, 4294967296.0);
+    const int64_t w = (int64_t)m;
+    out[i] = (int32_t)(uint32_t)(w & 0xffffffffLL);
+  }
+}

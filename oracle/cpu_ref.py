@@ -1,0 +1,444 @@
+"""numpy front end of the CPU oracle (libcpu_ref.so) — TEST INFRASTRUCTURE ONLY.
+
+Mirrors the method names of tfjs-core's MathBackendCPU
+(tfjs-core/src/backends/cpu/backend_cpu.ts) on numpy arrays so that parity tests read
+like the reference's own op tests.  Only tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py may import this module; the product path never does.
+
+The shape math restated here follows tfjs-core/src/ops/conv_util.ts:66-182,391-435,
+ops/broadcast_util.ts:27-87 and ops/axis_util.ts:49-95.
+"""
+import ctypes as C
+import math
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libcpu_ref.so")
+
+
+def build(force=False):
+    """Compile libcpu_ref.so with the Makefile next to this file."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libcpu_ref.so"],
+                              stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+class Conv2DInfoC(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "batch", "in_h", "in_w", "in_c", "out_h", "out_w", "out_c", "stride_h", "stride_w",
+        "dilation_h", "dilation_w", "filter_h", "filter_w", "pad_top", "pad_left",
+        "pad_bottom", "pad_right")]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_LIB_PATH)
+    return _lib
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _p(a, t=C.c_float):
+    return a.ctypes.data_as(C.POINTER(t))
+
+
+# ---------------------------------------------------------------------------------------
+# shape math (ops/conv_util.ts)
+# ---------------------------------------------------------------------------------------
+def _tuple2(v):
+    return (v, v) if isinstance(v, int) else (int(v[0]), int(v[1]))
+
+
+def _eff(filter_size, dilation):  # conv_util.ts:391-397
+    return filter_size if dilation <= 1 else filter_size + (filter_size - 1) * (dilation - 1)
+
+
+def _cond_round(v, mode):  # conv_util.ts:499-517
+    if not mode:
+        return v
+    if mode == "round":
+        return math.floor(v + 0.5)  # Math.round
+    if mode == "ceil":
+        return math.ceil(v)
+    if mode == "floor":
+        return math.floor(v)
+    raise ValueError("Unknown roundingMode %s" % mode)
+
+
+def compute_conv2d_info(in_shape, filter_shape, strides, dilations, pad, rounding_mode=None,
+                        depthwise=False):
+    """computeConv2DInfo (conv_util.ts:123-182) + getPadAndOutInfo (:399-435), NHWC."""
+    batch, in_h, in_w, in_c = in_shape
+    f_h, f_w, _, f_c = filter_shape
+    s_h, s_w = _tuple2(strides)
+    d_h, d_w = _tuple2(dilations)
+    e_h, e_w = _eff(f_h, d_h), _eff(f_w, d_w)
+    if isinstance(pad, (int, float)) and not isinstance(pad, bool):
+        top = bottom = left = right = pad
+        # computeOutputShape2D (conv_util.ts:271-296) uses the *height* filter and stride
+        out_h = _cond_round((in_h - e_h + 2 * pad) / s_h + 1, rounding_mode)
+        out_w = _cond_round((in_w - e_h + 2 * pad) / s_h + 1, rounding_mode)
+        if out_h != int(out_h) or out_w != int(out_w):
+            raise ValueError("The output # of rows/columns must be an integer. "
+                             "Change the stride and/or zero pad parameters")
+        out_h, out_w = int(out_h), int(out_w)
+        ptype = "VALID" if pad == 0 else "NUMBER"
+    elif pad == "same":
+        out_h, out_w = math.ceil(in_h / s_h), math.ceil(in_w / s_w)
+        pah = max(0, (out_h - 1) * s_h + e_h - in_h)
+        paw = max(0, (out_w - 1) * s_w + e_w - in_w)
+        top, left = pah // 2, paw // 2
+        bottom, right = pah - top, paw - left
+        ptype = "SAME"
+    elif pad == "valid":
+        top = bottom = left = right = 0
+        out_h = math.ceil((in_h - e_h + 1) / s_h)
+        out_w = math.ceil((in_w - e_w + 1) / s_w)
+        ptype = "VALID"
+    else:
+        raise ValueError("Unknown padding parameter: %s" % pad)
+    out_c = f_c * in_c if depthwise else f_c
+    return dict(batchSize=batch, inHeight=in_h, inWidth=in_w, inChannels=in_c,
+                outHeight=out_h, outWidth=out_w, outChannels=out_c,
+                strideHeight=s_h, strideWidth=s_w, dilationHeight=d_h, dilationWidth=d_w,
+                filterHeight=f_h, filterWidth=f_w, effectiveFilterHeight=e_h,
+                effectiveFilterWidth=e_w,
+                padInfo=dict(top=top, bottom=bottom, left=left, right=right, type=ptype),
+                inShape=tuple(in_shape), outShape=(batch, out_h, out_w, out_c),
+                filterShape=tuple(filter_shape))
+
+
+def compute_pool2d_info(in_shape, filter_size, strides, dilations, pad, rounding_mode=None):
+    """computePool2DInfo (conv_util.ts:66-86)."""
+    f_h, f_w = _tuple2(filter_size)
+    return compute_conv2d_info(in_shape, (f_h, f_w, in_shape[3], in_shape[3]), strides,
+                               dilations, pad, rounding_mode, False)
+
+
+def _info_c(ci):
+    p = ci["padInfo"]
+    return Conv2DInfoC(ci["batchSize"], ci["inHeight"], ci["inWidth"], ci["inChannels"],
+                       ci["outHeight"], ci["outWidth"], ci["outChannels"], ci["strideHeight"],
+                       ci["strideWidth"], ci["dilationHeight"], ci["dilationWidth"],
+                       ci["filterHeight"], ci["filterWidth"], int(p["top"]), int(p["left"]),
+                       int(p["bottom"]), int(p["right"]))
+
+
+def broadcast_shape(sa, sb):
+    """assertAndGetBroadcastShape (ops/broadcast_util.ts:61-87)."""
+    out = []
+    n = max(len(sa), len(sb))
+    for i in range(n):
+        a = sa[len(sa) - 1 - i] if i < len(sa) else 1
+        b = sb[len(sb) - 1 - i] if i < len(sb) else 1
+        if a == 1:
+            out.insert(0, b)
+        elif b == 1:
+            out.insert(0, a)
+        elif a != b:
+            raise ValueError("Operands could not be broadcast together with shapes "
+                             "%s and %s." % (",".join(map(str, sa)), ",".join(map(str, sb))))
+        else:
+            out.insert(0, a)
+    return tuple(out)
+
+
+# ---------------------------------------------------------------------------------------
+# kernels
+# ---------------------------------------------------------------------------------------
+def batch_matmul(a, b, transpose_a=False, transpose_b=False):
+    a, b = _f32(a), _f32(b)
+    batch = a.shape[0]
+    m = a.shape[2] if transpose_a else a.shape[1]
+    k = a.shape[1] if transpose_a else a.shape[2]
+    n = b.shape[1] if transpose_b else b.shape[2]
+    out = np.empty((batch, m, n), np.float32)
+    lib().ref_batch_matmul(_p(a), _p(b), _p(out), batch, m, n, k, int(transpose_a),
+                           int(transpose_b))
+    return out
+
+
+def _activation(x, activation, prelu_weights):
+    """mapActivation (backend_cpu.ts:50-62); 'relu6' = clip(x,0,6) (:1265-1275)."""
+    if activation in (None, "linear"):
+        return x
+    if activation == "relu":
+        return relu(x)
+    if activation == "prelu":
+        return prelu(x, prelu_weights)
+    if activation == "relu6":
+        return clip(x, 0.0, 6.0)
+    raise ValueError("Activation %s has not been implemented for the CPU backend." % activation)
+
+
+def fused_batch_matmul(a, b, transpose_a=False, transpose_b=False, bias=None, activation=None,
+                       prelu_weights=None):
+    """backend_cpu.ts:542-555: matmul, then add, then activation, as separate passes."""
+    r = batch_matmul(a, b, transpose_a, transpose_b)
+    if bias is not None:
+        r = add(r, bias)
+    return _activation(r, activation, prelu_weights)
+
+
+def conv2d(x, w, ci):
+    x, w = _f32(x), _f32(w)
+    y = np.empty(ci["outShape"], np.float32)
+    info = _info_c(ci)
+    lib().ref_conv2d(_p(x), _p(w), _p(y), C.byref(info))
+    return y
+
+
+def fused_conv2d(x, w, ci, bias=None, activation=None, prelu_weights=None):
+    """backend_cpu.ts:1536-1550."""
+    r = conv2d(x, w, ci)
+    if bias is not None:
+        r = add(r, bias)
+    return _activation(r, activation, prelu_weights)
+
+
+def depthwise_conv2d(x, w, ci, pad_quirk=False):
+    x, w = _f32(x), _f32(w)
+    y = np.empty(ci["outShape"], np.float32)
+    info = _info_c(ci)
+    lib().ref_depthwise_conv2d(_p(x), _p(w), _p(y), C.byref(info), int(pad_quirk))
+    return y
+
+
+def _pool(x, ci, kind):
+    x = _f32(x)
+    y = np.empty(ci["outShape"], np.float32)
+    info = _info_c(ci)
+    lib().ref_pool2d(_p(x), _p(y), C.byref(info), kind)
+    return y
+
+
+def avg_pool(x, ci):
+    return _pool(x, ci, 0)
+
+
+def max_pool(x, ci):
+    return _pool(x, ci, 1)
+
+
+_BIN = dict(add=0, sub=1, mul=2, div=3, prelu=4, maximum=5, minimum=6)
+
+
+def _store(values_f64, dtype):
+    """Typed-array store semantics: Float32Array rounds, Int32Array applies ToInt32."""
+    dtype = np.dtype(dtype)
+    if dtype == np.float32:
+        with np.errstate(over="ignore", invalid="ignore"):
+            return values_f64.astype(np.float32)
+    if dtype == np.int32:
+        v = np.where(np.isfinite(values_f64), np.trunc(values_f64), 0.0)
+        v = np.fmod(v, 4294967296.0).astype(np.int64) & 0xFFFFFFFF
+        return v.astype(np.uint32).view(np.int32).reshape(values_f64.shape)
+    if dtype == np.bool_ or dtype == np.uint8:
+        # Uint8Array store: ToUint8 (truncate, wrap modulo 256)
+        v = np.where(np.isfinite(values_f64), np.trunc(values_f64), 0.0)
+        return (np.fmod(v, 256.0).astype(np.int64) & 0xFF).astype(np.uint8)
+    raise ValueError(dtype)
+
+
+def _binary(op, a, b, out_dtype=None):
+    a, b = np.asarray(a), np.asarray(b)
+    if out_dtype is None:
+        out_dtype = np.result_type(a.dtype, b.dtype)
+        if out_dtype == np.float64:
+            out_dtype = np.float32
+    out_shape = broadcast_shape(a.shape, b.shape)
+    a64 = np.ascontiguousarray(a, np.float64)
+    b64 = np.ascontiguousarray(b, np.float64)
+    out = np.empty(out_shape, np.float64)
+    sa = (C.c_int32 * max(1, a.ndim))(*a.shape)
+    sb = (C.c_int32 * max(1, b.ndim))(*b.shape)
+    so = (C.c_int32 * max(1, len(out_shape)))(*out_shape)
+    rc = lib().ref_binary(_BIN[op], _p(a64, C.c_double), sa, a.ndim, _p(b64, C.c_double), sb,
+                          b.ndim, _p(out, C.c_double), so, len(out_shape))
+    assert rc == 0
+    return _store(out, out_dtype)
+
+
+def add(a, b):
+    return _binary("add", a, b)
+
+
+def subtract(a, b):
+    return _binary("sub", a, b)
+
+
+def multiply(a, b):
+    return _binary("mul", a, b)
+
+
+def real_divide(a, b):
+    return _binary("div", a, b, np.float32)  # backend_cpu.ts:574-580: float32 result
+
+
+def prelu(x, alpha):
+    return _binary("prelu", x, alpha, np.asarray(x).dtype)
+
+
+def maximum(a, b):
+    return _binary("maximum", a, b)
+
+
+def minimum(a, b):
+    return _binary("minimum", a, b)
+
+
+_UN = dict(relu=0, clip=1, exp=2, log=3, neg=4, abs=5, sigmoid=6, sqrt=7, square=8, tanh=9,
+           rsqrt=10)
+
+
+def _unary(op, x, p0=0.0, p1=0.0):
+    x = _f32(x)
+    out = np.empty(x.shape, np.float32)
+    lib().ref_unary(_UN[op], _p(x), _p(out), C.c_int64(x.size), C.c_float(p0), C.c_float(p1))
+    return out
+
+
+def relu(x):
+    return _unary("relu", x)
+
+
+def clip(x, lo, hi):
+    return _unary("clip", x, lo, hi)
+
+
+def exp(x):
+    return _unary("exp", x)
+
+
+def log(x):
+    return _unary("log", x)
+
+
+def neg(x):
+    return _unary("neg", x)
+
+
+def abs_(x):
+    return _unary("abs", x)
+
+
+def sigmoid(x):
+    return _unary("sigmoid", x)
+
+
+def sqrt(x):
+    return _unary("sqrt", x)
+
+
+def square(x):
+    return _unary("square", x)
+
+
+def tanh(x):
+    return _unary("tanh", x)
+
+
+def rsqrt(x):
+    return _unary("rsqrt", x)
+
+
+_RED = dict(sum=0, max=1, min=2, argmax=3, argmin=4)
+
+
+def _reduce(op, x, n_axes=1):
+    """Reduce the innermost n_axes dims (assertAxesAreInnerMostDims, axis_util.ts:24-34)."""
+    x = np.asarray(x)
+    out_shape = x.shape[:x.ndim - n_axes]
+    inner = int(np.prod(x.shape[x.ndim - n_axes:], dtype=np.int64))
+    outer = int(np.prod(out_shape, dtype=np.int64))
+    x64 = np.ascontiguousarray(x, np.float64)
+    out = np.empty(out_shape, np.float64)
+    lib().ref_reduce(_RED[op], _p(x64, C.c_double), _p(out, C.c_double), C.c_int64(outer),
+                     C.c_int64(inner))
+    return out
+
+
+def sum_(x, n_axes=1):
+    x = np.asarray(x)
+    # upcastType(x.dtype, 'int32') (types.ts:130-138): bool -> int32
+    dt = np.float32 if x.dtype == np.float32 else np.int32
+    return _store(_reduce("sum", x, n_axes), dt)
+
+
+def max_(x, n_axes=1):
+    x = np.asarray(x)
+    return _store(_reduce("max", x, n_axes), x.dtype)
+
+
+def min_(x, n_axes=1):
+    x = np.asarray(x)
+    return _store(_reduce("min", x, n_axes), x.dtype)
+
+
+def arg_max(x):
+    return _reduce("argmax", x).astype(np.int32)
+
+
+def arg_min(x):
+    return _reduce("argmin", x).astype(np.int32)
+
+
+def softmax(x):
+    x = _f32(x)
+    cols = x.shape[-1]
+    rows = x.size // cols if cols else 0
+    out = np.empty(x.shape, np.float32)
+    lib().ref_softmax_rows(_p(x), _p(out), C.c_int64(rows), C.c_int64(cols))
+    return out
+
+
+def gather(x, indices, axis=0):
+    x = np.ascontiguousarray(x)
+    assert x.dtype.itemsize == 4
+    idx = np.ascontiguousarray(indices, np.int32).ravel()
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    out_shape = x.shape[:axis] + (idx.size,) + x.shape[axis + 1:]
+    out = np.empty(out_shape, x.dtype)
+    lib().ref_gather(_p(x.view(np.int32), C.c_int32), _p(idx, C.c_int32),
+                     _p(out.view(np.int32), C.c_int32), C.c_int64(outer),
+                     C.c_int64(x.shape[axis]), C.c_int64(inner), C.c_int64(idx.size))
+    return out
+
+
+def transpose(x, perm):
+    x = np.ascontiguousarray(x)
+    assert x.dtype.itemsize == 4
+    out = np.empty(tuple(x.shape[p] for p in perm), x.dtype)
+    shape = (C.c_int32 * x.ndim)(*x.shape)
+    pm = (C.c_int32 * x.ndim)(*perm)
+    rc = lib().ref_transpose(_p(x.view(np.int32), C.c_int32), shape, x.ndim, pm,
+                             _p(out.view(np.int32), C.c_int32))
+    assert rc == 0
+    return out
+
+
+def dequantize_u8(q, scale, min_):
+    q = np.ascontiguousarray(q, np.uint8)
+    out = np.empty(q.shape, np.float32)
+    lib().ref_dequantize_u8(_p(q, C.c_uint8), _p(out), C.c_int64(q.size), C.c_double(scale),
+                            C.c_double(min_))
+    return out
+
+
+def to_int(x):
+    x = _f32(x)
+    out = np.empty(x.shape, np.int32)
+    lib().ref_float_to_int(_p(x), _p(out, C.c_int32), C.c_int64(x.size))
+    return out

@@ -1,0 +1,204 @@
+#!/usr/bin/env python3
+"""Pull the known-answer vectors of the reference's own op tests into JSON fixtures.
+
+Run in the build container (it reads the reference checkout as TEXT; nothing is imported
+or executed):
+
+    python tests/golden/extract_golden.py [/root/reference]
+
+For every forward (non-gradient, non-error) `it('<title>', ...)` block of the describe
+blocks listed in CASES the script records, in order of appearance, each numeric array
+literal of the block (data arrays, shapes, expected values) and each scalar/string
+`const` (stride, pad, dilation ...).  The tests under tests/ give each position its
+meaning.
+Arrays whose elements are not numeric literals are stored as null so positions stay
+stable.  Output: tests/golden/<name>.json, one file per reference test file.
+"""
+import json
+import os
+import re
+import sys
+
+REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+OUT = os.path.dirname(os.path.abspath(__file__))
+
+# fixture name -> (reference test file, describe blocks to take (None = whole file))
+CASES = {
+    "matmul": ("tfjs-core/src/ops/matmul_test.ts", ["matmul", "matmulBatch", "dot"]),
+    "matmul_webgpu": ("tfjs-webgpu/src/matmul_test.ts", None),
+    "fused": ("tfjs-core/src/ops/fused_test.ts", ["fused matmul", "fused conv2d"]),
+    "conv2d": ("tfjs-core/src/ops/conv2d_test.ts", ["conv2d"]),
+    "depthwise": ("tfjs-core/src/ops/conv2d_depthwise_test.ts", ["depthwiseConv2D"]),
+    "separable": ("tfjs-core/src/ops/conv2d_separable_test.ts", ["separableConv2d"]),
+    "pool": ("tfjs-core/src/ops/pool_test.ts", ["maxPool", "avgPool", "pool"]),
+    "softmax": ("tfjs-core/src/ops/softmax_test.ts", ["softmax"]),
+    "reduction": ("tfjs-core/src/ops/reduction_ops_test.ts",
+                  ["Reduction: max", "Reduction: min", "Reduction: argmax",
+                   "Reduction: argmin", "Reduction: sum", "Reduction: logSumExp"]),
+    "unary": ("tfjs-core/src/ops/unary_ops_test.ts",
+              ["relu", "clip", "exp", "log", "neg", "abs", "sigmoid", "sqrt", "square",
+               "tanh", "rsqrt"]),
+    "binary": ("tfjs-core/src/ops/binary_ops_test.ts", ["prelu", "maximum", "minimum"]),
+    "arithmetic": ("tfjs-core/src/ops/arithmetic_test.ts", ["add", "sub", "mul", "div"]),
+    "gather": ("tfjs-core/src/ops/array_ops_test.ts", ["gather"]),
+    "transpose": ("tfjs-core/src/ops/transpose_test.ts", ["transpose"]),
+    "dequant": ("tfjs-core/src/io/io_utils_test.ts", ["decodeWeights"]),
+}
+# blocks whose title matches are not forward known-answer cases
+SKIP = re.compile(r"grad|throw|raises|tensor-like|TensorLike|does not match|do not match|"
+                  r"dont match|non-tensor|string tensor|Unsupported|error", re.I)
+
+_NUM = re.compile(r"[-+]?(?:NaN|Infinity|(?:\d+\.?\d*|\.\d+)(?:[eE][-+]?\d+)?)")
+
+
+_CONST = re.compile(r"\bconst\s+([A-Za-z_$][\w$]*)(?::[^=;]+)?\s*=\s*"
+                    r"(?:(-?\d+\.?\d*(?:[eE][-+]?\d+)?)|'([^']*)'|(true|false))\s*;")
+
+
+def _match_paren(src, j):
+    """src[j-1] == '(' ; return index just past the matching ')'."""
+    depth, in_str = 1, None
+    while j < len(src) and depth:
+        c = src[j]
+        if in_str:
+            if c == "\\":
+                j += 1
+            elif c == in_str:
+                in_str = None
+        elif c in "'\"`":
+            in_str = c
+        elif c == "/" and src[j + 1] == "/":
+            j = src.index("\n", j)
+        elif c == "(":
+            depth += 1
+        elif c == ")":
+            depth -= 1
+        j += 1
+    return j
+
+
+def blocks_of(src, describes):
+    """Yield (describe, title, body) for each it() block of the wanted describe blocks."""
+    scopes = []
+    for m in re.finditer(r"\bdescribe\w*\(\s*['\"]([^'\"]*)['\"]", src):
+        end = _match_paren(src, src.index("(", m.start()) + 1)
+        scopes.append((m.group(1), m.start(), end))
+    if not scopes:
+        scopes = [(None, 0, len(src))]
+    for name, start, end in scopes:
+        if describes is not None and name not in describes:
+            continue
+        for m in re.finditer(r"\bit\(\s*(['\"])((?:(?!\1)[^\\]|\\.)*)\1\s*,", src[start:end]):
+            j = start + m.start()
+            stop = _match_paren(src, src.index("(", j) + 1)
+            yield name, m.group(2), src[start + m.end():stop]
+
+
+def consts_of(body):
+    out = {}
+    for m in _CONST.finditer(body):
+        if m.group(2) is not None:
+            t = m.group(2)
+            out[m.group(1)] = float(t) if re.search(r"[.eE]", t) else int(t)
+        elif m.group(3) is not None:
+            out[m.group(1)] = m.group(3)
+        else:
+            out[m.group(1)] = m.group(4) == "true"
+    return out
+
+
+def parse_array(body, i):
+    """Parse a bracketed literal starting at body[i]=='['. Returns (value|None, end)."""
+    assert body[i] == "["
+    out, ok = [], True
+    i += 1
+    while True:
+        while i < len(body) and body[i] in " \t\r\n,":
+            i += 1
+        if body.startswith("//", i):
+            i = body.index("\n", i)
+            continue
+        if body[i] == "]":
+            return (out if ok else None), i + 1
+        if body[i] == "[":
+            v, i = parse_array(body, i)
+            if v is None:
+                ok = False
+            out.append(v)
+            continue
+        m = _NUM.match(body, i)
+        nxt = body[m.end()] if m and m.end() < len(body) else ""
+        if m and (nxt in " \t\r\n,]"):
+            t = m.group(0)
+            out.append(float(t) if re.search(r"[.eEN]|Infinity", t) else int(t))
+            i = m.end()
+            continue
+        m2 = re.match(r"(true|false)\b", body[i:])
+        if m2:
+            out.append(1 if m2.group(1) == "true" else 0)
+            i += m2.end()
+            continue
+        # not a literal element: skip to the matching close, mark the array unusable
+        ok = False
+        depth = 0
+        while True:
+            c = body[i]
+            if c in "([{":
+                depth += 1
+            elif c in ")]}":
+                if depth == 0:
+                    break
+                depth -= 1
+            elif c == "," and depth == 0:
+                break
+            i += 1
+
+
+def arrays_of(body):
+    res, i = [], 0
+    while i < len(body):
+        c = body[i]
+        if c in "'\"`":  # skip strings
+            j = i + 1
+            while body[j] != c:
+                j += 2 if body[j] == "\\" else 1
+            i = j + 1
+            continue
+        if body.startswith("//", i):
+            i = body.index("\n", i)
+            continue
+        if c == "[":
+            k = i - 1
+            while k >= 0 and body[k] in " \t\r\n":
+                k -= 1
+            prev = body[k] if k >= 0 else ""
+            if prev.isalnum() or prev in "_)]>":  # indexing / type syntax, not a literal
+                v, j = parse_array(body, i)
+                i = j
+                continue
+            v, j = parse_array(body, i)
+            res.append(v)
+            i = j
+            continue
+        i += 1
+    return res
+
+
+def main():
+    for name, (rel, describes) in CASES.items():
+        src = open(os.path.join(REF, rel)).read()
+        out = {"source": rel, "cases": []}
+        for describe, title, body in blocks_of(src, describes):
+            if SKIP.search(title):
+                continue
+            out["cases"].append({"describe": describe, "title": title,
+                                 "consts": consts_of(body), "arrays": arrays_of(body)})
+        path = os.path.join(OUT, name + ".json")
+        with open(path, "w") as f:
+            json.dump(out, f, separators=(",", ":"))
+            f.write("\n")
+        print(name, len(out["cases"]), "cases", os.path.getsize(path), "bytes")
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,151 @@
+"""`ops` providers for tests/golden_recipes.py and the parity tests.
+
+Both expose the same tf-like calls on numpy arrays:
+  OracleOps — the CPU restatement of backend_cpu (oracle/cpu_ref.py);
+  HipOps    — the hip backend through the C ABI (tfhip python driver): every call uploads
+              its operands, runs the device kernels and reads the result back.
+"""
+import numpy as np
+
+
+class OracleOps:
+    name = "oracle"
+
+    def __init__(self):
+        from oracle import cpu_ref
+        self.r = cpu_ref
+
+    def matmul(self, a, b, ta=False, tb=False, bias=None, activation=None, prelu=None):
+        if a.size == 0 or b.size == 0:
+            m = a.shape[2] if ta else a.shape[1]
+            n = b.shape[1] if tb else b.shape[2]
+            return np.zeros((a.shape[0], m, n), np.float32)
+        return self.r.fused_batch_matmul(a, b, ta, tb, bias, activation, prelu)
+
+    def conv2d(self, x, w, strides, pad, dilations=1, bias=None, activation=None, prelu=None,
+               rounding=None):
+        ci = self.r.compute_conv2d_info(x.shape, w.shape, strides, dilations, pad, rounding)
+        return self.r.fused_conv2d(x, w, ci, bias, activation, prelu)
+
+    def depthwise_conv2d(self, x, w, strides, pad, dilations=1, bias=None, activation=None,
+                         rounding=None):
+        ci = self.r.compute_conv2d_info(x.shape, w.shape, strides, dilations, pad, rounding,
+                                        depthwise=True)
+        y = self.r.depthwise_conv2d(x, w, ci, pad_quirk=True)
+        if bias is not None:
+            y = self.r.add(y, bias)
+        return self.r._activation(y, activation, None)
+
+    def avg_pool(self, x, fsize, strides, pad, dilations=1, rounding=None):
+        return self.r.avg_pool(x, self.r.compute_pool2d_info(x.shape, fsize, strides, dilations,
+                                                              pad, rounding))
+
+    def max_pool(self, x, fsize, strides, pad, dilations=1, rounding=None):
+        return self.r.max_pool(x, self.r.compute_pool2d_info(x.shape, fsize, strides, dilations,
+                                                              pad, rounding))
+
+    def add(self, a, b): return self.r.add(a, b)
+    def sub(self, a, b): return self.r.subtract(a, b)
+    def mul(self, a, b): return self.r.multiply(a, b)
+    def div(self, a, b): return self.r.real_divide(a, b)
+    def prelu(self, x, alpha): return self.r.prelu(x, alpha)
+    def maximum(self, a, b): return self.r.maximum(a, b)
+    def minimum(self, a, b): return self.r.minimum(a, b)
+    def relu(self, x): return self.r.relu(x)
+    def clip(self, x, lo, hi): return self.r.clip(x, lo, hi)
+    def exp(self, x): return self.r.exp(x)
+    def log(self, x): return self.r.log(x)
+    def unary(self, name, x): return self.r._unary(name, x)
+    def sum(self, x): return self.r.sum_(x)
+    def max(self, x): return self.r.max_(x)
+    def min(self, x): return self.r.min_(x)
+    def argmax(self, x): return self.r.arg_max(x)
+    def argmin(self, x): return self.r.arg_min(x)
+    def softmax(self, x): return self.r.softmax(x)
+    def gather(self, x, idx, axis): return self.r.gather(x, idx, axis)
+    def transpose(self, x, perm): return self.r.transpose(x, perm)
+    def dequantize(self, q, scale, min_): return self.r.dequantize_u8(q, scale, min_)
+    def to_int(self, x): return self.r.to_int(x)
+
+
+class HipOps:
+    name = "hip"
+
+    def __init__(self):
+        import tfhip
+        self.tf = tfhip
+        self.tf.set_backend("hip")
+
+    def _run(self, fn, *arrays):
+        tf = self.tf
+        with tf.tidy():
+            ts = [None if a is None else tf.tensor(a) for a in arrays]
+            return fn(*ts).data_sync()
+
+    def matmul(self, a, b, ta=False, tb=False, bias=None, activation=None, prelu=None):
+        tf = self.tf
+        if bias is None and activation is None:
+            return self._run(lambda x, y: tf.matmul(x, y, ta, tb), a, b)
+        return self._run(lambda x, y, bi, pr: tf.fused.matmul(
+            x, y, ta, tb, bias=bi, activation=activation or "linear",
+            prelu_activation_weights=pr), a, b, bias, prelu)
+
+    def conv2d(self, x, w, strides, pad, dilations=1, bias=None, activation=None, prelu=None,
+               rounding=None):
+        tf = self.tf
+        if bias is None and activation is None:
+            return self._run(lambda a, b: tf.conv2d(a, b, strides, pad, "NHWC", dilations,
+                                                    rounding), x, w)
+        return self._run(lambda a, b, bi, pr: tf.fused.conv2d(
+            a, b, strides, pad, "NHWC", dilations, rounding, bias=bi,
+            activation=activation or "linear", prelu_activation_weights=pr), x, w, bias, prelu)
+
+    def depthwise_conv2d(self, x, w, strides, pad, dilations=1, bias=None, activation=None,
+                         rounding=None):
+        tf = self.tf
+        if bias is None and activation is None:
+            return self._run(lambda a, b: tf.depthwise_conv2d(a, b, strides, pad, "NHWC",
+                                                              dilations, rounding), x, w)
+        return self._run(lambda a, b, bi: tf.fused.depthwise_conv2d(
+            a, b, strides, pad, "NHWC", dilations, rounding, bias=bi,
+            activation=activation or "linear"), x, w, bias)
+
+    def avg_pool(self, x, fsize, strides, pad, dilations=1, rounding=None):
+        tf = self.tf
+        if dilations != 1:
+            return self._run(lambda a: tf.pool(a, fsize, "avg", pad, dilations, strides), x)
+        return self._run(lambda a: tf.avg_pool(a, fsize, strides, pad, rounding), x)
+
+    def max_pool(self, x, fsize, strides, pad, dilations=1, rounding=None):
+        tf = self.tf
+        if dilations != 1:
+            return self._run(lambda a: tf.pool(a, fsize, "max", pad, dilations, strides), x)
+        return self._run(lambda a: tf.max_pool(a, fsize, strides, pad, rounding), x)
+
+    def add(self, a, b): return self._run(self.tf.add, a, b)
+    def sub(self, a, b): return self._run(self.tf.sub, a, b)
+    def mul(self, a, b): return self._run(self.tf.mul, a, b)
+    def div(self, a, b): return self._run(self.tf.div, a, b)
+    def prelu(self, x, alpha): return self._run(self.tf.prelu, x, alpha)
+    def maximum(self, a, b): return self._run(self.tf.maximum, a, b)
+    def minimum(self, a, b): return self._run(self.tf.minimum, a, b)
+    def relu(self, x): return self._run(self.tf.relu, x)
+    def clip(self, x, lo, hi): return self._run(lambda t: self.tf.clip_by_value(t, lo, hi), x)
+    def exp(self, x): return self._run(self.tf.exp, x)
+    def log(self, x): return self._run(self.tf.log, x)
+    def unary(self, name, x): return self._run(getattr(self.tf, name), x)
+    def sum(self, x): return self._run(lambda t: self.tf.sum(t, -1), x)
+    def max(self, x): return self._run(lambda t: self.tf.max(t, -1), x)
+    def min(self, x): return self._run(lambda t: self.tf.min(t, -1), x)
+    def argmax(self, x): return self._run(lambda t: self.tf.arg_max(t, -1), x)
+    def argmin(self, x): return self._run(lambda t: self.tf.arg_min(t, -1), x)
+    def softmax(self, x): return self._run(self.tf.softmax, x)
+    def gather(self, x, idx, axis): return self._run(lambda t, i: self.tf.gather(t, i, axis), x, idx)
+    def transpose(self, x, perm): return self._run(lambda t: self.tf.transpose(t, perm), x)
+
+    def dequantize(self, q, scale, min_):
+        tf = self.tf
+        with tf.tidy():
+            return tf.dequantize(tf.quantized_tensor(q, scale, min_)).data_sync()
+
+    def to_int(self, x): return self._run(lambda t: self.tf.cast(t, "int32"), x)
