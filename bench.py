@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Headline benchmark: random-init MobileNetV1-1.0-224, fp32 NHWC, batch 64, one forward
+pass per step through the tf.* graph on the hip backend (one MI355X).
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 64] [--quant] [--no-cpu]
+
+Prints ONE JSON line: whole-job images/s (inputs resident in HBM before the timed region),
+the roofline of the kernel that takes the largest share of the step, timed live with HIP
+events on the backend's stream, and the CPU oracle timed on this host beside it.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "tfjs-core_amd", "python")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+RIDGE = PEAK_FP32_MFMA_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
+
+
+def per_layer_times(tf, mobilenet, w, x, reps):
+    """Time every layer of the forward pass on its real input with an event pair on the
+    backend's stream around `reps` back-to-back launches.  Returns rows with the kernel
+    variant the library chose, its average duration and its algorithmic work."""
+    be = tf.backend()
+    rows = []
+
+    def timed(fn):
+        out = fn()            # warm-up launch, also yields the layer's output
+        tf.dispose(out)
+        def many():
+            for _ in range(reps):
+                tf.dispose(fn())
+        ms = tf.time(many)["kernelMs"] / reps
+        kernel = be.lib.tfhip_last_kernel(be.ctx).decode()
+        return fn(), ms, kernel
+
+    table = mobilenet.layer_table(batch=x.shape[0])
+    h = x
+    ti = iter(table)
+    keep = []
+    row = next(ti)
+    h2, ms, k = timed(lambda: tf.fused.conv2d(h, w["stem_w"], 2, "same", bias=w["stem_b"],
+                                              activation="relu6"))
+    rows.append(dict(row, ms=ms, kernel=k))
+    keep.append(h2)
+    h = h2
+    for i, (_, s) in enumerate(mobilenet.BLOCKS, 1):
+        row = next(ti)
+        hin = h
+        h2, ms, k = timed(lambda: tf.fused.depthwise_conv2d(
+            hin, w["dw%d_w" % i], s, "same", bias=w["dw%d_b" % i], activation="relu6"))
+        rows.append(dict(row, ms=ms, kernel=k))
+        keep.append(h2)
+        row = next(ti)
+        hmid = h2
+        h3, ms, k = timed(lambda: tf.fused.conv2d(
+            hmid, w["pw%d_w" % i], 1, "same", bias=w["pw%d_b" % i], activation="relu6"))
+        rows.append(dict(row, ms=ms, kernel=k))
+        keep.append(h3)
+        h = h3
+    row = next(ti)
+    hin = h
+    h2, ms, k = timed(lambda: tf.avg_pool(hin, (hin.shape[1], hin.shape[2]), 1, "valid"))
+    rows.append(dict(row, ms=ms, kernel=k))
+    keep.append(h2)
+    row = next(ti)
+    flat = tf.reshape(h2, (h2.shape[0], h2.shape[3]))
+    keep.append(flat)
+    h3, ms, k = timed(lambda: tf.fused.matmul(flat, w["fc_w"], False, False, bias=w["fc_b"]))
+    rows.append(dict(row, ms=ms, kernel=k))
+    keep.append(h3)
+    tf.dispose(keep)
+    return rows
+
+
+def roofline_of_dominant_kernel(rows):
+    """Group the per-layer rows by kernel variant (what a profiler reports as one kernel
+    name), pick the variant with the largest share of the step, and price it: dense
+    variants against the fp32 matrix peak, streaming variants against HBM."""
+    groups = {}
+    for r in rows:
+        g = groups.setdefault(r["kernel"], dict(ms=0.0, flops=0.0, bytes=0.0, launches=0, layers=[]))
+        g["ms"] += r["ms"]
+        g["flops"] += 2.0 * r["macs"]
+        g["bytes"] += r["bytes"]
+        g["launches"] += 1
+        g["layers"].append(r["name"])
+    name, g = max(groups.items(), key=lambda kv: kv[1]["ms"])
+    ai = g["flops"] / g["bytes"]
+    sec = g["ms"] * 1e-3
+    if name.startswith("gemm") and ai >= RIDGE:
+        achieved = g["flops"] / sec / 1e12
+        roof = dict(bound="mfma", achieved=round(achieved, 3), peak=PEAK_FP32_MFMA_TFLOPS,
+                    unit="TFLOP/s", frac=round(achieved / PEAK_FP32_MFMA_TFLOPS, 4))
+    else:
+        achieved = g["bytes"] / sec / 1e9
+        roof = dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                    frac=round(achieved / PEAK_HBM_GBS, 4))
+    roof.update(kernel=name, launches_per_step=g["launches"], layers=g["layers"],
+                avg_launch_us=round(g["ms"] * 1e3 / g["launches"], 2),
+                share_of_step=round(g["ms"] / sum(r["ms"] for r in rows), 3), traffic=None)
+    return roof, groups
+
+
+def cpu_baseline(mobilenet, params, budget_s=20.0):
+    """The CPU oracle (restatement of backend_cpu's loops, one thread) on batch-1 forwards
+    of the same network: a bounded sample, reported as images/s."""
+    import numpy as np
+    from oracle import cpu_ref
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from providers import OracleOps
+    from providers import oracle_mobilenet_forward as oracle_forward
+    cpu_ref.build()
+    ref = OracleOps()
+    x = np.random.default_rng(5).uniform(0, 1, (1, 224, 224, 3)).astype(np.float32)
+    n, t0 = 0, time.perf_counter()
+    while True:
+        oracle_forward(ref, params, x)
+        n += 1
+        el = time.perf_counter() - t0
+        if el + el / n > budget_s or n >= 8:
+            break
+    return dict(value=round(n / el, 4), unit="images/s", cores=1, kind="port",
+                sample="%d batch-1 forward passes of the same MobileNetV1 (%.1f s), C restatement "
+                       "of backend_cpu at -O2, 1 thread" % (n, el))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--quant", action="store_true", help="uint8 weights dequantised in-kernel")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
+                 "(the path shards by batch, see DESIGN.md)" % args.gpus)
+
+    import numpy as np
+    import tfhip as tf
+    from tfhip import mobilenet
+    tf.set_backend("hip")
+    be = tf.backend()
+
+    params = mobilenet.make_params(seed=0)
+    dev_params = mobilenet.quantize_params(params) if args.quant else params
+    w = mobilenet.upload(tf, dev_params)
+    x_host = np.random.default_rng(1).uniform(0, 1, (args.batch, 224, 224, 3)).astype(np.float32)
+    x = tf.tensor(x_host)          # resident in HBM before the timed region
+    be.sync()
+
+    def step():
+        logits, probs = mobilenet.forward(tf, w, x)
+        tf.dispose([logits, probs])
+
+    for _ in range(args.warmup):
+        step()
+    be.sync()
+    t0 = time.perf_counter()
+    info = tf.time(lambda: [step() for _ in range(args.steps)])
+    be.sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    value = args.batch * args.steps / wall
+
+    rows = per_layer_times(tf, mobilenet, w, x, reps=20)
+    roof, groups = roofline_of_dominant_kernel(rows)
+    if args.layers:
+        for r in rows:
+            ai = 2.0 * r["macs"] / r["bytes"]
+            print("%-8s %-28s %8.1f us  %7.2f TFLOP/s  %7.1f GB/s  AI %6.1f" % (
+                r["name"], r["kernel"], r["ms"] * 1e3, 2e-9 * r["macs"] / r["ms"],
+                1e-6 * r["bytes"] / r["ms"], ai), file=sys.stderr)
+        print("sum of layer times: %.3f ms; step (events): %.3f ms; step (wall): %.3f ms" % (
+            sum(r["ms"] for r in rows), info["kernelMs"] / args.steps, ms_per_step), file=sys.stderr)
+
+    out = {
+        "metric": "MobileNetV1-224 images/s at batch 64" if args.batch == 64 and not args.quant
+                  else "MobileNetV1-224 images/s at batch %d%s" % (args.batch, " (uint8 weights)" if args.quant else ""),
+        "value": round(value, 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "MobileNetV1-1.0-224 random-init fp32 NHWC forward + softmax, "
+                               "batch %d%s, tf.* graph on the hip backend" % (
+                                   args.batch, ", uint8 weights" if args.quant else ""),
+                   "global_batch": args.batch, "host": "python ctypes driver over the C ABI"},
+        "gpu_ms_per_step_events": round(info["kernelMs"] / args.steps, 4),
+        "dense_tflops": round(sum(2e-9 * r["macs"] for r in rows if r["kernel"].startswith("gemm"))
+                              / sum(r["ms"] for r in rows if r["kernel"].startswith("gemm")), 2),
+        "roofline": roof,
+        "kernel_groups": {k: dict(ms=round(g["ms"], 4), launches=g["launches"],
+                                  tflops=round(g["flops"] / g["ms"] * 1e-9, 2),
+                                  gbs=round(g["bytes"] / g["ms"] * 1e-6, 1))
+                          for k, g in groups.items()},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(mobilenet, params)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

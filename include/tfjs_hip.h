@@ -89,32 +89,44 @@ int tfhip_sync(tfhip_ctx* ctx);
 /* KernelBackend.time (backend.ts:92, backend_cpu.ts:239-244): event pair on the stream. */
 int tfhip_time_begin(tfhip_ctx* ctx);
 int tfhip_time_end(tfhip_ctx* ctx, float* ms);
+/* Name of the kernel variant the last dense / image call launched (tile shape, operand
+ * layout), for matching launches to profiler rows.  Not part of the reference interface. */
+const char* tfhip_last_kernel(tfhip_ctx* ctx);
 /* Raw device address of an id's buffer (for callers that share the device, e.g. a
  * harness that generates inputs in HBM).  Not part of the reference interface. */
 int tfhip_device_ptr(tfhip_ctx* ctx, int64_t id, void** ptr, size_t* nbytes);
 
 /* ---- dense contractions ------------------------------------------------------------ */
+/* How a bias / prelu-alpha operand lines up with the [rows, N] result of a dense kernel.
+ * The reference accepts any shape broadcastable to the result (ops/fused_ops.ts:114-120,
+ * 340-346); the three layouts below are fused into the epilogue, any other shape is
+ * handled by the host as the reference's separate add / prelu pass. */
+enum {
+  TFHIP_BCAST_NONE = 0,    /* operand absent (id ignored) */
+  TFHIP_BCAST_SCALAR = 1,  /* 1 element */
+  TFHIP_BCAST_COLUMN = 2,  /* N elements, one per output column / channel */
+  TFHIP_BCAST_FULL = 3     /* same number of elements as the result */
+};
 /* batchMatMul / fusedBatchMatMul (backend.ts:128-138; backend_cpu.ts:491-555).
  * a: [batch,M,K] (or [batch,K,M] when transpose_a), b: [batch,K,N] (or [batch,N,K]),
- * out: [batch,M,N] float32.  bias / prelu: data id or -1; each must hold 1, N or
- * batch*M*N elements (scalar, per-column, full).  q: non-NULL iff b is TFHIP_UINT8Q. */
+ * out: [batch,M,N] float32.  q: non-NULL iff b is stored as TFHIP_UINT8Q. */
 int tfhip_matmul(tfhip_ctx* ctx, int64_t a, int64_t b, int64_t out, int batch, int m, int n,
-                 int k, int transpose_a, int transpose_b, int64_t bias, int act,
-                 int64_t prelu, const tfhip_qparams* q);
+                 int k, int transpose_a, int transpose_b, int64_t bias, int bias_kind, int act,
+                 int64_t prelu, int prelu_kind, const tfhip_qparams* q);
 /* conv2d / fusedConv2d (backend.ts:414-421; backend_cpu.ts:1536-1616): x NHWC,
  * filter [fh,fw,in_c,out_c], out NHWC float32.  bias/prelu/q as for tfhip_matmul with
- * N = out_c. */
+ * N = out_c and rows = batch*out_h*out_w. */
 int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t out,
-                 const tfhip_conv2d_info* info, int64_t bias, int act, int64_t prelu,
-                 const tfhip_qparams* q);
+                 const tfhip_conv2d_info* info, int64_t bias, int bias_kind, int act,
+                 int64_t prelu, int prelu_kind, const tfhip_qparams* q);
 
 /* ---- memory-bound image kernels ------------------------------------------------------ */
 /* depthwiseConv2D (backend.ts:431-434; backend_cpu.ts:1979-2035): filter
- * [fh,fw,in_c,ch_mul], out_c = in_c*ch_mul.  bias (-1 or out_c elements) and act
- * (LINEAR/RELU/RELU6) fold the add + clip that follow it in MobileNet into the same pass;
- * the reference issues them as separate add/clip calls.  q: filter may be UINT8Q. */
+ * [fh,fw,in_c,ch_mul], out_c = in_c*ch_mul.  bias (NONE / SCALAR / COLUMN over out_c) and
+ * act (LINEAR/RELU/RELU6) fold the add + clip that follow it in MobileNet into the same
+ * pass; the reference issues them as separate add/clip calls.  q: filter may be UINT8Q. */
 int tfhip_depthwise_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t out,
-                           const tfhip_conv2d_info* info, int64_t bias, int act,
+                           const tfhip_conv2d_info* info, int64_t bias, int bias_kind, int act,
                            const tfhip_qparams* q);
 /* avgPool / maxPool (backend.ts:453-462; backend_cpu.ts:2273-2345, 2869-2873). */
 enum { TFHIP_POOL_AVG = 0, TFHIP_POOL_MAX = 1 };
@@ -143,6 +155,10 @@ int tfhip_unary(tfhip_ctx* ctx, int op, int64_t x, int64_t out, float p0, float 
  * converts from x's stored dtype to out's stored dtype (float->int32 truncates,
  * ->bool is x != 0). */
 int tfhip_cast(tfhip_ctx* ctx, int64_t x, int64_t out);
+/* decodeWeights, quantised branch (io/io_utils.ts:122-147): x TFHIP_UINT8Q -> out float32,
+ * w = q*scale + min in double, rounded once.  The dense kernels do this while staging
+ * their B tile; this entry materialises the float weights for any other consumer. */
+int tfhip_dequantize(tfhip_ctx* ctx, int64_t x, int64_t out, const tfhip_qparams* q);
 /* fill/zerosLike/onesLike (backend.ts:629-640; backend_cpu.ts:3816-3836). */
 int tfhip_fill(tfhip_ctx* ctx, int64_t out, double value);
 
@@ -160,7 +176,7 @@ int tfhip_softmax_rows(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t rows, int
  * [outer, axis_dim, inner]; out [outer, n_indices, inner]; indices int32. */
 int tfhip_gather(tfhip_ctx* ctx, int64_t x, int64_t indices, int64_t out, int64_t outer,
                  int64_t axis_dim, int64_t inner, int64_t n_indices);
-/* transpose (backend.ts:497; backend_cpu.ts:2166-2202), rank <= 6. */
+/* transpose (backend.ts:497; backend_cpu.ts:2178-2200), rank <= 6. */
 int tfhip_transpose(tfhip_ctx* ctx, int64_t x, const int32_t* x_shape, int rank,
                     const int32_t* perm, int64_t out);
 /* Device-to-device copy between ids of equal byte size (identity / clone). */

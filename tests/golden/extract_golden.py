@@ -184,7 +184,114 @@ def arrays_of(body):
     return res
 
 
+def _eval_expr(tok, env):
+    """Evaluate a literal / identifier / array-of-those from the conv_util tests."""
+    tok = tok.strip()
+    if tok.startswith("["):
+        inner, parts, depth, cur = tok[1:-1], [], 0, ""
+        for ch in inner:
+            if ch == "[":
+                depth += 1
+            elif ch == "]":
+                depth -= 1
+            if ch == "," and depth == 0:
+                parts.append(cur)
+                cur = ""
+            else:
+                cur += ch
+        if cur.strip():
+            parts.append(cur)
+        return [_eval_expr(p, env) for p in parts]
+    if tok in ("null", "undefined"):
+        return None
+    if tok in ("true", "false"):
+        return tok == "true"
+    if tok[0] in "'\"":
+        return tok[1:-1]
+    if re.fullmatch(r"-?\d+", tok):
+        return int(tok)
+    if re.fullmatch(r"-?\d*\.\d+", tok):
+        return float(tok)
+    if tok in env:
+        return env[tok]
+    raise KeyError(tok)
+
+
+def _split_args(s):
+    parts, depth, cur = [], 0, ""
+    for ch in s:
+        if ch in "[(":
+            depth += 1
+        elif ch in "])":
+            depth -= 1
+        if ch == "," and depth == 0:
+            parts.append(cur)
+            cur = ""
+        else:
+            cur += ch
+    if cur.strip():
+        parts.append(cur)
+    return parts
+
+
+_DECL = re.compile(r"\bconst\s+([A-Za-z_$][\w$]*)\s*(?::[^=]+?)?=\s*([^;]+);")
+
+
+def extract_conv_util():
+    """ops/conv_util_test.ts: every computeConv2DInfo / computePool2DInfo call with literal
+    arguments, and the fields the test expects of the result (or that it must throw)."""
+    rel = "tfjs-core/src/ops/conv_util_test.ts"
+    src = open(os.path.join(REF, rel)).read()
+    out = {"source": rel, "cases": []}
+    for m in re.finditer(r"\bdescribe\(\s*'([^']*)'", src):
+        name = m.group(1)
+        if "3D" in name or "3d" in name or "convertConv2DDataFormat" in name:
+            continue
+        end = _match_paren(src, src.index("(", m.start()) + 1)
+        body = src[m.start():end]
+        first_it = body.find("it(")
+        env0 = {}
+        for d in _DECL.finditer(body[:first_it]):
+            try:
+                env0[d.group(1)] = _eval_expr(" ".join(d.group(2).split()), env0)
+            except KeyError:
+                pass
+        for it in re.finditer(r"\bit\(\s*'([^']*)'\s*,", body):
+            stop = _match_paren(body, body.index("(", it.start()) + 1)
+            blk = body[it.end():stop]
+            env = dict(env0)
+            for d in _DECL.finditer(blk):
+                try:
+                    env[d.group(1)] = _eval_expr(" ".join(d.group(2).split()), env)
+                except (KeyError, IndexError):
+                    pass
+            call = re.search(r"conv_util\.(computeConv2DInfo|computePool2DInfo)\(", blk)
+            if not call:
+                continue
+            cend = _match_paren(blk, call.end())
+            try:
+                args = [_eval_expr(" ".join(a.split()), env)
+                        for a in _split_args(blk[call.end():cend - 1])]
+            except KeyError:
+                continue
+            expect = {}
+            for e in re.finditer(r"expect\(\w+\.([\w.]+)\)\s*\.(?:toEqual|toBe)\(([^;]+)\);", blk):
+                try:
+                    expect[e.group(1)] = _eval_expr(" ".join(e.group(2).split()), env)
+                except KeyError:
+                    pass
+            out["cases"].append({"describe": name, "title": it.group(1), "fn": call.group(1),
+                                 "args": args, "throws": "toThrowError" in blk,
+                                 "expect": expect})
+    path = os.path.join(OUT, "conv_util.json")
+    with open(path, "w") as f:
+        json.dump(out, f, separators=(",", ":"))
+        f.write("\n")
+    print("conv_util", len(out["cases"]), "cases", os.path.getsize(path), "bytes")
+
+
 def main():
+    extract_conv_util()
     for name, (rel, describes) in CASES.items():
         src = open(os.path.join(REF, rel)).read()
         out = {"source": rel, "cases": []}

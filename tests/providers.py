@@ -149,3 +149,18 @@ class HipOps:
             return tf.dequantize(tf.quantized_tensor(q, scale, min_)).data_sync()
 
     def to_int(self, x): return self._run(lambda t: self.tf.cast(t, "int32"), x)
+
+
+def oracle_mobilenet_forward(ref, params, x):
+    """Same graph on the oracle: conv -> add -> clip(0,6) as backend_cpu would run it."""
+    from tfhip.mobilenet import BLOCKS
+    h = ref.conv2d(x, params["stem_w"], 2, "same", bias=params["stem_b"], activation="relu6")
+    for i, (_, s) in enumerate(BLOCKS, 1):
+        h = ref.depthwise_conv2d(h, params["dw%d_w" % i], s, "same", bias=params["dw%d_b" % i],
+                                 activation="relu6")
+        h = ref.conv2d(h, params["pw%d_w" % i], 1, "same", bias=params["pw%d_b" % i],
+                       activation="relu6")
+    h = ref.avg_pool(h, (h.shape[1], h.shape[2]), 1, "valid")
+    h = h.reshape(h.shape[0], h.shape[3])
+    logits = ref.matmul(h[None], params["fc_w"][None], bias=params["fc_b"])[0]
+    return logits, ref.softmax(logits)

@@ -1,0 +1,364 @@
+"""Parity of the hip backend with the CPU oracle on seeded random inputs, per op:
+float32 within 1e-4 relative / 1e-5 absolute, int32 / index results bit-exact."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def close(actual, expected, rtol=RTOL, atol=ATOL):
+    a = np.asarray(actual, np.float64)
+    e = np.asarray(expected, np.float64)
+    assert a.shape == e.shape, (a.shape, e.shape)
+    both_nan = np.isnan(a) & np.isnan(e)
+    err = np.abs(a - e)
+    ok = both_nan | (err <= atol + rtol * np.abs(e)) | (a == e)
+    assert ok.all(), "max err %g at %s (got %s want %s), %d bad of %d" % (
+        np.nanmax(np.where(ok, 0, err)), np.argwhere(~ok)[0], a[~ok][0], e[~ok][0],
+        (~ok).sum(), ok.size)
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from providers import HipOps
+    return HipOps()
+
+
+@pytest.fixture(scope="module")
+def ref(oracle):
+    from providers import OracleOps
+    return OracleOps()
+
+
+def rng_for(*key):
+    return np.random.default_rng(abs(hash(key)) % (2 ** 32))
+
+
+# ---------------------------------------------------------------- matmul ----
+def test_c1_matmul_256x512x256(hip, ref):
+    rng = np.random.default_rng(1)
+    a = rng.uniform(-1, 1, (1, 256, 512)).astype(np.float32)
+    b = rng.uniform(-1, 1, (1, 512, 256)).astype(np.float32)
+    close(hip.matmul(a, b), ref.matmul(a, b))
+
+
+@pytest.mark.parametrize("batch,m,k,n", [
+    (1, 1, 1, 1), (1, 7, 5, 3), (3, 33, 17, 65), (2, 129, 130, 131), (1, 300, 48, 10),
+    (1, 64, 1000, 32), (5, 2, 3, 2), (1, 257, 64, 64), (1, 513, 31, 40), (1, 40, 96, 257)])
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_matmul_shapes_and_transposes(hip, ref, batch, m, k, n, ta, tb):
+    print("matmul", batch, m, k, n, ta, tb, flush=True)
+    rng = np.random.default_rng(m * 1000 + k * 10 + n)
+    a = rng.uniform(-1, 1, (batch, k, m) if ta else (batch, m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (batch, n, k) if tb else (batch, k, n)).astype(np.float32)
+    close(hip.matmul(a, b, bool(ta), bool(tb)), ref.matmul(a, b, bool(ta), bool(tb)))
+
+
+@pytest.mark.parametrize("act", ["linear", "relu", "relu6", "prelu"])
+@pytest.mark.parametrize("bias_shape", [None, (), (24,), (1, 24), (2, 19, 24), (19, 1)])
+def test_fused_matmul_bias_and_activation(hip, ref, act, bias_shape):
+    rng = np.random.default_rng(11)
+    a = rng.standard_normal((2, 19, 40)).astype(np.float32) * 2
+    b = rng.standard_normal((2, 40, 24)).astype(np.float32)
+    bias = None if bias_shape is None else rng.standard_normal(bias_shape).astype(np.float32)
+    prelu = rng.uniform(0.1, 0.5, (24,)).astype(np.float32) if act == "prelu" else None
+    close(hip.matmul(a, b, bias=bias, activation=act, prelu=prelu),
+          ref.matmul(a, b, bias=bias, activation=act, prelu=prelu))
+
+
+def test_matmul_nan_and_inf_propagate(hip, ref):
+    a = np.ones((1, 4, 8), np.float32)
+    b = np.ones((1, 8, 4), np.float32)
+    a[0, 1, 3] = np.nan
+    b[0, 2, 2] = np.inf
+    close(hip.matmul(a, b, activation="relu"), ref.matmul(a, b, activation="relu"))
+
+
+def test_matmul_mixed_storage_dtypes(hip):
+    """float32 x int32 and int32 x bool (ops/matmul_test.ts:77-93)."""
+    import tfhip as tf
+    with tf.tidy():
+        a = tf.tensor(np.array([1, 2, 3, 4, 5, 6]), (2, 3), "float32")
+        b = tf.tensor(np.array([0, 1, -3, 2, 2, 1]), (3, 2), "int32")
+        c = tf.matmul(a, b)
+        assert c.dtype == "float32" and c.data_sync().ravel().tolist() == [0, 8, -3, 20]
+        a = tf.tensor(np.array([1, 2, 3, 4, 5, 6]), (2, 3), "int32")
+        b = tf.tensor(np.array([0, 1, -3, 2, 2, 1]), (3, 2), "bool")
+        c = tf.matmul(a, b)
+        assert c.dtype == "int32" and c.data_sync().ravel().tolist() == [5, 6, 11, 15]
+
+
+def test_c2_mlp_softmax_argmax(hip, ref):
+    """3-layer MLP 784->1024->1024->10 via fused matmul(bias+relu); batch cut to 256 so the
+    scalar oracle finishes in seconds.  argMax is checked bit-exactly on identical logits."""
+    rng = np.random.default_rng(2)
+    x = rng.uniform(0, 1, (1, 256, 784)).astype(np.float32)
+    dims = [784, 1024, 1024, 10]
+    hs, hr = x, x
+    for i in range(3):
+        w = (rng.standard_normal((1, dims[i], dims[i + 1])) * np.sqrt(2.0 / dims[i])).astype(np.float32)
+        bias = np.zeros(dims[i + 1], np.float32)
+        act = "relu" if i < 2 else "linear"
+        hs = hip.matmul(hs, w, bias=bias, activation=act)
+        hr = ref.matmul(hr, w, bias=bias, activation=act)
+        close(hs, hr)
+    logits = hr[0]
+    close(hip.softmax(logits), ref.softmax(logits))
+    assert np.array_equal(hip.argmax(logits), ref.argmax(logits))
+
+
+# ---------------------------------------------------------------- conv2d ----
+@pytest.mark.parametrize("xs,fs,stride,pad,dil", [
+    ((2, 12, 12, 8), (3, 3, 8, 16), 1, "same", 1),
+    ((1, 15, 13, 4), (3, 3, 4, 40), 2, "same", 1),
+    ((2, 16, 16, 3), (3, 3, 3, 32), 2, "same", 1),      # stem-like: Cin = 3
+    ((1, 9, 9, 5), (3, 3, 5, 7), 1, "valid", 1),        # Cin % 4 != 0
+    ((1, 14, 14, 64), (1, 1, 64, 128), 1, "same", 1),   # pointwise -> plain GEMM
+    ((1, 14, 14, 6), (1, 1, 6, 10), 2, "same", 1),      # 1x1 stride 2 stays implicit
+    ((1, 11, 11, 8), (5, 5, 8, 8), 1, "same", 1),
+    ((1, 13, 13, 4), (3, 3, 4, 8), 1, "same", 2),
+    ((1, 10, 12, 8), (2, 4, 8, 8), (1, 2), "valid", 1),
+    ((3, 7, 7, 32), (3, 3, 32, 200), 1, 1, 1),
+])
+def test_conv2d_shapes(hip, ref, xs, fs, stride, pad, dil):
+    print("conv2d", xs, fs, stride, pad, dil, flush=True)
+    rng = np.random.default_rng(sum(xs) + sum(fs))
+    x = rng.uniform(0, 1, xs).astype(np.float32)
+    w = (rng.standard_normal(fs) * np.sqrt(2.0 / (fs[0] * fs[1] * fs[2]))).astype(np.float32)
+    close(hip.conv2d(x, w, stride, pad, dil), ref.conv2d(x, w, stride, pad, dil))
+
+
+@pytest.mark.parametrize("act", ["linear", "relu", "relu6", "prelu"])
+@pytest.mark.parametrize("bias_kind", ["none", "scalar", "channel", "full", "odd"])
+def test_fused_conv2d_epilogues(hip, ref, act, bias_kind):
+    rng = np.random.default_rng(21)
+    x = rng.uniform(0, 1, (2, 10, 10, 8)).astype(np.float32)
+    w = rng.standard_normal((3, 3, 8, 12)).astype(np.float32)
+    bias = {"none": None, "scalar": rng.standard_normal(()).astype(np.float32),
+            "channel": rng.standard_normal(12).astype(np.float32),
+            "full": rng.standard_normal((2, 10, 10, 12)).astype(np.float32),
+            "odd": rng.standard_normal((10, 1)).astype(np.float32)}[bias_kind]
+    prelu = rng.uniform(0.1, 0.5, (1, 1, 12)).astype(np.float32) if act == "prelu" else None
+    close(hip.conv2d(x, w, 1, "same", bias=bias, activation=act, prelu=prelu),
+          ref.conv2d(x, w, 1, "same", bias=bias, activation=act, prelu=prelu))
+
+
+def test_c3_conv_and_depthwise_reduced_batch(hip, ref):
+    """Config 3 at its real spatial/channel shape, batch cut to 1 for the scalar oracle:
+    fusedConv2d 3x3 s1 same 64->128 + bias + relu6, depthwise 3x3 s1 on 128 ch + bias + relu6."""
+    rng = np.random.default_rng(3)
+    x = rng.uniform(0, 1, (1, 112, 112, 64)).astype(np.float32)
+    w = (rng.standard_normal((3, 3, 64, 128)) * np.sqrt(2.0 / 576)).astype(np.float32)
+    b = (rng.standard_normal(128) * 0.1).astype(np.float32)
+    y_ref = ref.conv2d(x, w, 1, "same", bias=b, activation="relu6")
+    y = hip.conv2d(x, w, 1, "same", bias=b, activation="relu6")
+    close(y, y_ref)
+    wd = (rng.standard_normal((3, 3, 128, 1)) * np.sqrt(2.0 / 9)).astype(np.float32)
+    bd = (rng.standard_normal(128) * 0.1).astype(np.float32)
+    close(hip.depthwise_conv2d(y_ref, wd, 1, "same", bias=bd, activation="relu6"),
+          ref.depthwise_conv2d(y_ref, wd, 1, "same", bias=bd, activation="relu6"))
+
+
+def test_c3_full_size_spot_check_against_float64():
+    """Config 3 at full size [32,112,112,64]: 400 random output positions of the conv and of
+    the depthwise recomputed in float64 from the inputs."""
+    import tfhip as tf
+    rng = np.random.default_rng(33)
+    x = rng.uniform(0, 1, (32, 112, 112, 64)).astype(np.float32)
+    w = (rng.standard_normal((3, 3, 64, 128)) * np.sqrt(2.0 / 576)).astype(np.float32)
+    b = (rng.standard_normal(128) * 0.1).astype(np.float32)
+    wd = (rng.standard_normal((3, 3, 128, 1)) * np.sqrt(2.0 / 9)).astype(np.float32)
+    with tf.tidy():
+        xt = tf.tensor(x)
+        yt = tf.fused.conv2d(xt, tf.tensor(w), 1, "same", bias=tf.tensor(b), activation="relu6")
+        zt = tf.fused.depthwise_conv2d(yt, tf.tensor(wd), 1, "same", bias=tf.tensor(b),
+                                       activation="relu6")
+        y, z = yt.data_sync(), zt.data_sync()
+    xp = np.pad(x, ((0, 0), (1, 1), (1, 1), (0, 0)))
+    yp = np.pad(y, ((0, 0), (1, 1), (1, 1), (0, 0)))
+    for _ in range(400):
+        n, i, j = rng.integers(32), rng.integers(112), rng.integers(112)
+        patch = xp[n, i:i + 3, j:j + 3, :].astype(np.float64)
+        want = np.einsum("abc,abco->o", patch, w.astype(np.float64)) + b
+        close(y[n, i, j], np.clip(want, 0, 6), rtol=1e-4, atol=1e-5)
+        dpatch = yp[n, i:i + 3, j:j + 3, :].astype(np.float64)
+        dwant = np.einsum("abc,abc->c", dpatch, wd[..., 0].astype(np.float64)) + b
+        close(z[n, i, j], np.clip(dwant, 0, 6), rtol=1e-4, atol=1e-5)
+
+
+# ------------------------------------------------------------- depthwise ----
+@pytest.mark.parametrize("xs,fs,stride,pad,dil", [
+    ((2, 14, 14, 32), (3, 3, 32, 1), 1, "same", 1),     # fast path, stride 1
+    ((2, 15, 13, 16), (3, 3, 16, 1), 2, "same", 1),     # fast path, stride 2, odd extent
+    ((1, 16, 16, 8), (3, 3, 8, 1), 2, "same", 1),       # stride 2, even extent: pad 0/1
+    ((1, 9, 9, 4), (3, 3, 4, 1), 1, "valid", 1),
+    ((1, 9, 9, 6), (3, 3, 6, 1), 1, "same", 1),         # C % 4 != 0 -> generic kernel
+    ((2, 8, 8, 4), (3, 3, 4, 2), 1, "same", 1),         # channel multiplier 2
+    ((1, 12, 12, 4), (5, 5, 4, 1), 1, "same", 1),
+    ((1, 12, 12, 4), (3, 3, 4, 1), 1, "same", 2),
+    ((1, 7, 7, 1024), (3, 3, 1024, 1), 1, "same", 1),
+])
+def test_depthwise_shapes(hip, ref, xs, fs, stride, pad, dil):
+    print("depthwise", xs, fs, stride, pad, dil, flush=True)
+    rng = np.random.default_rng(sum(xs) * 7 + sum(fs))
+    x = rng.uniform(0, 1, xs).astype(np.float32)
+    w = rng.standard_normal(fs).astype(np.float32)
+    close(hip.depthwise_conv2d(x, w, stride, pad, dil), ref.depthwise_conv2d(x, w, stride, pad, dil))
+    bias = rng.standard_normal(fs[2] * fs[3]).astype(np.float32)
+    for act in ("linear", "relu", "relu6"):
+        close(hip.depthwise_conv2d(x, w, stride, pad, dil, bias=bias, activation=act),
+              ref.depthwise_conv2d(x, w, stride, pad, dil, bias=bias, activation=act))
+
+
+# ------------------------------------------------------------------ pool ----
+@pytest.mark.parametrize("xs,f,s,pad", [
+    ((4, 7, 7, 1024), 7, 1, "valid"), ((2, 8, 8, 6), 2, 2, "valid"), ((1, 9, 9, 4), 3, 2, "same"),
+    ((2, 5, 7, 3), (2, 3), 1, "same"), ((1, 7, 7, 10), 7, 1, "valid")])
+def test_pool_shapes(hip, ref, xs, f, s, pad):
+    rng = np.random.default_rng(sum(xs))
+    x = rng.standard_normal(xs).astype(np.float32)
+    close(hip.avg_pool(x, f, s, pad), ref.avg_pool(x, f, s, pad))
+    assert np.array_equal(hip.max_pool(x, f, s, pad), ref.max_pool(x, f, s, pad))
+
+
+# ----------------------------------------------------------- elementwise ----
+@pytest.mark.parametrize("sa,sb", [
+    ((1024,), (1024,)), ((33, 7), (33, 7)), ((64, 128), (128,)), ((128,), (64, 128)),
+    ((5, 6), ()), ((), (5, 6)), ((4, 1, 3), (1, 5, 3)), ((2, 3, 4, 5), (3, 1, 5)),
+    ((7, 1), (1, 9)), ((2, 2, 2, 2, 2, 2), (2, 2))])
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div", "maximum", "minimum", "prelu"])
+def test_binary_broadcast(hip, ref, op, sa, sb):
+    rng = np.random.default_rng(len(sa) * 10 + len(sb))
+    a = rng.standard_normal(sa).astype(np.float32)
+    b = rng.standard_normal(sb).astype(np.float32) + np.float32(3.0 if op == "div" else 0.0)
+    if op == "prelu" and len(sb) > len(sa):
+        pytest.skip("prelu alpha broadcasts onto x")
+    close(getattr(hip, op)(a, b), getattr(ref, op)(a, b), rtol=1e-6, atol=1e-7)
+
+
+def test_binary_int32_and_nan(hip, ref):
+    a = np.array([[1, -2, 3], [40000, 5, -6]], np.int32)
+    b = np.array([7, 8, -9], np.int32)
+    for op in ("add", "sub", "mul"):
+        r = getattr(hip, op)(a, b)
+        assert r.dtype == np.int32 and np.array_equal(r, getattr(ref, op)(a, b))
+    x = np.array([1, np.nan, -1, np.inf], np.float32)
+    y = np.array([np.nan, 2, 3, -np.inf], np.float32)
+    for op in ("add", "mul", "maximum", "minimum"):
+        close(getattr(hip, op)(x, y), getattr(ref, op)(x, y))
+
+
+@pytest.mark.parametrize("name", ["relu", "exp", "log", "neg", "abs", "sigmoid", "sqrt", "square",
+                                  "tanh", "rsqrt"])
+def test_unary(hip, ref, name):
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((37, 29)) * 4).astype(np.float32)
+    if name in ("log", "sqrt", "rsqrt"):
+        x = np.abs(x) + np.float32(0.01)
+    x.ravel()[:3] = [np.nan, np.inf, -np.inf] if name not in ("log", "sqrt", "rsqrt") else [np.nan, np.inf, 1]
+    close(hip.unary(name, x), ref.unary(name, x), rtol=1e-5, atol=1e-6)
+    close(hip.unary(name, x.ravel()[:1000]), ref.unary(name, x.ravel()[:1000]), rtol=1e-5, atol=1e-6)
+
+
+def test_clip_relu6_nan(hip, ref):
+    x = np.array([-3, 0, 2.5, 6, 7.5, np.nan, np.inf, -np.inf], np.float32)
+    close(hip.clip(x, 0, 6), ref.clip(x, 0, 6))
+    assert np.isnan(hip.clip(x, 0, 6)[5]) and np.isnan(hip.relu(x)[5])
+
+
+def test_exp_log_accuracy_at_large_arguments(hip, ref):
+    x = np.linspace(-87, 88, 4001, dtype=np.float32)
+    close(hip.exp(x), ref.exp(x), rtol=1e-5, atol=0)
+    y = np.logspace(-37, 38, 4001, dtype=np.float32)
+    close(hip.log(y), ref.log(y), rtol=1e-6, atol=1e-6)
+
+
+# ------------------------------------------------------------ reductions ----
+@pytest.mark.parametrize("rows,cols", [(1, 1), (4096, 10), (64, 1000), (3, 63), (5, 64), (7, 65),
+                                       (2, 5000)])
+def test_reductions(hip, ref, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    close(hip.sum(x), ref.sum(x), rtol=1e-6, atol=1e-6)
+    assert np.array_equal(hip.max(x), ref.max(x))
+    assert np.array_equal(hip.min(x), ref.min(x))
+    a, e = hip.argmax(x), ref.argmax(x)
+    assert a.dtype == np.int32 and np.array_equal(a, e)
+    assert np.array_equal(hip.argmin(x), ref.argmin(x))
+    close(hip.softmax(x), ref.softmax(x), rtol=1e-4, atol=1e-7)
+
+
+def test_argmax_ties_nan_and_windows(hip, ref):
+    x = np.zeros((6, 200), np.float32)
+    x[0, [5, 70, 130]] = 1          # tie across lanes: first index wins
+    x[1, 0] = np.nan                # NaN in slot 0 keeps index 0
+    x[1, 50] = 9
+    x[2, 3] = np.nan                # NaN elsewhere is skipped
+    x[2, 199] = 2
+    x[3, :] = -np.inf
+    x[4, 64] = 1                    # first element of the second lane sweep
+    x[5, :] = np.arange(200)[::-1]
+    assert np.array_equal(hip.argmax(x), ref.argmax(x))
+    assert np.array_equal(hip.argmin(x), ref.argmin(x))
+    close(hip.max(x), ref.max(x))
+    close(hip.min(x), ref.min(x))
+
+
+def test_sum_int32_and_bool(hip):
+    import tfhip as tf
+    with tf.tidy():
+        r = tf.sum(tf.tensor(np.array([[1, 5], [7, 3]], np.int32)), -1)
+        assert r.dtype == "int32" and r.data_sync().tolist() == [6, 10]
+        r = tf.sum(tf.tensor(np.array([True, False, False, True, True])))
+        assert r.dtype == "int32" and r.data_sync().tolist() == 3
+        r = tf.sum(tf.tensor(np.arange(12, dtype=np.float32).reshape(3, 4)), 0)  # via transpose
+        assert r.data_sync().tolist() == [12, 15, 18, 21]
+        r = tf.arg_max(tf.tensor(np.array([[3, -1, 0], [100, -7, 2]], np.float32)), 0)
+        assert r.data_sync().tolist() == [1, 0, 1]
+
+
+# -------------------------------------------------------- data movement ----
+def test_gather_transpose_cast(hip, ref):
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((5, 6, 7)).astype(np.float32)
+    idx = np.array([4, 0, 0, 3, 2], np.int32)
+    for axis in (0, 1, 2):
+        assert np.array_equal(hip.gather(x, idx, axis), ref.gather(x, idx, axis))
+    xi = rng.integers(-50, 50, (9, 4)).astype(np.int32)
+    r = hip.gather(xi, np.array([8, 1], np.int32), 0)
+    assert r.dtype == np.int32 and np.array_equal(r, xi[[8, 1]])
+    for perm in ([2, 0, 1], [1, 0, 2], [0, 2, 1], [2, 1, 0]):
+        assert np.array_equal(hip.transpose(x, perm), ref.transpose(x, perm))
+    v = np.array([1.9, -1.9, 0.5, np.nan, np.inf, 3e9, -7.0], np.float32)
+    assert np.array_equal(hip.to_int(v), ref.to_int(v))
+
+
+# ------------------------------------------------------------ quantised ----
+def test_uint8_weights_dequantised_in_kernel(hip, ref):
+    """matmul / conv2d / depthwise with uint8 affine-quantised weights vs the oracle run on
+    the weights decodeWeights would produce (q*scale+min in double, rounded once)."""
+    import tfhip as tf
+    rng = np.random.default_rng(12)
+    scale, mn = 0.0137, -1.73
+    q = rng.integers(0, 256, (40, 24)).astype(np.uint8)
+    assert np.array_equal(hip.dequantize(q, scale, mn), ref.dequantize(q, scale, mn))
+    a = rng.standard_normal((1, 19, 40)).astype(np.float32)
+    w = ref.dequantize(q, scale, mn)
+    with tf.tidy():
+        r = tf.fused.matmul(tf.tensor(a[0]), tf.quantized_tensor(q, scale, mn), False, False,
+                            bias=tf.tensor(np.ones(24, np.float32)), activation="relu").data_sync()
+    close(r, ref.matmul(a, w[None], bias=np.ones(24, np.float32), activation="relu")[0])
+    x = rng.uniform(0, 1, (2, 9, 9, 8)).astype(np.float32)
+    for fs in ((3, 3, 8, 12), (1, 1, 8, 16), (3, 3, 8, 5)):
+        qf = rng.integers(0, 256, fs).astype(np.uint8)
+        with tf.tidy():
+            r = tf.conv2d(tf.tensor(x), tf.quantized_tensor(qf, scale, mn), 1, "same").data_sync()
+        close(r, ref.conv2d(x, ref.dequantize(qf, scale, mn), 1, "same"))
+    for fs, c in (((3, 3, 8, 1), 8), ((3, 3, 8, 2), 8)):
+        qf = rng.integers(0, 256, fs).astype(np.uint8)
+        with tf.tidy():
+            r = tf.depthwise_conv2d(tf.tensor(x), tf.quantized_tensor(qf, scale, mn), 1,
+                                    "same").data_sync()
+        close(r, ref.depthwise_conv2d(x, ref.dequantize(qf, scale, mn), 1, "same"))

@@ -1,0 +1,145 @@
+"""Storage contract of the backend (register / write / read / dispose / memory / time /
+moveData) through the C ABI, after tfjs-backend-wasm/src/index_test.ts:29-49,
+backends/cpu/backend_cpu_test.ts:135-175 and engine_test.ts:307-368, 452-609."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tf():
+    import tfhip
+    tfhip.set_backend("hip")
+    return tfhip
+
+
+def test_write_read_round_trip_all_dtypes(tf):
+    with tf.tidy():
+        f = tf.tensor(np.array([1.5, -2.25, 3e10], np.float32))
+        i = tf.tensor(np.array([1, -2, 2 ** 31 - 1], np.int32))
+        b = tf.tensor(np.array([True, False, True]))
+        assert f.data_sync().tolist() == [1.5, -2.25, 3e10] and f.dtype == "float32"
+        assert i.data_sync().tolist() == [1, -2, 2 ** 31 - 1] and i.dtype == "int32"
+        assert b.data_sync().tolist() == [1, 0, 1] and b.dtype == "bool"
+        z = tf.tensor(np.zeros((0, 3), np.float32))
+        assert z.data_sync().shape == (0, 3)
+
+
+def test_overwrite_live_buffer(tf):
+    with tf.tidy():
+        t = tf.tensor(np.zeros(4, np.float32))
+        tf.backend().write(t.data_id, np.arange(4, dtype=np.float32))
+        assert t.data_sync().tolist() == [0, 1, 2, 3]
+
+
+def test_register_twice_and_null_write_throw(tf):
+    be = tf.backend()
+    with tf.tidy():
+        t = tf.tensor(np.zeros(4, np.float32))
+        with pytest.raises(RuntimeError, match="already registered"):
+            be.register(t.data_id, (4,), "float32")
+        with pytest.raises(ValueError, match="can not be null"):
+            be.write(t.data_id, None)
+    # the C ABI itself reports the same two conditions
+    h = 10 ** 9
+    shape = (C.c_int32 * 1)(4)
+    assert be.lib.tfhip_register(be.ctx, h, shape, 1, 0) == 0
+    assert be.lib.tfhip_register(be.ctx, h, shape, 1, 0) != 0
+    assert b"already registered" in be.lib.tfhip_last_error(be.ctx)
+    assert be.lib.tfhip_write(be.ctx, h, None, 16) != 0
+    assert be.lib.tfhip_write(be.ctx, h, None, 8) != 0      # wrong size
+    assert be.lib.tfhip_read(be.ctx, h + 1, None, 0) != 0   # unknown id
+    assert be.lib.tfhip_dispose(be.ctx, h) == 0
+    assert be.lib.tfhip_dispose(be.ctx, h) == 0             # disposing again is a no-op
+
+
+def test_memory_accounting_and_pool_reuse(tf):
+    """Freed blocks are reused: allocate / free cycles do not grow the device footprint
+    (index_test.ts:41-49 'allocation reuse')."""
+    be = tf.backend()
+    base = tf.memory()
+    t = tf.tensor(np.zeros(1000, np.float32))
+    m1 = tf.memory()
+    assert m1["numTensors"] == base["numTensors"] + 1
+    assert m1["numBytes"] == base["numBytes"] + 4000
+    assert m1["numDeviceBuffers"] == base["numDeviceBuffers"] + 1
+    ptr = C.c_void_p()
+    be._ck(be.lib.tfhip_device_ptr(be.ctx, be._h(t), C.byref(ptr), None))
+    first = ptr.value
+    t.dispose()
+    total = lambda m: m["numBytesInGPU"] + m["numBytesInGPUPool"]
+    footprint = total(tf.memory())
+    for _ in range(5):
+        t = tf.tensor(np.ones(1000, np.float32))
+        be._ck(be.lib.tfhip_device_ptr(be.ctx, be._h(t), C.byref(ptr), None))
+        assert ptr.value == first, "the freed block should be handed out again"
+        t.dispose()
+    assert total(tf.memory()) == footprint
+    assert tf.memory()["numTensors"] == base["numTensors"]
+
+
+def test_reshape_and_widening_cast_alias_the_buffer(tf):
+    with tf.tidy():
+        a = tf.tensor(np.array([1, 2, 3, 4], np.int32))
+        n0 = tf.memory()["numDataBuffers"]
+        r = tf.reshape(a, (2, 2))
+        f = tf.cast(a, "float32")       # int32 -> float32: same data id, int32 storage
+        assert tf.memory()["numDataBuffers"] == n0
+        assert r.data_id is a.data_id and f.data_id is a.data_id
+        # kernels convert from the stored dtype
+        s = tf.add(f, tf.tensor(np.float32(0.5)))
+        assert s.dtype == "float32" and s.data_sync().tolist() == [1.5, 2.5, 3.5, 4.5]
+        m = tf.matmul(tf.reshape(f, (2, 2)), tf.tensor(np.eye(2, dtype=np.float32)))
+        assert m.data_sync().ravel().tolist() == [1, 2, 3, 4]
+        a.dispose()
+        assert r.data_sync().ravel().tolist() == [1, 2, 3, 4], "alias keeps the buffer alive"
+        i = tf.cast(tf.tensor(np.array([1.9, -1.9], np.float32)), "int32")   # narrowing: copy
+        assert i.data_sync().tolist() == [1, -1]
+        b = tf.cast(tf.tensor(np.array([0.0, 2.0, np.nan], np.float32)), "bool")
+        assert b.data_sync().tolist() == [0, 1, 1]
+
+
+def test_move_data_from_another_backend(tf):
+    """A tensor created on another backend is moved on first use (engine.ts:361-363)."""
+    from test_host_logic import FakeBackend
+    from tfhip.engine import ENGINE
+    fake = FakeBackend()
+    tf.register_backend("fake-move", lambda: fake, 0)
+    try:
+        tf.set_backend("fake-move")
+        a = tf.tensor(np.array([1, 2, 3], np.float32))
+        assert len(fake.live) == 1
+        tf.set_backend("hip")
+        r = tf.add(a, tf.tensor(np.float32(1)))
+        assert r.data_sync().tolist() == [2, 3, 4]
+        assert len(fake.live) == 0, "data left the source backend"
+        a.dispose()
+        r.dispose()
+    finally:
+        tf.set_backend("hip")
+        tf.remove_backend("fake-move")
+
+
+def test_time_returns_kernel_ms(tf):
+    with tf.tidy():
+        a = tf.tensor(np.ones((512, 512), np.float32))
+        info = tf.time(lambda: tf.matmul(a, a))
+        assert info["kernelMs"] > 0
+    assert tf.backend().float_precision() == 32 and tf.backend().epsilon() == 1e-7
+
+
+def test_errors_come_back_as_exceptions(tf):
+    with tf.tidy():
+        a = tf.tensor(np.ones((2, 3), np.float32))
+        with pytest.raises(ValueError, match="inner shapes"):
+            tf.matmul(a, a)
+        with pytest.raises(ValueError, match="could not be broadcast"):
+            tf.add(a, tf.tensor(np.ones((2, 2), np.float32)))
+        with pytest.raises(ValueError, match="has not been implemented"):
+            tf.fused.matmul(a, tf.tensor(np.ones((3, 2), np.float32)), activation="elu")
+        with pytest.raises(ValueError, match="depth of input"):
+            tf.conv2d(tf.tensor(np.ones((1, 4, 4, 3), np.float32)),
+                      tf.tensor(np.ones((3, 3, 2, 8), np.float32)), 1, "same")

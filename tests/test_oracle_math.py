@@ -1,0 +1,175 @@
+"""Pins the CPU oracle against what the mathematics fixes (float64 brute force, identities,
+closed forms), so a dropped term, swapped index or wrong sign in the restatement fails
+here.  No GPU needed."""
+import numpy as np
+import pytest
+
+from providers import OracleOps
+
+
+@pytest.fixture(scope="module")
+def ops(oracle):
+    return OracleOps()
+
+
+def rel_close(a, e, rel=1e-5, ab=1e-6):
+    a, e = np.asarray(a, np.float64), np.asarray(e, np.float64)
+    assert a.shape == e.shape
+    assert np.all(np.abs(a - e) <= ab + rel * np.abs(e)), float(np.max(np.abs(a - e)))
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_matmul_vs_float64(ops, ta, tb):
+    rng = np.random.default_rng(1)
+    a = rng.uniform(-1, 1, (3, 37, 101)).astype(np.float32)
+    b = rng.uniform(-1, 1, (3, 101, 53)).astype(np.float32)
+    want = np.matmul(a.astype(np.float64), b.astype(np.float64))
+    aa = np.ascontiguousarray(a.transpose(0, 2, 1)) if ta else a
+    bb = np.ascontiguousarray(b.transpose(0, 2, 1)) if tb else b
+    rel_close(ops.matmul(aa, bb, bool(ta), bool(tb)), want)
+
+
+def test_matmul_identity_and_k_blocking(ops):
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal((1, 50, 97)).astype(np.float32)  # K=97 spans three 48-blocks
+    eye = np.eye(97, dtype=np.float32)[None]
+    assert np.array_equal(ops.matmul(a, eye), a)
+
+
+def _conv_brute(x, w, sh, sw, dh, dw, pt, pl, oh, ow):
+    n, h, wd, c = x.shape
+    fh, fw, _, oc = w.shape
+    y = np.zeros((n, oh, ow, oc))
+    for i in range(oh):
+        for j in range(ow):
+            for a in range(fh):
+                for b in range(fw):
+                    r, q = i * sh - pt + a * dh, j * sw - pl + b * dw
+                    if 0 <= r < h and 0 <= q < wd:
+                        y[:, i, j, :] += x[:, r, q, :].astype(np.float64) @ w[a, b].astype(np.float64)
+    return y
+
+
+@pytest.mark.parametrize("shape,fshape,stride,pad,dil", [
+    ((2, 9, 7, 5), (3, 3, 5, 6), 1, "same", 1),
+    ((1, 10, 10, 3), (3, 3, 3, 8), 2, "same", 1),    # even size, stride 2: pad 0 / 1
+    ((1, 11, 9, 4), (3, 3, 4, 4), 2, "same", 1),     # odd size, stride 2: pad 1 / 1
+    ((1, 8, 8, 2), (2, 3, 2, 3), (1, 2), "valid", 1),
+    ((1, 9, 9, 2), (3, 3, 2, 2), 1, "same", 2),
+    ((2, 6, 6, 4), (1, 1, 4, 7), 1, 0, 1),
+])
+def test_conv2d_vs_float64_brute_force(ops, oracle, shape, fshape, stride, pad, dil):
+    rng = np.random.default_rng(3)
+    x = rng.uniform(0, 1, shape).astype(np.float32)
+    w = rng.standard_normal(fshape).astype(np.float32)
+    ci = oracle.compute_conv2d_info(shape, fshape, stride, dil, pad)
+    p = ci["padInfo"]
+    want = _conv_brute(x, w, ci["strideHeight"], ci["strideWidth"], ci["dilationHeight"],
+                       ci["dilationWidth"], p["top"], p["left"], ci["outHeight"], ci["outWidth"])
+    rel_close(ops.conv2d(x, w, stride, pad, dil), want, rel=1e-5, ab=1e-5)
+
+
+def test_pointwise_conv_is_matmul(ops):
+    rng = np.random.default_rng(4)
+    x = rng.uniform(0, 1, (2, 5, 5, 16)).astype(np.float32)
+    w = rng.standard_normal((1, 1, 16, 8)).astype(np.float32)
+    y = ops.conv2d(x, w, 1, "same")
+    mm = ops.matmul(x.reshape(1, 50, 16), w.reshape(1, 16, 8))
+    rel_close(y.reshape(50, 8), mm[0], rel=1e-5)
+
+
+@pytest.mark.parametrize("stride,ch_mul,pad", [(1, 1, "same"), (2, 1, "same"), (1, 2, "valid")])
+def test_depthwise_is_grouped_conv(ops, stride, ch_mul, pad):
+    rng = np.random.default_rng(5)
+    c = 6
+    x = rng.uniform(0, 1, (2, 8, 8, c)).astype(np.float32)
+    w = rng.standard_normal((3, 3, c, ch_mul)).astype(np.float32)
+    y = ops.depthwise_conv2d(x, w, stride, pad)
+    # one dense conv per input channel, picking that channel's filters
+    for ch in range(c):
+        dense = ops.conv2d(x[..., ch:ch + 1], w[:, :, ch:ch + 1, :], stride, pad)
+        rel_close(y[..., ch * ch_mul:(ch + 1) * ch_mul], dense, rel=1e-5)
+
+
+def test_avg_pool_counts_only_in_bounds_pixels(ops):
+    x = np.arange(1, 10, dtype=np.float32).reshape(1, 3, 3, 1)
+    y = ops.avg_pool(x, 2, 1, "same")[0, :, :, 0]
+    want = np.array([[3, 4, 4.5], [6, 7, 7.5], [7.5, 8.5, 9]])
+    rel_close(y, want)
+    g = ops.avg_pool(np.ones((2, 7, 7, 8), np.float32) * 3, 7, 1, "valid")
+    assert g.shape == (2, 1, 1, 8) and np.all(g == 3)
+
+
+def test_softmax_closed_form_and_rows_sum_to_one(ops):
+    rng = np.random.default_rng(6)
+    x = (rng.standard_normal((17, 1000)) * 5).astype(np.float32)
+    y = ops.softmax(x)
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(-1, keepdims=True))
+    rel_close(y, e / e.sum(-1, keepdims=True), rel=1e-4, ab=1e-7)
+    rel_close(y.sum(-1), np.ones(17), rel=1e-5)
+
+
+def test_argmax_first_max_wins_and_nan_rules(ops):
+    assert ops.argmax(np.array([[1, 5, 5, 2]], np.float32)).tolist() == [1]
+    assert ops.argmax(np.array([[np.nan, 5, 7]], np.float32)).tolist() == [0]
+    assert ops.argmax(np.array([[1, np.nan, 7]], np.float32)).tolist() == [2]
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((64, 1000)).astype(np.float32)
+    assert np.array_equal(ops.argmax(x), np.argmax(x, -1).astype(np.int32))
+    assert np.array_equal(ops.argmin(x), np.argmin(x, -1).astype(np.int32))
+
+
+def test_reductions_and_elementwise_closed_forms(ops):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((9, 33)).astype(np.float32)
+    rel_close(ops.sum(x), x.astype(np.float64).sum(-1), rel=1e-6)
+    assert np.array_equal(ops.max(x), x.max(-1))
+    assert np.array_equal(ops.min(x), x.min(-1))
+    b = rng.standard_normal(33).astype(np.float32)
+    assert np.array_equal(ops.add(x, b), x + b)
+    assert np.array_equal(ops.sub(x, b), x - b)
+    assert np.array_equal(ops.mul(x, b), x * b)
+    col = rng.standard_normal((9, 1)).astype(np.float32)
+    assert np.array_equal(ops.add(x, col), x + col)      # general broadcast path
+    assert np.array_equal(ops.relu(x), np.maximum(x, 0))
+    assert np.array_equal(ops.clip(x * 10, 0, 6), np.clip(x * 10, 0, 6))
+    rel_close(ops.exp(x), np.exp(x.astype(np.float64)), rel=1e-6)
+    rel_close(ops.log(np.abs(x) + 1), np.log(np.abs(x.astype(np.float64)) + 1), rel=1e-6)
+    ints = np.array([1, 2, 3], np.int32)
+    r = ops.add(ints, np.array([10, 20, 30], np.int32))
+    assert r.dtype == np.int32 and r.tolist() == [11, 22, 33]
+
+
+def test_fused_is_matmul_then_add_then_activation(ops):
+    rng = np.random.default_rng(9)
+    a = rng.standard_normal((2, 6, 10)).astype(np.float32)
+    b = rng.standard_normal((2, 10, 4)).astype(np.float32)
+    bias = rng.standard_normal(4).astype(np.float32)
+    base = ops.matmul(a, b)
+    assert np.array_equal(ops.matmul(a, b, bias=bias, activation="relu"),
+                          np.maximum(base + bias, 0))
+    assert np.array_equal(ops.matmul(a, b, bias=bias, activation="relu6"),
+                          np.clip(base + bias, 0, 6))
+    alpha = np.float32(0.25)
+    z = base + bias
+    assert np.array_equal(ops.matmul(a, b, bias=bias, activation="prelu",
+                                     prelu=np.array([alpha], np.float32)),
+                          np.where(z < 0, alpha * z, z))
+
+
+def test_dequantize_is_double_then_round(ops):
+    q = np.arange(256, dtype=np.uint8)
+    scale, mn = 0.0123456789, -1.57
+    want = (q.astype(np.float64) * scale + mn).astype(np.float32)
+    assert np.array_equal(ops.dequantize(q, scale, mn), want)
+
+
+def test_gather_transpose_to_int(ops):
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((3, 4, 5)).astype(np.float32)
+    idx = np.array([3, 0, 0, 2], np.int32)
+    assert np.array_equal(ops.gather(x, idx, 1), np.take(x, idx, 1))
+    assert np.array_equal(ops.transpose(x, [2, 0, 1]), x.transpose(2, 0, 1))
+    v = np.array([1.9, -1.9, 0.5, np.nan, np.inf, 3e9], np.float32)
+    assert ops.to_int(v).tolist() == [1, -1, 0, 0, 0, int(np.int64(3000000000) - 2**32)]

@@ -1,0 +1,352 @@
+// Memory-bound NHWC image kernels: depthwiseConv2D (+ folded bias / relu / relu6) and
+// avg / max pooling.  Replaces backend_cpu.ts:1979-2035 and :2273-2345 of the reference.
+//
+// Both stream the activation tensor through HBM once.  Lanes run along the channel axis
+// (4 channels = 16 bytes per lane) so every wavefront access is a run of contiguous
+// 16-byte pieces; the 3x3 kernel keeps a TH x TW patch of outputs per lane in registers so
+// each input vector fetched is used by up to 9 multiply-adds without going back to L2.
+#include <type_traits>
+
+#include "tfhip_internal.h"
+
+namespace tfhip {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float dq(unsigned q, double scale, double mn) {
+#pragma clang fp contract(off)
+  double v = (double)q * scale;
+  v = v + mn;
+  return (float)v;
+}
+
+__device__ __forceinline__ float act_f(float v, int act) {
+  switch (act) {
+    case TFHIP_ACT_RELU: return (v > 0.f || v != v) ? v : 0.f;
+    case TFHIP_ACT_RELU6: return v > 6.f ? 6.f : (v < 0.f ? 0.f : v);
+    default: return v;
+  }
+}
+
+struct DwArgs {
+  const float* x;
+  const void* w;
+  const float* bias;
+  float* y;
+  tfhip_conv2d_info ci;
+  int ch_mul;
+  int bias_kind, act;
+  int quant;
+  double qscale, qmin;
+  int tiles_w, tiles_h, c4;  // fast path: patch grid and channel quads
+};
+
+// 3x3, dilation 1, channel multiplier 1, C % 4 == 0, stride S.  One lane = one channel
+// quad of a TH x TW output patch.  Lane order: channel quad fastest, then patch column,
+// patch row, image — neighbours in a wavefront touch neighbouring addresses.
+template <int S, int TH, int TW>
+__global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p) {
+  constexpr int IH = (TH - 1) * S + 3, IW = (TW - 1) * S + 3;
+  const tfhip_conv2d_info& ci = p.ci;
+  const int64_t total = (int64_t)ci.batch * p.tiles_h * p.tiles_w * p.c4;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= total) return;
+  const int cq = (int)(gid % p.c4);
+  int64_t t = gid / p.c4;
+  const int tw = (int)(t % p.tiles_w);
+  t /= p.tiles_w;
+  const int th = (int)(t % p.tiles_h);
+  const int n = (int)(t / p.tiles_h);
+  const int c = cq * 4;
+  const int C = ci.in_c;
+
+  f32x4 w[9];
+  if (p.quant) {
+    const unsigned char* wq = static_cast<const unsigned char*>(p.w);
+#pragma unroll
+    for (int i = 0; i < 9; i++) {
+      const unsigned v = *reinterpret_cast<const unsigned*>(wq + (int64_t)i * C + c);
+#pragma unroll
+      for (int e = 0; e < 4; e++) w[i][e] = dq((v >> (8 * e)) & 0xffu, p.qscale, p.qmin);
+    }
+  } else {
+    const float* wf = static_cast<const float*>(p.w);
+#pragma unroll
+    for (int i = 0; i < 9; i++) w[i] = *reinterpret_cast<const f32x4*>(wf + (int64_t)i * C + c);
+  }
+
+  const int oh0 = th * TH, ow0 = tw * TW;
+  const int ih0 = oh0 * S - ci.pad_top, iw0 = ow0 * S - ci.pad_left;
+  const float* xn = p.x + (int64_t)n * ci.in_h * ci.in_w * C + c;
+
+  f32x4 acc[TH][TW];
+#pragma unroll
+  for (int i = 0; i < TH; i++)
+#pragma unroll
+    for (int j = 0; j < TW; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // Accumulation order per output is filter row, then filter column (as the reference's
+  // loops, backend_cpu.ts:1996-2030), because input rows are visited in ascending order.
+#pragma unroll
+  for (int r = 0; r < IH; r++) {
+    const int ih = ih0 + r;
+    const bool row_ok = (unsigned)ih < (unsigned)ci.in_h;
+    f32x4 in[IW];
+#pragma unroll
+    for (int q = 0; q < IW; q++) {
+      const int iw = iw0 + q;
+      in[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (row_ok && (unsigned)iw < (unsigned)ci.in_w)
+        in[q] = *reinterpret_cast<const f32x4*>(xn + ((int64_t)ih * ci.in_w + iw) * C);
+    }
+#pragma unroll
+    for (int i = 0; i < TH; i++) {
+      const int kh = r - i * S;
+      if (kh < 0 || kh > 2) continue;
+#pragma unroll
+      for (int j = 0; j < TW; j++)
+#pragma unroll
+        for (int kw = 0; kw < 3; kw++) acc[i][j] += in[j * S + kw] * w[kh * 3 + kw];
+    }
+  }
+
+  f32x4 b = {0.f, 0.f, 0.f, 0.f};
+  if (p.bias_kind == TFHIP_BCAST_COLUMN) b = *reinterpret_cast<const f32x4*>(p.bias + c);
+  else if (p.bias_kind == TFHIP_BCAST_SCALAR) b = f32x4{p.bias[0], p.bias[0], p.bias[0], p.bias[0]};
+#pragma unroll
+  for (int i = 0; i < TH; i++) {
+    const int oh = oh0 + i;
+    if (oh >= ci.out_h) continue;
+#pragma unroll
+    for (int j = 0; j < TW; j++) {
+      const int ow = ow0 + j;
+      if (ow >= ci.out_w) continue;
+      f32x4 v = acc[i][j] + b;
+#pragma unroll
+      for (int e = 0; e < 4; e++) v[e] = act_f(v[e], p.act);
+      *reinterpret_cast<f32x4*>(p.y + (((int64_t)n * ci.out_h + oh) * ci.out_w + ow) * C + c) = v;
+    }
+  }
+}
+
+// Any filter size, stride, dilation and channel multiplier: one lane per output element,
+// output channel fastest.
+__global__ void depthwise_generic_kernel(const DwArgs p) {
+  const tfhip_conv2d_info& ci = p.ci;
+  const int64_t total = (int64_t)ci.batch * ci.out_h * ci.out_w * ci.out_c;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; gid < total; gid += stride) {
+    const int oc = (int)(gid % ci.out_c);
+    int64_t t = gid / ci.out_c;
+    const int ow = (int)(t % ci.out_w);
+    t /= ci.out_w;
+    const int oh = (int)(t % ci.out_h);
+    const int n = (int)(t / ci.out_h);
+    const int c = oc / p.ch_mul, q = oc - c * p.ch_mul;
+    float acc = 0.f;
+    for (int kh = 0; kh < ci.filter_h; kh++) {
+      const int ih = oh * ci.stride_h - ci.pad_top + kh * ci.dilation_h;
+      if ((unsigned)ih >= (unsigned)ci.in_h) continue;
+      for (int kw = 0; kw < ci.filter_w; kw++) {
+        const int iw = ow * ci.stride_w - ci.pad_left + kw * ci.dilation_w;
+        if ((unsigned)iw >= (unsigned)ci.in_w) continue;
+        const int64_t wi = (((int64_t)kh * ci.filter_w + kw) * ci.in_c + c) * p.ch_mul + q;
+        const float wv = p.quant ? dq(static_cast<const unsigned char*>(p.w)[wi], p.qscale, p.qmin)
+                                 : static_cast<const float*>(p.w)[wi];
+        acc += p.x[(((int64_t)n * ci.in_h + ih) * ci.in_w + iw) * ci.in_c + c] * wv;
+      }
+    }
+    if (p.bias_kind == TFHIP_BCAST_COLUMN) acc += p.bias[oc];
+    else if (p.bias_kind == TFHIP_BCAST_SCALAR) acc += p.bias[0];
+    p.y[gid] = act_f(acc, p.act);
+  }
+}
+
+// avg: mean over the in-bounds part of the window (count = visited pixels,
+// backend_cpu.ts:2312-2336); max: NaN never wins (`pixel > max`).  Channel fastest.
+__global__ void pool2d_kernel(const float* x, float* y, const tfhip_conv2d_info ci, int kind) {
+  const int eff_h = ci.filter_h + (ci.filter_h - 1) * (ci.dilation_h - 1);
+  const int eff_w = ci.filter_w + (ci.filter_w - 1) * (ci.dilation_w - 1);
+  const int64_t total = (int64_t)ci.batch * ci.out_h * ci.out_w * ci.out_c;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; gid < total; gid += stride) {
+    const int c = (int)(gid % ci.out_c);
+    int64_t t = gid / ci.out_c;
+    const int ow = (int)(t % ci.out_w);
+    t /= ci.out_w;
+    const int oh = (int)(t % ci.out_h);
+    const int n = (int)(t / ci.out_h);
+    const int r0 = oh * ci.stride_h - ci.pad_top, c0 = ow * ci.stride_w - ci.pad_left;
+    const int r_min = r0 > 0 ? r0 : 0, c_min = c0 > 0 ? c0 : 0;
+    const int r_max = ci.in_h < eff_h + r0 ? ci.in_h : eff_h + r0;
+    const int c_max = ci.in_w < eff_w + c0 ? ci.in_w : eff_w + c0;
+    double sum = 0.0;
+    float mx = -INFINITY;
+    int count = 0;
+    for (int r = r_min; r < r_max; r += ci.dilation_h)
+      for (int q = c_min; q < c_max; q += ci.dilation_w) {
+        const float v = x[(((int64_t)n * ci.in_h + r) * ci.in_w + q) * ci.in_c + c];
+        if (kind == TFHIP_POOL_MAX) {
+          if (v > mx) mx = v;
+        } else {
+          sum += (double)v;
+          count++;
+        }
+      }
+    y[gid] = kind == TFHIP_POOL_AVG ? (float)(sum / (double)count) : mx;
+  }
+}
+
+// Global average pool (window = whole image, 'valid'): x [N, HW, C] -> y [N, C].  One lane
+// per (image, channel quad); consecutive lanes read consecutive channel quads.
+__global__ void global_avgpool_kernel(const float* x, float* y, int n_img, int hw, int c4) {
+  const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= n_img * c4) return;
+  const int n = gid / c4, cq = gid - n * c4;
+  const f32x4* src = reinterpret_cast<const f32x4*>(x) + (int64_t)n * hw * c4 + cq;
+  double s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+  for (int i = 0; i < hw; i++) {
+    const f32x4 v = src[(int64_t)i * c4];
+    s0 += v[0]; s1 += v[1]; s2 += v[2]; s3 += v[3];
+  }
+  const double d = (double)hw;
+  reinterpret_cast<f32x4*>(y)[gid] = f32x4{(float)(s0 / d), (float)(s1 / d), (float)(s2 / d), (float)(s3 / d)};
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <int S, int TH, int TW>
+static void launch_dw3x3(tfhip_ctx* ctx, DwArgs& p) {
+  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise3x3_s%d_%dx%d", S, TH, TW);
+  p.tiles_h = (int)ceil_div(p.ci.out_h, TH);
+  p.tiles_w = (int)ceil_div(p.ci.out_w, TW);
+  const int64_t total = (int64_t)p.ci.batch * p.tiles_h * p.tiles_w * p.c4;
+  hipLaunchKernelGGL((depthwise3x3_kernel<S, TH, TW>), dim3((unsigned)ceil_div(total, 256)),
+                     dim3(256), 0, ctx->stream, p);
+}
+
+static int check_geometry(tfhip_ctx* ctx, const char* op, const tfhip_conv2d_info* ci) {
+  if (ci->batch < 0 || ci->in_h < 0 || ci->in_w < 0 || ci->in_c < 0 || ci->out_h < 0 ||
+      ci->out_w < 0 || ci->out_c < 0 || ci->filter_h <= 0 || ci->filter_w <= 0 ||
+      ci->stride_h <= 0 || ci->stride_w <= 0 || ci->dilation_h <= 0 || ci->dilation_w <= 0)
+    return ctx->fail(TFHIP_EINVAL, "%s: bad geometry", op);
+  return TFHIP_OK;
+}
+
+}  // namespace tfhip
+
+using namespace tfhip;
+
+extern "C" int tfhip_depthwise_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t out,
+                                      const tfhip_conv2d_info* ci, int64_t bias, int bias_kind,
+                                      int act, const tfhip_qparams* q) {
+  if (!ctx || !ci) return TFHIP_EINVAL;
+  int rc;
+  if ((rc = check_geometry(ctx, "depthwiseConv2D", ci))) return rc;
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bw, filter);
+  TFHIP_GET(ctx, bo, out);
+  if (ci->in_c <= 0 || ci->out_c % ci->in_c != 0)
+    return ctx->fail(TFHIP_EINVAL, "depthwiseConv2D: out channels must be a multiple of in channels");
+  const int ch_mul = ci->out_c / ci->in_c;
+  const int64_t x_n = (int64_t)ci->batch * ci->in_h * ci->in_w * ci->in_c;
+  const int64_t w_n = (int64_t)ci->filter_h * ci->filter_w * ci->out_c;
+  const int64_t o_n = (int64_t)ci->batch * ci->out_h * ci->out_w * ci->out_c;
+  if (bx->numel != x_n || bw->numel != w_n || bo->numel != o_n)
+    return ctx->fail(TFHIP_EINVAL, "depthwiseConv2D: buffer sizes do not match the geometry");
+  if (bo->dtype != TFHIP_FLOAT32)
+    return ctx->fail(TFHIP_EINVAL, "depthwiseConv2D: output buffer must be float32");
+  if (act != TFHIP_ACT_LINEAR && act != TFHIP_ACT_RELU && act != TFHIP_ACT_RELU6)
+    return ctx->fail(TFHIP_EINVAL, "depthwiseConv2D: activation %d is not folded here", act);
+  if (bias_kind != TFHIP_BCAST_NONE && bias_kind != TFHIP_BCAST_SCALAR &&
+      bias_kind != TFHIP_BCAST_COLUMN)
+    return ctx->fail(TFHIP_EINVAL, "depthwiseConv2D: bias layout %d is not folded here", bias_kind);
+  const bool quant = bw->dtype == TFHIP_UINT8Q;
+  if (quant != (q != nullptr))
+    return ctx->fail(TFHIP_EINVAL, "depthwiseConv2D: qparams must be given exactly for a quantised filter");
+  if (o_n == 0) return TFHIP_OK;
+
+  Temp tx(ctx), tw(ctx), tb(ctx);
+  DwArgs p = {};
+  if ((rc = as_f32(ctx, bx, &tx, &p.x))) return rc;
+  if (quant) {
+    p.w = bw->ptr;
+    p.quant = 1;
+    p.qscale = q->scale;
+    p.qmin = q->min;
+  } else {
+    const float* wf;
+    if ((rc = as_f32(ctx, bw, &tw, &wf))) return rc;
+    p.w = wf;
+  }
+  if (bias_kind != TFHIP_BCAST_NONE) {
+    TFHIP_GET(ctx, bb, bias);
+    if (bb->numel != (bias_kind == TFHIP_BCAST_SCALAR ? 1 : ci->out_c))
+      return ctx->fail(TFHIP_EINVAL, "depthwiseConv2D: bias size does not match its layout");
+    if ((rc = as_f32(ctx, bb, &tb, &p.bias))) return rc;
+  }
+  p.y = static_cast<float*>(bo->ptr);
+  p.ci = *ci;
+  p.ch_mul = ch_mul;
+  p.bias_kind = bias_kind;
+  p.act = act;
+
+  const bool fast = ci->filter_h == 3 && ci->filter_w == 3 && ci->dilation_h == 1 &&
+                    ci->dilation_w == 1 && ch_mul == 1 && ci->in_c % 4 == 0 &&
+                    ci->stride_h == ci->stride_w && (ci->stride_h == 1 || ci->stride_h == 2) &&
+                    aligned16(p.x) && aligned16(p.w) && aligned16(p.y) &&
+                    (bias_kind != TFHIP_BCAST_COLUMN || aligned16(p.bias));
+  if (fast) {
+    p.c4 = ci->in_c / 4;
+    if (ci->stride_h == 1) launch_dw3x3<1, 2, 4>(ctx, p);
+    else launch_dw3x3<2, 1, 4>(ctx, p);
+  } else {
+    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise_generic");
+    const int64_t blocks = ceil_div(o_n, 256);
+    const int64_t cap = (int64_t)ctx->num_cus * 16;
+    hipLaunchKernelGGL(depthwise_generic_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)),
+                       dim3(256), 0, ctx->stream, p);
+  }
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+extern "C" int tfhip_pool2d(tfhip_ctx* ctx, int64_t x, int64_t out, const tfhip_conv2d_info* ci,
+                            int kind) {
+  if (!ctx || !ci) return TFHIP_EINVAL;
+  int rc;
+  if ((rc = check_geometry(ctx, "pool", ci))) return rc;
+  if (kind != TFHIP_POOL_AVG && kind != TFHIP_POOL_MAX)
+    return ctx->fail(TFHIP_EINVAL, "pool: unknown kind %d", kind);
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bo, out);
+  if (ci->in_c != ci->out_c) return ctx->fail(TFHIP_EINVAL, "pool: channel counts differ");
+  const int64_t x_n = (int64_t)ci->batch * ci->in_h * ci->in_w * ci->in_c;
+  const int64_t o_n = (int64_t)ci->batch * ci->out_h * ci->out_w * ci->out_c;
+  if (bx->numel != x_n || bo->numel != o_n)
+    return ctx->fail(TFHIP_EINVAL, "pool: buffer sizes do not match the geometry");
+  if (bo->dtype != TFHIP_FLOAT32) return ctx->fail(TFHIP_EINVAL, "pool: output must be float32");
+  if (o_n == 0) return TFHIP_OK;
+  Temp tx(ctx);
+  const float* xf;
+  if ((rc = as_f32(ctx, bx, &tx, &xf))) return rc;
+  float* y = static_cast<float*>(bo->ptr);
+  const bool global = kind == TFHIP_POOL_AVG && ci->out_h == 1 && ci->out_w == 1 &&
+                      ci->filter_h == ci->in_h && ci->filter_w == ci->in_w && ci->pad_top == 0 &&
+                      ci->pad_left == 0 && ci->dilation_h == 1 && ci->dilation_w == 1 &&
+                      ci->in_c % 4 == 0 && aligned16(xf) && aligned16(y);
+  if (global) {
+    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "global_avgpool");
+    const int items = ci->batch * (ci->in_c / 4);
+    hipLaunchKernelGGL(global_avgpool_kernel, dim3((unsigned)ceil_div(items, 64)), dim3(64), 0,
+                       ctx->stream, xf, y, ci->batch, ci->in_h * ci->in_w, ci->in_c / 4);
+  } else {
+    const int64_t blocks = ceil_div(o_n, 256);
+    const int64_t cap = (int64_t)ctx->num_cus * 16;
+    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "pool2d");
+    hipLaunchKernelGGL(pool2d_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0,
+                       ctx->stream, xf, y, *ci, kind);
+  }
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}

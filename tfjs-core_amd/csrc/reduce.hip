@@ -1,0 +1,255 @@
+// Row reductions (sum / max / min / argMax / argMin), one-pass row softmax, gather and
+// transpose.  Replaces backend_cpu.ts:590-611, 658-712, 861-929, 2178-2223 and the softmax
+// composite of ops/softmax.ts:45-79 + ops/reduction_ops.ts:56-74 of the reference.
+//
+// A row is reduced by one wavefront: lanes stride over the row (coalesced), then combine
+// with cross-lane shuffles.  The result is independent of the launch shape, so argMax /
+// argMin are deterministic and bit-exact against a sequential scan.
+#include "tfhip_internal.h"
+
+namespace tfhip {
+
+__device__ __forceinline__ float ld(const void* p, int dt, int64_t i) {
+  switch (dt) {
+    case TFHIP_FLOAT32: return static_cast<const float*>(p)[i];
+    case TFHIP_INT32: return (float)static_cast<const int32_t*>(p)[i];
+    default: return (float)static_cast<const uint8_t*>(p)[i];
+  }
+}
+
+constexpr int WAVE = 64;
+constexpr int ROWS_PER_BLOCK = 4;  // 4 wavefronts per workgroup, one row each
+
+// max / min follow backend_cpu: the accumulator starts at element 0 and only a strictly
+// greater (smaller) value replaces it, so NaN survives only from slot 0.  arg* return the
+// first index of the strict extremum; ties and NaN keep the earlier index.
+template <typename OutT>
+__global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void reduce_rows_kernel(
+    int op, const void* x, int x_dt, OutT* out, int64_t outer, int64_t inner) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+  if (row >= outer) return;
+  const int64_t base = row * inner;
+  if (op == TFHIP_SUM) {
+    double s = 0.0;
+    for (int64_t j = lane; j < inner; j += WAVE) s += (double)ld(x, x_dt, base + j);
+    for (int off = WAVE / 2; off > 0; off >>= 1) s += __shfl_down(s, off, WAVE);
+    if (lane == 0) {
+      if (std::is_same<OutT, float>::value) out[row] = (OutT)(float)s;
+      else out[row] = (OutT)(int32_t)(uint32_t)(int64_t)s;
+    }
+    return;
+  }
+  const bool want_max = op == TFHIP_MAX || op == TFHIP_ARGMAX;
+  const float first = ld(x, x_dt, base);
+  float best = first;
+  int64_t idx = 0;
+  for (int64_t j = lane; j < inner; j += WAVE) {
+    const float v = ld(x, x_dt, base + j);
+    if (want_max ? v > best : v < best) {
+      best = v;
+      idx = j;
+    }
+  }
+  for (int off = WAVE / 2; off > 0; off >>= 1) {
+    const float ob = __shfl_down(best, off, WAVE);
+    const int64_t oi = __shfl_down(idx, off, WAVE);
+    const bool better = want_max ? ob > best : ob < best;
+    if (better || (ob == best && oi < idx)) {
+      best = ob;
+      idx = oi;
+    }
+  }
+  if (lane == 0) {
+    if (op == TFHIP_ARGMAX || op == TFHIP_ARGMIN) out[row] = (OutT)idx;
+    else if (std::is_same<OutT, float>::value) out[row] = (OutT)best;
+    else out[row] = (OutT)(int32_t)best;
+  }
+}
+
+// softmax over the last axis with the rounding points of the reference composite:
+// m = max(x); e = exp(x - m); s = sum(e); lse = m + log(s); y = exp(x - lse).
+__global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void softmax_rows_kernel(
+    const float* x, float* y, int64_t rows, int64_t cols) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float* xr = x + row * cols;
+  float* yr = y + row * cols;
+  float m = xr[0];
+  for (int64_t j = lane; j < cols; j += WAVE) {
+    const float v = xr[j];
+    if (v > m) m = v;
+  }
+  for (int off = WAVE / 2; off > 0; off >>= 1) {
+    const float o = __shfl_xor(m, off, WAVE);
+    if (o > m) m = o;
+  }
+  // a NaN in slot 0 makes every lane's m NaN already (all start from xr[0])
+  double s = 0.0;
+  for (int64_t j = lane; j < cols; j += WAVE) s += (double)expf(xr[j] - m);
+  for (int off = WAVE / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
+  const float lse = m + logf((float)s);
+  for (int64_t j = lane; j < cols; j += WAVE) yr[j] = expf(xr[j] - lse);
+}
+
+// out[o, i, :] = x[o, indices[i], :] for 4-byte or 1-byte elements.
+template <typename T>
+__global__ void gather_kernel(const T* x, const int32_t* indices, T* out, int64_t outer,
+                              int64_t axis_dim, int64_t inner, int64_t n_idx) {
+  const int64_t total = outer * n_idx * inner;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += stride) {
+    const int64_t in = g % inner;
+    const int64_t t = g / inner;
+    const int64_t i = t % n_idx, o = t / n_idx;
+    const int64_t src = indices[i];
+    // an index outside the axis reads nothing (the reference would yield undefined)
+    out[g] = (src >= 0 && src < axis_dim) ? x[(o * axis_dim + src) * inner + in] : T(0);
+  }
+}
+
+constexpr int MAXR = 6;
+struct PermArgs {
+  int rank;
+  int out_dim[MAXR];
+  int64_t in_stride[MAXR];  // stride in x of the dimension that lands on out dim d
+};
+
+template <typename T>
+__global__ void transpose_kernel(const T* x, T* out, int64_t n, PermArgs pa) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < n; g += stride) {
+    int64_t rem = g, src = 0;
+#pragma unroll
+    for (int d = MAXR - 1; d >= 0; d--) {
+      if (d < pa.rank) {
+        src += (rem % pa.out_dim[d]) * pa.in_stride[d];
+        rem /= pa.out_dim[d];
+      }
+    }
+    out[g] = x[src];
+  }
+}
+
+static unsigned grid_cap(tfhip_ctx* ctx, int64_t items, int block) {
+  const int64_t want = ceil_div(items, block), cap = (int64_t)ctx->num_cus * 16;
+  return (unsigned)(want < 1 ? 1 : (want > cap ? cap : want));
+}
+
+}  // namespace tfhip
+
+using namespace tfhip;
+
+extern "C" int tfhip_reduce(tfhip_ctx* ctx, int op, int64_t x, int64_t out, int64_t outer,
+                            int64_t inner) {
+  if (!ctx) return TFHIP_EINVAL;
+  if (op < TFHIP_SUM || op > TFHIP_ARGMIN) return ctx->fail(TFHIP_EINVAL, "reduce: unknown op %d", op);
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bo, out);
+  if (outer < 0 || inner < 0 || bx->numel != outer * inner || bo->numel != outer)
+    return ctx->fail(TFHIP_EINVAL, "reduce: buffers hold %lld and %lld elements, need %lld and %lld",
+                     (long long)bx->numel, (long long)bo->numel, (long long)(outer * inner),
+                     (long long)outer);
+  if (bx->dtype == TFHIP_UINT8Q) return ctx->fail(TFHIP_EINVAL, "reduce: quantised input");
+  const bool arg = op == TFHIP_ARGMAX || op == TFHIP_ARGMIN;
+  if (arg && bo->dtype != TFHIP_INT32)
+    return ctx->fail(TFHIP_EINVAL, "reduce: argMax/argMin write int32");
+  if (bo->dtype != TFHIP_INT32 && bo->dtype != TFHIP_FLOAT32)
+    return ctx->fail(TFHIP_EINVAL, "reduce: output must be float32 or int32");
+  if (outer == 0) return TFHIP_OK;
+  if (inner == 0) {
+    if (op != TFHIP_SUM) return ctx->fail(TFHIP_EINVAL, "reduce: empty axis has no extremum");
+    return tfhip_fill(ctx, out, 0.0);
+  }
+  if (ceil_div(outer, ROWS_PER_BLOCK) > 0x7fffffffLL) return ctx->fail(TFHIP_ENOTSUP, "reduce: too many rows");
+  const dim3 grid((unsigned)ceil_div(outer, ROWS_PER_BLOCK)), block(WAVE * ROWS_PER_BLOCK);
+  if (bo->dtype == TFHIP_FLOAT32)
+    hipLaunchKernelGGL(reduce_rows_kernel<float>, grid, block, 0, ctx->stream, op, bx->ptr,
+                       bx->dtype, (float*)bo->ptr, outer, inner);
+  else
+    hipLaunchKernelGGL(reduce_rows_kernel<int32_t>, grid, block, 0, ctx->stream, op, bx->ptr,
+                       bx->dtype, (int32_t*)bo->ptr, outer, inner);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+extern "C" int tfhip_softmax_rows(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t rows,
+                                  int64_t cols) {
+  if (!ctx) return TFHIP_EINVAL;
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bo, out);
+  if (rows < 0 || cols < 0 || bx->numel != rows * cols || bo->numel != rows * cols)
+    return ctx->fail(TFHIP_EINVAL, "softmax: buffer sizes do not match rows x cols");
+  if (bo->dtype != TFHIP_FLOAT32) return ctx->fail(TFHIP_EINVAL, "softmax: output must be float32");
+  if (rows * cols == 0) return TFHIP_OK;
+  Temp tx(ctx);
+  const float* xf;
+  int rc;
+  if ((rc = as_f32(ctx, bx, &tx, &xf))) return rc;
+  hipLaunchKernelGGL(softmax_rows_kernel, dim3((unsigned)ceil_div(rows, ROWS_PER_BLOCK)),
+                     dim3(WAVE * ROWS_PER_BLOCK), 0, ctx->stream, xf, (float*)bo->ptr, rows, cols);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+extern "C" int tfhip_gather(tfhip_ctx* ctx, int64_t x, int64_t indices, int64_t out,
+                            int64_t outer, int64_t axis_dim, int64_t inner, int64_t n_indices) {
+  if (!ctx) return TFHIP_EINVAL;
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bi, indices);
+  TFHIP_GET(ctx, bo, out);
+  if (outer < 0 || axis_dim < 0 || inner < 0 || n_indices < 0 ||
+      bx->numel != outer * axis_dim * inner || bi->numel != n_indices ||
+      bo->numel != outer * n_indices * inner)
+    return ctx->fail(TFHIP_EINVAL, "gather: buffer sizes do not match the shapes given");
+  if (bi->dtype != TFHIP_INT32) return ctx->fail(TFHIP_EINVAL, "gather: indices must be int32");
+  if (dtype_size(bx->dtype) != dtype_size(bo->dtype))
+    return ctx->fail(TFHIP_EINVAL, "gather: input and output element sizes differ");
+  const int64_t total = bo->numel;
+  if (total == 0) return TFHIP_OK;
+  const dim3 grid(grid_cap(ctx, total, 256)), block(256);
+  if (dtype_size(bx->dtype) == 4)
+    hipLaunchKernelGGL(gather_kernel<int32_t>, grid, block, 0, ctx->stream, (const int32_t*)bx->ptr,
+                       (const int32_t*)bi->ptr, (int32_t*)bo->ptr, outer, axis_dim, inner, n_indices);
+  else
+    hipLaunchKernelGGL(gather_kernel<uint8_t>, grid, block, 0, ctx->stream, (const uint8_t*)bx->ptr,
+                       (const int32_t*)bi->ptr, (uint8_t*)bo->ptr, outer, axis_dim, inner, n_indices);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+extern "C" int tfhip_transpose(tfhip_ctx* ctx, int64_t x, const int32_t* x_shape, int rank,
+                               const int32_t* perm, int64_t out) {
+  if (!ctx) return TFHIP_EINVAL;
+  if (rank < 0 || rank > MAXR) return ctx->fail(TFHIP_ENOTSUP, "transpose: rank above %d", MAXR);
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bo, out);
+  int64_t n = 1, strides[MAXR];
+  bool seen[MAXR] = {false};
+  for (int i = rank - 1; i >= 0; i--) {
+    strides[i] = n;
+    n *= x_shape[i];
+  }
+  PermArgs pa = {};
+  pa.rank = rank;
+  for (int d = 0; d < rank; d++) {
+    const int s = perm[d];
+    if (s < 0 || s >= rank || seen[s]) return ctx->fail(TFHIP_EINVAL, "transpose: bad permutation");
+    seen[s] = true;
+    pa.out_dim[d] = x_shape[s];  // newShape[i] = x.shape[perm[i]] (backend_cpu.ts:2181-2184)
+    pa.in_stride[d] = strides[s];
+  }
+  if (bx->numel != n || bo->numel != n || dtype_size(bx->dtype) != dtype_size(bo->dtype))
+    return ctx->fail(TFHIP_EINVAL, "transpose: buffer sizes do not match the shape given");
+  if (n == 0) return TFHIP_OK;
+  const dim3 grid(grid_cap(ctx, n, 256)), block(256);
+  if (dtype_size(bx->dtype) == 4)
+    hipLaunchKernelGGL(transpose_kernel<int32_t>, grid, block, 0, ctx->stream,
+                       (const int32_t*)bx->ptr, (int32_t*)bo->ptr, n, pa);
+  else
+    hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, block, 0, ctx->stream,
+                       (const uint8_t*)bx->ptr, (uint8_t*)bo->ptr, n, pa);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}

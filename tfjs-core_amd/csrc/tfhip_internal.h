@@ -1,0 +1,97 @@
+// Internal declarations shared by the translation units of libtfjs_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <map>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "tfjs_hip.h"
+
+namespace tfhip {
+
+struct Buf {
+  void* ptr = nullptr;
+  size_t nbytes = 0;  // logical bytes (numel * element size)
+  size_t cap = 0;     // bytes of the pool block behind ptr
+  int dtype = TFHIP_FLOAT32;
+  int64_t numel = 0;
+  int rank = 0;
+  int32_t shape[8] = {0};
+};
+
+inline size_t dtype_size(int dtype) {
+  return (dtype == TFHIP_BOOL || dtype == TFHIP_UINT8Q) ? 1 : 4;
+}
+
+}  // namespace tfhip
+
+// One device, one in-order stream, one size-bucketed pool of device blocks.  Freed blocks
+// go back to the pool at once: every consumer is queued on the same stream, so a block
+// handed out again can only be touched after the work that last used it.
+struct tfhip_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev_begin = nullptr, ev_end = nullptr;
+  bool timing = false;
+  std::unordered_map<int64_t, tfhip::Buf> bufs;
+  std::multimap<size_t, void*> pool;  // capacity -> free block
+  size_t in_use = 0, pooled = 0;
+  std::string err;
+  char last_kernel[96] = "";  // variant chosen by the last dense / image launch
+  int num_cus = 256;
+
+  int fail(int code, const char* fmt, ...);
+  tfhip::Buf* find(int64_t id);          // sets err when missing
+  void* alloc(size_t nbytes, size_t* cap);  // nullptr + err on failure (nbytes > 0)
+  void release(void* p, size_t cap);
+  void trim();
+};
+
+#define TFHIP_HIP(ctx, expr)                                                          \
+  do {                                                                                \
+    hipError_t e_ = (expr);                                                           \
+    if (e_ != hipSuccess)                                                             \
+      return (ctx)->fail(TFHIP_EDEVICE, "%s: %s", #expr, hipGetErrorString(e_));      \
+  } while (0)
+
+#define TFHIP_GET(ctx, var, id)           \
+  tfhip::Buf* var = (ctx)->find(id);      \
+  if (!var) return TFHIP_ENOENT
+
+#define TFHIP_LAUNCH_CHECK(ctx) TFHIP_HIP(ctx, hipGetLastError())
+
+namespace tfhip {
+
+// Scoped device scratch taken from the pool (returned when the object dies; safe because
+// later users are ordered behind the kernels already queued on the stream).
+struct Temp {
+  tfhip_ctx* ctx;
+  void* ptr = nullptr;
+  size_t cap = 0;
+  explicit Temp(tfhip_ctx* c) : ctx(c) {}
+  bool get(size_t nbytes) {
+    ptr = ctx->alloc(nbytes, &cap);
+    return ptr != nullptr;
+  }
+  ~Temp() {
+    if (ptr) ctx->release(ptr, cap);
+  }
+};
+
+// Returns a float32 view of `b`: the buffer itself when it is stored as float32, else a
+// converted copy in `tmp` (int32 / bool storage under a float32 tensor: widening casts
+// alias the same data id, backends/backend_util.ts:49-55).
+int as_f32(tfhip_ctx* ctx, const Buf* b, Temp* tmp, const float** out);
+
+// elementwise.hip
+int launch_convert(tfhip_ctx* ctx, const void* src, int src_dtype, void* dst, int dst_dtype,
+                   int64_t n);
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace tfhip

@@ -1,0 +1,83 @@
+"""ctypes binding of libtfjs_hip.so (include/tfjs_hip.h).  No fallback: if the library is
+missing or no gfx950 device answers, callers get an exception."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "..", "libtfjs_hip.so"))
+
+FLOAT32, INT32, BOOL, UINT8Q = 0, 1, 2, 3
+ACT = {"linear": 0, None: 0, "relu": 1, "prelu": 2, "relu6": 3}
+BCAST_NONE, BCAST_SCALAR, BCAST_COLUMN, BCAST_FULL = 0, 1, 2, 3
+BINARY = dict(add=0, sub=1, mul=2, div=3, prelu=4, maximum=5, minimum=6)
+UNARY = dict(relu=0, clip=1, exp=2, log=3, neg=4, abs=5, sigmoid=6, sqrt=7, square=8, tanh=9,
+             rsqrt=10)
+REDUCE = dict(sum=0, max=1, min=2, argmax=3, argmin=4)
+POOL = dict(avg=0, max=1)
+
+
+class Conv2DInfoC(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "batch", "in_h", "in_w", "in_c", "out_h", "out_w", "out_c", "stride_h", "stride_w",
+        "dilation_h", "dilation_w", "filter_h", "filter_w", "pad_top", "pad_left",
+        "pad_bottom", "pad_right")]
+
+
+class QParams(C.Structure):
+    _fields_ = [("scale", C.c_double), ("min", C.c_double)]
+
+
+_lib = None
+
+_I64, _INT, _PTR = C.c_int64, C.c_int, C.c_void_p
+_SIGNATURES = {
+    "tfhip_init": [_INT, C.POINTER(_PTR)],
+    "tfhip_destroy": [_PTR],
+    "tfhip_last_error": [_PTR],
+    "tfhip_register": [_PTR, _I64, C.POINTER(C.c_int32), _INT, _INT],
+    "tfhip_write": [_PTR, _I64, _PTR, C.c_size_t],
+    "tfhip_read": [_PTR, _I64, _PTR, C.c_size_t],
+    "tfhip_dispose": [_PTR, _I64],
+    "tfhip_mem_info": [_PTR, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
+    "tfhip_sync": [_PTR],
+    "tfhip_time_begin": [_PTR],
+    "tfhip_time_end": [_PTR, C.POINTER(C.c_float)],
+    "tfhip_last_kernel": [_PTR],
+    "tfhip_device_ptr": [_PTR, _I64, C.POINTER(_PTR), C.POINTER(C.c_size_t)],
+    "tfhip_matmul": [_PTR, _I64, _I64, _I64, _INT, _INT, _INT, _INT, _INT, _INT, _I64, _INT, _INT,
+                     _I64, _INT, C.POINTER(QParams)],
+    "tfhip_conv2d": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC), _I64, _INT, _INT, _I64, _INT,
+                     C.POINTER(QParams)],
+    "tfhip_depthwise_conv2d": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC), _I64, _INT, _INT,
+                               C.POINTER(QParams)],
+    "tfhip_pool2d": [_PTR, _I64, _I64, C.POINTER(Conv2DInfoC), _INT],
+    "tfhip_binary": [_PTR, _INT, _I64, C.POINTER(C.c_int32), _INT, _I64, C.POINTER(C.c_int32),
+                     _INT, _I64],
+    "tfhip_unary": [_PTR, _INT, _I64, _I64, C.c_float, C.c_float],
+    "tfhip_cast": [_PTR, _I64, _I64],
+    "tfhip_dequantize": [_PTR, _I64, _I64, C.POINTER(QParams)],
+    "tfhip_fill": [_PTR, _I64, C.c_double],
+    "tfhip_reduce": [_PTR, _INT, _I64, _I64, _I64, _I64],
+    "tfhip_softmax_rows": [_PTR, _I64, _I64, _I64, _I64],
+    "tfhip_gather": [_PTR, _I64, _I64, _I64, _I64, _I64, _I64, _I64],
+    "tfhip_transpose": [_PTR, _I64, C.POINTER(C.c_int32), _INT, C.POINTER(C.c_int32), _I64],
+    "tfhip_copy": [_PTR, _I64, _I64],
+}
+
+
+def lib():
+    """Load libtfjs_hip.so (built by tfjs-core_amd/build.py); raises if it is not there."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libtfjs_hip.so is not built (%s): run `python "
+                               "tfjs-core_amd/build.py`; the hip backend has no CPU fallback"
+                               % LIB_PATH)
+        l = C.CDLL(LIB_PATH)
+        for name, args in _SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.argtypes = args
+            fn.restype = None if name == "tfhip_destroy" else (
+                C.c_char_p if name in ("tfhip_last_error", "tfhip_last_kernel") else C.c_int)
+        _lib = l
+    return _lib

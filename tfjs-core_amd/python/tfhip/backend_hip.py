@@ -1,0 +1,420 @@
+"""MathBackendHIP: the KernelBackend of tfjs-core (tfjs-core/src/backends/backend.ts:91-649)
+on libtfjs_hip.so, Python twin of js/backend_hip.js.  Method names are the reference's in
+snake_case; every kernel returns a device-resident Tensor at once (work is queued on the
+context's stream), only read_sync / time wait for the device."""
+import ctypes as C
+import itertools
+
+import numpy as np
+
+from . import _capi as capi
+from . import shape_util as su
+from .engine import ENGINE, NP_DTYPE, Tensor
+
+_DTYPE_CODE = {"float32": capi.FLOAT32, "int32": capi.INT32, "bool": capi.BOOL,
+               "uint8q": capi.UINT8Q}
+_NP_OF_CODE = {capi.FLOAT32: np.float32, capi.INT32: np.int32, capi.BOOL: np.uint8,
+               capi.UINT8Q: np.uint8}
+
+
+def _shape_arr(shape):
+    return (C.c_int32 * max(1, len(shape)))(*shape)
+
+
+def _info_c(ci):
+    p = ci["padInfo"]
+    if ci.get("dataFormat", "channelsLast") != "channelsLast":
+        raise NotImplementedError("hip backend: only NHWC (channelsLast) is implemented")
+    for k in ("top", "left", "bottom", "right"):
+        if int(p[k]) != p[k]:
+            raise ValueError("hip backend: fractional padding")
+    return capi.Conv2DInfoC(
+        ci["batchSize"], ci["inHeight"], ci["inWidth"], ci["inChannels"], ci["outHeight"],
+        ci["outWidth"], ci["outChannels"], ci["strideHeight"], ci["strideWidth"],
+        ci["dilationHeight"], ci["dilationWidth"], ci["filterHeight"], ci["filterWidth"],
+        int(p["top"]), int(p["left"]), int(p["bottom"]), int(p["right"]))
+
+
+class MathBackendHIP(object):
+    def __init__(self, device=0):
+        self.lib = capi.lib()
+        ctx = C.c_void_p()
+        rc = self.lib.tfhip_init(device, C.byref(ctx))
+        if rc != 0:
+            raise RuntimeError("hip backend: %s" % self.lib.tfhip_last_error(None).decode())
+        self.ctx = ctx
+        self.data = {}      # DataId -> (handle, storage dtype code, numel)
+        self._ids = itertools.count(1)
+
+    # ---- errors ----
+    def _ck(self, rc):
+        if rc != 0:
+            raise RuntimeError(self.lib.tfhip_last_error(self.ctx).decode())
+
+    # ---- TensorStorage (backend.ts:33-44) ----
+    def register(self, data_id, shape, dtype):
+        if data_id in self.data:
+            raise RuntimeError("Data buffer is already registered")
+        code = _DTYPE_CODE[dtype]
+        h = next(self._ids)
+        self._ck(self.lib.tfhip_register(self.ctx, h, _shape_arr(shape), len(shape), code))
+        self.data[data_id] = (h, code, su.size_from_shape(shape))
+
+    def write(self, data_id, values):
+        if values is None:
+            raise ValueError("MathBackendHIP.write(): values can not be null")
+        h, code, numel = self.data[data_id]
+        arr = np.ascontiguousarray(values, dtype=_NP_OF_CODE[code]).ravel()
+        if arr.size != numel:
+            raise ValueError("write: %d values for a buffer of %d" % (arr.size, numel))
+        self._ck(self.lib.tfhip_write(self.ctx, h, arr.ctypes.data_as(C.c_void_p), arr.nbytes))
+
+    def read_sync(self, data_id):
+        h, code, numel = self.data[data_id]
+        out = np.empty(numel, _NP_OF_CODE[code])
+        self._ck(self.lib.tfhip_read(self.ctx, h, out.ctypes.data_as(C.c_void_p), out.nbytes))
+        return out
+
+    def read(self, data_id):
+        return self.read_sync(data_id)
+
+    def dispose_data(self, data_id):
+        rec = self.data.pop(data_id, None)
+        if rec is not None:
+            self._ck(self.lib.tfhip_dispose(self.ctx, rec[0]))
+
+    def memory(self):
+        a, b, c = C.c_size_t(), C.c_size_t(), C.c_size_t()
+        self._ck(self.lib.tfhip_mem_info(self.ctx, C.byref(a), C.byref(b), C.byref(c)))
+        return dict(unreliable=False, numBytesInGPU=a.value, numBytesInGPUPool=b.value,
+                    numDeviceBuffers=c.value)
+
+    def time(self, f):
+        self._ck(self.lib.tfhip_time_begin(self.ctx))
+        f()
+        ms = C.c_float()
+        self._ck(self.lib.tfhip_time_end(self.ctx, C.byref(ms)))
+        return dict(kernelMs=ms.value)
+
+    def sync(self):
+        self._ck(self.lib.tfhip_sync(self.ctx))
+
+    def float_precision(self):
+        return 32
+
+    def epsilon(self):
+        return 1e-7  # EPSILON_FLOAT32 (backend.ts:23)
+
+    def dispose(self):
+        if self.ctx is not None:
+            self.lib.tfhip_destroy(self.ctx)
+            self.ctx = None
+            self.data.clear()
+
+    # ---- helpers ----
+    def _h(self, t):
+        rec = self.data.get(t.data_id)
+        if rec is None:
+            # data living on another backend: moveData (backend.ts:52-57, engine.ts:361-363)
+            src = ENGINE.ref[t.data_id]
+            values = src[1].read_sync(t.data_id)
+            src[1].dispose_data(t.data_id)
+            self.register(t.data_id, t.shape, t.dtype)
+            self.write(t.data_id, values)
+            src[1] = self
+            rec = self.data[t.data_id]
+        return rec[0]
+
+    def _out(self, shape, dtype="float32"):
+        return Tensor.make(shape, {}, dtype, self)
+
+    def _out_like_storage(self, shape, x):
+        """Output of a pure data-movement kernel: same tensor dtype and same stored element
+        type as x (they differ after a widening cast that aliased the buffer)."""
+        self._h(x)
+        code = self.data[x.data_id][1]
+        name = [k for k, v in _DTYPE_CODE.items() if v == code][0]
+        return Tensor(shape, x.dtype, None, None, self, None, name)
+
+    @staticmethod
+    def _q(t):
+        return C.byref(capi.QParams(t.quant[0], t.quant[1])) if t.quant else None
+
+    def _epilogue_kind(self, operand, out_shape):
+        """Which fused layout (if any) an epilogue operand has against the result."""
+        if operand is None:
+            return capi.BCAST_NONE
+        n = out_shape[-1]
+        if operand.size == 1:
+            return capi.BCAST_SCALAR
+        if operand.size == n and operand.shape[-1] == n:
+            return capi.BCAST_COLUMN
+        if tuple(operand.shape) == tuple(out_shape):
+            return capi.BCAST_FULL
+        return None  # some other broadcast: done as a separate pass
+
+    def _map_activation(self, x, activation, prelu_weights):
+        """mapActivation (backend_cpu.ts:50-62) for the unfused fall-back."""
+        if activation in (None, "linear"):
+            return x
+        if activation == "relu":
+            return self.relu(x)
+        if activation == "prelu":
+            return self.prelu(x, prelu_weights)
+        if activation == "relu6":
+            return self.clip(x, 0, 6)
+        raise ValueError("Activation %s has not been implemented for the HIP backend."
+                         % activation)
+
+    # ---- dense contractions ----
+    def batch_mat_mul(self, a, b, transpose_a, transpose_b):
+        return self.fused_batch_mat_mul(a, b, transpose_a, transpose_b, None, None, None)
+
+    def fused_batch_mat_mul(self, a, b, transpose_a, transpose_b, bias=None, activation=None,
+                            prelu_activation_weights=None):
+        if activation not in capi.ACT:
+            raise ValueError("Activation %s has not been implemented for the HIP backend."
+                             % activation)
+        batch = a.shape[0]
+        k = a.shape[1] if transpose_a else a.shape[2]
+        m = a.shape[2] if transpose_a else a.shape[1]
+        n = b.shape[1] if transpose_b else b.shape[2]
+        out_shape = (batch, m, n)
+        bk = self._epilogue_kind(bias, out_shape)
+        pk = self._epilogue_kind(prelu_activation_weights, out_shape) \
+            if activation == "prelu" else capi.BCAST_NONE
+        out_dtype = "float32"
+        if bk is None or pk is None or a.dtype != "float32":
+            # reference order: matmul, add, activation (backend_cpu.ts:542-555)
+            r = self._matmul(a, b, batch, m, n, k, transpose_a, transpose_b, None, 0, "linear",
+                             None, 0)
+            if a.dtype != "float32":  # int32 x bool -> int32 (backend_cpu.ts:511)
+                r = self.cast(r, a.dtype)
+            if bias is not None:
+                r = self.add(r, bias)
+            return self._map_activation(r, activation, prelu_activation_weights)
+        del out_dtype
+        return self._matmul(a, b, batch, m, n, k, transpose_a, transpose_b, bias, bk, activation,
+                            prelu_activation_weights, pk)
+
+    def _matmul(self, a, b, batch, m, n, k, ta, tb, bias, bk, activation, prelu, pk):
+        out = self._out((batch, m, n))
+        self._ck(self.lib.tfhip_matmul(
+            self.ctx, self._h(a), self._h(b), self._h(out), batch, m, n, k, int(bool(ta)),
+            int(bool(tb)), self._h(bias) if bk else -1, bk, capi.ACT[activation],
+            self._h(prelu) if pk else -1, pk, self._q(b)))
+        return out
+
+    def conv2d(self, x, filter, conv_info):
+        return self.fused_conv2d(x, filter, conv_info, None, None, None)
+
+    def fused_conv2d(self, x, filter, conv_info, bias=None, activation=None,
+                     prelu_activation_weights=None):
+        if activation not in capi.ACT:
+            raise ValueError("Activation %s has not been implemented for the HIP backend."
+                             % activation)
+        out_shape = conv_info["outShape"]
+        bk = self._epilogue_kind(bias, out_shape)
+        pk = self._epilogue_kind(prelu_activation_weights, out_shape) \
+            if activation == "prelu" else capi.BCAST_NONE
+        if bk is None or pk is None:
+            r = self.fused_conv2d(x, filter, conv_info)
+            if bias is not None:
+                r = self.add(r, bias)
+            return self._map_activation(r, activation, prelu_activation_weights)
+        out = self._out(out_shape)
+        info = _info_c(conv_info)
+        self._ck(self.lib.tfhip_conv2d(
+            self.ctx, self._h(x), self._h(filter), self._h(out), C.byref(info),
+            self._h(bias) if bk else -1, bk, capi.ACT[activation],
+            self._h(prelu_activation_weights) if pk else -1, pk, self._q(filter)))
+        return out
+
+    # ---- memory-bound image kernels ----
+    def depthwise_conv2d(self, x, filter, conv_info):
+        return self.fused_depthwise_conv2d(x, filter, conv_info, None, None)
+
+    def fused_depthwise_conv2d(self, x, filter, conv_info, bias=None, activation=None):
+        """Extension of the plug-in API: depthwiseConv2D with the add(bias) + relu / clip(0,6)
+        that follow it folded into the same pass."""
+        out_shape = conv_info["outShape"]
+        bk = self._epilogue_kind(bias, out_shape)
+        if bk in (None, capi.BCAST_FULL) or activation not in (None, "linear", "relu", "relu6"):
+            r = self.fused_depthwise_conv2d(x, filter, conv_info)
+            if bias is not None:
+                r = self.add(r, bias)
+            return self._map_activation(r, activation, None)
+        out = self._out(out_shape)
+        info = _info_c(conv_info)
+        self._ck(self.lib.tfhip_depthwise_conv2d(
+            self.ctx, self._h(x), self._h(filter), self._h(out), C.byref(info),
+            self._h(bias) if bk else -1, bk, capi.ACT[activation], self._q(filter)))
+        return out
+
+    def _pool(self, x, conv_info, kind):
+        out = self._out(conv_info["outShape"])
+        info = _info_c(conv_info)
+        self._ck(self.lib.tfhip_pool2d(self.ctx, self._h(x), self._h(out), C.byref(info),
+                                       capi.POOL[kind]))
+        return out
+
+    def avg_pool(self, x, conv_info):
+        return self._pool(x, conv_info, "avg")
+
+    def max_pool(self, x, conv_info):
+        r = self._pool(x, conv_info, "max")
+        return r if x.dtype == "float32" else self.cast(r, x.dtype)
+
+    # ---- elementwise ----
+    def _binary(self, op, a, b, out_dtype):
+        out_shape = su.broadcast_shape(a.shape, b.shape)
+        out = self._out(out_shape, out_dtype)
+        self._ck(self.lib.tfhip_binary(self.ctx, capi.BINARY[op], self._h(a), _shape_arr(a.shape),
+                                       a.rank, self._h(b), _shape_arr(b.shape), b.rank,
+                                       self._h(out)))
+        return out
+
+    @staticmethod
+    def _arith_dtype(a, b):
+        dt = su.upcast_type(a.dtype, b.dtype)
+        return "int32" if dt == "bool" else dt
+
+    def add(self, a, b):
+        return self._binary("add", a, b, self._arith_dtype(a, b))
+
+    def subtract(self, a, b):
+        return self._binary("sub", a, b, self._arith_dtype(a, b))
+
+    def multiply(self, a, b):
+        return self._binary("mul", a, b, self._arith_dtype(a, b))
+
+    def real_divide(self, a, b):
+        return self._binary("div", a, b, "float32")
+
+    def prelu(self, x, a):
+        return self._binary("prelu", x, a, "float32" if x.dtype == "float32" else "int32")
+
+    def maximum(self, a, b):
+        return self._binary("maximum", a, b, self._arith_dtype(a, b))
+
+    def minimum(self, a, b):
+        return self._binary("minimum", a, b, self._arith_dtype(a, b))
+
+    def _unary(self, op, x, out_dtype="float32", p0=0.0, p1=0.0):
+        out = self._out(x.shape, out_dtype)
+        self._ck(self.lib.tfhip_unary(self.ctx, capi.UNARY[op], self._h(x), self._h(out), p0, p1))
+        return out
+
+    def relu(self, x):  # keeps the input dtype (backend_cpu.ts:1194)
+        return self._unary("relu", x, "int32" if x.dtype != "float32" else "float32")
+
+    def clip(self, x, lo, hi):
+        return self._unary("clip", x, "float32", float(lo), float(hi))
+
+    def exp(self, x): return self._unary("exp", x)
+    def log(self, x): return self._unary("log", x)
+    def neg(self, x): return self._unary("neg", x, "int32" if x.dtype != "float32" else "float32")
+    def abs(self, x): return self._unary("abs", x)
+    def sigmoid(self, x): return self._unary("sigmoid", x)
+    def sqrt(self, x): return self._unary("sqrt", x)
+    def square(self, x): return self._unary("square", x)
+    def tanh(self, x): return self._unary("tanh", x)
+    def rsqrt(self, x): return self._unary("rsqrt", x)
+
+    def cast(self, x, dtype):
+        """castTensor (backends/backend_util.ts:34-71): widening casts alias the data id."""
+        if dtype == x.dtype:
+            return Tensor.make(x.shape, {"dataId": x.data_id}, dtype, self)
+        order = {"bool": 0, "int32": 1, "float32": 2}
+        if order[dtype] > order[x.dtype] and not x.quant:
+            return Tensor.make(x.shape, {"dataId": x.data_id}, dtype, self)
+        out = self._out(x.shape, dtype)
+        self._ck(self.lib.tfhip_cast(self.ctx, self._h(x), self._h(out)))
+        return out
+
+    def int(self, x):
+        out = self._out(x.shape, "int32")
+        self._ck(self.lib.tfhip_cast(self.ctx, self._h(x), self._h(out)))
+        return out
+
+    def dequantize(self, x):
+        out = self._out(x.shape, "float32")
+        self._ck(self.lib.tfhip_dequantize(self.ctx, self._h(x), self._h(out), self._q(x)))
+        return out
+
+    def fill(self, shape, value, dtype="float32"):
+        out = self._out(shape, dtype)
+        self._ck(self.lib.tfhip_fill(self.ctx, self._h(out), float(value)))
+        return out
+
+    def zeros_like(self, x):
+        return self.fill(x.shape, 0, x.dtype)
+
+    def ones_like(self, x):
+        return self.fill(x.shape, 1, x.dtype)
+
+    def reshape(self, x, shape):
+        """reshapeTensor (backends/backend_util.ts:79-82): same data id, new shape."""
+        shape = list(shape)
+        if -1 in shape:
+            known = su.size_from_shape([d for d in shape if d != -1])
+            shape[shape.index(-1)] = x.size // known if known else 0
+        if su.size_from_shape(shape) != x.size:
+            raise ValueError("Size(%d) must match the product of shape %s" % (x.size, shape))
+        t = Tensor(shape, x.dtype, x.data_id, None, self)
+        t.quant = x.quant
+        return t
+
+    # ---- reductions (innermost axes) ----
+    def _reduce(self, op, x, axes, out_dtype):
+        if not su.axes_are_inner_most_dims(axes, x.rank):
+            raise ValueError("%s must be called with innermost axes, got %s for rank %d"
+                             % (op, axes, x.rank))
+        out_shape, red_shape = su.compute_out_and_reduce_shapes(x.shape, axes)
+        out = self._out(out_shape, out_dtype)
+        self._ck(self.lib.tfhip_reduce(self.ctx, capi.REDUCE[op], self._h(x), self._h(out),
+                                       su.size_from_shape(out_shape),
+                                       su.size_from_shape(red_shape)))
+        return out
+
+    def sum(self, x, axes):
+        return self._reduce("sum", x, axes, su.upcast_type(x.dtype, "int32"))
+
+    def max(self, x, axes):
+        return self._reduce("max", x, axes, "float32" if x.dtype == "float32" else "int32")
+
+    def min(self, x, axes):
+        return self._reduce("min", x, axes, "float32" if x.dtype == "float32" else "int32")
+
+    def arg_max(self, x, axis):
+        return self._reduce("argmax", x, [axis], "int32")
+
+    def arg_min(self, x, axis):
+        return self._reduce("argmin", x, [axis], "int32")
+
+    def softmax(self, logits, dim):
+        """One-pass row softmax; the reference composes it from max/sub/exp/sum/log/add
+        (ops/softmax.ts:45-79)."""
+        cols = logits.shape[-1]
+        rows = logits.size // cols if cols else 0
+        out = self._out(logits.shape)
+        self._ck(self.lib.tfhip_softmax_rows(self.ctx, self._h(logits), self._h(out), rows, cols))
+        return out
+
+    # ---- data movement ----
+    def gather(self, x, indices, axis):
+        out_shape = list(x.shape)
+        out_shape[axis] = indices.size
+        out = self._out_like_storage(out_shape, x)
+        outer = su.size_from_shape(x.shape[:axis])
+        inner = su.size_from_shape(x.shape[axis + 1:])
+        idx = indices if indices.dtype == "int32" else self.int(indices)
+        self._ck(self.lib.tfhip_gather(self.ctx, self._h(x), self._h(idx), self._h(out), outer,
+                                       x.shape[axis], inner, indices.size))
+        return out
+
+    def transpose(self, x, perm):
+        out = self._out_like_storage([x.shape[p] for p in perm], x)
+        self._ck(self.lib.tfhip_transpose(self.ctx, self._h(x), _shape_arr(x.shape), x.rank,
+                                          _shape_arr(perm), self._h(out)))
+        return out

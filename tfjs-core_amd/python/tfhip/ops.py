@@ -1,0 +1,431 @@
+"""Op wrappers of the Node-free driver: argument validation and shape math in front of one
+backend call each, after tfjs-core/src/ops/{matmul,fused_ops,conv,pool,relu_ops,unary_ops,
+binary_ops,reduction_ops,softmax,segment_ops,transpose}.ts.  Python twin of js/ops.js."""
+import numpy as np
+
+from . import shape_util as su
+from .engine import ENGINE, NP_DTYPE, Tensor
+
+
+def _dtype_of(arr):
+    if arr.dtype == np.bool_:
+        return "bool"
+    if np.issubdtype(arr.dtype, np.integer):
+        return "int32"
+    return "float32"
+
+
+def tensor(values, shape=None, dtype=None):
+    """tf.tensor (ops/tensor_ops.ts:55-59, 108-112)."""
+    if isinstance(values, Tensor):
+        return values
+    arr = np.asarray(values)
+    if dtype is None:
+        dtype = _dtype_of(arr)
+    if shape is None:
+        shape = arr.shape
+    if su.size_from_shape(shape) != arr.size:
+        raise ValueError("Based on the provided shape, [%s], the tensor should have %d values "
+                         "but has %d" % (",".join(map(str, shape)), su.size_from_shape(shape),
+                                         arr.size))
+    if dtype == "bool":
+        arr = arr != 0
+    return Tensor(shape, dtype, None, np.ascontiguousarray(arr, NP_DTYPE[dtype]))
+
+
+def quantized_tensor(q, scale, min_, shape=None):
+    """A float32 weight tensor kept as uint8 affine-quantised bytes in HBM
+    (io/types.ts:100-107); consumers dequantise w = q*scale + min on load."""
+    arr = np.ascontiguousarray(q, np.uint8)
+    return Tensor(shape if shape is not None else arr.shape, "float32", None, arr, None,
+                  (float(scale), float(min_)))
+
+
+def dequantize(t):
+    return ENGINE.run_kernel(lambda b: b.dequantize(t))
+
+
+def _conv(x, name, op):
+    if not isinstance(x, Tensor):
+        x = tensor(x)
+    return x
+
+
+def _types_match(a, b):
+    """makeTypesMatch (tensor_util.ts:22-28)."""
+    if a.dtype == b.dtype:
+        return a, b
+    dt = su.upcast_type(a.dtype, b.dtype)
+    return cast(a, dt), cast(b, dt)
+
+
+def cast(x, dtype):
+    x = _conv(x, "x", "cast")
+    return ENGINE.run_kernel(lambda b: b.cast(x, dtype))
+
+
+def reshape(x, shape):
+    return ENGINE.run_kernel(lambda b: b.reshape(x, shape))
+
+
+# ---- matmul (ops/matmul.ts:41-124, ops/fused_ops.ts:52-220) ----
+def _matmul_prep(a, b, transpose_a, transpose_b, name):
+    a, b = _types_match(_conv(a, "a", name), _conv(b, "b", name))
+    if not (a.rank >= 2 and b.rank >= 2 and a.rank == b.rank):
+        raise ValueError("Error in %s: inputs must have the same rank of at least 2, got ranks "
+                         "%d and %d." % (name, a.rank, b.rank))
+    inner_a = a.shape[-2] if transpose_a else a.shape[-1]
+    inner_b = b.shape[-1] if transpose_b else b.shape[-2]
+    outer_a = a.shape[-1] if transpose_a else a.shape[-2]
+    outer_b = b.shape[-2] if transpose_b else b.shape[-1]
+    dims_a, dims_b = a.shape[:-2], b.shape[:-2]
+    if dims_a != dims_b:
+        raise ValueError("Error in %s: outer dimensions (%s) and (%s) of Tensors with shapes %s "
+                         "and %s must match." % (name, dims_a, dims_b, a.shape, b.shape))
+    if inner_a != inner_b:
+        raise ValueError("Error in %s: inner shapes (%d) and (%d) of Tensors with shapes %s and "
+                         "%s and transposeA=%s and transposeB=%s must match."
+                         % (name, inner_a, inner_b, a.shape, b.shape, transpose_a, transpose_b))
+    batch = su.size_from_shape(dims_a)
+    out_shape = tuple(dims_a) + (outer_a, outer_b)
+    a3 = (batch, inner_a, outer_a) if transpose_a else (batch, outer_a, inner_a)
+    b3 = (batch, outer_b, inner_b) if transpose_b else (batch, inner_b, outer_b)
+    return a, b, a3, b3, out_shape
+
+
+def matmul(a, b, transpose_a=False, transpose_b=False):
+    a, b, a3, b3, out_shape = _matmul_prep(a, b, transpose_a, transpose_b, "matMul")
+
+    def fwd(be):
+        r = be.batch_mat_mul(be.reshape(a, a3), be.reshape(b, b3), transpose_a, transpose_b)
+        return be.reshape(r, out_shape)
+    return ENGINE.run_kernel(fwd)
+
+
+def fused_matmul(a, b, transpose_a=False, transpose_b=False, bias=None, activation="linear",
+                 prelu_activation_weights=None):
+    a, b, a3, b3, out_shape = _matmul_prep(a, b, transpose_a, transpose_b, "fused matMul")
+    if bias is not None:
+        bias = _conv(bias, "bias", "fused matMul")
+        bias, _ = _types_match(bias, a)
+        su.broadcast_shape(out_shape, bias.shape)
+    if prelu_activation_weights is not None:
+        prelu_activation_weights = _conv(prelu_activation_weights, "prelu weights", "fused matMul")
+
+    def fwd(be):
+        r = be.fused_batch_mat_mul(be.reshape(a, a3), be.reshape(b, b3), transpose_a, transpose_b,
+                                   bias, activation, prelu_activation_weights)
+        return be.reshape(r, out_shape)
+    return ENGINE.run_kernel(fwd)
+
+
+# ---- convolutions (ops/conv.ts:145-217, 470-540; ops/fused_ops.ts:276-425) ----
+def _conv_prep(x, filt, strides, pad, data_format, dilations, rounding, name, depthwise=False):
+    x, filt = _conv(x, "x", name), _conv(filt, "filter", name)
+    lifted = x.rank == 3
+    x4 = reshape(x, (1,) + x.shape) if lifted else x
+    if x4.rank != 4:
+        raise ValueError("Error in %s: input must be rank 4, but got rank %d." % (name, x4.rank))
+    if filt.rank != 4:
+        raise ValueError("Error in %s: filter must be rank 4, but got rank %d." % (name, filt.rank))
+    if rounding is not None and not (isinstance(pad, (int, float)) and float(pad) == int(pad)):
+        raise ValueError("Error in %s: pad must be an integer when using, dimRoundingMode %s but "
+                         "got pad %s." % (name, rounding, pad))
+    if x4.shape[3] != filt.shape[2]:
+        raise ValueError("Error in %s: depth of input (%d) must match input depth for filter %d."
+                         % (name, x4.shape[3], filt.shape[2]))
+    if dilations is None:
+        dilations = (1, 1)
+    if not su.either_strides_or_dilations_are_one(strides, dilations):
+        raise ValueError("Error in %s: Either strides or dilations must be 1. Got strides %s and "
+                         "dilations '%s'" % (name, strides, dilations))
+    if data_format != "NHWC":
+        raise ValueError("Error in %s: got dataFormat of %s but only NHWC is currently supported."
+                         % (name, data_format))
+    ci = su.compute_conv2d_info(x4.shape, filt.shape, strides, dilations, pad, rounding, depthwise)
+    return x4, filt, ci, lifted
+
+
+def _lower(r, lifted):
+    return reshape(r, r.shape[1:]) if lifted else r
+
+
+def conv2d(x, filt, strides, pad, data_format="NHWC", dilations=(1, 1), dim_rounding_mode=None):
+    def run():
+        x4, f, ci, lifted = _conv_prep(x, filt, strides, pad, data_format, dilations,
+                                       dim_rounding_mode, "conv2d")
+        return _lower(ENGINE.run_kernel(lambda be: be.conv2d(x4, f, ci)), lifted)
+    return ENGINE.tidy(run)
+
+
+def fused_conv2d(x, filt, strides, pad, data_format="NHWC", dilations=(1, 1),
+                 dim_rounding_mode=None, bias=None, activation="linear",
+                 prelu_activation_weights=None):
+    def run():
+        x4, f, ci, lifted = _conv_prep(x, filt, strides, pad, data_format, dilations,
+                                       dim_rounding_mode, "fused conv2d")
+        bi = bias
+        if bi is not None:
+            bi, _ = _types_match(_conv(bi, "bias", "fused conv2d"), x4)
+            su.broadcast_shape(ci["outShape"], bi.shape)
+        r = ENGINE.run_kernel(lambda be: be.fused_conv2d(x4, f, ci, bi, activation,
+                                                         prelu_activation_weights))
+        return _lower(r, lifted)
+    return ENGINE.tidy(run)
+
+
+def depthwise_conv2d(x, filt, strides, pad, data_format="NHWC", dilations=(1, 1),
+                     dim_rounding_mode=None):
+    def run():
+        x4, f, ci, lifted = _conv_prep(x, filt, strides, pad, data_format, dilations,
+                                       dim_rounding_mode, "depthwiseConv2d", True)
+        return _lower(ENGINE.run_kernel(lambda be: be.depthwise_conv2d(x4, f, ci)), lifted)
+    return ENGINE.tidy(run)
+
+
+def fused_depthwise_conv2d(x, filt, strides, pad, data_format="NHWC", dilations=(1, 1),
+                           dim_rounding_mode=None, bias=None, activation="linear"):
+    """depthwiseConv2d + add(bias) + relu|clip(0,6).  Backends without the fused method run
+    the three reference calls (feature detection, as the harness does for backend_cpu)."""
+    def run():
+        x4, f, ci, lifted = _conv_prep(x, filt, strides, pad, data_format, dilations,
+                                       dim_rounding_mode, "fused depthwiseConv2d", True)
+
+        def fwd(be):
+            if hasattr(be, "fused_depthwise_conv2d"):
+                return be.fused_depthwise_conv2d(x4, f, ci, bias, activation)
+            r = be.depthwise_conv2d(x4, f, ci)
+            if bias is not None:
+                r = be.add(r, bias)
+            if activation == "relu":
+                r = be.relu(r)
+            elif activation == "relu6":
+                r = be.clip(r, 0, 6)
+            return r
+        return _lower(ENGINE.run_kernel(fwd), lifted)
+    return ENGINE.tidy(run)
+
+
+# ---- pooling (ops/pool.ts:56-203, 266-340) ----
+def _pool_impl(x, filter_size, strides, dilations, pad, rounding, kind):
+    def run():
+        xt = _conv(x, "x", kind + "Pool")
+        lifted = xt.rank == 3
+        x4 = reshape(xt, (1,) + xt.shape) if lifted else xt
+        if x4.rank != 4:
+            raise ValueError("Error in %sPool: x must be rank 4 but got rank %d." % (kind, x4.rank))
+        dil = (1, 1) if dilations is None else dilations
+        if not su.either_strides_or_dilations_are_one(strides, dil):
+            raise ValueError("Error in %sPool: Either strides or dilations must be 1. Got strides "
+                             "%s and dilations '%s'" % (kind, strides, dil))
+        if rounding is not None and not (isinstance(pad, (int, float)) and float(pad) == int(pad)):
+            raise ValueError("Error in %sPool: pad must be an integer when using, dimRoundingMode "
+                             "%s but got pad %s." % (kind, rounding, pad))
+        ci = su.compute_pool2d_info(x4.shape, filter_size, strides, dil, pad, rounding)
+        r = ENGINE.run_kernel(lambda be: be.avg_pool(x4, ci) if kind == "avg"
+                              else be.max_pool(x4, ci))
+        if kind == "avg" and r.dtype != xt.dtype:
+            r = cast(r, xt.dtype)  # ops/pool.ts:197
+        return _lower(r, lifted)
+    return ENGINE.tidy(run)
+
+
+def avg_pool(x, filter_size, strides, pad, dim_rounding_mode=None):
+    return _pool_impl(x, filter_size, strides, None, pad, dim_rounding_mode, "avg")
+
+
+def max_pool(x, filter_size, strides, pad, dim_rounding_mode=None):
+    return _pool_impl(x, filter_size, strides, None, pad, dim_rounding_mode, "max")
+
+
+def pool(x, window_shape, pooling_type, pad, dilations=None, strides=None):
+    """tf.pool (ops/pool.ts:266-340) for dilation rates the backend handles directly."""
+    return _pool_impl(x, window_shape, 1 if strides is None else strides,
+                      1 if dilations is None else dilations, pad, None, pooling_type)
+
+
+# ---- elementwise ----
+def _binary(name, method, a, b):
+    a, b = _types_match(_conv(a, "a", name), _conv(b, "b", name))
+    su.broadcast_shape(a.shape, b.shape)
+    return ENGINE.run_kernel(lambda be: getattr(be, method)(a, b))
+
+
+def add(a, b): return _binary("add", "add", a, b)
+def sub(a, b): return _binary("sub", "subtract", a, b)
+def mul(a, b): return _binary("mul", "multiply", a, b)
+def div(a, b): return _binary("div", "real_divide", a, b)
+def maximum(a, b): return _binary("maximum", "maximum", a, b)
+def minimum(a, b): return _binary("minimum", "minimum", a, b)
+
+
+def prelu(x, alpha):
+    x, alpha = _conv(x, "x", "prelu"), _conv(alpha, "alpha", "prelu")
+    return ENGINE.run_kernel(lambda be: be.prelu(x, alpha))
+
+
+def _unary(method):
+    def op(x):
+        x = _conv(x, "x", method)
+        return ENGINE.run_kernel(lambda be: getattr(be, method)(x))
+    op.__name__ = method
+    return op
+
+
+relu = _unary("relu")
+exp = _unary("exp")
+log = _unary("log")
+neg = _unary("neg")
+abs = _unary("abs")  # noqa: A001  (tf.abs)
+sigmoid = _unary("sigmoid")
+sqrt = _unary("sqrt")
+square = _unary("square")
+tanh = _unary("tanh")
+rsqrt = _unary("rsqrt")
+
+
+def clip_by_value(x, lo, hi):
+    """ops/unary_ops.ts:442-464."""
+    x = _conv(x, "x", "clipByValue")
+    if not lo <= hi:
+        raise ValueError("Error in clip: min (%s) must be less than or equal to max (%s)."
+                         % (lo, hi))
+    return ENGINE.run_kernel(lambda be: be.clip(x, lo, hi))
+
+
+def relu6(x):
+    return clip_by_value(x, 0, 6)
+
+
+# ---- reductions (ops/reduction_ops.ts) ----
+def _reduce(method, x, axis, keep_dims):
+    x = _conv(x, "x", method)
+
+    def run():
+        axes = su.parse_axis_param(axis, x.shape)
+        perm = su.get_axes_permutation(axes, x.rank)
+        xt, red = x, axes
+        if perm is not None:
+            xt = transpose(x, perm)
+            red = su.get_inner_most_axes(len(axes), x.rank)
+        r = ENGINE.run_kernel(lambda be: getattr(be, method)(xt, red))
+        if keep_dims:
+            out_shape, _ = su.compute_out_and_reduce_shapes(x.shape, axes)
+            r = reshape(r, su.expand_shape_to_keep_dim(out_shape, axes))
+        return r
+    return ENGINE.tidy(run)
+
+
+def sum(x, axis=None, keep_dims=False):  # noqa: A001
+    xt = _conv(x, "x", "sum")
+    if xt.dtype == "bool":
+        xt = cast(xt, "int32")
+    return _reduce("sum", xt, axis, keep_dims)
+
+
+def max(x, axis=None, keep_dims=False):  # noqa: A001
+    return _reduce("max", x, axis, keep_dims)
+
+
+def min(x, axis=None, keep_dims=False):  # noqa: A001
+    return _reduce("min", x, axis, keep_dims)
+
+
+def _arg(method, x, axis):
+    x = _conv(x, "x", method)
+
+    def run():
+        ax = 0 if axis is None else axis
+        axes = su.parse_axis_param(ax, x.shape)
+        perm = su.get_axes_permutation(axes, x.rank)
+        xt = x
+        if perm is not None:
+            xt = transpose(x, perm)
+            axes = su.get_inner_most_axes(1, x.rank)
+        return ENGINE.run_kernel(lambda be: getattr(be, method)(xt, axes[0]))
+    return ENGINE.tidy(run)
+
+
+def arg_max(x, axis=0):
+    return _arg("arg_max", x, axis)
+
+
+def arg_min(x, axis=0):
+    return _arg("arg_min", x, axis)
+
+
+def log_sum_exp(x, axis=None, keep_dims=False):
+    """ops/reduction_ops.ts:56-74."""
+    x = _conv(x, "x", "logSumExp")
+
+    def run():
+        axes = su.parse_axis_param(axis, x.shape)
+        x_max = max(x, axes, True)
+        c = sum(exp(sub(x, x_max)), axes)
+        d = log(c)
+        res = add(reshape(x_max, d.shape), d)
+        if keep_dims:
+            res = reshape(res, su.expand_shape_to_keep_dim(res.shape, axes))
+        return res
+    return ENGINE.tidy(run)
+
+
+def softmax(logits, dim=-1):
+    """ops/softmax.ts:45-79; uses the backend's one-pass kernel when it offers one, else the
+    reference composite exp(x - logSumExp(x))."""
+    logits = _conv(logits, "logits", "softmax")
+    if dim == -1:
+        dim = logits.rank - 1
+    if dim != logits.rank - 1:
+        raise ValueError("Softmax along a non-last dimension is not yet supported. Logits was "
+                         "rank %d and dim was %d" % (logits.rank, dim))
+    if hasattr(ENGINE.backend, "softmax"):
+        lf = cast(logits, "float32")
+        return ENGINE.run_kernel(lambda be: be.softmax(lf, dim))
+    return ENGINE.tidy(lambda: exp(sub(cast(logits, "float32"), log_sum_exp(logits, [dim], True))))
+
+
+# ---- data movement ----
+def gather(x, indices, axis=0):
+    """ops/segment_ops.ts:91-136."""
+    x = _conv(x, "x", "gather")
+    indices = _conv(indices, "indices", "gather")
+    if indices.dtype != "int32":
+        raise ValueError("Argument 'indices' passed to 'gather' must be int32 tensor")
+    axis = su.parse_axis_param(axis, x.shape)[0]
+
+    def run():
+        flat = reshape(indices, (indices.size,))
+        r = ENGINE.run_kernel(lambda be: be.gather(x, flat, axis))
+        out_shape = x.shape[:axis] + indices.shape + x.shape[axis + 1:]
+        return reshape(r, out_shape)
+    return ENGINE.tidy(run)
+
+
+def transpose(x, perm=None):
+    """ops/transpose.ts:42-66."""
+    x = _conv(x, "x", "transpose")
+    if perm is None:
+        perm = list(range(x.rank))[::-1]
+    if x.rank != len(perm):
+        raise ValueError("Error in transpose: rank of input %d must match length of perm %s."
+                         % (x.rank, perm))
+    for p in perm:
+        if not 0 <= p < x.rank:
+            raise ValueError("All entries in 'perm' must be between 0 and %d but got %s"
+                             % (x.rank - 1, perm))
+    if x.rank <= 1:
+        return ENGINE.run_kernel(lambda be: be.reshape(x, x.shape))
+    return ENGINE.run_kernel(lambda be: be.transpose(x, list(perm)))
+
+
+def fill(shape, value, dtype="float32"):
+    return ENGINE.run_kernel(lambda be: be.fill(shape, value, dtype))
+
+
+def zeros(shape, dtype="float32"):
+    return fill(shape, 0, dtype)
+
+
+def ones(shape, dtype="float32"):
+    return fill(shape, 1, dtype)
