@@ -109,7 +109,7 @@ def roofline_of_dominant_kernel(rows):
     return roof, groups
 
 
-def cpu_baseline(mobilenet, params, budget_s=20.0):
+def cpu_baseline(mobilenet, params, budget_s=15.0):
     """The CPU oracle (restatement of backend_cpu's loops, one thread) on batch-1 forwards
     of the same network: a bounded sample, reported as images/s."""
     import numpy as np
@@ -125,7 +125,7 @@ def cpu_baseline(mobilenet, params, budget_s=20.0):
         oracle_forward(ref, params, x)
         n += 1
         el = time.perf_counter() - t0
-        if el + el / n > budget_s or n >= 8:
+        if el + el / n > budget_s:
             break
     return dict(value=round(n / el, 4), unit="images/s", cores=1, kind="port",
                 sample="%d batch-1 forward passes of the same MobileNetV1 (%.1f s), C restatement "
