@@ -132,6 +132,52 @@ def cpu_baseline(mobilenet, params, budget_s=15.0):
                        "of backend_cpu at -O2, 1 thread" % (n, el))
 
 
+def write_weight_files(params, bin_path, manifest_path):
+    """Weights as a tfjs-style flat binary + manifest entries (name, shape, dtype and, for
+    uint8 affine-quantised tensors, quantization {dtype, scale, min})."""
+    import numpy as np
+    from tfhip import mobilenet  # noqa: F401
+    order = ["stem_w", "stem_b"]
+    for i in range(1, 14):
+        order += ["dw%d_w" % i, "dw%d_b" % i, "pw%d_w" % i, "pw%d_b" % i]
+    order += ["fc_w", "fc_b"]
+    manifest = []
+    with open(bin_path, "wb") as f:
+        for name in order:
+            v = params[name]
+            if isinstance(v, tuple):
+                q, scale, mn = v
+                f.write(np.ascontiguousarray(q, np.uint8).tobytes())
+                manifest.append(dict(name=name, shape=list(q.shape), dtype="float32",
+                                     quantization=dict(dtype="uint8", scale=scale, min=mn)))
+            else:
+                f.write(np.ascontiguousarray(v, np.float32).tobytes())
+                manifest.append(dict(name=name, shape=list(v.shape), dtype="float32"))
+    with open(manifest_path, "w") as f:
+        json.dump(manifest, f)
+
+
+def js_host_leg(params, x_host, batch, steps, warmup):
+    """The same step driven by the JavaScript host (tf.* graph in Node.js over the N-API
+    addon), as a child process on the same bytes.  None when node is not installed."""
+    import shutil
+    import subprocess
+    import tempfile
+    node = shutil.which("node")
+    js = os.path.join(ROOT, "tfjs-core_amd", "js")
+    if node is None or not os.path.exists(os.path.join(js, "tfjs_hip.node")):
+        return None
+    with tempfile.TemporaryDirectory() as d:
+        wb, mf, xb = (os.path.join(d, n) for n in ("w.bin", "manifest.json", "x.bin"))
+        write_weight_files(params, wb, mf)
+        x_host.tofile(xb)
+        r = subprocess.run([node, os.path.join(js, "bench_mobilenet.js"), wb, mf, xb, str(batch),
+                            str(steps), str(warmup)], capture_output=True, text=True, timeout=600)
+    if r.returncode != 0:
+        return dict(error=(r.stderr or r.stdout)[-400:])
+    return json.loads(r.stdout.strip().splitlines()[-1])
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -140,6 +186,7 @@ def main():
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--quant", action="store_true", help="uint8 weights dequantised in-kernel")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-js", action="store_true", help="skip the Node.js host leg")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -184,6 +231,17 @@ def main():
         print("sum of layer times: %.3f ms; step (events): %.3f ms; step (wall): %.3f ms" % (
             sum(r["ms"] for r in rows), info["kernelMs"] / args.steps, ms_per_step), file=sys.stderr)
 
+    # The product's host is JavaScript: when node is present the headline value is the step
+    # rate of the tf.* graph driven from Node.js; the Python driver's rate is kept beside it.
+    python_driver = dict(images_per_s=round(value, 1), ms_per_step=round(ms_per_step, 4),
+                         gpu_ms_per_step_events=round(info["kernelMs"] / args.steps, 4))
+    host = "python ctypes driver over the C ABI"
+    events_ms = info["kernelMs"] / args.steps
+    js = None if args.no_js else js_host_leg(dev_params, x_host, args.batch, args.steps, args.warmup)
+    if js is not None and "error" not in js:
+        value, ms_per_step, events_ms = js["images_per_s"], js["ms_per_step"], js["gpu_ms_per_step_events"]
+        host = "JavaScript tf.* graph in Node.js %s over the N-API addon" % js["node"]
+
     out = {
         "metric": "MobileNetV1-224 images/s at batch 64" if args.batch == 64 and not args.quant
                   else "MobileNetV1-224 images/s at batch %d%s" % (args.batch, " (uint8 weights)" if args.quant else ""),
@@ -193,8 +251,10 @@ def main():
         "config": {"workload": "MobileNetV1-1.0-224 random-init fp32 NHWC forward + softmax, "
                                "batch %d%s, tf.* graph on the hip backend" % (
                                    args.batch, ", uint8 weights" if args.quant else ""),
-                   "global_batch": args.batch, "host": "python ctypes driver over the C ABI"},
-        "gpu_ms_per_step_events": round(info["kernelMs"] / args.steps, 4),
+                   "global_batch": args.batch, "host": host},
+        "gpu_ms_per_step_events": round(events_ms, 4),
+        "python_driver": python_driver,
+        "js_host": js,
         "dense_tflops": round(sum(2e-9 * r["macs"] for r in rows if r["kernel"].startswith("gemm"))
                               / sum(r["ms"] for r in rows if r["kernel"].startswith("gemm")), 2),
         "roofline": roof,

@@ -1,0 +1,216 @@
+"""The JavaScript host path on the GPU: tf.* -> engine -> MathBackendHIP -> N-API addon ->
+libtfjs_hip.so, compared with the CPU oracle on the same bytes."""
+import json
+import os
+import shutil
+import subprocess
+
+import numpy as np
+import pytest
+
+from conftest import ROOT
+
+pytestmark = pytest.mark.gpu
+
+JS = os.path.join(ROOT, "tfjs-core_amd", "js")
+NODE = shutil.which("node")
+NP = {"float32": np.float32, "int32": np.int32, "bool": np.uint8}
+
+
+class Cases(object):
+    def __init__(self, d):
+        self.dir = str(d)
+        self.cases = []
+        self.expect = {}
+
+    def _put(self, name, arr, quant=None):
+        arr = np.asarray(arr)
+        dtype = "bool" if arr.dtype == np.bool_ else ("int32" if arr.dtype.kind in "iu" and not quant
+                                                      else "float32")
+        f = "%s.bin" % name
+        data = arr.astype(np.uint8) if quant else arr.astype(NP[dtype])
+        data.tofile(os.path.join(self.dir, f))
+        spec = {"file": f, "shape": list(arr.shape), "dtype": dtype}
+        if quant:
+            spec["quant"] = {"scale": quant[0], "min": quant[1]}
+        return spec
+
+    def add(self, name, op, inputs, attrs, expected, rtol=1e-4, atol=1e-5, exact=False):
+        specs = {}
+        for k, v in inputs.items():
+            if v is None:
+                continue
+            if isinstance(v, tuple):
+                specs[k] = self._put("%s_%s" % (name, k), v[0], (v[1], v[2]))
+            else:
+                specs[k] = self._put("%s_%s" % (name, k), v)
+        self.cases.append({"name": name, "op": op, "inputs": specs, "attrs": attrs})
+        self.expect[name] = (np.asarray(expected), rtol, atol, exact)
+
+    def run(self):
+        with open(os.path.join(self.dir, "cases.json"), "w") as f:
+            json.dump({"cases": self.cases}, f)
+        r = subprocess.run([NODE, os.path.join(JS, "test", "run_cases.js"), self.dir],
+                           capture_output=True, text=True, timeout=600)
+        assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-3000:]
+        with open(os.path.join(self.dir, "results.json")) as f:
+            return json.load(f)
+
+    def check(self, results):
+        for name, (want, rtol, atol, exact) in self.expect.items():
+            res = results["results"][name]
+            assert "error" not in res, "%s: %s" % (name, res.get("error"))
+            got = np.fromfile(os.path.join(self.dir, name + ".out.bin"), NP[res["dtype"]])
+            got = got.reshape(res["shape"])
+            assert list(got.shape) == list(want.shape), (name, got.shape, want.shape)
+            if exact:
+                assert np.array_equal(got, want), name
+            else:
+                g, e = got.astype(np.float64), want.astype(np.float64)
+                ok = (np.isnan(g) & np.isnan(e)) | (np.abs(g - e) <= atol + rtol * np.abs(e)) | (g == e)
+                assert ok.all(), "%s: max err %g" % (name, np.nanmax(np.abs(g - e)))
+            assert res["leaked"] == 0, "%s leaked %d tensors" % (name, res["leaked"])
+
+
+@pytest.fixture(scope="module")
+def ref(oracle):
+    from providers import OracleOps
+    return OracleOps()
+
+
+@pytest.mark.skipif(NODE is None, reason="node is not installed")
+def test_js_ops_match_oracle(tmp_path, ref):
+    rng = np.random.default_rng(42)
+    c = Cases(tmp_path)
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)
+    u = lambda *s: rng.uniform(0, 1, s).astype(np.float32)
+
+    # config 1 and transposes
+    a, b = rng.uniform(-1, 1, (256, 512)).astype(np.float32), rng.uniform(-1, 1, (512, 256)).astype(np.float32)
+    c.add("c1_matmul", "matMul", dict(a=a, b=b), {}, ref.matmul(a[None], b[None])[0])
+    a2, b2 = f(3, 33, 17), f(3, 65, 17)
+    c.add("matmul_bt", "matMul", dict(a=a2, b=b2), dict(transposeB=True), ref.matmul(a2, b2, False, True))
+    a3 = f(2, 2, 17, 9)
+    b3 = f(2, 2, 17, 5)
+    c.add("matmul_4d_at", "matMul", dict(a=a3, b=b3), dict(transposeA=True),
+          ref.matmul(a3.reshape(4, 17, 9), b3.reshape(4, 17, 5), True, False).reshape(2, 2, 9, 5))
+    bias, alpha = f(24), u(24)
+    am, bm = f(19, 40), f(40, 24)
+    for act in ("linear", "relu", "relu6", "prelu"):
+        c.add("fused_mm_" + act, "fusedMatMul", dict(a=am, b=bm, bias=bias, prelu=alpha if act == "prelu" else None),
+              dict(activation=act),
+              ref.matmul(am[None], bm[None], bias=bias, activation=act, prelu=alpha if act == "prelu" else None)[0])
+    odd_bias = f(19, 1)
+    c.add("fused_mm_oddbias", "fusedMatMul", dict(a=am, b=bm, bias=odd_bias), dict(activation="relu"),
+          ref.matmul(am[None], bm[None], bias=odd_bias, activation="relu")[0])
+    ai = rng.integers(-5, 5, (4, 6)).astype(np.int32)
+    bi = rng.integers(-5, 5, (6, 3)).astype(np.int32)
+    c.add("matmul_int32", "matMul", dict(a=ai, b=bi), {}, (ai @ bi).astype(np.int32), exact=True)
+    c.add("matmul_zero", "matMul", dict(a=np.zeros((0, 3), np.float32), b=f(3, 2)), {}, np.zeros((0, 2), np.float32))
+
+    # convolutions
+    x, w, cb = u(2, 12, 12, 8), f(3, 3, 8, 16) * 0.2, f(16)
+    c.add("conv", "conv2d", dict(x=x, filter=w), dict(strides=1, pad="same"), ref.conv2d(x, w, 1, "same"))
+    c.add("conv_s2", "conv2d", dict(x=x, filter=w), dict(strides=2, pad="same"), ref.conv2d(x, w, 2, "same"))
+    c.add("conv_rank3", "conv2d", dict(x=x[0], filter=w), dict(strides=1, pad="valid"), ref.conv2d(x[:1], w, 1, "valid")[0])
+    for act in ("linear", "relu", "relu6"):
+        c.add("fconv_" + act, "fusedConv2d", dict(x=x, filter=w, bias=cb), dict(strides=1, pad="same", activation=act),
+              ref.conv2d(x, w, 1, "same", bias=cb, activation=act))
+    c.add("conv_unfused_relu6", "unfusedRelu6Conv", dict(x=x, filter=w, bias=cb), dict(strides=1, pad="same"),
+          ref.conv2d(x, w, 1, "same", bias=cb, activation="relu6"))
+    xs, ws = u(1, 16, 16, 3), f(3, 3, 3, 32) * 0.3
+    sb = f(32)
+    c.add("conv_stem", "fusedConv2d", dict(x=xs, filter=ws, bias=sb), dict(strides=2, pad="same", activation="relu6"),
+          ref.conv2d(xs, ws, 2, "same", bias=sb, activation="relu6"))
+    wd, db = f(3, 3, 8, 1), f(8)
+    c.add("dw", "depthwiseConv2d", dict(x=x, filter=wd), dict(strides=1, pad="same"), ref.depthwise_conv2d(x, wd, 1, "same"))
+    c.add("fdw_s2", "fusedDepthwiseConv2d", dict(x=x, filter=wd, bias=db), dict(strides=2, pad="same", activation="relu6"),
+          ref.depthwise_conv2d(x, wd, 2, "same", bias=db, activation="relu6"))
+    wd2 = f(3, 3, 8, 2)
+    c.add("dw_chmul2", "depthwiseConv2d", dict(x=x, filter=wd2), dict(strides=1, pad="valid"),
+          ref.depthwise_conv2d(x, wd2, 1, "valid"))
+    q = rng.integers(0, 256, (3, 3, 8, 16)).astype(np.uint8)
+    c.add("conv_uint8", "conv2d", dict(x=x, filter=(q, 0.011, -1.4)), dict(strides=1, pad="same"),
+          ref.conv2d(x, ref.dequantize(q, 0.011, -1.4), 1, "same"))
+
+    # pooling
+    xp = f(2, 7, 7, 16)
+    c.add("avgpool_global", "avgPool", dict(x=xp), dict(filterSize=7, strides=1, pad="valid"), ref.avg_pool(xp, 7, 1, "valid"))
+    c.add("avgpool_same", "avgPool", dict(x=xp), dict(filterSize=3, strides=2, pad="same"), ref.avg_pool(xp, 3, 2, "same"))
+    c.add("maxpool", "maxPool", dict(x=xp), dict(filterSize=2, strides=2, pad="valid"), ref.max_pool(xp, 2, 2, "valid"), exact=True)
+
+    # elementwise and reductions
+    e1, e2 = f(6, 5, 12), f(5, 1)
+    for op in ("add", "sub", "mul", "div", "maximum", "minimum"):
+        c.add("bin_" + op, op, dict(a=e1, b=e2 + np.float32(3)), {}, getattr(ref, op)(e1, e2 + np.float32(3)), rtol=1e-6)
+    al = u(12)
+    c.add("prelu", "prelu", dict(x=e1, alpha=al), {}, ref.prelu(e1, al))
+    nanx = np.array([-3, 0, 2.5, 6, 7.5, np.nan, np.inf, -np.inf], np.float32)
+    c.add("relu_nan", "relu", dict(x=nanx), {}, ref.relu(nanx))
+    c.add("relu6_nan", "relu6", dict(x=nanx), {}, ref.clip(nanx, 0, 6))
+    c.add("clip", "clipByValue", dict(x=e1), dict(min=-0.5, max=0.25), ref.clip(e1, -0.5, 0.25))
+    c.add("exp", "exp", dict(x=e1), {}, ref.exp(e1), rtol=1e-5)
+    c.add("log", "log", dict(x=np.abs(e1) + np.float32(0.1)), {}, ref.log(np.abs(e1) + np.float32(0.1)), rtol=1e-5, atol=1e-6)
+    r2 = f(64, 1000)
+    c.add("sum_last", "sum", dict(x=r2), dict(axis=-1), ref.sum(r2), rtol=1e-5)
+    c.add("sum_axis0_keep", "sum", dict(x=r2[:, :9]), dict(axis=0, keepDims=True),
+          ref.sum(np.ascontiguousarray(r2[:, :9].T))[None], rtol=1e-5)
+    c.add("max_last", "max", dict(x=r2), dict(axis=1), ref.max(r2), exact=True)
+    c.add("min_all", "min", dict(x=r2[:3, :7]), dict(), ref.min(np.ascontiguousarray(r2[:3, :7]).reshape(1, -1)).reshape(()), exact=True)
+    c.add("argmax", "argMax", dict(x=r2), dict(axis=-1), ref.argmax(r2), exact=True)
+    c.add("argmax_axis0", "argMax", dict(x=r2[:, :5]), dict(axis=0), ref.argmax(np.ascontiguousarray(r2[:, :5].T)), exact=True)
+    c.add("argmin", "argMin", dict(x=r2), dict(axis=1), ref.argmin(r2), exact=True)
+    c.add("softmax", "softmax", dict(x=r2), {}, ref.softmax(r2), atol=1e-7)
+    c.add("softmax_composite", "softmaxComposite", dict(x=r2), {}, ref.softmax(r2), atol=1e-7)
+    lse = np.log(np.exp(r2.astype(np.float64)).sum(-1))
+    c.add("logsumexp", "logSumExp", dict(x=r2), dict(axis=-1), lse.astype(np.float32), rtol=1e-5)
+    idx = np.array([3, 0, 0, 2], np.int32)
+    g = f(5, 4, 6)
+    c.add("gather_axis1", "gather", dict(x=g, indices=idx), dict(axis=1), ref.gather(g, idx, 1), exact=True)
+    c.add("gather_2d_idx", "gather", dict(x=g, indices=idx.reshape(2, 2)), dict(axis=0),
+          ref.gather(g, idx, 0).reshape(2, 2, 4, 6), exact=True)
+    c.add("transpose", "transpose", dict(x=g), dict(perm=[2, 0, 1]), ref.transpose(g, [2, 0, 1]), exact=True)
+    cv = np.array([1.9, -1.9, 0.5, np.nan, 3e9, -7.0], np.float32)
+    c.add("cast_int", "cast", dict(x=cv), dict(dtype="int32"), ref.to_int(cv), exact=True)
+    c.add("cast_bool", "cast", dict(x=cv), dict(dtype="bool"), (cv != 0).astype(np.uint8), exact=True)
+    ch = f(3, 8)
+    c.add("chain_methods", "chainMethods", dict(x=ch), {},
+          np.float32((np.maximum(ch, 0).astype(np.float64) * ch).sum()), rtol=1e-5)
+
+    results = c.run()
+    c.check(results)
+    assert results["kernelMs"] > 0 and results["lastKernel"].startswith("gemm_")
+    assert any("matMul" in line for line in results["debugLog"]), "DEBUG mode logs each kernel"
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
+@pytest.mark.skipif(NODE is None, reason="node is not installed")
+@pytest.mark.parametrize("quant", [False, True])
+def test_js_mobilenet_matches_oracle(tmp_path, ref, quant):
+    """MobileNetV1 through the JS graph with weights loaded from a tfjs-style manifest +
+    binary; uint8 weights stay bytes in HBM (decodeWeightsToDevice)."""
+    from providers import oracle_mobilenet_forward
+    from tfhip import mobilenet
+    import bench
+    params = mobilenet.make_params(seed=21)
+    x = np.random.default_rng(22).uniform(0, 1, (1, 224, 224, 3)).astype(np.float32)
+    store = mobilenet.quantize_params(params) if quant else params
+    bench.write_weight_files(store, str(tmp_path / "w.bin"), str(tmp_path / "manifest.json"))
+    if quant:
+        params = {k: (ref.dequantize(*v) if isinstance(v, tuple) else v) for k, v in store.items()}
+    want, _ = oracle_mobilenet_forward(ref, params, x)
+    c = Cases(tmp_path)
+    c.cases.append({"name": "mobilenet", "op": "mobilenet",
+                    "inputs": {"x": c._put("mobilenet_x", x)},
+                    "attrs": {"weights": "w.bin", "manifest": "manifest.json", "onDevice": True}})
+    results = c.run()
+    res = results["results"]["mobilenet"]
+    assert "error" not in res, res.get("error")
+    got = np.fromfile(os.path.join(c.dir, "mobilenet.out.bin"), np.float32).reshape(res["shape"])
+    err = np.abs(got.astype(np.float64) - want)
+    assert np.all(err <= 1e-3 + 1e-3 * np.abs(want)), "max logit error %g" % err.max()
+    assert abs(res["probSum"][0] - 1) < 1e-4 and res["leaked"] == 0
+    gap = np.sort(want[0])
+    if gap[-1] - gap[-2] > 2e-3:
+        top = np.fromfile(os.path.join(c.dir, "mobilenet.top.bin"), np.int32)
+        assert top[0] == int(np.argmax(want[0]))

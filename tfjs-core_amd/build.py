@@ -68,8 +68,10 @@ def build_addon(force=False, verbose=False):
     if not force and not _stale(ADDON, [src, os.path.join(INCLUDE, "tfjs_hip.h")]):
         return ADDON
     os.makedirs(os.path.dirname(ADDON), exist_ok=True)
-    cmd = ["gcc", "-O2", "-fPIC", "-shared", "-Wall", "-I" + NODE_INCLUDE, "-I" + INCLUDE, src,
-           "-o", ADDON, "-ldl"]
+    # the addon sits in js/, the library one directory up
+    cmd = ["gcc", "-O2", "-fPIC", "-shared", "-Wall", "-DNODE_GYP_MODULE_NAME=tfjs_hip",
+           "-I" + NODE_INCLUDE, "-I" + INCLUDE, src, "-o", ADDON, "-L" + HERE, "-ltfjs_hip",
+           "-Wl,-rpath,$ORIGIN/.."]
     if verbose:
         print(" ".join(cmd))
     subprocess.check_call(cmd)

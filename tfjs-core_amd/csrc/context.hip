@@ -36,11 +36,12 @@ static size_t round_cap(size_t n) {
 
 void* tfhip_ctx::alloc(size_t nbytes, size_t* cap) {
   const size_t want = round_cap(nbytes);
-  auto it = pool.lower_bound(want);
-  if (it != pool.end() && it->first == want) {
-    void* p = it->second;
-    pooled -= it->first;
-    pool.erase(it);
+  auto it = pool.find(want);
+  if (it != pool.end() && !it->second.empty()) {
+    // most recently freed block first: it is the one most likely still in L2 / MALL
+    void* p = it->second.back();
+    it->second.pop_back();
+    pooled -= want;
     in_use += want;
     *cap = want;
     return p;
@@ -66,13 +67,14 @@ void tfhip_ctx::release(void* p, size_t cap) {
   if (!p) return;
   in_use -= cap;
   pooled += cap;
-  pool.emplace(cap, p);
+  pool[cap].push_back(p);
 }
 
 void tfhip_ctx::trim() {
   if (pool.empty()) return;
   (void)hipStreamSynchronize(stream);
-  for (auto& kv : pool) (void)hipFree(kv.second);
+  for (auto& kv : pool)
+    for (void* p : kv.second) (void)hipFree(p);
   pool.clear();
   pooled = 0;
 }
@@ -124,7 +126,8 @@ void tfhip_destroy(tfhip_ctx* ctx) {
   (void)hipStreamSynchronize(ctx->stream);
   for (auto& kv : ctx->bufs)
     if (kv.second.ptr) (void)hipFree(kv.second.ptr);
-  for (auto& kv : ctx->pool) (void)hipFree(kv.second);
+  for (auto& kv : ctx->pool)
+    for (void* p : kv.second) (void)hipFree(p);
   (void)hipEventDestroy(ctx->ev_begin);
   (void)hipEventDestroy(ctx->ev_end);
   (void)hipStreamDestroy(ctx->stream);

@@ -17,6 +17,8 @@
 // k = r (low half) with k = 4+r (high half): a permutation of the summation order only.
 // Likewise lane j of accumulator tile tj owns column TN*j + tj, so a lane reads its TN B
 // values with one access and writes TN adjacent results.
+#include <type_traits>
+
 #include "tfhip_internal.h"
 
 namespace tfhip {
@@ -47,6 +49,7 @@ struct GemmArgs {
 
 constexpr int BK = 16;
 constexpr int LDA_S = BK + 4;
+constexpr int TILES_PER_KBLOCK = 48 / BK;
 
 // w = q*scale + min evaluated in double, rounded once (io/io_utils.ts:133-136).
 __device__ __forceinline__ float dequant(unsigned q, double scale, double mn) {
@@ -79,7 +82,7 @@ __device__ __forceinline__ int xcd_remap(int bid, int total) {
   return start + i;
 }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN, int AMODE, int BMODE>
+template <int WAVES_M, int WAVES_N, int TM, int TN, int AMODE, int BMODE, bool KBLOCKED>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmArgs p) {
   constexpr int THREADS = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 32;
@@ -282,13 +285,21 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     }
   };
 
-  f32x16 acc[TM][TN];
+  // KBLOCKED (matMul): two-level accumulation.  The matrix cores sum 48 consecutive k into
+  // `blk`, which is then added to `acc` — the block structure of the reference's matmul
+  // (backend_cpu.ts:83, 516-535: 48-wide k blocks, one float32 rounding per block).  It
+  // keeps float32 round-off from growing with K: partial sums stay small inside a block.
+  // Convolutions accumulate straight through, as the reference's conv2d does (:1601-1604).
+  f32x16 acc[TM][TN], blk[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
     for (int j = 0; j < TN; j++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 16; r++) {
+        acc[i][j][r] = 0.f;
+        blk[i][j][r] = 0.f;
+      }
 
   f32x4 a_reg[A_PER], b_reg[B_PER];
   const int k_tiles = (p.K + BK - 1) / BK;
@@ -299,7 +310,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   store_b(Bs[0], b_reg);
   __syncthreads();
 
-  for (int kt = 0; kt < k_tiles; kt++) {
+  // One tile step: prefetch tile kt+1 into registers, run the matrix cores on tile kt out
+  // of LDS, park the prefetched tile in the other LDS buffer.  `fresh` (compile time) makes
+  // the first MFMA of each accumulator start from zero instead of from `blk`.
+  auto tile_step = [&](int kt, auto fresh_tag) {
+    constexpr bool fresh = decltype(fresh_tag)::value;
     const int cur = kt & 1;
     if (kt + 1 < k_tiles) {
       load_a((kt + 1) * BK, a_reg);
@@ -335,14 +350,40 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
-          for (int j = 0; j < TN; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][r], b[r][j], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < TN; j++) {
+            if (fresh && kc == 0 && r == 0) {
+              const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
+                                   0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+              blk[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][r], b[r][j], zero, 0, 0, 0);
+            } else {
+              blk[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][r], b[r][j], blk[i][j], 0, 0, 0);
+            }
+          }
     }
     if (kt + 1 < k_tiles) {
       store_a(As[cur ^ 1], a_reg);
       store_b(Bs[cur ^ 1], b_reg);
     }
     __syncthreads();
+  };
+
+  if (KBLOCKED) {
+    for (int kt = 0; kt < k_tiles; kt += TILES_PER_KBLOCK) {
+      tile_step(kt, std::true_type{});
+#pragma unroll
+      for (int t = 1; t < TILES_PER_KBLOCK; t++)
+        if (kt + t < k_tiles) tile_step(kt + t, std::false_type{});
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] += blk[i][j];
+    }
+  } else {
+    for (int kt = 0; kt < k_tiles; kt++) tile_step(kt, std::false_type{});
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) acc[i][j] = blk[i][j];
   }
 
   // ---- epilogue: bias, activation, store.  Accumulator register r of a 32x32 tile holds
@@ -411,23 +452,23 @@ struct TileCfg {
   static constexpr int BM = WM_ * TM_ * 32, BN = WN_ * TN_ * 32;
 };
 
-template <class T, int AMODE, int BMODE>
+template <class T, int AMODE, int BMODE, bool KBLOCKED>
 static void launch_cfg(tfhip_ctx* ctx, GemmArgs& p, int batch) {
   static const char* const a_names[] = {"rowmajor", "transposed", "im2col"};
   static const char* const b_names[] = {"f32", "f32t", "u8"};
-  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "gemm_%dx%d_%s_%s", T::BM, T::BN,
-           a_names[AMODE], b_names[BMODE]);
+  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "gemm_%dx%d_%s_%s%s", T::BM, T::BN,
+           a_names[AMODE], b_names[BMODE], KBLOCKED ? "_kb48" : "");
   hipStream_t s = ctx->stream;
   p.tiles_m = (p.M + T::BM - 1) / T::BM;
   p.tiles_n = (p.N + T::BN - 1) / T::BN;
   dim3 grid(p.tiles_m * p.tiles_n, 1, batch);
-  hipLaunchKernelGGL((gemm_kernel<T::WM, T::WN, T::TM, T::TN, AMODE, BMODE>), grid,
+  hipLaunchKernelGGL((gemm_kernel<T::WM, T::WN, T::TM, T::TN, AMODE, BMODE, KBLOCKED>), grid,
                      dim3(T::WM * T::WN * 64), 0, s, p);
 }
 
 // Tile choice: the widest tile whose grid still gives every CU work; narrow-N tiles for
 // the early MobileNet layers (N = 32/64) so no matrix-core columns are wasted.
-template <int AMODE, int BMODE>
+template <int AMODE, int BMODE, bool KBLOCKED>
 static void launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
   using Big = TileCfg<2, 2, 2, 2>;     // 128 x 128
   using Mid = TileCfg<2, 2, 2, 1>;     // 128 x 64
@@ -438,33 +479,36 @@ static void launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
     return (long long)ceil_div(p.M, bm) * ceil_div(p.N, bn) * batch;
   };
   if (p.N <= 32) {
-    launch_cfg<Thin, AMODE, BMODE>(ctx, p, batch);
+    launch_cfg<Thin, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
   } else if (p.N <= 64) {
-    if (blocks(128, 64) >= cus) launch_cfg<Mid, AMODE, BMODE>(ctx, p, batch);
-    else launch_cfg<Small, AMODE, BMODE>(ctx, p, batch);
+    if (blocks(128, 64) >= cus) launch_cfg<Mid, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
+    else launch_cfg<Small, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
   } else if (blocks(128, 128) >= 2 * cus) {
-    launch_cfg<Big, AMODE, BMODE>(ctx, p, batch);
+    launch_cfg<Big, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
   } else if (blocks(128, 64) >= 2 * cus) {
-    launch_cfg<Mid, AMODE, BMODE>(ctx, p, batch);
+    launch_cfg<Mid, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
   } else {
-    launch_cfg<Small, AMODE, BMODE>(ctx, p, batch);
+    launch_cfg<Small, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
   }
 }
 
-static int launch_gemm(tfhip_ctx* ctx, GemmArgs& p, int batch, int amode, int bmode) {
-#define TFHIP_CASE(AM, BM_)                                      \
-  if (amode == AM && bmode == BM_) {                             \
-    launch_mode<AM, BM_>(ctx, p, batch);                         \
+static int launch_gemm(tfhip_ctx* ctx, GemmArgs& p, int batch, int amode, int bmode,
+                       bool kblocked) {
+#define TFHIP_CASE(AM, BM_, KB)                                  \
+  if (amode == AM && bmode == BM_ && kblocked == KB) {           \
+    launch_mode<AM, BM_, KB>(ctx, p, batch);                     \
     TFHIP_LAUNCH_CHECK(ctx);                                     \
     return TFHIP_OK;                                             \
   }
-  TFHIP_CASE(A_ROWMAJOR, B_ROWMAJOR)
-  TFHIP_CASE(A_ROWMAJOR, B_TRANSPOSED)
-  TFHIP_CASE(A_ROWMAJOR, B_UINT8)
-  TFHIP_CASE(A_TRANSPOSED, B_ROWMAJOR)
-  TFHIP_CASE(A_TRANSPOSED, B_TRANSPOSED)
-  TFHIP_CASE(A_IM2COL, B_ROWMAJOR)
-  TFHIP_CASE(A_IM2COL, B_UINT8)
+  TFHIP_CASE(A_ROWMAJOR, B_ROWMAJOR, true)
+  TFHIP_CASE(A_ROWMAJOR, B_TRANSPOSED, true)
+  TFHIP_CASE(A_ROWMAJOR, B_UINT8, true)
+  TFHIP_CASE(A_TRANSPOSED, B_ROWMAJOR, true)
+  TFHIP_CASE(A_TRANSPOSED, B_TRANSPOSED, true)
+  TFHIP_CASE(A_ROWMAJOR, B_ROWMAJOR, false)
+  TFHIP_CASE(A_ROWMAJOR, B_UINT8, false)
+  TFHIP_CASE(A_IM2COL, B_ROWMAJOR, false)
+  TFHIP_CASE(A_IM2COL, B_UINT8, false)
 #undef TFHIP_CASE
   return ctx->fail(TFHIP_ENOTSUP, "matmul: operand layout combination not built "
                                   "(transposed A with quantised B)");
@@ -563,7 +607,7 @@ extern "C" int tfhip_matmul(tfhip_ctx* ctx, int64_t a, int64_t b, int64_t out, i
     return ctx->fail(TFHIP_ENOTSUP, "matmul: transposed quantised b is not built");
   p.a_vec = aligned16(p.A) && (p.lda % 4 == 0) && (p.strideA % 4 == 0);
   p.b_vec = aligned16(p.B) && (p.ldb % 4 == 0) && (p.strideB % 4 == 0);
-  return launch_gemm(ctx, p, batch, amode, bmode);
+  return launch_gemm(ctx, p, batch, amode, bmode, /*kblocked=*/true);
 }
 
 extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t out,
@@ -650,5 +694,5 @@ extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t o
     p.pt = ci->pad_top; p.pl = ci->pad_left;
     p.a_vec = aligned16(p.A) && (ci->in_c % 4 == 0);
   }
-  return launch_gemm(ctx, p, 1, amode, quant ? B_UINT8 : B_ROWMAJOR);
+  return launch_gemm(ctx, p, 1, amode, quant ? B_UINT8 : B_ROWMAJOR, /*kblocked=*/false);
 }

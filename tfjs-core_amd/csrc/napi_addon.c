@@ -1,0 +1,427 @@
+/*
+ * tfjs_hip.node — raw N-API binding of the C ABI in include/tfjs_hip.h.
+ *
+ * Deliberately thin: every exported function converts its JavaScript arguments to plain
+ * C values, calls the entry point of the same name in libtfjs_hip.so and turns a non-zero
+ * status into a thrown Error carrying tfhip_last_error().  Tensors never cross this
+ * boundary except in write() (TypedArray -> device) and read() (device -> TypedArray);
+ * kernels are addressed by integer data ids.  Plays the role of the Emscripten glue of
+ * the reference's WASM backend (tfjs-backend-wasm/src/backend_wasm.ts:166-187).
+ */
+#include <node_api.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "tfjs_hip.h"
+
+#define MAX_ARGS 18
+
+#define NAPI_OK(env, call)                                              \
+  do {                                                                  \
+    if ((call) != napi_ok) {                                            \
+      napi_throw_error((env), NULL, "tfjs_hip.node: N-API call failed: " #call); \
+      return NULL;                                                      \
+    }                                                                   \
+  } while (0)
+
+static napi_value throw_status(napi_env env, tfhip_ctx* ctx, int rc) {
+  const char* msg = tfhip_last_error(ctx);
+  char buf[640];
+  snprintf(buf, sizeof buf, "%s", (msg && msg[0]) ? msg : "hip backend call failed");
+  (void)rc;
+  napi_throw_error(env, NULL, buf);
+  return NULL;
+}
+
+static napi_value undefined(napi_env env) {
+  napi_value u;
+  napi_get_undefined(env, &u);
+  return u;
+}
+
+/* ---- argument helpers -------------------------------------------------------------- */
+static int get_args(napi_env env, napi_callback_info info, size_t want, napi_value* argv) {
+  size_t argc = MAX_ARGS;
+  if (napi_get_cb_info(env, info, &argc, argv, NULL, NULL) != napi_ok || argc < want) {
+    napi_throw_type_error(env, NULL, "tfjs_hip.node: wrong number of arguments");
+    return 0;
+  }
+  return 1;
+}
+
+static int arg_ctx(napi_env env, napi_value v, tfhip_ctx** out) {
+  void* p = NULL;
+  if (napi_get_value_external(env, v, &p) != napi_ok || !p) {
+    napi_throw_type_error(env, NULL, "tfjs_hip.node: first argument must be a context");
+    return 0;
+  }
+  *out = (tfhip_ctx*)p;
+  return 1;
+}
+
+static int arg_i64(napi_env env, napi_value v, int64_t* out) {
+  double d;
+  if (napi_get_value_double(env, v, &d) != napi_ok) {
+    napi_throw_type_error(env, NULL, "tfjs_hip.node: expected a number");
+    return 0;
+  }
+  *out = (int64_t)d;
+  return 1;
+}
+
+static int arg_int(napi_env env, napi_value v, int* out) {
+  int64_t t;
+  if (!arg_i64(env, v, &t)) return 0;
+  *out = (int)t;
+  return 1;
+}
+
+static int arg_f64(napi_env env, napi_value v, double* out) {
+  if (napi_get_value_double(env, v, out) != napi_ok) {
+    napi_throw_type_error(env, NULL, "tfjs_hip.node: expected a number");
+    return 0;
+  }
+  return 1;
+}
+
+/* Int32Array -> pointer + length */
+static int arg_i32_array(napi_env env, napi_value v, const int32_t** data, size_t* len) {
+  napi_typedarray_type type;
+  void* p;
+  if (napi_get_typedarray_info(env, v, &type, len, &p, NULL, NULL) != napi_ok ||
+      type != napi_int32_array) {
+    napi_throw_type_error(env, NULL, "tfjs_hip.node: expected an Int32Array");
+    return 0;
+  }
+  *data = (const int32_t*)p;
+  return 1;
+}
+
+/* any TypedArray -> pointer + byte length */
+static int arg_bytes(napi_env env, napi_value v, void** data, size_t* nbytes) {
+  napi_typedarray_type type;
+  size_t len;
+  if (napi_get_typedarray_info(env, v, &type, &len, data, NULL, NULL) != napi_ok) {
+    napi_throw_type_error(env, NULL, "tfjs_hip.node: expected a TypedArray");
+    return 0;
+  }
+  size_t w = 1;
+  switch (type) {
+    case napi_int8_array: case napi_uint8_array: case napi_uint8_clamped_array: w = 1; break;
+    case napi_int16_array: case napi_uint16_array: w = 2; break;
+    case napi_int32_array: case napi_uint32_array: case napi_float32_array: w = 4; break;
+    default: w = 8; break;
+  }
+  *nbytes = len * w;
+  return 1;
+}
+
+/* [scale, min] Float64Array(2) or null/undefined */
+static int arg_qparams(napi_env env, napi_value v, tfhip_qparams* q, const tfhip_qparams** out) {
+  napi_valuetype t;
+  napi_typeof(env, v, &t);
+  if (t == napi_undefined || t == napi_null) {
+    *out = NULL;
+    return 1;
+  }
+  napi_typedarray_type type;
+  size_t len;
+  void* p;
+  if (napi_get_typedarray_info(env, v, &type, &len, &p, NULL, NULL) != napi_ok ||
+      type != napi_float64_array || len != 2) {
+    napi_throw_type_error(env, NULL, "tfjs_hip.node: qparams must be a Float64Array(2)");
+    return 0;
+  }
+  q->scale = ((double*)p)[0];
+  q->min = ((double*)p)[1];
+  *out = q;
+  return 1;
+}
+
+static int arg_conv_info(napi_env env, napi_value v, tfhip_conv2d_info* ci) {
+  const int32_t* p;
+  size_t len;
+  if (!arg_i32_array(env, v, &p, &len)) return 0;
+  if (len * sizeof(int32_t) != sizeof(tfhip_conv2d_info)) {
+    napi_throw_type_error(env, NULL, "tfjs_hip.node: conv info must be an Int32Array(17)");
+    return 0;
+  }
+  memcpy(ci, p, sizeof *ci);
+  return 1;
+}
+
+#define ARGS(n)                                  \
+  napi_value argv[MAX_ARGS];                     \
+  tfhip_ctx* ctx;                                \
+  if (!get_args(env, info, (n), argv)) return NULL; \
+  if (!arg_ctx(env, argv[0], &ctx)) return NULL
+#define I64(i, name) int64_t name; if (!arg_i64(env, argv[i], &name)) return NULL
+#define INT(i, name) int name; if (!arg_int(env, argv[i], &name)) return NULL
+#define F64(i, name) double name; if (!arg_f64(env, argv[i], &name)) return NULL
+#define CHECK(rc) do { int rc_ = (rc); if (rc_) return throw_status(env, ctx, rc_); } while (0)
+
+/* ---- context / storage ------------------------------------------------------------- */
+/* Contexts are destroyed explicitly by backend.dispose() (KernelBackend.dispose,
+ * backend.ts:646); the external carries no finalizer so a context still referenced by
+ * queued work is never torn down by the garbage collector. */
+static napi_value js_init(napi_env env, napi_callback_info info) {
+  napi_value argv[MAX_ARGS];
+  if (!get_args(env, info, 1, argv)) return NULL;
+  int device;
+  if (!arg_int(env, argv[0], &device)) return NULL;
+  tfhip_ctx* ctx = NULL;
+  int rc = tfhip_init(device, &ctx);
+  if (rc) return throw_status(env, NULL, rc);
+  napi_value ext;
+  NAPI_OK(env, napi_create_external(env, ctx, NULL, NULL, &ext));
+  return ext;
+}
+
+static napi_value js_destroy(napi_env env, napi_callback_info info) {
+  ARGS(1);
+  tfhip_destroy(ctx);
+  return undefined(env);
+}
+
+static napi_value js_register(napi_env env, napi_callback_info info) {
+  ARGS(4);
+  I64(1, id);
+  const int32_t* shape; size_t rank;
+  if (!arg_i32_array(env, argv[2], &shape, &rank)) return NULL;
+  INT(3, dtype);
+  CHECK(tfhip_register(ctx, id, shape, (int)rank, dtype));
+  return undefined(env);
+}
+
+static napi_value js_write(napi_env env, napi_callback_info info) {
+  ARGS(3);
+  I64(1, id);
+  void* data; size_t nbytes;
+  if (!arg_bytes(env, argv[2], &data, &nbytes)) return NULL;
+  CHECK(tfhip_write(ctx, id, data, nbytes));
+  return undefined(env);
+}
+
+static napi_value js_read(napi_env env, napi_callback_info info) {
+  ARGS(3);
+  I64(1, id);
+  void* data; size_t nbytes;
+  if (!arg_bytes(env, argv[2], &data, &nbytes)) return NULL;
+  CHECK(tfhip_read(ctx, id, data, nbytes));
+  return argv[2];
+}
+
+static napi_value js_dispose(napi_env env, napi_callback_info info) {
+  ARGS(2);
+  I64(1, id);
+  CHECK(tfhip_dispose(ctx, id));
+  return undefined(env);
+}
+
+static napi_value js_mem_info(napi_env env, napi_callback_info info) {
+  ARGS(1);
+  size_t in_use, pooled, ids;
+  CHECK(tfhip_mem_info(ctx, &in_use, &pooled, &ids));
+  napi_value arr, v;
+  NAPI_OK(env, napi_create_array_with_length(env, 3, &arr));
+  napi_create_double(env, (double)in_use, &v); napi_set_element(env, arr, 0, v);
+  napi_create_double(env, (double)pooled, &v); napi_set_element(env, arr, 1, v);
+  napi_create_double(env, (double)ids, &v); napi_set_element(env, arr, 2, v);
+  return arr;
+}
+
+static napi_value js_sync(napi_env env, napi_callback_info info) {
+  ARGS(1);
+  CHECK(tfhip_sync(ctx));
+  return undefined(env);
+}
+
+static napi_value js_time_begin(napi_env env, napi_callback_info info) {
+  ARGS(1);
+  CHECK(tfhip_time_begin(ctx));
+  return undefined(env);
+}
+
+static napi_value js_time_end(napi_env env, napi_callback_info info) {
+  ARGS(1);
+  float ms = 0;
+  CHECK(tfhip_time_end(ctx, &ms));
+  napi_value v;
+  NAPI_OK(env, napi_create_double(env, ms, &v));
+  return v;
+}
+
+static napi_value js_last_kernel(napi_env env, napi_callback_info info) {
+  ARGS(1);
+  napi_value v;
+  NAPI_OK(env, napi_create_string_utf8(env, tfhip_last_kernel(ctx), NAPI_AUTO_LENGTH, &v));
+  return v;
+}
+
+/* ---- kernels ----------------------------------------------------------------------- */
+/* matmul(ctx, a, b, out, batch, m, n, k, tA, tB, bias, biasKind, act, prelu, preluKind, q) */
+static napi_value js_matmul(napi_env env, napi_callback_info info) {
+  ARGS(16);
+  I64(1, a); I64(2, b); I64(3, out);
+  INT(4, batch); INT(5, m); INT(6, n); INT(7, k); INT(8, ta); INT(9, tb);
+  I64(10, bias); INT(11, bias_kind); INT(12, act); I64(13, prelu); INT(14, prelu_kind);
+  tfhip_qparams q; const tfhip_qparams* qp;
+  if (!arg_qparams(env, argv[15], &q, &qp)) return NULL;
+  CHECK(tfhip_matmul(ctx, a, b, out, batch, m, n, k, ta, tb, bias, bias_kind, act, prelu,
+                     prelu_kind, qp));
+  return undefined(env);
+}
+
+/* conv2d(ctx, x, filter, out, info, bias, biasKind, act, prelu, preluKind, q) */
+static napi_value js_conv2d(napi_env env, napi_callback_info info) {
+  ARGS(11);
+  I64(1, x); I64(2, w); I64(3, out);
+  tfhip_conv2d_info ci;
+  if (!arg_conv_info(env, argv[4], &ci)) return NULL;
+  I64(5, bias); INT(6, bias_kind); INT(7, act); I64(8, prelu); INT(9, prelu_kind);
+  tfhip_qparams q; const tfhip_qparams* qp;
+  if (!arg_qparams(env, argv[10], &q, &qp)) return NULL;
+  CHECK(tfhip_conv2d(ctx, x, w, out, &ci, bias, bias_kind, act, prelu, prelu_kind, qp));
+  return undefined(env);
+}
+
+/* depthwiseConv2d(ctx, x, filter, out, info, bias, biasKind, act, q) */
+static napi_value js_depthwise(napi_env env, napi_callback_info info) {
+  ARGS(9);
+  I64(1, x); I64(2, w); I64(3, out);
+  tfhip_conv2d_info ci;
+  if (!arg_conv_info(env, argv[4], &ci)) return NULL;
+  I64(5, bias); INT(6, bias_kind); INT(7, act);
+  tfhip_qparams q; const tfhip_qparams* qp;
+  if (!arg_qparams(env, argv[8], &q, &qp)) return NULL;
+  CHECK(tfhip_depthwise_conv2d(ctx, x, w, out, &ci, bias, bias_kind, act, qp));
+  return undefined(env);
+}
+
+/* pool2d(ctx, x, out, info, kind) */
+static napi_value js_pool2d(napi_env env, napi_callback_info info) {
+  ARGS(5);
+  I64(1, x); I64(2, out);
+  tfhip_conv2d_info ci;
+  if (!arg_conv_info(env, argv[3], &ci)) return NULL;
+  INT(4, kind);
+  CHECK(tfhip_pool2d(ctx, x, out, &ci, kind));
+  return undefined(env);
+}
+
+/* binary(ctx, op, a, aShape, b, bShape, out) */
+static napi_value js_binary(napi_env env, napi_callback_info info) {
+  ARGS(7);
+  INT(1, op); I64(2, a);
+  const int32_t* as; size_t ar;
+  if (!arg_i32_array(env, argv[3], &as, &ar)) return NULL;
+  I64(4, b);
+  const int32_t* bs; size_t br;
+  if (!arg_i32_array(env, argv[5], &bs, &br)) return NULL;
+  I64(6, out);
+  CHECK(tfhip_binary(ctx, op, a, as, (int)ar, b, bs, (int)br, out));
+  return undefined(env);
+}
+
+/* unary(ctx, op, x, out, p0, p1) */
+static napi_value js_unary(napi_env env, napi_callback_info info) {
+  ARGS(6);
+  INT(1, op); I64(2, x); I64(3, out); F64(4, p0); F64(5, p1);
+  CHECK(tfhip_unary(ctx, op, x, out, (float)p0, (float)p1));
+  return undefined(env);
+}
+
+static napi_value js_cast(napi_env env, napi_callback_info info) {
+  ARGS(3);
+  I64(1, x); I64(2, out);
+  CHECK(tfhip_cast(ctx, x, out));
+  return undefined(env);
+}
+
+static napi_value js_copy(napi_env env, napi_callback_info info) {
+  ARGS(3);
+  I64(1, x); I64(2, out);
+  CHECK(tfhip_copy(ctx, x, out));
+  return undefined(env);
+}
+
+/* dequantize(ctx, x, out, q) */
+static napi_value js_dequantize(napi_env env, napi_callback_info info) {
+  ARGS(4);
+  I64(1, x); I64(2, out);
+  tfhip_qparams q; const tfhip_qparams* qp;
+  if (!arg_qparams(env, argv[3], &q, &qp)) return NULL;
+  CHECK(tfhip_dequantize(ctx, x, out, qp));
+  return undefined(env);
+}
+
+static napi_value js_fill(napi_env env, napi_callback_info info) {
+  ARGS(3);
+  I64(1, out); F64(2, value);
+  CHECK(tfhip_fill(ctx, out, value));
+  return undefined(env);
+}
+
+/* reduce(ctx, op, x, out, outer, inner) */
+static napi_value js_reduce(napi_env env, napi_callback_info info) {
+  ARGS(6);
+  INT(1, op); I64(2, x); I64(3, out); I64(4, outer); I64(5, inner);
+  CHECK(tfhip_reduce(ctx, op, x, out, outer, inner));
+  return undefined(env);
+}
+
+static napi_value js_softmax_rows(napi_env env, napi_callback_info info) {
+  ARGS(5);
+  I64(1, x); I64(2, out); I64(3, rows); I64(4, cols);
+  CHECK(tfhip_softmax_rows(ctx, x, out, rows, cols));
+  return undefined(env);
+}
+
+/* gather(ctx, x, indices, out, outer, axisDim, inner, nIndices) */
+static napi_value js_gather(napi_env env, napi_callback_info info) {
+  ARGS(8);
+  I64(1, x); I64(2, idx); I64(3, out); I64(4, outer); I64(5, axis_dim); I64(6, inner); I64(7, n);
+  CHECK(tfhip_gather(ctx, x, idx, out, outer, axis_dim, inner, n));
+  return undefined(env);
+}
+
+/* transpose(ctx, x, xShape, perm, out) */
+static napi_value js_transpose(napi_env env, napi_callback_info info) {
+  ARGS(5);
+  I64(1, x);
+  const int32_t* shape; size_t rank;
+  if (!arg_i32_array(env, argv[2], &shape, &rank)) return NULL;
+  const int32_t* perm; size_t plen;
+  if (!arg_i32_array(env, argv[3], &perm, &plen)) return NULL;
+  I64(4, out);
+  if (plen != rank) {
+    napi_throw_type_error(env, NULL, "tfjs_hip.node: perm and shape differ in length");
+    return NULL;
+  }
+  CHECK(tfhip_transpose(ctx, x, shape, (int)rank, perm, out));
+  return undefined(env);
+}
+
+static napi_value module_init(napi_env env, napi_value exports) {
+  static const struct { const char* name; napi_callback fn; } fns[] = {
+      {"init", js_init}, {"destroy", js_destroy}, {"register", js_register},
+      {"write", js_write}, {"read", js_read}, {"dispose", js_dispose},
+      {"memInfo", js_mem_info}, {"sync", js_sync}, {"timeBegin", js_time_begin},
+      {"timeEnd", js_time_end}, {"lastKernel", js_last_kernel}, {"matmul", js_matmul},
+      {"conv2d", js_conv2d}, {"depthwiseConv2d", js_depthwise}, {"pool2d", js_pool2d},
+      {"binary", js_binary}, {"unary", js_unary}, {"cast", js_cast}, {"copy", js_copy},
+      {"dequantize", js_dequantize}, {"fill", js_fill}, {"reduce", js_reduce},
+      {"softmaxRows", js_softmax_rows}, {"gather", js_gather}, {"transpose", js_transpose}};
+  for (size_t i = 0; i < sizeof fns / sizeof fns[0]; i++) {
+    napi_value f;
+    if (napi_create_function(env, fns[i].name, NAPI_AUTO_LENGTH, fns[i].fn, NULL, &f) != napi_ok ||
+        napi_set_named_property(env, exports, fns[i].name, f) != napi_ok) {
+      napi_throw_error(env, NULL, "tfjs_hip.node: could not export a function");
+      return NULL;
+    }
+  }
+  return exports;
+}
+
+NAPI_MODULE(NODE_GYP_MODULE_NAME, module_init)

@@ -39,7 +39,7 @@ struct tfhip_ctx {
   hipEvent_t ev_begin = nullptr, ev_end = nullptr;
   bool timing = false;
   std::unordered_map<int64_t, tfhip::Buf> bufs;
-  std::multimap<size_t, void*> pool;  // capacity -> free block
+  std::map<size_t, std::vector<void*>> pool;  // capacity -> free blocks, reused LIFO
   size_t in_use = 0, pooled = 0;
   std::string err;
   char last_kernel[96] = "";  // variant chosen by the last dense / image launch

@@ -1,0 +1,392 @@
+'use strict';
+// MathBackendHIP: the reference's KernelBackend (tfjs-core/src/backends/backend.ts:91-649)
+// on an AMD MI355X.  Every kernel method queues device work through the N-API addon
+// (tfjs_hip.node -> libtfjs_hip.so) and returns a device-resident Tensor immediately; only
+// write (host -> device), read/readSync (device -> host) and time wait for the GPU.
+// Storage follows the WASM backend's scheme: an integer handle per dataId
+// (tfjs-backend-wasm/src/backend_wasm.ts:35-51).  There is no CPU fallback: if the addon
+// or the device is missing the factory throws and the engine reports it.
+const path = require('path');
+const util = require('./util');
+const axis_util = require('./axis_util');
+const broadcast_util = require('./broadcast_util');
+const {DataStorage, KernelBackend} = require('./backend');
+const {Tensor} = require('./tensor');
+const {ENGINE} = require('./engine');
+const {ENV} = require('./environment');
+
+const DTYPE = {float32: 0, int32: 1, bool: 2, uint8q: 3};
+const ACT = {linear: 0, relu: 1, prelu: 2, relu6: 3};
+const BCAST = {NONE: 0, SCALAR: 1, COLUMN: 2, FULL: 3};
+const BINARY = {add: 0, sub: 1, mul: 2, div: 3, prelu: 4, maximum: 5, minimum: 6};
+const UNARY = {relu: 0, clip: 1, exp: 2, log: 3, neg: 4, abs: 5, sigmoid: 6, sqrt: 7, square: 8,
+               tanh: 9, rsqrt: 10};
+const REDUCE = {sum: 0, max: 1, min: 2, argMax: 3, argMin: 4};
+const POOL = {avg: 0, max: 1};
+
+let addon = null;
+function loadAddon() {
+  if (addon == null) {
+    try {
+      addon = require(path.join(__dirname, 'tfjs_hip.node'));
+    } catch (err) {
+      throw new Error('hip backend: the native addon tfjs_hip.node could not be loaded (' +
+                      err.message + '); build it with `python tfjs-core_amd/build.py`. ' +
+                      'There is no CPU fallback.');
+    }
+  }
+  return addon;
+}
+
+function typedArrayFor(code, n) {
+  if (code === DTYPE.float32) return new Float32Array(n);
+  if (code === DTYPE.int32) return new Int32Array(n);
+  return new Uint8Array(n);
+}
+
+function convInfoArray(ci) {
+  if (ci.dataFormat != null && ci.dataFormat !== 'channelsLast') {
+    throw new Error('hip backend: only NHWC (channelsLast) convolutions are implemented');
+  }
+  const p = ci.padInfo;
+  return Int32Array.from([
+    ci.batchSize, ci.inHeight, ci.inWidth, ci.inChannels, ci.outHeight, ci.outWidth,
+    ci.outChannels, ci.strideHeight, ci.strideWidth, ci.dilationHeight, ci.dilationWidth,
+    ci.filterHeight, ci.filterWidth, p.top, p.left, p.bottom, p.right
+  ]);
+}
+
+class MathBackendHIP extends KernelBackend {
+  constructor(device) {
+    super();
+    this.napi = loadAddon();
+    this.ctx = this.napi.init(device == null ? ENV.get('HIP_DEVICE') : device);
+    this.data = new DataStorage(this, ENGINE);
+    this.nextHandle = 1;
+    this.pendingReads = 0;
+  }
+
+  // ---- storage (backend.ts:33-44; CPU behaviour backend_cpu.ts:102-129, 199-254) ----
+  register(dataId, shape, dtype) {
+    if (this.data.has(dataId)) throw new Error('Data buffer is already registered');
+    const code = DTYPE[dtype];
+    if (code == null) throw new Error(`hip backend: dtype ${dtype} is not supported`);
+    const handle = this.nextHandle++;
+    this.napi.register(this.ctx, handle, Int32Array.from(shape), code);
+    this.data.set(dataId, {handle, code, size: util.sizeFromShape(shape)});
+  }
+
+  write(dataId, values) {
+    if (values == null) throw new Error('MathBackendHIP.write(): values can not be null');
+    const rec = this.data.get(dataId);
+    let arr = values;
+    const want = rec.code === DTYPE.float32 ? Float32Array :
+        rec.code === DTYPE.int32 ? Int32Array : Uint8Array;
+    if (!(arr instanceof want)) arr = want.from(arr);
+    this.napi.write(this.ctx, rec.handle, arr);
+  }
+
+  readSync(dataId) {
+    const rec = this.data.get(dataId);
+    return this.napi.read(this.ctx, rec.handle, typedArrayFor(rec.code, rec.size));
+  }
+
+  // The device queue is in order, so a read issued now sees every kernel queued before it;
+  // the copy itself completes inside the call and the promise resolves on the next tick.
+  read(dataId) {
+    try {
+      return Promise.resolve(this.readSync(dataId));
+    } catch (err) {
+      return Promise.reject(err);
+    }
+  }
+
+  disposeData(dataId) {
+    if (this.data.has(dataId)) {
+      this.napi.dispose(this.ctx, this.data.get(dataId).handle);
+      this.data.delete(dataId);
+    }
+  }
+
+  memory() {
+    const [inUse, pooled, ids] = this.napi.memInfo(this.ctx);
+    return {unreliable: false, numBytesInGPU: inUse, numBytesInGPUPool: pooled, numDeviceBuffers: ids};
+  }
+
+  // Event pair on the backend's stream around everything f() queues (backend.ts:27-31).
+  async time(f) {
+    this.napi.timeBegin(this.ctx);
+    let kernelMs;
+    try {
+      f();
+    } finally {
+      kernelMs = this.napi.timeEnd(this.ctx);
+    }
+    return {kernelMs, getExtraProfileInfo: () => this.napi.lastKernel(this.ctx)};
+  }
+
+  sync() { this.napi.sync(this.ctx); }
+  lastKernel() { return this.napi.lastKernel(this.ctx); }
+  floatPrecision() { return 32; }
+
+  dispose() {
+    if (this.ctx != null) {
+      this.napi.destroy(this.ctx);
+      this.ctx = null;
+    }
+  }
+
+  fromPixels() {
+    throw new Error('fromPixels is a browser-only entry point; not available in the hip backend');
+  }
+
+  // ---- helpers ----
+  h(t) { return this.data.get(t.dataId).handle; }
+  storageCode(t) { return this.data.get(t.dataId).code; }
+  out(shape, dtype) { return Tensor.make(shape, {}, dtype || 'float32', this); }
+  q(t) { return t.quantization ? Float64Array.of(t.quantization.scale, t.quantization.min) : null; }
+
+  // Output of a pure data-movement kernel: x's dtype over x's stored element type.
+  outLikeStorage(shape, x) {
+    const code = this.storageCode(x);
+    const name = Object.keys(DTYPE).filter(k => DTYPE[k] === code)[0];
+    return new Tensor(shape, x.dtype, null, null, this, name);
+  }
+
+  // Layout of a bias / prelu operand against the result (null = not fusable).
+  epilogueKind(operand, outShape) {
+    if (operand == null) return BCAST.NONE;
+    if (!ENV.get('HIP_FUSE_EPILOGUE')) return null;
+    const n = outShape[outShape.length - 1];
+    if (operand.size === 1) return BCAST.SCALAR;
+    if (operand.size === n && operand.shape[operand.rank - 1] === n) return BCAST.COLUMN;
+    if (util.arraysEqual(operand.shape, outShape)) return BCAST.FULL;
+    return null;
+  }
+
+  mapActivation(x, activation, preluWeights) {
+    if (activation == null || activation === 'linear') return x;
+    if (activation === 'relu') return this.relu(x);
+    if (activation === 'prelu') return this.prelu(x, preluWeights);
+    if (activation === 'relu6') return this.clip(x, 0, 6);
+    throw new Error(`Activation ${activation} has not been implemented for the HIP backend.`);
+  }
+
+  checkActivation(activation) {
+    if (activation != null && ACT[activation] == null) {
+      throw new Error(`Activation ${activation} has not been implemented for the HIP backend.`);
+    }
+  }
+
+  // ---- dense contractions (backend.ts:128-138, 414-421) ----
+  batchMatMul(a, b, transposeA, transposeB) {
+    return this.fusedBatchMatMul({a, b, transposeA, transposeB});
+  }
+
+  fusedBatchMatMul({a, b, transposeA, transposeB, bias, activation, preluActivationWeights}) {
+    this.checkActivation(activation);
+    const batch = a.shape[0];
+    const k = transposeA ? a.shape[1] : a.shape[2];
+    const m = transposeA ? a.shape[2] : a.shape[1];
+    const n = transposeB ? b.shape[1] : b.shape[2];
+    const outShape = [batch, m, n];
+    const bk = this.epilogueKind(bias, outShape);
+    const pk = activation === 'prelu' ? this.epilogueKind(preluActivationWeights, outShape) : BCAST.NONE;
+    if (bk == null || pk == null || a.dtype !== 'float32') {
+      // the reference's own order: matmul, add, activation (backend_cpu.ts:542-555)
+      let r = this.matmulImpl(a, b, batch, m, n, k, transposeA, transposeB, null, 0, 'linear', null, 0);
+      if (a.dtype !== 'float32') r = this.cast(r, a.dtype);  // int32 x bool -> int32 (:511)
+      if (bias != null) r = this.add(r, bias);
+      return this.mapActivation(r, activation, preluActivationWeights);
+    }
+    return this.matmulImpl(a, b, batch, m, n, k, transposeA, transposeB, bias, bk,
+                           activation || 'linear', preluActivationWeights, pk);
+  }
+
+  matmulImpl(a, b, batch, m, n, k, tA, tB, bias, bk, activation, prelu, pk) {
+    const out = this.out([batch, m, n]);
+    this.napi.matmul(this.ctx, this.h(a), this.h(b), this.h(out), batch, m, n, k, tA ? 1 : 0,
+                     tB ? 1 : 0, bk ? this.h(bias) : -1, bk, ACT[activation],
+                     pk ? this.h(prelu) : -1, pk, this.q(b));
+    return out;
+  }
+
+  conv2d(x, filter, convInfo) {
+    return this.fusedConv2d(x, filter, convInfo);
+  }
+
+  fusedConv2d(x, filter, convInfo, bias, activation, preluActivationWeights) {
+    this.checkActivation(activation);
+    const outShape = convInfo.outShape;
+    const bk = this.epilogueKind(bias, outShape);
+    const pk = activation === 'prelu' ? this.epilogueKind(preluActivationWeights, outShape) : BCAST.NONE;
+    if (bk == null || pk == null) {
+      let r = this.fusedConv2d(x, filter, convInfo);
+      if (bias != null) r = this.add(r, bias);
+      return this.mapActivation(r, activation, preluActivationWeights);
+    }
+    const out = this.out(outShape);
+    this.napi.conv2d(this.ctx, this.h(x), this.h(filter), this.h(out), convInfoArray(convInfo),
+                     bk ? this.h(bias) : -1, bk, ACT[activation || 'linear'],
+                     pk ? this.h(preluActivationWeights) : -1, pk, this.q(filter));
+    return out;
+  }
+
+  // ---- memory-bound image kernels (backend.ts:431-434, 453-462) ----
+  depthwiseConv2D(x, filter, convInfo) {
+    return this.fusedDepthwiseConv2D(x, filter, convInfo);
+  }
+
+  // Extension of the plug-in API (feature-detected by the op wrapper): depthwiseConv2D with
+  // the add(bias) and relu / clip(0,6) that follow it folded into the same pass.
+  fusedDepthwiseConv2D(x, filter, convInfo, bias, activation) {
+    const outShape = convInfo.outShape;
+    const bk = this.epilogueKind(bias, outShape);
+    const foldable = activation == null || activation === 'linear' || activation === 'relu' ||
+        activation === 'relu6';
+    if (bk == null || bk === BCAST.FULL || !foldable) {
+      let r = this.fusedDepthwiseConv2D(x, filter, convInfo);
+      if (bias != null) r = this.add(r, bias);
+      return this.mapActivation(r, activation, null);
+    }
+    const out = this.out(outShape);
+    this.napi.depthwiseConv2d(this.ctx, this.h(x), this.h(filter), this.h(out),
+                              convInfoArray(convInfo), bk ? this.h(bias) : -1, bk,
+                              ACT[activation || 'linear'], this.q(filter));
+    return out;
+  }
+
+  pool(x, convInfo, kind) {
+    const out = this.out(convInfo.outShape);
+    this.napi.pool2d(this.ctx, this.h(x), this.h(out), convInfoArray(convInfo), POOL[kind]);
+    return out;
+  }
+  avgPool(x, convInfo) { return this.pool(x, convInfo, 'avg'); }
+  maxPool(x, convInfo) {
+    const r = this.pool(x, convInfo, 'max');
+    return x.dtype === 'float32' ? r : this.cast(r, x.dtype);
+  }
+
+  // ---- elementwise (backend.ts:160-177, 247, 258, 300-357, 392) ----
+  binary(op, a, b, outDtype) {
+    const outShape = broadcast_util.assertAndGetBroadcastShape(a.shape, b.shape);
+    const out = this.out(outShape, outDtype);
+    this.napi.binary(this.ctx, BINARY[op], this.h(a), Int32Array.from(a.shape), this.h(b),
+                     Int32Array.from(b.shape), this.h(out));
+    return out;
+  }
+  arithDtype(a, b) {
+    const dt = util.upcastType(a.dtype, b.dtype);
+    return dt === 'bool' ? 'int32' : dt;
+  }
+  add(a, b) { return this.binary('add', a, b, this.arithDtype(a, b)); }
+  subtract(a, b) { return this.binary('sub', a, b, this.arithDtype(a, b)); }
+  multiply(a, b) { return this.binary('mul', a, b, this.arithDtype(a, b)); }
+  realDivide(a, b) { return this.binary('div', a, b, 'float32'); }
+  prelu(x, a) { return this.binary('prelu', x, a, x.dtype === 'float32' ? 'float32' : 'int32'); }
+  maximum(a, b) { return this.binary('maximum', a, b, this.arithDtype(a, b)); }
+  minimum(a, b) { return this.binary('minimum', a, b, this.arithDtype(a, b)); }
+
+  unary(op, x, outDtype, p0, p1) {
+    const out = this.out(x.shape, outDtype || 'float32');
+    this.napi.unary(this.ctx, UNARY[op], this.h(x), this.h(out), p0 || 0, p1 || 0);
+    return out;
+  }
+  relu(x) { return this.unary('relu', x, x.dtype === 'float32' ? 'float32' : 'int32'); }
+  clip(x, min, max) { return this.unary('clip', x, 'float32', min, max); }
+  exp(x) { return this.unary('exp', x); }
+  log(x) { return this.unary('log', x); }
+  neg(x) { return this.unary('neg', x, x.dtype === 'float32' ? 'float32' : 'int32'); }
+  abs(x) { return this.unary('abs', x); }
+  sigmoid(x) { return this.unary('sigmoid', x); }
+  sqrt(x) { return this.unary('sqrt', x); }
+  square(x) { return this.unary('square', x); }
+  tanh(x) { return this.unary('tanh', x); }
+  rsqrt(x) { return this.unary('rsqrt', x); }
+
+  // castTensor (backends/backend_util.ts:34-71): loss-free casts alias the same dataId.
+  cast(x, dtype) {
+    if (dtype === x.dtype || (!util.hasEncodingLoss(x.dtype, dtype) && !x.quantization)) {
+      return Tensor.make(x.shape, {dataId: x.dataId}, dtype, this);
+    }
+    const out = this.out(x.shape, dtype);
+    this.napi.cast(this.ctx, this.h(x), this.h(out));
+    return out;
+  }
+  int(x) {
+    const out = this.out(x.shape, 'int32');
+    this.napi.cast(this.ctx, this.h(x), this.h(out));
+    return out;
+  }
+  dequantize(x) {
+    const out = this.out(x.shape, 'float32');
+    this.napi.dequantize(this.ctx, this.h(x), this.h(out), this.q(x));
+    return out;
+  }
+  clone(x) {
+    const out = this.outLikeStorage(x.shape, x);
+    this.napi.copy(this.ctx, this.h(x), this.h(out));
+    return out;
+  }
+  fill(shape, value, dtype) {
+    const out = this.out(shape, dtype || 'float32');
+    this.napi.fill(this.ctx, this.h(out), +value);
+    return out;
+  }
+  onesLike(x) { return this.fill(x.shape, 1, x.dtype); }
+  zerosLike(x) { return this.fill(x.shape, 0, x.dtype); }
+
+  // reshapeTensor (backends/backend_util.ts:79-82)
+  reshape(x, shape) {
+    const t = Tensor.make(shape, {dataId: x.dataId}, x.dtype, this);
+    t.quantization = x.quantization;
+    return t;
+  }
+
+  // ---- reductions over the innermost axes (backend.ts:183, 195-200, 244, 255) ----
+  reduce(op, x, axes, outDtype) {
+    axis_util.assertAxesAreInnerMostDims(op, axes, x.rank);
+    const [outShape, reduceShape] = axis_util.computeOutAndReduceShapes(x.shape, axes);
+    const out = this.out(outShape, outDtype);
+    this.napi.reduce(this.ctx, REDUCE[op], this.h(x), this.h(out), util.sizeFromShape(outShape),
+                     util.sizeFromShape(reduceShape));
+    return out;
+  }
+  sum(x, axes) { return this.reduce('sum', x, axes, util.upcastType(x.dtype, 'int32')); }
+  max(x, axes) { return this.reduce('max', x, axes, x.dtype === 'float32' ? 'float32' : 'int32'); }
+  min(x, axes) { return this.reduce('min', x, axes, x.dtype === 'float32' ? 'float32' : 'int32'); }
+  argMax(x, axis) { return this.reduce('argMax', x, [axis], 'int32'); }
+  argMin(x, axis) { return this.reduce('argMin', x, [axis], 'int32'); }
+
+  // One-pass row softmax (extension; the reference composes it from ten backend calls,
+  // ops/softmax.ts:45-79 + ops/reduction_ops.ts:56-74).
+  softmax(logits, dim) {
+    const cols = logits.shape[logits.rank - 1];
+    const rows = cols ? logits.size / cols : 0;
+    const out = this.out(logits.shape);
+    this.napi.softmaxRows(this.ctx, this.h(logits), this.h(out), rows, cols);
+    return out;
+  }
+
+  // ---- data movement (backend.ts:497, 501) ----
+  gather(x, indices, axis) {
+    const newShape = x.shape.slice();
+    newShape[axis] = indices.size;
+    const out = this.outLikeStorage(newShape, x);
+    const outer = util.sizeFromShape(x.shape.slice(0, axis));
+    const inner = util.sizeFromShape(x.shape.slice(axis + 1));
+    const idx = this.storageCode(indices) === DTYPE.int32 ? indices : this.int(indices);
+    this.napi.gather(this.ctx, this.h(x), this.h(idx), this.h(out), outer, x.shape[axis], inner,
+                     indices.size);
+    return out;
+  }
+
+  transpose(x, perm) {
+    const out = this.outLikeStorage(perm.map(p => x.shape[p]), x);
+    this.napi.transpose(this.ctx, this.h(x), Int32Array.from(x.shape), Int32Array.from(perm),
+                        this.h(out));
+    return out;
+  }
+}
+
+module.exports = {MathBackendHIP, loadAddon};

@@ -1,0 +1,44 @@
+'use strict';
+// Throughput of the MobileNetV1 forward pass through the JavaScript host:
+//   node bench_mobilenet.js <weights.bin> <manifest.json> <input.bin> <batch> <steps> <warmup>
+// Weights / input are read from files written by the Python harness (so both hosts run the
+// same bytes); the input is uploaded once, before the timed region.  Prints one JSON line.
+const fs = require('fs');
+const tf = require('./index.js');
+const mobilenet = require('./mobilenet.js');
+
+function toArrayBuffer(buf) {
+  return buf.buffer.slice(buf.byteOffset, buf.byteOffset + buf.byteLength);
+}
+
+async function main() {
+  const [wPath, mPath, xPath, batchArg, stepsArg, warmArg] = process.argv.slice(2);
+  const batch = +batchArg, steps = +stepsArg, warmup = +warmArg;
+  await tf.setBackend('hip');
+  const manifest = JSON.parse(fs.readFileSync(mPath, 'utf8'));
+  const w = tf.io.decodeWeightsToDevice(toArrayBuffer(fs.readFileSync(wPath)), manifest);
+  const xHost = new Float32Array(toArrayBuffer(fs.readFileSync(xPath)));
+  const x = tf.tensor(xHost, [batch, 224, 224, 3]);
+  const be = tf.backend();
+  const step = () => {
+    const out = mobilenet.forward(tf, w, x);
+    out.logits.dispose();
+    out.probs.dispose();
+  };
+  for (let i = 0; i < warmup; i++) step();
+  be.sync();
+  const t0 = process.hrtime.bigint();
+  const info = await tf.time(() => { for (let i = 0; i < steps; i++) step(); });
+  be.sync();
+  const wallMs = Number(process.hrtime.bigint() - t0) / 1e6;
+  // host-only cost of queueing one step (no waiting on the device in between)
+  const out = mobilenet.forward(tf, w, x);
+  const top = tf.argMax(out.logits, -1).dataSync();
+  console.log(JSON.stringify({
+    images_per_s: batch * steps / (wallMs / 1e3), ms_per_step: wallMs / steps,
+    gpu_ms_per_step_events: info.kernelMs / steps, batch, steps, warmup,
+    node: process.version, top1_first: top[0], tensors: tf.memory().numTensors
+  }));
+}
+
+main().catch(err => { console.error(err.stack || err); process.exit(1); });

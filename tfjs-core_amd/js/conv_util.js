@@ -1,0 +1,130 @@
+'use strict';
+// Shape math of convolution and pooling: the Conv2DInfo the backend receives.
+// After tfjs-core/src/ops/conv_util.ts:43-182 (Conv2DInfo, computePool2DInfo,
+// computeConv2DInfo), :296-320 (computeOutputShape2D), :338-357 (parseTupleParam),
+// :391-435 (getEffectiveFilterSize, getPadAndOutInfo), :499-554.
+const util = require('./util');
+
+function parseTupleParam(param) {
+  if (typeof param === 'number') return [param, param, param];
+  if (param.length === 2) return [param[0], param[1], 1];
+  return param;
+}
+
+function tupleValuesAreOne(param) {
+  const [a, b, c] = parseTupleParam(param);
+  return a === 1 && b === 1 && c === 1;
+}
+
+function eitherStridesOrDilationsAreOne(strides, dilations) {
+  return tupleValuesAreOne(strides) || tupleValuesAreOne(dilations);
+}
+
+function getEffectiveFilterSize(filterSize, dilation) {
+  if (dilation <= 1) return filterSize;
+  return filterSize + (filterSize - 1) * (dilation - 1);
+}
+
+function conditionalRound(value, roundingMode) {
+  if (!roundingMode) return value;
+  switch (roundingMode) {
+    case 'round': return Math.round(value);
+    case 'ceil': return Math.ceil(value);
+    case 'floor': return Math.floor(value);
+    default: throw new Error(`Unknown roundingMode ${roundingMode}`);
+  }
+}
+
+function computeOutputShape2D(inShape, fieldSize, stride, zeroPad, roundingMode) {
+  const outputRows = conditionalRound((inShape[0] - fieldSize + 2 * zeroPad) / stride + 1, roundingMode);
+  util.assert(util.isInt(outputRows),
+              () => `The output # of rows (${outputRows}) must be an integer. ` +
+                  `Change the stride and/or zero pad parameters`);
+  const outputCols = conditionalRound((inShape[1] - fieldSize + 2 * zeroPad) / stride + 1, roundingMode);
+  util.assert(util.isInt(outputCols),
+              () => `The output # of columns (${outputCols}) must be an integer. ` +
+                  `Change the stride and/or zero pad parameters`);
+  return [outputRows, outputCols];
+}
+
+function getPadAndOutInfo(pad, inHeight, inWidth, strideHeight, strideWidth, filterHeight,
+                          filterWidth, roundingMode) {
+  let padInfo, outHeight, outWidth;
+  if (typeof pad === 'number') {
+    const padType = (pad === 0) ? 'VALID' : 'NUMBER';
+    padInfo = {top: pad, bottom: pad, left: pad, right: pad, type: padType};
+    const outShape = computeOutputShape2D([inHeight, inWidth], filterHeight, strideHeight, pad, roundingMode);
+    outHeight = outShape[0];
+    outWidth = outShape[1];
+  } else if (pad === 'same') {
+    outHeight = Math.ceil(inHeight / strideHeight);
+    outWidth = Math.ceil(inWidth / strideWidth);
+    const padAlongHeight = Math.max(0, (outHeight - 1) * strideHeight + filterHeight - inHeight);
+    const padAlongWidth = Math.max(0, (outWidth - 1) * strideWidth + filterWidth - inWidth);
+    const top = Math.floor(padAlongHeight / 2);
+    const left = Math.floor(padAlongWidth / 2);
+    padInfo = {top, bottom: padAlongHeight - top, left, right: padAlongWidth - left, type: 'SAME'};
+  } else if (pad === 'valid') {
+    padInfo = {top: 0, bottom: 0, left: 0, right: 0, type: 'VALID'};
+    outHeight = Math.ceil((inHeight - filterHeight + 1) / strideHeight);
+    outWidth = Math.ceil((inWidth - filterWidth + 1) / strideWidth);
+  } else {
+    throw Error(`Unknown padding parameter: ${pad}`);
+  }
+  return {padInfo, outHeight, outWidth};
+}
+
+function computeConv2DInfo(inShape, filterShape, strides, dilations, pad, roundingMode,
+                           depthwise, dataFormat) {
+  depthwise = depthwise || false;
+  dataFormat = dataFormat || 'channelsLast';
+  let batchSize, inHeight, inWidth, inChannels;
+  if (dataFormat === 'channelsLast') {
+    [batchSize, inHeight, inWidth, inChannels] = inShape;
+  } else if (dataFormat === 'channelsFirst') {
+    [batchSize, inChannels, inHeight, inWidth] = inShape;
+  } else {
+    throw new Error(`Unknown dataFormat ${dataFormat}`);
+  }
+  const filterHeight = filterShape[0], filterWidth = filterShape[1], filterChannels = filterShape[3];
+  const [strideHeight, strideWidth] = parseTupleParam(strides);
+  const [dilationHeight, dilationWidth] = parseTupleParam(dilations);
+  const effectiveFilterHeight = getEffectiveFilterSize(filterHeight, dilationHeight);
+  const effectiveFilterWidth = getEffectiveFilterSize(filterWidth, dilationWidth);
+  const {padInfo, outHeight, outWidth} = getPadAndOutInfo(
+      pad, inHeight, inWidth, strideHeight, strideWidth, effectiveFilterHeight,
+      effectiveFilterWidth, roundingMode);
+  const outChannels = depthwise ? filterChannels * inChannels : filterChannels;
+  const outShape = dataFormat === 'channelsFirst' ?
+      [batchSize, outChannels, outHeight, outWidth] : [batchSize, outHeight, outWidth, outChannels];
+  return {
+    batchSize, dataFormat, inHeight, inWidth, inChannels, outHeight, outWidth, outChannels,
+    padInfo, strideHeight, strideWidth, filterHeight, filterWidth, effectiveFilterHeight,
+    effectiveFilterWidth, dilationHeight, dilationWidth, inShape, outShape, filterShape
+  };
+}
+
+function computePool2DInfo(inShape, filterSize, strides, dilations, pad, roundingMode, dataFormat) {
+  dataFormat = dataFormat || 'channelsLast';
+  const [filterHeight, filterWidth] = parseTupleParam(filterSize);
+  let filterShape;
+  if (dataFormat === 'channelsLast') {
+    filterShape = [filterHeight, filterWidth, inShape[3], inShape[3]];
+  } else if (dataFormat === 'channelsFirst') {
+    filterShape = [filterHeight, filterWidth, inShape[1], inShape[1]];
+  } else {
+    throw new Error(`Unknown dataFormat ${dataFormat}`);
+  }
+  return computeConv2DInfo(inShape, filterShape, strides, dilations, pad, roundingMode, false, dataFormat);
+}
+
+function convertConv2DDataFormat(dataFormat) {
+  if (dataFormat === 'NHWC') return 'channelsLast';
+  if (dataFormat === 'NCHW') return 'channelsFirst';
+  throw new Error(`Unknown dataFormat ${dataFormat}`);
+}
+
+module.exports = {
+  parseTupleParam, tupleValuesAreOne, eitherStridesOrDilationsAreOne, getEffectiveFilterSize,
+  computeConv2DInfo, computePool2DInfo, convertConv2DDataFormat
+};

@@ -1,0 +1,328 @@
+'use strict';
+// Host-logic tests of the JavaScript side that need no GPU: shape math against the
+// reference's conv_util vectors, engine registry / scopes / reference counts / data
+// movement with storage-only test backends, flags, weight decoding.
+//   node test/host_test.js <path to tests/golden>
+// Test patterns follow tfjs-core/src/engine_test.ts:25-368, 452-609,
+// jasmine_util.ts:201-203 (TestKernelBackend) and io/io_utils_test.ts:468-494.
+const assert = require('assert');
+const fs = require('fs');
+const path = require('path');
+const tf = require('../index.js');
+const {Engine} = require('../engine.js');
+const {KernelBackend, DataStorage} = require('../backend.js');
+const {Tensor} = require('../tensor.js');
+
+const golden = process.argv[2] || path.join(__dirname, '..', '..', '..', 'tests', 'golden');
+const tests = [];
+const test = (name, fn) => tests.push({name, fn});
+
+// A backend that only stores typed arrays: enough for the engine, no kernels.
+class StorageBackend extends KernelBackend {
+  constructor() {
+    super();
+    this.data = new DataStorage(this, tf.engine());
+    this.disposed = 0;
+    this.live = 0;
+  }
+  register(dataId, shape, dtype) {
+    if (this.data.has(dataId)) throw new Error('Data buffer is already registered');
+    this.data.set(dataId, {dtype, values: null});
+    this.live++;
+  }
+  write(dataId, values) { this.data.get(dataId).values = values; }
+  readSync(dataId) { return this.data.get(dataId).values; }
+  async read(dataId) { return this.readSync(dataId); }
+  disposeData(dataId) {
+    if (this.data.has(dataId)) {
+      this.data.delete(dataId);
+      this.live--;
+      this.disposed++;
+    }
+  }
+  memory() { return {unreliable: true}; }
+  floatPrecision() { return 32; }
+  reshape(x, shape) { return Tensor.make(shape, {dataId: x.dataId}, x.dtype, this); }
+  cast(x, dtype) { return Tensor.make(x.shape, {dataId: x.dataId}, dtype, this); }
+  async time(f) { f(); return {kernelMs: 0}; }
+  dispose() {}
+}
+
+function quiet(fn) {
+  const w = console.warn;
+  const msgs = [];
+  console.warn = m => msgs.push(String(m));
+  try {
+    return {result: fn(), msgs};
+  } finally {
+    console.warn = w;
+  }
+}
+
+async function withBackend(name, backend, fn) {
+  tf.registerBackend(name, () => backend, 0);
+  const prev = tf.getBackend();
+  try {
+    await tf.setBackend(name);
+    await fn();
+  } finally {
+    tf.removeBackend(name);
+    if (prev && tf.findBackendFactory(prev)) tf.engine().backendName = prev;
+  }
+}
+
+test('conv_util vectors of the reference', () => {
+  const cases = JSON.parse(fs.readFileSync(path.join(golden, 'conv_util.json'), 'utf8')).cases;
+  const cu = tf.backend_util;
+  let checked = 0;
+  cases.forEach(c => {
+    const a = c.args.slice();
+    const call = () => c.fn === 'computePool2DInfo' ?
+        cu.computePool2DInfo(a[0], a[1], a[2], a[3], a[4], a[5]) :
+        cu.computeConv2DInfo(a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[7]);
+    if (c.throws) {
+      assert.throws(call, /must be an integer/);
+      return;
+    }
+    const info = call();
+    Object.keys(c.expect).forEach(p => {
+      const got = p.split('.').reduce((o, k) => o[k], info);
+      assert.deepStrictEqual(got, c.expect[p], `${c.title}: ${p}`);
+      checked++;
+    });
+  });
+  assert(checked > 100, 'too few expectations checked');
+});
+
+test('MobileNet stem: same padding on even input puts the pad at bottom/right', () => {
+  const ci = tf.backend_util.computeConv2DInfo([64, 224, 224, 3], [3, 3, 3, 32], 2, 1, 'same');
+  assert.deepStrictEqual(ci.outShape, [64, 112, 112, 32]);
+  assert.deepStrictEqual([ci.padInfo.top, ci.padInfo.bottom, ci.padInfo.left, ci.padInfo.right], [0, 1, 0, 1]);
+  const dw = tf.backend_util.computeConv2DInfo([1, 112, 112, 64], [3, 3, 64, 1], 2, 1, 'same', null, true);
+  assert.deepStrictEqual(dw.outShape, [1, 56, 56, 64]);
+});
+
+test('broadcast and axis helpers', () => {
+  const bu = tf.backend_util;
+  assert.deepStrictEqual(bu.assertAndGetBroadcastShape([2, 1], [1, 3]), [2, 3]);
+  assert.deepStrictEqual(bu.assertAndGetBroadcastShape([], [4]), [4]);
+  assert.throws(() => bu.assertAndGetBroadcastShape([2, 3], [2]), /could not be broadcast/);
+  assert.deepStrictEqual(bu.getBroadcastDims([1, 3], [2, 3]), [0]);
+  assert.deepStrictEqual(bu.getAxesPermutation([0], 3), [1, 2, 0]);
+  assert.strictEqual(bu.getAxesPermutation([2], 3), null);
+  assert.deepStrictEqual(bu.computeOutAndReduceShapes([2, 3, 4], [2]), [[2, 3], [4]]);
+  assert.deepStrictEqual(bu.expandShapeToKeepDim([2, 3], [2]), [2, 3, 1]);
+  assert.strictEqual(tf.util.upcastType('int32', 'bool'), 'int32');
+  assert.strictEqual(tf.util.hasEncodingLoss('int32', 'float32'), false);
+  assert.strictEqual(tf.util.hasEncodingLoss('float32', 'int32'), true);
+});
+
+test('registerBackend: duplicate name is refused with a warning', () => {
+  const e = new Engine();
+  assert.strictEqual(e.registerBackend('a', () => new StorageBackend()), true);
+  const {result, msgs} = quiet(() => e.registerBackend('a', () => new StorageBackend()));
+  assert.strictEqual(result, false);
+  assert(/already registered/.test(msgs[0]));
+});
+
+test('backend priority, failing factory falls back, sync init usable at once', () => {
+  const e = new Engine();
+  const good = new StorageBackend();
+  e.registerBackend('broken', () => { throw new Error('no device'); }, 5);
+  e.registerBackend('good', () => good, 1);
+  const {result} = quiet(() => e.backend);
+  assert.strictEqual(result, good);
+  assert.strictEqual(e.backendName, 'good');
+  assert.throws(() => e.setBackend('missing'), /not found in registry/);
+});
+
+test('async factory: backend getter throws until ready() resolves', async () => {
+  const be = new StorageBackend();
+  const factory = () => new Promise(r => setTimeout(() => r(be), 5));
+  const e0 = new Engine();
+  e0.registerBackend('async', factory, 1);
+  assert.throws(() => e0.backend, /has not yet been initialized/);
+  const e = new Engine();
+  e.registerBackend('async', factory, 1);
+  await e.ready();
+  assert.strictEqual(e.backend, be);
+  const e1 = new Engine();
+  e1.registerBackend('async', factory, 1);
+  assert.strictEqual(await e1.setBackend('async'), true);
+  assert.strictEqual(e1.backend, be);
+  // a rejected async factory reports false and the engine stays usable
+  const e2 = new Engine();
+  e2.registerBackend('rejects', () => Promise.reject(new Error('boom')), 2);
+  e2.registerBackend('ok', () => be, 1);
+  const w = console.warn;
+  console.warn = () => {};
+  try {
+    assert.strictEqual(await e2.setBackend('rejects'), false);
+    await e2.setBackend('ok');
+  } finally {
+    console.warn = w;
+  }
+  assert.strictEqual(e2.backend, be);
+});
+
+test('removeBackend disposes the instance and unsets the active backend', () => {
+  const e = new Engine();
+  let disposed = 0;
+  const be = new StorageBackend();
+  be.dispose = () => { disposed++; };
+  e.registerBackend('x', () => be, 1);
+  e.setBackend('x');
+  e.removeBackend('x');
+  assert.strictEqual(disposed, 1);
+  assert.strictEqual(e.backendName, null);
+  assert.throws(() => e.removeBackend('x'), /not found in registry/);
+});
+
+test('reference counts: aliases keep the buffer, tidy keeps results', async () => {
+  const be = new StorageBackend();
+  await withBackend('storage-test', be, async () => {
+    const before = tf.memory().numTensors;
+    const a = tf.tensor([1, 2, 3, 4]);
+    const b = tf.reshape(a, [2, 2]);
+    const c = tf.cast(a, 'float32');
+    assert.strictEqual(be.live, 1);
+    assert.strictEqual(tf.memory().numTensors, before + 3);
+    assert.strictEqual(tf.memory().numDataBuffers, 1);
+    assert.strictEqual(tf.memory().numBytes, 16);
+    a.dispose();
+    c.dispose();
+    assert.strictEqual(be.live, 1, 'aliased buffer must survive');
+    assert.deepStrictEqual(Array.from(b.dataSync()), [1, 2, 3, 4]);
+    b.dispose();
+    assert.strictEqual(be.live, 0);
+    assert.throws(() => b.dataSync(), /Tensor is disposed/);
+    b.dispose();  // disposing twice is harmless
+
+    let inner;
+    const kept = tf.tidy(() => {
+      inner = tf.tensor([5]);
+      tf.tensor([6]);
+      const k = tf.keep(tf.tensor([7]));
+      k.scratch = true;
+      return tf.tensor([8, 9]);
+    });
+    assert.strictEqual(inner.isDisposed, true);
+    assert.strictEqual(kept.isDisposed, false);
+    assert.strictEqual(be.live, 2, 'the result and the kept tensor remain');
+    assert.deepStrictEqual(await kept.data(), new Float32Array([8, 9]));
+    assert.deepStrictEqual(kept.arraySync(), [8, 9]);
+    // nested tidy: the result is re-tracked by the parent scope and dies with it
+    tf.tidy(() => { tf.tidy(() => tf.tensor([1])); });
+    assert.strictEqual(be.live, 2);
+    assert.throws(() => tf.tidy('name'), /provide a function/);
+  });
+});
+
+test('register twice / write null follow backend_cpu', async () => {
+  const be = new StorageBackend();
+  await withBackend('storage-test2', be, async () => {
+    const t = tf.tensor([1, 2]);
+    assert.throws(() => be.register(t.dataId, [2], 'float32'), /already registered/);
+    t.dispose();
+  });
+});
+
+test('moveData: a tensor made on another backend moves on first use', async () => {
+  const src = new StorageBackend(), dst = new StorageBackend();
+  tf.registerBackend('src-test', () => src, 0);
+  tf.registerBackend('dst-test', () => dst, 0);
+  try {
+    await tf.setBackend('src-test');
+    const t = tf.tensor([1, 2, 3]);
+    assert.strictEqual(src.live, 1);
+    await tf.setBackend('dst-test');
+    assert.deepStrictEqual(Array.from(dst.data.get(t.dataId).values), [1, 2, 3]);
+    assert.strictEqual(src.live, 0, 'data left the source backend');
+    assert.strictEqual(dst.live, 1);
+    assert.deepStrictEqual(Array.from(t.dataSync()), [1, 2, 3]);
+    t.dispose();
+    assert.strictEqual(dst.live, 0);
+  } finally {
+    tf.removeBackend('src-test');
+    tf.removeBackend('dst-test');
+  }
+});
+
+test('unimplemented kernels throw, as the base class promises', async () => {
+  const be = new StorageBackend();
+  await withBackend('storage-test3', be, async () => {
+    assert.throws(() => tf.matMul(tf.tensor([[1]]), tf.tensor([[1]])), /Not yet implemented/);
+    assert.strictEqual(tf.memory().numTensors >= 0, true);
+  });
+  assert.strictEqual(new KernelBackend().epsilon.call({floatPrecision: () => 32}), 1e-7);
+  assert.strictEqual(new KernelBackend().epsilon.call({floatPrecision: () => 16}), 1e-4);
+});
+
+test('op wrappers validate before touching the backend', async () => {
+  const be = new StorageBackend();
+  await withBackend('storage-test4', be, async () => {
+    const a = tf.tensor([[1, 2, 3], [4, 5, 6]]);
+    assert.throws(() => tf.matMul(a, a), /inner shapes \(3\) and \(2\)/);
+    assert.throws(() => tf.matMul(a, tf.tensor([1, 2, 3])), /same rank of at least 2/);
+    assert.throws(() => tf.add(a, tf.tensor([[1, 2], [3, 4]])), /could not be broadcast/);
+    assert.throws(() => tf.conv2d(tf.zeros ? tf.tensor(new Float32Array(48), [1, 4, 4, 3]) : null,
+                                  tf.tensor(new Float32Array(144), [3, 3, 2, 8]), 1, 'same'),
+                  /depth of input \(3\) must match input depth for filter 2/);
+    assert.throws(() => tf.conv2d(tf.tensor(new Float32Array(48), [1, 4, 4, 3]),
+                                  tf.tensor(new Float32Array(216), [3, 3, 3, 8]), 2, 'same', 'NHWC', 2),
+                  /Either strides or dilations must be 1/);
+    assert.throws(() => tf.clipByValue(a, 1, -1), /min \(1\) must be less than or equal to max/);
+    assert.throws(() => tf.softmax(a, 0), /non-last dimension/);
+    assert.throws(() => tf.tensor([1, 2, 3], [2, 2]), /should have 4 values but has 3/);
+    assert.throws(() => tf.transpose(a, [0]), /must match length of perm/);
+    assert.throws(() => tf.add(a, {}), /must be a Tensor or TensorLike/);
+  });
+});
+
+test('flags: lazy evaluation, set hook, unknown flag', () => {
+  const env = tf.ENV;
+  assert.strictEqual(env.getBool('DEBUG'), false);
+  assert.strictEqual(env.get('HIP_FUSE_EPILOGUE'), true);
+  assert.throws(() => env.set('NOPE', 1), /has not been registered/);
+  let hooked = null;
+  env.registerFlag('TEST_FLAG', () => 41, v => { hooked = v; });
+  assert.strictEqual(env.get('TEST_FLAG'), 41);
+  env.set('TEST_FLAG', 42);
+  assert.strictEqual(hooked, 42);
+});
+
+test('decodeWeights: uint8 affine quantisation (io_utils_test.ts:468-494)', async () => {
+  const be = new StorageBackend();
+  await withBackend('storage-test5', be, async () => {
+    const manifest = [
+      {name: 'w0', dtype: 'float32', shape: [3], quantization: {min: -1, scale: 0.1, dtype: 'uint8'}},
+      {name: 'w1', dtype: 'int32', shape: [3], quantization: {min: -1, scale: 0.1, dtype: 'uint8'}},
+      {name: 'w2', dtype: 'float32', shape: [2]}
+    ];
+    const buf = new ArrayBuffer(14);
+    new Uint8Array(buf).set([0, 48, 255, 0, 48, 255]);
+    new Uint8Array(buf).set(new Uint8Array(new Float32Array([1.5, -2]).buffer), 6);
+    const w = tf.io.decodeWeights(buf, manifest);
+    assert.deepStrictEqual(Array.from(w.w0.dataSync()), Array.from(new Float32Array([-1, 3.8, 24.5])));
+    assert.deepStrictEqual(Array.from(w.w1.dataSync()), [-1, 4, 25]);
+    assert.deepStrictEqual(Array.from(w.w2.dataSync()), [1.5, -2]);
+    assert.throws(() => tf.io.decodeWeights(buf, [{name: 'x', dtype: 'float32', shape: [1],
+                                                    quantization: {min: 0, scale: 1, dtype: 'int8'}}]),
+                  /unknown quantization dtype/);
+  });
+});
+
+(async () => {
+  let failed = 0;
+  for (const t of tests) {
+    try {
+      await t.fn();
+      console.log('ok   ' + t.name);
+    } catch (err) {
+      failed++;
+      console.log('FAIL ' + t.name + '\n' + (err.stack || err));
+    }
+  }
+  console.log(`${tests.length - failed} passed, ${failed} failed`);
+  process.exit(failed ? 1 : 0);
+})();

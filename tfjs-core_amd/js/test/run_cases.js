@@ -1,0 +1,120 @@
+'use strict';
+// Replays op cases written by the Python test harness on the hip backend through the
+// JavaScript host (tf.* -> engine -> MathBackendHIP -> N-API -> libtfjs_hip.so):
+//   node test/run_cases.js <dir>
+// <dir>/cases.json lists {name, op, attrs, inputs:{arg:{file,shape,dtype,quant}}}; every
+// result is written to <dir>/<name>.out.bin and described in <dir>/results.json.  The
+// harness compares them with the CPU oracle; nothing is checked here except that no tensor
+// is leaked.
+const fs = require('fs');
+const path = require('path');
+const tf = require('../index.js');
+const mobilenet = require('../mobilenet.js');
+
+const dir = process.argv[2];
+
+function toArrayBuffer(buf) {
+  return buf.buffer.slice(buf.byteOffset, buf.byteOffset + buf.byteLength);
+}
+
+function load(spec) {
+  const ab = toArrayBuffer(fs.readFileSync(path.join(dir, spec.file)));
+  if (spec.quant) return tf.quantizedTensor(new Uint8Array(ab), spec.shape, spec.quant.scale, spec.quant.min);
+  const arr = spec.dtype === 'float32' ? new Float32Array(ab) :
+      spec.dtype === 'int32' ? new Int32Array(ab) : new Uint8Array(ab);
+  return tf.tensor(arr, spec.shape, spec.dtype);
+}
+
+const OPS = {
+  matMul: (i, a) => tf.matMul(i.a, i.b, a.transposeA, a.transposeB),
+  fusedMatMul: (i, a) => tf.fused.matMul({
+    a: i.a, b: i.b, transposeA: a.transposeA, transposeB: a.transposeB, bias: i.bias,
+    activation: a.activation, preluActivationWeights: i.prelu}),
+  conv2d: (i, a) => tf.conv2d(i.x, i.filter, a.strides, a.pad, 'NHWC', a.dilations, a.dimRoundingMode),
+  fusedConv2d: (i, a) => tf.fused.conv2d({
+    x: i.x, filter: i.filter, strides: a.strides, pad: a.pad, dilations: a.dilations,
+    bias: i.bias, activation: a.activation, preluActivationWeights: i.prelu}),
+  depthwiseConv2d: (i, a) => tf.depthwiseConv2d(i.x, i.filter, a.strides, a.pad, 'NHWC', a.dilations),
+  fusedDepthwiseConv2d: (i, a) => tf.fused.depthwiseConv2d({
+    x: i.x, filter: i.filter, strides: a.strides, pad: a.pad, dilations: a.dilations,
+    bias: i.bias, activation: a.activation}),
+  unfusedRelu6Conv: (i, a) => tf.clipByValue(tf.add(tf.conv2d(i.x, i.filter, a.strides, a.pad), i.bias), 0, 6),
+  avgPool: (i, a) => tf.avgPool(i.x, a.filterSize, a.strides, a.pad, a.dimRoundingMode),
+  maxPool: (i, a) => tf.maxPool(i.x, a.filterSize, a.strides, a.pad, a.dimRoundingMode),
+  add: i => tf.add(i.a, i.b), sub: i => tf.sub(i.a, i.b), mul: i => tf.mul(i.a, i.b),
+  div: i => tf.div(i.a, i.b), maximum: i => tf.maximum(i.a, i.b), minimum: i => tf.minimum(i.a, i.b),
+  prelu: i => tf.prelu(i.x, i.alpha),
+  relu: i => tf.relu(i.x), exp: i => tf.exp(i.x), log: i => tf.log(i.x),
+  clipByValue: (i, a) => tf.clipByValue(i.x, a.min, a.max), relu6: i => tf.relu6(i.x),
+  sum: (i, a) => tf.sum(i.x, a.axis, a.keepDims), max: (i, a) => tf.max(i.x, a.axis, a.keepDims),
+  min: (i, a) => tf.min(i.x, a.axis, a.keepDims),
+  argMax: (i, a) => tf.argMax(i.x, a.axis), argMin: (i, a) => tf.argMin(i.x, a.axis),
+  softmax: i => tf.softmax(i.x), logSumExp: (i, a) => tf.logSumExp(i.x, a.axis, a.keepDims),
+  softmaxComposite: i => tf.exp(tf.sub(i.x, tf.logSumExp(i.x, [i.x.rank - 1], true))),
+  gather: (i, a) => tf.gather(i.x, i.indices, a.axis),
+  transpose: (i, a) => tf.transpose(i.x, a.perm),
+  cast: (i, a) => tf.cast(i.x, a.dtype),
+  chainMethods: i => i.x.reshape([i.x.size]).relu().mul(i.x.reshape([i.x.size])).sum(),
+};
+
+async function main() {
+  await tf.setBackend('hip');
+  const spec = JSON.parse(fs.readFileSync(path.join(dir, 'cases.json'), 'utf8'));
+  const results = {};
+  const base = tf.memory().numTensors;
+  for (const c of spec.cases) {
+    const entry = {};
+    try {
+      if (c.op === 'mobilenet') {
+        const manifest = JSON.parse(fs.readFileSync(path.join(dir, c.attrs.manifest), 'utf8'));
+        const wbuf = toArrayBuffer(fs.readFileSync(path.join(dir, c.attrs.weights)));
+        const w = c.attrs.onDevice ? tf.io.decodeWeightsToDevice(wbuf, manifest) : tf.io.decodeWeights(wbuf, manifest);
+        const x = load(c.inputs.x);
+        const out = mobilenet.forward(tf, w, x);
+        const logits = await out.logits.data();   // asynchronous read path
+        const top = tf.argMax(out.logits, -1);
+        fs.writeFileSync(path.join(dir, c.name + '.out.bin'), Buffer.from(logits.buffer));
+        fs.writeFileSync(path.join(dir, c.name + '.top.bin'), Buffer.from(top.dataSync().buffer));
+        entry.shape = out.logits.shape;
+        entry.dtype = out.logits.dtype;
+        entry.probSum = tf.tidy(() => Array.from(tf.sum(out.probs, -1).dataSync()));
+        tf.dispose([w, x, out, top]);
+      } else {
+        const inputs = {};
+        Object.keys(c.inputs).forEach(k => { inputs[k] = load(c.inputs[k]); });
+        const r = tf.tidy(() => OPS[c.op](inputs, c.attrs || {}));
+        const vals = r.dataSync();
+        fs.writeFileSync(path.join(dir, c.name + '.out.bin'),
+                         Buffer.from(vals.buffer, vals.byteOffset, vals.byteLength));
+        entry.shape = r.shape;
+        entry.dtype = r.dtype;
+        r.dispose();
+        tf.dispose(inputs);
+      }
+    } catch (err) {
+      entry.error = String(err.message || err);
+    }
+    entry.leaked = tf.memory().numTensors - base;
+    results[c.name] = entry;
+  }
+  // backend.time and DEBUG mode smoke (profiler downloads every kernel output)
+  const a = tf.tensor(new Float32Array(256 * 256).fill(1), [256, 256]);
+  const timing = await tf.time(() => tf.matMul(a, a).dispose());
+  const logs = [];
+  const origLog = console.log, origWarn = console.warn;
+  console.log = m => logs.push(String(m));
+  console.warn = () => {};
+  tf.ENV.set('DEBUG', true);
+  tf.matMul(a, a).dispose();
+  await new Promise(r => setTimeout(r, 10));
+  tf.ENV.set('DEBUG', false);
+  console.log = origLog;
+  console.warn = origWarn;
+  a.dispose();
+  const mem = tf.memory();
+  fs.writeFileSync(path.join(dir, 'results.json'), JSON.stringify({
+    results, kernelMs: timing.kernelMs, lastKernel: timing.getExtraProfileInfo(), debugLog: logs,
+    memory: mem, node: process.version}));
+}
+
+main().catch(err => { console.error(err.stack || err); process.exit(1); });
