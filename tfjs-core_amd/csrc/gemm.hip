@@ -17,6 +17,8 @@
 // k = r (low half) with k = 4+r (high half): a permutation of the summation order only.
 // Likewise lane j of accumulator tile tj owns column TN*j + tj, so a lane reads its TN B
 // values with one access and writes TN adjacent results.
+#include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
 #include "tfhip_internal.h"
@@ -26,6 +28,7 @@ namespace tfhip {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 enum { A_ROWMAJOR = 0, A_TRANSPOSED = 1, A_IM2COL = 2 };
 enum { B_ROWMAJOR = 0, B_TRANSPOSED = 1, B_UINT8 = 2 };
@@ -44,12 +47,32 @@ struct GemmArgs {
   // implicit-GEMM geometry (A_IM2COL): rows are (n, oh, ow), k is (kh, kw, c)
   int H, W, Cin, OH, OW, KH, KW, sh, sw, dh, dw, pt, pl;
   double qscale, qmin;
-  int tiles_m, tiles_n;
+  // schedule (see work_item)
+  int tiles_m, tiles_n, k_tiles, rounds, tail_tiles, splits, kt_per;
+  float* partials;  // [tail_tiles * splits][BM * BN] partial tiles when splits > 1
+  unsigned a_bytes, b_bytes;  // per-batch byte extents of A and B (buffer-load range check)
 };
 
 constexpr int BK = 16;
 constexpr int LDA_S = BK + 4;
 constexpr int TILES_PER_KBLOCK = 48 / BK;
+constexpr int NBUF = 2;  // LDS double buffer
+
+// Buffer descriptor over [base, base + bytes): loads through it return 0 for any offset at or
+// beyond `bytes`, which is how out-of-range items of a tile are zero-filled without a branch
+// or a select on the loaded value.  OOB_OFFSET is such an offset for every extent below 2 GiB.
+constexpr unsigned OOB_OFFSET = 0x80000000u;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+  // the base is the same for the whole workgroup: say so, or the descriptor lands in VGPRs
+  const unsigned long long b = reinterpret_cast<unsigned long long>(base);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+  void* ub = reinterpret_cast<void*>(((unsigned long long)hi << 32) | lo);
+  return __builtin_amdgcn_make_buffer_rsrc(ub, (short)0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ f32x4 buffer_load_f32x4(__amdgpu_buffer_rsrc_t r, unsigned byte_off) {
+  return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0));
+}
 
 // w = q*scale + min evaluated in double, rounded once (io/io_utils.ts:133-136).
 __device__ __forceinline__ float dequant(unsigned q, double scale, double mn) {
@@ -70,19 +93,33 @@ __device__ __forceinline__ float activate(float v, int act, float alpha) {
   }
 }
 
-// Workgroups are handed to the 8 XCDs round-robin by linear id; remap so that each XCD
-// (own L2) receives a contiguous run of tiles, i.e. neighbours that share A rows / B
-// columns hit the same L2.
-__device__ __forceinline__ int xcd_remap(int bid, int total) {
-  constexpr int XCDS = 8;
-  const int per = total / XCDS, rem = total % XCDS;
-  const int x = bid % XCDS, i = bid / XCDS;
-  // XCD x owns `per` tiles (+1 for the first `rem` XCDs)
-  const int start = x * per + (x < rem ? x : rem);
-  return start + i;
+// The work of one workgroup: a whole output tile, or (when tiles are split along K to fill
+// the machine) the k range [kt0, kt1) of one, written to a partial slot.
+struct WorkItem {
+  int tile;     // linear tile index over (batch, tile row, tile column); -1 = none
+  int kt0, kt1;
+  int slot;     // partial slot, -1 = finish the tile here
+};
+
+// Schedule: `rounds` is 0 in every plan the host makes today, so workgroup g takes k range
+// g % splits of tile g / splits (kt_per steps each); with splits == 1 that is tile g whole.
+// The rounds branch serves a grid smaller than the tile count, should a plan ask for one.
+__device__ __forceinline__ WorkItem work_item(const GemmArgs& p, int g, int G, int it) {
+  WorkItem w = {-1, 0, 0, -1};
+  if (it < p.rounds) {
+    w.tile = it * G + g;
+    w.kt1 = p.k_tiles;
+  } else if (it == p.rounds && g < p.tail_tiles * p.splits) {
+    w.tile = p.rounds * G + g / p.splits;
+    const int s = g % p.splits;
+    w.kt0 = s * p.kt_per;
+    w.kt1 = min(p.k_tiles, w.kt0 + p.kt_per);
+    if (p.splits > 1) w.slot = g;
+  }
+  return w;
 }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN, int AMODE, int BMODE, bool KBLOCKED>
+template <int WAVES_M, int WAVES_N, int TM, int TN, int AMODE, int BMODE, bool KBLOCKED, bool FAST>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmArgs p) {
   constexpr int THREADS = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 32;
@@ -93,64 +130,103 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   constexpr int A_PER = (A_ITEMS + THREADS - 1) / THREADS;
   constexpr int B_PER = (B_ITEMS + THREADS - 1) / THREADS;
 
-  __shared__ __attribute__((aligned(16))) float As[2][BM * LDA_S];
-  __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB_S];
+  __shared__ __attribute__((aligned(16))) float As[NBUF][BM * LDA_S];
+  __shared__ __attribute__((aligned(16))) float Bs[NBUF][BK * LDB_S];
 
   const int tid = threadIdx.x;
+  __builtin_assume(tid >= 0 && tid < THREADS);
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int l32 = lane & 31, g = lane >> 5;
+  const int G = gridDim.x;
+  const int wg = xcd_remap(blockIdx.x, G);
+  const int tiles_per_batch = p.tiles_m * p.tiles_n;
 
-  const int tile = xcd_remap(blockIdx.x, p.tiles_m * p.tiles_n);
-  const int bm0 = (tile / p.tiles_n) * BM;
-  const int bn0 = (tile % p.tiles_n) * BN;
-  const int batch = blockIdx.z;
-
-  const float* __restrict__ A = p.A + batch * p.strideA;
-  const float* __restrict__ Bf = static_cast<const float*>(p.B) + batch * p.strideB;
-  const unsigned char* __restrict__ Bq =
-      static_cast<const unsigned char*>(p.B) + batch * p.strideB;
-  float* __restrict__ C = p.C + batch * p.strideC;
-
-  // ---- per-thread description of the A items it stages (fixed over the K loop) ----
+  // ---- per-tile description of the A/B items this thread stages ----
   // A_ROWMAJOR / A_IM2COL: item = (row, k-quad); A_TRANSPOSED: item = (k, row-quad).
-  int a_row[A_PER], a_kq[A_PER];
-  long long a_base[A_PER];  // row-major: row*lda ; im2col: n*H*W*Cin
-  int a_ih0[A_PER], a_iw0[A_PER];
-  bool a_ok[A_PER];
+  struct Loader {
+    const float* A;
+    const float* Bf;
+    const unsigned char* Bq;
+    int bm0, bn0;
+    int a_row[A_PER], a_kq[A_PER];
+    long long a_base[A_PER];  // row-major: row*lda ; im2col: n*H*W*Cin
+    int a_ih0[A_PER], a_iw0[A_PER];
+    bool a_ok[A_PER];
+  };
+
+  auto setup = [&](Loader& L, int tile) {
+    const int batch = tile / tiles_per_batch;
+    const int t = tile - batch * tiles_per_batch;
+    L.bm0 = (t / p.tiles_n) * BM;
+    L.bn0 = (t % p.tiles_n) * BN;
+    L.A = p.A + batch * p.strideA;
+    L.Bf = static_cast<const float*>(p.B) + batch * p.strideB;
+    L.Bq = static_cast<const unsigned char*>(p.B) + batch * p.strideB;
 #pragma unroll
-  for (int i = 0; i < A_PER; i++) {
-    const int item = tid + i * THREADS;
-    a_ok[i] = item < A_ITEMS;
-    if (AMODE == A_TRANSPOSED) {
-      a_kq[i] = item / (BM / 4);           // k within the tile
-      a_row[i] = (item % (BM / 4)) * 4;    // first of 4 rows
-      a_base[i] = 0;
-    } else {
-      a_row[i] = item / (BK / 4);
-      a_kq[i] = (item % (BK / 4)) * 4;
-      const int m = bm0 + a_row[i];
-      if (m >= p.M) a_ok[i] = false;
-      if (AMODE == A_ROWMAJOR) {
-        a_base[i] = (long long)m * p.lda;
+    for (int i = 0; i < A_PER; i++) {
+      const int item = tid + i * THREADS;
+      L.a_ok[i] = item < A_ITEMS;
+      L.a_base[i] = 0;
+      L.a_ih0[i] = L.a_iw0[i] = 0;
+      if (AMODE == A_TRANSPOSED) {
+        L.a_kq[i] = item / (BM / 4);           // k within the tile
+        L.a_row[i] = (item % (BM / 4)) * 4;    // first of 4 rows
       } else {
-        const int ow = m % p.OW, t = m / p.OW;
-        const int oh = t % p.OH, n = t / p.OH;
-        a_base[i] = (long long)n * p.H * p.W * p.Cin;
-        a_ih0[i] = oh * p.sh - p.pt;
-        a_iw0[i] = ow * p.sw - p.pl;
+        L.a_row[i] = item / (BK / 4);
+        L.a_kq[i] = (item % (BK / 4)) * 4;
+        const int m = L.bm0 + L.a_row[i];
+        if (m >= p.M) L.a_ok[i] = false;
+        if (AMODE == A_ROWMAJOR) {
+          L.a_base[i] = (long long)m * p.lda;
+        } else {
+          const int ow = m % p.OW, r = m / p.OW;
+          const int oh = r % p.OH, n = r / p.OH;
+          L.a_base[i] = (long long)n * p.H * p.W * p.Cin;
+          L.a_ih0[i] = oh * p.sh - p.pt;
+          L.a_iw0[i] = ow * p.sw - p.pl;
+        }
       }
     }
-  }
+  };
 
-  auto load_a = [&](int k0, f32x4 (&reg)[A_PER]) {
+  // FAST: both operands allow aligned 16-byte accesses (K, N, Cin multiples of 4) and span
+  // less than 2 GiB per batch entry.  The loaders are then straight-line buffer loads with
+  // 32-bit offsets — an item that is out of range gets OOB_OFFSET and reads as zero — so the
+  // loads of a step are issued back to back and nothing touches their result until the
+  // matrix cores are done with the step.
+  __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b;
+  auto load_a = [&](const Loader& L, int k0, f32x4 (&reg)[A_PER]) {
+    if (FAST) {
+#pragma unroll
+      for (int i = 0; i < A_PER; i++) {
+        const int k = k0 + L.a_kq[i];
+        bool ok = L.a_ok[i] && k < p.K;
+        unsigned off;
+        if (AMODE == A_ROWMAJOR) {
+          off = (unsigned)L.a_base[i] + k;
+        } else if (AMODE == A_TRANSPOSED) {
+          const int m = L.bm0 + L.a_row[i];
+          ok = ok && m < p.M;  // M % 4 == 0: the quad is inside or outside as a whole
+          off = (unsigned)k * p.lda + m;
+        } else {
+          const int tap = k / p.Cin, c = k - tap * p.Cin;
+          const int kh = tap / p.KW, kw = tap - kh * p.KW;
+          const int ih = L.a_ih0[i] + kh * p.dh, iw = L.a_iw0[i] + kw * p.dw;
+          ok = ok && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+          off = (unsigned)L.a_base[i] + (unsigned)(ih * p.W + iw) * p.Cin + c;
+        }
+        reg[i] = buffer_load_f32x4(rsrc_a, ok ? off * 4u : OOB_OFFSET);
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < A_PER; i++) {
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
-      if (a_ok[i]) {
+      if (L.a_ok[i]) {
         if (AMODE == A_ROWMAJOR) {
-          const int k = k0 + a_kq[i];
-          const float* src = A + a_base[i] + k;
+          const int k = k0 + L.a_kq[i];
+          const float* src = L.A + L.a_base[i] + k;
           if (p.a_vec && k + 3 < p.K) {
             v = *reinterpret_cast<const f32x4*>(src);
           } else {
@@ -159,10 +235,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
               if (k + e < p.K) v[e] = src[e];
           }
         } else if (AMODE == A_TRANSPOSED) {
-          const int k = k0 + a_kq[i];
-          const int m = bm0 + a_row[i];
+          const int k = k0 + L.a_kq[i];
+          const int m = L.bm0 + L.a_row[i];
           if (k < p.K) {
-            const float* src = A + (long long)k * p.lda + m;
+            const float* src = L.A + (long long)k * p.lda + m;
             if (p.a_vec && m + 3 < p.M) {
               v = *reinterpret_cast<const f32x4*>(src);
             } else {
@@ -172,15 +248,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
             }
           }
         } else {  // A_IM2COL
-          const int k = k0 + a_kq[i];
+          const int k = k0 + L.a_kq[i];
           if (p.a_vec) {  // Cin % 4 == 0: the 4 elements share one filter tap
             if (k < p.K) {
               const int tap = k / p.Cin, c = k - tap * p.Cin;
               const int kh = tap / p.KW, kw = tap - kh * p.KW;
-              const int ih = a_ih0[i] + kh * p.dh, iw = a_iw0[i] + kw * p.dw;
+              const int ih = L.a_ih0[i] + kh * p.dh, iw = L.a_iw0[i] + kw * p.dw;
               if ((unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W)
                 v = *reinterpret_cast<const f32x4*>(
-                    A + a_base[i] + ((long long)ih * p.W + iw) * p.Cin + c);
+                    L.A + L.a_base[i] + ((long long)ih * p.W + iw) * p.Cin + c);
             }
           } else {
 #pragma unroll
@@ -189,9 +265,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
               if (ke < p.K) {
                 const int tap = ke / p.Cin, c = ke - tap * p.Cin;
                 const int kh = tap / p.KW, kw = tap - kh * p.KW;
-                const int ih = a_ih0[i] + kh * p.dh, iw = a_iw0[i] + kw * p.dw;
+                const int ih = L.a_ih0[i] + kh * p.dh, iw = L.a_iw0[i] + kw * p.dw;
                 if ((unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W)
-                  v[e] = A[a_base[i] + ((long long)ih * p.W + iw) * p.Cin + c];
+                  v[e] = L.A[L.a_base[i] + ((long long)ih * p.W + iw) * p.Cin + c];
               }
             }
           }
@@ -201,33 +277,62 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     }
   };
 
-  auto store_a = [&](float* as, const f32x4 (&reg)[A_PER]) {
+  auto store_a = [&](const Loader& L, float* as, const f32x4 (&reg)[A_PER]) {
 #pragma unroll
     for (int i = 0; i < A_PER; i++) {
       const int item = tid + i * THREADS;
       if (item < A_ITEMS) {
         if (AMODE == A_TRANSPOSED) {
 #pragma unroll
-          for (int e = 0; e < 4; e++) as[(a_row[i] + e) * LDA_S + a_kq[i]] = reg[i][e];
+          for (int e = 0; e < 4; e++) as[(L.a_row[i] + e) * LDA_S + L.a_kq[i]] = reg[i][e];
         } else {
-          *reinterpret_cast<f32x4*>(&as[a_row[i] * LDA_S + a_kq[i]]) = reg[i];
+          *reinterpret_cast<f32x4*>(&as[L.a_row[i] * LDA_S + L.a_kq[i]]) = reg[i];
         }
       }
     }
   };
 
   // B items: B_ROWMAJOR / B_UINT8: (k, col-quad); B_TRANSPOSED: (col, k-quad)
-  auto load_b = [&](int k0, f32x4 (&reg)[B_PER]) {
+  auto load_b = [&](const Loader& L, int k0, f32x4 (&reg)[B_PER]) {
+    if (FAST) {
+#pragma unroll
+      for (int i = 0; i < B_PER; i++) {
+        const int item = tid + i * THREADS;
+        int k, n;
+        unsigned off;
+        if (BMODE == B_TRANSPOSED) {
+          n = L.bn0 + item / (BK / 4);
+          k = k0 + (item % (BK / 4)) * 4;
+          off = (unsigned)n * p.ldb + k;
+        } else {
+          k = k0 + item / (BN / 4);
+          n = L.bn0 + (item % (BN / 4)) * 4;
+          off = (unsigned)k * p.ldb + n;
+        }
+        const bool ok = item < B_ITEMS && k < p.K && n < p.N;
+        if (BMODE == B_UINT8) {
+          const unsigned w =
+              __builtin_amdgcn_raw_buffer_load_b32(rsrc_b, (int)(ok ? off : OOB_OFFSET), 0, 0);
+          f32x4 v;
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] = dequant((w >> (8 * e)) & 0xffu, p.qscale, p.qmin);
+          reg[i] = ok ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+        } else {
+          reg[i] = buffer_load_f32x4(rsrc_b, ok ? off * 4u : OOB_OFFSET);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < B_PER; i++) {
       const int item = tid + i * THREADS;
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
       if (item < B_ITEMS) {
         if (BMODE == B_TRANSPOSED) {
-          const int n = bn0 + item / (BK / 4);
+          const int n = L.bn0 + item / (BK / 4);
           const int k = k0 + (item % (BK / 4)) * 4;
           if (n < p.N) {
-            const float* src = Bf + (long long)n * p.ldb + k;
+            const float* src = L.Bf + (long long)n * p.ldb + k;
             if (p.b_vec && k + 3 < p.K) {
               v = *reinterpret_cast<const f32x4*>(src);
             } else {
@@ -238,27 +343,27 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
           }
         } else {
           const int k = k0 + item / (BN / 4);
-          const int n = bn0 + (item % (BN / 4)) * 4;
+          const int n = L.bn0 + (item % (BN / 4)) * 4;
           if (k < p.K && n < p.N) {
             const long long off = (long long)k * p.ldb + n;
             if (BMODE == B_ROWMAJOR) {
               if (p.b_vec && n + 3 < p.N) {
-                v = *reinterpret_cast<const f32x4*>(Bf + off);
+                v = *reinterpret_cast<const f32x4*>(L.Bf + off);
               } else {
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                  if (n + e < p.N) v[e] = Bf[off + e];
+                  if (n + e < p.N) v[e] = L.Bf[off + e];
               }
             } else {  // B_UINT8
               if (p.b_vec && n + 3 < p.N) {
-                const unsigned w = *reinterpret_cast<const unsigned*>(Bq + off);
+                const unsigned w = *reinterpret_cast<const unsigned*>(L.Bq + off);
 #pragma unroll
                 for (int e = 0; e < 4; e++)
                   v[e] = dequant((w >> (8 * e)) & 0xffu, p.qscale, p.qmin);
               } else {
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                  if (n + e < p.N) v[e] = dequant(Bq[off + e], p.qscale, p.qmin);
+                  if (n + e < p.N) v[e] = dequant(L.Bq[off + e], p.qscale, p.qmin);
               }
             }
           }
@@ -285,11 +390,29 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     }
   };
 
+  Loader L;
+  const WorkItem cur = work_item(p, wg, G, 0);
+  if (cur.tile < 0) return;
+  setup(L, cur.tile);
+  const int n_steps = cur.kt1 - cur.kt0;
+  rsrc_a = make_rsrc(L.A, p.a_bytes);
+  rsrc_b = make_rsrc(BMODE == B_UINT8 ? (const void*)L.Bq : (const void*)L.Bf, p.b_bytes);
+
+  // Software pipeline: while the matrix cores work on step i out of LDS buffer i&1, the
+  // global loads of step i+1 are in flight into registers; they are parked in the other LDS
+  // buffer at the end of the step, and one barrier per step hands the buffers over.
+  f32x4 a_reg[A_PER], b_reg[B_PER];
+  load_a(L, cur.kt0 * BK, a_reg);
+  load_b(L, cur.kt0 * BK, b_reg);
+  store_a(L, As[0], a_reg);
+  store_b(Bs[0], b_reg);
+  __syncthreads();
+
   // KBLOCKED (matMul): two-level accumulation.  The matrix cores sum 48 consecutive k into
-  // `blk`, which is then added to `acc` — the block structure of the reference's matmul
-  // (backend_cpu.ts:83, 516-535: 48-wide k blocks, one float32 rounding per block).  It
-  // keeps float32 round-off from growing with K: partial sums stay small inside a block.
-  // Convolutions accumulate straight through, as the reference's conv2d does (:1601-1604).
+  // `blk` (its first MFMA starts from the inline zero), which is then added to `acc` — the
+  // block structure of the reference's matmul (backend_cpu.ts:83, 516-535: 48-wide k
+  // blocks, one float32 rounding per block).  It keeps float32 round-off from growing with
+  // K.  Convolutions accumulate straight through, as the reference conv does (:1601-1604).
   f32x16 acc[TM][TN], blk[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; i++)
@@ -301,34 +424,24 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
         blk[i][j][r] = 0.f;
       }
 
-  f32x4 a_reg[A_PER], b_reg[B_PER];
-  const int k_tiles = (p.K + BK - 1) / BK;
-
-  load_a(0, a_reg);
-  load_b(0, b_reg);
-  store_a(As[0], a_reg);
-  store_b(Bs[0], b_reg);
-  __syncthreads();
-
-  // One tile step: prefetch tile kt+1 into registers, run the matrix cores on tile kt out
-  // of LDS, park the prefetched tile in the other LDS buffer.  `fresh` (compile time) makes
-  // the first MFMA of each accumulator start from zero instead of from `blk`.
-  auto tile_step = [&](int kt, auto fresh_tag) {
+  auto step = [&](int i, int buf, auto fresh_tag) {
     constexpr bool fresh = decltype(fresh_tag)::value;
-    const int cur = kt & 1;
-    if (kt + 1 < k_tiles) {
-      load_a((kt + 1) * BK, a_reg);
-      load_b((kt + 1) * BK, b_reg);
+    if (FAST || i + 1 < n_steps) {
+      load_a(L, (cur.kt0 + i + 1) * BK, a_reg);
+      load_b(L, (cur.kt0 + i + 1) * BK, b_reg);
     }
-    const float* as = As[cur] + (wm * TM * 32 + l32) * LDA_S + g * 4;
-    const float* bs = Bs[cur] + g * 4 * LDB_S + wn * TN * 32 + TN * l32;
+    // keep the global loads ahead of the matrix-core work: left alone, the scheduler sinks
+    // them next to their LDS stores and their latency is paid in full every step
+    __builtin_amdgcn_sched_barrier(0);
+    const float* as = As[buf] + (wm * TM * 32 + l32) * LDA_S + g * 4;
+    const float* bs = Bs[buf] + g * 4 * LDB_S + wn * TN * 32 + TN * l32;
 #pragma unroll
     for (int kc = 0; kc < BK; kc += 8) {
       f32x4 a[TM];
       float b[4][TN];
 #pragma unroll
-      for (int i = 0; i < TM; i++)
-        a[i] = *reinterpret_cast<const f32x4*>(as + i * 32 * LDA_S + kc);
+      for (int ii = 0; ii < TM; ii++)
+        a[ii] = *reinterpret_cast<const f32x4*>(as + ii * 32 * LDA_S + kc);
 #pragma unroll
       for (int r = 0; r < 4; r++) {
         const float* src = bs + (kc + r) * LDB_S;
@@ -348,47 +461,75 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
 #pragma unroll
       for (int r = 0; r < 4; r++)
 #pragma unroll
-        for (int i = 0; i < TM; i++)
+        for (int ii = 0; ii < TM; ii++)
 #pragma unroll
           for (int j = 0; j < TN; j++) {
             if (fresh && kc == 0 && r == 0) {
               const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
                                    0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-              blk[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][r], b[r][j], zero, 0, 0, 0);
+              blk[ii][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ii][r], b[r][j], zero, 0, 0, 0);
             } else {
-              blk[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][r], b[r][j], blk[i][j], 0, 0, 0);
+              blk[ii][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ii][r], b[r][j], blk[ii][j], 0, 0, 0);
             }
           }
     }
-    if (kt + 1 < k_tiles) {
-      store_a(As[cur ^ 1], a_reg);
-      store_b(Bs[cur ^ 1], b_reg);
+    __builtin_amdgcn_sched_barrier(0);
+    if (FAST || i + 1 < n_steps) {
+      const int nb = buf == NBUF - 1 ? 0 : buf + 1;
+      store_a(L, As[nb], a_reg);
+      store_b(Bs[nb], b_reg);
     }
     __syncthreads();
   };
 
-  if (KBLOCKED) {
-    for (int kt = 0; kt < k_tiles; kt += TILES_PER_KBLOCK) {
-      tile_step(kt, std::true_type{});
-#pragma unroll
-      for (int t = 1; t < TILES_PER_KBLOCK; t++)
-        if (kt + t < k_tiles) tile_step(kt + t, std::false_type{});
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] += blk[i][j];
-    }
-  } else {
-    for (int kt = 0; kt < k_tiles; kt++) tile_step(kt, std::false_type{});
+  auto flush = [&]() {
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-      for (int j = 0; j < TN; j++) acc[i][j] = blk[i][j];
-  }
+      for (int j = 0; j < TN; j++) acc[i][j] += blk[i][j];
+  };
 
-  // ---- epilogue: bias, activation, store.  Accumulator register r of a 32x32 tile holds
-  // row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
+  int buf = 0;
+  if (KBLOCKED) {
+    for (int i = 0; i < n_steps; i += TILES_PER_KBLOCK) {
+      step(i, buf, std::true_type{});
+      buf ^= 1;
+#pragma unroll
+      for (int t = 1; t < TILES_PER_KBLOCK; t++)
+        if (i + t < n_steps) {
+          step(i + t, buf, std::false_type{});
+          buf ^= 1;
+        }
+      flush();
+    }
+  } else {
+    for (int i = 0; i < n_steps; i++) {
+      step(i, buf, std::false_type{});
+      buf ^= 1;
+    }
+  }
+  f32x16(&res)[TM][TN] = KBLOCKED ? acc : blk;
+
+  // ---- store.  Accumulator register r of a 32x32 tile holds row
+  // 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
+  const int bm0 = L.bm0, bn0 = L.bn0;
+  const int batch = cur.tile / tiles_per_batch;
   const int col0 = bn0 + wn * TN * 32 + TN * l32;
+  if (cur.slot >= 0) {
+    // partial sum of a k range: raw accumulators into the tile-shaped slot
+    float* slot = p.partials + (long long)cur.slot * (BM * BN);
+    const int lc = wn * TN * 32 + TN * l32;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int lr = wm * TM * 32 + i * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
+#pragma unroll
+        for (int j = 0; j < TN; j++) slot[lr * BN + lc + j] = res[i][j][r];
+      }
+    return;
+  }
+  float* __restrict__ C = p.C + batch * p.strideC;
   float bias_c[TN], alpha_c[TN];
 #pragma unroll
   for (int j = 0; j < TN; j++) {
@@ -413,7 +554,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       float out[TN];
 #pragma unroll
       for (int j = 0; j < TN; j++) {
-        float v = acc[i][j][r];
+        float v = res[i][j][r];
         const bool in = col0 + j < p.N;
         if (full_bias) {
           if (in) v += p.bias[batch * p.strideC + base + j];
@@ -443,6 +584,44 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   }
 }
 
+// Finishes the tiles that were split along K: adds the `splits` partial tiles in ascending
+// k order (fixed order, so the result does not depend on scheduling), then bias,
+// activation and store.  One thread per 4 columns of a tile row.
+__global__ void splitk_finish_kernel(const GemmArgs p, int BM, int BN, int first_tile) {
+  const int tiles_per_batch = p.tiles_m * p.tiles_n;
+  const int quads = BM * BN / 4;
+  const long long total = (long long)p.tail_tiles * quads;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long q = (long long)blockIdx.x * blockDim.x + threadIdx.x; q < total; q += stride) {
+    const int tt = (int)(q / quads);
+    const int e = (int)(q - (long long)tt * quads) * 4;
+    const int lr = e / BN, lc = e - lr * BN;
+    const int tile = first_tile + tt;
+    const int batch = tile / tiles_per_batch;
+    const int t = tile - batch * tiles_per_batch;
+    const int row = (t / p.tiles_n) * BM + lr;
+    const int col = (t % p.tiles_n) * BN + lc;
+    if (row >= p.M || col >= p.N) continue;
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    const float* src = p.partials + ((long long)tt * p.splits) * (BM * BN) + e;
+    for (int s = 0; s < p.splits; s++) v += *reinterpret_cast<const f32x4*>(src + (long long)s * (BM * BN));
+    const long long base = (long long)batch * p.strideC + (long long)row * p.N + col;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      if (col + j >= p.N) break;
+      float x = v[j];
+      if (p.bias_kind == TFHIP_BCAST_SCALAR) x += p.bias[0];
+      else if (p.bias_kind == TFHIP_BCAST_COLUMN) x += p.bias[col + j];
+      else if (p.bias_kind == TFHIP_BCAST_FULL) x += p.bias[base + j];
+      float al = 0.f;
+      if (p.prelu_kind == TFHIP_BCAST_SCALAR) al = p.prelu[0];
+      else if (p.prelu_kind == TFHIP_BCAST_COLUMN) al = p.prelu[col + j];
+      else if (p.prelu_kind == TFHIP_BCAST_FULL) al = p.prelu[base + j];
+      p.C[base + j] = activate(x, p.act, al);
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
@@ -452,54 +631,152 @@ struct TileCfg {
   static constexpr int BM = WM_ * TM_ * 32, BN = WN_ * TN_ * 32;
 };
 
-template <class T, int AMODE, int BMODE, bool KBLOCKED>
-static void launch_cfg(tfhip_ctx* ctx, GemmArgs& p, int batch) {
-  static const char* const a_names[] = {"rowmajor", "transposed", "im2col"};
-  static const char* const b_names[] = {"f32", "f32t", "u8"};
-  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "gemm_%dx%d_%s_%s%s", T::BM, T::BN,
-           a_names[AMODE], b_names[BMODE], KBLOCKED ? "_kb48" : "");
-  hipStream_t s = ctx->stream;
-  p.tiles_m = (p.M + T::BM - 1) / T::BM;
-  p.tiles_n = (p.N + T::BN - 1) / T::BN;
-  dim3 grid(p.tiles_m * p.tiles_n, 1, batch);
-  hipLaunchKernelGGL((gemm_kernel<T::WM, T::WN, T::TM, T::TN, AMODE, BMODE, KBLOCKED>), grid,
-                     dim3(T::WM * T::WN * 64), 0, s, p);
+// How one tile shape would run a problem: grid, split along K, and a cost in units of MFMA
+// work on the busiest CU (larger tiles do the same flops with less LDS traffic).
+struct Plan {
+  int grid = 0, rounds = 0, tail_tiles = 0, splits = 1, kt_per = 0, tiles_m = 0, tiles_n = 0;
+  double cost = 0;
+};
+
+static Plan make_plan(const GemmArgs& p, int batch, int bm, int bn, int resident, int cus,
+                      double efficiency, bool kblocked) {
+  Plan pl;
+  pl.tiles_m = (int)ceil_div(p.M, bm);
+  pl.tiles_n = (int)ceil_div(p.N, bn);
+  const long long tiles = (long long)pl.tiles_m * pl.tiles_n * batch;
+  const int slots = cus * resident;
+  const int k_tiles = (int)ceil_div(p.K, BK);
+  // one workgroup per work item; tiles are split along K only when the whole problem has
+  // fewer tiles than half the machine's workgroup slots
+  pl.rounds = 0;
+  pl.tail_tiles = (int)tiles;
+  pl.splits = 1;
+  pl.kt_per = k_tiles;
+  if (pl.tail_tiles > 0 && pl.tail_tiles * 2 <= slots && k_tiles >= 8) {
+    // cut each tail tile into k ranges of at least 4 steps (whole 48-wide blocks for matMul)
+    const int unit = kblocked ? TILES_PER_KBLOCK : 1;
+    int want = slots / pl.tail_tiles;
+    int per = (int)ceil_div(k_tiles, want);
+    if (per < 4) per = 4;
+    per = (int)ceil_div(per, unit) * unit;
+    pl.kt_per = per;
+    pl.splits = (int)ceil_div(k_tiles, per);
+  }
+  pl.grid = pl.tail_tiles * pl.splits;
+  if (pl.grid < 1) pl.grid = 1;
+  // work on the busiest CU: its share of the workgroups, each one tile or one k range
+  const double per_wg = pl.splits > 1 ? (double)pl.kt_per / k_tiles : 1.0;
+  const int wgs_on_busiest_cu = (int)ceil_div(pl.grid, cus);
+  pl.cost = per_wg * wgs_on_busiest_cu * (double)bm * bn / efficiency;
+  if (pl.splits > 1) pl.cost += 0.15 * bm * bn;  // second pass over the partial tiles
+  return pl;
 }
 
-// Tile choice: the widest tile whose grid still gives every CU work; narrow-N tiles for
-// the early MobileNet layers (N = 32/64) so no matrix-core columns are wasted.
-template <int AMODE, int BMODE, bool KBLOCKED>
-static void launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
+template <class T, int AMODE, int BMODE, bool KBLOCKED, bool FAST>
+static int resident_blocks(tfhip_ctx* ctx) {
+  static int cached = 0;
+  if (!cached) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(
+            &n, gemm_kernel<T::WM, T::WN, T::TM, T::TN, AMODE, BMODE, KBLOCKED, FAST>,
+            T::WM * T::WN * 64, 0) != hipSuccess || n < 1) {
+      (void)hipGetLastError();
+      n = 1;
+    }
+    cached = n;
+  }
+  (void)ctx;
+  return cached;
+}
+
+template <class T, int AMODE, int BMODE, bool KBLOCKED, bool FAST>
+static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
+  static const char* const a_names[] = {"rowmajor", "transposed", "im2col"};
+  static const char* const b_names[] = {"f32", "f32t", "u8"};
+  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "gemm_%dx%d_%s_%s%s%s", T::BM, T::BN,
+           a_names[AMODE], b_names[BMODE], KBLOCKED ? "_kb48" : "", pl.splits > 1 ? "_splitk" : "");
+  if (!FAST) strncat(ctx->last_kernel, "_unaligned", sizeof ctx->last_kernel - strlen(ctx->last_kernel) - 1);
+  p.tiles_m = pl.tiles_m;
+  p.tiles_n = pl.tiles_n;
+  p.rounds = pl.rounds;
+  p.tail_tiles = pl.tail_tiles;
+  p.splits = pl.splits;
+  p.kt_per = pl.kt_per;
+  p.k_tiles = (int)ceil_div(p.K, BK);
+  Temp partials(ctx);
+  p.partials = nullptr;
+  if (pl.splits > 1) {
+    if (!partials.get((size_t)pl.tail_tiles * pl.splits * T::BM * T::BN * sizeof(float)))
+      return TFHIP_EDEVICE;
+    p.partials = static_cast<float*>(partials.ptr);
+  }
+  hipLaunchKernelGGL((gemm_kernel<T::WM, T::WN, T::TM, T::TN, AMODE, BMODE, KBLOCKED, FAST>),
+                     dim3(pl.grid), dim3(T::WM * T::WN * 64), 0, ctx->stream, p);
+  TFHIP_LAUNCH_CHECK(ctx);
+  if (pl.splits > 1) {
+    const long long quads = (long long)pl.tail_tiles * T::BM * T::BN / 4;
+    const long long blocks = ceil_div(quads, 256);
+    const long long cap = (long long)ctx->num_cus * 8;
+    hipLaunchKernelGGL(splitk_finish_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256),
+                       0, ctx->stream, p, T::BM, T::BN, pl.rounds * pl.grid);
+    TFHIP_LAUNCH_CHECK(ctx);
+  }
+  return TFHIP_OK;
+}
+
+// Tile choice: every shape is planned (grid, split along K) and the one with the least work
+// on the busiest CU wins.  Narrow-N tiles exist for the early MobileNet
+// layers (N = 32 / 64) so that no matrix-core columns are wasted.
+template <int AMODE, int BMODE, bool KBLOCKED, bool FAST>
+static int launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
   using Big = TileCfg<2, 2, 2, 2>;     // 128 x 128
   using Mid = TileCfg<2, 2, 2, 1>;     // 128 x 64
   using Thin = TileCfg<4, 1, 2, 1>;    // 256 x 32
   using Small = TileCfg<2, 2, 1, 1>;   // 64 x 64
-  const long long cus = ctx->num_cus;
-  auto blocks = [&](int bm, int bn) {
-    return (long long)ceil_div(p.M, bm) * ceil_div(p.N, bn) * batch;
-  };
-  if (p.N <= 32) {
-    launch_cfg<Thin, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
-  } else if (p.N <= 64) {
-    if (blocks(128, 64) >= cus) launch_cfg<Mid, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
-    else launch_cfg<Small, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
-  } else if (blocks(128, 128) >= 2 * cus) {
-    launch_cfg<Big, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
-  } else if (blocks(128, 64) >= 2 * cus) {
-    launch_cfg<Mid, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
-  } else {
-    launch_cfg<Small, AMODE, BMODE, KBLOCKED>(ctx, p, batch);
+  const int cus = ctx->num_cus;
+  Plan plans[4];
+  plans[0] = make_plan(p, batch, Big::BM, Big::BN, resident_blocks<Big, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 1.00, KBLOCKED);
+  plans[1] = make_plan(p, batch, Mid::BM, Mid::BN, resident_blocks<Mid, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.95, KBLOCKED);
+  plans[2] = make_plan(p, batch, Thin::BM, Thin::BN, resident_blocks<Thin, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.80, KBLOCKED);
+  plans[3] = make_plan(p, batch, Small::BM, Small::BN, resident_blocks<Small, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.85, KBLOCKED);
+  // columns beyond N are wasted matrix-core work: charge it
+  const int bns[4] = {Big::BN, Mid::BN, Thin::BN, Small::BN};
+  const int bms[4] = {Big::BM, Mid::BM, Thin::BM, Small::BM};
+  int best = -1;
+  for (int i = 0; i < 4; i++) {
+    const double useful = ((double)p.N / (ceil_div(p.N, bns[i]) * bns[i])) *
+                          ((double)p.M / (ceil_div(p.M, bms[i]) * bms[i]));
+    plans[i].cost /= useful;
+    if (best < 0 || plans[i].cost < plans[best].cost) best = i;
+  }
+  switch (best) {
+    case 0: return launch_cfg<Big, AMODE, BMODE, KBLOCKED, FAST>(ctx, p, plans[0]);
+    case 1: return launch_cfg<Mid, AMODE, BMODE, KBLOCKED, FAST>(ctx, p, plans[1]);
+    case 2: return launch_cfg<Thin, AMODE, BMODE, KBLOCKED, FAST>(ctx, p, plans[2]);
+    default: return launch_cfg<Small, AMODE, BMODE, KBLOCKED, FAST>(ctx, p, plans[3]);
   }
 }
 
 static int launch_gemm(tfhip_ctx* ctx, GemmArgs& p, int batch, int amode, int bmode,
                        bool kblocked) {
-#define TFHIP_CASE(AM, BM_, KB)                                  \
-  if (amode == AM && bmode == BM_ && kblocked == KB) {           \
-    launch_mode<AM, BM_, KB>(ctx, p, batch);                     \
-    TFHIP_LAUNCH_CHECK(ctx);                                     \
-    return TFHIP_OK;                                             \
-  }
+  // Byte extents of one batch entry of A and B, for the range check of the buffer loads.
+  long long a_el, b_el;
+  if (amode == A_ROWMAJOR) a_el = (long long)(p.M - 1) * p.lda + p.K;
+  else if (amode == A_TRANSPOSED) a_el = (long long)(p.K - 1) * p.lda + p.M;
+  else a_el = p.OH * p.OW > 0 ? (long long)(p.M / (p.OH * p.OW)) * p.H * p.W * p.Cin : 0;
+  if (bmode == B_TRANSPOSED) b_el = (long long)(p.N - 1) * p.ldb + p.K;
+  else b_el = (long long)(p.K - 1) * p.ldb + p.N;
+  const long long a_bytes = a_el * 4, b_bytes = b_el * (bmode == B_UINT8 ? 1 : 4);
+  const long long lim = 0x7fffffffLL;
+  // (an empty contraction has no readable operand bytes: keep it on the guarded path)
+  const bool fast = p.a_vec && p.b_vec && p.K > 0 && p.M > 0 && p.N > 0 && a_bytes <= lim &&
+                    b_bytes <= lim;
+  p.a_bytes = fast ? (unsigned)a_bytes : 0;
+  p.b_bytes = fast ? (unsigned)b_bytes : 0;
+#define TFHIP_CASE(AM, BM_, KB)                                \
+  if (amode == AM && bmode == BM_ && kblocked == KB)           \
+    return fast ? launch_mode<AM, BM_, KB, true>(ctx, p, batch) \
+                : launch_mode<AM, BM_, KB, false>(ctx, p, batch);
   TFHIP_CASE(A_ROWMAJOR, B_ROWMAJOR, true)
   TFHIP_CASE(A_ROWMAJOR, B_TRANSPOSED, true)
   TFHIP_CASE(A_ROWMAJOR, B_UINT8, true)

@@ -49,7 +49,9 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p) {
   constexpr int IH = (TH - 1) * S + 3, IW = (TW - 1) * S + 3;
   const tfhip_conv2d_info& ci = p.ci;
   const int64_t total = (int64_t)ci.batch * p.tiles_h * p.tiles_w * p.c4;
-  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  // contiguous image regions per XCD: the halo rows two patch rows share are then served
+  // by that XCD's L2 instead of being fetched once per XCD
+  const int64_t gid = (int64_t)xcd_remap(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x;
   if (gid >= total) return;
   const int cq = (int)(gid % p.c4);
   int64_t t = gid / p.c4;
@@ -298,8 +300,14 @@ extern "C" int tfhip_depthwise_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter,
                     (bias_kind != TFHIP_BCAST_COLUMN || aligned16(p.bias));
   if (fast) {
     p.c4 = ci->in_c / 4;
-    if (ci->stride_h == 1) launch_dw3x3<1, 2, 4>(ctx, p);
-    else launch_dw3x3<2, 1, 4>(ctx, p);
+    // Patch shapes picked by measurement on MI355X (fp32, batch 32-64): 2x8 patches for wide,
+    // deep rows, 2x2 elsewhere; stride 2 streams best with one output per lane.
+    if (ci->stride_h == 1) {
+      if (ci->out_w >= 112 && ci->in_c >= 128 && ci->out_w % 8 == 0) launch_dw3x3<1, 2, 8>(ctx, p);
+      else launch_dw3x3<1, 2, 2>(ctx, p);
+    } else {
+      launch_dw3x3<2, 1, 1>(ctx, p);
+    }
   } else {
     snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise_generic");
     const int64_t blocks = ceil_div(o_n, 256);

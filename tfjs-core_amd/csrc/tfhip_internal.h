@@ -94,4 +94,17 @@ int launch_convert(tfhip_ctx* ctx, const void* src, int src_dtype, void* dst, in
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its own
+// L2.  Remap the id so that every XCD receives one contiguous run of the work: neighbours
+// that share data (A rows / B columns of a GEMM, halo rows of a convolution) then meet in
+// the same L2 instead of each fetching its own copy over the fabric.
+__device__ __forceinline__ int xcd_remap(int bid, int total) {
+  constexpr int XCDS = 8;
+  const int per = total / XCDS, rem = total % XCDS;
+  const int x = bid % XCDS, i = bid / XCDS;
+  // XCD x owns `per` items (+1 for the first `rem` XCDs)
+  const int start = x * per + (x < rem ? x : rem);
+  return start + i;
+}
+
 }  // namespace tfhip
