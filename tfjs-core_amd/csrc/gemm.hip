@@ -56,7 +56,7 @@ struct GemmArgs {
 constexpr int BK = 16;
 constexpr int LDA_S = BK + 4;
 constexpr int TILES_PER_KBLOCK = 48 / BK;
-constexpr int NBUF = 2;  // LDS double buffer
+constexpr int NBUF = 2;  // LDS double buffer (the pipeline below relies on exactly two)
 
 // Buffer descriptor over [base, base + bytes): loads through it return 0 for any offset at or
 // beyond `bytes`, which is how out-of-range items of a tile are zero-filled without a branch
@@ -83,14 +83,23 @@ __device__ __forceinline__ float dequant(unsigned q, double scale, double mn) {
 }
 
 // Activation of the reference (backend_cpu.ts:50-62) with JavaScript's NaN behaviour:
-// Math.max(0, NaN) is NaN (:1191-1201), clip keeps NaN (:1265-1275).
-__device__ __forceinline__ float activate(float v, int act, float alpha) {
-  switch (act) {
-    case TFHIP_ACT_RELU: return (v > 0.f || v != v) ? v : 0.f;
-    case TFHIP_ACT_RELU6: return v > 6.f ? 6.f : (v < 0.f ? 0.f : v);
-    case TFHIP_ACT_PRELU: return v < 0.f ? alpha * v : v;
-    default: return v;
-  }
+// Math.max(0, NaN) is NaN (:1191-1201), clip keeps NaN (:1265-1275).  Branch-free: the kind
+// is unpacked once into flags that are the same for every lane.
+struct ActCfg {
+  bool linear, use_alpha;
+  float hi;
+};
+__device__ __forceinline__ ActCfg act_cfg(int act) {
+  ActCfg c;
+  c.linear = act == TFHIP_ACT_LINEAR;
+  c.use_alpha = act == TFHIP_ACT_PRELU;
+  c.hi = act == TFHIP_ACT_RELU6 ? 6.f : __builtin_inff();
+  return c;
+}
+__device__ __forceinline__ float activate(float v, const ActCfg& c, float alpha) {
+  const float neg = c.linear ? v : (c.use_alpha ? alpha * v : 0.f);
+  const float r = v < 0.f ? neg : v;  // NaN is not < 0: it passes through
+  return r > c.hi ? c.hi : r;
 }
 
 // The work of one workgroup: a whole output tile, or (when tiles are split along K to fill
@@ -398,16 +407,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   rsrc_a = make_rsrc(L.A, p.a_bytes);
   rsrc_b = make_rsrc(BMODE == B_UINT8 ? (const void*)L.Bq : (const void*)L.Bf, p.b_bytes);
 
-  // Software pipeline: while the matrix cores work on step i out of LDS buffer i&1, the
-  // global loads of step i+1 are in flight into registers; they are parked in the other LDS
-  // buffer at the end of the step, and one barrier per step hands the buffers over.
-  f32x4 a_reg[A_PER], b_reg[B_PER];
-  load_a(L, cur.kt0 * BK, a_reg);
-  load_b(L, cur.kt0 * BK, b_reg);
-  store_a(L, As[0], a_reg);
-  store_b(Bs[0], b_reg);
-  __syncthreads();
-
   // KBLOCKED (matMul): two-level accumulation.  The matrix cores sum 48 consecutive k into
   // `blk` (its first MFMA starts from the inline zero), which is then added to `acc` — the
   // block structure of the reference's matmul (backend_cpu.ts:83, 516-535: 48-wide k
@@ -424,62 +423,104 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
         blk[i][j][r] = 0.f;
       }
 
-  auto step = [&](int i, int buf, auto fresh_tag) {
-    constexpr bool fresh = decltype(fresh_tag)::value;
-    if (FAST || i + 1 < n_steps) {
-      load_a(L, (cur.kt0 + i + 1) * BK, a_reg);
-      load_b(L, (cur.kt0 + i + 1) * BK, b_reg);
-    }
-    // keep the global loads ahead of the matrix-core work: left alone, the scheduler sinks
-    // them next to their LDS stores and their latency is paid in full every step
-    __builtin_amdgcn_sched_barrier(0);
-    const float* as = As[buf] + (wm * TM * 32 + l32) * LDA_S + g * 4;
-    const float* bs = Bs[buf] + g * 4 * LDB_S + wn * TN * 32 + TN * l32;
+  // The operands of 8 consecutive k of a step, as one wavefront feeds them to the matrix
+  // cores: a[ii] = 4 k of this lane's row of accumulator row ii, b[r][j] = k r of its column.
+  struct Frag {
+    f32x4 a[TM];
+    float b[4][TN];
+  };
+  auto read_frag = [&](int buf, int kc, Frag& f) {
+    const float* as = As[buf] + (wm * TM * 32 + l32) * LDA_S + g * 4 + kc;
+    const float* bs = Bs[buf] + (g * 4 + kc) * LDB_S + wn * TN * 32 + TN * l32;
 #pragma unroll
-    for (int kc = 0; kc < BK; kc += 8) {
-      f32x4 a[TM];
-      float b[4][TN];
+    for (int ii = 0; ii < TM; ii++)
+      f.a[ii] = *reinterpret_cast<const f32x4*>(as + ii * 32 * LDA_S);
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const float* src = bs + r * LDB_S;
+      if (TN == 2) {
+        const f32x2 t = *reinterpret_cast<const f32x2*>(src);
+        f.b[r][0] = t[0];
+        f.b[r][TN - 1] = t[1];
+      } else if (TN == 4) {
+        const f32x4 t = *reinterpret_cast<const f32x4*>(src);
+#pragma unroll
+        for (int j = 0; j < TN; j++) f.b[r][j] = t[j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < TN; j++) f.b[r][j] = src[j];
+      }
+    }
+  };
+  // MFMAs r0..r1-1 of a fragment; with `fresh` the very first one starts `blk` from zero.
+  auto mfma_rows = [&](const Frag& f, int r0, int r1, bool fresh) {
+#pragma unroll
+    for (int r = r0; r < r1; r++)
 #pragma unroll
       for (int ii = 0; ii < TM; ii++)
-        a[ii] = *reinterpret_cast<const f32x4*>(as + ii * 32 * LDA_S + kc);
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
-        const float* src = bs + (kc + r) * LDB_S;
-        if (TN == 2) {
-          const f32x2 t = *reinterpret_cast<const f32x2*>(src);
-          b[r][0] = t[0];
-          b[r][TN - 1] = t[1];
-        } else if (TN == 4) {
-          const f32x4 t = *reinterpret_cast<const f32x4*>(src);
-#pragma unroll
-          for (int j = 0; j < TN; j++) b[r][j] = t[j];
-        } else {
-#pragma unroll
-          for (int j = 0; j < TN; j++) b[r][j] = src[j];
-        }
-      }
-#pragma unroll
-      for (int r = 0; r < 4; r++)
-#pragma unroll
-        for (int ii = 0; ii < TM; ii++)
-#pragma unroll
-          for (int j = 0; j < TN; j++) {
-            if (fresh && kc == 0 && r == 0) {
-              const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
-                                   0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-              blk[ii][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ii][r], b[r][j], zero, 0, 0, 0);
-            } else {
-              blk[ii][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[ii][r], b[r][j], blk[ii][j], 0, 0, 0);
-            }
+        for (int j = 0; j < TN; j++) {
+          if (fresh && r == r0) {
+            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
+                                 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            blk[ii][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[ii][r], f.b[r][j], zero, 0, 0, 0);
+          } else {
+            blk[ii][j] =
+                __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[ii][r], f.b[r][j], blk[ii][j], 0, 0, 0);
           }
-    }
+        }
+  };
+
+  // Software pipeline over the k steps (BK = 16 = two fragments of 8 k each).  In flight at
+  // any time: the matrix cores on tile i out of LDS buffer i&1, tile i+1 on its way from
+  // registers into the other LDS buffer, and the global loads of tile i+2 into registers.
+  // One step, for tile i:
+  //   read fragment 1 of tile i          (LDS latency hidden by the next MFMAs)
+  //   MFMAs of fragment 0, first half
+  //   park tile i+1 in the other LDS buffer; issue the global loads of tile i+2
+  //   MFMAs of fragment 0, second half
+  //   barrier                            (tile i+1 visible, buffer i&1 free next step)
+  //   read fragment 0 of tile i+1        (latency hidden by the MFMAs of fragment 1)
+  //   MFMAs of fragment 1
+  // sched_barrier(0) pins that order: left alone, the scheduler sinks the global loads next
+  // to their LDS stores and every step pays their latency in full.  With FAST loaders the
+  // loads past the last tile are range-checked to zero and parked in an unused buffer, so
+  // the loop body has no branches.
+  f32x4 a_reg[A_PER], b_reg[B_PER];
+  Frag f0, f1;
+  load_a(L, cur.kt0 * BK, a_reg);
+  load_b(L, cur.kt0 * BK, b_reg);
+  store_a(L, As[0], a_reg);
+  store_b(Bs[0], b_reg);
+  if (FAST || 1 < n_steps) {
+    load_a(L, (cur.kt0 + 1) * BK, a_reg);
+    load_b(L, (cur.kt0 + 1) * BK, b_reg);
+  }
+  __syncthreads();
+  read_frag(0, 0, f0);
+
+  auto step = [&](int i, int buf, auto fresh_tag) {
+    constexpr bool fresh = decltype(fresh_tag)::value;
+    read_frag(buf, 8, f1);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_rows(f0, 0, 2, fresh);
     __builtin_amdgcn_sched_barrier(0);
     if (FAST || i + 1 < n_steps) {
-      const int nb = buf == NBUF - 1 ? 0 : buf + 1;
-      store_a(L, As[nb], a_reg);
-      store_b(Bs[nb], b_reg);
+      store_a(L, As[buf ^ 1], a_reg);
+      store_b(Bs[buf ^ 1], b_reg);
     }
+    if (FAST || i + 2 < n_steps) {
+      load_a(L, (cur.kt0 + i + 2) * BK, a_reg);
+      load_b(L, (cur.kt0 + i + 2) * BK, b_reg);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_rows(f0, 2, 4, false);
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
+    read_frag(buf ^ 1, 0, f0);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_rows(f1, 0, 4, false);
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   auto flush = [&]() {
@@ -544,44 +585,49 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   const bool full_bias = p.bias_kind == TFHIP_BCAST_FULL;
   const bool full_alpha = p.prelu_kind == TFHIP_BCAST_FULL;
   const bool vec_store = (TN == 2 || TN == 4) && (p.N % TN == 0);
+  const ActCfg act = act_cfg(p.act);
+  const int row0 = bm0 + wm * TM * 32 + 4 * g;
+  // FULL: bias or prelu weights with one value per output element (rare) read them here
+  auto store = [&](auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
 #pragma unroll
-  for (int i = 0; i < TM; i++) {
+    for (int i = 0; i < TM; i++) {
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int row = bm0 + wm * TM * 32 + i * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
-      if (row >= p.M) continue;
-      const long long base = (long long)row * p.N + col0;
-      float out[TN];
+      for (int r = 0; r < 16; r++) {
+        const int row = row0 + i * 32 + 8 * (r >> 2) + (r & 3);
+        if (row >= p.M) continue;
+        const long long base = (long long)row * p.N + col0;
+        float out[TN];
 #pragma unroll
-      for (int j = 0; j < TN; j++) {
-        float v = res[i][j][r];
-        const bool in = col0 + j < p.N;
-        if (full_bias) {
-          if (in) v += p.bias[batch * p.strideC + base + j];
-        } else {
-          v += bias_c[j];
+        for (int j = 0; j < TN; j++) {
+          float bv = bias_c[j], al = alpha_c[j];
+          if (FULL) {
+            const bool in = col0 + j < p.N;
+            if (full_bias && in) bv = p.bias[batch * p.strideC + base + j];
+            if (full_alpha && in) al = p.prelu[batch * p.strideC + base + j];
+          }
+          out[j] = activate(res[i][j][r] + bv, act, al);
         }
-        float al = alpha_c[j];
-        if (full_alpha && in) al = p.prelu[batch * p.strideC + base + j];
-        out[j] = activate(v, p.act, al);
-      }
-      if (vec_store && col0 + TN - 1 < p.N) {
-        if (TN == 2) {
-          f32x2 t = {out[0], out[TN - 1]};
-          *reinterpret_cast<f32x2*>(C + base) = t;
+        if (vec_store && col0 + TN - 1 < p.N) {
+          if (TN == 2) {
+            f32x2 t = {out[0], out[TN - 1]};
+            *reinterpret_cast<f32x2*>(C + base) = t;
+          } else {
+            f32x4 t;
+#pragma unroll
+            for (int j = 0; j < TN; j++) t[j] = out[j];
+            *reinterpret_cast<f32x4*>(C + base) = t;
+          }
         } else {
-          f32x4 t;
 #pragma unroll
-          for (int j = 0; j < TN; j++) t[j] = out[j];
-          *reinterpret_cast<f32x4*>(C + base) = t;
+          for (int j = 0; j < TN; j++)
+            if (col0 + j < p.N) C[base + j] = out[j];
         }
-      } else {
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-          if (col0 + j < p.N) C[base + j] = out[j];
       }
     }
-  }
+  };
+  if (full_bias || full_alpha) store(std::true_type{});
+  else store(std::false_type{});
 }
 
 // Finishes the tiles that were split along K: adds the `splits` partial tiles in ascending
@@ -617,7 +663,188 @@ __global__ void splitk_finish_kernel(const GemmArgs p, int BM, int BN, int first
       if (p.prelu_kind == TFHIP_BCAST_SCALAR) al = p.prelu[0];
       else if (p.prelu_kind == TFHIP_BCAST_COLUMN) al = p.prelu[col + j];
       else if (p.prelu_kind == TFHIP_BCAST_FULL) al = p.prelu[base + j];
-      p.C[base + j] = activate(x, p.act, al);
+      p.C[base + j] = activate(x, act_cfg(p.act), al);
+    }
+  }
+}
+
+// Convolution with a short contraction (KH*KW*Cin <= 32, e.g. a 3x3 stem over RGB) and at
+// most 64 output channels.  The im2col rows of such a layer are 27 scattered, unaligned
+// floats per pixel, which the tiled kernel above can only gather element by element; here a
+// workgroup takes output rows (n, oh) in turn: it copies the KH input rows that the row reads into
+// LDS with coalesced loads (zeros where the padding is), and every wavefront then builds the
+// MFMA operand of 32 output pixels straight out of LDS.  The whole filter lives in
+// registers (k = 8q + 4*(lane/32) + e of MFMA group q, the same summation-order permutation
+// as above).  HBM traffic is the input once (rows shared by neighbouring output rows come out
+// of L2) plus the output once.
+template <int TN, bool QUANT>
+__global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int row_floats,
+                                                          int n_rows) {
+  extern __shared__ __attribute__((aligned(16))) float rows[];  // [KH][row_floats]
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  // this lane's 16 contraction indices k = 8q + 4g + e: LDS offset of (kh, kw, c), or -1 past
+  // K, and row k of the filter.  (kh, kw, c) is counted up with k, which keeps the walk in
+  // scalar registers; the filter loads are unconditional (clamped index) so that they are
+  // all in flight together.
+  int a_off[4][4];
+  float b[4][4][TN];
+  {
+    int kh = 0, kw = 0, c = 0;
+#pragma unroll
+    for (int k = 0; k < 32; k++) {
+      const int q = k >> 3, gk = (k >> 2) & 1, e = k & 3;
+      const bool k_ok = k < p.K;
+      const int off = k_ok ? kh * row_floats + kw * p.dw * p.Cin + c : -1;
+      if (g == gk) a_off[q][e] = off;
+      if (++c == p.Cin) {
+        c = 0;
+        if (++kw == p.KW) {
+          kw = 0;
+          kh++;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 4; q++)
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const int k = 8 * q + 4 * g + e, col = 32 * j + l32;
+        const bool ok = k < p.K && col < p.N;
+        const int at = ok ? k * p.N + col : 0;
+        float w;
+        if (QUANT) w = dequant(static_cast<const unsigned char*>(p.B)[at], p.qscale, p.qmin);
+        else w = static_cast<const float*>(p.B)[at];
+        b[q][e][j] = ok ? w : 0.f;
+      }
+  float bias_c[TN], alpha_c[TN];
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int col = 32 * j + l32;
+    bias_c[j] = alpha_c[j] = 0.f;
+    if (p.bias_kind == TFHIP_BCAST_SCALAR) bias_c[j] = p.bias[0];
+    if (p.bias_kind == TFHIP_BCAST_COLUMN && col < p.N) bias_c[j] = p.bias[col];
+    if (p.prelu_kind == TFHIP_BCAST_SCALAR) alpha_c[j] = p.prelu[0];
+    if (p.prelu_kind == TFHIP_BCAST_COLUMN && col < p.N) alpha_c[j] = p.prelu[col];
+  }
+
+  // Staging plan of this lane: elements i = tid + 256u of the [KH][row_floats] block, as
+  // (kh, offset in the input row); fixed for the lifetime of the workgroup.  A block of up to
+  // 2048 floats is one pass, and then the next output row's loads are issued before the
+  // current row is computed, so that their latency is hidden behind the matrix-core work.
+  const int row_in = p.W * p.Cin;
+  const int stage_n = p.KH * row_floats;
+  const bool one_pass = stage_n <= 256 * 8;
+  int st_kh[8], st_e[8];
+#pragma unroll
+  for (int u = 0; u < 8; u++) {
+    const int i = tid + u * 256;
+    const int kh = i / row_floats;
+    st_kh[u] = i < stage_n ? kh : -1;
+    st_e[u] = i - kh * row_floats - p.pl * p.Cin;
+  }
+  auto stage_load = [&](int row, float (&v)[8]) {
+    const int n = row / p.OH, oh = row - n * p.OH;
+    const int ih0 = oh * p.sh - p.pt;
+    const float* img = p.A + (long long)n * p.H * row_in;  // same for the whole workgroup
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const int ih = ih0 + st_kh[u] * p.dh;
+      const bool ok = st_kh[u] >= 0 && (unsigned)ih < (unsigned)p.H &&
+                      (unsigned)st_e[u] < (unsigned)row_in;
+      const int at = ok ? ih * row_in + st_e[u] : 0;
+      const float x = img[at];
+      v[u] = ok ? x : 0.f;
+    }
+  };
+  float v[8];
+  if (one_pass && (int)blockIdx.x < n_rows) stage_load(blockIdx.x, v);
+  for (int row = blockIdx.x; row < n_rows; row += gridDim.x) {
+    const int n = row / p.OH, oh = row - n * p.OH;
+    __syncthreads();  // the previous row's readers are done
+    if (one_pass) {
+#pragma unroll
+      for (int u = 0; u < 8; u++)
+        if (st_kh[u] >= 0) rows[tid + u * 256] = v[u];
+    } else {
+      for (int i0 = tid; i0 < stage_n; i0 += 256 * 8) {
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const int i = i0 + u * 256;
+          const int kh = i / row_floats, r = i - kh * row_floats;
+          const int ih = oh * p.sh - p.pt + kh * p.dh;
+          const int e = r - p.pl * p.Cin;
+          const bool ok = i < stage_n && (unsigned)ih < (unsigned)p.H && (unsigned)e < (unsigned)row_in;
+          const long long at = ok ? ((long long)n * p.H + ih) * row_in + e : 0;
+          const float x = p.A[at];
+          t[u] = ok ? x : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const int i = i0 + u * 256;
+          if (i < stage_n) rows[i] = t[u];
+        }
+      }
+    }
+    __syncthreads();
+    if (one_pass && row + (int)gridDim.x < n_rows) stage_load(row + gridDim.x, v);
+
+    const long long out_at = (((long long)n * p.OH + oh) * p.OW) * p.N;  // workgroup-uniform
+    float* __restrict__ crow = p.C + out_at;
+    const ActCfg act = act_cfg(p.act);
+    const float* bias_row = p.bias_kind == TFHIP_BCAST_FULL ? p.bias + out_at : nullptr;
+    const float* alpha_row = p.prelu_kind == TFHIP_BCAST_FULL ? p.prelu + out_at : nullptr;
+    for (int strip = wave; strip * 32 < p.OW; strip += 4) {
+      const int ow = min(strip * 32 + l32, p.OW - 1);  // clamped: lanes past the row compute a copy
+      const int base = ow * p.sw * p.Cin;
+      f32x16 acc[TN];
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        float a[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float x = rows[max(a_off[q][e], 0) + base];
+          a[e] = a_off[q][e] >= 0 ? x : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[q][e][j], acc[j], 0, 0, 0);
+      }
+      // accumulator register r holds pixel 8*(r/4) + 4*(lane/32) + r%4 of the strip
+      const int px0 = strip * 32 + 4 * g;
+      auto store = [&](auto full_tag) {
+        constexpr bool full = decltype(full_tag)::value;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int px = px0 + 8 * (r >> 2) + (r & 3);
+#pragma unroll
+          for (int j = 0; j < TN; j++) {
+            const int col = 32 * j + l32;
+            if (px < p.OW && col < p.N) {
+              const int at = px * p.N + col;
+              float bv = bias_c[j], al = alpha_c[j];
+              if (full) {
+                if (bias_row) bv = bias_row[at];
+                if (alpha_row) al = alpha_row[at];
+              }
+              crow[at] = activate(acc[j][r] + bv, act, al);
+            }
+          }
+        }
+      };
+      if (bias_row || alpha_row) store(std::true_type{});
+      else store(std::false_type{});
     }
   }
 }
@@ -970,6 +1197,41 @@ extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t o
     p.dh = ci->dilation_h; p.dw = ci->dilation_w;
     p.pt = ci->pad_top; p.pl = ci->pad_left;
     p.a_vec = aligned16(p.A) && (ci->in_c % 4 == 0);
+  }
+  if (amode == A_IM2COL && !p.a_vec && p.K >= 1 && p.K <= 32 && p.N <= 64 &&
+      (int64_t)ci->in_h * ci->in_w * ci->in_c < (1LL << 31) &&
+      (int64_t)ci->out_w * ci->out_c < (1LL << 31)) {
+    // columns the output row reads, from -pad_left on
+    const long long span = (long long)(ci->out_w - 1) * ci->stride_w +
+                           (long long)(ci->filter_w - 1) * ci->dilation_w + 1;
+    const long long row_floats = span * ci->in_c;
+    const long long lds = row_floats * ci->filter_h * (long long)sizeof(float);
+    if (lds <= 64 * 1024) {
+      const int n_rows = ci->batch * ci->out_h;
+      // one workgroup per resident slot: each walks its share of the output rows
+      auto launch = [&](auto kernel, const char* name) {
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, (size_t)lds) !=
+                hipSuccess || per_cu < 1) {
+          (void)hipGetLastError();
+          per_cu = 1;
+        }
+        const long long cap = (long long)ctx->num_cus * per_cu;
+        const unsigned grid = (unsigned)(n_rows < cap ? n_rows : cap);
+        snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "%s_%s", name, quant ? "u8" : "f32");
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), (size_t)lds, ctx->stream, p,
+                           (int)row_floats, n_rows);
+      };
+      if (p.N <= 32) {
+        if (quant) launch(conv_smallk_kernel<1, true>, "conv_smallk_n32");
+        else launch(conv_smallk_kernel<1, false>, "conv_smallk_n32");
+      } else {
+        if (quant) launch(conv_smallk_kernel<2, true>, "conv_smallk_n64");
+        else launch(conv_smallk_kernel<2, false>, "conv_smallk_n64");
+      }
+      TFHIP_LAUNCH_CHECK(ctx);
+      return TFHIP_OK;
+    }
   }
   return launch_gemm(ctx, p, 1, amode, quant ? B_UINT8 : B_ROWMAJOR, /*kblocked=*/false);
 }
