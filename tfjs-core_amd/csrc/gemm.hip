@@ -570,7 +570,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       }
     return;
   }
-  float* __restrict__ C = p.C + batch * p.strideC;
   float bias_c[TN], alpha_c[TN];
 #pragma unroll
   for (int j = 0; j < TN; j++) {
@@ -586,48 +585,56 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   const bool full_alpha = p.prelu_kind == TFHIP_BCAST_FULL;
   const bool vec_store = (TN == 2 || TN == 4) && (p.N % TN == 0);
   const ActCfg act = act_cfg(p.act);
-  const int row0 = bm0 + wm * TM * 32 + 4 * g;
-  // FULL: bias or prelu weights with one value per output element (rare) read them here
-  auto store = [&](auto full_tag) {
+  // FULL: bias or prelu weights with one value per output element (rare) are read here.
+  // INTERIOR: the whole tile lies inside the matrix, so no store needs a bounds check.
+  // Addresses are a tile base that is the same for the whole wavefront plus a 32-bit offset.
+  const int lrow0 = wm * TM * 32 + 4 * g;        // this lane's first row within the tile
+  const int lcol0 = wn * TN * 32 + TN * l32;     // its first column within the tile
+  const long long tile_at = batch * p.strideC + (long long)bm0 * p.N + bn0;
+  float* __restrict__ Ct = p.C + tile_at;
+  auto store = [&](auto full_tag, auto interior_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
+    constexpr bool INTERIOR = decltype(interior_tag)::value;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const int row = row0 + i * 32 + 8 * (r >> 2) + (r & 3);
-        if (row >= p.M) continue;
-        const long long base = (long long)row * p.N + col0;
+        const int lrow = lrow0 + i * 32 + 8 * (r >> 2) + (r & 3);
+        if (!INTERIOR && bm0 + lrow >= p.M) continue;
+        const int at = lrow * p.N + lcol0;
         float out[TN];
 #pragma unroll
         for (int j = 0; j < TN; j++) {
           float bv = bias_c[j], al = alpha_c[j];
           if (FULL) {
             const bool in = col0 + j < p.N;
-            if (full_bias && in) bv = p.bias[batch * p.strideC + base + j];
-            if (full_alpha && in) al = p.prelu[batch * p.strideC + base + j];
+            if (full_bias && in) bv = p.bias[tile_at + at + j];
+            if (full_alpha && in) al = p.prelu[tile_at + at + j];
           }
           out[j] = activate(res[i][j][r] + bv, act, al);
         }
-        if (vec_store && col0 + TN - 1 < p.N) {
+        if (vec_store && (INTERIOR || col0 + TN - 1 < p.N)) {
           if (TN == 2) {
             f32x2 t = {out[0], out[TN - 1]};
-            *reinterpret_cast<f32x2*>(C + base) = t;
+            *reinterpret_cast<f32x2*>(Ct + at) = t;
           } else {
             f32x4 t;
 #pragma unroll
             for (int j = 0; j < TN; j++) t[j] = out[j];
-            *reinterpret_cast<f32x4*>(C + base) = t;
+            *reinterpret_cast<f32x4*>(Ct + at) = t;
           }
         } else {
 #pragma unroll
           for (int j = 0; j < TN; j++)
-            if (col0 + j < p.N) C[base + j] = out[j];
+            if (INTERIOR || col0 + j < p.N) Ct[at + j] = out[j];
         }
       }
     }
   };
-  if (full_bias || full_alpha) store(std::true_type{});
-  else store(std::false_type{});
+  const bool interior = bm0 + BM <= p.M && bn0 + BN <= p.N;
+  if (full_bias || full_alpha) store(std::true_type{}, std::false_type{});
+  else if (interior) store(std::false_type{}, std::true_type{});
+  else store(std::false_type{}, std::false_type{});
 }
 
 // Finishes the tiles that were split along K: adds the `splits` partial tiles in ascending
@@ -986,6 +993,8 @@ static int launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
 
 static int launch_gemm(tfhip_ctx* ctx, GemmArgs& p, int batch, int amode, int bmode,
                        bool kblocked) {
+  if ((long long)p.N * 256 >= (1LL << 31))
+    return ctx->fail(TFHIP_ENOTSUP, "matmul/conv2d: more than 2^23 output columns");
   // Byte extents of one batch entry of A and B, for the range check of the buffer loads.
   long long a_el, b_el;
   if (amode == A_ROWMAJOR) a_el = (long long)(p.M - 1) * p.lda + p.K;
