@@ -486,32 +486,43 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   // to their LDS stores and every step pays their latency in full.  With FAST loaders the
   // loads past the last tile are range-checked to zero and parked in an unused buffer, so
   // the loop body has no branches.
-  f32x4 a_reg[A_PER], b_reg[B_PER];
+  // Staging registers.  Convolutions (not KBLOCKED) keep two sets and run the global loads
+  // three tiles ahead of the matrix cores instead of two: a step of a lone wavefront is
+  // shorter than a trip to HBM.
+  constexpr int AHEAD = KBLOCKED ? 2 : 3;
+  f32x4 a_reg[2][A_PER], b_reg[2][B_PER];
   Frag f0, f1;
-  load_a(L, cur.kt0 * BK, a_reg);
-  load_b(L, cur.kt0 * BK, b_reg);
-  store_a(L, As[0], a_reg);
-  store_b(Bs[0], b_reg);
+  load_a(L, cur.kt0 * BK, a_reg[0]);
+  load_b(L, cur.kt0 * BK, b_reg[0]);
+  store_a(L, As[0], a_reg[0]);
+  store_b(Bs[0], b_reg[0]);
+  // tile 1 goes to set 1 (set 0 when there is one set), tile 2 to set 0
+  constexpr int SET1 = AHEAD == 3 ? 1 : 0;
   if (FAST || 1 < n_steps) {
-    load_a(L, (cur.kt0 + 1) * BK, a_reg);
-    load_b(L, (cur.kt0 + 1) * BK, b_reg);
+    load_a(L, (cur.kt0 + 1) * BK, a_reg[SET1]);
+    load_b(L, (cur.kt0 + 1) * BK, b_reg[SET1]);
+  }
+  if (AHEAD == 3 && (FAST || 2 < n_steps)) {
+    load_a(L, (cur.kt0 + 2) * BK, a_reg[0]);
+    load_b(L, (cur.kt0 + 2) * BK, b_reg[0]);
   }
   __syncthreads();
   read_frag(0, 0, f0);
 
-  auto step = [&](int i, int buf, auto fresh_tag) {
+  // step i: `set` holds tile i+1 on entry and receives tile i+AHEAD
+  auto step = [&](int i, int buf, f32x4 (&ar)[A_PER], f32x4 (&br)[B_PER], auto fresh_tag) {
     constexpr bool fresh = decltype(fresh_tag)::value;
     read_frag(buf, 8, f1);
     __builtin_amdgcn_sched_barrier(0);
     mfma_rows(f0, 0, 2, fresh);
     __builtin_amdgcn_sched_barrier(0);
     if (FAST || i + 1 < n_steps) {
-      store_a(L, As[buf ^ 1], a_reg);
-      store_b(Bs[buf ^ 1], b_reg);
+      store_a(L, As[buf ^ 1], ar);
+      store_b(Bs[buf ^ 1], br);
     }
-    if (FAST || i + 2 < n_steps) {
-      load_a(L, (cur.kt0 + i + 2) * BK, a_reg);
-      load_b(L, (cur.kt0 + i + 2) * BK, b_reg);
+    if (FAST || i + AHEAD < n_steps) {
+      load_a(L, (cur.kt0 + i + AHEAD) * BK, ar);
+      load_b(L, (cur.kt0 + i + AHEAD) * BK, br);
     }
     __builtin_amdgcn_sched_barrier(0);
     mfma_rows(f0, 2, 4, false);
@@ -530,23 +541,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       for (int j = 0; j < TN; j++) acc[i][j] += blk[i][j];
   };
 
-  int buf = 0;
   if (KBLOCKED) {
+    int buf = 0;
     for (int i = 0; i < n_steps; i += TILES_PER_KBLOCK) {
-      step(i, buf, std::true_type{});
+      step(i, buf, a_reg[0], b_reg[0], std::true_type{});
       buf ^= 1;
 #pragma unroll
       for (int t = 1; t < TILES_PER_KBLOCK; t++)
         if (i + t < n_steps) {
-          step(i + t, buf, std::false_type{});
+          step(i + t, buf, a_reg[0], b_reg[0], std::false_type{});
           buf ^= 1;
         }
       flush();
     }
   } else {
-    for (int i = 0; i < n_steps; i++) {
-      step(i, buf, std::false_type{});
-      buf ^= 1;
+    for (int i = 0; i < n_steps; i += 2) {
+      step(i, 0, a_reg[1], b_reg[1], std::false_type{});
+      if (i + 1 < n_steps) step(i + 1, 1, a_reg[0], b_reg[0], std::false_type{});
     }
   }
   f32x16(&res)[TM][TN] = KBLOCKED ? acc : blk;
@@ -872,6 +883,20 @@ struct Plan {
   double cost = 0;
 };
 
+// Cost of a plan in microseconds: matrix-core time of the busiest CU (its workgroups share
+// the CU's 4 matrix pipes: 2 flop * 256 MACs per clock at 2.4 GHz = 0.614 Mflop/us), and for a
+// split along K the partial tiles written and read back (about 4 TB/s) plus the launch of the
+// finishing kernel.  The numbers need only rank the candidates of one problem.
+static void price_plan(Plan& pl, const GemmArgs& p, int bm, int bn, int cus, double efficiency,
+                       int k_tiles) {
+  const double tile_us = 2.0 * bm * bn * (double)k_tiles * BK / 0.614e6 / efficiency;
+  const double per_wg = pl.splits > 1 ? (double)pl.kt_per / k_tiles : 1.0;
+  const int wgs_on_busiest_cu = (int)ceil_div(pl.grid, cus);
+  pl.cost = per_wg * wgs_on_busiest_cu * tile_us;
+  if (pl.splits > 1)
+    pl.cost += 3.0 + 2.0 * pl.grid * (double)bm * bn * sizeof(float) / 4.0e6;
+}
+
 static Plan make_plan(const GemmArgs& p, int batch, int bm, int bn, int resident, int cus,
                       double efficiency, bool kblocked) {
   Plan pl;
@@ -880,29 +905,28 @@ static Plan make_plan(const GemmArgs& p, int batch, int bm, int bn, int resident
   const long long tiles = (long long)pl.tiles_m * pl.tiles_n * batch;
   const int slots = cus * resident;
   const int k_tiles = (int)ceil_div(p.K, BK);
-  // one workgroup per work item; tiles are split along K only when the whole problem has
-  // fewer tiles than half the machine's workgroup slots
+  // one workgroup per work item
   pl.rounds = 0;
   pl.tail_tiles = (int)tiles;
   pl.splits = 1;
   pl.kt_per = k_tiles;
+  pl.grid = pl.tail_tiles < 1 ? 1 : pl.tail_tiles;
+  price_plan(pl, p, bm, bn, cus, efficiency, k_tiles);
+  // candidate: when the problem has fewer tiles than half the machine's workgroup slots, cut
+  // every tile into k ranges of at least 4 steps (whole 48-wide blocks for matMul)
   if (pl.tail_tiles > 0 && pl.tail_tiles * 2 <= slots && k_tiles >= 8) {
-    // cut each tail tile into k ranges of at least 4 steps (whole 48-wide blocks for matMul)
+    Plan sp = pl;
     const int unit = kblocked ? TILES_PER_KBLOCK : 1;
     int want = slots / pl.tail_tiles;
     int per = (int)ceil_div(k_tiles, want);
     if (per < 4) per = 4;
     per = (int)ceil_div(per, unit) * unit;
-    pl.kt_per = per;
-    pl.splits = (int)ceil_div(k_tiles, per);
+    sp.kt_per = per;
+    sp.splits = (int)ceil_div(k_tiles, per);
+    sp.grid = sp.tail_tiles * sp.splits;
+    price_plan(sp, p, bm, bn, cus, efficiency, k_tiles);
+    if (sp.splits > 1 && sp.cost < pl.cost) pl = sp;
   }
-  pl.grid = pl.tail_tiles * pl.splits;
-  if (pl.grid < 1) pl.grid = 1;
-  // work on the busiest CU: its share of the workgroups, each one tile or one k range
-  const double per_wg = pl.splits > 1 ? (double)pl.kt_per / k_tiles : 1.0;
-  const int wgs_on_busiest_cu = (int)ceil_div(pl.grid, cus);
-  pl.cost = per_wg * wgs_on_busiest_cu * (double)bm * bn / efficiency;
-  if (pl.splits > 1) pl.cost += 0.15 * bm * bn;  // second pass over the partial tiles
   return pl;
 }
 
