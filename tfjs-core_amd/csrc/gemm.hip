@@ -982,26 +982,33 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
   return TFHIP_OK;
 }
 
-// Tile choice: every shape is planned (grid, split along K) and the one with the least work
-// on the busiest CU wins.  Narrow-N tiles exist for the early MobileNet
-// layers (N = 32 / 64) so that no matrix-core columns are wasted.
+// Tile choice: every shape is planned (grid, split along K) and priced, and the cheapest
+// wins; ties go to the larger tile.  Measured on MI355X, at the sizes of a batch-64 MobileNet
+// the 64 x 64 tile (four wavefronts of one 32 x 32 accumulator) is as efficient per flop as
+// the large ones: its small register footprint lets eight workgroups share a CU, and that
+// occupancy hides latency better than a deeper software pipeline in fewer, larger waves;
+// its finer grain also balances the CUs.  The 128 x 128 tile (eight wavefronts of 32 x 64)
+// needs half the LDS traffic per flop and wins on large problems.
 template <int AMODE, int BMODE, bool KBLOCKED, bool FAST>
 static int launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
-  using Big = TileCfg<2, 2, 2, 2>;     // 128 x 128
-  using Mid = TileCfg<2, 2, 2, 1>;     // 128 x 64
-  using Thin = TileCfg<4, 1, 2, 1>;    // 256 x 32
-  using Small = TileCfg<2, 2, 1, 1>;   // 64 x 64
+  using Big = TileCfg<4, 2, 1, 2>;     // 128 x 128, 8 wavefronts of 32 x 64
+  using Mid = TileCfg<2, 2, 2, 1>;     // 128 x 64, 4 wavefronts of 64 x 32
+  using Wide = TileCfg<2, 4, 1, 1>;    // 64 x 128, 8 wavefronts of 32 x 32
+  using Thin = TileCfg<4, 1, 2, 1>;    // 256 x 32, 4 wavefronts of 64 x 32 (N <= 32)
+  using Small = TileCfg<2, 2, 1, 1>;   // 64 x 64, 4 wavefronts of 32 x 32
+  constexpr int NCFG = 5;
   const int cus = ctx->num_cus;
-  Plan plans[4];
+  Plan plans[NCFG];
   plans[0] = make_plan(p, batch, Big::BM, Big::BN, resident_blocks<Big, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 1.00, KBLOCKED);
   plans[1] = make_plan(p, batch, Mid::BM, Mid::BN, resident_blocks<Mid, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.95, KBLOCKED);
-  plans[2] = make_plan(p, batch, Thin::BM, Thin::BN, resident_blocks<Thin, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.80, KBLOCKED);
-  plans[3] = make_plan(p, batch, Small::BM, Small::BN, resident_blocks<Small, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.85, KBLOCKED);
-  // columns beyond N are wasted matrix-core work: charge it
-  const int bns[4] = {Big::BN, Mid::BN, Thin::BN, Small::BN};
-  const int bms[4] = {Big::BM, Mid::BM, Thin::BM, Small::BM};
+  plans[2] = make_plan(p, batch, Wide::BM, Wide::BN, resident_blocks<Wide, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 1.00, KBLOCKED);
+  plans[3] = make_plan(p, batch, Thin::BM, Thin::BN, resident_blocks<Thin, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.80, KBLOCKED);
+  plans[4] = make_plan(p, batch, Small::BM, Small::BN, resident_blocks<Small, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.98, KBLOCKED);
+  // rows and columns beyond M and N are wasted matrix-core work: charge it
+  const int bns[NCFG] = {Big::BN, Mid::BN, Wide::BN, Thin::BN, Small::BN};
+  const int bms[NCFG] = {Big::BM, Mid::BM, Wide::BM, Thin::BM, Small::BM};
   int best = -1;
-  for (int i = 0; i < 4; i++) {
+  for (int i = 0; i < NCFG; i++) {
     const double useful = ((double)p.N / (ceil_div(p.N, bns[i]) * bns[i])) *
                           ((double)p.M / (ceil_div(p.M, bms[i]) * bms[i]));
     plans[i].cost /= useful;
@@ -1010,8 +1017,9 @@ static int launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
   switch (best) {
     case 0: return launch_cfg<Big, AMODE, BMODE, KBLOCKED, FAST>(ctx, p, plans[0]);
     case 1: return launch_cfg<Mid, AMODE, BMODE, KBLOCKED, FAST>(ctx, p, plans[1]);
-    case 2: return launch_cfg<Thin, AMODE, BMODE, KBLOCKED, FAST>(ctx, p, plans[2]);
-    default: return launch_cfg<Small, AMODE, BMODE, KBLOCKED, FAST>(ctx, p, plans[3]);
+    case 2: return launch_cfg<Wide, AMODE, BMODE, KBLOCKED, FAST>(ctx, p, plans[2]);
+    case 3: return launch_cfg<Thin, AMODE, BMODE, KBLOCKED, FAST>(ctx, p, plans[3]);
+    default: return launch_cfg<Small, AMODE, BMODE, KBLOCKED, FAST>(ctx, p, plans[4]);
   }
 }
 
