@@ -23,6 +23,21 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 RIDGE = PEAK_FP32_MFMA_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
 
+# HBM bytes per launch (fetch + write), averaged over the launches of each kernel variant in
+# one batch-64 step, from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in
+# profiles/mobilenet_b64_fp32_hbm_traffic.txt (counters scaled by what a streaming kernel of
+# known size reads: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Counters cannot be read from inside
+# this process, so the figures are carried here; they apply to batch 64, fp32 weights.
+MIB = 1 << 20
+MEASURED_HBM_BYTES_PER_LAUNCH = {
+    "gemm_64x64_rowmajor_f32": 103.8 * MIB,
+    "gemm_64x128_rowmajor_f32": 47.3 * MIB,
+    "depthwise3x3_s1_2x2": 84.7 * MIB,
+    "depthwise3x3_s2_1x1": 115.0 * MIB,
+    "conv_smallk_n32_f32": 153.3 * MIB,
+    "global_avgpool": 12.5 * MIB,
+}
+
 
 def per_layer_times(tf, mobilenet, w, x, reps):
     """Time every layer of the forward pass on its real input with an event pair on the
@@ -105,7 +120,9 @@ def roofline_of_dominant_kernel(rows):
                     frac=round(achieved / PEAK_HBM_GBS, 4))
     roof.update(kernel=name, launches_per_step=g["launches"], layers=g["layers"],
                 avg_launch_us=round(g["ms"] * 1e3 / g["launches"], 2),
-                share_of_step=round(g["ms"] / sum(r["ms"] for r in rows), 3), traffic=None)
+                share_of_step=round(g["ms"] / sum(r["ms"] for r in rows), 3),
+                algorithmic_bytes_per_launch=round(g["bytes"] / g["launches"]),
+                algorithmic_flops_per_launch=round(g["flops"] / g["launches"]), traffic=None)
     return roof, groups
 
 
@@ -188,6 +205,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-js", action="store_true", help="skip the Node.js host leg")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
+    ap.add_argument("--calibrate-counters", action="store_true",
+                    help="only launch a streaming kernel of known size (relu over 256 MiB: reads "
+                         "256 MiB, writes 256 MiB) three times, to scale FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
@@ -198,6 +218,15 @@ def main():
     from tfhip import mobilenet
     tf.set_backend("hip")
     be = tf.backend()
+
+    if args.calibrate_counters:
+        big = tf.tensor(np.ones((64, 1024, 1024), np.float32))
+        for _ in range(3):
+            tf.dispose(tf.relu(big))
+        be.sync()
+        print(json.dumps({"calibration_kernel": "unary_f32_vec_kernel (relu)",
+                          "bytes_read": big.size * 4, "bytes_written": big.size * 4}))
+        return
 
     params = mobilenet.make_params(seed=0)
     dev_params = mobilenet.quantize_params(params) if args.quant else params
@@ -243,6 +272,8 @@ def main():
 
     rows = per_layer_times(tf, mobilenet, w, x, reps=20)
     roof, groups = roofline_of_dominant_kernel(rows)
+    if args.batch == 64 and not args.quant and roof["kernel"] in MEASURED_HBM_BYTES_PER_LAUNCH:
+        roof["traffic"] = round(MEASURED_HBM_BYTES_PER_LAUNCH[roof["kernel"]])
     if args.layers:
         for r in rows:
             ai = 2.0 * r["macs"] / r["bytes"]
