@@ -48,7 +48,7 @@ struct GemmArgs {
   int H, W, Cin, OH, OW, KH, KW, sh, sw, dh, dw, pt, pl;
   double qscale, qmin;
   // schedule (see work_item)
-  int tiles_m, tiles_n, k_tiles, rounds, tail_tiles, splits, kt_per;
+  int tiles_m, tiles_n, k_tiles, full_tiles, tail_tiles, splits, kt_per;
   float* partials;  // [tail_tiles * splits][BM * BN] partial tiles when splits > 1
   unsigned a_bytes, b_bytes;  // per-batch byte extents of A and B (buffer-load range check)
 };
@@ -110,20 +110,22 @@ struct WorkItem {
   int slot;     // partial slot, -1 = finish the tile here
 };
 
-// Schedule: `rounds` is 0 in every plan the host makes today, so workgroup g takes k range
-// g % splits of tile g / splits (kt_per steps each); with splits == 1 that is tile g whole.
-// The rounds branch serves a grid smaller than the tile count, should a plan ask for one.
-__device__ __forceinline__ WorkItem work_item(const GemmArgs& p, int g, int G, int it) {
+// Schedule: the first `full_tiles` workgroups take one whole tile each (ids remapped per
+// XCD); the remaining tail_tiles * splits workgroups take k range h % splits of tail tile
+// h / splits.  The tail workgroups are dispatched last and in hardware order, so the short
+// items spread over all XCDs and CUs.
+__device__ __forceinline__ WorkItem work_item(const GemmArgs& p, int block) {
   WorkItem w = {-1, 0, 0, -1};
-  if (it < p.rounds) {
-    w.tile = it * G + g;
+  if (block < p.full_tiles) {
+    w.tile = xcd_remap(block, p.full_tiles);
     w.kt1 = p.k_tiles;
-  } else if (it == p.rounds && g < p.tail_tiles * p.splits) {
-    w.tile = p.rounds * G + g / p.splits;
-    const int s = g % p.splits;
+  } else if (block - p.full_tiles < p.tail_tiles * p.splits) {
+    const int h = block - p.full_tiles;
+    w.tile = p.full_tiles + h / p.splits;
+    const int s = h % p.splits;
     w.kt0 = s * p.kt_per;
     w.kt1 = min(p.k_tiles, w.kt0 + p.kt_per);
-    if (p.splits > 1) w.slot = g;
+    if (p.splits > 1) w.slot = h;
   }
   return w;
 }
@@ -147,8 +149,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int l32 = lane & 31, g = lane >> 5;
-  const int G = gridDim.x;
-  const int wg = xcd_remap(blockIdx.x, G);
   const int tiles_per_batch = p.tiles_m * p.tiles_n;
 
   // ---- per-tile description of the A/B items this thread stages ----
@@ -400,7 +400,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   };
 
   Loader L;
-  const WorkItem cur = work_item(p, wg, G, 0);
+  const WorkItem cur = work_item(p, blockIdx.x);
   if (cur.tile < 0) return;
   setup(L, cur.tile);
   const int n_steps = cur.kt1 - cur.kt0;
@@ -876,10 +876,9 @@ struct TileCfg {
   static constexpr int BM = WM_ * TM_ * 32, BN = WN_ * TN_ * 32;
 };
 
-// How one tile shape would run a problem: grid, split along K, and a cost in units of MFMA
-// work on the busiest CU (larger tiles do the same flops with less LDS traffic).
+// How one tile shape would run a problem: whole tiles, tiles split along K, and a cost.
 struct Plan {
-  int grid = 0, rounds = 0, tail_tiles = 0, splits = 1, kt_per = 0, tiles_m = 0, tiles_n = 0;
+  int grid = 0, full_tiles = 0, tail_tiles = 0, splits = 1, kt_per = 0, tiles_m = 0, tiles_n = 0;
   double cost = 0;
 };
 
@@ -887,14 +886,28 @@ struct Plan {
 // the CU's 4 matrix pipes: 2 flop * 256 MACs per clock at 2.4 GHz = 0.614 Mflop/us), and for a
 // split along K the partial tiles written and read back (about 4 TB/s) plus the launch of the
 // finishing kernel.  The numbers need only rank the candidates of one problem.
-static void price_plan(Plan& pl, const GemmArgs& p, int bm, int bn, int cus, double efficiency,
-                       int k_tiles) {
+static void price_plan(Plan& pl, int bm, int bn, int cus, double efficiency, int k_tiles) {
   const double tile_us = 2.0 * bm * bn * (double)k_tiles * BK / 0.614e6 / efficiency;
-  const double per_wg = pl.splits > 1 ? (double)pl.kt_per / k_tiles : 1.0;
-  const int wgs_on_busiest_cu = (int)ceil_div(pl.grid, cus);
-  pl.cost = per_wg * wgs_on_busiest_cu * tile_us;
-  if (pl.splits > 1)
-    pl.cost += 3.0 + 2.0 * pl.grid * (double)bm * bn * sizeof(float) / 4.0e6;
+  const double per_split = (double)pl.kt_per / k_tiles;
+  const long long split_wgs = (long long)pl.tail_tiles * pl.splits;
+  pl.cost = tile_us * (ceil_div(pl.full_tiles, cus) +
+                       (pl.splits > 1 ? per_split * ceil_div(split_wgs, cus)
+                                      : (double)ceil_div(pl.tail_tiles, cus)));
+  if (pl.splits > 1) pl.cost += 3.0 + 2.0 * split_wgs * (double)bm * bn * sizeof(float) / 4.0e6;
+}
+
+// k ranges for `tail` tiles cut `want` ways: at least 4 steps each (whole 48-wide blocks for
+// matMul).  Returns false when that leaves a single range.
+static bool split_tail(Plan& pl, int tail, int want, int k_tiles, bool kblocked) {
+  const int unit = kblocked ? TILES_PER_KBLOCK : 1;
+  if (want < 2 || k_tiles < 8) return false;
+  int per = (int)ceil_div(k_tiles, want);
+  if (per < 4) per = 4;
+  per = (int)ceil_div(per, unit) * unit;
+  pl.kt_per = per;
+  pl.splits = (int)ceil_div(k_tiles, per);
+  pl.tail_tiles = tail;
+  return pl.splits > 1;
 }
 
 static Plan make_plan(const GemmArgs& p, int batch, int bm, int bn, int resident, int cus,
@@ -902,30 +915,37 @@ static Plan make_plan(const GemmArgs& p, int batch, int bm, int bn, int resident
   Plan pl;
   pl.tiles_m = (int)ceil_div(p.M, bm);
   pl.tiles_n = (int)ceil_div(p.N, bn);
-  const long long tiles = (long long)pl.tiles_m * pl.tiles_n * batch;
+  const int tiles = (int)((long long)pl.tiles_m * pl.tiles_n * batch);
   const int slots = cus * resident;
   const int k_tiles = (int)ceil_div(p.K, BK);
-  // one workgroup per work item
-  pl.rounds = 0;
-  pl.tail_tiles = (int)tiles;
+  // candidate 1: one workgroup per tile
+  pl.full_tiles = tiles;
+  pl.tail_tiles = 0;
   pl.splits = 1;
   pl.kt_per = k_tiles;
-  pl.grid = pl.tail_tiles < 1 ? 1 : pl.tail_tiles;
-  price_plan(pl, p, bm, bn, cus, efficiency, k_tiles);
-  // candidate: when the problem has fewer tiles than half the machine's workgroup slots, cut
-  // every tile into k ranges of at least 4 steps (whole 48-wide blocks for matMul)
-  if (pl.tail_tiles > 0 && pl.tail_tiles * 2 <= slots && k_tiles >= 8) {
+  pl.grid = tiles < 1 ? 1 : tiles;
+  price_plan(pl, bm, bn, cus, efficiency, k_tiles);
+  // candidate 2: fewer tiles than half the machine's workgroup slots: cut every tile
+  if (tiles > 0 && tiles * 2 <= slots) {
     Plan sp = pl;
-    const int unit = kblocked ? TILES_PER_KBLOCK : 1;
-    int want = slots / pl.tail_tiles;
-    int per = (int)ceil_div(k_tiles, want);
-    if (per < 4) per = 4;
-    per = (int)ceil_div(per, unit) * unit;
-    sp.kt_per = per;
-    sp.splits = (int)ceil_div(k_tiles, per);
-    sp.grid = sp.tail_tiles * sp.splits;
-    price_plan(sp, p, bm, bn, cus, efficiency, k_tiles);
-    if (sp.splits > 1 && sp.cost < pl.cost) pl = sp;
+    sp.full_tiles = 0;
+    if (split_tail(sp, tiles, slots / tiles, k_tiles, kblocked)) {
+      sp.grid = sp.tail_tiles * sp.splits;
+      price_plan(sp, bm, bn, cus, efficiency, k_tiles);
+      if (sp.cost < pl.cost) pl = sp;
+    }
+  }
+  // candidate 3: whole rounds of one tile per CU, and the tiles left over (at most half a
+  // round) cut so that every CU gets one short piece instead of some CUs a whole extra tile
+  const int left = tiles % cus;
+  if (tiles > cus && left > 0 && left * 2 <= cus) {
+    Plan sp = pl;
+    sp.full_tiles = tiles - left;
+    if (split_tail(sp, left, cus / left, k_tiles, kblocked)) {
+      sp.grid = sp.full_tiles + sp.tail_tiles * sp.splits;
+      price_plan(sp, bm, bn, cus, efficiency, k_tiles);
+      if (sp.cost < pl.cost) pl = sp;
+    }
   }
   return pl;
 }
@@ -952,11 +972,12 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
   static const char* const a_names[] = {"rowmajor", "transposed", "im2col"};
   static const char* const b_names[] = {"f32", "f32t", "u8"};
   snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "gemm_%dx%d_%s_%s%s%s", T::BM, T::BN,
-           a_names[AMODE], b_names[BMODE], KBLOCKED ? "_kb48" : "", pl.splits > 1 ? "_splitk" : "");
+           a_names[AMODE], b_names[BMODE], KBLOCKED ? "_kb48" : "",
+           pl.splits > 1 ? (pl.full_tiles ? "_tailk" : "_splitk") : "");
   if (!FAST) strncat(ctx->last_kernel, "_unaligned", sizeof ctx->last_kernel - strlen(ctx->last_kernel) - 1);
   p.tiles_m = pl.tiles_m;
   p.tiles_n = pl.tiles_n;
-  p.rounds = pl.rounds;
+  p.full_tiles = pl.full_tiles;
   p.tail_tiles = pl.tail_tiles;
   p.splits = pl.splits;
   p.kt_per = pl.kt_per;
@@ -976,7 +997,7 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
     const long long blocks = ceil_div(quads, 256);
     const long long cap = (long long)ctx->num_cus * 8;
     hipLaunchKernelGGL(splitk_finish_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256),
-                       0, ctx->stream, p, T::BM, T::BN, pl.rounds * pl.grid);
+                       0, ctx->stream, p, T::BM, T::BN, pl.full_tiles);
     TFHIP_LAUNCH_CHECK(ctx);
   }
   return TFHIP_OK;
