@@ -141,8 +141,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   constexpr int A_PER = (A_ITEMS + THREADS - 1) / THREADS;
   constexpr int B_PER = (B_ITEMS + THREADS - 1) / THREADS;
 
-  __shared__ __attribute__((aligned(16))) float As[NBUF][BM * LDA_S];
-  __shared__ __attribute__((aligned(16))) float Bs[NBUF][BK * LDB_S];
+  // One LDS block: the A and B double buffers of the k loop, reused after the loop as the
+  // staging area of the output tile (tiles with one accumulator column per wavefront).
+  constexpr int A_FLOATS = NBUF * BM * LDA_S, B_FLOATS = NBUF * BK * LDB_S;
+  constexpr bool STAGED_STORE = TN == 1;
+  constexpr int LDC_S = BN + 4;
+  constexpr int C_FLOATS = STAGED_STORE ? BM * LDC_S : 0;
+  constexpr int LDS_FLOATS = A_FLOATS + B_FLOATS > C_FLOATS ? A_FLOATS + B_FLOATS : C_FLOATS;
+  __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
+  float (*As)[BM * LDA_S] = reinterpret_cast<float (*)[BM * LDA_S]>(lds);
+  float (*Bs)[BK * LDB_S] = reinterpret_cast<float (*)[BK * LDB_S]>(lds + A_FLOATS);
 
   const int tid = threadIdx.x;
   __builtin_assume(tid >= 0 && tid < THREADS);
@@ -643,9 +651,47 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     }
   };
   const bool interior = bm0 + BM <= p.M && bn0 + BN <= p.N;
-  if (full_bias || full_alpha) store(std::true_type{}, std::false_type{});
-  else if (interior) store(std::false_type{}, std::true_type{});
-  else store(std::false_type{}, std::false_type{});
+  if (full_bias || full_alpha) {
+    store(std::true_type{}, std::false_type{});
+  } else if (!interior) {
+    store(std::false_type{}, std::false_type{});
+  } else if (STAGED_STORE && (p.N & 3) == 0) {
+    // One accumulator column per lane would mean 4-byte stores (two 128-byte runs per
+    // instruction).  Pass the tile through LDS instead and store it as 16 bytes per lane,
+    // whole 256/512-byte row segments per instruction: a quarter of the store instructions.
+    // (Ct is 16-byte aligned: buffers are, bn0 is a multiple of 64 and N of 4.)
+    __syncthreads();  // every wavefront is done with the k-loop buffers
+    float* cs = lds + lrow0 * LDC_S + lcol0;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+        cs[(i * 32 + 8 * (r >> 2) + (r & 3)) * LDC_S] = res[i][0][r];
+    __syncthreads();
+    constexpr int QUADS_PER_ROW = BN / 4;
+    constexpr int ROWS_PER_PASS = THREADS / QUADS_PER_ROW;
+    static_assert(THREADS % QUADS_PER_ROW == 0 && BM % ROWS_PER_PASS == 0, "tile / block shape");
+    const int cq = tid % QUADS_PER_ROW, r0 = tid / QUADS_PER_ROW;
+    f32x4 bv = {0.f, 0.f, 0.f, 0.f}, al = {0.f, 0.f, 0.f, 0.f};
+    if (p.bias_kind == TFHIP_BCAST_SCALAR) bv = f32x4{p.bias[0], p.bias[0], p.bias[0], p.bias[0]};
+    if (p.bias_kind == TFHIP_BCAST_COLUMN)
+#pragma unroll
+      for (int e = 0; e < 4; e++) bv[e] = p.bias[bn0 + 4 * cq + e];
+    if (p.prelu_kind == TFHIP_BCAST_SCALAR) al = f32x4{p.prelu[0], p.prelu[0], p.prelu[0], p.prelu[0]};
+    if (p.prelu_kind == TFHIP_BCAST_COLUMN)
+#pragma unroll
+      for (int e = 0; e < 4; e++) al[e] = p.prelu[bn0 + 4 * cq + e];
+#pragma unroll
+    for (int pass = 0; pass < BM / ROWS_PER_PASS; pass++) {
+      const int row = r0 + pass * ROWS_PER_PASS;
+      f32x4 v = *reinterpret_cast<const f32x4*>(lds + row * LDC_S + 4 * cq);
+#pragma unroll
+      for (int e = 0; e < 4; e++) v[e] = activate(v[e] + bv[e], act, al[e]);
+      *reinterpret_cast<f32x4*>(Ct + row * p.N + 4 * cq) = v;
+    }
+  } else {
+    store(std::false_type{}, std::true_type{});
+  }
 }
 
 // Finishes the tiles that were split along K: adds the `splits` partial tiles in ascending
