@@ -714,7 +714,17 @@ __global__ void splitk_finish_kernel(const GemmArgs p, int BM, int BN, int first
     if (row >= p.M || col >= p.N) continue;
     f32x4 v = {0.f, 0.f, 0.f, 0.f};
     const float* src = p.partials + ((long long)tt * p.splits) * (BM * BN) + e;
-    for (int s = 0; s < p.splits; s++) v += *reinterpret_cast<const f32x4*>(src + (long long)s * (BM * BN));
+    // four partial tiles in flight at a time; added in ascending k order
+    int s = 0;
+    for (; s + 4 <= p.splits; s += 4) {
+      f32x4 t[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+        t[u] = *reinterpret_cast<const f32x4*>(src + (long long)(s + u) * (BM * BN));
+#pragma unroll
+      for (int u = 0; u < 4; u++) v += t[u];
+    }
+    for (; s < p.splits; s++) v += *reinterpret_cast<const f32x4*>(src + (long long)s * (BM * BN));
     const long long base = (long long)batch * p.strideC + (long long)row * p.N + col;
 #pragma unroll
     for (int j = 0; j < 4; j++) {

@@ -207,7 +207,18 @@ __global__ void global_avgpool_kernel(const float* x, float* y, int n_img, int h
   const int n = gid / c4, cq = gid - n * c4;
   const f32x4* src = reinterpret_cast<const f32x4*>(x) + (int64_t)n * hw * c4 + cq;
   double s0 = 0, s1 = 0, s2 = 0, s3 = 0;
-  for (int i = 0; i < hw; i++) {
+  // seven loads in flight at a time (a 7x7 window is 7 such groups); summed in pixel order
+  int i = 0;
+  for (; i + 7 <= hw; i += 7) {
+    f32x4 v[7];
+#pragma unroll
+    for (int u = 0; u < 7; u++) v[u] = src[(int64_t)(i + u) * c4];
+#pragma unroll
+    for (int u = 0; u < 7; u++) {
+      s0 += v[u][0]; s1 += v[u][1]; s2 += v[u][2]; s3 += v[u][3];
+    }
+  }
+  for (; i < hw; i++) {
     const f32x4 v = src[(int64_t)i * c4];
     s0 += v[0]; s1 += v[1]; s2 += v[2]; s3 += v[3];
   }

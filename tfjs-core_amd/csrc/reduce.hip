@@ -77,6 +77,32 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void softmax_rows_kernel(
   const float* xr = x + row * cols;
   float* yr = y + row * cols;
   float m = xr[0];
+  if (cols <= WAVE * 16) {
+    // the row fits the wavefront's registers: one pass over memory, all loads in flight
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const int64_t j = lane + i * WAVE;
+      v[i] = xr[j < cols ? j : 0];
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      if (v[i] > m) m = v[i];
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const float o = __shfl_xor(m, off, WAVE);
+      if (o > m) m = o;
+    }
+    double s = 0.0;
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      if (lane + i * WAVE < cols) s += (double)expf(v[i] - m);
+    for (int off = WAVE / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
+    const float lse = m + logf((float)s);
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      if (lane + i * WAVE < cols) yr[lane + i * WAVE] = expf(v[i] - lse);
+    return;
+  }
   for (int64_t j = lane; j < cols; j += WAVE) {
     const float v = xr[j];
     if (v > m) m = v;
