@@ -940,8 +940,10 @@ struct Plan {
 
 // Cost of a plan in microseconds: matrix-core time of the busiest CU (its workgroups share
 // the CU's 4 matrix pipes: 2 flop * 256 MACs per clock at 2.4 GHz = 0.614 Mflop/us), and for a
-// split along K the partial tiles written and read back (about 4 TB/s) plus the launch of the
-// finishing kernel.  The numbers need only rank the candidates of one problem.
+// split along K the partial tiles written and read back (about 4 TB/s) plus the finishing
+// kernel (a second launch costs about 5 us in a busy stream; summing the partials inside the
+// first kernel instead was tried and is slower: a device-scope fence writes back the whole L2
+// of the XCD it is issued on).  The numbers need only rank the candidates of one problem.
 static void price_plan(Plan& pl, int bm, int bn, int cus, double efficiency, int k_tiles) {
   const double tile_us = 2.0 * bm * bn * (double)k_tiles * BK / 0.614e6 / efficiency;
   const double per_split = (double)pl.kt_per / k_tiles;
@@ -949,7 +951,7 @@ static void price_plan(Plan& pl, int bm, int bn, int cus, double efficiency, int
   pl.cost = tile_us * (ceil_div(pl.full_tiles, cus) +
                        (pl.splits > 1 ? per_split * ceil_div(split_wgs, cus)
                                       : (double)ceil_div(pl.tail_tiles, cus)));
-  if (pl.splits > 1) pl.cost += 3.0 + 2.0 * split_wgs * (double)bm * bn * sizeof(float) / 4.0e6;
+  if (pl.splits > 1) pl.cost += 6.0 + 2.0 * split_wgs * (double)bm * bn * sizeof(float) / 4.0e6;
 }
 
 // k ranges for `tail` tiles cut `want` ways: at least 4 steps each (whole 48-wide blocks for
