@@ -1,0 +1,160 @@
+"""Every kernel variant the dense path can choose is exercised on purpose, and the test checks
+which variant ran (tfhip_last_kernel), so a change of the planner cannot silently leave a
+variant untested.  Small cases are compared with the CPU oracle; large ones (too slow for the
+scalar oracle) with a float64 numpy contraction of the same inputs.  fp32 tolerance
+1e-4 relative / 1e-5 absolute."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def close(actual, expected, rtol=RTOL, atol=ATOL):
+    a = np.asarray(actual, np.float64)
+    e = np.asarray(expected, np.float64)
+    assert a.shape == e.shape, (a.shape, e.shape)
+    err = np.abs(a - e)
+    ok = (np.isnan(a) & np.isnan(e)) | (err <= atol + rtol * np.abs(e)) | (a == e)
+    assert ok.all(), "max err %g, %d bad of %d" % (np.nanmax(np.where(ok, 0, err)), (~ok).sum(),
+                                                     ok.size)
+
+
+@pytest.fixture(scope="module")
+def tf():
+    import tfhip
+    tfhip.set_backend("hip")
+    return tfhip
+
+
+@pytest.fixture(scope="module")
+def ref(oracle):
+    from providers import OracleOps
+    return OracleOps()
+
+
+def last_kernel(tf):
+    be = tf.backend()
+    return be.lib.tfhip_last_kernel(be.ctx).decode()
+
+
+def act64(v, act):
+    if act == "relu":
+        return np.maximum(v, 0)
+    if act == "relu6":
+        return np.clip(v, 0, 6)
+    return v
+
+
+# ------------------------------------------------- short-contraction conv ----
+@pytest.mark.parametrize("xs,fs,stride,pad,dil,act,bias_kind,want", [
+    ((2, 224, 224, 3), (3, 3, 3, 32), 2, "same", 1, "relu6", "channel", "conv_smallk_n32_f32"),
+    ((1, 33, 29, 3), (3, 3, 3, 32), 2, "same", 1, "linear", "none", "conv_smallk_n32_f32"),
+    ((2, 17, 40, 1), (5, 5, 1, 7), (1, 2), "same", 1, "relu", "scalar", "conv_smallk_n32_f32"),
+    ((1, 21, 21, 2), (3, 3, 2, 64), 1, "valid", 2, "prelu", "channel", "conv_smallk_n64_f32"),
+    ((3, 9, 70, 3), (3, 3, 3, 40), 1, "same", 1, "relu6", "full", "conv_smallk_n64_f32"),
+    ((1, 8, 300, 3), (1, 3, 3, 33), 1, "same", 1, "linear", "channel", "conv_smallk_n64_f32"),
+])
+def test_conv_smallk(tf, ref, xs, fs, stride, pad, dil, act, bias_kind, want):
+    print("smallk", xs, fs, stride, pad, dil, act, bias_kind, flush=True)
+    rng = np.random.default_rng(sum(xs) * 7 + sum(fs))
+    x = rng.uniform(-1, 1, xs).astype(np.float32)
+    w = (rng.standard_normal(fs) * 0.3).astype(np.float32)
+    cout = fs[3]
+    want_y = ref.conv2d(x, w, stride, pad, dil)
+    bias = {"none": None, "scalar": np.float32(0.25),
+            "channel": rng.standard_normal(cout).astype(np.float32),
+            "full": rng.standard_normal(want_y.shape).astype(np.float32)}[bias_kind]
+    prelu = rng.uniform(0.1, 0.5, cout).astype(np.float32) if act == "prelu" else None
+    want_y = ref.conv2d(x, w, stride, pad, dil, bias=bias, activation=act, prelu=prelu)
+    with tf.tidy():
+        y = tf.fused.conv2d(tf.tensor(x), tf.tensor(w), stride, pad, dilations=dil,
+                            bias=None if bias is None else tf.tensor(bias), activation=act,
+                            prelu_activation_weights=None if prelu is None else tf.tensor(prelu))
+        got = y.data_sync()
+        assert last_kernel(tf) == want
+    close(got, want_y)
+
+
+def test_conv_smallk_uint8_filter_and_nan(tf, ref):
+    rng = np.random.default_rng(5)
+    x = rng.uniform(0, 1, (1, 20, 20, 3)).astype(np.float32)
+    q = rng.integers(0, 256, (3, 3, 3, 16)).astype(np.uint8)
+    scale, mn = 0.011, -1.2
+    with tf.tidy():
+        got = tf.conv2d(tf.tensor(x), tf.quantized_tensor(q, scale, mn), 2, "same").data_sync()
+        assert last_kernel(tf) == "conv_smallk_n32_u8"
+    close(got, ref.conv2d(x, ref.dequantize(q, scale, mn), 2, "same"))
+    # a NaN pixel reaches exactly the outputs whose window covers it
+    x[0, 10, 10, 1] = np.nan
+    w = rng.standard_normal((3, 3, 3, 8)).astype(np.float32)
+    with tf.tidy():
+        got = tf.conv2d(tf.tensor(x), tf.tensor(w), 1, "same").data_sync()
+    want = ref.conv2d(x, w, 1, "same")
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    close(got, want)
+
+
+# ------------------------------------------------------- GEMM tile shapes ----
+@pytest.mark.parametrize("n,h,cin,cout,act,want", [
+    (4, 28, 128, 256, "relu6", "gemm_64x64_rowmajor_f32"),            # staged 16-byte store
+    (64, 7, 512, 1024, "relu6", "gemm_64x128_rowmajor_f32"),          # 8 wavefronts of 32x32
+    (64, 7, 1024, 1024, "relu", "gemm_64x64_rowmajor_f32_tailk"),     # leftover tiles split on K
+    (16, 32, 256, 512, "linear", "gemm_128x128_rowmajor_f32"),        # 8 wavefronts of 32x64
+    (2, 30, 36, 30, "relu6", None),                                   # N % 4 != 0: guarded store
+    (1, 5, 1024, 24, "linear", None),                                 # few tiles: split along K
+])
+def test_pointwise_conv_tiles(tf, n, h, cin, cout, act, want):
+    print("pointwise", n, h, cin, cout, act, flush=True)
+    rng = np.random.default_rng(n * 1000 + h * 10 + cin + cout)
+    x = rng.uniform(-1, 1, (n, h, h, cin)).astype(np.float32)
+    w = (rng.standard_normal((1, 1, cin, cout)) * np.sqrt(2.0 / cin)).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32)
+    with tf.tidy():
+        got = tf.fused.conv2d(tf.tensor(x), tf.tensor(w), 1, "same", bias=tf.tensor(b),
+                              activation=act).data_sync()
+        k = last_kernel(tf)
+    if want is not None:
+        assert k == want, k
+    else:
+        assert k.startswith("gemm_"), k
+    want_y = act64(x.reshape(-1, cin).astype(np.float64) @ w.reshape(cin, cout).astype(np.float64)
+                   + b, act).reshape(n, h, h, cout)
+    close(got, want_y)
+
+
+@pytest.mark.parametrize("m,k,n,want_prefix", [
+    (4096, 784, 1024, "gemm_128x128_rowmajor_f32_kb48"),
+    (256, 512, 256, "gemm_64x64_rowmajor_f32_kb48_splitk"),
+    (64, 1024, 1000, "gemm_64x64_rowmajor_f32_kb48_splitk"),
+    (4096, 1024, 10, "gemm_256x32_rowmajor_f32_kb48"),
+])
+def test_matmul_tiles_against_float64(tf, m, k, n, want_prefix):
+    print("matmul", m, k, n, flush=True)
+    rng = np.random.default_rng(m + k + n)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    with tf.tidy():
+        got = tf.matmul(tf.tensor(a), tf.tensor(b)).data_sync()
+        kern = last_kernel(tf)
+    assert kern.startswith(want_prefix), kern
+    close(got, a.astype(np.float64) @ b.astype(np.float64), atol=1e-4)
+
+
+def test_implicit_gemm_3x3_tiles(tf):
+    """3x3 convolutions through the im2col loaders at sizes that take the 64x64 and wider
+    tiles, against float64 on sampled output positions."""
+    rng = np.random.default_rng(9)
+    for (n, h, cin, cout) in ((8, 56, 64, 128), (2, 28, 32, 48), (1, 14, 256, 512)):
+        x = rng.uniform(-1, 1, (n, h, h, cin)).astype(np.float32)
+        w = (rng.standard_normal((3, 3, cin, cout)) * np.sqrt(2.0 / (9 * cin))).astype(np.float32)
+        with tf.tidy():
+            got = tf.conv2d(tf.tensor(x), tf.tensor(w), 1, "same").data_sync()
+            assert "im2col" in last_kernel(tf)
+        xp = np.pad(x, ((0, 0), (1, 1), (1, 1), (0, 0))).astype(np.float64)
+        w64 = w.astype(np.float64)
+        for _ in range(200):
+            b, i, j = rng.integers(n), rng.integers(h), rng.integers(h)
+            want = np.einsum("abc,abco->o", xp[b, i:i + 3, j:j + 3, :], w64)
+            close(got[b, i, j], want)

@@ -951,6 +951,10 @@ static void price_plan(Plan& pl, int bm, int bn, int cus, double efficiency, int
   pl.cost = tile_us * (ceil_div(pl.full_tiles, cus) +
                        (pl.splits > 1 ? per_split * ceil_div(split_wgs, cus)
                                       : (double)ceil_div(pl.tail_tiles, cus)));
+  // a k step is a chain of global load, LDS store, barrier, LDS read and MFMAs: about 0.4 us
+  // even when the matrix cores would be done sooner, which is what a sparse grid pays
+  const double chain_us = 0.4 * (pl.full_tiles > 0 || pl.splits == 1 ? k_tiles : pl.kt_per);
+  if (pl.cost < chain_us) pl.cost = chain_us;
   if (pl.splits > 1) pl.cost += 6.0 + 2.0 * split_wgs * (double)bm * bn * sizeof(float) / 4.0e6;
 }
 
