@@ -149,29 +149,37 @@ def cpu_baseline(mobilenet, params, budget_s=15.0):
                        "of backend_cpu at -O2, 1 thread" % (n, el))
 
 
-def write_weight_files(params, bin_path, manifest_path):
-    """Weights as a tfjs-style flat binary + manifest entries (name, shape, dtype and, for
-    uint8 affine-quantised tensors, quantization {dtype, scale, min})."""
+def write_weight_files(params, directory, shard_bytes=4 << 20):
+    """Weights in the tfjs on-disk format (io/types.ts:39-108): `weights_manifest.json` with
+    one group {paths, weights} and the group's bytes cut into shard files of `shard_bytes`
+    (weights straddle shard boundaries, as tfjs-converter writes them).  uint8 affine-quantised
+    tensors carry quantization {dtype, scale, min}.  Returns the manifest path."""
     import numpy as np
-    from tfhip import mobilenet  # noqa: F401
     order = ["stem_w", "stem_b"]
     for i in range(1, 14):
         order += ["dw%d_w" % i, "dw%d_b" % i, "pw%d_w" % i, "pw%d_b" % i]
     order += ["fc_w", "fc_b"]
-    manifest = []
-    with open(bin_path, "wb") as f:
-        for name in order:
-            v = params[name]
-            if isinstance(v, tuple):
-                q, scale, mn = v
-                f.write(np.ascontiguousarray(q, np.uint8).tobytes())
-                manifest.append(dict(name=name, shape=list(q.shape), dtype="float32",
-                                     quantization=dict(dtype="uint8", scale=scale, min=mn)))
-            else:
-                f.write(np.ascontiguousarray(v, np.float32).tobytes())
-                manifest.append(dict(name=name, shape=list(v.shape), dtype="float32"))
+    entries, blob = [], bytearray()
+    for name in order:
+        v = params[name]
+        if isinstance(v, tuple):
+            q, scale, mn = v
+            blob += np.ascontiguousarray(q, np.uint8).tobytes()
+            entries.append(dict(name=name, shape=list(q.shape), dtype="float32",
+                                quantization=dict(dtype="uint8", scale=scale, min=mn)))
+        else:
+            blob += np.ascontiguousarray(v, np.float32).tobytes()
+            entries.append(dict(name=name, shape=list(v.shape), dtype="float32"))
+    n_shards = max(1, -(-len(blob) // shard_bytes))
+    paths = []
+    for i in range(n_shards):
+        paths.append("group1-shard%dof%d" % (i + 1, n_shards))
+        with open(os.path.join(directory, paths[-1]), "wb") as f:
+            f.write(blob[i * shard_bytes:(i + 1) * shard_bytes])
+    manifest_path = os.path.join(directory, "weights_manifest.json")
     with open(manifest_path, "w") as f:
-        json.dump(manifest, f)
+        json.dump([dict(paths=paths, weights=entries)], f)
+    return manifest_path
 
 
 def js_host_leg(params, x_host, batch, steps, warmup):
@@ -185,10 +193,10 @@ def js_host_leg(params, x_host, batch, steps, warmup):
     if node is None or not os.path.exists(os.path.join(js, "tfjs_hip.node")):
         return None
     with tempfile.TemporaryDirectory() as d:
-        wb, mf, xb = (os.path.join(d, n) for n in ("w.bin", "manifest.json", "x.bin"))
-        write_weight_files(params, wb, mf)
+        xb = os.path.join(d, "x.bin")
+        mf = write_weight_files(params, d)
         x_host.tofile(xb)
-        r = subprocess.run([node, os.path.join(js, "bench_mobilenet.js"), wb, mf, xb, str(batch),
+        r = subprocess.run([node, os.path.join(js, "bench_mobilenet.js"), mf, xb, str(batch),
                             str(steps), str(warmup)], capture_output=True, text=True, timeout=600)
     if r.returncode != 0:
         return dict(error=(r.stderr or r.stdout)[-400:])

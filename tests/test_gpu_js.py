@@ -187,22 +187,23 @@ def test_js_ops_match_oracle(tmp_path, ref):
 @pytest.mark.skipif(NODE is None, reason="node is not installed")
 @pytest.mark.parametrize("quant", [False, True])
 def test_js_mobilenet_matches_oracle(tmp_path, ref, quant):
-    """MobileNetV1 through the JS graph with weights loaded from a tfjs-style manifest +
-    binary; uint8 weights stay bytes in HBM (decodeWeightsToDevice)."""
+    """MobileNetV1 through the JS graph with weights loaded from a tfjs weights manifest and
+    its shard files (weights_loader.js); uint8 weights stay bytes in HBM."""
     from providers import oracle_mobilenet_forward
     from tfhip import mobilenet
     import bench
     params = mobilenet.make_params(seed=21)
     x = np.random.default_rng(22).uniform(0, 1, (1, 224, 224, 3)).astype(np.float32)
     store = mobilenet.quantize_params(params) if quant else params
-    bench.write_weight_files(store, str(tmp_path / "w.bin"), str(tmp_path / "manifest.json"))
+    manifest = bench.write_weight_files(store, str(tmp_path), shard_bytes=1 << 20)
+    assert len(os.listdir(str(tmp_path))) > (4 if quant else 10)   # really sharded
     if quant:
         params = {k: (ref.dequantize(*v) if isinstance(v, tuple) else v) for k, v in store.items()}
     want, _ = oracle_mobilenet_forward(ref, params, x)
     c = Cases(tmp_path)
     c.cases.append({"name": "mobilenet", "op": "mobilenet",
                     "inputs": {"x": c._put("mobilenet_x", x)},
-                    "attrs": {"weights": "w.bin", "manifest": "manifest.json", "onDevice": True}})
+                    "attrs": {"manifest": os.path.basename(manifest), "onDevice": True}})
     results = c.run()
     res = results["results"]["mobilenet"]
     assert "error" not in res, res.get("error")

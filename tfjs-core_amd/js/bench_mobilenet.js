@@ -1,8 +1,8 @@
 'use strict';
 // Throughput of the MobileNetV1 forward pass through the JavaScript host:
-//   node bench_mobilenet.js <weights.bin> <manifest.json> <input.bin> <batch> <steps> <warmup>
-// Weights / input are read from files written by the Python harness (so both hosts run the
-// same bytes); the input is uploaded once, before the timed region.  Prints one JSON line.
+//   node bench_mobilenet.js <weights_manifest.json> <input.bin> <batch> <steps> <warmup>
+// Weights (tfjs manifest + shard files) and input are written by the Python harness, so both
+// hosts run the same bytes; uint8 weights go to the device as bytes; the input is uploaded once, before the timed region.  Prints one JSON line.
 const fs = require('fs');
 const tf = require('./index.js');
 const mobilenet = require('./mobilenet.js');
@@ -12,11 +12,10 @@ function toArrayBuffer(buf) {
 }
 
 async function main() {
-  const [wPath, mPath, xPath, batchArg, stepsArg, warmArg] = process.argv.slice(2);
+  const [mPath, xPath, batchArg, stepsArg, warmArg] = process.argv.slice(2);
   const batch = +batchArg, steps = +stepsArg, warmup = +warmArg;
   await tf.setBackend('hip');
-  const manifest = JSON.parse(fs.readFileSync(mPath, 'utf8'));
-  const w = tf.io.decodeWeightsToDevice(toArrayBuffer(fs.readFileSync(wPath)), manifest);
+  const w = await tf.io.loadWeightsFromDisk(mPath, null, {toDevice: true});
   const xHost = new Float32Array(toArrayBuffer(fs.readFileSync(xPath)));
   const x = tf.tensor(xHost, [batch, 224, 224, 3]);
   const be = tf.backend();

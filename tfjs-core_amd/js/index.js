@@ -12,7 +12,7 @@ const util = require('./util');
 const conv_util = require('./conv_util');
 const broadcast_util = require('./broadcast_util');
 const axis_util = require('./axis_util');
-const io = require('./io_utils');
+const io = Object.assign({}, require('./io_utils'), require('./weights_loader'));
 
 const tf = Object.assign({}, ops, {
   Tensor, KernelBackend, DataStorage, ENV, util, io,

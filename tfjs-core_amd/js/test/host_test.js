@@ -312,6 +312,159 @@ test('decodeWeights: uint8 affine quantisation (io_utils_test.ts:468-494)', asyn
   });
 });
 
+// Known-answer cases of tfjs-core/src/io/weights_loader_test.ts:34-545, with the fetch spy
+// replaced by an in-memory file table that counts requests.
+function fakeFiles(table) {
+  const calls = [];
+  const fetch = async urls => urls.map(u => {
+    calls.push(u);
+    if (!(u in table)) throw new Error('no such file ' + u);
+    return table[u];
+  });
+  return {fetch, calls};
+}
+
+test('loadWeights: groups, name filter, dtypes (weights_loader_test.ts:34-176)', async () => {
+  await withBackend('storage-wl1', new StorageBackend(), async () => {
+    const f = fakeFiles({'./weightfile0': new Float32Array([1, 2, 3, 4, 5])});
+    const manifest = [{paths: ['weightfile0'], weights: [
+      {name: 'weight0', dtype: 'float32', shape: [2]},
+      {name: 'weight1', dtype: 'float32', shape: [3]}]}];
+    const load = tf.io.weightsLoaderFactory(f.fetch);
+    let w = await load(manifest, './', ['weight1']);
+    assert.deepStrictEqual(Object.keys(w), ['weight1']);
+    assert.deepStrictEqual(Array.from(w.weight1.dataSync()), [3, 4, 5]);
+    assert.deepStrictEqual(w.weight1.shape, [3]);
+    assert.strictEqual(f.calls.length, 1);
+    w = await load(manifest, './');   // no names: everything
+    assert.deepStrictEqual(Object.keys(w).sort(), ['weight0', 'weight1']);
+    assert.deepStrictEqual(Array.from(w.weight0.dataSync()), [1, 2]);
+
+    const buffer = new ArrayBuffer(5 * 4 + 1);
+    const view = new DataView(buffer);
+    view.setInt32(0, 1, true); view.setInt32(4, 2, true); view.setUint8(8, 1);
+    view.setFloat32(9, 3, true); view.setFloat32(13, 4, true); view.setFloat32(17, 5, true);
+    const g = fakeFiles({'./weightfile0': buffer});
+    const mixed = [{paths: ['weightfile0'], weights: [
+      {name: 'weight0', dtype: 'int32', shape: [2]},
+      {name: 'weight1', dtype: 'bool', shape: []},
+      {name: 'weight2', dtype: 'float32', shape: [3]}]}];
+    w = await tf.io.weightsLoaderFactory(g.fetch)(mixed, './', ['weight0', 'weight1', 'weight2']);
+    assert.deepStrictEqual(Array.from(w.weight0.dataSync()), [1, 2]);
+    assert.strictEqual(w.weight0.dtype, 'int32');
+    assert.deepStrictEqual(Array.from(w.weight1.dataSync()), [1]);
+    assert.strictEqual(w.weight1.dtype, 'bool');
+    assert.deepStrictEqual(w.weight1.shape, []);
+    assert.deepStrictEqual(Array.from(w.weight2.dataSync()), [3, 4, 5]);
+  });
+});
+
+test('loadWeights: weights sharded across files (weights_loader_test.ts:178-249)', async () => {
+  await withBackend('storage-wl2', new StorageBackend(), async () => {
+    let f = fakeFiles({'./weightfile0': new Float32Array([1, 2, 3, 4, 5]),
+                       './weightsfile1': new Float32Array([1.1, 2.2]),
+                       './weightsfile2': new Float32Array([10, 20, 30])});
+    let w = await tf.io.weightsLoaderFactory(f.fetch)(
+        [{paths: ['weightfile0', 'weightsfile1', 'weightsfile2'],
+          weights: [{name: 'weight0', dtype: 'float32', shape: [5, 2]}]}], './', ['weight0']);
+    assert.strictEqual(f.calls.length, 3);
+    assert.deepStrictEqual(Array.from(w.weight0.dataSync()),
+                           Array.from(new Float32Array([1, 2, 3, 4, 5, 1.1, 2.2, 10, 20, 30])));
+    assert.deepStrictEqual(w.weight0.shape, [5, 2]);
+
+    const shard1 = new ArrayBuffer(5 * 4);   // end of the first weight, start of the second
+    new Int32Array(shard1, 0, 2).set([10, 20]);
+    new Float32Array(shard1, 8, 3).set([3, 4, 5]);
+    f = fakeFiles({'./weightfile0': new Int32Array([1, 2, 3, 4, 5]), './weightsfile1': shard1,
+                   './weightsfile2': new Float32Array([10, 20, 30])});
+    w = await tf.io.weightsLoaderFactory(f.fetch)(
+        [{paths: ['weightfile0', 'weightsfile1', 'weightsfile2'],
+          weights: [{name: 'weight0', dtype: 'int32', shape: [7, 1]},
+                    {name: 'weight1', dtype: 'float32', shape: [3, 2]}]}], './',
+        ['weight0', 'weight1']);
+    assert.deepStrictEqual(Array.from(w.weight0.dataSync()), [1, 2, 3, 4, 5, 10, 20]);
+    assert.deepStrictEqual(Array.from(w.weight1.dataSync()), [3, 4, 5, 10, 20, 30]);
+  });
+});
+
+test('loadWeights: two groups, only the needed group is fetched (weights_loader_test.ts:251-385)', async () => {
+  await withBackend('storage-wl3', new StorageBackend(), async () => {
+    const files = {'./weightfile0': new Float32Array([1, 2, 3, 4, 5]),
+                   './weightfile1': new Float32Array([6, 7, 8, 9])};
+    const manifest = [
+      {paths: ['weightfile0'], weights: [{name: 'weight0', dtype: 'float32', shape: [2]},
+                                         {name: 'weight1', dtype: 'float32', shape: [3]}]},
+      {paths: ['weightfile1'], weights: [{name: 'weight2', dtype: 'float32', shape: [3, 1]},
+                                         {name: 'weight3', dtype: 'float32', shape: []}]}];
+    let f = fakeFiles(files);
+    let w = await tf.io.weightsLoaderFactory(f.fetch)(manifest, './', ['weight0', 'weight1']);
+    assert.deepStrictEqual(f.calls, ['./weightfile0']);
+    assert.deepStrictEqual(Array.from(w.weight1.dataSync()), [3, 4, 5]);
+    f = fakeFiles(files);
+    w = await tf.io.weightsLoaderFactory(f.fetch)(manifest, './', ['weight0', 'weight2']);
+    assert.strictEqual(f.calls.length, 2);
+    assert.deepStrictEqual(Array.from(w.weight0.dataSync()), [1, 2]);
+    assert.deepStrictEqual(Array.from(w.weight2.dataSync()), [6, 7, 8]);
+    assert.deepStrictEqual(w.weight2.shape, [3, 1]);
+    f = fakeFiles(files);
+    w = await tf.io.weightsLoaderFactory(f.fetch)(manifest, './');
+    assert.deepStrictEqual(Object.keys(w).sort(), ['weight0', 'weight1', 'weight2', 'weight3']);
+    assert.deepStrictEqual(Array.from(w.weight3.dataSync()), [9]);
+  });
+});
+
+test('loadWeights: missing name, unknown dtype, quantised groups (weights_loader_test.ts:387-545)', async () => {
+  await withBackend('storage-wl4', new StorageBackend(), async () => {
+    const f = fakeFiles({'./weightfile0': new Float32Array([1, 2, 3])});
+    const load = tf.io.weightsLoaderFactory(f.fetch);
+    await assert.rejects(load([{paths: ['weightfile0'], weights: [
+      {name: 'weight0', dtype: 'float32', shape: [3]}]}], './', ['doesntexist']),
+      /Could not find weights in manifest with names: doesntexist/);
+    await assert.rejects(load([{paths: ['weightfile0'], weights: [
+      {name: 'weight0', dtype: 'null', shape: [3]}]}], './', ['weight0']), /Unsupported dtype/);
+    for (const [qd, Arr] of [['uint8', Uint8Array], ['uint16', Uint16Array]]) {
+      const q = fakeFiles({'./weightfile0': new Arr([0, 48, 255, 0, 48, 255]),
+                           './weightfile1': new Float32Array([6, 7, 8, 9])});
+      const w = await tf.io.weightsLoaderFactory(q.fetch)([
+        {paths: ['weightfile0'], weights: [
+          {name: 'weight0', dtype: 'float32', shape: [3], quantization: {min: -1, scale: 0.1, dtype: qd}},
+          {name: 'weight1', dtype: 'int32', shape: [3], quantization: {min: -1, scale: 0.1, dtype: qd}}]},
+        {paths: ['weightfile1'], weights: [{name: 'weight2', dtype: 'float32', shape: [3, 1]},
+                                           {name: 'weight3', dtype: 'float32', shape: []}]}],
+        './', ['weight0', 'weight1', 'weight2']);
+      assert.deepStrictEqual(Array.from(w.weight0.dataSync()), Array.from(new Float32Array([-1, 3.8, 24.5])));
+      assert.deepStrictEqual(Array.from(w.weight1.dataSync()), [-1, 4, 25]);
+      assert.deepStrictEqual(Array.from(w.weight2.dataSync()), [6, 7, 8]);
+    }
+    // a group whose files are too short for its manifest is an error, not silent zeros
+    const short = fakeFiles({'./w': new Float32Array([1, 2])});
+    await assert.rejects(tf.io.weightsLoaderFactory(short.fetch)(
+        [{paths: ['w'], weights: [{name: 'a', dtype: 'float32', shape: [3]}]}], '.'),
+        /needs bytes 0\.\.12/);
+  });
+});
+
+test('loadWeightsFromDisk: manifest next to its shard files', async () => {
+  await withBackend('storage-wl5', new StorageBackend(), async () => {
+    const os = require('os');
+    const dir = fs.mkdtempSync(path.join(os.tmpdir(), 'tfhip-wl-'));
+    try {
+      fs.writeFileSync(path.join(dir, 'group1-shard1of2'), Buffer.from(new Float32Array([1, 2, 3]).buffer));
+      fs.writeFileSync(path.join(dir, 'group1-shard2of2'), Buffer.from(new Uint8Array([0, 48, 255]).buffer));
+      fs.writeFileSync(path.join(dir, 'model.json'), JSON.stringify({weightsManifest: [
+        {paths: ['group1-shard1of2', 'group1-shard2of2'], weights: [
+          {name: 'a', dtype: 'float32', shape: [3]},
+          {name: 'b', dtype: 'float32', shape: [3], quantization: {min: -1, scale: 0.1, dtype: 'uint8'}}]}]}));
+      const w = await tf.io.loadWeightsFromDisk(path.join(dir, 'model.json'));
+      assert.deepStrictEqual(Array.from(w.a.dataSync()), [1, 2, 3]);
+      assert.deepStrictEqual(Array.from(w.b.dataSync()), Array.from(new Float32Array([-1, 3.8, 24.5])));
+    } finally {
+      for (const f of fs.readdirSync(dir)) fs.unlinkSync(path.join(dir, f));
+      fs.rmdirSync(dir);
+    }
+  });
+});
+
 (async () => {
   let failed = 0;
   for (const t of tests) {

@@ -66,9 +66,8 @@ async function main() {
     const entry = {};
     try {
       if (c.op === 'mobilenet') {
-        const manifest = JSON.parse(fs.readFileSync(path.join(dir, c.attrs.manifest), 'utf8'));
-        const wbuf = toArrayBuffer(fs.readFileSync(path.join(dir, c.attrs.weights)));
-        const w = c.attrs.onDevice ? tf.io.decodeWeightsToDevice(wbuf, manifest) : tf.io.decodeWeights(wbuf, manifest);
+        const w = await tf.io.loadWeightsFromDisk(path.join(dir, c.attrs.manifest), null,
+                                                  {toDevice: !!c.attrs.onDevice});
         const x = load(c.inputs.x);
         const out = mobilenet.forward(tf, w, x);
         const logits = await out.logits.data();   // asynchronous read path
