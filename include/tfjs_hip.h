@@ -139,7 +139,12 @@ int tfhip_pool2d(tfhip_ctx* ctx, int64_t x, int64_t out, const tfhip_conv2d_info
  * (ops/broadcast_util.ts:27-87).  Shapes are right-aligned, rank <= 6. */
 enum {
   TFHIP_ADD = 0, TFHIP_SUB = 1, TFHIP_MUL = 2, TFHIP_DIV = 3, TFHIP_PRELU = 4,
-  TFHIP_MAXIMUM = 5, TFHIP_MINIMUM = 6
+  TFHIP_MAXIMUM = 5, TFHIP_MINIMUM = 6,
+  /* equal/notEqual/less/lessEqual/greater/greaterEqual/logicalAnd/logicalOr
+   * (backend.ts:202-233; backend_cpu.ts:747-820): out must be TFHIP_BOOL; NaN compares
+   * like JavaScript (only != is true). */
+  TFHIP_EQUAL = 7, TFHIP_NOT_EQUAL = 8, TFHIP_LESS = 9, TFHIP_LESS_EQUAL = 10,
+  TFHIP_GREATER = 11, TFHIP_GREATER_EQUAL = 12, TFHIP_LOGICAL_AND = 13, TFHIP_LOGICAL_OR = 14
 };
 int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_shape, int a_rank,
                  int64_t b, const int32_t* b_shape, int b_rank, int64_t out);
@@ -181,6 +186,35 @@ int tfhip_transpose(tfhip_ctx* ctx, int64_t x, const int32_t* x_shape, int rank,
                     const int32_t* perm, int64_t out);
 /* Device-to-device copy between ids of equal byte size (identity / clone). */
 int tfhip_copy(tfhip_ctx* ctx, int64_t x, int64_t out);
+/* Copy of a rank-d box between two strided views (rank <= 8, element strides, may be zero or
+ * negative on the source side):
+ *   out[out_offset + sum_d i_d*out_strides[d]] = x[x_offset + sum_d i_d*x_strides[d]],
+ *   0 <= i_d < region[d].
+ * One entry point for slice / stridedSlice / reverse (backend.ts:140-158; backend_cpu.ts:292-391),
+ * concat (backend.ts:160; backend_cpu.ts:393-433), pad (backend.ts:486; backend_cpu.ts:2157-2176, after
+ * tfhip_fill with the constant) and tile (backend.ts:484; backend_cpu.ts:2152-2155): the host
+ * states the box.  x and out must have the same element size; every touched index is checked
+ * against the buffers on the host. */
+int tfhip_strided_copy(tfhip_ctx* ctx, int64_t x, int64_t out, int rank, const int32_t* region,
+                       const int64_t* x_strides, int64_t x_offset, const int64_t* out_strides,
+                       int64_t out_offset);
+
+/* ---- further forward kernels of converter graphs ---------------------------------------- */
+/* logicalNot (backend.ts:225; backend_cpu.ts:795-804): bool -> bool. */
+int tfhip_logical_not(tfhip_ctx* ctx, int64_t x, int64_t out);
+/* batchNormalization (backend.ts:464-468; backend_cpu.ts:3167-3213):
+ *   out[i] = offset[i % |offset|] + (x[i] - mean[i % |mean|]) * scale[i % |scale|] /
+ *            sqrt(variance[i % |variance|] + epsilon);  scale / offset may be -1 (1 and 0). */
+int tfhip_batchnorm(tfhip_ctx* ctx, int64_t x, int64_t mean, int64_t variance, int64_t offset,
+                    int64_t scale, float epsilon, int64_t out);
+/* resizeBilinear (backend.ts:589-592; backend_cpu.ts:2875-2936): x [batch, in_h, in_w, c] ->
+ * out [batch, out_h, out_w, c] float32. */
+int tfhip_resize_bilinear(tfhip_ctx* ctx, int64_t x, int64_t out, int batch, int in_h, int in_w,
+                          int channels, int out_h, int out_w, int align_corners);
+/* oneHot (backend.ts:614-616; backend_cpu.ts:3325-3339): indices int32 [n] -> out [n, depth]
+ * (int32 or float32 storage); an index outside [0, depth) leaves its row at off_value. */
+int tfhip_one_hot(tfhip_ctx* ctx, int64_t indices, int64_t out, int depth, float on_value,
+                  float off_value);
 
 #ifdef __cplusplus
 }

@@ -442,3 +442,190 @@ def to_int(x):
     out = np.empty(x.shape, np.int32)
     lib().ref_float_to_int(_p(x), _p(out, C.c_int32), C.c_int64(x.size))
     return out
+
+
+# ---------------------------------------------------------------------------------------
+# data movement and pointwise kernels of converter graphs (numpy restatements; pinned by
+# the reference's slice/strided_slice/reverse/concat/pad/array_ops/compare/logical/
+# batchnorm/resize_bilinear tests in tests/golden)
+# ---------------------------------------------------------------------------------------
+def slice_(x, begin, size):
+    """backend_cpu.ts:292-313: out[loc] = x[loc + begin]."""
+    x = np.asarray(x)
+    out = np.empty(tuple(size), x.dtype)
+    for loc in np.ndindex(*size):
+        out[loc] = x[tuple(l + b for l, b in zip(loc, begin))]
+    return out
+
+
+def strided_slice(x, begin_index, size, strides):
+    """backend_cpu.ts:315-345: out[loc] = x[loc * strides + beginIndex] (beginIndex and
+    size from getStridedSlicedInfo, ops/slice_util.ts:48-93)."""
+    x = np.asarray(x)
+    out = np.empty(tuple(size), x.dtype)
+    for loc in np.ndindex(*size):
+        out[loc] = x[tuple(l * s + b for l, s, b in zip(loc, strides, begin_index))]
+    return out
+
+
+def reverse(x, axes):
+    """backend_cpu.ts:377-391."""
+    x = np.asarray(x)
+    out = np.empty_like(x)
+    for loc in np.ndindex(*x.shape):
+        src = list(loc)
+        for a in axes:
+            src[a] = x.shape[a] - 1 - src[a]
+        out[loc] = x[tuple(src)]
+    return out
+
+
+def concat(tensors, axis):
+    """backend_cpu.ts:393-433: every tensor as [outer, inner] rows written side by side."""
+    ts = [np.asarray(t) for t in tensors]
+    t2 = [t.reshape(-1, int(np.prod(t.shape[axis:], dtype=np.int64))) for t in ts]
+    rows = t2[0].shape[0]
+    out = np.empty((rows, sum(t.shape[1] for t in t2)), ts[0].dtype)
+    col = 0
+    for t in t2:
+        for r in range(rows):
+            out[r, col:col + t.shape[1]] = t[r]
+        col += t.shape[1]
+    shape = list(ts[0].shape)
+    shape[axis] = sum(t.shape[axis] for t in ts)
+    return out.reshape(shape)
+
+
+def pad(x, paddings, constant_value=0):
+    """backend_cpu.ts:2157-2176."""
+    x = np.asarray(x)
+    out = np.full([p[0] + d + p[1] for p, d in zip(paddings, x.shape)], constant_value, x.dtype)
+    for loc in np.ndindex(*x.shape):
+        out[tuple(c + p[0] for c, p in zip(loc, paddings))] = x[loc]
+    return out
+
+
+def tile(x, reps):
+    """ops/array_ops.ts tile / backends/backend_util tile: out[loc] = x[loc % x.shape]."""
+    x = np.asarray(x)
+    out = np.empty([d * r for d, r in zip(x.shape, reps)], x.dtype)
+    for loc in np.ndindex(*out.shape):
+        out[loc] = x[tuple(l % d for l, d in zip(loc, x.shape))]
+    return out
+
+
+def one_hot(indices, depth, on_value=1, off_value=0):
+    """backend_cpu.ts:3325-3339: int32 [n, depth]."""
+    idx = np.asarray(indices).ravel()
+    res = np.full((idx.size, depth), off_value, np.float32)
+    for e in range(idx.size):
+        if 0 <= idx[e] < depth:
+            res[e, idx[e]] = on_value
+    return _store(res.astype(np.float64), np.int32)
+
+
+def _compare(fn, a, b):
+    """broadcastedBinaryOp with a bool result (backend_cpu.ts:747-820, 3515-3549)."""
+    a, b = np.asarray(a), np.asarray(b)
+    shape = broadcast_shape(a.shape, b.shape)
+    a64 = np.broadcast_to(a.astype(np.float64), shape)
+    b64 = np.broadcast_to(b.astype(np.float64), shape)
+    out = np.empty(shape, np.uint8)
+    for loc in np.ndindex(*shape):
+        out[loc] = 1 if fn(float(a64[loc]), float(b64[loc])) else 0
+    return out
+
+
+def equal(a, b): return _compare(lambda p, q: p == q, a, b)
+def not_equal(a, b): return _compare(lambda p, q: p != q, a, b)
+def less(a, b): return _compare(lambda p, q: p < q, a, b)
+def less_equal(a, b): return _compare(lambda p, q: p <= q, a, b)
+def greater(a, b): return _compare(lambda p, q: p > q, a, b)
+def greater_equal(a, b): return _compare(lambda p, q: p >= q, a, b)
+def logical_and(a, b): return _compare(lambda p, q: bool(p) and bool(q), a, b)
+def logical_or(a, b): return _compare(lambda p, q: bool(p) or bool(q), a, b)
+
+
+def logical_not(x):
+    """backend_cpu.ts:795-804."""
+    return np.where(np.asarray(x) != 0, 0, 1).astype(np.uint8)
+
+
+def batch_normalization(x, mean, variance, variance_epsilon, scale=None, offset=None):
+    """backend_cpu.ts:3167-3213: flat loop, statistics indexed modulo their length, double
+    arithmetic, one float32 rounding at the store."""
+    x = np.asarray(x, np.float32)
+    xv = x.ravel().astype(np.float64)
+    m = np.asarray(mean, np.float32).ravel().astype(np.float64)
+    v = np.asarray(variance, np.float32).ravel().astype(np.float64)
+    s = np.ones(1) if scale is None else np.asarray(scale, np.float32).ravel().astype(np.float64)
+    o = np.zeros(1) if offset is None else np.asarray(offset, np.float32).ravel().astype(np.float64)
+    eps = float(variance_epsilon)
+    out = np.empty(xv.size, np.float64)
+    for i in range(xv.size):
+        out[i] = o[i % o.size] + (xv[i] - m[i % m.size]) * s[i % s.size] / math.sqrt(
+            v[i % v.size] + eps)
+    return _store(out, np.float32).reshape(x.shape)
+
+
+def resize_bilinear(x, new_height, new_width, align_corners):
+    """backend_cpu.ts:2875-2936."""
+    x = np.asarray(x, np.float32)
+    batch, old_h, old_w, ch = x.shape
+    xv = x.astype(np.float64)
+    eff_in = ((old_h - 1) if (align_corners and new_height > 1) else old_h,
+              (old_w - 1) if (align_corners and new_width > 1) else old_w)
+    eff_out = ((new_height - 1) if (align_corners and new_height > 1) else new_height,
+               (new_width - 1) if (align_corners and new_width > 1) else new_width)
+    ratio_r, ratio_c = eff_in[0] / eff_out[0], eff_in[1] / eff_out[1]
+    out = np.empty((batch, new_height, new_width, ch), np.float64)
+    for b in range(batch):
+        for r in range(new_height):
+            fr = ratio_r * r
+            r0 = math.floor(fr)
+            wr = fr - r0
+            r1 = min(old_h - 1, math.ceil(fr))
+            for c in range(new_width):
+                fc = ratio_c * c
+                c0 = math.floor(fc)
+                wc = fc - c0
+                c1 = min(old_w - 1, math.ceil(fc))
+                top = xv[b, r0, c0] + (xv[b, r0, c1] - xv[b, r0, c0]) * wc
+                bot = xv[b, r1, c0] + (xv[b, r1, c1] - xv[b, r1, c0]) * wc
+                out[b, r, c] = top + (bot - top) * wr
+    return _store(out, np.float32)
+
+
+def strided_slice_info(shape, begin, end, strides, begin_mask=0, end_mask=0,
+                       shrink_axis_mask=0):
+    """getStridedSlicedInfo / startForAxis / stopForAxis (ops/slice_util.ts:48-188)."""
+    big = float(2 ** 53 - 1)
+    starts, stops, shrink = [], [], []
+    for axis, n in enumerate(shape):
+        stride = (strides[axis] if axis < len(strides) else 0) or 1
+        start = begin[axis] if axis < len(begin) else None
+        if (begin_mask >> axis) & 1 or start is None:
+            start = -big if stride > 0 else big
+        if start < 0:
+            start += n
+        start = int(min(max(start, 0), n - 1))
+        stop = end[axis] if axis < len(end) else None
+        if (end_mask >> axis) & 1 or stop is None:
+            stop = big if stride > 0 else -big
+        if stop < 0:
+            stop += n
+        stop = int(min(max(stop, 0), n)) if stride > 0 else int(min(max(stop, -1), n - 1))
+        if (shrink_axis_mask >> axis) & 1:
+            stop = start + 1
+            shrink.append(axis)
+        starts.append(start)
+        stops.append(stop)
+    sizes = []
+    for axis in range(len(shape)):
+        stride = (strides[axis] if axis < len(strides) else 0) or 1
+        if stride > 0:
+            count = len(range(starts[axis], stops[axis], stride))
+        else:
+            count = len(range(starts[axis], stops[axis], stride))
+        sizes.append(count)
+    return starts, sizes, shrink

@@ -43,6 +43,21 @@ CASES = {
     "gather": ("tfjs-core/src/ops/array_ops_test.ts", ["gather"]),
     "transpose": ("tfjs-core/src/ops/transpose_test.ts", ["transpose"]),
     "dequant": ("tfjs-core/src/io/io_utils_test.ts", ["decodeWeights"]),
+    "slice": ("tfjs-core/src/ops/slice_test.ts",
+              ["slice1d", "slice2d", "slice3d", "slice4d", "slice5d", "slice6d"]),
+    "strided_slice": ("tfjs-core/src/ops/strided_slice_test.ts", ["stridedSlice"]),
+    "reverse": ("tfjs-core/src/ops/reverse_test.ts",
+                ["reverse1d", "reverse2d", "reverse3d", "reverse4d"]),
+    "concat": ("tfjs-core/src/ops/concat_test.ts", ["concat1d", "concat2d", "concat3d"]),
+    "pad": ("tfjs-core/src/ops/pad_test.ts", ["pad1d", "pad2d", "pad4d", "pad"]),
+    "tile_onehot": ("tfjs-core/src/ops/array_ops_test.ts", ["tile", "oneHot"]),
+    "compare": ("tfjs-core/src/ops/compare_ops_test.ts",
+                ["equal", "notEqual", "less", "lessEqual", "greater", "greaterEqual"]),
+    "logical": ("tfjs-core/src/ops/logical_ops_test.ts",
+                ["logicalNot", "logicalAnd", "logicalOr"]),
+    "batchnorm": ("tfjs-core/src/ops/batchnorm_test.ts",
+                  ["batchNorm4D", "batchNorm3D", "batchNorm2D"]),
+    "resize_bilinear": ("tfjs-core/src/ops/resize_bilinear_test.ts", ["resizeBilinear"]),
 }
 # blocks whose title matches are not forward known-answer cases
 SKIP = re.compile(r"grad|throw|raises|tensor-like|TensorLike|does not match|do not match|"

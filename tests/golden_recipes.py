@@ -448,3 +448,289 @@ def dequant_uint8_known_answer(ops):
     a = golden_case("dequant", "support quantization uint8 weights")["arrays"]
     q = np.array(a[1][:3], np.uint8)  # bytes [0,48,255]; scale 0.1, min -1 (io_utils_test.ts:470-477)
     expect_close(ops.dequantize(q, 0.1, -1.0), a[2], eps=1e-6)
+
+
+# ---- ops/slice_test.ts, strided_slice_test.ts, reverse_test.ts ---------------------------
+@recipe
+def slice_known_answers(ops):
+    g = lambda d, t: golden_case("slice", t, d)["arrays"]
+    a = g("slice1d", "slices 5x1 into shape 2x1 starting at 3")      # a.slice1d... begin 3, size 2
+    assert ops.slice(f32(a[0]), [3], [2]).tolist() == a[2]
+    a = g("slice1d", "slices 5x1 into shape 3x1 starting at 1")
+    assert ops.slice(f32(a[0]), [1], [3]).tolist() == a[2]
+    a = g("slice2d", "returns the rectangle specified")
+    assert ops.slice(f32(a[0], a[1]), a[2], a[3]).ravel().tolist() == a[4]
+    a = g("slice2d", "slice a tensor that was not continous in memory")
+    assert ops.slice(f32(a[0]), a[1], [3, 3]).ravel().tolist() == a[3]
+    for d, titles in (("slice3d", ("slices 2x2x2 array into 1x2x2 starting at [1, 0, 0]",
+                                   "slices 2x2x2 array into 2x1x1 starting at [0, 1, 1]")),
+                      ("slice4d", ("slices 2x2x2x2 array into 1x2x2x2 starting at [1, 0, 0, 0]",
+                                   "slices 2x2x2x2 array into 2x1x1x1 starting at [0, 1, 1, 1]")),
+                      ("slice5d", ("slices 2x2x2x2x2 array into 1x2x2x2x2 starting at [1,0,0,0,0]",
+                                   "slices 2x2x2x2x2 array into 2x1x1x1x1 starting at [0,1,1,1,1]")),
+                      ("slice6d", ("slices 2x2x2x2x2x2 array into 1x2x2x2x2x2 starting at [1,0,0,0,0,0]",
+                                   "slices 2x2x2x2x2x2 array into 2x1x1x1x1x1 starting at [0,1,1,1,1,1]"))):
+        for t in titles:
+            a = g(d, t)   # [x, x shape, begin, size, result shape, expected]
+            r = ops.slice(f32(a[0], a[1]), a[2], a[3])
+            assert list(r.shape) == a[4] and r.ravel().tolist() == [float(v) for v in a[5]]
+
+
+# (title, beginMask, endMask, shrinkAxisMask) — the masks are call arguments of
+# ops/strided_slice_test.ts:92,133,140,204,212,219,273 that the extractor does not see
+_STRIDED_1D = [("stridedSlice should support 1d tensor", 0, 0, 0),
+               ("stridedSlice should support 1d tensor empty result", 0, 0, 0),
+               ("stridedSlice should support 1d tensor negative begin", 0, 0, 0),
+               ("stridedSlice should support 1d tensor out of range begin", 0, 0, 0),
+               ("stridedSlice should support 1d tensor negative end", 0, 0, 0),
+               ("stridedSlice should support 1d tensor out of range end", 0, 0, 0),
+               ("stridedSlice should support 1d tensor begin mask", 1, 0, 0),
+               ("stridedSlice should support 1d tensor nagtive begin and stride", 0, 0, 0),
+               ("stridedSlice should support 1d tensor nagtive end and stride", 0, 0, 0),
+               ("stridedSlice should support 1d tensor end mask", 0, 1, 0),
+               ("stridedSlice should support 1d tensor shrink axis mask", 0, 0, 1),
+               ("stridedSlice should support 1d tensor negative stride", 0, 0, 0),
+               ("stridedSlice should support 1d tensor even length stride", 0, 0, 0),
+               ("stridedSlice should support 1d tensor odd length stride", 0, 0, 0)]
+_STRIDED_ND = [("stridedSlice should support 2d tensor identity", 0, 0, 0),
+               ("stridedSlice should support 2d tensor", 0, 0, 0),
+               ("stridedSlice should support 2d tensor strides", 0, 0, 0),
+               ("stridedSlice should support 2d tensor negative strides", 0, 0, 0),
+               ("stridedSlice should support 2d tensor begin mask", 1, 0, 0),
+               ("stridedSlice should support 2d tensor shrink mask", 0, 0, 1),
+               ("stridedSlice should support 2d tensor end mask", 0, 2, 0),
+               ("stridedSlice should support 3d tensor identity", 0, 0, 0),
+               ("stridedSlice should support 3d tensor negative stride", 0, 0, 0),
+               ("stridedSlice should support 3d tensor strided 2", 0, 0, 0),
+               ("stridedSlice should support 3d tensor shrink mask", 0, 0, 1),
+               ("stridedSlice should support 3d with smaller length of begin array", 0, 0, 0),
+               ("stridedSlice should support 3d with smaller length of end array", 0, 0, 0),
+               ("stridedSlice should support 3d with smaller length of stride array", 0, 0, 0)]
+
+
+@recipe
+def strided_slice_known_answers(ops):
+    for title, bm, em, sm in _STRIDED_1D:
+        a = golden_case("strided_slice", title)["arrays"]   # [x, begin, end, strides, shape, expected]
+        r = ops.strided_slice(f32(a[0]), a[1], a[2], a[3], bm, em, sm)
+        assert list(r.shape) == a[4], (title, r.shape)
+        assert r.ravel().tolist() == [float(v) for v in a[5]], title
+    for title, bm, em, sm in _STRIDED_ND:
+        a = golden_case("strided_slice", title)["arrays"]   # [x, x shape, begin, end, strides, shape, expected]
+        r = ops.strided_slice(f32(a[0], a[1]), a[2], a[3], a[4], bm, em, sm)
+        assert list(r.shape) == a[5], (title, r.shape)
+        assert r.ravel().tolist() == [float(v) for v in a[6]], title
+
+
+@recipe
+def reverse_known_answers(ops):
+    g = lambda d, t: golden_case("reverse", t, d)["arrays"]
+    for t in ("reverse a 1D array", "reverse a 1D array, even length"):
+        a = g("reverse1d", t)
+        assert ops.reverse(f32(a[0]), [0]).tolist() == a[1]
+    for t in ("reverse a 2D array at axis [0]", "reverse a 2D array at axis [1]",
+              "reverse a 2D array odd rows and columns at axis [0, 1]"):
+        a = g("reverse2d", t)   # [axes, x, shape, expected]
+        assert ops.reverse(f32(a[1], a[2]), a[0]).ravel().tolist() == a[3]
+    # reverse_test.ts:145-149, 249-254: the inputs are 0..23 as [2,3,4] and 0..71 as [3,2,3,4]
+    x3 = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    for axes in ("[0]", "[1]", "[2]", "[0, 1]", "[0, 2]", "[1, 2]"):
+        a = g("reverse3d", "reverse a 3D array at axis " + axes)
+        assert ops.reverse(x3, a[0]).ravel().tolist() == a[1]
+    x4 = np.arange(72, dtype=np.float32).reshape(3, 2, 3, 4)
+    for axes in ("[0]", "[1]", "[2]", "[3]", "[0, 2]", "[1, 3]"):
+        a = g("reverse4d", "reverse a 4D array at axis " + axes)
+        assert ops.reverse(x4, a[0]).ravel().tolist() == a[1]
+
+
+# ---- ops/concat_test.ts, pad_test.ts, array_ops_test.ts (tile, oneHot) -------------------
+@recipe
+def concat_known_answers(ops):
+    g = lambda d, t: golden_case("concat", t, d)
+    for t in ("3 + 5", "3 + [5,7]", "[3,5] + 7"):
+        a = g("concat1d", t)["arrays"]
+        assert ops.concat([f32(a[0]), f32(a[1])], 0).tolist() == a[3]
+    a = g("concat1d", "3 + 5 + 7 + 9")["arrays"]
+    assert ops.concat([f32(v) for v in a[:4]], 0).tolist() == a[5]
+    for t in ("[[3]] + [[5]], axis=0", "[[3]] + [[5]], axis=1",
+              "[[1, 2], [3, 4]] + [[5, 6]], axis=0", "[[1, 2], [3, 4]] + [[5, 6], [7, 8]], axis=1"):
+        c = g("concat2d", t)
+        a = c["arrays"]   # [a, a shape, b, b shape, -, expected, expected shape]
+        r = ops.concat([f32(a[0], a[1]), f32(a[2], a[3])], c["consts"]["axis"])
+        assert list(r.shape) == a[6] and r.ravel().tolist() == a[5]
+    for t in ("[[1, 2],[3, 4]] + [[5, 6]] + [[7, 8]], axis=0",
+              "[[1, 2],[3, 4]] + [[5, 6],[7, 8]] + [[9, 10],[11, 12]], axis=1"):
+        c = g("concat2d", t)
+        a = c["arrays"]   # [a, b, c, -, expected, expected shape]
+        r = ops.concat([f32(a[0]), f32(a[1]), f32(a[2])], c["consts"]["axis"])
+        assert list(r.shape) == a[5] and r.ravel().tolist() == a[4]
+    for t, axis in (("concat axis=0", 0), ("concat axis=1", 1), ("concat axis=2", 2)):
+        a = g("concat3d", t)["arrays"]   # [a, a shape, b, b shape, -, expected shape, expected]
+        r = ops.concat([f32(a[0], a[1]), f32(a[2], a[3])], axis)
+        assert list(r.shape) == a[5] and r.ravel().tolist() == a[6]
+
+
+@recipe
+def pad_known_answers(ops):
+    g = lambda d, t: golden_case("pad", t, d)["arrays"]
+    a = g("pad1d", "Should pad 1D arrays")
+    expect_close(ops.pad(f32(a[0]), [tuple(a[1])]), a[2], eps=0)
+    a = g("pad1d", "Should handle padding with custom value")   # values 9 and 1.1 (pad_test.ts:40-52)
+    expect_close(ops.pad(f32(a[0]), [tuple(a[1])], 9), a[2], eps=0)
+    expect_close(ops.pad(f32(a[3]), [tuple(a[4])], 1.1), a[5], eps=1e-6)
+    a = g("pad1d", "Should handle NaNs with 1D arrays")
+    expect_close(ops.pad(f32(a[0]), [tuple(a[1])]), a[2], eps=0)
+    a = g("pad2d", "Should pad 2D arrays")   # [x, shape, paddings, expected] twice
+    for k in (0, 4):
+        r = ops.pad(f32(a[k], a[k + 1]), [tuple(p) for p in a[k + 2]])
+        expect_close(r, a[k + 3], eps=0)
+    a = g("pad2d", "Should handle padding with custom value")   # value 10 (pad_test.ts:121)
+    expect_close(ops.pad(f32(a[0], a[1]), [tuple(p) for p in a[2]], 10), a[3], eps=0)
+    a = g("pad4d", "Should pad 4D arrays")
+    r = ops.pad(f32(a[0], a[1]), [tuple(p) for p in a[2]])
+    assert list(r.shape) == a[4]
+    expect_close(r, np.array(a[3], np.float32), eps=0)
+
+
+@recipe
+def tile_and_one_hot_known_answers(ops):
+    g = lambda d, t: golden_case("tile_onehot", t, d)["arrays"]
+    a = g("tile", "1D (tile)")   # [x, reps, shape, expected]
+    r = ops.tile(f32(a[0]), a[1])
+    assert list(r.shape) == a[2] and r.tolist() == a[3]
+    a = g("tile", "2D (tile)")   # [x, x shape] then (reps, shape, expected) x3
+    x = f32(a[0], a[1])
+    for k in (2, 5, 8):
+        r = ops.tile(x, a[k])
+        assert list(r.shape) == a[k + 1] and r.ravel().tolist() == a[k + 2]
+    for t in ("3D (tile)", "4D (tile)"):
+        a = g("tile", t)   # [x, x shape, reps, shape, expected]
+        r = ops.tile(f32(a[0], a[1]), a[2])
+        assert list(r.shape) == a[3] and r.ravel().tolist() == a[4]
+    a = g("tile", "propagates NaNs")
+    expect_close(ops.tile(f32(a[0]), a[1]), a[3], eps=0)
+    a = g("tile", "2D int32 (tile)")
+    r = ops.tile(np.array(a[0], np.int32).reshape(a[1]), a[2])
+    assert r.dtype == np.int32 and r.ravel().tolist() == a[4]
+    a = g("tile", "1D bool (tile)")
+    r = ops.tile(np.array(a[0], np.bool_), a[1])
+    assert r.ravel().astype(int).tolist() == a[3]
+    for t, depth, on, off in (("Depth 2, diagonal", 2, 1, 0), ("Depth 2, transposed diagonal", 2, 1, 0),
+                              ("Depth 3, 4 events", 3, 1, 0),
+                              ("Out of range events do not trigger onValue", 5, 1, 0),
+                              ("Depth 2 onValue=3, offValue=-2", 2, 3, -2)):
+        a = g("oneHot", t)   # [indices, shape, expected]
+        r = ops.one_hot(np.array(a[0], np.int32), depth, on, off)
+        assert list(r.shape) == a[1] and r.ravel().tolist() == a[2], t
+    a = g("oneHot", "oneHot with indices as 2d")
+    r = ops.one_hot(np.array(a[0], np.int32), 4)
+    assert list(r.shape) == [2, 2, 4] and r.ravel().tolist() == a[3]
+
+
+# ---- ops/compare_ops_test.ts, logical_ops_test.ts -----------------------------------------
+_COMPARE = {"equal": "equal", "notEqual": "not_equal", "less": "less", "lessEqual": "less_equal",
+            "greater": "greater", "greaterEqual": "greater_equal"}
+
+
+def _typed(a, shape, dtype):
+    return np.array(a, dtype=dtype).reshape(shape) if shape is not None else np.array(a, dtype=dtype)
+
+
+@recipe
+def compare_known_answers(ops):
+    for describe, method in _COMPARE.items():
+        for kind, dt in (("int32", np.int32), ("float32", np.float32)):
+            a = golden_case("compare", "Tensor1D - " + kind, describe)["arrays"]
+            for k in range(0, len(a), 3):
+                r = ops.compare(method, _typed(a[k], None, dt), _typed(a[k + 1], None, dt))
+                assert r.astype(int).tolist() == a[k + 2], (describe, kind, k)
+            for rank in ("2D", "3D", "4D"):
+                a = golden_case("compare", "Tensor%s - %s" % (rank, kind), describe)["arrays"]
+                for k in range(0, len(a), 5):
+                    r = ops.compare(method, _typed(a[k], a[k + 1], dt), _typed(a[k + 2], a[k + 3], dt))
+                    assert r.ravel().astype(int).tolist() == a[k + 4], (describe, rank, kind, k)
+                try:
+                    a = golden_case("compare", "broadcasting Tensor%s shapes - %s" % (rank, kind),
+                                    describe)["arrays"]
+                except KeyError:   # a few blocks spell the title without "shapes -"
+                    a = golden_case("compare", "broadcasting Tensor%s %s" % (rank, kind),
+                                    describe)["arrays"]
+                r = ops.compare(method, _typed(a[0], a[1], dt), _typed(a[2], a[3], dt))
+                assert r.ravel().astype(int).tolist() == a[4], (describe, rank, kind)
+        a = golden_case("compare", "NaNs in Tensor1D - float32", describe)["arrays"]
+        r = ops.compare(method, f32(a[0]), f32(a[1]))
+        assert r.astype(int).tolist() == a[2], describe
+        for rank in ("2D", "3D", "4D"):
+            a = golden_case("compare", "NaNs in Tensor%s - float32" % rank, describe)["arrays"]
+            r = ops.compare(method, f32(a[0], a[1]), f32(a[2], a[3]))
+            assert r.ravel().astype(int).tolist() == a[4], (describe, rank)
+
+
+@recipe
+def logical_known_answers(ops):
+    b = lambda a, shape=None: _typed(a, shape, np.bool_)
+    a = golden_case("logical", "Tensor1D.", "logicalNot")["arrays"]
+    for k in range(0, len(a), 2):
+        assert ops.logical_not(b(a[k])).astype(int).tolist() == a[k + 1]
+    a = golden_case("logical", "Tensor2D", "logicalNot")["arrays"]
+    for k in range(0, len(a), 3):
+        assert ops.logical_not(b(a[k], a[k + 1])).ravel().astype(int).tolist() == a[k + 2]
+    for describe, method in (("logicalAnd", "logical_and"), ("logicalOr", "logical_or")):
+        a = golden_case("logical", "Tensor1D.", describe)["arrays"]
+        for k in range(0, len(a), 3):
+            assert ops.compare(method, b(a[k]), b(a[k + 1])).astype(int).tolist() == a[k + 2]
+        for rank in ("2D", "3D", "4D"):
+            a = golden_case("logical", "Tensor" + rank, describe)["arrays"]
+            for k in range(0, len(a), 5):
+                r = ops.compare(method, b(a[k], a[k + 1]), b(a[k + 2], a[k + 3]))
+                assert r.ravel().astype(int).tolist() == np.ravel(a[k + 4]).tolist(), (describe, rank, k)
+            a = golden_case("logical", "broadcasting Tensor%s shapes" % rank, describe)["arrays"]
+            r = ops.compare(method, b(a[0], a[1]), b(a[2], a[3]))
+            assert r.ravel().astype(int).tolist() == a[4], (describe, rank)
+
+
+# ---- ops/batchnorm_test.ts, resize_bilinear_test.ts ----------------------------------------
+@recipe
+def batchnorm_known_answers(ops):
+    # batchnorm_test.ts:23-152 and twins: the expected values are the closed form itself,
+    # evaluated here in float64; varianceEpsilon = .001
+    eps = 0.001
+    for describe, rank in (("batchNorm4D", "4D"), ("batchNorm3D", "3D"), ("batchNorm2D", "2D")):
+        dims = {"4D": "2x1x1x2", "3D": "2x1x2", "2D": "2x2"}[rank]
+        for variant in ("no offset or scale", "no offset", "no scale", "full"):
+            title = "simple batchnorm%s, %s%s" % (rank, "" if variant == "full" else variant + ", ", dims)
+            a = golden_case("batchnorm", title, describe)["arrays"]
+            x, mean, var = f32(a[0], a[1]), f32(a[2]), f32(a[3])
+            scale = offset = None
+            if variant == "no offset":
+                scale = f32(a[4])
+            elif variant == "no scale":
+                offset = f32(a[4])
+            elif variant == "full":
+                offset, scale = f32(a[4]), f32(a[5])   # offsetT then scaleT (batchnorm_test.ts:104-106)
+            want = ((x.astype(np.float64) - mean) * (1 if scale is None else scale.astype(np.float64))
+                    / np.sqrt(var.astype(np.float64) + eps) + (0 if offset is None else offset))
+            expect_close(ops.batch_norm(x, mean, var, offset, scale, eps), want)
+    a = golden_case("batchnorm", "batchnorm2D matches tensorflow, 3x3", "batchNorm2D")["arrays"]
+    # [x, shape, mean, variance, offset, scale, expected] with varianceEpsilon .001 (:884-904)
+    expect_close(ops.batch_norm(f32(a[0], a[1]), f32(a[2]), f32(a[3]), f32(a[4]), f32(a[5]), eps),
+                 a[6])
+    a = golden_case("batchnorm", "batchnorm matches tensorflow, 2x3x3", "batchNorm3D")["arrays"]
+    expect_close(ops.batch_norm(f32(a[0], a[1]), f32(a[2]), f32(a[3]), f32(a[4]), f32(a[5]), eps),
+                 a[6])
+
+
+@recipe
+def resize_bilinear_known_answers(ops):
+    g = lambda t: golden_case("resize_bilinear", t)["arrays"]
+    a = g("simple alignCorners=false")   # expected holds 10/3 (resize_bilinear_test.ts:27-28)
+    expect_close(ops.resize_bilinear(f32(a[0], a[1]), a[2], False),
+                 [2, 2, 2, 10 / 3, 10 / 3, 10 / 3, 4, 4, 4])
+    a = g("simple alignCorners=true")
+    expect_close(ops.resize_bilinear(f32(a[0], a[1]), a[2], True), a[3])
+    for t, align in (("matches tensorflow w/ random numbers alignCorners=false", False),
+                     ("matches tensorflow w/ random numbers alignCorners=true", True)):
+        a = g(t)   # [x, shape, size, expected]
+        expect_close(ops.resize_bilinear(f32(a[0], a[1]), a[2], align), a[3])
+    a = g("batch of 2, simple, alignCorners=true")
+    expect_close(ops.resize_bilinear(f32(a[0], a[1]), a[2], True), a[3])

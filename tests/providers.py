@@ -66,6 +66,37 @@ class OracleOps:
     def transpose(self, x, perm): return self.r.transpose(x, perm)
     def dequantize(self, q, scale, min_): return self.r.dequantize_u8(q, scale, min_)
     def to_int(self, x): return self.r.to_int(x)
+    def slice(self, x, begin, size): return self.r.slice_(x, begin, size)
+
+    def strided_slice(self, x, begin, end, strides, begin_mask=0, end_mask=0, shrink_mask=0):
+        strides = list(strides) + [1] * (np.ndim(x) - len(strides))
+        start, size, shrink = self.r.strided_slice_info(np.shape(x), begin, end, strides,
+                                                        begin_mask, end_mask, shrink_mask)
+        shape = [d for i, d in enumerate(size) if i not in shrink]
+        if 0 in shape:
+            return np.zeros(shape, np.asarray(x).dtype)
+        return self.r.strided_slice(x, start, size, strides).reshape(shape)
+
+    def reverse(self, x, axes): return self.r.reverse(x, axes)
+    def concat(self, xs, axis): return self.r.concat(xs, axis)
+    def pad(self, x, paddings, value=0): return self.r.pad(x, paddings, value)
+    def tile(self, x, reps): return self.r.tile(x, reps)
+
+    def one_hot(self, idx, depth, on=1, off=0):
+        idx = np.asarray(idx)
+        return self.r.one_hot(idx, depth, on, off).reshape(idx.shape + (depth,))
+
+    def compare(self, name, a, b): return getattr(self.r, name)(a, b)
+    def logical_not(self, x): return self.r.logical_not(x)
+
+    def batch_norm(self, x, mean, variance, offset=None, scale=None, eps=0.001):
+        return self.r.batch_normalization(x, mean, variance, eps, scale, offset)
+
+    def resize_bilinear(self, x, size, align_corners=False):
+        x = np.asarray(x, np.float32)
+        x4 = x if x.ndim == 4 else x[None]
+        r = self.r.resize_bilinear(x4, size[0], size[1], align_corners)
+        return r if x.ndim == 4 else r[0]
 
 
 class HipOps:
@@ -149,6 +180,33 @@ class HipOps:
             return tf.dequantize(tf.quantized_tensor(q, scale, min_)).data_sync()
 
     def to_int(self, x): return self._run(lambda t: self.tf.cast(t, "int32"), x)
+    def slice(self, x, begin, size): return self._run(lambda t: self.tf.slice(t, begin, size), x)
+
+    def strided_slice(self, x, begin, end, strides, begin_mask=0, end_mask=0, shrink_mask=0):
+        return self._run(lambda t: self.tf.strided_slice(t, begin, end, strides, begin_mask,
+                                                         end_mask, 0, 0, shrink_mask), x)
+
+    def reverse(self, x, axes): return self._run(lambda t: self.tf.reverse(t, axes), x)
+    def concat(self, xs, axis): return self._run(lambda *ts: self.tf.concat(list(ts), axis), *xs)
+    def pad(self, x, paddings, value=0): return self._run(lambda t: self.tf.pad(t, paddings, value), x)
+    def tile(self, x, reps): return self._run(lambda t: self.tf.tile(t, reps), x)
+    def one_hot(self, idx, depth, on=1, off=0):
+        return self._run(lambda t: self.tf.one_hot(t, depth, on, off), np.asarray(idx, np.int32))
+    def compare(self, name, a, b): return self._run(getattr(self.tf, name), a, b)
+    def logical_not(self, x): return self._run(self.tf.logical_not, x)
+
+    def batch_norm(self, x, mean, variance, offset=None, scale=None, eps=0.001):
+        arrs = [x, mean, variance] + [a for a in (offset, scale) if a is not None]
+
+        def run(xt, mt, vt, *rest):
+            rest = list(rest)
+            ot = rest.pop(0) if offset is not None else None
+            st = rest.pop(0) if scale is not None else None
+            return self.tf.batch_norm(xt, mt, vt, ot, st, eps)
+        return self._run(run, *arrs)
+
+    def resize_bilinear(self, x, size, align_corners=False):
+        return self._run(lambda t: self.tf.resize_bilinear(t, size, align_corners), x)
 
 
 def oracle_mobilenet_forward(ref, params, x):

@@ -184,6 +184,68 @@ def test_js_ops_match_oracle(tmp_path, ref):
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
 
 
+def test_js_graph_ops_match_oracle(tmp_path, ref):
+    """The data-movement and pointwise kernels of converter graphs through the JS host."""
+    rng = np.random.default_rng(43)
+    c = Cases(tmp_path)
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)
+    x = f(3, 9, 7, 5)
+    c.add("slice", "slice", dict(x=x), dict(begin=[1, 2, 0, 1], size=[2, 5, 7, 3]),
+          ref.slice(x, [1, 2, 0, 1], [2, 5, 7, 3]), exact=True)
+    c.add("slice_short", "slice", dict(x=x), dict(begin=[1], size=[1]),
+          ref.slice(x, [1, 0, 0, 0], [1, 9, 7, 5]), exact=True)
+    c.add("strided", "stridedSlice", dict(x=x),
+          dict(begin=[2, 8, 0, 0], end=[-4, 0, 7, 5], strides=[-1, -3, 2, 1], beginMask=0,
+               endMask=0, shrinkAxisMask=0),
+          ref.strided_slice(x, [2, 8, 0, 0], [-4, 0, 7, 5], [-1, -3, 2, 1]), exact=True)
+    c.add("strided_shrink", "stridedSlice", dict(x=x),
+          dict(begin=[1, 0, 0, 0], end=[3, 9, 7, 5], strides=[1, 2, 1, 1], beginMask=0, endMask=0,
+               shrinkAxisMask=1),
+          ref.strided_slice(x, [1, 0, 0, 0], [3, 9, 7, 5], [1, 2, 1, 1], 0, 0, 1), exact=True)
+    c.add("reverse", "reverse", dict(x=x), dict(axis=[1, 3]), ref.reverse(x, [1, 3]), exact=True)
+    a, b, d = f(2, 3, 4), f(2, 5, 4), f(2, 1, 4)
+    c.add("concat3", "concat", dict(a=a, b=b, c=d), dict(axis=1), ref.concat([a, b, d], 1), exact=True)
+    ai = rng.integers(-9, 9, (2, 3)).astype(np.int32)
+    bi = rng.integers(-9, 9, (4, 3)).astype(np.int32)
+    c.add("concat_int", "concat", dict(a=ai, b=bi), dict(axis=0), ref.concat([ai, bi], 0), exact=True)
+    pads = [[0, 0], [1, 2], [3, 0], [0, 1]]
+    c.add("pad", "pad", dict(x=x), dict(paddings=pads, constantValue=-1.5),
+          ref.pad(x, [tuple(p) for p in pads], -1.5), exact=True)
+    t = f(2, 3, 2)
+    c.add("tile", "tile", dict(x=t), dict(reps=[2, 1, 3]), ref.tile(t, [2, 1, 3]), exact=True)
+    idx = np.array([[0, 3], [9, -1]], np.int32)
+    c.add("one_hot", "oneHot", dict(indices=idx), dict(depth=5, onValue=4, offValue=-2),
+          ref.one_hot(idx, 5, 4, -2), exact=True)
+    p, q = f(4, 1, 6), f(5, 6)
+    p[0, 0, 1], q[1, 2] = np.nan, np.nan
+    q[0, :] = p[1, 0, :]
+    for name, py in (("equal", "equal"), ("notEqual", "not_equal"), ("less", "less"),
+                     ("lessEqual", "less_equal"), ("greater", "greater"),
+                     ("greaterEqual", "greater_equal")):
+        c.add("cmp_" + name, "compare", dict(a=p, b=q), dict(name=name), ref.compare(py, p, q), exact=True)
+    ba, bb = rng.integers(0, 2, (3, 1, 4)).astype(np.bool_), rng.integers(0, 2, (2, 4)).astype(np.bool_)
+    c.add("logical_and", "compare", dict(a=ba, b=bb), dict(name="logicalAnd"),
+          ref.compare("logical_and", ba, bb), exact=True)
+    c.add("logical_or", "compare", dict(a=ba, b=bb), dict(name="logicalOr"),
+          ref.compare("logical_or", ba, bb), exact=True)
+    c.add("logical_not", "logicalNot", dict(x=ba), {}, ref.logical_not(ba), exact=True)
+    xb, mean, var = f(2, 4, 4, 8) * 2, f(8), rng.uniform(0.2, 2, 8).astype(np.float32)
+    off, sc = f(8), f(8)
+    c.add("batchnorm_full", "batchNorm", dict(x=xb, mean=mean, variance=var, offset=off, scale=sc),
+          dict(varianceEpsilon=1e-3), ref.batch_norm(xb, mean, var, off, sc, 1e-3))
+    c.add("batchnorm_plain_2d", "batchNorm", dict(x=xb.reshape(32, 8), mean=mean, variance=var), {},
+          ref.batch_norm(xb.reshape(32, 8), mean, var, None, None, 0.001))
+    img = f(2, 5, 6, 3)
+    for align in (False, True):
+        c.add("resize_%s" % align, "resizeBilinear", dict(x=img), dict(size=[9, 4], alignCorners=align),
+              ref.resize_bilinear(img, [9, 4], align))
+    c.add("resize_rank3", "resizeBilinear", dict(x=img[0]), dict(size=[10, 12], alignCorners=False),
+          ref.resize_bilinear(img[0], [10, 12], False))
+    results = c.run()
+    c.check(results)
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
 @pytest.mark.skipif(NODE is None, reason="node is not installed")
 @pytest.mark.parametrize("quant", [False, True])
 def test_js_mobilenet_matches_oracle(tmp_path, ref, quant):

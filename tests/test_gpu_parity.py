@@ -362,3 +362,109 @@ def test_uint8_weights_dequantised_in_kernel(hip, ref):
             r = tf.depthwise_conv2d(tf.tensor(x), tf.quantized_tensor(qf, scale, mn), 1,
                                     "same").data_sync()
         close(r, ref.depthwise_conv2d(x, ref.dequantize(qf, scale, mn), 1, "same"))
+
+
+# ------------------------------------- data movement around the convolutions ----
+@pytest.mark.parametrize("dtype", [np.float32, np.int32, np.bool_])
+def test_box_copies_bit_exact(hip, ref, dtype):
+    """slice / stridedSlice / reverse / concat / pad / tile move elements unchanged."""
+    rng = np.random.default_rng(77)
+
+    def arr(*shape):
+        if dtype == np.bool_:
+            return rng.integers(0, 2, shape).astype(np.bool_)
+        if dtype == np.int32:
+            return rng.integers(-1000, 1000, shape).astype(np.int32)
+        return rng.standard_normal(shape).astype(np.float32)
+
+    x = arr(3, 17, 9, 5)
+    for begin, size in (([0, 0, 0, 0], [3, 17, 9, 5]), ([1, 4, 2, 1], [2, 9, 6, 3]),
+                        ([2, 16, 8, 4], [1, 1, 1, 1]), ([0, 3, 0, 0], [3, 5, 9, 5])):
+        assert np.array_equal(hip.slice(x, begin, size), ref.slice(x, begin, size))
+    for begin, end, strides, bm, em, sm in (
+            ([0, 0, 0, 0], [3, 17, 9, 5], [1, 2, 3, 1], 0, 0, 0),
+            ([2, 16, -1, 4], [-4, 0, -10, -6], [-1, -3, -2, -1], 0, 0, 0),
+            ([1, 2, 3, 1], [2, 9, 7, 4], [1, 1, 2, 2], 5, 10, 0),
+            ([1, 5, 0, 0], [3, 17, 9, 5], [1, 4, 1, 1], 0, 0, 1)):
+        assert np.array_equal(hip.strided_slice(x, begin, end, strides, bm, em, sm),
+                              ref.strided_slice(x, begin, end, strides, bm, em, sm))
+    for axes in ([0], [3], [1, 2], [0, 1, 2, 3]):
+        assert np.array_equal(hip.reverse(x, axes), ref.reverse(x, axes))
+    for axis, shapes in ((0, [(2, 5, 4), (3, 5, 4), (1, 5, 4)]), (1, [(2, 1, 4), (2, 7, 4)]),
+                         (2, [(3, 3, 64), (3, 3, 1), (3, 3, 33)])):
+        xs = [arr(*s) for s in shapes]
+        assert np.array_equal(hip.concat(xs, axis), ref.concat(xs, axis))
+    y = arr(2, 6, 7, 3)
+    for pads, value in (([(0, 0), (1, 1), (1, 1), (0, 0)], 0), ([(1, 0), (0, 2), (3, 1), (2, 2)], 1)):
+        assert np.array_equal(hip.pad(y, pads, value), ref.pad(y, pads, value))
+    for shape, reps in (((5,), [3]), ((2, 3), [2, 2]), ((2, 3, 4), [1, 2, 3]), ((1, 2, 2, 3), [2, 1, 3, 2])):
+        t = arr(*shape)
+        assert np.array_equal(hip.tile(t, reps), ref.tile(t, reps))
+
+
+def test_pad_float_constant_and_nan(hip, ref):
+    x = np.array([[1.5, np.nan], [-2.0, 4.0]], np.float32)
+    got, want = hip.pad(x, [(1, 2), (2, 0)], -0.75), ref.pad(x, [(1, 2), (2, 0)], -0.75)
+    assert np.array_equal(got, want, equal_nan=True)
+
+
+@pytest.mark.parametrize("name", ["equal", "not_equal", "less", "less_equal", "greater",
+                                  "greater_equal"])
+@pytest.mark.parametrize("sa,sb", [((4, 5), (4, 5)), ((4, 1), (1, 5)), ((), (3, 2)), ((2, 3, 4), (4,))])
+def test_comparisons_bit_exact(hip, ref, name, sa, sb):
+    rng = np.random.default_rng(5)
+    a = rng.integers(-3, 4, sa).astype(np.float32)
+    b = rng.integers(-3, 4, sb).astype(np.float32)
+    if a.size > 3:
+        a.flat[1], a.flat[2] = np.nan, np.inf
+    if b.size > 3:
+        b.flat[2], b.flat[3] = np.inf, np.nan
+    got = hip.compare(name, a, b)
+    assert got.dtype in (np.uint8, np.bool_)
+    assert np.array_equal(got.astype(np.uint8), ref.compare(name, a, b))
+    ai, bi = rng.integers(-3, 4, sa).astype(np.int32), rng.integers(-3, 4, sb).astype(np.int32)
+    assert np.array_equal(hip.compare(name, ai, bi).astype(np.uint8), ref.compare(name, ai, bi))
+    big = np.array([16777217, 16777216], np.int32)   # differ only beyond float32 precision
+    assert np.array_equal(hip.compare(name, big, big[::-1].copy()).astype(np.uint8),
+                          ref.compare(name, big, big[::-1].copy()))
+
+
+def test_logical_ops_bit_exact(hip, ref):
+    rng = np.random.default_rng(6)
+    a = rng.integers(0, 2, (3, 1, 5)).astype(np.bool_)
+    b = rng.integers(0, 2, (4, 5)).astype(np.bool_)
+    for name in ("logical_and", "logical_or"):
+        assert np.array_equal(hip.compare(name, a, b).astype(np.uint8), ref.compare(name, a, b))
+    assert np.array_equal(hip.logical_not(a).astype(np.uint8), ref.logical_not(a))
+
+
+@pytest.mark.parametrize("stat_shape", ["channel", "full", "row"])
+@pytest.mark.parametrize("with_scale,with_offset", [(False, False), (True, False), (False, True),
+                                                    (True, True)])
+def test_batch_norm(hip, ref, stat_shape, with_scale, with_offset):
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((2, 5, 6, 8)).astype(np.float32) * 3
+    shape = {"channel": (8,), "full": x.shape, "row": (1, 1, 6, 8)}[stat_shape]
+    mean = rng.standard_normal(shape).astype(np.float32)
+    var = rng.uniform(0.1, 2.0, shape).astype(np.float32)
+    scale = rng.standard_normal(shape).astype(np.float32) if with_scale else None
+    offset = rng.standard_normal(shape).astype(np.float32) if with_offset else None
+    close(hip.batch_norm(x, mean, var, offset, scale, 1e-3),
+          ref.batch_norm(x, mean, var, offset, scale, 1e-3))
+
+
+@pytest.mark.parametrize("in_hw,out_hw", [((5, 7), (10, 14)), ((9, 6), (4, 3)), ((4, 4), (7, 1)),
+                                          ((3, 5), (1, 9)), ((1, 1), (3, 3)), ((8, 8), (8, 8))])
+@pytest.mark.parametrize("align", [False, True])
+def test_resize_bilinear(hip, ref, in_hw, out_hw, align):
+    rng = np.random.default_rng(in_hw[0] * 100 + out_hw[1])
+    x = rng.standard_normal((2,) + in_hw + (3,)).astype(np.float32)
+    close(hip.resize_bilinear(x, out_hw, align), ref.resize_bilinear(x, out_hw, align))
+    x3 = x[0]
+    close(hip.resize_bilinear(x3, out_hw, align), ref.resize_bilinear(x3, out_hw, align))
+
+
+def test_one_hot_bit_exact(hip, ref):
+    idx = np.array([[0, 3, -1], [7, 2, 99]], np.int32)
+    got = hip.one_hot(idx, 8, 5, -1)
+    assert got.dtype == np.int32 and np.array_equal(got, ref.one_hot(idx, 8, 5, -1))

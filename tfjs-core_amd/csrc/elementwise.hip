@@ -39,7 +39,15 @@ __device__ __forceinline__ float bin_f(int op, float a, float b) {
     case TFHIP_DIV: return a / b;
     case TFHIP_PRELU: return a < 0.f ? b * a : a;
     case TFHIP_MAXIMUM: return (a != a || b != b) ? NAN : (a > b ? a : b);
-    default: return (a != a || b != b) ? NAN : (a < b ? a : b);
+    case TFHIP_MINIMUM: return (a != a || b != b) ? NAN : (a < b ? a : b);
+    case TFHIP_EQUAL: return a == b;
+    case TFHIP_NOT_EQUAL: return a != b;
+    case TFHIP_LESS: return a < b;
+    case TFHIP_LESS_EQUAL: return a <= b;
+    case TFHIP_GREATER: return a > b;
+    case TFHIP_GREATER_EQUAL: return a >= b;
+    case TFHIP_LOGICAL_AND: return (a != 0.f) && (b != 0.f);
+    default: return (a != 0.f) || (b != 0.f);
   }
 }
 __device__ __forceinline__ int64_t bin_i(int op, int64_t a, int64_t b) {
@@ -49,7 +57,15 @@ __device__ __forceinline__ int64_t bin_i(int op, int64_t a, int64_t b) {
     case TFHIP_MUL: return a * b;
     case TFHIP_PRELU: return a < 0 ? b * a : a;
     case TFHIP_MAXIMUM: return a > b ? a : b;
-    default: return a < b ? a : b;
+    case TFHIP_MINIMUM: return a < b ? a : b;
+    case TFHIP_EQUAL: return a == b;
+    case TFHIP_NOT_EQUAL: return a != b;
+    case TFHIP_LESS: return a < b;
+    case TFHIP_LESS_EQUAL: return a <= b;
+    case TFHIP_GREATER: return a > b;
+    case TFHIP_GREATER_EQUAL: return a >= b;
+    case TFHIP_LOGICAL_AND: return a && b;
+    default: return a || b;
   }
 }
 
@@ -88,14 +104,15 @@ __global__ void binary_kernel(int op, const void* a, int a_dt, int64_t a_len, co
         }
       }
     }
-    if (sizeof(OutT) == 4 && ((a_dt != TFHIP_FLOAT32 && b_dt != TFHIP_FLOAT32 && op != TFHIP_DIV))) {
+    if (a_dt != TFHIP_FLOAT32 && b_dt != TFHIP_FLOAT32 && op != TFHIP_DIV) {
       // integer arithmetic when neither operand is float (int32 / bool tensors)
       const int64_t r = bin_i(op, load_i(a, a_dt, ia), load_i(b, b_dt, ib));
       if (std::is_same<OutT, float>::value) out[i] = (OutT)r;
-      else out[i] = (OutT)(int32_t)(uint32_t)r;
+      else out[i] = (OutT)(int32_t)(uint32_t)r;   // comparisons yield 0 / 1
     } else {
       const float r = bin_f(op, load_f(a, a_dt, ia), load_f(b, b_dt, ib));
       if (std::is_same<OutT, float>::value) out[i] = (OutT)r;
+      else if (sizeof(OutT) == 1) out[i] = (OutT)(r != 0.f);
       else out[i] = (OutT)to_int32(r);
     }
   }
@@ -226,15 +243,17 @@ extern "C" int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_
                             int a_rank, int64_t b, const int32_t* b_shape, int b_rank,
                             int64_t out) {
   if (!ctx) return TFHIP_EINVAL;
-  if (op < TFHIP_ADD || op > TFHIP_MINIMUM) return ctx->fail(TFHIP_EINVAL, "binary: unknown op %d", op);
+  if (op < TFHIP_ADD || op > TFHIP_LOGICAL_OR) return ctx->fail(TFHIP_EINVAL, "binary: unknown op %d", op);
+  const bool predicate = op >= TFHIP_EQUAL;
   if (a_rank < 0 || b_rank < 0 || a_rank > MAXR || b_rank > MAXR)
     return ctx->fail(TFHIP_ENOTSUP, "binary: rank above %d", MAXR);
   TFHIP_GET(ctx, ba, a);
   TFHIP_GET(ctx, bb, b);
   TFHIP_GET(ctx, bo, out);
   if (ba->dtype == TFHIP_UINT8Q || bb->dtype == TFHIP_UINT8Q || bo->dtype == TFHIP_UINT8Q ||
-      bo->dtype == TFHIP_BOOL)
-    return ctx->fail(TFHIP_EINVAL, "binary: unsupported storage dtype");
+      (bo->dtype == TFHIP_BOOL) != predicate)
+    return ctx->fail(TFHIP_EINVAL, "binary: unsupported storage dtype (comparisons and logical "
+                                   "ops write bool, arithmetic writes float32 or int32)");
   // assertAndGetBroadcastShape (ops/broadcast_util.ts:61-87)
   const int rank = a_rank > b_rank ? a_rank : b_rank;
   BcastArgs bc = {};
@@ -269,7 +288,7 @@ extern "C" int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_
   const bool all_f32 = ba->dtype == TFHIP_FLOAT32 && bb->dtype == TFHIP_FLOAT32 &&
                        bo->dtype == TFHIP_FLOAT32;
   const int block = 256;
-  if (all_f32 && a_len == n && b_len == n && n % 4 == 0 && aligned16(ba->ptr) &&
+  if (!predicate && all_f32 && a_len == n && b_len == n && n % 4 == 0 && aligned16(ba->ptr) &&
       aligned16(bb->ptr) && aligned16(bo->ptr)) {
     hipLaunchKernelGGL(binary_f32_vec_kernel, dim3(grid_for(ctx, n / 4, block)), dim3(block), 0,
                        ctx->stream, op, (const f32x4*)ba->ptr, (const f32x4*)bb->ptr,
@@ -278,7 +297,7 @@ extern "C" int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_
     return TFHIP_OK;
   }
   const int last = rank ? bc.out_dim[rank - 1] : 1;
-  if (all_f32 && !a_bcast && !b_bcast && last % 4 == 0 && aligned16(ba->ptr) &&
+  if (!predicate && all_f32 && !a_bcast && !b_bcast && last % 4 == 0 && aligned16(ba->ptr) &&
       aligned16(bb->ptr) && aligned16(bo->ptr) &&
       ((a_len == n && b_len == last) || (b_len == n && a_len == last))) {
     const bool b_small = b_len == last && a_len == n;
@@ -294,6 +313,9 @@ extern "C" int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_
   if (bo->dtype == TFHIP_FLOAT32)
     hipLaunchKernelGGL(binary_kernel<float>, grid, dim3(block), 0, ctx->stream, op, ba->ptr,
                        ba->dtype, a_len, bb->ptr, bb->dtype, b_len, (float*)bo->ptr, n, mode, bc);
+  else if (bo->dtype == TFHIP_BOOL)
+    hipLaunchKernelGGL(binary_kernel<uint8_t>, grid, dim3(block), 0, ctx->stream, op, ba->ptr,
+                       ba->dtype, a_len, bb->ptr, bb->dtype, b_len, (uint8_t*)bo->ptr, n, mode, bc);
   else
     hipLaunchKernelGGL(binary_kernel<int32_t>, grid, dim3(block), 0, ctx->stream, op, ba->ptr,
                        ba->dtype, a_len, bb->ptr, bb->dtype, b_len, (int32_t*)bo->ptr, n, mode, bc);

@@ -403,6 +403,86 @@ static napi_value js_transpose(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+/* Float64Array -> pointer + length (element strides and offsets: exact up to 2^53) */
+static int arg_f64_array(napi_env env, napi_value v, const double** data, size_t* len) {
+  napi_typedarray_type type;
+  void* p;
+  if (napi_get_typedarray_info(env, v, &type, len, &p, NULL, NULL) != napi_ok ||
+      type != napi_float64_array) {
+    napi_throw_type_error(env, NULL, "tfjs_hip.node: expected a Float64Array");
+    return 0;
+  }
+  *data = (const double*)p;
+  return 1;
+}
+
+/* stridedCopy(ctx, x, out, region Int32Array, xStrides Float64Array, xOffset,
+ *             outStrides Float64Array, outOffset) */
+static napi_value js_strided_copy(napi_env env, napi_callback_info info) {
+  ARGS(8);
+  I64(1, x); I64(2, out);
+  const int32_t* region; size_t rank;
+  if (!arg_i32_array(env, argv[3], &region, &rank)) return NULL;
+  const double *xs, *os; size_t nx, no;
+  if (!arg_f64_array(env, argv[4], &xs, &nx)) return NULL;
+  I64(5, x_off);
+  if (!arg_f64_array(env, argv[6], &os, &no)) return NULL;
+  I64(7, out_off);
+  if (nx != rank || no != rank || rank > 8) {
+    napi_throw_type_error(env, NULL, "tfjs_hip.node: box arrays differ in length or rank > 8");
+    return NULL;
+  }
+  int64_t xs64[8], os64[8];
+  for (size_t i = 0; i < rank; i++) {
+    xs64[i] = (int64_t)xs[i];
+    os64[i] = (int64_t)os[i];
+  }
+  CHECK(tfhip_strided_copy(ctx, x, out, (int)rank, region, xs64, x_off, os64, out_off));
+  return undefined(env);
+}
+
+/* logicalNot(ctx, x, out) */
+static napi_value js_logical_not(napi_env env, napi_callback_info info) {
+  ARGS(3);
+  I64(1, x); I64(2, out);
+  CHECK(tfhip_logical_not(ctx, x, out));
+  return undefined(env);
+}
+
+/* batchnorm(ctx, x, mean, variance, offset|-1, scale|-1, epsilon, out) */
+static napi_value js_batchnorm(napi_env env, napi_callback_info info) {
+  ARGS(8);
+  I64(1, x); I64(2, mean); I64(3, variance); I64(4, offset); I64(5, scale);
+  double eps;
+  if (!arg_f64(env, argv[6], &eps)) return NULL;
+  I64(7, out);
+  CHECK(tfhip_batchnorm(ctx, x, mean, variance, offset, scale, (float)eps, out));
+  return undefined(env);
+}
+
+/* resizeBilinear(ctx, x, out, batch, inH, inW, channels, outH, outW, alignCorners) */
+static napi_value js_resize_bilinear(napi_env env, napi_callback_info info) {
+  ARGS(10);
+  I64(1, x); I64(2, out);
+  int v[7];
+  for (int i = 0; i < 7; i++)
+    if (!arg_int(env, argv[3 + i], &v[i])) return NULL;
+  CHECK(tfhip_resize_bilinear(ctx, x, out, v[0], v[1], v[2], v[3], v[4], v[5], v[6]));
+  return undefined(env);
+}
+
+/* oneHot(ctx, indices, out, depth, onValue, offValue) */
+static napi_value js_one_hot(napi_env env, napi_callback_info info) {
+  ARGS(6);
+  I64(1, idx); I64(2, out);
+  int depth;
+  if (!arg_int(env, argv[3], &depth)) return NULL;
+  double on, off;
+  if (!arg_f64(env, argv[4], &on) || !arg_f64(env, argv[5], &off)) return NULL;
+  CHECK(tfhip_one_hot(ctx, idx, out, depth, (float)on, (float)off));
+  return undefined(env);
+}
+
 static napi_value module_init(napi_env env, napi_value exports) {
   static const struct { const char* name; napi_callback fn; } fns[] = {
       {"init", js_init}, {"destroy", js_destroy}, {"register", js_register},
@@ -412,7 +492,10 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"conv2d", js_conv2d}, {"depthwiseConv2d", js_depthwise}, {"pool2d", js_pool2d},
       {"binary", js_binary}, {"unary", js_unary}, {"cast", js_cast}, {"copy", js_copy},
       {"dequantize", js_dequantize}, {"fill", js_fill}, {"reduce", js_reduce},
-      {"softmaxRows", js_softmax_rows}, {"gather", js_gather}, {"transpose", js_transpose}};
+      {"softmaxRows", js_softmax_rows}, {"gather", js_gather}, {"transpose", js_transpose},
+      {"stridedCopy", js_strided_copy}, {"logicalNot", js_logical_not},
+      {"batchnorm", js_batchnorm}, {"resizeBilinear", js_resize_bilinear},
+      {"oneHot", js_one_hot}};
   for (size_t i = 0; i < sizeof fns / sizeof fns[0]; i++) {
     napi_value f;
     if (napi_create_function(env, fns[i].name, NAPI_AUTO_LENGTH, fns[i].fn, NULL, &f) != napi_ok ||

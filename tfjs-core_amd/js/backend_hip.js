@@ -18,7 +18,9 @@ const {ENV} = require('./environment');
 const DTYPE = {float32: 0, int32: 1, bool: 2, uint8q: 3};
 const ACT = {linear: 0, relu: 1, prelu: 2, relu6: 3};
 const BCAST = {NONE: 0, SCALAR: 1, COLUMN: 2, FULL: 3};
-const BINARY = {add: 0, sub: 1, mul: 2, div: 3, prelu: 4, maximum: 5, minimum: 6};
+const BINARY = {add: 0, sub: 1, mul: 2, div: 3, prelu: 4, maximum: 5, minimum: 6, equal: 7,
+                notEqual: 8, less: 9, lessEqual: 10, greater: 11, greaterEqual: 12,
+                logicalAnd: 13, logicalOr: 14};
 const UNARY = {relu: 0, clip: 1, exp: 2, log: 3, neg: 4, abs: 5, sigmoid: 6, sqrt: 7, square: 8,
                tanh: 9, rsqrt: 10};
 const REDUCE = {sum: 0, max: 1, min: 2, argMax: 3, argMin: 4};
@@ -378,6 +380,131 @@ class MathBackendHIP extends KernelBackend {
     const idx = this.storageCode(indices) === DTYPE.int32 ? indices : this.int(indices);
     this.napi.gather(this.ctx, this.h(x), this.h(idx), this.h(out), outer, x.shape[axis], inner,
                      indices.size);
+    return out;
+  }
+
+  // ---- strided box copies (backend.ts:140-160, 484-486): slice / stridedSlice / reverse /
+  //      concat / pad / tile all state a box for the one stridedCopy entry point ----
+  boxCopy(x, out, region, xStrides, xOffset, outStrides, outOffset) {
+    this.napi.stridedCopy(this.ctx, this.h(x), this.h(out), Int32Array.from(region),
+                          Float64Array.from(xStrides), xOffset, Float64Array.from(outStrides),
+                          outOffset);
+  }
+  // x with its stored element type equal to its dtype (a widening cast aliases narrower
+  // storage, backends/backend_util.ts:34-71)
+  materialized(x) {
+    this.h(x);
+    if (this.storageCode(x) === DTYPE[x.dtype]) return x;
+    const out = this.out(x.shape, x.dtype);
+    this.napi.cast(this.ctx, this.h(x), this.h(out));
+    return out;
+  }
+  slice(x, begin, size) {
+    const out = this.outLikeStorage(size.slice(), x);
+    const xs = util.computeStrides(x.shape).concat([1]);
+    const at = begin.reduce((acc, b, i) => acc + b * xs[i], 0);
+    if (util.sizeFromShape(size) > 0) {
+      this.boxCopy(x, out, size, xs, at, util.computeStrides(size).concat([1]), 0);
+    }
+    return out;
+  }
+  // after getStridedSlicedInfo (ops/slice_util.ts:48-93): out[loc] = x[loc * strides + begin]
+  stridedSliceBox(x, beginIndex, size, strides) {
+    const out = this.outLikeStorage(size.slice(), x);
+    const xs = util.computeStrides(x.shape).concat([1]);
+    const at = beginIndex.reduce((acc, b, i) => acc + b * xs[i], 0);
+    this.boxCopy(x, out, size, xs.map((s, i) => s * strides[i]), at,
+                 util.computeStrides(size).concat([1]), 0);
+    return out;
+  }
+  reverse(x, axis) {
+    const out = this.outLikeStorage(x.shape.slice(), x);
+    if (x.size === 0) return out;
+    const xs = util.computeStrides(x.shape).concat([1]);
+    const at = axis.reduce((acc, a) => acc + (x.shape[a] - 1) * xs[a], 0);
+    this.boxCopy(x, out, x.shape, xs.map((s, i) => axis.indexOf(i) >= 0 ? -s : s), at, xs, 0);
+    return out;
+  }
+  concat(tensors, axis) {
+    tensors = tensors.map(t => this.materialized(t));
+    const outShape = tensors[0].shape.slice();
+    outShape[axis] = tensors.reduce((acc, t) => acc + t.shape[axis], 0);
+    const out = this.out(outShape, tensors[0].dtype);
+    const os = util.computeStrides(outShape).concat([1]);
+    let at = 0;
+    for (const t of tensors) {
+      if (t.size > 0) {
+        this.boxCopy(t, out, t.shape, util.computeStrides(t.shape).concat([1]), 0, os,
+                     at * os[axis]);
+      }
+      at += t.shape[axis];
+    }
+    return out;
+  }
+  pad(x, paddings, constantValue) {
+    const outShape = paddings.map((p, i) => p[0] + x.shape[i] + p[1]);
+    const out = this.outLikeStorage(outShape, x);
+    this.napi.fill(this.ctx, this.h(out), +constantValue);
+    const os = util.computeStrides(outShape).concat([1]);
+    if (x.size > 0) {
+      this.boxCopy(x, out, x.shape, util.computeStrides(x.shape).concat([1]), 0, os,
+                   paddings.reduce((acc, p, i) => acc + p[0] * os[i], 0));
+    }
+    return out;
+  }
+  // out[loc] = x[loc % x.shape]: a box of rank 2*rank whose repetition axes read with stride 0
+  tile(x, reps) {
+    const outShape = x.shape.map((d, i) => d * reps[i]);
+    const out = this.outLikeStorage(outShape, x);
+    if (util.sizeFromShape(outShape) === 0) return out;
+    if (2 * x.rank > 8) throw new Error('hip backend: tile of rank above 4 is not implemented');
+    const xs = util.computeStrides(x.shape).concat([1]);
+    const os = util.computeStrides(outShape).concat([1]);
+    const region = [], xst = [], ost = [];
+    for (let d = 0; d < x.rank; d++) {
+      region.push(reps[d], x.shape[d]);
+      xst.push(0, xs[d]);
+      ost.push(os[d] * x.shape[d], os[d]);
+    }
+    this.boxCopy(x, out, region, xst, 0, ost, 0);
+    return out;
+  }
+
+  // ---- comparison / logical (backend.ts:202-233) ----
+  equal(a, b) { return this.binary('equal', a, b, 'bool'); }
+  notEqual(a, b) { return this.binary('notEqual', a, b, 'bool'); }
+  less(a, b) { return this.binary('less', a, b, 'bool'); }
+  lessEqual(a, b) { return this.binary('lessEqual', a, b, 'bool'); }
+  greater(a, b) { return this.binary('greater', a, b, 'bool'); }
+  greaterEqual(a, b) { return this.binary('greaterEqual', a, b, 'bool'); }
+  logicalAnd(a, b) { return this.binary('logicalAnd', a, b, 'bool'); }
+  logicalOr(a, b) { return this.binary('logicalOr', a, b, 'bool'); }
+  logicalNot(x) {
+    x = this.materialized(x);
+    const out = this.out(x.shape, 'bool');
+    this.napi.logicalNot(this.ctx, this.h(x), this.h(out));
+    return out;
+  }
+
+  // ---- batchNormalization / resizeBilinear / oneHot (backend.ts:464-468, 589-592, 614-616) ----
+  batchNormalization(x, mean, variance, varianceEpsilon, scale, offset) {
+    const out = this.out(x.shape, 'float32');
+    this.napi.batchnorm(this.ctx, this.h(x), this.h(mean), this.h(variance),
+                        offset == null ? -1 : this.h(offset), scale == null ? -1 : this.h(scale),
+                        varianceEpsilon, this.h(out));
+    return out;
+  }
+  resizeBilinear(x, newHeight, newWidth, alignCorners) {
+    const [batch, h, w, c] = x.shape;
+    const out = this.out([batch, newHeight, newWidth, c], 'float32');
+    this.napi.resizeBilinear(this.ctx, this.h(x), this.h(out), batch, h, w, c, newHeight, newWidth,
+                             alignCorners ? 1 : 0);
+    return out;
+  }
+  oneHot(indices, depth, onValue, offValue) {
+    const idx = this.materialized(indices);
+    const out = this.out([indices.size, depth], 'int32');
+    this.napi.oneHot(this.ctx, this.h(idx), this.h(out), depth, onValue, offValue);
     return out;
   }
 

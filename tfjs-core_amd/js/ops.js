@@ -456,6 +456,229 @@ const transpose = op('transpose', (x, perm) => {
   return ENGINE.runKernel(backend => backend.transpose($x, perm), {$x});
 });
 
+// ---- slice / stridedSlice / reverse (ops/slice.ts, ops/slice_util.ts, ops/strided_slice.ts,
+//      ops/reverse.ts) ----
+const slice = op('slice', (x, begin, size) => {
+  const $x = convertToTensor(x, 'x', 'slice');
+  if ($x.rank === 0) throw new Error('Slicing scalar is not possible');
+  let begin_;
+  if (typeof begin === 'number') begin_ = [begin].concat(new Array($x.rank - 1).fill(0));
+  else if (begin.length < $x.rank) begin_ = begin.concat(new Array($x.rank - begin.length).fill(0));
+  else begin_ = begin.slice();
+  let size_;
+  if (size == null) size_ = new Array($x.rank).fill(-1);
+  else if (typeof size === 'number') size_ = [size].concat(new Array($x.rank - 1).fill(-1));
+  else if (size.length < $x.rank) size_ = size.concat(new Array($x.rank - size.length).fill(-1));
+  else size_ = size;
+  size_ = size_.map((d, i) => {
+    if (d >= 0) return d;
+    util.assert(d === -1, () => 'Bad value in size');
+    return $x.shape[i] - begin_[i];
+  });
+  util.assert($x.rank === begin_.length,
+              () => `Error in slice${$x.rank}D: Length of begin ${begin_} must match the rank of ` +
+                    `the array (${$x.rank}).`);
+  util.assert($x.rank === size_.length,
+              () => `Error in slice${$x.rank}D: Length of size ${size_} must match the rank of ` +
+                    `the array (${$x.rank}).`);
+  for (let i = 0; i < $x.rank; ++i) {
+    util.assert(begin_[i] + size_[i] <= $x.shape[i],
+                () => `Error in slice${$x.rank}D: begin[${i}] + size[${i}] ` +
+                      `(${begin_[i] + size_[i]}) would overflow input.shape[${i}] (${$x.shape[i]})`);
+  }
+  return ENGINE.runKernel(backend => backend.slice($x, begin_, size_), {$x});
+});
+
+const clampInt = (lo, v, hi) => Math.max(lo, Math.min(v, hi));
+
+// getStridedSlicedInfo (ops/slice_util.ts:48-188): [begin index, size, shrunk axes, strides]
+function stridedSliceInfo(shape, begin, end, strides, beginMask, endMask, ellipsisMask,
+                          newAxisMask, shrinkAxisMask) {
+  if (ellipsisMask) throw new Error('ellipsis mask is not yet supported');
+  if (newAxisMask) throw new Error('new axis mask is not yet supported');
+  const full = shape.map((d, i) => strides[i] || 1);
+  const startIndex = [], endIndex = [], shrinkAxis = [];
+  for (let i = 0; i < shape.length; i++) {
+    const n = shape[i], stride = full[i];
+    let start = begin[i];
+    if (beginMask & (1 << i) || start == null) {
+      start = stride > 0 ? Number.MIN_SAFE_INTEGER : Number.MAX_SAFE_INTEGER;
+    }
+    if (start < 0) start += n;
+    start = clampInt(0, start, n - 1);
+    let stop = end[i];
+    if (endMask & (1 << i) || stop == null) {
+      stop = stride > 0 ? Number.MAX_SAFE_INTEGER : Number.MIN_SAFE_INTEGER;
+    }
+    if (stop < 0) stop += n;
+    stop = stride > 0 ? clampInt(0, stop, n) : clampInt(-1, stop, n - 1);
+    if (shrinkAxisMask & (1 << i)) {
+      stop = start + 1;
+      shrinkAxis.push(i);
+    }
+    startIndex.push(start);
+    endIndex.push(stop);
+  }
+  const size = shape.map((d, i) => {
+    let count = 0;
+    for (let s = startIndex[i]; !(full[i] > 0 ? s >= endIndex[i] : s <= endIndex[i]); s += full[i]) {
+      count++;
+    }
+    return count;
+  });
+  return [startIndex, size, shrinkAxis, full];
+}
+
+const stridedSlice = op('stridedSlice', (x, begin, end, strides, beginMask, endMask, ellipsisMask,
+                                         newAxisMask, shrinkAxisMask) => {
+  const $x = convertToTensor(x, 'x', 'stridedSlice');
+  if (strides == null) strides = new Array(begin.length).fill(1);
+  const [start, size, shrink, full] = stridedSliceInfo(
+      $x.shape, begin, end, strides, beginMask | 0, endMask | 0, ellipsisMask | 0, newAxisMask | 0,
+      shrinkAxisMask | 0);
+  const shape = size.filter((v, i) => shrink.indexOf(i) === -1);
+  if (shape.some(d => d === 0)) return tensor([], shape, $x.dtype);
+  const res = ENGINE.runKernel(backend => backend.stridedSliceBox($x, start, size, full), {$x});
+  return reshape(res, shape);
+});
+
+const reverse = op('reverse', (x, axis) => {
+  const $x = convertToTensor(x, 'x', 'reverse');
+  if ($x.rank === 0) return clone($x);
+  const axes = util.parseAxisParam(axis, $x.shape);
+  return ENGINE.runKernel(backend => backend.reverse($x, axes), {$x});
+});
+
+// ---- concat (ops/concat_split.ts:163-196, ops/concat_util.ts) ----
+const concat = op('concat', (tensors, axis) => {
+  util.assert(tensors.length >= 1, () => 'Pass at least one tensor to concat');
+  let $tensors = tensors.map((t, i) => convertToTensor(t, `tensors[${i}]`, 'concat'));
+  axis = util.parseAxisParam(axis == null ? 0 : axis, $tensors[0].shape)[0];
+  const outShape = $tensors[0].shape.slice();
+  for (let i = 1; i < $tensors.length; i++) outShape[axis] += $tensors[i].shape[axis];
+  if (util.sizeFromShape(outShape) === 0) return tensor([], outShape, $tensors[0].dtype);
+  $tensors = $tensors.filter(t => t.size > 0);
+  if ($tensors.length === 1) return $tensors[0];
+  const shapes = $tensors.map(t => t.shape);
+  const rank = shapes[0].length;
+  shapes.forEach((shape, i) => {
+    util.assert(shape.length === rank,
+                () => `Error in concat${rank}D: rank of tensors[${i}] must be the same ` +
+                      `as the rank of the rest (${rank})`);
+  });
+  util.assert(axis >= 0 && axis < rank,
+              () => `Error in concat${rank}D: axis must be between 0 and ${rank - 1}.`);
+  shapes.forEach((shape, i) => {
+    for (let r = 0; r < rank; r++) {
+      util.assert(r === axis || shape[r] === shapes[0][r],
+                  () => `Error in concat${rank}D: Shape of tensors[${i}] (${shape}) ` +
+                        `does not match the shape of the rest (${shapes[0]}) ` +
+                        `along the non-concatenated axis ${i}.`);
+    }
+  });
+  return ENGINE.runKernel(backend => backend.concat($tensors, axis), {});
+});
+
+// ---- pad / tile / oneHot (ops/array_ops.ts:325-343, 455-528, 602-618) ----
+const pad = op('pad', (x, paddings, constantValue) => {
+  const $x = convertToTensor(x, 'x', 'pad');
+  if ($x.rank === 0) throw new Error('pad(scalar) is not defined. Pass non-scalar to pad');
+  util.assert(paddings.length === $x.rank,
+              () => `pad: paddings must give [before, after] for each of the ${$x.rank} dimensions`);
+  return ENGINE.runKernel(backend => backend.pad($x, paddings, constantValue || 0), {$x});
+});
+
+const tile = op('tile', (x, reps) => {
+  const $x = convertToTensor(x, 'x', 'tile');
+  util.assert($x.rank === reps.length,
+              () => `Error in transpose: rank of input ${$x.rank} must match length of reps ${reps}.`);
+  return ENGINE.runKernel(backend => backend.tile($x, reps), {$x});
+});
+
+const oneHot = op('oneHot', (indices, depth, onValue, offValue) => {
+  if (depth < 2) throw new Error(`Error in oneHot: depth must be >=2, but it is ${depth}`);
+  let $indices = convertToTensor(indices, 'indices', 'oneHot', 'int32');
+  if ($indices.dtype !== 'int32') $indices = cast($indices, 'int32');
+  const outShape = $indices.shape.concat([depth]);
+  const flat = reshape($indices, [$indices.size]);
+  const res = ENGINE.runKernel(
+      backend => backend.oneHot(flat, depth, onValue == null ? 1 : onValue, offValue || 0),
+      {$indices: flat});
+  return reshape(res, outShape);
+});
+
+// ---- comparison and logical ops (ops/compare.ts, ops/logical_ops.ts) ----
+function compareOp(name) {
+  return op(name, (a, b) => {
+    let $a = convertToTensor(a, 'a', name);
+    let $b = convertToTensor(b, 'b', name);
+    [$a, $b] = makeTypesMatch($a, $b);
+    broadcast_util.assertAndGetBroadcastShape($a.shape, $b.shape);
+    return ENGINE.runKernel(backend => backend[name]($a, $b), {$a, $b});
+  });
+}
+const equal = compareOp('equal'), notEqual = compareOp('notEqual'), less = compareOp('less');
+const lessEqual = compareOp('lessEqual'), greater = compareOp('greater');
+const greaterEqual = compareOp('greaterEqual');
+
+function logicalOp(name) {
+  return op(name, (a, b) => {
+    const $a = convertToTensor(a, 'a', name, 'bool');
+    const $b = convertToTensor(b, 'b', name, 'bool');
+    for (const [t, arg] of [[$a, 'a'], [$b, 'b']]) {
+      util.assert(t.dtype === 'bool',
+                  () => `Argument '${arg}' passed to '${name}' must be bool tensor, but got ${t.dtype} tensor`);
+    }
+    broadcast_util.assertAndGetBroadcastShape($a.shape, $b.shape);
+    return ENGINE.runKernel(backend => backend[name]($a, $b), {$a, $b});
+  });
+}
+const logicalAnd = logicalOp('logicalAnd'), logicalOr = logicalOp('logicalOr');
+const logicalNot = op('logicalNot', x => {
+  const $x = convertToTensor(x, 'x', 'logicalNot', 'bool');
+  util.assert($x.dtype === 'bool',
+              () => `Argument 'x' passed to 'logicalNot' must be bool tensor, but got ${$x.dtype} tensor`);
+  return ENGINE.runKernel(backend => backend.logicalNot($x), {$x});
+});
+
+// ---- batchNorm (ops/batchnorm.ts:268-370), resizeBilinear (ops/image_ops.ts:35-85) ----
+const batchNorm = op('batchNorm', (x, mean, variance, offset, scale, varianceEpsilon) => {
+  if (varianceEpsilon == null) varianceEpsilon = 0.001;
+  const $x = convertToTensor(x, 'x', 'batchNorm');
+  const $mean = convertToTensor(mean, 'mean', 'batchNorm');
+  const $variance = convertToTensor(variance, 'variance', 'batchNorm');
+  const $scale = scale == null ? null : convertToTensor(scale, 'scale', 'batchNorm');
+  const $offset = offset == null ? null : convertToTensor(offset, 'offset', 'batchNorm');
+  util.assert($mean.rank === $variance.rank,
+              () => 'Batch normalization gradient requires mean and variance to have equal ranks.');
+  util.assert($offset == null || $mean.rank === $offset.rank,
+              () => 'Batch normalization gradient requires mean and offset to have equal ranks.');
+  util.assert($scale == null || $mean.rank === $scale.rank,
+              () => 'Batch normalization gradient requires mean and scale to have equal ranks.');
+  let shape4;
+  if ($x.rank === 0 || $x.rank === 1) shape4 = [1, 1, 1, $x.size];
+  else if ($x.rank === 2) shape4 = [1, 1, $x.shape[0], $x.shape[1]];
+  else if ($x.rank === 3) shape4 = [1, $x.shape[0], $x.shape[1], $x.shape[2]];
+  else shape4 = $x.shape;
+  const x4D = reshape($x, shape4);
+  const res = ENGINE.runKernel(
+      backend => backend.batchNormalization(x4D, $mean, $variance, varianceEpsilon, $scale, $offset),
+      {$x, $mean, $variance});
+  return reshape(res, $x.shape);
+});
+
+const resizeBilinear = op('resizeBilinear', (images, size, alignCorners) => {
+  const $images = convertToTensor(images, 'images', 'resizeBilinear');
+  util.assert($images.rank === 3 || $images.rank === 4,
+              () => `Error in resizeBilinear: x must be rank 3 or 4, but got rank ${$images.rank}.`);
+  util.assert(size.length === 2,
+              () => `Error in resizeBilinear: new shape must 2D, but got ${size}.`);
+  const batchImages = $images.rank === 4 ? $images : reshape($images, [1].concat($images.shape));
+  const res = ENGINE.runKernel(
+      backend => backend.resizeBilinear(batchImages, size[0], size[1], !!alignCorners), {batchImages});
+  return $images.rank === 4 ? res : reshape(res, res.shape.slice(1));
+});
+
 const opHandler = {
   reshape, cast, clone, matMul, add, sub, mul, div, relu, prelu, clipByValue, exp, log, sum, max,
   min, argMax, argMin, logSumExp, softmax, transpose, gather, conv2d, depthwiseConv2d, avgPool, maxPool
@@ -468,5 +691,7 @@ module.exports = {
   fused: {matMul: fusedMatMul, conv2d: fusedConv2d, depthwiseConv2d: fusedDepthwiseConv2d},
   conv2d, depthwiseConv2d, separableConv2d, avgPool, maxPool, pool, add, sub, mul, div, maximum,
   minimum, prelu, relu, relu6, exp, log, neg, abs, sigmoid, sqrt, square, tanh, rsqrt,
-  clipByValue, sum, max, min, argMax, argMin, logSumExp, softmax, gather, transpose
+  clipByValue, sum, max, min, argMax, argMin, logSumExp, softmax, gather, transpose,
+  slice, stridedSlice, reverse, concat, pad, tile, oneHot, equal, notEqual, less, lessEqual,
+  greater, greaterEqual, logicalAnd, logicalOr, logicalNot, batchNorm, resizeBilinear
 };

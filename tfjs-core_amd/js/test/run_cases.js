@@ -55,6 +55,18 @@ const OPS = {
   transpose: (i, a) => tf.transpose(i.x, a.perm),
   cast: (i, a) => tf.cast(i.x, a.dtype),
   chainMethods: i => i.x.reshape([i.x.size]).relu().mul(i.x.reshape([i.x.size])).sum(),
+  slice: (i, a) => tf.slice(i.x, a.begin, a.size),
+  stridedSlice: (i, a) => tf.stridedSlice(i.x, a.begin, a.end, a.strides, a.beginMask, a.endMask, 0, 0,
+                                          a.shrinkAxisMask),
+  reverse: (i, a) => tf.reverse(i.x, a.axis),
+  concat: (i, a) => tf.concat([i.a, i.b, i.c].filter(t => t != null), a.axis),
+  pad: (i, a) => tf.pad(i.x, a.paddings, a.constantValue),
+  tile: (i, a) => tf.tile(i.x, a.reps),
+  oneHot: (i, a) => tf.oneHot(i.indices, a.depth, a.onValue, a.offValue),
+  compare: (i, a) => tf[a.name](i.a, i.b),
+  logicalNot: i => tf.logicalNot(i.x),
+  batchNorm: (i, a) => tf.batchNorm(i.x, i.mean, i.variance, i.offset, i.scale, a.varianceEpsilon),
+  resizeBilinear: (i, a) => tf.resizeBilinear(i.x, a.size, a.alignCorners),
 };
 
 async function main() {

@@ -15,6 +15,16 @@ function sizeFromShape(shape) {
   return size;
 }
 
+// Row-major strides of all but the last dimension (util.ts computeStrides): [] below rank 2.
+function computeStrides(shape) {
+  const rank = shape.length;
+  if (rank < 2) return [];
+  const strides = new Array(rank - 1);
+  strides[rank - 2] = shape[rank - 1];
+  for (let i = rank - 3; i >= 0; --i) strides[i] = strides[i + 1] * shape[i + 1];
+  return strides;
+}
+
 function arraysEqual(a, b) {
   if (a === b) return true;
   if (a == null || b == null || a.length !== b.length) return false;
@@ -155,7 +165,7 @@ function inferFromImplicitShape(shape, size) {
 }
 
 module.exports = {
-  assert, sizeFromShape, arraysEqual, isInt, isTypedArray, inferShape, flatten, inferDtype,
+  assert, sizeFromShape, computeStrides, arraysEqual, isInt, isTypedArray, inferShape, flatten, inferDtype,
   getTypedArrayFromDType, toTypedArray, bytesPerElement, upcastType, hasEncodingLoss,
   parseAxisParam, inferFromImplicitShape
 };

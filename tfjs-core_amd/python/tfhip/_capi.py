@@ -9,7 +9,8 @@ LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "..", "libtfjs_hip.so"))
 FLOAT32, INT32, BOOL, UINT8Q = 0, 1, 2, 3
 ACT = {"linear": 0, None: 0, "relu": 1, "prelu": 2, "relu6": 3}
 BCAST_NONE, BCAST_SCALAR, BCAST_COLUMN, BCAST_FULL = 0, 1, 2, 3
-BINARY = dict(add=0, sub=1, mul=2, div=3, prelu=4, maximum=5, minimum=6)
+BINARY = dict(add=0, sub=1, mul=2, div=3, prelu=4, maximum=5, minimum=6, equal=7, not_equal=8,
+              less=9, less_equal=10, greater=11, greater_equal=12, logical_and=13, logical_or=14)
 UNARY = dict(relu=0, clip=1, exp=2, log=3, neg=4, abs=5, sigmoid=6, sqrt=7, square=8, tanh=9,
              rsqrt=10)
 REDUCE = dict(sum=0, max=1, min=2, argmax=3, argmin=4)
@@ -62,6 +63,12 @@ _SIGNATURES = {
     "tfhip_gather": [_PTR, _I64, _I64, _I64, _I64, _I64, _I64, _I64],
     "tfhip_transpose": [_PTR, _I64, C.POINTER(C.c_int32), _INT, C.POINTER(C.c_int32), _I64],
     "tfhip_copy": [_PTR, _I64, _I64],
+    "tfhip_strided_copy": [_PTR, _I64, _I64, _INT, C.POINTER(C.c_int32), C.POINTER(C.c_int64), _I64,
+                           C.POINTER(C.c_int64), _I64],
+    "tfhip_logical_not": [_PTR, _I64, _I64],
+    "tfhip_batchnorm": [_PTR, _I64, _I64, _I64, _I64, _I64, C.c_float, _I64],
+    "tfhip_resize_bilinear": [_PTR, _I64, _I64, _INT, _INT, _INT, _INT, _INT, _INT, _INT],
+    "tfhip_one_hot": [_PTR, _I64, _I64, _INT, C.c_float, C.c_float],
 }
 
 

@@ -413,6 +413,143 @@ class MathBackendHIP(object):
                                        x.shape[axis], inner, indices.size))
         return out
 
+    # ---- strided box copies: slice / stridedSlice / reverse / concat / pad / tile ----
+    @staticmethod
+    def _strides(shape):
+        st, n = [0] * len(shape), 1
+        for i in range(len(shape) - 1, -1, -1):
+            st[i] = n
+            n *= shape[i]
+        return st
+
+    def _box_copy(self, x, out, region, x_strides, x_offset, out_strides, out_offset):
+        r = len(region)
+        i64 = C.c_int64 * max(1, r)
+        self._ck(self.lib.tfhip_strided_copy(self.ctx, self._h(x), self._h(out), r,
+                                             _shape_arr(region), i64(*x_strides), x_offset,
+                                             i64(*out_strides), out_offset))
+
+    def _materialized(self, x):
+        """x with its stored element type equal to its dtype (a widening cast may have
+        aliased narrower storage)."""
+        self._h(x)
+        if self.data[x.data_id][1] == _DTYPE_CODE[x.dtype]:
+            return x
+        out = self._out(x.shape, x.dtype)
+        self._ck(self.lib.tfhip_cast(self.ctx, self._h(x), self._h(out)))
+        return out
+
+    def slice(self, x, begin, size):
+        """backend_cpu.ts:292-313."""
+        out = self._out_like_storage(list(size), x)
+        xs = self._strides(x.shape)
+        self._box_copy(x, out, list(size), xs, sum(b * s for b, s in zip(begin, xs)),
+                       self._strides(size), 0)
+        return out
+
+    def strided_slice(self, x, begin_index, size, strides):
+        """backend_cpu.ts:315-345 after getStridedSlicedInfo: out[loc] = x[loc*strides+begin]."""
+        out = self._out_like_storage(list(size), x)
+        xs = self._strides(x.shape)
+        self._box_copy(x, out, list(size), [s * k for s, k in zip(xs, strides)],
+                       sum(b * s for b, s in zip(begin_index, xs)), self._strides(size), 0)
+        return out
+
+    def reverse(self, x, axes):
+        """backend_cpu.ts:377-391."""
+        out = self._out_like_storage(list(x.shape), x)
+        xs = self._strides(x.shape)
+        off = sum((x.shape[a] - 1) * xs[a] for a in axes)
+        self._box_copy(x, out, list(x.shape), [-s if a in axes else s for a, s in enumerate(xs)],
+                       off, xs, 0)
+        return out
+
+    def concat(self, tensors, axis):
+        """backend_cpu.ts:393-433."""
+        tensors = [self._materialized(t) for t in tensors]
+        out_shape = list(tensors[0].shape)
+        out_shape[axis] = sum(t.shape[axis] for t in tensors)
+        out = self._out(out_shape, tensors[0].dtype)
+        os_ = self._strides(out_shape)
+        at = 0
+        for t in tensors:
+            if t.size:
+                self._box_copy(t, out, list(t.shape), self._strides(t.shape), 0, os_,
+                               at * os_[axis])
+            at += t.shape[axis]
+        return out
+
+    def pad(self, x, paddings, constant_value):
+        """backend_cpu.ts:2157-2176."""
+        out_shape = [p[0] + d + p[1] for p, d in zip(paddings, x.shape)]
+        out = self._out_like_storage(out_shape, x)
+        self._ck(self.lib.tfhip_fill(self.ctx, self._h(out), float(constant_value)))
+        os_ = self._strides(out_shape)
+        if x.size:
+            self._box_copy(x, out, list(x.shape), self._strides(x.shape), 0, os_,
+                           sum(p[0] * s for p, s in zip(paddings, os_)))
+        return out
+
+    def tile(self, x, reps):
+        """backend_cpu.ts:2152-2155: out[i] = x[i % x.shape], as a box of rank 2*rank whose
+        repetition axes have source stride 0."""
+        out_shape = [d * r for d, r in zip(x.shape, reps)]
+        out = self._out_like_storage(out_shape, x)
+        if not su.size_from_shape(out_shape):
+            return out
+        if 2 * x.rank > 8:
+            raise NotImplementedError("hip backend: tile of rank above 4")
+        xs, os_ = self._strides(x.shape), self._strides(out_shape)
+        region, xst, ost = [], [], []
+        for d in range(x.rank):
+            region += [reps[d], x.shape[d]]
+            xst += [0, xs[d]]
+            ost += [os_[d] * x.shape[d], os_[d]]
+        self._box_copy(x, out, region, xst, 0, ost, 0)
+        return out
+
+    # ---- comparison / logical (backend_cpu.ts:747-820) ----
+    def equal(self, a, b): return self._binary("equal", a, b, "bool")
+    def not_equal(self, a, b): return self._binary("not_equal", a, b, "bool")
+    def less(self, a, b): return self._binary("less", a, b, "bool")
+    def less_equal(self, a, b): return self._binary("less_equal", a, b, "bool")
+    def greater(self, a, b): return self._binary("greater", a, b, "bool")
+    def greater_equal(self, a, b): return self._binary("greater_equal", a, b, "bool")
+    def logical_and(self, a, b): return self._binary("logical_and", a, b, "bool")
+    def logical_or(self, a, b): return self._binary("logical_or", a, b, "bool")
+
+    def logical_not(self, x):
+        x = self._materialized(x)
+        out = self._out(x.shape, "bool")
+        self._ck(self.lib.tfhip_logical_not(self.ctx, self._h(x), self._h(out)))
+        return out
+
+    # ---- batchNormalization / resizeBilinear / oneHot ----
+    def batch_normalization(self, x, mean, variance, variance_epsilon, scale=None, offset=None):
+        """backend_cpu.ts:3167-3213."""
+        out = self._out(x.shape, "float32")
+        self._ck(self.lib.tfhip_batchnorm(
+            self.ctx, self._h(x), self._h(mean), self._h(variance),
+            -1 if offset is None else self._h(offset), -1 if scale is None else self._h(scale),
+            float(variance_epsilon), self._h(out)))
+        return out
+
+    def resize_bilinear(self, x, new_height, new_width, align_corners):
+        """backend_cpu.ts:2875-2936."""
+        b, h, w, c = x.shape
+        out = self._out([b, new_height, new_width, c], "float32")
+        self._ck(self.lib.tfhip_resize_bilinear(self.ctx, self._h(x), self._h(out), b, h, w, c,
+                                                new_height, new_width, 1 if align_corners else 0))
+        return out
+
+    def one_hot(self, indices, depth, on_value, off_value):
+        """backend_cpu.ts:3325-3339 (int32 result)."""
+        out = self._out([indices.size, depth], "int32")
+        idx = self._materialized(indices)
+        self._ck(self.lib.tfhip_one_hot(self.ctx, self._h(idx), self._h(out), depth,
+                                        float(on_value), float(off_value)))
+        return out
+
     def transpose(self, x, perm):
         out = self._out_like_storage([x.shape[p] for p in perm], x)
         self._ck(self.lib.tfhip_transpose(self.ctx, self._h(x), _shape_arr(x.shape), x.rank,

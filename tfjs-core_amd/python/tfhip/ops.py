@@ -429,3 +429,265 @@ def zeros(shape, dtype="float32"):
 
 def ones(shape, dtype="float32"):
     return fill(shape, 1, dtype)
+
+
+# ---- slice / stridedSlice / reverse (ops/slice.ts, ops/slice_util.ts, ops/strided_slice.ts,
+#      ops/reverse.ts) ----
+def slice(x, begin, size=None):  # noqa: A001
+    x = _conv(x, "x", "slice")
+    if x.rank == 0:
+        raise ValueError("Slicing scalar is not possible")
+    if isinstance(begin, int):
+        begin = [begin] + [0] * (x.rank - 1)
+    begin = list(begin) + [0] * (x.rank - len(begin))
+    if size is None:
+        size = [-1] * x.rank
+    elif isinstance(size, int):
+        size = [size] + [-1] * (x.rank - 1)
+    size = list(size) + [-1] * (x.rank - len(size))
+    for i, d in enumerate(size):
+        if d < 0:
+            if d != -1:
+                raise ValueError("Bad value in size")
+            size[i] = x.shape[i] - begin[i]
+    if len(begin) != x.rank:
+        raise ValueError("Error in slice%dD: Length of begin %s must match the rank of the array "
+                         "(%d)." % (x.rank, begin, x.rank))
+    if len(size) != x.rank:
+        raise ValueError("Error in slice%dD: Length of size %s must match the rank of the array "
+                         "(%d)." % (x.rank, size, x.rank))
+    for i in range(x.rank):
+        if begin[i] + size[i] > x.shape[i]:
+            raise ValueError("Error in slice%dD: begin[%d] + size[%d] (%d) would overflow "
+                             "input.shape[%d] (%d)" % (x.rank, i, i, begin[i] + size[i], i,
+                                                       x.shape[i]))
+    return ENGINE.run_kernel(lambda be: be.slice(x, begin, size))
+
+
+_MAX_SAFE = 2 ** 53 - 1
+
+
+def _clamp(lo, v, hi):
+    return lo if v < lo else (hi if v > hi else v)
+
+
+def strided_slice_info(shape, begin, end, strides, begin_mask=0, end_mask=0, ellipsis_mask=0,
+                       new_axis_mask=0, shrink_axis_mask=0):
+    """getStridedSlicedInfo (ops/slice_util.ts:48-188): [start index, size, shrunk axes]."""
+    if ellipsis_mask != 0:
+        raise ValueError("ellipsis mask is not yet supported")
+    if new_axis_mask != 0:
+        raise ValueError("new axis mask is not yet supported")
+    start_index, end_index, shrink = [], [], []
+    strides = [(strides[i] if i < len(strides) else 0) or 1 for i in range(len(shape))]
+    for i, n in enumerate(shape):
+        stride = strides[i]
+        start = begin[i] if i < len(begin) else None
+        if begin_mask & (1 << i) or start is None:
+            start = -_MAX_SAFE if stride > 0 else _MAX_SAFE
+        if start < 0:
+            start += n
+        start = _clamp(0, start, n - 1)
+        stop = end[i] if i < len(end) else None
+        if end_mask & (1 << i) or stop is None:
+            stop = _MAX_SAFE if stride > 0 else -_MAX_SAFE
+        if stop < 0:
+            stop += n
+        stop = _clamp(0, stop, n) if stride > 0 else _clamp(-1, stop, n - 1)
+        if shrink_axis_mask & (1 << i):
+            stop = start + 1
+            shrink.append(i)
+        start_index.append(start)
+        end_index.append(stop)
+    size = []
+    for i in range(len(shape)):
+        stride = strides[i]
+        count, s = 0, start_index[i]
+        while not (s >= end_index[i] if stride > 0 else s <= end_index[i]):
+            count += 1
+            s += stride
+        size.append(count)
+    return start_index, size, shrink, strides
+
+
+def strided_slice(x, begin, end, strides=None, begin_mask=0, end_mask=0, ellipsis_mask=0,
+                  new_axis_mask=0, shrink_axis_mask=0):
+    x = _conv(x, "x", "stridedSlice")
+    if strides is None:
+        strides = [1] * len(begin)
+    start, size, shrink, strides = strided_slice_info(
+        x.shape, list(begin), list(end), list(strides), begin_mask, end_mask, ellipsis_mask,
+        new_axis_mask, shrink_axis_mask)
+    shape = [d for i, d in enumerate(size) if i not in shrink]
+    if any(d == 0 for d in shape):
+        return tensor(np.zeros(shape, NP_DTYPE[x.dtype]), shape, x.dtype)
+
+    def run():
+        r = ENGINE.run_kernel(lambda be: be.strided_slice(x, start, size, list(strides)))
+        return reshape(r, shape)
+    return ENGINE.tidy(run)
+
+
+def reverse(x, axis=None):
+    x = _conv(x, "x", "reverse")
+    if x.rank == 0:
+        return ENGINE.run_kernel(lambda be: be.reshape(x, x.shape))
+    axes = su.parse_axis_param(axis, x.shape)
+    return ENGINE.run_kernel(lambda be: be.reverse(x, list(axes)))
+
+
+# ---- concat (ops/concat_split.ts:163-196, ops/concat_util.ts) ----
+def concat(tensors, axis=0):
+    if len(tensors) < 1:
+        raise ValueError("Pass at least one tensor to concat")
+    ts = [_conv(t, "tensors", "concat") for t in tensors]
+    axis = su.parse_axis_param(axis, ts[0].shape)[0]
+    out_shape = list(ts[0].shape)
+    for t in ts[1:]:
+        out_shape[axis] += t.shape[axis]
+    if su.size_from_shape(out_shape) == 0:
+        return tensor(np.zeros(out_shape, NP_DTYPE[ts[0].dtype]), out_shape, ts[0].dtype)
+    ts = [t for t in ts if t.size > 0]
+    if len(ts) == 1:
+        return ts[0]
+    rank = ts[0].rank
+    for i, t in enumerate(ts):
+        if t.rank != rank:
+            raise ValueError("Error in concat%dD: rank of tensors[%d] must be the same as the "
+                             "rank of the rest (%d)" % (rank, i, rank))
+    if not 0 <= axis < rank:
+        raise ValueError("Error in concat%dD: axis must be between 0 and %d." % (rank, rank - 1))
+    for i, t in enumerate(ts):
+        for r in range(rank):
+            if r != axis and t.shape[r] != ts[0].shape[r]:
+                raise ValueError("Error in concat%dD: Shape of tensors[%d] (%s) does not match the "
+                                 "shape of the rest (%s) along the non-concatenated axis %d."
+                                 % (rank, i, list(t.shape), list(ts[0].shape), i))
+    return ENGINE.run_kernel(lambda be: be.concat(ts, axis))
+
+
+# ---- pad / tile / oneHot (ops/array_ops.ts:325-343, 455-528, 602-618) ----
+def pad(x, paddings, constant_value=0):
+    x = _conv(x, "x", "pad")
+    if x.rank == 0:
+        raise ValueError("pad(scalar) is not defined. Pass non-scalar to pad")
+    if len(paddings) != x.rank:
+        raise ValueError("pad: paddings must give [before, after] for each of the %d dimensions"
+                         % x.rank)
+    return ENGINE.run_kernel(lambda be: be.pad(x, [tuple(p) for p in paddings], constant_value))
+
+
+def tile(x, reps):
+    x = _conv(x, "x", "tile")
+    if x.rank != len(reps):
+        raise ValueError("Error in transpose: rank of input %d must match length of reps %s."
+                         % (x.rank, list(reps)))
+    return ENGINE.run_kernel(lambda be: be.tile(x, list(reps)))
+
+
+def one_hot(indices, depth, on_value=1, off_value=0):
+    if depth < 2:
+        raise ValueError("Error in oneHot: depth must be >=2, but it is %d" % depth)
+    indices = _conv(indices, "indices", "oneHot")
+    if indices.dtype != "int32":
+        indices = cast(indices, "int32")
+    out_shape = list(indices.shape) + [depth]
+
+    def run():
+        flat = reshape(indices, (indices.size,))
+        r = ENGINE.run_kernel(lambda be: be.one_hot(flat, depth, on_value, off_value))
+        return reshape(r, out_shape)
+    return ENGINE.tidy(run)
+
+
+# ---- comparison and logical ops (ops/compare.ts, ops/logical_ops.ts) ----
+def _compare(method, name):
+    def op(a, b):
+        a, b = _types_match(_conv(a, "a", name), _conv(b, "b", name))
+        su.broadcast_shape(a.shape, b.shape)
+        return ENGINE.run_kernel(lambda be: getattr(be, method)(a, b))
+    op.__name__ = method
+    return op
+
+
+equal = _compare("equal", "equal")
+not_equal = _compare("not_equal", "notEqual")
+less = _compare("less", "less")
+less_equal = _compare("less_equal", "lessEqual")
+greater = _compare("greater", "greater")
+greater_equal = _compare("greater_equal", "greaterEqual")
+
+
+def _logical(method, name):
+    def op(a, b):
+        a, b = _conv(a, "a", name), _conv(b, "b", name)
+        for t, arg in ((a, "a"), (b, "b")):
+            if t.dtype != "bool":
+                raise ValueError("Argument '%s' passed to '%s' must be bool tensor, but got %s "
+                                 "tensor" % (arg, name, t.dtype))
+        su.broadcast_shape(a.shape, b.shape)
+        return ENGINE.run_kernel(lambda be: getattr(be, method)(a, b))
+    op.__name__ = method
+    return op
+
+
+logical_and = _logical("logical_and", "logicalAnd")
+logical_or = _logical("logical_or", "logicalOr")
+
+
+def logical_not(x):
+    x = _conv(x, "x", "logicalNot")
+    if x.dtype != "bool":
+        raise ValueError("Argument 'x' passed to 'logicalNot' must be bool tensor, but got %s "
+                         "tensor" % x.dtype)
+    return ENGINE.run_kernel(lambda be: be.logical_not(x))
+
+
+# ---- batchNorm (ops/batchnorm.ts:268-370) and resizeBilinear (ops/image_ops.ts:35-85) ----
+def batch_norm(x, mean, variance, offset=None, scale=None, variance_epsilon=None):
+    if variance_epsilon is None:
+        variance_epsilon = 0.001
+    x = _conv(x, "x", "batchNorm")
+    mean = _conv(mean, "mean", "batchNorm")
+    variance = _conv(variance, "variance", "batchNorm")
+    scale = None if scale is None else _conv(scale, "scale", "batchNorm")
+    offset = None if offset is None else _conv(offset, "offset", "batchNorm")
+    if mean.rank != variance.rank:
+        raise ValueError("Batch normalization gradient requires mean and variance to have equal "
+                         "ranks.")
+    if offset is not None and mean.rank != offset.rank:
+        raise ValueError("Batch normalization gradient requires mean and offset to have equal "
+                         "ranks.")
+    if scale is not None and mean.rank != scale.rank:
+        raise ValueError("Batch normalization gradient requires mean and scale to have equal "
+                         "ranks.")
+    if x.rank <= 1:
+        shape4 = (1, 1, 1, x.size)
+    elif x.rank == 2:
+        shape4 = (1, 1) + tuple(x.shape)
+    elif x.rank == 3:
+        shape4 = (1,) + tuple(x.shape)
+    else:
+        shape4 = tuple(x.shape)
+
+    def run():
+        r = ENGINE.run_kernel(lambda be: be.batch_normalization(
+            be.reshape(x, shape4), mean, variance, variance_epsilon, scale, offset))
+        return reshape(r, x.shape)
+    return ENGINE.tidy(run)
+
+
+def resize_bilinear(images, size, align_corners=False):
+    images = _conv(images, "images", "resizeBilinear")
+    if images.rank not in (3, 4):
+        raise ValueError("Error in resizeBilinear: x must be rank 3 or 4, but got rank %d."
+                         % images.rank)
+    if len(size) != 2:
+        raise ValueError("Error in resizeBilinear: new shape must 2D, but got %s." % list(size))
+    new_h, new_w = size
+
+    def run():
+        x4 = images if images.rank == 4 else reshape(images, (1,) + tuple(images.shape))
+        r = ENGINE.run_kernel(lambda be: be.resize_bilinear(x4, new_h, new_w, align_corners))
+        return r if images.rank == 4 else reshape(r, r.shape[1:])
+    return ENGINE.tidy(run)
