@@ -150,3 +150,55 @@ def test_failing_factory_reports_and_falls_back():
                 tfhip.set_backend("broken-test")
     finally:
         tfhip.remove_backend("broken-test")
+
+
+def test_shape_op_wrappers_validate_before_the_backend():
+    """Argument checks of slice / stridedSlice / concat / pad / tile / oneHot / batchNorm /
+    resizeBilinear (ops/slice.ts, slice_util.ts, concat_util.ts, array_ops.ts, batchnorm.ts,
+    image_ops.ts) fire on the host; strided slice geometry follows slice_util.ts:48-188."""
+    import numpy as np
+    import tfhip
+    from tfhip import ops
+    from tfhip.engine import ENGINE
+    fake = FakeBackend()
+    tfhip.register_backend("fake-shape-test", lambda: fake, 0)
+    prev = ENGINE.backend_name
+    try:
+        tfhip.set_backend("fake-shape-test")
+        x = tfhip.tensor(np.zeros((4, 3), np.float32))
+        with pytest.raises(ValueError, match=r"begin\[0\] \+ size\[0\] \(5\) would overflow"):
+            tfhip.slice(x, [2, 0], [3, 3])
+        with pytest.raises(ValueError, match="Slicing scalar"):
+            tfhip.slice(tfhip.tensor(np.float32(1)), [0], [1])
+        with pytest.raises(ValueError, match="Bad value in size"):
+            tfhip.slice(x, [0, 0], [-2, 1])
+        with pytest.raises(ValueError, match="rank of tensors\\[1\\] must be the same"):
+            tfhip.concat([x, tfhip.tensor(np.zeros(3, np.float32))], 0)
+        with pytest.raises(ValueError, match="does not match the shape of the rest"):
+            tfhip.concat([x, tfhip.tensor(np.zeros((4, 2), np.float32))], 0)
+        with pytest.raises(ValueError, match="pad\\(scalar\\)"):
+            tfhip.pad(tfhip.tensor(np.float32(1)), [])
+        with pytest.raises(ValueError, match="must match length of reps"):
+            tfhip.tile(x, [2])
+        with pytest.raises(ValueError, match="depth must be >=2"):
+            tfhip.one_hot(np.array([0], np.int32), 1)
+        with pytest.raises(ValueError, match="ellipsis mask"):
+            tfhip.strided_slice(x, [0, 0], [1, 1], [1, 1], 0, 0, 1)
+        with pytest.raises(ValueError, match="mean and variance to have equal ranks"):
+            tfhip.batch_norm(x, np.zeros(3, np.float32), np.zeros((1, 3), np.float32))
+        with pytest.raises(ValueError, match="rank 3 or 4"):
+            tfhip.resize_bilinear(x, [2, 2])
+        with pytest.raises(ValueError, match="must be bool tensor"):
+            tfhip.logical_and(x, x)
+    finally:
+        tfhip.remove_backend("fake-shape-test")
+        if prev:
+            ENGINE.set_backend(prev)
+    # (start, size, shrunk axes, strides) of strided_slice_test.ts:92-140, 197-237
+    assert ops.strided_slice_info([4], [1], [3], [1], 1)[:2] == ([0], [3])
+    assert ops.strided_slice_info([4], [1], [3], [1], 0, 1)[:2] == ([1], [3])
+    assert ops.strided_slice_info([4], [1], [3], [1], 0, 0, 0, 0, 1)[:3] == ([1], [1], [0])
+    assert ops.strided_slice_info([4], [-1], [-4], [-1])[:2] == ([3], [3])
+    assert ops.strided_slice_info([2, 3], [1, -1], [2, -4], [2, -1])[:2] == ([1, 2], [1, 3])
+    assert ops.strided_slice_info([2, 3, 1, 2], [1, 0, 0, 0], [2, 3, 1, 2], [1, 1])[:2] == (
+        [1, 0, 0, 0], [1, 3, 1, 2])
