@@ -12,6 +12,7 @@
 namespace tfhip {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float dq(unsigned q, double scale, double mn) {
 #pragma clang fp contract(off)
@@ -26,6 +27,23 @@ __device__ __forceinline__ float act_f(float v, int act) {
     case TFHIP_ACT_RELU6: return v > 6.f ? 6.f : (v < 0.f ? 0.f : v);
     default: return v;
   }
+}
+
+// The same activations without branches: the kind is unpacked once into values that are
+// the same for every lane.  NaN passes through (it is neither < 0 nor > hi).
+struct ActFlags {
+  bool linear;
+  float hi;
+};
+__device__ __forceinline__ ActFlags act_flags(int act) {
+  ActFlags f;
+  f.linear = act != TFHIP_ACT_RELU && act != TFHIP_ACT_RELU6;
+  f.hi = act == TFHIP_ACT_RELU6 ? 6.f : __builtin_inff();
+  return f;
+}
+__device__ __forceinline__ float act_fast(float v, const ActFlags& f) {
+  const float r = v < 0.f ? (f.linear ? v : 0.f) : v;
+  return r > f.hi ? f.hi : r;
 }
 
 struct DwArgs {
@@ -112,6 +130,7 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p) {
     }
   }
 
+  const ActFlags af = act_flags(p.act);
   f32x4 b = {0.f, 0.f, 0.f, 0.f};
   if (p.bias_kind == TFHIP_BCAST_COLUMN) b = *reinterpret_cast<const f32x4*>(p.bias + c);
   else if (p.bias_kind == TFHIP_BCAST_SCALAR) b = f32x4{p.bias[0], p.bias[0], p.bias[0], p.bias[0]};
@@ -125,9 +144,141 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p) {
       if (ow >= ci.out_w) continue;
       f32x4 v = acc[i][j] + b;
 #pragma unroll
-      for (int e = 0; e < 4; e++) v[e] = act_f(v[e], p.act);
+      for (int e = 0; e < 4; e++) v[e] = act_fast(v[e], af);
       *reinterpret_cast<f32x4*>(p.y + (((int64_t)n * ci.out_h + oh) * ci.out_w + ow) * C + c) = v;
     }
+  }
+}
+
+// 3x3, stride 1, dilation 1, channel multiplier 1, C % 4 == 0, for large images: one lane =
+// one channel quad of a strip TW outputs wide, walked down `rows` output rows.  Every input
+// row of the strip is fetched once (TW + 2 vectors, the next row already in flight) and
+// feeds the three output rows it belongs to, which live in three rotating accumulator rows;
+// nothing is read twice vertically, and the two halo columns are shared with the
+// neighbouring lane's loads of the same moment.  Each output sums its taps in the order
+// filter row, then filter column, as the patch kernel above and the reference do.
+template <int TW>
+__global__ __launch_bounds__(256) void depthwise3x3_rows_kernel(const DwArgs p, int rows,
+                                                                int chunks, unsigned x_bytes,
+                                                                unsigned y_bytes) {
+  constexpr int IW = TW + 2;
+  constexpr unsigned OOB = 0x80000000u;  // beyond any extent below 2 GiB: loads give 0, stores vanish
+  const tfhip_conv2d_info& ci = p.ci;
+  const int64_t total = (int64_t)ci.batch * chunks * p.tiles_w * p.c4;
+  const int64_t gid = (int64_t)xcd_remap(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x;
+  if (gid >= total) return;
+  const int cq = (int)(gid % p.c4);
+  int64_t t = gid / p.c4;
+  const int tw = (int)(t % p.tiles_w);
+  t /= p.tiles_w;
+  const int chunk = (int)(t % chunks);
+  const int n = (int)(t / chunks);
+  const int c = cq * 4;
+  const int C = ci.in_c;
+
+  f32x4 w[9];
+  if (p.quant) {
+    const unsigned char* wq = static_cast<const unsigned char*>(p.w);
+#pragma unroll
+    for (int i = 0; i < 9; i++) {
+      const unsigned v = *reinterpret_cast<const unsigned*>(wq + (int64_t)i * C + c);
+#pragma unroll
+      for (int e = 0; e < 4; e++) w[i][e] = dq((v >> (8 * e)) & 0xffu, p.qscale, p.qmin);
+    }
+  } else {
+    const float* wf = static_cast<const float*>(p.w);
+#pragma unroll
+    for (int i = 0; i < 9; i++) w[i] = *reinterpret_cast<const f32x4*>(wf + (int64_t)i * C + c);
+  }
+  f32x4 b = {0.f, 0.f, 0.f, 0.f};
+  if (p.bias_kind == TFHIP_BCAST_COLUMN) b = *reinterpret_cast<const f32x4*>(p.bias + c);
+  else if (p.bias_kind == TFHIP_BCAST_SCALAR) b = f32x4{p.bias[0], p.bias[0], p.bias[0], p.bias[0]};
+
+  // All addresses are 32-bit byte offsets into buffer descriptors over x and y: padding,
+  // rows outside the chunk and columns outside the image get OOB instead of a branch.
+  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(p.x), (short)0, (int)x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ry =
+      __builtin_amdgcn_make_buffer_rsrc(p.y, (short)0, (int)y_bytes, 0x00020000);
+  const ActFlags af = act_flags(p.act);
+  const int oh0 = chunk * rows;
+  const int oh1 = min(ci.out_h, oh0 + rows);
+  const int ow0 = tw * TW;
+  const int iw0 = ow0 - ci.pad_left;
+  const unsigned x_img = ((unsigned)n * ci.in_h * ci.in_w * C + c) * 4u;
+  const unsigned y_img = ((unsigned)n * ci.out_h * ci.out_w * C + c) * 4u;
+  const unsigned x_row = (unsigned)ci.in_w * C * 4u, y_row = (unsigned)ci.out_w * C * 4u;
+  unsigned col_in[IW], col_out[TW];
+#pragma unroll
+  for (int q = 0; q < IW; q++)
+    col_in[q] = (unsigned)(iw0 + q) < (unsigned)ci.in_w ? x_img + (unsigned)(iw0 + q) * C * 4u : OOB;
+#pragma unroll
+  for (int j = 0; j < TW; j++)
+    col_out[j] = ow0 + j < ci.out_w ? y_img + (unsigned)(ow0 + j) * C * 4u : OOB;
+  const int ih_first = oh0 - ci.pad_top;         // filter row 0 of output row oh0
+  const int ih_last = oh1 - 1 - ci.pad_top + 2;  // filter row 2 of output row oh1 - 1
+
+  auto load_row = [&](int ih, f32x4 (&in)[IW]) {
+    const bool row_ok = (unsigned)ih < (unsigned)ci.in_h && ih <= ih_last;
+    const unsigned at = (unsigned)ih * x_row;
+#pragma unroll
+    for (int q = 0; q < IW; q++)
+      in[q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                            rx, (int)(row_ok ? at + col_in[q] : OOB), 0, 0));
+  };
+  auto store_row = [&](int oh, const f32x4 (&acc)[TW]) {
+    const bool row_ok = oh >= oh0 && oh < oh1;
+    const unsigned at = (unsigned)oh * y_row;
+#pragma unroll
+    for (int j = 0; j < TW; j++) {
+      f32x4 v = acc[j] + b;
+#pragma unroll
+      for (int e = 0; e < 4; e++) v[e] = act_fast(v[e], af);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), ry,
+                                             (int)(row_ok ? at + col_out[j] : OOB), 0, 0);
+    }
+  };
+  // Input row ih is filter row kh of output row ih + pad_top - kh: `newest` starts with it
+  // (kh = 0), `middle` gets its second filter row, `oldest` its last and is complete.
+  auto feed = [&](const f32x4 (&in)[IW], f32x4 (&oldest)[TW], f32x4 (&middle)[TW],
+                  f32x4 (&newest)[TW]) {
+#pragma unroll
+    for (int j = 0; j < TW; j++) {
+      f32x4 a = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kw = 0; kw < 3; kw++) a += in[j + kw] * w[kw];
+      newest[j] = a;
+#pragma unroll
+      for (int kw = 0; kw < 3; kw++) middle[j] += in[j + kw] * w[3 + kw];
+#pragma unroll
+      for (int kw = 0; kw < 3; kw++) oldest[j] += in[j + kw] * w[6 + kw];
+    }
+  };
+  // One step: start the loads of the next input row, feed the current one, store the output
+  // row it completes (input row ih completes output row ih + pad_top - 2).
+  auto step = [&](int ih, const f32x4 (&in)[IW], f32x4 (&next)[IW], f32x4 (&oldest)[TW],
+                  f32x4 (&middle)[TW], f32x4 (&newest)[TW]) {
+    load_row(ih + 1, next);
+    __builtin_amdgcn_sched_barrier(0);  // loads first, and none from a later step
+    feed(in, oldest, middle, newest);
+    store_row(ih + ci.pad_top - 2, oldest);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  f32x4 r0[TW], r1[TW], r2[TW];
+#pragma unroll
+  for (int j = 0; j < TW; j++) r0[j] = r1[j] = r2[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  f32x4 cur[IW], nxt[IW];
+  load_row(ih_first, cur);
+  // Two row buffers and three accumulator rows take turns: the pattern repeats every 6 rows.
+  // Steps past ih_last load nothing and store nothing.
+  for (int ih = ih_first; ih <= ih_last; ih += 6) {
+    step(ih, cur, nxt, r0, r1, r2);
+    step(ih + 1, nxt, cur, r1, r2, r0);
+    step(ih + 2, cur, nxt, r2, r0, r1);
+    step(ih + 3, nxt, cur, r0, r1, r2);
+    step(ih + 4, cur, nxt, r1, r2, r0);
+    step(ih + 5, nxt, cur, r2, r0, r1);
   }
 }
 
@@ -238,6 +389,18 @@ static void launch_dw3x3(tfhip_ctx* ctx, DwArgs& p) {
                      dim3(256), 0, ctx->stream, p);
 }
 
+template <int TW>
+static void launch_dw3x3_rows(tfhip_ctx* ctx, DwArgs& p, int rows) {
+  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise3x3_s1_rows_w%d", TW);
+  const int chunks = (int)ceil_div(p.ci.out_h, rows);
+  p.tiles_w = (int)ceil_div(p.ci.out_w, TW);
+  const int64_t total = (int64_t)p.ci.batch * chunks * p.tiles_w * p.c4;
+  hipLaunchKernelGGL((depthwise3x3_rows_kernel<TW>), dim3((unsigned)ceil_div(total, 256)),
+                     dim3(256), 0, ctx->stream, p, rows, chunks,
+                     (unsigned)((int64_t)p.ci.batch * p.ci.in_h * p.ci.in_w * p.ci.in_c * 4),
+                     (unsigned)((int64_t)p.ci.batch * p.ci.out_h * p.ci.out_w * p.ci.out_c * 4));
+}
+
 static int check_geometry(tfhip_ctx* ctx, const char* op, const tfhip_conv2d_info* ci) {
   if (ci->batch < 0 || ci->in_h < 0 || ci->in_w < 0 || ci->in_c < 0 || ci->out_h < 0 ||
       ci->out_w < 0 || ci->out_c < 0 || ci->filter_h <= 0 || ci->filter_w <= 0 ||
@@ -313,7 +476,23 @@ extern "C" int tfhip_depthwise_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter,
     p.c4 = ci->in_c / 4;
     // Patch shapes picked by measurement on MI355X (fp32, batch 32-64): 2x8 patches for wide,
     // deep rows, 2x2 elsewhere; stride 2 streams best with one output per lane.
-    if (ci->stride_h == 1) {
+    // Stride 1: the row-walking kernel when the image is large enough to give every SIMD a
+    // few wavefronts (it fetches each input row once), else 2x2 patches.  Measured on MI355X
+    // (fp32, batch 32-64): 28-row chunks stream best; halve them when that would leave a
+    // second, nearly empty round of wavefronts, or too few wavefronts.
+    int rows = 0;
+    if (ci->stride_h == 1 && x_n * 4 < (1ll << 31) && o_n * 4 < (1ll << 31)) {
+      const int64_t lanes_per_chunk = (int64_t)ci->batch * ceil_div(ci->out_w, 2) * p.c4;
+      const int64_t slots = (int64_t)ctx->num_cus * 12;  // 3 wavefronts per SIMD
+      auto waves = [&](int r) { return lanes_per_chunk * ceil_div(ci->out_h, r) / 64; };
+      rows = ci->out_h < 28 ? ci->out_h : 28;
+      while (rows > 7 && waves(rows) < slots / 2) rows = (rows + 1) / 2;
+      if (rows > 7 && waves(rows) > slots && waves(rows) * 2 < slots * 3) rows = (rows + 1) / 2;
+      if (waves(rows) < slots / 4) rows = 0;
+    }
+    if (rows > 0) {
+      launch_dw3x3_rows<2>(ctx, p, rows);
+    } else if (ci->stride_h == 1) {
       if (ci->out_w >= 112 && ci->in_c >= 128 && ci->out_w % 8 == 0) launch_dw3x3<1, 2, 8>(ctx, p);
       else launch_dw3x3<1, 2, 2>(ctx, p);
     } else {
