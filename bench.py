@@ -30,11 +30,12 @@ RIDGE = PEAK_FP32_MFMA_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
 # this process, so the figures are carried here; they apply to batch 64, fp32 weights.
 MIB = 1 << 20
 MEASURED_HBM_BYTES_PER_LAUNCH = {
-    "gemm_64x64_rowmajor_f32": 103.8 * MIB,
-    "gemm_64x128_rowmajor_f32": 47.3 * MIB,
-    "depthwise3x3_s1_2x2": 84.7 * MIB,
+    "gemm_64x64_rowmajor_f32": 104.3 * MIB,
+    "gemm_64x128_rowmajor_f32": 35.4 * MIB,
+    "gemm_64x64_rowmajor_f32_tailk": 66.9 * MIB,
+    "depthwise3x3_s1_rows_w2": 87.6 * MIB,
     "depthwise3x3_s2_1x1": 115.0 * MIB,
-    "conv_smallk_n32_f32": 153.3 * MIB,
+    "conv_smallk_n32_f32": 153.2 * MIB,
     "global_avgpool": 12.5 * MIB,
 }
 
@@ -126,6 +127,67 @@ def roofline_of_dominant_kernel(rows):
     return roof, groups
 
 
+def op_level_configs(tf, np):
+    """Configs 1-3 of BASELINE.json (single matMul, the 3-layer MLP, one fused conv2d and one
+    depthwiseConv2D) at their full sizes: every op timed with an event pair on the backend's
+    stream around back-to-back launches, priced by its algorithmic flops and bytes (operands
+    and result counted once) against the fp32 matrix peak and the HBM peak."""
+    be = tf.backend()
+    rng = np.random.default_rng(1)
+    out = []
+
+    def timed(name, fn, reps, flops, nbytes):
+        tf.dispose(fn())
+        def many():
+            for _ in range(reps):
+                tf.dispose(fn())
+        tf.time(many)                       # brings the clocks up
+        ms = min(tf.time(many)["kernelMs"] for _ in range(3)) / reps
+        tfl, gbs = flops / ms * 1e-9, nbytes / ms * 1e-6
+        dense = flops / nbytes >= RIDGE
+        out.append(dict(op=name, kernel=be.lib.tfhip_last_kernel(be.ctx).decode(),
+                        us=round(ms * 1e3, 2), tflops=round(tfl, 2), gbs=round(gbs, 1),
+                        bound="mfma" if dense else "hbm",
+                        frac=round(tfl / PEAK_FP32_MFMA_TFLOPS if dense else gbs / PEAK_HBM_GBS, 4)))
+
+    def f32(a):
+        return tf.tensor(np.asarray(a, np.float32))
+
+    a, b = f32(rng.uniform(-1, 1, (256, 512))), f32(rng.uniform(-1, 1, (512, 256)))
+    timed("config 1: matMul [256,512]x[512,256]", lambda: tf.matmul(a, b), 1000,
+          2.0 * 256 * 512 * 256, 4.0 * (256 * 512 + 512 * 256 + 256 * 256))
+    tf.dispose([a, b])
+
+    h = f32(rng.uniform(0, 1, (4096, 784)))
+    keep = [h]
+    for i, (cin, cout, act) in enumerate(((784, 1024, "relu"), (1024, 1024, "relu"), (1024, 10, "linear"))):
+        wt = f32(rng.standard_normal((cin, cout)) * np.sqrt(2.0 / cin))
+        bias = f32(np.zeros(cout))
+        layer = lambda h=h, wt=wt, bias=bias, act=act: tf.fused.matmul(h, wt, False, False, bias=bias,
+                                                                       activation=act)
+        timed("config 2: fused matMul 4096x%d->%d %s" % (cin, cout, act), layer, 200,
+              2.0 * 4096 * cin * cout, 4.0 * (4096 * cin + cin * cout + 4096 * cout + cout))
+        h = layer()
+        keep += [wt, bias, h]
+    tf.dispose(keep)
+
+    x = f32(rng.uniform(0, 1, (32, 112, 112, 64)))
+    wt = f32(rng.standard_normal((3, 3, 64, 128)) * np.sqrt(2.0 / (9 * 64)))
+    bias = f32(rng.standard_normal(128) * 0.1)
+    timed("config 3: fused conv2d 3x3 [32,112,112,64]->128 bias relu6",
+          lambda: tf.fused.conv2d(x, wt, 1, "same", bias=bias, activation="relu6"), 50,
+          2.0 * 32 * 112 * 112 * 128 * 9 * 64, 4.0 * (32 * 112 * 112 * (64 + 128) + 9 * 64 * 128 + 128))
+    tf.dispose([x, wt, bias])
+    x = f32(rng.uniform(0, 1, (32, 112, 112, 128)))
+    wt = f32(rng.standard_normal((3, 3, 128, 1)) * np.sqrt(2.0 / 9))
+    bias = f32(rng.standard_normal(128) * 0.1)
+    timed("config 3: fused depthwiseConv2D 3x3 [32,112,112,128] bias relu6",
+          lambda: tf.fused.depthwise_conv2d(x, wt, 1, "same", bias=bias, activation="relu6"), 100,
+          2.0 * 32 * 112 * 112 * 128 * 9, 4.0 * (2 * 32 * 112 * 112 * 128 + 9 * 128 + 128))
+    tf.dispose([x, wt, bias])
+    return out
+
+
 def cpu_baseline(mobilenet, params, budget_s=15.0):
     """The CPU oracle (restatement of backend_cpu's loops, one thread) on batch-1 forwards
     of the same network: a bounded sample, reported as images/s."""
@@ -212,6 +274,8 @@ def main():
     ap.add_argument("--quant", action="store_true", help="uint8 weights dequantised in-kernel")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-js", action="store_true", help="skip the Node.js host leg")
+    ap.add_argument("--no-ops", action="store_true",
+                    help="skip the op-level configs (single matMul, MLP layers, conv2d, depthwise)")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
     ap.add_argument("--calibrate-counters", action="store_true",
                     help="only launch a streaming kernel of known size (relu over 256 MiB: reads "
@@ -324,6 +388,13 @@ def main():
                                   gbs=round(g["bytes"] / g["ms"] * 1e-6, 1))
                           for k, g in groups.items()},
     }
+    if not args.no_ops:
+        out["op_configs"] = op_level_configs(tf, np)
+        if args.layers:
+            for r in out["op_configs"]:
+                print("%-66s %-36s %9.2f us %7.2f TFLOP/s %7.1f GB/s  %s %.3f" % (
+                    r["op"], r["kernel"], r["us"], r["tflops"], r["gbs"], r["bound"], r["frac"]),
+                    file=sys.stderr)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(mobilenet, params)
     print(json.dumps(out))

@@ -69,6 +69,9 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void reduce_rows_kernel(
 
 // softmax over the last axis with the rounding points of the reference composite:
 // m = max(x); e = exp(x - m); s = sum(e); lse = m + log(s); y = exp(x - lse).
+// SLOTS > 0: the row fits SLOTS registers per lane (cols <= 64 * SLOTS): one pass over
+// memory with all loads in flight.  SLOTS == 0: any length, three passes.
+template <int SLOTS>
 __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void softmax_rows_kernel(
     const float* x, float* y, int64_t rows, int64_t cols) {
   const int lane = threadIdx.x & (WAVE - 1);
@@ -77,16 +80,16 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void softmax_rows_kernel(
   const float* xr = x + row * cols;
   float* yr = y + row * cols;
   float m = xr[0];
-  if (cols <= WAVE * 16) {
-    // the row fits the wavefront's registers: one pass over memory, all loads in flight
-    float v[16];
+  if (SLOTS > 0) {
+    constexpr int S = SLOTS > 0 ? SLOTS : 1;
+    float v[S];
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
+    for (int i = 0; i < S; i++) {
       const int64_t j = lane + i * WAVE;
       v[i] = xr[j < cols ? j : 0];
     }
 #pragma unroll
-    for (int i = 0; i < 16; i++)
+    for (int i = 0; i < S; i++)
       if (v[i] > m) m = v[i];
     for (int off = WAVE / 2; off > 0; off >>= 1) {
       const float o = __shfl_xor(m, off, WAVE);
@@ -94,12 +97,12 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void softmax_rows_kernel(
     }
     double s = 0.0;
 #pragma unroll
-    for (int i = 0; i < 16; i++)
+    for (int i = 0; i < S; i++)
       if (lane + i * WAVE < cols) s += (double)expf(v[i] - m);
     for (int off = WAVE / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, WAVE);
     const float lse = m + logf((float)s);
 #pragma unroll
-    for (int i = 0; i < 16; i++)
+    for (int i = 0; i < S; i++)
       if (lane + i * WAVE < cols) yr[lane + i * WAVE] = expf(v[i] - lse);
     return;
   }
@@ -213,8 +216,16 @@ extern "C" int tfhip_softmax_rows(tfhip_ctx* ctx, int64_t x, int64_t out, int64_
   const float* xf;
   int rc;
   if ((rc = as_f32(ctx, bx, &tx, &xf))) return rc;
-  hipLaunchKernelGGL(softmax_rows_kernel, dim3((unsigned)ceil_div(rows, ROWS_PER_BLOCK)),
-                     dim3(WAVE * ROWS_PER_BLOCK), 0, ctx->stream, xf, (float*)bo->ptr, rows, cols);
+  const dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK)), block(WAVE * ROWS_PER_BLOCK);
+  float* yf = static_cast<float*>(bo->ptr);
+  if (cols <= WAVE)
+    hipLaunchKernelGGL(softmax_rows_kernel<1>, grid, block, 0, ctx->stream, xf, yf, rows, cols);
+  else if (cols <= WAVE * 4)
+    hipLaunchKernelGGL(softmax_rows_kernel<4>, grid, block, 0, ctx->stream, xf, yf, rows, cols);
+  else if (cols <= WAVE * 16)
+    hipLaunchKernelGGL(softmax_rows_kernel<16>, grid, block, 0, ctx->stream, xf, yf, rows, cols);
+  else
+    hipLaunchKernelGGL(softmax_rows_kernel<0>, grid, block, 0, ctx->stream, xf, yf, rows, cols);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }
