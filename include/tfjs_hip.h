@@ -216,6 +216,30 @@ int tfhip_resize_bilinear(tfhip_ctx* ctx, int64_t x, int64_t out, int batch, int
 int tfhip_one_hot(tfhip_ctx* ctx, int64_t indices, int64_t out, int depth, float on_value,
                   float off_value);
 
+/* ---- backward kernels (training) ---------------------------------------------------------- */
+/* `info` is the Conv2DInfo of the FORWARD op in every call below (in_* = x, out_* = y).
+ * conv2dDerInput (backend.ts:423-425; backend_cpu.ts:1686-1762): dy [batch,out_h,out_w,out_c],
+ * filter [fh,fw,in_c,out_c] -> dx [batch,in_h,in_w,in_c] float32.  Also the forward pass of
+ * conv2dTranspose (ops/conv.ts:783-790).  Dilation must be 1 (ops/conv.ts:240-243). */
+int tfhip_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int64_t filter, int64_t dx,
+                           const tfhip_conv2d_info* info);
+/* conv2dDerFilter (backend.ts:427-429; backend_cpu.ts:1849-1898): x, dy -> dW
+ * [fh,fw,in_c,out_c] float32. */
+int tfhip_conv2d_der_filter(tfhip_ctx* ctx, int64_t x, int64_t dy, int64_t dw,
+                            const tfhip_conv2d_info* info);
+/* depthwiseConv2DDerInput / depthwiseConv2DDerFilter (backend.ts:435-441;
+ * backend_cpu.ts:2037-2150): filter and dW are [fh,fw,in_c,ch_mul]. */
+int tfhip_depthwise_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int64_t filter, int64_t dx,
+                                     const tfhip_conv2d_info* info);
+int tfhip_depthwise_conv2d_der_filter(tfhip_ctx* ctx, int64_t x, int64_t dy, int64_t dw,
+                                      const tfhip_conv2d_info* info);
+/* maxPoolBackprop / avgPoolBackprop (backend.ts:456-465; backend_cpu.ts:2347-2509): dy, the
+ * forward input x (values used by TFHIP_POOL_MAX only; first strict maximum of a window wins,
+ * NaN never does) -> dx float32.  avg multiplies by 1 / (fh * fw) whatever part of a window
+ * lay inside the image, as the reference does.  Dilation is allowed (tf.pool). */
+int tfhip_pool2d_backprop(tfhip_ctx* ctx, int64_t dy, int64_t x, int64_t dx,
+                          const tfhip_conv2d_info* info, int kind);
+
 #ifdef __cplusplus
 }
 #endif

@@ -178,6 +178,221 @@ void ref_pool2d(const float* x, float* y, const ref_conv2d_info* ci, int kind) {
       }
 }
 
+/* ---- backward kernels --------------------------------------------------------------- */
+
+/* backends/cpu/backend_cpu.ts:1686-1762 (channelsLast).  The loop bounds are JavaScript
+ * numbers: yRMax = min(outHeight, (filterHeight + xRCorner) / strideHeight) is fractional and
+ * compared with `<`; one double dot product per dx element, stored to float once. */
+void ref_conv2d_der_input(const float* dy, const float* w, float* dx, const ref_conv2d_info* ci) {
+  const int fh = ci->filter_h, fw = ci->filter_w, ic = ci->in_c, oc = ci->out_c;
+  const int top_pad = fh - 1 - ci->pad_top, left_pad = fw - 1 - ci->pad_left;
+  const int64_t x_row = (int64_t)ci->in_w * ic, x_b = x_row * ci->in_h;
+  const int64_t y_row = (int64_t)ci->out_w * oc, y_b = y_row * ci->out_h;
+  const int64_t w_s0 = (int64_t)fw * ic * oc, w_s1 = (int64_t)ic * oc, w_s2 = oc;
+  for (int b = 0; b < ci->batch; ++b)
+    for (int d1 = 0; d1 < ic; ++d1)
+      for (int xr = 0; xr < ci->in_h; ++xr) {
+        const int xr_corner = xr - top_pad;
+        const double yr_min = fmax(0.0, ceil((double)xr_corner / ci->stride_h));
+        const double yr_max = fmin((double)ci->out_h, (double)(fh + xr_corner) / ci->stride_h);
+        for (int xc = 0; xc < ci->in_w; ++xc) {
+          const int xc_corner = xc - left_pad;
+          const double yc_min = fmax(0.0, ceil((double)xc_corner / ci->stride_w));
+          const double yc_max = fmin((double)ci->out_w, (double)(fw + xc_corner) / ci->stride_w);
+          double dot = 0.0;
+          for (int yr = (int)yr_min; yr < yr_max; ++yr) {
+            const int wr = yr * ci->stride_h - xr_corner;
+            for (int yc = (int)yc_min; yc < yc_max; ++yc) {
+              const int wc = yc * ci->stride_w - xc_corner;
+              const float* dyp = dy + b * y_b + yr * y_row + (int64_t)yc * oc;
+              const float* wp = w + w_s0 * (fh - 1 - wr) + w_s1 * (fw - 1 - wc) + w_s2 * d1;
+              for (int d2 = 0; d2 < oc; ++d2) dot += (double)dyp[d2] * (double)wp[d2];
+            }
+          }
+          dx[b * x_b + xr * x_row + (int64_t)xc * ic + d1] = (float)dot;
+        }
+      }
+}
+
+/* backends/cpu/backend_cpu.ts:1849-1898 (channelsLast): per filter element one double dot
+ * product over batch, output rows and columns, stored to float once. */
+void ref_conv2d_der_filter(const float* x, const float* dy, float* dw, const ref_conv2d_info* ci) {
+  const int fh = ci->filter_h, fw = ci->filter_w, ic = ci->in_c, oc = ci->out_c;
+  const int64_t x_row = (int64_t)ci->in_w * ic, x_b = x_row * ci->in_h;
+  const int64_t y_row = (int64_t)ci->out_w * oc, y_b = y_row * ci->out_h;
+  for (int wr = 0; wr < fh; ++wr) {
+    const double yr_min = fmax(0.0, ceil((double)(ci->pad_top - wr) / ci->stride_h));
+    const double yr_max = fmin((double)ci->out_h, (double)(ci->in_h + ci->pad_top - wr) / ci->stride_h);
+    for (int wc = 0; wc < fw; ++wc) {
+      const double yc_min = fmax(0.0, ceil((double)(ci->pad_left - wc) / ci->stride_w));
+      const double yc_max = fmin((double)ci->out_w, (double)(ci->in_w + ci->pad_left - wc) / ci->stride_w);
+      for (int d1 = 0; d1 < ic; ++d1)
+        for (int d2 = 0; d2 < oc; ++d2) {
+          double dot = 0.0;
+          for (int b = 0; b < ci->batch; ++b)
+            for (int yr = (int)yr_min; yr < yr_max; ++yr) {
+              const int xr = wr + yr * ci->stride_h - ci->pad_top;
+              for (int yc = (int)yc_min; yc < yc_max; ++yc) {
+                const int xc = wc + yc * ci->stride_w - ci->pad_left;
+                dot += (double)x[b * x_b + xr * x_row + (int64_t)xc * ic + d1] *
+                       (double)dy[b * y_b + yr * y_row + (int64_t)yc * oc + d2];
+              }
+            }
+          dw[(((int64_t)wr * fw + wc) * ic + d1) * oc + d2] = (float)dot;
+        }
+    }
+  }
+}
+
+/* backends/cpu/backend_cpu.ts:2037-2103. */
+void ref_depthwise_conv2d_der_input(const float* dy, const float* w, float* dx,
+                                    const ref_conv2d_info* ci) {
+  const int fh = ci->filter_h, fw = ci->filter_w, ic = ci->in_c, oc = ci->out_c;
+  const int ch_mul = oc / ic;
+  const int top_pad = fh - 1 - ci->pad_top, left_pad = fw - 1 - ci->pad_left;
+  const int64_t x_row = (int64_t)ci->in_w * ic, x_b = x_row * ci->in_h;
+  const int64_t y_row = (int64_t)ci->out_w * oc, y_b = y_row * ci->out_h;
+  const int64_t w_s0 = (int64_t)fw * ic * ch_mul, w_s1 = (int64_t)ic * ch_mul, w_s2 = ch_mul;
+  for (int b = 0; b < ci->batch; ++b)
+    for (int d1 = 0; d1 < ic; ++d1)
+      for (int xr = 0; xr < ci->in_h; ++xr) {
+        const int xr_corner = xr - top_pad;
+        const double yr_min = fmax(0.0, ceil((double)xr_corner / ci->stride_h));
+        const double yr_max = fmin((double)ci->out_h, (double)(fh + xr_corner) / ci->stride_h);
+        for (int xc = 0; xc < ci->in_w; ++xc) {
+          const int xc_corner = xc - left_pad;
+          const double yc_min = fmax(0.0, ceil((double)xc_corner / ci->stride_w));
+          const double yc_max = fmin((double)ci->out_w, (double)(fw + xc_corner) / ci->stride_w);
+          double dot = 0.0;
+          for (int yr = (int)yr_min; yr < yr_max; ++yr) {
+            const int wr = yr * ci->stride_h - xr_corner;
+            for (int yc = (int)yc_min; yc < yc_max; ++yc) {
+              const int wc = yc * ci->stride_w - xc_corner;
+              const float* dyp = dy + b * y_b + yr * y_row + (int64_t)yc * oc;
+              const float* wp = w + w_s0 * (fh - 1 - wr) + w_s1 * (fw - 1 - wc) + w_s2 * d1;
+              for (int dm = 0; dm < ch_mul; ++dm)
+                dot += (double)dyp[d1 * ch_mul + dm] * (double)wp[dm];
+            }
+          }
+          dx[b * x_b + xr * x_row + (int64_t)xc * ic + d1] = (float)dot;
+        }
+      }
+}
+
+/* backends/cpu/backend_cpu.ts:2105-2150. */
+void ref_depthwise_conv2d_der_filter(const float* x, const float* dy, float* dw,
+                                     const ref_conv2d_info* ci) {
+  const int fh = ci->filter_h, fw = ci->filter_w, ic = ci->in_c, oc = ci->out_c;
+  const int ch_mul = oc / ic;
+  const int64_t x_row = (int64_t)ci->in_w * ic, x_b = x_row * ci->in_h;
+  const int64_t y_row = (int64_t)ci->out_w * oc, y_b = y_row * ci->out_h;
+  for (int wr = 0; wr < fh; ++wr) {
+    const double yr_min = fmax(0.0, ceil((double)(ci->pad_top - wr) / ci->stride_h));
+    const double yr_max = fmin((double)ci->out_h, (double)(ci->in_h + ci->pad_top - wr) / ci->stride_h);
+    for (int wc = 0; wc < fw; ++wc) {
+      const double yc_min = fmax(0.0, ceil((double)(ci->pad_left - wc) / ci->stride_w));
+      const double yc_max = fmin((double)ci->out_w, (double)(ci->in_w + ci->pad_left - wc) / ci->stride_w);
+      for (int d2 = 0; d2 < oc; ++d2) {
+        const int d1 = d2 / ch_mul, dm = d2 % ch_mul;
+        double dot = 0.0;
+        for (int b = 0; b < ci->batch; ++b)
+          for (int yr = (int)yr_min; yr < yr_max; ++yr) {
+            const int xr = wr + yr * ci->stride_h - ci->pad_top;
+            for (int yc = (int)yc_min; yc < yc_max; ++yc) {
+              const int xc = wc + yc * ci->stride_w - ci->pad_left;
+              dot += (double)x[b * x_b + xr * x_row + (int64_t)xc * ic + d1] *
+                     (double)dy[b * y_b + yr * y_row + (int64_t)yc * oc + d2];
+            }
+          }
+        dw[(((int64_t)wr * fw + wc) * ic + d1) * ch_mul + dm] = (float)dot;
+      }
+    }
+  }
+}
+
+/* backends/cpu/backend_cpu.ts:2347-2398: position (within the dilated window, row-major over
+ * the effective filter) of the first strict maximum; -1 when nothing beats -inf. */
+void ref_max_pool_positions(const float* x, int32_t* pos, const ref_conv2d_info* ci) {
+  const int eff_h = ci->filter_h + (ci->filter_h - 1) * (ci->dilation_h - 1);
+  const int eff_w = ci->filter_w + (ci->filter_w - 1) * (ci->dilation_w - 1);
+  const int64_t x_row = (int64_t)ci->in_w * ci->in_c, x_b = x_row * ci->in_h;
+  const int64_t y_row = (int64_t)ci->out_w * ci->out_c, y_b = y_row * ci->out_h;
+  for (int b = 0; b < ci->batch; ++b)
+    for (int d = 0; d < ci->in_c; ++d)
+      for (int yr = 0; yr < ci->out_h; ++yr) {
+        const int xr_corner = yr * ci->stride_h - ci->pad_top;
+        int xr_min = xr_corner;
+        while (xr_min < 0) xr_min += ci->dilation_h;
+        const int xr_max = ci->in_h < eff_h + xr_corner ? ci->in_h : eff_h + xr_corner;
+        for (int yc = 0; yc < ci->out_w; ++yc) {
+          const int xc_corner = yc * ci->stride_w - ci->pad_left;
+          int xc_min = xc_corner;
+          while (xc_min < 0) xc_min += ci->dilation_w;
+          const int xc_max = ci->in_w < eff_w + xc_corner ? ci->in_w : eff_w + xc_corner;
+          double max_value = -INFINITY;
+          int max_position = -1;
+          for (int xr = xr_min; xr < xr_max; xr += ci->dilation_h) {
+            const int wr = xr - xr_corner;
+            for (int xc = xc_min; xc < xc_max; xc += ci->dilation_w) {
+              const int wc = xc - xc_corner;
+              const double pixel = (double)x[b * x_b + xr * x_row + (int64_t)xc * ci->in_c + d];
+              if (pixel > max_value) {
+                max_value = pixel;
+                max_position = wr * eff_w + wc;
+              }
+            }
+          }
+          pos[b * y_b + yr * y_row + (int64_t)yc * ci->out_c + d] = max_position;
+        }
+      }
+}
+
+/* backends/cpu/backend_cpu.ts:2400-2457 (kind 1, needs x) and :2459-2509 (kind 0: the sum of
+ * the dy that cover the pixel times 1 / (filterHeight * filterWidth), whatever part of the
+ * window was inside the image). */
+void ref_pool2d_backprop(const float* dy, const float* x, float* dx, const ref_conv2d_info* ci,
+                         int kind) {
+  const int eff_h = ci->filter_h + (ci->filter_h - 1) * (ci->dilation_h - 1);
+  const int eff_w = ci->filter_w + (ci->filter_w - 1) * (ci->dilation_w - 1);
+  const int pad_left = eff_w - 1 - ci->pad_left, pad_top = eff_h - 1 - ci->pad_top;
+  const int64_t x_row = (int64_t)ci->in_w * ci->in_c, x_b = x_row * ci->in_h;
+  const int64_t y_row = (int64_t)ci->out_w * ci->out_c, y_b = y_row * ci->out_h;
+  const double avg_multiplier = 1.0 / (double)(ci->filter_h * ci->filter_w);
+  int32_t* pos = NULL;
+  if (kind == 1) {
+    pos = (int32_t*)malloc(sizeof(int32_t) * (size_t)(y_b * ci->batch));
+    ref_max_pool_positions(x, pos, ci);
+  }
+  for (int b = 0; b < ci->batch; ++b)
+    for (int d = 0; d < ci->in_c; ++d)
+      for (int dxr = 0; dxr < ci->in_h; ++dxr)
+        for (int dxc = 0; dxc < ci->in_w; ++dxc) {
+          const int dyr_corner = dxr - pad_top, dyc_corner = dxc - pad_left;
+          double dot = 0.0;
+          for (int wr = 0; wr < eff_h; wr += ci->dilation_h) {
+            const int num_r = dyr_corner + wr;
+            if (num_r < 0 || num_r % ci->stride_h != 0) continue;
+            const int dyr = num_r / ci->stride_h;
+            if (dyr >= ci->out_h) continue;
+            for (int wc = 0; wc < eff_w; wc += ci->dilation_w) {
+              const int num_c = dyc_corner + wc;
+              if (num_c < 0 || num_c % ci->stride_w != 0) continue;
+              const int dyc = num_c / ci->stride_w;
+              if (dyc >= ci->out_w) continue;
+              const int64_t at = b * y_b + dyr * y_row + (int64_t)dyc * ci->out_c + d;
+              if (kind == 1) {
+                const int max_pos = eff_h * eff_w - 1 - pos[at];
+                if (max_pos != wr * eff_w + wc) continue;
+              }
+              dot += (double)dy[at];
+            }
+          }
+          dx[b * x_b + dxr * x_row + (int64_t)dxc * ci->in_c + d] =
+              (float)(kind == 1 ? dot : dot * avg_multiplier);
+        }
+  free(pos);
+}
+
 /* ---- elementwise ------------------------------------------------------------------- */
 enum { REF_ADD = 0, REF_SUB, REF_MUL, REF_DIV, REF_PRELU, REF_MAXIMUM, REF_MINIMUM };
 

@@ -231,6 +231,64 @@ def max_pool(x, ci):
     return _pool(x, ci, 1)
 
 
+# ---- backward kernels (backends/cpu/backend_cpu.ts:1686-1762, 1849-1898, 2037-2150,
+# 2347-2509).  `ci` is the Conv2DInfo of the forward op.
+def conv2d_der_input(dy, w, ci):
+    dy, w = _f32(dy), _f32(w)
+    dx = np.empty(ci["inShape"], np.float32)
+    info = _info_c(ci)
+    lib().ref_conv2d_der_input(_p(dy), _p(w), _p(dx), C.byref(info))
+    return dx
+
+
+def conv2d_der_filter(x, dy, ci):
+    x, dy = _f32(x), _f32(dy)
+    dw = np.empty(ci["filterShape"], np.float32)
+    info = _info_c(ci)
+    lib().ref_conv2d_der_filter(_p(x), _p(dy), _p(dw), C.byref(info))
+    return dw
+
+
+def depthwise_conv2d_der_input(dy, w, ci):
+    dy, w = _f32(dy), _f32(w)
+    dx = np.empty(ci["inShape"], np.float32)
+    info = _info_c(ci)
+    lib().ref_depthwise_conv2d_der_input(_p(dy), _p(w), _p(dx), C.byref(info))
+    return dx
+
+
+def depthwise_conv2d_der_filter(x, dy, ci):
+    x, dy = _f32(x), _f32(dy)
+    dw = np.empty(ci["filterShape"], np.float32)
+    info = _info_c(ci)
+    lib().ref_depthwise_conv2d_der_filter(_p(x), _p(dy), _p(dw), C.byref(info))
+    return dw
+
+
+def max_pool_positions(x, ci):
+    x = _f32(x)
+    pos = np.empty(ci["outShape"], np.int32)
+    info = _info_c(ci)
+    lib().ref_max_pool_positions(_p(x), _p(pos, C.c_int32), C.byref(info))
+    return pos
+
+
+def _pool_backprop(dy, x, ci, kind):
+    dy, x = _f32(dy), _f32(x)
+    dx = np.empty(ci["inShape"], np.float32)
+    info = _info_c(ci)
+    lib().ref_pool2d_backprop(_p(dy), _p(x), _p(dx), C.byref(info), kind)
+    return dx
+
+
+def avg_pool_backprop(dy, x, ci):
+    return _pool_backprop(dy, x, ci, 0)
+
+
+def max_pool_backprop(dy, x, ci):
+    return _pool_backprop(dy, x, ci, 1)
+
+
 _BIN = dict(add=0, sub=1, mul=2, div=3, prelu=4, maximum=5, minimum=6)
 
 

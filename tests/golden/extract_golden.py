@@ -59,6 +59,19 @@ CASES = {
                   ["batchNorm4D", "batchNorm3D", "batchNorm2D"]),
     "resize_bilinear": ("tfjs-core/src/ops/resize_bilinear_test.ts", ["resizeBilinear"]),
 }
+# fixture name -> (reference test file, describe blocks, title filter): the gradient blocks,
+# whose expected values pin the backward kernels (conv2dDerInput / conv2dDerFilter behind
+# tf.grads of conv2d and behind conv2dTranspose, the depthwise and pooling backprops).  A
+# describe's beforeEach block is recorded as a case titled "beforeEach".
+GRAD_CASES = {
+    "conv2d_grad": ("tfjs-core/src/ops/conv2d_test.ts", ["conv2d"], r"^gradient(?!.*NCHW)"),
+    "conv2d_transpose": ("tfjs-core/src/ops/conv2d_transpose_test.ts", ["conv2dTranspose"],
+                         r"^(input=|gradient)"),
+    "depthwise_grad": ("tfjs-core/src/ops/conv2d_depthwise_test.ts",
+                       ["depthwiseConv2d gradients"], r"^(beforeEach|wrt )"),
+    "pool_grad": ("tfjs-core/src/ops/pool_test.ts", ["maxPoolBackprop", "avgPool", "poolBackprop"],
+                  r"gradient"),
+}
 # blocks whose title matches are not forward known-answer cases
 SKIP = re.compile(r"grad|throw|raises|tensor-like|TensorLike|does not match|do not match|"
                   r"dont match|non-tensor|string tensor|Unsupported|error", re.I)
@@ -92,8 +105,9 @@ def _match_paren(src, j):
     return j
 
 
-def blocks_of(src, describes):
-    """Yield (describe, title, body) for each it() block of the wanted describe blocks."""
+def blocks_of(src, describes, before_each=False):
+    """Yield (describe, title, body) for each it() block of the wanted describe blocks (and,
+    on request, for their beforeEach blocks under the title "beforeEach")."""
     scopes = []
     for m in re.finditer(r"\bdescribe\w*\(\s*['\"]([^'\"]*)['\"]", src):
         end = _match_paren(src, src.index("(", m.start()) + 1)
@@ -107,6 +121,10 @@ def blocks_of(src, describes):
             j = start + m.start()
             stop = _match_paren(src, src.index("(", j) + 1)
             yield name, m.group(2), src[start + m.end():stop]
+        for m in re.finditer(r"\bbeforeEach\(", src[start:end] if before_each else ""):
+            j = start + m.start()
+            stop = _match_paren(src, src.index("(", j) + 1)
+            yield name, "beforeEach", src[j:stop]
 
 
 def consts_of(body):
@@ -312,6 +330,19 @@ def main():
         out = {"source": rel, "cases": []}
         for describe, title, body in blocks_of(src, describes):
             if SKIP.search(title):
+                continue
+            out["cases"].append({"describe": describe, "title": title,
+                                 "consts": consts_of(body), "arrays": arrays_of(body)})
+        path = os.path.join(OUT, name + ".json")
+        with open(path, "w") as f:
+            json.dump(out, f, separators=(",", ":"))
+            f.write("\n")
+        print(name, len(out["cases"]), "cases", os.path.getsize(path), "bytes")
+    for name, (rel, describes, keep) in GRAD_CASES.items():
+        src = open(os.path.join(REF, rel)).read()
+        out = {"source": rel, "cases": []}
+        for describe, title, body in blocks_of(src, describes, before_each=True):
+            if not re.search(keep, title) or re.search(r"throw|tensor-like", title, re.I):
                 continue
             out["cases"].append({"describe": describe, "title": title,
                                  "consts": consts_of(body), "arrays": arrays_of(body)})

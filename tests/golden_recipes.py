@@ -734,3 +734,132 @@ def resize_bilinear_known_answers(ops):
         expect_close(ops.resize_bilinear(f32(a[0], a[1]), a[2], align), a[3])
     a = g("batch of 2, simple, alignCorners=true")
     expect_close(ops.resize_bilinear(f32(a[0], a[1]), a[2], True), a[3])
+
+
+# ---- gradient blocks: conv2d_test.ts, conv2d_transpose_test.ts, conv2d_depthwise_test.ts,
+# pool_test.ts.  tf.grads of conv2d = (conv2dDerInput, conv2dDerFilter) (ops/conv.ts:236-250);
+# conv2dTranspose = conv2dDerInput on the output shape (:783-790), and its gradients are
+# conv2d(dy, filter) and conv2dDerFilter(dy, x) (:395-405).
+def _lift(a):
+    return a[None] if a.ndim == 3 else a
+
+
+@recipe
+def conv2d_gradients(ops):
+    for title, xs, dys in (("gradient with clones input=[3,3,1] f=[2,2,1,1] s=1 p=0",
+                            (1, 3, 3, 1), (1, 2, 2, 1)),
+                           ("gradient x=[2,3,3,1] f=[2,2,1,1] s=1 p=0", (2, 3, 3, 1), (2, 2, 2, 1))):
+        a = golden_case("conv2d_grad", title)["arrays"]
+        x, dy = f32(a[4], xs), f32(a[5], dys)
+        w = np.ones((2, 2, 1, 1), np.float32)
+        expect_close(ops.conv2d_der_input(xs, dy, w, 1, 0), a[8])
+        want_dw = a[9] if a[9] is not None else [26, 38, 62, 74]   # written as 13 * 2 ... there
+        expect_close(ops.conv2d_der_filter(x, dy, (2, 2, 1, 1), 1, 0), want_dw)
+
+
+@recipe
+def conv2d_transpose_known_answers(ops):
+    for title, xs, out in (("input=2x2x1,d2=1,f=2,s=1,p=0", (1, 1, 1, 1), (1, 2, 2, 1)),
+                           ("input=2x2x1,d2=1,f=2,s=1,p=0, batch=2", (2, 1, 1, 1), (2, 2, 2, 1))):
+        a = golden_case("conv2d_transpose", title)["arrays"]
+        x, w = f32(a[2], xs), f32(a[3], (2, 2, 1, 1))
+        expect_close(ops.conv2d_der_input(out, x, w, 1, 0), a[6])
+
+
+@recipe
+def conv2d_transpose_gradients(ops):
+    # (title, positions of x, filter, expected dx, expected dfilter, x shape, output shape, stride, pad)
+    for title, ix, iw, idx, idw, xs, out, stride, pad in (
+            ("gradient input=[1,3,3,1] f=[2,2,2,1] s=[1,1] padding=same", 6, 7, 11, 12,
+             (1, 3, 3, 1), (1, 3, 3, 2), 1, "same"),
+            ("gradient input=[1,2,2,2] f=[2,2,2,1] s=[2,2] padding=same", 6, 7, 11, 13,
+             (1, 2, 2, 2), (1, 3, 3, 2), 2, "same")):
+        a = golden_case("conv2d_transpose", title)["arrays"]
+        x = f32(np.array(a[ix]).ravel(), xs)
+        w = f32(np.array(a[iw]).ravel(), (2, 2, 2, xs[3]))
+        dy = np.ones(out, np.float32)
+        # forward value: the transposed convolution itself is conv2dDerInput
+        y = ops.conv2d_der_input(out, x, w, stride, pad)
+        assert y.shape == out
+        expect_close(ops.conv2d(dy, w, stride, pad), np.array(a[idx]).ravel())
+        expect_close(ops.conv2d_der_filter(dy, x, w.shape, stride, pad), np.array(a[idw]).ravel())
+
+
+@recipe
+def depthwise_gradients(ops):
+    g = lambda t: golden_case("depthwise_grad", t)["arrays"]
+    b = g("beforeEach")
+    images = f32(np.array(b[0]).ravel(), (2, 2, 2, 3))
+    filt = f32(np.array(b[1]).ravel(), (2, 2, 3, 2))
+    result = f32(np.array(b[2]).ravel(), (2, 2, 2, 6))
+    expect_close(ops.depthwise_conv2d(images, filt, 1, "same"), result)
+    ones = np.ones_like(result)
+    expect_close(ops.depthwise_der_input(images.shape, ones, filt, 1, "same"),
+                 np.array(g("wrt input")[0]).ravel())
+    expect_close(ops.depthwise_der_filter(images, ones, filt.shape, 1, "same"),
+                 np.array(g("wrt filter")[0]).ravel())
+    # d/dx of square(y) = derInput(2 y)
+    expect_close(ops.depthwise_der_input(images.shape, 2 * result, filt, 1, "same"),
+                 np.array(g("wrt input, squared output")[0]).ravel())
+    expect_close(ops.depthwise_der_filter(images, 2 * result, filt.shape, 1, "same"),
+                 np.array(g("wrt filter, squared output")[0]).ravel())
+    y2 = ops.depthwise_conv2d(images, filt, 2, "valid")
+    expect_close(ops.depthwise_der_input(images.shape, np.ones_like(y2), filt, 2, "valid"),
+                 g("wrt input, stride=2, pad=valid")[0])
+    expect_close(ops.depthwise_der_filter(images, np.ones_like(y2), filt.shape, 2, "valid"),
+                 g("wrt filter, stride=2, pad=valid")[0])
+
+
+@recipe
+def max_pool_gradients(ops):
+    for title, f, s in (
+            ("gradients x=[3,3,1] f=[2,2] s=1 no dup max value, test #1", 2, 1),
+            ("gradients x=[3,3,1] f=[2,2] s=1 no dup max value, test #2", 2, 1),
+            ("gradients x=[2,3,3,1] f=[2,2] s=1 no duplicate max value", 2, 1),
+            ("gradient x=[3,3,1] f=[2,2] s=1 dup max value, test 1", 2, 1),
+            ("gradient x=[3,3,1] f=[2,2] s=1 dup max value, test 2", 2, 1),
+            ("gradient x=[2,3,3,1] f=[2,2] s=1 dup max value in 2nd input", 2, 1),
+            ("gradient x=[4,4,1] f=[2,2] s=2 test #1", 2, 2),
+            ("gradient x=[4,4,1] f=[2,2] s=2 test #2", 2, 2),
+            ("gradient x=[5,5,1] f=[3,3] s=2 no duplicate max value", 3, 2),
+            ("gradient x=[5,5,1] f=[3,3] s=2 duplicate max value", 3, 2),
+            ("gradient x=[3,3,2] f=[2,2] s=1, no duplicate max value", 2, 1),
+            ("gradient x=[3,3,2] f=[2,2] s=1 duplicate max value", 2, 1),
+            ("gradient x=[4,4,2] f=[2,2] s=1", 2, 2),   # the block calls maxPool(2, 2, 0)
+            ("gradient x=5x5x2, f=3, s=2 no duplicate max value", 3, 2)):
+        a = golden_case("pool_grad", title, "maxPoolBackprop")["arrays"]
+        dy, x = _lift(f32(a[0], a[1])), _lift(f32(a[2], a[3]))
+        expect_close(ops.max_pool_backprop(dy, x, f, s, 0), a[4])
+    for title in ("max gradients x=[3,3,1] f=[2,2] s=1 d=1 no dup max value",
+                  "max gradients x=[3,3,1] f=[2,2] s=1 d=2 no dup max value, test #1",
+                  "max gradients x=[3,3,1] f=[2,2] s=1 d=2 no dup max value, test #2",
+                  "max gradient x=[3,3,1] f=[2,2] s=1 d=2 dup max value"):
+        c = golden_case("pool_grad", title, "poolBackprop")
+        a, d = c["arrays"], c["consts"].get("dilationRate", 1)
+        dy, x = _lift(f32(a[0], a[1])), _lift(f32(a[2], a[3]))
+        expect_close(ops.max_pool_backprop(dy, x, 2, 1, 0, dilations=d), a[4])
+
+
+@recipe
+def avg_pool_gradients(ops):
+    a = golden_case("pool_grad", "gradient x=[1,1,1] f=[1,1] s=1 [0] => [0]", "avgPool")["arrays"]
+    expect_close(ops.avg_pool_backprop(_lift(f32(a[2], a[3])), _lift(f32(a[0], a[1])), 1, 1, 0), a[4])
+    # expected values are written there as products with avgMultiplier = 1 / (2 * 2):
+    # every dy spreads a quarter of itself over its 2x2 window
+    for title in ("gradient x=[3,3,1] f=[2,2] s=1", "gradient x=[2,3,3,1] f=[2,2], s=1"):
+        a = golden_case("pool_grad", title, "avgPool")["arrays"]
+        x, dy = _lift(f32(a[0], a[1])), _lift(f32(a[2], a[3]))
+        want = np.zeros(x.shape, np.float64)
+        for i in range(2):
+            for j in range(2):
+                want[:, i:i + 2, j:j + 2, :] += dy[:, i:i + 1, j:j + 1, :] * 0.25
+        expect_close(ops.avg_pool_backprop(dy, x, 2, 1, 0), want.ravel())
+    a = golden_case("pool_grad", "avg gradient x=[4,4,1] f=[2,2] s=1 d=2", "poolBackprop")["arrays"]
+    x, dy = _lift(f32(a[0], a[1])), _lift(f32(a[2], a[3]))
+    want = np.zeros(x.shape, np.float64)
+    for i in range(3):
+        for j in range(3):
+            for di in (0, 2):
+                for dj in (0, 2):
+                    want[0, i + di, j + dj, 0] += dy[0, i, j, 0] * 0.25
+    expect_close(ops.avg_pool_backprop(dy, x, 2, 1, 0, dilations=2), want.ravel())

@@ -44,6 +44,33 @@ class OracleOps:
         return self.r.max_pool(x, self.r.compute_pool2d_info(x.shape, fsize, strides, dilations,
                                                               pad, rounding))
 
+    # backward kernels; the Conv2DInfo is that of the forward op (ops/conv.ts:354-420,
+    # 466-520, ops/pool.ts:333-397), dilation 1 for the convolutions
+    def conv2d_der_input(self, x_shape, dy, w, strides, pad, rounding=None):
+        ci = self.r.compute_conv2d_info(x_shape, w.shape, strides, 1, pad, rounding)
+        return self.r.conv2d_der_input(dy, w, ci)
+
+    def conv2d_der_filter(self, x, dy, filter_shape, strides, pad, rounding=None):
+        ci = self.r.compute_conv2d_info(x.shape, filter_shape, strides, 1, pad, rounding)
+        return self.r.conv2d_der_filter(x, dy, ci)
+
+    def depthwise_der_input(self, x_shape, dy, w, strides, pad):
+        ci = self.r.compute_conv2d_info(x_shape, w.shape, strides, 1, pad, None, depthwise=True)
+        return self.r.depthwise_conv2d_der_input(dy, w, ci)
+
+    def depthwise_der_filter(self, x, dy, filter_shape, strides, pad):
+        ci = self.r.compute_conv2d_info(x.shape, filter_shape, strides, 1, pad, None,
+                                        depthwise=True)
+        return self.r.depthwise_conv2d_der_filter(x, dy, ci)
+
+    def max_pool_backprop(self, dy, x, fsize, strides, pad, dilations=1):
+        return self.r.max_pool_backprop(dy, x, self.r.compute_pool2d_info(
+            x.shape, fsize, strides, dilations, pad))
+
+    def avg_pool_backprop(self, dy, x, fsize, strides, pad, dilations=1):
+        return self.r.avg_pool_backprop(dy, x, self.r.compute_pool2d_info(
+            x.shape, fsize, strides, dilations, pad))
+
     def add(self, a, b): return self.r.add(a, b)
     def sub(self, a, b): return self.r.subtract(a, b)
     def mul(self, a, b): return self.r.multiply(a, b)
@@ -152,6 +179,36 @@ class HipOps:
         if dilations != 1:
             return self._run(lambda a: tf.pool(a, fsize, "max", pad, dilations, strides), x)
         return self._run(lambda a: tf.max_pool(a, fsize, strides, pad, rounding), x)
+
+    def conv2d_der_input(self, x_shape, dy, w, strides, pad, rounding=None):
+        tf = self.tf
+        return self._run(lambda d, f: tf.conv2d_der_input(x_shape, d, f, strides, pad, "NHWC",
+                                                          rounding), dy, w)
+
+    def conv2d_der_filter(self, x, dy, filter_shape, strides, pad, rounding=None):
+        tf = self.tf
+        return self._run(lambda a, d: tf.conv2d_der_filter(a, d, filter_shape, strides, pad,
+                                                           "NHWC", rounding), x, dy)
+
+    def depthwise_der_input(self, x_shape, dy, w, strides, pad):
+        tf = self.tf
+        return self._run(lambda d, f: tf.depthwise_conv2d_der_input(x_shape, d, f, strides, pad),
+                         dy, w)
+
+    def depthwise_der_filter(self, x, dy, filter_shape, strides, pad):
+        tf = self.tf
+        return self._run(lambda a, d: tf.depthwise_conv2d_der_filter(a, d, filter_shape, strides,
+                                                                     pad), x, dy)
+
+    def max_pool_backprop(self, dy, x, fsize, strides, pad, dilations=1):
+        tf = self.tf
+        return self._run(lambda d, a: tf.max_pool_backprop(d, a, fsize, strides, pad, dilations),
+                         dy, x)
+
+    def avg_pool_backprop(self, dy, x, fsize, strides, pad, dilations=1):
+        tf = self.tf
+        return self._run(lambda d, a: tf.avg_pool_backprop(d, a, fsize, strides, pad, dilations),
+                         dy, x)
 
     def add(self, a, b): return self._run(self.tf.add, a, b)
     def sub(self, a, b): return self._run(self.tf.sub, a, b)

@@ -277,3 +277,44 @@ def test_js_mobilenet_matches_oracle(tmp_path, ref, quant):
     if gap[-1] - gap[-2] > 2e-3:
         top = np.fromfile(os.path.join(c.dir, "mobilenet.top.bin"), np.int32)
         assert top[0] == int(np.argmax(want[0]))
+
+
+def test_js_backward_ops_match_oracle(tmp_path, ref):
+    """conv2dDerInput / conv2dDerFilter / conv2dTranspose, the depthwise and pooling backprops
+    through the JS host and the N-API addon."""
+    rng = np.random.default_rng(47)
+    c = Cases(tmp_path)
+    f = lambda *s: rng.uniform(-1, 1, s).astype(np.float32)
+    x, w = f(2, 9, 11, 8), f(3, 3, 8, 12) * 0.3
+    for tag, stride, pad in (("s1", 1, "same"), ("s2", 2, "same"), ("valid", [2, 1], "valid")):
+        dy = f(*ref.conv2d(x, w, stride, pad).shape)
+        c.add("der_input_" + tag, "conv2dDerInput", dict(dy=dy, filter=w),
+              dict(xShape=list(x.shape), strides=stride, pad=pad),
+              ref.conv2d_der_input(x.shape, dy, w, stride, pad), atol=2e-5)
+        c.add("der_filter_" + tag, "conv2dDerFilter", dict(x=x, dy=dy),
+              dict(filterShape=list(w.shape), strides=stride, pad=pad),
+              ref.conv2d_der_filter(x, dy, w.shape, stride, pad), atol=1e-4)
+    small, wt = f(5, 5, 6), f(4, 4, 3, 6) * 0.3      # rank-3 input: batch of 1 assumed
+    c.add("transpose_rank3", "conv2dTranspose", dict(x=small, filter=wt),
+          dict(outputShape=[10, 10, 3], strides=2, pad="same"),
+          ref.conv2d_der_input((1, 10, 10, 3), small[None], wt, 2, "same")[0], atol=2e-5)
+    xd, wd = f(2, 8, 8, 6), f(3, 3, 6, 2)
+    for tag, stride, pad in (("s1", 1, "same"), ("s2", 2, "valid")):
+        dy = f(*ref.depthwise_conv2d(xd, wd, stride, pad).shape)
+        c.add("dw_der_input_" + tag, "depthwiseConv2dDerInput", dict(dy=dy, filter=wd),
+              dict(xShape=list(xd.shape), strides=stride, pad=pad),
+              ref.depthwise_der_input(xd.shape, dy, wd, stride, pad))
+        c.add("dw_der_filter_" + tag, "depthwiseConv2dDerFilter", dict(x=xd, dy=dy),
+              dict(filterShape=list(wd.shape), strides=stride, pad=pad),
+              ref.depthwise_der_filter(xd, dy, wd.shape, stride, pad), atol=2e-5)
+    xp = rng.integers(0, 5, (2, 9, 9, 3)).astype(np.float32)
+    for tag, fs, stride, pad, dil in (("f2s2", 2, 2, "valid", 1), ("f3s1same", 3, 1, "same", 1), ("d2", 2, 1, 0, 2)):
+        dy = f(*ref.max_pool(xp, fs, stride, pad, dilations=dil).shape)
+        args = dict(filterSize=fs, strides=stride, pad=pad, dilations=dil)
+        c.add("max_backprop_" + tag, "maxPoolBackprop", dict(dy=dy, x=xp), args,
+              ref.max_pool_backprop(dy, xp, fs, stride, pad, dil))
+        c.add("avg_backprop_" + tag, "avgPoolBackprop", dict(dy=dy, x=xp), args,
+              ref.avg_pool_backprop(dy, xp, fs, stride, pad, dil))
+    results = c.run()
+    c.check(results)
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0

@@ -158,3 +158,52 @@ def test_implicit_gemm_3x3_tiles(tf):
             b, i, j = rng.integers(n), rng.integers(h), rng.integers(h)
             want = np.einsum("abc,abco->o", xp[b, i:i + 3, j:j + 3, :], w64)
             close(got[b, i, j], want)
+
+
+# ------------------------------------- row lengths that are not multiples of 4 ----
+@pytest.mark.parametrize("m,k,n,ta,tb", [
+    (67, 37, 10, False, False), (67, 37, 10, True, False), (67, 37, 10, False, True),
+    (67, 37, 10, True, True), (130, 49, 33, False, False), (5, 3, 2, False, False),
+    (4096, 1024, 10, False, False), (257, 1001, 7, False, True), (66, 50, 129, True, False),
+])
+def test_matmul_odd_row_lengths(tf, m, k, n, ta, tb):
+    """Row lengths that are not multiples of 4 (the element-wise loaders): a NaN at the start
+    of the next row in memory must not leak into a row's result."""
+    print("odd matmul", m, k, n, ta, tb, flush=True)
+    rng = np.random.default_rng(m * 7 + k * 3 + n + 2 * ta + tb)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    if m > 8 and k > 8:
+        a[m // 2 + 1, 0] = np.nan      # follows the end of row m//2 in memory (row-major A)
+        b[k // 2 + 1, 0] = np.nan      # follows the end of row k//2 (row-major B)
+    a_in = np.ascontiguousarray(a.T) if ta else a
+    b_in = np.ascontiguousarray(b.T) if tb else b
+    with tf.tidy():
+        got = tf.matmul(tf.tensor(a_in), tf.tensor(b_in), ta, tb).data_sync()
+        kern = last_kernel(tf)
+    assert kern.startswith("gemm_"), kern
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    close(got, want, atol=1e-4)
+
+
+def test_batched_matmul_odd_strides(tf):
+    rng = np.random.default_rng(77)
+    a = rng.uniform(-1, 1, (3, 9, 7)).astype(np.float32)
+    b = rng.uniform(-1, 1, (3, 7, 5)).astype(np.float32)
+    with tf.tidy():
+        got = tf.matmul(tf.tensor(a), tf.tensor(b)).data_sync()
+    close(got, a.astype(np.float64) @ b.astype(np.float64))
+
+
+def test_pointwise_conv_odd_channels(tf):
+    rng = np.random.default_rng(78)
+    x = rng.uniform(-1, 1, (2, 9, 11, 37)).astype(np.float32)
+    w = (rng.standard_normal((1, 1, 37, 21)) * 0.2).astype(np.float32)
+    x[1, 3, 4, 0] = np.inf
+    with tf.tidy():
+        got = tf.conv2d(tf.tensor(x), tf.tensor(w), 1, "same").data_sync()
+    want = (x.reshape(-1, 37).astype(np.float64) @ w.reshape(37, 21).astype(np.float64)).reshape(2, 9, 11, 21)
+    assert np.array_equal(np.isfinite(got), np.isfinite(want))
+    ok = np.isfinite(want)
+    close(got[ok], want[ok])

@@ -468,3 +468,80 @@ def test_one_hot_bit_exact(hip, ref):
     idx = np.array([[0, 3, -1], [7, 2, 99]], np.int32)
     got = hip.one_hot(idx, 8, 5, -1)
     assert got.dtype == np.int32 and np.array_equal(got, ref.one_hot(idx, 8, 5, -1))
+
+
+# ------------------------------------------------------- backward kernels ----
+@pytest.mark.parametrize("xs,fs,stride,pad", [
+    ((2, 12, 12, 8), (3, 3, 8, 16), 1, "same"),        # buffer-load path (channels % 4 == 0)
+    ((1, 15, 13, 4), (3, 3, 4, 40), 2, "same"),        # stride 2: dy stretched by the stride
+    ((2, 16, 16, 3), (3, 3, 3, 32), 2, "same"),        # Cin = 3: element-wise loaders
+    ((1, 9, 9, 5), (3, 3, 5, 7), 1, "valid"),
+    ((1, 14, 14, 64), (1, 1, 64, 128), 1, "same"),     # pointwise
+    ((1, 14, 14, 8), (1, 1, 8, 12), 2, "same"),        # 1x1 stride 2: most of dx is zero
+    ((1, 11, 11, 8), (5, 5, 8, 8), 1, "same"),
+    ((1, 10, 12, 8), (2, 4, 8, 8), (1, 2), "valid"),
+    ((3, 7, 7, 32), (3, 3, 32, 200), 1, 1),
+    ((2, 9, 9, 4), (3, 3, 4, 4), 3, "same"),
+    ((4, 28, 28, 32), (3, 3, 32, 64), 1, "same"),      # long contraction for dW: split along K
+])
+def test_conv2d_backward(hip, ref, xs, fs, stride, pad):
+    print("conv2d backward", xs, fs, stride, pad, flush=True)
+    rng = np.random.default_rng(sum(xs) * 3 + sum(fs))
+    x = rng.uniform(-1, 1, xs).astype(np.float32)
+    w = (rng.standard_normal(fs) * np.sqrt(2.0 / (fs[0] * fs[1] * fs[2]))).astype(np.float32)
+    y = ref.conv2d(x, w, stride, pad)
+    dy = rng.uniform(-1, 1, y.shape).astype(np.float32)
+    close(hip.conv2d_der_input(xs, dy, w, stride, pad), ref.conv2d_der_input(xs, dy, w, stride, pad),
+          atol=2e-5)
+    close(hip.conv2d_der_filter(x, dy, fs, stride, pad), ref.conv2d_der_filter(x, dy, fs, stride, pad),
+          atol=1e-4)
+
+
+def test_conv2d_transpose_upsamples(hip, ref):
+    """conv2dTranspose (= conv2dDerInput on the output shape) of a 7x7 map to 14x14, and a NaN
+    in dy reaches exactly the dx pixels whose window covers it."""
+    rng = np.random.default_rng(21)
+    x = rng.uniform(-1, 1, (2, 7, 7, 16)).astype(np.float32)
+    w = (rng.standard_normal((4, 4, 8, 16)) * 0.2).astype(np.float32)   # [fh, fw, outDepth, inDepth]
+    close(hip.conv2d_der_input((2, 14, 14, 8), x, w, 2, "same"),
+          ref.conv2d_der_input((2, 14, 14, 8), x, w, 2, "same"), atol=2e-5)
+    x[1, 3, 3, 5] = np.nan
+    got = hip.conv2d_der_input((2, 14, 14, 8), x, w, 2, "same")
+    want = ref.conv2d_der_input((2, 14, 14, 8), x, w, 2, "same")
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+
+
+@pytest.mark.parametrize("xs,fs,stride,pad", [
+    ((2, 12, 12, 8), (3, 3, 8, 1), 1, "same"),
+    ((1, 15, 15, 4), (3, 3, 4, 2), 2, "same"),
+    ((2, 9, 9, 3), (3, 3, 3, 3), 2, "valid"),
+    ((1, 10, 10, 130), (3, 3, 130, 1), 1, "same"),     # more than one block of 64 channels
+    ((3, 8, 8, 5), (5, 5, 5, 1), 1, "same"),
+    ((2, 28, 28, 32), (3, 3, 32, 1), (2, 1), "valid"),
+])
+def test_depthwise_backward(hip, ref, xs, fs, stride, pad):
+    print("depthwise backward", xs, fs, stride, pad, flush=True)
+    rng = np.random.default_rng(sum(xs) * 5 + sum(fs))
+    x = rng.uniform(-1, 1, xs).astype(np.float32)
+    w = rng.standard_normal(fs).astype(np.float32)
+    # dy shape from the hip forward op (square inputs: the reference's pad quirk does not bite)
+    y = hip.depthwise_conv2d(x, w, stride, pad)
+    dy = rng.uniform(-1, 1, y.shape).astype(np.float32)
+    close(hip.depthwise_der_input(xs, dy, w, stride, pad), ref.depthwise_der_input(xs, dy, w, stride, pad))
+    close(hip.depthwise_der_filter(x, dy, fs, stride, pad), ref.depthwise_der_filter(x, dy, fs, stride, pad),
+          atol=2e-5)
+
+
+@pytest.mark.parametrize("xs,f,s,pad,dil", [
+    ((2, 12, 12, 8), 2, 2, 0, 1), ((1, 13, 13, 3), 3, 2, "same", 1), ((2, 7, 7, 5), 3, 1, "same", 1),
+    ((1, 9, 9, 4), 2, 1, 0, 2), ((1, 14, 14, 64), (2, 3), (2, 1), "valid", 1),
+])
+def test_pool_backprop(hip, ref, xs, f, s, pad, dil):
+    print("pool backprop", xs, f, s, pad, dil, flush=True)
+    rng = np.random.default_rng(sum(xs) + 17)
+    x = rng.integers(0, 6, xs).astype(np.float32)        # many ties: the first maximum wins
+    x[0, 2, 2, 0] = np.nan                               # NaN never wins
+    y = ref.max_pool(x, f, s, pad, dilations=dil)
+    dy = rng.uniform(-1, 1, y.shape).astype(np.float32)
+    close(hip.max_pool_backprop(dy, x, f, s, pad, dil), ref.max_pool_backprop(dy, x, f, s, pad, dil))
+    close(hip.avg_pool_backprop(dy, x, f, s, pad, dil), ref.avg_pool_backprop(dy, x, f, s, pad, dil))

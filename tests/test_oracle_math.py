@@ -173,3 +173,67 @@ def test_gather_transpose_to_int(ops):
     assert np.array_equal(ops.transpose(x, [2, 0, 1]), x.transpose(2, 0, 1))
     v = np.array([1.9, -1.9, 0.5, np.nan, np.inf, 3e9], np.float32)
     assert ops.to_int(v).tolist() == [1, -1, 0, 0, 0, int(np.int64(3000000000) - 2**32)]
+
+
+# ---- backward kernels: pinned by adjointness / directional derivatives, which a wrong
+# sign, flipped filter index, swapped padding or stride fails ---------------------------
+@pytest.mark.parametrize("stride,pad", [(1, "valid"), (1, "same"), ((2, 1), "same"), (2, "valid"),
+                                        (2, 1), (3, "same")])
+def test_conv2d_backward_kernels_are_the_adjoints(ops, stride, pad):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((2, 7, 9, 3)).astype(np.float32)
+    w = rng.standard_normal((3, 2, 3, 4)).astype(np.float32)
+    if pad == 1:
+        x = x[:, :, :8]          # a numeric pad needs integral output sizes: (8 - 3 + 2) / 2
+        x = x[:, :7]
+    try:
+        y = ops.conv2d(x, w, stride, pad)
+    except ValueError:
+        pytest.skip("non-integral output size for this numeric pad")
+    dy = rng.standard_normal(y.shape).astype(np.float32)
+    lhs = float((y.astype(np.float64) * dy).sum())
+    dx = ops.conv2d_der_input(x.shape, dy, w, stride, pad)
+    dw = ops.conv2d_der_filter(x, dy, w.shape, stride, pad)
+    assert dx.shape == x.shape and dw.shape == w.shape
+    assert abs(float((dx.astype(np.float64) * x).sum()) - lhs) < 1e-3 * max(1, abs(lhs))
+    assert abs(float((dw.astype(np.float64) * w).sum()) - lhs) < 1e-3 * max(1, abs(lhs))
+
+
+@pytest.mark.parametrize("stride,pad,ch_mul", [(1, "same", 1), (2, "same", 2), (2, "valid", 3),
+                                               ((1, 2), "valid", 1)])
+def test_depthwise_backward_kernels_are_the_adjoints(ops, oracle, stride, pad, ch_mul):
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((2, 6, 6, 3)).astype(np.float32)   # square: padLeft == padTop
+    w = rng.standard_normal((3, 3, 3, ch_mul)).astype(np.float32)
+    y = ops.depthwise_conv2d(x, w, stride, pad)
+    dy = rng.standard_normal(y.shape).astype(np.float32)
+    lhs = float((y.astype(np.float64) * dy).sum())
+    dx = ops.depthwise_der_input(x.shape, dy, w, stride, pad)
+    dw = ops.depthwise_der_filter(x, dy, w.shape, stride, pad)
+    assert abs(float((dx.astype(np.float64) * x).sum()) - lhs) < 1e-3 * max(1, abs(lhs))
+    assert abs(float((dw.astype(np.float64) * w).sum()) - lhs) < 1e-3 * max(1, abs(lhs))
+
+
+@pytest.mark.parametrize("fsize,stride,dil", [(2, 1, 1), (3, 2, 1), (2, 1, 2), (3, 1, 1)])
+def test_pool_backprops(ops, fsize, stride, dil):
+    rng = np.random.default_rng(13)
+    x = rng.permutation(2 * 7 * 7 * 2).reshape(2, 7, 7, 2).astype(np.float32)  # no ties
+    v = rng.standard_normal(x.shape).astype(np.float32)
+    y = ops.max_pool(x, fsize, stride, "valid", dilations=dil)
+    dy = rng.standard_normal(y.shape).astype(np.float32)
+    # max: y(x + eps v) - y(x) = eps * J v while the winners do not change (values differ by
+    # at least 1, |eps v| stays below 0.5); <dy, J v> = <J^T dy, v>
+    eps = 0.1
+    v = np.clip(v, -4, 4)
+    jv = (ops.max_pool(x + eps * v, fsize, stride, "valid", dilations=dil).astype(np.float64) - y) / eps
+    dx = ops.max_pool_backprop(dy, x, fsize, stride, "valid", dilations=dil)
+    assert abs(float((jv * dy).sum()) - float((dx.astype(np.float64) * v).sum())) < 1e-2
+    # avg with valid padding: every window is whole, so backprop is the exact adjoint
+    ya = ops.avg_pool(v, fsize, stride, "valid", dilations=dil)
+    dxa = ops.avg_pool_backprop(dy, x, fsize, stride, "valid", dilations=dil)
+    assert abs(float((ya.astype(np.float64) * dy).sum()) -
+               float((dxa.astype(np.float64) * v).sum())) < 1e-3
+    # and with 'same' padding the multiplier stays 1 / (f * f) although windows are cut
+    dxs = ops.avg_pool_backprop(np.ones((1, 3, 3, 1), np.float32), np.zeros((1, 3, 3, 1), np.float32),
+                                2, 1, "same")
+    assert np.allclose(dxs.ravel(), np.array([1, 2, 2, 2, 4, 4, 2, 4, 4]) / 4.0)

@@ -30,7 +30,11 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
-enum { A_ROWMAJOR = 0, A_TRANSPOSED = 1, A_IM2COL = 2 };
+// A_IM2COL_UP: the gather of conv2dDerInput (rows are input pixels, k is (filter row, filter
+// column, output channel) of the flipped filter; the image gathered from is dy, stretched by
+// the forward stride).  A_IM2COL_T: the gather of conv2dDerFilter (rows are (filter row,
+// filter column, input channel), k runs over the output pixels (n, oh, ow)).
+enum { A_ROWMAJOR = 0, A_TRANSPOSED = 1, A_IM2COL = 2, A_IM2COL_UP = 3, A_IM2COL_T = 4 };
 enum { B_ROWMAJOR = 0, B_TRANSPOSED = 1, B_UINT8 = 2 };
 
 struct GemmArgs {
@@ -46,6 +50,7 @@ struct GemmArgs {
   int a_vec, b_vec;  // operands allow aligned 4-element accesses
   // implicit-GEMM geometry (A_IM2COL): rows are (n, oh, ow), k is (kh, kw, c)
   int H, W, Cin, OH, OW, KH, KW, sh, sw, dh, dw, pt, pl;
+  int up_h, up_w;  // A_IM2COL_UP: forward strides (dy is read at row / up_h when divisible)
   double qscale, qmin;
   // schedule (see work_item)
   int tiles_m, tiles_n, k_tiles, full_tiles, tail_tiles, splits, kt_per;
@@ -189,6 +194,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       if (AMODE == A_TRANSPOSED) {
         L.a_kq[i] = item / (BM / 4);           // k within the tile
         L.a_row[i] = (item % (BM / 4)) * 4;    // first of 4 rows
+      } else if (AMODE == A_IM2COL_T) {
+        L.a_kq[i] = item / (BM / 4);
+        L.a_row[i] = (item % (BM / 4)) * 4;
+        const int m = L.bm0 + L.a_row[i];      // (filter row, filter column, channel)
+        if (m >= p.M) L.a_ok[i] = false;
+        const int tap = m / p.Cin, c = m - tap * p.Cin;
+        const int kh = tap / p.KW, kw = tap - kh * p.KW;
+        L.a_base[i] = c;
+        L.a_ih0[i] = kh * p.dh - p.pt;
+        L.a_iw0[i] = kw * p.dw - p.pl;
       } else {
         L.a_row[i] = item / (BK / 4);
         L.a_kq[i] = (item % (BK / 4)) * 4;
@@ -226,10 +241,22 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
           const int m = L.bm0 + L.a_row[i];
           ok = ok && m < p.M;  // M % 4 == 0: the quad is inside or outside as a whole
           off = (unsigned)k * p.lda + m;
+        } else if (AMODE == A_IM2COL_T) {
+          // k is an output pixel (n, oh, ow); the item's tap and channel quad are fixed
+          const int ow = k % p.OW, r = k / p.OW;
+          const int oh = r % p.OH, n = r / p.OH;
+          const int ih = L.a_ih0[i] + oh * p.sh, iw = L.a_iw0[i] + ow * p.sw;
+          ok = ok && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+          off = (unsigned)((n * p.H + ih) * p.W + iw) * p.Cin + (unsigned)L.a_base[i];
         } else {
           const int tap = k / p.Cin, c = k - tap * p.Cin;
           const int kh = tap / p.KW, kw = tap - kh * p.KW;
-          const int ih = L.a_ih0[i] + kh * p.dh, iw = L.a_iw0[i] + kw * p.dw;
+          int ih = L.a_ih0[i] + kh * p.dh, iw = L.a_iw0[i] + kw * p.dw;
+          if (AMODE == A_IM2COL_UP) {
+            ok = ok && ih >= 0 && iw >= 0 && ih % p.up_h == 0 && iw % p.up_w == 0;
+            ih /= p.up_h;
+            iw /= p.up_w;
+          }
           ok = ok && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
           off = (unsigned)L.a_base[i] + (unsigned)(ih * p.W + iw) * p.Cin + c;
         }
@@ -264,14 +291,42 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
                 if (m + e < p.M) v[e] = src[e];
             }
           }
-        } else {  // A_IM2COL
+        } else if (AMODE == A_IM2COL_T) {
           const int k = k0 + L.a_kq[i];
+          if (k < p.K) {
+            const int ow = k % p.OW, r = k / p.OW;
+            const int oh = r % p.OH, n = r / p.OH;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const int m = L.bm0 + L.a_row[i] + e;
+              if (m < p.M) {
+                const int tap = m / p.Cin, c = m - tap * p.Cin;
+                const int kh = tap / p.KW, kw = tap - kh * p.KW;
+                const int ih = kh * p.dh - p.pt + oh * p.sh, iw = kw * p.dw - p.pl + ow * p.sw;
+                if ((unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W)
+                  v[e] = L.A[(((long long)n * p.H + ih) * p.W + iw) * p.Cin + c];
+              }
+            }
+          }
+        } else {  // A_IM2COL, A_IM2COL_UP
+          const int k = k0 + L.a_kq[i];
+          // dy row / column of a tap: stretched by the forward stride for A_IM2COL_UP
+          auto source = [&](int kh, int kw, int& ih, int& iw) {
+            ih = L.a_ih0[i] + kh * p.dh;
+            iw = L.a_iw0[i] + kw * p.dw;
+            if (AMODE == A_IM2COL_UP) {
+              if (ih < 0 || iw < 0 || ih % p.up_h != 0 || iw % p.up_w != 0) return false;
+              ih /= p.up_h;
+              iw /= p.up_w;
+            }
+            return (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+          };
           if (p.a_vec) {  // Cin % 4 == 0: the 4 elements share one filter tap
             if (k < p.K) {
               const int tap = k / p.Cin, c = k - tap * p.Cin;
               const int kh = tap / p.KW, kw = tap - kh * p.KW;
-              const int ih = L.a_ih0[i] + kh * p.dh, iw = L.a_iw0[i] + kw * p.dw;
-              if ((unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W)
+              int ih, iw;
+              if (source(kh, kw, ih, iw))
                 v = *reinterpret_cast<const f32x4*>(
                     L.A + L.a_base[i] + ((long long)ih * p.W + iw) * p.Cin + c);
             }
@@ -282,8 +337,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
               if (ke < p.K) {
                 const int tap = ke / p.Cin, c = ke - tap * p.Cin;
                 const int kh = tap / p.KW, kw = tap - kh * p.KW;
-                const int ih = L.a_ih0[i] + kh * p.dh, iw = L.a_iw0[i] + kw * p.dw;
-                if ((unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W)
+                int ih, iw;
+                if (source(kh, kw, ih, iw))
                   v[e] = L.A[L.a_base[i] + ((long long)ih * p.W + iw) * p.Cin + c];
               }
             }
@@ -299,7 +354,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     for (int i = 0; i < A_PER; i++) {
       const int item = tid + i * THREADS;
       if (item < A_ITEMS) {
-        if (AMODE == A_TRANSPOSED) {
+        if (AMODE == A_TRANSPOSED || AMODE == A_IM2COL_T) {
 #pragma unroll
           for (int e = 0; e < 4; e++) as[(L.a_row[i] + e) * LDA_S + L.a_kq[i]] = reg[i][e];
         } else {
@@ -1031,7 +1086,7 @@ static int resident_blocks(tfhip_ctx* ctx) {
 
 template <class T, int AMODE, int BMODE, bool KBLOCKED, bool FAST>
 static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
-  static const char* const a_names[] = {"rowmajor", "transposed", "im2col"};
+  static const char* const a_names[] = {"rowmajor", "transposed", "im2col", "im2col_up", "im2col_t"};
   static const char* const b_names[] = {"f32", "f32t", "u8"};
   snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "gemm_%dx%d_%s_%s%s%s", T::BM, T::BN,
            a_names[AMODE], b_names[BMODE], KBLOCKED ? "_kb48" : "",
@@ -1114,6 +1169,8 @@ static int launch_gemm(tfhip_ctx* ctx, GemmArgs& p, int batch, int amode, int bm
   long long a_el, b_el;
   if (amode == A_ROWMAJOR) a_el = (long long)(p.M - 1) * p.lda + p.K;
   else if (amode == A_TRANSPOSED) a_el = (long long)(p.K - 1) * p.lda + p.M;
+  else if (amode == A_IM2COL_T)
+    a_el = p.OH * p.OW > 0 ? (long long)(p.K / (p.OH * p.OW)) * p.H * p.W * p.Cin : 0;
   else a_el = p.OH * p.OW > 0 ? (long long)(p.M / (p.OH * p.OW)) * p.H * p.W * p.Cin : 0;
   if (bmode == B_TRANSPOSED) b_el = (long long)(p.N - 1) * p.ldb + p.K;
   else b_el = (long long)(p.K - 1) * p.ldb + p.N;
@@ -1137,6 +1194,8 @@ static int launch_gemm(tfhip_ctx* ctx, GemmArgs& p, int batch, int amode, int bm
   TFHIP_CASE(A_ROWMAJOR, B_UINT8, false)
   TFHIP_CASE(A_IM2COL, B_ROWMAJOR, false)
   TFHIP_CASE(A_IM2COL, B_UINT8, false)
+  TFHIP_CASE(A_IM2COL_UP, B_ROWMAJOR, false)
+  TFHIP_CASE(A_IM2COL_T, B_ROWMAJOR, false)
 #undef TFHIP_CASE
   return ctx->fail(TFHIP_ENOTSUP, "matmul: operand layout combination not built "
                                   "(transposed A with quantised B)");
@@ -1358,4 +1417,140 @@ extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t o
     }
   }
   return launch_gemm(ctx, p, 1, amode, quant ? B_UINT8 : B_ROWMAJOR, /*kblocked=*/false);
+}
+
+namespace tfhip {
+// out[(kh, kw, co)][ci] = w[KH - 1 - kh][KW - 1 - kw][ci][co]: the filter as conv2dDerInput
+// reads it (backend_cpu.ts:1741-1742), laid out as the row-major B operand of the product.
+__global__ void flip_filter_kernel(const float* w, float* out, int KH, int KW, int Cin, int Cout) {
+  const int total = KH * KW * Cin * Cout;
+  for (int g = blockIdx.x * blockDim.x + threadIdx.x; g < total; g += gridDim.x * blockDim.x) {
+    const int ci = g % Cin;
+    int t = g / Cin;
+    const int co = t % Cout;
+    t /= Cout;
+    const int kw = t % KW, kh = t / KW;
+    out[g] = w[(((KH - 1 - kh) * KW + (KW - 1 - kw)) * Cin + ci) * Cout + co];
+  }
+}
+
+static int check_backward_geometry(tfhip_ctx* ctx, const char* op, const tfhip_conv2d_info* ci) {
+  if (ci->batch < 0 || ci->in_h < 0 || ci->in_w < 0 || ci->in_c < 0 || ci->out_h < 0 ||
+      ci->out_w < 0 || ci->out_c < 0 || ci->filter_h <= 0 || ci->filter_w <= 0 ||
+      ci->stride_h <= 0 || ci->stride_w <= 0)
+    return ctx->fail(TFHIP_EINVAL, "%s: bad geometry", op);
+  // the reference's gradient of conv2D rejects dilation rates above 1 (ops/conv.ts:240-243)
+  if (ci->dilation_h != 1 || ci->dilation_w != 1)
+    return ctx->fail(TFHIP_EINVAL, "%s: dilation rates greater than 1 are not yet supported", op);
+  if ((int64_t)(ci->out_h - 1) * ci->stride_h - ci->pad_top >= ci->in_h ||
+      (int64_t)(ci->out_w - 1) * ci->stride_w - ci->pad_left >= ci->in_w)
+    return ctx->fail(TFHIP_EINVAL, "%s: output extent does not fit the input", op);
+  return TFHIP_OK;
+}
+}  // namespace tfhip
+
+extern "C" int tfhip_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int64_t filter, int64_t dx,
+                                      const tfhip_conv2d_info* ci) {
+  if (!ctx || !ci) return TFHIP_EINVAL;
+  int rc;
+  if ((rc = check_backward_geometry(ctx, "conv2dDerInput", ci))) return rc;
+  TFHIP_GET(ctx, bdy, dy);
+  TFHIP_GET(ctx, bw, filter);
+  TFHIP_GET(ctx, bdx, dx);
+  const int64_t x_n = (int64_t)ci->batch * ci->in_h * ci->in_w * ci->in_c;
+  const int64_t w_n = (int64_t)ci->filter_h * ci->filter_w * ci->in_c * ci->out_c;
+  const int64_t y_n = (int64_t)ci->batch * ci->out_h * ci->out_w * ci->out_c;
+  if (bdy->numel != y_n || bw->numel != w_n || bdx->numel != x_n)
+    return ctx->fail(TFHIP_EINVAL, "conv2dDerInput: buffer sizes do not match the geometry");
+  if (bdx->dtype != TFHIP_FLOAT32 || bw->dtype == TFHIP_UINT8Q)
+    return ctx->fail(TFHIP_EINVAL, "conv2dDerInput: dx must be float32 and the filter not quantised");
+  if (x_n == 0) return TFHIP_OK;
+  if ((int64_t)ci->batch * ci->in_h * ci->in_w > 0x7fffffffLL || w_n > 0x7fffffffLL)
+    return ctx->fail(TFHIP_ENOTSUP, "conv2dDerInput: more than 2^31 input pixels");
+  if (y_n == 0 || ci->out_c == 0) {  // nothing flows back
+    if (hipMemsetAsync(bdx->ptr, 0, (size_t)x_n * sizeof(float), ctx->stream) != hipSuccess)
+      return ctx->fail(TFHIP_EDEVICE, "conv2dDerInput: memset failed");
+    return TFHIP_OK;
+  }
+  Temp tdy(ctx), tw(ctx), tflip(ctx);
+  GemmArgs p = {};
+  const float* wf;
+  if ((rc = as_f32(ctx, bdy, &tdy, &p.A))) return rc;
+  if ((rc = as_f32(ctx, bw, &tw, &wf))) return rc;
+  if (!tflip.get((size_t)w_n * sizeof(float))) return TFHIP_EDEVICE;
+  {
+    const int64_t blocks = ceil_div(w_n, 256);
+    hipLaunchKernelGGL(flip_filter_kernel, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256),
+                       0, ctx->stream, wf, static_cast<float*>(tflip.ptr), ci->filter_h,
+                       ci->filter_w, ci->in_c, ci->out_c);
+    TFHIP_LAUNCH_CHECK(ctx);
+  }
+  p.B = tflip.ptr;
+  p.C = static_cast<float*>(bdx->ptr);
+  p.bias_kind = p.prelu_kind = TFHIP_BCAST_NONE;
+  p.act = TFHIP_ACT_LINEAR;
+  p.M = ci->batch * ci->in_h * ci->in_w;   // rows: input pixels
+  p.N = ci->in_c;
+  p.K = ci->filter_h * ci->filter_w * ci->out_c;
+  p.ldb = ci->in_c;
+  p.b_vec = aligned16(p.B) && (p.ldb % 4 == 0);
+  // the image gathered from is dy: "input" geometry of the loader = dy, rows = dx pixels
+  p.H = ci->out_h; p.W = ci->out_w; p.Cin = ci->out_c;
+  p.OH = ci->in_h; p.OW = ci->in_w;
+  p.KH = ci->filter_h; p.KW = ci->filter_w;
+  p.sh = p.sw = 1;
+  p.dh = p.dw = 1;
+  p.pt = ci->filter_h - 1 - ci->pad_top;   // may be negative (padding larger than the filter)
+  p.pl = ci->filter_w - 1 - ci->pad_left;
+  p.up_h = ci->stride_h; p.up_w = ci->stride_w;
+  p.a_vec = aligned16(p.A) && (ci->out_c % 4 == 0);
+  return launch_gemm(ctx, p, 1, A_IM2COL_UP, B_ROWMAJOR, /*kblocked=*/false);
+}
+
+extern "C" int tfhip_conv2d_der_filter(tfhip_ctx* ctx, int64_t x, int64_t dy, int64_t dw,
+                                       const tfhip_conv2d_info* ci) {
+  if (!ctx || !ci) return TFHIP_EINVAL;
+  int rc;
+  if ((rc = check_backward_geometry(ctx, "conv2dDerFilter", ci))) return rc;
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bdy, dy);
+  TFHIP_GET(ctx, bdw, dw);
+  const int64_t x_n = (int64_t)ci->batch * ci->in_h * ci->in_w * ci->in_c;
+  const int64_t w_n = (int64_t)ci->filter_h * ci->filter_w * ci->in_c * ci->out_c;
+  const int64_t y_n = (int64_t)ci->batch * ci->out_h * ci->out_w * ci->out_c;
+  if (bx->numel != x_n || bdy->numel != y_n || bdw->numel != w_n)
+    return ctx->fail(TFHIP_EINVAL, "conv2dDerFilter: buffer sizes do not match the geometry");
+  if (bdw->dtype != TFHIP_FLOAT32)
+    return ctx->fail(TFHIP_EINVAL, "conv2dDerFilter: dW must be float32");
+  if (w_n == 0) return TFHIP_OK;
+  if ((int64_t)ci->batch * ci->out_h * ci->out_w > 0x7fffffffLL || w_n > 0x7fffffffLL ||
+      x_n > (1LL << 40))
+    return ctx->fail(TFHIP_ENOTSUP, "conv2dDerFilter: more than 2^31 output pixels");
+  if (x_n == 0 || y_n == 0) {
+    if (hipMemsetAsync(bdw->ptr, 0, (size_t)w_n * sizeof(float), ctx->stream) != hipSuccess)
+      return ctx->fail(TFHIP_EDEVICE, "conv2dDerFilter: memset failed");
+    return TFHIP_OK;
+  }
+  Temp tx(ctx), tdy(ctx);
+  GemmArgs p = {};
+  const float* dyf;
+  if ((rc = as_f32(ctx, bx, &tx, &p.A))) return rc;
+  if ((rc = as_f32(ctx, bdy, &tdy, &dyf))) return rc;
+  p.B = dyf;
+  p.C = static_cast<float*>(bdw->ptr);
+  p.bias_kind = p.prelu_kind = TFHIP_BCAST_NONE;
+  p.act = TFHIP_ACT_LINEAR;
+  p.M = ci->filter_h * ci->filter_w * ci->in_c;   // rows: (filter row, filter column, channel)
+  p.N = ci->out_c;
+  p.K = ci->batch * ci->out_h * ci->out_w;        // contraction over the output pixels
+  p.ldb = ci->out_c;
+  p.b_vec = aligned16(p.B) && (p.ldb % 4 == 0);
+  p.H = ci->in_h; p.W = ci->in_w; p.Cin = ci->in_c;
+  p.OH = ci->out_h; p.OW = ci->out_w;
+  p.KH = ci->filter_h; p.KW = ci->filter_w;
+  p.sh = ci->stride_h; p.sw = ci->stride_w;
+  p.dh = p.dw = 1;
+  p.pt = ci->pad_top; p.pl = ci->pad_left;
+  p.a_vec = aligned16(p.A) && (ci->in_c % 4 == 0);
+  return launch_gemm(ctx, p, 1, A_IM2COL_T, B_ROWMAJOR, /*kblocked=*/false);
 }

@@ -310,6 +310,34 @@ static napi_value js_pool2d(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+/* Backward kernels: name(ctx, a, b, out, info) with info = the forward op's Conv2DInfo.
+ * conv2dDerInput(ctx, dy, filter, dx, info), conv2dDerFilter(ctx, x, dy, dW, info) and their
+ * depthwise twins. */
+#define BACKWARD_BINDING(js_fn, c_fn)                                   \
+  static napi_value js_fn(napi_env env, napi_callback_info info) {      \
+    ARGS(5);                                                            \
+    I64(1, a); I64(2, b); I64(3, out);                                  \
+    tfhip_conv2d_info ci;                                               \
+    if (!arg_conv_info(env, argv[4], &ci)) return NULL;                 \
+    CHECK(c_fn(ctx, a, b, out, &ci));                                   \
+    return undefined(env);                                              \
+  }
+BACKWARD_BINDING(js_conv2d_der_input, tfhip_conv2d_der_input)
+BACKWARD_BINDING(js_conv2d_der_filter, tfhip_conv2d_der_filter)
+BACKWARD_BINDING(js_depthwise_der_input, tfhip_depthwise_conv2d_der_input)
+BACKWARD_BINDING(js_depthwise_der_filter, tfhip_depthwise_conv2d_der_filter)
+
+/* pool2dBackprop(ctx, dy, x, dx, info, kind) */
+static napi_value js_pool2d_backprop(napi_env env, napi_callback_info info) {
+  ARGS(6);
+  I64(1, dy); I64(2, x); I64(3, dx);
+  tfhip_conv2d_info ci;
+  if (!arg_conv_info(env, argv[4], &ci)) return NULL;
+  INT(5, kind);
+  CHECK(tfhip_pool2d_backprop(ctx, dy, x, dx, &ci, kind));
+  return undefined(env);
+}
+
 /* binary(ctx, op, a, aShape, b, bShape, out) */
 static napi_value js_binary(napi_env env, napi_callback_info info) {
   ARGS(7);
@@ -495,7 +523,11 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"softmaxRows", js_softmax_rows}, {"gather", js_gather}, {"transpose", js_transpose},
       {"stridedCopy", js_strided_copy}, {"logicalNot", js_logical_not},
       {"batchnorm", js_batchnorm}, {"resizeBilinear", js_resize_bilinear},
-      {"oneHot", js_one_hot}};
+      {"oneHot", js_one_hot}, {"conv2dDerInput", js_conv2d_der_input},
+      {"conv2dDerFilter", js_conv2d_der_filter},
+      {"depthwiseConv2dDerInput", js_depthwise_der_input},
+      {"depthwiseConv2dDerFilter", js_depthwise_der_filter},
+      {"pool2dBackprop", js_pool2d_backprop}};
   for (size_t i = 0; i < sizeof fns / sizeof fns[0]; i++) {
     napi_value f;
     if (napi_create_function(env, fns[i].name, NAPI_AUTO_LENGTH, fns[i].fn, NULL, &f) != napi_ok ||

@@ -263,6 +263,34 @@ class MathBackendHIP extends KernelBackend {
     this.napi.pool2d(this.ctx, this.h(x), this.h(out), convInfoArray(convInfo), POOL[kind]);
     return out;
   }
+  // ---- backward kernels (backend.ts:423-441, 456-465); convInfo is the forward op's ----
+  backward(fn, a, b, outShape, convInfo, extra) {
+    const out = this.out(outShape);
+    const args = [this.ctx, this.h(a), this.h(b), this.h(out), convInfoArray(convInfo)];
+    if (extra !== undefined) args.push(extra);
+    this.napi[fn].apply(this.napi, args);
+    return out;
+  }
+  conv2dDerInput(dy, filter, convInfo) {
+    return this.backward('conv2dDerInput', dy, filter, convInfo.inShape, convInfo);
+  }
+  conv2dDerFilter(x, dy, convInfo) {
+    return this.backward('conv2dDerFilter', x, dy, convInfo.filterShape, convInfo);
+  }
+  depthwiseConv2DDerInput(dy, filter, convInfo) {
+    return this.backward('depthwiseConv2dDerInput', dy, filter, convInfo.inShape, convInfo);
+  }
+  depthwiseConv2DDerFilter(x, dy, convInfo) {
+    return this.backward('depthwiseConv2dDerFilter', x, dy, convInfo.filterShape, convInfo);
+  }
+  // y (the forward result) is part of the plug-in signature; the kernel finds the winners of
+  // each window from x, as backend_cpu does
+  maxPoolBackprop(dy, x, y, convInfo) {
+    return this.backward('pool2dBackprop', dy, x, x.shape, convInfo, POOL.max);
+  }
+  avgPoolBackprop(dy, x, convInfo) {
+    return this.backward('pool2dBackprop', dy, x, x.shape, convInfo, POOL.avg);
+  }
   avgPool(x, convInfo) { return this.pool(x, convInfo, 'avg'); }
   maxPool(x, convInfo) {
     const r = this.pool(x, convInfo, 'max');

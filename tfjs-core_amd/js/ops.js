@@ -311,6 +311,129 @@ const pool = op('pool', (input, windowShape, poolingType, pad, dilations, stride
     poolImpl(input, windowShape, strides == null ? 1 : strides, dilations == null ? 1 : dilations,
              pad, null, poolingType));
 
+// ---- backward ops (ops/conv.ts:242-468, 678-716; ops/pool.ts:333-445) ----------------------
+function as4D(t) {
+  return t.rank === 3 ? reshape(t, [1, t.shape[0], t.shape[1], t.shape[2]]) : t;
+}
+function sameShape(a, b) {
+  return a.length === b.length && a.every((v, i) => v === b[i]);
+}
+const conv2dDerInput = op('conv2dDerInput', (xShape, dy, filter, strides, pad, dataFormat, dimRoundingMode) => {
+  const $dy = convertToTensor(dy, 'dy', 'conv2dDerInput');
+  const $filter = convertToTensor(filter, 'filter', 'conv2dDerInput');
+  util.assert(xShape.length === $dy.rank,
+              () => `Length of inShape (${xShape.length}) and rank of dy (${$dy.rank}) must match`);
+  const reshapedTo4D = $dy.rank === 3;
+  const dy4D = as4D($dy);
+  const xShape4D = reshapedTo4D ? [1, xShape[0], xShape[1], xShape[2]] : xShape.slice();
+  util.assert(xShape4D.length === 4,
+              () => `Error in conv2dDerInput: inShape must be length 4, but got length ${xShape4D.length}.`);
+  util.assert(dy4D.rank === 4, () => `Error in conv2dDerInput: dy must be rank 4, but got rank ${dy4D.rank}`);
+  util.assert($filter.rank === 4,
+              () => `Error in conv2dDerInput: filter must be rank 4, but got rank ${$filter.rank}`);
+  if (dataFormat == null) dataFormat = 'NHWC';
+  util.assert(dataFormat === 'NHWC',
+              () => `Error in conv2dDerInput: got dataFormat of ${dataFormat} but only NHWC is currently supported.`);
+  util.assert(xShape4D[3] === $filter.shape[2],
+              () => `Error in conv2dDerInput: depth of input (${xShape4D[3]}) must ` +
+                  `match input depth for filter ${$filter.shape[2]}.`);
+  util.assert(dy4D.shape[3] === $filter.shape[3],
+              () => `Error in conv2dDerInput: depth of output (${dy4D.shape[3]}) must ` +
+                  `match output depth for filter ${$filter.shape[3]}.`);
+  if (dimRoundingMode != null) {
+    util.assert(util.isInt(pad), () => `Error in conv2dDerInput: pad must be an integer when using, ` +
+        `dimRoundingMode ${dimRoundingMode} but got pad ${pad}.`);
+  }
+  const convInfo = conv_util.computeConv2DInfo(xShape4D, $filter.shape, strides, 1, pad, dimRoundingMode, false);
+  util.assert(sameShape(convInfo.outShape, dy4D.shape),
+              () => `Error in conv2dDerInput: dy has shape ${dy4D.shape}, the convolution of an ` +
+                  `input of shape ${xShape4D} gives ${convInfo.outShape}`);
+  const res = ENGINE.runKernel(backend => backend.conv2dDerInput(dy4D, $filter, convInfo), {dy4D, $filter});
+  return lower(res, reshapedTo4D);
+});
+const conv2dDerFilter = op('conv2dDerFilter', (x, dy, filterShape, strides, pad, dataFormat, dimRoundingMode) => {
+  const x4D = as4D(convertToTensor(x, 'x', 'conv2dDerFilter'));
+  const dy4D = as4D(convertToTensor(dy, 'dy', 'conv2dDerFilter'));
+  util.assert(x4D.rank === 4, () => `Error in conv2dDerFilter: input must be rank 4, but got shape ${x4D.shape}.`);
+  util.assert(dy4D.rank === 4, () => `Error in conv2dDerFilter: dy must be rank 4, but got shape ${dy4D.shape}.`);
+  util.assert(filterShape.length === 4,
+              () => `Error in conv2dDerFilter: filterShape must be length 4, but got ${filterShape}.`);
+  if (dataFormat == null) dataFormat = 'NHWC';
+  util.assert(dataFormat === 'NHWC',
+              () => `Error in conv2dDerFilter: got dataFormat of ${dataFormat} but only NHWC is currently supported.`);
+  util.assert(x4D.shape[3] === filterShape[2],
+              () => `Error in conv2dDerFilter: depth of input ${x4D.shape[3]}) must ` +
+                  `match input depth in filter (${filterShape[2]}.`);
+  util.assert(dy4D.shape[3] === filterShape[3],
+              () => `Error in conv2dDerFilter: depth of dy (${dy4D.shape[3]}) must ` +
+                  `match output depth for filter (${filterShape[3]}).`);
+  if (dimRoundingMode != null) {
+    util.assert(util.isInt(pad), () => `Error in conv2dDerFilter: pad must be an integer when using, ` +
+        `dimRoundingMode ${dimRoundingMode} but got pad ${pad}.`);
+  }
+  const convInfo = conv_util.computeConv2DInfo(x4D.shape, filterShape, strides, 1, pad, dimRoundingMode, false);
+  util.assert(sameShape(convInfo.outShape, dy4D.shape),
+              () => `Error in conv2dDerFilter: dy has shape ${dy4D.shape}, the convolution gives ${convInfo.outShape}`);
+  return ENGINE.runKernel(backend => backend.conv2dDerFilter(x4D, dy4D, convInfo), {x4D, dy4D});
+});
+// ops/conv.ts:413-424: the transposed convolution is conv2dDerInput on the output shape.
+const conv2dTranspose = op('conv2dTranspose', (x, filter, outputShape, strides, pad, dimRoundingMode) =>
+    conv2dDerInput(outputShape, convertToTensor(x, 'x', 'conv2dTranspose'),
+                   convertToTensor(filter, 'filter', 'conv2dTranspose'), strides, pad, 'NHWC', dimRoundingMode));
+const depthwiseConv2dDerInput = op('depthwiseConv2dDerInput', (xShape, dy, filter, strides, pad, dilations, dimRoundingMode) => {
+  const $dy = convertToTensor(dy, 'dy', 'depthwiseConv2dDerInput');
+  const $filter = convertToTensor(filter, 'filter', 'depthwiseConv2dDerInput');
+  const reshapedTo4D = $dy.rank === 3;
+  const dy4D = as4D($dy);
+  const xShape4D = xShape.length === 3 ? [1, xShape[0], xShape[1], xShape[2]] : xShape.slice();
+  const convInfo = conv_util.computeConv2DInfo(xShape4D, $filter.shape, strides, dilations == null ? 1 : dilations,
+                                               pad, dimRoundingMode, true);
+  util.assert(sameShape(convInfo.outShape, dy4D.shape),
+              () => `Error in depthwiseConv2dDerInput: dy has shape ${dy4D.shape}, the convolution gives ${convInfo.outShape}`);
+  const res = ENGINE.runKernel(backend => backend.depthwiseConv2DDerInput(dy4D, $filter, convInfo), {dy4D});
+  return lower(res, reshapedTo4D);
+});
+const depthwiseConv2dDerFilter = op('depthwiseConv2dDerFilter', (x, dy, filterShape, strides, pad, dilations, dimRoundingMode) => {
+  const x4D = as4D(convertToTensor(x, 'x', 'depthwiseConv2dDerFilter'));
+  const dy4D = as4D(convertToTensor(dy, 'dy', 'depthwiseConv2dDerFilter'));
+  const convInfo = conv_util.computeConv2DInfo(x4D.shape, filterShape, strides, dilations == null ? 1 : dilations,
+                                               pad, dimRoundingMode, true);
+  util.assert(sameShape(convInfo.outShape, dy4D.shape),
+              () => `Error in depthwiseConv2dDerFilter: dy has shape ${dy4D.shape}, the convolution gives ${convInfo.outShape}`);
+  return ENGINE.runKernel(backend => backend.depthwiseConv2DDerFilter(x4D, dy4D, convInfo), {x4D, dy4D});
+});
+function poolBackprop(name, dy, input, filterSize, strides, dilations, pad, dimRoundingMode, kind) {
+  const $dy = convertToTensor(dy, 'dy', name);
+  const $input = convertToTensor(input, 'input', name);
+  util.assert($input.rank === $dy.rank,
+              () => `Rank of input (${$input.rank}) does not match rank of dy (${$dy.rank})`);
+  if (dilations == null) dilations = [1, 1];
+  util.assert(conv_util.eitherStridesOrDilationsAreOne(strides, dilations),
+              () => `Error in ${name}: Either strides or dilations must be 1. ` +
+                  `Got strides ${strides} and dilations '${dilations}'`);
+  const reshapedTo4D = $input.rank === 3;
+  const input4D = as4D($input), dy4D = as4D($dy);
+  util.assert(dy4D.rank === 4, () => `Error in ${name}: dy must be rank 4 but got rank ${dy4D.rank}.`);
+  util.assert(input4D.rank === 4, () => `Error in ${name}: input must be rank 4 but got rank ${input4D.rank}.`);
+  if (dimRoundingMode != null) {
+    util.assert(util.isInt(pad), () => `Error in ${name}: pad must be an integer when using, ` +
+        `dimRoundingMode ${dimRoundingMode} but got pad ${pad}.`);
+  }
+  const convInfo = conv_util.computePool2DInfo(input4D.shape, filterSize, strides, dilations, pad, dimRoundingMode);
+  util.assert(sameShape(convInfo.outShape, dy4D.shape),
+              () => `Error in ${name}: dy has shape ${dy4D.shape}, the pooling gives ${convInfo.outShape}`);
+  const res = ENGINE.runKernel(
+      backend => kind === 'max' ? backend.maxPoolBackprop(dy4D, input4D, null, convInfo)
+                                : backend.avgPoolBackprop(dy4D, input4D, convInfo),
+      {dy4D, input4D});
+  return lower(res, reshapedTo4D);
+}
+// ops/pool.ts:333-383 (the forward result of the reference signature is not needed) / :397-445
+const maxPoolBackprop = op('maxPoolBackprop', (dy, input, filterSize, strides, pad, dilations, dimRoundingMode) =>
+    poolBackprop('maxPoolBackprop', dy, input, filterSize, strides, dilations, pad, dimRoundingMode, 'max'));
+const avgPoolBackprop = op('avgPoolBackprop', (dy, input, filterSize, strides, pad, dilations) =>
+    poolBackprop('avgPoolBackprop', dy, input, filterSize, strides, dilations, pad, null, 'avg'));
+
 // ---- elementwise ------------------------------------------------------------------------
 function binaryOp(name, method) {
   return op(name, (a, b) => {
@@ -693,5 +816,7 @@ module.exports = {
   minimum, prelu, relu, relu6, exp, log, neg, abs, sigmoid, sqrt, square, tanh, rsqrt,
   clipByValue, sum, max, min, argMax, argMin, logSumExp, softmax, gather, transpose,
   slice, stridedSlice, reverse, concat, pad, tile, oneHot, equal, notEqual, less, lessEqual,
-  greater, greaterEqual, logicalAnd, logicalOr, logicalNot, batchNorm, resizeBilinear
+  greater, greaterEqual, logicalAnd, logicalOr, logicalNot, batchNorm, resizeBilinear,
+  conv2dDerInput, conv2dDerFilter, conv2dTranspose, depthwiseConv2dDerInput,
+  depthwiseConv2dDerFilter, maxPoolBackprop, avgPoolBackprop
 };

@@ -67,6 +67,13 @@ const OPS = {
   logicalNot: i => tf.logicalNot(i.x),
   batchNorm: (i, a) => tf.batchNorm(i.x, i.mean, i.variance, i.offset, i.scale, a.varianceEpsilon),
   resizeBilinear: (i, a) => tf.resizeBilinear(i.x, a.size, a.alignCorners),
+  conv2dDerInput: (i, a) => tf.conv2dDerInput(a.xShape, i.dy, i.filter, a.strides, a.pad),
+  conv2dDerFilter: (i, a) => tf.conv2dDerFilter(i.x, i.dy, a.filterShape, a.strides, a.pad),
+  conv2dTranspose: (i, a) => tf.conv2dTranspose(i.x, i.filter, a.outputShape, a.strides, a.pad),
+  depthwiseConv2dDerInput: (i, a) => tf.depthwiseConv2dDerInput(a.xShape, i.dy, i.filter, a.strides, a.pad),
+  depthwiseConv2dDerFilter: (i, a) => tf.depthwiseConv2dDerFilter(i.x, i.dy, a.filterShape, a.strides, a.pad),
+  maxPoolBackprop: (i, a) => tf.maxPoolBackprop(i.dy, i.x, a.filterSize, a.strides, a.pad, a.dilations),
+  avgPoolBackprop: (i, a) => tf.avgPoolBackprop(i.dy, i.x, a.filterSize, a.strides, a.pad, a.dilations),
 };
 
 async function main() {

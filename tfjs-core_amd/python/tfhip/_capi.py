@@ -52,6 +52,11 @@ _SIGNATURES = {
     "tfhip_depthwise_conv2d": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC), _I64, _INT, _INT,
                                C.POINTER(QParams)],
     "tfhip_pool2d": [_PTR, _I64, _I64, C.POINTER(Conv2DInfoC), _INT],
+    "tfhip_conv2d_der_input": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC)],
+    "tfhip_conv2d_der_filter": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC)],
+    "tfhip_depthwise_conv2d_der_input": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC)],
+    "tfhip_depthwise_conv2d_der_filter": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC)],
+    "tfhip_pool2d_backprop": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC), _INT],
     "tfhip_binary": [_PTR, _INT, _I64, C.POINTER(C.c_int32), _INT, _I64, C.POINTER(C.c_int32),
                      _INT, _I64],
     "tfhip_unary": [_PTR, _INT, _I64, _I64, C.c_float, C.c_float],

@@ -265,6 +265,39 @@ class MathBackendHIP(object):
         r = self._pool(x, conv_info, "max")
         return r if x.dtype == "float32" else self.cast(r, x.dtype)
 
+    # ---- backward kernels (backend.ts:423-441, 456-465); conv_info is the forward op's ----
+    def _backward(self, fn, a, b, out_shape, conv_info, *extra):
+        out = self._out(out_shape)
+        info = _info_c(conv_info)
+        self._ck(fn(self.ctx, self._h(a), self._h(b), self._h(out), C.byref(info), *extra))
+        return out
+
+    def conv2d_der_input(self, dy, filter, conv_info):
+        return self._backward(self.lib.tfhip_conv2d_der_input, dy, filter, conv_info["inShape"],
+                              conv_info)
+
+    def conv2d_der_filter(self, x, dy, conv_info):
+        return self._backward(self.lib.tfhip_conv2d_der_filter, x, dy, conv_info["filterShape"],
+                              conv_info)
+
+    def depthwise_conv2d_der_input(self, dy, filter, conv_info):
+        return self._backward(self.lib.tfhip_depthwise_conv2d_der_input, dy, filter,
+                              conv_info["inShape"], conv_info)
+
+    def depthwise_conv2d_der_filter(self, x, dy, conv_info):
+        return self._backward(self.lib.tfhip_depthwise_conv2d_der_filter, x, dy,
+                              conv_info["filterShape"], conv_info)
+
+    def max_pool_backprop(self, dy, x, y, conv_info):
+        # y (the forward result) is part of the plug-in signature; the kernel finds the winners
+        # from x, as backend_cpu does
+        return self._backward(self.lib.tfhip_pool2d_backprop, dy, x, x.shape, conv_info,
+                              capi.POOL["max"])
+
+    def avg_pool_backprop(self, dy, x, conv_info):
+        return self._backward(self.lib.tfhip_pool2d_backprop, dy, x, x.shape, conv_info,
+                              capi.POOL["avg"])
+
     # ---- elementwise ----
     def _binary(self, op, a, b, out_dtype):
         out_shape = su.broadcast_shape(a.shape, b.shape)

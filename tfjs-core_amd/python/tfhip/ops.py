@@ -691,3 +691,160 @@ def resize_bilinear(images, size, align_corners=False):
         r = ENGINE.run_kernel(lambda be: be.resize_bilinear(x4, new_h, new_w, align_corners))
         return r if images.rank == 4 else reshape(r, r.shape[1:])
     return ENGINE.tidy(run)
+
+
+# ---- backward ops (ops/conv.ts:242-468, 678-716; ops/pool.ts:333-445) ----
+def _as4d(t):
+    return reshape(t, (1,) + tuple(t.shape)) if t.rank == 3 else t
+
+
+def conv2d_der_input(x_shape, dy, filt, strides, pad, data_format="NHWC", dim_rounding_mode=None):
+    def run():
+        dyt, f = _conv(dy, "dy", "conv2dDerInput"), _conv(filt, "filter", "conv2dDerInput")
+        xs = tuple(int(v) for v in x_shape)
+        if len(xs) != dyt.rank:
+            raise ValueError("Length of inShape (%d) and rank of dy (%d) must match"
+                             % (len(xs), dyt.rank))
+        lifted = dyt.rank == 3
+        dy4 = _as4d(dyt)
+        xs4 = (1,) + xs if lifted else xs
+        if len(xs4) != 4:
+            raise ValueError("Error in conv2dDerInput: inShape must be length 4, but got length "
+                             "%d." % len(xs4))
+        if dy4.rank != 4:
+            raise ValueError("Error in conv2dDerInput: dy must be rank 4, but got rank %d" % dy4.rank)
+        if f.rank != 4:
+            raise ValueError("Error in conv2dDerInput: filter must be rank 4, but got rank %d" % f.rank)
+        if data_format != "NHWC":
+            raise ValueError("Error in conv2dDerInput: got dataFormat of %s but only NHWC is "
+                             "currently supported." % data_format)
+        if xs4[3] != f.shape[2]:
+            raise ValueError("Error in conv2dDerInput: depth of input (%d) must match input depth "
+                             "for filter %d." % (xs4[3], f.shape[2]))
+        if dy4.shape[3] != f.shape[3]:
+            raise ValueError("Error in conv2dDerInput: depth of output (%d) must match output depth "
+                             "for filter %d." % (dy4.shape[3], f.shape[3]))
+        if dim_rounding_mode is not None and not (isinstance(pad, (int, float)) and
+                                                  float(pad) == int(pad)):
+            raise ValueError("Error in conv2dDerInput: pad must be an integer when using, "
+                             "dimRoundingMode %s but got pad %s." % (dim_rounding_mode, pad))
+        ci = su.compute_conv2d_info(xs4, f.shape, strides, 1, pad, dim_rounding_mode, False)
+        if tuple(ci["outShape"]) != tuple(dy4.shape):
+            raise ValueError("Error in conv2dDerInput: dy has shape %s, the convolution of an input "
+                             "of shape %s gives %s" % (list(dy4.shape), list(xs4),
+                                                       list(ci["outShape"])))
+        return _lower(ENGINE.run_kernel(lambda be: be.conv2d_der_input(dy4, f, ci)), lifted)
+    return ENGINE.tidy(run)
+
+
+def conv2d_der_filter(x, dy, filter_shape, strides, pad, data_format="NHWC", dim_rounding_mode=None):
+    def run():
+        x4 = _as4d(_conv(x, "x", "conv2dDerFilter"))
+        dy4 = _as4d(_conv(dy, "dy", "conv2dDerFilter"))
+        fs = tuple(int(v) for v in filter_shape)
+        if x4.rank != 4:
+            raise ValueError("Error in conv2dDerFilter: input must be rank 4, but got shape %s."
+                             % list(x4.shape))
+        if dy4.rank != 4:
+            raise ValueError("Error in conv2dDerFilter: dy must be rank 4, but got shape %s."
+                             % list(dy4.shape))
+        if len(fs) != 4:
+            raise ValueError("Error in conv2dDerFilter: filterShape must be length 4, but got %s."
+                             % list(fs))
+        if data_format != "NHWC":
+            raise ValueError("Error in conv2dDerFilter: got dataFormat of %s but only NHWC is "
+                             "currently supported." % data_format)
+        if x4.shape[3] != fs[2]:
+            raise ValueError("Error in conv2dDerFilter: depth of input %d) must match input depth "
+                             "in filter (%d." % (x4.shape[3], fs[2]))
+        if dy4.shape[3] != fs[3]:
+            raise ValueError("Error in conv2dDerFilter: depth of dy (%d) must match output depth "
+                             "for filter (%d)." % (dy4.shape[3], fs[3]))
+        if dim_rounding_mode is not None and not (isinstance(pad, (int, float)) and
+                                                  float(pad) == int(pad)):
+            raise ValueError("Error in conv2dDerFilter: pad must be an integer when using, "
+                             "dimRoundingMode %s but got pad %s." % (dim_rounding_mode, pad))
+        ci = su.compute_conv2d_info(x4.shape, fs, strides, 1, pad, dim_rounding_mode, False)
+        if tuple(ci["outShape"]) != tuple(dy4.shape):
+            raise ValueError("Error in conv2dDerFilter: dy has shape %s, the convolution gives %s"
+                             % (list(dy4.shape), list(ci["outShape"])))
+        return ENGINE.run_kernel(lambda be: be.conv2d_der_filter(x4, dy4, ci))
+    return ENGINE.tidy(run)
+
+
+def conv2d_transpose(x, filt, output_shape, strides, pad, dim_rounding_mode=None):
+    """ops/conv.ts:413-424: the transposed convolution is conv2dDerInput on the output shape."""
+    return conv2d_der_input(output_shape, _conv(x, "x", "conv2dTranspose"),
+                            _conv(filt, "filter", "conv2dTranspose"), strides, pad, "NHWC",
+                            dim_rounding_mode)
+
+
+def depthwise_conv2d_der_input(x_shape, dy, filt, strides, pad, dilations=(1, 1),
+                               dim_rounding_mode=None):
+    """ops/conv.ts:678-694; the Conv2DInfo is the forward op's (:530-540)."""
+    def run():
+        dyt, f = _conv(dy, "dy", "depthwiseConv2dDerInput"), _conv(filt, "filter", "depthwiseConv2dDerInput")
+        lifted = dyt.rank == 3
+        dy4 = _as4d(dyt)
+        xs = tuple(int(v) for v in x_shape)
+        xs4 = (1,) + xs if len(xs) == 3 else xs
+        ci = su.compute_conv2d_info(xs4, f.shape, strides, dilations, pad, dim_rounding_mode, True)
+        if tuple(ci["outShape"]) != tuple(dy4.shape):
+            raise ValueError("Error in depthwiseConv2dDerInput: dy has shape %s, the convolution "
+                             "gives %s" % (list(dy4.shape), list(ci["outShape"])))
+        return _lower(ENGINE.run_kernel(lambda be: be.depthwise_conv2d_der_input(dy4, f, ci)), lifted)
+    return ENGINE.tidy(run)
+
+
+def depthwise_conv2d_der_filter(x, dy, filter_shape, strides, pad, dilations=(1, 1),
+                                dim_rounding_mode=None):
+    """ops/conv.ts:696-716."""
+    def run():
+        x4 = _as4d(_conv(x, "x", "depthwiseConv2dDerFilter"))
+        dy4 = _as4d(_conv(dy, "dy", "depthwiseConv2dDerFilter"))
+        fs = tuple(int(v) for v in filter_shape)
+        ci = su.compute_conv2d_info(x4.shape, fs, strides, dilations, pad, dim_rounding_mode, True)
+        if tuple(ci["outShape"]) != tuple(dy4.shape):
+            raise ValueError("Error in depthwiseConv2dDerFilter: dy has shape %s, the convolution "
+                             "gives %s" % (list(dy4.shape), list(ci["outShape"])))
+        return ENGINE.run_kernel(lambda be: be.depthwise_conv2d_der_filter(x4, dy4, ci))
+    return ENGINE.tidy(run)
+
+
+def _pool_backprop(name, dy, x, filter_size, strides, dilations, pad, rounding, kind):
+    def run():
+        dyt, xt = _conv(dy, "dy", name), _conv(x, "input", name)
+        if xt.rank != dyt.rank:
+            raise ValueError("Rank of input (%d) does not match rank of dy (%d)" % (xt.rank, dyt.rank))
+        dil = (1, 1) if dilations is None else dilations
+        if not su.either_strides_or_dilations_are_one(strides, dil):
+            raise ValueError("Error in %s: Either strides or dilations must be 1. Got strides %s "
+                             "and dilations '%s'" % (name, strides, dil))
+        lifted = xt.rank == 3
+        x4, dy4 = _as4d(xt), _as4d(dyt)
+        if dy4.rank != 4:
+            raise ValueError("Error in %s: dy must be rank 4 but got rank %d." % (name, dy4.rank))
+        if x4.rank != 4:
+            raise ValueError("Error in %s: input must be rank 4 but got rank %d." % (name, x4.rank))
+        if rounding is not None and not (isinstance(pad, (int, float)) and float(pad) == int(pad)):
+            raise ValueError("Error in %s: pad must be an integer when using, dimRoundingMode %s "
+                             "but got pad %s." % (name, rounding, pad))
+        ci = su.compute_pool2d_info(x4.shape, filter_size, strides, dil, pad, rounding)
+        if tuple(ci["outShape"]) != tuple(dy4.shape):
+            raise ValueError("Error in %s: dy has shape %s, the pooling gives %s"
+                             % (name, list(dy4.shape), list(ci["outShape"])))
+        r = ENGINE.run_kernel(lambda be: be.max_pool_backprop(dy4, x4, None, ci) if kind == "max"
+                              else be.avg_pool_backprop(dy4, x4, ci))
+        return _lower(r, lifted)
+    return ENGINE.tidy(run)
+
+
+def max_pool_backprop(dy, x, filter_size, strides, pad, dilations=None, dim_rounding_mode=None):
+    """ops/pool.ts:333-383 (the forward result `y` of the reference signature is not needed)."""
+    return _pool_backprop("maxPoolBackprop", dy, x, filter_size, strides, dilations, pad,
+                          dim_rounding_mode, "max")
+
+
+def avg_pool_backprop(dy, x, filter_size, strides, pad, dilations=None):
+    """ops/pool.ts:397-445."""
+    return _pool_backprop("avgPoolBackprop", dy, x, filter_size, strides, dilations, pad, None, "avg")
