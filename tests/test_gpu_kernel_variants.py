@@ -207,3 +207,44 @@ def test_pointwise_conv_odd_channels(tf):
     assert np.array_equal(np.isfinite(got), np.isfinite(want))
     ok = np.isfinite(want)
     close(got[ok], want[ok])
+
+
+# ------------------------------------------------------- backward variants ----
+def test_backward_kernel_variants(tf):
+    """Which kernel each backward op takes: the two gather modes of the product kernel (the
+    filter gradient split along its long contraction), the plain product for a pointwise
+    layer, the vectorised depthwise kernels and their general fallbacks."""
+    rng = np.random.default_rng(31)
+    f = lambda *s: rng.uniform(-1, 1, s).astype(np.float32)
+    seen = {}
+
+    def run(name, fn):
+        with tf.tidy():
+            fn().data_sync()
+            seen[name] = last_kernel(tf)
+
+    x, w = tf.tensor(f(4, 28, 28, 32)), tf.tensor(f(3, 3, 32, 64))
+    dy = tf.tensor(f(4, 28, 28, 64))
+    run("der_input", lambda: tf.conv2d_der_input((4, 28, 28, 32), dy, w, 1, "same"))
+    run("der_filter", lambda: tf.conv2d_der_filter(x, dy, (3, 3, 32, 64), 1, "same"))
+    w1 = tf.tensor(f(1, 1, 32, 64))
+    run("der_input_1x1", lambda: tf.conv2d_der_input((4, 28, 28, 32), dy, w1, 1, "same"))
+    x3, w3, dy3 = tf.tensor(f(1, 9, 9, 3)), tf.tensor(f(3, 3, 3, 8)), tf.tensor(f(1, 9, 9, 8))
+    run("der_input_c3", lambda: tf.conv2d_der_input((1, 9, 9, 3), dy3, w3, 1, "same"))
+    run("der_filter_c3", lambda: tf.conv2d_der_filter(x3, dy3, (3, 3, 3, 8), 1, "same"))
+    xd, wd, dyd = tf.tensor(f(2, 16, 16, 8)), tf.tensor(f(3, 3, 8, 1)), tf.tensor(f(2, 16, 16, 8))
+    run("dw_der_input", lambda: tf.depthwise_conv2d_der_input((2, 16, 16, 8), dyd, wd, 1, "same"))
+    run("dw_der_filter", lambda: tf.depthwise_conv2d_der_filter(xd, dyd, (3, 3, 8, 1), 1, "same"))
+    wm, dym = tf.tensor(f(3, 3, 8, 2)), tf.tensor(f(2, 16, 16, 16))
+    run("dw_der_input_mul2", lambda: tf.depthwise_conv2d_der_input((2, 16, 16, 8), dym, wm, 1, "same"))
+    run("dw_der_filter_mul2", lambda: tf.depthwise_conv2d_der_filter(xd, dym, (3, 3, 8, 2), 1, "same"))
+    tf.dispose([x, w, dy, w1, x3, w3, dy3, xd, wd, dyd, wm, dym])
+    assert "im2col_up_f32" in seen["der_input"], seen
+    assert "im2col_t_f32" in seen["der_filter"] and seen["der_filter"].endswith("_splitk"), seen
+    assert "rowmajor_f32" in seen["der_input_1x1"], seen
+    assert seen["der_input_c3"].endswith("im2col_up_f32_unaligned") or "_unaligned" in seen["der_input_c3"], seen
+    assert "im2col_t" in seen["der_filter_c3"] and "_unaligned" in seen["der_filter_c3"], seen
+    assert seen["dw_der_input"] == "depthwise_der_input_vec_s1", seen
+    assert seen["dw_der_filter"] == "depthwise3x3_der_filter", seen
+    assert seen["dw_der_input_mul2"] == "depthwise_der_input", seen
+    assert seen["dw_der_filter_mul2"] == "depthwise_der_filter", seen

@@ -94,6 +94,116 @@ __global__ void depthwise_der_filter_finish_kernel(const double* partial, float*
   dw[g] = (float)s;
 }
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Fast variants for channel multiplier 1, C % 4 == 0 and 16-byte aligned buffers: a lane owns
+// 4 consecutive channels (16-byte accesses) and sums in float in the same tap order.
+// S = 1, 2: the forward stride, known at compile time (no integer division); S = 0: any.
+template <int S>
+__global__ __launch_bounds__(256) void depthwise_der_input_vec_kernel(
+    const float* __restrict__ dy, const float* __restrict__ w, float* __restrict__ dx,
+    const tfhip_conv2d_info ci) {
+  const int c4 = ci.in_c / 4;
+  const int64_t total = (int64_t)ci.batch * ci.in_h * ci.in_w * c4;
+  const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (g >= total) return;
+  const int cq = (int)(g % c4);
+  int64_t t = g / c4;
+  const int xc = (int)(t % ci.in_w);
+  t /= ci.in_w;
+  const int xr = (int)(t % ci.in_h);
+  const int n = (int)(t / ci.in_h);
+  const int sh = S ? S : ci.stride_h, sw = S ? S : ci.stride_w;
+  const int xr_corner = xr - (ci.filter_h - 1 - ci.pad_top);
+  const int xc_corner = xc - (ci.filter_w - 1 - ci.pad_left);
+  const float* dyn = dy + (int64_t)n * ci.out_h * ci.out_w * ci.out_c + cq * 4;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int wr = 0; wr < ci.filter_h; wr++) {
+    const int num_r = xr_corner + wr;
+    const int yr = num_r / sh;
+    if (num_r < 0 || yr * sh != num_r || yr >= ci.out_h) continue;
+    for (int wc = 0; wc < ci.filter_w; wc++) {
+      const int num_c = xc_corner + wc;
+      const int yc = num_c / sw;
+      if (num_c < 0 || yc * sw != num_c || yc >= ci.out_w) continue;
+      const f32x4 d = *reinterpret_cast<const f32x4*>(dyn + ((int64_t)yr * ci.out_w + yc) * ci.out_c);
+      const f32x4 f = *reinterpret_cast<const f32x4*>(
+          w + ((int64_t)(ci.filter_h - 1 - wr) * ci.filter_w + (ci.filter_w - 1 - wc)) * ci.in_c + cq * 4);
+      acc += d * f;
+    }
+  }
+  *reinterpret_cast<f32x4*>(dx + g * 4) = acc;
+}
+
+// dW of a 3x3 depthwise filter (multiplier 1): one pass over the output pixels of a slice;
+// a lane owns a channel quad and keeps the nine taps' sums, so dy is read once and the nine
+// x vectors of a pixel come from neighbouring rows that stay in cache.  The lanes of a
+// workgroup that share a quad (several pixels per wavefront when C / 4 < 64, and the four
+// wavefronts) are then added in a fixed order through LDS.  partial[slice][tap][c] in double.
+__global__ __launch_bounds__(256) void depthwise3x3_der_filter_partial_kernel(
+    const float* __restrict__ x, const float* __restrict__ dy, double* __restrict__ partial,
+    const tfhip_conv2d_info ci, int quads_per_wave, int64_t pixels_per_slice) {
+  extern __shared__ __attribute__((aligned(16))) float red[];  // [256 lanes][9 taps][4]
+  const int tid = threadIdx.x;
+  const int c4 = ci.in_c / 4;
+  const int q_local = tid % quads_per_wave;            // quad within the channel block
+  const int sub = tid / quads_per_wave;                // which of the workgroup's pixel lanes
+  const int subs = 256 / quads_per_wave;
+  const int cq = blockIdx.x * quads_per_wave + q_local;
+  const bool live = cq < c4;
+  const int64_t pixels = (int64_t)ci.batch * ci.out_h * ci.out_w;
+  const int64_t p0 = (int64_t)blockIdx.y * pixels_per_slice;
+  const int64_t p1 = p0 + pixels_per_slice < pixels ? p0 + pixels_per_slice : pixels;
+  f32x4 acc[9];
+#pragma unroll
+  for (int k = 0; k < 9; k++) acc[k] = f32x4{0.f, 0.f, 0.f, 0.f};
+  if (live) {
+    for (int64_t px = p0 + sub; px < p1; px += subs) {
+      const int yc = (int)(px % ci.out_w);
+      const int64_t t = px / ci.out_w;
+      const int yr = (int)(t % ci.out_h);
+      const int n = (int)(t / ci.out_h);
+      const f32x4 d = *reinterpret_cast<const f32x4*>(dy + px * ci.out_c + cq * 4);
+      const int xr0 = yr * ci.stride_h - ci.pad_top, xc0 = yc * ci.stride_w - ci.pad_left;
+      const float* xn = x + (int64_t)n * ci.in_h * ci.in_w * ci.in_c + cq * 4;
+#pragma unroll
+      for (int wr = 0; wr < 3; wr++) {
+        const int xr = xr0 + wr;
+#pragma unroll
+        for (int wc = 0; wc < 3; wc++) {
+          const int xc = xc0 + wc;
+          f32x4 v = {0.f, 0.f, 0.f, 0.f};
+          if ((unsigned)xr < (unsigned)ci.in_h && (unsigned)xc < (unsigned)ci.in_w)
+            v = *reinterpret_cast<const f32x4*>(xn + ((int64_t)xr * ci.in_w + xc) * ci.in_c);
+          acc[wr * 3 + wc] += v * d;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 9; k++) *reinterpret_cast<f32x4*>(red + (tid * 9 + k) * 4) = acc[k];
+  __syncthreads();
+  // thread -> (tap, quad): add the `subs` lanes of that quad in ascending order, in double
+  for (int item = tid; item < 9 * quads_per_wave; item += 256) {
+    const int k = item / quads_per_wave, q = item % quads_per_wave;
+    const int c = (blockIdx.x * quads_per_wave + q) * 4;
+    if (c >= ci.in_c) continue;
+    double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+    for (int r = 0; r < subs; r++) {
+      const float* v = red + ((r * quads_per_wave + q) * 9 + k) * 4;
+      s0 += (double)v[0];
+      s1 += (double)v[1];
+      s2 += (double)v[2];
+      s3 += (double)v[3];
+    }
+    double* out = partial + ((int64_t)blockIdx.y * 9 + k) * ci.in_c + c;
+    out[0] = s0;
+    out[1] = s1;
+    out[2] = s2;
+    out[3] = s3;
+  }
+}
+
 // Position (row-major over the dilated window) of the first strict maximum of the window of
 // output pixel (yr, yc), as maxPoolPositions finds it; -1 when nothing is greater than -inf.
 __device__ __forceinline__ int max_position(const float* x, const tfhip_conv2d_info& ci, int eff_h,
@@ -168,6 +278,8 @@ static int check_geometry(tfhip_ctx* ctx, const char* op, const tfhip_conv2d_inf
   return TFHIP_OK;
 }
 
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
 static unsigned grid_for(tfhip_ctx* ctx, int64_t elements) {
   const int64_t blocks = ceil_div(elements, 256);
   const int64_t cap = (int64_t)ctx->num_cus * 16;
@@ -201,9 +313,26 @@ extern "C" int tfhip_depthwise_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int6
   const float *dyf, *wf;
   if ((rc = as_f32(ctx, bdy, &tdy, &dyf))) return rc;
   if ((rc = as_f32(ctx, bw, &tw, &wf))) return rc;
+  float* dxf = static_cast<float*>(bdx->ptr);
+  if (ch_mul == 1 && ci->in_c % 4 == 0 && aligned16(dyf) && aligned16(wf) && aligned16(dxf)) {
+    const unsigned blocks = (unsigned)ceil_div(x_n / 4, 256);
+    const int s = ci->stride_h == ci->stride_w && ci->stride_h <= 2 ? ci->stride_h : 0;
+    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise_der_input_vec_s%d", s);
+    if (s == 1)
+      hipLaunchKernelGGL(depthwise_der_input_vec_kernel<1>, dim3(blocks), dim3(256), 0, ctx->stream,
+                         dyf, wf, dxf, *ci);
+    else if (s == 2)
+      hipLaunchKernelGGL(depthwise_der_input_vec_kernel<2>, dim3(blocks), dim3(256), 0, ctx->stream,
+                         dyf, wf, dxf, *ci);
+    else
+      hipLaunchKernelGGL(depthwise_der_input_vec_kernel<0>, dim3(blocks), dim3(256), 0, ctx->stream,
+                         dyf, wf, dxf, *ci);
+    TFHIP_LAUNCH_CHECK(ctx);
+    return TFHIP_OK;
+  }
   snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise_der_input");
   hipLaunchKernelGGL(depthwise_der_input_kernel, dim3(grid_for(ctx, x_n)), dim3(256), 0, ctx->stream,
-                     dyf, wf, static_cast<float*>(bdx->ptr), *ci, ch_mul);
+                     dyf, wf, dxf, *ci, ch_mul);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }
@@ -233,8 +362,34 @@ extern "C" int tfhip_depthwise_conv2d_der_filter(tfhip_ctx* ctx, int64_t x, int6
   const float *xf, *dyf;
   if ((rc = as_f32(ctx, bx, &tx, &xf))) return rc;
   if ((rc = as_f32(ctx, bdy, &tdy, &dyf))) return rc;
-  // enough pixel slices to fill the machine, at least 64 pixels each
   const int64_t pixels = (int64_t)ci->batch * ci->out_h * ci->out_w;
+  if (ch_mul == 1 && ci->filter_h == 3 && ci->filter_w == 3 && ci->in_c % 4 == 0 && aligned16(xf) &&
+      aligned16(dyf) && pixels > 0) {
+    const int c4 = ci->in_c / 4;
+    int qpw = 1;                       // channel quads per workgroup: a power of two <= 64
+    while (qpw < 64 && qpw < c4) qpw *= 2;
+    const int64_t blocks_c = ceil_div(c4, qpw);
+    const int subs = 256 / qpw;
+    // two workgroups per CU, and at least 32 pixels per lane so that the reduction through
+    // LDS and the partial sums stay a small part of the work
+    int64_t slices = ceil_div((int64_t)ctx->num_cus * 2, blocks_c);
+    if (slices > ceil_div(pixels, (int64_t)subs * 32)) slices = ceil_div(pixels, (int64_t)subs * 32);
+    if (slices < 1) slices = 1;
+    if (slices > 65535) slices = 65535;
+    const int64_t per_slice = ceil_div(pixels, slices);
+    if (!tpart.get((size_t)(slices * w_n) * sizeof(double))) return TFHIP_EDEVICE;
+    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise3x3_der_filter");
+    hipLaunchKernelGGL(depthwise3x3_der_filter_partial_kernel, dim3((unsigned)blocks_c, (unsigned)slices),
+                       dim3(256), (size_t)(256 * 9 * 4 * sizeof(float)), ctx->stream, xf, dyf,
+                       static_cast<double*>(tpart.ptr), *ci, qpw, per_slice);
+    TFHIP_LAUNCH_CHECK(ctx);
+    hipLaunchKernelGGL(depthwise_der_filter_finish_kernel, dim3((unsigned)ceil_div(w_n, 256)), dim3(256),
+                       0, ctx->stream, static_cast<const double*>(tpart.ptr),
+                       static_cast<float*>(bdw->ptr), w_n, (int)slices);
+    TFHIP_LAUNCH_CHECK(ctx);
+    return TFHIP_OK;
+  }
+  // enough pixel slices to fill the machine, at least 64 pixels each
   const int64_t channel_blocks = ceil_div(ci->out_c, 64);
   int64_t slices = ceil_div((int64_t)ctx->num_cus * 8, channel_blocks * taps);
   if (slices > ceil_div(pixels, 64)) slices = ceil_div(pixels, 64);

@@ -1504,6 +1504,13 @@ extern "C" int tfhip_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int64_t filter
   p.pl = ci->filter_w - 1 - ci->pad_left;
   p.up_h = ci->stride_h; p.up_w = ci->stride_w;
   p.a_vec = aligned16(p.A) && (ci->out_c % 4 == 0);
+  if (ci->filter_h == 1 && ci->filter_w == 1 && ci->stride_h == 1 && ci->stride_w == 1 &&
+      ci->pad_top == 0 && ci->pad_left == 0 && ci->out_h == ci->in_h && ci->out_w == ci->in_w) {
+    // pointwise: dx = dy [pixels, out_c] x W^T [out_c, in_c], a plain product
+    p.lda = ci->out_c;
+    p.a_vec = aligned16(p.A) && (p.lda % 4 == 0);
+    return launch_gemm(ctx, p, 1, A_ROWMAJOR, B_ROWMAJOR, /*kblocked=*/false);
+  }
   return launch_gemm(ctx, p, 1, A_IM2COL_UP, B_ROWMAJOR, /*kblocked=*/false);
 }
 
