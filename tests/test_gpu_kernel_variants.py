@@ -248,3 +248,24 @@ def test_backward_kernel_variants(tf):
     assert seen["dw_der_filter"] == "depthwise3x3_der_filter", seen
     assert seen["dw_der_input_mul2"] == "depthwise_der_input", seen
     assert seen["dw_der_filter_mul2"] == "depthwise_der_filter", seen
+
+
+@pytest.mark.parametrize("xs,fs,stride,pad", [
+    ((20, 56, 56, 64), (3, 3, 64, 128), 2, "same"),      # 3x3 stride 2: classes of 1, 2, 2, 4 taps
+    ((24, 60, 61, 32), (5, 5, 32, 64), 3, "same"),       # stride 3, 5x5, odd width
+    ((40, 56, 56, 128), (1, 1, 128, 256), 2, "same"),    # 1x1 stride 2: three classes are all zero
+    ((16, 57, 59, 64), (4, 4, 64, 96), (2, 1), "valid"), # stride on rows only
+])
+def test_conv2d_der_input_by_parity(tf, ref, xs, fs, stride, pad):
+    """Large strided layers: dx is computed one pixel-parity class at a time on the forward
+    kernels; compared with the oracle."""
+    print("by parity", xs, fs, stride, pad, flush=True)
+    rng = np.random.default_rng(sum(xs) + sum(fs))
+    w = (rng.standard_normal(fs) * np.sqrt(2.0 / (fs[0] * fs[1] * fs[3]))).astype(np.float32)
+    from oracle import cpu_ref
+    ci = cpu_ref.compute_conv2d_info(xs, fs, stride, 1, pad)
+    dy = rng.uniform(-1, 1, ci["outShape"]).astype(np.float32)
+    with tf.tidy():
+        got = tf.conv2d_der_input(xs, tf.tensor(dy), tf.tensor(w), stride, pad).data_sync()
+        assert last_kernel(tf).endswith("_by_parity"), last_kernel(tf)
+    close(got, ref.conv2d_der_input(xs, dy, w, stride, pad), atol=2e-5)

@@ -1434,6 +1434,38 @@ __global__ void flip_filter_kernel(const float* w, float* out, int KH, int KW, i
   }
 }
 
+// The same for the taps wr = r0 + sr * i (i < KHc), wc = c0 + sc * j (j < KWc) only:
+// out[(i, j, co)][ci] = w[KH - 1 - wr][KW - 1 - wc][ci][co].
+__global__ void flip_filter_taps_kernel(const float* w, float* out, int KH, int KW, int Cin,
+                                        int Cout, int r0, int sr, int KHc, int c0, int sc, int KWc) {
+  const int total = KHc * KWc * Cin * Cout;
+  for (int g = blockIdx.x * blockDim.x + threadIdx.x; g < total; g += gridDim.x * blockDim.x) {
+    const int ci = g % Cin;
+    int t = g / Cin;
+    const int co = t % Cout;
+    t /= Cout;
+    const int j = t % KWc, i = t / KWc;
+    const int wr = r0 + sr * i, wc = c0 + sc * j;
+    out[g] = w[(((KH - 1 - wr) * KW + (KW - 1 - wc)) * Cin + ci) * Cout + co];
+  }
+}
+
+// dx[n, r0 + sr * i, c0 + sc * j, :] = src[(n, i, j), :] for a [batch * Hc * Wc, C] block.
+__global__ void scatter_pixels_kernel(const float* __restrict__ src, float* __restrict__ dx,
+                                      int64_t total, int Hc, int Wc, int C, int in_h, int in_w,
+                                      int r0, int sr, int c0, int sc) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += stride) {
+    const int c = (int)(g % C);
+    int64_t t = g / C;
+    const int j = (int)(t % Wc);
+    t /= Wc;
+    const int i = (int)(t % Hc);
+    const int64_t n = t / Hc;
+    dx[((n * in_h + r0 + sr * i) * in_w + c0 + sc * j) * C + c] = src[g];
+  }
+}
+
 static int check_backward_geometry(tfhip_ctx* ctx, const char* op, const tfhip_conv2d_info* ci) {
   if (ci->batch < 0 || ci->in_h < 0 || ci->in_w < 0 || ci->in_c < 0 || ci->out_h < 0 ||
       ci->out_w < 0 || ci->out_c < 0 || ci->filter_h <= 0 || ci->filter_w <= 0 ||
@@ -1504,6 +1536,67 @@ extern "C" int tfhip_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int64_t filter
   p.pl = ci->filter_w - 1 - ci->pad_left;
   p.up_h = ci->stride_h; p.up_w = ci->stride_w;
   p.a_vec = aligned16(p.A) && (ci->out_c % 4 == 0);
+  // Stride above 1 on a large layer: dx pixels of one parity class (row % stride_h, column %
+  // stride_w) all use the same subset of filter taps, and over that subset the gather is an
+  // ordinary stride-1 convolution of dy.  One product per class on the forward kernels, none of
+  // them multiplying the zeros of a stretched dy; the class results are scattered into dx.
+  // (Small layers stay on the single stretched-gather launch: a class costs three launches.)
+  if ((ci->stride_h > 1 || ci->stride_w > 1) &&
+      2.0 * p.M * (double)p.N * p.K >= 8e9 && ci->stride_h * ci->stride_w <= 16) {
+    const int top_pad = ci->filter_h - 1 - ci->pad_top, left_pad = ci->filter_w - 1 - ci->pad_left;
+    auto mod = [](int a, int m) { return ((a % m) + m) % m; };
+    bool some_empty = false;
+    for (int r0 = 0; r0 < ci->stride_h && !some_empty; r0++)
+      for (int c0 = 0; c0 < ci->stride_w; c0++)
+        if (mod(top_pad - r0, ci->stride_h) >= ci->filter_h ||
+            mod(left_pad - c0, ci->stride_w) >= ci->filter_w)
+          some_empty = true;
+    if (some_empty &&
+        hipMemsetAsync(bdx->ptr, 0, (size_t)x_n * sizeof(float), ctx->stream) != hipSuccess)
+      return ctx->fail(TFHIP_EDEVICE, "conv2dDerInput: memset failed");
+    for (int r0 = 0; r0 < ci->stride_h; r0++)
+      for (int c0 = 0; c0 < ci->stride_w; c0++) {
+        const int Hc = (int)ceil_div(ci->in_h - r0, ci->stride_h);
+        const int Wc = (int)ceil_div(ci->in_w - c0, ci->stride_w);
+        const int wr0 = mod(top_pad - r0, ci->stride_h), wc0 = mod(left_pad - c0, ci->stride_w);
+        if (Hc <= 0 || Wc <= 0 || wr0 >= ci->filter_h || wc0 >= ci->filter_w) continue;
+        const int KHc = (int)ceil_div(ci->filter_h - wr0, ci->stride_h);
+        const int KWc = (int)ceil_div(ci->filter_w - wc0, ci->stride_w);
+        const int64_t taps_n = (int64_t)KHc * KWc * ci->in_c * ci->out_c;
+        const int64_t rows = (int64_t)ci->batch * Hc * Wc;
+        Temp tsub(ctx), tout(ctx);
+        if (!tsub.get((size_t)taps_n * sizeof(float)) ||
+            !tout.get((size_t)(rows * ci->in_c) * sizeof(float)))
+          return TFHIP_EDEVICE;
+        const int64_t fb = ceil_div(taps_n, 256);
+        hipLaunchKernelGGL(flip_filter_taps_kernel, dim3((unsigned)(fb > 4096 ? 4096 : fb)), dim3(256),
+                           0, ctx->stream, wf, static_cast<float*>(tsub.ptr), ci->filter_h,
+                           ci->filter_w, ci->in_c, ci->out_c, wr0, ci->stride_h, KHc, wc0,
+                           ci->stride_w, KWc);
+        TFHIP_LAUNCH_CHECK(ctx);
+        GemmArgs q = p;
+        q.B = tsub.ptr;
+        q.C = static_cast<float*>(tout.ptr);
+        q.M = (int)rows;
+        q.K = KHc * KWc * ci->out_c;
+        q.OH = Hc; q.OW = Wc;
+        q.KH = KHc; q.KW = KWc;
+        // dy row of tap i for class row a: a + i + (r0 - top_pad + wr0) / stride_h
+        q.pt = -((r0 - top_pad + wr0) / ci->stride_h);
+        q.pl = -((c0 - left_pad + wc0) / ci->stride_w);
+        q.up_h = q.up_w = 1;
+        q.b_vec = aligned16(q.B) && (q.ldb % 4 == 0);
+        if ((rc = launch_gemm(ctx, q, 1, A_IM2COL, B_ROWMAJOR, /*kblocked=*/false))) return rc;
+        const int64_t total = rows * ci->in_c;
+        const int64_t sb = ceil_div(total, 256), cap = (int64_t)ctx->num_cus * 16;
+        hipLaunchKernelGGL(scatter_pixels_kernel, dim3((unsigned)(sb > cap ? cap : sb)), dim3(256), 0,
+                           ctx->stream, static_cast<const float*>(tout.ptr), p.C, total, Hc, Wc,
+                           ci->in_c, ci->in_h, ci->in_w, r0, ci->stride_h, c0, ci->stride_w);
+        TFHIP_LAUNCH_CHECK(ctx);
+      }
+    strncat(ctx->last_kernel, "_by_parity", sizeof ctx->last_kernel - strlen(ctx->last_kernel) - 1);
+    return TFHIP_OK;
+  }
   if (ci->filter_h == 1 && ci->filter_w == 1 && ci->stride_h == 1 && ci->stride_w == 1 &&
       ci->pad_top == 0 && ci->pad_left == 0 && ci->out_h == ci->in_h && ci->out_w == ci->in_w) {
     // pointwise: dx = dy [pixels, out_c] x W^T [out_c, in_c], a plain product
