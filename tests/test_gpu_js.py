@@ -318,3 +318,106 @@ def test_js_backward_ops_match_oracle(tmp_path, ref):
     results = c.run()
     c.check(results)
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
+def _golden(name, title, describe=None):
+    with open(os.path.join(ROOT, "tests", "golden", name + ".json")) as f:
+        cases = json.load(f)["cases"]
+    hits = [c for c in cases if c["title"] == title and (describe is None or c["describe"] == describe)]
+    assert len(hits) == 1, (name, title, len(hits))
+    return hits[0]
+
+
+def test_js_gradients_through_the_tape(tmp_path, ref):
+    """tf.grad / tf.grads on the hip backend: the reference's own gradient blocks (conv2d,
+    conv2dTranspose, depthwiseConv2d, maxPool, avgPool), then composites against closed forms
+    and against the oracle's backward kernels chained by hand."""
+    rng = np.random.default_rng(53)
+    c = Cases(tmp_path)
+    f = lambda *s: rng.uniform(-1, 1, s).astype(np.float32)
+    flat = lambda a: np.asarray(a, np.float32).ravel()
+
+    # ops/conv2d_test.ts: gradient with clones
+    a = _golden("conv2d_grad", "gradient with clones input=[3,3,1] f=[2,2,1,1] s=1 p=0")["arrays"]
+    x, dy, w = flat(a[4]).reshape(3, 3, 1), flat(a[5]).reshape(2, 2, 1), np.ones((2, 2, 1, 1), np.float32)
+    c.add("conv2d_dx", "gradConv2d", dict(x=x, filter=w, dy=dy), dict(strides=1, pad=0, wrt=0),
+          flat(a[8]).reshape(3, 3, 1), atol=1e-3)
+    c.add("conv2d_dw", "gradConv2d", dict(x=x, filter=w, dy=dy), dict(strides=1, pad=0, wrt=1),
+          flat(a[9]).reshape(2, 2, 1, 1), atol=1e-3)
+    # ops/conv2d_transpose_test.ts: stride 2, 'same', two channels
+    a = _golden("conv2d_transpose", "gradient input=[1,2,2,2] f=[2,2,2,1] s=[2,2] padding=same")["arrays"]
+    x, w = flat(a[6]).reshape(1, 2, 2, 2), flat(a[7]).reshape(2, 2, 2, 2)
+    ones = np.ones((1, 3, 3, 2), np.float32)
+    attrs = dict(outputShape=[1, 3, 3, 2], strides=2, pad="same")
+    c.add("transpose_dx", "gradConv2dTranspose", dict(x=x, filter=w, dy=ones), dict(attrs, wrt=0),
+          flat(a[11]).reshape(1, 2, 2, 2), atol=1e-3)
+    c.add("transpose_dw", "gradConv2dTranspose", dict(x=x, filter=w, dy=ones), dict(attrs, wrt=1),
+          flat(a[13]).reshape(2, 2, 2, 2), atol=1e-3)
+    # ops/conv2d_depthwise_test.ts: depthwiseConv2d gradients
+    g = lambda t: _golden("depthwise_grad", t)["arrays"]
+    b = g("beforeEach")
+    images, filt = flat(b[0]).reshape(2, 2, 2, 3), flat(b[1]).reshape(2, 2, 3, 2)
+    for tag, title, wrt, sq in (("dx", "wrt input", 0, False), ("dw", "wrt filter", 1, False),
+                                ("dx_sq", "wrt input, squared output", 0, True),
+                                ("dw_sq", "wrt filter, squared output", 1, True)):
+        c.add("depthwise_" + tag, "gradDepthwise", dict(x=images, filter=filt),
+              dict(strides=1, pad="same", wrt=wrt, squared=sq),
+              flat(g(title)[0]).reshape(images.shape if wrt == 0 else filt.shape), atol=1e-3)
+    # ops/pool_test.ts
+    a = _golden("pool_grad", "gradient x=[5,5,1] f=[3,3] s=2 duplicate max value", "maxPoolBackprop")["arrays"]
+    c.add("maxpool_dup", "gradPool", dict(x=flat(a[2]).reshape(a[3]), dy=flat(a[0]).reshape(a[1])),
+          dict(kind="max", filterSize=3, strides=2, pad=0), flat(a[4]).reshape(a[3]), atol=1e-3)
+    a = _golden("pool_grad", "gradient x=[2,3,3,1] f=[2,2], s=1", "avgPool")["arrays"]
+    xa, dya = flat(a[0]).reshape(a[1]), flat(a[2]).reshape(a[3])
+    c.add("avgpool", "gradPool", dict(x=xa, dy=dya), dict(kind="avg", filterSize=2, strides=1, pad=0),
+          ref.avg_pool_backprop(dya, xa, 2, 1, 0))
+
+    # a two-layer perceptron against the closed form in float64
+    x, t = f(17, 12), f(17, 5)
+    w1, b1, w2 = f(12, 9) * 0.5, f(9) * 0.1, f(9, 5) * 0.5
+    pre = x.astype(np.float64) @ w1 + b1
+    h = np.maximum(pre, 0)
+    dout = 2 * (h @ w2 - t)
+    dpre = (dout @ w2.T.astype(np.float64)) * (pre > 0)
+    want = [x.T.astype(np.float64) @ dpre, dpre.sum(0), h.T @ dout]
+    for k, name in enumerate(("w1", "b1", "w2")):
+        for op in ("gradMlp", "gradFusedMlp"):
+            c.add("%s_d%s" % (op, name), op, dict(x=x, t=t, w1=w1, b1=b1, w2=w2), dict(wrt=k),
+                  want[k].astype(np.float32), atol=1e-4)
+    logits = f(6, 10) * 3
+    labels = np.eye(10, dtype=np.float32)[rng.integers(0, 10, 6)]
+    e = np.exp(logits.astype(np.float64) - logits.max(1, keepdims=True))
+    c.add("softmax_xent", "gradSoftmaxXent", dict(logits=logits, labels=labels), {},
+          (e / e.sum(1, keepdims=True) - labels).astype(np.float32), atol=1e-5)
+
+    # the conv net: backward pass chained by hand from the oracle's kernels
+    x, t = f(3, 8, 8, 4), f(3, 6)
+    cw, cb, dw, fw = f(3, 3, 4, 8) * 0.3, f(8) * 0.1, f(3, 3, 8, 1) * 0.3, f(2 * 2 * 8, 6) * 0.3
+    z = ref.conv2d(x, cw, 1, "same") + cb
+    h1 = np.maximum(z, 0)
+    p1 = ref.max_pool(h1, 2, 2, "valid")
+    d1 = ref.depthwise_conv2d(p1, dw, 1, "same")
+    p2 = ref.avg_pool(d1, 2, 2, "valid")
+    flatten = p2.reshape(3, -1)
+    dout = 2 * (flatten.astype(np.float64) @ fw - t)
+    want_fw = flatten.T.astype(np.float64) @ dout
+    dp2 = (dout @ fw.T.astype(np.float64)).reshape(p2.shape).astype(np.float32)
+    dd1 = ref.avg_pool_backprop(dp2, d1, 2, 2, "valid")
+    want_dw = ref.depthwise_der_filter(p1, dd1, dw.shape, 1, "same")
+    dp1 = ref.depthwise_der_input(p1.shape, dd1, dw, 1, "same")
+    dh1 = ref.max_pool_backprop(dp1, h1, 2, 2, "valid")
+    dz = dh1 * (z > 0)
+    want_cw = ref.conv2d_der_filter(x, dz, cw.shape, 1, "same")
+    want_cb = dz.astype(np.float64).sum((0, 1, 2))
+    ins = dict(x=x, t=t, cw=cw, cb=cb, dw=dw, fw=fw)
+    for k, (name, want_k) in enumerate((("cw", want_cw), ("cb", want_cb), ("dw", want_dw), ("fw", want_fw))):
+        c.add("convnet_d" + name, "gradConvNet", ins, dict(wrt=k), np.asarray(want_k, np.float32),
+              rtol=1e-3, atol=1e-4)
+    # SGD on the same net: the mean squared error must fall
+    c.add("train", "trainConvNet", ins, dict(steps=12, lr=0.05), np.zeros(12, np.float32), atol=1e9)
+    results = c.run()
+    c.check(results)
+    losses = np.fromfile(os.path.join(str(tmp_path), "train.out.bin"), np.float32)
+    assert losses.shape == (12,) and np.all(np.isfinite(losses))
+    assert losses[-1] < 0.7 * losses[0] and np.all(np.diff(losses) < 1e-3), losses
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0

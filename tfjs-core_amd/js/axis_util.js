@@ -48,7 +48,13 @@ function getInnerMostAxes(numAxes, rank) {
   return res;
 }
 
+// The permutation that undoes `axes` (axis_util.ts:150-154).
+function getUndoAxesPermutation(axes) {
+  return axes.map((axis, i) => [i, axis]).sort((a, b) => a[1] - b[1]).map(x => x[0]);
+}
+
 module.exports = {
+  getUndoAxesPermutation,
   axesAreInnerMostDims, assertAxesAreInnerMostDims, computeOutAndReduceShapes,
   expandShapeToKeepDim, getAxesPermutation, getInnerMostAxes
 };

@@ -35,4 +35,16 @@ function assertAndGetBroadcastShape(shapeA, shapeB) {
   return result;
 }
 
-module.exports = {getBroadcastDims, assertAndGetBroadcastShape};
+// Axes of the broadcast result over which a gradient must be summed to get back the shape of
+// an operand (broadcast_util.ts:48-59).
+function getReductionAxes(inShape, outShape) {
+  const result = [];
+  for (let i = 0; i < outShape.length; i++) {
+    const inDim = inShape[inShape.length - i - 1];
+    const outAxis = outShape.length - i - 1;
+    if (inDim == null || (inDim === 1 && outShape[outAxis] > 1)) result.unshift(outAxis);
+  }
+  return result;
+}
+
+module.exports = {getBroadcastDims, assertAndGetBroadcastShape, getReductionAxes};

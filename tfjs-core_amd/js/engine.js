@@ -3,12 +3,13 @@
 // dispatch, per-dataId reference counts, tidy scopes, cross-backend data movement, memory
 // and timing.  After tfjs-core/src/engine.ts: registry/init :149-359, moveData :361-363,
 // tidy/scopes :365-411, 675-718, runKernel :435-498, registerTensor/disposeTensor
-// :502-572, memory/profile :588-622, write/read :833-877.  Autodiff is not part of this
-// path, so runKernel never records a tape (save() is a no-op, as at :445-453).
+// :502-572, memory/profile :588-622, write/read :833-877, tape and gradients :435-498,
+// 628-774, customGrad :776-831 (the tape algorithm itself is in tape.js).
 const util = require('./util');
 const {Tensor, setTensorTracker} = require('./tensor');
 const {Profiler} = require('./profiler');
 const {ENV} = require('./environment');
+const {getFilteredNodesXToY, backpropagateGradients} = require('./tape');
 
 class Engine {
   constructor() {
@@ -28,7 +29,7 @@ class Engine {
       tensorInfo: new WeakMap(), numTensors: 0, numBytes: 0, numDataBuffers: 0,
       scopeStack: [], activeScope: null, kernelDepth: 0, profiling: false,
       activeProfile: {newBytes: 0, newTensors: 0, peakBytes: 0, kernels: [], result: null},
-      nextScopeId: 0
+      nextScopeId: 0, activeTape: null, gradientDepth: 0, nextTapeNodeId: 0
     };
   }
 
@@ -267,10 +268,17 @@ class Engine {
   }
 
   // ---- kernels --------------------------------------------------------------------
-  runKernel(forwardFunc, inputs) {
+  // backwardsFunc(dy, saved) -> {inputName: () => Tensor}; forwardFunc may hand tensors the
+  // gradient needs to save(), which keeps clones of them until the tape is released.
+  runKernel(forwardFunc, inputs, backwardsFunc) {
     let result;
+    let saved = [];
     const scopeName = this.state.activeScope != null ? this.state.activeScope.name : '';
-    const save = () => {};  // no tape on this path
+    const tapeOn = this.isTapeOn();
+    const save = tensors => {
+      if (!tapeOn) return;
+      saved = tensors.map(t => this.keep(this.taped(t)));
+    };
     const startingBytes = this.state.numBytes;
     const startingTensors = this.state.numTensors;
     this.scopedRun(() => this.state.kernelDepth++, () => this.state.kernelDepth--, () => {
@@ -280,6 +288,13 @@ class Engine {
         result = this.profiler.profileKernel(scopeName, () => forwardFunc(this.backend, save));
       }
     });
+    if (tapeOn) {
+      this.state.activeTape.push({
+        id: this.state.nextTapeNodeId++, name: scopeName, inputs: inputs || {},
+        outputs: Array.isArray(result) ? result : [result], saved,
+        gradient: backwardsFunc == null ? null : dy => backwardsFunc(dy, saved)
+      });
+    }
     if (this.state.profiling) {
       this.state.activeProfile.kernels.push({
         name: scopeName,
@@ -292,6 +307,101 @@ class Engine {
       });
     }
     return result;
+  }
+
+  // ---- tape ------------------------------------------------------------------------
+  isTapeOn() { return this.state.gradientDepth > 0 && this.state.kernelDepth === 0; }
+
+  // A second tensor over the same buffer (reference count + 1), outside any tape.
+  aliasOf(t) { return Tensor.make(t.shape, {dataId: t.dataId}, t.dtype); }
+
+  // An alias that the tape knows to be the same value as `t` (engine.ts:426-432): gradient
+  // functions compute with saved aliases, and a higher-order gradient must see through them.
+  taped(t) {
+    const y = this.aliasOf(t);
+    this.state.activeTape.push({
+      id: this.state.nextTapeNodeId++, name: 'clone', inputs: {0: t}, outputs: [y], saved: [],
+      gradient: dy => ({0: () => dy.toFloat()})
+    });
+    return y;
+  }
+
+  startTape() {
+    if (this.state.gradientDepth === 0) this.state.activeTape = [];
+    this.state.gradientDepth++;
+  }
+  endTape() { this.state.gradientDepth--; }
+
+  // value = f() and d value / d xs[i], with dy (default ones) flowing into value
+  // (engine.ts:726-774).  `ops` = {ones, zeros, add} of the op layer.
+  gradients(f, xs, dy, allowNoGradients, ops) {
+    util.assert(xs.length > 0, () => 'gradients() received an empty list of xs.');
+    if (dy != null && dy.dtype !== 'float32') {
+      throw new Error(`dy must have 'float32' dtype, but has '${dy.dtype}'`);
+    }
+    const y = this.scopedRun(() => this.startTape(), () => this.endTape(), () => this.tidy('forward', f));
+    util.assert(y instanceof Tensor, () => 'The result y returned by f() must be a tensor.');
+    const filteredTape = getFilteredNodesXToY(this.state.activeTape, xs, y);
+    if (!allowNoGradients && filteredTape.length === 0 && xs.length > 0) {
+      throw new Error('Cannot compute gradient of y=f(x) with respect to x. Make sure ' +
+                      'that the f you passed encloses all operations that lead from x to y.');
+    }
+    const release = () => {
+      if (this.state.gradientDepth === 0 && this.state.activeTape != null) {
+        this.state.activeTape.forEach(node => node.saved.forEach(t => t.dispose()));
+        this.state.activeTape = null;
+      }
+    };
+    try {
+      return this.tidy('backward', () => {
+        const map = {};
+        map[y.id] = dy == null ? ops.ones(y.shape) : dy;
+        backpropagateGradients(map, filteredTape, fn => this.tidy(fn), ops.zeros, ops.add,
+                               util.arraysEqual);
+        const grads = xs.map(x => map[x.id]);
+        return {value: y, grads};
+      });
+    } finally {
+      release();
+    }
+  }
+
+  // f(...inputs, save) -> {value, gradFunc(dy, saved)} (engine.ts:776-831).
+  customGrad(f) {
+    util.assert(typeof f === 'function', () => 'The f passed in customGrad(f) must be a function.');
+    return (...inputs) => {
+      util.assert(inputs.every(t => t instanceof Tensor),
+                  () => 'The args passed in customGrad(f)(x1, x2,...) must all be tensors');
+      let res;
+      const inputMap = {};
+      inputs.forEach((input, i) => { inputMap[i] = input; });
+      return this.runKernel(
+          (_, save) => {
+            res = f.apply(null, inputs.concat([save]));
+            util.assert(res.value instanceof Tensor,
+                        () => 'The function f passed in customGrad(f) must return an ' +
+                            'object where `obj.value` is a tensor');
+            util.assert(typeof res.gradFunc === 'function',
+                        () => 'The function f passed in customGrad(f) must return an ' +
+                            'object where `obj.gradFunc` is a function.');
+            return res.value;
+          },
+          inputMap,
+          (dy, saved) => {
+            const gradRes = res.gradFunc(dy, saved);
+            const grads = Array.isArray(gradRes) ? gradRes : [gradRes];
+            util.assert(grads.length === inputs.length,
+                        () => 'The function f passed in customGrad(f) must return an object ' +
+                            'where `obj.gradFunc` is a function that returns the same ' +
+                            'number of tensors as inputs passed to f(...).');
+            util.assert(grads.every(t => t instanceof Tensor),
+                        () => 'The function f passed in customGrad(f) must return an object ' +
+                            'where `obj.gradFunc` is a function that returns a list of only tensors.');
+            const gradMap = {};
+            grads.forEach((g, i) => { gradMap[i] = () => g; });
+            return gradMap;
+          });
+    };
   }
 
   // ---- tensor bookkeeping ---------------------------------------------------------

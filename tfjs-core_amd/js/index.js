@@ -13,8 +13,9 @@ const conv_util = require('./conv_util');
 const broadcast_util = require('./broadcast_util');
 const axis_util = require('./axis_util');
 const io = Object.assign({}, require('./io_utils'), require('./weights_loader'));
+const gradients = require('./gradients');
 
-const tf = Object.assign({}, ops, {
+const tf = Object.assign({}, ops, gradients, {
   Tensor, KernelBackend, DataStorage, ENV, util, io,
   backend_util: Object.assign({}, conv_util, broadcast_util, axis_util),
   engine: () => ENGINE,

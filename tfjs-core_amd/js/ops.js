@@ -79,6 +79,24 @@ function makeTypesMatch(a, b) {  // tensor_util.ts:22-28
   return [cast(a, dtype), cast(b, dtype)];
 }
 
+// ---- gradient helpers ---------------------------------------------------------------------
+// dy of a broadcast result, summed back to the shape of one operand (binary_ops.ts:76-96).
+function unbroadcast(g, shape) {
+  const axes = broadcast_util.getReductionAxes(shape, g.shape);
+  const r = axes.length > 0 ? sum(g, axes) : g;
+  return reshape(r, shape);
+}
+// 1 where x > 0, else 0 (the reference's step(x) up to NaN, which it passes through).
+function stepOf(x) {
+  return cast(greater(x, zeros([], x.dtype)), 'float32');
+}
+// dy through a fused activation (fused_ops.ts:38-49).
+function fusedDyActivation(dy, y, activation) {
+  if (activation == null || activation === 'linear') return dy;
+  if (activation === 'relu') return mul(dy, stepOf(y));
+  throw new Error(`Gradient for activation ${activation} has not been implemented yet.`);
+}
+
 const fill = (shape, value, dtype) => ENGINE.runKernel(b => b.fill(shape, value, dtype), {});
 const zeros = (shape, dtype) => fill(shape, 0, dtype || 'float32');
 const ones = (shape, dtype) => fill(shape, 1, dtype || 'float32');
@@ -90,19 +108,20 @@ const reshape = op('reshape', (x, shape) => {
   const $x = convertToTensor(x, 'x', 'reshape');
   shape = util.inferFromImplicitShape(shape, $x.size);
   util.assert($x.size === util.sizeFromShape(shape), 'new shape and old shape must have the same number of elements.');
-  return ENGINE.runKernel(b => b.reshape($x, shape), {$x});
+  return ENGINE.runKernel(b => b.reshape($x, shape), {$x}, dy => ({$x: () => reshape(dy, $x.shape)}));
 });
 
 const cast = op('cast', (x, dtype) => {
   const $x = convertToTensor(x, 'x', 'cast');
   util.assert(['float32', 'int32', 'bool'].indexOf(dtype) !== -1, `Failed to cast to unknown dtype ${dtype}`);
-  return ENGINE.runKernel(b => b.cast($x, dtype), {$x});
+  return ENGINE.runKernel(b => b.cast($x, dtype), {$x}, dy => ({$x: () => clone(dy)}));
 });
 
 const clone = op('clone', x => {
   const $x = convertToTensor(x, 'x', 'clone');
   // same dataId, as the reference (tensor_ops.ts: clone -> Tensor.make(shape, {dataId}))
-  return ENGINE.runKernel(() => Tensor.make($x.shape, {dataId: $x.dataId}, $x.dtype), {$x});
+  return ENGINE.runKernel(() => Tensor.make($x.shape, {dataId: $x.dataId}, $x.dtype), {$x},
+                          dy => ({$x: () => cast(dy, 'float32')}));
 });
 
 const dequantize = op('dequantize', x => {
@@ -145,10 +164,24 @@ const matMul = op('matMul', (a, b, transposeA, transposeB) => {
   transposeA = !!transposeA;
   transposeB = !!transposeB;
   const {a3D, b3D, outShape} = matMulPrep(a, b, transposeA, transposeB, 'matMul');
-  const res = ENGINE.runKernel(backend => backend.batchMatMul(a3D, b3D, transposeA, transposeB),
-                               {$a: a3D, $b: b3D});
+  const res = ENGINE.runKernel((backend, save) => {
+    save([a3D, b3D]);
+    return backend.batchMatMul(a3D, b3D, transposeA, transposeB);
+  }, {$a: a3D, $b: b3D}, (dy, saved) => matMulGrads(dy, saved[0], saved[1], transposeA, transposeB));
   return reshape(res, outShape);
 });
+
+// d/da and d/db of a (batched) product for the four transpose combinations (matmul.ts:100-130).
+function matMulGrads(dy, a3D, b3D, transposeA, transposeB) {
+  if (!transposeA && !transposeB) {
+    return {$a: () => matMul(dy, b3D, false, true), $b: () => matMul(a3D, dy, true, false)};
+  } else if (!transposeA && transposeB) {
+    return {$a: () => matMul(dy, b3D, false, false), $b: () => matMul(dy, a3D, true, false)};
+  } else if (transposeA && !transposeB) {
+    return {$a: () => matMul(b3D, dy, false, true), $b: () => matMul(a3D, dy, false, false)};
+  }
+  return {$a: () => matMul(b3D, dy, true, true), $b: () => matMul(dy, a3D, true, true)};
+}
 
 const fusedMatMul = op('fusedMatMul', (config) => {
   const transposeA = !!config.transposeA, transposeB = !!config.transposeB;
@@ -164,12 +197,25 @@ const fusedMatMul = op('fusedMatMul', (config) => {
   if (config.preluActivationWeights != null) {
     $prelu = convertToTensor(config.preluActivationWeights, 'prelu weights', 'fused matMul');
   }
+  const inputs = {$a: a3D, $b: b3D};
+  if ($bias != null) inputs.$bias = $bias;
+  if ($prelu != null) inputs.$prelu = $prelu;
   const res = ENGINE.runKernel(
-      backend => backend.fusedBatchMatMul({
-        a: a3D, b: b3D, transposeA, transposeB, bias: $bias, activation,
-        preluActivationWeights: $prelu
-      }),
-      {$a: a3D, $b: b3D});
+      (backend, save) => {
+        const y = backend.fusedBatchMatMul({
+          a: a3D, b: b3D, transposeA, transposeB, bias: $bias, activation,
+          preluActivationWeights: $prelu
+        });
+        save([a3D, b3D, y]);
+        return y;
+      },
+      inputs,
+      (dy, saved) => {  // fused_ops.ts:150-210
+        const dyAct = fusedDyActivation(dy, saved[2], activation);
+        const g = matMulGrads(dyAct, saved[0], saved[1], transposeA, transposeB);
+        if ($bias != null) g.$bias = () => unbroadcast(dyAct, $bias.shape);
+        return g;
+      });
   return reshape(res, outShape);
 });
 
@@ -212,9 +258,24 @@ function lower(res, reshapedTo4D) {
 const conv2d = op('conv2d', (x, filter, strides, pad, dataFormat, dilations, dimRoundingMode) => {
   const {x4D, $filter, convInfo, reshapedTo4D} =
       convPrep(x, filter, strides, pad, dataFormat, dilations, dimRoundingMode, 'conv2d', false);
-  const res = ENGINE.runKernel(backend => backend.conv2d(x4D, $filter, convInfo), {x: x4D, $filter});
+  const res = ENGINE.runKernel((backend, save) => {
+    save([$filter, x4D]);
+    return backend.conv2d(x4D, $filter, convInfo);
+  }, {x: x4D, $filter}, (dy, saved) => conv2dGrads(dy, saved[1], saved[0], strides, pad, dilations));
   return lower(res, reshapedTo4D);
 });
+
+// ops/conv.ts:236-250
+function conv2dGrads(dy, x4D, filter, strides, pad, dilations) {
+  if (dilations == null) dilations = [1, 1];
+  util.assert(conv_util.tupleValuesAreOne(dilations),
+              () => 'Error in gradient of conv2D: dilation rates greater than 1 ' +
+                  `are not yet supported in gradients. Got dilations '${dilations}'`);
+  return {
+    x: () => conv2dDerInput(x4D.shape, dy, filter, strides, pad, 'NHWC'),
+    $filter: () => conv2dDerFilter(x4D, dy, filter.shape, strides, pad, 'NHWC')
+  };
+}
 
 const fusedConv2d = op('fusedConv2d', (config) => {
   const activation = config.activation || 'linear';
@@ -231,16 +292,41 @@ const fusedConv2d = op('fusedConv2d', (config) => {
   if (config.preluActivationWeights != null) {
     $prelu = convertToTensor(config.preluActivationWeights, 'prelu weights', 'fused conv2d');
   }
+  const inputs = {x: x4D, $filter};
+  if ($bias != null) inputs.$bias = $bias;
+  if ($prelu != null) inputs.$prelu = $prelu;
   const res = ENGINE.runKernel(
-      backend => backend.fusedConv2d(x4D, $filter, convInfo, $bias, activation, $prelu),
-      {x: x4D, $filter});
+      (backend, save) => {
+        const y = backend.fusedConv2d(x4D, $filter, convInfo, $bias, activation, $prelu);
+        save([$filter, x4D, y]);
+        return y;
+      },
+      inputs,
+      (dy, saved) => {  // fused_ops.ts:361-400
+        const dyAct = fusedDyActivation(dy, saved[2], activation);
+        const g = conv2dGrads(dyAct, saved[1], saved[0], config.strides, config.pad, config.dilations);
+        if ($bias != null) g.$bias = () => unbroadcast(dyAct, $bias.shape);
+        return g;
+      });
   return lower(res, reshapedTo4D);
 });
 
 const depthwiseConv2d = op('depthwiseConv2d', (x, filter, strides, pad, dataFormat, dilations, dimRoundingMode) => {
   const {x4D, $filter, convInfo, reshapedTo4D} = convPrep(
       x, filter, strides, pad, dataFormat, dilations, dimRoundingMode, 'depthwiseConv2d', true);
-  const res = ENGINE.runKernel(backend => backend.depthwiseConv2D(x4D, $filter, convInfo), {x: x4D, $filter});
+  const res = ENGINE.runKernel((backend, save) => {
+    save([x4D, $filter]);
+    return backend.depthwiseConv2D(x4D, $filter, convInfo);
+  }, {x: x4D, $filter}, (dy, saved) => {  // ops/conv.ts:520-540
+    const dil = dilations == null ? [1, 1] : dilations;
+    util.assert(conv_util.tupleValuesAreOne(dil),
+                () => 'Error in gradient of depthwiseConv2d: dilation rates greater than ' +
+                    `1 are not yet supported. Got dilations '${dil}'`);
+    return {
+      x: () => depthwiseConv2dDerInput(saved[0].shape, dy, saved[1], strides, pad, dil, dimRoundingMode),
+      $filter: () => depthwiseConv2dDerFilter(saved[0], dy, saved[1].shape, strides, pad, dil, dimRoundingMode)
+    };
+  });
   return lower(res, reshapedTo4D);
 });
 
@@ -297,8 +383,13 @@ function poolImpl(x, filterSize, strides, dilations, pad, dimRoundingMode, kind)
         `dimRoundingMode ${dimRoundingMode} but got pad ${pad}.`);
   }
   const convInfo = conv_util.computePool2DInfo(x4D.shape, filterSize, strides, dilations, pad, dimRoundingMode);
-  let res = ENGINE.runKernel(
-      backend => kind === 'avg' ? backend.avgPool(x4D, convInfo) : backend.maxPool(x4D, convInfo), {x: x4D});
+  let res = ENGINE.runKernel((backend, save) => {
+    save([x4D]);
+    return kind === 'avg' ? backend.avgPool(x4D, convInfo) : backend.maxPool(x4D, convInfo);
+  }, {x: x4D}, (dy, saved) => ({  // ops/pool.ts:80-90, 180-185
+    x: () => kind === 'avg' ? avgPoolBackprop(dy, saved[0], filterSize, strides, pad, dilations)
+                            : maxPoolBackprop(dy, saved[0], filterSize, strides, pad, dilations)
+  }));
   if (kind === 'avg') res = cast(res, $x.dtype);  // ops/pool.ts:197
   return lower(res, reshapedTo4D);
 }
@@ -348,7 +439,13 @@ const conv2dDerInput = op('conv2dDerInput', (xShape, dy, filter, strides, pad, d
   util.assert(sameShape(convInfo.outShape, dy4D.shape),
               () => `Error in conv2dDerInput: dy has shape ${dy4D.shape}, the convolution of an ` +
                   `input of shape ${xShape4D} gives ${convInfo.outShape}`);
-  const res = ENGINE.runKernel(backend => backend.conv2dDerInput(dy4D, $filter, convInfo), {dy4D, $filter});
+  const res = ENGINE.runKernel((backend, save) => {
+    save([$filter, dy4D]);
+    return backend.conv2dDerInput(dy4D, $filter, convInfo);
+  }, {dy4D, $filter}, (ddx, saved) => ({  // ops/conv.ts:299-311
+    dy4D: () => conv2d(ddx, saved[0], strides, pad, 'NHWC', 1, dimRoundingMode),
+    $filter: () => conv2dDerFilter(ddx, saved[1], saved[0].shape, strides, pad, 'NHWC', dimRoundingMode)
+  }));
   return lower(res, reshapedTo4D);
 });
 const conv2dDerFilter = op('conv2dDerFilter', (x, dy, filterShape, strides, pad, dataFormat, dimRoundingMode) => {
@@ -435,13 +532,31 @@ const avgPoolBackprop = op('avgPoolBackprop', (dy, input, filterSize, strides, p
     poolBackprop('avgPoolBackprop', dy, input, filterSize, strides, dilations, pad, null, 'avg'));
 
 // ---- elementwise ------------------------------------------------------------------------
+// Gradients of the broadcasting arithmetic ops (binary_ops.ts:76-96, 253-279, 406-437, 530-556);
+// maximum / minimum record no gradient function, so a backward pass through them throws.
+const BINARY_GRADS = {
+  add: (dy, a, b) => ({$a: () => unbroadcast(dy, a.shape), $b: () => unbroadcast(dy, b.shape)}),
+  sub: (dy, a, b) => ({$a: () => unbroadcast(dy, a.shape), $b: () => unbroadcast(neg(dy), b.shape)}),
+  mul: (dy, a, b) => ({
+    $a: () => unbroadcast(mul(dy, cast(b, 'float32')), a.shape),
+    $b: () => unbroadcast(mul(dy, cast(a, 'float32')), b.shape)
+  }),
+  div: (dy, a, b) => ({
+    $a: () => unbroadcast(div(dy, cast(b, 'float32')), a.shape),
+    $b: () => neg(div(unbroadcast(mul(dy, cast(a, 'float32')), b.shape), cast(square(b), 'float32')))
+  })
+};
 function binaryOp(name, method) {
   return op(name, (a, b) => {
     let $a = convertToTensor(a, 'a', name);
     let $b = convertToTensor(b, 'b', name);
     [$a, $b] = makeTypesMatch($a, $b);
     broadcast_util.assertAndGetBroadcastShape($a.shape, $b.shape);
-    return ENGINE.runKernel(backend => backend[method]($a, $b), {$a, $b});
+    const g = BINARY_GRADS[name];
+    return ENGINE.runKernel((backend, save) => {
+      save([$a, $b]);
+      return backend[method]($a, $b);
+    }, {$a, $b}, g == null ? null : (dy, saved) => g(dy, saved[0], saved[1]));
   });
 }
 const add = binaryOp('add', 'add');
@@ -457,10 +572,26 @@ const prelu = op('prelu', (x, alpha) => {
   return ENGINE.runKernel(backend => backend.prelu($x, $alpha), {$x, $alpha});
 });
 
+// Gradients of the unary ops (unary_ops.ts, relu_ops.ts); x and y are the saved input and result.
+const UNARY_GRADS = {
+  relu: (dy, x) => mul(dy, stepOf(x)),
+  exp: (dy, x, y) => mul(dy, y),
+  log: (dy, x) => div(dy, cast(x, 'float32')),
+  neg: dy => neg(dy),
+  square: (dy, x) => mul(dy, mul(cast(x, 'float32'), scalar(2))),
+  sqrt: (dy, x) => div(dy, mul(sqrt(cast(x, 'float32')), scalar(2))),
+  sigmoid: (dy, x, y) => mul(dy, mul(y, sub(scalar(1), y))),
+  tanh: (dy, x, y) => mul(sub(scalar(1), square(y)), dy)
+};
 function unaryOp(name, method) {
   return op(name, x => {
     const $x = convertToTensor(x, 'x', name);
-    return ENGINE.runKernel(backend => backend[method || name]($x), {$x});
+    const g = UNARY_GRADS[name];
+    return ENGINE.runKernel((backend, save) => {
+      const y = backend[method || name]($x);
+      save([$x, y]);
+      return y;
+    }, {$x}, g == null ? null : (dy, saved) => ({$x: () => g(dy, saved[0], saved[1])}));
   });
 }
 const relu = unaryOp('relu');
@@ -478,7 +609,13 @@ const clipByValue = op('clipByValue', (x, clipValueMin, clipValueMax) => {
   const $x = convertToTensor(x, 'x', 'clipByValue');
   util.assert(clipValueMin <= clipValueMax,
               () => `Error in clip: min (${clipValueMin}) must be less than or equal to max (${clipValueMax}).`);
-  return ENGINE.runKernel(backend => backend.clip($x, clipValueMin, clipValueMax), {$x});
+  return ENGINE.runKernel((backend, save) => {
+    save([$x]);
+    return backend.clip($x, clipValueMin, clipValueMax);
+  }, {$x}, (dy, saved) => ({  // unary_ops.ts:584-592: dy where min <= x <= max, else 0
+    $x: () => mul(dy, cast(logicalAnd(greaterEqual(saved[0], scalar(clipValueMin)),
+                                      lessEqual(saved[0], scalar(clipValueMax))), 'float32'))
+  }));
 });
 const relu6 = op('relu6', x => clipByValue(x, 0, 6));
 
@@ -495,7 +632,19 @@ function reduceOp(name, method) {
       reduceInput = transpose($x, permutedAxes);
       axes = axis_util.getInnerMostAxes(axes.length, $x.rank);
     }
-    const res = ENGINE.runKernel(backend => backend[method](reduceInput, axes), {$x: reduceInput});
+    // dy (and y) stretched back over the reduced axes, which are the innermost ones here
+    const expand = t => reshape(t, reduceInput.shape.map((d, i) => axes.indexOf(i) === -1 ? d : 1));
+    const res = ENGINE.runKernel((backend, save) => {
+      const y = backend[method](reduceInput, axes);
+      save([reduceInput, y]);
+      return y;
+    }, {$x: reduceInput}, (dy, saved) => ({
+      // reduction_ops.ts:163-172 (sum: dy spread over the axes), :41-52 (max / min: dy where
+      // the element equals the extremum)
+      $x: () => name === 'sum' ?
+          mul(expand(dy), ones(saved[0].shape, 'float32')) :
+          mul(expand(dy), cast(equal(saved[0], expand(saved[1])), 'float32'))
+    }));
     if (keepDims) {
       return reshape(res, axis_util.expandShapeToKeepDim(res.shape, origAxes));
     }
@@ -548,7 +697,16 @@ const softmax = op('softmax', (logits, dim) => {
   }
   if (typeof ENGINE.backend.softmax === 'function') {
     const lf = cast($logits, 'float32');
-    return ENGINE.runKernel(backend => backend.softmax(lf, dim), {logits: lf});
+    return ENGINE.runKernel((backend, save) => {
+      const y = backend.softmax(lf, dim);
+      save([y]);
+      return y;
+    }, {logits: lf}, (dy, saved) => ({  // ops/softmax.ts:64-72
+      logits: () => {
+        const dyTimesY = mul(dy, saved[0]);
+        return sub(dyTimesY, mul(sum(dyTimesY, [dim], true), saved[0]));
+      }
+    }));
   }
   const lse = logSumExp($logits, [dim], true);
   return exp(sub(cast($logits, 'float32'), lse));
@@ -576,7 +734,8 @@ const transpose = op('transpose', (x, perm) => {
                 () => `All entries in 'perm' must be between 0 and ${$x.rank - 1} but got ${perm}`);
   });
   if ($x.rank <= 1) return clone($x);
-  return ENGINE.runKernel(backend => backend.transpose($x, perm), {$x});
+  return ENGINE.runKernel(backend => backend.transpose($x, perm), {$x},
+                          dy => ({$x: () => transpose(dy, axis_util.getUndoAxesPermutation(perm))}));
 });
 
 // ---- slice / stridedSlice / reverse (ops/slice.ts, ops/slice_util.ts, ops/strided_slice.ts,

@@ -279,6 +279,122 @@ test('op wrappers validate before touching the backend', async () => {
   });
 });
 
+// Enough kernels in plain JavaScript (same-shape or scalar operands) to drive the tape.
+class ArithBackend extends StorageBackend {
+  make(shape, values, dtype) {
+    return Tensor.make(shape, {values}, dtype || 'float32', this);
+  }
+  zip(a, b, f) {
+    const av = this.readSync(a.dataId), bv = this.readSync(b.dataId);
+    const big = a.size >= b.size ? a : b;
+    const out = new Float32Array(big.size);
+    for (let i = 0; i < big.size; i++) out[i] = f(av[a.size === 1 ? 0 : i], bv[b.size === 1 ? 0 : i]);
+    return this.make(big.shape, out);
+  }
+  map(x, f) { return this.make(x.shape, Float32Array.from(this.readSync(x.dataId), f)); }
+  add(a, b) { return this.zip(a, b, (p, q) => p + q); }
+  subtract(a, b) { return this.zip(a, b, (p, q) => p - q); }
+  multiply(a, b) { return this.zip(a, b, (p, q) => p * q); }
+  realDivide(a, b) { return this.zip(a, b, (p, q) => p / q); }
+  neg(x) { return this.map(x, v => -v); }
+  square(x) { return this.map(x, v => v * v); }
+  exp(x) { return this.map(x, v => Math.exp(v)); }
+  relu(x) { return this.map(x, v => Math.max(0, v)); }
+  greater(a, b) {
+    const r = this.zip(a, b, (p, q) => p > q ? 1 : 0);
+    return Tensor.make(r.shape, {dataId: r.dataId}, 'bool', this);
+  }
+  cast(x, dtype) {
+    if (dtype === 'float32' && x.dtype === 'bool') return this.map(x, v => v);
+    return Tensor.make(x.shape, {dataId: x.dataId}, dtype, this);
+  }
+  fill(shape, value, dtype) {
+    return this.make(shape, new Float32Array(shape.reduce((a, b) => a * b, 1)).fill(value), dtype);
+  }
+  sum(x, axes) {
+    util.assert(axes.length === x.rank, 'ArithBackend.sum reduces every axis');
+    return this.make([], Float32Array.of(Array.from(this.readSync(x.dataId)).reduce((a, b) => a + b, 0)));
+  }
+}
+
+function closeTo(actual, expected, eps) {
+  assert.strictEqual(actual.length, expected.length);
+  for (let i = 0; i < expected.length; i++) {
+    assert.ok(Math.abs(actual[i] - expected[i]) <= (eps || 1e-5), `${Array.from(actual)} vs ${expected}`);
+  }
+}
+
+test('tape: grad, grads, twice, second order (gradients_test.ts:61-112, 291-316)', async () => {
+  await withBackend('arith-grad', new ArithBackend(), async () => {
+    const grad = tf.grad(x => tf.square(x));
+    closeTo(grad(tf.tensor1d([.1, .2])).dataSync(), [.2, .4]);
+    closeTo(grad(tf.tensor1d([.1, .4])).dataSync(), [.2, .8]);
+    closeTo(tf.grads(x => tf.square(x))([tf.tensor1d([.1, .2])])[0].dataSync(), [.2, .4]);
+    // dy scales the result; its shape must match f(x)
+    closeTo(grad(tf.tensor1d([1, 2]), tf.tensor1d([10, 100])).dataSync(), [20, 400]);
+    assert.throws(() => grad(tf.tensor1d([1, 2]), tf.tensor1d([1, 2, 3])));   // dy of another shape
+    assert.strictEqual(tf.engine().isTapeOn(), false);
+    const x = tf.tensor1d([.1, .2]);
+    const before = tf.memory().numTensors;
+    const gg = tf.grad(tf.grad(t => tf.mul(tf.mul(t, t), t)))(x);
+    assert.strictEqual(tf.memory().numTensors, before + 1);   // nothing but the result survives
+    closeTo(gg.dataSync(), [.6, 1.2]);
+    closeTo(tf.grad(tf.grad(t => tf.square(t)))(tf.scalar(3)).dataSync(), [2]);
+    const g3 = tf.grads(t => tf.mul(tf.mul(t, t), t));
+    closeTo(tf.grads(t => g3([t])[0])([tf.tensor1d([.1, .2])])[0].dataSync(), [.6, 1.2]);
+    // two arguments, a shared subexpression, accumulation over two uses of a
+    const [da, db] = tf.grads((a, b) => tf.add(tf.mul(a, b), tf.square(a)))([tf.scalar(3), tf.scalar(5)]);
+    closeTo(da.dataSync(), [5 + 6]);
+    closeTo(db.dataSync(), [3]);
+    const r = tf.valueAndGrad(t => tf.exp(t))(tf.scalar(0));
+    closeTo(r.value.dataSync(), [1]);
+    closeTo(r.grad.dataSync(), [1]);
+  });
+});
+
+test('tape: errors leave no tape behind, pruned ops need no gradient (gradients_test.ts:76-161)', async () => {
+  await withBackend('arith-grad2', new ArithBackend(), async () => {
+    const e = tf.engine();
+    assert.throws(() => tf.grad(() => { throw new Error('failed forward pass'); })(tf.zeros([])));
+    assert.strictEqual(e.isTapeOn(), false);
+    const bad = tf.customGrad(x => ({value: x, gradFunc: () => { throw new Error('failed backward pass'); }}));
+    assert.throws(() => tf.grad(x => bad(x))(tf.zeros([])), /failed backward pass/);
+    assert.strictEqual(e.isTapeOn(), false);
+    assert.strictEqual(e.state.activeTape, null);
+    // y does not depend on x
+    assert.throws(() => tf.grad(x => tf.scalar(2))(tf.scalar(1)), /Cannot compute gradient of y=f\(x\)/);
+    // an op without a gradient function off the x -> y path is fine, on it it is an error
+    const noGrad = t => e.runKernel(b => b.neg(t), {t});
+    closeTo(tf.grad(x => { noGrad(tf.scalar(7)); return tf.square(x); })(tf.scalar(2)).dataSync(), [4]);
+    assert.throws(() => tf.grad(x => noGrad(x))(tf.scalar(2)), /gradient function not found/);
+  });
+});
+
+test('tape: customGrad value / gradFunc / save, no leaks (gradients_test.ts:192-211, 317-370)', async () => {
+  await withBackend('arith-grad3', new ArithBackend(), async () => {
+    const a = tf.scalar(3), dy = tf.scalar(4);
+    const customSquare = tf.customGrad(t => ({value: tf.square(t), gradFunc: d => tf.mul(d, tf.scalar(0.1))}));
+    const {value, grad} = tf.valueAndGrad(t => customSquare(t))(a, dy);
+    closeTo(value.dataSync(), [9]);
+    closeTo(grad.dataSync(), [.4]);
+    // saved tensors reach gradFunc and are released afterwards
+    const before = tf.memory().numTensors;
+    const withSave = tf.customGrad((t, save) => {
+      save([t]);
+      return {value: tf.square(t), gradFunc: (d, saved) => tf.mul(d, tf.mul(saved[0], tf.scalar(2)))};
+    });
+    const g = tf.grad(t => withSave(t))(a);
+    closeTo(g.dataSync(), [6]);
+    assert.strictEqual(tf.memory().numTensors, before + 1);
+    g.dispose();
+    // outside a gradient nothing is saved
+    const y = withSave(a);
+    assert.strictEqual(tf.memory().numTensors, before + 1);
+    y.dispose();
+    assert.throws(() => tf.customGrad(t => ({value: 3, gradFunc: d => d}))(a), /`obj.value` is a tensor/);
+  });
+});
+
 test('flags: lazy evaluation, set hook, unknown flag', () => {
   const env = tf.ENV;
   assert.strictEqual(env.getBool('DEBUG'), false);

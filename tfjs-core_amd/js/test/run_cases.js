@@ -74,6 +74,62 @@ const OPS = {
   depthwiseConv2dDerFilter: (i, a) => tf.depthwiseConv2dDerFilter(i.x, i.dy, a.filterShape, a.strides, a.pad),
   maxPoolBackprop: (i, a) => tf.maxPoolBackprop(i.dy, i.x, a.filterSize, a.strides, a.pad, a.dilations),
   avgPoolBackprop: (i, a) => tf.avgPoolBackprop(i.dy, i.x, a.filterSize, a.strides, a.pad, a.dilations),
+  // gradients through the tape (tf.grad / tf.grads); `wrt` picks the argument
+  gradConv2d: (i, a) => tf.grads((x, f) => tf.conv2d(x.clone(), f.clone(), a.strides, a.pad).clone())(
+      [i.x, i.filter], i.dy)[a.wrt],
+  gradConv2dTranspose: (i, a) => tf.grads((x, f) => tf.conv2dTranspose(x, f, a.outputShape, a.strides, a.pad))(
+      [i.x, i.filter], i.dy)[a.wrt],
+  gradDepthwise: (i, a) => tf.grads((x, f) => {
+    const y = tf.depthwiseConv2d(x, f, a.strides, a.pad);
+    return a.squared ? tf.square(y) : y;
+  })([i.x, i.filter])[a.wrt],
+  gradPool: (i, a) => tf.grad(x => a.kind === 'max' ? tf.maxPool(x, a.filterSize, a.strides, a.pad)
+                                                    : tf.avgPool(x, a.filterSize, a.strides, a.pad))(i.x, i.dy),
+  // loss = sum((relu(x w1 + b1) w2 - t)^2): d loss / d (w1 | b1 | w2)
+  gradMlp: (i, a) => tf.grads((w1, b1, w2) => {
+    const h = tf.relu(tf.add(tf.matMul(i.x, w1), b1));
+    return tf.sum(tf.square(tf.sub(tf.matMul(h, w2), i.t)));
+  })([i.w1, i.b1, i.w2])[a.wrt],
+  gradFusedMlp: (i, a) => tf.grads((w1, b1, w2) => {
+    const h = tf.fused.matMul({a: i.x, b: w1, bias: b1, activation: 'relu'});
+    return tf.sum(tf.square(tf.sub(tf.matMul(h, w2), i.t)));
+  })([i.w1, i.b1, i.w2])[a.wrt],
+  // loss = -sum(labels * log(softmax(logits)))
+  gradSoftmaxXent: i => tf.grad(l => tf.neg(tf.sum(tf.mul(i.labels, tf.log(tf.softmax(l))))))(i.logits),
+  // a small conv net: conv(3x3, bias, relu) -> maxPool 2 -> depthwise 3x3 -> avgPool -> dense -> sum of squares
+  gradConvNet: (i, a) => tf.grads((cw, cb, dw, fw) => {
+    let h = tf.relu(tf.add(tf.conv2d(i.x, cw, 1, 'same'), cb));
+    h = tf.maxPool(h, 2, 2, 'valid');
+    h = tf.depthwiseConv2d(h, dw, 1, 'same');
+    h = tf.avgPool(h, 2, 2, 'valid');
+    const flat = tf.reshape(h, [h.shape[0], h.shape[1] * h.shape[2] * h.shape[3]]);
+    return tf.sum(tf.square(tf.sub(tf.matMul(flat, fw), i.t)));
+  })([i.cw, i.cb, i.dw, i.fw])[a.wrt],
+  // one SGD step on the same net, repeated: the loss after `steps` updates
+  trainConvNet: (i, a) => {
+    const lossOf = (cw, cb, dw, fw) => {
+      let h = tf.relu(tf.add(tf.conv2d(i.x, cw, 1, 'same'), cb));
+      h = tf.maxPool(h, 2, 2, 'valid');
+      h = tf.depthwiseConv2d(h, dw, 1, 'same');
+      h = tf.avgPool(h, 2, 2, 'valid');
+      const flat = tf.reshape(h, [h.shape[0], h.shape[1] * h.shape[2] * h.shape[3]]);
+      return tf.div(tf.sum(tf.square(tf.sub(tf.matMul(flat, fw), i.t))), tf.scalar(i.t.size));
+    };
+    let params = [i.cw, i.cb, i.dw, i.fw];
+    const losses = [];
+    for (let s = 0; s < a.steps; s++) {
+      const next = tf.tidy(() => {
+        const {value, grads} = tf.valueAndGrads(lossOf)(params);
+        losses.push(value.dataSync()[0]);
+        return params.map((p, k) => tf.sub(p, tf.mul(grads[k], tf.scalar(a.lr))));
+      });
+      if (s > 0) tf.dispose(params);
+      params = next;
+    }
+    const out = tf.tensor(new Float32Array(losses), [losses.length]);
+    tf.dispose(params);
+    return out;
+  },
 };
 
 async function main() {
