@@ -277,6 +277,9 @@ def main():
     ap.add_argument("--no-ops", action="store_true",
                     help="skip the op-level configs (single matMul, MLP layers, conv2d, depthwise)")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
+    ap.add_argument("--loop-pointwise", type=int, default=0, metavar="REPS",
+                    help="only launch the 512->512 pointwise layer of the network (pw7: "
+                         "[64,14,14,512] x [512,512], bias + relu6) REPS times, for counter runs")
     ap.add_argument("--calibrate-counters", action="store_true",
                     help="only launch a streaming kernel of known size (relu over 256 MiB: reads "
                          "256 MiB, writes 256 MiB) three times, to scale FETCH_SIZE / WRITE_SIZE")
@@ -298,6 +301,19 @@ def main():
         be.sync()
         print(json.dumps({"calibration_kernel": "unary_f32_vec_kernel (relu)",
                           "bytes_read": big.size * 4, "bytes_written": big.size * 4}))
+        return
+
+    if args.loop_pointwise > 0:
+        rng = np.random.default_rng(1)
+        x = tf.tensor(rng.uniform(0, 1, (args.batch, 14, 14, 512)).astype(np.float32))
+        wt = tf.tensor((rng.standard_normal((1, 1, 512, 512)) * 0.05).astype(np.float32))
+        bias = tf.tensor(np.zeros(512, np.float32))
+        for _ in range(args.loop_pointwise):
+            tf.dispose(tf.fused.conv2d(x, wt, 1, "same", bias=bias, activation="relu6"))
+        be.sync()
+        print(json.dumps({"kernel": be.lib.tfhip_last_kernel(be.ctx).decode(),
+                          "launches": args.loop_pointwise,
+                          "flops_per_launch": 2.0 * args.batch * 196 * 512 * 512}))
         return
 
     params = mobilenet.make_params(seed=0)
