@@ -235,6 +235,9 @@ def test_backward_kernel_variants(tf):
     xd, wd, dyd = tf.tensor(f(2, 16, 16, 8)), tf.tensor(f(3, 3, 8, 1)), tf.tensor(f(2, 16, 16, 8))
     run("dw_der_input", lambda: tf.depthwise_conv2d_der_input((2, 16, 16, 8), dyd, wd, 1, "same"))
     run("dw_der_filter", lambda: tf.depthwise_conv2d_der_filter(xd, dyd, (3, 3, 8, 1), 1, "same"))
+    dys2 = tf.tensor(f(2, 8, 8, 8))
+    run("dw_der_input_s2", lambda: tf.depthwise_conv2d_der_input((2, 16, 16, 8), dys2, wd, 2, "same"))
+    dys2.dispose()
     wm, dym = tf.tensor(f(3, 3, 8, 2)), tf.tensor(f(2, 16, 16, 16))
     run("dw_der_input_mul2", lambda: tf.depthwise_conv2d_der_input((2, 16, 16, 8), dym, wm, 1, "same"))
     run("dw_der_filter_mul2", lambda: tf.depthwise_conv2d_der_filter(xd, dym, (3, 3, 8, 2), 1, "same"))
@@ -244,7 +247,8 @@ def test_backward_kernel_variants(tf):
     assert "rowmajor_f32" in seen["der_input_1x1"], seen
     assert seen["der_input_c3"].endswith("im2col_up_f32_unaligned") or "_unaligned" in seen["der_input_c3"], seen
     assert "im2col_t" in seen["der_filter_c3"] and "_unaligned" in seen["der_filter_c3"], seen
-    assert seen["dw_der_input"] == "depthwise_der_input_vec_s1", seen
+    assert seen["dw_der_input"].startswith("depthwise3x3_s1") and seen["dw_der_input"].endswith("_as_der_input"), seen
+    assert seen["dw_der_input_s2"] == "depthwise_der_input_vec_s2", seen
     assert seen["dw_der_filter"] == "depthwise3x3_der_filter", seen
     assert seen["dw_der_input_mul2"] == "depthwise_der_input", seen
     assert seen["dw_der_filter_mul2"] == "depthwise_der_filter", seen

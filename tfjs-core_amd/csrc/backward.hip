@@ -8,6 +8,8 @@
 // respect to the depthwise filter is a reduction over every output pixel: lanes run along
 // the channels, workgroups split the pixels, and a second kernel adds the partial sums in a
 // fixed order, so the result does not depend on scheduling.
+#include <cstring>
+
 #include "tfhip_internal.h"
 
 namespace tfhip {
@@ -95,6 +97,15 @@ __global__ void depthwise_der_filter_finish_kernel(const double* partial, float*
 }
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// out[kh][kw][c] = w[KH - 1 - kh][KW - 1 - kw][c] (channel multiplier 1).
+__global__ void flip_depthwise_filter_kernel(const float* w, float* out, int KH, int KW, int C) {
+  const int g = blockIdx.x * blockDim.x + threadIdx.x;
+  if (g >= KH * KW * C) return;
+  const int c = g % C, t = g / C;
+  const int kw = t % KW, kh = t / KW;
+  out[g] = w[((KH - 1 - kh) * KW + (KW - 1 - kw)) * C + c];
+}
 
 // Fast variants for channel multiplier 1, C % 4 == 0 and 16-byte aligned buffers: a lane owns
 // 4 consecutive channels (16-byte accesses) and sums in float in the same tap order.
@@ -267,6 +278,70 @@ __global__ void pool2d_backprop_kernel(const float* dy, const float* x, float* d
   }
 }
 
+// The same with a lane owning 4 consecutive channels (C % 4 == 0, 16-byte aligned buffers):
+// the window scan and the dy gather are 16-byte accesses, the winner is tracked per channel.
+__global__ __launch_bounds__(256) void pool2d_backprop_vec_kernel(
+    const float* __restrict__ dy, const float* __restrict__ x, float* __restrict__ dx,
+    const tfhip_conv2d_info ci, int kind) {
+  const int eff_h = ci.filter_h + (ci.filter_h - 1) * (ci.dilation_h - 1);
+  const int eff_w = ci.filter_w + (ci.filter_w - 1) * (ci.dilation_w - 1);
+  const int pad_top = eff_h - 1 - ci.pad_top, pad_left = eff_w - 1 - ci.pad_left;
+  const int c4 = ci.in_c / 4;
+  const int64_t total = (int64_t)ci.batch * ci.in_h * ci.in_w * c4;
+  const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (g >= total) return;
+  const int cq = (int)(g % c4);
+  int64_t t = g / c4;
+  const int xc = (int)(t % ci.in_w);
+  t /= ci.in_w;
+  const int xr = (int)(t % ci.in_h);
+  const int n = (int)(t / ci.in_h);
+  const float* xn = x + (int64_t)n * ci.in_h * ci.in_w * ci.in_c + cq * 4;
+  const float* dyn = dy + (int64_t)n * ci.out_h * ci.out_w * ci.out_c + cq * 4;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int wr = 0; wr < eff_h; wr += ci.dilation_h) {
+    const int num_r = xr - pad_top + wr;
+    const int yr = num_r / ci.stride_h;
+    if (num_r < 0 || yr * ci.stride_h != num_r || yr >= ci.out_h) continue;
+    for (int wc = 0; wc < eff_w; wc += ci.dilation_w) {
+      const int num_c = xc - pad_left + wc;
+      const int yc = num_c / ci.stride_w;
+      if (num_c < 0 || yc * ci.stride_w != num_c || yc >= ci.out_w) continue;
+      const f32x4 d = *reinterpret_cast<const f32x4*>(dyn + ((int64_t)yr * ci.out_w + yc) * ci.out_c);
+      if (kind != TFHIP_POOL_MAX) {
+        acc += d;
+        continue;
+      }
+      // first strict maximum of window (yr, yc), per channel; this pixel sits at the
+      // flipped position (eff_h - 1 - wr, eff_w - 1 - wc) of that window
+      const int xr0 = yr * ci.stride_h - ci.pad_top, xc0 = yc * ci.stride_w - ci.pad_left;
+      f32x4 best = {-__builtin_inff(), -__builtin_inff(), -__builtin_inff(), -__builtin_inff()};
+      int pos[4] = {-1, -1, -1, -1};
+      for (int fr = 0; fr < eff_h; fr += ci.dilation_h) {
+        const int r = xr0 + fr;
+        if ((unsigned)r >= (unsigned)ci.in_h) continue;
+        for (int fc = 0; fc < eff_w; fc += ci.dilation_w) {
+          const int c = xc0 + fc;
+          if ((unsigned)c >= (unsigned)ci.in_w) continue;
+          const f32x4 v = *reinterpret_cast<const f32x4*>(xn + ((int64_t)r * ci.in_w + c) * ci.in_c);
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+            if (v[e] > best[e]) {
+              best[e] = v[e];
+              pos[e] = fr * eff_w + fc;
+            }
+        }
+      }
+      const int mine = (eff_h - 1 - wr) * eff_w + (eff_w - 1 - wc);
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        if (pos[e] == mine) acc[e] += d[e];
+    }
+  }
+  if (kind != TFHIP_POOL_MAX) acc *= 1.0f / (float)(ci.filter_h * ci.filter_w);
+  *reinterpret_cast<f32x4*>(dx + g * 4) = acc;
+}
+
 static int check_geometry(tfhip_ctx* ctx, const char* op, const tfhip_conv2d_info* ci,
                           bool dilation_allowed) {
   if (ci->batch < 0 || ci->in_h < 0 || ci->in_w < 0 || ci->in_c < 0 || ci->out_h < 0 ||
@@ -314,6 +389,26 @@ extern "C" int tfhip_depthwise_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int6
   if ((rc = as_f32(ctx, bdy, &tdy, &dyf))) return rc;
   if ((rc = as_f32(ctx, bw, &tw, &wf))) return rc;
   float* dxf = static_cast<float*>(bdx->ptr);
+  if (ch_mul == 1 && ci->stride_h == 1 && ci->stride_w == 1 && y_n > 0) {
+    // stride 1: dx is the depthwise convolution of dy with the filter flipped in both spatial
+    // directions and the padding filter - 1 - pad: the forward kernels do it at their speed
+    Temp tflip(ctx);
+    if (!tflip.get((size_t)w_n * sizeof(float))) return TFHIP_EDEVICE;
+    hipLaunchKernelGGL(flip_depthwise_filter_kernel, dim3((unsigned)ceil_div(w_n, 256)), dim3(256), 0,
+                       ctx->stream, wf, static_cast<float*>(tflip.ptr), ci->filter_h, ci->filter_w,
+                       ci->in_c);
+    TFHIP_LAUNCH_CHECK(ctx);
+    tfhip_conv2d_info back = *ci;
+    back.in_h = ci->out_h; back.in_w = ci->out_w;
+    back.out_h = ci->in_h; back.out_w = ci->in_w;
+    back.out_c = ci->in_c;
+    back.pad_top = ci->filter_h - 1 - ci->pad_top;
+    back.pad_left = ci->filter_w - 1 - ci->pad_left;
+    back.pad_bottom = back.pad_right = 0;   // (not read by the kernels)
+    if ((rc = depthwise_forward_f32(ctx, dyf, static_cast<const float*>(tflip.ptr), dxf, &back))) return rc;
+    strncat(ctx->last_kernel, "_as_der_input", sizeof ctx->last_kernel - strlen(ctx->last_kernel) - 1);
+    return TFHIP_OK;
+  }
   if (ch_mul == 1 && ci->in_c % 4 == 0 && aligned16(dyf) && aligned16(wf) && aligned16(dxf)) {
     const unsigned blocks = (unsigned)ceil_div(x_n / 4, 256);
     const int s = ci->stride_h == ci->stride_w && ci->stride_h <= 2 ? ci->stride_h : 0;
@@ -430,6 +525,15 @@ extern "C" int tfhip_pool2d_backprop(tfhip_ctx* ctx, int64_t dy, int64_t x, int6
   const float *dyf, *xf;
   if ((rc = as_f32(ctx, bdy, &tdy, &dyf))) return rc;
   if ((rc = as_f32(ctx, bx, &tx, &xf))) return rc;
+  float* dxf = static_cast<float*>(bdx->ptr);
+  if (ci->in_c % 4 == 0 && aligned16(dyf) && aligned16(xf) && aligned16(dxf)) {
+    snprintf(ctx->last_kernel, sizeof ctx->last_kernel,
+             kind == TFHIP_POOL_MAX ? "max_pool_backprop_vec" : "avg_pool_backprop_vec");
+    hipLaunchKernelGGL(pool2d_backprop_vec_kernel, dim3((unsigned)ceil_div(x_n / 4, 256)), dim3(256), 0,
+                       ctx->stream, dyf, xf, dxf, *ci, kind);
+    TFHIP_LAUNCH_CHECK(ctx);
+    return TFHIP_OK;
+  }
   snprintf(ctx->last_kernel, sizeof ctx->last_kernel,
            kind == TFHIP_POOL_MAX ? "max_pool_backprop" : "avg_pool_backprop");
   hipLaunchKernelGGL(pool2d_backprop_kernel, dim3(grid_for(ctx, x_n)), dim3(256), 0, ctx->stream, dyf,

@@ -409,6 +409,68 @@ static int check_geometry(tfhip_ctx* ctx, const char* op, const tfhip_conv2d_inf
   return TFHIP_OK;
 }
 
+// Picks and launches the kernel for a filled-in DwArgs (p.x, p.w, p.y, bias, act, quant set).
+static int dispatch_depthwise(tfhip_ctx* ctx, DwArgs& p, const tfhip_conv2d_info* ci, int ch_mul,
+                              int bias_kind, int64_t x_n, int64_t o_n) {
+  const bool fast = ci->filter_h == 3 && ci->filter_w == 3 && ci->dilation_h == 1 &&
+                    ci->dilation_w == 1 && ch_mul == 1 && ci->in_c % 4 == 0 &&
+                    ci->stride_h == ci->stride_w && (ci->stride_h == 1 || ci->stride_h == 2) &&
+                    aligned16(p.x) && aligned16(p.w) && aligned16(p.y) &&
+                    (bias_kind != TFHIP_BCAST_COLUMN || aligned16(p.bias));
+  if (fast) {
+    p.c4 = ci->in_c / 4;
+    // Stride 2 streams best with one output per lane (measured on MI355X, fp32, batch 32-64).
+    // Stride 1: the row-walking kernel when the image is large enough to give every SIMD a
+    // few wavefronts (it fetches each input row once), else 2x2 patches.  Measured on MI355X
+    // (fp32, batch 32-64): 28-row chunks stream best; halve them when that would leave a
+    // second, nearly empty round of wavefronts, or too few wavefronts.
+    int rows = 0;
+    if (ci->stride_h == 1 && x_n * 4 < (1ll << 31) && o_n * 4 < (1ll << 31)) {
+      const int64_t lanes_per_chunk = (int64_t)ci->batch * ceil_div(ci->out_w, 2) * p.c4;
+      const int64_t slots = (int64_t)ctx->num_cus * 12;  // 3 wavefronts per SIMD
+      auto waves = [&](int r) { return lanes_per_chunk * ceil_div(ci->out_h, r) / 64; };
+      rows = ci->out_h < 28 ? ci->out_h : 28;
+      while (rows > 7 && waves(rows) < slots / 2) rows = (rows + 1) / 2;
+      if (rows > 7 && waves(rows) > slots && waves(rows) * 2 < slots * 3) rows = (rows + 1) / 2;
+      if (waves(rows) < slots / 4) rows = 0;
+    }
+    if (rows > 0) {
+      launch_dw3x3_rows<2>(ctx, p, rows);
+    } else if (ci->stride_h == 1) {
+      if (ci->out_w >= 112 && ci->in_c >= 128 && ci->out_w % 8 == 0) launch_dw3x3<1, 2, 8>(ctx, p);
+      else launch_dw3x3<1, 2, 2>(ctx, p);
+    } else {
+      launch_dw3x3<2, 1, 1>(ctx, p);
+    }
+  } else {
+    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise_generic");
+    const int64_t blocks = ceil_div(o_n, 256);
+    const int64_t cap = (int64_t)ctx->num_cus * 16;
+    hipLaunchKernelGGL(depthwise_generic_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)),
+                       dim3(256), 0, ctx->stream, p);
+  }
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+// depthwiseConv2D of float32 device buffers without bias or activation: the forward kernels
+// reused by depthwiseConv2DDerInput (stride 1: dx is the depthwise convolution of dy with the
+// spatially flipped filter).
+int depthwise_forward_f32(tfhip_ctx* ctx, const float* x, const float* w, float* y,
+                          const tfhip_conv2d_info* ci) {
+  DwArgs p = {};
+  p.x = x;
+  p.w = w;
+  p.y = y;
+  p.ci = *ci;
+  p.ch_mul = ci->out_c / ci->in_c;
+  p.bias_kind = TFHIP_BCAST_NONE;
+  p.act = TFHIP_ACT_LINEAR;
+  return dispatch_depthwise(ctx, p, ci, p.ch_mul, TFHIP_BCAST_NONE,
+                            (int64_t)ci->batch * ci->in_h * ci->in_w * ci->in_c,
+                            (int64_t)ci->batch * ci->out_h * ci->out_w * ci->out_c);
+}
+
 }  // namespace tfhip
 
 using namespace tfhip;
@@ -467,46 +529,7 @@ extern "C" int tfhip_depthwise_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter,
   p.bias_kind = bias_kind;
   p.act = act;
 
-  const bool fast = ci->filter_h == 3 && ci->filter_w == 3 && ci->dilation_h == 1 &&
-                    ci->dilation_w == 1 && ch_mul == 1 && ci->in_c % 4 == 0 &&
-                    ci->stride_h == ci->stride_w && (ci->stride_h == 1 || ci->stride_h == 2) &&
-                    aligned16(p.x) && aligned16(p.w) && aligned16(p.y) &&
-                    (bias_kind != TFHIP_BCAST_COLUMN || aligned16(p.bias));
-  if (fast) {
-    p.c4 = ci->in_c / 4;
-    // Patch shapes picked by measurement on MI355X (fp32, batch 32-64): 2x8 patches for wide,
-    // deep rows, 2x2 elsewhere; stride 2 streams best with one output per lane.
-    // Stride 1: the row-walking kernel when the image is large enough to give every SIMD a
-    // few wavefronts (it fetches each input row once), else 2x2 patches.  Measured on MI355X
-    // (fp32, batch 32-64): 28-row chunks stream best; halve them when that would leave a
-    // second, nearly empty round of wavefronts, or too few wavefronts.
-    int rows = 0;
-    if (ci->stride_h == 1 && x_n * 4 < (1ll << 31) && o_n * 4 < (1ll << 31)) {
-      const int64_t lanes_per_chunk = (int64_t)ci->batch * ceil_div(ci->out_w, 2) * p.c4;
-      const int64_t slots = (int64_t)ctx->num_cus * 12;  // 3 wavefronts per SIMD
-      auto waves = [&](int r) { return lanes_per_chunk * ceil_div(ci->out_h, r) / 64; };
-      rows = ci->out_h < 28 ? ci->out_h : 28;
-      while (rows > 7 && waves(rows) < slots / 2) rows = (rows + 1) / 2;
-      if (rows > 7 && waves(rows) > slots && waves(rows) * 2 < slots * 3) rows = (rows + 1) / 2;
-      if (waves(rows) < slots / 4) rows = 0;
-    }
-    if (rows > 0) {
-      launch_dw3x3_rows<2>(ctx, p, rows);
-    } else if (ci->stride_h == 1) {
-      if (ci->out_w >= 112 && ci->in_c >= 128 && ci->out_w % 8 == 0) launch_dw3x3<1, 2, 8>(ctx, p);
-      else launch_dw3x3<1, 2, 2>(ctx, p);
-    } else {
-      launch_dw3x3<2, 1, 1>(ctx, p);
-    }
-  } else {
-    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise_generic");
-    const int64_t blocks = ceil_div(o_n, 256);
-    const int64_t cap = (int64_t)ctx->num_cus * 16;
-    hipLaunchKernelGGL(depthwise_generic_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)),
-                       dim3(256), 0, ctx->stream, p);
-  }
-  TFHIP_LAUNCH_CHECK(ctx);
-  return TFHIP_OK;
+  return dispatch_depthwise(ctx, p, ci, ch_mul, bias_kind, x_n, o_n);
 }
 
 extern "C" int tfhip_pool2d(tfhip_ctx* ctx, int64_t x, int64_t out, const tfhip_conv2d_info* ci,

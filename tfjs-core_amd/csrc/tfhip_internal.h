@@ -92,6 +92,10 @@ int as_f32(tfhip_ctx* ctx, const Buf* b, Temp* tmp, const float** out);
 int launch_convert(tfhip_ctx* ctx, const void* src, int src_dtype, void* dst, int dst_dtype,
                    int64_t n);
 
+// image.hip
+int depthwise_forward_f32(tfhip_ctx* ctx, const float* x, const float* w, float* y,
+                          const tfhip_conv2d_info* ci);
+
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its own
