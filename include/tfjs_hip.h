@@ -216,6 +216,17 @@ int tfhip_resize_bilinear(tfhip_ctx* ctx, int64_t x, int64_t out, int batch, int
 int tfhip_one_hot(tfhip_ctx* ctx, int64_t indices, int64_t out, int depth, float on_value,
                   float off_value);
 
+/* resizeNearestNeighbor (backend.ts:594-598; backend_cpu.ts:3016-3067): as resizeBilinear, the
+ * source pixel is floor(ratio * r), or Math.round(ratio * r) with align_corners. */
+int tfhip_resize_nearest(tfhip_ctx* ctx, int64_t x, int64_t out, int batch, int in_h, int in_w,
+                         int channels, int out_h, int out_w, int align_corners);
+/* select (backend.ts:236-238; backend_cpu.ts:822-845): out[i] = condition[i / inner] ? a[i] :
+ * b[i]; inner = 1 when the condition has the shape of a, = the size of a row of `a` when the
+ * condition is rank 1 over the first axis (ops/logical_ops.ts:140-156).  a, b, out share one
+ * storage dtype (the host upcasts, backend_cpu.ts:828). */
+int tfhip_select(tfhip_ctx* ctx, int64_t condition, int64_t a, int64_t b, int64_t out,
+                 int64_t inner);
+
 /* ---- backward kernels (training) ---------------------------------------------------------- */
 /* `info` is the Conv2DInfo of the FORWARD op in every call below (in_* = x, out_* = y).
  * conv2dDerInput (backend.ts:423-425; backend_cpu.ts:1686-1762): dy [batch,out_h,out_w,out_c],

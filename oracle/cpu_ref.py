@@ -687,3 +687,44 @@ def strided_slice_info(shape, begin, end, strides, begin_mask=0, end_mask=0,
             count = len(range(starts[axis], stops[axis], stride))
         sizes.append(count)
     return starts, sizes, shrink
+
+
+def resize_nearest_neighbor(x, new_height, new_width, align_corners):
+    """backends/cpu/backend_cpu.ts:3016-3067 (ratios and source coordinates in double,
+    Math.round = floor(v + 0.5) for the non-negative values met here)."""
+    x = _f32(x)
+    b, oh, ow, c = x.shape
+    eih = oh - 1 if (align_corners and new_height > 1) else oh
+    eiw = ow - 1 if (align_corners and new_width > 1) else ow
+    eoh = new_height - 1 if (align_corners and new_height > 1) else new_height
+    eow = new_width - 1 if (align_corners and new_width > 1) else new_width
+    rr, rc = eih / eoh, eiw / eow
+    pick = (lambda v: math.floor(v + 0.5)) if align_corners else math.floor
+    rows = [min(oh - 1, pick(rr * r)) for r in range(new_height)]
+    cols = [min(ow - 1, pick(rc * q)) for q in range(new_width)]
+    return x[:, rows][:, :, cols].copy()
+
+
+def select(condition, a, b):
+    """tf.where (ops/logical_ops.ts:129-175) as its tests state it: element-wise when the
+    condition has the shape of a, whole slices along the first axis when it is rank 1.
+    (backend_cpu.ts:822-845 reads a[i] / b[i] with the condition index for a rank-1
+    condition, which only its constant-row tests tolerate; the TensorFlow semantics are
+    restated here.)"""
+    a, b = np.asarray(a), np.asarray(b)
+    cond = np.asarray(condition).astype(bool)
+    # upcastType (types.ts:130-138)
+    kinds = [a.dtype.kind, b.dtype.kind]
+    dtype = np.float32 if "f" in kinds else (np.int32 if "i" in kinds else np.bool_)
+    if cond.ndim == 1 and a.ndim > 1:
+        cond = cond.reshape((-1,) + (1,) * (a.ndim - 1))
+    return np.where(cond, a, b).astype(dtype)
+
+
+def mean(x, n_axes=None):
+    """ops/reduction_ops.ts:201-238 over the innermost n_axes axes (all when None): each
+    element divided by the count (float32), then summed."""
+    x = _f32(x)
+    n_axes = x.ndim if n_axes is None else n_axes
+    count = int(np.prod(x.shape[x.ndim - n_axes:])) if n_axes else 1
+    return sum_(real_divide(x, np.float32(count)), n_axes)

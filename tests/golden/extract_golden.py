@@ -58,6 +58,12 @@ CASES = {
     "batchnorm": ("tfjs-core/src/ops/batchnorm_test.ts",
                   ["batchNorm4D", "batchNorm3D", "batchNorm2D"]),
     "resize_bilinear": ("tfjs-core/src/ops/resize_bilinear_test.ts", ["resizeBilinear"]),
+    "resize_nearest": ("tfjs-core/src/ops/resize_nearest_neighbor_test.ts",
+                       ["resizeNearestNeighbor"]),
+    "where": ("tfjs-core/src/ops/logical_ops_test.ts", ["where"]),
+    "array_extra": ("tfjs-core/src/ops/array_ops_test.ts",
+                    ["stack", "unstack", "split", "expandDims"]),
+    "mean": ("tfjs-core/src/ops/reduction_ops_test.ts", ["Reduction: mean"]),
 }
 # fixture name -> (reference test file, describe blocks, title filter): the gradient blocks,
 # whose expected values pin the backward kernels (conv2dDerInput / conv2dDerFilter behind

@@ -863,3 +863,111 @@ def avg_pool_gradients(ops):
                 for dj in (0, 2):
                     want[0, i + di, j + dj, 0] += dy[0, i, j, 0] * 0.25
     expect_close(ops.avg_pool_backprop(dy, x, 2, 1, 0, dilations=2), want.ravel())
+
+
+# ---- resize_nearest_neighbor_test.ts, logical_ops_test.ts (where), array_ops_test.ts (stack,
+# unstack, split, expandDims), reduction_ops_test.ts (mean) ---------------------------------
+@recipe
+def resize_nearest_known_answers(ops):
+    for title, align in (("simple alignCorners=false", False), ("simple alignCorners=true", True),
+                         ("matches tensorflow w/ random numbers alignCorners=false", False),
+                         ("matches tensorflow w/ random numbers alignCorners=true", True),
+                         ("batch of 2, simple, alignCorners=true", True)):
+        a = golden_case("resize_nearest", title)["arrays"]
+        r = ops.resize_nearest(f32(a[0], a[1]), a[2], align)
+        expect_close(r, a[3])
+
+
+@recipe
+def where_known_answers(ops):
+    g = lambda t: golden_case("where", t)["arrays"]
+    flat = lambda v: np.array(v).ravel()
+    a = g("Tensor1D")
+    expect_close(ops.where(np.array(a[0], bool), f32(a[1]), f32(a[2])), a[3])
+    for t in ("Tensor2D", "Tensor3D", "Tensor4D"):
+        a = g(t)
+        cond = flat(a[0]).astype(bool).reshape(a[1])
+        expect_close(ops.where(cond, f32(flat(a[2]), a[3]), f32(flat(a[4]), a[5])), a[6])
+    # rank-1 condition: whole slices along the first axis
+    a = g("Tensor2D different `a` dimension w/ condition rank=1")
+    cond = np.array(a[0], bool)
+    expect_close(ops.where(cond, f32(flat(a[5]), a[6]), f32(flat(a[7]), a[8])), a[9])
+    expect_close(ops.where(cond, np.full((4, 2), 10, np.float32), f32(flat(a[12]), a[13])), a[14])
+    a = g("Tensor4D different `a` dimension w/ condition rank=1")
+    expect_close(ops.where(np.array(a[0], bool), f32(a[10], a[11]), f32(a[12], a[13])), a[14])
+    # rows that are not constant: a slice of a where the condition holds, of b elsewhere
+    x = np.arange(12, dtype=np.float32).reshape(4, 3)
+    got = ops.where(np.array([1, 0, 0, 1], bool), x, -x)
+    expect_close(got, np.where(np.array([1, 0, 0, 1], bool)[:, None], x, -x))
+    # int32 and float32 operands give float32; bool operands stay bool
+    r = ops.where(np.array([True, False]), np.array([1, 2], np.int32), np.array([.5, .25], np.float32))
+    assert r.dtype == np.float32 and list(r) == [1.0, 0.25]
+    r = ops.where(np.array([True, False]), np.array([True, True]), np.array([False, False]))
+    assert r.dtype in (np.bool_, np.uint8) and [bool(v) for v in r] == [True, False]   # Uint8Array storage
+
+
+@recipe
+def mean_known_answers(ops):
+    g = lambda t: golden_case("mean", t, "Reduction: mean")["arrays"]
+    a = g("basic")
+    expect_close(ops.mean(f32(a[0], a[1])), 7 / 6)
+    a = g("propagates NaNs")
+    assert np.isnan(ops.mean(f32(a[0], a[1])))
+    r = ops.mean(np.array(g("mean(int32) => float32")[0], np.int32))
+    assert r.dtype == np.float32
+    expect_close(r, 4)
+    expect_close(ops.mean(np.array(g("mean(bool) => float32")[0], bool)), 3 / 5)
+    a = g("axis=1 in 2D array")
+    expect_close(ops.mean(f32(a[0], a[1]), a[2]), a[4])
+    a = g("axis = -1 in 2D array")
+    expect_close(ops.mean(f32(a[0], a[1]), a[2]), a[4])
+    a = g("axis=0 in 2D array, keepDims")
+    r = ops.mean(f32(a[0], a[1]), a[2], True)
+    assert list(r.shape) == a[3]
+    expect_close(r, [4 / 3, 1])
+    a = g("axis=0,1 in 2D array")
+    expect_close(ops.mean(f32(a[0], a[1]), a[2]), 7 / 6)
+
+
+@recipe
+def stack_unstack_split_expand_dims_known_answers(ops):
+    g = lambda t, d: golden_case("array_extra", t, d)["arrays"]
+    a = g("[1,2], [3,4] and [5,6], axis=1", "stack")
+    r = ops.stack([f32(a[0]), f32(a[1]), f32(a[2])], 1)
+    assert list(r.shape) == a[4]
+    expect_close(r, a[5])
+    a = g("[[1,2],[3,4]] and [[5, 6], [7, 8]], axis=2", "stack")
+    r = ops.stack([f32(np.array(v).ravel(), (2, 2)) for v in a[:3]], 2)
+    assert list(r.shape) == a[4]
+    expect_close(r, a[5])
+    a = g("scalars 3, 5 and 7", "stack")
+    expect_close(ops.stack([f32(3), f32(5), f32(7)]), a[2])
+    a = g("unstack with negative integer axis", "unstack")
+    x = f32(a[0], a[1])
+    for k, part in enumerate(ops.unstack(x, -1)):
+        assert list(part.shape) == a[2 + 2 * k]
+        expect_close(part, a[3 + 2 * k])
+    a = g("unstack rank 3 tensor with axis=1", "unstack")
+    parts = ops.unstack(f32(a[0], a[1]), 1)
+    expect_close(parts[0], a[3])
+    expect_close(parts[1], a[5])
+    a = g("split by number", "split")
+    parts = ops.split(f32(a[0], a[1]), 2, 1)
+    assert list(parts[0].shape) == a[2]
+    expect_close(parts[0], a[3])
+    expect_close(parts[1], a[5])
+    a = g("split by sizes", "split")
+    parts = ops.split(f32(a[0], a[1]), a[2], 1)
+    for k in range(3):
+        assert list(parts[k].shape) == a[3 + 2 * k]
+        expect_close(parts[k], a[4 + 2 * k])
+    for title in ("1d, axis=-2", "1d, axis=-1", "1d, axis=0", "1d, axis=1"):
+        a = g(title, "expandDims")
+        r = ops.expand_dims(f32(a[0]), int(title.split("=")[1]))
+        assert list(r.shape) == a[1]
+        expect_close(r, a[2])
+    for title in ("2d, axis=-3", "2d, axis=-2", "2d, axis=-1", "2d, axis=0", "2d, axis=1", "2d, axis=2"):
+        a = g(title, "expandDims")
+        r = ops.expand_dims(f32(np.array(a[0]).ravel(), (3, 2)), int(title.split("=")[1]))
+        assert list(r.shape) == a[1]
+        expect_close(r, a[2])

@@ -44,6 +44,36 @@ class OracleOps:
         return self.r.max_pool(x, self.r.compute_pool2d_info(x.shape, fsize, strides, dilations,
                                                               pad, rounding))
 
+    # further ops of converter graphs
+    def resize_nearest(self, x, size, align):
+        x4 = x[None] if x.ndim == 3 else x
+        r = self.r.resize_nearest_neighbor(x4, size[0], size[1], align)
+        return r[0] if x.ndim == 3 else r
+
+    def where(self, cond, a, b): return self.r.select(cond, a, b)
+
+    def mean(self, x, axis=None, keep_dims=False):
+        x = np.asarray(x)
+        axes = list(range(x.ndim)) if axis is None else [a % x.ndim for a in np.atleast_1d(axis)]
+        rest = [i for i in range(x.ndim) if i not in axes]
+        moved = np.transpose(x, rest + axes) if x.ndim else x
+        r = self.r.mean(moved.astype(np.float32), len(axes))
+        if keep_dims:
+            r = r.reshape([1 if i in axes else d for i, d in enumerate(x.shape)])
+        return r
+
+    def expand_dims(self, x, axis=0):
+        x = np.asarray(x)
+        return np.expand_dims(x, axis if axis >= 0 else x.ndim + axis + 1)
+
+    def stack(self, xs, axis=0): return np.stack([np.asarray(x) for x in xs], axis)
+    def unstack(self, x, axis=0): return [np.take(x, i, axis) for i in range(np.shape(x)[axis])]
+
+    def split(self, x, num_or_sizes, axis=0):
+        if isinstance(num_or_sizes, int):
+            return np.split(np.asarray(x), num_or_sizes, axis)
+        return np.split(np.asarray(x), np.cumsum(num_or_sizes)[:-1], axis)
+
     # backward kernels; the Conv2DInfo is that of the forward op (ops/conv.ts:354-420,
     # 466-520, ops/pool.ts:333-397), dilation 1 for the convolutions
     def conv2d_der_input(self, x_shape, dy, w, strides, pad, rounding=None):
@@ -179,6 +209,29 @@ class HipOps:
         if dilations != 1:
             return self._run(lambda a: tf.pool(a, fsize, "max", pad, dilations, strides), x)
         return self._run(lambda a: tf.max_pool(a, fsize, strides, pad, rounding), x)
+
+    def resize_nearest(self, x, size, align):
+        return self._run(lambda a: self.tf.resize_nearest_neighbor(a, size, align), x)
+
+    def where(self, cond, a, b): return self._run(self.tf.where, cond, a, b)
+
+    def mean(self, x, axis=None, keep_dims=False):
+        return self._run(lambda a: self.tf.mean(a, axis, keep_dims), x)
+
+    def expand_dims(self, x, axis=0): return self._run(lambda a: self.tf.expand_dims(a, axis), x)
+
+    def stack(self, xs, axis=0):
+        return self._run(lambda *ts: self.tf.stack(list(ts), axis), *xs)
+
+    def _run_list(self, fn, *arrays):
+        tf = self.tf
+        with tf.tidy():
+            return [t.data_sync() for t in fn(*[tf.tensor(a) for a in arrays])]
+
+    def unstack(self, x, axis=0): return self._run_list(lambda a: self.tf.unstack(a, axis), x)
+
+    def split(self, x, num_or_sizes, axis=0):
+        return self._run_list(lambda a: self.tf.split(a, num_or_sizes, axis), x)
 
     def conv2d_der_input(self, x_shape, dy, w, strides, pad, rounding=None):
         tf = self.tf

@@ -241,6 +241,22 @@ def test_js_graph_ops_match_oracle(tmp_path, ref):
               ref.resize_bilinear(img, [9, 4], align))
     c.add("resize_rank3", "resizeBilinear", dict(x=img[0]), dict(size=[10, 12], alignCorners=False),
           ref.resize_bilinear(img[0], [10, 12], False))
+    for align in (False, True):
+        c.add("nearest_%s" % align, "resizeNearestNeighbor", dict(x=img), dict(size=[9, 4], alignCorners=align),
+              ref.resize_nearest(img, [9, 4], align), exact=True)
+    cond = rng.integers(0, 2, (4, 3, 5)).astype(np.bool_)
+    wa, wb = f(4, 3, 5), f(4, 3, 5)
+    c.add("where_same_shape", "where", dict(condition=cond, a=wa, b=wb), {}, ref.where(cond, wa, wb), exact=True)
+    c.add("where_rank1", "where", dict(condition=cond[:, 0, 0], a=wa, b=wb), {},
+          ref.where(cond[:, 0, 0], wa, wb), exact=True)
+    m = f(5, 7, 3)
+    c.add("mean_all", "mean", dict(x=m), {}, ref.mean(m))
+    c.add("mean_axes", "mean", dict(x=m), dict(axis=[0, 2], keepDims=True), ref.mean(m, [0, 2], True))
+    sx = f(3, 8, 2)
+    c.add("split_stack", "splitStack", dict(x=sx), dict(sizes=4, axis=1, stackAxis=0),
+          np.stack(np.split(sx, 4, 1), 0), exact=True)
+    c.add("unstack_concat", "unstackConcat", dict(x=sx), dict(axis=2, concatAxis=0),
+          np.concatenate([sx[:, :, 0], sx[:, :, 1]], 0), exact=True)
     results = c.run()
     c.check(results)
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0

@@ -545,3 +545,38 @@ def test_pool_backprop(hip, ref, xs, f, s, pad, dil):
     dy = rng.uniform(-1, 1, y.shape).astype(np.float32)
     close(hip.max_pool_backprop(dy, x, f, s, pad, dil), ref.max_pool_backprop(dy, x, f, s, pad, dil))
     close(hip.avg_pool_backprop(dy, x, f, s, pad, dil), ref.avg_pool_backprop(dy, x, f, s, pad, dil))
+
+
+# ---------------------------------------- further ops of converter graphs ----
+@pytest.mark.parametrize("in_hw,out_hw,align", [((5, 6), (9, 4), False), ((5, 6), (9, 4), True),
+                                                ((7, 7), (1, 1), True), ((3, 4), (12, 20), False),
+                                                ((16, 16), (5, 7), True)])
+def test_resize_nearest_bit_exact(hip, ref, in_hw, out_hw, align):
+    x = rng_for("nearest", in_hw, out_hw).standard_normal((2,) + in_hw + (3,)).astype(np.float32)
+    assert np.array_equal(hip.resize_nearest(x, out_hw, align), ref.resize_nearest(x, out_hw, align))
+
+
+def test_where_bit_exact(hip, ref):
+    rng = rng_for("where")
+    for shape in ((7,), (5, 6), (2, 3, 4, 5)):
+        cond = rng.integers(0, 2, shape).astype(np.bool_)
+        a, b = rng.standard_normal(shape).astype(np.float32), rng.standard_normal(shape).astype(np.float32)
+        a.flat[0] = np.nan
+        got, want = hip.where(cond, a, b), ref.where(cond, a, b)
+        assert np.array_equal(got, want, equal_nan=True)
+        if len(shape) > 1:
+            got, want = hip.where(cond[(slice(None),) + (0,) * (len(shape) - 1)], a, b), \
+                ref.where(cond[(slice(None),) + (0,) * (len(shape) - 1)], a, b)
+            assert np.array_equal(got, want, equal_nan=True)
+    ai = rng.integers(-5, 5, (4, 3)).astype(np.int32)
+    bf = rng.standard_normal((4, 3)).astype(np.float32)
+    cond = rng.integers(0, 2, (4, 3)).astype(np.bool_)
+    got = hip.where(cond, ai, bf)
+    assert got.dtype == np.float32 and np.array_equal(got, ref.where(cond, ai, bf))
+
+
+@pytest.mark.parametrize("shape,axis,keep", [((6, 5), None, False), ((6, 5), 0, True), ((4, 3, 5), [0, 2], False),
+                                             ((2, 1000), 1, False)])
+def test_mean(hip, ref, shape, axis, keep):
+    x = rng_for("mean", shape).standard_normal(shape).astype(np.float32)
+    close(hip.mean(x, axis, keep), ref.mean(x, axis, keep))

@@ -310,6 +310,23 @@ static napi_value js_pool2d(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+/* resizeNearest(ctx, x, out, batch, inH, inW, channels, outH, outW, alignCorners) */
+static napi_value js_resize_nearest(napi_env env, napi_callback_info info) {
+  ARGS(10);
+  I64(1, x); I64(2, out);
+  INT(3, batch); INT(4, in_h); INT(5, in_w); INT(6, ch); INT(7, out_h); INT(8, out_w); INT(9, align);
+  CHECK(tfhip_resize_nearest(ctx, x, out, batch, in_h, in_w, ch, out_h, out_w, align));
+  return undefined(env);
+}
+
+/* select(ctx, condition, a, b, out, inner) */
+static napi_value js_select(napi_env env, napi_callback_info info) {
+  ARGS(6);
+  I64(1, c); I64(2, a); I64(3, b); I64(4, out); I64(5, inner);
+  CHECK(tfhip_select(ctx, c, a, b, out, inner));
+  return undefined(env);
+}
+
 /* Backward kernels: name(ctx, a, b, out, info) with info = the forward op's Conv2DInfo.
  * conv2dDerInput(ctx, dy, filter, dx, info), conv2dDerFilter(ctx, x, dy, dW, info) and their
  * depthwise twins. */
@@ -527,7 +544,8 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"conv2dDerFilter", js_conv2d_der_filter},
       {"depthwiseConv2dDerInput", js_depthwise_der_input},
       {"depthwiseConv2dDerFilter", js_depthwise_der_filter},
-      {"pool2dBackprop", js_pool2d_backprop}};
+      {"pool2dBackprop", js_pool2d_backprop}, {"resizeNearest", js_resize_nearest},
+      {"select", js_select}};
   for (size_t i = 0; i < sizeof fns / sizeof fns[0]; i++) {
     napi_value f;
     if (napi_create_function(env, fns[i].name, NAPI_AUTO_LENGTH, fns[i].fn, NULL, &f) != napi_ok ||

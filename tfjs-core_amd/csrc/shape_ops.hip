@@ -85,6 +85,36 @@ __global__ void resize_bilinear_kernel(const float* x, float* out, int batch, in
   }
 }
 
+// Nearest neighbour: source row / column = min(in - 1, floor(ratio * r)), or round half up
+// (JavaScript's Math.round) with align_corners, in double as the reference computes them.
+__global__ void resize_nearest_kernel(const float* x, float* out, int batch, int in_h, int in_w,
+                                      int ch, int out_h, int out_w, double ratio_h,
+                                      double ratio_w, int align_corners) {
+  const int64_t n = (int64_t)batch * out_h * out_w * ch;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const int d = (int)(i % ch);
+    int64_t t = i / ch;
+    const int c = (int)(t % out_w);
+    t /= out_w;
+    const int r = (int)(t % out_h);
+    const int b = (int)(t / out_h);
+    const double fr = ratio_h * r, fc = ratio_w * c;
+    const int sr = min(in_h - 1, (int)(align_corners ? floor(fr + 0.5) : floor(fr)));
+    const int sc = min(in_w - 1, (int)(align_corners ? floor(fc + 0.5) : floor(fc)));
+    out[i] = x[(((int64_t)b * in_h + sr) * in_w + sc) * ch + d];
+  }
+}
+
+// out[i] = cond[i / inner] ? a[i] : b[i]; T = 4-byte (float32 / int32) or 1-byte (bool) elements.
+template <typename T>
+__global__ void select_kernel(const uint8_t* cond, const T* a, const T* b, T* out, int64_t n,
+                              int64_t inner) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    out[i] = cond[i / inner] == 1 ? a[i] : b[i];
+}
+
 template <typename T>
 __global__ void one_hot_kernel(const int32_t* idx, T* out, int64_t n_idx, int depth, T on, T off) {
   const int64_t n = n_idx * depth;
@@ -245,6 +275,65 @@ extern "C" int tfhip_one_hot(tfhip_ctx* ctx, int64_t indices, int64_t out, int d
     hipLaunchKernelGGL(one_hot_kernel<float>, grid, block, 0, ctx->stream,
                        (const int32_t*)bi->ptr, (float*)bo->ptr, bi->numel, depth, on_value,
                        off_value);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+extern "C" int tfhip_resize_nearest(tfhip_ctx* ctx, int64_t x, int64_t out, int batch, int in_h,
+                                    int in_w, int channels, int out_h, int out_w,
+                                    int align_corners) {
+  if (!ctx) return TFHIP_EINVAL;
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bo, out);
+  if (batch < 0 || in_h < 0 || in_w < 0 || channels < 0 || out_h < 0 || out_w < 0)
+    return ctx->fail(TFHIP_EINVAL, "resizeNearestNeighbor: bad geometry");
+  if (bx->numel != (int64_t)batch * in_h * in_w * channels ||
+      bo->numel != (int64_t)batch * out_h * out_w * channels || bo->dtype != TFHIP_FLOAT32)
+    return ctx->fail(TFHIP_EINVAL, "resizeNearestNeighbor: buffers do not match the shapes given");
+  if (bo->numel == 0) return TFHIP_OK;
+  if (in_h == 0 || in_w == 0) return ctx->fail(TFHIP_EINVAL, "resizeNearestNeighbor: empty input image");
+  Temp tx(ctx);
+  const float* xf;
+  int rc;
+  if ((rc = as_f32(ctx, bx, &tx, &xf))) return rc;
+  // effective sizes and ratios (backend_cpu.ts:3025-3038)
+  const double eh_in = (align_corners && out_h > 1) ? in_h - 1 : in_h;
+  const double ew_in = (align_corners && out_w > 1) ? in_w - 1 : in_w;
+  const double eh_out = (align_corners && out_h > 1) ? out_h - 1 : out_h;
+  const double ew_out = (align_corners && out_w > 1) ? out_w - 1 : out_w;
+  hipLaunchKernelGGL(resize_nearest_kernel, dim3(grid_for(ctx, bo->numel, 256)), dim3(256), 0,
+                     ctx->stream, xf, (float*)bo->ptr, batch, in_h, in_w, channels, out_h, out_w,
+                     eh_in / eh_out, ew_in / ew_out, align_corners ? 1 : 0);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+extern "C" int tfhip_select(tfhip_ctx* ctx, int64_t condition, int64_t a, int64_t b, int64_t out,
+                            int64_t inner) {
+  if (!ctx) return TFHIP_EINVAL;
+  TFHIP_GET(ctx, bc, condition);
+  TFHIP_GET(ctx, ba, a);
+  TFHIP_GET(ctx, bb, b);
+  TFHIP_GET(ctx, bo, out);
+  if (bc->dtype != TFHIP_BOOL) return ctx->fail(TFHIP_EINVAL, "select: condition must be bool");
+  if (ba->dtype == TFHIP_UINT8Q || ba->dtype != bb->dtype || ba->dtype != bo->dtype)
+    return ctx->fail(TFHIP_EINVAL, "select: a, b and the result must share one storage dtype");
+  if (inner < 1 || ba->numel != bb->numel || ba->numel != bo->numel ||
+      bc->numel * inner != ba->numel)
+    return ctx->fail(TFHIP_EINVAL, "select: sizes do not match (condition %lld x %lld, a %lld, b %lld)",
+                     (long long)bc->numel, (long long)inner, (long long)ba->numel,
+                     (long long)bb->numel);
+  if (bo->numel == 0) return TFHIP_OK;
+  const dim3 grid(grid_for(ctx, bo->numel, 256)), block(256);
+  const uint8_t* c = static_cast<const uint8_t*>(bc->ptr);
+  if (dtype_size(ba->dtype) == 4)
+    hipLaunchKernelGGL(select_kernel<int32_t>, grid, block, 0, ctx->stream, c,
+                       (const int32_t*)ba->ptr, (const int32_t*)bb->ptr, (int32_t*)bo->ptr,
+                       bo->numel, inner);
+  else
+    hipLaunchKernelGGL(select_kernel<uint8_t>, grid, block, 0, ctx->stream, c,
+                       (const uint8_t*)ba->ptr, (const uint8_t*)bb->ptr, (uint8_t*)bo->ptr,
+                       bo->numel, inner);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }

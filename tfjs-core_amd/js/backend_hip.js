@@ -529,6 +529,24 @@ class MathBackendHIP extends KernelBackend {
                              alignCorners ? 1 : 0);
     return out;
   }
+  resizeNearestNeighbor(x, newHeight, newWidth, alignCorners) {
+    const [batch, h, w, c] = x.shape;
+    const out = this.out([batch, newHeight, newWidth, c], 'float32');
+    this.napi.resizeNearest(this.ctx, this.h(x), this.h(out), batch, h, w, c, newHeight, newWidth,
+                            alignCorners ? 1 : 0);
+    return out;
+  }
+  // backend_cpu.ts:822-845; a rank-1 condition picks whole slices along the first axis
+  // (ops/logical_ops.ts:140-156)
+  select(condition, a, b) {
+    const dtype = util.upcastType(a.dtype, b.dtype);
+    const $a = this.materialized(this.cast(a, dtype)), $b = this.materialized(this.cast(b, dtype));
+    const cond = this.materialized(condition);
+    const inner = condition.rank === 1 && a.rank > 1 ? util.sizeFromShape(a.shape.slice(1)) : 1;
+    const out = this.out(a.shape, dtype);
+    this.napi.select(this.ctx, this.h(cond), this.h($a), this.h($b), this.h(out), inner);
+    return out;
+  }
   oneHot(indices, depth, onValue, offValue) {
     const idx = this.materialized(indices);
     const out = this.out([indices.size, depth], 'int32');

@@ -961,6 +961,149 @@ const resizeBilinear = op('resizeBilinear', (images, size, alignCorners) => {
   return $images.rank === 4 ? res : reshape(res, res.shape.slice(1));
 });
 
+// ---- further ops of converter graphs -------------------------------------------------------
+// ops/image_ops.ts:105-150
+const resizeNearestNeighbor = op('resizeNearestNeighbor', (images, size, alignCorners) => {
+  const $images = convertToTensor(images, 'images', 'resizeNearestNeighbor');
+  util.assert($images.rank === 3 || $images.rank === 4,
+              () => `Error in resizeNearestNeighbor: x must be rank 3 or 4, but got rank ${$images.rank}.`);
+  util.assert(size.length === 2,
+              () => `Error in resizeNearestNeighbor: new shape must 2D, but got ${size}.`);
+  util.assert($images.dtype === 'float32' || $images.dtype === 'int32',
+              () => '`images` must have `int32` or `float32` as dtype');
+  const batchImages = $images.rank === 4 ? $images : reshape($images, [1].concat($images.shape));
+  const res = ENGINE.runKernel(
+      backend => backend.resizeNearestNeighbor(batchImages, size[0], size[1], !!alignCorners), {batchImages});
+  return $images.rank === 4 ? res : reshape(res, res.shape.slice(1));
+});
+
+// ops/logical_ops.ts:129-175
+const where = op('where', (condition, a, b) => {
+  const $a = convertToTensor(a, 'a', 'where');
+  const $b = convertToTensor(b, 'b', 'where');
+  const $condition = convertToTensor(condition, 'condition', 'where', 'bool');
+  util.assert($condition.dtype === 'bool',
+              () => `Argument 'condition' passed to 'where' must be bool tensor, but got ${$condition.dtype} tensor`);
+  util.assert(util.arraysEqual($a.shape, $b.shape),
+              () => `Error in where:  Shapes ${$a.shape} and ${$b.shape} must match`);
+  if ($condition.rank === 1) {
+    util.assert($condition.shape[0] === $a.shape[0],
+                () => 'The first dimension of `a` must match the size of `condition`.');
+  } else {
+    util.assert(util.arraysEqual($condition.shape, $b.shape),
+                () => `Error in where:  Shapes ${$condition.shape} and ${$b.shape} must match`);
+  }
+  return ENGINE.runKernel((backend, save) => {
+    save([$condition]);
+    return backend.select($condition, $a, $b);
+  }, {$condition, $a, $b}, (dy, saved) => ({
+    $condition: () => cast(zerosLike(saved[0]), 'float32'),
+    $a: () => mul(dy, cast(saved[0], dy.dtype)),
+    $b: () => mul(dy, cast(logicalNot(saved[0]), dy.dtype))
+  }));
+});
+
+// ops/reduction_ops.ts:201-238: every element is divided by the count, then the quotients are
+// summed (so the gradient is the composite's: dy / count spread over the reduced axes).
+const mean = op('mean', (x, axis, keepDims) => {
+  const $x = convertToTensor(x, 'x', 'mean');
+  const axes = util.parseAxisParam(axis, $x.shape);
+  const reduceSize = util.sizeFromShape(axes.map(a => $x.shape[a]));
+  const xf = $x.dtype === 'float32' ? $x : cast($x, 'float32');
+  return sum(div(xf, scalar(reduceSize)), axis, keepDims);
+});
+
+// ops/array_ops.ts:905-920
+const expandDims = op('expandDims', (x, axis) => {
+  if (axis == null) axis = 0;
+  const $x = convertToTensor(x, 'x', 'expandDims');
+  util.assert(axis <= $x.rank, () => 'Axis must be <= rank of the tensor');
+  const newShape = $x.shape.slice();
+  if (axis < 0) {
+    util.assert(-($x.rank + 1) <= axis, () => `Axis must be in the interval [${- ($x.rank + 1)}, ${$x.rank}]`);
+    axis = $x.rank + axis + 1;
+  }
+  newShape.splice(axis, 0, 1);
+  return reshape($x, newShape);
+});
+
+// ops/array_ops.ts:820-826 with squeezeShape of util.ts:238-275
+const squeeze = op('squeeze', (x, axis) => {
+  const $x = convertToTensor(x, 'x', 'squeeze');
+  const axes = axis == null ? null : util.parseAxisParam(axis, $x.shape).sort((p, q) => p - q);
+  const newShape = [];
+  let j = 0;
+  for (let i = 0; i < $x.shape.length; ++i) {
+    if (axes != null) {
+      if (axes[j] === i && $x.shape[i] !== 1) {
+        throw new Error(`Can't squeeze axis ${i} since its dim '${$x.shape[i]}' is not 1`);
+      }
+      if ((axes[j] == null || axes[j] > i) && $x.shape[i] === 1) newShape.push($x.shape[i]);
+      if (axes[j] <= i) j++;
+    }
+    if ($x.shape[i] !== 1) newShape.push($x.shape[i]);
+  }
+  return reshape($x, newShape);
+});
+
+// ops/array_ops.ts:744-765
+const stack = op('stack', (tensors, axis) => {
+  if (axis == null) axis = 0;
+  const $tensors = tensors.map((t, i) => convertToTensor(t, `tensors[${i}]`, 'stack'));
+  util.assert($tensors.length >= 1, () => 'Pass at least one tensor to tf.stack');
+  if ($tensors.length === 1) return expandDims($tensors[0], axis);
+  const rank = $tensors[0].rank, shape = $tensors[0].shape, dtype = $tensors[0].dtype;
+  util.assert(axis <= rank, () => 'Axis must be <= rank of the tensor');
+  $tensors.forEach(t => {
+    util.assert(util.arraysEqual(shape, t.shape), () => 'All tensors passed to stack must have matching shapes');
+    util.assert(dtype === t.dtype, () => 'All tensors passed to stack must have matching dtypes');
+  });
+  return concat($tensors.map(t => expandDims(t, axis)), axis);
+});
+
+// ops/array_ops.ts:860-892
+const unstack = op('unstack', (x, axis) => {
+  if (axis == null) axis = 0;
+  const $x = convertToTensor(x, 'x', 'unstack');
+  util.assert(axis >= -$x.shape.length && axis < $x.shape.length,
+              () => `Axis = ${axis} is not in [-${$x.shape.length}, ${$x.shape.length})`);
+  if (axis < 0) axis += $x.shape.length;
+  const outputShape = $x.shape.filter((d, i) => i !== axis);
+  const res = [];
+  for (let i = 0; i < $x.shape[axis]; i++) {
+    const begin = new Array($x.rank).fill(0);
+    const size = $x.shape.slice();
+    begin[axis] = i;
+    size[axis] = 1;
+    res.push(reshape(slice($x, begin, size), outputShape));
+  }
+  return res;
+});
+
+// ops/concat_split.ts:182-218
+const split = op('split', (x, numOrSizeSplits, axis) => {
+  if (axis == null) axis = 0;
+  const $x = convertToTensor(x, 'x', 'split');
+  axis = util.parseAxisParam(axis, $x.shape)[0];
+  let splitSizes;
+  if (typeof numOrSizeSplits === 'number') {
+    util.assert($x.shape[axis] % numOrSizeSplits === 0, () => 'Number of splits must evenly divide the axis.');
+    splitSizes = new Array(numOrSizeSplits).fill($x.shape[axis] / numOrSizeSplits);
+  } else {
+    util.assert($x.shape[axis] === numOrSizeSplits.reduce((p, q) => p + q),
+                () => 'The sum of sizes must match the size of the axis dimension.');
+    splitSizes = numOrSizeSplits;
+  }
+  const begin = new Array($x.rank).fill(0);
+  const size = $x.shape.slice();
+  return splitSizes.map(s => {
+    size[axis] = s;
+    const piece = slice($x, begin.slice(), size.slice());
+    begin[axis] += s;
+    return piece;
+  });
+});
+
 const opHandler = {
   reshape, cast, clone, matMul, add, sub, mul, div, relu, prelu, clipByValue, exp, log, sum, max,
   min, argMax, argMin, logSumExp, softmax, transpose, gather, conv2d, depthwiseConv2d, avgPool, maxPool
@@ -977,5 +1120,6 @@ module.exports = {
   slice, stridedSlice, reverse, concat, pad, tile, oneHot, equal, notEqual, less, lessEqual,
   greater, greaterEqual, logicalAnd, logicalOr, logicalNot, batchNorm, resizeBilinear,
   conv2dDerInput, conv2dDerFilter, conv2dTranspose, depthwiseConv2dDerInput,
-  depthwiseConv2dDerFilter, maxPoolBackprop, avgPoolBackprop
+  depthwiseConv2dDerFilter, maxPoolBackprop, avgPoolBackprop, resizeNearestNeighbor, where, mean,
+  expandDims, squeeze, stack, unstack, split
 };

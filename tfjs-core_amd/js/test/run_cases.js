@@ -74,6 +74,12 @@ const OPS = {
   depthwiseConv2dDerFilter: (i, a) => tf.depthwiseConv2dDerFilter(i.x, i.dy, a.filterShape, a.strides, a.pad),
   maxPoolBackprop: (i, a) => tf.maxPoolBackprop(i.dy, i.x, a.filterSize, a.strides, a.pad, a.dilations),
   avgPoolBackprop: (i, a) => tf.avgPoolBackprop(i.dy, i.x, a.filterSize, a.strides, a.pad, a.dilations),
+  resizeNearestNeighbor: (i, a) => tf.resizeNearestNeighbor(i.x, a.size, a.alignCorners),
+  where: i => tf.where(i.condition, i.a, i.b),
+  mean: (i, a) => tf.mean(i.x, a.axis, a.keepDims),
+  // stack of the pieces of a split / an unstack along another axis: one tensor exercising all three
+  splitStack: (i, a) => tf.stack(tf.split(i.x, a.sizes, a.axis).map(t => tf.squeeze(tf.expandDims(t, 0), [0])), a.stackAxis),
+  unstackConcat: (i, a) => tf.concat(tf.unstack(i.x, a.axis), a.concatAxis),
   // gradients through the tape (tf.grad / tf.grads); `wrt` picks the argument
   gradConv2d: (i, a) => tf.grads((x, f) => tf.conv2d(x.clone(), f.clone(), a.strides, a.pad).clone())(
       [i.x, i.filter], i.dy)[a.wrt],

@@ -52,6 +52,8 @@ _SIGNATURES = {
     "tfhip_depthwise_conv2d": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC), _I64, _INT, _INT,
                                C.POINTER(QParams)],
     "tfhip_pool2d": [_PTR, _I64, _I64, C.POINTER(Conv2DInfoC), _INT],
+    "tfhip_resize_nearest": [_PTR, _I64, _I64, _INT, _INT, _INT, _INT, _INT, _INT, _INT],
+    "tfhip_select": [_PTR, _I64, _I64, _I64, _I64, _I64],
     "tfhip_conv2d_der_input": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC)],
     "tfhip_conv2d_der_filter": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC)],
     "tfhip_depthwise_conv2d_der_input": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC)],

@@ -575,6 +575,29 @@ class MathBackendHIP(object):
                                                 new_height, new_width, 1 if align_corners else 0))
         return out
 
+    def resize_nearest_neighbor(self, x, new_height, new_width, align_corners):
+        """backend_cpu.ts:3016-3067."""
+        b, h, w, c = x.shape
+        out = self._out([b, new_height, new_width, c], "float32")
+        self._ck(self.lib.tfhip_resize_nearest(self.ctx, self._h(x), self._h(out), b, h, w, c,
+                                               new_height, new_width, 1 if align_corners else 0))
+        return out
+
+    def select(self, condition, a, b):
+        """backend_cpu.ts:822-845; a rank-1 condition picks whole slices along the first axis
+        (ops/logical_ops.ts:140-156)."""
+        dtype = su.upcast_type(a.dtype, b.dtype)
+        a, b = self.cast(a, dtype), self.cast(b, dtype)
+        a, b, cond = self._materialized(a), self._materialized(b), self._materialized(condition)
+        inner = 1
+        if condition.rank == 1 and a.rank > 1:
+            for d in a.shape[1:]:
+                inner *= d
+        out = self._out(a.shape, dtype)
+        self._ck(self.lib.tfhip_select(self.ctx, self._h(cond), self._h(a), self._h(b), self._h(out),
+                                       inner))
+        return out
+
     def one_hot(self, indices, depth, on_value, off_value):
         """backend_cpu.ts:3325-3339 (int32 result)."""
         out = self._out([indices.size, depth], "int32")

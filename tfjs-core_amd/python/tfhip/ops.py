@@ -3,7 +3,10 @@ backend call each, after tfjs-core/src/ops/{matmul,fused_ops,conv,pool,relu_ops,
 binary_ops,reduction_ops,softmax,segment_ops,transpose}.ts.  Python twin of js/ops.js."""
 import numpy as np
 
+import builtins
 from . import shape_util as su
+
+builtins_sum = builtins.sum
 from .engine import ENGINE, NP_DTYPE, Tensor
 
 
@@ -848,3 +851,151 @@ def max_pool_backprop(dy, x, filter_size, strides, pad, dilations=None, dim_roun
 def avg_pool_backprop(dy, x, filter_size, strides, pad, dilations=None):
     """ops/pool.ts:397-445."""
     return _pool_backprop("avgPoolBackprop", dy, x, filter_size, strides, dilations, pad, None, "avg")
+
+
+# ---- further ops of converter graphs: resizeNearestNeighbor, where, mean, and the shape ops
+# that are compositions of reshape / slice / concat ----
+def resize_nearest_neighbor(images, size, align_corners=False):
+    """ops/image_ops.ts:105-150."""
+    images = _conv(images, "images", "resizeNearestNeighbor")
+    if images.rank not in (3, 4):
+        raise ValueError("Error in resizeNearestNeighbor: x must be rank 3 or 4, but got rank %d."
+                         % images.rank)
+    if len(size) != 2:
+        raise ValueError("Error in resizeNearestNeighbor: new shape must 2D, but got %s."
+                         % list(size))
+    if images.dtype not in ("float32", "int32"):
+        raise ValueError("`images` must have `int32` or `float32` as dtype")
+    new_h, new_w = size
+
+    def run():
+        x4 = images if images.rank == 4 else reshape(images, (1,) + tuple(images.shape))
+        r = ENGINE.run_kernel(lambda be: be.resize_nearest_neighbor(x4, new_h, new_w, align_corners))
+        return r if images.rank == 4 else reshape(r, r.shape[1:])
+    return ENGINE.tidy(run)
+
+
+def where(condition, a, b):
+    """ops/logical_ops.ts:129-175."""
+    a, b = _conv(a, "a", "where"), _conv(b, "b", "where")
+    condition = _conv(condition, "condition", "where")
+    if condition.dtype != "bool":
+        raise ValueError("Argument 'condition' passed to 'where' must be bool tensor, but got %s "
+                         "tensor" % condition.dtype)
+    if tuple(a.shape) != tuple(b.shape):
+        raise ValueError("Error in where:  Shapes %s and %s must match" % (list(a.shape), list(b.shape)))
+    if condition.rank == 1:
+        if condition.shape[0] != (a.shape[0] if a.rank else None):
+            raise ValueError("The first dimension of `a` must match the size of `condition`.")
+    elif tuple(condition.shape) != tuple(b.shape):
+        raise ValueError("Error in where:  Shapes %s and %s must match"
+                         % (list(condition.shape), list(b.shape)))
+    return ENGINE.tidy(lambda: ENGINE.run_kernel(lambda be: be.select(condition, a, b)))
+
+
+def mean(x, axis=None, keep_dims=False):
+    """ops/reduction_ops.ts:201-238: every element is divided by the number of reduced elements
+    first, then the quotients are summed."""
+    def run():
+        xt = _conv(x, "x", "mean")
+        axes = su.parse_axis_param(axis, xt.shape)
+        n = 1
+        for a in axes:
+            n *= xt.shape[a]
+        xf = xt if xt.dtype == "float32" else cast(xt, "float32")
+        return sum(div(xf, tensor(float(n))), axis, keep_dims)
+    return ENGINE.tidy(run)
+
+
+def expand_dims(x, axis=0):
+    """ops/array_ops.ts:905-920."""
+    x = _conv(x, "x", "expandDims")
+    if axis > x.rank:
+        raise ValueError("Axis must be <= rank of the tensor")
+    shape = list(x.shape)
+    if axis < 0:
+        if -(x.rank + 1) > axis:
+            raise ValueError("Axis must be in the interval [%d, %d]" % (-(x.rank + 1), x.rank))
+        axis = x.rank + axis + 1
+    shape.insert(axis, 1)
+    return reshape(x, shape)
+
+
+def squeeze(x, axis=None):
+    """ops/array_ops.ts:820-826, util.ts:238-275 (squeezeShape)."""
+    x = _conv(x, "x", "squeeze")
+    axes = None if axis is None else sorted(su.parse_axis_param(axis, x.shape))
+    shape, j = [], 0
+    for i, d in enumerate(x.shape):
+        if axes is not None:
+            if j < len(axes) and axes[j] == i:
+                if d != 1:
+                    raise ValueError("Can't squeeze axis %d since its dim '%d' is not 1" % (i, d))
+                j += 1
+                continue
+            shape.append(d)
+        elif d != 1:
+            shape.append(d)
+    return reshape(x, shape)
+
+
+def stack(tensors, axis=0):
+    """ops/array_ops.ts:744-765."""
+    ts = [_conv(t, "tensors[%d]" % i, "stack") for i, t in enumerate(tensors)]
+    if len(ts) < 1:
+        raise ValueError("Pass at least one tensor to tf.stack")
+    if len(ts) == 1:
+        return expand_dims(ts[0], axis)
+    for t in ts:
+        if tuple(t.shape) != tuple(ts[0].shape):
+            raise ValueError("All tensors passed to stack must have matching shapes")
+        if t.dtype != ts[0].dtype:
+            raise ValueError("All tensors passed to stack must have matching dtypes")
+    if axis > ts[0].rank:
+        raise ValueError("Axis must be <= rank of the tensor")
+    return ENGINE.tidy(lambda: concat([expand_dims(t, axis) for t in ts], axis))
+
+
+def unstack(x, axis=0):
+    """ops/array_ops.ts:860-892."""
+    x = _conv(x, "x", "unstack")
+    if not (-x.rank <= axis < x.rank):
+        raise ValueError("Axis = %d is not in [-%d, %d)" % (axis, x.rank, x.rank))
+    if axis < 0:
+        axis += x.rank
+    out_shape = [d for i, d in enumerate(x.shape) if i != axis]
+
+    def run():
+        res = []
+        for i in range(x.shape[axis]):
+            begin = [0] * x.rank
+            size = list(x.shape)
+            begin[axis], size[axis] = i, 1
+            res.append(reshape(slice(x, begin, size), out_shape))
+        return res
+    return ENGINE.tidy(run)
+
+
+def split(x, num_or_size_splits, axis=0):
+    """ops/concat_split.ts:182-218."""
+    x = _conv(x, "x", "split")
+    axis = su.parse_axis_param(axis, x.shape)[0]
+    if isinstance(num_or_size_splits, int):
+        if x.shape[axis] % num_or_size_splits != 0:
+            raise ValueError("Number of splits must evenly divide the axis.")
+        sizes = [x.shape[axis] // num_or_size_splits] * num_or_size_splits
+    else:
+        sizes = list(num_or_size_splits)
+        if x.shape[axis] != builtins_sum(sizes):
+            raise ValueError("The sum of sizes must match the size of the axis dimension.")
+
+    def run():
+        begin = [0] * x.rank
+        res = []
+        for sz in sizes:
+            size = list(x.shape)
+            size[axis] = sz
+            res.append(slice(x, list(begin), size))
+            begin[axis] += sz
+        return res
+    return ENGINE.tidy(run)
