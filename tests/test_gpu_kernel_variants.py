@@ -124,6 +124,67 @@ def test_pointwise_conv_tiles(tf, n, h, cin, cout, act, want):
     close(got, want_y)
 
 
+# -------------------------------------- many rows times a small matrix ----
+@pytest.mark.parametrize("n,h,w_,cin,cout,act,bias,quant,want", [
+    (16, 112, 112, 32, 64, "relu6", True, False, "gemm_rowstream_k32xn64_f32"),
+    (1, 449, 449, 32, 64, "prelu", True, False, "gemm_rowstream_k32xn64_f32"),   # odd row count
+    (3, 256, 257, 32, 64, "linear", False, False, "gemm_rowstream_k32xn64_f32"),
+    (5, 200, 201, 32, 64, "relu", True, True, "gemm_rowstream_k32xn64_u8"),
+    (2, 320, 331, 32, 64, "linear", True, True, "gemm_rowstream_k32xn64_u8"),
+    (1, 449, 449, 64, 128, "relu6", True, False, "gemm_64x64_rowmajor_f32"),    # stays tiled
+])
+def test_rowstream_products(tf, ref, n, h, w_, cin, cout, act, bias, quant, want):
+    """Pointwise convolutions with enough pixels for the row-streaming kernel (B resident in
+    LDS, A straight into the MFMA operand registers), against a float64 contraction; the last
+    32-row block is partial in the odd cases."""
+    print("rowstream", n, h, w_, cin, cout, act, bias, quant, flush=True)
+    rng = np.random.default_rng(n + h + cin + cout)
+    x = rng.uniform(-1, 1, (n, h, w_, cin)).astype(np.float32)
+    if quant:
+        q = rng.integers(0, 256, (1, 1, cin, cout)).astype(np.uint8)
+        scale, mn = 0.004, -0.5
+        w = ref.dequantize(q, scale, mn)
+    else:
+        w = (rng.standard_normal((1, 1, cin, cout)) * np.sqrt(2.0 / cin)).astype(np.float32)
+    b = rng.standard_normal(cout).astype(np.float32) if bias else None
+    alpha = rng.uniform(0.1, 0.5, cout).astype(np.float32) if act == "prelu" else None
+    with tf.tidy():
+        wt = tf.quantized_tensor(q, scale, mn) if quant else tf.tensor(w)
+        got = tf.fused.conv2d(
+            tf.tensor(x), wt, 1, "same", bias=None if b is None else tf.tensor(b), activation=act,
+            prelu_activation_weights=None if alpha is None else tf.tensor(alpha)).data_sync()
+        assert last_kernel(tf) == want, last_kernel(tf)
+    y = x.reshape(-1, cin).astype(np.float64) @ np.asarray(w, np.float64).reshape(cin, cout)
+    if b is not None:
+        y = y + b
+    y = np.where(y < 0, alpha * y, y) if act == "prelu" else act64(y, act)
+    close(got, y.reshape(n, h, w_, cout))
+    # a NaN in one row of A stays in that row
+    x2 = x[:1, :40].copy()
+    x2[0, 7, 5, 3] = np.nan
+    with tf.tidy():
+        got2 = tf.conv2d(tf.tensor(x2), tf.tensor(np.asarray(w, np.float32)), 1, "same").data_sync()
+    nan_rows = np.isnan(got2).any(axis=-1)
+    assert nan_rows.sum() == 1 and nan_rows[0, 7, 5]
+
+
+def test_rowstream_matmul_and_small_fallback(tf):
+    """tf.matMul of the same shape class takes the row-streaming kernel; below the row threshold
+    and with a full-shape bias the tiled kernels keep the product."""
+    rng = np.random.default_rng(77)
+    m = 256 * 8 * 32 * 3 + 5
+    a = rng.uniform(-1, 1, (m, 32)).astype(np.float32)
+    b = rng.uniform(-1, 1, (32, 64)).astype(np.float32)
+    with tf.tidy():
+        got = tf.matmul(tf.tensor(a), tf.tensor(b)).data_sync()
+        assert last_kernel(tf) == "gemm_rowstream_k32xn64_f32", last_kernel(tf)
+    close(got, a.astype(np.float64) @ b.astype(np.float64))
+    with tf.tidy():
+        got = tf.matmul(tf.tensor(a[:5000]), tf.tensor(b)).data_sync()
+        assert last_kernel(tf).startswith("gemm_64x64"), last_kernel(tf)
+    close(got, a[:5000].astype(np.float64) @ b.astype(np.float64))
+
+
 @pytest.mark.parametrize("m,k,n,want_prefix", [
     (4096, 784, 1024, "gemm_128x128_rowmajor_f32_kb48"),
     (256, 512, 256, "gemm_64x64_rowmajor_f32_kb48_splitk"),

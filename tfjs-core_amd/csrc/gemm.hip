@@ -56,6 +56,7 @@ struct GemmArgs {
   int tiles_m, tiles_n, k_tiles, full_tiles, tail_tiles, splits, kt_per;
   float* partials;  // [tail_tiles * splits][BM * BN] partial tiles when splits > 1
   unsigned a_bytes, b_bytes;  // per-batch byte extents of A and B (buffer-load range check)
+  int reverse;  // walk the tiles / row blocks of every XCD's run from the end
 };
 
 constexpr int BK = 16;
@@ -122,7 +123,7 @@ struct WorkItem {
 __device__ __forceinline__ WorkItem work_item(const GemmArgs& p, int block) {
   WorkItem w = {-1, 0, 0, -1};
   if (block < p.full_tiles) {
-    w.tile = xcd_remap(block, p.full_tiles);
+    w.tile = xcd_remap_dir(block, p.full_tiles, p.reverse);
     w.kt1 = p.k_tiles;
   } else if (block - p.full_tiles < p.tail_tiles * p.splits) {
     const int h = block - p.full_tiles;
@@ -978,6 +979,147 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
   }
 }
 
+// Products of many rows with a small right-hand side (K <= 128, K * N floats <= 64 KB: the
+// first pointwise layers of a MobileNet are [802816, 32] x [32, 64] ... [200704, 128] x
+// [128, 128]).  A tile of such a product has only K / 16 steps, so the tiled kernel above
+// spends its time filling and draining its pipeline.  Here B is copied into LDS once per
+// workgroup, already in operand order, and every wavefront streams blocks of 32 rows of A
+// straight from memory into the registers that the MFMA reads (lane = row, 16-byte loads of 4
+// consecutive k), with the next block's loads in flight while the current one is multiplied and
+// stored.  Same summation-order permutation as above: MFMA e of group q multiplies
+// k = 8q + e (lanes 0..31) and k = 8q + 4 + e (lanes 32..63).
+template <int KQ, int NJ>
+__global__ __launch_bounds__(256, 2) void gemm_rowstream_kernel(const GemmArgs p, int n_blocks,
+                                                                int quant) {
+  constexpr int K = 8 * KQ, N = 32 * NJ;
+  extern __shared__ __attribute__((aligned(16))) float bl[];  // B as [K / 4][N][4] = (k / 4, col, k % 4)
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, g = lane >> 5;
+  {
+    // B into operand order: an item is 4 consecutive k of one column (one 16-byte LDS write,
+    // lanes side by side along the column); all loads first, they are independent
+    constexpr int PER = K / 4 * N / 256;
+    auto fill = [&](auto quant_tag) {
+      f32x4 w[PER];
+#pragma unroll
+      for (int u = 0; u < PER; u++) {
+        const int item = tid + 256 * u;
+        const int k4 = item / N, col = item - k4 * N;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int at = (4 * k4 + e) * N + col;
+          if (decltype(quant_tag)::value)
+            w[u][e] = dequant(static_cast<const unsigned char*>(p.B)[at], p.qscale, p.qmin);
+          else
+            w[u][e] = static_cast<const float*>(p.B)[at];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < PER; u++)
+        *reinterpret_cast<f32x4*>(&bl[(tid + 256 * u) * 4]) = w[u];
+    };
+    if (quant) fill(std::true_type{});
+    else fill(std::false_type{});
+  }
+  float bias_c[NJ], alpha_c[NJ];  // of column 32j + l32
+#pragma unroll
+  for (int j = 0; j < NJ; j++) {
+    const int col = 32 * j + l32;
+    bias_c[j] = alpha_c[j] = 0.f;
+    if (p.bias_kind == TFHIP_BCAST_SCALAR) bias_c[j] = p.bias[0];
+    if (p.bias_kind == TFHIP_BCAST_COLUMN) bias_c[j] = p.bias[col];
+    if (p.prelu_kind == TFHIP_BCAST_SCALAR) alpha_c[j] = p.prelu[0];
+    if (p.prelu_kind == TFHIP_BCAST_COLUMN) alpha_c[j] = p.prelu[col];
+  }
+  const ActCfg act = act_cfg(p.act);
+  __syncthreads();
+
+  // The 32-row blocks are cut into 8 runs, one per XCD (workgroup b runs on XCD b % 8; the grid
+  // is a multiple of 8): the kernels before and after this one split their rows the same way,
+  // so what an XCD leaves in its L2 is what the same XCD reads next.  Within its run this
+  // wavefront takes blocks first, first + stride, ... (the same for all its lanes).
+  const int xcd = (int)blockIdx.x & 7;
+  const int per = n_blocks >> 3, rem = n_blocks & 7;
+  const int run0 = xcd * per + (xcd < rem ? xcd : rem);
+  const int run1 = run0 + per + (xcd < rem ? 1 : 0);
+  const int first = __builtin_amdgcn_readfirstlane(run0 + ((int)blockIdx.x >> 3) * 4 + wave);
+  const int stride = ((int)gridDim.x >> 3) * 4;
+  const unsigned a_at = (unsigned)((l32 * K + 4 * g) * 4);
+  const unsigned c_at = (unsigned)((4 * g * N + l32) * 4);
+
+  // One descriptor per block over its rows that exist: rows at or past M (and whole blocks
+  // past the end of the run) read as zeros and their stores are dropped.
+  auto load = [&](int blk, f32x4 (&a)[KQ]) {
+    const long long row0 = (long long)(p.reverse ? run0 + run1 - 1 - blk : blk) * 32;
+    const long long left = (long long)p.M - row0;
+    const unsigned bytes = blk >= run1 ? 0u : (unsigned)((left < 32 ? left : 32) * K * 4);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A + row0 * K, bytes);
+#pragma unroll
+    for (int q = 0; q < KQ; q++) a[q] = buffer_load_f32x4(ra, a_at + 32 * q);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto multiply_store = [&](int blk, const f32x4 (&a)[KQ]) {
+    f32x16 acc[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+    // B operands of group q + 1 are read while group q is multiplied; the order is pinned so
+    // that no more than two groups of them are ever live
+    f32x4 b[2][NJ];
+    auto read_b = [&](int q, f32x4 (&dst)[NJ]) {
+#pragma unroll
+      for (int j = 0; j < NJ; j++)
+        dst[j] = *reinterpret_cast<const f32x4*>(&bl[((q * 2 + g) * N + 32 * j + l32) * 4]);
+    };
+    read_b(0, b[0]);
+#pragma unroll
+    for (int q = 0; q < KQ; q++) {
+      if (q + 1 < KQ) read_b(q + 1, b[(q + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+          acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q][e], b[q & 1][j][e], acc[j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // accumulator register r holds row 8*(r/4) + 4*(lane/32) + r%4 of the block, column l32 of
+    // column block j: a store writes two runs of 32 consecutive floats.  The part of the address
+    // that is known at compile time rides in the scalar offset, which the range check of the
+    // descriptor does not see: in the one block that is cut short by M the rows past the end are
+    // therefore turned away through the lane's own offset.
+    const long long row0 = (long long)(p.reverse ? run0 + run1 - 1 - blk : blk) * 32;
+    const int left = (int)((long long)p.M - row0 < 32 ? (long long)p.M - row0 : 32);
+    const __amdgpu_buffer_rsrc_t rc = make_rsrc(p.C + row0 * N, (unsigned)(left * N * 4));
+    auto store = [&](auto whole_tag) {
+      constexpr bool whole = decltype(whole_tag)::value;
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+          const int row_c = 8 * (r >> 2) + (r & 3);  // + 4 * g
+          const float v = activate(acc[j][r] + bias_c[j], act, alpha_c[j]);
+          const unsigned at = whole || row_c + 4 * g < left ? c_at : OOB_OFFSET;
+          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rc, (int)at,
+                                                /*scalar offset=*/(row_c * N + 32 * j) * 4, 0);
+        }
+    };
+    if (left == 32) store(std::true_type{});
+    else store(std::false_type{});
+  };
+
+  f32x4 a0[KQ], a1[KQ];
+  load(first, a0);
+  for (int blk = first; blk < run1; blk += 2 * stride) {
+    load(blk + stride, a1);
+    multiply_store(blk, a0);
+    load(blk + 2 * stride, a0);
+    if (blk + stride < run1) multiply_store(blk + stride, a1);
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
@@ -1099,6 +1241,7 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
   p.splits = pl.splits;
   p.kt_per = pl.kt_per;
   p.k_tiles = (int)ceil_div(p.K, BK);
+  p.reverse = ctx->take_sweep();
   Temp partials(ctx);
   p.partials = nullptr;
   if (pl.splits > 1) {
@@ -1161,8 +1304,58 @@ static int launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
   }
 }
 
+// The row-streaming kernel for the shapes it is built for; returns -1 when the product is not
+// one of them (the tiled kernels take it then).
+template <int KQ, int NJ>
+static int launch_rowstream_cfg(tfhip_ctx* ctx, const GemmArgs& p, int quant) {
+  auto kernel = gemm_rowstream_kernel<KQ, NJ>;
+  const size_t lds = (size_t)KQ * 8 * NJ * 32 * sizeof(float);
+  static int per_cu = 0;
+  if (!per_cu) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, lds) != hipSuccess || n < 1) {
+      (void)hipGetLastError();
+      n = 1;
+    }
+    per_cu = n;
+  }
+  const int n_blocks = (int)ceil_div(p.M, 32);
+  const long long slots = (long long)ctx->num_cus * per_cu / 8 * 8;  // a multiple of the XCD count
+  const long long want = ceil_div(ceil_div(n_blocks, 8), 4) * 8;
+  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "gemm_rowstream_k%dxn%d_%s", KQ * 8, NJ * 32,
+           quant ? "u8" : "f32");
+  GemmArgs q = p;
+  q.reverse = ctx->take_sweep();
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(want < slots || slots < 8 ? want : slots)), dim3(256),
+                     lds, ctx->stream, q, n_blocks, quant);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+static int launch_rowstream(tfhip_ctx* ctx, const GemmArgs& p, int batch, int amode, int bmode) {
+  if (batch != 1 || amode != A_ROWMAJOR || (bmode != B_ROWMAJOR && bmode != B_UINT8)) return -1;
+  if (p.lda != p.K || p.ldb != p.N || !p.a_vec || !p.b_vec) return -1;
+  if (p.bias_kind == TFHIP_BCAST_FULL || p.prelu_kind == TFHIP_BCAST_FULL) return -1;
+  // enough 32-row blocks to give every wavefront of a full machine several
+  if ((long long)p.M < (long long)ctx->num_cus * 8 * 32 * 3) return -1;
+  const int quant = bmode == B_UINT8;
+#define TFHIP_ROWSTREAM(KK, NN) \
+  if (p.K == KK && p.N == NN) return launch_rowstream_cfg<KK / 8, NN / 32>(ctx, p, quant);
+  // Measured on MI355X inside a batch-64 MobileNet: [802816, 32] x [32, 64] (bound by HBM) runs
+  // 58 us here against 66 us tiled; at K = 64 and 128 with N = 128 the tiled kernel, whose
+  // tiles balance better over the CUs (24.5 per CU against 6.1 row blocks per SIMD), stays
+  // 4 us ahead, so those shapes are not routed here.
+  TFHIP_ROWSTREAM(32, 64)
+#undef TFHIP_ROWSTREAM
+  return -1;
+}
+
 static int launch_gemm(tfhip_ctx* ctx, GemmArgs& p, int batch, int amode, int bmode,
                        bool kblocked) {
+  {
+    const int rc = launch_rowstream(ctx, p, batch, amode, bmode);
+    if (rc >= 0) return rc;
+  }
   if ((long long)p.N * 256 >= (1LL << 31))
     return ctx->fail(TFHIP_ENOTSUP, "matmul/conv2d: more than 2^23 output columns");
   // Byte extents of one batch entry of A and B, for the range check of the buffer loads.
@@ -1402,6 +1595,7 @@ extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t o
         const long long cap = (long long)ctx->num_cus * per_cu;
         const unsigned grid = (unsigned)(n_rows < cap ? n_rows : cap);
         snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "%s_%s", name, quant ? "u8" : "f32");
+        ctx->sweep = 1;  // this kernel walks the rows forward: its consumer should start at the end
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), (size_t)lds, ctx->stream, p,
                            (int)row_floats, n_rows);
       };

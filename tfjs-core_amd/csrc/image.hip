@@ -57,6 +57,7 @@ struct DwArgs {
   int quant;
   double qscale, qmin;
   int tiles_w, tiles_h, c4;  // fast path: patch grid and channel quads
+  int reverse;               // fast path: walk the rows of every XCD's run from the end
 };
 
 // 3x3, dilation 1, channel multiplier 1, C % 4 == 0, stride S.  One lane = one channel
@@ -69,7 +70,8 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p) {
   const int64_t total = (int64_t)ci.batch * p.tiles_h * p.tiles_w * p.c4;
   // contiguous image regions per XCD: the halo rows two patch rows share are then served
   // by that XCD's L2 instead of being fetched once per XCD
-  const int64_t gid = (int64_t)xcd_remap(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x;
+  const int64_t gid =
+      (int64_t)xcd_remap_dir(blockIdx.x, gridDim.x, p.reverse) * blockDim.x + threadIdx.x;
   if (gid >= total) return;
   const int cq = (int)(gid % p.c4);
   int64_t t = gid / p.c4;
@@ -165,7 +167,8 @@ __global__ __launch_bounds__(256) void depthwise3x3_rows_kernel(const DwArgs p, 
   constexpr unsigned OOB = 0x80000000u;  // beyond any extent below 2 GiB: loads give 0, stores vanish
   const tfhip_conv2d_info& ci = p.ci;
   const int64_t total = (int64_t)ci.batch * chunks * p.tiles_w * p.c4;
-  const int64_t gid = (int64_t)xcd_remap(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x;
+  const int64_t gid =
+      (int64_t)xcd_remap_dir(blockIdx.x, gridDim.x, p.reverse) * blockDim.x + threadIdx.x;
   if (gid >= total) return;
   const int cq = (int)(gid % p.c4);
   int64_t t = gid / p.c4;
@@ -385,6 +388,7 @@ static void launch_dw3x3(tfhip_ctx* ctx, DwArgs& p) {
   p.tiles_h = (int)ceil_div(p.ci.out_h, TH);
   p.tiles_w = (int)ceil_div(p.ci.out_w, TW);
   const int64_t total = (int64_t)p.ci.batch * p.tiles_h * p.tiles_w * p.c4;
+  p.reverse = ctx->take_sweep();
   hipLaunchKernelGGL((depthwise3x3_kernel<S, TH, TW>), dim3((unsigned)ceil_div(total, 256)),
                      dim3(256), 0, ctx->stream, p);
 }
@@ -395,6 +399,7 @@ static void launch_dw3x3_rows(tfhip_ctx* ctx, DwArgs& p, int rows) {
   const int chunks = (int)ceil_div(p.ci.out_h, rows);
   p.tiles_w = (int)ceil_div(p.ci.out_w, TW);
   const int64_t total = (int64_t)p.ci.batch * chunks * p.tiles_w * p.c4;
+  p.reverse = ctx->take_sweep();
   hipLaunchKernelGGL((depthwise3x3_rows_kernel<TW>), dim3((unsigned)ceil_div(total, 256)),
                      dim3(256), 0, ctx->stream, p, rows, chunks,
                      (unsigned)((int64_t)p.ci.batch * p.ci.in_h * p.ci.in_w * p.ci.in_c * 4),
