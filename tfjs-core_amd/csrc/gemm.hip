@@ -891,9 +891,20 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
       v[u] = ok ? x : 0.f;
     }
   };
+  // A grid that is a multiple of 8 cuts the output rows into one run per XCD (workgroup b runs
+  // on XCD b % 8): neighbouring output rows, which share input rows, then meet in one L2, and
+  // the kernel that reads the result cuts it the same way.
+  int row_first = blockIdx.x, row_step = gridDim.x, row_end = n_rows;
+  if ((gridDim.x & 7) == 0) {
+    const int xcd = (int)blockIdx.x & 7, per = n_rows >> 3, rem = n_rows & 7;
+    const int run0 = xcd * per + (xcd < rem ? xcd : rem);
+    row_end = run0 + per + (xcd < rem ? 1 : 0);
+    row_first = run0 + ((int)blockIdx.x >> 3);
+    row_step = (int)gridDim.x >> 3;
+  }
   float v[8];
-  if (one_pass && (int)blockIdx.x < n_rows) stage_load(blockIdx.x, v);
-  for (int row = blockIdx.x; row < n_rows; row += gridDim.x) {
+  if (one_pass && row_first < row_end) stage_load(row_first, v);
+  for (int row = row_first; row < row_end; row += row_step) {
     const int n = row / p.OH, oh = row - n * p.OH;
     __syncthreads();  // the previous row's readers are done
     if (one_pass) {
@@ -922,7 +933,7 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
       }
     }
     __syncthreads();
-    if (one_pass && row + (int)gridDim.x < n_rows) stage_load(row + gridDim.x, v);
+    if (one_pass && row + row_step < row_end) stage_load(row + row_step, v);
 
     const long long out_at = (((long long)n * p.OH + oh) * p.OW) * p.N;  // workgroup-uniform
     float* __restrict__ crow = p.C + out_at;
@@ -1593,7 +1604,8 @@ extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t o
           per_cu = 1;
         }
         const long long cap = (long long)ctx->num_cus * per_cu;
-        const unsigned grid = (unsigned)(n_rows < cap ? n_rows : cap);
+        unsigned grid = (unsigned)(n_rows < cap ? n_rows : cap);
+        if (grid >= 64) grid &= ~7u;  // a multiple of the XCD count: one run of rows per XCD
         snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "%s_%s", name, quant ? "u8" : "f32");
         ctx->sweep = 1;  // this kernel walks the rows forward: its consumer should start at the end
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), (size_t)lds, ctx->stream, p,
