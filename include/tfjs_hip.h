@@ -144,7 +144,13 @@ enum {
    * (backend.ts:202-233; backend_cpu.ts:747-820): out must be TFHIP_BOOL; NaN compares
    * like JavaScript (only != is true). */
   TFHIP_EQUAL = 7, TFHIP_NOT_EQUAL = 8, TFHIP_LESS = 9, TFHIP_LESS_EQUAL = 10,
-  TFHIP_GREATER = 11, TFHIP_GREATER_EQUAL = 12, TFHIP_LOGICAL_AND = 13, TFHIP_LOGICAL_OR = 14
+  TFHIP_GREATER = 11, TFHIP_GREATER_EQUAL = 12, TFHIP_LOGICAL_AND = 13, TFHIP_LOGICAL_OR = 14,
+  /* pow/squaredDifference/mod/floorDiv/atan2/eluDer (backend.ts:166-181, 260-262, 363-366;
+   * backend_cpu.ts:483-489, 582-588, 893-904, 984-991, 1227-1242, 1425-1431) with JavaScript's
+   * Math.pow (1 ** +-Infinity and x ** NaN are NaN) and % (sign of the dividend).  floorDiv
+   * writes int32.  eluDer(dy, y) = y >= 1 ? dy : dy * (y + 1). */
+  TFHIP_POW = 15, TFHIP_SQUARED_DIFFERENCE = 16, TFHIP_MOD = 17, TFHIP_FLOOR_DIV = 18,
+  TFHIP_ATAN2 = 19, TFHIP_ELU_DER = 20
 };
 int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_shape, int a_rank,
                  int64_t b, const int32_t* b_shape, int b_rank, int64_t out);
@@ -153,7 +159,19 @@ int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_shape, int 
 enum {
   TFHIP_RELU = 0, TFHIP_CLIP = 1, TFHIP_EXP = 2, TFHIP_LOG = 3, TFHIP_NEG = 4,
   TFHIP_ABS = 5, TFHIP_SIGMOID = 6, TFHIP_SQRT = 7, TFHIP_SQUARE = 8, TFHIP_TANH = 9,
-  TFHIP_RSQRT = 10
+  TFHIP_RSQRT = 10,
+  /* floor/ceil/round/sign/expm1/log1p/reciprocal, the trigonometric and hyperbolic functions
+   * and their inverses, erf/elu/selu/softplus/step (backend.ts:264-298, 306-322, 330-338,
+   * 344-390; backend_cpu.ts:993-1030, 1071-1189, 1211-1225, 1244-1263, 1321-1535): round is
+   * round-half-to-even, sign(NaN) = 0, erf is the reference's polynomial (also for x < 0),
+   * step(x) = NaN for NaN, 1 for x > 0, else p0. */
+  TFHIP_FLOOR = 11, TFHIP_CEIL = 12, TFHIP_ROUND = 13, TFHIP_SIGN = 14, TFHIP_EXPM1 = 15,
+  TFHIP_LOG1P = 16, TFHIP_RECIPROCAL = 17, TFHIP_SIN = 18, TFHIP_COS = 19, TFHIP_TAN = 20,
+  TFHIP_ASIN = 21, TFHIP_ACOS = 22, TFHIP_ATAN = 23, TFHIP_SINH = 24, TFHIP_COSH = 25,
+  TFHIP_ASINH = 26, TFHIP_ACOSH = 27, TFHIP_ATANH = 28, TFHIP_ERF = 29, TFHIP_ELU = 30,
+  TFHIP_SELU = 31, TFHIP_SOFTPLUS = 32, TFHIP_STEP = 33,
+  /* isNaN/isInf/isFinite (backend.ts:284-290; backend_cpu.ts:1032-1069): out must be TFHIP_BOOL */
+  TFHIP_IS_NAN = 34, TFHIP_IS_INF = 35, TFHIP_IS_FINITE = 36
 };
 int tfhip_unary(tfhip_ctx* ctx, int op, int64_t x, int64_t out, float p0, float p1);
 /* cast / int (backend.ts:340, 484; backend_cpu.ts:1299-1308, 2861-2863; backends/backend_util.ts:34-71):
@@ -170,7 +188,12 @@ int tfhip_fill(tfhip_ctx* ctx, int64_t out, double value);
 /* ---- reductions over the innermost axis ---------------------------------------------- */
 /* sum/max/min/argMax/argMin (backend.ts:183, 195-200, 244, 255; backend_cpu.ts:590-611,686-712,906-929):
  * x viewed as [outer, inner]; out has `outer` elements (int32 for ARG*). */
-enum { TFHIP_SUM = 0, TFHIP_MAX = 1, TFHIP_MIN = 2, TFHIP_ARGMAX = 3, TFHIP_ARGMIN = 4 };
+enum {
+  TFHIP_SUM = 0, TFHIP_MAX = 1, TFHIP_MIN = 2, TFHIP_ARGMAX = 3, TFHIP_ARGMIN = 4,
+  /* prod/all/any (backend.ts:185-193, 249-253; backend_cpu.ts:613-633, 938-982): prod like sum;
+   * all/any read and write bool */
+  TFHIP_PROD = 5, TFHIP_ALL = 6, TFHIP_ANY = 7
+};
 int tfhip_reduce(tfhip_ctx* ctx, int op, int64_t x, int64_t out, int64_t outer, int64_t inner);
 /* One-pass row softmax; same result as the reference's 10-call composite
  * (ops/softmax.ts:45-79, ops/reduction_ops.ts:56-74) within float32 tolerance. */

@@ -394,7 +394,18 @@ void ref_pool2d_backprop(const float* dy, const float* x, float* dx, const ref_c
 }
 
 /* ---- elementwise ------------------------------------------------------------------- */
-enum { REF_ADD = 0, REF_SUB, REF_MUL, REF_DIV, REF_PRELU, REF_MAXIMUM, REF_MINIMUM };
+enum {
+  REF_ADD = 0, REF_SUB, REF_MUL, REF_DIV, REF_PRELU, REF_MAXIMUM, REF_MINIMUM,
+  REF_POW, REF_SQUARED_DIFFERENCE, REF_MOD, REF_FLOOR_DIV, REF_ATAN2, REF_ELU_DER
+};
+
+/* Math.pow of ECMAScript: a NaN exponent gives NaN (also for base 1), and (+-1) ** +-Infinity
+ * is NaN; everything else is C's pow. */
+static double js_pow(double a, double b) {
+  if (isnan(b)) return NAN;
+  if (fabs(a) == 1.0 && isinf(b)) return NAN;
+  return pow(a, b);
+}
 
 static double binary_eval(int op, double a, double b) {
   switch (op) {
@@ -405,6 +416,16 @@ static double binary_eval(int op, double a, double b) {
     case REF_PRELU: return a < 0 ? b * a : a;         /* :1203-1209 */
     case REF_MAXIMUM: return (isnan(a) || isnan(b)) ? NAN : (a > b ? a : b); /* Math.max :931-936 */
     case REF_MINIMUM: return (isnan(a) || isnan(b)) ? NAN : (a < b ? a : b); /* Math.min :886-891 */
+    case REF_POW: return js_pow(a, b);                /* :483-489 */
+    case REF_SQUARED_DIFFERENCE: return (a - b) * (a - b); /* :984-991 */
+    case REF_MOD: {                                   /* :893-904; % is fmod */
+      const double rem = fmod(a, b);
+      if ((a < 0 && b < 0) || (a >= 0 && b >= 0)) return rem;
+      return fmod(rem + b, b);
+    }
+    case REF_FLOOR_DIV: return floor(a / b);          /* :582-588 */
+    case REF_ATAN2: return atan2(a, b);               /* :1425-1431 */
+    case REF_ELU_DER: return b >= 1 ? a : a * (b + 1); /* eluDer(dy, y) :1227-1242 */
   }
   return NAN;
 }
@@ -462,7 +483,11 @@ int ref_binary(int op, const double* a, const int32_t* a_shape, int a_rank, cons
 
 enum {
   REF_RELU = 0, REF_CLIP, REF_EXP, REF_LOG, REF_NEG, REF_ABS, REF_SIGMOID, REF_SQRT,
-  REF_SQUARE, REF_TANH, REF_RSQRT
+  REF_SQUARE, REF_TANH, REF_RSQRT,
+  REF_FLOOR, REF_CEIL, REF_ROUND, REF_SIGN, REF_EXPM1, REF_LOG1P, REF_RECIPROCAL, REF_SIN,
+  REF_COS, REF_TAN, REF_ASIN, REF_ACOS, REF_ATAN, REF_SINH, REF_COSH, REF_ASINH, REF_ACOSH,
+  REF_ATANH, REF_ERF, REF_ELU, REF_SELU, REF_SOFTPLUS, REF_STEP, REF_IS_NAN, REF_IS_INF,
+  REF_IS_FINITE
 };
 
 /* backends/cpu/backend_cpu.ts: relu :1191-1201 (Math.max(0,x), NaN-propagating), clip
@@ -485,6 +510,54 @@ void ref_unary(int op, const float* x, float* out, int64_t n, float p0, float p1
       case REF_SQUARE: r = v * v; break;
       case REF_TANH: r = tanh(v); break;
       case REF_RSQRT: r = 1.0 / sqrt(v); break;
+      case REF_FLOOR: r = floor(v); break;            /* backend_cpu.ts:1004-1013 */
+      case REF_CEIL: r = ceil(v); break;              /* :993-1002 */
+      case REF_ROUND: {                               /* :1071-1092, banker's rounding */
+        const double base = floor(v);
+        if (v - base < 0.5) r = floor(v);
+        else if (v - base > 0.5) r = ceil(v);
+        else r = fmod(base, 2.0) == 0.0 ? base : base + 1.0;
+        break;
+      }
+      case REF_SIGN: r = v < 0 ? -1 : (v > 0 ? 1 : 0); break; /* :1015-1030 */
+      case REF_EXPM1: r = expm1(v); break;            /* :1105-1114 */
+      case REF_LOG1P: r = log1p(v); break;            /* :1128-1138 */
+      case REF_RECIPROCAL: r = 1.0 / v; break;        /* :1176-1185 */
+      case REF_SIN: r = sin(v); break;                /* :1359-1368 */
+      case REF_COS: r = cos(v); break;                /* :1370-1379 */
+      case REF_TAN: r = tan(v); break;                /* :1381-1390 */
+      case REF_ASIN: r = asin(v); break;              /* :1392-1401 */
+      case REF_ACOS: r = acos(v); break;              /* :1403-1412 */
+      case REF_ATAN: r = atan(v); break;              /* :1414-1423 */
+      case REF_SINH: r = sinh(v); break;              /* :1433-1442 */
+      case REF_COSH: r = cosh(v); break;              /* :1444-1453 */
+      case REF_ASINH: r = asinh(v); break;            /* :1466-1475 */
+      case REF_ACOSH: r = acosh(v); break;            /* :1477-1486 */
+      case REF_ATANH: r = atanh(v); break;            /* :1488-1497 */
+      case REF_ERF: {                                 /* :1499-1518, ops/erf_util.ts:18-23 */
+        const double p = 0.3275911, a1 = 0.254829592, a2 = -0.284496736, a3 = 1.421413741,
+                     a4 = -1.453152027, a5 = 1.061405429;
+        const double t = 1.0 / (1.0 + p * v);
+        r = 1.0 - (((((a5 * t + a4) * t) + a3) * t + a2) * t + a1) * t * exp(-v * v);
+        break;
+      }
+      case REF_ELU: r = v >= 0 ? v : exp(v) - 1; break; /* :1211-1225 */
+      case REF_SELU:                                  /* :1244-1263, ops/selu_util.ts:18-19 */
+        r = v >= 0 ? 1.0507009873554804934193349852946 * v
+                   : 1.7580993408473768599402175208123 * (exp(v) - 1);
+        break;
+      case REF_SOFTPLUS: {                            /* :1321-1357 */
+        const double threshold = log(1.1920928955078125e-7) + 2.0;
+        const double e = exp(v);
+        if (v < threshold) r = e;
+        else if (v > -threshold) r = v;
+        else r = log(1.0 + e);
+        break;
+      }
+      case REF_STEP: r = isnan(v) ? NAN : (v > 0 ? 1 : (double)p0); break; /* :1520-1535 */
+      case REF_IS_NAN: r = isnan(v) ? 1 : 0; break;   /* :1032-1043 */
+      case REF_IS_INF: r = isinf(v) ? 1 : 0; break;   /* :1045-1056 */
+      case REF_IS_FINITE: r = isfinite(v) ? 1 : 0; break; /* :1058-1069 */
       default: r = NAN;
     }
     out[i] = (float)r;
@@ -492,7 +565,7 @@ void ref_unary(int op, const float* x, float* out, int64_t n, float p0, float p1
 }
 
 /* ---- reductions over the innermost axis ---------------------------------------------- */
-enum { REF_SUM = 0, REF_MAX, REF_MIN, REF_ARGMAX, REF_ARGMIN };
+enum { REF_SUM = 0, REF_MAX, REF_MIN, REF_ARGMAX, REF_ARGMIN, REF_PROD, REF_ALL, REF_ANY };
 
 /* sum backend_cpu.ts:590-611 (double accumulator, one rounding); max :906-929 and min
  * :861-884 (seeded with element 0, strict compare, so a NaN only survives in slot 0);
@@ -501,7 +574,8 @@ enum { REF_SUM = 0, REF_MAX, REF_MIN, REF_ARGMAX, REF_ARGMIN };
 void ref_reduce(int op, const double* x, double* out, int64_t outer, int64_t inner) {
   for (int64_t i = 0; i < outer; i++) {
     const double* row = x + i * inner;
-    double acc = (op == REF_SUM) ? 0.0 : row[0];
+    /* prod :613-633 starts at 1; all :938-959 and any :961-982 start from element 0 */
+    double acc = (op == REF_SUM) ? 0.0 : (op == REF_PROD) ? 1.0 : row[0];
     int64_t idx = 0;
     for (int64_t j = 0; j < inner; j++) {
       const double v = row[j];
@@ -511,6 +585,9 @@ void ref_reduce(int op, const double* x, double* out, int64_t outer, int64_t inn
         case REF_MIN: if (v < acc) acc = v; break;
         case REF_ARGMAX: if (v > acc) { acc = v; idx = j; } break;
         case REF_ARGMIN: if (v < acc) { acc = v; idx = j; } break;
+        case REF_PROD: acc *= v; break;
+        case REF_ALL: acc = (acc != 0 && !isnan(acc)) ? v : acc; break; /* all = all && value */
+        case REF_ANY: acc = (acc != 0 && !isnan(acc)) ? acc : v; break; /* any = any || value */
       }
     }
     out[i] = (op == REF_ARGMAX || op == REF_ARGMIN) ? (double)idx : acc;

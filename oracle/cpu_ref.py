@@ -289,7 +289,8 @@ def max_pool_backprop(dy, x, ci):
     return _pool_backprop(dy, x, ci, 1)
 
 
-_BIN = dict(add=0, sub=1, mul=2, div=3, prelu=4, maximum=5, minimum=6)
+_BIN = dict(add=0, sub=1, mul=2, div=3, prelu=4, maximum=5, minimum=6, pow=7,
+            squared_difference=8, mod=9, floor_div=10, atan2=11, elu_der=12)
 
 
 def _store(values_f64, dtype):
@@ -357,7 +358,10 @@ def minimum(a, b):
 
 
 _UN = dict(relu=0, clip=1, exp=2, log=3, neg=4, abs=5, sigmoid=6, sqrt=7, square=8, tanh=9,
-           rsqrt=10)
+           rsqrt=10, floor=11, ceil=12, round=13, sign=14, expm1=15, log1p=16, reciprocal=17,
+           sin=18, cos=19, tan=20, asin=21, acos=22, atan=23, sinh=24, cosh=25, asinh=26,
+           acosh=27, atanh=28, erf=29, elu=30, selu=31, softplus=32, step=33, is_nan=34,
+           is_inf=35, is_finite=36)
 
 
 def _unary(op, x, p0=0.0, p1=0.0):
@@ -411,7 +415,49 @@ def rsqrt(x):
     return _unary("rsqrt", x)
 
 
-_RED = dict(sum=0, max=1, min=2, argmax=3, argmin=4)
+def unary(op, x, p0=0.0):
+    """floor ... step by name (the table above): float32 in, float32 out, evaluated in double
+    like backend_cpu's Math.* calls and rounded once by the Float32Array store."""
+    return _unary(op, x, p0)
+
+
+def is_nan(x):
+    return _unary("is_nan", x).astype(np.bool_)
+
+
+def is_inf(x):
+    return _unary("is_inf", x).astype(np.bool_)
+
+
+def is_finite(x):
+    return _unary("is_finite", x).astype(np.bool_)
+
+
+def pow_(a, b):
+    return _binary("pow", a, b, np.asarray(a).dtype)  # backend_cpu.ts:483-489: a.dtype
+
+
+def squared_difference(a, b):
+    return _binary("squared_difference", a, b, np.asarray(a).dtype)
+
+
+def mod(a, b):
+    return _binary("mod", a, b, np.asarray(a).dtype)
+
+
+def floor_div(a, b):
+    return _binary("floor_div", a, b, np.int32)  # backend_cpu.ts:586
+
+
+def atan2(a, b):
+    return _binary("atan2", a, b, np.asarray(a).dtype)
+
+
+def elu_der(dy, y):
+    return _binary("elu_der", dy, y, np.float32)
+
+
+_RED = dict(sum=0, max=1, min=2, argmax=3, argmin=4, prod=5, all=6, any=7)
 
 
 def _reduce(op, x, n_axes=1):
@@ -432,6 +478,20 @@ def sum_(x, n_axes=1):
     # upcastType(x.dtype, 'int32') (types.ts:130-138): bool -> int32
     dt = np.float32 if x.dtype == np.float32 else np.int32
     return _store(_reduce("sum", x, n_axes), dt)
+
+
+def prod(x, n_axes=1):
+    x = np.asarray(x)
+    dt = np.float32 if x.dtype == np.float32 else np.int32
+    return _store(_reduce("prod", x, n_axes), dt)
+
+
+def all_(x, n_axes=1):
+    return _store(_reduce("all", x, n_axes), np.bool_).astype(np.bool_)
+
+
+def any_(x, n_axes=1):
+    return _store(_reduce("any", x, n_axes), np.bool_).astype(np.bool_)
 
 
 def max_(x, n_axes=1):

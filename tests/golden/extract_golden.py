@@ -64,6 +64,17 @@ CASES = {
     "array_extra": ("tfjs-core/src/ops/array_ops_test.ts",
                     ["stack", "unstack", "split", "expandDims"]),
     "mean": ("tfjs-core/src/ops/reduction_ops_test.ts", ["Reduction: mean"]),
+    "unary_extra": ("tfjs-core/src/ops/unary_ops_test.ts",
+                    ["step", "logSigmoid", "softplus", "reciprocal", "log1p", "ceil", "floor", "sign",
+                     "isNaN", "isInf", "isFinite", "expm1", "sin", "cos", "tan", "asin", "acos",
+                     "atan", "sinh", "cosh", "leakyRelu", "elu", "selu", "round", "asinh", "acosh",
+                     "atanh", "erf"]),
+    "binary_extra": ("tfjs-core/src/ops/binary_ops_test.ts",
+                     ["squaredDifference", "mod", "atan2"]),
+    "arithmetic_extra": ("tfjs-core/src/ops/arithmetic_test.ts", ["pow", "addN"]),
+    "reduction_extra": ("tfjs-core/src/ops/reduction_ops_test.ts",
+                        ["Reduction: prod", "Reduction: all", "Reduction: any",
+                         "Reduction: moments", "Reduction: norm"]),
 }
 # fixture name -> (reference test file, describe blocks, title filter): the gradient blocks,
 # whose expected values pin the backward kernels (conv2dDerInput / conv2dDerFilter behind

@@ -113,6 +113,27 @@ class OracleOps:
     def exp(self, x): return self.r.exp(x)
     def log(self, x): return self.r.log(x)
     def unary(self, name, x): return self.r._unary(name, x)
+    def step(self, x, alpha=0.0): return self.r.unary("step", x, alpha)
+
+    def binary(self, name, a, b):
+        fn = dict(pow=self.r.pow_, squared_difference=self.r.squared_difference, mod=self.r.mod,
+                  floor_div=self.r.floor_div, atan2=self.r.atan2)[name]
+        return fn(a, b)
+
+    def reduce(self, name, x):
+        return dict(prod=self.r.prod, all=self.r.all_, any=self.r.any_)[name](x)
+
+    def add_n(self, xs):
+        acc = xs[0]
+        for x in xs[1:]:   # backend_cpu.ts:454-467 sums in the first tensor's dtype
+            acc = self.r.add(acc, x)
+        return acc
+
+    def leaky_relu(self, x, alpha=0.2):
+        return self.r.maximum(self.r.multiply(np.float32(alpha), x), x)
+
+    def log_sigmoid(self, x):
+        return self.r.neg(self.r.unary("softplus", self.r.neg(x)))
     def sum(self, x): return self.r.sum_(x)
     def max(self, x): return self.r.max_(x)
     def min(self, x): return self.r.min_(x)
@@ -275,6 +296,12 @@ class HipOps:
     def exp(self, x): return self._run(self.tf.exp, x)
     def log(self, x): return self._run(self.tf.log, x)
     def unary(self, name, x): return self._run(getattr(self.tf, name), x)
+    def step(self, x, alpha=0.0): return self._run(lambda t: self.tf.step(t, alpha), x)
+    def binary(self, name, a, b): return self._run(getattr(self.tf, name), a, b)
+    def reduce(self, name, x): return self._run(lambda t: getattr(self.tf, name)(t, -1), x)
+    def add_n(self, xs): return self._run(lambda *ts: self.tf.add_n(list(ts)), *xs)
+    def leaky_relu(self, x, alpha=0.2): return self._run(lambda t: self.tf.leaky_relu(t, alpha), x)
+    def log_sigmoid(self, x): return self._run(self.tf.log_sigmoid, x)
     def sum(self, x): return self._run(lambda t: self.tf.sum(t, -1), x)
     def max(self, x): return self._run(lambda t: self.tf.max(t, -1), x)
     def min(self, x): return self._run(lambda t: self.tf.min(t, -1), x)

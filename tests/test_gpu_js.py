@@ -295,6 +295,94 @@ def test_js_mobilenet_matches_oracle(tmp_path, ref, quant):
         assert top[0] == int(np.argmax(want[0]))
 
 
+def test_js_math_ops_match_oracle(tmp_path, ref):
+    """floor ... erf, pow / mod / squaredDifference / floorDiv / atan2, prod / all / any and addN
+    through the JS host, and their gradient functions against closed forms in float64."""
+    rng = np.random.default_rng(61)
+    c = Cases(tmp_path)
+    dom = dict(asin=(-1, 1), acos=(-1, 1), atanh=(-0.99, 0.99), acosh=(1, 30), log1p=(-0.9, 30),
+               tan=(-1.4, 1.4), erf=(-2, 4))
+    js = dict(is_nan="isNaN", is_inf="isInf", is_finite="isFinite")
+    for name in ("floor", "ceil", "round", "sign", "expm1", "log1p", "reciprocal", "sin", "cos", "tan",
+                 "asin", "acos", "atan", "sinh", "cosh", "asinh", "acosh", "atanh", "erf", "elu",
+                 "selu", "softplus", "is_nan", "is_inf", "is_finite"):
+        lo, hi = dom.get(name, (-8, 8))
+        x = rng.uniform(lo, hi, (9, 13)).astype(np.float32)
+        x.ravel()[:5] = [np.nan, 0.5, 1.5, 2.5, -0.5] if name != "erf" else [np.nan, 0.5, 1.5, 2.5, 0]
+        if name.startswith("is_"):
+            x.ravel()[5:7] = [np.inf, -np.inf]
+            c.add(name, "unaryNamed", dict(x=x), dict(name=js[name]), ref.unary(name, x).astype(np.bool_),
+                  exact=True)
+        else:
+            c.add(name, "unaryNamed", dict(x=x), dict(name=name), ref.unary(name, x))
+    v = np.array([-2, 0, 3, np.nan], np.float32)
+    c.add("step", "unaryNamed", dict(x=v), dict(name="step", alpha=0.25), ref.step(v, 0.25))
+    w = (rng.standard_normal(300) * 6).astype(np.float32)
+    c.add("leaky_relu", "unaryNamed", dict(x=w), dict(name="leakyRelu", alpha=0.1), ref.leaky_relu(w, 0.1))
+    c.add("log_sigmoid", "unaryNamed", dict(x=w), dict(name="logSigmoid"), ref.log_sigmoid(w))
+    a = (np.abs(rng.standard_normal((4, 1, 5))) + 0.2).astype(np.float32)
+    b = rng.uniform(-3, 3, (3, 5)).astype(np.float32)
+    b = np.where(np.abs(b) < 0.2, np.float32(0.9), b)
+    for name, jsname in (("pow", "pow"), ("squared_difference", "squaredDifference"), ("mod", "mod"),
+                         ("floor_div", "floorDiv"), ("atan2", "atan2")):
+        c.add(name, "binaryNamed", dict(a=a, b=b), dict(name=jsname), ref.binary(name, a, b),
+              exact=name == "floor_div")
+    ai, bi = rng.integers(-9, 10, (6,)).astype(np.int32), rng.integers(1, 5, (6,)).astype(np.int32)
+    for name, jsname in (("pow", "pow"), ("mod", "mod"), ("floor_div", "floorDiv")):
+        c.add(name + "_int", "binaryNamed", dict(a=ai, b=bi), dict(name=jsname), ref.binary(name, ai, bi),
+              exact=True)
+    m = rng.uniform(0.8, 1.2, (4, 6, 5)).astype(np.float32)
+    c.add("prod_inner", "reduceNamed", dict(x=m), dict(name="prod", axis=-1), ref.reduce("prod", m))
+    c.add("prod_outer_keep", "reduceNamed", dict(x=m), dict(name="prod", axis=[0], keepDims=True),
+          np.prod(m.astype(np.float64), 0, keepdims=True).astype(np.float32))
+    bm = rng.uniform(0, 1, (5, 7)) < 0.8
+    c.add("all", "reduceNamed", dict(x=bm), dict(name="all", axis=1), ref.reduce("all", bm), exact=True)
+    c.add("any", "reduceNamed", dict(x=~bm), dict(name="any", axis=0), np.any(~bm, 0), exact=True)
+    xs = [rng.standard_normal((3, 4)).astype(np.float32) for _ in range(3)]
+    c.add("add_n", "addN", dict(a=xs[0], b=xs[1], c=xs[2]), {}, ref.add_n(xs))
+
+    # gradient functions: d/dx of each op, times dy (unary_ops.ts, relu_ops.ts, binary_ops.ts)
+    sq = lambda t: t.astype(np.float64)
+    ders = dict(
+        expm1=lambda t: np.exp(t), log1p=lambda t: 1 / (1 + t), reciprocal=lambda t: -1 / t ** 2,
+        sin=np.cos, cos=lambda t: -np.sin(t), tan=lambda t: 1 / np.cos(t) ** 2,
+        asin=lambda t: 1 / np.sqrt(1 - t ** 2), acos=lambda t: -1 / np.sqrt(1 - t ** 2),
+        atan=lambda t: 1 / (1 + t ** 2), sinh=np.cosh, cosh=np.sinh,
+        asinh=lambda t: 1 / np.sqrt(1 + t ** 2), acosh=lambda t: 1 / np.sqrt(t ** 2 - 1),
+        atanh=lambda t: 1 / (1 - t ** 2), softplus=lambda t: 1 / (1 + np.exp(-t)),
+        erf=lambda t: 2 / np.sqrt(np.pi) * np.exp(-t ** 2),
+        # eluDer of the reference (backend_cpu.ts:1227-1242): dy where y >= 1, else dy * (y + 1)
+        elu=lambda t: np.where(t >= 1, 1.0, np.where(t >= 0, t + 1, np.exp(t))),
+        selu=lambda t: np.where(t > 0, 1.0507009873554805, 1.7580993408473768 * np.exp(t)),
+        floor=lambda t: 0 * t, round=lambda t: 0 * t, sign=lambda t: 0 * t,
+        logSigmoid=lambda t: 1 / (1 + np.exp(t)))
+    gdom = dict(asin=(-0.9, 0.9), acos=(-0.9, 0.9), atanh=(-0.9, 0.9), acosh=(1.2, 9), log1p=(-0.5, 9),
+                tan=(-1.2, 1.2), reciprocal=(0.3, 4), sinh=(-4, 4), cosh=(-4, 4), expm1=(-4, 4))
+    for name, der in ders.items():
+        lo, hi = gdom.get(name, (-3, 3))
+        x = rng.uniform(lo, hi, (23,)).astype(np.float32)
+        dy = rng.uniform(-1, 1, (23,)).astype(np.float32)
+        c.add("grad_" + name, "gradUnaryNamed", dict(x=x, dy=dy), dict(name=name),
+              (der(sq(x)) * dy).astype(np.float32), atol=1e-4)
+    a = rng.uniform(0.4, 3, (4, 5)).astype(np.float32)
+    b = rng.uniform(0.5, 2.5, (5,)).astype(np.float32)
+    dy = rng.uniform(-1, 1, (4, 5)).astype(np.float32)
+    A, B, D = sq(a), sq(b), sq(dy)
+    wants = dict(
+        pow=(D * B * A ** (B - 1), (D * A ** B * np.log(A)).sum(0)),
+        squaredDifference=(D * 2 * (A - B), (D * 2 * (B - A)).sum(0)),
+        atan2=(D * B / (A ** 2 + B ** 2), (-D * A / (A ** 2 + B ** 2)).sum(0)),
+        mod=(D, (-D * np.floor(A / B)).sum(0)))
+    for name, (da, db) in wants.items():
+        c.add("grad_%s_a" % name, "gradBinaryNamed", dict(a=a, b=b, dy=dy), dict(name=name, wrt=0),
+              da.astype(np.float32), atol=1e-4)
+        c.add("grad_%s_b" % name, "gradBinaryNamed", dict(a=a, b=b, dy=dy), dict(name=name, wrt=1),
+              db.astype(np.float32), atol=1e-4)
+    results = c.run()
+    c.check(results)
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
 def test_js_backward_ops_match_oracle(tmp_path, ref):
     """conv2dDerInput / conv2dDerFilter / conv2dTranspose, the depthwise and pooling backprops
     through the JS host and the N-API addon."""

@@ -262,6 +262,102 @@ def test_unary(hip, ref, name):
     close(hip.unary(name, x.ravel()[:1000]), ref.unary(name, x.ravel()[:1000]), rtol=1e-5, atol=1e-6)
 
 
+_DOMAIN = dict(asin=(-1, 1), acos=(-1, 1), atanh=(-0.999, 0.999), acosh=(1, 50), log1p=(-0.99, 50),
+               sinh=(-20, 20), cosh=(-20, 20), expm1=(-30, 30), tan=(-1.5, 1.5))
+
+
+@pytest.mark.parametrize("name", ["floor", "ceil", "round", "sign", "expm1", "log1p", "reciprocal",
+                                  "sin", "cos", "tan", "asin", "acos", "atan", "sinh", "cosh",
+                                  "asinh", "acosh", "atanh", "erf", "elu", "selu", "softplus"])
+def test_unary_more(hip, ref, name):
+    """fp32 1e-4 relative / 1e-5 absolute against the oracle's double evaluation; NaN, the
+    infinities and values outside the function's domain behave as in the oracle."""
+    rng = np.random.default_rng(6)
+    lo, hi = _DOMAIN.get(name, (-12, 12))
+    x = rng.uniform(lo, hi, (41, 31)).astype(np.float32)
+    x.ravel()[:6] = [np.nan, np.inf, -np.inf, 0.0, -0.0, 100.0]
+    x.ravel()[6:12] = [0.5, 1.5, 2.5, -0.5, -1.5, -2.5]      # round: ties to even
+    if name == "erf":
+        x = np.clip(x, -3, 12)   # the polynomial overflows below -1 / 0.3275911
+        x.ravel()[:3] = [np.nan, np.inf, 0.25]
+    got, want = hip.unary(name, x), ref.unary(name, x)
+    assert got.dtype == np.float32
+    close(got, want, rtol=1e-4, atol=1e-5)
+    xi = rng.integers(-3, 4, 50).astype(np.int32)            # int32 storage, float32 result
+    if name not in ("acosh", "reciprocal", "log1p", "atanh", "asin", "acos"):
+        close(hip.unary(name, xi), ref.unary(name, xi.astype(np.float32)), rtol=1e-4, atol=1e-5)
+
+
+def test_step_predicates_and_composites(hip, ref):
+    x = np.array([-2, -0.0, 0.0, 3, np.nan, np.inf, -np.inf, 1e-30], np.float32)
+    for alpha in (0.0, 0.3, -2.0):
+        close(hip.step(x, alpha), ref.step(x, alpha))
+    for name in ("is_nan", "is_inf", "is_finite"):
+        got = hip.unary(name, x)
+        assert got.dtype in (np.bool_, np.uint8)
+        assert np.asarray(got).astype(int).tolist() == ref.unary(name, x).astype(int).tolist()
+    rng = np.random.default_rng(8)
+    v = (rng.standard_normal(777) * 10).astype(np.float32)
+    close(hip.leaky_relu(v, 0.1), ref.leaky_relu(v, 0.1), rtol=1e-5, atol=1e-6)
+    close(hip.log_sigmoid(v), ref.log_sigmoid(v), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("sa,sb", [((5, 7), (5, 7)), ((5, 1), (1, 7)), ((), (6,)), ((2, 3, 4), (4,))])
+@pytest.mark.parametrize("name", ["pow", "squared_difference", "mod", "floor_div", "atan2"])
+def test_binary_more(hip, ref, name, sa, sb):
+    rng = np.random.default_rng(len(sa) * 10 + len(sb))
+    a = rng.uniform(-4, 4, sa).astype(np.float32)
+    b = rng.uniform(-4, 4, sb).astype(np.float32)
+    if name == "pow":
+        a = np.abs(a) + np.float32(0.1)
+    if name in ("mod", "floor_div"):
+        b = np.where(np.abs(b) < 0.2, np.float32(0.7), b)
+    got, want = hip.binary(name, a, b), ref.binary(name, a, b)
+    assert got.dtype == want.dtype, (got.dtype, want.dtype)
+    if name == "floor_div":
+        assert np.array_equal(got, want)
+    else:
+        close(got, want, rtol=1e-4, atol=1e-5)
+    ai = rng.integers(-9, 10, sa).astype(np.int32)
+    bi = rng.integers(1, 6, sb).astype(np.int32)
+    got, want = hip.binary(name, ai, bi), ref.binary(name, ai, bi)
+    assert got.dtype == want.dtype == np.int32
+    assert np.array_equal(got, want), name
+
+
+def test_pow_mod_special_values(hip, ref):
+    a = np.array([1, -1, 1, 2, np.nan, -8, 0, 0, np.inf, -2, -2], np.float32)
+    b = np.array([np.inf, -np.inf, np.nan, 0, 0, 1 / 3, 0, -1, 2, 3, 0.5], np.float32)
+    close(hip.binary("pow", a, b), ref.binary("pow", a, b))
+    a = np.array([5, -5, 5, -5, 5.5, np.nan, 3, 0], np.float32)
+    b = np.array([3, 3, -3, -3, 2, 2, np.nan, 4], np.float32)
+    close(hip.binary("mod", a, b), ref.binary("mod", a, b))
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (37, 10), (3, 64), (5, 65), (2, 3000)])
+def test_prod_all_any(hip, ref, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = rng.uniform(0.9, 1.1, (rows, cols)).astype(np.float32)
+    x[0, cols // 2] = -1.5
+    close(hip.reduce("prod", x), ref.reduce("prod", x), rtol=1e-4, atol=1e-5)
+    xi = rng.integers(1, 3, (rows, min(cols, 20))).astype(np.int32)
+    got = hip.reduce("prod", xi)
+    assert got.dtype == np.int32 and np.array_equal(got, ref.reduce("prod", xi))
+    m = rng.uniform(0, 1, (rows, cols)) < 0.97
+    m[-1, :] = True
+    n = rng.uniform(0, 1, (rows, cols)) < 0.02
+    n[0, :] = False
+    for name, v in (("all", m), ("any", n)):
+        got = hip.reduce(name, v)
+        assert np.asarray(got).astype(bool).tolist() == ref.reduce(name, v).tolist(), name
+
+
+def test_add_n(hip, ref):
+    rng = np.random.default_rng(3)
+    xs = [rng.standard_normal((6, 5)).astype(np.float32) for _ in range(4)]
+    close(hip.add_n(xs), ref.add_n(xs), rtol=1e-6, atol=1e-6)
+
+
 def test_clip_relu6_nan(hip, ref):
     x = np.array([-3, 0, 2.5, 6, 7.5, np.nan, np.inf, -np.inf], np.float32)
     close(hip.clip(x, 0, 6), ref.clip(x, 0, 6))

@@ -47,7 +47,20 @@ __device__ __forceinline__ float bin_f(int op, float a, float b) {
     case TFHIP_GREATER: return a > b;
     case TFHIP_GREATER_EQUAL: return a >= b;
     case TFHIP_LOGICAL_AND: return (a != 0.f) && (b != 0.f);
-    default: return (a != 0.f) || (b != 0.f);
+    case TFHIP_LOGICAL_OR: return (a != 0.f) || (b != 0.f);
+    case TFHIP_POW:
+      // Math.pow: NaN exponent and (+-1) ** +-Infinity give NaN where C gives 1
+      if (b != b || (fabsf(a) == 1.f && isinf(b))) return NAN;
+      return powf(a, b);
+    case TFHIP_SQUARED_DIFFERENCE: return (a - b) * (a - b);
+    case TFHIP_MOD: {
+      const float rem = fmodf(a, b);
+      if ((a < 0.f && b < 0.f) || (a >= 0.f && b >= 0.f)) return rem;
+      return fmodf(rem + b, b);
+    }
+    case TFHIP_FLOOR_DIV: return floorf(a / b);
+    case TFHIP_ATAN2: return atan2f(a, b);
+    default: return b >= 1.f ? a : a * (b + 1.f);  // eluDer(dy, y)
   }
 }
 __device__ __forceinline__ int64_t bin_i(int op, int64_t a, int64_t b) {
@@ -104,7 +117,7 @@ __global__ void binary_kernel(int op, const void* a, int a_dt, int64_t a_len, co
         }
       }
     }
-    if (a_dt != TFHIP_FLOAT32 && b_dt != TFHIP_FLOAT32 && op != TFHIP_DIV) {
+    if (a_dt != TFHIP_FLOAT32 && b_dt != TFHIP_FLOAT32 && op != TFHIP_DIV && op < TFHIP_POW) {
       // integer arithmetic when neither operand is float (int32 / bool tensors)
       const int64_t r = bin_i(op, load_i(a, a_dt, ia), load_i(b, b_dt, ib));
       if (std::is_same<OutT, float>::value) out[i] = (OutT)r;
@@ -156,7 +169,47 @@ __device__ __forceinline__ float unary_f(int op, float v, float p0, float p1) {
     case TFHIP_SQRT: return sqrtf(v);
     case TFHIP_SQUARE: return v * v;
     case TFHIP_TANH: return tanhf(v);
-    default: return 1.f / sqrtf(v);
+    case TFHIP_RSQRT: return 1.f / sqrtf(v);
+    case TFHIP_FLOOR: return floorf(v);
+    case TFHIP_CEIL: return ceilf(v);
+    case TFHIP_ROUND: return rintf(v);  // round half to even (backend_cpu.ts:1077-1090)
+    case TFHIP_SIGN: return v < 0.f ? -1.f : (v > 0.f ? 1.f : 0.f);
+    case TFHIP_EXPM1: return expm1f(v);
+    case TFHIP_LOG1P: return log1pf(v);
+    case TFHIP_RECIPROCAL: return 1.f / v;
+    case TFHIP_SIN: return sinf(v);
+    case TFHIP_COS: return cosf(v);
+    case TFHIP_TAN: return tanf(v);
+    case TFHIP_ASIN: return asinf(v);
+    case TFHIP_ACOS: return acosf(v);
+    case TFHIP_ATAN: return atanf(v);
+    case TFHIP_SINH: return sinhf(v);
+    case TFHIP_COSH: return coshf(v);
+    case TFHIP_ASINH: return asinhf(v);
+    case TFHIP_ACOSH: return acoshf(v);
+    case TFHIP_ATANH: return atanhf(v);
+    case TFHIP_ERF: {
+      // ops/erf_util.ts:18-23, backend_cpu.ts:1509-1516 (no sign handling: as the reference)
+      const float t = 1.f / (1.f + 0.3275911f * v);
+      const float poly = ((((1.061405429f * t + -1.453152027f) * t + 1.421413741f) * t +
+                           -0.284496736f) * t + 0.254829592f) * t;
+      return 1.f - poly * expf(-v * v);
+    }
+    case TFHIP_ELU: return v >= 0.f ? v : expm1f(v);
+    case TFHIP_SELU:  // ops/selu_util.ts:18-19
+      return v >= 0.f ? 1.0507009873554804934193349852946f * v
+                      : 1.7580993408473768599402175208123f * expm1f(v);
+    case TFHIP_SOFTPLUS: {
+      // backend_cpu.ts:1326-1353: threshold = log(2^-23) + 2
+      const float threshold = -13.942385f;
+      if (v < threshold) return expf(v);
+      if (v > -threshold) return v;
+      return log1pf(expf(v));
+    }
+    case TFHIP_STEP: return v != v ? NAN : (v > 0.f ? 1.f : p0);
+    case TFHIP_IS_NAN: return v != v;
+    case TFHIP_IS_INF: return isinf(v);
+    default: return isfinite(v);
   }
 }
 
@@ -167,6 +220,7 @@ __global__ void unary_kernel(int op, const void* x, int x_dt, OutT* out, int64_t
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
     const float r = unary_f(op, load_f(x, x_dt, i), p0, p1);
     if (std::is_same<OutT, float>::value) out[i] = (OutT)r;
+    else if (sizeof(OutT) == 1) out[i] = (OutT)(r != 0.f);
     else out[i] = (OutT)to_int32(r);
   }
 }
@@ -243,8 +297,8 @@ extern "C" int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_
                             int a_rank, int64_t b, const int32_t* b_shape, int b_rank,
                             int64_t out) {
   if (!ctx) return TFHIP_EINVAL;
-  if (op < TFHIP_ADD || op > TFHIP_LOGICAL_OR) return ctx->fail(TFHIP_EINVAL, "binary: unknown op %d", op);
-  const bool predicate = op >= TFHIP_EQUAL;
+  if (op < TFHIP_ADD || op > TFHIP_ELU_DER) return ctx->fail(TFHIP_EINVAL, "binary: unknown op %d", op);
+  const bool predicate = op >= TFHIP_EQUAL && op <= TFHIP_LOGICAL_OR;
   if (a_rank < 0 || b_rank < 0 || a_rank > MAXR || b_rank > MAXR)
     return ctx->fail(TFHIP_ENOTSUP, "binary: rank above %d", MAXR);
   TFHIP_GET(ctx, ba, a);
@@ -325,12 +379,15 @@ extern "C" int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_
 
 extern "C" int tfhip_unary(tfhip_ctx* ctx, int op, int64_t x, int64_t out, float p0, float p1) {
   if (!ctx) return TFHIP_EINVAL;
-  if (op < TFHIP_RELU || op > TFHIP_RSQRT) return ctx->fail(TFHIP_EINVAL, "unary: unknown op %d", op);
+  if (op < TFHIP_RELU || op > TFHIP_IS_FINITE) return ctx->fail(TFHIP_EINVAL, "unary: unknown op %d", op);
+  const bool predicate = op >= TFHIP_IS_NAN;
   TFHIP_GET(ctx, bx, x);
   TFHIP_GET(ctx, bo, out);
   if (bx->numel != bo->numel) return ctx->fail(TFHIP_EINVAL, "unary: size mismatch");
-  if (bx->dtype == TFHIP_UINT8Q || bo->dtype == TFHIP_UINT8Q || bo->dtype == TFHIP_BOOL)
-    return ctx->fail(TFHIP_EINVAL, "unary: unsupported storage dtype");
+  if (bx->dtype == TFHIP_UINT8Q || bo->dtype == TFHIP_UINT8Q ||
+      (bo->dtype == TFHIP_BOOL) != predicate)
+    return ctx->fail(TFHIP_EINVAL, "unary: unsupported storage dtype (isNaN/isInf/isFinite write "
+                                   "bool, the others float32 or int32)");
   const int64_t n = bx->numel;
   if (n == 0) return TFHIP_OK;
   const int block = 256;
@@ -341,6 +398,9 @@ extern "C" int tfhip_unary(tfhip_ctx* ctx, int op, int64_t x, int64_t out, float
   } else if (bo->dtype == TFHIP_FLOAT32) {
     hipLaunchKernelGGL(unary_kernel<float>, dim3(grid_for(ctx, n, block)), dim3(block), 0,
                        ctx->stream, op, bx->ptr, bx->dtype, (float*)bo->ptr, n, p0, p1);
+  } else if (bo->dtype == TFHIP_BOOL) {
+    hipLaunchKernelGGL(unary_kernel<uint8_t>, dim3(grid_for(ctx, n, block)), dim3(block), 0,
+                       ctx->stream, op, bx->ptr, bx->dtype, (uint8_t*)bo->ptr, n, p0, p1);
   } else {
     hipLaunchKernelGGL(unary_kernel<int32_t>, dim3(grid_for(ctx, n, block)), dim3(block), 0,
                        ctx->stream, op, bx->ptr, bx->dtype, (int32_t*)bo->ptr, n, p0, p1);

@@ -40,6 +40,23 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void reduce_rows_kernel(
     }
     return;
   }
+  if (op == TFHIP_PROD) {
+    double s = 1.0;
+    for (int64_t j = lane; j < inner; j += WAVE) s *= (double)ld(x, x_dt, base + j);
+    for (int off = WAVE / 2; off > 0; off >>= 1) s *= __shfl_down(s, off, WAVE);
+    if (lane == 0) {
+      if (std::is_same<OutT, float>::value) out[row] = (OutT)(float)s;
+      else out[row] = (OutT)(int32_t)(uint32_t)(int64_t)s;
+    }
+    return;
+  }
+  if (op == TFHIP_ALL || op == TFHIP_ANY) {
+    int hit = 0;  // any: a non-zero element; all: a zero element
+    for (int64_t j = lane; j < inner; j += WAVE) hit |= (ld(x, x_dt, base + j) != 0.f) == (op == TFHIP_ANY);
+    for (int off = WAVE / 2; off > 0; off >>= 1) hit |= __shfl_down(hit, off, WAVE);
+    if (lane == 0) out[row] = (OutT)(op == TFHIP_ANY ? hit : !hit);
+    return;
+  }
   const bool want_max = op == TFHIP_MAX || op == TFHIP_ARGMAX;
   const float first = ld(x, x_dt, base);
   float best = first;
@@ -173,7 +190,7 @@ using namespace tfhip;
 extern "C" int tfhip_reduce(tfhip_ctx* ctx, int op, int64_t x, int64_t out, int64_t outer,
                             int64_t inner) {
   if (!ctx) return TFHIP_EINVAL;
-  if (op < TFHIP_SUM || op > TFHIP_ARGMIN) return ctx->fail(TFHIP_EINVAL, "reduce: unknown op %d", op);
+  if (op < TFHIP_SUM || op > TFHIP_ANY) return ctx->fail(TFHIP_EINVAL, "reduce: unknown op %d", op);
   TFHIP_GET(ctx, bx, x);
   TFHIP_GET(ctx, bo, out);
   if (outer < 0 || inner < 0 || bx->numel != outer * inner || bo->numel != outer)
@@ -184,10 +201,12 @@ extern "C" int tfhip_reduce(tfhip_ctx* ctx, int op, int64_t x, int64_t out, int6
   const bool arg = op == TFHIP_ARGMAX || op == TFHIP_ARGMIN;
   if (arg && bo->dtype != TFHIP_INT32)
     return ctx->fail(TFHIP_EINVAL, "reduce: argMax/argMin write int32");
-  if (bo->dtype != TFHIP_INT32 && bo->dtype != TFHIP_FLOAT32)
-    return ctx->fail(TFHIP_EINVAL, "reduce: output must be float32 or int32");
+  const bool logical = op == TFHIP_ALL || op == TFHIP_ANY;
+  if (logical ? bo->dtype != TFHIP_BOOL : (bo->dtype != TFHIP_INT32 && bo->dtype != TFHIP_FLOAT32))
+    return ctx->fail(TFHIP_EINVAL, "reduce: output must be float32 or int32 (bool for all/any)");
   if (outer == 0) return TFHIP_OK;
   if (inner == 0) {
+    if (op == TFHIP_PROD) return tfhip_fill(ctx, out, 1.0);
     if (op != TFHIP_SUM) return ctx->fail(TFHIP_EINVAL, "reduce: empty axis has no extremum");
     return tfhip_fill(ctx, out, 0.0);
   }
@@ -196,6 +215,9 @@ extern "C" int tfhip_reduce(tfhip_ctx* ctx, int op, int64_t x, int64_t out, int6
   if (bo->dtype == TFHIP_FLOAT32)
     hipLaunchKernelGGL(reduce_rows_kernel<float>, grid, block, 0, ctx->stream, op, bx->ptr,
                        bx->dtype, (float*)bo->ptr, outer, inner);
+  else if (bo->dtype == TFHIP_BOOL)
+    hipLaunchKernelGGL(reduce_rows_kernel<uint8_t>, grid, block, 0, ctx->stream, op, bx->ptr,
+                       bx->dtype, (uint8_t*)bo->ptr, outer, inner);
   else
     hipLaunchKernelGGL(reduce_rows_kernel<int32_t>, grid, block, 0, ctx->stream, op, bx->ptr,
                        bx->dtype, (int32_t*)bo->ptr, outer, inner);

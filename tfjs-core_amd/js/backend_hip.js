@@ -20,10 +20,14 @@ const ACT = {linear: 0, relu: 1, prelu: 2, relu6: 3};
 const BCAST = {NONE: 0, SCALAR: 1, COLUMN: 2, FULL: 3};
 const BINARY = {add: 0, sub: 1, mul: 2, div: 3, prelu: 4, maximum: 5, minimum: 6, equal: 7,
                 notEqual: 8, less: 9, lessEqual: 10, greater: 11, greaterEqual: 12,
-                logicalAnd: 13, logicalOr: 14};
+                logicalAnd: 13, logicalOr: 14, pow: 15, squaredDifference: 16, mod: 17,
+                floorDiv: 18, atan2: 19, eluDer: 20};
 const UNARY = {relu: 0, clip: 1, exp: 2, log: 3, neg: 4, abs: 5, sigmoid: 6, sqrt: 7, square: 8,
-               tanh: 9, rsqrt: 10};
-const REDUCE = {sum: 0, max: 1, min: 2, argMax: 3, argMin: 4};
+               tanh: 9, rsqrt: 10, floor: 11, ceil: 12, round: 13, sign: 14, expm1: 15, log1p: 16,
+               reciprocal: 17, sin: 18, cos: 19, tan: 20, asin: 21, acos: 22, atan: 23, sinh: 24,
+               cosh: 25, asinh: 26, acosh: 27, atanh: 28, erf: 29, elu: 30, selu: 31,
+               softplus: 32, step: 33, isNaN: 34, isInf: 35, isFinite: 36};
+const REDUCE = {sum: 0, max: 1, min: 2, argMax: 3, argMin: 4, prod: 5, all: 6, any: 7};
 const POOL = {avg: 0, max: 1};
 
 let addon = null;
@@ -333,6 +337,40 @@ class MathBackendHIP extends KernelBackend {
   square(x) { return this.unary('square', x); }
   tanh(x) { return this.unary('tanh', x); }
   rsqrt(x) { return this.unary('rsqrt', x); }
+  // float32 results whatever the input dtype (backend_cpu.ts:993-1030, 1071-1189, 1359-1518)
+  floor(x) { return this.unary('floor', x); }
+  ceil(x) { return this.unary('ceil', x); }
+  round(x) { return this.unary('round', x); }
+  sign(x) { return this.unary('sign', x); }
+  expm1(x) { return this.unary('expm1', x); }
+  log1p(x) { return this.unary('log1p', x); }
+  reciprocal(x) { return this.unary('reciprocal', x); }
+  sin(x) { return this.unary('sin', x); }
+  cos(x) { return this.unary('cos', x); }
+  tan(x) { return this.unary('tan', x); }
+  asin(x) { return this.unary('asin', x); }
+  acos(x) { return this.unary('acos', x); }
+  atan(x) { return this.unary('atan', x); }
+  sinh(x) { return this.unary('sinh', x); }
+  cosh(x) { return this.unary('cosh', x); }
+  asinh(x) { return this.unary('asinh', x); }
+  acosh(x) { return this.unary('acosh', x); }
+  atanh(x) { return this.unary('atanh', x); }
+  erf(x) { return this.unary('erf', x); }
+  elu(x) { return this.unary('elu', x); }
+  selu(x) { return this.unary('selu', x); }
+  softplus(x) { return this.unary('softplus', x); }
+  step(x, alpha) { return this.unary('step', x, 'float32', alpha || 0); }
+  isNaN(x) { return this.unary('isNaN', x, 'bool'); }
+  isInf(x) { return this.unary('isInf', x, 'bool'); }
+  isFinite(x) { return this.unary('isFinite', x, 'bool'); }
+  // results keep a's dtype (backend_cpu.ts:483-489, 893-904, 984-991, 1425-1431); floorDiv is int32
+  pow(a, b) { return this.binary('pow', a, b, a.dtype === 'bool' ? 'int32' : a.dtype); }
+  squaredDifference(a, b) { return this.binary('squaredDifference', a, b, a.dtype === 'bool' ? 'int32' : a.dtype); }
+  mod(a, b) { return this.binary('mod', a, b, a.dtype === 'bool' ? 'int32' : a.dtype); }
+  floorDiv(a, b) { return this.binary('floorDiv', a, b, 'int32'); }
+  atan2(a, b) { return this.binary('atan2', a, b, a.dtype === 'bool' ? 'int32' : a.dtype); }
+  eluDer(dy, y) { return this.binary('eluDer', dy, y, 'float32'); }
 
   // castTensor (backends/backend_util.ts:34-71): loss-free casts alias the same dataId.
   cast(x, dtype) {
@@ -383,6 +421,9 @@ class MathBackendHIP extends KernelBackend {
     return out;
   }
   sum(x, axes) { return this.reduce('sum', x, axes, util.upcastType(x.dtype, 'int32')); }
+  prod(x, axes) { return this.reduce('prod', x, axes, util.upcastType(x.dtype, 'int32')); }
+  all(x, axes) { return this.reduce('all', x, axes, 'bool'); }
+  any(x, axes) { return this.reduce('any', x, axes, 'bool'); }
   max(x, axes) { return this.reduce('max', x, axes, x.dtype === 'float32' ? 'float32' : 'int32'); }
   min(x, axes) { return this.reduce('min', x, axes, x.dtype === 'float32' ? 'float32' : 'int32'); }
   argMax(x, axis) { return this.reduce('argMax', x, [axis], 'int32'); }

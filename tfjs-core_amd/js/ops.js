@@ -559,12 +559,68 @@ function binaryOp(name, method) {
     }, {$a, $b}, g == null ? null : (dy, saved) => g(dy, saved[0], saved[1]));
   });
 }
+// (pow, squaredDifference, atan2, mod: binary_ops.ts:254-276, 547-565, 751-757, 808-829)
+Object.assign(BINARY_GRADS, {
+  squaredDifference: (dy, a, b) => ({
+    $a: () => unbroadcast(mul(dy, mul(sub(a, b), scalar(2))), a.shape),
+    $b: () => unbroadcast(mul(dy, mul(sub(b, a), scalar(2))), b.shape)
+  }),
+  atan2: (dy, a, b) => ({
+    $a: () => unbroadcast(mul(dy, div(b, add(square(a), square(b)))), a.shape),
+    $b: () => unbroadcast(mul(dy, neg(div(a, add(square(a), square(b))))), b.shape)
+  }),
+  mod: (dy, a, b) => ({
+    $a: () => unbroadcast(dy, a.shape),
+    $b: () => unbroadcast(mul(dy, neg(floor(div(a, b)))), b.shape)
+  })
+});
 const add = binaryOp('add', 'add');
 const sub = binaryOp('sub', 'subtract');
 const mul = binaryOp('mul', 'multiply');
 const div = binaryOp('div', 'realDivide');
 const maximum = binaryOp('maximum', 'maximum');
 const minimum = binaryOp('minimum', 'minimum');
+
+const squaredDifference = binaryOp('squaredDifference', 'squaredDifference');
+const mod = binaryOp('mod', 'mod');
+const floorDiv = binaryOp('floorDiv', 'floorDiv');
+const atan2 = binaryOp('atan2', 'atan2');
+// binary_ops.ts:246-282: the kernel sees the operands as given; the result has base's dtype
+const pow = op('pow', (base, exponent) => {
+  const $base = convertToTensor(base, 'base', 'pow');
+  const $exp = convertToTensor(exponent, 'exp', 'pow');
+  broadcast_util.assertAndGetBroadcastShape($base.shape, $exp.shape);
+  return ENGINE.runKernel((backend, save) => {
+    const y = backend.pow($base, $exp);
+    save([$base, $exp, y]);
+    return y;
+  }, {$base, $exp}, (dy, saved) => {
+    const [b, e, y] = saved;
+    return {
+      $base: () => {
+        const ef = cast(e, 'float32');
+        return unbroadcast(mul(dy, mul(ef, pow(b, sub(ef, scalar(1))))), b.shape);
+      },
+      $exp: () => {
+        const logBase = where(greater(b, scalar(0)), log(cast(b, 'float32')), zerosLike(cast(b, 'float32')));
+        return unbroadcast(mul(dy, mul(y, logBase)), e.shape);
+      }
+    };
+  });
+});
+// binary_ops.ts:97-133
+const addN = op('addN', tensors => {
+  util.assert(Array.isArray(tensors), () => 'The argument passed to tf.addN() must be a list of tensors');
+  util.assert(tensors.length >= 1,
+              () => `Must pass at least one tensor to tf.addN(), but got ${tensors.length}`);
+  const $tensors = tensors.map((t, i) => convertToTensor(t, `tensors${i}`, 'addN'));
+  $tensors.forEach(t => {
+    if (t.dtype !== $tensors[0].dtype) throw new Error('All tensors passed to tf.addN() must have the same dtype');
+    if (!util.arraysEqual(t.shape, $tensors[0].shape)) throw new Error('All tensors passed to tf.addN() must have the same shape');
+  });
+  if ($tensors.length === 1) return clone($tensors[0]);
+  return ENGINE.tidy(() => $tensors.slice(1).reduce((acc, t) => add(acc, t), $tensors[0]));
+});
 
 const prelu = op('prelu', (x, alpha) => {
   const $x = convertToTensor(x, 'x', 'prelu');
@@ -594,6 +650,33 @@ function unaryOp(name, method) {
     }, {$x}, g == null ? null : (dy, saved) => ({$x: () => g(dy, saved[0], saved[1])}));
   });
 }
+// unary_ops.ts:88-188 (ceil, floor, sign, round: zero gradient), :229-348 (expm1, log1p,
+// reciprocal), :377-400 (softplus), :490-740 (trigonometric and hyperbolic functions),
+// relu_ops.ts:58-95 (elu, selu)
+const SELU_SCALEALPHA = 1.7580993408473768599402175208123, SELU_SCALE = 1.0507009873554804934193349852946;
+Object.assign(UNARY_GRADS, {
+  floor: dy => zerosLike(dy), ceil: dy => zerosLike(dy), round: dy => zerosLike(dy),
+  sign: dy => zerosLike(dy),
+  expm1: (dy, x) => mul(dy, exp(x)),
+  log1p: (dy, x) => div(dy, add(x, scalar(1))),
+  reciprocal: (dy, x) => div(dy, neg(square(x))),
+  sin: (dy, x) => mul(cos(cast(x, 'float32')), dy),
+  cos: (dy, x) => mul(neg(sin(cast(x, 'float32'))), dy),
+  tan: (dy, x) => div(dy, square(cos(x))),
+  asin: (dy, x) => div(dy, sqrt(sub(scalar(1), square(cast(x, 'float32'))))),
+  acos: (dy, x) => neg(div(dy, sqrt(sub(scalar(1), square(cast(x, 'float32')))))),
+  atan: (dy, x) => div(dy, add(square(cast(x, 'float32')), scalar(1))),
+  sinh: (dy, x) => mul(cosh(cast(x, 'float32')), dy),
+  cosh: (dy, x) => mul(sinh(cast(x, 'float32')), dy),
+  asinh: (dy, x) => div(dy, sqrt(add(scalar(1), square(cast(x, 'float32'))))),
+  acosh: (dy, x) => div(dy, sqrt(sub(square(cast(x, 'float32')), scalar(1)))),
+  atanh: (dy, x) => div(dy, sub(scalar(1), square(cast(x, 'float32')))),
+  softplus: (dy, x) => mul(dy, sigmoid(x)),
+  erf: (dy, x) => mul(dy, mul(exp(neg(square(x))), scalar(2 / Math.sqrt(Math.PI)))),
+  elu: (dy, x, y) => ENGINE.runKernel(backend => backend.eluDer(dy, y), {dy, y}),
+  selu: (dy, x) => where(greater(x, scalar(0)), mul(dy, scalar(SELU_SCALE)),
+                         mul(mul(dy, scalar(SELU_SCALEALPHA)), exp(cast(x, 'float32'))))
+});
 const relu = unaryOp('relu');
 const exp = unaryOp('exp');
 const log = unaryOp('log');
@@ -604,6 +687,56 @@ const sqrt = unaryOp('sqrt');
 const square = unaryOp('square');
 const tanh = unaryOp('tanh');
 const rsqrt = unaryOp('rsqrt');
+const floor = unaryOp('floor');
+const ceil = unaryOp('ceil');
+const round = unaryOp('round');
+const sign = unaryOp('sign');
+const expm1 = unaryOp('expm1');
+const log1p = unaryOp('log1p');
+const reciprocal = unaryOp('reciprocal');
+const sin = unaryOp('sin');
+const cos = unaryOp('cos');
+const tan = unaryOp('tan');
+const asin = unaryOp('asin');
+const acos = unaryOp('acos');
+const atan = unaryOp('atan');
+const sinh = unaryOp('sinh');
+const cosh = unaryOp('cosh');
+const asinh = unaryOp('asinh');
+const acosh = unaryOp('acosh');
+const atanh = unaryOp('atanh');
+const elu = unaryOp('elu');
+const selu = unaryOp('selu');
+const softplus = unaryOp('softplus');
+const isNaN_ = unaryOp('isNaN');
+const isInf = unaryOp('isInf');
+const isFinite_ = unaryOp('isFinite');
+// unary_ops.ts:864-885
+const erfOp = unaryOp('erf');
+const erf = op('erf', x => {
+  const $x = convertToTensor(x, 'x', 'erf');
+  util.assert($x.dtype === 'int32' || $x.dtype === 'float32', () => 'Input dtype must be `int32` or `float32`.');
+  return erfOp($x.dtype === 'int32' ? cast($x, 'float32') : $x);
+});
+// unary_ops.ts:909-924: the gradient is zero everywhere
+const step = op('step', (x, alpha) => {
+  const $x = convertToTensor(x, 'x', 'step');
+  return ENGINE.runKernel(backend => backend.step($x, alpha == null ? 0 : alpha), {$x},
+                          dy => ({$x: () => zerosLike(dy)}));
+});
+// relu_ops.ts:104-108
+const leakyRelu = op('leakyRelu', (x, alpha) => {
+  const $x = convertToTensor(x, 'x', 'leakyRelu');
+  return maximum(mul(scalar(alpha == null ? 0.2 : alpha), $x), $x);
+});
+// unary_ops.ts:326-339: -softplus(-x) with gradient dy * sigmoid(-x)
+const logSigmoid = op('logSigmoid', x => {
+  const $x = convertToTensor(x, 'x', 'logSigmoid');
+  return ENGINE.customGrad(t => ({
+    value: neg(softplus(neg(t))),
+    gradFunc: dy => mul(dy, sigmoid(neg(t)))
+  }))($x);
+});
 
 const clipByValue = op('clipByValue', (x, clipValueMin, clipValueMax) => {
   const $x = convertToTensor(x, 'x', 'clipByValue');
@@ -623,7 +756,10 @@ const relu6 = op('relu6', x => clipByValue(x, 0, 6));
 function reduceOp(name, method) {
   return op(name, (x, axis, keepDims) => {
     let $x = convertToTensor(x, 'x', name);
-    if (name === 'sum' && $x.dtype === 'bool') $x = cast($x, 'int32');
+    if ((name === 'sum' || name === 'prod') && $x.dtype === 'bool') $x = cast($x, 'int32');
+    if (name === 'all' || name === 'any') {  // reduction_ops.ts:366-429
+      util.assert($x.dtype === 'bool', () => `Error Tensor must be of type bool. Got: ${$x.dtype}`);
+    }
     const origAxes = util.parseAxisParam(axis, $x.shape);
     let axes = origAxes;
     const permutedAxes = axis_util.getAxesPermutation(axes, $x.rank);
@@ -638,7 +774,7 @@ function reduceOp(name, method) {
       const y = backend[method](reduceInput, axes);
       save([reduceInput, y]);
       return y;
-    }, {$x: reduceInput}, (dy, saved) => ({
+    }, {$x: reduceInput}, ['sum', 'max', 'min'].indexOf(name) === -1 ? null : (dy, saved) => ({
       // reduction_ops.ts:163-172 (sum: dy spread over the axes), :41-52 (max / min: dy where
       // the element equals the extremum)
       $x: () => name === 'sum' ?
@@ -652,6 +788,9 @@ function reduceOp(name, method) {
   });
 }
 const sum = reduceOp('sum', 'sum');
+const prod = reduceOp('prod', 'prod');
+const all = reduceOp('all', 'all');
+const any = reduceOp('any', 'any');
 const max = reduceOp('max', 'max');
 const min = reduceOp('min', 'min');
 
@@ -1121,5 +1260,8 @@ module.exports = {
   greater, greaterEqual, logicalAnd, logicalOr, logicalNot, batchNorm, resizeBilinear,
   conv2dDerInput, conv2dDerFilter, conv2dTranspose, depthwiseConv2dDerInput,
   depthwiseConv2dDerFilter, maxPoolBackprop, avgPoolBackprop, resizeNearestNeighbor, where, mean,
-  expandDims, squeeze, stack, unstack, split
+  expandDims, squeeze, stack, unstack, split,
+  floor, ceil, round, sign, expm1, log1p, reciprocal, sin, cos, tan, asin, acos, atan, sinh, cosh,
+  asinh, acosh, atanh, erf, elu, selu, softplus, step, leakyRelu, logSigmoid, isNaN: isNaN_, isInf,
+  isFinite: isFinite_, pow, squaredDifference, mod, floorDiv, atan2, addN, prod, all, any
 };

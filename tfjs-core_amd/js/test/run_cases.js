@@ -64,6 +64,12 @@ const OPS = {
   tile: (i, a) => tf.tile(i.x, a.reps),
   oneHot: (i, a) => tf.oneHot(i.indices, a.depth, a.onValue, a.offValue),
   compare: (i, a) => tf[a.name](i.a, i.b),
+  unaryNamed: (i, a) => tf[a.name](i.x, a.alpha),
+  binaryNamed: (i, a) => tf[a.name](i.a, i.b),
+  reduceNamed: (i, a) => tf[a.name](i.x, a.axis, a.keepDims),
+  addN: i => tf.addN([i.a, i.b, i.c]),
+  gradUnaryNamed: (i, a) => tf.grad(x => tf[a.name](x, a.alpha))(i.x, i.dy),
+  gradBinaryNamed: (i, a) => tf.grads((p, q) => tf[a.name](p, q))([i.a, i.b], i.dy)[a.wrt],
   logicalNot: i => tf.logicalNot(i.x),
   batchNorm: (i, a) => tf.batchNorm(i.x, i.mean, i.variance, i.offset, i.scale, a.varianceEpsilon),
   resizeBilinear: (i, a) => tf.resizeBilinear(i.x, a.size, a.alignCorners),

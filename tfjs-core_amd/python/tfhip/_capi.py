@@ -10,10 +10,14 @@ FLOAT32, INT32, BOOL, UINT8Q = 0, 1, 2, 3
 ACT = {"linear": 0, None: 0, "relu": 1, "prelu": 2, "relu6": 3}
 BCAST_NONE, BCAST_SCALAR, BCAST_COLUMN, BCAST_FULL = 0, 1, 2, 3
 BINARY = dict(add=0, sub=1, mul=2, div=3, prelu=4, maximum=5, minimum=6, equal=7, not_equal=8,
-              less=9, less_equal=10, greater=11, greater_equal=12, logical_and=13, logical_or=14)
+              less=9, less_equal=10, greater=11, greater_equal=12, logical_and=13, logical_or=14,
+              pow=15, squared_difference=16, mod=17, floor_div=18, atan2=19, elu_der=20)
 UNARY = dict(relu=0, clip=1, exp=2, log=3, neg=4, abs=5, sigmoid=6, sqrt=7, square=8, tanh=9,
-             rsqrt=10)
-REDUCE = dict(sum=0, max=1, min=2, argmax=3, argmin=4)
+             rsqrt=10, floor=11, ceil=12, round=13, sign=14, expm1=15, log1p=16, reciprocal=17,
+             sin=18, cos=19, tan=20, asin=21, acos=22, atan=23, sinh=24, cosh=25, asinh=26,
+             acosh=27, atanh=28, erf=29, elu=30, selu=31, softplus=32, step=33, is_nan=34,
+             is_inf=35, is_finite=36)
+REDUCE = dict(sum=0, max=1, min=2, argmax=3, argmin=4, prod=5, all=6, any=7)
 POOL = dict(avg=0, max=1)
 
 

@@ -354,6 +354,43 @@ class MathBackendHIP(object):
     def tanh(self, x): return self._unary("tanh", x)
     def rsqrt(self, x): return self._unary("rsqrt", x)
 
+    # float32 results whatever the input dtype (backend_cpu.ts:993-1030, 1071-1189, 1359-1518)
+    def floor(self, x): return self._unary("floor", x)
+    def ceil(self, x): return self._unary("ceil", x)
+    def round(self, x): return self._unary("round", x)
+    def sign(self, x): return self._unary("sign", x)
+    def expm1(self, x): return self._unary("expm1", x)
+    def log1p(self, x): return self._unary("log1p", x)
+    def reciprocal(self, x): return self._unary("reciprocal", x)
+    def sin(self, x): return self._unary("sin", x)
+    def cos(self, x): return self._unary("cos", x)
+    def tan(self, x): return self._unary("tan", x)
+    def asin(self, x): return self._unary("asin", x)
+    def acos(self, x): return self._unary("acos", x)
+    def atan(self, x): return self._unary("atan", x)
+    def sinh(self, x): return self._unary("sinh", x)
+    def cosh(self, x): return self._unary("cosh", x)
+    def asinh(self, x): return self._unary("asinh", x)
+    def acosh(self, x): return self._unary("acosh", x)
+    def atanh(self, x): return self._unary("atanh", x)
+    def erf(self, x): return self._unary("erf", x)
+    def elu(self, x): return self._unary("elu", x)
+    def selu(self, x): return self._unary("selu", x)
+    def softplus(self, x): return self._unary("softplus", x)
+    def step(self, x, alpha=0.0): return self._unary("step", x, "float32", float(alpha))
+    def is_nan(self, x): return self._unary("is_nan", x, "bool")
+    def is_inf(self, x): return self._unary("is_inf", x, "bool")
+    def is_finite(self, x): return self._unary("is_finite", x, "bool")
+
+    # results keep a's dtype (backend_cpu.ts:483-489, 893-904, 984-991, 1425-1431); floorDiv is int32
+    def _a_dtype(self, a): return "int32" if a.dtype == "bool" else a.dtype
+    def pow(self, a, b): return self._binary("pow", a, b, self._a_dtype(a))
+    def squared_difference(self, a, b): return self._binary("squared_difference", a, b, self._a_dtype(a))
+    def mod(self, a, b): return self._binary("mod", a, b, self._a_dtype(a))
+    def floor_div(self, a, b): return self._binary("floor_div", a, b, "int32")
+    def atan2(self, a, b): return self._binary("atan2", a, b, self._a_dtype(a))
+    def elu_der(self, dy, y): return self._binary("elu_der", dy, y, "float32")
+
     def cast(self, x, dtype):
         """castTensor (backends/backend_util.ts:34-71): widening casts alias the data id."""
         if dtype == x.dtype:
@@ -412,6 +449,15 @@ class MathBackendHIP(object):
 
     def sum(self, x, axes):
         return self._reduce("sum", x, axes, su.upcast_type(x.dtype, "int32"))
+
+    def prod(self, x, axes):
+        return self._reduce("prod", x, axes, su.upcast_type(x.dtype, "int32"))
+
+    def all(self, x, axes):
+        return self._reduce("all", x, axes, "bool")
+
+    def any(self, x, axes):
+        return self._reduce("any", x, axes, "bool")
 
     def max(self, x, axes):
         return self._reduce("max", x, axes, "float32" if x.dtype == "float32" else "int32")

@@ -7,6 +7,7 @@ import builtins
 from . import shape_util as su
 
 builtins_sum = builtins.sum
+builtins_any = builtins.any
 from .engine import ENGINE, NP_DTYPE, Tensor
 
 
@@ -285,6 +286,95 @@ sqrt = _unary("sqrt")
 square = _unary("square")
 tanh = _unary("tanh")
 rsqrt = _unary("rsqrt")
+# ops/unary_ops.ts: floor :108, ceil :88, round :188, sign :128, expm1 :229, log1p :270,
+# reciprocal :348, sin :490, cos :508, tan :527, asin :546, acos :567, atan :590, sinh :609,
+# cosh :631, asinh :675, acosh :696, atanh :718, elu (ops/relu_ops.ts:58), selu (:81),
+# softplus :377, isNaN :149, isInf :165, isFinite :181
+floor = _unary("floor")
+ceil = _unary("ceil")
+round = _unary("round")  # noqa: A001  (tf.round: half to even)
+sign = _unary("sign")
+expm1 = _unary("expm1")
+log1p = _unary("log1p")
+reciprocal = _unary("reciprocal")
+sin = _unary("sin")
+cos = _unary("cos")
+tan = _unary("tan")
+asin = _unary("asin")
+acos = _unary("acos")
+atan = _unary("atan")
+sinh = _unary("sinh")
+cosh = _unary("cosh")
+asinh = _unary("asinh")
+acosh = _unary("acosh")
+atanh = _unary("atanh")
+elu = _unary("elu")
+selu = _unary("selu")
+softplus = _unary("softplus")
+is_nan = _unary("is_nan")
+is_inf = _unary("is_inf")
+is_finite = _unary("is_finite")
+
+
+def erf(x):
+    """ops/unary_ops.ts:864-885: int32 or float32 only."""
+    x = _conv(x, "x", "erf")
+    if x.dtype not in ("int32", "float32"):
+        raise ValueError("Input dtype must be `int32` or `float32`.")
+    return ENGINE.run_kernel(lambda be: be.erf(x))
+
+
+def step(x, alpha=0.0):
+    """ops/unary_ops.ts:909-924."""
+    x = _conv(x, "x", "step")
+    return ENGINE.run_kernel(lambda be: be.step(x, alpha))
+
+
+def leaky_relu(x, alpha=0.2):
+    """ops/relu_ops.ts:104-108: maximum(alpha * x, x)."""
+    x = _conv(x, "x", "leakyRelu")
+    return ENGINE.tidy(lambda: maximum(mul(tensor(np.float32(alpha)), x), x))
+
+
+def log_sigmoid(x):
+    """ops/unary_ops.ts:326-339: -softplus(-x)."""
+    x = _conv(x, "x", "logSigmoid")
+    return ENGINE.tidy(lambda: neg(softplus(neg(x))))
+
+
+def pow(base, exp):  # noqa: A001
+    """ops/binary_ops.ts:246-282: the kernel sees the operands as given; result in base's dtype."""
+    base, exp = _conv(base, "base", "pow"), _conv(exp, "exp", "pow")
+    su.broadcast_shape(base.shape, exp.shape)
+    return ENGINE.run_kernel(lambda be: be.pow(base, exp))
+
+
+def squared_difference(a, b): return _binary("squaredDifference", "squared_difference", a, b)
+def mod(a, b): return _binary("mod", "mod", a, b)
+def floor_div(a, b): return _binary("floorDiv", "floor_div", a, b)
+def atan2(a, b): return _binary("atan2", "atan2", a, b)
+
+
+def add_n(tensors):
+    """ops/binary_ops.ts:97-133: same dtype and shape for all."""
+    if not isinstance(tensors, (list, tuple)) or len(tensors) < 1:
+        raise ValueError("Must pass at least one tensor to tf.addN(), but got %d"
+                         % (len(tensors) if isinstance(tensors, (list, tuple)) else 0))
+    ts = [_conv(t, "tensors%d" % i, "addN") for i, t in enumerate(tensors)]
+    for t in ts:
+        if t.dtype != ts[0].dtype:
+            raise ValueError("All tensors passed to tf.addN() must have the same dtype")
+        if list(t.shape) != list(ts[0].shape):
+            raise ValueError("All tensors passed to tf.addN() must have the same shape")
+    if len(ts) == 1:
+        return reshape(ts[0], ts[0].shape)
+
+    def run():
+        acc = ts[0]
+        for t in ts[1:]:
+            acc = add(acc, t)
+        return acc
+    return ENGINE.tidy(run)
 
 
 def clip_by_value(x, lo, hi):
@@ -324,6 +414,30 @@ def sum(x, axis=None, keep_dims=False):  # noqa: A001
     if xt.dtype == "bool":
         xt = cast(xt, "int32")
     return _reduce("sum", xt, axis, keep_dims)
+
+
+def prod(x, axis=None, keep_dims=False):
+    """ops/reduction_ops.ts:166-199."""
+    xt = _conv(x, "x", "prod")
+    if xt.dtype == "bool":
+        xt = cast(xt, "int32")
+    return _reduce("prod", xt, axis, keep_dims)
+
+
+def all(x, axis=None, keep_dims=False):  # noqa: A001
+    """ops/reduction_ops.ts:366-384: bool only."""
+    xt = _conv(x, "x", "all")
+    if xt.dtype != "bool":
+        raise ValueError("Error Tensor must be of type bool. Got: %s" % xt.dtype)
+    return _reduce("all", xt, axis, keep_dims)
+
+
+def any(x, axis=None, keep_dims=False):  # noqa: A001
+    """ops/reduction_ops.ts:411-429: bool only."""
+    xt = _conv(x, "x", "any")
+    if xt.dtype != "bool":
+        raise ValueError("Error Tensor must be of type bool. Got: %s" % xt.dtype)
+    return _reduce("any", xt, axis, keep_dims)
 
 
 def max(x, axis=None, keep_dims=False):  # noqa: A001
@@ -522,7 +636,7 @@ def strided_slice(x, begin, end, strides=None, begin_mask=0, end_mask=0, ellipsi
         x.shape, list(begin), list(end), list(strides), begin_mask, end_mask, ellipsis_mask,
         new_axis_mask, shrink_axis_mask)
     shape = [d for i, d in enumerate(size) if i not in shrink]
-    if any(d == 0 for d in shape):
+    if builtins_any(d == 0 for d in shape):
         return tensor(np.zeros(shape, NP_DTYPE[x.dtype]), shape, x.dtype)
 
     def run():
