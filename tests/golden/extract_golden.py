@@ -72,6 +72,13 @@ CASES = {
     "binary_extra": ("tfjs-core/src/ops/binary_ops_test.ts",
                      ["squaredDifference", "mod", "atan2"]),
     "arithmetic_extra": ("tfjs-core/src/ops/arithmetic_test.ts", ["pow", "addN"]),
+    "optimizer_sgd": ("tfjs-core/src/optimizers/sgd_optimizer_test.ts", None),
+    "optimizer_momentum": ("tfjs-core/src/optimizers/momentum_optimizer_test.ts", None),
+    "optimizer_adagrad": ("tfjs-core/src/optimizers/adagrad_optimizer_test.ts", None),
+    "optimizer_adadelta": ("tfjs-core/src/optimizers/adadelta_optimizer_test.ts", None),
+    "optimizer_adam": ("tfjs-core/src/optimizers/adam_optimizer_test.ts", None),
+    "optimizer_adamax": ("tfjs-core/src/optimizers/adamax_optimizer_test.ts", None),
+    "optimizer_rmsprop": ("tfjs-core/src/optimizers/rmsprop_optimizer_test.ts", None),
     "reduction_extra": ("tfjs-core/src/ops/reduction_ops_test.ts",
                         ["Reduction: prod", "Reduction: all", "Reduction: any",
                          "Reduction: moments", "Reduction: norm"]),

@@ -383,6 +383,77 @@ def test_js_math_ops_match_oracle(tmp_path, ref):
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
 
 
+def _optimizer_reference(name, args, x, w, t, steps):
+    """The update rules of tfjs-core/src/optimizers/*_optimizer.ts in float64 (closed forms of
+    the published algorithms; epsilon 1e-7 as KernelBackend.epsilon() gives for float32)."""
+    x = x.astype(np.float64).copy()
+    st = {}
+    eps = 1e-7
+    for it in range(steps):
+        g = 2 * (x * w - t) * w
+        if name == "sgd":
+            x -= args[0] * g
+        elif name == "momentum":
+            lr, m = args[0], args[1]
+            nesterov = len(args) > 2 and args[2]
+            st["a"] = m * st.get("a", 0) + g
+            x -= lr * ((g + m * st["a"]) if nesterov else st["a"])
+        elif name == "adagrad":
+            st["a"] = st.get("a", args[1]) + g * g
+            x -= args[0] * g / np.sqrt(st["a"] + eps)
+        elif name == "adadelta":
+            lr, rho = args
+            ag, au = st.get("g", 0 * x), st.get("u", 0 * x)
+            upd = np.sqrt(au + eps) / np.sqrt(ag + eps) * g
+            st["g"] = rho * ag + (1 - rho) * g * g
+            st["u"] = rho * au + (1 - rho) * upd * upd
+            x -= lr * upd
+        elif name == "adam":
+            lr, b1, b2 = args
+            st["m"] = b1 * st.get("m", 0) + (1 - b1) * g
+            st["v"] = b2 * st.get("v", 0) + (1 - b2) * g * g
+            mh, vh = st["m"] / (1 - b1 ** (it + 1)), st["v"] / (1 - b2 ** (it + 1))
+            x -= lr * mh / (np.sqrt(vh) + eps)
+        elif name == "adamax":
+            lr, b1, b2, _, decay = args
+            st["m"] = b1 * st.get("m", 0) + (1 - b1) * g
+            st["v"] = np.maximum(b2 * st.get("v", 0 * x), np.abs(g))
+            x -= lr / (1 + decay * it) / (1 - b1 ** (it + 1)) * st["m"] / (st["v"] + eps)
+        elif name == "rmsprop":
+            lr, decay, mom, e, centered = args
+            st["r"] = decay * st.get("r", 0) + (1 - decay) * g * g
+            if centered:
+                st["g"] = decay * st.get("g", 0) + (1 - decay) * g
+                den = np.sqrt(st["r"] - (st["g"] ** 2 + e))
+            else:
+                den = np.sqrt(st["r"] + e)
+            st["m"] = mom * st.get("m", 0) + lr * g / den
+            x -= st["m"]
+    return x.astype(np.float32)
+
+
+def test_js_optimizers_on_the_gpu(tmp_path):
+    """tf.train.* on the hip backend: five steps on a 2000-element least-squares problem against
+    the float64 update rules; no tensor or device buffer is left behind."""
+    rng = np.random.default_rng(71)
+    c = Cases(tmp_path)
+    x = rng.uniform(-1, 1, (40, 50)).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, (40, 50)).astype(np.float32)
+    t = rng.uniform(-1, 1, (40, 50)).astype(np.float32)
+    for tag, name, args in (("sgd", "sgd", [0.05]), ("momentum", "momentum", [0.05, 0.6]),
+                            ("nesterov", "momentum", [0.05, 0.6, True]), ("adagrad", "adagrad", [0.1, 0.1]),
+                            ("adadelta", "adadelta", [0.5, 0.9]), ("adam", "adam", [0.05, 0.8, 0.9]),
+                            ("adamax", "adamax", [0.05, 0.8, 0.9, None, 0.1]),
+                            ("rmsprop", "rmsprop", [0.02, 0.9, 0.3, 1e-7, False]),
+                            ("rmsprop_centered", "rmsprop", [0.02, 0.9, 0.3, 1e-7, True])):
+        want = _optimizer_reference(name, args, x, w.astype(np.float64), t.astype(np.float64), 5)
+        c.add(tag, "optimizerSteps", dict(x=x, w=w, t=t), dict(name=name, args=args, steps=5), want,
+              rtol=1e-3, atol=1e-4)
+    results = c.run()
+    c.check(results)
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
 def test_js_backward_ops_match_oracle(tmp_path, ref):
     """conv2dDerInput / conv2dDerFilter / conv2dTranspose, the depthwise and pooling backprops
     through the JS host and the N-API addon."""

@@ -6,7 +6,7 @@
 // :502-572, memory/profile :588-622, write/read :833-877, tape and gradients :435-498,
 // 628-774, customGrad :776-831 (the tape algorithm itself is in tape.js).
 const util = require('./util');
-const {Tensor, setTensorTracker} = require('./tensor');
+const {Tensor, Variable, setTensorTracker} = require('./tensor');
 const {Profiler} = require('./profiler');
 const {ENV} = require('./environment');
 const {getFilteredNodesXToY, backpropagateGradients} = require('./tape');
@@ -22,6 +22,8 @@ class Engine {
     this.profiler = null;
     this.state = this.freshState();
     this.tensorId = 0;
+    this.variableId = 0;
+    this.registeredVariables = {};
   }
 
   freshState() {
@@ -418,7 +420,23 @@ class Engine {
       owner.register(a.dataId, a.shape, dt);
     }
     this.state.tensorInfo.get(a.dataId).refCount++;
-    this.track(a);
+    if (!Variable.constructing) this.track(a);  // engine.ts:654-656: variables outlive scopes
+  }
+
+  // ---- variables (engine.ts:660-673, 600-611) -----------------------------------------
+  nextVariableId() { return this.variableId++; }
+  registerVariable(v) {
+    if (this.registeredVariables[v.name] != null) {
+      throw new Error(`Variable with name ${v.name} was already registered`);
+    }
+    this.registeredVariables[v.name] = v;
+  }
+  disposeVariable(v) {
+    this.disposeTensor(v);
+    if (this.registeredVariables[v.name] === v) delete this.registeredVariables[v.name];
+  }
+  disposeVariables() {
+    Object.keys(this.registeredVariables).forEach(name => this.registeredVariables[name].dispose());
   }
 
   disposeTensor(a) {

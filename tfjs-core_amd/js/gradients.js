@@ -1,9 +1,8 @@
 'use strict';
 // tf.grad / tf.grads / tf.valueAndGrad / tf.valueAndGrads / tf.customGrad, after
-// tfjs-core/src/gradients.ts:30-388 (same argument checks and messages; variableGrads is
-// not built: this host has no Variable).
+// tfjs-core/src/gradients.ts:30-388 (same argument checks and messages).
 const {ENGINE} = require('./engine');
-const {Tensor} = require('./tensor');
+const {Tensor, Variable} = require('./tensor');
 const util = require('./util');
 const ops = require('./ops');
 
@@ -22,6 +21,36 @@ function checkGrads(grads) {
     throw new Error(`Cannot compute gradient of y=f(x) with respect to x. Make sure that
     the f you passed encloses all operations that lead from x to y.`);
   }
+}
+
+// d f() / d variable for every trainable variable of varList (default: all registered ones),
+// keyed by variable name; f must return a scalar (gradients.ts:268-350).
+function variableGrads(f, varList) {
+  util.assert(typeof f === 'function', () => 'The f passed in variableGrads(f) must be a function');
+  util.assert(varList == null || (Array.isArray(varList) && varList.every(v => v instanceof Variable)),
+              () => 'The varList passed in variableGrads(f, varList) must be an array of variables');
+  const given = varList != null;
+  if (!given) varList = Object.keys(ENGINE.registeredVariables).map(n => ENGINE.registeredVariables[n]);
+  const frozen = given ? varList.filter(v => !v.trainable) : null;
+  const count = varList.length;
+  varList = varList.filter(v => v.trainable);
+  util.assert(varList.length > 0,
+              () => `variableGrads() expects at least one of the input variables to be trainable, ` +
+                  `but none of the ${count} variables is trainable.`);
+  const {value, grads} = ENGINE.gradients(f, varList, null, true, TAPE_OPS);
+  util.assert(grads.some(g => g != null),
+              () => 'Cannot find a connection between any variable and the result of the loss ' +
+                  'function y=f(x). Please make sure the operations that use variables are inside ' +
+                  'the function f passed to minimize().');
+  util.assert(value.rank === 0,
+              () => `The f passed in variableGrads(f) must return a scalar, but it returned a ` +
+                  `rank-${value.rank} tensor`);
+  const named = {};
+  varList.forEach((v, i) => {
+    if (grads[i] != null) named[v.name] = grads[i];
+  });
+  if (frozen != null) frozen.forEach(v => named[v.name] = null);
+  return {value, grads: named};
 }
 
 function grad(f) {
@@ -93,4 +122,4 @@ function customGrad(f) {
   return ENGINE.customGrad(f);
 }
 
-module.exports = {grad, grads, valueAndGrad, valueAndGrads, customGrad};
+module.exports = {grad, grads, valueAndGrad, valueAndGrads, customGrad, variableGrads};

@@ -5,7 +5,7 @@
 // (tfjs-backend-wasm/src/backend_wasm.ts:154-157): tf.registerBackend('hip', factory, 3).
 const {ENGINE} = require('./engine');
 const {ENV} = require('./environment');
-const {Tensor} = require('./tensor');
+const {Tensor, Variable} = require('./tensor');
 const {KernelBackend, DataStorage} = require('./backend');
 const ops = require('./ops');
 const util = require('./util');
@@ -14,9 +14,12 @@ const broadcast_util = require('./broadcast_util');
 const axis_util = require('./axis_util');
 const io = Object.assign({}, require('./io_utils'), require('./weights_loader'));
 const gradients = require('./gradients');
+const optimizers = require('./optimizers');
 
 const tf = Object.assign({}, ops, gradients, {
-  Tensor, KernelBackend, DataStorage, ENV, util, io,
+  Tensor, Variable, KernelBackend, DataStorage, ENV, util, io,
+  train: optimizers.train, Optimizer: optimizers.Optimizer,
+  variable: (initialValue, trainable, name, dtype) => Variable.variable(initialValue, trainable, name, dtype),
   backend_util: Object.assign({}, conv_util, broadcast_util, axis_util),
   engine: () => ENGINE,
   registerBackend: (name, factory, priority) => ENGINE.registerBackend(name, factory, priority),
@@ -37,7 +40,7 @@ const tf = Object.assign({}, ops, gradients, {
   time: f => ENGINE.time(f),
   profile: f => ENGINE.profile(f),
   enableDebugMode: () => ENV.set('DEBUG', true),
-  disposeVariables: () => {},
+  disposeVariables: () => ENGINE.disposeVariables(),
 });
 
 ENGINE.registerBackend('hip', () => {

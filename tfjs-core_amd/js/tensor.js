@@ -112,6 +112,59 @@ class Tensor {
   toString() { return `Tensor(shape=[${this.shape}], dtype=${this.dtype})`; }
 }
 
+// A mutable tensor: a name in the engine's variable registry over a buffer that assign()
+// swaps (tensor.ts:1467-1552).  Variables are not tracked by tidy scopes.
+class Variable extends Tensor {
+  constructor(initialValue, trainable, name) {
+    Variable.constructing = true;   // registerTensor must not put it into the active scope
+    try {
+      super(initialValue.shape, initialValue.dtype, null, initialValue.dataId);
+    } finally {
+      Variable.constructing = false;
+    }
+    this.trainable = trainable == null ? true : trainable;
+    this.name = name != null ? name : engine().nextVariableId().toString();
+    try {
+      engine().registerVariable(this);
+    } catch (ex) {
+      engine().disposeTensor(this);
+      throw ex;
+    }
+  }
+  static variable(initialValue, trainable, name, dtype) {
+    if (dtype != null && dtype !== initialValue.dtype) initialValue = initialValue.asType(dtype);
+    return new Variable(initialValue, trainable, name);
+  }
+  assign(newValue) {
+    if (newValue.dtype !== this.dtype) {
+      throw new Error(`dtype of the new value (${newValue.dtype}) and ` +
+                      `previous value (${this.dtype}) must match`);
+    }
+    if (!util.arraysEqual(newValue.shape, this.shape)) {
+      throw new Error(`shape of the new value (${newValue.shape}) and ` +
+                      `previous value (${this.shape}) must match`);
+    }
+    engine().disposeTensor(this);
+    this.dataId = newValue.dataId;
+    Variable.constructing = true;
+    try {
+      engine().registerTensor(this);
+    } finally {
+      Variable.constructing = false;
+    }
+  }
+  dispose() {
+    if (this.isDisposedInternal) return;
+    engine().disposeVariable(this);
+    this.isDisposedInternal = true;
+  }
+}
+Variable.constructing = false;
+Tensor.prototype.variable = function(trainable, name, dtype) {
+  this.throwIfDisposed();
+  return Variable.variable(this, trainable, name, dtype);
+};
+
 function toNestedArray(shape, a) {
   if (shape.length === 0) return a[0];
   const size = shape.reduce((acc, c) => acc * c, 1);
@@ -126,4 +179,4 @@ function toNestedArray(shape, a) {
   return rec(0, shape);
 }
 
-module.exports = {Tensor, setTensorTracker, setOpHandler, computeStrides};
+module.exports = {Tensor, Variable, setTensorTracker, setOpHandler, computeStrides};

@@ -300,6 +300,10 @@ class ArithBackend extends StorageBackend {
   square(x) { return this.map(x, v => v * v); }
   exp(x) { return this.map(x, v => Math.exp(v)); }
   relu(x) { return this.map(x, v => Math.max(0, v)); }
+  sqrt(x) { return this.map(x, v => Math.sqrt(v)); }
+  abs(x) { return this.map(x, v => Math.abs(v)); }
+  maximum(a, b) { return this.zip(a, b, (p, q) => Math.max(p, q)); }
+  zerosLike(x) { return this.fill(x.shape, 0, x.dtype); }
   greater(a, b) {
     const r = this.zip(a, b, (p, q) => p > q ? 1 : 0);
     return Tensor.make(r.shape, {dataId: r.dataId}, 'bool', this);
@@ -312,7 +316,7 @@ class ArithBackend extends StorageBackend {
     return this.make(shape, new Float32Array(shape.reduce((a, b) => a * b, 1)).fill(value), dtype);
   }
   sum(x, axes) {
-    util.assert(axes.length === x.rank, 'ArithBackend.sum reduces every axis');
+    assert.strictEqual(axes.length, x.rank, 'ArithBackend.sum reduces every axis');
     return this.make([], Float32Array.of(Array.from(this.readSync(x.dataId)).reduce((a, b) => a + b, 0)));
   }
 }
@@ -392,6 +396,99 @@ test('tape: customGrad value / gradFunc / save, no leaks (gradients_test.ts:192-
     assert.strictEqual(tf.memory().numTensors, before + 1);
     y.dispose();
     assert.throws(() => tf.customGrad(t => ({value: 3, gradFunc: d => d}))(a), /`obj.value` is a tensor/);
+  });
+});
+
+// Known answers of tfjs-core/src/optimizers/*_optimizer_test.ts ('basic' blocks): the start
+// value and x after one and two steps of minimising sum(x^2), from tests/golden/optimizer_*.json;
+// the constructor arguments are those of the blocks (lines cited per optimizer).
+function goldenOptimizer(name, title) {
+  const file = path.join(__dirname, '..', '..', '..', 'tests', 'golden', `optimizer_${name}.json`);
+  const found = JSON.parse(fs.readFileSync(file, 'utf8')).cases.filter(c => c.title === title);
+  assert.strictEqual(found.length, 1, `${name}: ${title}`);
+  return found[0].arrays;
+}
+
+test('variables: registry, assign, tidy keeps them, variableGrads (variable_test.ts, gradients.ts:268-350)', async () => {
+  await withBackend('arith-var', new ArithBackend(), async () => {
+    const before = tf.memory().numTensors;
+    const v = tf.tidy(() => tf.variable(tf.tensor1d([1, 2, 3]), true, 'host-test-v'));
+    assert.strictEqual(tf.memory().numTensors, before + 1);     // the initial value went with the scope
+    assert.strictEqual(tf.engine().registeredVariables['host-test-v'], v);
+    assert.throws(() => tf.tidy(() => tf.variable(tf.scalar(1), true, 'host-test-v')), /already registered/);
+    tf.tidy(() => v.assign(tf.tensor1d([4, 5, 6])));
+    closeTo(v.dataSync(), [4, 5, 6]);
+    assert.strictEqual(tf.memory().numTensors, before + 1);
+    assert.throws(() => tf.tidy(() => v.assign(tf.tensor1d([1, 2]))), /shape of the new value/);
+    assert.throws(() => tf.tidy(() => v.assign(tf.tensor1d([1, 2, 3], 'int32'))), /dtype of the new value/);
+    const frozen = tf.scalar(2).variable(false, 'host-test-frozen');
+    const {value, grads} = tf.variableGrads(() => tf.sum(tf.mul(tf.square(v), frozen)));
+    closeTo(value.dataSync(), [2 * (16 + 25 + 36)]);
+    assert.deepStrictEqual(Object.keys(grads), ['host-test-v']);
+    closeTo(grads['host-test-v'].dataSync(), [16, 20, 24]);
+    assert.throws(() => tf.variableGrads(() => tf.sum(tf.square(v)), [frozen]), /none of the 1 variables is trainable/);
+    assert.throws(() => tf.variableGrads(() => tf.square(v)), /must return a scalar/);
+    tf.dispose([value, grads]);
+    tf.disposeVariables();
+    assert.strictEqual(Object.keys(tf.engine().registeredVariables).length, 0);
+    assert.strictEqual(v.isDisposed, true);
+  });
+});
+
+test('optimizers: two steps each against the reference vectors, tensor counts (optimizers/*_test.ts)', async () => {
+  await withBackend('arith-opt', new ArithBackend(), async () => {
+    const cases = [
+      // [fixture, block, factory]  (constructor arguments: the const lines of each block)
+      ['momentum', 'basic', () => tf.train.momentum(0.1, 0.5)],                   // :24-26
+      ['momentum', 'basic - with Nesterov', () => tf.train.momentum(0.1, 0.5, true)],   // :71-74
+      // (its second vector carries a slip of the reference's hand calculation, checked there
+      // at 1e-2 for that reason, adagrad_optimizer_test.ts:53-60)
+      ['adagrad', 'basic', () => tf.train.adagrad(0.1, 0.1), 1e-2],               // :24-26
+      ['adadelta', 'basic', () => tf.train.adadelta(0.1, 0.95)],                  // :24-26
+      ['adam', 'basic', () => tf.train.adam(0.1, 0.8, 0.9)],                      // :24-27
+      ['adamax', 'basic', () => tf.train.adamax(0.1, 0.8, 0.9, undefined, 0.1)],  // :24-29
+      ['rmsprop', 'Save and load weigths: centered = false', () => tf.train.rmsprop(0.1, 0.95, 0.1)],  // :152-155
+      ['rmsprop', 'Save, load weigths and continue training: centered = true',
+       () => tf.train.rmsprop(0.1, 0.95, 0.1, 1e-8, true)]                        // :84-88
+    ];
+    for (const [name, title, make, eps2] of cases) {
+      const [start, after1, after2] = goldenOptimizer(name, title);
+      const opt = make();
+      const x = tf.tensor1d(start).variable();
+      const f = () => tf.sum(tf.square(x));
+      let count = tf.memory().numTensors;
+      let cost = opt.minimize(f, true);
+      const slots = opt.getSlotVariables().length;
+      assert.strictEqual(tf.memory().numTensors, count + 1 + slots, `${name}: cost and slots only`);
+      closeTo(x.dataSync(), after1, 1e-3);
+      closeTo(cost.dataSync(), [start[0] * start[0] + start[1] * start[1]], 1e-3);
+      cost.dispose();
+      count = tf.memory().numTensors;
+      cost = opt.minimize(f, false);
+      assert.strictEqual(cost, null);
+      assert.strictEqual(tf.memory().numTensors, count, `${name}: a step allocates nothing that stays`);
+      closeTo(x.dataSync(), after2, eps2 || 1e-3);
+      assert.strictEqual(opt.iterations, 2);
+      x.dispose();
+      opt.dispose();
+    }
+    // SGD (sgd_optimizer_test.ts:24-56): x = 4, lr = 0.1, cost x^2
+    const opt = tf.train.sgd(0.1);
+    const x = tf.scalar(4).variable();
+    const count = tf.memory().numTensors;
+    const cost = opt.minimize(() => tf.square(x), true);
+    assert.strictEqual(tf.memory().numTensors, count + 1);
+    closeTo(x.dataSync(), [-2 * 4 * 0.1 + 4]);
+    closeTo(cost.dataSync(), [16]);
+    opt.minimize(() => tf.square(x));
+    closeTo(x.dataSync(), [-2 * 3.2 * 0.1 + 3.2]);
+    // varList restricts the update; a variable off the path keeps its value
+    const y = tf.scalar(7).variable();
+    opt.minimize(() => tf.add(tf.square(x), tf.square(y)), false, [x]);
+    closeTo(y.dataSync(), [7]);
+    assert.throws(() => tf.train.sgd(0.1).minimize(() => tf.scalar(3)), /Cannot find a connection/);
+    tf.dispose([cost]);
+    tf.disposeVariables();
   });
 });
 

@@ -64,6 +64,16 @@ const OPS = {
   tile: (i, a) => tf.tile(i.x, a.reps),
   oneHot: (i, a) => tf.oneHot(i.indices, a.depth, a.onValue, a.offValue),
   compare: (i, a) => tf[a.name](i.a, i.b),
+  // a.steps of minimising sum((x * w - t)^2) over the variable made from i.x
+  optimizerSteps: (i, a) => {
+    const x = i.x.variable();
+    const opt = tf.train[a.name].apply(null, a.args);
+    for (let k = 0; k < a.steps; k++) opt.minimize(() => tf.sum(tf.square(tf.sub(tf.mul(x, i.w), i.t))));
+    const out = tf.add(x, tf.scalar(0));
+    x.dispose();
+    opt.dispose();
+    return out;
+  },
   unaryNamed: (i, a) => tf[a.name](i.x, a.alpha),
   binaryNamed: (i, a) => tf[a.name](i.a, i.b),
   reduceNamed: (i, a) => tf[a.name](i.x, a.axis, a.keepDims),
