@@ -222,6 +222,17 @@ int tfhip_strided_copy(tfhip_ctx* ctx, int64_t x, int64_t out, int rank, const i
                        const int64_t* x_strides, int64_t x_offset, const int64_t* out_strides,
                        int64_t out_offset);
 
+/* cumsum along the innermost axis (backend.ts:240-242; backend_cpu.ts:714-745): x viewed as
+ * [outer, inner]; out float32 or int32 (upcastType(x.dtype, 'int32')). */
+int tfhip_cumsum(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t outer, int64_t inner,
+                 int exclusive, int reverse);
+/* localResponseNormalization4D and LRNGrad (backend.ts:600-610; backend_cpu.ts:3211-3281) over
+ * [pixels, channels] float32: the window is the channels within depth_radius of each one. */
+int tfhip_lrn(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t pixels, int channels,
+              int depth_radius, float bias, float alpha, float beta);
+int tfhip_lrn_grad(tfhip_ctx* ctx, int64_t dy, int64_t x, int64_t y, int64_t dx, int64_t pixels,
+                   int channels, int depth_radius, float bias, float alpha, float beta);
+
 /* ---- further forward kernels of converter graphs ---------------------------------------- */
 /* logicalNot (backend.ts:225; backend_cpu.ts:795-804): bool -> bool. */
 int tfhip_logical_not(tfhip_ctx* ctx, int64_t x, int64_t out);

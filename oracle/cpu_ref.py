@@ -788,3 +788,54 @@ def mean(x, n_axes=None):
     n_axes = x.ndim if n_axes is None else n_axes
     count = int(np.prod(x.shape[x.ndim - n_axes:])) if n_axes else 1
     return sum_(real_divide(x, np.float32(count)), n_axes)
+
+
+def cumsum(x, exclusive=False, reverse=False):
+    """backend_cpu.ts:714-745 along the innermost axis: every partial sum is stored into the
+    result array (Float32Array / Int32Array) before the next one is formed."""
+    x = np.asarray(x)
+    dt = np.float32 if x.dtype == np.float32 else np.int32
+    src = x.astype(dt)
+    if reverse:
+        src = src[..., ::-1]
+    out = np.zeros(src.shape, dt)
+    n = src.shape[-1] if src.ndim else 0
+    with np.errstate(over="ignore", invalid="ignore"):
+        for j in range(n):
+            if j == 0:
+                out[..., 0] = 0 if exclusive else src[..., 0]
+            else:
+                prev = out[..., j - 1].astype(np.float64)
+                term = (src[..., j - 1] if exclusive else src[..., j]).astype(np.float64)
+                out[..., j] = _store(term + prev, dt)
+    return out[..., ::-1].copy() if reverse else out
+
+
+def local_response_normalization(x, depth_radius=5, bias=1.0, alpha=1.0, beta=0.5):
+    """backend_cpu.ts:3211-3244 on NHWC (any leading dims): doubles, one Float32Array store."""
+    x = _f32(x)
+    c = x.shape[-1]
+    x64 = x.astype(np.float64)
+    sq = x64 * x64
+    out = np.empty_like(x64)
+    for ch in range(c):
+        lo, hi = max(0, ch - depth_radius), min(ch + depth_radius, c - 1)
+        s = sq[..., lo:hi + 1].sum(-1)
+        out[..., ch] = x64[..., ch] * np.power(bias + alpha * s, -beta)
+    return out.astype(np.float32)
+
+
+def lrn_grad(dy, x, y, depth_radius=5, bias=1.0, alpha=1.0, beta=0.5):
+    """backend_cpu.ts:3246-3281: scatter of every output channel's term over its window."""
+    dy64, x64, y64 = (np.asarray(a, np.float32).astype(np.float64) for a in (dy, x, y))
+    c = x64.shape[-1]
+    res = np.zeros_like(x64)
+    for o in range(c):
+        lo, hi = max(0, o - depth_radius), min(c, o + depth_radius + 1)
+        norm = alpha * (x64[..., lo:hi] ** 2).sum(-1) + bias
+        for k in range(lo, hi):
+            d = -2 * alpha * beta * x64[..., k] * y64[..., o] / norm
+            if k == o:
+                d = d + np.power(norm, -beta)
+            res[..., k] += d * dy64[..., o]
+    return res.astype(np.float32)

@@ -72,6 +72,11 @@ CASES = {
     "binary_extra": ("tfjs-core/src/ops/binary_ops_test.ts",
                      ["squaredDifference", "mod", "atan2"]),
     "arithmetic_extra": ("tfjs-core/src/ops/arithmetic_test.ts", ["pow", "addN"]),
+    "lrn": ("tfjs-core/src/ops/lrn_test.ts", ["localResponseNormalization with Tensor3D",
+                                              "localResponseNormalization with Tensor4D"]),
+    "cumsum": ("tfjs-core/src/ops/array_ops_test.ts", ["cumsum"]),
+    "space_batch_depth": ("tfjs-core/src/ops/array_ops_test.ts",
+                          ["batchToSpaceND", "spaceToBatchND", "depthToSpace"]),
     "optimizer_sgd": ("tfjs-core/src/optimizers/sgd_optimizer_test.ts", None),
     "optimizer_momentum": ("tfjs-core/src/optimizers/momentum_optimizer_test.ts", None),
     "optimizer_adagrad": ("tfjs-core/src/optimizers/adagrad_optimizer_test.ts", None),

@@ -1146,3 +1146,46 @@ def add_n_prod_all_any_known_answers(ops):
             v = _typed(a[k], None, np.bool_)[None]
             want = bool(np.all(v)) if name == "all" else bool(np.any(v))
             assert bool(np.asarray(ops.reduce(name, v))[0]) == want
+
+
+# ---- ops/lrn_test.ts, ops/array_ops_test.ts (cumsum) ---------------------------------------
+@recipe
+def lrn_known_answers(ops):
+    d3, d4 = "localResponseNormalization with Tensor3D", "localResponseNormalization with Tensor4D"
+    # TensorFlow's tf.nn.lrn(t, depth_radius=2) on the same input (lrn_test.ts:158-226, 334-470)
+    c = golden_case("lrn", "yields same result as tensorflow", d3)
+    x, want = f32(c["arrays"][0]), f32(c["arrays"][1])
+    expect_close(ops.lrn(x[None], 2)[0], want)
+    c = golden_case("lrn", "yields same result as tensorflow", d4)
+    expect_close(ops.lrn(f32(c["arrays"][0]), 2), f32(c["arrays"][1]))
+    c = golden_case("lrn", "yields same result as tensorflow with inner most dims of odd shape", d4)
+    expect_close(ops.lrn(f32(c["arrays"][0]), 2), f32(c["arrays"][1]))
+    # the closed form the spec writes out (lrn_test.ts:52-70): x / sqrt(1 + sum of squares)
+    c = golden_case("lrn", "computes simple normalization across channels", d3)
+    x = f32(c["arrays"][0]).reshape(1, 1, 1, 4)   # [1, 20, 300, 4]
+    v = x.ravel().astype(np.float64)
+    want = [v[0] / np.sqrt(1 + v[0] ** 2 + v[1] ** 2), v[1] / np.sqrt(1 + v[0] ** 2 + v[1] ** 2 + v[2] ** 2),
+            v[2] / np.sqrt(1 + v[1] ** 2 + v[2] ** 2 + v[3] ** 2), v[3] / np.sqrt(1 + v[2] ** 2 + v[3] ** 2)]
+    expect_close(ops.lrn(x, 1, 1, 1, 0.5).ravel(), want)
+    for beta in (1.0, 0.75):
+        want_b = [v[0] * (1 + v[0] ** 2 + v[1] ** 2) ** -beta, v[1] * (1 + v[0] ** 2 + v[1] ** 2 + v[2] ** 2) ** -beta,
+                  v[2] * (1 + v[1] ** 2 + v[2] ** 2 + v[3] ** 2) ** -beta, v[3] * (1 + v[2] ** 2 + v[3] ** 2) ** -beta]
+        expect_close(ops.lrn(x, 1, 1, 1, beta).ravel(), want_b)
+
+
+@recipe
+def cumsum_known_answers(ops):
+    g = lambda t: golden_case("cumsum", t, "cumsum")["arrays"]
+    for t, kw in (("1D standard", {}), ("1D reverse", dict(reverse=True)),
+                  ("1D exclusive", dict(exclusive=True)),
+                  ("1D exclusive reverse", dict(exclusive=True, reverse=True))):
+        a = g(t)
+        expect_close(ops.cumsum(f32(a[0]), 0, **kw), a[2])
+    a = g("2D standard")
+    expect_close(ops.cumsum(f32(a[0]), 1), a[2])
+    a = g("2D reverse exclusive")
+    expect_close(ops.cumsum(f32(a[0]), 1, exclusive=True, reverse=True), a[2])
+    a = g("2D axis=0")
+    expect_close(ops.cumsum(f32(a[0]), 0), a[2])
+    a = g("3D standard")
+    expect_close(ops.cumsum(f32(a[0]), 2), a[2])

@@ -115,6 +115,17 @@ class OracleOps:
     def unary(self, name, x): return self.r._unary(name, x)
     def step(self, x, alpha=0.0): return self.r.unary("step", x, alpha)
 
+    def cumsum(self, x, axis=0, exclusive=False, reverse=False):
+        x = np.asarray(x)
+        moved = np.moveaxis(x, axis, -1)
+        return np.moveaxis(self.r.cumsum(moved, exclusive, reverse), -1, axis)
+
+    def lrn(self, x, radius=5, bias=1.0, alpha=1.0, beta=0.5):
+        return self.r.local_response_normalization(x, radius, bias, alpha, beta)
+
+    def lrn_grad(self, dy, x, y, radius=5, bias=1.0, alpha=1.0, beta=0.5):
+        return self.r.lrn_grad(dy, x, y, radius, bias, alpha, beta)
+
     def binary(self, name, a, b):
         fn = dict(pow=self.r.pow_, squared_difference=self.r.squared_difference, mod=self.r.mod,
                   floor_div=self.r.floor_div, atan2=self.r.atan2)[name]
@@ -297,6 +308,15 @@ class HipOps:
     def log(self, x): return self._run(self.tf.log, x)
     def unary(self, name, x): return self._run(getattr(self.tf, name), x)
     def step(self, x, alpha=0.0): return self._run(lambda t: self.tf.step(t, alpha), x)
+
+    def cumsum(self, x, axis=0, exclusive=False, reverse=False):
+        return self._run(lambda t: self.tf.cumsum(t, axis, exclusive, reverse), x)
+
+    def lrn(self, x, radius=5, bias=1.0, alpha=1.0, beta=0.5):
+        return self._run(lambda t: self.tf.local_response_normalization(t, radius, bias, alpha, beta), x)
+
+    def lrn_grad(self, dy, x, y, radius=5, bias=1.0, alpha=1.0, beta=0.5):
+        return self._run(lambda d, a, b: self.tf.lrn_grad(d, a, b, radius, bias, alpha, beta), dy, x, y)
     def binary(self, name, a, b): return self._run(getattr(self.tf, name), a, b)
     def reduce(self, name, x): return self._run(lambda t: getattr(self.tf, name)(t, -1), x)
     def add_n(self, xs): return self._run(lambda *ts: self.tf.add_n(list(ts)), *xs)

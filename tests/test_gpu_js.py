@@ -454,6 +454,59 @@ def test_js_optimizers_on_the_gpu(tmp_path):
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
 
 
+def test_js_scan_lrn_and_rearrangements(tmp_path, ref):
+    """cumsum and localResponseNormalization (kernels + gradients) against the oracle, and
+    batchToSpaceND / spaceToBatchND / depthToSpace against the reference's own vectors
+    (array_ops_test.ts) through the JS host."""
+    rng = np.random.default_rng(83)
+    c = Cases(tmp_path)
+    x = rng.standard_normal((3, 70, 4)).astype(np.float32)
+    for axis, ex, rev in ((1, False, False), (1, True, True), (2, False, True), (0, True, False)):
+        c.add("cumsum_%d_%d_%d" % (axis, ex, rev), "cumsum", dict(x=x), dict(axis=axis, exclusive=ex, reverse=rev),
+              ref.cumsum(x, axis, ex, rev), atol=1e-4)
+    dy = rng.standard_normal(x.shape).astype(np.float32)
+    # d cumsum: the scan of dy from the other end (array_ops.ts:718-723)
+    c.add("cumsum_grad", "gradCumsum", dict(x=x, dy=dy), dict(axis=1, exclusive=False, reverse=False),
+          ref.cumsum(dy, 1, False, True), atol=1e-4)
+    xi = rng.integers(-40, 40, (6, 33)).astype(np.int32)
+    c.add("cumsum_int", "cumsum", dict(x=xi), dict(axis=1), ref.cumsum(xi, 1), exact=True)
+    img = rng.uniform(-2, 2, (2, 6, 5, 24)).astype(np.float32)
+    attrs = dict(radius=2, bias=2.0, alpha=1e-2, beta=0.75)
+    y = ref.lrn(img, 2, 2.0, 1e-2, 0.75)
+    c.add("lrn", "lrn", dict(x=img), attrs, y)
+    c.add("lrn_rank3", "lrn", dict(x=img[0]), attrs, y[0])
+    dyi = rng.uniform(-1, 1, img.shape).astype(np.float32)
+    c.add("lrn_grad", "gradLrn", dict(x=img, dy=dyi), attrs, ref.lrn_grad(dyi, img, y, 2, 2.0, 1e-2, 0.75))
+    flat = lambda a: np.asarray(a, np.float32).ravel()
+    for describe, op, key in (("batchToSpaceND", "batchToSpaceND", "crops"),
+                              ("spaceToBatchND", "spaceToBatchND", "paddings")):
+        for k, case in enumerate(cc for cc in _golden_all("space_batch_depth") if cc["describe"] == describe):
+            a = case["arrays"]
+            if len(a) != 6 or a[0] is None:
+                continue
+            c.add("%s_%d" % (op, k), op, dict(x=flat(a[0]).reshape(a[1])), {"blockShape": a[2], key: a[3]},
+                  flat(a[5]).reshape(a[4]), exact=True)
+    for k, case in enumerate(cc for cc in _golden_all("space_batch_depth") if cc["describe"] == "depthToSpace"):
+        a = case["arrays"]
+        xin = np.asarray(a[0], np.float32)
+        c.add("depthToSpace_%d" % k, "depthToSpace", dict(x=xin), dict(blockSize=2), flat(a[2]).reshape(a[1]),
+              exact=True)
+    # and at a size where the blocks are not trivial, against numpy's own reshuffle
+    big = rng.standard_normal((2, 5, 7, 36)).astype(np.float32)
+    want = big.reshape(2, 5, 7, 3, 3, 4).transpose(0, 1, 3, 2, 4, 5).reshape(2, 15, 21, 4)
+    c.add("depthToSpace_big", "depthToSpace", dict(x=big), dict(blockSize=3), want, exact=True)
+    sp = rng.standard_normal((3, 7, 10, 5)).astype(np.float32)
+    padded = np.pad(sp, ((0, 0), (1, 0), (0, 2), (0, 0)))
+    s2b = padded.reshape(3, 4, 2, 4, 3, 5).transpose(2, 4, 0, 1, 3, 5).reshape(18, 4, 4, 5)
+    c.add("spaceToBatch_big", "spaceToBatchND", dict(x=sp), dict(blockShape=[2, 3], paddings=[[1, 0], [0, 2]]),
+          s2b, exact=True)
+    c.add("batchToSpace_big", "batchToSpaceND", dict(x=s2b), dict(blockShape=[2, 3], crops=[[1, 0], [0, 2]]),
+          sp, exact=True)
+    results = c.run()
+    c.check(results)
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
 def test_js_backward_ops_match_oracle(tmp_path, ref):
     """conv2dDerInput / conv2dDerFilter / conv2dTranspose, the depthwise and pooling backprops
     through the JS host and the N-API addon."""
@@ -493,6 +546,11 @@ def test_js_backward_ops_match_oracle(tmp_path, ref):
     results = c.run()
     c.check(results)
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
+def _golden_all(name):
+    with open(os.path.join(os.path.dirname(__file__), "golden", name + ".json")) as fh:
+        return json.load(fh)["cases"]
 
 
 def _golden(name, title, describe=None):

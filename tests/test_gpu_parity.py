@@ -358,6 +358,32 @@ def test_add_n(hip, ref):
     close(hip.add_n(xs), ref.add_n(xs), rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("shape,axis", [((7,), 0), ((5, 64), 1), ((3, 65, 4), 1), ((2, 3, 1000), 2),
+                                        ((4, 6, 5), 0)])
+@pytest.mark.parametrize("exclusive,reverse", [(False, False), (True, False), (False, True), (True, True)])
+def test_cumsum(hip, ref, shape, axis, exclusive, reverse):
+    rng = np.random.default_rng(sum(shape) + axis)
+    x = rng.standard_normal(shape).astype(np.float32)
+    close(hip.cumsum(x, axis, exclusive, reverse), ref.cumsum(x, axis, exclusive, reverse),
+          rtol=1e-4, atol=1e-4)
+    xi = rng.integers(-50, 50, shape).astype(np.int32)
+    got = hip.cumsum(xi, axis, exclusive, reverse)
+    assert got.dtype == np.int32 and np.array_equal(got, ref.cumsum(xi, axis, exclusive, reverse))
+
+
+@pytest.mark.parametrize("shape,radius,bias,alpha,beta", [
+    ((2, 5, 7, 16), 2, 1.0, 1e-4, 0.75), ((1, 3, 3, 8), 5, 1.0, 1.0, 0.5), ((3, 4, 4, 1), 1, 2.0, 0.5, 1.0),
+    ((2, 9, 9, 96), 2, 2.0, 2e-5, 0.75), ((1, 2, 2, 5), 0, 1.0, 1.0, 0.5)])
+def test_local_response_normalization_and_gradient(hip, ref, shape, radius, bias, alpha, beta):
+    rng = np.random.default_rng(shape[-1] + radius)
+    x = rng.uniform(-2, 2, shape).astype(np.float32)
+    y = ref.lrn(x, radius, bias, alpha, beta)
+    close(hip.lrn(x, radius, bias, alpha, beta), y, rtol=1e-4, atol=1e-5)
+    dy = rng.uniform(-1, 1, shape).astype(np.float32)
+    close(hip.lrn_grad(dy, x, y, radius, bias, alpha, beta), ref.lrn_grad(dy, x, y, radius, bias, alpha, beta),
+          rtol=1e-4, atol=1e-5)
+
+
 def test_clip_relu6_nan(hip, ref):
     x = np.array([-3, 0, 2.5, 6, 7.5, np.nan, np.inf, -np.inf], np.float32)
     close(hip.clip(x, 0, 6), ref.clip(x, 0, 6))

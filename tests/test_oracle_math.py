@@ -237,3 +237,42 @@ def test_pool_backprops(ops, fsize, stride, dil):
     dxs = ops.avg_pool_backprop(np.ones((1, 3, 3, 1), np.float32), np.zeros((1, 3, 3, 1), np.float32),
                                 2, 1, "same")
     assert np.allclose(dxs.ravel(), np.array([1, 2, 2, 2, 4, 4, 2, 4, 4]) / 4.0)
+
+
+def test_lrn_gradient_is_the_derivative_of_the_forward_pass(oracle):
+    """LRNGrad restated from backend_cpu.ts:3246-3281 against central differences of the forward
+    restatement evaluated in float64 (numpy), which a wrong window bound or sign would miss."""
+    from oracle import cpu_ref as r
+    rng = np.random.default_rng(12)
+    radius, bias, alpha, beta = 2, 1.5, 0.3, 0.75
+    x = rng.uniform(-1, 1, (1, 2, 2, 7)).astype(np.float32)
+    dy = rng.uniform(-1, 1, x.shape).astype(np.float32)
+
+    def fwd64(v):
+        out = np.empty_like(v)
+        c = v.shape[-1]
+        for ch in range(c):
+            lo, hi = max(0, ch - radius), min(ch + radius, c - 1)
+            out[..., ch] = v[..., ch] * (bias + alpha * (v[..., lo:hi + 1] ** 2).sum(-1)) ** -beta
+        return out
+    x64 = x.astype(np.float64)
+    want = np.zeros_like(x64)
+    eps = 1e-6
+    for idx in np.ndindex(*x.shape):
+        p, m = x64.copy(), x64.copy()
+        p[idx] += eps
+        m[idx] -= eps
+        want[idx] = ((fwd64(p) - fwd64(m)) / (2 * eps) * dy).sum()
+    y = r.local_response_normalization(x, radius, bias, alpha, beta)
+    np.testing.assert_allclose(y, fwd64(x64), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(r.lrn_grad(dy, x, y, radius, bias, alpha, beta), want, rtol=1e-4, atol=1e-5)
+
+
+def test_cumsum_matches_numpy_in_all_four_modes(oracle):
+    from oracle import cpu_ref as r
+    rng = np.random.default_rng(13)
+    x = rng.integers(-9, 9, (3, 11)).astype(np.int32)
+    assert np.array_equal(r.cumsum(x), np.cumsum(x, -1))
+    assert np.array_equal(r.cumsum(x, reverse=True), np.cumsum(x[:, ::-1], -1)[:, ::-1])
+    assert np.array_equal(r.cumsum(x, exclusive=True), np.cumsum(x, -1) - x)
+    assert np.array_equal(r.cumsum(x, True, True), np.cumsum(x[:, ::-1], -1)[:, ::-1] - x)

@@ -380,6 +380,57 @@ __global__ void global_avgpool_kernel(const float* x, float* y, int n_img, int h
   reinterpret_cast<f32x4*>(y)[gid] = f32x4{(float)(s0 / d), (float)(s1 / d), (float)(s2 / d), (float)(s3 / d)};
 }
 
+// localResponseNormalization4D (backend_cpu.ts:3211-3244): out = x * (bias + alpha * sum of
+// x^2 over the channels within depth_radius of this one) ^ -beta.  One lane per element; the
+// window of neighbouring lanes overlaps, so the loads come out of L1.
+__global__ void lrn_kernel(const float* __restrict__ x, float* __restrict__ out, int64_t n,
+                           int channels, int radius, float bias, float alpha, float beta) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const int c = (int)(i % channels);
+    const int64_t px = i - c;
+    const int lo = c - radius > 0 ? c - radius : 0;
+    const int hi = c + radius < channels - 1 ? c + radius : channels - 1;
+    float sum = 0.f;
+    for (int k = lo; k <= hi; k++) {
+      const float z = x[px + k];
+      sum += z * z;
+    }
+    out[i] = x[i] * powf(bias + alpha * sum, -beta);
+  }
+}
+
+// LRNGrad (backend_cpu.ts:3246-3281), gathered: element k collects, from every channel o of its
+// pixel whose window holds k, dy[o] * (-2 alpha beta x[k] y[o] / norm[o] + [o == k] norm[o]^-beta)
+// with norm[o] = bias + alpha * sum of x^2 over the window of o.
+__global__ void lrn_grad_kernel(const float* __restrict__ dy, const float* __restrict__ x,
+                                const float* __restrict__ y, float* __restrict__ dx, int64_t n,
+                                int channels, int radius, float bias, float alpha, float beta) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const int k = (int)(i % channels);
+    const int64_t px = i - k;
+    const int o_lo = k - radius > 0 ? k - radius : 0;
+    const int o_hi = k + radius < channels - 1 ? k + radius : channels - 1;
+    const float xk = x[i];
+    float acc = 0.f;
+    for (int o = o_lo; o <= o_hi; o++) {
+      const int lo = o - radius > 0 ? o - radius : 0;
+      const int hi = o + radius < channels - 1 ? o + radius : channels - 1;
+      float sum = 0.f;
+      for (int q = lo; q <= hi; q++) {
+        const float z = x[px + q];
+        sum += z * z;
+      }
+      const float norm = alpha * sum + bias;
+      float d = -2.f * alpha * beta * xk * y[px + o] / norm;
+      if (o == k) d += powf(norm, -beta);
+      acc += d * dy[px + o];
+    }
+    dx[i] = acc;
+  }
+}
+
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 template <int S, int TH, int TW>
@@ -573,6 +624,56 @@ extern "C" int tfhip_pool2d(tfhip_ctx* ctx, int64_t x, int64_t out, const tfhip_
     hipLaunchKernelGGL(pool2d_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0,
                        ctx->stream, xf, y, *ci, kind);
   }
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+static int lrn_check(tfhip_ctx* ctx, const char* op, const Buf* const* bufs, int n_bufs, int64_t pixels,
+                     int channels, int radius) {
+  if (pixels < 0 || channels < 0 || radius < 0) return ctx->fail(TFHIP_EINVAL, "%s: bad geometry", op);
+  for (int i = 0; i < n_bufs; i++) {
+    if (bufs[i]->numel != pixels * channels)
+      return ctx->fail(TFHIP_EINVAL, "%s: a buffer holds %lld elements, the shape needs %lld", op,
+                       (long long)bufs[i]->numel, (long long)(pixels * channels));
+    if (bufs[i]->dtype != TFHIP_FLOAT32) return ctx->fail(TFHIP_EINVAL, "%s: float32 buffers only", op);
+  }
+  return TFHIP_OK;
+}
+
+extern "C" int tfhip_lrn(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t pixels, int channels,
+                         int depth_radius, float bias, float alpha, float beta) {
+  if (!ctx) return TFHIP_EINVAL;
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bo, out);
+  const Buf* bufs[] = {bx, bo};
+  int rc;
+  if ((rc = lrn_check(ctx, "localResponseNormalization", bufs, 2, pixels, channels, depth_radius))) return rc;
+  const int64_t n = bx->numel;
+  if (n == 0) return TFHIP_OK;
+  const int64_t blocks = ceil_div(n, 256), cap = (int64_t)ctx->num_cus * 16;
+  hipLaunchKernelGGL(lrn_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, ctx->stream,
+                     (const float*)bx->ptr, (float*)bo->ptr, n, channels, depth_radius, bias, alpha, beta);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+extern "C" int tfhip_lrn_grad(tfhip_ctx* ctx, int64_t dy, int64_t x, int64_t y, int64_t dx,
+                              int64_t pixels, int channels, int depth_radius, float bias,
+                              float alpha, float beta) {
+  if (!ctx) return TFHIP_EINVAL;
+  TFHIP_GET(ctx, bdy, dy);
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, by, y);
+  TFHIP_GET(ctx, bdx, dx);
+  const Buf* bufs[] = {bdy, bx, by, bdx};
+  int rc;
+  if ((rc = lrn_check(ctx, "LRNGrad", bufs, 4, pixels, channels, depth_radius))) return rc;
+  const int64_t n = bx->numel;
+  if (n == 0) return TFHIP_OK;
+  const int64_t blocks = ceil_div(n, 256), cap = (int64_t)ctx->num_cus * 16;
+  hipLaunchKernelGGL(lrn_grad_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0,
+                     ctx->stream, (const float*)bdy->ptr, (const float*)bx->ptr, (const float*)by->ptr,
+                     (float*)bdx->ptr, n, channels, depth_radius, bias, alpha, beta);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }

@@ -319,6 +319,33 @@ static napi_value js_resize_nearest(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+/* cumsum(ctx, x, out, outer, inner, exclusive, reverse) */
+static napi_value js_cumsum(napi_env env, napi_callback_info info) {
+  ARGS(7);
+  I64(1, x); I64(2, out); I64(3, outer); I64(4, inner); INT(5, exclusive); INT(6, reverse);
+  CHECK(tfhip_cumsum(ctx, x, out, outer, inner, exclusive, reverse));
+  return undefined(env);
+}
+
+/* lrn(ctx, x, out, pixels, channels, depthRadius, bias, alpha, beta) */
+static napi_value js_lrn(napi_env env, napi_callback_info info) {
+  ARGS(9);
+  I64(1, x); I64(2, out); I64(3, pixels); INT(4, channels); INT(5, radius);
+  F64(6, bias); F64(7, alpha); F64(8, beta);
+  CHECK(tfhip_lrn(ctx, x, out, pixels, channels, radius, (float)bias, (float)alpha, (float)beta));
+  return undefined(env);
+}
+
+/* lrnGrad(ctx, dy, x, y, dx, pixels, channels, depthRadius, bias, alpha, beta) */
+static napi_value js_lrn_grad(napi_env env, napi_callback_info info) {
+  ARGS(11);
+  I64(1, dy); I64(2, x); I64(3, y); I64(4, dx); I64(5, pixels); INT(6, channels); INT(7, radius);
+  F64(8, bias); F64(9, alpha); F64(10, beta);
+  CHECK(tfhip_lrn_grad(ctx, dy, x, y, dx, pixels, channels, radius, (float)bias, (float)alpha,
+                       (float)beta));
+  return undefined(env);
+}
+
 /* select(ctx, condition, a, b, out, inner) */
 static napi_value js_select(napi_env env, napi_callback_info info) {
   ARGS(6);
@@ -545,7 +572,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"depthwiseConv2dDerInput", js_depthwise_der_input},
       {"depthwiseConv2dDerFilter", js_depthwise_der_filter},
       {"pool2dBackprop", js_pool2d_backprop}, {"resizeNearest", js_resize_nearest},
-      {"select", js_select}};
+      {"select", js_select}, {"cumsum", js_cumsum}, {"lrn", js_lrn}, {"lrnGrad", js_lrn_grad}};
   for (size_t i = 0; i < sizeof fns / sizeof fns[0]; i++) {
     napi_value f;
     if (napi_create_function(env, fns[i].name, NAPI_AUTO_LENGTH, fns[i].fn, NULL, &f) != napi_ok ||

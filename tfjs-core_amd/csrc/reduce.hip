@@ -139,6 +139,36 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void softmax_rows_kernel(
   for (int64_t j = lane; j < cols; j += WAVE) yr[j] = expf(xr[j] - lse);
 }
 
+// cumsum along the innermost axis (backend_cpu.ts:714-745): one wavefront per row walks the row
+// 64 elements at a time, a shuffle scan inside the group and a running carry between groups.
+// Floats are summed in double and rounded once per element, int32 wraps like Int32Array.
+template <typename OutT>
+__global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void cumsum_rows_kernel(
+    const void* x, int x_dt, OutT* out, int64_t rows, int64_t cols, int exclusive, int reverse) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int64_t base = row * cols;
+  double carry = 0.0;
+  for (int64_t j0 = 0; j0 < cols; j0 += WAVE) {
+    const int64_t j = j0 + lane;                       // position along the scan direction
+    const int64_t at = base + (reverse ? cols - 1 - j : j);
+    const double v = j < cols ? (double)ld(x, x_dt, at) : 0.0;
+    double s = v;
+    for (int off = 1; off < WAVE; off <<= 1) {
+      const double o = __shfl_up(s, off, WAVE);
+      if (lane >= off) s += o;
+    }
+    const double incl = carry + s;
+    const double r = exclusive ? incl - v : incl;
+    if (j < cols) {
+      if (std::is_same<OutT, float>::value) out[at] = (OutT)(float)r;
+      else out[at] = (OutT)(int32_t)(uint32_t)(int64_t)r;
+    }
+    carry = __shfl(incl, WAVE - 1, WAVE);
+  }
+}
+
 // out[o, i, :] = x[o, indices[i], :] for 4-byte or 1-byte elements.
 template <typename T>
 __global__ void gather_kernel(const T* x, const int32_t* indices, T* out, int64_t outer,
@@ -309,6 +339,29 @@ extern "C" int tfhip_transpose(tfhip_ctx* ctx, int64_t x, const int32_t* x_shape
   else
     hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, block, 0, ctx->stream,
                        (const uint8_t*)bx->ptr, (uint8_t*)bo->ptr, n, pa);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+extern "C" int tfhip_cumsum(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t outer, int64_t inner,
+                            int exclusive, int reverse) {
+  if (!ctx) return TFHIP_EINVAL;
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bo, out);
+  if (outer < 0 || inner < 0 || bx->numel != outer * inner || bo->numel != outer * inner)
+    return ctx->fail(TFHIP_EINVAL, "cumsum: buffers hold %lld and %lld elements, need %lld",
+                     (long long)bx->numel, (long long)bo->numel, (long long)(outer * inner));
+  if (bx->dtype == TFHIP_UINT8Q || (bo->dtype != TFHIP_FLOAT32 && bo->dtype != TFHIP_INT32))
+    return ctx->fail(TFHIP_EINVAL, "cumsum: output must be float32 or int32");
+  if (outer * inner == 0) return TFHIP_OK;
+  if (ceil_div(outer, ROWS_PER_BLOCK) > 0x7fffffffLL) return ctx->fail(TFHIP_ENOTSUP, "cumsum: too many rows");
+  const dim3 grid((unsigned)ceil_div(outer, ROWS_PER_BLOCK)), block(WAVE * ROWS_PER_BLOCK);
+  if (bo->dtype == TFHIP_FLOAT32)
+    hipLaunchKernelGGL(cumsum_rows_kernel<float>, grid, block, 0, ctx->stream, bx->ptr, bx->dtype,
+                       (float*)bo->ptr, outer, inner, exclusive, reverse);
+  else
+    hipLaunchKernelGGL(cumsum_rows_kernel<int32_t>, grid, block, 0, ctx->stream, bx->ptr, bx->dtype,
+                       (int32_t*)bo->ptr, outer, inner, exclusive, reverse);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }

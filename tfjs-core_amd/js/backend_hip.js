@@ -421,6 +421,29 @@ class MathBackendHIP extends KernelBackend {
     return out;
   }
   sum(x, axes) { return this.reduce('sum', x, axes, util.upcastType(x.dtype, 'int32')); }
+  cumsum(x, axis, exclusive, reverse) {
+    if (axis !== x.rank - 1) {   // backend_cpu.ts:718-722
+      throw new Error(`backend.cumsum expects an inner-most axis=${x.rank - 1} but got axis=${axis}`);
+    }
+    const out = this.out(x.shape, util.upcastType(x.dtype, 'int32'));
+    const inner = x.rank ? x.shape[x.rank - 1] : 1;
+    this.napi.cumsum(this.ctx, this.h(x), this.h(out), inner ? x.size / inner : 0, inner,
+                     exclusive ? 1 : 0, reverse ? 1 : 0);
+    return out;
+  }
+  localResponseNormalization4D(x, radius, bias, alpha, beta) {
+    const out = this.out(x.shape, 'float32');
+    const c = x.shape[3];
+    this.napi.lrn(this.ctx, this.h(x), this.h(out), c ? x.size / c : 0, c, radius, bias, alpha, beta);
+    return out;
+  }
+  LRNGrad(dy, inputImage, outputImage, radius, bias, alpha, beta) {
+    const out = this.out(inputImage.shape, 'float32');
+    const c = inputImage.shape[3];
+    this.napi.lrnGrad(this.ctx, this.h(dy), this.h(inputImage), this.h(outputImage), this.h(out),
+                      c ? inputImage.size / c : 0, c, radius, bias, alpha, beta);
+    return out;
+  }
   prod(x, axes) { return this.reduce('prod', x, axes, util.upcastType(x.dtype, 'int32')); }
   all(x, axes) { return this.reduce('all', x, axes, 'bool'); }
   any(x, axes) { return this.reduce('any', x, axes, 'bool'); }

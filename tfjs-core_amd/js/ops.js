@@ -1249,6 +1249,119 @@ const opHandler = {
 };
 setOpHandler(opHandler);
 
+// ---- cumsum, localResponseNormalization, space / batch / depth rearrangements ---------------
+// array_ops.ts:703-731: the axis is brought innermost, scanned and put back; the gradient is
+// the scan of dy in the other direction.
+const cumsum = op('cumsum', (x, axis, exclusive, reverse) => {
+  const $x = convertToTensor(x, 'x', 'cumsum');
+  axis = util.parseAxisParam([axis | 0], $x.shape)[0];
+  exclusive = !!exclusive;
+  reverse = !!reverse;
+  const perm = axis_util.getAxesPermutation([axis], $x.rank);
+  const permutedX = perm == null ? $x : transpose($x, perm);
+  const inner = axis_util.getInnerMostAxes(1, $x.rank)[0];
+  let value = ENGINE.runKernel(backend => backend.cumsum(permutedX, inner, exclusive, reverse), {permutedX},
+                               dy => ({permutedX: () => cumsum(dy, inner, exclusive, !reverse)}));
+  if (perm != null) value = transpose(value, axis_util.getUndoAxesPermutation(perm));
+  return value;
+});
+
+// ops/lrn.ts:41-91
+const localResponseNormalization = op('localResponseNormalization', (x, depthRadius, bias, alpha, beta) => {
+  const $x = convertToTensor(x, 'x', 'localResponseNormalization');
+  if (depthRadius == null) depthRadius = 5;
+  if (bias == null) bias = 1;
+  if (alpha == null) alpha = 1;
+  if (beta == null) beta = 0.5;
+  util.assert($x.rank === 4 || $x.rank === 3,
+              () => `Error in localResponseNormalization: x must be rank 3 or 4 but got rank ${$x.rank}.`);
+  util.assert(util.isInt(depthRadius),
+              () => `Error in localResponseNormalization: depthRadius must be an integer but got ` +
+                  `depthRadius ${depthRadius}.`);
+  const reshapedTo4D = $x.rank === 3;
+  const x4D = as4D($x);
+  const res = ENGINE.runKernel((backend, save) => {
+    const y = backend.localResponseNormalization4D(x4D, depthRadius, bias, alpha, beta);
+    save([x4D, y]);
+    return y;
+  }, {x4D}, (dy, saved) => ({
+    x4D: () => ENGINE.runKernel(backend => backend.LRNGrad(dy, saved[0], saved[1], depthRadius, bias, alpha, beta), {})
+  }));
+  return lower(res, reshapedTo4D);
+});
+
+// array_ops.ts:708-741 / backend_cpu.ts:2225-2245 over this host's reshape, transpose and slice:
+// [B, s1..sM, rest] -> [b1..bM, B/prod, s1..sM, rest] -> interleave (si, bi) -> crop.
+const batchToSpaceND = op('batchToSpaceND', (x, blockShape, crops) => {
+  const $x = convertToTensor(x, 'x', 'batchToSpaceND');
+  const M = blockShape.length;
+  const prod = blockShape.reduce((a, b) => a * b);
+  util.assert($x.rank >= 1 + M,
+              () => `input rank is ${$x.rank} but should be > than blockShape.length ${M}`);
+  util.assert(crops.length === M,
+              () => `crops.length is ${crops.length} but should be equal to blockShape.length  ${M}`);
+  util.assert($x.shape[0] % prod === 0,
+              () => `input tensor batch is ${$x.shape[0]} but is not divisible by the product of ` +
+                  `the elements of blockShape ${blockShape.join(' * ')} === ${prod}`);
+  const rest = $x.shape.slice(1 + M);
+  const split = blockShape.concat([$x.shape[0] / prod], $x.shape.slice(1));
+  const perm = [M];
+  for (let i = 0; i < M; i++) perm.push(M + 1 + i, i);
+  for (let i = 0; i < rest.length; i++) perm.push(2 * M + 1 + i);
+  const merged = [$x.shape[0] / prod].concat(blockShape.map((b, i) => b * $x.shape[1 + i]), rest);
+  const begin = [0].concat(crops.map(c => c[0]), rest.map(() => 0));
+  const size = [merged[0]].concat(crops.map((c, i) => merged[1 + i] - c[0] - c[1]), rest);
+  return ENGINE.tidy(() => slice(reshape(transpose(reshape($x, split), perm), merged), begin, size));
+});
+
+// array_ops.ts:786-824 / backend_cpu.ts:2247-2271: pad, split every spatial dim into
+// (si / bi, bi), move the bi in front of the batch, merge.
+const spaceToBatchND = op('spaceToBatchND', (x, blockShape, paddings) => {
+  const $x = convertToTensor(x, 'x', 'spaceToBatchND');
+  const M = blockShape.length;
+  util.assert($x.rank >= 1 + M,
+              () => `input rank ${$x.rank} should be > than [blockShape] ${M}`);
+  util.assert(paddings.length === M,
+              () => `paddings.shape[0] ${paddings.length} must be equal to [blockShape] ${M}`);
+  util.assert($x.shape.reduce((ok, d, i) => (i > 0 && i <= M) ?
+      ok && ((d + paddings[i - 1][0] + paddings[i - 1][1]) % blockShape[i - 1] === 0) : ok, true),
+              () => `input spatial dimensions ${$x.shape.slice(1)} with paddings ${paddings.toString()} ` +
+                  `must be divisible by blockShapes ${blockShape.toString()}`);
+  const prod = blockShape.reduce((a, b) => a * b);
+  const rest = $x.shape.slice(1 + M);
+  const full = [[0, 0]].concat(paddings, rest.map(() => [0, 0]));
+  return ENGINE.tidy(() => {
+    const padded = pad($x, full);
+    const split = [padded.shape[0]];
+    for (let i = 0; i < M; i++) split.push(padded.shape[1 + i] / blockShape[i], blockShape[i]);
+    const perm = [];
+    for (let i = 0; i < M; i++) perm.push(2 + 2 * i);
+    perm.push(0);
+    for (let i = 0; i < M; i++) perm.push(1 + 2 * i);
+    for (let i = 0; i < rest.length; i++) perm.push(2 * M + 1 + i);
+    const merged = [padded.shape[0] * prod].concat(blockShape.map((b, i) => padded.shape[1 + i] / b), rest);
+    return reshape(transpose(reshape(padded, split.concat(rest)), perm), merged);
+  });
+});
+
+// array_ops.ts:960-1001 / backend_cpu.ts:3469-3512 (NHWC): out[b, h, w, d] =
+// x[b, h / bs, w / bs, ((h % bs) * bs + w % bs) * outDepth + d], i.e. a 6-d transpose.
+const depthToSpace = op('depthToSpace', (x, blockSize, dataFormat) => {
+  const $x = convertToTensor(x, 'x', 'depthToSpace');
+  if (dataFormat == null) dataFormat = 'NHWC';
+  util.assert(dataFormat === 'NHWC', () => `Only NHWC dataFormat supported for depthToSpace. Got ${dataFormat}`);
+  util.assert($x.rank === 4, () => `depthToSpace expects a rank-4 tensor, got rank ${$x.rank}`);
+  util.assert(blockSize > 1, () => `blockSize should be > 1 for depthToSpace, but was: ${blockSize}`);
+  const [b, h, w, d] = $x.shape;
+  util.assert(d % (blockSize * blockSize) === 0,
+              () => `Dimension size must be evenly divisible by ${blockSize * blockSize} but is ${d} ` +
+                  `for depthToSpace with input shape ${$x.shape}`);
+  const outD = d / (blockSize * blockSize);
+  return ENGINE.tidy(() => reshape(
+      transpose(reshape($x, [b, h, w, blockSize, blockSize, outD]), [0, 1, 3, 2, 4, 5]),
+      [b, h * blockSize, w * blockSize, outD]));
+});
+
 module.exports = {
   op, tensor, scalar, tensor1d, tensor2d, tensor3d, tensor4d, quantizedTensor, convertToTensor,
   fill, zeros, ones, zerosLike, onesLike, reshape, cast, clone, dequantize, matMul,
@@ -1263,5 +1376,6 @@ module.exports = {
   expandDims, squeeze, stack, unstack, split,
   floor, ceil, round, sign, expm1, log1p, reciprocal, sin, cos, tan, asin, acos, atan, sinh, cosh,
   asinh, acosh, atanh, erf, elu, selu, softplus, step, leakyRelu, logSigmoid, isNaN: isNaN_, isInf,
-  isFinite: isFinite_, pow, squaredDifference, mod, floorDiv, atan2, addN, prod, all, any
+  isFinite: isFinite_, pow, squaredDifference, mod, floorDiv, atan2, addN, prod, all, any,
+  cumsum, localResponseNormalization, batchToSpaceND, spaceToBatchND, depthToSpace
 };

@@ -74,6 +74,13 @@ const OPS = {
     opt.dispose();
     return out;
   },
+  cumsum: (i, a) => tf.cumsum(i.x, a.axis, a.exclusive, a.reverse),
+  gradCumsum: (i, a) => tf.grad(x => tf.cumsum(x, a.axis, a.exclusive, a.reverse))(i.x, i.dy),
+  lrn: (i, a) => tf.localResponseNormalization(i.x, a.radius, a.bias, a.alpha, a.beta),
+  gradLrn: (i, a) => tf.grad(x => tf.localResponseNormalization(x, a.radius, a.bias, a.alpha, a.beta))(i.x, i.dy),
+  batchToSpaceND: (i, a) => tf.batchToSpaceND(i.x, a.blockShape, a.crops),
+  spaceToBatchND: (i, a) => tf.spaceToBatchND(i.x, a.blockShape, a.paddings),
+  depthToSpace: (i, a) => tf.depthToSpace(i.x, a.blockSize),
   unaryNamed: (i, a) => tf[a.name](i.x, a.alpha),
   binaryNamed: (i, a) => tf[a.name](i.a, i.b),
   reduceNamed: (i, a) => tf[a.name](i.x, a.axis, a.keepDims),

@@ -450,6 +450,33 @@ class MathBackendHIP(object):
     def sum(self, x, axes):
         return self._reduce("sum", x, axes, su.upcast_type(x.dtype, "int32"))
 
+    def cumsum(self, x, axis, exclusive, reverse):
+        if axis != x.rank - 1:   # backend_cpu.ts:718-722
+            raise ValueError("backend.cumsum expects an inner-most axis=%d but got axis=%d"
+                             % (x.rank - 1, axis))
+        out = self._out(x.shape, su.upcast_type(x.dtype, "int32"))
+        inner = x.shape[-1] if x.rank else 1
+        self._ck(self.lib.tfhip_cumsum(self.ctx, self._h(x), self._h(out),
+                                       su.size_from_shape(x.shape) // inner if inner else 0, inner,
+                                       int(bool(exclusive)), int(bool(reverse))))
+        return out
+
+    def local_response_normalization4d(self, x, radius, bias, alpha, beta):
+        out = self._out(x.shape, "float32")
+        c = x.shape[3]
+        self._ck(self.lib.tfhip_lrn(self.ctx, self._h(x), self._h(out),
+                                    su.size_from_shape(x.shape) // c if c else 0, c, int(radius),
+                                    float(bias), float(alpha), float(beta)))
+        return out
+
+    def lrn_grad(self, dy, x, y, radius, bias, alpha, beta):
+        out = self._out(x.shape, "float32")
+        c = x.shape[3]
+        self._ck(self.lib.tfhip_lrn_grad(self.ctx, self._h(dy), self._h(x), self._h(y), self._h(out),
+                                         su.size_from_shape(x.shape) // c if c else 0, c,
+                                         int(radius), float(bias), float(alpha), float(beta)))
+        return out
+
     def prod(self, x, axes):
         return self._reduce("prod", x, axes, su.upcast_type(x.dtype, "int32"))
 

@@ -416,6 +416,41 @@ def sum(x, axis=None, keep_dims=False):  # noqa: A001
     return _reduce("sum", xt, axis, keep_dims)
 
 
+def cumsum(x, axis=0, exclusive=False, reverse=False):
+    """ops/array_ops.ts:703-731: the axis is brought innermost, scanned, and put back."""
+    x = _conv(x, "x", "cumsum")
+
+    def run():
+        ax = su.parse_axis_param([axis], x.shape)[0]
+        perm = su.get_axes_permutation([ax], x.rank)
+        xt = x if perm is None else transpose(x, perm)
+        inner = su.get_inner_most_axes(1, x.rank)[0]
+        r = ENGINE.run_kernel(lambda be: be.cumsum(xt, inner, exclusive, reverse))
+        if perm is not None:
+            r = transpose(r, su.get_undo_axes_permutation(perm))
+        return r
+    return ENGINE.tidy(run)
+
+
+def local_response_normalization(x, depth_radius=5, bias=1.0, alpha=1.0, beta=0.5):
+    """ops/lrn.ts:41-91: rank 3 or 4, integer depthRadius."""
+    x = _conv(x, "x", "localResponseNormalization")
+    if x.rank not in (3, 4):
+        raise ValueError("Error in localResponseNormalization: x must be rank 3 or 4 but got rank %d."
+                         % x.rank)
+    if int(depth_radius) != depth_radius:
+        raise ValueError("Error in localResponseNormalization: depthRadius must be an integer but "
+                         "got depthRadius %s." % depth_radius)
+    x4 = reshape(x, (1,) + tuple(x.shape)) if x.rank == 3 else x
+    r = ENGINE.run_kernel(lambda be: be.local_response_normalization4d(x4, depth_radius, bias, alpha, beta))
+    return reshape(r, r.shape[1:]) if x.rank == 3 else r
+
+
+def lrn_grad(dy, x, y, depth_radius=5, bias=1.0, alpha=1.0, beta=0.5):
+    dy, x, y = _conv(dy, "dy", "LRNGrad"), _conv(x, "x", "LRNGrad"), _conv(y, "y", "LRNGrad")
+    return ENGINE.run_kernel(lambda be: be.lrn_grad(dy, x, y, depth_radius, bias, alpha, beta))
+
+
 def prod(x, axis=None, keep_dims=False):
     """ops/reduction_ops.ts:166-199."""
     xt = _conv(x, "x", "prod")

@@ -173,6 +173,11 @@ def get_axes_permutation(axes, rank):
     return [i for i in range(rank) if i not in axes] + list(axes)
 
 
+def get_undo_axes_permutation(axes):
+    """ops/axis_util.ts:172-176: the permutation that reverses `axes`."""
+    return [i for i, _ in sorted(enumerate(axes), key=lambda p: p[1])]
+
+
 def get_inner_most_axes(num_axes, rank):
     return list(range(rank - num_axes, rank))
 
