@@ -397,6 +397,9 @@ def main():
         "python_driver": python_driver,
         "js_host": js,
         "pcie_inclusive": pcie,
+        # the same step recorded once with tf.captureGraph and replayed (one launch per step); an
+        # extension of this backend, reported beside `value`, which stays the eager tf.* path
+        "graph_replay": js.get("graph_replay") if js else None,
         "dense_tflops": round(sum(2e-9 * r["macs"] for r in rows if r["kernel"].startswith("gemm"))
                               / sum(r["ms"] for r in rows if r["kernel"].startswith("gemm")), 2),
         "roofline": roof,

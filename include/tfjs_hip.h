@@ -89,6 +89,24 @@ int tfhip_sync(tfhip_ctx* ctx);
 /* KernelBackend.time (backend.ts:92, backend_cpu.ts:239-244): event pair on the stream. */
 int tfhip_time_begin(tfhip_ctx* ctx);
 int tfhip_time_end(tfhip_ctx* ctx, float* ms);
+/* Captured graphs: no counterpart in the reference, whose backends run every op eagerly.  A
+ * chain of small kernels (a batch-1 forward pass is 32 launches of a few microseconds) is bound by
+ * the host's cost per launch; captured once, it replays with a single launch.
+ *   tfhip_graph_begin  starts recording the work queued on the context's stream.  Until
+ *                      tfhip_graph_end, write / read / sync / time fail, and the pool must already
+ *                      hold every block the work needs (run it once before capturing it).
+ *   tfhip_graph_end    stops recording and returns a graph id.  The blocks the recorded work
+ *                      used stay out of the pool while the graph lives: a replay writes them again.
+ *   tfhip_graph_launch queues one replay.  The tensors the recorded work read that were created
+ *                      before the capture (weights, the input) must still exist; new input data is
+ *                      written into the same tensor with tfhip_write.  Results appear in the buffers
+ *                      of the tensors the recorded work produced.
+ *   tfhip_graph_destroy waits for queued replays and gives the blocks back. */
+int tfhip_graph_begin(tfhip_ctx* ctx);
+int tfhip_graph_end(tfhip_ctx* ctx, int64_t* graph_id);
+int tfhip_graph_launch(tfhip_ctx* ctx, int64_t graph_id);
+int tfhip_graph_destroy(tfhip_ctx* ctx, int64_t graph_id);
+
 /* Name of the kernel variant the last dense / image call launched (tile shape, operand
  * layout), for matching launches to profiler rows.  Not part of the reference interface. */
 const char* tfhip_last_kernel(tfhip_ctx* ctx);

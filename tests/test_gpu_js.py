@@ -507,6 +507,21 @@ def test_js_scan_lrn_and_rearrangements(tmp_path, ref):
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
 
 
+def test_js_captured_graph_replays_equal_eager(tmp_path):
+    """tf.captureGraph on the hip backend: a conv net recorded once, then replayed four times
+    with new input data and eager ops in between; every replay equals the eager result bit
+    for bit, and nothing is left behind."""
+    rng = np.random.default_rng(97)
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)
+    c = Cases(tmp_path)
+    inputs = dict(x=f(2, 16, 16, 3), x2=f(2, 16, 16, 3), w0=f(3, 3, 3, 16) * 0.3, b0=f(16) * 0.1,
+                  dw=f(3, 3, 16, 1) * 0.3, w1=f(1, 1, 16, 32) * 0.3, fc=f(2 * 2 * 32, 10) * 0.2)
+    c.add("capture", "captureReplay", inputs, dict(replays=4), np.zeros((2, 10), np.float32), exact=True)
+    results = c.run()
+    c.check(results)
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
 def test_js_backward_ops_match_oracle(tmp_path, ref):
     """conv2dDerInput / conv2dDerFilter / conv2dTranspose, the depthwise and pooling backprops
     through the JS host and the N-API addon."""

@@ -137,3 +137,63 @@ def test_errors_come_back_as_exceptions(tf):
         with pytest.raises(ValueError, match="depth of input"):
             tf.conv2d(tf.tensor(np.ones((1, 4, 4, 3), np.float32)),
                       tf.tensor(np.ones((3, 3, 2, 8), np.float32)), 1, "same")
+
+
+def test_captured_graph_replays_match_eager_runs():
+    """A chain of conv / depthwise / pointwise / pool / matmul / softmax kernels captured once and
+    replayed several times, with eager work, new input data and synchronisations between the
+    replays: every replay must equal the eager result for the input then in place, the blocks
+    the graph wrote must not be handed to other tensors while it lives, and destroying it returns
+    them to the pool."""
+    import tfhip as tf
+    tf.set_backend("hip")
+    rng = np.random.default_rng(91)
+    f32 = lambda *s: rng.standard_normal(s).astype(np.float32)
+    w0, b0 = f32(3, 3, 3, 16) * 0.3, f32(16) * 0.1
+    dw, w1, b1 = f32(3, 3, 16, 1) * 0.3, f32(1, 1, 16, 32) * 0.3, f32(32) * 0.1
+    fc = f32(32, 10) * 0.3
+    with tf.tidy():
+        wt = [tf.tensor(a) for a in (w0, b0, dw, w1, b1, fc)]
+        x = tf.tensor(f32(2, 16, 16, 3))
+
+        def net():
+            h = tf.fused.conv2d(x, wt[0], 2, "same", bias=wt[1], activation="relu6")
+            h = tf.depthwise_conv2d(h, wt[2], 1, "same")
+            h = tf.fused.conv2d(h, wt[3], 1, "same", bias=wt[4], activation="relu")
+            h = tf.avg_pool(h, 8, 8, "valid")
+            return tf.softmax(tf.matmul(tf.reshape(h, (2, 32)), wt[5]))
+
+        def eager():
+            with tf.tidy():
+                return net().data_sync()
+
+        before = tf.memory()
+        g = tf.capture_graph(net)
+        out = g.outputs
+        for k in range(4):
+            new_x = f32(2, 16, 16, 3)
+            tf.backend().write(x.data_id, new_x)          # new data into the same tensor
+            want = eager()                                 # eager work between the replays
+            junk = [tf.tensor(f32(2, 8, 8, 16)) for _ in range(6)]   # takes blocks from the pool
+            junk_want = [t.data_sync() for t in junk]
+            g.replay()
+            got = out.data_sync()                          # synchronises
+            np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-7, err_msg="replay %d" % k)
+            for t, wv in zip(junk, junk_want):             # the replay wrote none of their blocks
+                assert np.array_equal(t.data_sync(), wv)
+                t.dispose()
+        # write / read are refused inside a capture and the capture still ends cleanly
+        tf.backend().lib.tfhip_graph_begin(tf.backend().ctx)
+        with pytest.raises(Exception, match="graph capture"):
+            with tf.tidy():
+                tf.tensor(f32(4))
+        import ctypes
+        gid = ctypes.c_int64()
+        if tf.backend().lib.tfhip_graph_end(tf.backend().ctx, ctypes.byref(gid)) == 0:
+            assert tf.backend().lib.tfhip_graph_destroy(tf.backend().ctx, gid.value) == 0
+        with tf.tidy():
+            assert tf.tensor(f32(4)).data_sync().shape == (4,)  # eager work goes on afterwards
+        g.dispose()
+        after = tf.memory()
+        assert after["numDeviceBuffers"] == before["numDeviceBuffers"]
+        assert after["numBytesInGPU"] == before["numBytesInGPU"]

@@ -44,7 +44,15 @@ void* tfhip_ctx::alloc(size_t nbytes, size_t* cap) {
     pooled -= want;
     in_use += want;
     *cap = want;
+    if (capturing) capture_blocks.push_back(p);
     return p;
+  }
+  if (capturing) {
+    // a capture must find every block in the pool (the same work has run once before it):
+    // allocating here would put a device allocation into the middle of a stream capture
+    fail(TFHIP_EDEVICE, "graph capture needs a block of %zu bytes that the pool does not hold; "
+                        "run the captured work once before capturing it", want);
+    return nullptr;
   }
   void* p = nullptr;
   hipError_t e = hipMalloc(&p, want);
@@ -66,12 +74,18 @@ void* tfhip_ctx::alloc(size_t nbytes, size_t* cap) {
 void tfhip_ctx::release(void* p, size_t cap) {
   if (!p) return;
   in_use -= cap;
+  auto own = owner.find(p);
+  if (own != owner.end()) {  // a block that a captured graph writes on every replay
+    graphs[own->second].parked.emplace_back(p, cap);
+    return;
+  }
   pooled += cap;
   pool[cap].push_back(p);
 }
 
 void tfhip_ctx::trim() {
-  if (pool.empty()) return;
+  // (not while a graph exists: a replay may still read blocks that went back to the pool)
+  if (pool.empty() || capturing || !graphs.empty()) return;
   (void)hipStreamSynchronize(stream);
   for (auto& kv : pool)
     for (void* p : kv.second) (void)hipFree(p);
@@ -128,6 +142,11 @@ void tfhip_destroy(tfhip_ctx* ctx) {
     if (kv.second.ptr) (void)hipFree(kv.second.ptr);
   for (auto& kv : ctx->pool)
     for (void* p : kv.second) (void)hipFree(p);
+  for (auto& kv : ctx->graphs) {
+    (void)hipGraphExecDestroy(kv.second.exec);
+    (void)hipGraphDestroy(kv.second.graph);
+    for (auto& blk : kv.second.parked) (void)hipFree(blk.first);
+  }
   (void)hipEventDestroy(ctx->ev_begin);
   (void)hipEventDestroy(ctx->ev_end);
   (void)hipStreamDestroy(ctx->stream);
@@ -166,6 +185,9 @@ int tfhip_register(tfhip_ctx* ctx, int64_t id, const int32_t* shape, int rank, i
 
 int tfhip_write(tfhip_ctx* ctx, int64_t id, const void* host, size_t nbytes) {
   if (!ctx) return TFHIP_EINVAL;
+  if (ctx->capturing)
+    return ctx->fail(TFHIP_EINVAL, "write: host data cannot enter a graph capture (create the "
+                                   "tensor before capturing)");
   TFHIP_GET(ctx, b, id);
   if (!host && nbytes)  // backend_cpu.ts:125-127
     return ctx->fail(TFHIP_EINVAL, "MathBackendHIP.write(): values can not be null");
@@ -180,6 +202,7 @@ int tfhip_write(tfhip_ctx* ctx, int64_t id, const void* host, size_t nbytes) {
 
 int tfhip_read(tfhip_ctx* ctx, int64_t id, void* host, size_t nbytes) {
   if (!ctx) return TFHIP_EINVAL;
+  if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "read: not during a graph capture");
   TFHIP_GET(ctx, b, id);
   if (nbytes != b->nbytes)
     return ctx->fail(TFHIP_EINVAL, "read: asked %zu bytes of a buffer of %zu", nbytes, b->nbytes);
@@ -208,12 +231,14 @@ int tfhip_mem_info(tfhip_ctx* ctx, size_t* in_use, size_t* pooled, size_t* num_i
 
 int tfhip_sync(tfhip_ctx* ctx) {
   if (!ctx) return TFHIP_EINVAL;
+  if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "sync: not during a graph capture");
   TFHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
   return TFHIP_OK;
 }
 
 int tfhip_time_begin(tfhip_ctx* ctx) {
   if (!ctx) return TFHIP_EINVAL;
+  if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "time: not during a graph capture");
   TFHIP_HIP(ctx, hipEventRecord(ctx->ev_begin, ctx->stream));
   ctx->timing = true;
   return TFHIP_OK;
@@ -226,6 +251,79 @@ int tfhip_time_end(tfhip_ctx* ctx, float* ms) {
   TFHIP_HIP(ctx, hipEventRecord(ctx->ev_end, ctx->stream));
   TFHIP_HIP(ctx, hipEventSynchronize(ctx->ev_end));
   TFHIP_HIP(ctx, hipEventElapsedTime(ms, ctx->ev_begin, ctx->ev_end));
+  return TFHIP_OK;
+}
+
+// ---- captured graphs ---------------------------------------------------------------------
+int tfhip_graph_begin(tfhip_ctx* ctx) {
+  if (!ctx) return TFHIP_EINVAL;
+  if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "graph_begin: a capture is already running");
+  ctx->capture_blocks.clear();
+  TFHIP_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+  ctx->capturing = true;
+  return TFHIP_OK;
+}
+
+int tfhip_graph_end(tfhip_ctx* ctx, int64_t* graph_id) {
+  if (!ctx || !graph_id) return TFHIP_EINVAL;
+  if (!ctx->capturing) return ctx->fail(TFHIP_EINVAL, "graph_end without graph_begin");
+  ctx->capturing = false;
+  tfhip_ctx::Graph g;
+  hipError_t e = hipStreamEndCapture(ctx->stream, &g.graph);
+  if (e == hipSuccess) e = hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    if (g.graph) (void)hipGraphDestroy(g.graph);
+    ctx->capture_blocks.clear();
+    return ctx->fail(TFHIP_EDEVICE, "graph capture failed: %s", hipGetErrorString(e));
+  }
+  const int64_t id = ctx->next_graph++;
+  // Every block the capture handed out now belongs to the graph: those lying free in the pool
+  // are taken out of it, the others follow when their tensor lets go of them (release()).
+  for (void* p : ctx->capture_blocks) {
+    if (ctx->owner.count(p)) continue;
+    ctx->owner[p] = id;
+    for (auto& kv : ctx->pool) {
+      auto& v = kv.second;
+      for (size_t i = 0; i < v.size(); i++) {
+        if (v[i] != p) continue;
+        v.erase(v.begin() + i);
+        ctx->pooled -= kv.first;
+        g.parked.emplace_back(p, kv.first);
+        break;
+      }
+    }
+  }
+  ctx->capture_blocks.clear();
+  ctx->graphs.emplace(id, std::move(g));
+  *graph_id = id;
+  return TFHIP_OK;
+}
+
+int tfhip_graph_launch(tfhip_ctx* ctx, int64_t graph_id) {
+  if (!ctx) return TFHIP_EINVAL;
+  if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "graph_launch: not during a graph capture");
+  auto it = ctx->graphs.find(graph_id);
+  if (it == ctx->graphs.end()) return ctx->fail(TFHIP_ENOENT, "graph %lld does not exist", (long long)graph_id);
+  TFHIP_HIP(ctx, hipGraphLaunch(it->second.exec, ctx->stream));
+  return TFHIP_OK;
+}
+
+int tfhip_graph_destroy(tfhip_ctx* ctx, int64_t graph_id) {
+  if (!ctx) return TFHIP_EINVAL;
+  auto it = ctx->graphs.find(graph_id);
+  if (it == ctx->graphs.end()) return TFHIP_OK;
+  // queued replays may still run: wait before the blocks can be handed to anyone else
+  (void)hipStreamSynchronize(ctx->stream);
+  (void)hipGraphExecDestroy(it->second.exec);
+  (void)hipGraphDestroy(it->second.graph);
+  for (auto& blk : it->second.parked) {
+    ctx->pooled += blk.second;
+    ctx->pool[blk.second].push_back(blk.first);
+  }
+  for (auto o = ctx->owner.begin(); o != ctx->owner.end();)
+    o = o->second == graph_id ? ctx->owner.erase(o) : std::next(o);
+  ctx->graphs.erase(it);
   return TFHIP_OK;
 }
 

@@ -1706,9 +1706,7 @@ extern "C" int tfhip_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int64_t filter
   if ((int64_t)ci->batch * ci->in_h * ci->in_w > 0x7fffffffLL || w_n > 0x7fffffffLL)
     return ctx->fail(TFHIP_ENOTSUP, "conv2dDerInput: more than 2^31 input pixels");
   if (y_n == 0 || ci->out_c == 0) {  // nothing flows back
-    if (hipMemsetAsync(bdx->ptr, 0, (size_t)x_n * sizeof(float), ctx->stream) != hipSuccess)
-      return ctx->fail(TFHIP_EDEVICE, "conv2dDerInput: memset failed");
-    return TFHIP_OK;
+    return tfhip_fill(ctx, dx, 0.0);
   }
   Temp tdy(ctx), tw(ctx), tflip(ctx);
   GemmArgs p = {};
@@ -1757,9 +1755,10 @@ extern "C" int tfhip_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int64_t filter
         if (mod(top_pad - r0, ci->stride_h) >= ci->filter_h ||
             mod(left_pad - c0, ci->stride_w) >= ci->filter_w)
           some_empty = true;
-    if (some_empty &&
-        hipMemsetAsync(bdx->ptr, 0, (size_t)x_n * sizeof(float), ctx->stream) != hipSuccess)
-      return ctx->fail(TFHIP_EDEVICE, "conv2dDerInput: memset failed");
+    if (some_empty) {  // (a fill kernel, not a memset node: this may run inside a captured graph)
+      const int rc_fill = tfhip_fill(ctx, dx, 0.0);
+      if (rc_fill) return rc_fill;
+    }
     for (int r0 = 0; r0 < ci->stride_h; r0++)
       for (int c0 = 0; c0 < ci->stride_w; c0++) {
         const int Hc = (int)ceil_div(ci->in_h - r0, ci->stride_h);
@@ -1833,9 +1832,7 @@ extern "C" int tfhip_conv2d_der_filter(tfhip_ctx* ctx, int64_t x, int64_t dy, in
       x_n > (1LL << 40))
     return ctx->fail(TFHIP_ENOTSUP, "conv2dDerFilter: more than 2^31 output pixels");
   if (x_n == 0 || y_n == 0) {
-    if (hipMemsetAsync(bdw->ptr, 0, (size_t)w_n * sizeof(float), ctx->stream) != hipSuccess)
-      return ctx->fail(TFHIP_EDEVICE, "conv2dDerFilter: memset failed");
-    return TFHIP_OK;
+    return tfhip_fill(ctx, dw, 0.0);
   }
   Temp tx(ctx), tdy(ctx);
   GemmArgs p = {};

@@ -319,6 +319,33 @@ static napi_value js_resize_nearest(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+/* graphBegin(ctx), graphEnd(ctx) -> id, graphLaunch(ctx, id), graphDestroy(ctx, id) */
+static napi_value js_graph_begin(napi_env env, napi_callback_info info) {
+  ARGS(1);
+  CHECK(tfhip_graph_begin(ctx));
+  return undefined(env);
+}
+static napi_value js_graph_end(napi_env env, napi_callback_info info) {
+  ARGS(1);
+  int64_t id = 0;
+  CHECK(tfhip_graph_end(ctx, &id));
+  napi_value out;
+  if (napi_create_double(env, (double)id, &out) != napi_ok) return NULL;
+  return out;
+}
+static napi_value js_graph_launch(napi_env env, napi_callback_info info) {
+  ARGS(2);
+  I64(1, id);
+  CHECK(tfhip_graph_launch(ctx, id));
+  return undefined(env);
+}
+static napi_value js_graph_destroy(napi_env env, napi_callback_info info) {
+  ARGS(2);
+  I64(1, id);
+  CHECK(tfhip_graph_destroy(ctx, id));
+  return undefined(env);
+}
+
 /* cumsum(ctx, x, out, outer, inner, exclusive, reverse) */
 static napi_value js_cumsum(napi_env env, napi_callback_info info) {
   ARGS(7);
@@ -572,7 +599,9 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"depthwiseConv2dDerInput", js_depthwise_der_input},
       {"depthwiseConv2dDerFilter", js_depthwise_der_filter},
       {"pool2dBackprop", js_pool2d_backprop}, {"resizeNearest", js_resize_nearest},
-      {"select", js_select}, {"cumsum", js_cumsum}, {"lrn", js_lrn}, {"lrnGrad", js_lrn_grad}};
+      {"select", js_select}, {"cumsum", js_cumsum}, {"lrn", js_lrn}, {"lrnGrad", js_lrn_grad},
+      {"graphBegin", js_graph_begin}, {"graphEnd", js_graph_end}, {"graphLaunch", js_graph_launch},
+      {"graphDestroy", js_graph_destroy}};
   for (size_t i = 0; i < sizeof fns / sizeof fns[0]; i++) {
     napi_value f;
     if (napi_create_function(env, fns[i].name, NAPI_AUTO_LENGTH, fns[i].fn, NULL, &f) != napi_ok ||

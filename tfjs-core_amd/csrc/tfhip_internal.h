@@ -57,6 +57,20 @@ struct tfhip_ctx {
     return s;
   }
 
+  // Captured graphs (tfhip_graph_*): while `capturing`, every block handed out is noted; when
+  // the capture ends those blocks belong to the graph (`owner`), which keeps them out of the
+  // pool for as long as it lives, because a replay writes them again.
+  struct Graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    std::vector<std::pair<void*, size_t>> parked;  // owned blocks that no tensor holds
+  };
+  bool capturing = false;
+  std::vector<void*> capture_blocks;
+  std::unordered_map<void*, int64_t> owner;  // block -> graph that owns it
+  std::unordered_map<int64_t, Graph> graphs;
+  int64_t next_graph = 1;
+
   int fail(int code, const char* fmt, ...);
   tfhip::Buf* find(int64_t id);          // sets err when missing
   void* alloc(size_t nbytes, size_t* cap);  // nullptr + err on failure (nbytes > 0)

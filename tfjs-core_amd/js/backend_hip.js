@@ -119,6 +119,41 @@ class MathBackendHIP extends KernelBackend {
     return {unreliable: false, numBytesInGPU: inUse, numBytesInGPUPool: pooled, numDeviceBuffers: ids};
   }
 
+  // Records the kernels that f() queues into a graph that replays with one launch (an extension:
+  // the reference's backends run every op eagerly).  f runs twice: once eagerly, so that the pool
+  // holds every block it needs, then under capture.  Tensors that f reads and did not create
+  // (weights, the input) must outlive the graph; new input data goes into the same tensor
+  // (backend.write).  Returns {outputs, replay(), dispose()}: outputs is what f returned, and
+  // every replay() refreshes it in place.
+  captureGraph(f) {
+    const {ENGINE, getTensorsInContainer} = require('./engine');
+    getTensorsInContainer(ENGINE.tidy(f)).forEach(t => t.dispose());
+    this.napi.graphBegin(this.ctx);
+    let outputs;
+    try {
+      outputs = ENGINE.tidy(f);
+    } catch (e) {
+      try {
+        this.napi.graphDestroy(this.ctx, this.napi.graphEnd(this.ctx));
+      } catch (ignored) {}
+      throw e;
+    }
+    let id = this.napi.graphEnd(this.ctx);
+    return {
+      outputs,
+      replay: () => {
+        this.napi.graphLaunch(this.ctx, id);
+        return outputs;
+      },
+      dispose: () => {
+        if (id == null) return;
+        getTensorsInContainer(outputs).forEach(t => t.dispose());
+        this.napi.graphDestroy(this.ctx, id);
+        id = null;
+      }
+    };
+  }
+
   // Event pair on the backend's stream around everything f() queues (backend.ts:27-31).
   async time(f) {
     this.napi.timeBegin(this.ctx);

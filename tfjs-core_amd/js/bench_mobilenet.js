@@ -30,13 +30,28 @@ async function main() {
   const info = await tf.time(() => { for (let i = 0; i < steps; i++) step(); });
   be.sync();
   const wallMs = Number(process.hrtime.bigint() - t0) / 1e6;
-  // host-only cost of queueing one step (no waiting on the device in between)
   const out = mobilenet.forward(tf, w, x);
   const top = tf.argMax(out.logits, -1).dataSync();
+  const eagerProbs = out.probs.dataSync();
+  // The same step captured once and replayed with one launch per step (tf.captureGraph, an
+  // extension of this backend): what is left when the host's cost per op is taken away.
+  const graph = tf.captureGraph(() => mobilenet.forward(tf, w, x).probs);
+  for (let i = 0; i < warmup; i++) graph.replay();
+  be.sync();
+  const g0 = process.hrtime.bigint();
+  for (let i = 0; i < steps; i++) graph.replay();
+  be.sync();
+  const graphMs = Number(process.hrtime.bigint() - g0) / 1e6;
+  const replayProbs = graph.outputs.dataSync();
+  let maxDiff = 0;
+  for (let i = 0; i < eagerProbs.length; i++) maxDiff = Math.max(maxDiff, Math.abs(eagerProbs[i] - replayProbs[i]));
+  graph.dispose();
   console.log(JSON.stringify({
     images_per_s: batch * steps / (wallMs / 1e3), ms_per_step: wallMs / steps,
     gpu_ms_per_step_events: info.kernelMs / steps, batch, steps, warmup,
-    node: process.version, top1_first: top[0], tensors: tf.memory().numTensors
+    node: process.version, top1_first: top[0], tensors: tf.memory().numTensors,
+    graph_replay: {images_per_s: batch * steps / (graphMs / 1e3), ms_per_step: graphMs / steps,
+                   max_abs_diff_vs_eager: maxDiff}
   }));
 }
 

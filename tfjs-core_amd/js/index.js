@@ -41,6 +41,13 @@ const tf = Object.assign({}, ops, gradients, {
   profile: f => ENGINE.profile(f),
   enableDebugMode: () => ENV.set('DEBUG', true),
   disposeVariables: () => ENGINE.disposeVariables(),
+  // not in the reference: see MathBackendHIP.captureGraph
+  captureGraph: f => {
+    if (typeof ENGINE.backend.captureGraph !== 'function') {
+      throw new Error(`The ${ENGINE.backendName} backend cannot capture graphs`);
+    }
+    return ENGINE.backend.captureGraph(f);
+  },
 });
 
 ENGINE.registerBackend('hip', () => {

@@ -74,6 +74,30 @@ const OPS = {
     opt.dispose();
     return out;
   },
+  // replay(x2) - eager(x2) of a small conv net captured on x: zeros when a replay computes what
+  // the eager ops compute for the data then in the input tensor
+  captureReplay: (i, a) => {
+    const net = () => {
+      let h = tf.fused.conv2d({x: i.x, filter: i.w0, strides: 2, pad: 'same', bias: i.b0, activation: 'relu'});
+      h = tf.depthwiseConv2d(h, i.dw, 1, 'same');
+      h = tf.relu6(tf.conv2d(h, i.w1, 1, 'same'));
+      h = tf.avgPool(h, 4, 4, 'valid');
+      return tf.softmax(tf.matMul(tf.reshape(h, [h.shape[0], h.size / h.shape[0]]), i.fc));
+    };
+    const graph = tf.captureGraph(net);
+    let worst = tf.zerosLike(graph.outputs);
+    for (let k = 0; k < a.replays; k++) {
+      const fresh = tf.add(i.x2, tf.scalar(k));                 // eager work between replays
+      tf.backend().write(i.x.dataId, fresh.dataSync());         // new data into the captured input
+      const eager = net();
+      graph.replay();
+      const next = tf.maximum(worst, tf.abs(tf.sub(graph.outputs, eager)));
+      tf.dispose([worst, fresh, eager]);
+      worst = next;
+    }
+    graph.dispose();
+    return worst;
+  },
   cumsum: (i, a) => tf.cumsum(i.x, a.axis, a.exclusive, a.reverse),
   gradCumsum: (i, a) => tf.grad(x => tf.cumsum(x, a.axis, a.exclusive, a.reverse))(i.x, i.dy),
   lrn: (i, a) => tf.localResponseNormalization(i.x, a.radius, a.bias, a.alpha, a.beta),

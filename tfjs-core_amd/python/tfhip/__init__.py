@@ -53,6 +53,12 @@ def tidy(fn=None):
     return ENGINE.tidy(fn)
 
 
+def capture_graph(f):
+    """backend().capture_graph(f): the kernels f() queues, recorded once and replayed with one
+    launch (backend_hip.MathBackendHIP.capture_graph)."""
+    return ENGINE.backend.capture_graph(f, ENGINE.tidy)
+
+
 def memory():
     return ENGINE.memory()
 

@@ -58,6 +58,10 @@ _SIGNATURES = {
     "tfhip_pool2d": [_PTR, _I64, _I64, C.POINTER(Conv2DInfoC), _INT],
     "tfhip_resize_nearest": [_PTR, _I64, _I64, _INT, _INT, _INT, _INT, _INT, _INT, _INT],
     "tfhip_select": [_PTR, _I64, _I64, _I64, _I64, _I64],
+    "tfhip_graph_begin": [_PTR],
+    "tfhip_graph_end": [_PTR, C.POINTER(C.c_int64)],
+    "tfhip_graph_launch": [_PTR, _I64],
+    "tfhip_graph_destroy": [_PTR, _I64],
     "tfhip_cumsum": [_PTR, _I64, _I64, _I64, _I64, _INT, _INT],
     "tfhip_lrn": [_PTR, _I64, _I64, _I64, _INT, _INT, C.c_float, C.c_float, C.c_float],
     "tfhip_lrn_grad": [_PTR, _I64, _I64, _I64, _I64, _I64, _INT, _INT, C.c_float, C.c_float, C.c_float],

@@ -35,6 +35,24 @@ def _info_c(ci):
         int(p["top"]), int(p["left"]), int(p["bottom"]), int(p["right"]))
 
 
+class _CapturedGraph(object):
+    def __init__(self, backend, gid, outputs):
+        self.backend, self.gid, self.outputs = backend, gid, outputs
+
+    def replay(self):
+        self.backend._ck(self.backend.lib.tfhip_graph_launch(self.backend.ctx, self.gid))
+        return self.outputs
+
+    def dispose(self):
+        if self.gid is None:
+            return
+        outs = self.outputs if isinstance(self.outputs, (list, tuple)) else [self.outputs]
+        for t in outs:
+            t.dispose()
+        self.backend._ck(self.backend.lib.tfhip_graph_destroy(self.backend.ctx, self.gid))
+        self.gid = None
+
+
 class MathBackendHIP(object):
     def __init__(self, device=0):
         self.lib = capi.lib()
@@ -98,6 +116,28 @@ class MathBackendHIP(object):
 
     def sync(self):
         self._ck(self.lib.tfhip_sync(self.ctx))
+
+    def capture_graph(self, f, tidy):
+        """Records the kernels that f() queues into a graph that replays with one launch (an
+        extension: the reference's backends run every op eagerly).  f runs twice: once eagerly, so
+        that the pool holds every block it needs, then under capture.  Tensors that f reads and
+        did not create (weights, the input) must outlive the graph; new input data goes into the
+        same tensor.  Returns an object with .outputs (what f returned, refreshed by every
+        .replay()) and .dispose()."""
+        warm = tidy(f)
+        for t in (warm if isinstance(warm, (list, tuple)) else [warm]):
+            t.dispose()
+        self._ck(self.lib.tfhip_graph_begin(self.ctx))
+        try:
+            outputs = tidy(f)
+        except Exception:
+            gid = C.c_int64()
+            if self.lib.tfhip_graph_end(self.ctx, C.byref(gid)) == 0:
+                self.lib.tfhip_graph_destroy(self.ctx, gid.value)
+            raise
+        gid = C.c_int64()
+        self._ck(self.lib.tfhip_graph_end(self.ctx, C.byref(gid)))
+        return _CapturedGraph(self, gid.value, outputs)
 
     def float_precision(self):
         return 32
