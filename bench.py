@@ -287,7 +287,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported "
-                 "(the path shards by batch, see DESIGN.md)" % args.gpus)
+                 "(the forward pass shards by batch: images are independent, weights replicated)"
+                 % args.gpus)
 
     import numpy as np
     import tfhip as tf

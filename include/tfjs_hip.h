@@ -244,6 +244,11 @@ int tfhip_strided_copy(tfhip_ctx* ctx, int64_t x, int64_t out, int rank, const i
  * [outer, inner]; out float32 or int32 (upcastType(x.dtype, 'int32')). */
 int tfhip_cumsum(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t outer, int64_t inner,
                  int exclusive, int reverse);
+/* topk along the innermost axis (backend.ts:236-238; backends/topk_impl.ts:25-60): x viewed as
+ * [rows, cols] (float32 or int32); values [rows, k] in x's dtype, indices [rows, k] int32, in
+ * descending value order, equal values in ascending index order. */
+int tfhip_topk(tfhip_ctx* ctx, int64_t x, int64_t values, int64_t indices, int64_t rows,
+               int64_t cols, int k);
 /* localResponseNormalization4D and LRNGrad (backend.ts:600-610; backend_cpu.ts:3211-3281) over
  * [pixels, channels] float32: the window is the channels within depth_radius of each one. */
 int tfhip_lrn(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t pixels, int channels,

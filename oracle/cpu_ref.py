@@ -839,3 +839,11 @@ def lrn_grad(dy, x, y, depth_radius=5, bias=1.0, alpha=1.0, beta=0.5):
                 d = d + np.power(norm, -beta)
             res[..., k] += d * dy64[..., o]
     return res.astype(np.float32)
+
+
+def topk(x, k=1):
+    """backends/topk_impl.ts:25-60 along the innermost axis: a stable sort by descending value
+    (equal values keep ascending index order), then the first k."""
+    x = np.asarray(x)
+    order = np.argsort(-x.astype(np.float64), axis=-1, kind="stable")[..., :k]
+    return np.take_along_axis(x, order, -1), order.astype(np.int32)

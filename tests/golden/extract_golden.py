@@ -75,6 +75,7 @@ CASES = {
     "lrn": ("tfjs-core/src/ops/lrn_test.ts", ["localResponseNormalization with Tensor3D",
                                               "localResponseNormalization with Tensor4D"]),
     "cumsum": ("tfjs-core/src/ops/array_ops_test.ts", ["cumsum"]),
+    "topk": ("tfjs-core/src/ops/topk_test.ts", ["topk"]),
     "space_batch_depth": ("tfjs-core/src/ops/array_ops_test.ts",
                           ["batchToSpaceND", "spaceToBatchND", "depthToSpace"]),
     "optimizer_sgd": ("tfjs-core/src/optimizers/sgd_optimizer_test.ts", None),

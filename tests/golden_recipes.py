@@ -1189,3 +1189,18 @@ def cumsum_known_answers(ops):
     expect_close(ops.cumsum(f32(a[0]), 0), a[2])
     a = g("3D standard")
     expect_close(ops.cumsum(f32(a[0]), 2), a[2])
+
+
+# ---- ops/topk_test.ts ----------------------------------------------------------------------
+@recipe
+def topk_known_answers_bit_exact(ops):
+    g = lambda t: golden_case("topk", t, "topk")["arrays"]
+    for title, k, dt in (("1d array with default k", 1, np.float32), ("2d array with default k", 1, np.float32),
+                         ("2d array with k=2", 2, np.float32), ("3d array with k=3", 3, np.float32),
+                         ("topk(int32) propagates int32 dtype", 1, np.int32),
+                         ("lower-index element appears first, k=4", 4, np.float32)):
+        a = g(title)
+        values, indices = ops.topk(np.asarray(a[0], dt), k)
+        assert values.dtype == dt and indices.dtype == np.int32, title
+        assert list(values.shape) == a[1] and list(indices.shape) == a[2], title
+        assert values.ravel().tolist() == a[3] and indices.ravel().tolist() == a[4], title

@@ -120,6 +120,8 @@ class OracleOps:
         moved = np.moveaxis(x, axis, -1)
         return np.moveaxis(self.r.cumsum(moved, exclusive, reverse), -1, axis)
 
+    def topk(self, x, k=1): return self.r.topk(x, k)
+
     def lrn(self, x, radius=5, bias=1.0, alpha=1.0, beta=0.5):
         return self.r.local_response_normalization(x, radius, bias, alpha, beta)
 
@@ -311,6 +313,9 @@ class HipOps:
 
     def cumsum(self, x, axis=0, exclusive=False, reverse=False):
         return self._run(lambda t: self.tf.cumsum(t, axis, exclusive, reverse), x)
+
+    def topk(self, x, k=1):
+        return self._run_list(lambda t: list(self.tf.topk(t, k)), x)
 
     def lrn(self, x, radius=5, bias=1.0, alpha=1.0, beta=0.5):
         return self._run(lambda t: self.tf.local_response_normalization(t, radius, bias, alpha, beta), x)

@@ -491,6 +491,11 @@ def test_js_scan_lrn_and_rearrangements(tmp_path, ref):
         xin = np.asarray(a[0], np.float32)
         c.add("depthToSpace_%d" % k, "depthToSpace", dict(x=xin), dict(blockSize=2), flat(a[2]).reshape(a[1]),
               exact=True)
+    probs = rng.uniform(0, 1, (6, 1000)).astype(np.float32)
+    probs[:, 10:20] = 2.0                      # ties: the lower index comes first
+    tv, ti = ref.topk(probs, 5)
+    c.add("topk_values", "topkValues", dict(x=probs), dict(k=5), tv, exact=True)
+    c.add("topk_indices", "topkIndices", dict(x=probs), dict(k=5), ti, exact=True)
     # and at a size where the blocks are not trivial, against numpy's own reshuffle
     big = rng.standard_normal((2, 5, 7, 36)).astype(np.float32)
     want = big.reshape(2, 5, 7, 3, 3, 4).transpose(0, 1, 3, 2, 4, 5).reshape(2, 15, 21, 4)

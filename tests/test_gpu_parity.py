@@ -384,6 +384,21 @@ def test_local_response_normalization_and_gradient(hip, ref, shape, radius, bias
           rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("shape,k", [((1000,), 5), ((64, 1000), 5), ((3, 7, 130), 130), ((5, 1), 1),
+                                     ((4, 65), 17), ((2, 4000), 64)])
+def test_topk_bit_exact(hip, ref, shape, k):
+    rng = np.random.default_rng(sum(shape) + k)
+    x = rng.standard_normal(shape).astype(np.float32)
+    x[..., ::7] = np.float32(0.25)            # many ties: ascending index order among equals
+    gv, gi = hip.topk(x, k)
+    wv, wi = ref.topk(x, k)
+    assert np.array_equal(gi, wi) and np.array_equal(gv, wv)
+    xi = rng.integers(-5, 6, shape).astype(np.int32)
+    gv, gi = hip.topk(xi, k)
+    wv, wi = ref.topk(xi, k)
+    assert gv.dtype == np.int32 and np.array_equal(gi, wi) and np.array_equal(gv, wv)
+
+
 def test_clip_relu6_nan(hip, ref):
     x = np.array([-3, 0, 2.5, 6, 7.5, np.nan, np.inf, -np.inf], np.float32)
     close(hip.clip(x, 0, 6), ref.clip(x, 0, 6))

@@ -346,6 +346,14 @@ static napi_value js_graph_destroy(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+/* topk(ctx, x, values, indices, rows, cols, k) */
+static napi_value js_topk(napi_env env, napi_callback_info info) {
+  ARGS(7);
+  I64(1, x); I64(2, values); I64(3, indices); I64(4, rows); I64(5, cols); INT(6, k);
+  CHECK(tfhip_topk(ctx, x, values, indices, rows, cols, k));
+  return undefined(env);
+}
+
 /* cumsum(ctx, x, out, outer, inner, exclusive, reverse) */
 static napi_value js_cumsum(napi_env env, napi_callback_info info) {
   ARGS(7);
@@ -601,7 +609,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"pool2dBackprop", js_pool2d_backprop}, {"resizeNearest", js_resize_nearest},
       {"select", js_select}, {"cumsum", js_cumsum}, {"lrn", js_lrn}, {"lrnGrad", js_lrn_grad},
       {"graphBegin", js_graph_begin}, {"graphEnd", js_graph_end}, {"graphLaunch", js_graph_launch},
-      {"graphDestroy", js_graph_destroy}};
+      {"graphDestroy", js_graph_destroy}, {"topk", js_topk}};
   for (size_t i = 0; i < sizeof fns / sizeof fns[0]; i++) {
     napi_value f;
     if (napi_create_function(env, fns[i].name, NAPI_AUTO_LENGTH, fns[i].fn, NULL, &f) != napi_ok ||

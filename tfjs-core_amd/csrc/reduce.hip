@@ -169,6 +169,59 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void cumsum_rows_kernel(
   }
 }
 
+// topk along the innermost axis (backends/topk_impl.ts:25-60: a stable sort by descending value,
+// so equal values keep ascending index order).  One wavefront per row selects the k entries one
+// after the other: entry i is the largest element that comes after entry i-1 in that order
+// (smaller value, or equal value and larger index); ties go to the smallest index.  k passes over
+// the row, which stays in L1/L2; NaN elements are never selected (JavaScript's comparator leaves
+// their place unspecified) and rows that run out of candidates repeat index -1 / value NaN.
+template <typename T>
+__global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void topk_rows_kernel(
+    const T* __restrict__ x, T* __restrict__ values, int32_t* __restrict__ indices, int64_t rows,
+    int64_t cols, int k) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* xr = x + row * cols;
+  bool have_prev = false;
+  T prev_v = T(0);
+  int64_t prev_i = -1;
+  bool exhausted = false;  // (the same for every lane)
+  for (int out = 0; out < k; out++) {
+    bool found = false;
+    T best = T(0);
+    int64_t best_i = cols;
+    for (int64_t j = lane; j < cols && !exhausted; j += WAVE) {
+      const T v = xr[j];
+      if (v != v) continue;
+      if (have_prev && !(v < prev_v || (v == prev_v && j > prev_i))) continue;
+      if (!found || v > best) {  // ascending j within a lane: the first of equal values stays
+        best = v;
+        best_i = j;
+        found = true;
+      }
+    }
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const T ob = __shfl_xor(best, off, WAVE);
+      const int64_t oi = __shfl_xor(best_i, off, WAVE);
+      const int of = __shfl_xor((int)found, off, WAVE);
+      if (of && (!found || ob > best || (ob == best && oi < best_i))) {
+        best = ob;
+        best_i = oi;
+        found = true;
+      }
+    }
+    if (lane == 0) {
+      values[row * k + out] = found ? best : (T)NAN;
+      indices[row * k + out] = found ? (int32_t)best_i : -1;
+    }
+    have_prev = true;
+    prev_v = best;
+    prev_i = best_i;
+    exhausted = !found;
+  }
+}
+
 // out[o, i, :] = x[o, indices[i], :] for 4-byte or 1-byte elements.
 template <typename T>
 __global__ void gather_kernel(const T* x, const int32_t* indices, T* out, int64_t outer,
@@ -362,6 +415,33 @@ extern "C" int tfhip_cumsum(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t oute
   else
     hipLaunchKernelGGL(cumsum_rows_kernel<int32_t>, grid, block, 0, ctx->stream, bx->ptr, bx->dtype,
                        (int32_t*)bo->ptr, outer, inner, exclusive, reverse);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+extern "C" int tfhip_topk(tfhip_ctx* ctx, int64_t x, int64_t values, int64_t indices, int64_t rows,
+                          int64_t cols, int k) {
+  if (!ctx) return TFHIP_EINVAL;
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bv, values);
+  TFHIP_GET(ctx, bi, indices);
+  if (rows < 0 || cols < 0 || k < 0 || k > cols)
+    return ctx->fail(TFHIP_EINVAL, "'k' passed to topk() must be <= the last dimension (%lld) but got %d",
+                     (long long)cols, k);
+  if (bx->numel != rows * cols || bv->numel != rows * k || bi->numel != rows * k)
+    return ctx->fail(TFHIP_EINVAL, "topk: buffer sizes do not match rows x cols and rows x k");
+  if ((bx->dtype != TFHIP_FLOAT32 && bx->dtype != TFHIP_INT32) || bv->dtype != bx->dtype ||
+      bi->dtype != TFHIP_INT32)
+    return ctx->fail(TFHIP_EINVAL, "topk: values keep x's dtype (float32 or int32), indices are int32");
+  if (rows * k == 0) return TFHIP_OK;
+  if (ceil_div(rows, ROWS_PER_BLOCK) > 0x7fffffffLL) return ctx->fail(TFHIP_ENOTSUP, "topk: too many rows");
+  const dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK)), block(WAVE * ROWS_PER_BLOCK);
+  if (bx->dtype == TFHIP_FLOAT32)
+    hipLaunchKernelGGL(topk_rows_kernel<float>, grid, block, 0, ctx->stream, (const float*)bx->ptr,
+                       (float*)bv->ptr, (int32_t*)bi->ptr, rows, cols, k);
+  else
+    hipLaunchKernelGGL(topk_rows_kernel<int32_t>, grid, block, 0, ctx->stream, (const int32_t*)bx->ptr,
+                       (int32_t*)bv->ptr, (int32_t*)bi->ptr, rows, cols, k);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }

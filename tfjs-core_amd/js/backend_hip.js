@@ -456,6 +456,13 @@ class MathBackendHIP extends KernelBackend {
     return out;
   }
   sum(x, axes) { return this.reduce('sum', x, axes, util.upcastType(x.dtype, 'int32')); }
+  topk(x, k, sorted) {
+    const cols = x.shape[x.rank - 1];
+    const outShape = x.shape.slice(0, -1).concat([k]);
+    const values = this.out(outShape, x.dtype), indices = this.out(outShape, 'int32');
+    this.napi.topk(this.ctx, this.h(x), this.h(values), this.h(indices), cols ? x.size / cols : 0, cols, k);
+    return [values, indices];
+  }
   cumsum(x, axis, exclusive, reverse) {
     if (axis !== x.rank - 1) {   // backend_cpu.ts:718-722
       throw new Error(`backend.cumsum expects an inner-most axis=${x.rank - 1} but got axis=${axis}`);

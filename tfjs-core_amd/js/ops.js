@@ -1249,6 +1249,20 @@ const opHandler = {
 };
 setOpHandler(opHandler);
 
+// ops/topk.ts:47-63
+const topk = op('topk', (x, k, sorted) => {
+  let $x = convertToTensor(x, 'x', 'topk');
+  if (k == null) k = 1;
+  if ($x.rank === 0) throw new Error('topk() expects the input to be of rank 1 or higher');
+  const lastDim = $x.shape[$x.shape.length - 1];
+  if (k > lastDim) {
+    throw new Error(`'k' passed to topk() must be <= the last dimension (${lastDim}) but got ${k}`);
+  }
+  if ($x.dtype === 'bool') $x = cast($x, 'int32');
+  const [values, indices] = ENGINE.runKernel(b => b.topk($x, k, sorted == null ? true : sorted), {$x});
+  return {values, indices};
+});
+
 // ---- cumsum, localResponseNormalization, space / batch / depth rearrangements ---------------
 // array_ops.ts:703-731: the axis is brought innermost, scanned and put back; the gradient is
 // the scan of dy in the other direction.
@@ -1377,5 +1391,5 @@ module.exports = {
   floor, ceil, round, sign, expm1, log1p, reciprocal, sin, cos, tan, asin, acos, atan, sinh, cosh,
   asinh, acosh, atanh, erf, elu, selu, softplus, step, leakyRelu, logSigmoid, isNaN: isNaN_, isInf,
   isFinite: isFinite_, pow, squaredDifference, mod, floorDiv, atan2, addN, prod, all, any,
-  cumsum, localResponseNormalization, batchToSpaceND, spaceToBatchND, depthToSpace
+  cumsum, localResponseNormalization, batchToSpaceND, spaceToBatchND, depthToSpace, topk
 };

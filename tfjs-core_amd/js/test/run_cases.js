@@ -98,6 +98,8 @@ const OPS = {
     graph.dispose();
     return worst;
   },
+  topkValues: (i, a) => { const r = tf.topk(i.x, a.k); r.indices.dispose(); return r.values; },
+  topkIndices: (i, a) => { const r = tf.topk(i.x, a.k); r.values.dispose(); return r.indices; },
   cumsum: (i, a) => tf.cumsum(i.x, a.axis, a.exclusive, a.reverse),
   gradCumsum: (i, a) => tf.grad(x => tf.cumsum(x, a.axis, a.exclusive, a.reverse))(i.x, i.dy),
   lrn: (i, a) => tf.localResponseNormalization(i.x, a.radius, a.bias, a.alpha, a.beta),

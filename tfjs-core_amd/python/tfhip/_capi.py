@@ -62,6 +62,7 @@ _SIGNATURES = {
     "tfhip_graph_end": [_PTR, C.POINTER(C.c_int64)],
     "tfhip_graph_launch": [_PTR, _I64],
     "tfhip_graph_destroy": [_PTR, _I64],
+    "tfhip_topk": [_PTR, _I64, _I64, _I64, _I64, _I64, _INT],
     "tfhip_cumsum": [_PTR, _I64, _I64, _I64, _I64, _INT, _INT],
     "tfhip_lrn": [_PTR, _I64, _I64, _I64, _INT, _INT, C.c_float, C.c_float, C.c_float],
     "tfhip_lrn_grad": [_PTR, _I64, _I64, _I64, _I64, _I64, _INT, _INT, C.c_float, C.c_float, C.c_float],

@@ -490,6 +490,15 @@ class MathBackendHIP(object):
     def sum(self, x, axes):
         return self._reduce("sum", x, axes, su.upcast_type(x.dtype, "int32"))
 
+    def topk(self, x, k, is_sorted=True):
+        dt = x.dtype if x.dtype != "bool" else "int32"
+        cols = x.shape[-1]
+        out_shape = tuple(x.shape[:-1]) + (k,)
+        values, indices = self._out(out_shape, dt), self._out(out_shape, "int32")
+        self._ck(self.lib.tfhip_topk(self.ctx, self._h(x), self._h(values), self._h(indices),
+                                     su.size_from_shape(x.shape) // cols if cols else 0, cols, int(k)))
+        return [values, indices]
+
     def cumsum(self, x, axis, exclusive, reverse):
         if axis != x.rank - 1:   # backend_cpu.ts:718-722
             raise ValueError("backend.cumsum expects an inner-most axis=%d but got axis=%d"

@@ -416,6 +416,19 @@ def sum(x, axis=None, keep_dims=False):  # noqa: A001
     return _reduce("sum", xt, axis, keep_dims)
 
 
+def topk(x, k=1, is_sorted=True):
+    """ops/topk.ts:47-63: (values, indices) of the k largest entries along the last axis."""
+    x = _conv(x, "x", "topk")
+    if x.rank == 0:
+        raise ValueError("topk() expects the input to be of rank 1 or higher")
+    if k > x.shape[-1]:
+        raise ValueError("'k' passed to topk() must be <= the last dimension (%d) but got %d"
+                         % (x.shape[-1], k))
+    if x.dtype == "bool":
+        x = cast(x, "int32")
+    return ENGINE.run_kernel(lambda be: be.topk(x, k, is_sorted))
+
+
 def cumsum(x, axis=0, exclusive=False, reverse=False):
     """ops/array_ops.ts:703-731: the axis is brought innermost, scanned, and put back."""
     x = _conv(x, "x", "cumsum")
