@@ -496,6 +496,38 @@ def test_js_scan_lrn_and_rearrangements(tmp_path, ref):
     tv, ti = ref.topk(probs, 5)
     c.add("topk_values", "topkValues", dict(x=probs), dict(k=5), tv, exact=True)
     c.add("topk_indices", "topkIndices", dict(x=probs), dict(k=5), ti, exact=True)
+    m = rng.standard_normal((4, 6, 5)).astype(np.float32)
+    m64 = m.astype(np.float64)
+    c.add("moments_mean", "momentsMean", dict(x=m), dict(axis=[0, 2], keepDims=True),
+          m64.mean((0, 2), keepdims=True).astype(np.float32), atol=1e-5)
+    c.add("moments_var", "momentsVariance", dict(x=m), dict(axis=[0, 2], keepDims=False),
+          m64.var((0, 2)).astype(np.float32), atol=1e-5)
+    for case in _golden_all("reduction_extra"):          # reduction_ops_test.ts: norm, literal blocks
+        a = case["arrays"]
+        if case["describe"] != "Reduction: norm" or case["title"] not in (
+                "vector inf norm", "vector -inf norm", "vector 1 norm", "vector euclidean norm"):
+            continue
+        v = np.asarray(a[0], np.float32)                 # [1, -2, 3, -4]
+        ordv, want = {"vector inf norm": ("inf", 4), "vector -inf norm": ("-inf", 1),
+                      "vector 1 norm": (1, 10), "vector euclidean norm": ("euclidean", np.sqrt(30))}[case["title"]]
+        c.add("norm_" + case["title"].replace(" ", "_"), "norm", dict(x=v), dict(ord=ordv),
+              np.float32(want).reshape(()), atol=1e-5)
+    c.add("norm_fro", "norm", dict(x=m[0]), dict(ord="fro", axis=[0, 1]),
+          np.float32(np.sqrt((m64[0] ** 2).sum())).reshape(()), atol=1e-5)
+    c.add("norm_matrix_1_keep", "norm", dict(x=m[0]), dict(ord=1, axis=[0, 1], keepDims=True),
+          np.abs(m64[0]).sum(0).max().astype(np.float32).reshape(1, 1), atol=1e-5)
+    lg = (rng.standard_normal((7, 33)) * 4).astype(np.float32)
+    l64 = lg.astype(np.float64)
+    lse = np.log(np.exp(l64 - l64.max(1, keepdims=True)).sum(1, keepdims=True)) + l64.max(1, keepdims=True)
+    c.add("log_softmax", "logSoftmax", dict(x=lg), {}, (l64 - lse).astype(np.float32), atol=1e-5)
+    dyl = rng.standard_normal(lg.shape).astype(np.float32)
+    c.add("log_softmax_grad", "gradLogSoftmax", dict(x=lg, dy=dyl), {},
+          (dyl - dyl.astype(np.float64).sum(1, keepdims=True) * np.exp(l64 - lse)).astype(np.float32), atol=1e-4)
+    ch = rng.uniform(0.5, 2, (3, 4)).astype(np.float32)
+    c64 = ch.astype(np.float64)
+    chained = np.maximum(np.sqrt(np.abs(c64)) + (c64 ** 2).mean(1, keepdims=True), -c64)[0:2, 1:4]
+    c.add("chain_more", "chainMore", dict(x=ch), {}, np.pad(chained, ((1, 0), (0, 1))).ravel().astype(np.float32),
+          atol=1e-5)
     # and at a size where the blocks are not trivial, against numpy's own reshuffle
     big = rng.standard_normal((2, 5, 7, 36)).astype(np.float32)
     want = big.reshape(2, 5, 7, 3, 3, 4).transpose(0, 1, 3, 2, 4, 5).reshape(2, 15, 21, 4)

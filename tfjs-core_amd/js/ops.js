@@ -1376,6 +1376,71 @@ const depthToSpace = op('depthToSpace', (x, blockSize, dataFormat) => {
       [b, h * blockSize, w * blockSize, outD]));
 });
 
+// ---- composites of reductions ------------------------------------------------------------
+// reduction_ops.ts:590-603
+const moments = op('moments', (x, axis, keepDims) => {
+  const $x = convertToTensor(x, 'x', 'moments');
+  const axes = util.parseAxisParam(axis == null ? null : axis, $x.shape);
+  const mu = mean($x, axes, !!keepDims);
+  const keepDimsShape = keepDims ? mu.shape : axis_util.expandShapeToKeepDim(mu.shape, axes);
+  const variance = ENGINE.tidy(() =>
+      mean(square(sub(cast($x, 'float32'), reshape(mu, keepDimsShape))), axes, !!keepDims));
+  return {mean: mu, variance};
+});
+
+// ops/norm.ts:64-135: vector norms (1, 2 / 'euclidean', +-Infinity) over one axis, matrix
+// norms (1, +-Infinity, 'fro' / 'euclidean') over two
+function normImpl(x, p, axis) {
+  if (x.rank === 0) return abs(x);
+  if (x.rank !== 1 && axis === null) return normImpl(reshape(x, [x.size]), p, axis);
+  if (x.rank === 1 || typeof axis === 'number' || (Array.isArray(axis) && axis.length === 1)) {
+    if (p === 1) return sum(abs(x), axis);
+    if (p === Infinity) return max(abs(x), axis);
+    if (p === -Infinity) return min(abs(x), axis);
+    if (p === 'euclidean' || p === 2) return sqrt(sum(pow(abs(x), scalar(2, 'int32')), axis));
+    throw new Error(`Error in norm: invalid ord value: ${p}`);
+  }
+  if (Array.isArray(axis) && axis.length === 2) {
+    if (p === 1) return max(sum(abs(x), axis[0]), axis[1] - 1);
+    if (p === Infinity) return max(sum(abs(x), axis[1]), axis[0]);
+    if (p === -Infinity) return min(sum(abs(x), axis[1]), axis[0]);
+    if (p === 'fro' || p === 'euclidean') return sqrt(sum(square(x), axis));
+    throw new Error(`Error in norm: invalid ord value: ${p}`);
+  }
+  throw new Error(`Error in norm: invalid axis: ${axis}`);
+}
+const norm = op('norm', (x, ord, axis, keepDims) => {
+  const $x = convertToTensor(x, 'x', 'norm');
+  if (ord == null) ord = 'euclidean';
+  if (axis === undefined) axis = null;
+  return ENGINE.tidy(() => {
+    const n = normImpl($x, ord, axis);
+    if (!keepDims) return n;
+    const axes = util.parseAxisParam(axis, $x.shape);
+    return reshape(n, axis_util.expandShapeToKeepDim(n.shape, axes));
+  });
+});
+
+// ops/softmax.ts:98-135: x - logSumExp(x) along the last axis, with its own gradient
+const logSoftmax = op('logSoftmax', (logits, axis) => {
+  const $logits = convertToTensor(logits, 'logits', 'logSoftmax');
+  if (axis == null || axis === -1) axis = $logits.rank - 1;
+  if (axis !== $logits.rank - 1) {
+    throw Error('Log Softmax along a non-last dimension is not yet supported. ' +
+                `Logits was rank ${$logits.rank} and axis was ${axis}`);
+  }
+  return ENGINE.customGrad((t, save) => {
+    const xMax = max(t, axis, true);
+    const shifted = sub(t, xMax);
+    const value = sub(cast(shifted, 'float32'), log(sum(exp(shifted), axis, true)));
+    save([value]);
+    return {
+      value,
+      gradFunc: (dy, saved) => sub(dy, mul(sum(dy, axis, true), exp(saved[0])))
+    };
+  })($logits);
+});
+
 module.exports = {
   op, tensor, scalar, tensor1d, tensor2d, tensor3d, tensor4d, quantizedTensor, convertToTensor,
   fill, zeros, ones, zerosLike, onesLike, reshape, cast, clone, dequantize, matMul,
@@ -1391,5 +1456,46 @@ module.exports = {
   floor, ceil, round, sign, expm1, log1p, reciprocal, sin, cos, tan, asin, acos, atan, sinh, cosh,
   asinh, acosh, atanh, erf, elu, selu, softplus, step, leakyRelu, logSigmoid, isNaN: isNaN_, isInf,
   isFinite: isFinite_, pow, squaredDifference, mod, floorDiv, atan2, addN, prod, all, any,
-  cumsum, localResponseNormalization, batchToSpaceND, spaceToBatchND, depthToSpace, topk
+  cumsum, localResponseNormalization, batchToSpaceND, spaceToBatchND, depthToSpace, topk,
+  moments, norm, logSoftmax
 };
+
+// Chaining methods (tensor.ts:700-1460 defines them one by one: x.square().sum() ...): every op
+// above whose first argument is the tensor itself, under the reference's method names.
+const CHAINED = [
+  'abs', 'neg', 'sigmoid', 'sqrt', 'square', 'tanh', 'rsqrt', 'floor', 'ceil', 'round', 'sign', 'expm1',
+  'log1p', 'reciprocal', 'sin', 'cos', 'tan', 'asin', 'acos', 'atan', 'sinh', 'cosh', 'asinh', 'acosh',
+  'atanh', 'erf', 'elu', 'selu', 'softplus', 'step', 'leakyRelu', 'logSigmoid', 'isNaN', 'isInf',
+  'isFinite', 'relu6', 'maximum', 'minimum', 'pow', 'squaredDifference', 'mod', 'floorDiv', 'atan2',
+  'equal', 'notEqual', 'less', 'lessEqual', 'greater', 'greaterEqual', 'logicalAnd', 'logicalOr',
+  'logicalNot', 'mean', 'prod', 'all', 'any', 'cumsum', 'topk', 'norm', 'logSoftmax', 'slice',
+  'stridedSlice', 'reverse', 'pad', 'tile', 'expandDims', 'squeeze', 'unstack', 'split',
+  'resizeBilinear', 'resizeNearestNeighbor', 'localResponseNormalization', 'batchToSpaceND',
+  'spaceToBatchND', 'depthToSpace', 'zerosLike', 'onesLike', 'separableConv2d', 'conv2dTranspose',
+  'pool', 'dequantize'
+];
+CHAINED.forEach(name => {
+  const fn = module.exports[name];
+  if (typeof fn !== 'function' || Tensor.prototype[name] != null) return;
+  Tensor.prototype[name] = function(...args) {
+    this.throwIfDisposed();
+    return fn(this, ...args);
+  };
+});
+Object.assign(Tensor.prototype, {
+  flatten() { return this.as1D(); },
+  asScalar() {
+    util.assert(this.size === 1, () => 'The array must have only 1 element.');
+    return this.reshape([]);
+  },
+  concat(x, axis) {
+    this.throwIfDisposed();
+    return module.exports.concat([this].concat(Array.isArray(x) ? x : [x]), axis);
+  },
+  stack(x, axis) { return module.exports.stack([this, x], axis); },
+  where(condition, x) { return module.exports.where(condition, this, x); },
+  batchNorm(mean, variance, offset, scale, varianceEpsilon) {
+    return module.exports.batchNorm(this, mean, variance, offset, scale, varianceEpsilon);
+  },
+  oneHot(depth, onValue, offValue) { return module.exports.oneHot(this, depth, onValue, offValue); }
+});

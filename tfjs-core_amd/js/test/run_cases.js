@@ -100,6 +100,14 @@ const OPS = {
   },
   topkValues: (i, a) => { const r = tf.topk(i.x, a.k); r.indices.dispose(); return r.values; },
   topkIndices: (i, a) => { const r = tf.topk(i.x, a.k); r.values.dispose(); return r.indices; },
+  momentsMean: (i, a) => { const r = tf.moments(i.x, a.axis, a.keepDims); r.variance.dispose(); return r.mean; },
+  momentsVariance: (i, a) => { const r = tf.moments(i.x, a.axis, a.keepDims); r.mean.dispose(); return r.variance; },
+  norm: (i, a) => tf.norm(i.x, a.ord === 'inf' ? Infinity : a.ord === '-inf' ? -Infinity : a.ord, a.axis, a.keepDims),
+  logSoftmax: i => tf.logSoftmax(i.x),
+  gradLogSoftmax: i => tf.grad(x => tf.logSoftmax(x))(i.x, i.dy),
+  // x.square().sum() style chains over the methods attached to Tensor
+  chainMore: i => i.x.abs().sqrt().add(i.x.square().mean(1, true)).maximum(i.x.neg()).slice([0, 1], [2, 3])
+      .pad([[1, 0], [0, 1]]).expandDims(0).squeeze([0]).flatten(),
   cumsum: (i, a) => tf.cumsum(i.x, a.axis, a.exclusive, a.reverse),
   gradCumsum: (i, a) => tf.grad(x => tf.cumsum(x, a.axis, a.exclusive, a.reverse))(i.x, i.dy),
   lrn: (i, a) => tf.localResponseNormalization(i.x, a.radius, a.bias, a.alpha, a.beta),
