@@ -861,6 +861,37 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
     if (p.prelu_kind == TFHIP_BCAST_SCALAR) alpha_c[j] = p.prelu[0];
     if (p.prelu_kind == TFHIP_BCAST_COLUMN && col < p.N) alpha_c[j] = p.prelu[col];
   }
+  // Where this lane reads its 16 operand values of a strip of 32 output pixels: the LDS index
+  // of (kh, kw, c) at its pixel, or a slot behind the staged rows that holds 0 for k past K.
+  // Every output row has the same strips, so the first strip's addresses are computed once.
+  const int zero_slot = p.KH * row_floats;
+  if (tid == 0) rows[zero_slot] = 0.f;
+  // (a copy of a lane constant that the optimiser cannot see through: the address arithmetic of
+  // the rarely taken paths below then stays inside them instead of being hoisted out of the row
+  // loop into registers that every row pays for)
+  auto opaque = [](int x) {
+    asm volatile("" : "+v"(x));
+    return x;
+  };
+  auto pixel_base = [&](int strip, int lane32) {
+    const int ow = min(strip * 32 + lane32, p.OW - 1);  // clamped: lanes past the row compute a copy
+    return ow * p.sw * p.Cin;
+  };
+  const int base_first = pixel_base(wave, l32);
+  int a_first[4][4];
+#pragma unroll
+  for (int q = 0; q < 4; q++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) a_first[q][e] = a_off[q][e] >= 0 ? a_off[q][e] + base_first : zero_slot;
+  // (rows wider than 128 output pixels: further strips shift the first strip's addresses)
+  auto strip_addresses = [&](int strip, int (&addr)[4][4]) {
+    const int shift = pixel_base(strip, opaque(l32)) - base_first;
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        addr[q][e] = a_first[q][e] == zero_slot ? zero_slot : a_first[q][e] + shift;
+  };
 
   // Staging plan of this lane: elements i = tid + 256u of the [KH][row_floats] block, as
   // (kh, offset in the input row); fixed for the lifetime of the workgroup.  A block of up to
@@ -868,28 +899,30 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
   // current row is computed, so that their latency is hidden behind the matrix-core work.
   const int row_in = p.W * p.Cin;
   const int stage_n = p.KH * row_floats;
-  const bool one_pass = stage_n <= 256 * 8;
-  int st_kh[8], st_e[8];
+  // (one pass also needs 32-bit byte offsets inside one image)
+  const bool one_pass = stage_n <= 256 * 8 && (long long)p.H * row_in * 4 < (1LL << 30);
+  // Per lane and staged element, fixed for the lifetime of the workgroup: the byte offset of
+  // (kh, column) relative to the first input row of an output row, or a value that stays out
+  // of range whatever row offset is added (elements past the block, columns in the padding).
+  // The rows above and below the image fall out of the descriptor's range by themselves: a
+  // negative offset wraps to a huge one.  So a staged element costs one add and one load.
+  unsigned ld_const[8];
 #pragma unroll
   for (int u = 0; u < 8; u++) {
     const int i = tid + u * 256;
     const int kh = i / row_floats;
-    st_kh[u] = i < stage_n ? kh : -1;
-    st_e[u] = i - kh * row_floats - p.pl * p.Cin;
+    const int e = i - kh * row_floats - p.pl * p.Cin;
+    const bool ok = i < stage_n && (unsigned)e < (unsigned)row_in;
+    ld_const[u] = ok ? (unsigned)((kh * p.dh * row_in + e) * 4) : OOB_OFFSET;
   }
-  auto stage_load = [&](int row, float (&v)[8]) {
-    const int n = row / p.OH, oh = row - n * p.OH;
-    const int ih0 = oh * p.sh - p.pt;
-    const float* img = p.A + (long long)n * p.H * row_in;  // same for the whole workgroup
+  const unsigned img_bytes = (unsigned)(p.H * row_in) * 4u;
+  auto stage_load = [&](int n, int oh, float (&v)[8]) {
+    const __amdgpu_buffer_rsrc_t rimg = make_rsrc(p.A + (long long)n * p.H * row_in, img_bytes);
+    const unsigned first = (unsigned)((oh * p.sh - p.pt) * row_in * 4);  // may be "negative"
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
-      const int ih = ih0 + st_kh[u] * p.dh;
-      const bool ok = st_kh[u] >= 0 && (unsigned)ih < (unsigned)p.H &&
-                      (unsigned)st_e[u] < (unsigned)row_in;
-      const int at = ok ? ih * row_in + st_e[u] : 0;
-      const float x = img[at];
-      v[u] = ok ? x : 0.f;
-    }
+    for (int u = 0; u < 8; u++)
+      v[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                           rimg, (int)(ld_const[u] + first), 0, 0));
   };
   // A grid that is a multiple of 8 cuts the output rows into one run per XCD (workgroup b runs
   // on XCD b % 8): neighbouring output rows, which share input rows, then meet in one L2, and
@@ -902,17 +935,31 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
     row_first = run0 + ((int)blockIdx.x >> 3);
     row_step = (int)gridDim.x >> 3;
   }
+  // (image, output row) of the current row and of the next one of this workgroup, advanced by
+  // additions: a division per row would run on the vector ALU
+  const int step_n = row_step / p.OH, step_oh = row_step - step_n * p.OH;
+  auto advance = [&](int& n, int& oh) {
+    n += step_n;
+    oh += step_oh;
+    if (oh >= p.OH) {
+      oh -= p.OH;
+      n++;
+    }
+  };
+  int n = row_first / p.OH, oh = row_first - n * p.OH;
+  int n_next = n, oh_next = oh;
+  advance(n_next, oh_next);
   float v[8];
-  if (one_pass && row_first < row_end) stage_load(row_first, v);
-  for (int row = row_first; row < row_end; row += row_step) {
-    const int n = row / p.OH, oh = row - n * p.OH;
+  if (one_pass && row_first < row_end) stage_load(n, oh, v);
+  for (int row = row_first; row < row_end;
+       row += row_step, n = n_next, oh = oh_next, advance(n_next, oh_next)) {
     __syncthreads();  // the previous row's readers are done
     if (one_pass) {
 #pragma unroll
       for (int u = 0; u < 8; u++)
-        if (st_kh[u] >= 0) rows[tid + u * 256] = v[u];
+        if (tid + u * 256 < stage_n) rows[tid + u * 256] = v[u];
     } else {
-      for (int i0 = tid; i0 < stage_n; i0 += 256 * 8) {
+      for (int i0 = opaque(tid); i0 < stage_n; i0 += 256 * 8) {
         float t[8];
 #pragma unroll
         for (int u = 0; u < 8; u++) {
@@ -933,59 +980,79 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
       }
     }
     __syncthreads();
-    if (one_pass && row + row_step < row_end) stage_load(row + row_step, v);
+    if (one_pass && row + row_step < row_end) stage_load(n_next, oh_next, v);
 
     const long long out_at = (((long long)n * p.OH + oh) * p.OW) * p.N;  // workgroup-uniform
     float* __restrict__ crow = p.C + out_at;
     const ActCfg act = act_cfg(p.act);
     const float* bias_row = p.bias_kind == TFHIP_BCAST_FULL ? p.bias + out_at : nullptr;
     const float* alpha_row = p.prelu_kind == TFHIP_BCAST_FULL ? p.prelu + out_at : nullptr;
+    // the output row as a descriptor: pixels past the row fall out of its range
+    const __amdgpu_buffer_rsrc_t rout = make_rsrc(crow, (unsigned)(p.OW * p.N) * 4u);
     for (int strip = wave; strip * 32 < p.OW; strip += 4) {
-      const int ow = min(strip * 32 + l32, p.OW - 1);  // clamped: lanes past the row compute a copy
-      const int base = ow * p.sw * p.Cin;
       f32x16 acc[TN];
 #pragma unroll
       for (int j = 0; j < TN; j++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+      auto multiply = [&](const int (&addr)[4][4]) {
 #pragma unroll
-      for (int q = 0; q < 4; q++) {
-        float a[4];
+        for (int q = 0; q < 4; q++) {
+          float a[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const float x = rows[max(a_off[q][e], 0) + base];
-          a[e] = a_off[q][e] >= 0 ? x : 0.f;
+          for (int e = 0; e < 4; e++) a[e] = rows[addr[q][e]];
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+              acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[q][e][j], acc[j], 0, 0, 0);
         }
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-#pragma unroll
-          for (int j = 0; j < TN; j++)
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[q][e][j], acc[j], 0, 0, 0);
+      };
+      if (strip == wave) {
+        multiply(a_first);
+      } else {
+        int addr[4][4];
+        strip_addresses(strip, addr);
+        multiply(addr);
       }
       // accumulator register r holds pixel 8*(r/4) + 4*(lane/32) + r%4 of the strip
       const int px0 = strip * 32 + 4 * g;
-      auto store = [&](auto full_tag) {
-        constexpr bool full = decltype(full_tag)::value;
+      if (bias_row || alpha_row) {
+        const int px0_ = opaque(px0), l32_ = opaque(l32);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          const int px = px0 + 8 * (r >> 2) + (r & 3);
+          const int px = px0_ + 8 * (r >> 2) + (r & 3);
 #pragma unroll
           for (int j = 0; j < TN; j++) {
-            const int col = 32 * j + l32;
+            const int col = 32 * j + l32_;
             if (px < p.OW && col < p.N) {
               const int at = px * p.N + col;
-              float bv = bias_c[j], al = alpha_c[j];
-              if (full) {
-                if (bias_row) bv = bias_row[at];
-                if (alpha_row) al = alpha_row[at];
-              }
+              const float bv = bias_row ? bias_row[at] : bias_c[j];
+              const float al = alpha_row ? alpha_row[at] : alpha_c[j];
               crow[at] = activate(acc[j][r] + bv, act, al);
             }
           }
         }
-      };
-      if (bias_row || alpha_row) store(std::true_type{});
-      else store(std::false_type{});
+      } else {
+        // one add per store: the lane's base offset (out of range for a column past N) plus
+        // the register's pixel offset, which is the same for all lanes
+        unsigned lane_at[TN];
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          const int col = 32 * j + l32;
+          lane_at[j] = col < p.N ? (unsigned)((px0 * p.N + col) * 4) : OOB_OFFSET;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const unsigned px_at = (unsigned)((8 * (r >> 2) + (r & 3)) * p.N * 4);
+#pragma unroll
+          for (int j = 0; j < TN; j++) {
+            const float v = activate(acc[j][r] + bias_c[j], act, alpha_c[j]);
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rout,
+                                                  (int)(lane_at[j] + px_at), 0, 0);
+          }
+        }
+      }
     }
   }
 }
@@ -1592,7 +1659,7 @@ extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t o
     const long long span = (long long)(ci->out_w - 1) * ci->stride_w +
                            (long long)(ci->filter_w - 1) * ci->dilation_w + 1;
     const long long row_floats = span * ci->in_c;
-    const long long lds = row_floats * ci->filter_h * (long long)sizeof(float);
+    const long long lds = (row_floats * ci->filter_h + 1) * (long long)sizeof(float);  // + the zero slot
     if (lds <= 64 * 1024) {
       const int n_rows = ci->batch * ci->out_h;
       // one workgroup per resident slot: each walks its share of the output rows
