@@ -168,6 +168,21 @@ def test_rowstream_products(tf, ref, n, h, w_, cin, cout, act, bias, quant, want
     assert nan_rows.sum() == 1 and nan_rows[0, 7, 5]
 
 
+def test_rowstream_scalar_bias_and_slope(tf):
+    """fused matMul with a scalar bias and a scalar prelu slope through the row-streaming kernel."""
+    rng = np.random.default_rng(78)
+    m = 256 * 8 * 32 * 3 + 11
+    a = rng.uniform(-1, 1, (m, 32)).astype(np.float32)
+    b = rng.uniform(-1, 1, (32, 64)).astype(np.float32)
+    with tf.tidy():
+        got = tf.fused.matmul(tf.tensor(a), tf.tensor(b), bias=tf.tensor(np.float32(0.25)),
+                              activation="prelu",
+                              prelu_activation_weights=tf.tensor(np.float32(0.1))).data_sync()
+        assert last_kernel(tf) == "gemm_rowstream_k32xn64_f32", last_kernel(tf)
+    y = a.astype(np.float64) @ b.astype(np.float64) + 0.25
+    close(got, np.where(y < 0, np.float64(np.float32(0.1)) * y, y))
+
+
 def test_rowstream_matmul_and_small_fallback(tf):
     """tf.matMul of the same shape class takes the row-streaming kernel; below the row threshold
     and with a full-shape bias the tiled kernels keep the product."""

@@ -1664,9 +1664,13 @@ extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t o
       const int n_rows = ci->batch * ci->out_h;
       // one workgroup per resident slot: each walks its share of the output rows
       auto launch = [&](auto kernel, const char* name) {
-        int per_cu = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, (size_t)lds) !=
-                hipSuccess || per_cu < 1) {
+        // resident workgroups per CU for this kernel and LDS size, asked once (the query
+        // costs microseconds, which a batch-1 step would pay on every call)
+        static std::map<size_t, int> resident;
+        int& per_cu = resident[(size_t)lds];
+        if (per_cu == 0 &&
+            (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, (size_t)lds) !=
+                 hipSuccess || per_cu < 1)) {
           (void)hipGetLastError();
           per_cu = 1;
         }
