@@ -283,6 +283,39 @@ int tfhip_resize_nearest(tfhip_ctx* ctx, int64_t x, int64_t out, int batch, int 
  * storage dtype (the host upcasts, backend_cpu.ts:828). */
 int tfhip_select(tfhip_ctx* ctx, int64_t condition, int64_t a, int64_t b, int64_t out,
                  int64_t inner);
+/* gatherND (backend.ts:499; backend_cpu.ts:3771-3803): x of shape x_shape[rank]; indices
+ * [num_slices, slice_rank] int32 address its first slice_rank dimensions; out
+ * [num_slices, product of the remaining dimensions] in x's element size.  An index outside x
+ * fails with "Invalid indices: <index> does not index into <shape>" (:3796-3799); the check
+ * waits for the device, so the call is not available during a graph capture. */
+int tfhip_gather_nd(tfhip_ctx* ctx, int64_t x, int64_t indices, int64_t out,
+                    const int32_t* x_shape, int rank, int64_t num_slices, int slice_rank);
+/* scatterND, sparseToDense and unsortedSegmentSum (backend.ts:193, 499-503, 624-627;
+ * backend_cpu.ts:635-660, 3759-3769, 3805-3814, 3842-3889): out of shape out_shape[rank]
+ * (float32 or int32) starts at default_value; update i (a slice of the trailing
+ * rank - slice_rank dimensions, or one value shared by all) goes to the slice
+ * indices[i, :] addresses, in ascending i.  flags:
+ *   TFHIP_SCATTER_SUM           add to what is there (scatterND); without it the update
+ *                               replaces it and the last one wins (sparseToDense)
+ *   TFHIP_SCATTER_SKIP_INVALID  an index outside the result is skipped (unsortedSegmentSum
+ *                               ignores such segment ids); without it the call fails as
+ *                               tfhip_gather_nd does
+ *   TFHIP_SCATTER_WIDE_SUM      float32 sums are kept in double and rounded once
+ *                               (unsortedSegmentSum); without it every addition rounds to
+ *                               float32 as the reference's typed array does */
+enum { TFHIP_SCATTER_SUM = 1, TFHIP_SCATTER_SKIP_INVALID = 2, TFHIP_SCATTER_WIDE_SUM = 4 };
+int tfhip_scatter_nd(tfhip_ctx* ctx, int64_t indices, int64_t updates, int64_t out,
+                     const int32_t* out_shape, int rank, int64_t num_updates, int slice_rank,
+                     double default_value, int flags);
+/* cropAndResize (backend.ts:612-616; backend_cpu.ts:3622-3757): images [batch,h,w,c]; boxes
+ * [num_boxes,4] float32 rows (y1,x1,y2,x2) in normalised coordinates; box_index [num_boxes]
+ * int32; out [num_boxes,crop_h,crop_w,c] float32.  Samples outside the image get
+ * extrapolation_value; a box whose image index is outside the batch yields zeros. */
+enum { TFHIP_RESIZE_BILINEAR = 0, TFHIP_RESIZE_NEAREST = 1 };
+int tfhip_crop_and_resize(tfhip_ctx* ctx, int64_t images, int64_t boxes, int64_t box_index,
+                          int64_t out, int batch, int image_h, int image_w, int channels,
+                          int64_t num_boxes, int crop_h, int crop_w, int method,
+                          float extrapolation_value);
 
 /* ---- backward kernels (training) ---------------------------------------------------------- */
 /* `info` is the Conv2DInfo of the FORWARD op in every call below (in_* = x, out_* = y).
@@ -307,6 +340,16 @@ int tfhip_depthwise_conv2d_der_filter(tfhip_ctx* ctx, int64_t x, int64_t dy, int
  * lay inside the image, as the reference does.  Dilation is allowed (tf.pool). */
 int tfhip_pool2d_backprop(tfhip_ctx* ctx, int64_t dy, int64_t x, int64_t dx,
                           const tfhip_conv2d_info* info, int kind);
+/* resizeBilinearBackprop / resizeNearestNeighborBackprop (backend.ts:591-598;
+ * backend_cpu.ts:2938-3013, 3070-3165): dy [batch,y_h,y_w,c] float32 -> dx [batch,x_h,x_w,c]
+ * float32, the gradient of the resize of an x_h x x_w image to y_h x y_w.  Contributions to
+ * one dx element are added in the reference's order, so the results do not depend on
+ * scheduling.  (The reference labels the bilinear result [batch,x_w,x_h,c]; the data is in
+ * [batch,x_h,x_w,c] order in both.) */
+int tfhip_resize_bilinear_backprop(tfhip_ctx* ctx, int64_t dy, int64_t dx, int batch, int x_h,
+                                   int x_w, int channels, int y_h, int y_w, int align_corners);
+int tfhip_resize_nearest_backprop(tfhip_ctx* ctx, int64_t dy, int64_t dx, int batch, int x_h,
+                                  int x_w, int channels, int y_h, int y_w, int align_corners);
 
 #ifdef __cplusplus
 }

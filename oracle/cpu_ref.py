@@ -847,3 +847,214 @@ def topk(x, k=1):
     x = np.asarray(x)
     order = np.argsort(-x.astype(np.float64), axis=-1, kind="stable")[..., :k]
     return np.take_along_axis(x, order, -1), order.astype(np.int32)
+
+
+def _slice_geometry(shape, slice_rank):
+    """Slice size and, in units of slices, the stride of each indexed dimension
+    (ops/gather_nd_util.ts:71-78, ops/scatter_nd_util.ts:131-147)."""
+    shape = [int(d) for d in shape]
+    slice_size = int(np.prod(shape[slice_rank:], dtype=np.int64))
+    strides = [int(np.prod(shape[j + 1:slice_rank], dtype=np.int64)) for j in range(slice_rank)]
+    return slice_size, strides
+
+
+def gather_nd(x, indices):
+    """backends/cpu/backend_cpu.ts:3771-3803: the loop over slices, with the reference's error
+    for an index outside x."""
+    x, indices = np.asarray(x), np.asarray(indices)
+    slice_rank = indices.shape[-1]
+    slice_size, strides = _slice_geometry(x.shape, slice_rank)
+    flat_x = x.reshape(-1, slice_size) if slice_size else x.reshape(0, 0)
+    rows = indices.reshape(-1, slice_rank)
+    out = np.zeros((rows.shape[0], slice_size), x.dtype)
+    for i, index in enumerate(rows):
+        flat = sum(int(d) * s for d, s in zip(index, strides))
+        if flat < 0 or flat >= flat_x.shape[0]:
+            raise ValueError("Invalid indices: %s does not index into %s"
+                             % (",".join(str(int(d)) for d in index), ",".join(map(str, x.shape))))
+        out[i] = flat_x[flat]
+    return out.reshape(tuple(indices.shape[:-1]) + tuple(x.shape[slice_rank:]))
+
+
+def scatter(indices, updates, shape, default_value=0, sum_dupe_indices=True):
+    """backends/cpu/backend_cpu.ts:3842-3889: scatterND (sums duplicates, default 0) and
+    sparseToDense (the last duplicate wins, any default) share this loop; updates are applied
+    one after the other, each sum rounded to the result's element type."""
+    indices, updates = np.asarray(indices), np.asarray(updates)
+    slice_rank = indices.shape[-1] if indices.ndim > 1 else 1
+    slice_size, strides = _slice_geometry(shape, slice_rank)
+    dtype = updates.dtype if updates.dtype != np.bool_ else np.int32
+    out = np.full((int(np.prod(shape, dtype=np.int64)) // max(slice_size, 1), slice_size), default_value, dtype)
+    rows = indices.reshape(-1, slice_rank) if indices.size else np.zeros((0, slice_rank), np.int32)
+    flat_updates = updates.reshape(-1)
+    for i, index in enumerate(rows):
+        flat = sum(int(d) * s for d, s in zip(index, strides))
+        if flat < 0 or flat >= out.shape[0]:
+            raise ValueError("Invalid indices: %s does not index into %s"
+                             % (",".join(str(int(d)) for d in index), ",".join(map(str, shape))))
+        for k in range(slice_size):
+            if sum_dupe_indices:
+                out[flat, k] = out[flat, k] + flat_updates[i * slice_size + k]
+            else:
+                out[flat, k] = flat_updates[0] if updates.ndim == 0 else flat_updates[i * slice_size + k]
+    return out.reshape(tuple(shape))
+
+
+def unsorted_segment_sum(x, segment_ids, num_segments):
+    """backends/cpu/backend_cpu.ts:635-660 for segments along axis 0: row s of the result is
+    sum over i of (segment_ids[i] == s) * x[i], a masked sum over every row in ascending i
+    (float32: accumulated in double, rounded once, as backend_cpu.ts:590-611 sums)."""
+    x = np.asarray(x)
+    ids = np.asarray(segment_ids).reshape((-1,) + (1,) * (x.ndim - 1))
+    rows = []
+    for s in range(num_segments):
+        masked = (ids == s).astype(np.float32) * x.astype(np.float32)
+        rows.append(masked.astype(np.float64).sum(axis=0).astype(np.float32))
+    return np.stack(rows) if rows else np.zeros((0,) + x.shape[1:], np.float32)
+
+
+def _resize_scales(x_h, x_w, y_h, y_w, align_corners):
+    ex_h = x_h - 1 if (align_corners and y_h > 1) else x_h
+    ex_w = x_w - 1 if (align_corners and y_w > 1) else x_w
+    ey_h = y_h - 1 if (align_corners and y_h > 1) else y_h
+    ey_w = y_w - 1 if (align_corners and y_w > 1) else y_w
+    return ex_h / ey_h, ex_w / ey_w
+
+
+def resize_bilinear_backprop(dy, x_shape, align_corners):
+    """backends/cpu/backend_cpu.ts:2938-3013: every dy pixel is spread over its four source
+    pixels, into a float32 array (each += is a double add rounded to float32)."""
+    dy = _f32(dy)
+    batch, x_h, x_w, depth = x_shape
+    _, y_h, y_w, _ = dy.shape
+    scale_h, scale_w = _resize_scales(x_h, x_w, y_h, y_w, align_corners)
+    out = np.zeros((batch, x_h, x_w, depth), np.float32)
+
+    def add(b, r, c, values):
+        out[b, r, c] = (out[b, r, c].astype(np.float64) + values).astype(np.float32)
+
+    for b in range(batch):
+        for r in range(y_h):
+            dx_r = r * scale_h
+            top, bottom = math.floor(dx_r), min(math.ceil(dx_r), x_h - 1)
+            lerp_r = dx_r - top
+            for c in range(y_w):
+                dx_c = c * scale_w
+                left, right = math.floor(dx_c), min(math.ceil(dx_c), x_w - 1)
+                lerp_c = dx_c - left
+                g = dy[b, r, c].astype(np.float64)
+                add(b, top, left, g * ((1.0 - lerp_r) * (1.0 - lerp_c)))
+                add(b, top, right, g * ((1.0 - lerp_r) * lerp_c))
+                add(b, bottom, left, g * (lerp_r * (1.0 - lerp_c)))
+                add(b, bottom, right, g * (lerp_r * lerp_c))
+    return out
+
+
+def resize_nearest_neighbor_backprop(dy, x_shape, align_corners):
+    """backends/cpu/backend_cpu.ts:3070-3165 restated from the forward side: dy pixel (r, c)
+    belongs to the x pixel the forward pass read for it; the reference's windowed search
+    visits exactly those pixels, in ascending (r, c), summing in double."""
+    dy = _f32(dy)
+    batch, x_h, x_w, depth = x_shape
+    _, y_h, y_w, _ = dy.shape
+    scale_h, scale_w = _resize_scales(x_h, x_w, y_h, y_w, align_corners)
+    pick = (lambda v: math.floor(v + 0.5)) if align_corners else math.floor
+    acc = np.zeros((batch, x_h, x_w, depth), np.float64)
+    for r in range(y_h):
+        sr = min(x_h - 1, pick(r * scale_h))
+        for c in range(y_w):
+            sc = min(x_w - 1, pick(c * scale_w))
+            acc[:, sr, sc] += dy[:, r, c]
+    return acc.astype(np.float32)
+
+
+def crop_and_resize(images, boxes, box_index, crop_size, method="bilinear", extrapolation_value=0.0):
+    """backends/cpu/backend_cpu.ts:3622-3757."""
+    images, boxes = _f32(images), _f32(boxes).astype(np.float64)
+    batch, img_h, img_w, ch = images.shape
+    crop_h, crop_w = crop_size
+    n = boxes.shape[0]
+    out = np.zeros((n, crop_h, crop_w, ch), np.float32)
+    im = images.astype(np.float64)
+    for b in range(n):
+        y1, x1, y2, x2 = boxes[b]
+        ind = int(np.asarray(box_index)[b])
+        if ind >= batch:
+            continue
+        scale_h = (y2 - y1) * (img_h - 1) / (crop_h - 1) if crop_h > 1 else 0.0
+        scale_w = (x2 - x1) * (img_w - 1) / (crop_w - 1) if crop_w > 1 else 0.0
+        for y in range(crop_h):
+            fy = y1 * (img_h - 1) + y * scale_h if crop_h > 1 else 0.5 * (y1 + y2) * (img_h - 1)
+            if fy < 0 or fy > img_h - 1:
+                out[b, y] = extrapolation_value
+                continue
+            for x in range(crop_w):
+                fx = x1 * (img_w - 1) + x * scale_w if crop_w > 1 else 0.5 * (x1 + x2) * (img_w - 1)
+                if fx < 0 or fx > img_w - 1:
+                    out[b, y, x] = extrapolation_value
+                    continue
+                if method == "bilinear":
+                    top, bottom = math.floor(fy), math.ceil(fy)
+                    left, right = math.floor(fx), math.ceil(fx)
+                    wy, wx = fy - top, fx - left
+                    up = im[ind, top, left] + (im[ind, top, right] - im[ind, top, left]) * wx
+                    down = im[ind, bottom, left] + (im[ind, bottom, right] - im[ind, bottom, left]) * wx
+                    out[b, y, x] = up + (down - up) * wy
+                else:
+                    out[b, y, x] = images[ind, math.floor(fy + 0.5), math.floor(fx + 0.5)]
+    return out
+
+
+def non_max_suppression(boxes, scores, max_output_size, iou_threshold=0.5, score_threshold=-math.inf):
+    """backends/non_max_suppression_impl.ts:25-102: candidates above the score threshold in
+    descending score (a stable sort keeps equal scores in index order), each kept unless it
+    overlaps an already selected box by iou_threshold or more."""
+    boxes = _f32(boxes).astype(np.float64).reshape(-1, 4)
+    scores = _f32(scores).astype(np.float64)
+    order = [i for i in sorted(range(len(scores)), key=lambda i: -scores[i]) if scores[i] > score_threshold]
+
+    def iou(i, j):
+        ymin_i, ymax_i = sorted((boxes[i][0], boxes[i][2]))
+        xmin_i, xmax_i = sorted((boxes[i][1], boxes[i][3]))
+        ymin_j, ymax_j = sorted((boxes[j][0], boxes[j][2]))
+        xmin_j, xmax_j = sorted((boxes[j][1], boxes[j][3]))
+        area_i = (ymax_i - ymin_i) * (xmax_i - xmin_i)
+        area_j = (ymax_j - ymin_j) * (xmax_j - xmin_j)
+        if area_i <= 0 or area_j <= 0:
+            return 0.0
+        inter = max(min(ymax_i, ymax_j) - max(ymin_i, ymin_j), 0.0) * \
+            max(min(xmax_i, xmax_j) - max(xmin_i, xmin_j), 0.0)
+        return inter / (area_i + area_j - inter)
+
+    selected = []
+    for i in order:
+        if len(selected) >= max_output_size:
+            break
+        if all(iou(i, j) < iou_threshold for j in reversed(selected)):
+            selected.append(i)
+    return np.asarray(selected, np.int32)
+
+
+def diag(x):
+    """backends/cpu/backend_cpu.ts:346-354 with the result shape of ops/diag.ts:45-49."""
+    x = np.asarray(x)
+    out = np.zeros((x.size, x.size), x.dtype)
+    out[np.arange(x.size), np.arange(x.size)] = x.ravel()
+    return out.reshape(x.shape + x.shape)
+
+
+def linspace(start, stop, num):
+    """backends/backend_util.ts:78-88: a running float32 sum of the double step."""
+    step = (stop - start) / (num - 1) if num != 1 else math.nan
+    values = np.zeros(num, np.float32)
+    if num:
+        values[0] = start
+    for i in range(1, num):
+        values[i] = np.float32(float(values[i - 1]) + step)
+    return values
+
+
+def where_indices(condition):
+    """backends/where_impl.ts:25-43: the coordinates of the true elements, row-major."""
+    condition = np.asarray(condition)
+    return np.argwhere(condition.astype(bool)).astype(np.int32).reshape(-1, condition.ndim)

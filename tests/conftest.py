@@ -33,6 +33,14 @@ def golden_case(fixture, title, describe=None):
     raise KeyError((fixture, describe, title))
 
 
+def golden_cases(fixture):
+    """All cases of a fixture, in the order of the reference's test file."""
+    if fixture not in _cache:
+        with open(os.path.join(GOLDEN, fixture + ".json")) as f:
+            _cache[fixture] = json.load(f)
+    return _cache[fixture]["cases"]
+
+
 def f32(a, shape=None):
     x = np.array(a, dtype=np.float32)
     return x.reshape(shape) if shape is not None else x

@@ -88,6 +88,13 @@ CASES = {
     "reduction_extra": ("tfjs-core/src/ops/reduction_ops_test.ts",
                         ["Reduction: prod", "Reduction: all", "Reduction: any",
                          "Reduction: moments", "Reduction: norm"]),
+    "gather_nd": ("tfjs-core/src/ops/gather_nd_test.ts", ["gatherND"]),
+    "scatter_nd": ("tfjs-core/src/ops/scatter_nd_test.ts", ["scatterND"]),
+    "sparse_to_dense": ("tfjs-core/src/ops/sparse_to_dense_test.ts", ["sparseToDense"]),
+    "segment": ("tfjs-core/src/ops/segment_ops_test.ts", ["unsortedSegmentSum"]),
+    "image": ("tfjs-core/src/ops/image_ops_test.ts", ["nonMaxSuppression", "cropAndResize"]),
+    "diag": ("tfjs-core/src/ops/diag_test.ts", ["diag"]),
+    "linspace_range": ("tfjs-core/src/ops/array_ops_test.ts", ["linspace", "range"]),
 }
 # fixture name -> (reference test file, describe blocks, title filter): the gradient blocks,
 # whose expected values pin the backward kernels (conv2dDerInput / conv2dDerFilter behind
@@ -101,6 +108,10 @@ GRAD_CASES = {
                        ["depthwiseConv2d gradients"], r"^(beforeEach|wrt )"),
     "pool_grad": ("tfjs-core/src/ops/pool_test.ts", ["maxPoolBackprop", "avgPool", "poolBackprop"],
                   r"gradient"),
+    "resize_bilinear_grad": ("tfjs-core/src/ops/resize_bilinear_test.ts", ["resizeBilinear gradients"],
+                             r"^(greyscale|color)"),
+    "resize_nearest_grad": ("tfjs-core/src/ops/resize_nearest_neighbor_test.ts",
+                            ["resizeNearestNeighbor gradients"], r"^(greyscale|color)"),
 }
 # blocks whose title matches are not forward known-answer cases
 SKIP = re.compile(r"grad|throw|raises|tensor-like|TensorLike|does not match|do not match|"

@@ -8,8 +8,9 @@ tf-like calls used below; the same recipes run against the CPU oracle (no GPU ne
 and against the hip backend through the C ABI (-m gpu).
 """
 import numpy as np
+import pytest
 
-from conftest import expect_close, f32, golden_case
+from conftest import expect_close, f32, golden_case, golden_cases
 
 RECIPES = []
 
@@ -1204,3 +1205,158 @@ def topk_known_answers_bit_exact(ops):
         assert values.dtype == dt and indices.dtype == np.int32, title
         assert list(values.shape) == a[1] and list(indices.shape) == a[2], title
         assert values.ravel().tolist() == a[3] and indices.ravel().tolist() == a[4], title
+
+
+# ---- ops/gather_nd_test.ts, scatter_nd_test.ts, sparse_to_dense_test.ts, segment_ops_test.ts --
+@recipe
+def gather_nd_known_answers_bit_exact(ops):
+    for c in golden_cases("gather_nd"):
+        a = c["arrays"]
+        if len(a) == 5:      # indices, indices shape, input (1-D), result shape, expected
+            idx, x = np.asarray(a[0], np.int32).reshape(a[1]), np.asarray(a[2], np.float32)
+            shape, want = a[3], a[4]
+        else:                # indices, indices shape, input, input shape, result shape, expected
+            idx, x = np.asarray(a[0], np.int32).reshape(a[1]), np.asarray(a[2], np.float32).reshape(a[3])
+            shape, want = a[4], a[5]
+        r = ops.gather_nd(x, idx)
+        assert list(r.shape) == shape and r.ravel().tolist() == want, c["title"]
+    # int32 and bool data keep their type; an index outside the tensor is an error
+    x = np.arange(24, dtype=np.int32).reshape(2, 3, 4)
+    r = ops.gather_nd(x, np.asarray([[1, 2], [0, 0]], np.int32))
+    assert r.dtype == np.int32 and r.tolist() == [x[1, 2].tolist(), x[0, 0].tolist()]
+    with pytest.raises(Exception, match="Invalid indices: 2,0 does not index into 2,3,4"):
+        ops.gather_nd(x, np.asarray([[1, 2], [2, 0]], np.int32))
+
+
+@recipe
+def scatter_nd_known_answers(ops):
+    g = lambda t: golden_case("scatter_nd", t)["arrays"]
+    a = g("should work for 2d")
+    r = ops.scatter_nd(np.asarray(a[0], np.int32), f32(a[1], a[2]), a[3])
+    assert list(r.shape) == a[3] and r.ravel().tolist() == a[4]
+    for title in ("should work for simple 1d", "should work for multiple 1d", "should sum the duplicated indices"):
+        a = g(title)
+        r = ops.scatter_nd(np.asarray(a[0], np.int32), f32(a[1]), a[2])
+        assert r.dtype == np.float32 and r.ravel().tolist() == a[3], title
+    a = g("should work for high rank updates")
+    r = ops.scatter_nd(np.asarray(a[0], np.int32).reshape(a[1]), f32(a[2], a[3]), a[4])
+    assert r.ravel().tolist() == a[5]
+    a = g("should work for high rank indices")
+    r = ops.scatter_nd(np.asarray(a[0], np.int32).reshape(a[1]), f32(a[2]), a[3])
+    assert r.ravel().tolist() == a[4]
+    a = g("should work for high rank indices and update")
+    r = ops.scatter_nd(np.asarray(a[0], np.int32).reshape(a[1]), np.ones(a[2], np.float32), a[3])
+    assert list(r.shape) == a[3]
+    assert r[1, 0].tolist() == [1.0] * 256 and r[0, 1].tolist() == [2.0] * 256 and not r[0, 0].any()
+    with pytest.raises(Exception, match="Invalid indices: 5 does not index into 5"):
+        ops.scatter_nd(np.asarray([0, 5], np.int32), f32([1, 2]), [5])
+
+
+@recipe
+def sparse_to_dense_known_answers(ops):
+    g = lambda t: golden_case("sparse_to_dense", t)["arrays"]
+    a = g("should work for scalar indices")
+    r = ops.sparse_to_dense(np.asarray(2, np.int32), np.asarray(100, np.int32), a[0], 0)
+    assert r.dtype == np.int32 and r.tolist() == a[1]
+    a = g("should work for vector")
+    r = ops.sparse_to_dense(np.asarray(a[0], np.int32), f32(a[1]), a[2], 0)
+    assert r.dtype == np.float32 and r.tolist() == a[3]
+    a = g("should work for scalar value")
+    r = ops.sparse_to_dense(np.asarray(a[0], np.int32), np.asarray(10, np.int32), a[1], 0)
+    assert r.tolist() == a[2]
+    for title, default in (("should work for matrix", 0), ("should allow setting default value", 1),
+                           ("no default value passed", 0)):
+        a = g(title)
+        r = ops.sparse_to_dense(np.asarray(a[0], np.int32).reshape(a[1]), f32(a[2]), a[3], default)
+        assert list(r.shape) == a[3] and r.ravel().tolist() == a[4], title
+    a = g("should work with 0-sized tensors")
+    r = ops.sparse_to_dense(np.zeros(a[0], np.int32), np.zeros(a[1], np.float32), a[2], 5)
+    assert r.tolist() == a[3]
+    # the last of several values for one index wins
+    r = ops.sparse_to_dense(np.asarray([1, 1, 3], np.int32), f32([7, 8, 9]), [4], -1)
+    assert r.tolist() == [-1, 8, -1, 9]
+
+
+@recipe
+def unsorted_segment_sum_known_answers(ops):
+    g = lambda t: golden_case("segment", t)
+    c = g("tensor1D")
+    expect_close(ops.unsorted_segment_sum(f32(c["arrays"][0]), np.asarray(c["arrays"][1], np.int32),
+                                          c["consts"]["numSegments"]), c["arrays"][3])
+    c = g("ignores negative segmentIds")
+    expect_close(ops.unsorted_segment_sum(f32(c["arrays"][0]), np.asarray(c["arrays"][1], np.int32),
+                                          c["consts"]["numSegments"]), c["arrays"][3])
+    for title in ("tensor2D", "tensor3D"):
+        c = g(title)
+        a = c["arrays"]
+        expect_close(ops.unsorted_segment_sum(f32(a[0], a[1]), np.asarray(a[2], np.int32),
+                                              c["consts"]["numSegments"]), a[4])
+
+
+# ---- ops/resize_bilinear_test.ts, resize_nearest_neighbor_test.ts (gradients), image_ops_test.ts,
+# diag_test.ts, array_ops_test.ts (linspace) ----------------------------------------------------
+@recipe
+def resize_gradients(ops):
+    for name, fn in (("resize_bilinear_grad", ops.resize_bilinear_grad),
+                     ("resize_nearest_grad", ops.resize_nearest_grad)):
+        cases = golden_cases(name)
+        assert len(cases) >= 19
+        for c in cases:
+            a = c["arrays"]
+            x, dy = np.asarray(a[0], np.float32), np.asarray(a[1], np.float32)
+            assert list(dy.shape[:2]) == a[3], c["title"]
+            dx = fn(x, dy, c["consts"]["alignCorners"])
+            assert dx.shape == x.shape, c["title"]
+            expect_close(dx, np.asarray(a[4], np.float32).ravel())
+
+
+@recipe
+def crop_and_resize_known_answers(ops):
+    cases = [c for c in golden_cases("image") if c["describe"] == "cropAndResize"]
+    assert len(cases) == 19
+    for c in cases:
+        a, title = c["arrays"], c["title"]
+        method = "nearest" if title.lower().endswith("nearest") else "bilinear"
+        extrapolation = c["consts"].get("val", 0)
+        r = ops.crop_and_resize(f32(a[0], a[1]), f32(a[2], a[3]), np.asarray(a[4], np.int32), a[5], method,
+                                extrapolation)
+        assert list(r.shape) == a[6], title
+        if a[7] is not None:
+            expect_close(r, a[7])
+        else:   # 2x2to3x3-Extrapolated: the box (-1,-1,1,1) keeps the image in its lower right quarter
+            v = extrapolation
+            expect_close(r, [v, v, v, v, 1, 2, v, 3, 4])
+
+
+@recipe
+def non_max_suppression_known_answers_bit_exact(ops):
+    for c in golden_cases("image"):
+        a, k = c["arrays"], c["consts"]
+        if c["describe"] != "nonMaxSuppression" or len(a) != 5 or a[0] is None:
+            continue
+        r = ops.non_max_suppression(f32(a[0], a[1]), f32(a[2]), k["maxOutputSize"], k["iouThreshold"],
+                                    k["scoreThreshold"])
+        assert r.dtype == np.int32 and list(r.shape) == a[3] and r.tolist() == a[4], c["title"]
+    # ten identical boxes with equal scores: the first one survives
+    r = ops.non_max_suppression(np.tile(f32([0, 0, 1, 1]), (10, 1)), np.full(10, 0.9, np.float32), 3, 0.5, 0)
+    assert r.tolist() == [0]
+
+
+@recipe
+def diag_and_linspace_known_answers(ops):
+    for title, dt in (("2d", np.float32), ("3d", np.float32), ("4d", np.float32)):
+        a = golden_case("diag", title)["arrays"]
+        r = ops.diag(np.asarray(a[0], dt).reshape(a[1]))
+        assert list(r.shape) == a[2] and r.ravel().tolist() == a[3], title
+    r = ops.diag(np.asarray([1, 2, 3], np.int32))
+    assert r.dtype == np.int32 and r.tolist() == [[1, 0, 0], [0, 2, 0], [0, 0, 3]]
+    g = lambda t: golden_case("linspace_range", t, "linspace")["arrays"]
+    a = g("start stop")
+    expect_close(ops.linspace(1, 10, 10), a[0])
+    expect_close(ops.linspace(12, 17, 8), a[2])
+    expect_close(ops.linspace(9, 0, 6), a[4])
+    expect_close(ops.linspace(-4, 5, 6), g("negative start stop")[0])
+    expect_close(ops.linspace(4, -5, 6), g("start negative stop")[0])
+    a = g("negative start negative stop")
+    expect_close(ops.linspace(-4, -5, 6), a[0])
+    expect_close(ops.linspace(-9, -4, 5), a[2])

@@ -128,6 +128,35 @@ class OracleOps:
     def lrn_grad(self, dy, x, y, radius=5, bias=1.0, alpha=1.0, beta=0.5):
         return self.r.lrn_grad(dy, x, y, radius, bias, alpha, beta)
 
+    def gather_nd(self, x, indices): return self.r.gather_nd(x, indices)
+
+    def scatter_nd(self, indices, updates, shape): return self.r.scatter(indices, updates, shape, 0, True)
+
+    def sparse_to_dense(self, indices, values, shape, default=0):
+        return self.r.scatter(indices, values, shape, default, False)
+
+    def unsorted_segment_sum(self, x, ids, num): return self.r.unsorted_segment_sum(x, ids, num)
+
+    def resize_bilinear_grad(self, x, dy, align):
+        r = self.r.resize_bilinear_backprop(dy[None] if x.ndim == 3 else dy,
+                                            (1,) + x.shape if x.ndim == 3 else x.shape, align)
+        return r[0] if x.ndim == 3 else r
+
+    def resize_nearest_grad(self, x, dy, align):
+        r = self.r.resize_nearest_neighbor_backprop(dy[None] if x.ndim == 3 else dy,
+                                                    (1,) + x.shape if x.ndim == 3 else x.shape, align)
+        return r[0] if x.ndim == 3 else r
+
+    def crop_and_resize(self, image, boxes, box_ind, crop_size, method="bilinear", extrapolation=0):
+        return self.r.crop_and_resize(image, boxes, box_ind, crop_size, method, extrapolation)
+
+    def non_max_suppression(self, boxes, scores, max_out, iou=0.5, score=-np.inf):
+        return self.r.non_max_suppression(boxes, scores, max_out, iou, score)
+
+    def diag(self, x): return self.r.diag(x)
+
+    def linspace(self, start, stop, num): return self.r.linspace(start, stop, num)
+
     def binary(self, name, a, b):
         fn = dict(pow=self.r.pow_, squared_difference=self.r.squared_difference, mod=self.r.mod,
                   floor_div=self.r.floor_div, atan2=self.r.atan2)[name]
@@ -322,6 +351,35 @@ class HipOps:
 
     def lrn_grad(self, dy, x, y, radius=5, bias=1.0, alpha=1.0, beta=0.5):
         return self._run(lambda d, a, b: self.tf.lrn_grad(d, a, b, radius, bias, alpha, beta), dy, x, y)
+
+    def gather_nd(self, x, indices): return self._run(self.tf.gather_nd, x, indices)
+
+    def scatter_nd(self, indices, updates, shape):
+        return self._run(lambda i, u: self.tf.scatter_nd(i, u, shape), indices, updates)
+
+    def sparse_to_dense(self, indices, values, shape, default=0):
+        return self._run(lambda i, v: self.tf.sparse_to_dense(i, v, shape, default), indices, values)
+
+    def unsorted_segment_sum(self, x, ids, num):
+        return self._run(lambda t, i: self.tf.unsorted_segment_sum(t, i, num), x, ids)
+
+    def resize_bilinear_grad(self, x, dy, align):
+        return self._run(lambda a, d: self.tf.resize_bilinear_backprop(d, a, align), x, dy)
+
+    def resize_nearest_grad(self, x, dy, align):
+        return self._run(lambda a, d: self.tf.resize_nearest_neighbor_backprop(d, a, align), x, dy)
+
+    def crop_and_resize(self, image, boxes, box_ind, crop_size, method="bilinear", extrapolation=0):
+        return self._run(lambda im, b, i: self.tf.crop_and_resize(im, b, i, crop_size, method, extrapolation),
+                         image, boxes, box_ind)
+
+    def non_max_suppression(self, boxes, scores, max_out, iou=0.5, score=-np.inf):
+        return self._run(lambda b, s: self.tf.non_max_suppression(b, s, max_out, iou, score), boxes, scores)
+
+    def diag(self, x): return self._run(self.tf.diag, x)
+
+    def linspace(self, start, stop, num): return self._run(lambda: self.tf.linspace(start, stop, num))
+
     def binary(self, name, a, b): return self._run(getattr(self.tf, name), a, b)
     def reduce(self, name, x): return self._run(lambda t: getattr(self.tf, name)(t, -1), x)
     def add_n(self, xs): return self._run(lambda *ts: self.tf.add_n(list(ts)), *xs)

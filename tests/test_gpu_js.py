@@ -706,3 +706,125 @@ def test_js_gradients_through_the_tape(tmp_path, ref):
     assert losses.shape == (12,) and np.all(np.isfinite(losses))
     assert losses[-1] < 0.7 * losses[0] and np.all(np.diff(losses) < 1e-3), losses
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
+def test_js_index_driven_ops_and_image_utilities(tmp_path, ref):
+    """gatherND, scatterND, sparseToDense, unsortedSegmentSum, cropAndResize, nonMaxSuppression,
+    diag, linspace, the resize gradients and the host-side where / multinomial through the JS
+    host: the reference's own vectors (gather_nd_test.ts, scatter_nd_test.ts,
+    sparse_to_dense_test.ts, segment_ops_test.ts, image_ops_test.ts, diag_test.ts,
+    resize_*_test.ts gradients) and seeded cases against the oracle."""
+    rng = np.random.default_rng(97)
+    c = Cases(tmp_path)
+    i32 = lambda a, shape=None: np.asarray(a, np.int32).reshape(shape if shape is not None else -1)
+    f = lambda a, shape=None: np.asarray(a, np.float32).reshape(shape if shape is not None else -1)
+    for k, case in enumerate(_golden_all("gather_nd")):
+        a = case["arrays"]
+        if len(a) == 5:
+            c.add("gather_nd_%d" % k, "gatherND", dict(x=f(a[2]), indices=i32(a[0], a[1])), {}, f(a[4], a[3]),
+                  exact=True)
+        else:
+            c.add("gather_nd_%d" % k, "gatherND", dict(x=f(a[2], a[3]), indices=i32(a[0], a[1])), {},
+                  f(a[5], a[4]), exact=True)
+    x = rng.standard_normal((5, 6, 7, 3)).astype(np.float32)
+    idx = np.stack([rng.integers(0, 5, 40), rng.integers(0, 6, 40)], 1).astype(np.int32).reshape(8, 5, 2)
+    c.add("gather_nd_seeded", "gatherND", dict(x=x, indices=idx), {}, ref.gather_nd(x, idx), exact=True)
+    g = lambda name, title: [cc for cc in _golden_all(name) if cc["title"] == title][0]["arrays"]
+    a = g("scatter_nd", "should work for 2d")
+    c.add("scatter_nd_2d", "scatterND", dict(indices=i32(a[0]), updates=f(a[1], a[2])), dict(shape=a[3]),
+          f(a[4], a[3]), exact=True)
+    a = g("scatter_nd", "should sum the duplicated indices")
+    c.add("scatter_nd_dupes", "scatterND", dict(indices=i32(a[0]), updates=f(a[1])), dict(shape=a[2]), f(a[3]),
+          exact=True)
+    a = g("scatter_nd", "should work for high rank updates")
+    c.add("scatter_nd_high_rank", "scatterND", dict(indices=i32(a[0], a[1]), updates=f(a[2], a[3])),
+          dict(shape=a[4]), f(a[5], a[4]), exact=True)
+    # many duplicates: the additions happen in update order, so the sums are bit-equal to the oracle's
+    sidx = rng.integers(0, 9, (300, 1)).astype(np.int32)
+    supd = rng.standard_normal((300, 17)).astype(np.float32)
+    c.add("scatter_nd_seeded", "scatterND", dict(indices=sidx, updates=supd), dict(shape=[9, 17]),
+          ref.r.scatter(sidx, supd, [9, 17], 0, True), exact=True)
+    a = g("sparse_to_dense", "should allow setting default value")
+    c.add("sparse_to_dense_default", "sparseToDense", dict(indices=i32(a[0], a[1]), values=f(a[2])),
+          dict(shape=a[3], defaultValue=1), f(a[4], a[3]), exact=True)
+    c.add("sparse_to_dense_last_wins", "sparseToDense", dict(indices=i32([1, 1, 3]), values=f([7, 8, 9])),
+          dict(shape=[4], defaultValue=-1), f([-1, 8, -1, 9]), exact=True)
+    for case in _golden_all("segment"):
+        a, n = case["arrays"], case["consts"]["numSegments"]
+        if a[0] is None:
+            continue
+        if len(a) == 4:
+            c.add("segment_" + case["title"].replace(" ", "_"), "unsortedSegmentSum", dict(x=f(a[0]), ids=i32(a[1])),
+                  dict(numSegments=n), f(a[3]))
+        else:
+            c.add("segment_" + case["title"], "unsortedSegmentSum", dict(x=f(a[0], a[1]), ids=i32(a[2])),
+                  dict(numSegments=n), f(a[4]).reshape([n] + a[1][1:]))
+    sx = rng.standard_normal((200, 4, 5)).astype(np.float32)
+    ids = rng.integers(-1, 7, 200).astype(np.int32)
+    c.add("segment_seeded", "unsortedSegmentSum", dict(x=sx, ids=ids), dict(numSegments=6),
+          ref.unsorted_segment_sum(sx, ids, 6), atol=1e-5)
+    sdy = rng.standard_normal((6, 4, 5)).astype(np.float32)
+    c.add("segment_grad", "gradUnsortedSegmentSum", dict(x=sx, ids=np.minimum(ids, 5), dy=sdy), dict(numSegments=6),
+          np.where((ids >= 0)[:, None, None], sdy[np.clip(ids, 0, 5)], 0).astype(np.float32), exact=True)
+    for k, case in enumerate(cc for cc in _golden_all("image") if cc["describe"] == "cropAndResize"):
+        a, title = case["arrays"], case["title"]
+        if a[7] is None or not a[2]:
+            continue
+        c.add("crop_%d" % k, "cropAndResize", dict(image=f(a[0], a[1]), boxes=f(a[2], a[3]), boxInd=i32(a[4])),
+              dict(cropSize=a[5], method="nearest" if title.lower().endswith("nearest") else "bilinear",
+                   extrapolationValue=0), f(a[7], a[6]), atol=1e-5)
+    img = rng.standard_normal((3, 9, 11, 4)).astype(np.float32)
+    boxes = rng.uniform(-0.2, 1.2, (7, 4)).astype(np.float32)
+    bind = rng.integers(0, 3, 7).astype(np.int32)
+    for method in ("bilinear", "nearest"):
+        c.add("crop_seeded_" + method, "cropAndResize", dict(image=img, boxes=boxes, boxInd=bind),
+              dict(cropSize=[5, 6], method=method, extrapolationValue=-7.5),
+              ref.crop_and_resize(img, boxes, bind, [5, 6], method, -7.5), atol=1e-5)
+    for k, case in enumerate(cc for cc in _golden_all("image") if cc["describe"] == "nonMaxSuppression"):
+        a, kk = case["arrays"], case["consts"]
+        if len(a) != 5 or a[0] is None or not a[0]:
+            continue
+        c.add("nms_%d" % k, "nonMaxSuppression", dict(boxes=f(a[0], a[1]), scores=f(a[2])),
+              dict(maxOutputSize=kk["maxOutputSize"], iouThreshold=kk["iouThreshold"],
+                   scoreThreshold=kk["scoreThreshold"]), i32(a[4]), exact=True)
+    nb = rng.uniform(0, 1, (60, 4)).astype(np.float32)
+    ns = rng.uniform(0, 1, 60).astype(np.float32)
+    c.add("nms_seeded", "nonMaxSuppression", dict(boxes=nb, scores=ns),
+          dict(maxOutputSize=20, iouThreshold=0.3, scoreThreshold=0.1),
+          ref.non_max_suppression(nb, ns, 20, 0.3, 0.1), exact=True)
+    a = g("diag", "3d")
+    c.add("diag_3d", "diag", dict(x=f(a[0], a[1])), {}, f(a[3], a[2]), exact=True)
+    c.add("linspace", "linspace", {}, dict(start=-9, stop=-4, num=5), ref.linspace(-9, -4, 5), exact=True)
+    cond = rng.uniform(0, 1, (4, 5, 3)) > 0.6
+    c.add("where_coordinates", "whereCoordinates", dict(x=cond), {}, ref.r.where_indices(cond), exact=True)
+    for name, op in (("resize_bilinear_grad", "gradResizeBilinear"), ("resize_nearest_grad", "gradResizeNearest")):
+        for k, case in enumerate(_golden_all(name)):
+            a = case["arrays"]
+            xin, dy = np.asarray(a[0], np.float32), np.asarray(a[1], np.float32)
+            c.add("%s_%d" % (name, k), op, dict(x=xin, dy=dy), dict(size=a[3], alignCorners=case["consts"]["alignCorners"]),
+                  np.asarray(a[4], np.float32).reshape(xin.shape), atol=1e-3)
+    # seeded shapes, batch and channels, both directions of scaling: equal to the oracle's scatter loop
+    for k, (xs, ys, align) in enumerate((((2, 5, 7, 3), (11, 4), False), ((2, 5, 7, 3), (11, 4), True),
+                                         ((1, 12, 9, 2), (5, 20), False), ((1, 12, 9, 2), (5, 20), True),
+                                         ((1, 1, 6, 2), (4, 1), True))):
+        xin = rng.standard_normal(xs).astype(np.float32)
+        dy = rng.standard_normal((xs[0],) + ys + (xs[3],)).astype(np.float32)
+        c.add("bilinear_grad_seeded_%d" % k, "gradResizeBilinear", dict(x=xin, dy=dy), dict(size=list(ys), alignCorners=align),
+              ref.r.resize_bilinear_backprop(dy, xs, align), exact=True)
+        c.add("nearest_grad_seeded_%d" % k, "gradResizeNearest", dict(x=xin, dy=dy), dict(size=list(ys), alignCorners=align),
+              ref.r.resize_nearest_neighbor_backprop(dy, xs, align), exact=True)
+    probs = np.asarray([0.1, 0.2, 0.3, 0.4], np.float32)
+    c.add("multinomial_frequencies", "multinomialFrequencies", dict(probs=probs), dict(numSamples=20000, seed=3),
+          probs, atol=0.02, rtol=0)
+    xs = rng.standard_normal((6, 8, 5)).astype(np.float32)
+    c.add("strided_slice", "stridedSlice", dict(x=xs),
+          dict(begin=[1, 7, 0], end=[6, 0, 5], strides=[2, -3, 1], beginMask=0, endMask=4, shrinkAxisMask=0),
+          xs[1:6:2, 7:0:-3, :], exact=True)
+    c.add("split_piece", "splitPiece", dict(x=xs), dict(sizes=[3, 1, 4], axis=1, pick=2), xs[:, 4:8], exact=True)
+    c.add("split_grad", "gradSplit", dict(x=xs), dict(sizes=[3, 5], axis=1),
+          np.concatenate([np.ones((6, 3, 5)), np.full((6, 5, 5), 2.0)], 1).astype(np.float32), exact=True)
+    dya = rng.standard_normal((3, 4)).astype(np.float32)
+    c.add("add_n_grad", "gradAddN", dict(a=xs[0, :3, :4], b=xs[1, :3, :4], dy=dya), {}, dya + dya, exact=True)
+    results = c.run()
+    c.check(results)
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0

@@ -399,6 +399,80 @@ def test_topk_bit_exact(hip, ref, shape, k):
     assert gv.dtype == np.int32 and np.array_equal(gi, wi) and np.array_equal(gv, wv)
 
 
+@pytest.mark.parametrize("x_shape,y_size,align", [
+    ((2, 7, 9, 5), (15, 4), False), ((2, 7, 9, 5), (15, 4), True), ((1, 16, 16, 8), (5, 5), False),
+    ((1, 16, 16, 8), (5, 5), True), ((3, 4, 4, 1), (4, 4), False), ((1, 1, 5, 3), (6, 1), True),
+    ((1, 3, 3, 2), (1, 1), True), ((1, 6, 1, 2), (13, 7), False)])
+def test_resize_backprops_bit_exact(hip, ref, x_shape, y_size, align):
+    """Both resize gradients equal the oracle's restatement of the reference's loops bit for
+    bit: contributions are added in the same order with the same roundings."""
+    rng = np.random.default_rng(sum(x_shape) + sum(y_size) + align)
+    x = rng.standard_normal(x_shape).astype(np.float32)
+    dy = rng.standard_normal((x_shape[0],) + y_size + (x_shape[3],)).astype(np.float32)
+    assert np.array_equal(hip.resize_bilinear_grad(x, dy, align), ref.resize_bilinear_grad(x, dy, align))
+    assert np.array_equal(hip.resize_nearest_grad(x, dy, align), ref.resize_nearest_grad(x, dy, align))
+
+
+def test_resize_bilinear_backprop_is_the_adjoint_of_the_forward_pass(hip):
+    """<resize(x), dy> == <x, backprop(dy)> for the linear map resizeBilinear, at a size the
+    pure-Python oracle would take minutes for."""
+    rng = np.random.default_rng(5)
+    for align in (False, True):
+        x = rng.standard_normal((4, 33, 47, 16)).astype(np.float32)
+        dy = rng.standard_normal((4, 70, 29, 16)).astype(np.float32)
+        y = hip.resize_bilinear(x, [70, 29], align)
+        dx = hip.resize_bilinear_grad(x, dy, align)
+        lhs = float((y.astype(np.float64) * dy).sum()), float((x.astype(np.float64) * dx).sum())
+        assert abs(lhs[0] - lhs[1]) <= 1e-4 * max(1.0, abs(lhs[0])), lhs
+        yn = hip.resize_nearest(x, [70, 29], align)
+        dxn = hip.resize_nearest_grad(x, dy, align)
+        rhs = float((yn.astype(np.float64) * dy).sum()), float((x.astype(np.float64) * dxn).sum())
+        assert abs(rhs[0] - rhs[1]) <= 1e-4 * max(1.0, abs(rhs[0])), rhs
+
+
+@pytest.mark.parametrize("method", ["bilinear", "nearest"])
+def test_crop_and_resize(hip, ref, method):
+    rng = np.random.default_rng(len(method))
+    img = rng.standard_normal((3, 12, 10, 6)).astype(np.float32)
+    boxes = rng.uniform(-0.3, 1.3, (9, 4)).astype(np.float32)
+    boxes[0] = [0, 0, 1, 1]
+    boxes[1] = [1, 1, 0, 0]                       # flipped
+    boxes[2] = [0.25, 0.25, 0.25, 0.25]           # degenerate
+    ind = rng.integers(0, 3, 9).astype(np.int32)
+    ind[3] = 3                                    # outside the batch: zeros
+    for crop in ([7, 5], [1, 1], [1, 4], [12, 10]):
+        got = hip.crop_and_resize(img, boxes, ind, crop, method, 2.5)
+        close(got, ref.crop_and_resize(img, boxes, ind, crop, method, 2.5), rtol=1e-6, atol=1e-6)
+        assert not got[3].any()
+
+
+def test_gather_nd_scatter_nd_round_trip_and_types(hip, ref):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((6, 5, 4, 33)).astype(np.float32)
+    for depth in (1, 2, 3, 4):
+        idx = np.stack([rng.integers(0, x.shape[d], 50) for d in range(depth)], 1).astype(np.int32)
+        assert np.array_equal(hip.gather_nd(x, idx), ref.gather_nd(x, idx))
+    xb = rng.uniform(0, 1, (7, 9)) > 0.5
+    idx = np.stack([rng.integers(0, 7, 20), rng.integers(0, 9, 20)], 1).astype(np.int32).reshape(4, 5, 2)
+    got = hip.gather_nd(xb, idx)
+    assert got.shape == (4, 5) and np.array_equal(got.astype(bool), ref.gather_nd(xb, idx))
+    # a permutation scattered and gathered back is the identity
+    perm = rng.permutation(40).astype(np.int32).reshape(40, 1)
+    rows = rng.standard_normal((40, 19)).astype(np.float32)
+    scattered = hip.scatter_nd(perm, rows, [40, 19])
+    assert np.array_equal(hip.gather_nd(scattered, perm), rows)
+    # duplicates: float sums in update order, int32 sums exact
+    idx = rng.integers(0, 5, (500, 1)).astype(np.int32)
+    upd = rng.standard_normal((500, 3)).astype(np.float32)
+    assert np.array_equal(hip.scatter_nd(idx, upd, [5, 3]), ref.scatter_nd(idx, upd, [5, 3]))
+    updi = rng.integers(-9, 9, (500, 3)).astype(np.int32)
+    got = hip.scatter_nd(idx, updi, [5, 3])
+    assert got.dtype == np.int32 and np.array_equal(got, ref.scatter_nd(idx, updi, [5, 3]))
+    ids = rng.integers(-2, 9, 300).astype(np.int32)
+    seg = rng.standard_normal((300, 6, 2)).astype(np.float32)
+    close(hip.unsorted_segment_sum(seg, ids, 7), ref.unsorted_segment_sum(seg, ids, 7), rtol=1e-6, atol=1e-6)
+
+
 def test_clip_relu6_nan(hip, ref):
     x = np.array([-3, 0, 2.5, 6, 7.5, np.nan, np.inf, -np.inf], np.float32)
     close(hip.clip(x, 0, 6), ref.clip(x, 0, 6))

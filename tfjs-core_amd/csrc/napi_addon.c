@@ -319,6 +319,56 @@ static napi_value js_resize_nearest(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+/* gatherND(ctx, x, indices, out, xShape:Int32Array, numSlices, sliceRank) */
+static napi_value js_gather_nd(napi_env env, napi_callback_info info) {
+  ARGS(7);
+  I64(1, x); I64(2, indices); I64(3, out);
+  const int32_t* shape; size_t rank;
+  if (!arg_i32_array(env, argv[4], &shape, &rank)) return NULL;
+  I64(5, num_slices); INT(6, slice_rank);
+  CHECK(tfhip_gather_nd(ctx, x, indices, out, shape, (int)rank, num_slices, slice_rank));
+  return undefined(env);
+}
+
+/* scatterND(ctx, indices, updates, out, outShape:Int32Array, numUpdates, sliceRank, defaultValue, sumDupes) */
+static napi_value js_scatter_nd(napi_env env, napi_callback_info info) {
+  ARGS(9);
+  I64(1, indices); I64(2, updates); I64(3, out);
+  const int32_t* shape; size_t rank;
+  if (!arg_i32_array(env, argv[4], &shape, &rank)) return NULL;
+  I64(5, num_updates); INT(6, slice_rank); F64(7, default_value); INT(8, sum_dupes);
+  CHECK(tfhip_scatter_nd(ctx, indices, updates, out, shape, (int)rank, num_updates, slice_rank,
+                         default_value, sum_dupes));
+  return undefined(env);
+}
+
+/* cropAndResize(ctx, images, boxes, boxIndex, out, batch, h, w, channels, numBoxes, cropH, cropW, method, extrapolation) */
+static napi_value js_crop_and_resize(napi_env env, napi_callback_info info) {
+  ARGS(14);
+  I64(1, images); I64(2, boxes); I64(3, box_index); I64(4, out);
+  INT(5, batch); INT(6, h); INT(7, w); INT(8, ch); I64(9, num_boxes); INT(10, crop_h); INT(11, crop_w);
+  INT(12, method); F64(13, extrapolation);
+  CHECK(tfhip_crop_and_resize(ctx, images, boxes, box_index, out, batch, h, w, ch, num_boxes, crop_h,
+                              crop_w, method, (float)extrapolation));
+  return undefined(env);
+}
+
+/* resizeBilinearBackprop / resizeNearestBackprop(ctx, dy, dx, batch, xH, xW, channels, yH, yW, alignCorners) */
+static napi_value js_resize_bilinear_backprop(napi_env env, napi_callback_info info) {
+  ARGS(10);
+  I64(1, dy); I64(2, dx);
+  INT(3, batch); INT(4, x_h); INT(5, x_w); INT(6, ch); INT(7, y_h); INT(8, y_w); INT(9, align);
+  CHECK(tfhip_resize_bilinear_backprop(ctx, dy, dx, batch, x_h, x_w, ch, y_h, y_w, align));
+  return undefined(env);
+}
+static napi_value js_resize_nearest_backprop(napi_env env, napi_callback_info info) {
+  ARGS(10);
+  I64(1, dy); I64(2, dx);
+  INT(3, batch); INT(4, x_h); INT(5, x_w); INT(6, ch); INT(7, y_h); INT(8, y_w); INT(9, align);
+  CHECK(tfhip_resize_nearest_backprop(ctx, dy, dx, batch, x_h, x_w, ch, y_h, y_w, align));
+  return undefined(env);
+}
+
 /* graphBegin(ctx), graphEnd(ctx) -> id, graphLaunch(ctx, id), graphDestroy(ctx, id) */
 static napi_value js_graph_begin(napi_env env, napi_callback_info info) {
   ARGS(1);
@@ -609,7 +659,10 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"pool2dBackprop", js_pool2d_backprop}, {"resizeNearest", js_resize_nearest},
       {"select", js_select}, {"cumsum", js_cumsum}, {"lrn", js_lrn}, {"lrnGrad", js_lrn_grad},
       {"graphBegin", js_graph_begin}, {"graphEnd", js_graph_end}, {"graphLaunch", js_graph_launch},
-      {"graphDestroy", js_graph_destroy}, {"topk", js_topk}};
+      {"graphDestroy", js_graph_destroy}, {"topk", js_topk}, {"gatherNd", js_gather_nd},
+      {"scatterNd", js_scatter_nd}, {"cropAndResize", js_crop_and_resize},
+      {"resizeBilinearBackprop", js_resize_bilinear_backprop},
+      {"resizeNearestBackprop", js_resize_nearest_backprop}};
   for (size_t i = 0; i < sizeof fns / sizeof fns[0]; i++) {
     napi_value f;
     if (napi_create_function(env, fns[i].name, NAPI_AUTO_LENGTH, fns[i].fn, NULL, &f) != napi_ok ||

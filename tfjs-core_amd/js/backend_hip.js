@@ -14,6 +14,7 @@ const {DataStorage, KernelBackend} = require('./backend');
 const {Tensor} = require('./tensor');
 const {ENGINE} = require('./engine');
 const {ENV} = require('./environment');
+const {stridedSliceInfo} = require('./slice_util');
 
 const DTYPE = {float32: 0, int32: 1, bool: 2, uint8q: 3};
 const ACT = {linear: 0, relu: 1, prelu: 2, relu6: 3};
@@ -660,6 +661,239 @@ class MathBackendHIP extends KernelBackend {
     return out;
   }
 
+  // ---- index-driven kernels (backend.ts:193, 499-503, 591-598, 612-627) ----
+  gatherND(x, indices) {
+    const sliceRank = indices.shape[indices.rank - 1];
+    const numSlices = util.sizeFromShape(indices.shape.slice(0, -1));
+    const outShape = indices.shape.slice(0, -1).concat(x.shape.slice(sliceRank));
+    const out = this.outLikeStorage(outShape, x);
+    const idx = this.storageCode(indices) === DTYPE.int32 ? indices : this.int(indices);
+    this.napi.gatherNd(this.ctx, this.h(x), this.h(idx), this.h(out), Int32Array.from(x.shape),
+                       numSlices, sliceRank);
+    return out;
+  }
+  // flags of tfhip_scatter_nd: 1 sum duplicates, 2 skip indices outside the result, 4 round
+  // float32 sums once
+  scatterImpl(indices, updates, shape, defaultValue, flags, sliceRank) {
+    if (sliceRank == null) sliceRank = indices.rank > 1 ? indices.shape[indices.rank - 1] : 1;
+    const numUpdates = sliceRank ? indices.size / sliceRank : 0;
+    const dtype = updates.dtype === 'bool' ? 'int32' : updates.dtype;
+    const out = this.out(shape.slice(), dtype);
+    const idx = this.materialized(indices.dtype === 'int32' ? indices : this.int(indices));
+    const upd = this.materialized(this.cast(updates, dtype));
+    this.napi.scatterNd(this.ctx, this.h(idx), this.h(upd), this.h(out), Int32Array.from(shape),
+                        numUpdates, sliceRank, defaultValue, flags);
+    return out;
+  }
+  scatterND(indices, updates, shape) { return this.scatterImpl(indices, updates, shape, 0, 1); }
+  // defaultValue is a scalar tensor (backend.ts:624-627); reading it waits for the device
+  sparseToDense(sparseIndices, sparseValues, outputShape, defaultValue) {
+    const value = typeof defaultValue === 'number' ? defaultValue : this.readSync(defaultValue.dataId)[0];
+    return this.scatterImpl(sparseIndices, sparseValues, outputShape, value, 0);
+  }
+  // backend_cpu.ts:635-660: segments along axis 0; ids outside [0, numSegments) add nothing
+  unsortedSegmentSum(x, segmentIds, numSegments) {
+    const $x = x.dtype === 'bool' ? this.cast(x, 'float32') : x;
+    return this.scatterImpl(segmentIds, $x, [numSegments].concat($x.shape.slice(1)), 0, 1 | 2 | 4, 1);
+  }
+  resizeBilinearBackprop(dy, x, alignCorners) {
+    const [batch, h, w, c] = x.shape;
+    const dx = this.out([batch, h, w, c], 'float32');
+    this.napi.resizeBilinearBackprop(this.ctx, this.h(this.materialized(dy)), this.h(dx), batch, h, w,
+                                     c, dy.shape[1], dy.shape[2], alignCorners ? 1 : 0);
+    return dx;
+  }
+  resizeNearestNeighborBackprop(dy, x, alignCorners) {
+    const [batch, h, w, c] = x.shape;
+    const dx = this.out([batch, h, w, c], 'float32');
+    this.napi.resizeNearestBackprop(this.ctx, this.h(this.materialized(dy)), this.h(dx), batch, h, w,
+                                    c, dy.shape[1], dy.shape[2], alignCorners ? 1 : 0);
+    return dx;
+  }
+  cropAndResize(images, boxes, boxIndex, cropSize, method, extrapolationValue) {
+    const [batch, h, w, c] = images.shape;
+    const numBoxes = boxes.shape[0];
+    const out = this.out([numBoxes, cropSize[0], cropSize[1], c], 'float32');
+    const idx = this.materialized(boxIndex.dtype === 'int32' ? boxIndex : this.int(boxIndex));
+    this.napi.cropAndResize(this.ctx, this.h(images), this.h(this.materialized(boxes)), this.h(idx),
+                            this.h(out), batch, h, w, c, numBoxes, cropSize[0], cropSize[1],
+                            method === 'bilinear' ? 0 : 1, extrapolationValue);
+    return out;
+  }
+
+  // ---- composites over the kernels above, as backend_cpu.ts builds them from its own ops ----
+  // backend_cpu.ts:454-468: the tensors are added one after the other, starting from the first
+  addN(tensors) {
+    if (tensors.length === 1) {
+      const out = this.outLikeStorage(tensors[0].shape.slice(), tensors[0]);
+      this.napi.copy(this.ctx, this.h(tensors[0]), this.h(out));
+      return out;
+    }
+    return tensors.slice(1).reduce((acc, t) => this.add(acc, t), tensors[0]);
+  }
+  // backend_cpu.ts:315-344
+  stridedSlice(x, begin, end, strides, beginMask, endMask, ellipsisMask, newAxisMask, shrinkAxisMask) {
+    const [start, size, shrink, full] = stridedSliceInfo(
+        x.shape, begin, end, strides, beginMask | 0, endMask | 0, ellipsisMask | 0, newAxisMask | 0,
+        shrinkAxisMask | 0);
+    const shape = size.filter((v, i) => shrink.indexOf(i) === -1);
+    if (shape.some(d => d === 0)) return this.out(shape, x.dtype);
+    return this.reshape(this.stridedSliceBox(x, start, size, full), shape);
+  }
+  // backend_cpu.ts:356-375
+  unstack(x, axis) {
+    const outShape = x.shape.filter((d, i) => i !== axis);
+    const res = [];
+    for (let i = 0; i < x.shape[axis]; i++) {
+      const begin = new Array(x.rank).fill(0), size = x.shape.slice();
+      begin[axis] = i;
+      size[axis] = 1;
+      res.push(this.reshape(this.slice(x, begin, size), outShape));
+    }
+    return res;
+  }
+  // backends/split_shared.ts:22-32
+  split(x, sizeSplits, axis) {
+    const begin = new Array(x.rank).fill(0), size = x.shape.slice();
+    return sizeSplits.map(s => {
+      size[axis] = s;
+      const piece = this.slice(x, begin.slice(), size.slice());
+      begin[axis] += s;
+      return piece;
+    });
+  }
+  // backend_cpu.ts:2225-2245: [B, s1..sM, rest] -> [b1..bM, B / prod, s1..sM, rest] ->
+  // interleave (si, bi) -> crop
+  batchToSpaceND(x, blockShape, crops) {
+    const M = blockShape.length;
+    const prod = blockShape.reduce((a, b) => a * b);
+    const rest = x.shape.slice(1 + M);
+    const split = blockShape.concat([x.shape[0] / prod], x.shape.slice(1));
+    const perm = [M];
+    for (let i = 0; i < M; i++) perm.push(M + 1 + i, i);
+    for (let i = 0; i < rest.length; i++) perm.push(2 * M + 1 + i);
+    const merged = [x.shape[0] / prod].concat(blockShape.map((b, i) => b * x.shape[1 + i]), rest);
+    const begin = [0].concat(crops.map(c => c[0]), rest.map(() => 0));
+    const size = [merged[0]].concat(crops.map((c, i) => merged[1 + i] - c[0] - c[1]), rest);
+    return this.slice(this.reshape(this.transpose(this.reshape(x, split), perm), merged), begin, size);
+  }
+  // backend_cpu.ts:2247-2271: pad, split every spatial dimension into (si / bi, bi), move the
+  // bi in front of the batch, merge
+  spaceToBatchND(x, blockShape, paddings) {
+    const M = blockShape.length;
+    const prod = blockShape.reduce((a, b) => a * b);
+    const rest = x.shape.slice(1 + M);
+    const padded = this.pad(x, [[0, 0]].concat(paddings, rest.map(() => [0, 0])), 0);
+    const split = [padded.shape[0]];
+    for (let i = 0; i < M; i++) split.push(padded.shape[1 + i] / blockShape[i], blockShape[i]);
+    const perm = [];
+    for (let i = 0; i < M; i++) perm.push(2 + 2 * i);
+    perm.push(0);
+    for (let i = 0; i < M; i++) perm.push(1 + 2 * i);
+    for (let i = 0; i < rest.length; i++) perm.push(2 * M + 1 + i);
+    const merged = [padded.shape[0] * prod].concat(blockShape.map((b, i) => padded.shape[1 + i] / b), rest);
+    return this.reshape(this.transpose(this.reshape(padded, split.concat(rest)), perm), merged);
+  }
+  // backend_cpu.ts:3469-3512 (NHWC): out[b, h, w, d] =
+  // x[b, h / bs, w / bs, ((h % bs) * bs + w % bs) * outDepth + d], a 6-d transpose
+  depthToSpace(x, blockSize, dataFormat) {
+    util.assert(dataFormat === 'NHWC',
+                () => `Only NHWC dataFormat supported on CPU for depthToSpace. Got ${dataFormat}`);
+    const [b, h, w, d] = x.shape;
+    const outD = d / (blockSize * blockSize);
+    return this.reshape(
+        this.transpose(this.reshape(x, [b, h, w, blockSize, blockSize, outD]), [0, 1, 3, 2, 4, 5]),
+        [b, h * blockSize, w * blockSize, outD]);
+  }
+  // backend_cpu.ts:346-354: the flattened x on the diagonal of a [size, size] matrix
+  diag(x) {
+    const n = x.size;
+    const out = this.fill([n, n], 0, x.dtype);
+    if (n > 0) this.boxCopy(this.materialized(x), out, [n], [1], 0, [n + 1], 0);
+    return out;
+  }
+
+  // ---- host-side routines: every backend of the reference runs these on values read back ----
+  fromHost(values, shape, dtype) { return Tensor.make(shape, {values}, dtype, this); }
+  // backends/backend_util.ts:78-88: a running float32 sum of the double step
+  linspace(start, stop, num) {
+    const step = (stop - start) / (num - 1);
+    const values = new Float32Array(num);
+    values[0] = start;
+    for (let i = 1; i < num; i++) values[i] = values[i - 1] + step;
+    return this.fromHost(values, [num], 'float32');
+  }
+  // backends/where_impl.ts:25-43: coordinates of the true elements, row-major
+  where(condition) {
+    const vals = this.readSync(condition.dataId);
+    const rank = condition.rank, strides = util.computeStrides(condition.shape).concat([1]);
+    const hits = [];
+    for (let i = 0; i < vals.length; i++) if (vals[i]) hits.push(i);
+    const out = new Int32Array(hits.length * rank);
+    hits.forEach((flat, i) => {
+      let rem = flat;
+      for (let d = 0; d < rank; d++) {
+        out[i * rank + d] = Math.floor(rem / strides[d]);
+        rem -= out[i * rank + d] * strides[d];
+      }
+    });
+    return this.fromHost(out, [hits.length, rank], 'int32');
+  }
+  // backends/non_max_suppression_impl.ts:25-102: candidates above the score threshold in
+  // descending score (equal scores in index order), each kept unless it overlaps an already
+  // selected box by iouThreshold or more
+  nonMaxSuppression(boxes, scores, maxOutputSize, iouThreshold, scoreThreshold) {
+    const b = this.readSync(boxes.dataId), s = this.readSync(scores.dataId);
+    const iou = (i, j) => {
+      const yminI = Math.min(b[4 * i], b[4 * i + 2]), ymaxI = Math.max(b[4 * i], b[4 * i + 2]);
+      const xminI = Math.min(b[4 * i + 1], b[4 * i + 3]), xmaxI = Math.max(b[4 * i + 1], b[4 * i + 3]);
+      const yminJ = Math.min(b[4 * j], b[4 * j + 2]), ymaxJ = Math.max(b[4 * j], b[4 * j + 2]);
+      const xminJ = Math.min(b[4 * j + 1], b[4 * j + 3]), xmaxJ = Math.max(b[4 * j + 1], b[4 * j + 3]);
+      const areaI = (ymaxI - yminI) * (xmaxI - xminI), areaJ = (ymaxJ - yminJ) * (xmaxJ - xminJ);
+      if (areaI <= 0 || areaJ <= 0) return 0;
+      const inter = Math.max(Math.min(ymaxI, ymaxJ) - Math.max(yminI, yminJ), 0) *
+          Math.max(Math.min(xmaxI, xmaxJ) - Math.max(xminI, xminJ), 0);
+      return inter / (areaI + areaJ - inter);
+    };
+    const order = Array.from(s, (score, i) => i).filter(i => s[i] > scoreThreshold)
+                      .sort((i, j) => (s[j] - s[i]) || (i - j));
+    const selected = [];
+    for (let k = 0; k < order.length && selected.length < maxOutputSize; k++) {
+      let keep = true;
+      for (let j = selected.length - 1; j >= 0 && keep; j--) {
+        if (iou(order[k], selected[j]) >= iouThreshold) keep = false;
+      }
+      if (keep) selected.push(order[k]);
+    }
+    return this.fromHost(Int32Array.from(selected), [selected.length], 'int32');
+  }
+  // backend_cpu.ts:3284-3323: inverse-CDF sampling of each row of `probabilities` on the host,
+  // with the Alea generator (Baagoe) that the reference takes from the seedrandom package.
+  // parity unpinned: the reference holds no sample vectors, only distribution checks.
+  multinomial(probabilities, normalized, numSamples, seed) {
+    const probs = normalized ? probabilities : this.softmax(probabilities, probabilities.rank - 1);
+    const [batch, numEvents] = probs.shape;
+    const p = this.readSync(probs.dataId);
+    const out = new Int32Array(batch * numSamples);
+    for (let b = 0; b < batch; b++) {
+      const cdf = new Float32Array(numEvents - 1);
+      if (numEvents > 1) cdf[0] = p[b * numEvents];
+      for (let e = 1; e < cdf.length; e++) cdf[e] = cdf[e - 1] + p[b * numEvents + e];
+      const random = alea(String(seed));
+      for (let n = 0; n < numSamples; n++) {
+        const r = random();
+        out[b * numSamples + n] = cdf.length;
+        for (let e = 0; e < cdf.length; e++) {
+          if (r < cdf[e]) {
+            out[b * numSamples + n] = e;
+            break;
+          }
+        }
+      }
+    }
+    return this.fromHost(out, [batch, numSamples], 'int32');
+  }
+
   transpose(x, perm) {
     const out = this.outLikeStorage(perm.map(p => x.shape[p]), x);
     this.napi.transpose(this.ctx, this.h(x), Int32Array.from(x.shape), Int32Array.from(perm),
@@ -668,4 +902,37 @@ class MathBackendHIP extends KernelBackend {
   }
 }
 
-module.exports = {MathBackendHIP, loadAddon};
+// Alea, Johannes Baagoe's generator, in the variant the seedrandom package (2.4.3, a dependency
+// of the reference: package.json) ships as seedrandom.alea; restated from its published
+// description.  Returns a function giving doubles in [0, 1).
+function alea(seed) {
+  let n = 0xefc8249d;
+  const mash = data => {
+    for (let i = 0; i < data.length; i++) {
+      n += data.charCodeAt(i);
+      let h = 0.02519603282416938 * n;
+      n = h >>> 0;
+      h -= n;
+      h *= n;
+      n = h >>> 0;
+      h -= n;
+      n += h * 0x100000000;  // 2^32
+    }
+    return (n >>> 0) * 2.3283064365386963e-10;  // 2^-32
+  };
+  let s0 = mash(' '), s1 = mash(' '), s2 = mash(' '), c = 1;
+  s0 -= mash(seed);
+  if (s0 < 0) s0 += 1;
+  s1 -= mash(seed);
+  if (s1 < 0) s1 += 1;
+  s2 -= mash(seed);
+  if (s2 < 0) s2 += 1;
+  return () => {
+    const t = 2091639 * s0 + c * 2.3283064365386963e-10;
+    s0 = s1;
+    s1 = s2;
+    return s2 = t - (c = t | 0);
+  };
+}
+
+module.exports = {MathBackendHIP, loadAddon, alea};

@@ -618,8 +618,14 @@ const addN = op('addN', tensors => {
     if (t.dtype !== $tensors[0].dtype) throw new Error('All tensors passed to tf.addN() must have the same dtype');
     if (!util.arraysEqual(t.shape, $tensors[0].shape)) throw new Error('All tensors passed to tf.addN() must have the same shape');
   });
-  if ($tensors.length === 1) return clone($tensors[0]);
-  return ENGINE.tidy(() => $tensors.slice(1).reduce((acc, t) => add(acc, t), $tensors[0]));
+  const inputs = {};
+  $tensors.forEach((t, i) => inputs[i] = t);
+  const grads = dy => {
+    const ders = {};
+    $tensors.forEach((t, i) => ders[i] = () => clone(dy));
+    return ders;
+  };
+  return ENGINE.runKernel(backend => backend.addN($tensors), inputs, grads);
 });
 
 const prelu = op('prelu', (x, alpha) => {
@@ -910,57 +916,13 @@ const slice = op('slice', (x, begin, size) => {
   return ENGINE.runKernel(backend => backend.slice($x, begin_, size_), {$x});
 });
 
-const clampInt = (lo, v, hi) => Math.max(lo, Math.min(v, hi));
-
-// getStridedSlicedInfo (ops/slice_util.ts:48-188): [begin index, size, shrunk axes, strides]
-function stridedSliceInfo(shape, begin, end, strides, beginMask, endMask, ellipsisMask,
-                          newAxisMask, shrinkAxisMask) {
-  if (ellipsisMask) throw new Error('ellipsis mask is not yet supported');
-  if (newAxisMask) throw new Error('new axis mask is not yet supported');
-  const full = shape.map((d, i) => strides[i] || 1);
-  const startIndex = [], endIndex = [], shrinkAxis = [];
-  for (let i = 0; i < shape.length; i++) {
-    const n = shape[i], stride = full[i];
-    let start = begin[i];
-    if (beginMask & (1 << i) || start == null) {
-      start = stride > 0 ? Number.MIN_SAFE_INTEGER : Number.MAX_SAFE_INTEGER;
-    }
-    if (start < 0) start += n;
-    start = clampInt(0, start, n - 1);
-    let stop = end[i];
-    if (endMask & (1 << i) || stop == null) {
-      stop = stride > 0 ? Number.MAX_SAFE_INTEGER : Number.MIN_SAFE_INTEGER;
-    }
-    if (stop < 0) stop += n;
-    stop = stride > 0 ? clampInt(0, stop, n) : clampInt(-1, stop, n - 1);
-    if (shrinkAxisMask & (1 << i)) {
-      stop = start + 1;
-      shrinkAxis.push(i);
-    }
-    startIndex.push(start);
-    endIndex.push(stop);
-  }
-  const size = shape.map((d, i) => {
-    let count = 0;
-    for (let s = startIndex[i]; !(full[i] > 0 ? s >= endIndex[i] : s <= endIndex[i]); s += full[i]) {
-      count++;
-    }
-    return count;
-  });
-  return [startIndex, size, shrinkAxis, full];
-}
-
 const stridedSlice = op('stridedSlice', (x, begin, end, strides, beginMask, endMask, ellipsisMask,
                                          newAxisMask, shrinkAxisMask) => {
   const $x = convertToTensor(x, 'x', 'stridedSlice');
   if (strides == null) strides = new Array(begin.length).fill(1);
-  const [start, size, shrink, full] = stridedSliceInfo(
-      $x.shape, begin, end, strides, beginMask | 0, endMask | 0, ellipsisMask | 0, newAxisMask | 0,
-      shrinkAxisMask | 0);
-  const shape = size.filter((v, i) => shrink.indexOf(i) === -1);
-  if (shape.some(d => d === 0)) return tensor([], shape, $x.dtype);
-  const res = ENGINE.runKernel(backend => backend.stridedSliceBox($x, start, size, full), {$x});
-  return reshape(res, shape);
+  return ENGINE.runKernel(
+      backend => backend.stridedSlice($x, begin, end, strides, beginMask | 0, endMask | 0, ellipsisMask | 0,
+                                      newAxisMask | 0, shrinkAxisMask | 0), {$x});
 });
 
 const reverse = op('reverse', (x, axis) => {
@@ -1096,7 +1058,14 @@ const resizeBilinear = op('resizeBilinear', (images, size, alignCorners) => {
               () => `Error in resizeBilinear: new shape must 2D, but got ${size}.`);
   const batchImages = $images.rank === 4 ? $images : reshape($images, [1].concat($images.shape));
   const res = ENGINE.runKernel(
-      backend => backend.resizeBilinear(batchImages, size[0], size[1], !!alignCorners), {batchImages});
+      (backend, save) => {
+        save([batchImages]);
+        return backend.resizeBilinear(batchImages, size[0], size[1], !!alignCorners);
+      },
+      {batchImages}, (dy, saved) => ({
+        batchImages: () => ENGINE.runKernel(
+            backend => backend.resizeBilinearBackprop(dy, saved[0], !!alignCorners), {})
+      }));
   return $images.rank === 4 ? res : reshape(res, res.shape.slice(1));
 });
 
@@ -1112,7 +1081,14 @@ const resizeNearestNeighbor = op('resizeNearestNeighbor', (images, size, alignCo
               () => '`images` must have `int32` or `float32` as dtype');
   const batchImages = $images.rank === 4 ? $images : reshape($images, [1].concat($images.shape));
   const res = ENGINE.runKernel(
-      backend => backend.resizeNearestNeighbor(batchImages, size[0], size[1], !!alignCorners), {batchImages});
+      (backend, save) => {
+        save([batchImages]);
+        return backend.resizeNearestNeighbor(batchImages, size[0], size[1], !!alignCorners);
+      },
+      {batchImages}, (dy, saved) => ({
+        batchImages: () => ENGINE.runKernel(
+            backend => backend.resizeNearestNeighborBackprop(dy, saved[0], !!alignCorners), {})
+      }));
   return $images.rank === 4 ? res : reshape(res, res.shape.slice(1));
 });
 
@@ -1207,16 +1183,7 @@ const unstack = op('unstack', (x, axis) => {
   util.assert(axis >= -$x.shape.length && axis < $x.shape.length,
               () => `Axis = ${axis} is not in [-${$x.shape.length}, ${$x.shape.length})`);
   if (axis < 0) axis += $x.shape.length;
-  const outputShape = $x.shape.filter((d, i) => i !== axis);
-  const res = [];
-  for (let i = 0; i < $x.shape[axis]; i++) {
-    const begin = new Array($x.rank).fill(0);
-    const size = $x.shape.slice();
-    begin[axis] = i;
-    size[axis] = 1;
-    res.push(reshape(slice($x, begin, size), outputShape));
-  }
-  return res;
+  return ENGINE.runKernel(backend => backend.unstack($x, axis), {$x}, dy => ({$x: () => stack(dy, axis)}));
 });
 
 // ops/concat_split.ts:182-218
@@ -1233,14 +1200,8 @@ const split = op('split', (x, numOrSizeSplits, axis) => {
                 () => 'The sum of sizes must match the size of the axis dimension.');
     splitSizes = numOrSizeSplits;
   }
-  const begin = new Array($x.rank).fill(0);
-  const size = $x.shape.slice();
-  return splitSizes.map(s => {
-    size[axis] = s;
-    const piece = slice($x, begin.slice(), size.slice());
-    begin[axis] += s;
-    return piece;
-  });
+  return ENGINE.runKernel(backend => backend.split($x, splitSizes, axis), {$x},
+                          dy => ({$x: () => concat(dy, axis)}));
 });
 
 const opHandler = {
@@ -1304,8 +1265,7 @@ const localResponseNormalization = op('localResponseNormalization', (x, depthRad
   return lower(res, reshapedTo4D);
 });
 
-// array_ops.ts:708-741 / backend_cpu.ts:2225-2245 over this host's reshape, transpose and slice:
-// [B, s1..sM, rest] -> [b1..bM, B/prod, s1..sM, rest] -> interleave (si, bi) -> crop.
+// array_ops.ts:708-741
 const batchToSpaceND = op('batchToSpaceND', (x, blockShape, crops) => {
   const $x = convertToTensor(x, 'x', 'batchToSpaceND');
   const M = blockShape.length;
@@ -1317,19 +1277,11 @@ const batchToSpaceND = op('batchToSpaceND', (x, blockShape, crops) => {
   util.assert($x.shape[0] % prod === 0,
               () => `input tensor batch is ${$x.shape[0]} but is not divisible by the product of ` +
                   `the elements of blockShape ${blockShape.join(' * ')} === ${prod}`);
-  const rest = $x.shape.slice(1 + M);
-  const split = blockShape.concat([$x.shape[0] / prod], $x.shape.slice(1));
-  const perm = [M];
-  for (let i = 0; i < M; i++) perm.push(M + 1 + i, i);
-  for (let i = 0; i < rest.length; i++) perm.push(2 * M + 1 + i);
-  const merged = [$x.shape[0] / prod].concat(blockShape.map((b, i) => b * $x.shape[1 + i]), rest);
-  const begin = [0].concat(crops.map(c => c[0]), rest.map(() => 0));
-  const size = [merged[0]].concat(crops.map((c, i) => merged[1 + i] - c[0] - c[1]), rest);
-  return ENGINE.tidy(() => slice(reshape(transpose(reshape($x, split), perm), merged), begin, size));
+  return ENGINE.runKernel(backend => backend.batchToSpaceND($x, blockShape, crops), {$x},
+                          dy => ({$x: () => spaceToBatchND(dy, blockShape, crops)}));
 });
 
-// array_ops.ts:786-824 / backend_cpu.ts:2247-2271: pad, split every spatial dim into
-// (si / bi, bi), move the bi in front of the batch, merge.
+// array_ops.ts:786-824
 const spaceToBatchND = op('spaceToBatchND', (x, blockShape, paddings) => {
   const $x = convertToTensor(x, 'x', 'spaceToBatchND');
   const M = blockShape.length;
@@ -1341,25 +1293,11 @@ const spaceToBatchND = op('spaceToBatchND', (x, blockShape, paddings) => {
       ok && ((d + paddings[i - 1][0] + paddings[i - 1][1]) % blockShape[i - 1] === 0) : ok, true),
               () => `input spatial dimensions ${$x.shape.slice(1)} with paddings ${paddings.toString()} ` +
                   `must be divisible by blockShapes ${blockShape.toString()}`);
-  const prod = blockShape.reduce((a, b) => a * b);
-  const rest = $x.shape.slice(1 + M);
-  const full = [[0, 0]].concat(paddings, rest.map(() => [0, 0]));
-  return ENGINE.tidy(() => {
-    const padded = pad($x, full);
-    const split = [padded.shape[0]];
-    for (let i = 0; i < M; i++) split.push(padded.shape[1 + i] / blockShape[i], blockShape[i]);
-    const perm = [];
-    for (let i = 0; i < M; i++) perm.push(2 + 2 * i);
-    perm.push(0);
-    for (let i = 0; i < M; i++) perm.push(1 + 2 * i);
-    for (let i = 0; i < rest.length; i++) perm.push(2 * M + 1 + i);
-    const merged = [padded.shape[0] * prod].concat(blockShape.map((b, i) => padded.shape[1 + i] / b), rest);
-    return reshape(transpose(reshape(padded, split.concat(rest)), perm), merged);
-  });
+  return ENGINE.runKernel(backend => backend.spaceToBatchND($x, blockShape, paddings), {$x},
+                          dy => ({$x: () => batchToSpaceND(dy, blockShape, paddings)}));
 });
 
-// array_ops.ts:960-1001 / backend_cpu.ts:3469-3512 (NHWC): out[b, h, w, d] =
-// x[b, h / bs, w / bs, ((h % bs) * bs + w % bs) * outDepth + d], i.e. a 6-d transpose.
+// array_ops.ts:960-1001
 const depthToSpace = op('depthToSpace', (x, blockSize, dataFormat) => {
   const $x = convertToTensor(x, 'x', 'depthToSpace');
   if (dataFormat == null) dataFormat = 'NHWC';
@@ -1370,10 +1308,213 @@ const depthToSpace = op('depthToSpace', (x, blockSize, dataFormat) => {
   util.assert(d % (blockSize * blockSize) === 0,
               () => `Dimension size must be evenly divisible by ${blockSize * blockSize} but is ${d} ` +
                   `for depthToSpace with input shape ${$x.shape}`);
-  const outD = d / (blockSize * blockSize);
-  return ENGINE.tidy(() => reshape(
-      transpose(reshape($x, [b, h, w, blockSize, blockSize, outD]), [0, 1, 3, 2, 4, 5]),
-      [b, h * blockSize, w * blockSize, outD]));
+  return ENGINE.runKernel(backend => backend.depthToSpace($x, blockSize, dataFormat), {$x});
+});
+
+// ---- index-driven ops and image utilities --------------------------------------------------
+// ops/gather_nd.ts:56-63 with the checks of ops/gather_nd_util.ts:29-55
+const gatherND = op('gatherND', (x, indices) => {
+  const $x = convertToTensor(x, 'x', 'gatherND');
+  const $indices = convertToTensor(indices, 'indices', 'gatherND', 'int32');
+  if ($x.rank < 1) {
+    throw new Error(`tf.gatherND() expects the input to be rank 1 or higher, but the rank was ${$x.rank}.`);
+  }
+  if ($indices.rank < 1) {
+    throw new Error(`tf.gatherND() expects the indices to be rank 1 or higher, but the rank was ${$indices.rank}.`);
+  }
+  if ($indices.dtype !== 'int32') {
+    throw new Error(`tf.gatherND() expects the indices to be int32 type, but the dtype was ${$indices.dtype}.`);
+  }
+  if ($indices.shape[$indices.rank - 1] > $x.rank) {
+    throw new Error('index innermost dimension length must be <= tensor rank; saw: ' +
+                    `${$indices.shape[$indices.rank - 1]} vs. ${$x.rank}`);
+  }
+  if ($x.size === 0) {
+    throw new Error(`Requested more than 0 entries, but input is empty. Input shape: ${$x.shape}.`);
+  }
+  return ENGINE.runKernel(backend => backend.gatherND($x, $indices), {$x, $indices});
+});
+
+// ops/scatter_nd_util.ts:28-125
+function validateScatter(updates, indices, shape) {
+  if (indices.rank < 1) {
+    throw new Error(`tf.scatterND() expects the indices to be rank 1 or higher, but the rank was ${indices.rank}.`);
+  }
+  if (updates.rank < 1) {
+    throw new Error(`tf.scatterND() expects the updates to be rank 1 or higher, but the rank was ${updates.rank}.`);
+  }
+  if (indices.dtype !== 'int32') {
+    throw new Error(`The dtype of 'indices' should be int32, but got dtype: ${indices.dtype}`);
+  }
+  if (shape.length < 1) {
+    throw new Error(`Output rank must be greater or equal to 1, but got shape: ${shape}`);
+  }
+  const sliceDim = indices.rank > 1 ? indices.shape[indices.rank - 1] : 1;
+  const batchDim = indices.rank > 1 ? indices.rank - 1 : 1;
+  const shapeError = 'Must have updates.shape = indices.shape[:batchDim] + ' +
+      `shape[sliceDim:], got updates.shape: ${updates.shape}, indices.shape: ${indices.shape}, ` +
+      `shape: ${shape}, sliceDim: ${sliceDim}, and batchDim: ${batchDim}.`;
+  if (updates.rank < batchDim) throw new Error(shapeError + ` update.rank < ${batchDim}. `);
+  if (shape.length < sliceDim + (updates.rank - batchDim)) {
+    throw new Error(shapeError + ` Output shape length < ${sliceDim + (updates.rank - batchDim)}`);
+  }
+  if (updates.rank !== batchDim + shape.length - sliceDim) {
+    throw new Error(shapeError + ` update.rank != ${batchDim + shape.length - sliceDim}`);
+  }
+  for (let d = 0; d < batchDim; ++d) {
+    if (updates.shape[d] !== indices.shape[d]) {
+      throw new Error(shapeError + ` updates.shape[${d}] (${updates.shape[d]}) != indices.shape[${d}] (${indices.shape[d]}).`);
+    }
+  }
+  for (let d = 0; d < updates.rank - batchDim; ++d) {
+    if (updates.shape[d + batchDim] !== shape[d + sliceDim]) {
+      throw new Error(shapeError + ` updates.shape[${d + batchDim}] (${updates.shape[d + batchDim]}) != ` +
+                      `shape[${d + batchDim}] (${shape[d + batchDim]})`);
+    }
+  }
+}
+
+// ops/scatter_nd.ts:44-53
+const scatterND = op('scatterND', (indices, updates, shape) => {
+  const $indices = convertToTensor(indices, 'indices', 'scatterND', 'int32');
+  const $updates = convertToTensor(updates, 'updates', 'scatterND');
+  validateScatter($updates, $indices, shape);
+  return ENGINE.runKernel(backend => backend.scatterND($indices, $updates, shape), {$indices, $updates});
+});
+
+// ops/sparse_to_dense.ts:61-79 with the checks of ops/sparse_to_dense_util.ts:28-64
+const sparseToDense = op('sparseToDense', (sparseIndices, sparseValues, outputShape, defaultValue) => {
+  const $sparseIndices = convertToTensor(sparseIndices, 'sparseIndices', 'sparseToDense', 'int32');
+  const $sparseValues = convertToTensor(sparseValues, 'sparseValues', 'sparseToDense');
+  const $defaultValue = convertToTensor(defaultValue == null ? 0 : defaultValue, 'defaultValue', 'sparseToDense',
+                                        $sparseValues.dtype);
+  if ($sparseIndices.dtype !== 'int32') {
+    throw new Error(`tf.sparseToDense() expects the indices to be int32 type, but the dtype was ${$sparseIndices.dtype}.`);
+  }
+  if ($sparseIndices.rank > 2) {
+    throw new Error(`sparseIndices should be a scalar, vector, or matrix, but got shape ${$sparseIndices.shape}.`);
+  }
+  const numElems = $sparseIndices.rank > 0 ? $sparseIndices.shape[0] : 1;
+  const numDims = $sparseIndices.rank > 1 ? $sparseIndices.shape[1] : 1;
+  if (outputShape.length !== numDims) {
+    throw new Error(`outputShape has incorrect number of elements:, ${outputShape.length}, should be: ${numDims}.`);
+  }
+  const numValues = $sparseValues.size;
+  if (!($sparseValues.rank === 0 || $sparseValues.rank === 1 && numValues === numElems)) {
+    throw new Error(`sparseValues has incorrect shape ${$sparseValues.shape}, should be [] or [${numElems}]`);
+  }
+  if ($sparseValues.dtype !== $defaultValue.dtype) {
+    throw new Error('sparseValues.dtype must match defaultValues.dtype');
+  }
+  return ENGINE.runKernel(
+      backend => backend.sparseToDense($sparseIndices, $sparseValues, outputShape, $defaultValue),
+      {$sparseIndices, $sparseValues, $defaultValue});
+});
+
+// ops/segment_ops.ts:43-69, 156-170: the gradient gathers dy by segment id, zero for negative ids
+const unsortedSegmentSum = op('unsortedSegmentSum', (x, segmentIds, numSegments) => {
+  const $x = convertToTensor(x, 'x', 'unsortedSegmentSum');
+  const $segmentIds = convertToTensor(segmentIds, 'segmentIds', 'unsortedSegmentSum', 'int32');
+  util.assert(util.isInt(numSegments), () => 'numSegments must be of dtype int');
+  return ENGINE.runKernel((backend, save) => {
+    save([$segmentIds]);
+    return backend.unsortedSegmentSum($x, $segmentIds, numSegments);
+  }, {$x}, (dy, saved) => ({
+    $x: () => {
+      const ids = saved[0];
+      const gathered = gather(dy, maximum(ids, zerosLike(ids)));
+      let isPositive = greaterEqual(ids, scalar(0, 'int32'));
+      for (let i = 0; i < gathered.rank - 1; ++i) isPositive = expandDims(isPositive, i + 1);
+      isPositive = logicalAnd(isPositive, ones(gathered.shape, 'bool'));
+      return where(isPositive, gathered, zerosLike(gathered));
+    }
+  }));
+});
+
+// ops/image_ops.ts:268-316
+const cropAndResize = op('cropAndResize', (image, boxes, boxInd, cropSize, method, extrapolationValue) => {
+  const $image = convertToTensor(image, 'image', 'cropAndResize', 'float32');
+  const $boxes = convertToTensor(boxes, 'boxes', 'cropAndResize', 'float32');
+  const $boxInd = convertToTensor(boxInd, 'boxInd', 'cropAndResize', 'int32');
+  method = method || 'bilinear';
+  extrapolationValue = extrapolationValue || 0;
+  const numBoxes = $boxes.shape[0];
+  util.assert($image.rank === 4,
+              () => `Error in cropAndResize: image must be rank 4,but got rank ${$image.rank}.`);
+  util.assert($boxes.rank === 2 && $boxes.shape[1] === 4,
+              () => `Error in cropAndResize: boxes must be have size [${numBoxes},4] but had shape ${$boxes.shape}.`);
+  util.assert($boxInd.rank === 1 && $boxInd.shape[0] === numBoxes,
+              () => `Error in cropAndResize: boxInd must be have size [${numBoxes}] but had shape ${$boxes.shape}.`);
+  util.assert(cropSize.length === 2,
+              () => `Error in cropAndResize: cropSize must be of length 2, but got length ${cropSize.length}.`);
+  util.assert(cropSize[0] >= 1 && cropSize[1] >= 1, () => `cropSize must be atleast [1,1], but was ${cropSize}`);
+  util.assert(method === 'bilinear' || method === 'nearest',
+              () => `method must be bilinear or nearest, but was ${method}`);
+  return ENGINE.runKernel(
+      backend => backend.cropAndResize($image, $boxes, $boxInd, cropSize, method, extrapolationValue),
+      {$image, $boxes});
+});
+
+// ops/image_ops.ts:214-247
+function nonMaxSuppSanityCheck(boxes, scores, maxOutputSize, iouThreshold, scoreThreshold) {
+  if (iouThreshold == null) iouThreshold = 0.5;
+  if (scoreThreshold == null) scoreThreshold = Number.NEGATIVE_INFINITY;
+  const numBoxes = boxes.shape[0];
+  maxOutputSize = Math.min(maxOutputSize, numBoxes);
+  util.assert(0 <= iouThreshold && iouThreshold <= 1, () => `iouThreshold must be in [0, 1], but was '${iouThreshold}'`);
+  util.assert(boxes.rank === 2, () => `boxes must be a 2D tensor, but was of rank '${boxes.rank}'`);
+  util.assert(boxes.shape[1] === 4, () => `boxes must have 4 columns, but 2nd dimension was ${boxes.shape[1]}`);
+  util.assert(scores.rank === 1, () => 'scores must be a 1D tensor');
+  util.assert(scores.shape[0] === numBoxes,
+              () => `scores has incompatible shape with boxes. Expected ${numBoxes}, but was ${scores.shape[0]}`);
+  return {maxOutputSize, iouThreshold, scoreThreshold};
+}
+// ops/image_ops.ts:165-180
+const nonMaxSuppression = op('nonMaxSuppression', (boxes, scores, maxOutputSize, iouThreshold, scoreThreshold) => {
+  const $boxes = convertToTensor(boxes, 'boxes', 'nonMaxSuppression');
+  const $scores = convertToTensor(scores, 'scores', 'nonMaxSuppression');
+  const p = nonMaxSuppSanityCheck($boxes, $scores, maxOutputSize, iouThreshold, scoreThreshold);
+  return ENGINE.runKernel(
+      backend => backend.nonMaxSuppression($boxes, $scores, p.maxOutputSize, p.iouThreshold, p.scoreThreshold),
+      {$boxes});
+});
+// ops/image_ops.ts:183-212: the same selection behind a promise
+async function nonMaxSuppressionAsync(boxes, scores, maxOutputSize, iouThreshold, scoreThreshold) {
+  return nonMaxSuppression(boxes, scores, maxOutputSize, iouThreshold, scoreThreshold);
+}
+
+// ops/diag.ts:43-50
+const diag = op('diag', x => {
+  const $x = convertToTensor(x, 'x', 'diag');
+  const flat = reshape($x, [$x.size]);
+  const res = ENGINE.runKernel(backend => backend.diag(flat), {$x: flat});
+  return reshape(res, $x.shape.concat($x.shape));
+});
+
+// ops/tensor_ops.ts:483-488
+const linspace = op('linspace', (start, stop, num) => {
+  if (num <= 0) throw new Error('The number of values should be positive.');
+  return ENGINE.runKernel(backend => backend.linspace(start, stop, num));
+});
+
+// ops/logical_ops.ts:189-197: coordinates of the true elements
+async function whereAsync(condition) {
+  const $condition = convertToTensor(condition, 'condition', 'whereAsync', 'bool');
+  return ENGINE.runKernel(backend => backend.where($condition), {$condition});
+}
+
+// ops/array_ops.ts:284-305
+const multinomial = op('multinomial', (logits, numSamples, seed, normalized) => {
+  const $logits = convertToTensor(logits, 'logits', 'multinomial');
+  const numOutcomes = $logits.size, origRank = $logits.rank;
+  if (numOutcomes < 2) {
+    throw new Error(`Error in multinomial: you need at least 2 outcomes, but got ${numOutcomes}.`);
+  }
+  if (origRank > 2) throw new Error(`Rank of probabilities must be 1 or 2, but is ${origRank}`);
+  seed = seed || Math.random();
+  const logits2D = origRank === 1 ? reshape($logits, [1, -1]) : $logits;
+  const res = ENGINE.runKernel(backend => backend.multinomial(logits2D, !!normalized, numSamples, seed), {logits2D});
+  return origRank === 1 ? reshape(res, [res.size]) : res;
 });
 
 // ---- composites of reductions ------------------------------------------------------------
@@ -1457,7 +1598,9 @@ module.exports = {
   asinh, acosh, atanh, erf, elu, selu, softplus, step, leakyRelu, logSigmoid, isNaN: isNaN_, isInf,
   isFinite: isFinite_, pow, squaredDifference, mod, floorDiv, atan2, addN, prod, all, any,
   cumsum, localResponseNormalization, batchToSpaceND, spaceToBatchND, depthToSpace, topk,
-  moments, norm, logSoftmax
+  moments, norm, logSoftmax, gatherND, scatterND, sparseToDense, unsortedSegmentSum, diag, linspace,
+  whereAsync, multinomial,
+  image: {resizeBilinear, resizeNearestNeighbor, cropAndResize, nonMaxSuppression, nonMaxSuppressionAsync}
 };
 
 // Chaining methods (tensor.ts:700-1460 defines them one by one: x.square().sum() ...): every op

@@ -108,6 +108,29 @@ const OPS = {
   // x.square().sum() style chains over the methods attached to Tensor
   chainMore: i => i.x.abs().sqrt().add(i.x.square().mean(1, true)).maximum(i.x.neg()).slice([0, 1], [2, 3])
       .pad([[1, 0], [0, 1]]).expandDims(0).squeeze([0]).flatten(),
+  gatherND: i => tf.gatherND(i.x, i.indices),
+  scatterND: (i, a) => tf.scatterND(i.indices, i.updates, a.shape),
+  sparseToDense: (i, a) => tf.sparseToDense(i.indices, i.values, a.shape, a.defaultValue),
+  unsortedSegmentSum: (i, a) => tf.unsortedSegmentSum(i.x, i.ids, a.numSegments),
+  gradUnsortedSegmentSum: (i, a) => tf.grad(x => tf.unsortedSegmentSum(x, i.ids, a.numSegments))(i.x, i.dy),
+  cropAndResize: (i, a) => tf.image.cropAndResize(i.image, i.boxes, i.boxInd, a.cropSize, a.method, a.extrapolationValue),
+  nonMaxSuppression: (i, a) => tf.image.nonMaxSuppression(i.boxes, i.scores, a.maxOutputSize, a.iouThreshold, a.scoreThreshold),
+  diag: i => tf.diag(i.x),
+  linspace: (i, a) => tf.linspace(a.start, a.stop, a.num),
+  whereCoordinates: i => tf.backend().where(i.x),
+  gradResizeBilinear: (i, a) => tf.grad(x => tf.image.resizeBilinear(x, a.size, a.alignCorners))(i.x, i.dy),
+  gradResizeNearest: (i, a) => tf.grad(x => tf.image.resizeNearestNeighbor(x, a.size, a.alignCorners))(i.x, i.dy),
+  // relative frequency of each outcome over a.numSamples draws (the reference's own tests check
+  // multinomial this way, multinomial_test.ts)
+  multinomialFrequencies: (i, a) => {
+    const draws = tf.multinomial(i.probs, a.numSamples, a.seed, true);
+    const counts = tf.sum(tf.cast(tf.oneHot(tf.reshape(draws, [draws.size]), i.probs.size), 'float32'), 0);
+    return tf.div(counts, tf.scalar(a.numSamples));
+  },
+  stridedSlice: (i, a) => tf.stridedSlice(i.x, a.begin, a.end, a.strides, a.beginMask, a.endMask, 0, 0, a.shrinkAxisMask),
+  splitPiece: (i, a) => { const parts = tf.split(i.x, a.sizes, a.axis); const keep = parts[a.pick]; parts.forEach((t, k) => k !== a.pick && t.dispose()); return keep; },
+  gradSplit: (i, a) => tf.grad(x => { const parts = tf.split(x, a.sizes, a.axis); return tf.add(tf.sum(parts[0]), tf.mul(tf.sum(parts[1]), tf.scalar(2))); })(i.x),
+  gradAddN: i => tf.grads((p, q) => tf.addN([p, q, p]))([i.a, i.b], i.dy)[0],
   cumsum: (i, a) => tf.cumsum(i.x, a.axis, a.exclusive, a.reverse),
   gradCumsum: (i, a) => tf.grad(x => tf.cumsum(x, a.axis, a.exclusive, a.reverse))(i.x, i.dy),
   lrn: (i, a) => tf.localResponseNormalization(i.x, a.radius, a.bias, a.alpha, a.beta),

@@ -168,6 +168,11 @@ class MathBackendHIP(object):
     def _out(self, shape, dtype="float32"):
         return Tensor.make(shape, {}, dtype, self)
 
+    def _from_host(self, values):
+        """A tensor of this backend holding a host array (float32 or int32)."""
+        dtype = "int32" if values.dtype.kind in "iu" else "float32"
+        return Tensor.make(values.shape, {"values": values}, dtype, self)
+
     def _out_like_storage(self, shape, x):
         """Output of a pure data-movement kernel: same tensor dtype and same stored element
         type as x (they differ after a widening cast that aliased the buffer)."""
@@ -704,6 +709,135 @@ class MathBackendHIP(object):
         self._ck(self.lib.tfhip_resize_nearest(self.ctx, self._h(x), self._h(out), b, h, w, c,
                                                new_height, new_width, 1 if align_corners else 0))
         return out
+
+    def resize_bilinear_backprop(self, dy, x, align_corners):
+        """backend_cpu.ts:2938-3013."""
+        b, h, w, c = x.shape
+        dx = self._out([b, h, w, c], "float32")
+        self._ck(self.lib.tfhip_resize_bilinear_backprop(
+            self.ctx, self._h(self._materialized(dy)), self._h(dx), b, h, w, c, dy.shape[1], dy.shape[2],
+            1 if align_corners else 0))
+        return dx
+
+    def resize_nearest_neighbor_backprop(self, dy, x, align_corners):
+        """backend_cpu.ts:3070-3165."""
+        b, h, w, c = x.shape
+        dx = self._out([b, h, w, c], "float32")
+        self._ck(self.lib.tfhip_resize_nearest_backprop(
+            self.ctx, self._h(self._materialized(dy)), self._h(dx), b, h, w, c, dy.shape[1], dy.shape[2],
+            1 if align_corners else 0))
+        return dx
+
+    def crop_and_resize(self, images, boxes, box_index, crop_size, method, extrapolation_value):
+        """backend_cpu.ts:3622-3757."""
+        b, h, w, c = images.shape
+        n = boxes.shape[0]
+        out = self._out([n, crop_size[0], crop_size[1], c], "float32")
+        idx = box_index if box_index.dtype == "int32" else self.int(box_index)
+        self._ck(self.lib.tfhip_crop_and_resize(
+            self.ctx, self._h(images), self._h(self._materialized(boxes)), self._h(idx), self._h(out),
+            b, h, w, c, n, crop_size[0], crop_size[1], 0 if method == "bilinear" else 1,
+            float(extrapolation_value)))
+        return out
+
+    def gather_nd(self, x, indices):
+        """backend_cpu.ts:3771-3803; shapes as ops/gather_nd_util.ts:29-78 derives them."""
+        slice_rank = indices.shape[-1]
+        num_slices = su.size_from_shape(indices.shape[:-1])
+        out_shape = list(indices.shape[:-1]) + list(x.shape[slice_rank:])
+        out = self._out_like_storage(out_shape, x)
+        idx = indices if indices.dtype == "int32" else self.int(indices)
+        shape = (C.c_int32 * max(1, x.rank))(*x.shape)
+        self._ck(self.lib.tfhip_gather_nd(self.ctx, self._h(x), self._h(idx), self._h(out), shape, x.rank,
+                                          num_slices, slice_rank))
+        return out
+
+    _SCATTER_SUM, _SCATTER_SKIP_INVALID, _SCATTER_WIDE_SUM = 1, 2, 4
+
+    def _scatter(self, indices, updates, shape, default_value, flags, slice_rank=None):
+        if slice_rank is None:
+            slice_rank = indices.shape[-1] if indices.rank > 1 else 1   # ops/scatter_nd_util.ts:118-120
+        num_updates = su.size_from_shape(indices.shape) // slice_rank if slice_rank else 0
+        dtype = updates.dtype if updates.dtype != "bool" else "int32"
+        out = self._out(list(shape), dtype)
+        idx = indices if indices.dtype == "int32" else self.int(indices)
+        upd = self._materialized(self.cast(updates, dtype))
+        dims = (C.c_int32 * max(1, len(shape)))(*shape)
+        self._ck(self.lib.tfhip_scatter_nd(self.ctx, self._h(self._materialized(idx)), self._h(upd),
+                                           self._h(out), dims, len(shape), num_updates, slice_rank,
+                                           float(default_value), flags))
+        return out
+
+    def scatter_nd(self, indices, updates, shape):
+        """backend_cpu.ts:3805-3814."""
+        return self._scatter(indices, updates, shape, 0.0, self._SCATTER_SUM)
+
+    def sparse_to_dense(self, sparse_indices, sparse_values, output_shape, default_value):
+        """backend_cpu.ts:3759-3769; default_value is a number here."""
+        return self._scatter(sparse_indices, sparse_values, output_shape, default_value, 0)
+
+    def unsorted_segment_sum(self, x, segment_ids, num_segments):
+        """backend_cpu.ts:635-660: x holds the segments along axis 0; ids outside
+        [0, num_segments) contribute nothing; each sum is rounded once."""
+        x = self.cast(x, "float32") if x.dtype == "bool" else x
+        return self._scatter(segment_ids, x, [num_segments] + list(x.shape[1:]), 0.0,
+                             self._SCATTER_SUM | self._SCATTER_SKIP_INVALID | self._SCATTER_WIDE_SUM, 1)
+
+    def diag(self, x):
+        """backend_cpu.ts:346-354: x flattened onto the diagonal of a [size, size] matrix."""
+        n = x.size
+        out = self.fill([n, n], 0, x.dtype)
+        if n:
+            flat = self._materialized(x)
+            self._box_copy(flat, out, [n], [1], 0, [n + 1], 0)
+        return out
+
+    def linspace(self, start, stop, num):
+        """backends/backend_util.ts:78-88: the values are made on the host, as every backend of
+        the reference does."""
+        import numpy as np
+        step = (stop - start) / (num - 1) if num != 1 else float("nan")
+        values = np.zeros(num, np.float32)
+        if num:
+            values[0] = start
+        for i in range(1, num):
+            values[i] = np.float32(float(values[i - 1]) + step)
+        return self._from_host(values)
+
+    def where(self, condition):
+        """backends/where_impl.ts:25-43 on the condition read back to the host, as every
+        backend of the reference does: the coordinates of the true elements, row-major."""
+        import numpy as np
+        cond = np.asarray(self.read_sync(condition.data_id)).reshape(condition.shape)
+        coords = np.argwhere(cond != 0).astype(np.int32).reshape(-1, condition.rank)
+        return self._from_host(coords)
+
+    def non_max_suppression(self, boxes, scores, max_output_size, iou_threshold, score_threshold):
+        """backends/non_max_suppression_impl.ts:25-102 on boxes and scores read back to the
+        host, as the reference's CPU and WebGL backends do."""
+        import numpy as np
+        b = np.asarray(self.read_sync(boxes.data_id), np.float64).reshape(-1, 4)
+        s = np.asarray(self.read_sync(scores.data_id), np.float64)
+        ymin, ymax = np.minimum(b[:, 0], b[:, 2]), np.maximum(b[:, 0], b[:, 2])
+        xmin, xmax = np.minimum(b[:, 1], b[:, 3]), np.maximum(b[:, 1], b[:, 3])
+        area = (ymax - ymin) * (xmax - xmin)
+        candidates = [i for i in np.argsort(-s, kind="stable") if s[i] > score_threshold]
+        selected = []
+        for i in candidates:
+            if len(selected) >= max_output_size:
+                break
+            keep = True
+            for j in reversed(selected):
+                if area[i] <= 0 or area[j] <= 0:
+                    continue
+                h = max(min(ymax[i], ymax[j]) - max(ymin[i], ymin[j]), 0.0)
+                w = max(min(xmax[i], xmax[j]) - max(xmin[i], xmin[j]), 0.0)
+                if h * w / (area[i] + area[j] - h * w) >= iou_threshold:
+                    keep = False
+                    break
+            if keep:
+                selected.append(int(i))
+        return self._from_host(np.asarray(selected, np.int32))
 
     def select(self, condition, a, b):
         """backend_cpu.ts:822-845; a rank-1 condition picks whole slices along the first axis

@@ -49,9 +49,11 @@ def dequantize(t):
     return ENGINE.run_kernel(lambda b: b.dequantize(t))
 
 
-def _conv(x, name, op):
+def _conv(x, name, op, dtype=None):
+    """convertToTensor (tensor_util_env.ts:92-124): a host value becomes a tensor of `dtype`
+    (inferred when None); a Tensor is taken as it is."""
     if not isinstance(x, Tensor):
-        x = tensor(x)
+        x = tensor(x, dtype=dtype)
     return x
 
 
@@ -1161,3 +1163,179 @@ def split(x, num_or_size_splits, axis=0):
             begin[axis] += sz
         return res
     return ENGINE.tidy(run)
+
+
+# ---- index-driven ops and the image utilities around them -------------------------------------
+def gather_nd(x, indices):
+    """ops/gather_nd.ts:56-63 with the checks of ops/gather_nd_util.ts:29-50."""
+    x, indices = _conv(x, "x", "gatherND"), _conv(indices, "indices", "gatherND", "int32")
+    if x.rank < 1:
+        raise ValueError("tf.gatherND() expects the input to be rank 1 or higher, but the rank was %d." % x.rank)
+    if indices.rank < 1:
+        raise ValueError("tf.gatherND() expects the indices to be rank 1 or higher, but the rank was %d."
+                         % indices.rank)
+    if indices.dtype != "int32":
+        raise ValueError("tf.gatherND() expects the indices to be int32 type, but the dtype was %s."
+                         % indices.dtype)
+    if indices.shape[-1] > x.rank:
+        raise ValueError("index innermost dimension length must be <= tensor rank; saw: %d vs. %d"
+                         % (indices.shape[-1], x.rank))
+    if x.size == 0:
+        raise ValueError("Requested more than 0 entries, but input is empty. Input shape: %s." % list(x.shape))
+    return ENGINE.run_kernel(lambda be: be.gather_nd(x, indices))
+
+
+def _check_scatter(op, indices, updates, shape):
+    """ops/scatter_nd_util.ts:28-125."""
+    if indices.dtype != "int32":
+        raise ValueError("The dtype of 'indices' should be int32, but got dtype: %s" % indices.dtype)
+    if len(shape) < 1:
+        raise ValueError("Output rank must be greater or equal to 1, but got shape: %s" % list(shape))
+    slice_dim = indices.shape[-1] if indices.rank > 1 else 1
+    batch_dim = indices.rank - 1 if indices.rank > 1 else 1
+    err = ("Must have updates.shape = indices.shape[:batchDim] + shape[sliceDim:], got updates.shape: %s, "
+           "indices.shape: %s, shape: %s, sliceDim: %d, and batchDim: %d."
+           % (list(updates.shape), list(indices.shape), list(shape), slice_dim, batch_dim))
+    if updates.rank < batch_dim or len(shape) < slice_dim + (updates.rank - batch_dim) or \
+            updates.rank != batch_dim + len(shape) - slice_dim:
+        raise ValueError(err)
+    if builtins_any(updates.shape[d] != indices.shape[d] for d in range(batch_dim)) or \
+            builtins_any(updates.shape[d + batch_dim] != shape[d + slice_dim]
+                         for d in range(updates.rank - batch_dim)):
+        raise ValueError(err)
+
+
+def scatter_nd(indices, updates, shape):
+    """ops/scatter_nd.ts:44-53."""
+    indices, updates = _conv(indices, "indices", "scatterND", "int32"), _conv(updates, "updates", "scatterND")
+    if indices.rank < 1:
+        raise ValueError("tf.scatterND() expects the indices to be rank 1 or higher, but the rank was %d."
+                         % indices.rank)
+    if updates.rank < 1:
+        raise ValueError("tf.scatterND() expects the updates to be rank 1 or higher, but the rank was %d."
+                         % updates.rank)
+    _check_scatter("scatterND", indices, updates, shape)
+    return ENGINE.run_kernel(lambda be: be.scatter_nd(indices, updates, list(shape)))
+
+
+def sparse_to_dense(sparse_indices, sparse_values, output_shape, default_value=0):
+    """ops/sparse_to_dense.ts:61-79 with the checks of ops/sparse_to_dense_util.ts:28-64;
+    default_value is a number."""
+    idx = _conv(sparse_indices, "sparseIndices", "sparseToDense", "int32")
+    vals = _conv(sparse_values, "sparseValues", "sparseToDense")
+    if idx.dtype != "int32":
+        raise ValueError("tf.sparseToDense() expects the indices to be int32 type, but the dtype was %s."
+                         % idx.dtype)
+    if idx.rank > 2:
+        raise ValueError("sparseIndices should be a scalar, vector, or matrix, but got shape %s."
+                         % list(idx.shape))
+    num_elems = idx.shape[0] if idx.rank > 0 else 1
+    num_dims = idx.shape[1] if idx.rank > 1 else 1
+    if len(output_shape) != num_dims:
+        raise ValueError("outputShape has incorrect number of elements:, %d, should be: %d."
+                         % (len(output_shape), num_dims))
+    if not (vals.rank == 0 or (vals.rank == 1 and vals.size == num_elems)):
+        raise ValueError("sparseValues has incorrect shape %s, should be [] or [%d]"
+                         % (list(vals.shape), num_elems))
+    return ENGINE.run_kernel(lambda be: be.sparse_to_dense(idx, vals, list(output_shape), default_value))
+
+
+def unsorted_segment_sum(x, segment_ids, num_segments):
+    """ops/segment_ops.ts:43-89 (forward)."""
+    x = _conv(x, "x", "unsortedSegmentSum")
+    ids = _conv(segment_ids, "segmentIds", "unsortedSegmentSum", "int32")
+    if int(num_segments) != num_segments:
+        raise ValueError("numSegments must be of dtype int")
+    return ENGINE.run_kernel(lambda be: be.unsorted_segment_sum(x, ids, int(num_segments)))
+
+
+def _resize_backprop(method, dy, x, align_corners):
+    dy, x = _conv(dy, "dy", method), _conv(x, "x", method)
+    lift = x.rank == 3
+
+    def run():
+        x4 = reshape(x, (1,) + tuple(x.shape)) if lift else x
+        dy4 = reshape(dy, (1,) + tuple(dy.shape)) if lift else dy
+        r = ENGINE.run_kernel(lambda be: getattr(be, method)(dy4, x4, align_corners))
+        return reshape(r, r.shape[1:]) if lift else r
+    return ENGINE.tidy(run)
+
+
+def resize_bilinear_backprop(dy, x, align_corners=False):
+    """The gradient of resizeBilinear with respect to its input (ops/image_ops.ts:84-89)."""
+    return _resize_backprop("resize_bilinear_backprop", dy, x, align_corners)
+
+
+def resize_nearest_neighbor_backprop(dy, x, align_corners=False):
+    """The gradient of resizeNearestNeighbor with respect to its input (ops/image_ops.ts:140-147)."""
+    return _resize_backprop("resize_nearest_neighbor_backprop", dy, x, align_corners)
+
+
+def crop_and_resize(image, boxes, box_ind, crop_size, method="bilinear", extrapolation_value=0):
+    """ops/image_ops.ts:268-316."""
+    image = _conv(image, "image", "cropAndResize", "float32")
+    boxes = _conv(boxes, "boxes", "cropAndResize", "float32")
+    box_ind = _conv(box_ind, "boxInd", "cropAndResize", "int32")
+    num_boxes = boxes.shape[0]
+    if image.rank != 4:
+        raise ValueError("Error in cropAndResize: image must be rank 4,but got rank %d." % image.rank)
+    if boxes.rank != 2 or boxes.shape[1] != 4:
+        raise ValueError("Error in cropAndResize: boxes must be have size [%d,4] but had shape %s."
+                         % (num_boxes, list(boxes.shape)))
+    if box_ind.rank != 1 or box_ind.shape[0] != num_boxes:
+        raise ValueError("Error in cropAndResize: boxInd must be have size [%d] but had shape %s."
+                         % (num_boxes, list(boxes.shape)))
+    if len(crop_size) != 2:
+        raise ValueError("Error in cropAndResize: cropSize must be of length 2, but got length %d."
+                         % len(crop_size))
+    if crop_size[0] < 1 or crop_size[1] < 1:
+        raise ValueError("cropSize must be atleast [1,1], but was %s" % list(crop_size))
+    if method not in ("bilinear", "nearest"):
+        raise ValueError("method must be bilinear or nearest, but was %s" % method)
+    return ENGINE.run_kernel(lambda be: be.crop_and_resize(image, boxes, box_ind, list(crop_size), method,
+                                                          extrapolation_value))
+
+
+def non_max_suppression(boxes, scores, max_output_size, iou_threshold=0.5, score_threshold=float("-inf")):
+    """ops/image_ops.ts:165-180 with the checks of :214-247."""
+    boxes = _conv(boxes, "boxes", "nonMaxSuppression")
+    scores = _conv(scores, "scores", "nonMaxSuppression")
+    num_boxes = boxes.shape[0]
+    max_output_size = builtins.min(int(max_output_size), num_boxes)
+    if not 0 <= iou_threshold <= 1:
+        raise ValueError("iouThreshold must be in [0, 1], but was '%s'" % iou_threshold)
+    if boxes.rank != 2:
+        raise ValueError("boxes must be a 2D tensor, but was of rank '%d'" % boxes.rank)
+    if boxes.shape[1] != 4:
+        raise ValueError("boxes must have 4 columns, but 2nd dimension was %d" % boxes.shape[1])
+    if scores.rank != 1:
+        raise ValueError("scores must be a 1D tensor")
+    if scores.shape[0] != num_boxes:
+        raise ValueError("scores has incompatible shape with boxes. Expected %d, but was %d"
+                         % (num_boxes, scores.shape[0]))
+    return ENGINE.run_kernel(lambda be: be.non_max_suppression(boxes, scores, max_output_size, iou_threshold,
+                                                              score_threshold))
+
+
+def diag(x):
+    """ops/diag.ts:43-50."""
+    x = _conv(x, "x", "diag")
+
+    def run():
+        flat = reshape(x, (x.size,))
+        r = ENGINE.run_kernel(lambda be: be.diag(flat))
+        return reshape(r, tuple(x.shape) + tuple(x.shape))
+    return ENGINE.tidy(run)
+
+
+def linspace(start, stop, num):
+    """ops/tensor_ops.ts:483-488."""
+    if num <= 0:
+        raise ValueError("The number of values should be positive.")
+    return ENGINE.run_kernel(lambda be: be.linspace(start, stop, int(num)))
+
+
+def where_indices(condition):
+    """tf.whereAsync (ops/logical_ops.ts:189-197): coordinates of the true elements."""
+    condition = _conv(condition, "condition", "whereAsync", "bool")
+    return ENGINE.run_kernel(lambda be: be.where(condition))
