@@ -828,3 +828,162 @@ def test_js_index_driven_ops_and_image_utilities(tmp_path, ref):
     results = c.run()
     c.check(results)
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
+def test_js_composite_surface(tmp_path, ref):
+    """The composed part of tf.*: strict variants, rank aliases, dot / outerProduct / eye / range,
+    conv1d, tf.losses with weights and reductions, softmaxCrossEntropy's custom gradient, LSTM
+    cells, movingAverage, confusionMatrix, signal windows and framing, gramSchmidt, seeded random
+    tensors and dropout.  Expected values: the literals of conv1d_test.ts, confusion_matrix_test.ts
+    and signal_ops_test.ts, and closed forms in float64 for the rest."""
+    rng = np.random.default_rng(101)
+    c = Cases(tmp_path)
+    f32 = lambda a: np.asarray(a, np.float32)
+    call = lambda name, fn, inputs, args, want, **kw: c.add(name, "call", inputs, dict(fn=fn, args=args), want, **kw)
+
+    a, b = rng.standard_normal((4, 6)).astype(np.float32), rng.standard_normal((4, 6)).astype(np.float32)
+    call("add_strict", "addStrict", dict(a=a, b=b), ["$a", "$b"], a + b, exact=True)
+    call("less_strict", "lessStrict", dict(a=a, b=b), ["$a", "$b"], a < b, exact=True)
+    call("pow_strict", "powStrict", dict(a=np.abs(a), b=b), ["$a", "$b"], np.abs(a).astype(np.float64) ** b)
+    call("xor", "logicalXor", dict(a=a > 0, b=b > 0), ["$a", "$b"], (a > 0) ^ (b > 0), exact=True)
+    call("concat2d", "concat2d", dict(a=a, b=b), [["$a", "$b"], 1], np.concatenate([a, b], 1), exact=True)
+    call("pad1d", "pad1d", dict(a=a[0]), ["$a", [2, 1], 7], np.pad(a[0], (2, 1), constant_values=7), exact=True)
+    call("reverse2d", "reverse2d", dict(a=a), ["$a", [0, 1]], a[::-1, ::-1], exact=True)
+    call("slice2d", "slice2d", dict(a=a), ["$a", [1, 2], [2, 3]], a[1:3, 2:5], exact=True)
+    v, w = a[0], b[0]
+    call("dot_vv", "dot", dict(a=v, b=w), ["$a", "$b"], f32(np.dot(v.astype(np.float64), w)).reshape(()))
+    call("dot_mv", "dot", dict(a=a, b=w), ["$a", "$b"], a.astype(np.float64) @ w)
+    call("dot_vm", "dot", dict(a=a[:, 0], b=b), ["$a", "$b"], a[:, 0].astype(np.float64) @ b)
+    call("outer", "outerProduct", dict(a=v, b=w), ["$a", "$b"], np.outer(v.astype(np.float64), w))
+    call("eye", "eye", {}, [3, 5, [2], "int32"], np.tile(np.eye(3, 5, dtype=np.int32), (2, 1, 1)), exact=True)
+    g = lambda t: [cc for cc in _golden_all("linspace_range") if cc["describe"] == "range" and cc["title"] == t][0]["arrays"]
+    call("range_step", "range", {}, [4, 15, 4], f32(g("start stop step")[0]), exact=True)         # array_ops_test.ts: [4, 8, 12]
+    call("range_neg", "range", {}, [4, -2], f32(g("start stop negative")[2]), exact=True)         # [4, 3, 2, 1, 0, -1]
+    call("range_int", "range", {}, [-3, 9, 2, "int32"], np.arange(-3, 9, 2, dtype=np.int32), exact=True)
+    # conv1d_test.ts: 2x2x1 'same' f=1 -> [3,6,9,12]; 4x1 'valid' f=2 -> [4,7,10]
+    call("conv1d_same", "conv1d", dict(x=f32([1, 2, 3, 4]).reshape(2, 2, 1), w=f32([3]).reshape(1, 1, 1)),
+         ["$x", "$w", 1, "same", "NWC", 1], f32([3, 6, 9, 12]).reshape(2, 2, 1))
+    call("conv1d_rank2", "conv1d", dict(x=f32([1, 2, 3, 4]).reshape(4, 1), w=f32([2, 1]).reshape(2, 1, 1)),
+         ["$x", "$w", 1, "valid", "NWC", 1], f32([4, 7, 10]).reshape(3, 1))
+    xs, ws = rng.standard_normal((3, 20, 5)).astype(np.float32), rng.standard_normal((4, 5, 7)).astype(np.float32)
+    want = np.zeros((3, 6, 7))
+    for o in range(6):                                   # stride 3, dilation 1, 'valid': (20 - 4) // 3 + 1 = 6
+        want[:, o] = np.einsum("bkc,kcd->bd", xs[:, 3 * o:3 * o + 4].astype(np.float64), ws)
+    call("conv1d_stride", "conv1d", dict(x=xs, w=ws), ["$x", "$w", 3, "valid"], want, atol=1e-4)
+
+    # tf.losses: labels l, predictions p, weights per row; reductions NONE 0 / MEAN 1 / SUM 2 / SUM_BY_NONZERO 3
+    l = rng.uniform(0, 1, (5, 4)).astype(np.float32)
+    p = rng.uniform(0.05, 0.95, (5, 4)).astype(np.float32)
+    wts = f32([[1.0], [0.0], [2.5], [0.5], [0.0]])
+    l64, p64, w64 = l.astype(np.float64), p.astype(np.float64), wts.astype(np.float64)
+
+    def reduced(losses, weights, reduction):
+        wl = losses if weights is None else losses * weights
+        if reduction == 0:
+            return wl
+        if reduction == 2:
+            return wl.sum()
+        if reduction == 1:
+            if weights is None:
+                return wl.mean()
+            return wl.sum() / weights.sum() / max(1.0, losses.size / weights.size) if losses.size / weights.size > 1 \
+                else wl.sum() / weights.sum()
+        if weights is None:
+            return wl.sum() / losses.size
+        return wl.sum() / np.count_nonzero(np.broadcast_to(weights, losses.shape))
+
+    sig = lambda z: 1 / (1 + np.exp(-z))
+    logits = rng.standard_normal((5, 4)).astype(np.float32) * 3
+    z64 = logits.astype(np.float64)
+    hub = np.abs(p64 - l64)
+    lse = np.log(np.exp(z64 - z64.max(1, keepdims=True)).sum(1, keepdims=True)) + z64.max(1, keepdims=True)
+    onehot = np.eye(4, dtype=np.float32)[rng.integers(0, 4, 5)]
+    smooth = onehot * (1 - 0.1) + 0.1 / 4
+    table = {
+        "absoluteDifference": (np.abs(l64 - p64), ["$l", "$p"]),
+        "meanSquaredError": ((l64 - p64) ** 2, ["$l", "$p"]),
+        "hingeLoss": (np.maximum(0, 1 - (2 * l64 - 1) * p64), ["$l", "$p"]),
+        "logLoss": (-l64 * np.log(p64 + 1e-7) - (1 - l64) * np.log(1 - p64 + 1e-7), ["$l", "$p"]),
+        "huberLoss": (0.5 * np.minimum(hub, 0.3) ** 2 + 0.3 * (hub - np.minimum(hub, 0.3)), ["$l", "$p"]),
+    }
+    extra = {"logLoss": [1e-7], "huberLoss": [0.3]}
+    for name, (losses, args) in table.items():
+        for red in (0, 1, 2, 3):
+            for use_w in (False, True):
+                wv = w64 if use_w else None
+                want = np.asarray(reduced(losses, wv, red), np.float64)
+                call("%s_r%d_w%d" % (name, red, use_w), "losses." + name, dict(l=l, p=p, w=wts if use_w else None),
+                     args + (["$w"] if use_w else [None]) + extra.get(name, []) + [red], f32(want), atol=1e-5)
+    cos = 1 - (l64 * p64).sum(1, keepdims=True)
+    call("cosine", "losses.cosineDistance", dict(l=l, p=p, w=wts), ["$l", "$p", 1, "$w", 3], f32(reduced(cos, w64, 3)).reshape(()))
+    sce = np.maximum(z64, 0) - z64 * (l64 * 0.8 + 0.1) + np.log1p(np.exp(-np.abs(z64)))
+    call("sigmoid_ce", "losses.sigmoidCrossEntropy", dict(l=l, p=logits, w=wts), ["$l", "$p", "$w", 0.2, 1],
+         f32(reduced(sce, w64, 1)).reshape(()), atol=1e-5)
+    sm = -(smooth * (z64 - lse)).sum(1)
+    call("softmax_ce", "losses.softmaxCrossEntropy", dict(l=onehot, p=logits), ["$l", "$p", None, 0.1, 0],
+         f32(sm), atol=1e-5)
+    # its custom gradient with respect to the logits: (softmax - labels) / batch under the default reduction
+    c.add("softmax_ce_grad", "gradCall", dict(x=logits, l=onehot), dict(fn="losses.softmaxCrossEntropy", args=["$l", "$x"]),
+          f32((np.exp(z64 - lse) - onehot) / 5), atol=1e-5)
+
+    # two stacked LSTM cells against numpy
+    def cell(kernel, bias, data, cc, hh):
+        r = np.concatenate([data, hh], 1) @ kernel + bias
+        i_, j_, f_, o_ = np.split(r, 4, 1)
+        new_c = sig(i_) * np.tanh(j_) + cc * sig(1.0 + f_)
+        return new_c, np.tanh(new_c) * sig(o_)
+    data = rng.standard_normal((3, 6))
+    k0, b0 = rng.standard_normal((6 + 5, 20)) * 0.3, rng.standard_normal(20) * 0.1
+    k1, b1 = rng.standard_normal((5 + 4, 16)) * 0.3, rng.standard_normal(16) * 0.1
+    c0, h0, c1, h1 = (rng.standard_normal(s) for s in ((3, 5), (3, 5), (3, 4), (3, 4)))
+    nc0, nh0 = cell(k0, b0, data, c0, h0)
+    nc1, nh1 = cell(k1, b1, nh0, c1, h1)
+    c.add("lstm_stack", "lstmStack", {k: f32(v) for k, v in dict(data=data, k0=k0, b0=b0, k1=k1, b1=b1, c0=c0, h0=h0,
+                                                                  c1=c1, h1=h1).items()}, {},
+          f32(np.concatenate([nc0, nc1, nh0, nh1], 1)), atol=1e-5)
+    call("moving_average", "movingAverage", dict(v=a, x=b), ["$v", "$x", 0.9, 3],
+         a + (b.astype(np.float64) - a) * (1 - 0.9) / (1 - 0.9 ** 3), atol=1e-5)
+    call("moving_average_plain", "movingAverage", dict(v=a, x=b), ["$v", "$x", 0.9, None, False],
+         a + (b.astype(np.float64) - a) * (1 - 0.9), atol=1e-5)
+    # confusion_matrix_test.ts: labels [0,1,2,1,0], predictions [2,1,2,1,0], 3 classes
+    call("confusion", "math.confusionMatrix", dict(l=np.asarray([0, 1, 2, 1, 0], np.int32), p=np.asarray([2, 1, 2, 1, 0], np.int32)),
+         ["$l", "$p", 3], np.asarray([[1, 0, 1], [0, 2, 0], [0, 0, 1]], np.int32), exact=True)
+    # signal_ops_test.ts
+    call("hann7", "signal.hannWindow", {}, [7], f32([0, 0.25, 0.75, 1, 0.75, 0.25, 0]), atol=1e-6)
+    call("hann6", "signal.hannWindow", {}, [6], f32([0., 0.25, 0.75, 1., 0.75, 0.25]), atol=1e-6)
+    call("hamming20", "signal.hammingWindow", {}, [20], f32([
+        0.08000001, 0.10251403, 0.16785222, 0.2696188, 0.3978522, 0.54, 0.68214786, 0.8103813, 0.9121479, 0.977486,
+        1., 0.977486, 0.9121478, 0.8103812, 0.6821477, 0.54, 0.39785212, 0.2696187, 0.16785222, 0.102514]), atol=1e-6)
+    sigl = np.arange(1, 11, dtype=np.float32)
+    call("frame", "signal.frame", dict(s=sigl), ["$s", 4, 3], np.stack([sigl[0:4], sigl[3:7], sigl[6:10]]), exact=True)
+    call("frame_pad", "signal.frame", dict(s=sigl), ["$s", 4, 4, True, -1], np.stack([sigl[0:4], sigl[4:8], np.r_[sigl[8:10], -1, -1]]),
+         exact=True)
+    # gramSchmidt: rows orthonormal, and each spans what the inputs so far span (QR of the transpose)
+    m = rng.standard_normal((4, 9)).astype(np.float32)
+    q, r = np.linalg.qr(m.astype(np.float64).T)
+    call("gram_schmidt", "linalg.gramSchmidt", dict(x=m), ["$x"], (q * np.sign(np.diag(r))).T, atol=1e-4)
+    # seeded random tensors: same seed, same values; moments and ranges as asked
+    c.add("random_normal", "randomMoments", {}, dict(fn="randomNormal", shape=[200, 100], args=[1.5, 2.0, "float32", 7]),
+          f32([1.5, 2.0, 0, 0, 1]), atol=1e9)
+    c.add("truncated_normal", "randomMoments", {}, dict(fn="truncatedNormal", shape=[200, 100], args=[0, 1.0, "float32", 7]),
+          f32([0, 0.88, 0, 0, 1]), atol=1e9)
+    c.add("random_uniform", "randomMoments", {}, dict(fn="randomUniform", shape=[200, 100], args=[-2, 6, "float32", 11]),
+          f32([2.0, 8 / np.sqrt(12), -2, 6, 1]), atol=1e9)
+    c.add("random_uniform_int", "randomMoments", {}, dict(fn="randomUniform", shape=[200, 100], args=[0, 10, "int32", 11]),
+          f32([5.0, 0, 0, 10, 1]), atol=1e9)
+    xd = rng.uniform(1, 2, (300, 50)).astype(np.float32)
+    c.add("dropout", "dropoutStats", dict(x=xd), dict(rate=0.25, seed=5), f32([0.75, 0]), atol=1e9)
+    results = c.run()
+    c.check(results)
+    out = lambda name: np.fromfile(os.path.join(str(tmp_path), name + ".out.bin"), np.float32)
+    mean, std, lo, hi, same = out("random_normal")
+    assert abs(mean - 1.5) < 0.05 and abs(std - 2.0) < 0.05 and same == 1
+    mean, std, lo, hi, same = out("truncated_normal")
+    assert abs(mean) < 0.03 and abs(std - 0.88) < 0.03 and lo >= -2 and hi <= 2 and same == 1
+    mean, std, lo, hi, same = out("random_uniform")
+    assert abs(mean - 2.0) < 0.06 and abs(std - 8 / np.sqrt(12)) < 0.05 and -2 <= lo < -1.95 and 5.95 < hi < 6 and same == 1
+    mean, std, lo, hi, same = out("random_uniform_int")
+    assert abs(mean - 5.0) < 0.1 and lo == 0 and hi == 10 and same == 1
+    kept, err = out("dropout")
+    assert abs(kept - 0.75) < 0.02 and err < 1e-5
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0

@@ -8,6 +8,7 @@ const {ENV} = require('./environment');
 const {Tensor, Variable} = require('./tensor');
 const {KernelBackend, DataStorage} = require('./backend');
 const ops = require('./ops');
+const opsExtra = require('./ops_extra');
 const util = require('./util');
 const conv_util = require('./conv_util');
 const broadcast_util = require('./broadcast_util');
@@ -16,7 +17,7 @@ const io = Object.assign({}, require('./io_utils'), require('./weights_loader'))
 const gradients = require('./gradients');
 const optimizers = require('./optimizers');
 
-const tf = Object.assign({}, ops, gradients, {
+const tf = Object.assign({}, ops, opsExtra, gradients, {
   Tensor, Variable, KernelBackend, DataStorage, ENV, util, io,
   train: optimizers.train, Optimizer: optimizers.Optimizer,
   variable: (initialValue, trainable, name, dtype) => Variable.variable(initialValue, trainable, name, dtype),

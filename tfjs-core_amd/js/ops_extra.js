@@ -1,0 +1,434 @@
+'use strict';
+// The part of the tf.* surface that is pure composition of the ops in ops.js: the *Strict
+// variants, the rank-suffixed aliases, small linear-algebra helpers, tf.losses, LSTM cells,
+// random tensors, dropout.  Each follows the reference file named above it; nothing here
+// touches the device except through those ops.
+const {ENGINE} = require('./engine');
+const {Tensor} = require('./tensor');
+const ops = require('./ops');
+const {customGrad} = require('./gradients');
+const axis_util = require('./axis_util');
+const util = require('./util');
+const {alea} = require('./alea');
+
+const {op, convertToTensor, scalar, reshape, cast} = ops;
+
+// ---- *Strict: same-shape operands only (binary_ops.ts, compare.ts: assertShapesMatch) ----
+const strict = (name, base) => op(name, (a, b) => {
+  const $a = convertToTensor(a, 'a', name), $b = convertToTensor(b, 'b', name);
+  util.assert(util.arraysEqual($a.shape, $b.shape),
+              () => `Error in ${name}: Shapes ${$a.shape} and ${$b.shape} must match`);
+  return base($a, $b);
+});
+const STRICT = {
+  addStrict: ops.add, subStrict: ops.sub, mulStrict: ops.mul, divStrict: ops.div, modStrict: ops.mod,
+  powStrict: ops.pow, maximumStrict: ops.maximum, minimumStrict: ops.minimum,
+  squaredDifferenceStrict: ops.squaredDifference, equalStrict: ops.equal, notEqualStrict: ops.notEqual,
+  lessStrict: ops.less, lessEqualStrict: ops.lessEqual, greaterStrict: ops.greater,
+  greaterEqualStrict: ops.greaterEqual
+};
+const strictOps = {};
+Object.keys(STRICT).forEach(name => strictOps[name] = strict(name, STRICT[name]));
+
+// ---- rank-suffixed aliases (concat.ts, pad.ts, reverse.ts, slice.ts, batchnorm.ts) ----
+const ranked = (name, rank, argIndex, base) => op(name, (...args) => {
+  const list = Array.isArray(args[argIndex]) && args[argIndex][0] instanceof Tensor ? args[argIndex] : [args[argIndex]];
+  list.forEach(t => {
+    const $t = convertToTensor(t, 'x', name);
+    util.assert($t.rank === rank, () => `Error in ${name}: x must be rank ${rank} but got rank ${$t.rank}.`);
+  });
+  return base(...args);
+});
+const aliases = {};
+[1, 2, 3, 4].forEach(r => {
+  aliases[`concat${r}d`] = op(`concat${r}d`, (tensors, axis) => ops.concat(tensors, r === 1 ? 0 : axis));
+  aliases[`pad${r}d`] = ranked(`pad${r}d`, r, 0, (x, paddings, value) => ops.pad(x, r === 1 ? [paddings] : paddings, value));
+  aliases[`reverse${r}d`] = ranked(`reverse${r}d`, r, 0, (x, axis) => ops.reverse(x, r === 1 ? 0 : axis));
+  aliases[`slice${r}d`] = ranked(`slice${r}d`, r, 0, (x, begin, size) => ops.slice(x, r === 1 ? [begin] : begin, r === 1 ? [size] : size));
+});
+[2, 3, 4].forEach(r => {
+  aliases[`batchNorm${r}d`] = ranked(`batchNorm${r}d`, r, 0, ops.batchNorm);
+  // the deprecated argument order (batchnorm.ts:33-100): (x, mean, variance, varianceEpsilon, scale, offset)
+  aliases[`batchNormalization${r}d`] = ranked(`batchNormalization${r}d`, r, 0,
+      (x, mean, variance, eps, scale, offset) => ops.batchNorm(x, mean, variance, offset, scale, eps));
+});
+aliases.batchNormalization = op('batchNormalization',
+    (x, mean, variance, eps, scale, offset) => ops.batchNorm(x, mean, variance, offset, scale, eps));
+
+// logical_ops.ts:104-112
+const logicalXor = op('logicalXor', (a, b) => {
+  const $a = convertToTensor(a, 'a', 'logicalXor', 'bool'), $b = convertToTensor(b, 'b', 'logicalXor', 'bool');
+  return ops.logicalAnd(ops.logicalOr($a, $b), ops.logicalNot(ops.logicalAnd($a, $b)));
+});
+
+// tensor_ops.ts (range): values made on the host
+function range(start, stop, step, dtype) {
+  if (step == null) step = 1;
+  if (dtype == null) dtype = 'float32';
+  if (step === 0) throw new Error('Cannot have a step of zero');
+  const sameStartStop = start === stop;
+  const increasingRangeNegativeStep = start < stop && step < 0;
+  const decreasingRangePositiveStep = stop < start && step > 1;
+  if (sameStartStop || increasingRangeNegativeStep || decreasingRangePositiveStep) return ops.zeros([0], dtype);
+  const numElements = Math.abs(Math.ceil((stop - start) / step));
+  const values = dtype === 'int32' ? new Int32Array(numElements) : new Float32Array(numElements);
+  if (stop < start && step === 1) step = -1;  // auto adjust the step's sign
+  values[0] = start;
+  for (let i = 1; i < values.length; i++) values[i] = values[i - 1] + step;
+  return ops.tensor1d(values, dtype);
+}
+
+// array_ops.ts (eye): an identity matrix, tiled over batchShape
+const eye = op('eye', (numRows, numColumns, batchShape, dtype) => {
+  if (numColumns == null) numColumns = numRows;
+  const n = Math.min(numRows, numColumns);
+  const values = new Float32Array(numRows * numColumns);
+  for (let i = 0; i < n; i++) values[i * numColumns + i] = 1;
+  const out = cast(ops.tensor2d(values, [numRows, numColumns]), dtype || 'float32');
+  if (batchShape == null) return out;
+  util.assert(batchShape.length >= 1 && batchShape.length <= 3,
+              () => `eye() currently supports only 1D and 2D batchShapes, but received ${batchShape.length}D.`);
+  const lifted = reshape(out, batchShape.map(() => 1).concat([numRows, numColumns]));
+  return ops.tile(lifted, batchShape.concat([1, 1]));
+});
+
+// matmul.ts (outerProduct, dot)
+const outerProduct = op('outerProduct', (v1, v2) => {
+  const $v1 = convertToTensor(v1, 'v1', 'outerProduct'), $v2 = convertToTensor(v2, 'v2', 'outerProduct');
+  util.assert($v1.rank === 1 && $v2.rank === 1,
+              () => `Error in outerProduct: inputs must be rank 1, but got ranks ${$v1.rank} and ${$v2.rank}.`);
+  return ops.matMul(reshape($v1, [-1, 1]), reshape($v2, [1, -1]));
+});
+const dot = op('dot', (t1, t2) => {
+  const $t1 = convertToTensor(t1, 't1', 'dot'), $t2 = convertToTensor(t2, 't2', 'dot');
+  util.assert(($t1.rank === 1 || $t1.rank === 2) && ($t2.rank === 1 || $t2.rank === 2),
+              () => `Error in dot: inputs must all be rank 1 or 2, but got ranks ${$t1.rank} and ${$t2.rank}.`);
+  const t1Inner = $t1.rank === 1 ? $t1.size : $t1.shape[1];
+  const t2Inner = $t2.rank === 1 ? $t2.size : $t2.shape[0];
+  util.assert(t1Inner === t2Inner,
+              () => `Error in dot: inner dimensions of inputs must match, but got ${t1Inner} and ${t2Inner}.`);
+  if ($t1.rank === 1 && $t2.rank === 1) return reshape(ops.matMul(reshape($t1, [1, -1]), reshape($t2, [-1, 1])), []);
+  if ($t1.rank === 1 && $t2.rank === 2) {
+    const r = ops.matMul(reshape($t1, [1, -1]), $t2);
+    return reshape(r, [r.size]);
+  }
+  if ($t1.rank === 2 && $t2.rank === 1) {
+    const r = ops.matMul($t1, reshape($t2, [-1, 1]));
+    return reshape(r, [r.size]);
+  }
+  return ops.matMul($t1, $t2);
+});
+
+// conv.ts (conv1d): a conv2d over an image of height 1
+const conv1d = op('conv1d', (x, filter, stride, pad, dataFormat, dilation, dimRoundingMode) => {
+  const $x = convertToTensor(x, 'x', 'conv1d'), $filter = convertToTensor(filter, 'filter', 'conv1d');
+  if (dataFormat == null) dataFormat = 'NWC';
+  if (dilation == null) dilation = 1;
+  const x3D = $x.rank === 2 ? reshape($x, [1, $x.shape[0], $x.shape[1]]) : $x;
+  util.assert(x3D.rank === 3, () => `Error in conv1d: input must be rank 3, but got rank ${x3D.rank}.`);
+  util.assert($filter.rank === 3, () => `Error in conv1d: filter must be rank 3, but got rank ${$filter.rank}.`);
+  util.assert(x3D.shape[2] === $filter.shape[1],
+              () => `Error in conv1d: depth of input (${x3D.shape[2]}) must match input depth for filter ${$filter.shape[1]}.`);
+  util.assert(dataFormat === 'NWC', () => `Error in conv1d: got dataFormat of ${dataFormat} but only NWC is currently supported.`);
+  const filter4D = reshape($filter, [1, $filter.shape[0], $filter.shape[1], $filter.shape[2]]);
+  const input4D = reshape(x3D, [x3D.shape[0], 1, x3D.shape[1], x3D.shape[2]]);
+  const res = ops.conv2d(input4D, filter4D, [1, stride], pad, 'NHWC', [1, dilation], dimRoundingMode);
+  return $x.rank === 2 ? reshape(res, [res.shape[2], res.shape[3]]) : reshape(res, [res.shape[0], res.shape[2], res.shape[3]]);
+});
+
+// moving_average.ts
+const movingAverage = op('movingAverage', (v, x, decay, step, zeroDebias) => {
+  if (zeroDebias == null) zeroDebias = true;
+  const $v = convertToTensor(v, 'v', 'movingAverage'), $x = convertToTensor(x, 'x', 'movingAverage');
+  const $decay = convertToTensor(decay, 'decay', 'movingAverage');
+  util.assert(util.arraysEqual($v.shape, $x.shape), () => `Error in movingAverage: Shapes ${$v.shape} and ${$x.shape} must match`);
+  const one = scalar(1);
+  let update = ops.mul(ops.sub($x, $v), ops.sub(one, $decay));
+  if (zeroDebias) {
+    util.assert(step != null, () => 'When using zeroDebias: true, step is required.');
+    const $step = convertToTensor(step, 'step', 'movingAverage');
+    update = ops.div(update, ops.sub(one, ops.pow($decay, $step)));
+  }
+  return ops.add($v, update);
+});
+
+// lstm.ts
+const basicLSTMCell = op('basicLSTMCell', (forgetBias, lstmKernel, lstmBias, data, c, h) => {
+  const $forgetBias = convertToTensor(forgetBias, 'forgetBias', 'basicLSTMCell');
+  const $lstmKernel = convertToTensor(lstmKernel, 'lstmKernel', 'basicLSTMCell');
+  const $lstmBias = convertToTensor(lstmBias, 'lstmBias', 'basicLSTMCell');
+  const $data = convertToTensor(data, 'data', 'basicLSTMCell');
+  const $c = convertToTensor(c, 'c', 'basicLSTMCell'), $h = convertToTensor(h, 'h', 'basicLSTMCell');
+  const combined = ops.concat([$data, $h], 1);
+  const res = ops.add(ops.matMul(combined, $lstmKernel), $lstmBias);
+  const batchSize = res.shape[0], sliceCols = res.shape[1] / 4;
+  const part = k => ops.slice(res, [0, k * sliceCols], [batchSize, sliceCols]);
+  const i = part(0), j = part(1), f = part(2), o = part(3);
+  const newC = strictOps.addStrict(strictOps.mulStrict(ops.sigmoid(i), ops.tanh(j)),
+                                   strictOps.mulStrict($c, ops.sigmoid(ops.add($forgetBias, f))));
+  const newH = strictOps.mulStrict(ops.tanh(newC), ops.sigmoid(o));
+  return [newC, newH];
+});
+const multiRNNCell = op('multiRNNCell', (lstmCells, data, c, h) => {
+  let input = convertToTensor(data, 'data', 'multiRNNCell');
+  const newC = [], newH = [];
+  lstmCells.forEach((cell, i) => {
+    const output = cell(input, convertToTensor(c[i], 'c', 'multiRNNCell'), convertToTensor(h[i], 'h', 'multiRNNCell'));
+    newC.push(output[0]);
+    newH.push(output[1]);
+    input = output[1];
+  });
+  return [newC, newH];
+});
+
+// confusion_matrix.ts
+const confusionMatrix = op('confusionMatrix', (labels, predictions, numClasses) => {
+  const $labels = convertToTensor(labels, 'labels', 'confusionMatrix');
+  const $predictions = convertToTensor(predictions, 'predictions', 'confusionMatrix');
+  util.assert(numClasses == null || numClasses > 0 && Number.isInteger(numClasses),
+              () => `If provided, numClasses must be a positive integer, but got ${numClasses}`);
+  util.assert($labels.rank === 1, () => `Expected the rank of labels to be 1, but got ${$labels.rank}`);
+  util.assert($predictions.rank === 1, () => `Expected the rank of predictions to be 1, but got ${$predictions.rank}`);
+  util.assert($labels.shape[0] === $predictions.shape[0],
+              () => `Mismatch in the number of examples: ${$labels.shape[0]} vs. ${$predictions.shape[0]}. ` +
+                  'Labels and predictions should have the same number of elements.');
+  const oneHotLabels = cast(ops.oneHot(cast($labels, 'int32'), numClasses), 'float32');
+  const oneHotPredictions = cast(ops.oneHot(cast($predictions, 'int32'), numClasses), 'float32');
+  return cast(ops.matMul(ops.transpose(oneHotLabels), oneHotPredictions), 'int32');
+});
+
+// ---- tf.losses (loss_ops.ts) ----
+const Reduction = {NONE: 0, MEAN: 1, SUM: 2, SUM_BY_NONZERO_WEIGHTS: 3};
+const computeWeightedLoss = op('computeWeightedLoss', (losses, weights, reduction) => {
+  if (reduction == null) reduction = Reduction.SUM_BY_NONZERO_WEIGHTS;
+  const $losses = convertToTensor(losses, 'losses', 'computeWeightedLoss');
+  const $weights = weights == null ? null : convertToTensor(weights, 'weights', 'computeWeightedLoss');
+  const weightedLoss = $weights == null ? $losses : ops.mul($losses, $weights);
+  if (reduction === Reduction.NONE) return weightedLoss;
+  if (reduction === Reduction.SUM) return ops.sum(weightedLoss);
+  if (reduction === Reduction.MEAN) {
+    if ($weights == null) return ops.mean(weightedLoss);
+    const broadcastFactor = $losses.size / $weights.size;
+    const result = ops.div(ops.sum(weightedLoss), ops.sum($weights));
+    return broadcastFactor > 1 ? ops.div(result, scalar(broadcastFactor)) : result;
+  }
+  if (reduction === Reduction.SUM_BY_NONZERO_WEIGHTS) {
+    if ($weights == null) return ops.div(ops.sum(weightedLoss), scalar($losses.size));
+    const broadcastedWeights = ops.mul($weights, ops.ones($losses.shape));
+    const numNonZeros = cast(ops.sum(ops.notEqual(broadcastedWeights, scalar(0))), 'float32');
+    return ops.div(ops.sum(weightedLoss), numNonZeros);
+  }
+  throw Error(`Unknown reduction: ${reduction}`);
+});
+// labels and predictions of one shape -> per-element losses -> computeWeightedLoss
+const pairLoss = (name, f) => op(name, (labels, predictions, ...rest) => {
+  const $labels = convertToTensor(labels, 'labels', name);
+  const $predictions = convertToTensor(predictions, 'predictions', name);
+  util.assert(util.arraysEqual($labels.shape, $predictions.shape),
+              () => `Error in ${name}: Shapes ${$labels.shape} and ${$predictions.shape} must match`);
+  return f($labels, $predictions, ...rest);
+});
+const absoluteDifference = pairLoss('absoluteDifference', (l, p, weights, reduction) =>
+    computeWeightedLoss(ops.abs(ops.sub(l, p)), weights, reduction));
+const meanSquaredError = pairLoss('meanSquaredError', (l, p, weights, reduction) =>
+    computeWeightedLoss(ops.squaredDifference(l, p), weights, reduction));
+const cosineDistance = pairLoss('cosineDistance', (l, p, axis, weights, reduction) =>
+    computeWeightedLoss(ops.sub(scalar(1), ops.sum(ops.mul(l, p), axis, true)), weights, reduction));
+const hingeLoss = pairLoss('hingeLoss', (l, p, weights, reduction) => {
+  const one = scalar(1);
+  const signed = ops.sub(ops.mul(scalar(2), l), one);
+  return computeWeightedLoss(ops.relu(ops.sub(one, ops.mul(signed, p))), weights, reduction);
+});
+const logLoss = pairLoss('logLoss', (l, p, weights, epsilon, reduction) => {
+  const one = scalar(1), eps = scalar(epsilon == null ? 1e-7 : epsilon);
+  const losses = ops.sub(ops.neg(ops.mul(l, ops.log(ops.add(p, eps)))),
+                         ops.mul(ops.sub(one, l), ops.log(ops.add(ops.sub(one, p), eps))));
+  return computeWeightedLoss(losses, weights, reduction);
+});
+const huberLoss = pairLoss('huberLoss', (l, p, weights, delta, reduction) => {
+  const deltaScalar = scalar(delta == null ? 1.0 : delta);
+  const error = ops.abs(ops.sub(p, l));
+  const quadratic = ops.minimum(error, deltaScalar);
+  const linear = ops.sub(error, quadratic);
+  const losses = ops.add(ops.mul(scalar(0.5), ops.square(quadratic)), ops.mul(deltaScalar, linear));
+  return computeWeightedLoss(losses, weights, reduction);
+});
+const sigmoidCrossEntropy = pairLoss('sigmoidCrossEntropy', (labels, logits, weights, labelSmoothing, reduction) => {
+  let l = labels;
+  if (labelSmoothing > 0) {
+    const s = scalar(labelSmoothing);
+    l = ops.add(ops.mul(l, ops.sub(scalar(1), s)), ops.mul(scalar(0.5), s));
+  }
+  // max(x, 0) - x * z + log(1 + exp(-|x|))
+  const losses = ops.add(ops.sub(ops.relu(logits), ops.mul(logits, l)), ops.log1p(ops.exp(ops.neg(ops.abs(logits)))));
+  return computeWeightedLoss(losses, weights, reduction);
+});
+function softmaxCrossEntropyWithLogits(labels, logits, dim) {
+  if (dim == null || dim === -1) dim = logits.rank - 1;
+  if (dim !== logits.rank - 1) {
+    throw Error('Softmax cross entropy along a non-last dimension is not yet supported. ' +
+                `Labels / logits was rank ${logits.rank} and dim was ${dim}`);
+  }
+  const customOp = customGrad((labels, logits, save) => {
+    const lse = ops.logSumExp(logits, [dim], true);
+    const logResult = ops.sub(cast(logits, 'float32'), lse);
+    save([labels, logResult]);
+    const value = ops.sum(ops.neg(ops.mul(logResult, labels)), [dim]);
+    const gradFunc = (dy, saved) => {
+      const [labels, logResult] = saved;
+      const dyShape = axis_util.expandShapeToKeepDim(dy.shape, [dim]);
+      return [
+        ops.mul(reshape(dy, dyShape), ops.sub(cast(labels, 'float32'), ops.exp(logResult))),
+        ops.mul(reshape(dy, dyShape), ops.sub(ops.exp(logResult), cast(labels, 'float32')))
+      ];
+    };
+    return {value, gradFunc};
+  });
+  return customOp(labels, logits);
+}
+const softmaxCrossEntropy = pairLoss('softmaxCrossEntropy', (onehotLabels, logits, weights, labelSmoothing, reduction) => {
+  let l = onehotLabels;
+  if (labelSmoothing > 0) {
+    const s = scalar(labelSmoothing);
+    l = ops.add(ops.mul(l, ops.sub(scalar(1), s)), ops.div(s, scalar(l.shape[1])));
+  }
+  return computeWeightedLoss(softmaxCrossEntropyWithLogits(l, logits), weights, reduction);
+});
+
+// ---- random tensors (array_ops.ts rand / randomNormal / truncatedNormal / randomUniform, rand.ts):
+// values are drawn on the host with the Alea generator and uploaded.  parity unpinned for the
+// exact streams (the generator is restated, its package is not vendored); the reference's
+// tests check moments and ranges.
+function rand(shape, randFunction, dtype) {
+  const size = util.sizeFromShape(shape);
+  const values = dtype === 'int32' ? new Int32Array(size) : dtype === 'bool' ? new Uint8Array(size) : new Float32Array(size);
+  for (let i = 0; i < size; i++) values[i] = randFunction();
+  return ops.tensor(values, shape, dtype || 'float32');
+}
+function gaussian(mean, stdDev, dtype, truncated, seed) {
+  const random = alea(String(seed ? seed : Math.random()));
+  const upper = mean + stdDev * 2, lower = mean - stdDev * 2;
+  const ok = v => !truncated || (v <= upper && v >= lower);
+  const convert = v => (dtype == null || dtype === 'float32') ? v : Math.round(v);
+  let nextVal = NaN;
+  // Marsaglia's polar method, two values per accepted pair (rand.ts:66-96)
+  return () => {
+    if (!isNaN(nextVal)) {
+      const value = nextVal;
+      nextVal = NaN;
+      return value;
+    }
+    let resultX, resultY;
+    for (;;) {
+      let v1, v2, s;
+      do {
+        v1 = 2 * random() - 1;
+        v2 = 2 * random() - 1;
+        s = v1 * v1 + v2 * v2;
+      } while (s >= 1 || s === 0);
+      const mul = Math.sqrt(-2.0 * Math.log(s) / s);
+      resultX = mean + stdDev * v1 * mul;
+      resultY = mean + stdDev * v2 * mul;
+      if (ok(resultX)) break;
+    }
+    if (ok(resultY)) nextVal = convert(resultY);
+    return convert(resultX);
+  };
+}
+function randomNormal(shape, mean, stdDev, dtype, seed) {
+  if (dtype === 'bool') throw new Error(`Unsupported data type ${dtype}`);
+  return rand(shape, gaussian(mean || 0, stdDev == null ? 1 : stdDev, dtype, false, seed), dtype);
+}
+function truncatedNormal(shape, mean, stdDev, dtype, seed) {
+  if (dtype === 'bool') throw new Error('Unsupported data type bool');
+  return rand(shape, gaussian(mean || 0, stdDev == null ? 1 : stdDev, dtype, true, seed), dtype);
+}
+function randomUniform(shape, minval, maxval, dtype, seed) {
+  if (minval == null) minval = 0;
+  if (maxval == null) maxval = 1;
+  const isFloat = dtype == null || dtype === 'float32';
+  if (!isFloat && maxval - minval <= 1) {
+    throw new Error(`The difference between ${minval} - ${maxval} <= 1 and dtype is not float`);
+  }
+  const random = alea(String(seed == null ? Math.random() : seed));
+  return rand(shape, () => {
+    const v = minval + (maxval - minval) * random();
+    return isFloat ? v : Math.round(v);
+  }, dtype);
+}
+
+// dropout.ts:48-73 (+ dropout_util.ts getNoiseShape)
+const dropout = op('dropout', (x, rate, noiseShape, seed) => {
+  const $x = convertToTensor(x, 'x', 'dropout');
+  util.assert($x.dtype === 'float32',
+              () => `x has to be a floating point tensor since it's going to be scaled, but got a ${$x.dtype} tensor instead.`);
+  util.assert(rate >= 0 && rate < 1, () => `rate must be a float in the range [0, 1), but got ${rate}.`);
+  if (rate === 0) return x instanceof Tensor ? ops.clone($x) : $x;
+  const shape = noiseShape == null ? $x.shape.slice() :
+      noiseShape.map((d, i) => d == null && $x.shape[i] != null ? $x.shape[i] : d);
+  const keepProb = 1 - rate;
+  const multiplier = ops.div(ops.floor(ops.add(randomUniform(shape, 0, 1, 'float32', seed), scalar(keepProb))),
+                             scalar(keepProb));
+  return ops.mul($x, multiplier);
+});
+
+// ---- tf.signal windows and framing (signal_ops.ts), tf.linalg.gramSchmidt (linalg_ops.ts:64-111) ----
+function cosineWindow(windowLength, a, b) {
+  const even = 1 - windowLength % 2;
+  const values = new Float32Array(windowLength);
+  for (let i = 0; i < windowLength; ++i) {
+    values[i] = a - b * Math.cos((2.0 * Math.PI * i) / (windowLength + even - 1));
+  }
+  return ops.tensor1d(values, 'float32');
+}
+const hannWindow = op('hannWindow', windowLength => cosineWindow(windowLength, 0.5, 0.5));
+const hammingWindow = op('hammingWindow', windowLength => cosineWindow(windowLength, 0.54, 0.46));
+const frame = op('frame', (signal, frameLength, frameStep, padEnd, padValue) => {
+  const $signal = convertToTensor(signal, 'signal', 'frame');
+  let start = 0;
+  const output = [];
+  while (start + frameLength <= $signal.size) {
+    output.push(ops.slice($signal, [start], [frameLength]));
+    start += frameStep;
+  }
+  if (padEnd) {
+    const padLen = (start + frameLength) - $signal.size;
+    output.push(ops.concat([ops.slice($signal, [start], [frameLength - padLen]), ops.fill([padLen], padValue || 0)], 0));
+  }
+  if (output.length === 0) return ops.tensor2d([], [0, frameLength]);
+  return reshape(ops.concat(output, 0), [output.length, frameLength]);
+});
+const gramSchmidt = op('gramSchmidt', xs => {
+  const inputIsTensor2D = !Array.isArray(xs);
+  let vectors;
+  if (inputIsTensor2D) {
+    vectors = ops.split(xs, xs.shape[0], 0).map(x => ops.squeeze(x, [0]));
+  } else {
+    util.assert(xs != null && xs.length > 0, () => 'Gram-Schmidt process: input must not be null, undefined, or empty');
+    const dim = xs[0].shape[0];
+    xs.forEach(x => util.assert(x.shape[0] === dim,
+        () => `Gram-Schmidt: Non-unique lengths found in the input vectors: (${x.shape[0]} vs. ${dim})`));
+    vectors = xs;
+  }
+  util.assert(vectors.length <= vectors[0].shape[0],
+              () => `Gram-Schmidt: Number of vectors (${vectors.length}) exceeds number of dimensions (${vectors[0].shape[0]}).`);
+  const ys = [];
+  for (let i = 0; i < vectors.length; ++i) {
+    ys.push(ENGINE.tidy(() => {
+      let x = vectors[i];
+      for (let j = 0; j < i; ++j) x = ops.sub(x, ops.mul(ops.sum(strictOps.mulStrict(ys[j], x)), ys[j]));
+      return ops.div(x, ops.norm(x, 'euclidean'));
+    }));
+  }
+  return inputIsTensor2D ? ops.stack(ys, 0) : ys;
+});
+
+module.exports = Object.assign({}, strictOps, aliases, {
+  signal: {hannWindow, hammingWindow, frame},
+  linalg: {gramSchmidt},
+  logicalXor, range, eye, outerProduct, dot, conv1d, movingAverage, basicLSTMCell, multiRNNCell,
+  rand, randomNormal, truncatedNormal, randomUniform, dropout, Reduction,
+  math: {confusionMatrix},
+  losses: {computeWeightedLoss, absoluteDifference, meanSquaredError, cosineDistance, hingeLoss, logLoss,
+           huberLoss, sigmoidCrossEntropy, softmaxCrossEntropy}
+});

@@ -108,6 +108,46 @@ const OPS = {
   // x.square().sum() style chains over the methods attached to Tensor
   chainMore: i => i.x.abs().sqrt().add(i.x.square().mean(1, true)).maximum(i.x.neg()).slice([0, 1], [2, 3])
       .pad([[1, 0], [0, 1]]).expandDims(0).squeeze([0]).flatten(),
+  // a.fn names a function of tf (dots walk namespaces); a.args are its arguments, with the
+  // string "$name" standing for the input tensor of that name (also inside arrays);
+  // a.pick selects one tensor of a returned list, the others are disposed
+  call: (i, a) => {
+    const resolve = v => typeof v === 'string' && v[0] === '$' ? i[v.slice(1)] :
+        Array.isArray(v) ? v.map(resolve) : v === 'Infinity' ? Infinity : v;
+    const fn = a.fn.split('.').reduce((o, k) => o[k], tf);
+    const out = fn(...a.args.map(resolve));
+    if (a.pick == null) return out;
+    const flat = [].concat(...out);
+    flat.forEach((t, k) => k !== a.pick && t.dispose());
+    return flat[a.pick];
+  },
+  gradCall: (i, a) => {
+    const resolve = (v, x) => v === '$x' ? x : typeof v === 'string' && v[0] === '$' ? i[v.slice(1)] : v;
+    const fn = a.fn.split('.').reduce((o, k) => o[k], tf);
+    return tf.grad(x => fn(...a.args.map(v => resolve(v, x))))(i.x);
+  },
+  lstmStack: i => {
+    const cell = (k, b) => (data, c, h) => tf.basicLSTMCell(tf.scalar(1.0), k, b, data, c, h);
+    const [c, h] = tf.multiRNNCell([cell(i.k0, i.b0), cell(i.k1, i.b1)], i.data, [i.c0, i.c1], [i.h0, i.h1]);
+    const out = tf.concat([c[0], c[1], h[0], h[1]], 1);
+    tf.dispose([c, h]);
+    return out;
+  },
+  randomMoments: (i, a) => {
+    const x = tf[a.fn](a.shape, ...a.args);
+    const again = tf[a.fn](a.shape, ...a.args);
+    const same = tf.cast(tf.all(tf.equal(x, again)), 'float32');
+    const m = tf.moments(tf.cast(x, 'float32'));
+    const out = tf.stack([m.mean, tf.sqrt(m.variance), tf.cast(tf.min(x), 'float32'), tf.cast(tf.max(x), 'float32'), same]);
+    tf.dispose([x, again, m]);
+    return out;
+  },
+  dropoutStats: (i, a) => {
+    const y = tf.dropout(i.x, a.rate, null, a.seed);
+    const kept = tf.notEqual(y, tf.scalar(0));
+    const out = tf.stack([tf.mean(tf.cast(kept, 'float32')), tf.max(tf.abs(tf.sub(tf.mul(tf.cast(kept, 'float32'), tf.div(i.x, tf.scalar(1 - a.rate))), y)))]);
+    return out;
+  },
   gatherND: i => tf.gatherND(i.x, i.indices),
   scatterND: (i, a) => tf.scatterND(i.indices, i.updates, a.shape),
   sparseToDense: (i, a) => tf.sparseToDense(i.indices, i.values, a.shape, a.defaultValue),
