@@ -94,6 +94,8 @@ CASES = {
     "segment": ("tfjs-core/src/ops/segment_ops_test.ts", ["unsortedSegmentSum"]),
     "image": ("tfjs-core/src/ops/image_ops_test.ts", ["nonMaxSuppression", "cropAndResize"]),
     "diag": ("tfjs-core/src/ops/diag_test.ts", ["diag"]),
+    "conv3d": ("tfjs-core/src/ops/conv3d_test.ts", ["conv3d"]),
+    "pool3d": ("tfjs-core/src/ops/pool_test.ts", ["maxPool3d", "avgPool3d"]),
     "linspace_range": ("tfjs-core/src/ops/array_ops_test.ts", ["linspace", "range"]),
 }
 # fixture name -> (reference test file, describe blocks, title filter): the gradient blocks,

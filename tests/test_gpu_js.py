@@ -987,3 +987,101 @@ def test_js_composite_surface(tmp_path, ref):
     kept, err = out("dropout")
     assert abs(kept - 0.75) < 0.02 and err < 1e-5
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
+def _conv3d_float64(x, w, strides, pad):
+    """Direct 3-D convolution in float64 with the 'same' / 'valid' geometry of
+    ops/conv_util.ts:469-497; returns (y, front/top/left padding)."""
+    b, d, h, wd, c = x.shape
+    fd, fh, fw, _, oc = w.shape
+    sd, sh, sw = strides
+    if pad == "same":
+        od, oh, ow = -(-d // sd), -(-h // sh), -(-wd // sw)
+        pads = [((o - 1) * s + f - n) // 2 for o, s, f, n in ((od, sd, fd, d), (oh, sh, fh, h), (ow, sw, fw, wd))]
+    else:
+        od, oh, ow = -(-(d - fd + 1) // sd), -(-(h - fh + 1) // sh), -(-(wd - fw + 1) // sw)
+        pads = [0, 0, 0]
+    xp = np.zeros((b, d + 2 * fd, h + 2 * fh, wd + 2 * fw, c))
+    xp[:, pads[0]:pads[0] + d, pads[1]:pads[1] + h, pads[2]:pads[2] + wd] = x
+    y = np.zeros((b, od, oh, ow, oc))
+    for z in range(od):
+        for r in range(oh):
+            for q in range(ow):
+                win = xp[:, z * sd:z * sd + fd, r * sh:r * sh + fh, q * sw:q * sw + fw]
+                y[:, z, r, q] = np.einsum("bdhwc,dhwco->bo", win, w)
+    return y, pads
+
+
+def test_js_conv3d_and_pool3d(tmp_path):
+    """conv3d (with both gradients), maxPool3d and avgPool3d, which the backend composes from its
+    2-D kernels, against the literals of conv3d_test.ts and pool_test.ts and a float64 direct
+    convolution on seeded shapes with strides and 'same' padding."""
+    import re
+    rng = np.random.default_rng(103)
+    c = Cases(tmp_path)
+    for k, case in enumerate(_golden_all("conv3d")):
+        m = re.match(r"x=\[(.*?)\] f=\[(.*?)\] s=(\[.*?\]|\d+) d=1 p=(\w+)", case["title"])
+        xs, fs = [int(v) for v in m.group(1).split(",")], [int(v) for v in m.group(2).split(",")]
+        strides = json.loads(m.group(3))
+        x = ((np.arange(np.prod(xs)) + 1) / np.prod(xs)).astype(np.float32).reshape(xs)   # generateCaseInputs
+        w = ((np.arange(np.prod(fs)) + 1) / np.prod(fs)).astype(np.float32).reshape(fs)
+        want = np.asarray(case["arrays"][-1], np.float32)
+        s3 = strides if isinstance(strides, list) else [strides] * 3
+        y64, _ = _conv3d_float64(x.astype(np.float64), w.astype(np.float64), s3, m.group(4))
+        assert y64.size == want.size and np.abs(y64.ravel() - want).max() < 1e-3, case["title"]   # pins the checker
+        c.add("conv3d_%d" % k, "call", dict(x=x, w=w), dict(fn="conv3d", args=["$x", "$w", strides, m.group(4)]),
+              want.reshape(y64.shape), atol=1e-4)
+    for k, case in enumerate(_golden_all("pool3d")):
+        a, title = case["arrays"], case["title"]
+        m = re.search(r"f=\[(.*?)\] s=(\d+)(?: p=(\w+))?", title)
+        pad = m.group(3) if m.group(3) else "0"
+        pad = int(pad) if pad.isdigit() else pad
+        shape, want = (a[2], a[3]) if len(a[2]) == len(a[1]) and int(np.prod(a[2])) == len(a[3]) else (a[3], a[2])
+        args = ["$x", [int(v) for v in m.group(1).split(",")], int(m.group(2)), pad]
+        if "roundingMode=floor" in title:
+            args.append("floor")
+        c.add("pool3d_%d" % k, "call", dict(x=np.asarray(a[0], np.float32).reshape(a[1])),
+              dict(fn=case["describe"], args=args), np.asarray(want, np.float32).reshape(shape), atol=1e-5)
+    for k, (xs, fs, strides, pad) in enumerate((((2, 7, 6, 5, 3), (3, 2, 3, 3, 4), [2, 1, 2], "same"),
+                                                ((1, 6, 5, 7, 2), (2, 3, 2, 2, 5), [1, 2, 1], "valid"),
+                                                ((2, 4, 4, 4, 8), (3, 3, 3, 8, 8), [1, 1, 1], "same"))):
+        x = rng.standard_normal(xs).astype(np.float32)
+        w = rng.standard_normal(fs).astype(np.float32)
+        y64, pads = _conv3d_float64(x.astype(np.float64), w.astype(np.float64), strides, pad)
+        c.add("conv3d_seeded_%d" % k, "call", dict(x=x, w=w), dict(fn="conv3d", args=["$x", "$w", strides, pad]), y64,
+              atol=1e-4)
+        # gradients in float64: dW by correlating windows with dy, dx by spreading dy through the filter
+        dy = rng.standard_normal(y64.shape).astype(np.float32)
+        fd, fh, fw = fs[:3]
+        xp = np.zeros((xs[0], xs[1] + 2 * fd, xs[2] + 2 * fh, xs[3] + 2 * fw, xs[4]))
+        xp[:, pads[0]:pads[0] + xs[1], pads[1]:pads[1] + xs[2], pads[2]:pads[2] + xs[3]] = x
+        dxp, dw = np.zeros_like(xp), np.zeros(fs)
+        for z in range(y64.shape[1]):
+            for r in range(y64.shape[2]):
+                for q in range(y64.shape[3]):
+                    sl = (slice(None), slice(z * strides[0], z * strides[0] + fd),
+                          slice(r * strides[1], r * strides[1] + fh), slice(q * strides[2], q * strides[2] + fw))
+                    dw += np.einsum("bdhwc,bo->dhwco", xp[sl], dy[:, z, r, q].astype(np.float64))
+                    dxp[sl] += np.einsum("bo,dhwco->bdhwc", dy[:, z, r, q].astype(np.float64), w.astype(np.float64))
+        dx = dxp[:, pads[0]:pads[0] + xs[1], pads[1]:pads[1] + xs[2], pads[2]:pads[2] + xs[3]]
+        c.add("conv3d_dx_%d" % k, "gradConv3d", dict(x=x, w=w, dy=dy), dict(strides=strides, pad=pad, wrt=0), dx,
+              atol=2e-4)
+        c.add("conv3d_dw_%d" % k, "gradConv3d", dict(x=x, w=w, dy=dy), dict(strides=strides, pad=pad, wrt=1), dw,
+              atol=2e-4)
+    # pools on a seeded volume with stride 2 and 'same' padding, against numpy windows
+    v = rng.standard_normal((2, 5, 6, 7, 3)).astype(np.float32)
+    od, oh, ow = 3, 3, 4
+    mx, av = np.zeros((2, od, oh, ow, 3)), np.zeros((2, od, oh, ow, 3))
+    pf, pt, pl = ((od - 1) * 2 + 3 - 5) // 2, ((oh - 1) * 2 + 3 - 6) // 2, ((ow - 1) * 2 + 3 - 7) // 2
+    for z in range(od):
+        for r in range(oh):
+            for q in range(ow):
+                win = v[:, max(0, 2 * z - pf):2 * z - pf + 3, max(0, 2 * r - pt):2 * r - pt + 3,
+                        max(0, 2 * q - pl):2 * q - pl + 3].astype(np.float64)
+                mx[:, z, r, q] = win.max((1, 2, 3))
+                av[:, z, r, q] = win.mean((1, 2, 3))
+    c.add("max_pool3d_seeded", "call", dict(x=v), dict(fn="maxPool3d", args=["$x", 3, 2, "same"]), mx, exact=True)
+    c.add("avg_pool3d_seeded", "call", dict(x=v), dict(fn="avgPool3d", args=["$x", 3, 2, "same"]), av, atol=1e-5)
+    results = c.run()
+    c.check(results)
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0

@@ -814,6 +814,107 @@ class MathBackendHIP extends KernelBackend {
     return out;
   }
 
+  // ---- 3-D convolutions and pools (backend.ts:443-451, 467-482) as sums over the filter's depth
+  //      taps of the 2-D kernels: out[:, od] = sum_kd conv2d(x[:, od * sd + kd * dd - front], f[kd]).
+  //      The planes a tap reads for all od form one strided box, so each tap is a single 2-D call
+  //      over a batch of batch * outDepth images. ----
+  info2dOf(ci) {
+    const n = ci.batchSize * ci.outDepth;
+    return {
+      batchSize: n, inHeight: ci.inHeight, inWidth: ci.inWidth, inChannels: ci.inChannels,
+      outHeight: ci.outHeight, outWidth: ci.outWidth, outChannels: ci.outChannels,
+      strideHeight: ci.strideHeight, strideWidth: ci.strideWidth, dilationHeight: ci.dilationHeight,
+      dilationWidth: ci.dilationWidth, filterHeight: ci.filterHeight, filterWidth: ci.filterWidth,
+      padInfo: ci.padInfo, dataFormat: 'channelsLast',
+      inShape: [n, ci.inHeight, ci.inWidth, ci.inChannels],
+      outShape: [n, ci.outHeight, ci.outWidth, ci.outChannels],
+      filterShape: [ci.filterHeight, ci.filterWidth, ci.inChannels, ci.outChannels]
+    };
+  }
+  // x padded along depth with `value`, so that every tap of every output plane exists
+  depthPadded(x, ci, value) {
+    const need = (ci.outDepth - 1) * ci.strideDepth + ci.effectiveFilterDepth;
+    const front = Math.max(ci.padInfo.front, 0);
+    const back = Math.max(need - front - ci.inDepth, 0);
+    return front || back ? this.pad(x, [[0, 0], [front, back], [0, 0], [0, 0], [0, 0]], value) : x;
+  }
+  // planes kd * dd + od * sd (od = 0 .. outDepth - 1) of a depth-padded x, as [batch * outDepth, h, w, c]
+  tapPlanes(xp, ci, kd) {
+    const [b, , h, w, c] = xp.shape;
+    const planes = this.stridedSliceBox(xp, [0, kd * ci.dilationDepth, 0, 0, 0], [b, ci.outDepth, h, w, c],
+                                        [1, ci.strideDepth, 1, 1, 1]);
+    return this.reshape(planes, [b * ci.outDepth, h, w, c]);
+  }
+  filterTap(filter, ci, kd) {
+    const [, fh, fw, inC, outC] = filter.shape;
+    return this.reshape(this.slice(filter, [kd, 0, 0, 0, 0], [1, fh, fw, inC, outC]), [fh, fw, inC, outC]);
+  }
+  conv3d(x, filter, ci) {
+    const xp = this.depthPadded(x, ci, 0), info = this.info2dOf(ci);
+    let acc = null;
+    for (let kd = 0; kd < ci.filterDepth; kd++) {
+      const y = this.conv2d(this.tapPlanes(xp, ci, kd), this.filterTap(filter, ci, kd), info);
+      acc = acc == null ? y : this.add(acc, y);
+    }
+    return this.reshape(acc, ci.outShape);
+  }
+  conv3dDerFilter(x, dy, ci) {
+    const xp = this.depthPadded(x, ci, 0), info = this.info2dOf(ci);
+    const dy4 = this.reshape(dy, info.outShape);
+    const taps = [];
+    for (let kd = 0; kd < ci.filterDepth; kd++) {
+      const dw = this.conv2dDerFilter(this.tapPlanes(xp, ci, kd), dy4, info);
+      taps.push(this.reshape(dw, [1].concat(dw.shape)));
+    }
+    return taps.length === 1 ? taps[0] : this.concat(taps, 0);
+  }
+  conv3dDerInput(dy, filter, ci) {
+    const info = this.info2dOf(ci);
+    const dy4 = this.reshape(dy, info.outShape);
+    const need = (ci.outDepth - 1) * ci.strideDepth + ci.effectiveFilterDepth;
+    const front = Math.max(ci.padInfo.front, 0);
+    const depth = Math.max(need, front + ci.inDepth);
+    const plane = ci.inHeight * ci.inWidth * ci.inChannels;
+    let acc = null;
+    for (let kd = 0; kd < ci.filterDepth; kd++) {
+      const dx4 = this.conv2dDerInput(dy4, this.filterTap(filter, ci, kd), info);
+      // plane od of this tap belongs to padded depth kd * dd + od * sd
+      const spread = this.fill([ci.batchSize, depth, ci.inHeight, ci.inWidth, ci.inChannels], 0, 'float32');
+      this.boxCopy(dx4, spread, [ci.batchSize, ci.outDepth, plane], [ci.outDepth * plane, plane, 1], 0,
+                   [depth * plane, ci.strideDepth * plane, 1], kd * ci.dilationDepth * plane);
+      acc = acc == null ? spread : this.add(acc, spread);
+    }
+    return this.slice(acc, [0, front, 0, 0, 0], ci.inShape);
+  }
+  maxPool3d(x, ci) {
+    const xp = this.depthPadded(x, ci, -Infinity), info = this.info2dOf(ci);
+    let acc = null;
+    for (let kd = 0; kd < ci.filterDepth; kd++) {
+      const y = this.maxPool(this.tapPlanes(xp, ci, kd), info);
+      acc = acc == null ? y : this.maximum(acc, y);
+    }
+    return this.reshape(acc, ci.outShape);
+  }
+  // backend_cpu.ts:2511-2581 divides the window's sum by the number of its elements inside the
+  // volume: both come from zero-padded window sums (a depthwise convolution with a filter of
+  // ones), the count from a volume of ones
+  avgPool3d(x, ci) {
+    const info = this.info2dOf(ci);
+    const ones = this.fill([ci.filterHeight, ci.filterWidth, ci.inChannels, 1], 1, 'float32');
+    const windowSums = v => {
+      const vp = this.depthPadded(v, ci, 0);
+      let acc = null;
+      for (let kd = 0; kd < ci.filterDepth; kd++) {
+        const y = this.depthwiseConv2D(this.tapPlanes(vp, ci, kd), ones, info);
+        acc = acc == null ? y : this.add(acc, y);
+      }
+      return acc;
+    };
+    const total = windowSums(this.cast(x, 'float32'));
+    const count = windowSums(this.fill(x.shape, 1, 'float32'));
+    return this.reshape(this.realDivide(total, count), ci.outShape);
+  }
+
   // ---- host-side routines: every backend of the reference runs these on values read back ----
   fromHost(values, shape, dtype) { return Tensor.make(shape, {values}, dtype, this); }
   // backends/backend_util.ts:78-88: a running float32 sum of the double step

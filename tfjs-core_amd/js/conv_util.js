@@ -118,6 +118,78 @@ function computePool2DInfo(inShape, filterSize, strides, dilations, pad, roundin
   return computeConv2DInfo(inShape, filterShape, strides, dilations, pad, roundingMode, false, dataFormat);
 }
 
+// ---- 3-D (conv_util.ts:91-118, 222-300, 322-356, 437-505) ----
+function parse3TupleParam(param) {
+  return typeof param === 'number' ? [param, param, param] : param;
+}
+// A numeric pad sizes all three output dimensions from the filter's depth and the depth
+// stride, as the reference does (conv_util.ts:463-468).
+function get3DPadAndOutInfo(pad, inDepth, inHeight, inWidth, strideDepth, strideHeight, strideWidth,
+                            filterDepth, filterHeight, filterWidth, roundingMode) {
+  let padInfo, outDepth, outHeight, outWidth;
+  if (typeof pad === 'number') {
+    padInfo = {top: pad, bottom: pad, left: pad, right: pad, front: pad, back: pad,
+               type: pad === 0 ? 'VALID' : 'NUMBER'};
+    const size = (n, what) => {
+      const v = conditionalRound((n - filterDepth + 2 * pad) / strideDepth + 1, roundingMode);
+      util.assert(util.isInt(v), () => `The output # of ${what} (${v}) must be an integer. ` +
+                                       'Change the stride and/or zero pad parameters');
+      return v;
+    };
+    outDepth = size(inDepth, 'depths');
+    outHeight = size(inHeight, 'rows');
+    outWidth = size(inWidth, 'columns');
+  } else if (pad === 'same') {
+    outDepth = Math.ceil(inDepth / strideDepth);
+    outHeight = Math.ceil(inHeight / strideHeight);
+    outWidth = Math.ceil(inWidth / strideWidth);
+    const alongDepth = (outDepth - 1) * strideDepth + filterDepth - inDepth;
+    const alongHeight = (outHeight - 1) * strideHeight + filterHeight - inHeight;
+    const alongWidth = (outWidth - 1) * strideWidth + filterWidth - inWidth;
+    const front = Math.floor(alongDepth / 2), top = Math.floor(alongHeight / 2), left = Math.floor(alongWidth / 2);
+    padInfo = {top, bottom: alongHeight - top, left, right: alongWidth - left, front, back: alongDepth - front,
+               type: 'SAME'};
+  } else if (pad === 'valid') {
+    padInfo = {top: 0, bottom: 0, left: 0, right: 0, front: 0, back: 0, type: 'VALID'};
+    outDepth = Math.ceil((inDepth - filterDepth + 1) / strideDepth);
+    outHeight = Math.ceil((inHeight - filterHeight + 1) / strideHeight);
+    outWidth = Math.ceil((inWidth - filterWidth + 1) / strideWidth);
+  } else {
+    throw Error(`Unknown padding parameter: ${pad}`);
+  }
+  return {padInfo, outDepth, outHeight, outWidth};
+}
+
+function computeConv3DInfo(inShape, filterShape, strides, dilations, pad, depthwise, dataFormat, roundingMode) {
+  if (dataFormat == null) dataFormat = 'channelsLast';
+  if (dataFormat !== 'channelsLast') throw new Error(`hip backend: only NDHWC 3-D convolutions are implemented`);
+  const [batchSize, inDepth, inHeight, inWidth, inChannels] = inShape;
+  const [filterDepth, filterHeight, filterWidth, , filterChannels] = filterShape;
+  const [strideDepth, strideHeight, strideWidth] = parse3TupleParam(strides);
+  const [dilationDepth, dilationHeight, dilationWidth] = parse3TupleParam(dilations);
+  const effectiveFilterDepth = getEffectiveFilterSize(filterDepth, dilationDepth);
+  const effectiveFilterHeight = getEffectiveFilterSize(filterHeight, dilationHeight);
+  const effectiveFilterWidth = getEffectiveFilterSize(filterWidth, dilationWidth);
+  const {padInfo, outDepth, outHeight, outWidth} = get3DPadAndOutInfo(
+      pad, inDepth, inHeight, inWidth, strideDepth, strideHeight, strideWidth, effectiveFilterDepth,
+      effectiveFilterHeight, effectiveFilterWidth, roundingMode);
+  const outChannels = depthwise ? filterChannels * inChannels : filterChannels;
+  return {
+    batchSize, dataFormat, inDepth, inHeight, inWidth, inChannels, outDepth, outHeight, outWidth, outChannels,
+    padInfo, strideDepth, strideHeight, strideWidth, filterDepth, filterHeight, filterWidth,
+    effectiveFilterDepth, effectiveFilterHeight, effectiveFilterWidth, dilationDepth, dilationHeight,
+    dilationWidth, inShape, outShape: [batchSize, outDepth, outHeight, outWidth, outChannels], filterShape
+  };
+}
+
+function computePool3DInfo(inShape, filterSize, strides, dilations, pad, roundingMode, dataFormat) {
+  if (dataFormat == null) dataFormat = 'NDHWC';
+  if (dataFormat !== 'NDHWC') throw new Error(`hip backend: only NDHWC 3-D pooling is implemented`);
+  const [filterDepth, filterHeight, filterWidth] = parse3TupleParam(filterSize);
+  return computeConv3DInfo(inShape, [filterDepth, filterHeight, filterWidth, inShape[4], inShape[4]], strides,
+                           dilations, pad, false, 'channelsLast', roundingMode);
+}
+
 function convertConv2DDataFormat(dataFormat) {
   if (dataFormat === 'NHWC') return 'channelsLast';
   if (dataFormat === 'NCHW') return 'channelsFirst';
@@ -126,5 +198,6 @@ function convertConv2DDataFormat(dataFormat) {
 
 module.exports = {
   parseTupleParam, tupleValuesAreOne, eitherStridesOrDilationsAreOne, getEffectiveFilterSize,
-  computeConv2DInfo, computePool2DInfo, convertConv2DDataFormat
+  computeConv2DInfo, computePool2DInfo, convertConv2DDataFormat, parse3TupleParam, computeConv3DInfo,
+  computePool3DInfo
 };

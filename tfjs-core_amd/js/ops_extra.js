@@ -9,6 +9,7 @@ const ops = require('./ops');
 const {customGrad} = require('./gradients');
 const axis_util = require('./axis_util');
 const util = require('./util');
+const conv_util = require('./conv_util');
 const {alea} = require('./alea');
 
 const {op, convertToTensor, scalar, reshape, cast} = ops;
@@ -372,6 +373,65 @@ const dropout = op('dropout', (x, rate, noiseShape, seed) => {
   return ops.mul($x, multiplier);
 });
 
+// ---- 3-D convolutions and pools (conv.ts:744-807, 833-905, pool.ts:461-560, 600-700) ----
+const as5D = (t, name) => {
+  const lifted = t.rank === 4;
+  const t5 = lifted ? reshape(t, [1].concat(t.shape)) : t;
+  util.assert(t5.rank === 5, () => `Error in ${name}: input must be rank 5, but got rank ${t5.rank}.`);
+  return [t5, lifted];
+};
+const conv3dDerInput = (xShape, dy, filter, strides, pad) => {
+  const ci = conv_util.computeConv3DInfo(xShape, filter.shape, strides, 1, pad);
+  return ENGINE.runKernel(backend => backend.conv3dDerInput(dy, filter, ci), {dy});
+};
+const conv3dDerFilter = (x, dy, filterShape, strides, pad) => {
+  const ci = conv_util.computeConv3DInfo(x.shape, filterShape, strides, 1, pad);
+  return ENGINE.runKernel(backend => backend.conv3dDerFilter(x, dy, ci), {x, dy});
+};
+const conv3d = op('conv3d', (x, filter, strides, pad, dataFormat, dilations) => {
+  const $x = convertToTensor(x, 'x', 'conv3d'), $filter = convertToTensor(filter, 'filter', 'conv3d');
+  if (dataFormat == null) dataFormat = 'NDHWC';
+  if (dilations == null) dilations = [1, 1, 1];
+  const [x5D, lifted] = as5D($x, 'conv3d');
+  util.assert($filter.rank === 5, () => `Error in conv3d: filter must be rank 5, but got rank ${$filter.rank}.`);
+  util.assert(x5D.shape[4] === $filter.shape[3],
+              () => `Error in conv3d: depth of input (${x5D.shape[4]}) must match input depth for filter ${$filter.shape[3]}.`);
+  util.assert(conv_util.eitherStridesOrDilationsAreOne(strides, dilations),
+              () => `Error in conv3D: Either strides or dilations must be 1. Got strides ${strides} and dilations '${dilations}'`);
+  util.assert(dataFormat === 'NDHWC', () => `Error in conv3d: got dataFormat of ${dataFormat} but only NDHWC is currently supported.`);
+  const ci = conv_util.computeConv3DInfo(x5D.shape, $filter.shape, strides, dilations, pad);
+  const res = ENGINE.runKernel((backend, save) => {
+    save([x5D, $filter]);
+    return backend.conv3d(x5D, $filter, ci);
+  }, {x: x5D, $filter}, (dy, saved) => {
+    util.assert(conv_util.tupleValuesAreOne(dilations),
+                () => `Error in gradient of conv3D: dilation rates greater than 1 are not yet supported in gradients. Got dilations '${dilations}'`);
+    return {
+      x: () => conv3dDerInput(saved[0].shape, dy, saved[1], strides, pad),
+      $filter: () => conv3dDerFilter(saved[0], dy, saved[1].shape, strides, pad)
+    };
+  });
+  return lifted ? reshape(res, res.shape.slice(1)) : res;
+});
+const pool3d = (name, method) => op(name, (x, filterSize, strides, pad, dimRoundingMode, dataFormat, dilations) => {
+  const $x = convertToTensor(x, 'x', name);
+  if (dataFormat == null) dataFormat = 'NDHWC';
+  if (dilations == null) dilations = [1, 1, 1];
+  const [x5D, lifted] = as5D($x, name);
+  util.assert(dataFormat === 'NDHWC', () => `Error in ${name}: Only NDHWC is currently supported, but got dataFormat of ${dataFormat}`);
+  util.assert(conv_util.eitherStridesOrDilationsAreOne(strides, dilations),
+              () => `Error in ${name}: Either strides or dilations must be 1. Got strides ${strides} and dilations '${dilations}'`);
+  if (dimRoundingMode != null) {
+    util.assert(util.isInt(pad), () => `Error in ${name}: pad must be an integer when using, dimRoundingMode ${dimRoundingMode} but got pad ${pad}.`);
+  }
+  util.assert(conv_util.tupleValuesAreOne(dilations), () => `Error in ${name}: the hip backend pools 3-D windows without dilation`);
+  const ci = conv_util.computePool3DInfo(x5D.shape, filterSize, strides, dilations, pad, dimRoundingMode, dataFormat);
+  let res = ENGINE.runKernel(backend => backend[method](x5D, ci), {x: x5D});
+  if (method === 'avgPool3d') res = cast(res, x5D.dtype);
+  return lifted ? reshape(res, res.shape.slice(1)) : res;
+});
+const maxPool3d = pool3d('maxPool3d', 'maxPool3d'), avgPool3d = pool3d('avgPool3d', 'avgPool3d');
+
 // ---- tf.signal windows and framing (signal_ops.ts), tf.linalg.gramSchmidt (linalg_ops.ts:64-111) ----
 function cosineWindow(windowLength, a, b) {
   const even = 1 - windowLength % 2;
@@ -426,7 +486,7 @@ const gramSchmidt = op('gramSchmidt', xs => {
 module.exports = Object.assign({}, strictOps, aliases, {
   signal: {hannWindow, hammingWindow, frame},
   linalg: {gramSchmidt},
-  logicalXor, range, eye, outerProduct, dot, conv1d, movingAverage, basicLSTMCell, multiRNNCell,
+  logicalXor, range, eye, outerProduct, dot, conv1d, conv3d, maxPool3d, avgPool3d, movingAverage, basicLSTMCell, multiRNNCell,
   rand, randomNormal, truncatedNormal, randomUniform, dropout, Reduction,
   math: {confusionMatrix},
   losses: {computeWeightedLoss, absoluteDifference, meanSquaredError, cosineDistance, hingeLoss, logLoss,

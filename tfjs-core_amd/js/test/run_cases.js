@@ -148,6 +148,7 @@ const OPS = {
     const out = tf.stack([tf.mean(tf.cast(kept, 'float32')), tf.max(tf.abs(tf.sub(tf.mul(tf.cast(kept, 'float32'), tf.div(i.x, tf.scalar(1 - a.rate))), y)))]);
     return out;
   },
+  gradConv3d: (i, a) => tf.grads((x, w) => tf.conv3d(x, w, a.strides, a.pad))([i.x, i.w], i.dy)[a.wrt],
   gatherND: i => tf.gatherND(i.x, i.indices),
   scatterND: (i, a) => tf.scatterND(i.indices, i.updates, a.shape),
   sparseToDense: (i, a) => tf.sparseToDense(i.indices, i.values, a.shape, a.defaultValue),
