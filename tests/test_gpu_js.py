@@ -839,7 +839,8 @@ def test_js_composite_surface(tmp_path, ref):
     rng = np.random.default_rng(101)
     c = Cases(tmp_path)
     f32 = lambda a: np.asarray(a, np.float32)
-    call = lambda name, fn, inputs, args, want, **kw: c.add(name, "call", inputs, dict(fn=fn, args=args), want, **kw)
+    def call(name, fn, inputs, args, want, pick=None, **kw):
+        c.add(name, "call", inputs, dict(fn=fn, args=args, **({} if pick is None else {"pick": pick})), want, **kw)
 
     a, b = rng.standard_normal((4, 6)).astype(np.float32), rng.standard_normal((4, 6)).astype(np.float32)
     call("add_strict", "addStrict", dict(a=a, b=b), ["$a", "$b"], a + b, exact=True)
@@ -971,6 +972,23 @@ def test_js_composite_surface(tmp_path, ref):
           f32([2.0, 8 / np.sqrt(12), -2, 6, 1]), atol=1e9)
     c.add("random_uniform_int", "randomMoments", {}, dict(fn="randomUniform", shape=[200, 100], args=[0, 10, "int32", 11]),
           f32([5.0, 0, 0, 10, 1]), atol=1e9)
+    c.add("random_gamma", "randomMoments", {}, dict(fn="randomGamma", shape=[200, 100], args=[2, 3, "float32", 13]),
+          f32([6.0, 4.243, 0, 0, 1]), atol=1e9)
+    # Householder QR: LAPACK (numpy) uses the same sign convention, r_jj = -sign(x_jj) |x|
+    for name, shape, full in (("qr_tall", (7, 4), False), ("qr_tall_full", (7, 4), True), ("qr_wide", (3, 6), False),
+                              ("qr_square", (5, 5), False)):
+        mat = rng.standard_normal(shape).astype(np.float32)
+        qn, rn = np.linalg.qr(mat.astype(np.float64), mode="complete" if full else "reduced")
+        if shape[0] <= shape[1]:
+            # the reference also reflects the final 1 x 1 block (tau = 2), LAPACK leaves it alone
+            qn[:, -1] *= -1
+            rn[-1, :] *= -1
+        call(name + "_q", "linalg.qr", dict(x=mat), ["$x", full], qn, atol=1e-4, pick=0)
+        call(name + "_r", "linalg.qr", dict(x=mat), ["$x", full], rn, atol=1e-4, pick=1)
+    batch = rng.standard_normal((2, 3, 4, 3)).astype(np.float32)
+    qn, rn = np.linalg.qr(batch.astype(np.float64))
+    call("qr_batched_q", "linalg.qr", dict(x=batch), ["$x"], qn, atol=1e-4, pick=0)
+    call("qr_batched_r", "linalg.qr", dict(x=batch), ["$x"], rn, atol=1e-4, pick=1)
     xd = rng.uniform(1, 2, (300, 50)).astype(np.float32)
     c.add("dropout", "dropoutStats", dict(x=xd), dict(rate=0.25, seed=5), f32([0.75, 0]), atol=1e9)
     results = c.run()
@@ -984,6 +1002,8 @@ def test_js_composite_surface(tmp_path, ref):
     assert abs(mean - 2.0) < 0.06 and abs(std - 8 / np.sqrt(12)) < 0.05 and -2 <= lo < -1.95 and 5.95 < hi < 6 and same == 1
     mean, std, lo, hi, same = out("random_uniform_int")
     assert abs(mean - 5.0) < 0.1 and lo == 0 and hi == 10 and same == 1
+    mean, std, lo, hi, same = out("random_gamma")
+    assert abs(mean - 6.0) < 0.15 and abs(std - 18 ** 0.5) < 0.15 and lo > 0 and same == 1
     kept, err = out("dropout")
     assert abs(kept - 0.75) < 0.02 and err < 1e-5
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
@@ -1068,6 +1088,8 @@ def test_js_conv3d_and_pool3d(tmp_path):
               atol=2e-4)
         c.add("conv3d_dw_%d" % k, "gradConv3d", dict(x=x, w=w, dy=dy), dict(strides=strides, pad=pad, wrt=1), dw,
               atol=2e-4)
+        c.add("conv3d_transpose_%d" % k, "call", dict(x=dy, w=w),
+              dict(fn="conv3dTranspose", args=["$x", "$w", list(xs), strides, pad]), dx, atol=2e-4)
     # pools on a seeded volume with stride 2 and 'same' padding, against numpy windows
     v = rng.standard_normal((2, 5, 6, 7, 3)).astype(np.float32)
     od, oh, ow = 3, 3, 4

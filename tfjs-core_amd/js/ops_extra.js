@@ -358,6 +358,36 @@ function randomUniform(shape, minval, maxval, dtype, seed) {
   }, dtype);
 }
 
+// array_ops.ts (randomGamma) over rand.ts:114-172: Marsaglia and Tsang's squeeze method on a
+// standard normal stream seeded from the first uniform draw.  The accepted value is multiplied
+// by beta (the reference converts the rate to a scale and then divides by that scale).
+function randomGamma(shape, alpha, beta, dtype, seed) {
+  if (beta == null) beta = 1;
+  if (dtype == null) dtype = 'float32';
+  if (dtype !== 'float32' && dtype !== 'int32') throw new Error(`Unsupported data type ${dtype}`);
+  const randu = alea(String(seed ? seed : Math.random()));
+  const randn = gaussian(0, 1, dtype, false, randu());
+  const d = alpha < 1 ? alpha + 2 / 3 : alpha - 1 / 3;
+  const c = 1 / Math.sqrt(9 * d);
+  return rand(shape, () => {
+    let v;
+    for (;;) {
+      let x;
+      do {
+        x = randn();
+        v = 1 + c * x;
+      } while (v <= 0);
+      v *= v * v;
+      const x2 = x * x;
+      const u = randu();
+      if (u < 1 - 0.331 * x2 * x2 || Math.log(u) < 0.5 * x2 + d * (1 - v + Math.log(v))) break;
+    }
+    v = beta * d * v;
+    if (alpha < 1) v *= Math.pow(randu(), 1 / alpha);
+    return dtype === 'float32' ? v : Math.round(v);
+  }, dtype);
+}
+
 // dropout.ts:48-73 (+ dropout_util.ts getNoiseShape)
 const dropout = op('dropout', (x, rate, noiseShape, seed) => {
   const $x = convertToTensor(x, 'x', 'dropout');
@@ -431,6 +461,23 @@ const pool3d = (name, method) => op(name, (x, filterSize, strides, pad, dimRound
   return lifted ? reshape(res, res.shape.slice(1)) : res;
 });
 const maxPool3d = pool3d('maxPool3d', 'maxPool3d'), avgPool3d = pool3d('avgPool3d', 'avgPool3d');
+// conv.ts:960-968: the transposed 3-D convolution is conv3d's gradient with respect to its input
+const conv3dTranspose = op('conv3dTranspose', (x, filter, outputShape, strides, pad) => {
+  const $x = convertToTensor(x, 'x', 'conv3dTranspose'), $filter = convertToTensor(filter, 'filter', 'conv3dTranspose');
+  util.assert(outputShape.length === 4 || outputShape.length === 5,
+              () => `Error in conv3dDerInput: outShape must be length 4 or 5, but got length ${outputShape.length}.`);
+  const lifted = $x.rank === 4;
+  const dy5D = lifted ? reshape($x, [1].concat($x.shape)) : $x;
+  const shape5D = outputShape.length === 4 ? [1].concat(outputShape) : outputShape;
+  util.assert(dy5D.rank === 5, () => `Error in conv3dDerInput: dy must be rank 5, but got rank ${dy5D.rank}`);
+  util.assert($filter.rank === 5, () => `Error in conv3dDerInput: filter must be rank 5, but got rank ${$filter.rank}`);
+  util.assert(shape5D[4] === $filter.shape[3],
+              () => `Error in conv3dDerInput: depth of input (${shape5D[4]}) must match input depth for filter ${$filter.shape[3]}.`);
+  util.assert(dy5D.shape[4] === $filter.shape[4],
+              () => `Error in conv3dDerInput: depth of output (${dy5D.shape[4]}) must match output depth for filter ${$filter.shape[4]}.`);
+  const res = conv3dDerInput(shape5D, dy5D, $filter, strides, pad);
+  return lifted ? reshape(res, res.shape.slice(1)) : res;
+});
 
 // ---- tf.signal windows and framing (signal_ops.ts), tf.linalg.gramSchmidt (linalg_ops.ts:64-111) ----
 function cosineWindow(windowLength, a, b) {
@@ -458,6 +505,54 @@ const frame = op('frame', (signal, frameLength, frameStep, padEnd, padValue) => 
   if (output.length === 0) return ops.tensor2d([], [0, frameLength]);
   return reshape(ops.concat(output, 0), [output.length, frameLength]);
 });
+// linalg_ops.ts:157-270: QR by Householder reflections, column by column.  For column j,
+// with x = r[j:, j]: s = -sign(x0) (+1 for x0 <= 0), u1 = x0 - s |x|, w = x / u1 with w0 = 1,
+// tau = -s u1 / |x|; then r[j:, :] -= tau w (w' r[j:, :]) and q[:, j:] -= (q[:, j:] w) (tau w)'.
+function qr2d(x, fullMatrices) {
+  return ENGINE.tidy(() => {
+    const [m, n] = x.shape;
+    let q = eye(m), r = ops.clone(x);
+    const one = ops.tensor2d([1], [1, 1]);
+    for (let j = 0; j < Math.min(m, n); ++j) {
+      const previous = [q, r];
+      [q, r] = ENGINE.tidy(() => {
+        const column = ops.slice(r, [j, j], [m - j, 1]);
+        const length = ops.norm(column);
+        const head = ops.slice(r, [j, j], [1, 1]);
+        const s = ops.where(ops.greater(head, scalar(0)), ops.tensor2d([-1], [1, 1]), ops.tensor2d([1], [1, 1]));
+        const u1 = ops.sub(head, ops.mul(s, length));
+        const scaled = ops.div(column, u1);
+        const w = m - j === 1 ? ops.clone(one) : ops.concat([one, ops.slice(scaled, [1, 0], [m - j - 1, 1])], 0);
+        const tau = ops.neg(ops.div(ops.matMul(s, u1), length));
+        const tauW = ops.mul(tau, w);
+        const below = ops.slice(r, [j, 0], [m - j, n]);
+        const reflected = ops.sub(below, ops.matMul(tauW, ops.matMul(w, below, true, false)));
+        const nextR = j === 0 ? reflected : ops.concat([ops.slice(r, [0, 0], [j, n]), reflected], 0);
+        const right = ops.slice(q, [0, j], [m, m - j]);
+        const rotated = ops.sub(right, ops.matMul(ops.matMul(right, w), tauW, false, true));
+        const nextQ = j === 0 ? rotated : ops.concat([ops.slice(q, [0, 0], [m, j]), rotated], 1);
+        return [nextQ, nextR];
+      });
+      previous.forEach(t => t.dispose());
+    }
+    if (!fullMatrices && m > n) {
+      q = ops.slice(q, [0, 0], [m, n]);
+      r = ops.slice(r, [0, 0], [n, n]);
+    }
+    return [q, r];
+  });
+}
+const qr = op('qr', (x, fullMatrices) => {
+  if (x.rank < 2) throw new Error(`qr() requires input tensor to have a rank >= 2, but got rank ${x.rank}`);
+  if (x.rank === 2) return qr2d(x, !!fullMatrices);
+  // leading dimensions are a batch of matrices
+  const rows = x.shape[x.rank - 2], cols = x.shape[x.rank - 1];
+  const outer = x.shape.slice(0, -2);
+  const parts = ops.unstack(reshape(x, [util.sizeFromShape(outer), rows, cols]), 0).map(m2 => qr2d(m2, !!fullMatrices));
+  const q = ops.stack(parts.map(p => p[0]), 0), r = ops.stack(parts.map(p => p[1]), 0);
+  return [reshape(q, outer.concat(q.shape.slice(1))), reshape(r, outer.concat(r.shape.slice(1)))];
+});
+
 const gramSchmidt = op('gramSchmidt', xs => {
   const inputIsTensor2D = !Array.isArray(xs);
   let vectors;
@@ -485,8 +580,8 @@ const gramSchmidt = op('gramSchmidt', xs => {
 
 module.exports = Object.assign({}, strictOps, aliases, {
   signal: {hannWindow, hammingWindow, frame},
-  linalg: {gramSchmidt},
-  logicalXor, range, eye, outerProduct, dot, conv1d, conv3d, maxPool3d, avgPool3d, movingAverage, basicLSTMCell, multiRNNCell,
+  linalg: {gramSchmidt, qr},
+  logicalXor, range, eye, outerProduct, dot, conv1d, conv3d, conv3dTranspose, maxPool3d, avgPool3d, randomGamma, movingAverage, basicLSTMCell, multiRNNCell,
   rand, randomNormal, truncatedNormal, randomUniform, dropout, Reduction,
   math: {confusionMatrix},
   losses: {computeWeightedLoss, absoluteDifference, meanSquaredError, cosineDistance, hingeLoss, logLoss,
