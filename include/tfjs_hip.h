@@ -307,6 +307,10 @@ enum { TFHIP_SCATTER_SUM = 1, TFHIP_SCATTER_SKIP_INVALID = 2, TFHIP_SCATTER_WIDE
 int tfhip_scatter_nd(tfhip_ctx* ctx, int64_t indices, int64_t updates, int64_t out,
                      const int32_t* out_shape, int rank, int64_t num_updates, int slice_rank,
                      double default_value, int flags);
+/* fft / ifft (backend.ts:618-622; backend_cpu.ts:3343-3467): x and out are float32 buffers
+ * holding batch rows of n interleaved (real, imaginary) pairs, which is how the host keeps a
+ * complex64 tensor; inverse = 1 changes the sign of the exponent and divides by n. */
+int tfhip_fft(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t batch, int64_t n, int inverse);
 /* cropAndResize (backend.ts:612-616; backend_cpu.ts:3622-3757): images [batch,h,w,c]; boxes
  * [num_boxes,4] float32 rows (y1,x1,y2,x2) in normalised coordinates; box_index [num_boxes]
  * int32; out [num_boxes,crop_h,crop_w,c] float32.  Samples outside the image get

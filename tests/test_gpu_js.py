@@ -1107,3 +1107,48 @@ def test_js_conv3d_and_pool3d(tmp_path):
     results = c.run()
     c.check(results)
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
+def test_js_complex_and_spectral(tmp_path):
+    """tf.complex / real / imag, fft, ifft, rfft, irfft and signal.stft through the JS host:
+    the literals of spectral_ops_test.ts and signal_ops_test.ts, and numpy.fft on seeded rows of
+    power-of-two, odd and prime lengths."""
+    rng = np.random.default_rng(107)
+    c = Cases(tmp_path)
+    f32 = lambda a: np.asarray(a, np.float32)
+    pairs = lambda z: np.stack([z.real, z.imag], -1)
+    # spectral_ops_test.ts: 1D FFT of 1+1i, 2+1i -> 3+2i, -1+0i;  of (1, 2, 3) -> 6, -1.5 +- 0.866i
+    c.add("fft_2", "spectral", dict(re=f32([1, 2]), im=f32([1, 1])), dict(fn="fft"), f32([[3, 2], [-1, 0]]))
+    c.add("fft_3", "spectral", dict(re=f32([1, 2, 3]), im=f32([0, 0, 0])), dict(fn="fft"),
+          f32([[6, 0], [-1.5, 0.866025], [-1.5, -0.866025]]), atol=1e-5)
+    # signal_ops_test.ts: stft of ones and of 1..5, frame 3, step 1, hann window
+    c.add("stft_ones", "spectral", dict(re=f32([1, 1, 1, 1, 1])), dict(fn="stft", frameLength=3, frameStep=1),
+          f32([1.0, 0.0, 0.0, -1.0, -1.0, 0.0] * 3).reshape(3, 3, 2), atol=1e-5)
+    c.add("stft_seq", "spectral", dict(re=f32([1, 2, 3, 4, 5])), dict(fn="stft", frameLength=3, frameStep=1),
+          f32([2.0, 0.0, 0.0, -2.0, -2.0, 0.0, 3.0, 0.0, 0.0, -3.0, -3.0, 0.0, 4.0, 0.0, 0.0, -4.0, -4.0, 0.0]).reshape(3, 3, 2),
+          atol=1e-5)
+    for n in (1, 8, 15, 64, 127, 1024):
+        re, im = rng.standard_normal((5, n)).astype(np.float32), rng.standard_normal((5, n)).astype(np.float32)
+        z = re.astype(np.float64) + 1j * im
+        tol = dict(rtol=1e-4, atol=1e-5 * max(1.0, n ** 0.5))
+        c.add("fft_%d" % n, "spectral", dict(re=re, im=im), dict(fn="fft"), pairs(np.fft.fft(z)), **tol)
+        c.add("ifft_%d" % n, "spectral", dict(re=re, im=im), dict(fn="ifft"), pairs(np.fft.ifft(z)), **tol)
+    sig = rng.standard_normal((3, 4, 50)).astype(np.float32)
+    for fft_len in (None, 32, 64):
+        c.add("rfft_%s" % fft_len, "spectral", dict(re=sig), dict(fn="rfft", fftLength=fft_len),
+              pairs(np.fft.rfft(sig.astype(np.float64), fft_len)), atol=1e-4)
+    half = np.fft.rfft(rng.standard_normal((6, 40)))
+    c.add("irfft", "spectral", dict(re=f32(half.real), im=f32(half.imag)), dict(fn="irfft"),
+          np.fft.irfft(f32(half.real).astype(np.float64) + 1j * f32(half.imag)), atol=1e-5)
+    re, im = rng.standard_normal((4, 9)).astype(np.float32), rng.standard_normal((4, 9)).astype(np.float32)
+    c.add("complex_abs", "spectral", dict(re=re, im=im), dict(fn="abs"), np.hypot(re.astype(np.float64), im), atol=1e-6)
+    c.add("complex_interleaved", "spectral", dict(re=re, im=im), dict(fn="interleaved"), np.stack([re, im], -1).ravel(),
+          exact=True)
+    wave = rng.standard_normal(400).astype(np.float32)
+    frames = np.stack([wave[s:s + 64] for s in range(0, 400 - 64 + 1, 24)]).astype(np.float64)
+    window = 0.54 - 0.46 * np.cos(2 * np.pi * np.arange(64) / 64)      # even length: periodic form
+    c.add("stft_hamming", "spectral", dict(re=wave), dict(fn="stft", frameLength=64, frameStep=24, fftLength=128, hamming=True),
+          pairs(np.fft.rfft(frames * window, 128)), atol=1e-4)
+    results = c.run()
+    c.check(results)
+    assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0

@@ -20,7 +20,7 @@ ADDON = os.path.join(HERE, "js", "tfjs_hip.node")
 NODE_INCLUDE = "/usr/include/node"
 
 HIP_SOURCES = ["context.hip", "gemm.hip", "image.hip", "elementwise.hip", "reduce.hip",
-               "shape_ops.hip", "backward.hip", "indexing.hip"]
+               "shape_ops.hip", "backward.hip", "indexing.hip", "spectral.hip"]
 # Packed fp32 VALU ops are switched off for every kernel (scalar/float2 code only).
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC,
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

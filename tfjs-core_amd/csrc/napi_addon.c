@@ -369,6 +369,14 @@ static napi_value js_resize_nearest_backprop(napi_env env, napi_callback_info in
   return undefined(env);
 }
 
+/* fft(ctx, x, out, batch, n, inverse) */
+static napi_value js_fft(napi_env env, napi_callback_info info) {
+  ARGS(6);
+  I64(1, x); I64(2, out); I64(3, batch); I64(4, n); INT(5, inverse);
+  CHECK(tfhip_fft(ctx, x, out, batch, n, inverse));
+  return undefined(env);
+}
+
 /* graphBegin(ctx), graphEnd(ctx) -> id, graphLaunch(ctx, id), graphDestroy(ctx, id) */
 static napi_value js_graph_begin(napi_env env, napi_callback_info info) {
   ARGS(1);
@@ -662,7 +670,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"graphDestroy", js_graph_destroy}, {"topk", js_topk}, {"gatherNd", js_gather_nd},
       {"scatterNd", js_scatter_nd}, {"cropAndResize", js_crop_and_resize},
       {"resizeBilinearBackprop", js_resize_bilinear_backprop},
-      {"resizeNearestBackprop", js_resize_nearest_backprop}};
+      {"resizeNearestBackprop", js_resize_nearest_backprop}, {"fft", js_fft}};
   for (size_t i = 0; i < sizeof fns / sizeof fns[0]; i++) {
     napi_value f;
     if (napi_create_function(env, fns[i].name, NAPI_AUTO_LENGTH, fns[i].fn, NULL, &f) != napi_ok ||

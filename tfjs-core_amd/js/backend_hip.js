@@ -77,11 +77,14 @@ class MathBackendHIP extends KernelBackend {
   // ---- storage (backend.ts:33-44; CPU behaviour backend_cpu.ts:102-129, 199-254) ----
   register(dataId, shape, dtype) {
     if (this.data.has(dataId)) throw new Error('Data buffer is already registered');
-    const code = DTYPE[dtype];
+    // a complex64 tensor is a float32 buffer of interleaved (real, imaginary) pairs
+    const complex = dtype === 'complex64';
+    const code = complex ? DTYPE.float32 : DTYPE[dtype];
     if (code == null) throw new Error(`hip backend: dtype ${dtype} is not supported`);
     const handle = this.nextHandle++;
-    this.napi.register(this.ctx, handle, Int32Array.from(shape), code);
-    this.data.set(dataId, {handle, code, size: util.sizeFromShape(shape)});
+    const stored = complex ? shape.concat([2]) : shape;
+    this.napi.register(this.ctx, handle, Int32Array.from(stored), code);
+    this.data.set(dataId, {handle, code, size: util.sizeFromShape(stored)});
   }
 
   write(dataId, values) {
@@ -914,6 +917,34 @@ class MathBackendHIP extends KernelBackend {
     const count = windowSums(this.fill(x.shape, 1, 'float32'));
     return this.reshape(this.realDivide(total, count), ci.outShape);
   }
+
+  // ---- complex numbers and Fourier transforms (backend.ts:618-640) ----
+  complex(real, imag) {
+    const out = this.out(real.shape, 'complex64');
+    const n = real.size;
+    if (n > 0) {
+      this.boxCopy(this.materialized(this.cast(real, 'float32')), out, [n], [1], 0, [2], 0);
+      this.boxCopy(this.materialized(this.cast(imag, 'float32')), out, [n], [1], 0, [2], 1);
+    }
+    return out;
+  }
+  complexPart(x, offset) {
+    const out = this.out(x.shape, 'float32');
+    if (x.size > 0) this.boxCopy(x, out, [x.size], [2], offset, [1], 0);
+    return out;
+  }
+  real(x) { return this.complexPart(x, 0); }
+  imag(x) { return this.complexPart(x, 1); }
+  complexAbs(x) {
+    return this.sqrt(this.add(this.square(this.real(x)), this.square(this.imag(x))));
+  }
+  fourier(x, inverse) {
+    const out = this.out(x.shape, 'complex64');
+    this.napi.fft(this.ctx, this.h(x), this.h(out), x.shape[0], x.shape[1], inverse);
+    return out;
+  }
+  fft(x) { return this.fourier(x, 0); }
+  ifft(x) { return this.fourier(x, 1); }
 
   // ---- host-side routines: every backend of the reference runs these on values read back ----
   fromHost(values, shape, dtype) { return Tensor.make(shape, {values}, dtype, this); }

@@ -479,6 +479,66 @@ const conv3dTranspose = op('conv3dTranspose', (x, filter, outputShape, strides, 
   return lifted ? reshape(res, res.shape.slice(1)) : res;
 });
 
+// ---- complex tensors and tf.spectral (complex_ops.ts, spectral_ops.ts) ----
+const complex = op('complex', (real, imag) => {
+  const $real = convertToTensor(real, 'real', 'complex'), $imag = convertToTensor(imag, 'imag', 'complex');
+  util.assert(util.arraysEqual($real.shape, $imag.shape),
+              () => `real and imag shapes, ${$real.shape} and ${$imag.shape}, must match in call to tf.complex().`);
+  return ENGINE.runKernel(backend => backend.complex($real, $imag), {$real, $imag});
+});
+const real = op('real', input => {
+  const $input = convertToTensor(input, 'input', 'real');
+  return ENGINE.runKernel(backend => backend.real($input), {$input});
+});
+const imag = op('imag', input => {
+  const $input = convertToTensor(input, 'input', 'imag');
+  return ENGINE.runKernel(backend => backend.imag($input), {$input});
+});
+const transform = (name, method) => op(name, input => {
+  util.assert(input.dtype === 'complex64',
+              () => `The dtype for tf.spectral.${name}() must be complex64 but got ${input.dtype}.`);
+  const inner = input.shape[input.shape.length - 1];
+  const input2D = reshape(input, [input.size / inner, inner]);
+  const ret = ENGINE.runKernel(backend => backend[method](input2D), {input});
+  return reshape(ret, input.shape);
+});
+const fft = transform('fft', 'fft'), ifft = transform('ifft', 'ifft');
+// the non-negative-frequency half of the transform of a real signal, cut or zero-padded to fftLength
+const rfft = op('rfft', (input, fftLength) => {
+  util.assert(input.dtype === 'float32', () => `The dtype for rfft() must be real value but got ${input.dtype}`);
+  const last = input.rank - 1;
+  let inner = input.shape[last], adjusted = input;
+  if (fftLength != null && fftLength < inner) {
+    const size = input.shape.slice();
+    size[last] = fftLength;
+    adjusted = ops.slice(input, input.shape.map(() => 0), size);
+    inner = fftLength;
+  } else if (fftLength != null && fftLength > inner) {
+    const zerosShape = input.shape.slice();
+    zerosShape[last] = fftLength - inner;
+    adjusted = ops.concat([input, ops.zeros(zerosShape)], last);
+    inner = fftLength;
+  }
+  const batch = adjusted.size / inner;
+  const ret = fft(reshape(complex(adjusted, ops.zerosLike(adjusted)), [batch, inner]));
+  const half = Math.floor(inner / 2) + 1;
+  const outputShape = adjusted.shape.slice();
+  outputShape[last] = half;
+  const keep = t => ops.slice(t, [0, 0], [batch, half]);
+  return reshape(complex(keep(real(ret)), keep(imag(ret))), outputShape);
+});
+// inverse of rfft: the missing half is the mirrored complex conjugate
+const irfft = op('irfft', input => {
+  const inner = input.shape[input.shape.length - 1];
+  const batch = input.size / inner;
+  if (inner <= 2) return real(ifft(reshape(input, [batch, inner])));
+  const re = reshape(real(input), [batch, inner]), im = reshape(imag(input), [batch, inner]);
+  const mirror = t => ops.reverse(ops.slice(t, [0, 1], [batch, inner - 2]), 1);
+  const full = complex(ops.concat([re, mirror(re)], 1), ops.concat([im, ops.neg(mirror(im))], 1));
+  return real(ifft(full));
+});
+const enclosingPowerOfTwo = value => Math.floor(Math.pow(2, Math.ceil(Math.log(value) / Math.log(2.0))));
+
 // ---- tf.signal windows and framing (signal_ops.ts), tf.linalg.gramSchmidt (linalg_ops.ts:64-111) ----
 function cosineWindow(windowLength, a, b) {
   const even = 1 - windowLength % 2;
@@ -553,6 +613,14 @@ const qr = op('qr', (x, fullMatrices) => {
   return [reshape(q, outer.concat(q.shape.slice(1))), reshape(r, outer.concat(r.shape.slice(1)))];
 });
 
+// signal_ops.ts (stft): windowed frames, each transformed with rfft
+const stft = op('stft', (signal, frameLength, frameStep, fftLength, windowFn) => {
+  if (fftLength == null) fftLength = enclosingPowerOfTwo(frameLength);
+  if (windowFn == null) windowFn = hannWindow;
+  const framed = frame(signal, frameLength, frameStep);
+  return rfft(ops.mul(framed, windowFn(frameLength)), fftLength);
+});
+
 const gramSchmidt = op('gramSchmidt', xs => {
   const inputIsTensor2D = !Array.isArray(xs);
   let vectors;
@@ -579,7 +647,9 @@ const gramSchmidt = op('gramSchmidt', xs => {
 });
 
 module.exports = Object.assign({}, strictOps, aliases, {
-  signal: {hannWindow, hammingWindow, frame},
+  signal: {hannWindow, hammingWindow, frame, stft},
+  spectral: {fft, ifft, rfft, irfft},
+  complex, real, imag, fft, ifft, rfft, irfft, stft,
   linalg: {gramSchmidt, qr},
   logicalXor, range, eye, outerProduct, dot, conv1d, conv3d, conv3dTranspose, maxPool3d, avgPool3d, randomGamma, movingAverage, basicLSTMCell, multiRNNCell,
   rand, randomNormal, truncatedNormal, randomUniform, dropout, Reduction,

@@ -149,6 +149,20 @@ const OPS = {
     return out;
   },
   gradConv3d: (i, a) => tf.grads((x, w) => tf.conv3d(x, w, a.strides, a.pad))([i.x, i.w], i.dy)[a.wrt],
+  // complex results come back as a float32 tensor with a trailing (real, imaginary) axis
+  spectral: (i, a) => {
+    const pairs = z => tf.stack([tf.real(z), tf.imag(z)], -1);
+    if (a.fn === 'fft' || a.fn === 'ifft') return pairs(tf.spectral[a.fn](tf.complex(i.re, i.im)));
+    if (a.fn === 'rfft') return pairs(tf.spectral.rfft(i.re, a.fftLength));
+    if (a.fn === 'irfft') return tf.spectral.irfft(tf.complex(i.re, i.im));
+    if (a.fn === 'stft') return pairs(tf.signal.stft(i.re, a.frameLength, a.frameStep, a.fftLength, a.hamming ? tf.signal.hammingWindow : undefined));
+    if (a.fn === 'abs') return tf.backend().complexAbs(tf.complex(i.re, i.im));
+    if (a.fn === 'interleaved') {   // what dataSync returns for a complex tensor
+      const z = tf.complex(i.re, i.im);
+      return tf.tensor1d(z.dataSync());
+    }
+    throw new Error('unknown spectral case ' + a.fn);
+  },
   gatherND: i => tf.gatherND(i.x, i.indices),
   scatterND: (i, a) => tf.scatterND(i.indices, i.updates, a.shape),
   sparseToDense: (i, a) => tf.sparseToDense(i.indices, i.values, a.shape, a.defaultValue),

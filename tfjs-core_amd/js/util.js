@@ -103,6 +103,7 @@ function toTypedArray(a, dtype) {
 function bytesPerElement(dtype) {
   if (dtype === 'float32' || dtype === 'int32') return 4;
   if (dtype === 'bool') return 1;
+  if (dtype === 'complex64') return 8;
   throw new Error(`Unknown dtype ${dtype}`);
 }
 

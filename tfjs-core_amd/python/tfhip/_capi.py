@@ -58,6 +58,7 @@ _SIGNATURES = {
     "tfhip_pool2d": [_PTR, _I64, _I64, C.POINTER(Conv2DInfoC), _INT],
     "tfhip_resize_nearest": [_PTR, _I64, _I64, _INT, _INT, _INT, _INT, _INT, _INT, _INT],
     "tfhip_select": [_PTR, _I64, _I64, _I64, _I64, _I64],
+    "tfhip_fft": [_PTR, _I64, _I64, _I64, _I64, _INT],
     "tfhip_gather_nd": [_PTR, _I64, _I64, _I64, C.POINTER(C.c_int32), _INT, _I64, _INT],
     "tfhip_scatter_nd": [_PTR, _I64, _I64, _I64, C.POINTER(C.c_int32), _INT, _I64, _INT, C.c_double, _INT],
     "tfhip_crop_and_resize": [_PTR, _I64, _I64, _I64, _I64, _INT, _INT, _INT, _INT, _I64, _INT, _INT, _INT,
