@@ -1102,6 +1102,37 @@ def test_js_conv3d_and_pool3d(tmp_path):
                         max(0, 2 * q - pl):2 * q - pl + 3].astype(np.float64)
                 mx[:, z, r, q] = win.max((1, 2, 3))
                 av[:, z, r, q] = win.mean((1, 2, 3))
+    # their gradients: dy to the first maximum of each window (depth, row, column order), or
+    # dy / 27 to every element of the window inside the volume
+    v[0, 1:4, 2:5, 3:6, 0] = 9.0                              # ties: a block of equal maxima
+    dyp = rng.standard_normal((2, od, oh, ow, 3)).astype(np.float32)
+    dmx, dav = np.zeros(v.shape), np.zeros(v.shape)
+    for z in range(od):
+        for r in range(oh):
+            for q in range(ow):
+                z0, r0, q0 = max(0, 2 * z - pf), max(0, 2 * r - pt), max(0, 2 * q - pl)
+                win = v[:, z0:2 * z - pf + 3, r0:2 * r - pt + 3, q0:2 * q - pl + 3]
+                dav[:, z0:2 * z - pf + 3, r0:2 * r - pt + 3, q0:2 * q - pl + 3] += dyp[:, z, r, q][:, None, None, None] / 27.0
+                flat = win.reshape(2, -1, 3)
+                first = flat.argmax(1)                        # numpy's argmax returns the first maximum
+                for b in range(2):
+                    for ch in range(3):
+                        dz, dr, dq = np.unravel_index(first[b, ch], win.shape[1:4])
+                        dmx[b, z0 + dz, r0 + dr, q0 + dq, ch] += dyp[b, z, r, q, ch]
+    for z in range(od):                                      # the forward maxima after the edit above
+        for r in range(oh):
+            for q in range(ow):
+                mx[:, z, r, q] = v[:, max(0, 2 * z - pf):2 * z - pf + 3, max(0, 2 * r - pt):2 * r - pt + 3,
+                                   max(0, 2 * q - pl):2 * q - pl + 3].max((1, 2, 3))
+                av[:, z, r, q] = v[:, max(0, 2 * z - pf):2 * z - pf + 3, max(0, 2 * r - pt):2 * r - pt + 3,
+                                   max(0, 2 * q - pl):2 * q - pl + 3].astype(np.float64).mean((1, 2, 3))
+    grad_attrs = dict(filterSize=3, strides=2, pad="same")
+    c.add("max_pool3d_grad", "gradPool3d", dict(x=v, dy=dyp), dict(fn="maxPool3d", **grad_attrs), dmx, atol=1e-5)
+    c.add("avg_pool3d_grad", "gradPool3d", dict(x=v, dy=dyp), dict(fn="avgPool3d", **grad_attrs), dav, atol=1e-5)
+    # pool_test.ts: maxPool3d(x, 2, 1, 0) of 1..8 sends dy = 1 to the last element
+    c.add("max_pool3d_grad_literal", "gradPool3d", dict(x=np.arange(1, 9, dtype=np.float32).reshape(1, 2, 2, 2, 1),
+                                                        dy=np.ones((1, 1, 1, 1, 1), np.float32)),
+          dict(fn="maxPool3d", filterSize=2, strides=1, pad=0), np.asarray([0, 0, 0, 0, 0, 0, 0, 1], np.float32).reshape(1, 2, 2, 2, 1))
     c.add("max_pool3d_seeded", "call", dict(x=v), dict(fn="maxPool3d", args=["$x", 3, 2, "same"]), mx, exact=True)
     c.add("avg_pool3d_seeded", "call", dict(x=v), dict(fn="avgPool3d", args=["$x", 3, 2, "same"]), av, atol=1e-5)
     results = c.run()

@@ -874,20 +874,8 @@ class MathBackendHIP extends KernelBackend {
   conv3dDerInput(dy, filter, ci) {
     const info = this.info2dOf(ci);
     const dy4 = this.reshape(dy, info.outShape);
-    const need = (ci.outDepth - 1) * ci.strideDepth + ci.effectiveFilterDepth;
-    const front = Math.max(ci.padInfo.front, 0);
-    const depth = Math.max(need, front + ci.inDepth);
-    const plane = ci.inHeight * ci.inWidth * ci.inChannels;
-    let acc = null;
-    for (let kd = 0; kd < ci.filterDepth; kd++) {
-      const dx4 = this.conv2dDerInput(dy4, this.filterTap(filter, ci, kd), info);
-      // plane od of this tap belongs to padded depth kd * dd + od * sd
-      const spread = this.fill([ci.batchSize, depth, ci.inHeight, ci.inWidth, ci.inChannels], 0, 'float32');
-      this.boxCopy(dx4, spread, [ci.batchSize, ci.outDepth, plane], [ci.outDepth * plane, plane, 1], 0,
-                   [depth * plane, ci.strideDepth * plane, 1], kd * ci.dilationDepth * plane);
-      acc = acc == null ? spread : this.add(acc, spread);
-    }
-    return this.slice(acc, [0, front, 0, 0, 0], ci.inShape);
+    // plane od of tap kd belongs to padded depth kd * dd + od * sd
+    return this.spreadTaps(ci, kd => this.conv2dDerInput(dy4, this.filterTap(filter, ci, kd), info));
   }
   maxPool3d(x, ci) {
     const xp = this.depthPadded(x, ci, -Infinity), info = this.info2dOf(ci);
@@ -916,6 +904,50 @@ class MathBackendHIP extends KernelBackend {
     const total = windowSums(this.cast(x, 'float32'));
     const count = windowSums(this.fill(x.shape, 1, 'float32'));
     return this.reshape(this.realDivide(total, count), ci.outShape);
+  }
+
+  // per-tap gradients [batch * outDepth, h, w, c] spread onto their depth planes and summed
+  spreadTaps(ci, tapGradient) {
+    const need = (ci.outDepth - 1) * ci.strideDepth + ci.effectiveFilterDepth;
+    const front = Math.max(ci.padInfo.front, 0);
+    const depth = Math.max(need, front + ci.inDepth);
+    const plane = ci.inHeight * ci.inWidth * ci.inChannels;
+    let acc = null;
+    for (let kd = 0; kd < ci.filterDepth; kd++) {
+      const spread = this.fill([ci.batchSize, depth, ci.inHeight, ci.inWidth, ci.inChannels], 0, 'float32');
+      this.boxCopy(tapGradient(kd), spread, [ci.batchSize, ci.outDepth, plane], [ci.outDepth * plane, plane, 1], 0,
+                   [depth * plane, ci.strideDepth * plane, 1], kd * ci.dilationDepth * plane);
+      acc = acc == null ? spread : this.add(acc, spread);
+    }
+    return this.slice(acc, [0, front, 0, 0, 0], ci.inShape);
+  }
+  // backend_cpu.ts:2583-2665: every window hands dy / (fd * fh * fw) to each of its elements
+  avgPool3dBackprop(dy, x, ci) {
+    const info = this.info2dOf(ci);
+    const dy4 = this.reshape(this.multiply(dy, this.fill([1], 1 / ci.filterDepth, 'float32')), info.outShape);
+    // the 2-D average rule reads only the shape of its second operand
+    const perTap = this.backward('pool2dBackprop', dy4, this.fill(info.inShape, 0, 'float32'), info.inShape, info,
+                                 POOL.avg);
+    return this.spreadTaps(ci, () => perTap);
+  }
+  // backend_cpu.ts:2667-2867: dy goes to the first maximum of each window in (depth, row, column)
+  // order: the first depth tap whose plane maximum equals the window maximum y, and inside that
+  // plane the 2-D rule
+  maxPool3dBackprop(dy, x, y, ci) {
+    const info = this.info2dOf(ci);
+    const xp = this.depthPadded(x, ci, -Infinity);
+    const y4 = this.reshape(y, info.outShape), dy4 = this.reshape(dy, info.outShape);
+    const zeros = this.fill(info.outShape, 0, 'float32');
+    let taken = null;
+    const taps = [];
+    for (let kd = 0; kd < ci.filterDepth; kd++) {
+      const planes = this.tapPlanes(xp, ci, kd);
+      let wins = this.equal(this.maxPool(planes, info), y4);
+      if (taken != null) wins = this.logicalAnd(wins, this.logicalNot(taken));
+      taken = taken == null ? wins : this.logicalOr(taken, wins);
+      taps.push(this.backward('pool2dBackprop', this.select(wins, dy4, zeros), planes, planes.shape, info, POOL.max));
+    }
+    return this.spreadTaps(ci, kd => taps[kd]);
   }
 
   // ---- complex numbers and Fourier transforms (backend.ts:618-640) ----

@@ -456,7 +456,14 @@ const pool3d = (name, method) => op(name, (x, filterSize, strides, pad, dimRound
   }
   util.assert(conv_util.tupleValuesAreOne(dilations), () => `Error in ${name}: the hip backend pools 3-D windows without dilation`);
   const ci = conv_util.computePool3DInfo(x5D.shape, filterSize, strides, dilations, pad, dimRoundingMode, dataFormat);
-  let res = ENGINE.runKernel(backend => backend[method](x5D, ci), {x: x5D});
+  let res = ENGINE.runKernel((backend, save) => {
+    const y = backend[method](x5D, ci);
+    save([x5D, y]);
+    return y;
+  }, {x: x5D}, (dy, saved) => ({
+    x: () => ENGINE.runKernel(backend => method === 'avgPool3d' ?
+        backend.avgPool3dBackprop(dy, saved[0], ci) : backend.maxPool3dBackprop(dy, saved[0], saved[1], ci), {})
+  }));
   if (method === 'avgPool3d') res = cast(res, x5D.dtype);
   return lifted ? reshape(res, res.shape.slice(1)) : res;
 });

@@ -163,6 +163,7 @@ const OPS = {
     }
     throw new Error('unknown spectral case ' + a.fn);
   },
+  gradPool3d: (i, a) => tf.grad(x => tf[a.fn](x, a.filterSize, a.strides, a.pad))(i.x, i.dy),
   gatherND: i => tf.gatherND(i.x, i.indices),
   scatterND: (i, a) => tf.scatterND(i.indices, i.updates, a.shape),
   sparseToDense: (i, a) => tf.sparseToDense(i.indices, i.values, a.shape, a.defaultValue),
