@@ -678,6 +678,85 @@ test('loadWeightsFromDisk: manifest next to its shard files', async () => {
   });
 });
 
+// conv_util_test.ts:271-520, 834-979: output sizes and paddings of 3-D convolutions and pools
+test('computeConv3DInfo / computePool3DInfo (conv_util_test.ts:271-520, 834-979)', () => {
+  const conv_util = require('../conv_util.js');
+  let ci = conv_util.computeConv3DInfo([1, 3, 3, 3, 1], [2, 2, 2, 1, 1], 1, 1, 'same');
+  assert.deepStrictEqual([ci.outDepth, ci.outHeight, ci.outWidth, ci.outChannels], [3, 3, 3, 1]);
+  assert.deepStrictEqual([ci.padInfo.front, ci.padInfo.back, ci.padInfo.left, ci.padInfo.right, ci.padInfo.top,
+                          ci.padInfo.bottom], [0, 1, 0, 1, 0, 1]);
+  ci = conv_util.computeConv3DInfo([1, 3, 3, 3, 1], [2, 2, 2, 1, 1], 1, 1, 'valid');
+  assert.deepStrictEqual([ci.outDepth, ci.outHeight, ci.outWidth], [2, 2, 2]);
+  ci = conv_util.computeConv3DInfo([1, 5, 5, 5, 1], [3, 3, 3, 1, 1], 2, 1, 'same');
+  assert.deepStrictEqual([ci.outDepth, ci.outHeight, ci.outWidth], [3, 3, 3]);
+  assert.deepStrictEqual([ci.padInfo.front, ci.padInfo.back, ci.padInfo.top, ci.padInfo.bottom], [1, 1, 1, 1]);
+  // a dilated 3 x 3 x 3 filter acts like a 5 x 5 x 5 one
+  ci = conv_util.computeConv3DInfo([1, 9, 9, 9, 2], [3, 3, 3, 2, 7], 1, 2, 'valid');
+  assert.deepStrictEqual([ci.effectiveFilterDepth, ci.outDepth, ci.outHeight, ci.outWidth, ci.outChannels],
+                         [5, 5, 5, 5, 7]);
+  // per-dimension strides; a numeric pad sizes every dimension from the filter depth and depth stride
+  ci = conv_util.computeConv3DInfo([2, 8, 6, 4, 1], [2, 3, 1, 1, 4], [2, 3, 1], 1, 'same');
+  assert.deepStrictEqual(ci.outShape, [2, 4, 2, 4, 4]);
+  ci = conv_util.computePool3DInfo([1, 2, 2, 2, 1], 2, 1, 1, 1, 'floor');
+  assert.deepStrictEqual([ci.outShape, ci.padInfo.front, ci.padInfo.type], [[1, 3, 3, 3, 1], 1, 'NUMBER']);
+  ci = conv_util.computePool3DInfo([1, 4, 4, 4, 3], [2, 2, 2], 2, 1, 'valid');
+  assert.deepStrictEqual(ci.outShape, [1, 2, 2, 2, 3]);
+  assert.throws(() => conv_util.computeConv3DInfo([1, 3, 3, 3, 1], [2, 2, 2, 1, 1], 1, 1, 'diagonal'), /Unknown padding/);
+});
+
+// host-side generators: they need a backend only to hold their values
+test('range, windows, seeded random tensors, losses over a host backend', async () => {
+  await withBackend('arith-extra', new ArithBackend(), async () => {
+    const before = tf.memory().numTensors;
+    tf.tidy(() => {
+      // array_ops_test.ts (range): sign of the step adjusted, empty for incompatible steps, dtype
+      assert.deepStrictEqual(Array.from(tf.range(0, 3).dataSync()), [0, 1, 2]);
+      assert.deepStrictEqual(Array.from(tf.range(4, -2).dataSync()), [4, 3, 2, 1, 0, -1]);
+      assert.deepStrictEqual(Array.from(tf.range(4, 15, 4).dataSync()), [4, 8, 12]);
+      assert.deepStrictEqual(tf.range(3, 3).shape, [0]);
+      assert.deepStrictEqual(tf.range(5, 1, 2).shape, [0]);
+      assert.strictEqual(tf.range(1, 4, 1, 'int32').dtype, 'int32');
+      assert.throws(() => tf.range(0, 3, 0), /step of zero/);
+      // signal_ops_test.ts: hann and hamming windows
+      closeTo(tf.signal.hannWindow(7).dataSync(), [0, 0.25, 0.75, 1, 0.75, 0.25, 0], 1e-6);
+      closeTo(tf.signal.hannWindow(6).dataSync(), [0, 0.25, 0.75, 1, 0.75, 0.25], 1e-6);
+      closeTo(tf.signal.hammingWindow(7).dataSync(), [0.08, 0.31, 0.77, 1, 0.77, 0.31, 0.08], 1e-6);
+      // Alea: a seed fixes the stream, different seeds differ, values lie in [0, 1)
+      const {alea} = require('../alea.js');
+      const a = alea('7'), b = alea('7'), c = alea('8');
+      const first = [a(), a(), a()];
+      assert.deepStrictEqual(first, [b(), b(), b()]);
+      assert.notDeepStrictEqual(first, [c(), c(), c()]);
+      for (let i = 0; i < 1000; i++) {
+        const v = a();
+        assert.ok(v >= 0 && v < 1);
+      }
+      const u = tf.randomUniform([4000], -1, 3, 'float32', 5).dataSync();
+      assert.deepStrictEqual(Array.from(u), Array.from(tf.randomUniform([4000], -1, 3, 'float32', 5).dataSync()));
+      const mean = u.reduce((p, q) => p + q, 0) / u.length;
+      assert.ok(Math.abs(mean - 1) < 0.1 && Math.min(...u) >= -1 && Math.max(...u) < 3);
+      const t = tf.truncatedNormal([4000], 2, 0.5, 'float32', 9).dataSync();
+      assert.ok(Math.min(...t) >= 1 && Math.max(...t) <= 3);
+      assert.throws(() => tf.randomUniform([4], 0, 1, 'int32', 1), /<= 1 and dtype is not float/);
+      const g = tf.randomGamma([4000], 2, 3, 'float32', 3).dataSync();
+      assert.ok(Math.abs(g.reduce((p, q) => p + q, 0) / g.length - 6) < 0.4 && Math.min(...g) > 0);
+      // loss_ops_test.ts: |l - p| with weights under the four reductions
+      const l = tf.tensor1d([1, 2, 3, 4]), p = tf.tensor1d([0.5, 2.5, 1, 4]), w = tf.tensor1d([1, 0, 2, 0.5]);
+      const R = tf.Reduction;
+      closeTo(tf.losses.absoluteDifference(l, p, w, R.NONE).dataSync(), [0.5, 0, 4, 0]);
+      closeTo(tf.losses.absoluteDifference(l, p, w, R.SUM).dataSync(), [4.5]);
+      closeTo(tf.losses.absoluteDifference(l, p, w, R.MEAN).dataSync(), [4.5 / 3.5]);
+      closeTo(tf.losses.absoluteDifference(l, p).dataSync(), [3 / 4]);
+      closeTo(tf.losses.hingeLoss(tf.tensor1d([0, 1, 1, 0]), tf.tensor1d([0.3, 0.7, -0.2, -1.5]), undefined, R.NONE).dataSync(),
+              [1.3, 0.3, 1.2, 0]);
+      assert.throws(() => tf.losses.absoluteDifference(l, tf.tensor1d([1, 2])), /must match/);
+      assert.throws(() => tf.addStrict(l, tf.tensor1d([1, 2])), /must match/);
+      closeTo(tf.addStrict(l, p).dataSync(), [1.5, 4.5, 4, 8]);
+    });
+    assert.strictEqual(tf.memory().numTensors, before);
+  });
+});
+
 (async () => {
   let failed = 0;
   for (const t of tests) {
