@@ -989,6 +989,13 @@ def test_js_composite_surface(tmp_path, ref):
     qn, rn = np.linalg.qr(batch.astype(np.float64))
     call("qr_batched_q", "linalg.qr", dict(x=batch), ["$x"], qn, atol=1e-4, pick=0)
     call("qr_batched_r", "linalg.qr", dict(x=batch), ["$x"], rn, atol=1e-4, pick=1)
+    # in_top_k_test.ts semantics: the target is among the k largest; equal values rank by index
+    preds = rng.standard_normal((40, 25)).astype(np.float32)
+    preds[:, 3] = preds[:, 11]                                # ties
+    targets = rng.integers(0, 25, 40).astype(np.int32)
+    order = np.argsort(-preds.astype(np.float64), axis=1, kind="stable")[:, :4]
+    c.add("in_top_k", "inTopK", dict(predictions=preds, targets=targets), dict(k=4), (order == targets[:, None]).any(1),
+          exact=True)
     xd = rng.uniform(1, 2, (300, 50)).astype(np.float32)
     c.add("dropout", "dropoutStats", dict(x=xd), dict(rate=0.25, seed=5), f32([0.75, 0]), atol=1e9)
     results = c.run()

@@ -653,7 +653,126 @@ const gramSchmidt = op('gramSchmidt', xs => {
   return inputIsTensor2D ? ops.stack(ys, 0) : ys;
 });
 
+// ---- host-side containers and helpers (tensor.ts TensorBuffer :44-160, array_ops.ts buffer /
+//      print / setdiff1dAsync, in_top_k.ts, browser_util.ts nextFrame, test_util.ts) ----
+class TensorBuffer {
+  constructor(shape, dtype, values) {
+    this.dtype = dtype || 'float32';
+    this.shape = shape.slice();
+    this.size = util.sizeFromShape(shape);
+    if (values != null) {
+      util.assert(values.length === this.size,
+                  () => `Length of values '${values.length}' does not match the size inferred by the shape '${this.size}'.`);
+    }
+    if (dtype === 'complex64') {
+      throw new Error('complex64 dtype TensorBuffers are not supported. Please create a TensorBuffer for the ' +
+                      'real and imaginary parts separately and call tf.complex(real, imag).');
+    }
+    this.values = values || util.getTypedArrayFromDType(this.dtype, this.size);
+    this.strides = util.computeStrides(shape);
+  }
+  get rank() { return this.shape.length; }
+  locToIndex(locs) {
+    if (this.rank === 0) return 0;
+    if (this.rank === 1) return locs[0];
+    let index = locs[locs.length - 1];
+    for (let i = 0; i < locs.length - 1; ++i) index += this.strides[i] * locs[i];
+    return index;
+  }
+  indexToLoc(index) {
+    if (this.rank === 0) return [];
+    if (this.rank === 1) return [index];
+    const locs = new Array(this.shape.length);
+    for (let i = 0; i < locs.length - 1; ++i) {
+      locs[i] = Math.floor(index / this.strides[i]);
+      index -= locs[i] * this.strides[i];
+    }
+    locs[locs.length - 1] = index;
+    return locs;
+  }
+  checkLocs(locs) {
+    if (locs.length === 0) locs = [0];
+    util.assert(locs.length === this.rank,
+                () => `The number of provided coordinates (${locs.length}) must match the rank (${this.rank})`);
+    locs.forEach((loc, i) => {
+      if (loc < 0 || loc >= this.shape[i]) {
+        throw new Error(`Requested out of range element at ${locs}.   Buffer shape=${this.shape}`);
+      }
+    });
+    return locs;
+  }
+  set(value, ...locs) { this.values[this.locToIndex(this.checkLocs(locs))] = value; }
+  get(...locs) { return this.values[this.locToIndex(this.checkLocs(locs))]; }
+  toTensor() { return ops.tensor(this.values, this.shape, this.dtype); }
+}
+const buffer = (shape, dtype, values) => new TensorBuffer(shape, dtype || 'float32', values);
+Tensor.prototype.bufferSync = function() { return buffer(this.shape, this.dtype, this.dataSync()); };
+Tensor.prototype.buffer = async function() { return buffer(this.shape, this.dtype, await this.data()); };
+function print(x, verbose) {
+  const values = Array.from(x.dataSync());
+  const nest = (shape, offset) => {
+    if (shape.length === 0) return values[offset];
+    const step = util.sizeFromShape(shape.slice(1));
+    return Array.from({length: shape[0]}, (v, i) => nest(shape.slice(1), offset + i * step));
+  };
+  const text = JSON.stringify(nest(x.shape, 0));
+  console.log(verbose ? `Tensor\n  dtype: ${x.dtype}\n  rank: ${x.rank}\n  shape: [${x.shape}]\n  values:\n    ${text}` :
+                        `Tensor\n    ${text}`);
+}
+const tensor5d = (values, shape, dtype) => ops.tensor(values, shape, dtype);
+const tensor6d = (values, shape, dtype) => ops.tensor(values, shape, dtype);
+// the elements of x that are not in y, and where they sit in x (array_ops.ts:1031-1068)
+async function setdiff1dAsync(x, y) {
+  const $x = convertToTensor(x, 'x', 'setdiff1d'), $y = convertToTensor(y, 'y', 'setdiff1d');
+  util.assert($x.dtype === $y.dtype, () => `x and y should have the same dtype, but got x (${$x.dtype}) and y (${$y.dtype}).`);
+  util.assert($x.rank === 1, () => `x should be 1D tensor, but got x (${$x.shape}).`);
+  util.assert($y.rank === 1, () => `y should be 1D tensor, but got y (${$y.shape}).`);
+  const xVals = await $x.data(), ySet = new Set(await $y.data());
+  const kept = [];
+  xVals.forEach((v, i) => ySet.has(v) || kept.push(i));
+  return [ops.tensor(kept.map(i => xVals[i]), [kept.length], $x.dtype), ops.tensor(Int32Array.from(kept), [kept.length], 'int32')];
+}
+// whether targets[b] is among the k largest of predictions[b, :] (in_top_k.ts:35-100); the
+// selection runs on the device (equal values: the lower index first, as a stable sort gives)
+async function inTopKAsync(predictions, targets, k) {
+  if (k == null) k = 1;
+  const $predictions = convertToTensor(predictions, 'predictions', 'inTopK');
+  const $targets = convertToTensor(targets, 'targets', 'inTopK');
+  util.assert($predictions.rank > 1, () => `inTopK() expects the predictions to be of rank 2 or higher, but got ${$predictions.rank}`);
+  util.assert($predictions.rank - 1 === $targets.rank,
+              () => `predictions rank should be 1 larger than targets rank, but got predictions rank ${$predictions.rank} and targets rank ${$targets.rank}`);
+  util.assert(util.arraysEqual($predictions.shape.slice(0, -1), $targets.shape),
+              () => `predictions's shape should be align with the targets' shape, except the last dimension.`);
+  const lastDim = $predictions.shape[$predictions.rank - 1];
+  util.assert(k > 0 && k <= lastDim,
+              () => `'k' passed to inTopK() must be > 0 && <= the predictions last dimension (${lastDim}), but got ${k}`);
+  const res = ENGINE.tidy(() => {
+    const {values, indices} = ops.topk($predictions, k);
+    values.dispose();
+    return ops.any(ops.equal(indices, ops.expandDims(cast($targets, 'int32'), -1)), -1);
+  });
+  if (predictions !== $predictions) $predictions.dispose();
+  if (targets !== $targets) $targets.dispose();
+  return res;
+}
+const nextFrame = () => new Promise(resolve => setImmediate(resolve));
+// expectArraysClose of test_util.ts:22-39, 121-138 (absolute epsilon 1e-3 on a 32-bit backend)
+const test_util = {
+  expectArraysClose(actual, expected, epsilon) {
+    if (epsilon == null) epsilon = 1e-3;
+    const a = Array.from(util.flatten(actual)), e = Array.from(util.flatten(expected));
+    if (a.length !== e.length) throw new Error(`Arrays have different lengths actual: ${a.length} vs expected: ${e.length}.`);
+    a.forEach((v, i) => {
+      const ok = (isNaN(v) && isNaN(e[i])) || Math.abs(v - e[i]) <= epsilon || v === e[i];
+      if (!ok) throw new Error(`Arrays differ: actual[${i}] = ${v}, expected[${i}] = ${e[i]}.`);
+    });
+  },
+  expectArraysEqual(actual, expected) { return test_util.expectArraysClose(actual, expected, 0); }
+};
+
 module.exports = Object.assign({}, strictOps, aliases, {
+  TensorBuffer, buffer, print, tensor5d, tensor6d, setdiff1dAsync, inTopKAsync, nextFrame, test_util,
+  version_core: '1.2.7-hip',
   signal: {hannWindow, hammingWindow, frame, stft},
   spectral: {fft, ifft, rfft, irfft},
   complex, real, imag, fft, ifft, rfft, irfft, stft,

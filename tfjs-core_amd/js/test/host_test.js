@@ -752,7 +752,25 @@ test('range, windows, seeded random tensors, losses over a host backend', async 
       assert.throws(() => tf.losses.absoluteDifference(l, tf.tensor1d([1, 2])), /must match/);
       assert.throws(() => tf.addStrict(l, tf.tensor1d([1, 2])), /must match/);
       closeTo(tf.addStrict(l, p).dataSync(), [1.5, 4.5, 4, 8]);
+      // tensor.ts TensorBuffer: coordinates, bounds, round trip
+      const buf = tf.buffer([2, 3], 'int32');
+      buf.set(7, 1, 2);
+      buf.set(-1, 0, 1);
+      assert.strictEqual(buf.get(1, 2), 7);
+      assert.deepStrictEqual(buf.indexToLoc(5), [1, 2]);
+      assert.throws(() => buf.get(2, 0), /out of range/);
+      const fromBuf = buf.toTensor();
+      assert.deepStrictEqual([fromBuf.dtype, fromBuf.shape, Array.from(fromBuf.dataSync())], ['int32', [2, 3], [0, -1, 0, 0, 0, 7]]);
+      assert.strictEqual(fromBuf.bufferSync().get(0, 1), -1);
+      assert.strictEqual(tf.tensor5d([1, 2], [1, 1, 1, 1, 2]).rank, 5);
+      tf.test_util.expectArraysClose([1, NaN, 2.0005], [1, NaN, 2]);
+      assert.throws(() => tf.test_util.expectArraysClose([1], [1.1]), /differ/);
     });
+    // array_ops_test.ts (setdiff1dAsync): values of x absent from y, with their positions
+    const sx = tf.tensor1d([1, 2, 3, 4, 5, 6]), sy = tf.tensor1d([1, 3, 5]);
+    const [diff, where] = await tf.setdiff1dAsync(sx, sy);
+    assert.deepStrictEqual([Array.from(diff.dataSync()), Array.from(where.dataSync())], [[2, 4, 6], [1, 3, 5]]);
+    tf.dispose([diff, where, sx, sy]);
     assert.strictEqual(tf.memory().numTensors, before);
   });
 });

@@ -164,6 +164,7 @@ const OPS = {
     throw new Error('unknown spectral case ' + a.fn);
   },
   gradPool3d: (i, a) => tf.grad(x => tf[a.fn](x, a.filterSize, a.strides, a.pad))(i.x, i.dy),
+  inTopK: async (i, a) => tf.inTopKAsync(i.predictions, i.targets, a.k),
   gatherND: i => tf.gatherND(i.x, i.indices),
   scatterND: (i, a) => tf.scatterND(i.indices, i.updates, a.shape),
   sparseToDense: (i, a) => tf.sparseToDense(i.indices, i.values, a.shape, a.defaultValue),
@@ -298,7 +299,10 @@ async function main() {
       } else {
         const inputs = {};
         Object.keys(c.inputs).forEach(k => { inputs[k] = load(c.inputs[k]); });
-        const r = tf.tidy(() => OPS[c.op](inputs, c.attrs || {}));
+        const fn = OPS[c.op];
+        // the *Async ops resolve after a read-back and cannot run inside a tidy
+        const r = fn.constructor.name === 'AsyncFunction' ? await fn(inputs, c.attrs || {}) :
+                                                            tf.tidy(() => fn(inputs, c.attrs || {}));
         const vals = r.dataSync();
         fs.writeFileSync(path.join(dir, c.name + '.out.bin'),
                          Buffer.from(vals.buffer, vals.byteOffset, vals.byteLength));
