@@ -129,7 +129,7 @@ def roofline_of_dominant_kernel(rows):
 
 
 def op_level_configs(tf, np):
-    """Configs 1-3 of BASELINE.json (single matMul, the 3-layer MLP, one fused conv2d and one
+    """The three op-level configurations (single matMul, the 3-layer MLP, one fused conv2d and one
     depthwiseConv2D) at their full sizes: every op timed with an event pair on the backend's
     stream around back-to-back launches, priced by its algorithmic flops and bytes (operands
     and result counted once) against the fp32 matrix peak and the HBM peak."""
