@@ -55,6 +55,17 @@ __global__ void gather_rows_kernel(const T* x, const int64_t* flat, T* out, int6
   }
 }
 
+// The same copy in 16-byte pieces, for slices that are a whole number of them.
+__global__ void gather_rows_vec_kernel(const uint4* x, const int64_t* flat, uint4* out, int64_t n_slices,
+                                       int64_t slice16) {
+  const int64_t total = n_slices * slice16;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += stride) {
+    const int64_t i = g / slice16, k = g - i * slice16;
+    out[g] = x[flat[i] * slice16 + k];
+  }
+}
+
 // One lane per result element (row, k): starts from the default value and walks the updates
 // in ascending order, adding (scatterND) or overwriting (sparseToDense: the last one wins)
 // whenever an update addresses its row, which is the order backend_cpu.ts:3858-3886 applies
@@ -307,7 +318,13 @@ extern "C" int tfhip_gather_nd(tfhip_ctx* ctx, int64_t x, int64_t indices, int64
     return ctx->fail(TFHIP_EINVAL, "gatherND: input and output element sizes differ");
   if (bo->numel == 0) return TFHIP_OK;
   const dim3 grid(blocks_for(ctx, bo->numel)), block(256);
-  if (dtype_size(bx->dtype) == 4)
+  const int64_t slice_bytes = slice * (int64_t)dtype_size(bx->dtype);
+  if (slice_bytes % 16 == 0 && reinterpret_cast<uintptr_t>(bx->ptr) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(bo->ptr) % 16 == 0)
+    hipLaunchKernelGGL(gather_rows_vec_kernel, dim3(blocks_for(ctx, num_slices * (slice_bytes / 16))), block, 0,
+                       ctx->stream, (const uint4*)bx->ptr, (const int64_t*)flat.ptr, (uint4*)bo->ptr, num_slices,
+                       slice_bytes / 16);
+  else if (dtype_size(bx->dtype) == 4)
     hipLaunchKernelGGL(gather_rows_kernel<int32_t>, grid, block, 0, ctx->stream, (const int32_t*)bx->ptr,
                        (const int64_t*)flat.ptr, (int32_t*)bo->ptr, num_slices, slice);
   else
