@@ -72,20 +72,40 @@ __global__ void gather_rows_vec_kernel(const uint4* x, const int64_t* flat, uint
 // them in.  Acc = T rounds every sum to the element type as a typed array does; Acc = double
 // rounds once at the end, as the masked sums of unsortedSegmentSum do.
 template <typename T, typename Acc>
-__global__ void scatter_rows_kernel(const int64_t* flat, const T* updates, T* out, int64_t rows,
-                                    int64_t slice, int64_t n_updates, T start, int sum_dupes,
-                                    int scalar_update) {
+__global__ __launch_bounds__(256) void scatter_rows_kernel(const int64_t* flat, const T* updates, T* out,
+                                                           int64_t rows, int64_t slice, int64_t n_updates,
+                                                           T start, int sum_dupes, int scalar_update) {
+  // the index list passes through LDS 256 entries at a time: every lane of the workgroup walks
+  // the same entries, which LDS serves as broadcasts
+  __shared__ int chunk[256];  // row of each update, -2 for none (rows fit an int: checked by the host)
   const int64_t total = rows * slice;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += stride) {
-    const int64_t row = g / slice, k = g - row * slice;
+  // all lanes of a workgroup make the same number of trips, so the barriers below are uniform
+  for (int64_t base = (int64_t)blockIdx.x * blockDim.x; base < total; base += stride) {
+    const int64_t g = base + threadIdx.x;
+    const bool live = g < total;
+    const int row = live ? (int)(g / slice) : -1;
+    const int64_t k = live ? g - (int64_t)row * slice : 0;
     Acc acc = start;
-    for (int64_t i = 0; i < n_updates; i++) {
-      if (flat[i] != row) continue;
-      const T u = updates[scalar_update ? 0 : i * slice + k];
-      acc = sum_dupes ? (Acc)(acc + u) : (Acc)u;
+    for (int64_t i0 = 0; i0 < n_updates; i0 += 256) {
+      __syncthreads();
+      const int64_t f = i0 + threadIdx.x < n_updates ? flat[i0 + threadIdx.x] : -2;
+      chunk[threadIdx.x] = f >= 0 && f < rows ? (int)f : -2;
+      __syncthreads();
+      // eight entries per trip, read together so that their LDS latencies overlap
+      for (int j0 = 0; j0 < 256; j0 += 8) {
+        int c[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) c[e] = chunk[j0 + e];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          if (c[e] != row) continue;
+          const T u = updates[scalar_update ? 0 : (i0 + j0 + e) * slice + k];
+          acc = sum_dupes ? (Acc)(acc + u) : (Acc)u;
+        }
+      }
     }
-    out[g] = (T)acc;
+    if (live) out[g] = (T)acc;
   }
 }
 
@@ -356,6 +376,7 @@ extern "C" int tfhip_scatter_nd(tfhip_ctx* ctx, int64_t indices, int64_t updates
   if ((bo->dtype != TFHIP_FLOAT32 && bo->dtype != TFHIP_INT32) || bu->dtype != bo->dtype)
     return ctx->fail(TFHIP_EINVAL, "scatterND: updates and result must both be float32 or both int32");
   if (bo->numel == 0) return TFHIP_OK;
+  if (rows > INT_MAX) return ctx->fail(TFHIP_ENOTSUP, "scatterND: more than 2^31 - 1 result slices");
   const dim3 grid(blocks_for(ctx, bo->numel)), block(256);
   const int sum = flags & TFHIP_SCATTER_SUM ? 1 : 0, one = scalar_update ? 1 : 0;
   const int64_t* fl = (const int64_t*)flat.ptr;
