@@ -783,3 +783,25 @@ module.exports = Object.assign({}, strictOps, aliases, {
   losses: {computeWeightedLoss, absoluteDifference, meanSquaredError, cosineDistance, hingeLoss, logLoss,
            huberLoss, sigmoidCrossEntropy, softmaxCrossEntropy}
 });
+
+// Chaining methods for the ops above (tensor.ts:700-1460): x.addStrict(y), x.fft(), x.dot(y) ...
+const CHAINED = Object.keys(STRICT).concat(['fft', 'ifft', 'rfft', 'irfft', 'dot', 'logicalXor', 'conv1d',
+                                              'batchNormalization']);
+CHAINED.forEach(name => {
+  const fn = module.exports[name];
+  if (typeof fn !== 'function' || Tensor.prototype[name] != null) return;
+  Tensor.prototype[name] = function(...args) {
+    this.throwIfDisposed();
+    return fn(this, ...args);
+  };
+});
+Tensor.prototype.unsortedSegmentSum = function(segmentIds, numSegments) {
+  this.throwIfDisposed();
+  return ops.unsortedSegmentSum(this, segmentIds, numSegments);
+};
+Tensor.prototype.as5D = function(rows, columns, depth, depth2, depth3) {
+  this.throwIfDisposed();
+  return reshape(this, [rows, columns, depth, depth2, depth3]);
+};
+Tensor.prototype.print = function(verbose) { return print(this, verbose); };
+

@@ -752,6 +752,9 @@ test('range, windows, seeded random tensors, losses over a host backend', async 
       assert.throws(() => tf.losses.absoluteDifference(l, tf.tensor1d([1, 2])), /must match/);
       assert.throws(() => tf.addStrict(l, tf.tensor1d([1, 2])), /must match/);
       closeTo(tf.addStrict(l, p).dataSync(), [1.5, 4.5, 4, 8]);
+      closeTo(l.addStrict(p).mulStrict(w).dataSync(), [1.5, 0, 8, 4]);          // chained forms
+      assert.deepStrictEqual(l.as5D(1, 1, 2, 1, 2).shape, [1, 1, 2, 1, 2]);
+      assert.throws(() => l.subStrict(tf.tensor1d([1])), /must match/);
       // tensor.ts TensorBuffer: coordinates, bounds, round trip
       const buf = tf.buffer([2, 3], 'int32');
       buf.set(7, 1, 2);
