@@ -7,6 +7,13 @@ cpu_baseline leg of bench.py may import this module; the product path never does
 
 The shape math restated here follows tfjs-core/src/ops/conv_util.ts:66-182,391-435,
 ops/broadcast_util.ts:27-87 and ops/axis_util.ts:49-95.
+
+Pinning: every function below is checked against the known-answer vectors of the reference's
+own *_test.ts files (tests/test_oracle_golden.py) or against closed forms, identities and
+brute force (tests/test_oracle_math.py).  Parity unpinned: depthwise_conv2d with asymmetric
+padding on non-square inputs (the `pad_quirk` argument chooses between backend_cpu's row /
+column swap and the TensorFlow semantics; no reference vector tells them apart), and
+where_indices, which is numpy.argwhere and has no reference vector extracted.
 """
 import ctypes as C
 import math
