@@ -83,12 +83,59 @@ int tfhip_register(tfhip_ctx* ctx, int64_t id, const int32_t* shape, int rank, i
 int tfhip_write(tfhip_ctx* ctx, int64_t id, const void* host, size_t nbytes);
 int tfhip_read(tfhip_ctx* ctx, int64_t id, void* host, size_t nbytes);
 int tfhip_dispose(tfhip_ctx* ctx, int64_t id);
+/* How the copies are ordered.  Kernels run on one in-order stream.  tfhip_write sends up to
+ * 64 KiB through a pinned slot on that stream and returns without waiting; larger writes run on
+ * a second stream, so that they overlap with the kernels queued before them, and the first
+ * kernel that uses the buffer waits for the copy (the device backends of the reference upload
+ * lazily for the same reason: tfjs-webgpu/src/backend_webgpu.ts:191-245,
+ * backends/webgl/backend_webgl.ts:425-499).  From ordinary memory the call returns when the
+ * copy is done (the caller's array is its own again).  From memory of tfhip_host_alloc the call
+ * returns at once and the copy reads the caller's buffer later: leave it unchanged until
+ * tfhip_sync, tfhip_read or a finished asynchronous read of a result that depends on it — the
+ * contract of the reference's CPU backend, whose write keeps the caller's array
+ * (backend_cpu.ts:122-129).
+ *
+ * Pinned host memory for such uploads.  Process-wide (no context), safe from any thread.
+ * tfhip_host_free waits for copies that still use the memory. */
+int tfhip_host_alloc(size_t nbytes, void** ptr);
+int tfhip_host_free(void* ptr);
+/* KernelBackend.read (backend.ts:33-35) returns a promise: a read in three steps, so that the
+ * host's thread never waits for the device.
+ *   tfhip_read_begin   queues, behind the kernels queued so far, a copy of the buffer into
+ *                      pinned staging memory on a third stream, and returns at once.  The
+ *                      buffer may be disposed or overwritten right away.
+ *   tfhip_read_wait    blocks until that copy is done.  The only call of this interface that may
+ *                      run on another thread than the context's (a worker of the host's thread
+ *                      pool); it touches nothing but the ticket.
+ *   tfhip_read_finish  copies the staged bytes to `host` (nbytes must be the buffer's size; NULL
+ *                      drops the data), waiting first if nobody has, and frees the ticket.  ctx
+ *                      may be NULL when the context was destroyed in the meantime. */
+typedef struct tfhip_pending_read tfhip_pending_read;
+int tfhip_read_begin(tfhip_ctx* ctx, int64_t id, tfhip_pending_read** out);
+int tfhip_read_wait(tfhip_pending_read* r);
+int tfhip_read_finish(tfhip_ctx* ctx, tfhip_pending_read* r, void* host, size_t nbytes);
 /* bytes held by live ids / bytes parked in the pool / number of live ids */
 int tfhip_mem_info(tfhip_ctx* ctx, size_t* in_use, size_t* pooled, size_t* num_ids);
 int tfhip_sync(tfhip_ctx* ctx);
-/* KernelBackend.time (backend.ts:92, backend_cpu.ts:239-244): event pair on the stream. */
+/* KernelBackend.time (backend.ts:92, backend_cpu.ts:239-244): device time of the work queued
+ * between the two calls.  Regions nest (up to 8 deep), as tf.time() calls may.
+ * BackendTimingInfo.getExtraProfileInfo (backend.ts:27-31) is fed by the per-kernel figures:
+ * while a region is open an event follows every kernel launch on the stream, and the time
+ * of a kernel is the distance from the event before it, so the figures of a region add up to
+ * its total (device idle time in front of a kernel counts towards that kernel).  The WebGL
+ * backend of the reference times each program the same way with timer queries
+ * (backends/webgl/backend_webgl.ts:547-620).
+ *   tfhip_time_kernel_count / tfhip_time_kernel  the launches of the region that ended last, in
+ *                      launch order: name of the kernel variant (as tfhip_last_kernel reports
+ *                      it; the entry point's name for kernels without variants) and its time.
+ *                      The name stays valid until the next tfhip_time_end.
+ *   tfhip_time_per_kernel(ctx, 0) switches the per-launch events off (one event pair per
+ *                      region, no figures per kernel); 1, the default, switches them on. */
 int tfhip_time_begin(tfhip_ctx* ctx);
 int tfhip_time_end(tfhip_ctx* ctx, float* ms);
+int tfhip_time_per_kernel(tfhip_ctx* ctx, int enable);
+int tfhip_time_kernel_count(tfhip_ctx* ctx, int* count);
+int tfhip_time_kernel(tfhip_ctx* ctx, int index, const char** name, float* ms);
 /* Captured graphs: no counterpart in the reference, whose backends run every op eagerly.  A
  * chain of small kernels (a batch-1 forward pass is 32 launches of a few microseconds) is bound by
  * the host's cost per launch; captured once, it replays with a single launch.

@@ -197,3 +197,170 @@ def test_captured_graph_replays_match_eager_runs():
         after = tf.memory()
         assert after["numDeviceBuffers"] == before["numDeviceBuffers"]
         assert after["numBytesInGPU"] == before["numBytesInGPU"]
+
+
+# ---- copies that overlap with kernels ------------------------------------------------------
+def _chain(tf, x, w):
+    """A few milliseconds of dependent kernels whose result depends on every element of x."""
+    h = x
+    for _ in range(6):
+        h = tf.relu(tf.matmul(h, w))
+    return h
+
+
+def test_large_pageable_and_pinned_uploads_arrive_whole(tf):
+    """Writes above the ring-slot size run on the upload stream; the first kernel that reads
+    the tensor waits for the copy.  Checked for ordinary and for page-locked source memory, on
+    fresh blocks and on blocks that come back from the pool with kernels still reading them."""
+    rng = np.random.default_rng(21)
+    n = 1 << 20
+    pinned = tf.pinned_array("float32", (n,))
+    for round_ in range(6):
+        src = rng.standard_normal(n).astype(np.float32)
+        if round_ % 2:
+            pinned[:] = src
+            src_arr = pinned
+        else:
+            src_arr = src
+        with tf.tidy():
+            t = tf.tensor(src_arr)
+            y = tf.add(tf.mul(t, t), t)      # reads the block while the next round's tensor ...
+            got = y.data_sync()
+        np.testing.assert_array_equal(got, src * src + src)
+        # ... is registered here into the block t just gave back
+
+
+def test_upload_overlapping_a_running_step_never_tears(tf):
+    """A pipelined loop as the benchmark runs it: batch i+1 is uploaded from pinned memory
+    while the kernels of batch i run, input blocks cycle through the pool, results are read
+    asynchronously two steps late.  Every result must equal the eager, fully synchronised
+    one: a kernel that read a half-written input, or an upload that overwrote an input still
+    being read, would differ."""
+    rng = np.random.default_rng(22)
+    m = 1024
+    w_np = (rng.standard_normal((m, m)) / np.sqrt(m)).astype(np.float32)
+    batches = [rng.standard_normal((m, m)).astype(np.float32) for _ in range(4)]
+    slots = [tf.pinned_array("float32", (m, m)) for _ in range(2)]
+    w = tf.tensor(w_np)
+    want = []
+    for b in batches:
+        with tf.tidy():
+            want.append(_chain(tf, tf.tensor(b), w).data_sync())
+        tf.backend().sync()
+    steps = 24
+    pending, got = [], []
+    slots[0][:] = batches[0]
+    nxt = tf.tensor(slots[0])
+    for i in range(steps):
+        cur = nxt
+        if i + 1 < steps:
+            # the slot was the source of batch i-1, whose result has been waited for below
+            slots[(i + 1) % 2][:] = batches[(i + 1) % 4]
+            nxt = tf.tensor(slots[(i + 1) % 2])          # upload overlaps with the step below
+        out = _chain(tf, cur, w)
+        cur.dispose()
+        pending.append(out.data())
+        out.dispose()                                     # disposed with the read in flight
+        if len(pending) > 1:
+            got.append(pending.pop(0).result())
+    got += [p.result() for p in pending]
+    w.dispose()
+    assert len(got) == steps
+    for i, g in enumerate(got):
+        np.testing.assert_array_equal(g, want[i % 4], err_msg="step %d" % i)
+
+
+def test_overwrite_of_a_tensor_that_queued_kernels_still_read(tf):
+    rng = np.random.default_rng(23)
+    a = rng.standard_normal((512, 512)).astype(np.float32)
+    b = rng.standard_normal((512, 512)).astype(np.float32)
+    w_np = (rng.standard_normal((512, 512)) / 22).astype(np.float32)
+    with tf.tidy():
+        w = tf.tensor(w_np)
+        t = tf.tensor(a)
+        ya = _chain(tf, t, w)
+        tf.backend().write(t.data_id, b)     # large write into a buffer with readers queued
+        yb = _chain(tf, t, w)
+        small = tf.tensor(np.zeros(8, np.float32))
+        s1 = tf.add(small, small)
+        tf.backend().write(small.data_id, np.arange(8, dtype=np.float32))  # ring-slot path
+        s2 = tf.add(small, small)
+        got_a, got_b = ya.data_sync(), yb.data_sync()
+        assert s1.data_sync().tolist() == [0] * 8
+        assert s2.data_sync().tolist() == [2 * i for i in range(8)]
+        t2 = tf.tensor(a)
+        want_a = _chain(tf, t2, w).data_sync()
+        t3 = tf.tensor(b)
+        want_b = _chain(tf, t3, w).data_sync()
+    np.testing.assert_array_equal(got_a, want_a)
+    np.testing.assert_array_equal(got_b, want_b)
+
+
+def test_many_small_writes_wrap_the_staging_ring(tf):
+    with tf.tidy():
+        ts = [tf.tensor(np.full(100, i, np.float32)) for i in range(200)]
+        total = ts[0]
+        for t in ts[1:]:
+            total = tf.add(total, t)
+        assert total.data_sync().tolist() == [sum(range(200))] * 100
+
+
+def test_async_read_returns_what_sync_read_returns(tf):
+    rng = np.random.default_rng(24)
+    with tf.tidy():
+        for dtype, vals in (("float32", rng.standard_normal(70000).astype(np.float32)),
+                            ("int32", rng.integers(-9, 9, 333).astype(np.int32)),
+                            ("bool", rng.integers(0, 2, 50) != 0)):
+            t = tf.tensor(vals)
+            p = t.data()
+            np.testing.assert_array_equal(p.result(), t.data_sync())
+        empty = tf.tensor(np.zeros((0, 4), np.float32))
+        assert empty.data().result().shape == (0, 4)
+    be = tf.backend()
+    ticket = C.c_void_p()
+    assert be.lib.tfhip_read_begin(be.ctx, 10 ** 9 + 7, C.byref(ticket)) != 0   # unknown id
+    assert b"unknown data id" in be.lib.tfhip_last_error(be.ctx)
+
+
+def test_time_reports_every_kernel_and_nests(tf):
+    """KernelBackend.time with the per-kernel figures behind getExtraProfileInfo
+    (backend.ts:27-31): one entry per launch, in order, adding up to the region's total."""
+    rng = np.random.default_rng(25)
+    with tf.tidy():
+        a = tf.tensor(rng.standard_normal((512, 512)).astype(np.float32))
+        x = tf.tensor(rng.standard_normal((2, 32, 32, 16)).astype(np.float32))
+        f = tf.tensor(rng.standard_normal((3, 3, 16, 1)).astype(np.float32))
+        inner = {}
+
+        def work():
+            tf.matmul(a, a)
+            inner.update(tf.time(lambda: tf.relu(a)))
+            tf.depthwise_conv2d(x, f, 1, "same")
+            tf.softmax(a)
+
+        tf.matmul(a, a)
+        info = tf.time(work)
+    names = [k[0] for k in info["kernelTimes"]]
+    if names[0].endswith("_splitk"):   # a product cut along K is two launches, each with its own line
+        assert names[1] == "splitk_finish", names
+        del names[1]
+    assert len(names) == 4, names
+    assert names[0].startswith("gemm_") and names[2].startswith("depthwise")
+    assert names[1] == "tfhip_unary" and names[3] == "tfhip_softmax_rows", names
+    assert all(ms > 0 for _, ms in info["kernelTimes"])
+    total = sum(ms for _, ms in info["kernelTimes"])
+    assert total <= info["kernelMs"] * 1.001 and total >= info["kernelMs"] * 0.8
+    assert [k[0] for k in inner["kernelTimes"]] == ["tfhip_unary"]
+    assert 0 < inner["kernelMs"] < info["kernelMs"]
+    assert info["getExtraProfileInfo"]().count(":") == len(info["kernelTimes"])
+    be = tf.backend()
+    ms = C.c_float()
+    assert be.lib.tfhip_time_end(be.ctx, C.byref(ms)) != 0      # no region is open
+    be.lib.tfhip_time_per_kernel(be.ctx, 0)
+    try:
+        with tf.tidy():
+            a = tf.tensor(np.ones((64, 64), np.float32))
+            quiet = tf.time(lambda: tf.matmul(a, a))
+        assert quiet["kernelTimes"] == [] and quiet["kernelMs"] > 0
+    finally:
+        be.lib.tfhip_time_per_kernel(be.ctx, 1)

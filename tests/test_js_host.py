@@ -37,8 +37,12 @@ def test_addon_exports_the_c_abi():
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
     declared = set(re.findall(r"\btfhip_([a-z0-9_]+)\s*\(", header))
     camel = lambda s: re.sub(r"_([a-z0-9])", lambda m: m.group(1).upper(), s)
+    # host_free is the finaliser of hostAlloc's buffer; the three steps of an asynchronous read
+    # are readAsync; the two per-kernel getters are timeKernels
     rename = {"last_error": None, "device_ptr": None, "softmax_rows": "softmaxRows",
-              "depthwise_conv2d": "depthwiseConv2d"}
+              "depthwise_conv2d": "depthwiseConv2d", "host_free": "hostAlloc",
+              "read_begin": "readAsync", "read_wait": "readAsync", "read_finish": "readAsync",
+              "time_kernel_count": "timeKernels", "time_kernel": "timeKernels"}
     for name in declared:
         js_name = rename.get(name, camel(name))
         if js_name is not None:

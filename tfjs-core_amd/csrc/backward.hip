@@ -412,7 +412,7 @@ extern "C" int tfhip_depthwise_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int6
   if (ch_mul == 1 && ci->in_c % 4 == 0 && aligned16(dyf) && aligned16(wf) && aligned16(dxf)) {
     const unsigned blocks = (unsigned)ceil_div(x_n / 4, 256);
     const int s = ci->stride_h == ci->stride_w && ci->stride_h <= 2 ? ci->stride_h : 0;
-    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise_der_input_vec_s%d", s);
+    ctx->name_kernel("depthwise_der_input_vec_s%d", s);
     if (s == 1)
       hipLaunchKernelGGL(depthwise_der_input_vec_kernel<1>, dim3(blocks), dim3(256), 0, ctx->stream,
                          dyf, wf, dxf, *ci);
@@ -425,7 +425,7 @@ extern "C" int tfhip_depthwise_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int6
     TFHIP_LAUNCH_CHECK(ctx);
     return TFHIP_OK;
   }
-  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise_der_input");
+  ctx->name_kernel("depthwise_der_input");
   hipLaunchKernelGGL(depthwise_der_input_kernel, dim3(grid_for(ctx, x_n)), dim3(256), 0, ctx->stream,
                      dyf, wf, dxf, *ci, ch_mul);
   TFHIP_LAUNCH_CHECK(ctx);
@@ -473,7 +473,7 @@ extern "C" int tfhip_depthwise_conv2d_der_filter(tfhip_ctx* ctx, int64_t x, int6
     if (slices > 65535) slices = 65535;
     const int64_t per_slice = ceil_div(pixels, slices);
     if (!tpart.get((size_t)(slices * w_n) * sizeof(double))) return TFHIP_EDEVICE;
-    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise3x3_der_filter");
+    ctx->name_kernel("depthwise3x3_der_filter");
     hipLaunchKernelGGL(depthwise3x3_der_filter_partial_kernel, dim3((unsigned)blocks_c, (unsigned)slices),
                        dim3(256), (size_t)(256 * 9 * 4 * sizeof(float)), ctx->stream, xf, dyf,
                        static_cast<double*>(tpart.ptr), *ci, qpw, per_slice);
@@ -492,7 +492,7 @@ extern "C" int tfhip_depthwise_conv2d_der_filter(tfhip_ctx* ctx, int64_t x, int6
   if (slices > 65535) slices = 65535;
   const int64_t per_slice = ceil_div(pixels > 0 ? pixels : 1, slices);
   if (!tpart.get((size_t)(slices * w_n) * sizeof(double))) return TFHIP_EDEVICE;
-  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise_der_filter");
+  ctx->name_kernel("depthwise_der_filter");
   hipLaunchKernelGGL(depthwise_der_filter_partial_kernel,
                      dim3((unsigned)channel_blocks, (unsigned)taps, (unsigned)slices), dim3(256), 0,
                      ctx->stream, xf, dyf, static_cast<double*>(tpart.ptr), *ci, ch_mul, per_slice);
@@ -527,14 +527,14 @@ extern "C" int tfhip_pool2d_backprop(tfhip_ctx* ctx, int64_t dy, int64_t x, int6
   if ((rc = as_f32(ctx, bx, &tx, &xf))) return rc;
   float* dxf = static_cast<float*>(bdx->ptr);
   if (ci->in_c % 4 == 0 && aligned16(dyf) && aligned16(xf) && aligned16(dxf)) {
-    snprintf(ctx->last_kernel, sizeof ctx->last_kernel,
+    ctx->name_kernel(
              kind == TFHIP_POOL_MAX ? "max_pool_backprop_vec" : "avg_pool_backprop_vec");
     hipLaunchKernelGGL(pool2d_backprop_vec_kernel, dim3((unsigned)ceil_div(x_n / 4, 256)), dim3(256), 0,
                        ctx->stream, dyf, xf, dxf, *ci, kind);
     TFHIP_LAUNCH_CHECK(ctx);
     return TFHIP_OK;
   }
-  snprintf(ctx->last_kernel, sizeof ctx->last_kernel,
+  ctx->name_kernel(
            kind == TFHIP_POOL_MAX ? "max_pool_backprop" : "avg_pool_backprop");
   hipLaunchKernelGGL(pool2d_backprop_kernel, dim3(grid_for(ctx, x_n)), dim3(256), 0, ctx->stream, dyf,
                      xf, static_cast<float*>(bdx->ptr), *ci, kind);

@@ -7,6 +7,53 @@ using tfhip::Buf;
 
 static thread_local std::string g_init_error;
 
+// Pinned host memory is process-wide: buffers handed to callers (tfhip_host_alloc) outlive any
+// one context, and finished reads leave their staging blocks here for the next read.
+static std::mutex g_host_mu;
+static std::map<uintptr_t, size_t> g_pinned;                  // start -> bytes
+static std::map<size_t, std::vector<void*>> g_staging;        // capacity -> free blocks
+
+namespace tfhip {
+static bool host_is_pinned(const void* p, size_t nbytes) {
+  std::lock_guard<std::mutex> lock(g_host_mu);
+  auto it = g_pinned.upper_bound((uintptr_t)p);
+  if (it == g_pinned.begin()) return false;
+  --it;
+  return (uintptr_t)p + nbytes <= it->first + it->second;
+}
+// Block sizes are rounded so that tensors of similar size share blocks: 512 B granules up
+// to 1 MiB, then 1/8-octave steps (at most 12.5 % slack on large activations).
+static size_t round_cap(size_t n) {
+  if (n <= (1u << 20)) return (n + 511) & ~size_t(511);
+  size_t step = size_t(1) << (63 - __builtin_clzll(n) - 3);
+  return (n + step - 1) & ~(step - 1);
+}
+
+static void* staging_get(size_t nbytes, size_t* cap) {
+  *cap = round_cap(nbytes);
+  {
+    std::lock_guard<std::mutex> lock(g_host_mu);
+    auto it = g_staging.find(*cap);
+    if (it != g_staging.end() && !it->second.empty()) {
+      void* p = it->second.back();
+      it->second.pop_back();
+      return p;
+    }
+  }
+  void* p = nullptr;
+  if (hipHostMalloc(&p, *cap, hipHostMallocDefault) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  return p;
+}
+static void staging_put(void* p, size_t cap) {
+  if (!p) return;
+  std::lock_guard<std::mutex> lock(g_host_mu);
+  g_staging[cap].push_back(p);
+}
+}  // namespace tfhip
+
 int tfhip_ctx::fail(int code, const char* fmt, ...) {
   char buf[512];
   va_list ap;
@@ -17,25 +64,97 @@ int tfhip_ctx::fail(int code, const char* fmt, ...) {
   return code;
 }
 
-Buf* tfhip_ctx::find(int64_t id) {
+void tfhip_ctx::name_kernel(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(last_kernel, sizeof last_kernel, fmt, ap);
+  va_end(ap);
+  kernel_named = true;
+}
+
+// One more event on the stream.  The begin and end marks of a region always get a slot (the
+// last one is kept for them); kernel marks beyond the limit are counted and left out.
+int tfhip_ctx::mark(const char* name) {
+  const bool bracket = name[0] == '(';
+  if (marks_used >= kMaxMarks - (bracket ? 0 : 2 * kMaxTimeDepth)) {
+    if (!bracket) {
+      marks_dropped++;
+      return -1;
+    }
+    if (marks_used >= kMaxMarks) {
+      fail(TFHIP_EINVAL, "time: too many nested regions after %d launches", kMaxMarks);
+      return -1;
+    }
+  }
+  if (marks_used == (int)mark_events.size()) {
+    hipEvent_t ev;
+    hipError_t e = hipEventCreate(&ev);
+    if (e != hipSuccess) {
+      fail(TFHIP_EDEVICE, "hipEventCreate: %s", hipGetErrorString(e));
+      return -1;
+    }
+    mark_events.push_back(ev);
+    mark_names.emplace_back();
+  }
+  hipError_t e = hipEventRecord(mark_events[marks_used], stream);
+  if (e != hipSuccess) {
+    fail(TFHIP_EDEVICE, "hipEventRecord: %s", hipGetErrorString(e));
+    return -1;
+  }
+  mark_names[marks_used] = name;
+  return marks_used++;
+}
+
+Buf* tfhip_ctx::find(int64_t id, bool touch) {
   auto it = bufs.find(id);
   if (it == bufs.end()) {
     fail(TFHIP_ENOENT, "unknown data id %lld", (long long)id);
     return nullptr;
   }
-  return &it->second;
+  Buf& b = it->second;
+  if (touch) {
+    if (b.uploaded) {  // the data is still on its way: the compute stream waits for the copy
+      (void)hipStreamWaitEvent(stream, b.uploaded, 0);
+      ev_put(b.uploaded);
+      b.uploaded = nullptr;
+    }
+    if (b.ready) {  // from here on the block is ordered by the compute stream alone
+      ev_put(b.ready);
+      b.ready = nullptr;
+    }
+    b.used = true;
+  }
+  return &b;
 }
 
-// Block sizes are rounded so that tensors of similar size share blocks: 512 B granules up
-// to 1 MiB, then 1/8-octave steps (at most 12.5 % slack on large activations).
-static size_t round_cap(size_t n) {
-  if (n <= (1u << 20)) return (n + 511) & ~size_t(511);
-  size_t step = size_t(1) << (63 - __builtin_clzll(n) - 3);
-  return (n + step - 1) & ~(step - 1);
+int tfhip_ctx::await_uploads() {
+  for (auto& kv : bufs) {
+    if (!kv.second.uploaded) continue;
+    TFHIP_HIP(this, hipStreamWaitEvent(stream, kv.second.uploaded, 0));
+    ev_put(kv.second.uploaded);
+    kv.second.uploaded = nullptr;
+  }
+  return TFHIP_OK;
 }
 
-void* tfhip_ctx::alloc(size_t nbytes, size_t* cap) {
-  const size_t want = round_cap(nbytes);
+hipEvent_t tfhip_ctx::ev_get() {
+  if (!free_events.empty()) {
+    hipEvent_t ev = free_events.back();
+    free_events.pop_back();
+    return ev;
+  }
+  hipEvent_t ev = nullptr;
+  if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  return ev;
+}
+
+void* tfhip_ctx::alloc(size_t nbytes, size_t* cap, hipEvent_t* ready, bool* recycled) {
+  const size_t want = tfhip::round_cap(nbytes);
+  if (ready) *ready = nullptr;
+  if (recycled) *recycled = false;
   auto it = pool.find(want);
   if (it != pool.end() && !it->second.empty()) {
     // most recently freed block first: it is the one most likely still in L2 / MALL
@@ -45,6 +164,15 @@ void* tfhip_ctx::alloc(size_t nbytes, size_t* cap) {
     in_use += want;
     *cap = want;
     if (capturing) capture_blocks.push_back(p);
+    if (recycled) *recycled = true;
+    if (!block_ready.empty()) {
+      auto ev = block_ready.find(p);
+      if (ev != block_ready.end()) {
+        if (ready) *ready = ev->second;
+        else ev_put(ev->second);  // the new owner is ordered by the compute stream
+        block_ready.erase(ev);
+      }
+    }
     return p;
   }
   if (capturing) {
@@ -71,9 +199,17 @@ void* tfhip_ctx::alloc(size_t nbytes, size_t* cap) {
   return p;
 }
 
-void tfhip_ctx::release(void* p, size_t cap) {
-  if (!p) return;
+void tfhip_ctx::release(void* p, size_t cap, hipEvent_t ready) {
+  if (!p) {
+    ev_put(ready);
+    return;
+  }
   in_use -= cap;
+  if (ready) {
+    auto old = block_ready.find(p);
+    if (old != block_ready.end()) ev_put(old->second);
+    block_ready[p] = ready;
+  }
   auto own = owner.find(p);
   if (own != owner.end()) {  // a block that a captured graph writes on every replay
     graphs[own->second].parked.emplace_back(p, cap);
@@ -83,12 +219,46 @@ void tfhip_ctx::release(void* p, size_t cap) {
   pool[cap].push_back(p);
 }
 
+// A buffer lets go of its block.  Copies still in flight on the other streams are put in
+// front of whatever the compute stream does with the block next; a block that was filled
+// through the upload stream leaves an event behind, so that the next upload into it waits for
+// the kernels that read it and for nothing queued later.
+void tfhip_ctx::release_buf(Buf& b) {
+  if (b.uploaded) {
+    (void)hipStreamWaitEvent(stream, b.uploaded, 0);
+    ev_put(b.uploaded);
+  }
+  if (b.read_done) (void)hipStreamWaitEvent(stream, b.read_done, 0);  // owned by the read's ticket
+  hipEvent_t left = nullptr;
+  if (b.ready) {
+    if (b.used) ev_put(b.ready);
+    else left = b.ready;  // never touched: the block's history is still what the event says
+  }
+  if (!left && b.ptr && b.upload_target && !capturing && (left = ev_get())) {
+    if (hipEventRecord(left, stream) != hipSuccess) {
+      (void)hipGetLastError();
+      ev_put(left);
+      left = nullptr;
+    }
+  }
+  release(b.ptr, b.cap, left);
+  b.ptr = nullptr;
+  b.uploaded = b.read_done = b.ready = nullptr;
+}
+
 void tfhip_ctx::trim() {
   // (not while a graph exists: a replay may still read blocks that went back to the pool)
   if (pool.empty() || capturing || !graphs.empty()) return;
   (void)hipStreamSynchronize(stream);
   for (auto& kv : pool)
-    for (void* p : kv.second) (void)hipFree(p);
+    for (void* p : kv.second) {
+      auto ev = block_ready.find(p);
+      if (ev != block_ready.end()) {
+        ev_put(ev->second);
+        block_ready.erase(ev);
+      }
+      (void)hipFree(p);
+    }
   pool.clear();
   pooled = 0;
 }
@@ -116,9 +286,12 @@ int tfhip_init(int device, tfhip_ctx** out) {
   if ((e = hipSetDevice(device)) != hipSuccess ||
       (e = hipGetDeviceProperties(&prop, device)) != hipSuccess ||
       (e = hipStreamCreate(&ctx->stream)) != hipSuccess ||
-      (e = hipEventCreate(&ctx->ev_begin)) != hipSuccess ||
-      (e = hipEventCreate(&ctx->ev_end)) != hipSuccess) {
+      (e = hipStreamCreateWithFlags(&ctx->upload, hipStreamNonBlocking)) != hipSuccess ||
+      (e = hipStreamCreateWithFlags(&ctx->download, hipStreamNonBlocking)) != hipSuccess) {
     g_init_error = std::string("device set-up failed: ") + hipGetErrorString(e);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    if (ctx->upload) (void)hipStreamDestroy(ctx->upload);
+    if (ctx->download) (void)hipStreamDestroy(ctx->download);
     delete ctx;
     return TFHIP_EDEVICE;
   }
@@ -126,6 +299,8 @@ int tfhip_init(int device, tfhip_ctx** out) {
     g_init_error = std::string("libtfjs_hip is built for gfx950 only, device is ") +
                    prop.gcnArchName;
     (void)hipStreamDestroy(ctx->stream);
+    (void)hipStreamDestroy(ctx->upload);
+    (void)hipStreamDestroy(ctx->download);
     delete ctx;
     return TFHIP_ENOTSUP;
   }
@@ -137,9 +312,21 @@ int tfhip_init(int device, tfhip_ctx** out) {
 void tfhip_destroy(tfhip_ctx* ctx) {
   if (!ctx) return;
   (void)hipSetDevice(ctx->device);
+  (void)hipStreamSynchronize(ctx->upload);
+  (void)hipStreamSynchronize(ctx->download);
   (void)hipStreamSynchronize(ctx->stream);
-  for (auto& kv : ctx->bufs)
+  // reads that were begun and not finished keep their ticket (tfhip_read_finish with a NULL
+  // context frees it); their events are theirs
+  for (auto& kv : ctx->bufs) {
     if (kv.second.ptr) (void)hipFree(kv.second.ptr);
+    if (kv.second.ready) (void)hipEventDestroy(kv.second.ready);
+    if (kv.second.uploaded) (void)hipEventDestroy(kv.second.uploaded);
+  }
+  for (auto& kv : ctx->block_ready) (void)hipEventDestroy(kv.second);
+  for (hipEvent_t ev : ctx->free_events) (void)hipEventDestroy(ev);
+  for (hipEvent_t ev : ctx->ring_done)
+    if (ev) (void)hipEventDestroy(ev);
+  if (ctx->ring) (void)hipHostFree(ctx->ring);
   for (auto& kv : ctx->pool)
     for (void* p : kv.second) (void)hipFree(p);
   for (auto& kv : ctx->graphs) {
@@ -147,8 +334,9 @@ void tfhip_destroy(tfhip_ctx* ctx) {
     (void)hipGraphDestroy(kv.second.graph);
     for (auto& blk : kv.second.parked) (void)hipFree(blk.first);
   }
-  (void)hipEventDestroy(ctx->ev_begin);
-  (void)hipEventDestroy(ctx->ev_end);
+  for (hipEvent_t ev : ctx->mark_events) (void)hipEventDestroy(ev);
+  (void)hipStreamDestroy(ctx->upload);
+  (void)hipStreamDestroy(ctx->download);
   (void)hipStreamDestroy(ctx->stream);
   delete ctx;
 }
@@ -176,27 +364,83 @@ int tfhip_register(tfhip_ctx* ctx, int64_t id, const int32_t* shape, int rank, i
   }
   b.nbytes = (size_t)b.numel * tfhip::dtype_size(dtype);
   if (b.nbytes) {
-    b.ptr = ctx->alloc(b.nbytes, &b.cap);
+    b.ptr = ctx->alloc(b.nbytes, &b.cap, &b.ready, &b.recycled);
     if (!b.ptr) return TFHIP_EDEVICE;
   }
   ctx->bufs.emplace(id, b);
   return TFHIP_OK;
 }
 
+// Host-to-device copies take one of three roads:
+//  * up to one ring slot (64 KiB): the bytes are copied into a pinned slot and from there by
+//    the compute stream itself, in order with the kernels, without any wait on the host;
+//  * larger, from memory of tfhip_host_alloc: a DMA on the upload stream straight from the
+//    caller's buffer, which returns at once and overlaps with the kernels already queued;
+//  * larger, from ordinary (pageable) memory: the same on the upload stream, and the host waits
+//    for that stream only, so kernels queued earlier keep running during the copy.
+// The upload stream may overwrite a block only after the compute-stream work that used it:
+// it waits for the event the block's last owner left (release_buf), or, when the history is
+// not known (a live buffer overwritten, a recycled block without an event), for everything
+// queued on the compute stream so far.  A buffer fresh from the driver needs no wait.
 int tfhip_write(tfhip_ctx* ctx, int64_t id, const void* host, size_t nbytes) {
   if (!ctx) return TFHIP_EINVAL;
   if (ctx->capturing)
     return ctx->fail(TFHIP_EINVAL, "write: host data cannot enter a graph capture (create the "
                                    "tensor before capturing)");
-  TFHIP_GET(ctx, b, id);
+  Buf* b = ctx->find(id, /*touch=*/false);
+  if (!b) return TFHIP_ENOENT;
   if (!host && nbytes)  // backend_cpu.ts:125-127
     return ctx->fail(TFHIP_EINVAL, "MathBackendHIP.write(): values can not be null");
   if (nbytes != b->nbytes)
     return ctx->fail(TFHIP_EINVAL, "write: got %zu bytes for a buffer of %zu", nbytes, b->nbytes);
   if (!nbytes) return TFHIP_OK;
-  // The caller may reuse or free `host` as soon as this returns, so wait for the copy.
-  TFHIP_HIP(ctx, hipMemcpyAsync(b->ptr, host, nbytes, hipMemcpyHostToDevice, ctx->stream));
-  TFHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+
+  if (nbytes <= tfhip_ctx::kSlotBytes) {
+    if (!ctx->ring)
+      TFHIP_HIP(ctx, hipHostMalloc((void**)&ctx->ring, tfhip_ctx::kSlotBytes * tfhip_ctx::kSlots,
+                                   hipHostMallocDefault));
+    const int slot = ctx->ring_next;
+    ctx->ring_next = (slot + 1) % tfhip_ctx::kSlots;
+    if (ctx->ring_done[slot]) TFHIP_HIP(ctx, hipEventSynchronize(ctx->ring_done[slot]));
+    else if (!(ctx->ring_done[slot] = ctx->ev_get()))
+      return ctx->fail(TFHIP_EDEVICE, "write: could not create an event");
+    char* staged = ctx->ring + (size_t)slot * tfhip_ctx::kSlotBytes;
+    memcpy(staged, host, nbytes);
+    b = ctx->find(id, /*touch=*/true);  // a copy on the compute stream is a use like any kernel
+    if (b->read_done) TFHIP_HIP(ctx, hipStreamWaitEvent(ctx->stream, b->read_done, 0));
+    TFHIP_HIP(ctx, hipMemcpyAsync(b->ptr, staged, nbytes, hipMemcpyHostToDevice, ctx->stream));
+    TFHIP_HIP(ctx, hipEventRecord(ctx->ring_done[slot], ctx->stream));
+    return TFHIP_OK;
+  }
+
+  if (b->used || (b->recycled && !b->ready)) {
+    hipEvent_t fence = ctx->ev_get();
+    if (!fence) return ctx->fail(TFHIP_EDEVICE, "write: could not create an event");
+    hipError_t e = hipEventRecord(fence, ctx->stream);
+    if (e == hipSuccess) e = hipStreamWaitEvent(ctx->upload, fence, 0);
+    ctx->ev_put(fence);  // the wait has been queued: the event may be recorded again
+    if (e != hipSuccess) return ctx->fail(TFHIP_EDEVICE, "write: %s", hipGetErrorString(e));
+  } else if (b->ready) {
+    TFHIP_HIP(ctx, hipStreamWaitEvent(ctx->upload, b->ready, 0));
+  }
+  ctx->ev_put(b->ready);
+  b->ready = nullptr;
+  if (b->read_done) TFHIP_HIP(ctx, hipStreamWaitEvent(ctx->upload, b->read_done, 0));
+  b->used = false;
+  b->recycled = false;
+  b->upload_target = true;
+  TFHIP_HIP(ctx, hipMemcpyAsync(b->ptr, host, nbytes, hipMemcpyHostToDevice, ctx->upload));
+  if (!tfhip::host_is_pinned(host, nbytes)) {
+    // the copy reads the caller's pages until it is done, and the caller may change or free
+    // them as soon as this returns
+    TFHIP_HIP(ctx, hipStreamSynchronize(ctx->upload));
+    ctx->ev_put(b->uploaded);
+    b->uploaded = nullptr;
+    return TFHIP_OK;
+  }
+  if (!b->uploaded && !(b->uploaded = ctx->ev_get()))
+    return ctx->fail(TFHIP_EDEVICE, "write: could not create an event");
+  TFHIP_HIP(ctx, hipEventRecord(b->uploaded, ctx->upload));
   return TFHIP_OK;
 }
 
@@ -212,11 +456,114 @@ int tfhip_read(tfhip_ctx* ctx, int64_t id, void* host, size_t nbytes) {
   return TFHIP_OK;
 }
 
+// ---- asynchronous read ----------------------------------------------------------------------
+int tfhip_read_begin(tfhip_ctx* ctx, int64_t id, tfhip_pending_read** out) {
+  if (!ctx || !out) return TFHIP_EINVAL;
+  *out = nullptr;
+  if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "read: not during a graph capture");
+  TFHIP_GET(ctx, b, id);
+  tfhip_pending_read* r = new tfhip_pending_read();
+  r->device = ctx->device;
+  r->nbytes = b->nbytes;
+  if (b->nbytes) {
+    r->staging = tfhip::staging_get(b->nbytes, &r->staging_cap);
+    hipEvent_t produced = ctx->ev_get();
+    r->done = ctx->ev_get();
+    hipError_t e = (r->staging && produced && r->done) ? hipSuccess : hipErrorOutOfMemory;
+    // the copy runs on the download stream, behind the kernels queued so far and no others
+    if (e == hipSuccess) e = hipEventRecord(produced, ctx->stream);
+    if (e == hipSuccess) e = hipStreamWaitEvent(ctx->download, produced, 0);
+    if (e == hipSuccess)
+      e = hipMemcpyAsync(r->staging, b->ptr, b->nbytes, hipMemcpyDeviceToHost, ctx->download);
+    if (e == hipSuccess) e = hipEventRecord(r->done, ctx->download);
+    ctx->ev_put(produced);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      tfhip::staging_put(r->staging, r->staging_cap);
+      ctx->ev_put(r->done);
+      delete r;
+      return ctx->fail(TFHIP_EDEVICE, "read: %s", hipGetErrorString(e));
+    }
+    b->read_done = r->done;
+  }
+  ctx->reads.emplace(r, id);
+  *out = r;
+  return TFHIP_OK;
+}
+
+int tfhip_read_wait(tfhip_pending_read* r) {
+  if (!r) return TFHIP_EINVAL;
+  if (!r->done) return TFHIP_OK;
+  // may run on a thread that has never used the device
+  if (hipSetDevice(r->device) != hipSuccess || hipEventSynchronize(r->done) != hipSuccess) {
+    (void)hipGetLastError();
+    r->failed = true;
+    return TFHIP_EDEVICE;
+  }
+  return TFHIP_OK;
+}
+
+int tfhip_read_finish(tfhip_ctx* ctx, tfhip_pending_read* r, void* host, size_t nbytes) {
+  if (!r) return TFHIP_EINVAL;
+  int rc = TFHIP_OK;
+  if (host && nbytes != r->nbytes) {
+    rc = ctx ? ctx->fail(TFHIP_EINVAL, "read: asked %zu bytes of a buffer of %zu", nbytes, r->nbytes)
+             : TFHIP_EINVAL;
+  } else if (r->done && (r->failed || hipEventSynchronize(r->done) != hipSuccess)) {
+    (void)hipGetLastError();
+    rc = ctx ? ctx->fail(TFHIP_EDEVICE, "read: the copy from the device failed") : TFHIP_EDEVICE;
+  } else if (host && nbytes) {
+    memcpy(host, r->staging, nbytes);
+  }
+  if (ctx) {
+    auto it = ctx->reads.find(r);
+    if (it != ctx->reads.end()) {
+      auto buf = ctx->bufs.find(it->second);
+      if (buf != ctx->bufs.end() && buf->second.read_done == r->done) buf->second.read_done = nullptr;
+      ctx->reads.erase(it);
+    }
+    ctx->ev_put(r->done);
+  } else if (r->done) {
+    (void)hipEventDestroy(r->done);
+  }
+  tfhip::staging_put(r->staging, r->staging_cap);
+  delete r;
+  return rc;
+}
+
+int tfhip_host_alloc(size_t nbytes, void** ptr) {
+  if (!ptr || !nbytes) return TFHIP_EINVAL;
+  *ptr = nullptr;
+  void* p = nullptr;
+  if (hipHostMalloc(&p, nbytes, hipHostMallocDefault) != hipSuccess) {
+    (void)hipGetLastError();
+    return TFHIP_EDEVICE;
+  }
+  std::lock_guard<std::mutex> lock(g_host_mu);
+  g_pinned[(uintptr_t)p] = nbytes;
+  *ptr = p;
+  return TFHIP_OK;
+}
+
+int tfhip_host_free(void* ptr) {
+  if (!ptr) return TFHIP_OK;
+  {
+    std::lock_guard<std::mutex> lock(g_host_mu);
+    if (!g_pinned.erase((uintptr_t)ptr)) return TFHIP_EINVAL;
+  }
+  // waits for copies that still read the memory
+  if (hipHostFree(ptr) != hipSuccess) {
+    (void)hipGetLastError();
+    return TFHIP_EDEVICE;
+  }
+  return TFHIP_OK;
+}
+
 int tfhip_dispose(tfhip_ctx* ctx, int64_t id) {
   if (!ctx) return TFHIP_EINVAL;
   auto it = ctx->bufs.find(id);
   if (it == ctx->bufs.end()) return TFHIP_OK;  // backend_cpu.ts:228-237: unknown id is a no-op
-  ctx->release(it->second.ptr, it->second.cap);
+  ctx->release_buf(it->second);
   ctx->bufs.erase(it);
   return TFHIP_OK;
 }
@@ -232,6 +579,7 @@ int tfhip_mem_info(tfhip_ctx* ctx, size_t* in_use, size_t* pooled, size_t* num_i
 int tfhip_sync(tfhip_ctx* ctx) {
   if (!ctx) return TFHIP_EINVAL;
   if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "sync: not during a graph capture");
+  TFHIP_HIP(ctx, hipStreamSynchronize(ctx->upload));  // pinned sources are free again after this
   TFHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
   return TFHIP_OK;
 }
@@ -239,18 +587,58 @@ int tfhip_sync(tfhip_ctx* ctx) {
 int tfhip_time_begin(tfhip_ctx* ctx) {
   if (!ctx) return TFHIP_EINVAL;
   if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "time: not during a graph capture");
-  TFHIP_HIP(ctx, hipEventRecord(ctx->ev_begin, ctx->stream));
-  ctx->timing = true;
+  if (ctx->time_depth == tfhip_ctx::kMaxTimeDepth)
+    return ctx->fail(TFHIP_EINVAL, "time: more than %d nested regions", tfhip_ctx::kMaxTimeDepth);
+  if (ctx->time_depth == 0) ctx->marks_used = ctx->marks_dropped = 0;
+  const int at = ctx->mark("(begin)");
+  if (at < 0) return TFHIP_EDEVICE;
+  ctx->time_stack[ctx->time_depth++] = at;
   return TFHIP_OK;
 }
 
 int tfhip_time_end(tfhip_ctx* ctx, float* ms) {
   if (!ctx || !ms) return TFHIP_EINVAL;
-  if (!ctx->timing) return ctx->fail(TFHIP_EINVAL, "time_end without time_begin");
-  ctx->timing = false;
-  TFHIP_HIP(ctx, hipEventRecord(ctx->ev_end, ctx->stream));
-  TFHIP_HIP(ctx, hipEventSynchronize(ctx->ev_end));
-  TFHIP_HIP(ctx, hipEventElapsedTime(ms, ctx->ev_begin, ctx->ev_end));
+  if (!ctx->time_depth) return ctx->fail(TFHIP_EINVAL, "time_end without time_begin");
+  const int first = ctx->time_stack[--ctx->time_depth];
+  const int last = ctx->mark("(end)");
+  if (last < 0) return TFHIP_EDEVICE;
+  TFHIP_HIP(ctx, hipEventSynchronize(ctx->mark_events[last]));
+  TFHIP_HIP(ctx, hipEventElapsedTime(ms, ctx->mark_events[first], ctx->mark_events[last]));
+  ctx->kernel_times.clear();
+  for (int i = first + 1; i <= last; i++) {
+    float d = 0;
+    TFHIP_HIP(ctx, hipEventElapsedTime(&d, ctx->mark_events[i - 1], ctx->mark_events[i]));
+    // the marks of this and of inner regions carry no kernel: their (tiny) share stays in the total
+    if (ctx->mark_names[i][0] == '(') continue;
+    ctx->kernel_times.push_back({ctx->mark_names[i], d});
+  }
+  if (ctx->marks_dropped) {
+    char note[64];
+    snprintf(note, sizeof note, "(%d launches not recorded)", ctx->marks_dropped);
+    ctx->kernel_times.push_back({note, 0.f});
+  }
+  return TFHIP_OK;
+}
+
+int tfhip_time_per_kernel(tfhip_ctx* ctx, int enable) {
+  if (!ctx) return TFHIP_EINVAL;
+  ctx->per_kernel = enable != 0;
+  return TFHIP_OK;
+}
+
+int tfhip_time_kernel_count(tfhip_ctx* ctx, int* count) {
+  if (!ctx || !count) return TFHIP_EINVAL;
+  *count = (int)ctx->kernel_times.size();
+  return TFHIP_OK;
+}
+
+int tfhip_time_kernel(tfhip_ctx* ctx, int index, const char** name, float* ms) {
+  if (!ctx) return TFHIP_EINVAL;
+  if (index < 0 || index >= (int)ctx->kernel_times.size())
+    return ctx->fail(TFHIP_EINVAL, "time_kernel: index %d not in 0..%zu", index,
+                     ctx->kernel_times.size());
+  if (name) *name = ctx->kernel_times[index].name.c_str();
+  if (ms) *ms = ctx->kernel_times[index].ms;
   return TFHIP_OK;
 }
 
@@ -259,6 +647,10 @@ int tfhip_graph_begin(tfhip_ctx* ctx) {
   if (!ctx) return TFHIP_EINVAL;
   if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "graph_begin: a capture is already running");
   ctx->capture_blocks.clear();
+  // uploads still on their way are waited for before the recording starts: a wait for an
+  // event of another stream must not become part of the graph
+  int rc = ctx->await_uploads();
+  if (rc) return rc;
   TFHIP_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
   ctx->capturing = true;
   return TFHIP_OK;
@@ -305,6 +697,10 @@ int tfhip_graph_launch(tfhip_ctx* ctx, int64_t graph_id) {
   if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "graph_launch: not during a graph capture");
   auto it = ctx->graphs.find(graph_id);
   if (it == ctx->graphs.end()) return ctx->fail(TFHIP_ENOENT, "graph %lld does not exist", (long long)graph_id);
+  // the recorded kernels read their inputs by address: new data written into those tensors
+  // through the upload stream has to arrive first
+  int rc = ctx->await_uploads();
+  if (rc) return rc;
   TFHIP_HIP(ctx, hipGraphLaunch(it->second.exec, ctx->stream));
   return TFHIP_OK;
 }

@@ -1308,7 +1308,7 @@ template <class T, int AMODE, int BMODE, bool KBLOCKED, bool FAST>
 static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
   static const char* const a_names[] = {"rowmajor", "transposed", "im2col", "im2col_up", "im2col_t"};
   static const char* const b_names[] = {"f32", "f32t", "u8"};
-  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "gemm_%dx%d_%s_%s%s%s", T::BM, T::BN,
+  ctx->name_kernel("gemm_%dx%d_%s_%s%s%s", T::BM, T::BN,
            a_names[AMODE], b_names[BMODE], KBLOCKED ? "_kb48" : "",
            pl.splits > 1 ? (pl.full_tiles ? "_tailk" : "_splitk") : "");
   if (!FAST) strncat(ctx->last_kernel, "_unaligned", sizeof ctx->last_kernel - strlen(ctx->last_kernel) - 1);
@@ -1336,7 +1336,7 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
     const long long cap = (long long)ctx->num_cus * 8;
     hipLaunchKernelGGL(splitk_finish_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256),
                        0, ctx->stream, p, T::BM, T::BN, pl.full_tiles);
-    TFHIP_LAUNCH_CHECK(ctx);
+    TFHIP_LAUNCH_CHECK_NAMED(ctx, "splitk_finish");
   }
   return TFHIP_OK;
 }
@@ -1400,7 +1400,7 @@ static int launch_rowstream_cfg(tfhip_ctx* ctx, const GemmArgs& p, int quant) {
   const int n_blocks = (int)ceil_div(p.M, 32);
   const long long slots = (long long)ctx->num_cus * per_cu / 8 * 8;  // a multiple of the XCD count
   const long long want = ceil_div(ceil_div(n_blocks, 8), 4) * 8;
-  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "gemm_rowstream_k%dxn%d_%s", KQ * 8, NJ * 32,
+  ctx->name_kernel("gemm_rowstream_k%dxn%d_%s", KQ * 8, NJ * 32,
            quant ? "u8" : "f32");
   GemmArgs q = p;
   q.reverse = ctx->take_sweep();
@@ -1677,7 +1677,7 @@ extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t o
         const long long cap = (long long)ctx->num_cus * per_cu;
         unsigned grid = (unsigned)(n_rows < cap ? n_rows : cap);
         if (grid >= 64) grid &= ~7u;  // a multiple of the XCD count: one run of rows per XCD
-        snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "%s_%s", name, quant ? "u8" : "f32");
+        ctx->name_kernel("%s_%s", name, quant ? "u8" : "f32");
         ctx->sweep = 1;  // this kernel walks the rows forward: its consumer should start at the end
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), (size_t)lds, ctx->stream, p,
                            (int)row_floats, n_rows);

@@ -435,7 +435,7 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 template <int S, int TH, int TW>
 static void launch_dw3x3(tfhip_ctx* ctx, DwArgs& p) {
-  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise3x3_s%d_%dx%d", S, TH, TW);
+  ctx->name_kernel("depthwise3x3_s%d_%dx%d", S, TH, TW);
   p.tiles_h = (int)ceil_div(p.ci.out_h, TH);
   p.tiles_w = (int)ceil_div(p.ci.out_w, TW);
   const int64_t total = (int64_t)p.ci.batch * p.tiles_h * p.tiles_w * p.c4;
@@ -446,7 +446,7 @@ static void launch_dw3x3(tfhip_ctx* ctx, DwArgs& p) {
 
 template <int TW>
 static void launch_dw3x3_rows(tfhip_ctx* ctx, DwArgs& p, int rows) {
-  snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise3x3_s1_rows_w%d", TW);
+  ctx->name_kernel("depthwise3x3_s1_rows_w%d", TW);
   const int chunks = (int)ceil_div(p.ci.out_h, rows);
   p.tiles_w = (int)ceil_div(p.ci.out_w, TW);
   const int64_t total = (int64_t)p.ci.batch * chunks * p.tiles_w * p.c4;
@@ -499,7 +499,7 @@ static int dispatch_depthwise(tfhip_ctx* ctx, DwArgs& p, const tfhip_conv2d_info
       launch_dw3x3<2, 1, 1>(ctx, p);
     }
   } else {
-    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "depthwise_generic");
+    ctx->name_kernel("depthwise_generic");
     const int64_t blocks = ceil_div(o_n, 256);
     const int64_t cap = (int64_t)ctx->num_cus * 16;
     hipLaunchKernelGGL(depthwise_generic_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)),
@@ -613,14 +613,14 @@ extern "C" int tfhip_pool2d(tfhip_ctx* ctx, int64_t x, int64_t out, const tfhip_
                       ci->pad_left == 0 && ci->dilation_h == 1 && ci->dilation_w == 1 &&
                       ci->in_c % 4 == 0 && aligned16(xf) && aligned16(y);
   if (global) {
-    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "global_avgpool");
+    ctx->name_kernel("global_avgpool");
     const int items = ci->batch * (ci->in_c / 4);
     hipLaunchKernelGGL(global_avgpool_kernel, dim3((unsigned)ceil_div(items, 64)), dim3(64), 0,
                        ctx->stream, xf, y, ci->batch, ci->in_h * ci->in_w, ci->in_c / 4);
   } else {
     const int64_t blocks = ceil_div(o_n, 256);
     const int64_t cap = (int64_t)ctx->num_cus * 16;
-    snprintf(ctx->last_kernel, sizeof ctx->last_kernel, "pool2d");
+    ctx->name_kernel("pool2d");
     hipLaunchKernelGGL(pool2d_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0,
                        ctx->stream, xf, y, *ci, kind);
   }

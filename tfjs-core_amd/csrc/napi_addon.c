@@ -11,6 +11,7 @@
 #include <node_api.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "tfjs_hip.h"
@@ -161,6 +162,20 @@ static int arg_conv_info(napi_env env, napi_value v, tfhip_conv2d_info* ci) {
 #define F64(i, name) double name; if (!arg_f64(env, argv[i], &name)) return NULL
 #define CHECK(rc) do { int rc_ = (rc); if (rc_) return throw_status(env, ctx, rc_); } while (0)
 
+/* contexts that js_destroy has not seen yet: a read may finish after its backend is gone */
+#define MAX_LIVE 64
+static tfhip_ctx* live_ctx[MAX_LIVE];
+static void ctx_born(tfhip_ctx* c) {
+  for (int i = 0; i < MAX_LIVE; i++) if (!live_ctx[i]) { live_ctx[i] = c; return; }
+}
+static void ctx_died(tfhip_ctx* c) {
+  for (int i = 0; i < MAX_LIVE; i++) if (live_ctx[i] == c) live_ctx[i] = NULL;
+}
+static int ctx_alive(tfhip_ctx* c) {
+  for (int i = 0; i < MAX_LIVE; i++) if (live_ctx[i] == c) return 1;
+  return 0;
+}
+
 /* ---- context / storage ------------------------------------------------------------- */
 /* Contexts are destroyed explicitly by backend.dispose() (KernelBackend.dispose,
  * backend.ts:646); the external carries no finalizer so a context still referenced by
@@ -173,6 +188,7 @@ static napi_value js_init(napi_env env, napi_callback_info info) {
   tfhip_ctx* ctx = NULL;
   int rc = tfhip_init(device, &ctx);
   if (rc) return throw_status(env, NULL, rc);
+  ctx_born(ctx);
   napi_value ext;
   NAPI_OK(env, napi_create_external(env, ctx, NULL, NULL, &ext));
   return ext;
@@ -180,6 +196,7 @@ static napi_value js_init(napi_env env, napi_callback_info info) {
 
 static napi_value js_destroy(napi_env env, napi_callback_info info) {
   ARGS(1);
+  ctx_died(ctx);
   tfhip_destroy(ctx);
   return undefined(env);
 }
@@ -250,6 +267,132 @@ static napi_value js_time_end(napi_env env, napi_callback_info info) {
   napi_value v;
   NAPI_OK(env, napi_create_double(env, ms, &v));
   return v;
+}
+
+/* timeKernels(ctx) -> [[name, ms], ...] of the time() region that ended last */
+static napi_value js_time_kernels(napi_env env, napi_callback_info info) {
+  ARGS(1);
+  int n = 0;
+  CHECK(tfhip_time_kernel_count(ctx, &n));
+  napi_value arr;
+  NAPI_OK(env, napi_create_array_with_length(env, (size_t)n, &arr));
+  for (int i = 0; i < n; i++) {
+    const char* name = "";
+    float ms = 0;
+    CHECK(tfhip_time_kernel(ctx, i, &name, &ms));
+    napi_value pair, vn, vm;
+    NAPI_OK(env, napi_create_array_with_length(env, 2, &pair));
+    NAPI_OK(env, napi_create_string_utf8(env, name, NAPI_AUTO_LENGTH, &vn));
+    NAPI_OK(env, napi_create_double(env, ms, &vm));
+    napi_set_element(env, pair, 0, vn);
+    napi_set_element(env, pair, 1, vm);
+    napi_set_element(env, arr, (uint32_t)i, pair);
+  }
+  return arr;
+}
+
+static napi_value js_time_per_kernel(napi_env env, napi_callback_info info) {
+  ARGS(2);
+  INT(1, enable);
+  CHECK(tfhip_time_per_kernel(ctx, enable));
+  return undefined(env);
+}
+
+/* hostAlloc(nbytes) -> ArrayBuffer over pinned host memory (freed when it is collected) */
+static void free_pinned(napi_env env, void* data, void* hint) {
+  (void)env; (void)hint;
+  tfhip_host_free(data);
+}
+
+static napi_value js_host_alloc(napi_env env, napi_callback_info info) {
+  napi_value argv[MAX_ARGS];
+  if (!get_args(env, info, 1, argv)) return NULL;
+  double nbytes;
+  if (!arg_f64(env, argv[0], &nbytes)) return NULL;
+  void* p = NULL;
+  if (nbytes < 1 || tfhip_host_alloc((size_t)nbytes, &p) != TFHIP_OK) {
+    napi_throw_error(env, NULL, "hip backend: could not allocate pinned host memory");
+    return NULL;
+  }
+  napi_value buf;
+  if (napi_create_external_arraybuffer(env, p, (size_t)nbytes, free_pinned, NULL, &buf) != napi_ok) {
+    tfhip_host_free(p);
+    napi_throw_error(env, NULL, "tfjs_hip.node: could not wrap pinned memory");
+    return NULL;
+  }
+  return buf;
+}
+
+/* readAsync(ctx, id) -> Promise<ArrayBuffer>: the copy is queued here, a worker of the thread
+ * pool waits for it, and the promise resolves on the JavaScript thread
+ * (KernelBackend.read, backend.ts:33-35). */
+typedef struct {
+  tfhip_ctx* ctx;
+  tfhip_pending_read* ticket;
+  size_t nbytes;
+  int wait_rc;
+  napi_deferred deferred;
+  napi_async_work work;
+} read_job;
+
+static void read_execute(napi_env env, void* data) {
+  (void)env;
+  read_job* job = (read_job*)data;
+  job->wait_rc = tfhip_read_wait(job->ticket);
+}
+
+static void read_complete(napi_env env, napi_status status, void* data) {
+  read_job* job = (read_job*)data;
+  tfhip_ctx* ctx = ctx_alive(job->ctx) ? job->ctx : NULL;
+  napi_value result = NULL, err = NULL, msg;
+  void* dst = NULL;
+  int rc = (status == napi_ok) ? job->wait_rc : TFHIP_EDEVICE;
+  if (rc == TFHIP_OK && napi_create_arraybuffer(env, job->nbytes, &dst, &result) != napi_ok) {
+    rc = TFHIP_EDEVICE;
+    dst = NULL;
+  }
+  int frc = tfhip_read_finish(ctx, job->ticket, rc == TFHIP_OK ? dst : NULL, job->nbytes);
+  if (rc == TFHIP_OK) rc = frc;
+  if (rc == TFHIP_OK) {
+    napi_resolve_deferred(env, job->deferred, result);
+  } else {
+    const char* text = ctx ? tfhip_last_error(ctx) : "";
+    napi_create_string_utf8(env, (text && text[0]) ? text : "hip backend: asynchronous read failed",
+                            NAPI_AUTO_LENGTH, &msg);
+    napi_create_error(env, NULL, msg, &err);
+    napi_reject_deferred(env, job->deferred, err);
+  }
+  napi_delete_async_work(env, job->work);
+  free(job);
+}
+
+static napi_value js_read_async(napi_env env, napi_callback_info info) {
+  ARGS(3);
+  I64(1, id);
+  F64(2, nbytes);
+  read_job* job = (read_job*)calloc(1, sizeof *job);
+  if (!job) {
+    napi_throw_error(env, NULL, "tfjs_hip.node: out of memory");
+    return NULL;
+  }
+  job->ctx = ctx;
+  job->nbytes = (size_t)nbytes;
+  int rc = tfhip_read_begin(ctx, id, &job->ticket);
+  if (rc) {
+    free(job);
+    return throw_status(env, ctx, rc);
+  }
+  napi_value promise, name;
+  if (napi_create_promise(env, &job->deferred, &promise) != napi_ok ||
+      napi_create_string_utf8(env, "tfhip.read", NAPI_AUTO_LENGTH, &name) != napi_ok ||
+      napi_create_async_work(env, NULL, name, read_execute, read_complete, job, &job->work) != napi_ok ||
+      napi_queue_async_work(env, job->work) != napi_ok) {
+    tfhip_read_finish(ctx, job->ticket, NULL, 0);
+    free(job);
+    napi_throw_error(env, NULL, "tfjs_hip.node: could not queue the read");
+    return NULL;
+  }
+  return promise;
 }
 
 static napi_value js_last_kernel(napi_env env, napi_callback_info info) {
@@ -653,7 +796,9 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"init", js_init}, {"destroy", js_destroy}, {"register", js_register},
       {"write", js_write}, {"read", js_read}, {"dispose", js_dispose},
       {"memInfo", js_mem_info}, {"sync", js_sync}, {"timeBegin", js_time_begin},
-      {"timeEnd", js_time_end}, {"lastKernel", js_last_kernel}, {"matmul", js_matmul},
+      {"timeEnd", js_time_end}, {"timeKernels", js_time_kernels},
+      {"timePerKernel", js_time_per_kernel}, {"hostAlloc", js_host_alloc},
+      {"readAsync", js_read_async}, {"lastKernel", js_last_kernel}, {"matmul", js_matmul},
       {"conv2d", js_conv2d}, {"depthwiseConv2d", js_depthwise}, {"pool2d", js_pool2d},
       {"binary", js_binary}, {"unary", js_unary}, {"cast", js_cast}, {"copy", js_copy},
       {"dequantize", js_dequantize}, {"fill", js_fill}, {"reduce", js_reduce},

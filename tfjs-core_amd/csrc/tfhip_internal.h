@@ -5,7 +5,9 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstring>
 #include <map>
+#include <mutex>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -22,6 +24,14 @@ struct Buf {
   int64_t numel = 0;
   int rank = 0;
   int32_t shape[8] = {0};
+  // Ordering between the compute stream and the copy streams (see tfhip_ctx::upload):
+  hipEvent_t ready = nullptr;      // compute work that last read the block, recorded when it went
+                                   // back to the pool: a copy stream waits for it before overwriting
+  hipEvent_t uploaded = nullptr;   // a copy on the upload stream that the first consumer waits for
+  hipEvent_t read_done = nullptr;  // the last asynchronous read of this buffer (owned by its ticket)
+  bool recycled = false;           // the block came out of the pool (its history is unknown)
+  bool used = false;               // queued work may have touched the buffer since it was written
+  bool upload_target = false;      // written through the upload stream: worth an event on release
 };
 
 inline size_t dtype_size(int dtype) {
@@ -30,19 +40,70 @@ inline size_t dtype_size(int dtype) {
 
 }  // namespace tfhip
 
+// An asynchronous read between tfhip_read_begin and tfhip_read_finish.  Self-contained, so that
+// a thread which only waits (tfhip_read_wait) never looks into the context.
+struct tfhip_pending_read {
+  int device = 0;
+  size_t nbytes = 0;
+  void* staging = nullptr;  // pinned; the device copies into it on the download stream
+  size_t staging_cap = 0;
+  hipEvent_t done = nullptr;  // recorded behind that copy
+  bool failed = false;
+};
+
 // One device, one in-order stream, one size-bucketed pool of device blocks.  Freed blocks
 // go back to the pool at once: every consumer is queued on the same stream, so a block
 // handed out again can only be touched after the work that last used it.
 struct tfhip_ctx {
   int device = 0;
-  hipStream_t stream = nullptr;
-  hipEvent_t ev_begin = nullptr, ev_end = nullptr;
-  bool timing = false;
+  hipStream_t stream = nullptr;  // every kernel runs here, in order
+  // Copies that overlap with kernels: host-to-device on `upload`, asynchronous reads on
+  // `download` (both at the default priority).  Events carry the order between the three.
+  hipStream_t upload = nullptr, download = nullptr;
+  std::vector<hipEvent_t> free_events;  // untimed events, reused
+  hipEvent_t ev_get();
+  void ev_put(hipEvent_t ev) {
+    if (ev) free_events.push_back(ev);
+  }
+  std::unordered_map<void*, hipEvent_t> block_ready;  // pool block -> Buf::ready of its last owner
+  // Small writes travel through a ring of pinned slots on the compute stream itself.
+  static constexpr size_t kSlotBytes = 64 << 10;
+  static constexpr int kSlots = 32;
+  char* ring = nullptr;
+  hipEvent_t ring_done[kSlots] = {nullptr};
+  int ring_next = 0;
+  std::unordered_map<tfhip_pending_read*, int64_t> reads;  // asynchronous reads not yet finished
   std::unordered_map<int64_t, tfhip::Buf> bufs;
   std::map<size_t, std::vector<void*>> pool;  // capacity -> free blocks, reused LIFO
   size_t in_use = 0, pooled = 0;
   std::string err;
   char last_kernel[96] = "";  // variant chosen by the last dense / image launch
+  bool kernel_named = false;  // last_kernel was written for the launch that is being queued
+  void name_kernel(const char* fmt, ...);
+
+  // KernelBackend.time with per-kernel figures (backends/backend.ts:27-31): while a time()
+  // region is open every launch is followed by an event on the stream (a "mark"); the time of
+  // a kernel is the distance between its mark and the one before it, so the figures of a
+  // region add up to its total and include whatever the device idled before that kernel.
+  // Regions nest: each remembers the mark it started at.
+  static constexpr int kMaxMarks = 1 << 16;
+  static constexpr int kMaxTimeDepth = 8;
+  struct KernelTime {
+    std::string name;
+    float ms;
+  };
+  std::vector<hipEvent_t> mark_events;  // created on demand, reused by later regions
+  std::vector<std::string> mark_names;
+  int marks_used = 0, marks_dropped = 0;
+  int time_stack[kMaxTimeDepth];
+  int time_depth = 0;
+  bool per_kernel = true;
+  std::vector<KernelTime> kernel_times;  // of the region that ended last
+  int mark(const char* name);  // index of the new mark, -1 when none could be recorded
+  void after_launch(const char* func) {
+    if (time_depth && per_kernel && !capturing) mark(kernel_named ? last_kernel : func);
+    kernel_named = false;
+  }
   int num_cus = 256;
   // Direction in which the next row-sweeping kernel should walk its rows: 1 = from the end.
   // A kernel leaves the rows it wrote last in the L2 of the XCD that wrote them (32 MB over the
@@ -72,9 +133,15 @@ struct tfhip_ctx {
   int64_t next_graph = 1;
 
   int fail(int code, const char* fmt, ...);
-  tfhip::Buf* find(int64_t id);          // sets err when missing
-  void* alloc(size_t nbytes, size_t* cap);  // nullptr + err on failure (nbytes > 0)
-  void release(void* p, size_t cap);
+  // Looks an id up (sets err when missing).  `touch` = the caller queues work on the compute
+  // stream that reads or writes the buffer: a pending upload is waited for first.
+  tfhip::Buf* find(int64_t id, bool touch = true);
+  // nullptr + err on failure (nbytes > 0).  *ready receives the event that the block's last
+  // owner left with it, or nullptr; *recycled whether the block was used before.
+  void* alloc(size_t nbytes, size_t* cap, hipEvent_t* ready = nullptr, bool* recycled = nullptr);
+  void release(void* p, size_t cap, hipEvent_t ready = nullptr);
+  void release_buf(tfhip::Buf& b);
+  int await_uploads();  // the compute stream waits for every upload still on its way
   void trim();
 };
 
@@ -89,7 +156,19 @@ struct tfhip_ctx {
   tfhip::Buf* var = (ctx)->find(id);      \
   if (!var) return TFHIP_ENOENT
 
-#define TFHIP_LAUNCH_CHECK(ctx) TFHIP_HIP(ctx, hipGetLastError())
+// After every kernel launch: report a launch error, and note the launch for an open time() region.
+#define TFHIP_LAUNCH_CHECK(ctx)            \
+  do {                                     \
+    TFHIP_HIP(ctx, hipGetLastError());     \
+    (ctx)->after_launch(__func__);         \
+  } while (0)
+// The same for a launch that has a name of its own (a second kernel of one call).
+#define TFHIP_LAUNCH_CHECK_NAMED(ctx, name) \
+  do {                                      \
+    TFHIP_HIP(ctx, hipGetLastError());      \
+    (ctx)->kernel_named = false;            \
+    (ctx)->after_launch(name);              \
+  } while (0)
 
 namespace tfhip {
 

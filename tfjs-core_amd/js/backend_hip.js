@@ -71,7 +71,6 @@ class MathBackendHIP extends KernelBackend {
     this.ctx = this.napi.init(device == null ? ENV.get('HIP_DEVICE') : device);
     this.data = new DataStorage(this, ENGINE);
     this.nextHandle = 1;
-    this.pendingReads = 0;
   }
 
   // ---- storage (backend.ts:33-44; CPU behaviour backend_cpu.ts:102-129, 199-254) ----
@@ -87,6 +86,13 @@ class MathBackendHIP extends KernelBackend {
     this.data.set(dataId, {handle, code, size: util.sizeFromShape(stored)});
   }
 
+  // Up to 64 KiB the bytes are staged and the call returns at once; a larger array is copied on
+  // a stream of its own, so that the upload overlaps with kernels already queued, and the first
+  // kernel that reads the tensor waits for it.  From an array made by pinnedArray() the copy
+  // is a DMA straight out of the caller's memory and the call returns before it has run: the
+  // record keeps the array (as the reference's CPU backend keeps the values it is given,
+  // backend_cpu.ts:122-129) and the caller leaves it unchanged until a result that depends on
+  // it has been read.
   write(dataId, values) {
     if (values == null) throw new Error('MathBackendHIP.write(): values can not be null');
     const rec = this.data.get(dataId);
@@ -95,6 +101,18 @@ class MathBackendHIP extends KernelBackend {
         rec.code === DTYPE.int32 ? Int32Array : Uint8Array;
     if (!(arr instanceof want)) arr = want.from(arr);
     this.napi.write(this.ctx, rec.handle, arr);
+    rec.source = arr.buffer != null && arr.buffer.hipPinned === true ? arr : null;
+  }
+
+  // A typed array over page-locked host memory (an extension): uploads out of it run at the
+  // full rate of the link and do not hold the JavaScript thread.
+  pinnedArray(dtype, length) {
+    const ctor = dtype === 'float32' ? Float32Array : dtype === 'int32' ? Int32Array :
+        dtype === 'bool' ? Uint8Array : null;
+    if (ctor == null) throw new Error(`hip backend: no pinned array of dtype ${dtype}`);
+    const buffer = this.napi.hostAlloc(Math.max(1, length) * ctor.BYTES_PER_ELEMENT);
+    buffer.hipPinned = true;
+    return new ctor(buffer, 0, length);
   }
 
   readSync(dataId) {
@@ -102,11 +120,19 @@ class MathBackendHIP extends KernelBackend {
     return this.napi.read(this.ctx, rec.handle, typedArrayFor(rec.code, rec.size));
   }
 
-  // The device queue is in order, so a read issued now sees every kernel queued before it;
-  // the copy itself completes inside the call and the promise resolves on the next tick.
+  // The copy is queued behind the kernels queued so far, on a stream of its own, into pinned
+  // staging memory; a worker thread waits for it and the promise resolves on this thread, which
+  // stays free to queue more work meanwhile (backend.ts:33-35).  The tensor may be disposed as
+  // soon as this returns.
   read(dataId) {
+    let rec;
     try {
-      return Promise.resolve(this.readSync(dataId));
+      rec = this.data.get(dataId);
+      const ctor = rec.code === DTYPE.float32 ? Float32Array :
+          rec.code === DTYPE.int32 ? Int32Array : Uint8Array;
+      if (rec.size === 0) return Promise.resolve(new ctor(0));
+      return this.napi.readAsync(this.ctx, rec.handle, rec.size * ctor.BYTES_PER_ELEMENT)
+          .then(buffer => new ctor(buffer, 0, rec.size));
     } catch (err) {
       return Promise.reject(err);
     }
@@ -159,7 +185,10 @@ class MathBackendHIP extends KernelBackend {
     };
   }
 
-  // Event pair on the backend's stream around everything f() queues (backend.ts:27-31).
+  // Device time of everything f() queues (backend.ts:27-31, 92).  Calls may nest.  While a
+  // region is open an event follows every kernel on the stream, which gives the time of each
+  // launch: getExtraProfileInfo() returns them as 'name: ms' pairs (the interface asks for a
+  // string), kernelTimes as [{name, ms}] in launch order.
   async time(f) {
     this.napi.timeBegin(this.ctx);
     let kernelMs;
@@ -168,7 +197,13 @@ class MathBackendHIP extends KernelBackend {
     } finally {
       kernelMs = this.napi.timeEnd(this.ctx);
     }
-    return {kernelMs, getExtraProfileInfo: () => this.napi.lastKernel(this.ctx)};
+    const kernelTimes = this.napi.timeKernels(this.ctx).map(([name, ms]) => ({name, ms}));
+    return {
+      kernelMs,
+      kernelTimes,
+      getExtraProfileInfo: () =>
+          kernelTimes.map(k => `${k.name}: ${k.ms.toFixed(4)}`).join(', ')
+    };
   }
 
   sync() { this.napi.sync(this.ctx); }

@@ -67,6 +67,11 @@ def time(f):
     return ENGINE.backend.time(f)
 
 
+def pinned_array(dtype, shape):
+    """Page-locked host array of the active backend (hip extension)."""
+    return ENGINE.backend.pinned_array(dtype, tuple(shape))
+
+
 def dispose(t):
     for x in (t if isinstance(t, (list, tuple)) else [t]):
         x.dispose()

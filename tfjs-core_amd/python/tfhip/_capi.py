@@ -47,6 +47,14 @@ _SIGNATURES = {
     "tfhip_sync": [_PTR],
     "tfhip_time_begin": [_PTR],
     "tfhip_time_end": [_PTR, C.POINTER(C.c_float)],
+    "tfhip_time_per_kernel": [_PTR, _INT],
+    "tfhip_time_kernel_count": [_PTR, C.POINTER(_INT)],
+    "tfhip_time_kernel": [_PTR, _INT, C.POINTER(C.c_char_p), C.POINTER(C.c_float)],
+    "tfhip_host_alloc": [C.c_size_t, C.POINTER(_PTR)],
+    "tfhip_host_free": [_PTR],
+    "tfhip_read_begin": [_PTR, _I64, C.POINTER(_PTR)],
+    "tfhip_read_wait": [_PTR],
+    "tfhip_read_finish": [_PTR, _PTR, _PTR, C.c_size_t],
     "tfhip_last_kernel": [_PTR],
     "tfhip_device_ptr": [_PTR, _I64, C.POINTER(_PTR), C.POINTER(C.c_size_t)],
     "tfhip_matmul": [_PTR, _I64, _I64, _I64, _INT, _INT, _INT, _INT, _INT, _INT, _I64, _INT, _INT,

@@ -53,6 +53,44 @@ class _CapturedGraph(object):
         self.gid = None
 
 
+class _PinnedBlock:
+    """Owns one tfhip_host_alloc block; numpy arrays made from .view keep it alive."""
+
+    def __init__(self, lib, address, nbytes):
+        self._lib, self._address = lib, address
+        self.view = (C.c_char * max(1, nbytes)).from_address(address)
+        self.view._owner = self  # the ctypes array is what numpy references
+
+    def __del__(self):
+        try:
+            self._lib.tfhip_host_free(self._address)
+        except Exception:
+            pass
+
+
+class _PendingRead:
+    def __init__(self, backend, ticket, out):
+        self._backend, self._ticket, self._out = backend, ticket, out
+
+    def result(self):
+        if self._ticket is not None:
+            b, ticket = self._backend, self._ticket
+            self._ticket = None
+            b.lib.tfhip_read_wait(ticket)  # releases the GIL while it waits
+            ctx = b.ctx if b.ctx else None
+            rc = b.lib.tfhip_read_finish(ctx, ticket, self._out.ctypes.data_as(C.c_void_p),
+                                         self._out.nbytes)
+            if rc != 0:
+                raise RuntimeError(b.lib.tfhip_last_error(ctx).decode() if ctx else
+                                   "hip backend: asynchronous read failed")
+        return self._out
+
+    def __del__(self):
+        if getattr(self, "_ticket", None) is not None:
+            b = self._backend
+            b.lib.tfhip_read_finish(b.ctx if b.ctx else None, self._ticket, None, 0)
+
+
 class MathBackendHIP(object):
     def __init__(self, device=0):
         self.lib = capi.lib()
@@ -94,7 +132,26 @@ class MathBackendHIP(object):
         return out
 
     def read(self, data_id):
-        return self.read_sync(data_id)
+        """The asynchronous read of KernelBackend.read (backend.ts:33-35): the copy is queued
+        behind the kernels queued so far, on a stream of its own, and the call returns at once
+        with a handle whose .result() waits for it; the tensor may be disposed meanwhile."""
+        h, code, numel = self.data[data_id]
+        ticket = C.c_void_p()
+        self._ck(self.lib.tfhip_read_begin(self.ctx, h, C.byref(ticket)))
+        return _PendingRead(self, ticket, np.empty(numel, _NP_OF_CODE[code]))
+
+    def pinned_array(self, dtype, shape):
+        """numpy array over page-locked host memory (an extension): tfhip_write out of it is a
+        DMA that returns at once and overlaps with the kernels queued before it.  The caller
+        leaves the array unchanged until a result that depends on it has been read."""
+        np_dtype = np.dtype(_NP_OF_CODE[_DTYPE_CODE[dtype]])
+        numel = int(np.prod(shape)) if len(shape) else 1
+        p = C.c_void_p()
+        if self.lib.tfhip_host_alloc(max(1, numel) * np_dtype.itemsize, C.byref(p)) != 0:
+            raise MemoryError("hip backend: could not allocate pinned host memory")
+        owner = _PinnedBlock(self.lib, p.value, numel * np_dtype.itemsize)
+        arr = np.frombuffer(owner.view, dtype=np_dtype, count=numel).reshape(shape)
+        return arr
 
     def dispose_data(self, data_id):
         rec = self.data.pop(data_id, None)
@@ -108,11 +165,25 @@ class MathBackendHIP(object):
                     numDeviceBuffers=c.value)
 
     def time(self, f):
+        """Device time of everything f() queues; calls may nest.  kernelTimes lists every launch
+        of the region in order as (kernel variant, ms): an event follows each kernel on the
+        stream while a region is open (BackendTimingInfo.getExtraProfileInfo, backend.ts:27-31)."""
         self._ck(self.lib.tfhip_time_begin(self.ctx))
-        f()
-        ms = C.c_float()
-        self._ck(self.lib.tfhip_time_end(self.ctx, C.byref(ms)))
-        return dict(kernelMs=ms.value)
+        try:
+            f()
+        finally:
+            ms = C.c_float()
+            rc = self.lib.tfhip_time_end(self.ctx, C.byref(ms))
+        self._ck(rc)
+        n = C.c_int()
+        self._ck(self.lib.tfhip_time_kernel_count(self.ctx, C.byref(n)))
+        kernels = []
+        for i in range(n.value):
+            name, k_ms = C.c_char_p(), C.c_float()
+            self._ck(self.lib.tfhip_time_kernel(self.ctx, i, C.byref(name), C.byref(k_ms)))
+            kernels.append((name.value.decode(), k_ms.value))
+        return dict(kernelMs=ms.value, kernelTimes=kernels,
+                    getExtraProfileInfo=lambda: ", ".join("%s: %.4f" % k for k in kernels))
 
     def sync(self):
         self._ck(self.lib.tfhip_sync(self.ctx))

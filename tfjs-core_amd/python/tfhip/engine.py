@@ -53,6 +53,20 @@ class Tensor(object):
             vals = vals.astype(np.uint8)
         return vals.reshape(self.shape)
 
+    def data(self):
+        """Tensor.data (tensor.ts:1060-1071): starts the read and returns at once; .result() of
+        the returned handle waits for the values (there is no event loop to resolve a promise
+        on).  The tensor may be disposed before the values are asked for."""
+        self._check()
+        pending = ENGINE.read(self.data_id)
+        shape, as_bool = self.shape, self.dtype == "bool"
+
+        class _Data(object):
+            def result(_self):
+                vals = pending.result()
+                return (vals.astype(np.uint8) if as_bool else vals).reshape(shape)
+        return _Data()
+
     def dispose(self):
         if not self.is_disposed:
             ENGINE.dispose_tensor(self)
@@ -158,6 +172,9 @@ class Engine(object):
 
     def read_sync(self, data_id):
         return self.ref[data_id][1].read_sync(data_id)
+
+    def read(self, data_id):
+        return self.ref[data_id][1].read(data_id)
 
     def dispose_tensor(self, t):
         rec = self.ref.get(t.data_id)
