@@ -10,10 +10,12 @@ ops/broadcast_util.ts:27-87 and ops/axis_util.ts:49-95.
 
 Pinning: every function below is checked against the known-answer vectors of the reference's
 own *_test.ts files (tests/test_oracle_golden.py) or against closed forms, identities and
-brute force (tests/test_oracle_math.py).  Parity unpinned: depthwise_conv2d with asymmetric
-padding on non-square inputs (the `pad_quirk` argument chooses between backend_cpu's row /
-column swap and the TensorFlow semantics; no reference vector tells them apart), and
-where_indices, which is numpy.argwhere and has no reference vector extracted.
+brute force (tests/test_oracle_math.py); where_indices against the whereAsync blocks of
+logical_ops_test.ts:742-780.  Parity unpinned: depthwise_conv2d with asymmetric padding on
+non-square inputs (the `pad_quirk` argument chooses between backend_cpu's row / column swap and
+the TensorFlow semantics; no reference vector tells them apart — pad_quirk=False is checked
+against a float64 grouped convolution, and pad_quirk=True is shown to differ from it, in
+tests/test_oracle_math.py).
 """
 import ctypes as C
 import math

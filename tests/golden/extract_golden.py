@@ -61,6 +61,7 @@ CASES = {
     "resize_nearest": ("tfjs-core/src/ops/resize_nearest_neighbor_test.ts",
                        ["resizeNearestNeighbor"]),
     "where": ("tfjs-core/src/ops/logical_ops_test.ts", ["where"]),
+    "where_async": ("tfjs-core/src/ops/logical_ops_test.ts", ["whereAsync"]),
     "array_extra": ("tfjs-core/src/ops/array_ops_test.ts",
                     ["stack", "unstack", "split", "expandDims"]),
     "mean": ("tfjs-core/src/ops/reduction_ops_test.ts", ["Reduction: mean"]),

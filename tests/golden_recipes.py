@@ -880,6 +880,19 @@ def resize_nearest_known_answers(ops):
 
 
 @recipe
+def where_async_known_answers(ops):
+    """logical_ops_test.ts:742-780: coordinates of the true elements, int32, row-major."""
+    for title in ("1d tensor", "2d tensor", "3d tensor"):
+        a = golden_case("where_async", title)["arrays"]
+        r = ops.where_indices(np.array(a[0], bool))
+        assert r.dtype == np.int32 and list(r.shape) == a[-2]
+        assert r.ravel().tolist() == a[-1]
+    a = golden_case("where_async", "returns tensor with 0 in shape when no values are true")["arrays"]
+    r = ops.where_indices(np.array(a[0], bool))
+    assert list(r.shape) == a[1] and r.size == 0
+
+
+@recipe
 def where_known_answers(ops):
     g = lambda t: golden_case("where", t)["arrays"]
     flat = lambda v: np.array(v).ravel()

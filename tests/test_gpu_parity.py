@@ -33,7 +33,8 @@ def ref(oracle):
 
 
 def rng_for(*key):
-    return np.random.default_rng(abs(hash(key)) % (2 ** 32))
+    import zlib
+    return np.random.default_rng(zlib.crc32(repr(key).encode()))  # the same in every process
 
 
 # ---------------------------------------------------------------- matmul ----
@@ -210,6 +211,36 @@ def test_depthwise_shapes(hip, ref, xs, fs, stride, pad, dil):
     for act in ("linear", "relu", "relu6"):
         close(hip.depthwise_conv2d(x, w, stride, pad, dil, bias=bias, activation=act),
               ref.depthwise_conv2d(x, w, stride, pad, dil, bias=bias, activation=act))
+
+
+@pytest.mark.parametrize("xs", [(1, 8, 5, 8), (2, 9, 6, 4), (1, 8, 5, 6), (2, 30, 17, 32)])
+def test_depthwise_asymmetric_padding(hip, oracle, xs):
+    """padInfo.top != padInfo.left (3x3 stride 2 'same', height and width of different parity):
+    rows take the top padding and columns the left one, as TensorFlow and the reference's
+    WebGL backend do.  Checked against the oracle with pad_quirk=False and against a float64
+    convolution per channel; backend_cpu's swapped form (backend_cpu.ts:1999, 2010) must
+    differ, so the case does tell the two apart."""
+    print("depthwise asymmetric", xs, flush=True)
+    rng = rng_for("dw-asym", xs)
+    c = xs[3]
+    x = rng.uniform(0, 1, xs).astype(np.float32)
+    w = rng.standard_normal((3, 3, c, 1)).astype(np.float32)
+    bias = rng.standard_normal(c).astype(np.float32)
+    ci = oracle.compute_conv2d_info(xs, w.shape, 2, 1, "same", depthwise=True)
+    p = ci["padInfo"]
+    assert p["top"] != p["left"]
+    got = hip.depthwise_conv2d(x, w, 2, "same")
+    close(got, oracle.depthwise_conv2d(x, w, ci, pad_quirk=False))
+    xp = np.pad(x.astype(np.float64), ((0, 0), (p["top"], p["bottom"]), (p["left"], p["right"]), (0, 0)))
+    want = np.zeros(got.shape)
+    for i in range(3):
+        for j in range(3):
+            want += xp[:, i:i + 2 * ci["outHeight"] - 1:2, j:j + 2 * ci["outWidth"] - 1:2, :] * \
+                w[i, j, :, 0].astype(np.float64)
+    close(got, want)
+    assert np.abs(oracle.depthwise_conv2d(x, w, ci, pad_quirk=True) - want).max() > 1e-2
+    close(hip.depthwise_conv2d(x, w, 2, "same", bias=bias, activation="relu6"),
+          np.clip(want + bias, 0, 6))
 
 
 # ------------------------------------------------------------------ pool ----

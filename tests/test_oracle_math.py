@@ -91,6 +91,30 @@ def test_depthwise_is_grouped_conv(ops, stride, ch_mul, pad):
         rel_close(y[..., ch * ch_mul:(ch + 1) * ch_mul], dense, rel=1e-5)
 
 
+@pytest.mark.parametrize("shape", [(1, 8, 5, 8), (2, 9, 6, 4)])
+def test_depthwise_asymmetric_padding_against_grouped_float64(ops, oracle, shape):
+    """3x3 stride 2 'same' on an image whose height and width differ in parity pads the top and
+    the left differently (conv_util.ts:415-426).  With pad_quirk=False rows take padInfo.top
+    and columns padInfo.left: checked against a float64 direct convolution per channel.
+    backend_cpu applies them the other way round (backend_cpu.ts:1999, 2010), which
+    pad_quirk=True reproduces; the two must differ here, or this test pins nothing."""
+    rng = np.random.default_rng(55)
+    c = shape[3]
+    x = rng.uniform(0, 1, shape).astype(np.float32)
+    w = rng.standard_normal((3, 3, c, 1)).astype(np.float32)
+    ci = oracle.compute_conv2d_info(shape, w.shape, 2, 1, "same", depthwise=True)
+    p = ci["padInfo"]
+    assert p["top"] != p["left"]
+    want = np.concatenate(
+        [_conv_brute(x[..., ch:ch + 1], w[:, :, ch:ch + 1, :], 2, 2, 1, 1, p["top"], p["left"],
+                     ci["outHeight"], ci["outWidth"]) for ch in range(c)], -1)
+    plain = oracle.depthwise_conv2d(x, w, ci, pad_quirk=False)
+    rel_close(plain, want, rel=1e-5, ab=1e-5)
+    rel_close(ops.depthwise_conv2d(x, w, 2, "same"), want, rel=1e-5, ab=1e-5)
+    swapped = oracle.depthwise_conv2d(x, w, ci, pad_quirk=True)
+    assert np.abs(swapped.astype(np.float64) - want).max() > 1e-2
+
+
 def test_avg_pool_counts_only_in_bounds_pixels(ops):
     x = np.arange(1, 10, dtype=np.float32).reshape(1, 3, 3, 1)
     y = ops.avg_pool(x, 2, 1, "same")[0, :, :, 0]
