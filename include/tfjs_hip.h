@@ -178,6 +178,21 @@ enum {
 int tfhip_matmul(tfhip_ctx* ctx, int64_t a, int64_t b, int64_t out, int batch, int m, int n,
                  int k, int transpose_a, int transpose_b, int64_t bias, int bias_kind, int act,
                  int64_t prelu, int prelu_kind, const tfhip_qparams* q);
+/* tfhip_matmul for callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, same kernels and same results as tfhip_matmul; it calls no
+ * hipMalloc / hipFree and takes no block from the pool.  Where tfhip_matmul would take scratch
+ * memory from the pool (the partial tiles of a product that is cut along K because it has too
+ * few tiles to fill the GPU), this entry point uses a static device array of 8 MiB that the
+ * library holds on every GPU it runs on until the process ends.  A product whose partial
+ * tiles need more fails with TFHIP_ENOTSUP, as does an operand that is not stored as float32
+ * (its converted copy would need a block; b may be TFHIP_UINT8Q).  All calls on one GPU share
+ * the array: calls that overlap on one GPU (two contexts, two threads) race on it; calls on
+ * one context are ordered by its stream. */
+int tfhip_matmul_noalloc(tfhip_ctx* ctx, int64_t a, int64_t b, int64_t out, int batch, int m,
+                         int n, int k, int transpose_a, int transpose_b, int64_t bias,
+                         int bias_kind, int act, int64_t prelu, int prelu_kind,
+                         const tfhip_qparams* q);
 /* conv2d / fusedConv2d (backend.ts:414-421; backend_cpu.ts:1536-1616): x NHWC,
  * filter [fh,fw,in_c,out_c], out NHWC float32.  bias/prelu/q as for tfhip_matmul with
  * N = out_c and rows = batch*out_h*out_w. */

@@ -87,6 +87,10 @@ int tfhip_ctx::mark(const char* name) {
     }
   }
   if (marks_used == (int)mark_events.size()) {
+    if (no_alloc) {  // no new event inside a call that promises to create nothing
+      marks_dropped++;
+      return -1;
+    }
     hipEvent_t ev;
     hipError_t e = hipEventCreate(&ev);
     if (e != hipSuccess) {
@@ -152,6 +156,10 @@ hipEvent_t tfhip_ctx::ev_get() {
 }
 
 void* tfhip_ctx::alloc(size_t nbytes, size_t* cap, hipEvent_t* ready, bool* recycled) {
+  if (no_alloc) {  // a mistake in the library, not in the caller: fail instead of allocating
+    fail(TFHIP_EDEVICE, "internal: a no-alloc entry point asked the pool for %zu bytes", nbytes);
+    return nullptr;
+  }
   const size_t want = tfhip::round_cap(nbytes);
   if (ready) *ready = nullptr;
   if (recycled) *recycled = false;
@@ -305,6 +313,14 @@ int tfhip_init(int device, tfhip_ctx** out) {
     return TFHIP_ENOTSUP;
   }
   ctx->num_cus = prop.multiProcessorCount;
+  if (tfhip::scratch_init(ctx) != TFHIP_OK) {
+    g_init_error = ctx->err;
+    (void)hipStreamDestroy(ctx->stream);
+    (void)hipStreamDestroy(ctx->upload);
+    (void)hipStreamDestroy(ctx->download);
+    delete ctx;
+    return TFHIP_EDEVICE;
+  }
   *out = ctx;
   return TFHIP_OK;
 }

@@ -1287,6 +1287,39 @@ static Plan make_plan(const GemmArgs& p, int batch, int bm, int bn, int resident
   return pl;
 }
 
+// Scratch memory of tfhip_matmul_noalloc: a static device array, one copy per GPU, that takes
+// the place of the pool block in which a product cut along K keeps its partial tiles.  Host
+// code reaches it only through the address hipGetSymbolAddress returns for the current
+// device (the array's name is not a device address on the host), asked once per device.
+constexpr size_t kScratchBytes = 8u << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+static void* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mu;
+
+int scratch_init(tfhip_ctx* ctx) {
+  if (ctx->device < 0 || ctx->device >= kMaxDevices)
+    return ctx->fail(TFHIP_EINVAL, "device index %d beyond %d", ctx->device, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[ctx->device]) {
+    void* ptr = nullptr;
+    // (the context's device is current: tfhip_init has just selected it)
+    hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      return ctx->fail(TFHIP_EDEVICE, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    }
+    g_scratch_ptr[ctx->device] = ptr;
+  }
+  ctx->scratch = g_scratch_ptr[ctx->device];
+  return TFHIP_OK;
+}
+
+static void* scratch_address(tfhip_ctx* ctx) {
+  if (!ctx->scratch) ctx->fail(TFHIP_EDEVICE, "static scratch memory was not set up");
+  return ctx->scratch;
+}
+
 template <class T, int AMODE, int BMODE, bool KBLOCKED, bool FAST>
 static int resident_blocks(tfhip_ctx* ctx) {
   static int cached = 0;
@@ -1323,9 +1356,20 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
   Temp partials(ctx);
   p.partials = nullptr;
   if (pl.splits > 1) {
-    if (!partials.get((size_t)pl.tail_tiles * pl.splits * T::BM * T::BN * sizeof(float)))
-      return TFHIP_EDEVICE;
-    p.partials = static_cast<float*>(partials.ptr);
+    const size_t need = (size_t)pl.tail_tiles * pl.splits * T::BM * T::BN * sizeof(float);
+    if (ctx->no_alloc) {
+      // the partial tiles go into the library's static device array instead of a pool block
+      if (need > kScratchBytes)
+        return ctx->fail(TFHIP_ENOTSUP,
+                         "matmul_noalloc: this product is cut along K and its partial tiles take "
+                         "%zu bytes, more than the %zu bytes of static scratch memory; use "
+                         "tfhip_matmul", need, kScratchBytes);
+      p.partials = static_cast<float*>(scratch_address(ctx));
+      if (!p.partials) return TFHIP_EDEVICE;
+    } else {
+      if (!partials.get(need)) return TFHIP_EDEVICE;
+      p.partials = static_cast<float*>(partials.ptr);
+    }
   }
   hipLaunchKernelGGL((gemm_kernel<T::WM, T::WN, T::TM, T::TN, AMODE, BMODE, KBLOCKED, FAST>),
                      dim3(pl.grid), dim3(T::WM * T::WN * 64), 0, ctx->stream, p);
@@ -1494,11 +1538,50 @@ static int epilogue_operand(tfhip_ctx* ctx, const char* what, int64_t id, int ki
 
 using namespace tfhip;
 
+static int matmul_impl(tfhip_ctx* ctx, int64_t a, int64_t b, int64_t out, int batch,
+                            int m, int n, int k, int transpose_a, int transpose_b,
+                            int64_t bias, int bias_kind, int act, int64_t prelu,
+                            int prelu_kind, const tfhip_qparams* q);
+
 extern "C" int tfhip_matmul(tfhip_ctx* ctx, int64_t a, int64_t b, int64_t out, int batch,
                             int m, int n, int k, int transpose_a, int transpose_b,
                             int64_t bias, int bias_kind, int act, int64_t prelu,
                             int prelu_kind, const tfhip_qparams* q) {
   if (!ctx) return TFHIP_EINVAL;
+  return matmul_impl(ctx, a, b, out, batch, m, n, k, transpose_a, transpose_b, bias, bias_kind,
+                     act, prelu, prelu_kind, q);
+}
+
+// The same product for callers that must not allocate device memory.  Nothing here or below
+// takes a block from the pool or asks the driver for memory: operands have to be stored as
+// float32 already (a converted copy would need a block), and the partial tiles of a product
+// cut along K live in the static array `scratch`.
+extern "C" int tfhip_matmul_noalloc(tfhip_ctx* ctx, int64_t a, int64_t b, int64_t out, int batch,
+                                    int m, int n, int k, int transpose_a, int transpose_b,
+                                    int64_t bias, int bias_kind, int act, int64_t prelu,
+                                    int prelu_kind, const tfhip_qparams* q) {
+  if (!ctx) return TFHIP_EINVAL;
+  const int64_t ids[4] = {a, b, bias_kind != TFHIP_BCAST_NONE ? bias : -1,
+                          (act == TFHIP_ACT_PRELU && prelu_kind != TFHIP_BCAST_NONE) ? prelu : -1};
+  for (int i = 0; i < 4; i++) {
+    if (ids[i] < 0 && i >= 2) continue;
+    TFHIP_GET(ctx, buf, ids[i]);
+    if (buf->dtype != TFHIP_FLOAT32 && !(i == 1 && buf->dtype == TFHIP_UINT8Q))
+      return ctx->fail(TFHIP_ENOTSUP, "matmul_noalloc: operand %d is not stored as float32 (a "
+                                      "converted copy would need device memory); use tfhip_matmul",
+                       i);
+  }
+  ctx->no_alloc = true;
+  const int rc = matmul_impl(ctx, a, b, out, batch, m, n, k, transpose_a, transpose_b, bias,
+                             bias_kind, act, prelu, prelu_kind, q);
+  ctx->no_alloc = false;
+  return rc;
+}
+
+static int matmul_impl(tfhip_ctx* ctx, int64_t a, int64_t b, int64_t out, int batch,
+                            int m, int n, int k, int transpose_a, int transpose_b,
+                            int64_t bias, int bias_kind, int act, int64_t prelu,
+                            int prelu_kind, const tfhip_qparams* q) {
   TFHIP_GET(ctx, ba, a);
   TFHIP_GET(ctx, bb, b);
   TFHIP_GET(ctx, bo, out);

@@ -416,6 +416,19 @@ static napi_value js_matmul(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+/* matmulNoalloc: the same arguments; allocates no device memory (tfhip_matmul_noalloc) */
+static napi_value js_matmul_noalloc(napi_env env, napi_callback_info info) {
+  ARGS(16);
+  I64(1, a); I64(2, b); I64(3, out);
+  INT(4, batch); INT(5, m); INT(6, n); INT(7, k); INT(8, ta); INT(9, tb);
+  I64(10, bias); INT(11, bias_kind); INT(12, act); I64(13, prelu); INT(14, prelu_kind);
+  tfhip_qparams q; const tfhip_qparams* qp;
+  if (!arg_qparams(env, argv[15], &q, &qp)) return NULL;
+  CHECK(tfhip_matmul_noalloc(ctx, a, b, out, batch, m, n, k, ta, tb, bias, bias_kind, act, prelu,
+                             prelu_kind, qp));
+  return undefined(env);
+}
+
 /* conv2d(ctx, x, filter, out, info, bias, biasKind, act, prelu, preluKind, q) */
 static napi_value js_conv2d(napi_env env, napi_callback_info info) {
   ARGS(11);
@@ -798,7 +811,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"memInfo", js_mem_info}, {"sync", js_sync}, {"timeBegin", js_time_begin},
       {"timeEnd", js_time_end}, {"timeKernels", js_time_kernels},
       {"timePerKernel", js_time_per_kernel}, {"hostAlloc", js_host_alloc},
-      {"readAsync", js_read_async}, {"lastKernel", js_last_kernel}, {"matmul", js_matmul},
+      {"readAsync", js_read_async}, {"lastKernel", js_last_kernel}, {"matmul", js_matmul}, {"matmulNoalloc", js_matmul_noalloc},
       {"conv2d", js_conv2d}, {"depthwiseConv2d", js_depthwise}, {"pool2d", js_pool2d},
       {"binary", js_binary}, {"unary", js_unary}, {"cast", js_cast}, {"copy", js_copy},
       {"dequantize", js_dequantize}, {"fill", js_fill}, {"reduce", js_reduce},

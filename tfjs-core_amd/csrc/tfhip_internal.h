@@ -132,6 +132,11 @@ struct tfhip_ctx {
   std::unordered_map<int64_t, Graph> graphs;
   int64_t next_graph = 1;
 
+  // tfhip_matmul_noalloc: this device's copy of the library's static scratch array (asked from
+  // the driver once, at init), and the flag that routes scratch needs there while it runs.
+  void* scratch = nullptr;
+  bool no_alloc = false;
+
   int fail(int code, const char* fmt, ...);
   // Looks an id up (sets err when missing).  `touch` = the caller queues work on the compute
   // stream that reads or writes the buffer: a pending upload is waited for first.
@@ -192,6 +197,9 @@ struct Temp {
 // converted copy in `tmp` (int32 / bool storage under a float32 tensor: widening casts
 // alias the same data id, backends/backend_util.ts:49-55).
 int as_f32(tfhip_ctx* ctx, const Buf* b, Temp* tmp, const float** out);
+
+// gemm.hip: looks up this device's address of the static scratch array (tfhip_init calls it)
+int scratch_init(tfhip_ctx* ctx);
 
 // elementwise.hip
 int launch_convert(tfhip_ctx* ctx, const void* src, int src_dtype, void* dst, int dst_dtype,

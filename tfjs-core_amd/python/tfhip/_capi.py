@@ -59,6 +59,8 @@ _SIGNATURES = {
     "tfhip_device_ptr": [_PTR, _I64, C.POINTER(_PTR), C.POINTER(C.c_size_t)],
     "tfhip_matmul": [_PTR, _I64, _I64, _I64, _INT, _INT, _INT, _INT, _INT, _INT, _I64, _INT, _INT,
                      _I64, _INT, C.POINTER(QParams)],
+    "tfhip_matmul_noalloc": [_PTR, _I64, _I64, _I64, _INT, _INT, _INT, _INT, _INT, _INT, _I64, _INT,
+                             _INT, _I64, _INT, C.POINTER(QParams)],
     "tfhip_conv2d": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC), _I64, _INT, _INT, _I64, _INT,
                      C.POINTER(QParams)],
     "tfhip_depthwise_conv2d": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC), _I64, _INT, _INT,
