@@ -4,9 +4,12 @@ pass per step through the tf.* graph on the hip backend (one MI355X).
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 64] [--quant] [--no-cpu]
 
-Prints ONE JSON line: whole-job images/s (inputs resident in HBM before the timed region),
-the roofline of the kernel that takes the largest share of the step, timed live with HIP
-events on the backend's stream, and the CPU oracle timed on this host beside it.
+Prints ONE JSON line.  `value` is the end-to-end rate: every step uploads its batch from host
+memory, runs the forward pass and reads the class probabilities back, with batch i+1 uploading
+while batch i computes; `resident_input` is the rate with the input already in HBM.  `roofline`
+prices the kernel variant that takes the largest share of the step from the times the kernels
+take inside the running step (a HIP event after every launch on the backend's stream);
+`cpu_baseline` is the CPU oracle timed on this host beside it.
 """
 import argparse
 import json
@@ -23,82 +26,63 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 RIDGE = PEAK_FP32_MFMA_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
 
-# HBM bytes per launch (fetch + write), averaged over the launches of each kernel variant in
-# one batch-64 step, from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised in
-# profiles/mobilenet_b64_fp32_hbm_traffic.txt (counters scaled by what a streaming kernel of
-# known size reads: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Counters cannot be read from inside
-# this process, so the figures are carried here; they apply to batch 64, fp32 weights.
-MIB = 1 << 20
-MEASURED_HBM_BYTES_PER_LAUNCH = {
-    "gemm_64x64_rowmajor_f32": 85.2 * MIB,
-    "gemm_rowstream_k32xn64_f32": 294.1 * MIB,
-    "gemm_64x128_rowmajor_f32": 35.4 * MIB,
-    "gemm_64x64_rowmajor_f32_tailk": 66.9 * MIB,
-    "depthwise3x3_s1_rows_w2": 87.6 * MIB,
-    "depthwise3x3_s2_1x1": 115.0 * MIB,
-    "conv_smallk_n32_f32": 135.0 * MIB,
-    "global_avgpool": 12.5 * MIB,
-}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "mobilenet_b64_fp32_hbm_traffic.txt")
+KERNEL_SOURCES = os.path.join(ROOT, "tfjs-core_amd", "csrc")
 
 
-def per_layer_times(tf, mobilenet, w, x, reps):
-    """Time every layer of the forward pass on its real input with an event pair on the
-    backend's stream around `reps` back-to-back launches.  Returns rows with the kernel
-    variant the library chose, its average duration and its algorithmic work."""
-    be = tf.backend()
-    rows = []
+def kernel_sources_sha1():
+    """Fingerprint of the device code: the traffic figures of a profile belong to the kernels
+    that were profiled, so the profile records this value and a run compares it."""
+    import hashlib
+    h = hashlib.sha1()
+    for name in sorted(os.listdir(KERNEL_SOURCES)):
+        if name.endswith((".hip", ".h")):
+            with open(os.path.join(KERNEL_SOURCES, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()
 
-    def timed(fn):
-        out = fn()            # warm-up launch, also yields the layer's output
-        tf.dispose(out)
-        def many():
-            for _ in range(reps):
-                tf.dispose(fn())
-        ms = tf.time(many)["kernelMs"] / reps
-        kernel = be.lib.tfhip_last_kernel(be.ctx).decode()
-        return fn(), ms, kernel
 
-    table = mobilenet.layer_table(batch=x.shape[0])
-    h = x
-    ti = iter(table)
-    keep = []
-    row = next(ti)
-    h2, ms, k = timed(lambda: tf.fused.conv2d(h, w["stem_w"], 2, "same", bias=w["stem_b"],
-                                              activation="relu6"))
-    rows.append(dict(row, ms=ms, kernel=k))
-    keep.append(h2)
-    h = h2
-    for i, (_, s) in enumerate(mobilenet.BLOCKS, 1):
-        row = next(ti)
-        hin = h
-        h2, ms, k = timed(lambda: tf.fused.depthwise_conv2d(
-            hin, w["dw%d_w" % i], s, "same", bias=w["dw%d_b" % i], activation="relu6"))
-        rows.append(dict(row, ms=ms, kernel=k))
-        keep.append(h2)
-        row = next(ti)
-        hmid = h2
-        h3, ms, k = timed(lambda: tf.fused.conv2d(
-            hmid, w["pw%d_w" % i], 1, "same", bias=w["pw%d_b" % i], activation="relu6"))
-        rows.append(dict(row, ms=ms, kernel=k))
-        keep.append(h3)
-        h = h3
-    row = next(ti)
-    hin = h
-    h2, ms, k = timed(lambda: tf.avg_pool(hin, (hin.shape[1], hin.shape[2]), 1, "valid"))
-    rows.append(dict(row, ms=ms, kernel=k))
-    keep.append(h2)
-    row = next(ti)
-    flat = tf.reshape(h2, (h2.shape[0], h2.shape[3]))
-    keep.append(flat)
-    h3, ms, k = timed(lambda: tf.fused.matmul(flat, w["fc_w"], False, False, bias=w["fc_b"]))
-    rows.append(dict(row, ms=ms, kernel=k))
-    keep.append(h3)
-    tf.dispose(keep)
-    return rows
+def measured_traffic():
+    """HBM bytes per launch of every kernel variant, read from the committed rocprofv3 counter
+    summary (FETCH_SIZE and WRITE_SIZE runs, scaled by a streaming kernel of known size; the
+    file states the commands).  Returns ({variant: bytes}, stale) where stale says that the
+    device code has changed since the profile was taken."""
+    import re
+    if not os.path.exists(TRAFFIC_PROFILE):
+        return {}, None
+    text = open(TRAFFIC_PROFILE).read()
+    out = {}
+    for m in re.finditer(r"^\s+(\S+)\s+launches\s+\d+\s+measured\s+([0-9.]+)\s+algorithmic", text, re.M):
+        out[m.group(1)] = float(m.group(2)) * (1 << 20)
+    m = re.search(r"kernel_sources_sha1:\s*([0-9a-f]{40})", text)
+    stale = True if m is None else m.group(1) != kernel_sources_sha1()
+    return out, stale
+
+
+def rows_of_one_step(kernel_times, table, batch):
+    """Pairs the launches of one step, in launch order, with the layers of the network.
+    kernel_times: [(kernel variant, ms)] from KernelBackend.time (an event after every launch on
+    the stream, so these are the times the kernels take inside the running step, inputs coming
+    from wherever the previous kernel left them).  The finishing launch of a product cut along K
+    is counted with its layer; the softmax launch is a row of its own."""
+    rows, layers = [], iter(table)
+    for name, ms in kernel_times:
+        if name == "splitk_finish":
+            rows[-1]["ms"] += ms
+            rows[-1]["launches"] += 1
+        elif name.startswith("tfhip_softmax"):
+            rows.append(dict(name="softmax", kind="softmax", macs=0, bytes=2 * 4 * batch * 1000,
+                             kernel="softmax_rows", ms=ms, launches=1))
+        else:
+            layer = next(layers, None)
+            if layer is None:
+                return None
+            rows.append(dict(layer, kernel=name, ms=ms, launches=1))
+    return rows if next(layers, None) is None else None
 
 
 def roofline_of_dominant_kernel(rows):
-    """Group the per-layer rows by kernel variant (what a profiler reports as one kernel
+    """Group the rows of one step by kernel variant (what a profiler reports as one kernel
     name), pick the variant with the largest share of the step, and price it: dense
     variants against the fp32 matrix peak, streaming variants against HBM."""
     groups = {}
@@ -112,7 +96,7 @@ def roofline_of_dominant_kernel(rows):
     name, g = max(groups.items(), key=lambda kv: kv[1]["ms"])
     ai = g["flops"] / g["bytes"]
     sec = g["ms"] * 1e-3
-    if name.startswith("gemm") and ai >= RIDGE:
+    if ai >= RIDGE:
         achieved = g["flops"] / sec / 1e12
         roof = dict(bound="mfma", achieved=round(achieved, 3), peak=PEAK_FP32_MFMA_TFLOPS,
                     unit="TFLOP/s", frac=round(achieved / PEAK_FP32_MFMA_TFLOPS, 4))
@@ -124,7 +108,8 @@ def roofline_of_dominant_kernel(rows):
                 avg_launch_us=round(g["ms"] * 1e3 / g["launches"], 2),
                 share_of_step=round(g["ms"] / sum(r["ms"] for r in rows), 3),
                 algorithmic_bytes_per_launch=round(g["bytes"] / g["launches"]),
-                algorithmic_flops_per_launch=round(g["flops"] / g["launches"]), traffic=None)
+                algorithmic_flops_per_launch=round(g["flops"] / g["launches"]), traffic=None,
+                timing="HIP event after every launch of the running step (KernelBackend.time)")
     return roof, groups
 
 
@@ -136,12 +121,14 @@ def op_level_configs(tf, np):
     be = tf.backend()
     rng = np.random.default_rng(1)
     out = []
+    be.lib.tfhip_time_per_kernel(be.ctx, 0)   # one event pair around each loop, none per launch
 
-    def timed(name, fn, reps, flops, nbytes):
-        tf.dispose(fn())
+    def timed(name, fn, reps, flops, nbytes, variants=1):
+        for v in range(variants):
+            tf.dispose(fn(v) if variants > 1 else fn())
         def many():
-            for _ in range(reps):
-                tf.dispose(fn())
+            for i in range(reps):
+                tf.dispose(fn(i % variants) if variants > 1 else fn())
         tf.time(many)                       # brings the clocks up
         ms = min(tf.time(many)["kernelMs"] for _ in range(3)) / reps
         tfl, gbs = flops / ms * 1e-9, nbytes / ms * 1e-6
@@ -172,26 +159,37 @@ def op_level_configs(tf, np):
         keep += [wt, bias, h]
     tf.dispose(keep)
 
-    x = f32(rng.uniform(0, 1, (32, 112, 112, 64)))
+    # Config 3 streams hundreds of MB per launch: the launches of the loop take their input from
+    # four tensors in turn (0.4 / 0.8 GB together, more than the 256 MB memory-side cache holds),
+    # so that every launch reads from HBM as it does inside a network.
+    xs = [f32(rng.uniform(0, 1, (32, 112, 112, 64))) for _ in range(4)]
     wt = f32(rng.standard_normal((3, 3, 64, 128)) * np.sqrt(2.0 / (9 * 64)))
     bias = f32(rng.standard_normal(128) * 0.1)
     timed("config 3: fused conv2d 3x3 [32,112,112,64]->128 bias relu6",
-          lambda: tf.fused.conv2d(x, wt, 1, "same", bias=bias, activation="relu6"), 50,
-          2.0 * 32 * 112 * 112 * 128 * 9 * 64, 4.0 * (32 * 112 * 112 * (64 + 128) + 9 * 64 * 128 + 128))
-    tf.dispose([x, wt, bias])
-    x = f32(rng.uniform(0, 1, (32, 112, 112, 128)))
+          lambda v: tf.fused.conv2d(xs[v], wt, 1, "same", bias=bias, activation="relu6"), 48,
+          2.0 * 32 * 112 * 112 * 128 * 9 * 64, 4.0 * (32 * 112 * 112 * (64 + 128) + 9 * 64 * 128 + 128),
+          variants=4)
+    tf.dispose(xs + [wt, bias])
+    xs = [f32(rng.uniform(0, 1, (32, 112, 112, 128))) for _ in range(4)]
     wt = f32(rng.standard_normal((3, 3, 128, 1)) * np.sqrt(2.0 / 9))
     bias = f32(rng.standard_normal(128) * 0.1)
     timed("config 3: fused depthwiseConv2D 3x3 [32,112,112,128] bias relu6",
-          lambda: tf.fused.depthwise_conv2d(x, wt, 1, "same", bias=bias, activation="relu6"), 100,
-          2.0 * 32 * 112 * 112 * 128 * 9, 4.0 * (2 * 32 * 112 * 112 * 128 + 9 * 128 + 128))
-    tf.dispose([x, wt, bias])
+          lambda v: tf.fused.depthwise_conv2d(xs[v], wt, 1, "same", bias=bias, activation="relu6"), 100,
+          2.0 * 32 * 112 * 112 * 128 * 9, 4.0 * (2 * 32 * 112 * 112 * 128 + 9 * 128 + 128),
+          variants=4)
+    tf.dispose(xs + [wt, bias])
+    be.lib.tfhip_time_per_kernel(be.ctx, 1)
     return out
 
 
-def cpu_baseline(mobilenet, params, budget_s=15.0):
-    """The CPU oracle (restatement of backend_cpu's loops, one thread) on batch-1 forwards
-    of the same network: a bounded sample, reported as images/s."""
+def cpu_baseline(mobilenet, params, budget_s=12.0):
+    """The CPU oracle on batch-1 forward passes of the same network, a bounded sample, as
+    images/s: (i) the C restatement of backend_cpu's loops at -O2 on one thread (`value`),
+    (ii) the plain-JavaScript restatement of the same loops under V8, the engine that runs the
+    reference's own backend_cpu (`javascript`), when node is installed."""
+    import shutil
+    import subprocess
+    import tempfile
     import numpy as np
     from oracle import cpu_ref
     sys.path.insert(0, os.path.join(ROOT, "tests"))
@@ -207,9 +205,42 @@ def cpu_baseline(mobilenet, params, budget_s=15.0):
         el = time.perf_counter() - t0
         if el + el / n > budget_s:
             break
-    return dict(value=round(n / el, 4), unit="images/s", cores=1, kind="port",
-                sample="%d batch-1 forward passes of the same MobileNetV1 (%.1f s), C restatement "
-                       "of backend_cpu at -O2, 1 thread" % (n, el))
+    cpu_model = ""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                cpu_model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    out = dict(value=round(n / el, 4), unit="images/s", cores=1, kind="port", cpu=cpu_model,
+               sample="%d batch-1 forward passes of the same MobileNetV1 (%.1f s), C restatement "
+                      "of backend_cpu at -O2, 1 thread" % (n, el))
+    node = shutil.which("node")
+    if node is not None:
+        order = ["stem_w", "stem_b"]
+        for i in range(1, 14):
+            order += ["dw%d_w" % i, "dw%d_b" % i, "pw%d_w" % i, "pw%d_b" % i]
+        order += ["fc_w", "fc_b"]
+        with tempfile.TemporaryDirectory() as d:
+            with open(os.path.join(d, "w.bin"), "wb") as f:
+                for name in order:
+                    f.write(np.ascontiguousarray(params[name], np.float32).tobytes())
+            with open(os.path.join(d, "specs.json"), "w") as f:
+                json.dump([dict(name=k, shape=list(params[k].shape)) for k in order], f)
+            r = subprocess.run([node, os.path.join(ROOT, "oracle", "cpu_ref.js"), "time",
+                                os.path.join(d, "w.bin"), os.path.join(d, "specs.json"),
+                                str(budget_s)], capture_output=True, text=True, timeout=600)
+        if r.returncode == 0:
+            j = json.loads(r.stdout.strip().splitlines()[-1])
+            out["javascript"] = dict(
+                value=round(j["images_per_s"], 4), unit="images/s", cores=1, kind="port",
+                sample="%d batch-1 forward passes (%.1f s), plain-JavaScript restatement of "
+                       "backend_cpu's loops under V8 (node %s), 1 thread" % (
+                           j["images"], j["seconds"], j["node"]))
+        else:
+            out["javascript"] = dict(error=(r.stderr or r.stdout)[-300:])
+    return out
 
 
 def write_weight_files(params, directory, shard_bytes=4 << 20):
@@ -322,8 +353,10 @@ def main():
     dev_params = mobilenet.quantize_params(params) if args.quant else params
     w = mobilenet.upload(tf, dev_params)
     x_host = np.random.default_rng(1).uniform(0, 1, (args.batch, 224, 224, 3)).astype(np.float32)
-    x = tf.tensor(x_host)          # resident in HBM before the timed region
     be.sync()
+
+    # ---- Python driver: input resident in HBM --------------------------------------------------
+    x = tf.tensor(x_host)
 
     def step():
         logits, probs = mobilenet.forward(tf, w, x)
@@ -333,81 +366,113 @@ def main():
         step()
     be.sync()
     t0 = time.perf_counter()
-    info = tf.time(lambda: [step() for _ in range(args.steps)])
+    for _ in range(args.steps):
+        step()
     be.sync()
     wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    value = args.batch * args.steps / wall
+    resident = dict(images_per_s=round(args.batch * args.steps / wall, 1),
+                    ms_per_step=round(wall * 1e3 / args.steps, 4))
+    # the same loop with an event after every launch: the times the kernels take in the step
+    info = tf.time(lambda: [step() for _ in range(args.steps)])
+    resident["gpu_ms_per_step_events"] = round(info["kernelMs"] / args.steps, 4)
+    per_step = len(info["kernelTimes"]) // args.steps
+    py_kernel_times = None
+    if per_step * args.steps == len(info["kernelTimes"]):
+        py_kernel_times = [(info["kernelTimes"][j][0],
+                            sum(info["kernelTimes"][s * per_step + j][1] for s in range(args.steps))
+                            / args.steps) for j in range(per_step)]
 
-    # The same step when the boundary is handed host buffers: input H2D (pageable host memory)
-    # before the forward pass and the class probabilities D2H after it.  Reported beside
-    # `value`, never as `value`.
-    def step_host():
-        xd = tf.tensor(x_host)
-        logits, probs = mobilenet.forward(tf, w, xd)
-        probs.data_sync()
-        tf.dispose([xd, logits, probs])
+    # ---- Python driver: end to end ---------------------------------------------------------------
+    # Every step uploads its batch (page-locked host arrays, upload stream), runs the forward
+    # pass and reads the probabilities back (asynchronous read, awaited two steps late); batch
+    # i+1 uploads while batch i computes.
+    slots = [tf.pinned_array("float32", x_host.shape) for _ in range(2)]
+    for sl in slots:
+        sl[...] = x_host
 
-    n_host = max(3, min(20, args.steps))
-    step_host()
-    be.sync()
+    def pipelined(n):
+        pending, last = [], None
+        nxt = tf.tensor(slots[0])
+        for i in range(n):
+            cur = nxt
+            if i + 1 < n:
+                nxt = tf.tensor(slots[(i + 1) % 2])
+            logits, probs = mobilenet.forward(tf, w, cur)
+            pending.append(probs.data())
+            tf.dispose([cur, logits, probs])
+            if len(pending) > 2:
+                last = pending.pop(0).result()
+        for p in pending:
+            last = p.result()
+        return last
+
+    pipelined(max(4, min(args.warmup, 10)))
     t0 = time.perf_counter()
-    for _ in range(n_host):
-        step_host()
-    host_wall = time.perf_counter() - t0
-    pcie = dict(images_per_s=round(args.batch * n_host / host_wall, 1),
-                ms_per_step=round(host_wall * 1e3 / n_host, 4), steps=n_host,
-                note="input upload (%.1f MB, pageable host memory) and probabilities readback "
-                     "inside the timed region" % (x_host.nbytes / 1e6))
+    last_probs = pipelined(args.steps)
+    wall = time.perf_counter() - t0
+    with tf.tidy():
+        want_probs = mobilenet.forward(tf, w, x)[1].data_sync()
+    py_end_to_end = dict(images_per_s=round(args.batch * args.steps / wall, 1),
+                         ms_per_step=round(wall * 1e3 / args.steps, 4),
+                         max_abs_diff_vs_resident=float(np.abs(last_probs - want_probs).max()))
 
-    rows = per_layer_times(tf, mobilenet, w, x, reps=20)
-    roof, groups = roofline_of_dominant_kernel(rows)
-    if args.batch == 64 and not args.quant and roof["kernel"] in MEASURED_HBM_BYTES_PER_LAUNCH:
-        roof["traffic"] = round(MEASURED_HBM_BYTES_PER_LAUNCH[roof["kernel"]])
-    if args.layers:
-        for r in rows:
-            ai = 2.0 * r["macs"] / r["bytes"]
-            print("%-8s %-28s %8.1f us  %7.2f TFLOP/s  %7.1f GB/s  AI %6.1f" % (
-                r["name"], r["kernel"], r["ms"] * 1e3, 2e-9 * r["macs"] / r["ms"],
-                1e-6 * r["bytes"] / r["ms"], ai), file=sys.stderr)
-        print("sum of layer times: %.3f ms; step (events): %.3f ms; step (wall): %.3f ms" % (
-            sum(r["ms"] for r in rows), info["kernelMs"] / args.steps, ms_per_step), file=sys.stderr)
-
-    # The product's host is JavaScript: when node is present the headline value is the step
-    # rate of the tf.* graph driven from Node.js; the Python driver's rate is kept beside it.
-    python_driver = dict(images_per_s=round(value, 1), ms_per_step=round(ms_per_step, 4),
-                         gpu_ms_per_step_events=round(info["kernelMs"] / args.steps, 4))
+    # ---- JavaScript host (the product's host) ----------------------------------------------------
     host = "python ctypes driver over the C ABI"
-    events_ms = info["kernelMs"] / args.steps
+    end_to_end, resident_input, kernel_times = py_end_to_end, resident, py_kernel_times
     js = None if args.no_js else js_host_leg(dev_params, x_host, args.batch, args.steps, args.warmup)
     if js is not None and "error" not in js:
-        value, ms_per_step, events_ms = js["images_per_s"], js["ms_per_step"], js["gpu_ms_per_step_events"]
         host = "JavaScript tf.* graph in Node.js %s over the N-API addon" % js["node"]
+        end_to_end, resident_input = js["end_to_end"], js["resident"]
+        if js.get("kernel_times"):
+            kernel_times = [tuple(k) for k in js["kernel_times"]]
 
+    # ---- roofline of the dominant kernel, from the times inside the running step ---------------
+    table = mobilenet.layer_table(batch=args.batch)
+    rows = rows_of_one_step(kernel_times, table, args.batch) if kernel_times else None
+    roof, groups = (roofline_of_dominant_kernel(rows) if rows else (None, {}))
+    traffic, stale = measured_traffic()
+    if roof is not None and args.batch == 64 and not args.quant:
+        roof["traffic"] = round(traffic[roof["kernel"]]) if roof["kernel"] in traffic else None
+        roof["traffic_source"] = "profiles/mobilenet_b64_fp32_hbm_traffic.txt"
+        roof["traffic_stale"] = stale
+    if args.layers and rows:
+        for r in rows:
+            ai = 2.0 * r["macs"] / r["bytes"]
+            print("%-8s %-36s %8.1f us  %7.2f TFLOP/s  %7.1f GB/s  AI %6.1f" % (
+                r["name"], r["kernel"], r["ms"] * 1e3, 2e-9 * r["macs"] / r["ms"],
+                1e-6 * r["bytes"] / r["ms"], ai), file=sys.stderr)
+        print("sum of kernel times: %.3f ms; step (wall, resident input): %.3f ms; end to end: %.3f ms"
+              % (sum(r["ms"] for r in rows), resident_input["ms_per_step"], end_to_end["ms_per_step"]),
+              file=sys.stderr)
+
+    dense = [r for r in (rows or []) if r["kind"] in ("conv", "matmul")]
     out = {
         "metric": "MobileNetV1-224 images/s at batch 64" if args.batch == 64 and not args.quant
                   else "MobileNetV1-224 images/s at batch %d%s" % (args.batch, " (uint8 weights)" if args.quant else ""),
-        "value": round(value, 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "value": round(end_to_end["images_per_s"], 1), "unit": "images/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(end_to_end["ms_per_step"], 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "MobileNetV1-1.0-224 random-init fp32 NHWC forward + softmax, "
-                               "batch %d%s, tf.* graph on the hip backend" % (
-                                   args.batch, ", uint8 weights" if args.quant else ""),
+                               "batch %d%s, tf.* graph on the hip backend; every step uploads its "
+                               "input batch from host memory and reads the class probabilities "
+                               "back (upload of batch i+1 overlapped with the kernels of batch i)"
+                               % (args.batch, ", uint8 weights" if args.quant else ""),
                    "global_batch": args.batch, "host": host},
-        "gpu_ms_per_step_events": round(events_ms, 4),
-        "python_driver": python_driver,
+        # the same step with the input uploaded once, before the timed region
+        "resident_input": resident_input,
+        "python_driver": {"end_to_end": py_end_to_end, "resident_input": resident},
         "js_host": js,
-        "pcie_inclusive": pcie,
-        # the same step recorded once with tf.captureGraph and replayed (one launch per step); an
-        # extension of this backend, reported beside `value`, which stays the eager tf.* path
-        "graph_replay": js.get("graph_replay") if js else None,
-        "dense_tflops": round(sum(2e-9 * r["macs"] for r in rows if r["kernel"].startswith("gemm"))
-                              / sum(r["ms"] for r in rows if r["kernel"].startswith("gemm")), 2),
+        "dense_tflops": round(sum(2e-9 * r["macs"] for r in dense) / sum(r["ms"] for r in dense), 2)
+                        if dense else None,
         "roofline": roof,
         "kernel_groups": {k: dict(ms=round(g["ms"], 4), launches=g["launches"],
                                   tflops=round(g["flops"] / g["ms"] * 1e-9, 2),
                                   gbs=round(g["bytes"] / g["ms"] * 1e-6, 1))
                           for k, g in groups.items()},
+        "layers": [dict(name=r["name"], kernel=r["kernel"], us=round(r["ms"] * 1e3, 2),
+                        tflops=round(2e-9 * r["macs"] / r["ms"], 2),
+                        gbs=round(1e-6 * r["bytes"] / r["ms"], 1)) for r in (rows or [])],
     }
     if not args.no_ops:
         out["op_configs"] = op_level_configs(tf, np)

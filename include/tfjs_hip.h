@@ -118,19 +118,19 @@ int tfhip_read_finish(tfhip_ctx* ctx, tfhip_pending_read* r, void* host, size_t 
 int tfhip_mem_info(tfhip_ctx* ctx, size_t* in_use, size_t* pooled, size_t* num_ids);
 int tfhip_sync(tfhip_ctx* ctx);
 /* KernelBackend.time (backend.ts:92, backend_cpu.ts:239-244): device time of the work queued
- * between the two calls.  Regions nest (up to 8 deep), as tf.time() calls may.
- * BackendTimingInfo.getExtraProfileInfo (backend.ts:27-31) is fed by the per-kernel figures:
- * while a region is open an event follows every kernel launch on the stream, and the time
- * of a kernel is the distance from the event before it, so the figures of a region add up to
- * its total (device idle time in front of a kernel counts towards that kernel).  The WebGL
- * backend of the reference times each program the same way with timer queries
+ * between the two calls (two events on the stream).  Regions nest (up to 8 deep), as tf.time()
+ * calls may.  BackendTimingInfo.getExtraProfileInfo (backend.ts:27-31) is fed by the per-kernel
+ * figures: while a region is open every kernel is launched with a start and a stop event
+ * attached to its own dispatch, so the time of a kernel is its execution on the device, as a
+ * profiler's kernel trace reports it (idle time between kernels is in the region's total
+ * only).  The WebGL backend of the reference times each program with timer queries
  * (backends/webgl/backend_webgl.ts:547-620).
  *   tfhip_time_kernel_count / tfhip_time_kernel  the launches of the region that ended last, in
  *                      launch order: name of the kernel variant (as tfhip_last_kernel reports
  *                      it; the entry point's name for kernels without variants) and its time.
  *                      The name stays valid until the next tfhip_time_end.
- *   tfhip_time_per_kernel(ctx, 0) switches the per-launch events off (one event pair per
- *                      region, no figures per kernel); 1, the default, switches them on. */
+ *   tfhip_time_per_kernel(ctx, 0) switches the per-launch events off (no figures per kernel);
+ *                      1, the default, switches them on. */
 int tfhip_time_begin(tfhip_ctx* ctx);
 int tfhip_time_end(tfhip_ctx* ctx, float* ms);
 int tfhip_time_per_kernel(tfhip_ctx* ctx, int enable);

@@ -394,8 +394,7 @@ extern "C" int tfhip_depthwise_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int6
     // directions and the padding filter - 1 - pad: the forward kernels do it at their speed
     Temp tflip(ctx);
     if (!tflip.get((size_t)w_n * sizeof(float))) return TFHIP_EDEVICE;
-    hipLaunchKernelGGL(flip_depthwise_filter_kernel, dim3((unsigned)ceil_div(w_n, 256)), dim3(256), 0,
-                       ctx->stream, wf, static_cast<float*>(tflip.ptr), ci->filter_h, ci->filter_w,
+    tfhip::launch(ctx, flip_depthwise_filter_kernel, dim3((unsigned)ceil_div(w_n, 256)), dim3(256), 0, wf, static_cast<float*>(tflip.ptr), ci->filter_h, ci->filter_w,
                        ci->in_c);
     TFHIP_LAUNCH_CHECK(ctx);
     tfhip_conv2d_info back = *ci;
@@ -414,19 +413,19 @@ extern "C" int tfhip_depthwise_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int6
     const int s = ci->stride_h == ci->stride_w && ci->stride_h <= 2 ? ci->stride_h : 0;
     ctx->name_kernel("depthwise_der_input_vec_s%d", s);
     if (s == 1)
-      hipLaunchKernelGGL(depthwise_der_input_vec_kernel<1>, dim3(blocks), dim3(256), 0, ctx->stream,
+      tfhip::launch(ctx, depthwise_der_input_vec_kernel<1>, dim3(blocks), dim3(256), 0,
                          dyf, wf, dxf, *ci);
     else if (s == 2)
-      hipLaunchKernelGGL(depthwise_der_input_vec_kernel<2>, dim3(blocks), dim3(256), 0, ctx->stream,
+      tfhip::launch(ctx, depthwise_der_input_vec_kernel<2>, dim3(blocks), dim3(256), 0,
                          dyf, wf, dxf, *ci);
     else
-      hipLaunchKernelGGL(depthwise_der_input_vec_kernel<0>, dim3(blocks), dim3(256), 0, ctx->stream,
+      tfhip::launch(ctx, depthwise_der_input_vec_kernel<0>, dim3(blocks), dim3(256), 0,
                          dyf, wf, dxf, *ci);
     TFHIP_LAUNCH_CHECK(ctx);
     return TFHIP_OK;
   }
   ctx->name_kernel("depthwise_der_input");
-  hipLaunchKernelGGL(depthwise_der_input_kernel, dim3(grid_for(ctx, x_n)), dim3(256), 0, ctx->stream,
+  tfhip::launch(ctx, depthwise_der_input_kernel, dim3(grid_for(ctx, x_n)), dim3(256), 0,
                      dyf, wf, dxf, *ci, ch_mul);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -474,12 +473,12 @@ extern "C" int tfhip_depthwise_conv2d_der_filter(tfhip_ctx* ctx, int64_t x, int6
     const int64_t per_slice = ceil_div(pixels, slices);
     if (!tpart.get((size_t)(slices * w_n) * sizeof(double))) return TFHIP_EDEVICE;
     ctx->name_kernel("depthwise3x3_der_filter");
-    hipLaunchKernelGGL(depthwise3x3_der_filter_partial_kernel, dim3((unsigned)blocks_c, (unsigned)slices),
-                       dim3(256), (size_t)(256 * 9 * 4 * sizeof(float)), ctx->stream, xf, dyf,
+    tfhip::launch(ctx, depthwise3x3_der_filter_partial_kernel, dim3((unsigned)blocks_c, (unsigned)slices),
+                       dim3(256), (size_t)(256 * 9 * 4 * sizeof(float)), xf, dyf,
                        static_cast<double*>(tpart.ptr), *ci, qpw, per_slice);
     TFHIP_LAUNCH_CHECK(ctx);
-    hipLaunchKernelGGL(depthwise_der_filter_finish_kernel, dim3((unsigned)ceil_div(w_n, 256)), dim3(256),
-                       0, ctx->stream, static_cast<const double*>(tpart.ptr),
+    tfhip::launch(ctx, depthwise_der_filter_finish_kernel, dim3((unsigned)ceil_div(w_n, 256)), dim3(256),
+                       0, static_cast<const double*>(tpart.ptr),
                        static_cast<float*>(bdw->ptr), w_n, (int)slices);
     TFHIP_LAUNCH_CHECK(ctx);
     return TFHIP_OK;
@@ -493,12 +492,11 @@ extern "C" int tfhip_depthwise_conv2d_der_filter(tfhip_ctx* ctx, int64_t x, int6
   const int64_t per_slice = ceil_div(pixels > 0 ? pixels : 1, slices);
   if (!tpart.get((size_t)(slices * w_n) * sizeof(double))) return TFHIP_EDEVICE;
   ctx->name_kernel("depthwise_der_filter");
-  hipLaunchKernelGGL(depthwise_der_filter_partial_kernel,
-                     dim3((unsigned)channel_blocks, (unsigned)taps, (unsigned)slices), dim3(256), 0,
-                     ctx->stream, xf, dyf, static_cast<double*>(tpart.ptr), *ci, ch_mul, per_slice);
+  tfhip::launch(ctx, depthwise_der_filter_partial_kernel,
+                     dim3((unsigned)channel_blocks, (unsigned)taps, (unsigned)slices), dim3(256), 0, xf, dyf, static_cast<double*>(tpart.ptr), *ci, ch_mul, per_slice);
   TFHIP_LAUNCH_CHECK(ctx);
-  hipLaunchKernelGGL(depthwise_der_filter_finish_kernel, dim3((unsigned)ceil_div(w_n, 256)), dim3(256),
-                     0, ctx->stream, static_cast<const double*>(tpart.ptr),
+  tfhip::launch(ctx, depthwise_der_filter_finish_kernel, dim3((unsigned)ceil_div(w_n, 256)), dim3(256),
+                     0, static_cast<const double*>(tpart.ptr),
                      static_cast<float*>(bdw->ptr), w_n, (int)slices);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -529,14 +527,13 @@ extern "C" int tfhip_pool2d_backprop(tfhip_ctx* ctx, int64_t dy, int64_t x, int6
   if (ci->in_c % 4 == 0 && aligned16(dyf) && aligned16(xf) && aligned16(dxf)) {
     ctx->name_kernel(
              kind == TFHIP_POOL_MAX ? "max_pool_backprop_vec" : "avg_pool_backprop_vec");
-    hipLaunchKernelGGL(pool2d_backprop_vec_kernel, dim3((unsigned)ceil_div(x_n / 4, 256)), dim3(256), 0,
-                       ctx->stream, dyf, xf, dxf, *ci, kind);
+    tfhip::launch(ctx, pool2d_backprop_vec_kernel, dim3((unsigned)ceil_div(x_n / 4, 256)), dim3(256), 0, dyf, xf, dxf, *ci, kind);
     TFHIP_LAUNCH_CHECK(ctx);
     return TFHIP_OK;
   }
   ctx->name_kernel(
            kind == TFHIP_POOL_MAX ? "max_pool_backprop" : "avg_pool_backprop");
-  hipLaunchKernelGGL(pool2d_backprop_kernel, dim3(grid_for(ctx, x_n)), dim3(256), 0, ctx->stream, dyf,
+  tfhip::launch(ctx, pool2d_backprop_kernel, dim3(grid_for(ctx, x_n)), dim3(256), 0, dyf,
                      xf, static_cast<float*>(bdx->ptr), *ci, kind);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;

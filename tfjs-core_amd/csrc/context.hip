@@ -72,25 +72,13 @@ void tfhip_ctx::name_kernel(const char* fmt, ...) {
   kernel_named = true;
 }
 
-// One more event on the stream.  The begin and end marks of a region always get a slot (the
-// last one is kept for them); kernel marks beyond the limit are counted and left out.
-int tfhip_ctx::mark(const char* name) {
-  const bool bracket = name[0] == '(';
-  if (marks_used >= kMaxMarks - (bracket ? 0 : 2 * kMaxTimeDepth)) {
-    if (!bracket) {
-      marks_dropped++;
-      return -1;
-    }
-    if (marks_used >= kMaxMarks) {
-      fail(TFHIP_EINVAL, "time: too many nested regions after %d launches", kMaxMarks);
-      return -1;
-    }
+// One more event on the stream, for the begin or the end of a region.
+int tfhip_ctx::mark() {
+  if (marks_used >= kMaxMarks) {
+    fail(TFHIP_EINVAL, "time: more than %d regions inside one", kMaxMarks / 2);
+    return -1;
   }
   if (marks_used == (int)mark_events.size()) {
-    if (no_alloc) {  // no new event inside a call that promises to create nothing
-      marks_dropped++;
-      return -1;
-    }
     hipEvent_t ev;
     hipError_t e = hipEventCreate(&ev);
     if (e != hipSuccess) {
@@ -98,15 +86,35 @@ int tfhip_ctx::mark(const char* name) {
       return -1;
     }
     mark_events.push_back(ev);
-    mark_names.emplace_back();
   }
   hipError_t e = hipEventRecord(mark_events[marks_used], stream);
   if (e != hipSuccess) {
     fail(TFHIP_EDEVICE, "hipEventRecord: %s", hipGetErrorString(e));
     return -1;
   }
-  mark_names[marks_used] = name;
   return marks_used++;
+}
+
+bool tfhip_ctx::next_rec(hipEvent_t* start, hipEvent_t* stop) {
+  if (recs_used >= kMaxKernelRecs || (recs_used == (int)recs.size() && no_alloc)) {
+    recs_dropped++;  // (a call that promises to create nothing creates no event either)
+    return false;
+  }
+  if (recs_used == (int)recs.size()) {
+    KernelRec r;
+    if (hipEventCreate(&r.start) != hipSuccess || hipEventCreate(&r.stop) != hipSuccess) {
+      (void)hipGetLastError();
+      if (r.start) (void)hipEventDestroy(r.start);
+      recs_dropped++;
+      return false;
+    }
+    recs.push_back(r);
+  }
+  *start = recs[recs_used].start;
+  *stop = recs[recs_used].stop;
+  recs[recs_used].name.clear();
+  pending_rec = recs_used++;
+  return true;
 }
 
 Buf* tfhip_ctx::find(int64_t id, bool touch) {
@@ -351,6 +359,10 @@ void tfhip_destroy(tfhip_ctx* ctx) {
     for (auto& blk : kv.second.parked) (void)hipFree(blk.first);
   }
   for (hipEvent_t ev : ctx->mark_events) (void)hipEventDestroy(ev);
+  for (auto& r : ctx->recs) {
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
   (void)hipStreamDestroy(ctx->upload);
   (void)hipStreamDestroy(ctx->download);
   (void)hipStreamDestroy(ctx->stream);
@@ -605,32 +617,30 @@ int tfhip_time_begin(tfhip_ctx* ctx) {
   if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "time: not during a graph capture");
   if (ctx->time_depth == tfhip_ctx::kMaxTimeDepth)
     return ctx->fail(TFHIP_EINVAL, "time: more than %d nested regions", tfhip_ctx::kMaxTimeDepth);
-  if (ctx->time_depth == 0) ctx->marks_used = ctx->marks_dropped = 0;
-  const int at = ctx->mark("(begin)");
+  if (ctx->time_depth == 0) ctx->marks_used = ctx->recs_used = ctx->recs_dropped = 0;
+  const int at = ctx->mark();
   if (at < 0) return TFHIP_EDEVICE;
-  ctx->time_stack[ctx->time_depth++] = at;
+  ctx->time_stack[ctx->time_depth++] = {at, ctx->recs_used};
   return TFHIP_OK;
 }
 
 int tfhip_time_end(tfhip_ctx* ctx, float* ms) {
   if (!ctx || !ms) return TFHIP_EINVAL;
   if (!ctx->time_depth) return ctx->fail(TFHIP_EINVAL, "time_end without time_begin");
-  const int first = ctx->time_stack[--ctx->time_depth];
-  const int last = ctx->mark("(end)");
+  const tfhip_ctx::Region first = ctx->time_stack[--ctx->time_depth];
+  const int last = ctx->mark();
   if (last < 0) return TFHIP_EDEVICE;
   TFHIP_HIP(ctx, hipEventSynchronize(ctx->mark_events[last]));
-  TFHIP_HIP(ctx, hipEventElapsedTime(ms, ctx->mark_events[first], ctx->mark_events[last]));
+  TFHIP_HIP(ctx, hipEventElapsedTime(ms, ctx->mark_events[first.mark], ctx->mark_events[last]));
   ctx->kernel_times.clear();
-  for (int i = first + 1; i <= last; i++) {
+  for (int i = first.rec; i < ctx->recs_used; i++) {
     float d = 0;
-    TFHIP_HIP(ctx, hipEventElapsedTime(&d, ctx->mark_events[i - 1], ctx->mark_events[i]));
-    // the marks of this and of inner regions carry no kernel: their (tiny) share stays in the total
-    if (ctx->mark_names[i][0] == '(') continue;
-    ctx->kernel_times.push_back({ctx->mark_names[i], d});
+    TFHIP_HIP(ctx, hipEventElapsedTime(&d, ctx->recs[i].start, ctx->recs[i].stop));
+    ctx->kernel_times.push_back({ctx->recs[i].name, d});
   }
-  if (ctx->marks_dropped) {
+  if (ctx->recs_dropped) {
     char note[64];
-    snprintf(note, sizeof note, "(%d launches not recorded)", ctx->marks_dropped);
+    snprintf(note, sizeof note, "(%d launches not recorded)", ctx->recs_dropped);
     ctx->kernel_times.push_back({note, 0.f});
   }
   return TFHIP_OK;

@@ -281,7 +281,7 @@ static int grid_for(tfhip_ctx* ctx, int64_t work_items, int block) {
 int launch_convert(tfhip_ctx* ctx, const void* src, int src_dtype, void* dst, int dst_dtype,
                    int64_t n) {
   if (n == 0) return TFHIP_OK;
-  hipLaunchKernelGGL(convert_kernel, dim3(grid_for(ctx, n, 256)), dim3(256), 0, ctx->stream, src,
+  tfhip::launch(ctx, convert_kernel, dim3(grid_for(ctx, n, 256)), dim3(256), 0, src,
                      src_dtype, dst, dst_dtype, n);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -344,8 +344,7 @@ extern "C" int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_
   const int block = 256;
   if (!predicate && all_f32 && a_len == n && b_len == n && n % 4 == 0 && aligned16(ba->ptr) &&
       aligned16(bb->ptr) && aligned16(bo->ptr)) {
-    hipLaunchKernelGGL(binary_f32_vec_kernel, dim3(grid_for(ctx, n / 4, block)), dim3(block), 0,
-                       ctx->stream, op, (const f32x4*)ba->ptr, (const f32x4*)bb->ptr,
+    tfhip::launch(ctx, binary_f32_vec_kernel, dim3(grid_for(ctx, n / 4, block)), dim3(block), 0, op, (const f32x4*)ba->ptr, (const f32x4*)bb->ptr,
                        (f32x4*)bo->ptr, n / 4);
     TFHIP_LAUNCH_CHECK(ctx);
     return TFHIP_OK;
@@ -355,8 +354,7 @@ extern "C" int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_
       aligned16(bb->ptr) && aligned16(bo->ptr) &&
       ((a_len == n && b_len == last) || (b_len == n && a_len == last))) {
     const bool b_small = b_len == last && a_len == n;
-    hipLaunchKernelGGL(binary_f32_rowvec_kernel, dim3(grid_for(ctx, n / 4, block)), dim3(block), 0,
-                       ctx->stream, op, (const f32x4*)(b_small ? ba->ptr : bb->ptr),
+    tfhip::launch(ctx, binary_f32_rowvec_kernel, dim3(grid_for(ctx, n / 4, block)), dim3(block), 0, op, (const f32x4*)(b_small ? ba->ptr : bb->ptr),
                        (const f32x4*)(b_small ? bb->ptr : ba->ptr), (f32x4*)bo->ptr, n / 4,
                        last / 4, b_small ? 0 : 1);
     TFHIP_LAUNCH_CHECK(ctx);
@@ -365,13 +363,13 @@ extern "C" int tfhip_binary(tfhip_ctx* ctx, int op, int64_t a, const int32_t* a_
   const int mode = (a_len == n && b_len == n) ? 0 : (!a_bcast && !b_bcast) ? 1 : 2;
   const dim3 grid(grid_for(ctx, n, block));
   if (bo->dtype == TFHIP_FLOAT32)
-    hipLaunchKernelGGL(binary_kernel<float>, grid, dim3(block), 0, ctx->stream, op, ba->ptr,
+    tfhip::launch(ctx, binary_kernel<float>, grid, dim3(block), 0, op, ba->ptr,
                        ba->dtype, a_len, bb->ptr, bb->dtype, b_len, (float*)bo->ptr, n, mode, bc);
   else if (bo->dtype == TFHIP_BOOL)
-    hipLaunchKernelGGL(binary_kernel<uint8_t>, grid, dim3(block), 0, ctx->stream, op, ba->ptr,
+    tfhip::launch(ctx, binary_kernel<uint8_t>, grid, dim3(block), 0, op, ba->ptr,
                        ba->dtype, a_len, bb->ptr, bb->dtype, b_len, (uint8_t*)bo->ptr, n, mode, bc);
   else
-    hipLaunchKernelGGL(binary_kernel<int32_t>, grid, dim3(block), 0, ctx->stream, op, ba->ptr,
+    tfhip::launch(ctx, binary_kernel<int32_t>, grid, dim3(block), 0, op, ba->ptr,
                        ba->dtype, a_len, bb->ptr, bb->dtype, b_len, (int32_t*)bo->ptr, n, mode, bc);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -393,17 +391,13 @@ extern "C" int tfhip_unary(tfhip_ctx* ctx, int op, int64_t x, int64_t out, float
   const int block = 256;
   if (bx->dtype == TFHIP_FLOAT32 && bo->dtype == TFHIP_FLOAT32 && n % 4 == 0 &&
       aligned16(bx->ptr) && aligned16(bo->ptr)) {
-    hipLaunchKernelGGL(unary_f32_vec_kernel, dim3(grid_for(ctx, n / 4, block)), dim3(block), 0,
-                       ctx->stream, op, (const f32x4*)bx->ptr, (f32x4*)bo->ptr, n / 4, p0, p1);
+    tfhip::launch(ctx, unary_f32_vec_kernel, dim3(grid_for(ctx, n / 4, block)), dim3(block), 0, op, (const f32x4*)bx->ptr, (f32x4*)bo->ptr, n / 4, p0, p1);
   } else if (bo->dtype == TFHIP_FLOAT32) {
-    hipLaunchKernelGGL(unary_kernel<float>, dim3(grid_for(ctx, n, block)), dim3(block), 0,
-                       ctx->stream, op, bx->ptr, bx->dtype, (float*)bo->ptr, n, p0, p1);
+    tfhip::launch(ctx, unary_kernel<float>, dim3(grid_for(ctx, n, block)), dim3(block), 0, op, bx->ptr, bx->dtype, (float*)bo->ptr, n, p0, p1);
   } else if (bo->dtype == TFHIP_BOOL) {
-    hipLaunchKernelGGL(unary_kernel<uint8_t>, dim3(grid_for(ctx, n, block)), dim3(block), 0,
-                       ctx->stream, op, bx->ptr, bx->dtype, (uint8_t*)bo->ptr, n, p0, p1);
+    tfhip::launch(ctx, unary_kernel<uint8_t>, dim3(grid_for(ctx, n, block)), dim3(block), 0, op, bx->ptr, bx->dtype, (uint8_t*)bo->ptr, n, p0, p1);
   } else {
-    hipLaunchKernelGGL(unary_kernel<int32_t>, dim3(grid_for(ctx, n, block)), dim3(block), 0,
-                       ctx->stream, op, bx->ptr, bx->dtype, (int32_t*)bo->ptr, n, p0, p1);
+    tfhip::launch(ctx, unary_kernel<int32_t>, dim3(grid_for(ctx, n, block)), dim3(block), 0, op, bx->ptr, bx->dtype, (int32_t*)bo->ptr, n, p0, p1);
   }
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -426,8 +420,7 @@ extern "C" int tfhip_dequantize(tfhip_ctx* ctx, int64_t x, int64_t out, const tf
   if (bx->dtype != TFHIP_UINT8Q || bo->dtype != TFHIP_FLOAT32 || bx->numel != bo->numel)
     return ctx->fail(TFHIP_EINVAL, "dequantize: needs a quantised input and a float32 output of equal size");
   if (bx->numel == 0) return TFHIP_OK;
-  hipLaunchKernelGGL(dequantize_kernel, dim3(grid_for(ctx, bx->numel, 256)), dim3(256), 0,
-                     ctx->stream, (const uint8_t*)bx->ptr, (float*)bo->ptr, bx->numel, q->scale,
+  tfhip::launch(ctx, dequantize_kernel, dim3(grid_for(ctx, bx->numel, 256)), dim3(256), 0, (const uint8_t*)bx->ptr, (float*)bo->ptr, bx->numel, q->scale,
                      q->min);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -440,13 +433,13 @@ extern "C" int tfhip_fill(tfhip_ctx* ctx, int64_t out, double value) {
   if (n == 0) return TFHIP_OK;
   const dim3 grid(grid_for(ctx, n, 256)), block(256);
   if (bo->dtype == TFHIP_FLOAT32)
-    hipLaunchKernelGGL(fill_kernel<float>, grid, block, 0, ctx->stream, (float*)bo->ptr, n,
+    tfhip::launch(ctx, fill_kernel<float>, grid, block, 0, (float*)bo->ptr, n,
                        (float)value);
   else if (bo->dtype == TFHIP_INT32)
-    hipLaunchKernelGGL(fill_kernel<int32_t>, grid, block, 0, ctx->stream, (int32_t*)bo->ptr, n,
+    tfhip::launch(ctx, fill_kernel<int32_t>, grid, block, 0, (int32_t*)bo->ptr, n,
                        (int32_t)value);
   else
-    hipLaunchKernelGGL(fill_kernel<uint8_t>, grid, block, 0, ctx->stream, (uint8_t*)bo->ptr, n,
+    tfhip::launch(ctx, fill_kernel<uint8_t>, grid, block, 0, (uint8_t*)bo->ptr, n,
                        (uint8_t)value);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;

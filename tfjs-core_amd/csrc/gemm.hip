@@ -1371,15 +1371,15 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
       p.partials = static_cast<float*>(partials.ptr);
     }
   }
-  hipLaunchKernelGGL((gemm_kernel<T::WM, T::WN, T::TM, T::TN, AMODE, BMODE, KBLOCKED, FAST>),
-                     dim3(pl.grid), dim3(T::WM * T::WN * 64), 0, ctx->stream, p);
+  tfhip::launch(ctx, (gemm_kernel<T::WM, T::WN, T::TM, T::TN, AMODE, BMODE, KBLOCKED, FAST>),
+                     dim3(pl.grid), dim3(T::WM * T::WN * 64), 0, p);
   TFHIP_LAUNCH_CHECK(ctx);
   if (pl.splits > 1) {
     const long long quads = (long long)pl.tail_tiles * T::BM * T::BN / 4;
     const long long blocks = ceil_div(quads, 256);
     const long long cap = (long long)ctx->num_cus * 8;
-    hipLaunchKernelGGL(splitk_finish_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256),
-                       0, ctx->stream, p, T::BM, T::BN, pl.full_tiles);
+    tfhip::launch(ctx, splitk_finish_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256),
+                       0, p, T::BM, T::BN, pl.full_tiles);
     TFHIP_LAUNCH_CHECK_NAMED(ctx, "splitk_finish");
   }
   return TFHIP_OK;
@@ -1448,8 +1448,8 @@ static int launch_rowstream_cfg(tfhip_ctx* ctx, const GemmArgs& p, int quant) {
            quant ? "u8" : "f32");
   GemmArgs q = p;
   q.reverse = ctx->take_sweep();
-  hipLaunchKernelGGL(kernel, dim3((unsigned)(want < slots || slots < 8 ? want : slots)), dim3(256),
-                     lds, ctx->stream, q, n_blocks, quant);
+  tfhip::launch(ctx, kernel, dim3((unsigned)(want < slots || slots < 8 ? want : slots)), dim3(256),
+                     lds, q, n_blocks, quant);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }
@@ -1762,7 +1762,7 @@ extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t o
         if (grid >= 64) grid &= ~7u;  // a multiple of the XCD count: one run of rows per XCD
         ctx->name_kernel("%s_%s", name, quant ? "u8" : "f32");
         ctx->sweep = 1;  // this kernel walks the rows forward: its consumer should start at the end
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), (size_t)lds, ctx->stream, p,
+        tfhip::launch(ctx, kernel, dim3(grid), dim3(256), (size_t)lds, p,
                            (int)row_floats, n_rows);
       };
       if (p.N <= 32) {
@@ -1870,8 +1870,8 @@ extern "C" int tfhip_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int64_t filter
   if (!tflip.get((size_t)w_n * sizeof(float))) return TFHIP_EDEVICE;
   {
     const int64_t blocks = ceil_div(w_n, 256);
-    hipLaunchKernelGGL(flip_filter_kernel, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256),
-                       0, ctx->stream, wf, static_cast<float*>(tflip.ptr), ci->filter_h,
+    tfhip::launch(ctx, flip_filter_kernel, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256),
+                       0, wf, static_cast<float*>(tflip.ptr), ci->filter_h,
                        ci->filter_w, ci->in_c, ci->out_c);
     TFHIP_LAUNCH_CHECK(ctx);
   }
@@ -1928,8 +1928,8 @@ extern "C" int tfhip_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int64_t filter
             !tout.get((size_t)(rows * ci->in_c) * sizeof(float)))
           return TFHIP_EDEVICE;
         const int64_t fb = ceil_div(taps_n, 256);
-        hipLaunchKernelGGL(flip_filter_taps_kernel, dim3((unsigned)(fb > 4096 ? 4096 : fb)), dim3(256),
-                           0, ctx->stream, wf, static_cast<float*>(tsub.ptr), ci->filter_h,
+        tfhip::launch(ctx, flip_filter_taps_kernel, dim3((unsigned)(fb > 4096 ? 4096 : fb)), dim3(256),
+                           0, wf, static_cast<float*>(tsub.ptr), ci->filter_h,
                            ci->filter_w, ci->in_c, ci->out_c, wr0, ci->stride_h, KHc, wc0,
                            ci->stride_w, KWc);
         TFHIP_LAUNCH_CHECK(ctx);
@@ -1948,8 +1948,7 @@ extern "C" int tfhip_conv2d_der_input(tfhip_ctx* ctx, int64_t dy, int64_t filter
         if ((rc = launch_gemm(ctx, q, 1, A_IM2COL, B_ROWMAJOR, /*kblocked=*/false))) return rc;
         const int64_t total = rows * ci->in_c;
         const int64_t sb = ceil_div(total, 256), cap = (int64_t)ctx->num_cus * 16;
-        hipLaunchKernelGGL(scatter_pixels_kernel, dim3((unsigned)(sb > cap ? cap : sb)), dim3(256), 0,
-                           ctx->stream, static_cast<const float*>(tout.ptr), p.C, total, Hc, Wc,
+        tfhip::launch(ctx, scatter_pixels_kernel, dim3((unsigned)(sb > cap ? cap : sb)), dim3(256), 0, static_cast<const float*>(tout.ptr), p.C, total, Hc, Wc,
                            ci->in_c, ci->in_h, ci->in_w, r0, ci->stride_h, c0, ci->stride_w);
         TFHIP_LAUNCH_CHECK(ctx);
       }

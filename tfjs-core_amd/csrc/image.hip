@@ -440,8 +440,8 @@ static void launch_dw3x3(tfhip_ctx* ctx, DwArgs& p) {
   p.tiles_w = (int)ceil_div(p.ci.out_w, TW);
   const int64_t total = (int64_t)p.ci.batch * p.tiles_h * p.tiles_w * p.c4;
   p.reverse = ctx->take_sweep();
-  hipLaunchKernelGGL((depthwise3x3_kernel<S, TH, TW>), dim3((unsigned)ceil_div(total, 256)),
-                     dim3(256), 0, ctx->stream, p);
+  tfhip::launch(ctx, (depthwise3x3_kernel<S, TH, TW>), dim3((unsigned)ceil_div(total, 256)),
+                     dim3(256), 0, p);
 }
 
 template <int TW>
@@ -451,8 +451,8 @@ static void launch_dw3x3_rows(tfhip_ctx* ctx, DwArgs& p, int rows) {
   p.tiles_w = (int)ceil_div(p.ci.out_w, TW);
   const int64_t total = (int64_t)p.ci.batch * chunks * p.tiles_w * p.c4;
   p.reverse = ctx->take_sweep();
-  hipLaunchKernelGGL((depthwise3x3_rows_kernel<TW>), dim3((unsigned)ceil_div(total, 256)),
-                     dim3(256), 0, ctx->stream, p, rows, chunks,
+  tfhip::launch(ctx, (depthwise3x3_rows_kernel<TW>), dim3((unsigned)ceil_div(total, 256)),
+                     dim3(256), 0, p, rows, chunks,
                      (unsigned)((int64_t)p.ci.batch * p.ci.in_h * p.ci.in_w * p.ci.in_c * 4),
                      (unsigned)((int64_t)p.ci.batch * p.ci.out_h * p.ci.out_w * p.ci.out_c * 4));
 }
@@ -502,8 +502,8 @@ static int dispatch_depthwise(tfhip_ctx* ctx, DwArgs& p, const tfhip_conv2d_info
     ctx->name_kernel("depthwise_generic");
     const int64_t blocks = ceil_div(o_n, 256);
     const int64_t cap = (int64_t)ctx->num_cus * 16;
-    hipLaunchKernelGGL(depthwise_generic_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)),
-                       dim3(256), 0, ctx->stream, p);
+    tfhip::launch(ctx, depthwise_generic_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)),
+                       dim3(256), 0, p);
   }
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -615,14 +615,12 @@ extern "C" int tfhip_pool2d(tfhip_ctx* ctx, int64_t x, int64_t out, const tfhip_
   if (global) {
     ctx->name_kernel("global_avgpool");
     const int items = ci->batch * (ci->in_c / 4);
-    hipLaunchKernelGGL(global_avgpool_kernel, dim3((unsigned)ceil_div(items, 64)), dim3(64), 0,
-                       ctx->stream, xf, y, ci->batch, ci->in_h * ci->in_w, ci->in_c / 4);
+    tfhip::launch(ctx, global_avgpool_kernel, dim3((unsigned)ceil_div(items, 64)), dim3(64), 0, xf, y, ci->batch, ci->in_h * ci->in_w, ci->in_c / 4);
   } else {
     const int64_t blocks = ceil_div(o_n, 256);
     const int64_t cap = (int64_t)ctx->num_cus * 16;
     ctx->name_kernel("pool2d");
-    hipLaunchKernelGGL(pool2d_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0,
-                       ctx->stream, xf, y, *ci, kind);
+    tfhip::launch(ctx, pool2d_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, xf, y, *ci, kind);
   }
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -651,7 +649,7 @@ extern "C" int tfhip_lrn(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t pixels,
   const int64_t n = bx->numel;
   if (n == 0) return TFHIP_OK;
   const int64_t blocks = ceil_div(n, 256), cap = (int64_t)ctx->num_cus * 16;
-  hipLaunchKernelGGL(lrn_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, ctx->stream,
+  tfhip::launch(ctx, lrn_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0,
                      (const float*)bx->ptr, (float*)bo->ptr, n, channels, depth_radius, bias, alpha, beta);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -671,8 +669,7 @@ extern "C" int tfhip_lrn_grad(tfhip_ctx* ctx, int64_t dy, int64_t x, int64_t y, 
   const int64_t n = bx->numel;
   if (n == 0) return TFHIP_OK;
   const int64_t blocks = ceil_div(n, 256), cap = (int64_t)ctx->num_cus * 16;
-  hipLaunchKernelGGL(lrn_grad_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0,
-                     ctx->stream, (const float*)bdy->ptr, (const float*)bx->ptr, (const float*)by->ptr,
+  tfhip::launch(ctx, lrn_grad_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, (const float*)bdy->ptr, (const float*)bx->ptr, (const float*)by->ptr,
                      (float*)bdx->ptr, n, channels, depth_radius, bias, alpha, beta);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;

@@ -285,8 +285,8 @@ static int flatten_checked(tfhip_ctx* ctx, const char* op, const Buf* bi, const 
   Temp flag(ctx);
   if (!flat->get((size_t)n * sizeof(int64_t)) || !flag.get(sizeof(int))) return TFHIP_EDEVICE;
   int* bad = static_cast<int*>(flag.ptr);
-  hipLaunchKernelGGL(set_int_kernel, dim3(1), dim3(1), 0, ctx->stream, bad, INT_MAX);
-  hipLaunchKernelGGL(flatten_indices_kernel, dim3(blocks_for(ctx, n)), dim3(256), 0, ctx->stream,
+  tfhip::launch(ctx, set_int_kernel, dim3(1), dim3(1), 0, bad, INT_MAX);
+  tfhip::launch(ctx, flatten_indices_kernel, dim3(blocks_for(ctx, n)), dim3(256), 0,
                      (const int32_t*)bi->ptr, (int64_t*)flat->ptr, n, s, rows, bad);
   TFHIP_LAUNCH_CHECK(ctx);
   if (!check) return TFHIP_OK;
@@ -341,14 +341,13 @@ extern "C" int tfhip_gather_nd(tfhip_ctx* ctx, int64_t x, int64_t indices, int64
   const int64_t slice_bytes = slice * (int64_t)dtype_size(bx->dtype);
   if (slice_bytes % 16 == 0 && reinterpret_cast<uintptr_t>(bx->ptr) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(bo->ptr) % 16 == 0)
-    hipLaunchKernelGGL(gather_rows_vec_kernel, dim3(blocks_for(ctx, num_slices * (slice_bytes / 16))), block, 0,
-                       ctx->stream, (const uint4*)bx->ptr, (const int64_t*)flat.ptr, (uint4*)bo->ptr, num_slices,
+    tfhip::launch(ctx, gather_rows_vec_kernel, dim3(blocks_for(ctx, num_slices * (slice_bytes / 16))), block, 0, (const uint4*)bx->ptr, (const int64_t*)flat.ptr, (uint4*)bo->ptr, num_slices,
                        slice_bytes / 16);
   else if (dtype_size(bx->dtype) == 4)
-    hipLaunchKernelGGL(gather_rows_kernel<int32_t>, grid, block, 0, ctx->stream, (const int32_t*)bx->ptr,
+    tfhip::launch(ctx, gather_rows_kernel<int32_t>, grid, block, 0, (const int32_t*)bx->ptr,
                        (const int64_t*)flat.ptr, (int32_t*)bo->ptr, num_slices, slice);
   else
-    hipLaunchKernelGGL(gather_rows_kernel<uint8_t>, grid, block, 0, ctx->stream, (const uint8_t*)bx->ptr,
+    tfhip::launch(ctx, gather_rows_kernel<uint8_t>, grid, block, 0, (const uint8_t*)bx->ptr,
                        (const int64_t*)flat.ptr, (uint8_t*)bo->ptr, num_slices, slice);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -381,15 +380,15 @@ extern "C" int tfhip_scatter_nd(tfhip_ctx* ctx, int64_t indices, int64_t updates
   const int sum = flags & TFHIP_SCATTER_SUM ? 1 : 0, one = scalar_update ? 1 : 0;
   const int64_t* fl = (const int64_t*)flat.ptr;
   if (bo->dtype == TFHIP_INT32)
-    hipLaunchKernelGGL((scatter_rows_kernel<int32_t, int32_t>), grid, block, 0, ctx->stream, fl,
+    tfhip::launch(ctx, (scatter_rows_kernel<int32_t, int32_t>), grid, block, 0, fl,
                        (const int32_t*)bu->ptr, (int32_t*)bo->ptr, rows, slice, num_updates,
                        (int32_t)default_value, sum, one);
   else if (flags & TFHIP_SCATTER_WIDE_SUM)
-    hipLaunchKernelGGL((scatter_rows_kernel<float, double>), grid, block, 0, ctx->stream, fl,
+    tfhip::launch(ctx, (scatter_rows_kernel<float, double>), grid, block, 0, fl,
                        (const float*)bu->ptr, (float*)bo->ptr, rows, slice, num_updates,
                        (float)default_value, sum, one);
   else
-    hipLaunchKernelGGL((scatter_rows_kernel<float, float>), grid, block, 0, ctx->stream, fl,
+    tfhip::launch(ctx, (scatter_rows_kernel<float, float>), grid, block, 0, fl,
                        (const float*)bu->ptr, (float*)bo->ptr, rows, slice, num_updates,
                        (float)default_value, sum, one);
   TFHIP_LAUNCH_CHECK(ctx);
@@ -410,8 +409,7 @@ extern "C" int tfhip_resize_bilinear_backprop(tfhip_ctx* ctx, int64_t dy, int64_
   const double eh_x = (align_corners && y_h > 1) ? x_h - 1 : x_h, ew_x = (align_corners && y_w > 1) ? x_w - 1 : x_w;
   const double eh_y = (align_corners && y_h > 1) ? y_h - 1 : y_h, ew_y = (align_corners && y_w > 1) ? y_w - 1 : y_w;
   if (bdy->numel == 0) return tfhip_fill(ctx, dx, 0.0);
-  hipLaunchKernelGGL(resize_bilinear_backprop_kernel, dim3(blocks_for(ctx, bdx->numel)), dim3(256), 0,
-                     ctx->stream, (const float*)bdy->ptr, (float*)bdx->ptr, batch, x_h, x_w, channels,
+  tfhip::launch(ctx, resize_bilinear_backprop_kernel, dim3(blocks_for(ctx, bdx->numel)), dim3(256), 0, (const float*)bdy->ptr, (float*)bdx->ptr, batch, x_h, x_w, channels,
                      y_h, y_w, eh_x / eh_y, ew_x / ew_y);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -432,8 +430,7 @@ extern "C" int tfhip_resize_nearest_backprop(tfhip_ctx* ctx, int64_t dy, int64_t
   // effective sizes and scales (backend_cpu.ts:3083-3094)
   const double eh_x = (align_corners && y_h > 1) ? x_h - 1 : x_h, ew_x = (align_corners && y_w > 1) ? x_w - 1 : x_w;
   const double eh_y = (align_corners && y_h > 1) ? y_h - 1 : y_h, ew_y = (align_corners && y_w > 1) ? y_w - 1 : y_w;
-  hipLaunchKernelGGL(resize_nearest_backprop_kernel, dim3(blocks_for(ctx, bdx->numel)), dim3(256), 0,
-                     ctx->stream, (const float*)bdy->ptr, (float*)bdx->ptr, batch, x_h, x_w, channels,
+  tfhip::launch(ctx, resize_nearest_backprop_kernel, dim3(blocks_for(ctx, bdx->numel)), dim3(256), 0, (const float*)bdy->ptr, (float*)bdx->ptr, batch, x_h, x_w, channels,
                      y_h, y_w, eh_x / eh_y, ew_x / ew_y, align_corners ? 1 : 0);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -463,7 +460,7 @@ extern "C" int tfhip_crop_and_resize(tfhip_ctx* ctx, int64_t images, int64_t box
   const float* imf;
   int rc;
   if ((rc = as_f32(ctx, bim, &tx, &imf))) return rc;
-  hipLaunchKernelGGL(crop_and_resize_kernel, dim3(blocks_for(ctx, bo->numel)), dim3(256), 0, ctx->stream,
+  tfhip::launch(ctx, crop_and_resize_kernel, dim3(blocks_for(ctx, bo->numel)), dim3(256), 0,
                      imf, (const float*)bb->ptr, (const int32_t*)bx->ptr, (float*)bo->ptr, batch, image_h,
                      image_w, channels, num_boxes, crop_h, crop_w, method == TFHIP_RESIZE_NEAREST ? 1 : 0,
                      extrapolation_value);

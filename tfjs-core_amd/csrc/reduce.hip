@@ -296,13 +296,13 @@ extern "C" int tfhip_reduce(tfhip_ctx* ctx, int op, int64_t x, int64_t out, int6
   if (ceil_div(outer, ROWS_PER_BLOCK) > 0x7fffffffLL) return ctx->fail(TFHIP_ENOTSUP, "reduce: too many rows");
   const dim3 grid((unsigned)ceil_div(outer, ROWS_PER_BLOCK)), block(WAVE * ROWS_PER_BLOCK);
   if (bo->dtype == TFHIP_FLOAT32)
-    hipLaunchKernelGGL(reduce_rows_kernel<float>, grid, block, 0, ctx->stream, op, bx->ptr,
+    tfhip::launch(ctx, reduce_rows_kernel<float>, grid, block, 0, op, bx->ptr,
                        bx->dtype, (float*)bo->ptr, outer, inner);
   else if (bo->dtype == TFHIP_BOOL)
-    hipLaunchKernelGGL(reduce_rows_kernel<uint8_t>, grid, block, 0, ctx->stream, op, bx->ptr,
+    tfhip::launch(ctx, reduce_rows_kernel<uint8_t>, grid, block, 0, op, bx->ptr,
                        bx->dtype, (uint8_t*)bo->ptr, outer, inner);
   else
-    hipLaunchKernelGGL(reduce_rows_kernel<int32_t>, grid, block, 0, ctx->stream, op, bx->ptr,
+    tfhip::launch(ctx, reduce_rows_kernel<int32_t>, grid, block, 0, op, bx->ptr,
                        bx->dtype, (int32_t*)bo->ptr, outer, inner);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -324,13 +324,13 @@ extern "C" int tfhip_softmax_rows(tfhip_ctx* ctx, int64_t x, int64_t out, int64_
   const dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK)), block(WAVE * ROWS_PER_BLOCK);
   float* yf = static_cast<float*>(bo->ptr);
   if (cols <= WAVE)
-    hipLaunchKernelGGL(softmax_rows_kernel<1>, grid, block, 0, ctx->stream, xf, yf, rows, cols);
+    tfhip::launch(ctx, softmax_rows_kernel<1>, grid, block, 0, xf, yf, rows, cols);
   else if (cols <= WAVE * 4)
-    hipLaunchKernelGGL(softmax_rows_kernel<4>, grid, block, 0, ctx->stream, xf, yf, rows, cols);
+    tfhip::launch(ctx, softmax_rows_kernel<4>, grid, block, 0, xf, yf, rows, cols);
   else if (cols <= WAVE * 16)
-    hipLaunchKernelGGL(softmax_rows_kernel<16>, grid, block, 0, ctx->stream, xf, yf, rows, cols);
+    tfhip::launch(ctx, softmax_rows_kernel<16>, grid, block, 0, xf, yf, rows, cols);
   else
-    hipLaunchKernelGGL(softmax_rows_kernel<0>, grid, block, 0, ctx->stream, xf, yf, rows, cols);
+    tfhip::launch(ctx, softmax_rows_kernel<0>, grid, block, 0, xf, yf, rows, cols);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }
@@ -352,10 +352,10 @@ extern "C" int tfhip_gather(tfhip_ctx* ctx, int64_t x, int64_t indices, int64_t 
   if (total == 0) return TFHIP_OK;
   const dim3 grid(grid_cap(ctx, total, 256)), block(256);
   if (dtype_size(bx->dtype) == 4)
-    hipLaunchKernelGGL(gather_kernel<int32_t>, grid, block, 0, ctx->stream, (const int32_t*)bx->ptr,
+    tfhip::launch(ctx, gather_kernel<int32_t>, grid, block, 0, (const int32_t*)bx->ptr,
                        (const int32_t*)bi->ptr, (int32_t*)bo->ptr, outer, axis_dim, inner, n_indices);
   else
-    hipLaunchKernelGGL(gather_kernel<uint8_t>, grid, block, 0, ctx->stream, (const uint8_t*)bx->ptr,
+    tfhip::launch(ctx, gather_kernel<uint8_t>, grid, block, 0, (const uint8_t*)bx->ptr,
                        (const int32_t*)bi->ptr, (uint8_t*)bo->ptr, outer, axis_dim, inner, n_indices);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -387,10 +387,10 @@ extern "C" int tfhip_transpose(tfhip_ctx* ctx, int64_t x, const int32_t* x_shape
   if (n == 0) return TFHIP_OK;
   const dim3 grid(grid_cap(ctx, n, 256)), block(256);
   if (dtype_size(bx->dtype) == 4)
-    hipLaunchKernelGGL(transpose_kernel<int32_t>, grid, block, 0, ctx->stream,
+    tfhip::launch(ctx, transpose_kernel<int32_t>, grid, block, 0,
                        (const int32_t*)bx->ptr, (int32_t*)bo->ptr, n, pa);
   else
-    hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, block, 0, ctx->stream,
+    tfhip::launch(ctx, transpose_kernel<uint8_t>, grid, block, 0,
                        (const uint8_t*)bx->ptr, (uint8_t*)bo->ptr, n, pa);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -410,10 +410,10 @@ extern "C" int tfhip_cumsum(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t oute
   if (ceil_div(outer, ROWS_PER_BLOCK) > 0x7fffffffLL) return ctx->fail(TFHIP_ENOTSUP, "cumsum: too many rows");
   const dim3 grid((unsigned)ceil_div(outer, ROWS_PER_BLOCK)), block(WAVE * ROWS_PER_BLOCK);
   if (bo->dtype == TFHIP_FLOAT32)
-    hipLaunchKernelGGL(cumsum_rows_kernel<float>, grid, block, 0, ctx->stream, bx->ptr, bx->dtype,
+    tfhip::launch(ctx, cumsum_rows_kernel<float>, grid, block, 0, bx->ptr, bx->dtype,
                        (float*)bo->ptr, outer, inner, exclusive, reverse);
   else
-    hipLaunchKernelGGL(cumsum_rows_kernel<int32_t>, grid, block, 0, ctx->stream, bx->ptr, bx->dtype,
+    tfhip::launch(ctx, cumsum_rows_kernel<int32_t>, grid, block, 0, bx->ptr, bx->dtype,
                        (int32_t*)bo->ptr, outer, inner, exclusive, reverse);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -437,10 +437,10 @@ extern "C" int tfhip_topk(tfhip_ctx* ctx, int64_t x, int64_t values, int64_t ind
   if (ceil_div(rows, ROWS_PER_BLOCK) > 0x7fffffffLL) return ctx->fail(TFHIP_ENOTSUP, "topk: too many rows");
   const dim3 grid((unsigned)ceil_div(rows, ROWS_PER_BLOCK)), block(WAVE * ROWS_PER_BLOCK);
   if (bx->dtype == TFHIP_FLOAT32)
-    hipLaunchKernelGGL(topk_rows_kernel<float>, grid, block, 0, ctx->stream, (const float*)bx->ptr,
+    tfhip::launch(ctx, topk_rows_kernel<float>, grid, block, 0, (const float*)bx->ptr,
                        (float*)bv->ptr, (int32_t*)bi->ptr, rows, cols, k);
   else
-    hipLaunchKernelGGL(topk_rows_kernel<int32_t>, grid, block, 0, ctx->stream, (const int32_t*)bx->ptr,
+    tfhip::launch(ctx, topk_rows_kernel<int32_t>, grid, block, 0, (const int32_t*)bx->ptr,
                        (int32_t*)bv->ptr, (int32_t*)bi->ptr, rows, cols, k);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;

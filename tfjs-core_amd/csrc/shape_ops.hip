@@ -175,10 +175,10 @@ extern "C" int tfhip_strided_copy(tfhip_ctx* ctx, int64_t x, int64_t out, int ra
   if (bx->ptr == bo->ptr) return ctx->fail(TFHIP_EINVAL, "strided copy: in place is not supported");
   const dim3 grid(grid_for(ctx, n, 256)), block(256);
   if (dtype_size(bx->dtype) == 4)
-    hipLaunchKernelGGL(strided_copy_kernel<int32_t>, grid, block, 0, ctx->stream,
+    tfhip::launch(ctx, strided_copy_kernel<int32_t>, grid, block, 0,
                        (const int32_t*)bx->ptr, (int32_t*)bo->ptr, n, b);
   else
-    hipLaunchKernelGGL(strided_copy_kernel<uint8_t>, grid, block, 0, ctx->stream,
+    tfhip::launch(ctx, strided_copy_kernel<uint8_t>, grid, block, 0,
                        (const uint8_t*)bx->ptr, (uint8_t*)bo->ptr, n, b);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -191,8 +191,7 @@ extern "C" int tfhip_logical_not(tfhip_ctx* ctx, int64_t x, int64_t out) {
   if (bx->dtype != TFHIP_BOOL || bo->dtype != TFHIP_BOOL || bx->numel != bo->numel)
     return ctx->fail(TFHIP_EINVAL, "logicalNot: operand and result must be bool of one size");
   if (bx->numel == 0) return TFHIP_OK;
-  hipLaunchKernelGGL(logical_not_kernel, dim3(grid_for(ctx, bx->numel, 256)), dim3(256), 0,
-                     ctx->stream, (const uint8_t*)bx->ptr, (uint8_t*)bo->ptr, bx->numel);
+  tfhip::launch(ctx, logical_not_kernel, dim3(grid_for(ctx, bx->numel, 256)), dim3(256), 0, (const uint8_t*)bx->ptr, (uint8_t*)bo->ptr, bx->numel);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }
@@ -220,8 +219,7 @@ extern "C" int tfhip_batchnorm(tfhip_ctx* ctx, int64_t x, int64_t mean, int64_t 
     return rc;
   if (boff && (rc = as_f32(ctx, boff, &to, &of))) return rc;
   if (bs && (rc = as_f32(ctx, bs, &ts, &sf))) return rc;
-  hipLaunchKernelGGL(batchnorm_kernel, dim3(grid_for(ctx, bx->numel, 256)), dim3(256), 0,
-                     ctx->stream, xf, mf, bm->numel, vf, bv->numel, of, boff ? boff->numel : 1, sf,
+  tfhip::launch(ctx, batchnorm_kernel, dim3(grid_for(ctx, bx->numel, 256)), dim3(256), 0, xf, mf, bm->numel, vf, bv->numel, of, boff ? boff->numel : 1, sf,
                      bs ? bs->numel : 1, epsilon, (float*)bo->ptr, bx->numel);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -249,8 +247,7 @@ extern "C" int tfhip_resize_bilinear(tfhip_ctx* ctx, int64_t x, int64_t out, int
   const double ew_in = (align_corners && out_w > 1) ? in_w - 1 : in_w;
   const double eh_out = (align_corners && out_h > 1) ? out_h - 1 : out_h;
   const double ew_out = (align_corners && out_w > 1) ? out_w - 1 : out_w;
-  hipLaunchKernelGGL(resize_bilinear_kernel, dim3(grid_for(ctx, bo->numel, 256)), dim3(256), 0,
-                     ctx->stream, xf, (float*)bo->ptr, batch, in_h, in_w, channels, out_h, out_w,
+  tfhip::launch(ctx, resize_bilinear_kernel, dim3(grid_for(ctx, bo->numel, 256)), dim3(256), 0, xf, (float*)bo->ptr, batch, in_h, in_w, channels, out_h, out_w,
                      eh_in / eh_out, ew_in / ew_out);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -268,11 +265,11 @@ extern "C" int tfhip_one_hot(tfhip_ctx* ctx, int64_t indices, int64_t out, int d
   if (bo->numel == 0) return TFHIP_OK;
   const dim3 grid(grid_for(ctx, bo->numel, 256)), block(256);
   if (bo->dtype == TFHIP_INT32)
-    hipLaunchKernelGGL(one_hot_kernel<int32_t>, grid, block, 0, ctx->stream,
+    tfhip::launch(ctx, one_hot_kernel<int32_t>, grid, block, 0,
                        (const int32_t*)bi->ptr, (int32_t*)bo->ptr, bi->numel, depth,
                        (int32_t)on_value, (int32_t)off_value);
   else
-    hipLaunchKernelGGL(one_hot_kernel<float>, grid, block, 0, ctx->stream,
+    tfhip::launch(ctx, one_hot_kernel<float>, grid, block, 0,
                        (const int32_t*)bi->ptr, (float*)bo->ptr, bi->numel, depth, on_value,
                        off_value);
   TFHIP_LAUNCH_CHECK(ctx);
@@ -301,8 +298,7 @@ extern "C" int tfhip_resize_nearest(tfhip_ctx* ctx, int64_t x, int64_t out, int 
   const double ew_in = (align_corners && out_w > 1) ? in_w - 1 : in_w;
   const double eh_out = (align_corners && out_h > 1) ? out_h - 1 : out_h;
   const double ew_out = (align_corners && out_w > 1) ? out_w - 1 : out_w;
-  hipLaunchKernelGGL(resize_nearest_kernel, dim3(grid_for(ctx, bo->numel, 256)), dim3(256), 0,
-                     ctx->stream, xf, (float*)bo->ptr, batch, in_h, in_w, channels, out_h, out_w,
+  tfhip::launch(ctx, resize_nearest_kernel, dim3(grid_for(ctx, bo->numel, 256)), dim3(256), 0, xf, (float*)bo->ptr, batch, in_h, in_w, channels, out_h, out_w,
                      eh_in / eh_out, ew_in / ew_out, align_corners ? 1 : 0);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
@@ -327,11 +323,11 @@ extern "C" int tfhip_select(tfhip_ctx* ctx, int64_t condition, int64_t a, int64_
   const dim3 grid(grid_for(ctx, bo->numel, 256)), block(256);
   const uint8_t* c = static_cast<const uint8_t*>(bc->ptr);
   if (dtype_size(ba->dtype) == 4)
-    hipLaunchKernelGGL(select_kernel<int32_t>, grid, block, 0, ctx->stream, c,
+    tfhip::launch(ctx, select_kernel<int32_t>, grid, block, 0, c,
                        (const int32_t*)ba->ptr, (const int32_t*)bb->ptr, (int32_t*)bo->ptr,
                        bo->numel, inner);
   else
-    hipLaunchKernelGGL(select_kernel<uint8_t>, grid, block, 0, ctx->stream, c,
+    tfhip::launch(ctx, select_kernel<uint8_t>, grid, block, 0, c,
                        (const uint8_t*)ba->ptr, (const uint8_t*)bb->ptr, (uint8_t*)bo->ptr,
                        bo->numel, inner);
   TFHIP_LAUNCH_CHECK(ctx);

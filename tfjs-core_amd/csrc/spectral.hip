@@ -57,7 +57,7 @@ extern "C" int tfhip_fft(tfhip_ctx* ctx, int64_t x, int64_t out, int64_t batch, 
   if (bx->ptr == bo->ptr && bo->numel) return ctx->fail(TFHIP_EINVAL, "fft: the transform is not in place");
   if (bo->numel == 0) return TFHIP_OK;
   const int64_t blocks = (batch * n + 255) / 256, cap = (int64_t)ctx->num_cus * 16;
-  hipLaunchKernelGGL(dft_rows_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0, ctx->stream,
+  tfhip::launch(ctx, dft_rows_kernel, dim3((unsigned)(blocks > cap ? cap : blocks)), dim3(256), 0,
                      (const float*)bx->ptr, (float*)bo->ptr, batch, n, inverse ? 1 : 0);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;

@@ -1,6 +1,7 @@
 // Internal declarations shared by the translation units of libtfjs_hip.so.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstdint>
@@ -9,7 +10,9 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <tuple>
 #include <unordered_map>
+#include <utility>
 #include <vector>
 
 #include "tfjs_hip.h"
@@ -81,29 +84,47 @@ struct tfhip_ctx {
   bool kernel_named = false;  // last_kernel was written for the launch that is being queued
   void name_kernel(const char* fmt, ...);
 
-  // KernelBackend.time with per-kernel figures (backends/backend.ts:27-31): while a time()
-  // region is open every launch is followed by an event on the stream (a "mark"); the time of
-  // a kernel is the distance between its mark and the one before it, so the figures of a
-  // region add up to its total and include whatever the device idled before that kernel.
-  // Regions nest: each remembers the mark it started at.
-  static constexpr int kMaxMarks = 1 << 16;
+  // KernelBackend.time with per-kernel figures (backends/backend.ts:27-31).  A region is
+  // bracketed by two events on the stream ("marks"); regions nest, each remembers the mark it
+  // started at.  While a region is open every kernel is launched with a start and a stop event
+  // attached to its own dispatch (hipExtLaunchKernel), so its time is the execution of that
+  // kernel on the device, as a profiler's kernel trace reports it, and no extra packet sits
+  // between two kernels.
+  static constexpr int kMaxMarks = 64;
+  static constexpr int kMaxKernelRecs = 1 << 16;
   static constexpr int kMaxTimeDepth = 8;
   struct KernelTime {
     std::string name;
     float ms;
   };
+  struct KernelRec {
+    hipEvent_t start = nullptr, stop = nullptr;
+    std::string name;
+  };
   std::vector<hipEvent_t> mark_events;  // created on demand, reused by later regions
-  std::vector<std::string> mark_names;
-  int marks_used = 0, marks_dropped = 0;
-  int time_stack[kMaxTimeDepth];
+  int marks_used = 0;
+  std::vector<KernelRec> recs;  // events created on demand, reused by later regions
+  int recs_used = 0, recs_dropped = 0;
+  struct Region {
+    int mark, rec;
+  };
+  Region time_stack[kMaxTimeDepth];
   int time_depth = 0;
   bool per_kernel = true;
   std::vector<KernelTime> kernel_times;  // of the region that ended last
-  int mark(const char* name);  // index of the new mark, -1 when none could be recorded
+  int mark();  // index of the new mark, -1 when none could be recorded
+  bool timing_kernels() const { return time_depth && per_kernel && !capturing; }
+  // The event pair for the next launch (false: launch without).
+  bool next_rec(hipEvent_t* start, hipEvent_t* stop);
+  int pending_rec = -1;  // record of the launch that is being queued, waiting for its name
   void after_launch(const char* func) {
-    if (time_depth && per_kernel && !capturing) mark(kernel_named ? last_kernel : func);
+    if (pending_rec >= 0) {
+      recs[pending_rec].name = kernel_named ? last_kernel : func;
+      pending_rec = -1;
+    }
     kernel_named = false;
   }
+
   int num_cus = 256;
   // Direction in which the next row-sweeping kernel should walk its rows: 1 = from the end.
   // A kernel leaves the rows it wrote last in the L2 of the XCD that wrote them (32 MB over the
@@ -210,6 +231,26 @@ int depthwise_forward_f32(tfhip_ctx* ctx, const float* x, const float* w, float*
                           const tfhip_conv2d_info* ci);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Every kernel of the library is launched through here, on the context's stream.  The
+// arguments are converted to the kernel's parameter types as a <<<>>> launch would.  Inside a
+// time() region the launch carries its own start / stop events.
+template <typename... Params, typename... Args>
+inline void launch(tfhip_ctx* ctx, void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds,
+                   Args&&... args) {
+  static_assert(sizeof...(Params) == sizeof...(Args), "wrong number of kernel arguments");
+  std::tuple<Params...> values{static_cast<Params>(std::forward<Args>(args))...};
+  void* ptrs[sizeof...(Params) ? sizeof...(Params) : 1];
+  {
+    int i = 0;
+    std::apply([&](auto&... v) { ((ptrs[i++] = (void*)&v), ...); }, values);
+  }
+  hipEvent_t start = nullptr, stop = nullptr;
+  if (ctx->timing_kernels() && ctx->next_rec(&start, &stop))
+    (void)hipExtLaunchKernel((const void*)kernel, grid, block, ptrs, lds, ctx->stream, start, stop, 0);
+  else
+    (void)hipLaunchKernel((const void*)kernel, grid, block, ptrs, lds, ctx->stream);
+}
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has its own
 // L2.  Remap the id so that every XCD receives one contiguous run of the work: neighbours

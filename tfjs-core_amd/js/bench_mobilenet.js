@@ -2,7 +2,20 @@
 // Throughput of the MobileNetV1 forward pass through the JavaScript host:
 //   node bench_mobilenet.js <weights_manifest.json> <input.bin> <batch> <steps> <warmup>
 // Weights (tfjs manifest + shard files) and input are written by the Python harness, so both
-// hosts run the same bytes; uint8 weights go to the device as bytes; the input is uploaded once, before the timed region.  Prints one JSON line.
+// hosts run the same bytes; uint8 weights go to the device as bytes.  Prints one JSON line:
+//   end_to_end      every step uploads its batch from host memory, runs the forward pass and
+//                   reads the class probabilities back.  The loop is pipelined the way an input
+//                   pipeline feeds a device backend: batch i+1 is uploaded (from page-locked
+//                   arrays, on the upload stream) while batch i computes, and the probabilities
+//                   are awaited two steps late (asynchronous read), so the JavaScript thread
+//                   never waits for the device inside a step.
+//   end_to_end_blocking  the same work with nothing overlapped: tf.tensor() of an ordinary
+//                   array, forward, await data(), one step after the other.
+//   resident        the input uploaded once, before the timed region.
+//   reference_graph resident input, the network written as conv -> add -> clipByValue.
+//   graph_replay    the resident step recorded once with tf.captureGraph and replayed.
+//   kernel_times    [name, ms] of every launch of one step, in launch order, averaged over the
+//                   steps of a tf.time() region (event after each launch on the stream).
 const fs = require('fs');
 const tf = require('./index.js');
 const mobilenet = require('./mobilenet.js');
@@ -11,47 +24,137 @@ function toArrayBuffer(buf) {
   return buf.buffer.slice(buf.byteOffset, buf.byteOffset + buf.byteLength);
 }
 
+const now = () => Number(process.hrtime.bigint()) / 1e6;
+
 async function main() {
   const [mPath, xPath, batchArg, stepsArg, warmArg] = process.argv.slice(2);
   const batch = +batchArg, steps = +stepsArg, warmup = +warmArg;
   await tf.setBackend('hip');
   const w = await tf.io.loadWeightsFromDisk(mPath, null, {toDevice: true});
   const xHost = new Float32Array(toArrayBuffer(fs.readFileSync(xPath)));
-  const x = tf.tensor(xHost, [batch, 224, 224, 3]);
+  const shape = [batch, 224, 224, 3];
   const be = tf.backend();
-  const step = () => {
-    const out = mobilenet.forward(tf, w, x);
+  const rate = ms => ({images_per_s: batch * steps / (ms / 1e3), ms_per_step: ms / steps});
+
+  // ---- input resident in HBM -------------------------------------------------------------
+  const x = tf.tensor(xHost, shape);
+  const step = fwd => {
+    const out = fwd(tf, w, x);
     out.logits.dispose();
     out.probs.dispose();
   };
-  for (let i = 0; i < warmup; i++) step();
+  for (let i = 0; i < warmup; i++) step(mobilenet.forward);
   be.sync();
-  const t0 = process.hrtime.bigint();
-  const info = await tf.time(() => { for (let i = 0; i < steps; i++) step(); });
+  let t0 = now();
+  for (let i = 0; i < steps; i++) step(mobilenet.forward);
   be.sync();
-  const wallMs = Number(process.hrtime.bigint() - t0) / 1e6;
+  const resident = rate(now() - t0);
+  const info = await tf.time(() => { for (let i = 0; i < steps; i++) step(mobilenet.forward); });
+  resident.gpu_ms_per_step_events = info.kernelMs / steps;
+  // per-launch times, averaged by position in the step
+  const perStep = info.kernelTimes.length / steps;
+  let kernelTimes = null;
+  if (Number.isInteger(perStep)) {
+    kernelTimes = [];
+    for (let j = 0; j < perStep; j++) {
+      let ms = 0;
+      for (let s = 0; s < steps; s++) ms += info.kernelTimes[s * perStep + j].ms;
+      kernelTimes.push([info.kernelTimes[j].name, ms / steps]);
+    }
+  }
+
+  // ---- the network as a graph of the reference's own ops ------------------------------------
+  for (let i = 0; i < Math.min(warmup, 5); i++) step(mobilenet.forwardReference);
+  be.sync();
+  t0 = now();
+  for (let i = 0; i < steps; i++) step(mobilenet.forwardReference);
+  be.sync();
+  const referenceGraph = rate(now() - t0);
+  {
+    const a = mobilenet.forward(tf, w, x), b = mobilenet.forwardReference(tf, w, x);
+    const pa = a.probs.dataSync(), pb = b.probs.dataSync();
+    let d = 0;
+    for (let i = 0; i < pa.length; i++) d = Math.max(d, Math.abs(pa[i] - pb[i]));
+    referenceGraph.max_abs_diff_vs_fused = d;
+    referenceGraph.backend_calls_per_step = 3 * 27 + 5;
+    [a.logits, a.probs, b.logits, b.probs].forEach(t => t.dispose());
+  }
+
+  // ---- end to end, pipelined ---------------------------------------------------------------
+  const slots = [be.pinnedArray('float32', xHost.length), be.pinnedArray('float32', xHost.length)];
+  slots.forEach(s => s.set(xHost));
+  const pipelined = async n => {
+    const pending = [];
+    let last = null;
+    let next = tf.tensor(slots[0], shape);
+    for (let i = 0; i < n; i++) {
+      const cur = next;
+      if (i + 1 < n) next = tf.tensor(slots[(i + 1) % 2], shape);   // overlaps with the step below
+      const out = mobilenet.forward(tf, w, cur);
+      cur.dispose();
+      out.logits.dispose();
+      pending.push(out.probs.data());
+      out.probs.dispose();
+      if (pending.length > 2) last = await pending.shift();
+    }
+    while (pending.length) last = await pending.shift();
+    return last;
+  };
+  await pipelined(Math.max(4, Math.min(warmup, 10)));
+  t0 = now();
+  const lastProbs = await pipelined(steps);
+  const endToEnd = rate(now() - t0);
+
+  // ---- end to end, nothing overlapped -------------------------------------------------------
+  const nBlocking = Math.max(3, Math.min(20, steps));
+  const blocking = async n => {
+    let probs = null;
+    for (let i = 0; i < n; i++) {
+      const xi = tf.tensor(xHost, shape);
+      const out = mobilenet.forward(tf, w, xi);
+      probs = await out.probs.data();
+      [xi, out.logits, out.probs].forEach(t => t.dispose());
+    }
+    return probs;
+  };
+  await blocking(2);
+  t0 = now();
+  const blockingProbs = await blocking(nBlocking);
+  const blockingMs = now() - t0;
+
   const out = mobilenet.forward(tf, w, x);
   const top = tf.argMax(out.logits, -1).dataSync();
   const eagerProbs = out.probs.dataSync();
-  // The same step captured once and replayed with one launch per step (tf.captureGraph, an
-  // extension of this backend): what is left when the host's cost per op is taken away.
+  let pipeDiff = 0, blockDiff = 0;
+  for (let i = 0; i < eagerProbs.length; i++) {
+    pipeDiff = Math.max(pipeDiff, Math.abs(eagerProbs[i] - lastProbs[i]));
+    blockDiff = Math.max(blockDiff, Math.abs(eagerProbs[i] - blockingProbs[i]));
+  }
+  endToEnd.max_abs_diff_vs_resident = pipeDiff;
+
+  // ---- captured graph ------------------------------------------------------------------------
   const graph = tf.captureGraph(() => mobilenet.forward(tf, w, x).probs);
   for (let i = 0; i < warmup; i++) graph.replay();
   be.sync();
-  const g0 = process.hrtime.bigint();
+  t0 = now();
   for (let i = 0; i < steps; i++) graph.replay();
   be.sync();
-  const graphMs = Number(process.hrtime.bigint() - g0) / 1e6;
+  const graphReplay = rate(now() - t0);
   const replayProbs = graph.outputs.dataSync();
   let maxDiff = 0;
   for (let i = 0; i < eagerProbs.length; i++) maxDiff = Math.max(maxDiff, Math.abs(eagerProbs[i] - replayProbs[i]));
+  graphReplay.max_abs_diff_vs_eager = maxDiff;
   graph.dispose();
+
   console.log(JSON.stringify({
-    images_per_s: batch * steps / (wallMs / 1e3), ms_per_step: wallMs / steps,
-    gpu_ms_per_step_events: info.kernelMs / steps, batch, steps, warmup,
-    node: process.version, top1_first: top[0], tensors: tf.memory().numTensors,
-    graph_replay: {images_per_s: batch * steps / (graphMs / 1e3), ms_per_step: graphMs / steps,
-                   max_abs_diff_vs_eager: maxDiff}
+    batch, steps, warmup, node: process.version, top1_first: top[0],
+    tensors: tf.memory().numTensors,
+    end_to_end: endToEnd,
+    end_to_end_blocking: {images_per_s: batch * nBlocking / (blockingMs / 1e3),
+                          ms_per_step: blockingMs / nBlocking, steps: nBlocking,
+                          max_abs_diff_vs_resident: blockDiff},
+    resident, reference_graph: referenceGraph, graph_replay: graphReplay,
+    kernel_times: kernelTimes
   }));
 }
 

@@ -44,4 +44,23 @@ function forward(tf, w, x) {
   });
 }
 
-module.exports = {BLOCKS, NUM_CLASSES, weightSpecs, forward};
+// The same network written only with calls that exist in the reference at this commit: every
+// layer is conv -> add -> clipByValue(0, 6), the dense layer matMul -> add, as a graph produced
+// for tfjs-core 1.2 states it.  Three backend calls per layer instead of one.
+function forwardReference(tf, w, x) {
+  return tf.tidy(() => {
+    const relu6 = (t, bias) => tf.clipByValue(tf.add(t, bias), 0, 6);
+    let h = relu6(tf.conv2d(x, w.stem_w, 2, 'same'), w.stem_b);
+    BLOCKS.forEach((b, i) => {
+      const n = i + 1;
+      h = relu6(tf.depthwiseConv2d(h, w[`dw${n}_w`], b[1], 'same'), w[`dw${n}_b`]);
+      h = relu6(tf.conv2d(h, w[`pw${n}_w`], 1, 'same'), w[`pw${n}_b`]);
+    });
+    h = tf.avgPool(h, [h.shape[1], h.shape[2]], 1, 'valid');
+    h = tf.reshape(h, [h.shape[0], h.shape[3]]);
+    const logits = tf.add(tf.matMul(h, w.fc_w), w.fc_b);
+    return {logits, probs: tf.softmax(logits)};
+  });
+}
+
+module.exports = {BLOCKS, NUM_CLASSES, weightSpecs, forward, forwardReference};
