@@ -200,6 +200,24 @@ int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t out,
                  const tfhip_conv2d_info* info, int64_t bias, int bias_kind, int act,
                  int64_t prelu, int prelu_kind, const tfhip_qparams* q);
 
+/* A depthwise convolution followed by a pointwise (1x1) one, the block of depthwise-separable
+ * networks (separableConv2d, ops/conv.ts:588-660, composes depthwiseConv2d and conv2d;
+ * backend_cpu.ts:1979-2035, 1552-1616), with the add + clip/relu that follows each folded in:
+ *   out = act_pw(conv1x1(act_dw(depthwise(x, dw_filter) + dw_bias), pw_filter) + pw_bias).
+ * dw_info is the Conv2DInfo of the depthwise half; pw_filter is [1,1,dw_info.out_c,out_c] and
+ * out [batch,out_h,out_w,out_c].  Biases NONE / SCALAR / COLUMN, activations LINEAR / RELU /
+ * RELU6; either filter may be TFHIP_UINT8Q with its qparams.  For 3x3 filters, multiplier 1 and
+ * (channels, stride) in {(32->64, 1), (64->128, 2)} on large images one kernel computes both
+ * halves and the intermediate never reaches HBM; every other shape runs the two kernels with
+ * the intermediate in a pool block.  Results are those of the two calls (the single kernel sums
+ * the pointwise products in another order: equal within float32 round-off).
+ * tfhip_separable_single_kernel(ctx, 0) forces the two-kernel form (1 restores the default). */
+int tfhip_separable_conv2d(tfhip_ctx* ctx, int64_t x, int64_t dw_filter, int64_t pw_filter,
+                           int64_t out, const tfhip_conv2d_info* dw_info, int64_t dw_bias,
+                           int dw_bias_kind, int dw_act, int64_t pw_bias, int pw_bias_kind,
+                           int pw_act, const tfhip_qparams* dw_q, const tfhip_qparams* pw_q);
+int tfhip_separable_single_kernel(tfhip_ctx* ctx, int enable);
+
 /* ---- memory-bound image kernels ------------------------------------------------------ */
 /* depthwiseConv2D (backend.ts:431-434; backend_cpu.ts:1979-2035): filter
  * [fh,fw,in_c,ch_mul], out_c = in_c*ch_mul.  bias (NONE / SCALAR / COLUMN over out_c) and

@@ -128,7 +128,7 @@ def test_mobilenet_uint8_batch256_matches_oracle(tf, ref):
         got, got_probs = out["l"].data_sync(), out["p"].data_sync()
     names = [k[0] for k in info["kernelTimes"]]
     print("kernels of the batch-256 uint8 step:", sorted(set(names)), flush=True)
-    dense = [n for n in names if n.startswith(("gemm_", "conv_smallk", "sep_"))]
+    dense = [n for n in names if n.startswith(("gemm_", "conv_smallk", "separable_"))]
     assert len(dense) >= 15 and all("u8" in n for n in dense), dense
     assert any(n.startswith("depthwise") for n in names)
     idx = np.arange(256) % 8

@@ -822,3 +822,85 @@ def test_where_bit_exact(hip, ref):
 def test_mean(hip, ref, shape, axis, keep):
     x = rng_for("mean", shape).standard_normal(shape).astype(np.float32)
     close(hip.mean(x, axis, keep), ref.mean(x, axis, keep))
+
+
+# ------------------------------------------------- depthwise + pointwise as one call ----
+def _separable_oracle(ref, x, dw, pw, stride, dbias, dact, pbias, pact):
+    mid = ref.depthwise_conv2d(x, dw, stride, "same", bias=dbias, activation=dact)
+    return ref.conv2d(mid, pw, 1, "valid", bias=pbias, activation=pact)
+
+
+@pytest.mark.parametrize("xs,cout,stride", [
+    ((16, 112, 112, 32), 64, 1),    # single kernel: K 32 -> N 64
+    ((64, 112, 112, 64), 128, 2),   # single kernel, stride 2 (top/left padding 0)
+    ((64, 56, 56, 128), 128, 1),    # K 128 -> N 128: the filter leaves no room for the panels, two kernels
+    ((17, 113, 111, 32), 64, 1),    # odd extents: blocks straddle rows and images, last block short
+    ((66, 111, 113, 64), 128, 2),   # stride 2 on odd extents (padding 1 on both sides)
+    ((2, 20, 20, 32), 64, 1),       # too few pixels for the single kernel: two-kernel form
+    ((1, 9, 9, 12), 20, 2),         # channel counts without a single-kernel variant
+])
+def test_separable_conv2d_matches_the_two_op_chain(hip, ref, xs, cout, stride):
+    """tf.fused.separableConv2d against the oracle's depthwise -> add -> clip -> conv2d -> add ->
+    clip chain, and bit for bit against the backend's own two-kernel form."""
+    print("separable", xs, cout, stride, flush=True)
+    tf = hip.tf
+    be = tf.backend()
+    rng = rng_for("separable", xs, cout, stride)
+    c = xs[3]
+    x = rng.uniform(0, 1, xs).astype(np.float32)
+    dw = (rng.standard_normal((3, 3, c, 1)) * np.sqrt(2.0 / 9)).astype(np.float32)
+    pw = (rng.standard_normal((1, 1, c, cout)) * np.sqrt(2.0 / c)).astype(np.float32)
+    dbias = (rng.standard_normal(c) * 0.1).astype(np.float32)
+    pbias = (rng.standard_normal(cout) * 0.1).astype(np.float32)
+
+    def run(dact, pact, db, pb):
+        with tf.tidy():
+            t = lambda a: None if a is None else tf.tensor(a)
+            info = tf.time(lambda: out.append(tf.fused.separable_conv2d(
+                t(x), t(dw), t(pw), stride, "same", depthwise_bias=t(db),
+                depthwise_activation=dact, bias=t(pb), activation=pact)))
+            return out.pop().data_sync(), [k[0] for k in info["kernelTimes"]]
+
+    out = []
+    # the oracle is scalar: compare a slice of the batch (first and last image) at full size
+    pick = [0, xs[0] - 1] if xs[1] > 50 else list(range(xs[0]))
+    for dact, pact, db, pb in (("relu6", "relu6", dbias, pbias), ("linear", "relu", None, pbias),
+                               ("relu", "linear", dbias[:1], None)):
+        got, kernels = run(dact, pact, db, pb)
+        single = len(kernels) == 1 and kernels[0].startswith("separable_")
+        pixels = xs[0] * -(-xs[1] // stride) * -(-xs[2] // stride)
+        expect_single = pixels >= 256 * 8 * 32 * 3 and \
+            (c, cout, stride) in ((32, 64, 1), (64, 128, 2))
+        assert single == expect_single, kernels
+        want = _separable_oracle(ref, x[pick], dw, pw, stride, db, dact, pb, pact)
+        close(got[pick], want)
+        if single:
+            be.lib.tfhip_separable_single_kernel(be.ctx, 0)
+            try:
+                two, kernels2 = run(dact, pact, db, pb)
+            finally:
+                be.lib.tfhip_separable_single_kernel(be.ctx, 1)
+            assert len(kernels2) == 2, kernels2
+            close(got, two, rtol=2e-5, atol=2e-6)
+
+
+def test_separable_conv2d_uint8_filters(hip, ref):
+    """Both filters kept as uint8 in HBM and dequantised inside the single kernel."""
+    tf = hip.tf
+    from tfhip import mobilenet
+    rng = rng_for("separable-u8")
+    x = rng.uniform(0, 1, (16, 112, 112, 32)).astype(np.float32)
+    params = {"dw_w": (rng.standard_normal((3, 3, 32, 1)) * 0.5).astype(np.float32),
+              "pw_w": (rng.standard_normal((1, 1, 32, 64)) * 0.25).astype(np.float32)}
+    q = mobilenet.quantize_params(params)
+    deq = {k: ref.dequantize(*v) for k, v in q.items()}
+    bias = (rng.standard_normal(64) * 0.1).astype(np.float32)
+    with tf.tidy():
+        out = []
+        info = tf.time(lambda: out.append(tf.fused.separable_conv2d(
+            tf.tensor(x), tf.quantized_tensor(*q["dw_w"]), tf.quantized_tensor(*q["pw_w"]), 1, "same",
+            depthwise_activation="relu6", bias=tf.tensor(bias), activation="relu6")))
+        got = out[0].data_sync()
+    assert [k[0] for k in info["kernelTimes"]] == ["separable_s1_k32xn64_u8"]
+    want = _separable_oracle(ref, x[:1], deq["dw_w"], deq["pw_w"], 1, None, "relu6", bias, "relu6")
+    close(got[:1], want)

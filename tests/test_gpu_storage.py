@@ -322,6 +322,37 @@ def test_async_read_returns_what_sync_read_returns(tf):
     assert b"unknown data id" in be.lib.tfhip_last_error(be.ctx)
 
 
+def test_dispose_during_an_async_read_keeps_the_block_out_of_reach(tf):
+    """A tensor disposed while its asynchronous read is still copying: the block neither goes to
+    the next tensor of that size before the copy is done (the pool holds it back until the read
+    is finished), nor is it lost (afterwards the pool hands it out again), and tf.memory() counts
+    it as pooled, not in use, from the dispose on."""
+    rng = np.random.default_rng(25)
+    n = 3 * 1000 * 1000 + 17                 # a size class no other test of this module uses
+    vals = [rng.standard_normal(n).astype(np.float32) for _ in range(4)]
+    be = tf.backend()
+    two = tf.tensor(np.float32(2.0))
+    base = tf.memory()["numBytesInGPU"]
+    reads = []
+    for i, v in enumerate(vals):
+        t = tf.tensor(v)
+        u = tf.mul(t, two)                     # queued work in front of the read
+        reads.append(u.data())
+        tf.dispose([t, u])                    # while the copy of u is (most likely) still running
+        # the next tensor of the same size must not land in u's block before the copy is over
+        w = tf.tensor(np.full(n, -7.0, np.float32))
+        tf.dispose(tf.add(w, w))
+        w.dispose()
+    assert tf.memory()["numBytesInGPU"] == base
+    for v, r in zip(vals, reads):
+        np.testing.assert_array_equal(r.result(), v * np.float32(2.0))
+    pooled = tf.memory()["numBytesInGPUPool"]
+    t = tf.tensor(vals[0])                    # comes out of the pool: no new device memory
+    assert tf.memory()["numBytesInGPUPool"] < pooled
+    np.testing.assert_array_equal(t.data_sync(), vals[0])
+    tf.dispose([t, two])
+
+
 def test_time_reports_every_kernel_and_nests(tf):
     """KernelBackend.time with the per-kernel figures behind getExtraProfileInfo
     (backend.ts:27-31): one entry per launch, in order, each the execution time of its kernel."""

@@ -20,7 +20,7 @@ ADDON = os.path.join(HERE, "js", "tfjs_hip.node")
 NODE_INCLUDE = "/usr/include/node"
 
 HIP_SOURCES = ["context.hip", "gemm.hip", "image.hip", "elementwise.hip", "reduce.hip",
-               "shape_ops.hip", "backward.hip", "indexing.hip", "spectral.hip"]
+               "shape_ops.hip", "backward.hip", "indexing.hip", "spectral.hip", "separable.hip"]
 # Packed fp32 VALU ops are switched off for every kernel (scalar/float2 code only).
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC,
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -36,7 +36,7 @@ def _stale(target, sources):
 
 def build_lib(force=False, verbose=False):
     srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
-    deps = srcs + [os.path.join(CSRC, "tfhip_internal.h"), os.path.join(INCLUDE, "tfjs_hip.h")]
+    deps = srcs + [os.path.join(CSRC, "tfhip_internal.h"), os.path.join(CSRC, "tfhip_device.h"), os.path.join(INCLUDE, "tfjs_hip.h")]
     if not force and not _stale(LIB, deps):
         return LIB
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"

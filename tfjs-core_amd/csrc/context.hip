@@ -191,6 +191,22 @@ void* tfhip_ctx::alloc(size_t nbytes, size_t* cap, hipEvent_t* ready, bool* recy
     }
     return p;
   }
+  for (size_t i = 0; i < held.size(); i++) {
+    if (held[i].cap != want) continue;
+    // no free block of this size, but one whose read is still copying: take it and put the copy
+    // in front of whatever the compute stream does next
+    const HeldBlock h = held[i];
+    held[i] = held.back();
+    held.pop_back();
+    (void)hipStreamWaitEvent(stream, h.done, 0);
+    ev_put(h.left);
+    pooled -= want;
+    in_use += want;
+    *cap = want;
+    if (capturing) capture_blocks.push_back(h.p);
+    if (recycled) *recycled = true;
+    return h.p;
+  }
   if (capturing) {
     // a capture must find every block in the pool (the same work has run once before it):
     // allocating here would put a device allocation into the middle of a stream capture
@@ -221,6 +237,11 @@ void tfhip_ctx::release(void* p, size_t cap, hipEvent_t ready) {
     return;
   }
   in_use -= cap;
+  pooled += cap;
+  park(p, cap, ready);
+}
+
+void tfhip_ctx::park(void* p, size_t cap, hipEvent_t ready) {
   if (ready) {
     auto old = block_ready.find(p);
     if (old != block_ready.end()) ev_put(old->second);
@@ -228,11 +249,23 @@ void tfhip_ctx::release(void* p, size_t cap, hipEvent_t ready) {
   }
   auto own = owner.find(p);
   if (own != owner.end()) {  // a block that a captured graph writes on every replay
+    pooled -= cap;
     graphs[own->second].parked.emplace_back(p, cap);
     return;
   }
-  pooled += cap;
   pool[cap].push_back(p);
+}
+
+void tfhip_ctx::unhold(hipEvent_t done) {
+  for (size_t i = 0; i < held.size();) {
+    if (held[i].done == done) {
+      park(held[i].p, held[i].cap, held[i].left);
+      held[i] = held.back();
+      held.pop_back();
+    } else {
+      i++;
+    }
+  }
 }
 
 // A buffer lets go of its block.  Copies still in flight on the other streams are put in
@@ -244,7 +277,6 @@ void tfhip_ctx::release_buf(Buf& b) {
     (void)hipStreamWaitEvent(stream, b.uploaded, 0);
     ev_put(b.uploaded);
   }
-  if (b.read_done) (void)hipStreamWaitEvent(stream, b.read_done, 0);  // owned by the read's ticket
   hipEvent_t left = nullptr;
   if (b.ready) {
     if (b.used) ev_put(b.ready);
@@ -257,7 +289,16 @@ void tfhip_ctx::release_buf(Buf& b) {
       left = nullptr;
     }
   }
-  release(b.ptr, b.cap, left);
+  if (b.read_done && b.ptr) {
+    // An asynchronous read is still copying out of the block: it goes back to the pool when the
+    // read's ticket is finished.  (Waiting for the copy on the compute stream here would hold up
+    // every kernel queued after this dispose for the length of a cross-stream round trip.)
+    in_use -= b.cap;
+    pooled += b.cap;
+    held.push_back({b.ptr, b.cap, b.read_done, left});
+  } else {
+    release(b.ptr, b.cap, left);
+  }
   b.ptr = nullptr;
   b.uploaded = b.read_done = b.ready = nullptr;
 }
@@ -277,6 +318,7 @@ void tfhip_ctx::trim() {
     }
   pool.clear();
   pooled = 0;
+  for (const HeldBlock& h : held) pooled += h.cap;  // (they wait for their reads, outside the pool)
 }
 
 extern "C" {
@@ -353,6 +395,10 @@ void tfhip_destroy(tfhip_ctx* ctx) {
   if (ctx->ring) (void)hipHostFree(ctx->ring);
   for (auto& kv : ctx->pool)
     for (void* p : kv.second) (void)hipFree(p);
+  for (auto& h : ctx->held) {
+    (void)hipFree(h.p);
+    if (h.left) (void)hipEventDestroy(h.left);
+  }
   for (auto& kv : ctx->graphs) {
     (void)hipGraphExecDestroy(kv.second.exec);
     (void)hipGraphDestroy(kv.second.graph);
@@ -550,6 +596,7 @@ int tfhip_read_finish(tfhip_ctx* ctx, tfhip_pending_read* r, void* host, size_t 
       if (buf != ctx->bufs.end() && buf->second.read_done == r->done) buf->second.read_done = nullptr;
       ctx->reads.erase(it);
     }
+    if (r->done) ctx->unhold(r->done);  // the copy is complete (or failed for good)
     ctx->ev_put(r->done);
   } else if (r->done) {
     (void)hipEventDestroy(r->done);

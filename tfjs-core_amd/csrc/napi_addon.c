@@ -455,6 +455,29 @@ static napi_value js_depthwise(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+/* separableConv2d(ctx, x, dwFilter, pwFilter, out, dwInfo, dwBias, dwBiasKind, dwAct, pwBias,
+ *                 pwBiasKind, pwAct, dwQ, pwQ) */
+static napi_value js_separable(napi_env env, napi_callback_info info) {
+  ARGS(14);
+  I64(1, x); I64(2, dw); I64(3, pw); I64(4, out);
+  tfhip_conv2d_info ci;
+  if (!arg_conv_info(env, argv[5], &ci)) return NULL;
+  I64(6, dw_bias); INT(7, dw_bias_kind); INT(8, dw_act);
+  I64(9, pw_bias); INT(10, pw_bias_kind); INT(11, pw_act);
+  tfhip_qparams dq, pq; const tfhip_qparams* dqp; const tfhip_qparams* pqp;
+  if (!arg_qparams(env, argv[12], &dq, &dqp) || !arg_qparams(env, argv[13], &pq, &pqp)) return NULL;
+  CHECK(tfhip_separable_conv2d(ctx, x, dw, pw, out, &ci, dw_bias, dw_bias_kind, dw_act, pw_bias,
+                               pw_bias_kind, pw_act, dqp, pqp));
+  return undefined(env);
+}
+
+static napi_value js_separable_single_kernel(napi_env env, napi_callback_info info) {
+  ARGS(2);
+  INT(1, enable);
+  CHECK(tfhip_separable_single_kernel(ctx, enable));
+  return undefined(env);
+}
+
 /* pool2d(ctx, x, out, info, kind) */
 static napi_value js_pool2d(napi_env env, napi_callback_info info) {
   ARGS(5);
@@ -812,7 +835,8 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"timeEnd", js_time_end}, {"timeKernels", js_time_kernels},
       {"timePerKernel", js_time_per_kernel}, {"hostAlloc", js_host_alloc},
       {"readAsync", js_read_async}, {"lastKernel", js_last_kernel}, {"matmul", js_matmul}, {"matmulNoalloc", js_matmul_noalloc},
-      {"conv2d", js_conv2d}, {"depthwiseConv2d", js_depthwise}, {"pool2d", js_pool2d},
+      {"conv2d", js_conv2d}, {"depthwiseConv2d", js_depthwise}, {"separableConv2d", js_separable},
+      {"separableSingleKernel", js_separable_single_kernel}, {"pool2d", js_pool2d},
       {"binary", js_binary}, {"unary", js_unary}, {"cast", js_cast}, {"copy", js_copy},
       {"dequantize", js_dequantize}, {"fill", js_fill}, {"reduce", js_reduce},
       {"softmaxRows", js_softmax_rows}, {"gather", js_gather}, {"transpose", js_transpose},

@@ -1,0 +1,591 @@
+// Depthwise 3x3 convolution and the pointwise (1x1) convolution that follows it, as one kernel:
+// the block a depthwise-separable network repeats (separableConv2d of the reference,
+// ops/conv.ts:588-660, composes depthwiseConv2d and conv2d at op level; backend_cpu.ts:1979-2035
+// and :1552-1616 run them), with the bias + activation that follows each of the two folded in.
+//
+// Why one kernel.  For the first blocks of such a network both halves are bound by HBM: the
+// depthwise kernel writes an activation that the pointwise product reads right back.  Here the
+// depthwise result never leaves the CU: a wavefront computes it for 32 output pixels into its
+// own panel in LDS and multiplies the panel by the pointwise filter on the matrix cores.
+// HBM sees the block's input once and its output once.
+//
+// Shape.  The pointwise filter [K, N] (K = input channels, N = output channels) lies in LDS in
+// operand order for the whole kernel, so this kernel serves the blocks whose filter fits
+// (K * N * 4 <= 64 KiB).  A wavefront works on its own: it takes a strip of SW output columns of
+// one image and walks down a chunk of output rows.
+//   depthwise stage: lanes run along the channels (a lane owns one quad of 4 channels and TW
+//     neighbouring output columns, so a wavefront access is a run of 16-byte pieces).  Every
+//     input row of the strip is fetched once (buffer loads whose offsets fall outside the
+//     descriptor where the padding is; PD rows in flight) and feeds the output rows it belongs
+//     to, which live in rotating accumulators; taps are summed in the order filter row, filter
+//     column, as the reference does.  A finished row gets its bias and activation and goes to
+//     the panel [pixel][k]; RB rows fill the panel's 32 pixels.
+//   pointwise stage: lane = pixel of the panel (16-byte LDS reads of 4 consecutive k; lanes
+//     0-31 take k = 0..3 and lanes 32-63 k = 4..7 of each group of 8, the operand order the
+//     filter was laid out in), v_mfma_f32_32x32x2f32 into N / 32 accumulators, bias + activation,
+//     dword stores of 128-byte runs.
+// Wavefronts of a workgroup share nothing but the filter, so there is no barrier after the set-up;
+// the other wavefronts of the SIMD fill the time one of them waits for memory or the matrix cores.
+#include <cstdlib>
+#include <type_traits>
+
+#include "tfhip_internal.h"
+#include "tfhip_device.h"
+
+namespace tfhip {
+
+// relu / relu6 / linear as a clamp to [lo, hi] that lets NaN through (no comparison with NaN
+// holds), which is what the reference's Math.max(0, x) and clip do (backend_cpu.ts:1191-1201,
+// :1265-1275): two compares and two selects per value.
+struct Clamp {
+  float lo, hi;
+};
+__device__ __forceinline__ Clamp clamp_of(int act) {
+  Clamp c;
+  c.lo = act == TFHIP_ACT_LINEAR ? -__builtin_inff() : 0.f;
+  c.hi = act == TFHIP_ACT_RELU6 ? 6.f : __builtin_inff();
+  return c;
+}
+__device__ __forceinline__ float clamp(float v, const Clamp& c) {
+  const float r = v < c.lo ? c.lo : v;
+  return r > c.hi ? c.hi : r;
+}
+
+struct SepArgs {
+  const float* x;
+  const void* dw;    // [3][3][K] float32 or uint8
+  const float* dwb;  // depthwise bias: nullptr, 1 element or K elements
+  const void* pw;    // [K][N] float32 or uint8
+  const float* pwb;  // pointwise bias: nullptr, 1 element or N elements
+  float* y;
+  int batch, H, W, OH, OW, pt, pl;
+  int dwb_kind, pwb_kind, dw_act, pw_act;
+  int dw_quant, pw_quant;
+  double dw_scale, dw_min, pw_scale, pw_min;
+  unsigned x_bytes, y_bytes;
+  int rh;      // output rows of a unit (a multiple of the panel's rows)
+  int chunks;  // units per strip of an image: ceil(OH / rh)
+  int strips;  // ceil(OW / SW)
+  int units;   // batch * chunks * strips
+  int reverse;
+};
+
+template <int KQ, int NJ, int S, int PD, int OCC>
+__global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
+  constexpr int K = 8 * KQ, N = 32 * NJ;
+  constexpr int QN = K / 4;            // channel quads = lanes side by side along the channels
+  constexpr int PX = 64 / QN;          // pixel slots of a wavefront
+  constexpr int TW = S == 1 ? 2 : 1;   // output columns of a lane
+  constexpr int SW = PX * TW;          // output columns of a strip
+  constexpr int RB = 32 / SW;          // output rows that fill a panel
+  constexpr int NV = (TW - 1) * S + 3; // input vectors of a lane per input row
+  constexpr int PITCH = K + 4;         // floats per panel row: 16-byte reads of a lane stay conflict-free
+  constexpr int LEAD = 3 - S;          // input rows of a unit before the first one that completes an output row
+  static_assert(QN <= 64 && 64 % QN == 0 && 32 % SW == 0, "a wavefront covers whole pixels and rows");
+  static_assert(LEAD <= PD && (PD % ((S * RB) % PD ? (S * RB) % PD : 1) == 0) && PD / ((S * RB) % PD ? (S * RB) % PD : PD) <= 4,
+                "row buffers take turns with a period of at most four panels");
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  float* bl = lds;  // pointwise filter as [K / 4][N][4] = (k / 4, col, k % 4)
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool producer = wave < 4;
+  const int pair = wave & 3;
+  const int l32 = lane & 31, g = lane >> 5;
+  float* panels = lds + K * N + pair * (2 * 32 * PITCH);  // the pair's two panels
+
+  {
+    // the pointwise filter into operand order: an item is 4 consecutive k of one column
+    constexpr int PER = (K / 4 * N + 511) / 512;
+    auto fill = [&](auto quant_tag) {
+      f32x4 w[PER];
+#pragma unroll
+      for (int u = 0; u < PER; u++) {
+        const int item = tid + 512 * u;
+        const int k4 = item / N, col = item - k4 * N;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int at = (4 * k4 + e) * N + col;
+          if (decltype(quant_tag)::value)
+            w[u][e] = dequant(static_cast<const unsigned char*>(p.pw)[at], p.pw_scale, p.pw_min);
+          else
+            w[u][e] = static_cast<const float*>(p.pw)[at];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < PER; u++)
+        *reinterpret_cast<f32x4*>(&bl[(tid + 512 * u) * 4]) = w[u];
+    };
+    static_assert(K / 4 * N % 512 == 0, "whole passes");
+    if (p.pw_quant) fill(std::true_type{});
+    else fill(std::false_type{});
+  }
+
+  // The units (image, chunk of rows, strip; strip fastest) are cut into 8 runs, one per XCD
+  // (workgroup b runs on XCD b % 8; the grid is a multiple of 8): the kernels before and after
+  // this one cut their rows the same way, so what an XCD leaves in its L2 is what it reads next.
+  // Within its run a workgroup takes four neighbouring units (they share their halo columns),
+  // one per pair of wavefronts, then the four `stride` further on, ...
+  const int xcd = (int)blockIdx.x & 7;
+  const int per = p.units >> 3, rem = p.units & 7;
+  const int run0 = xcd * per + (xcd < rem ? xcd : rem);
+  const int run1 = run0 + per + (xcd < rem ? 1 : 0);
+  const int wg_first = run0 + ((int)blockIdx.x >> 3) * 4;
+  const int stride = ((int)gridDim.x >> 3) * 4;
+  const int trips = wg_first < run1 ? (run1 - wg_first + stride - 1) / stride : 0;
+  const int iters = (p.rh + RB - 1) / RB;  // panels of a unit
+  const int total = trips * iters;
+  struct Unit {
+    bool live;
+    int n, o0, rows, strip;
+  };
+  auto unit_of = [&](int trip) {
+    Unit un;
+    const int u = wg_first + trip * stride + pair;
+    un.live = u < run1;
+    const int unit = p.reverse ? run0 + run1 - 1 - u : u;
+    un.strip = unit % p.strips;
+    const int rest = unit / p.strips;
+    const int chunk = rest % p.chunks;
+    un.n = rest / p.chunks;
+    un.o0 = chunk * p.rh;
+    un.rows = min(p.rh, p.OH - un.o0);
+    return un;
+  };
+
+  if (producer) {
+    // ---- depthwise wavefronts: input rows -> panel -------------------------------------------
+    const int quad = lane % QN, slot = lane / QN;
+    f32x4 w[9], dwb = {0.f, 0.f, 0.f, 0.f};
+    if (p.dw_quant) {
+      const unsigned char* wq = static_cast<const unsigned char*>(p.dw);
+#pragma unroll
+      for (int i = 0; i < 9; i++) {
+        const unsigned v = *reinterpret_cast<const unsigned*>(wq + i * K + 4 * quad);
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[i][e] = dequant((v >> (8 * e)) & 0xffu, p.dw_scale, p.dw_min);
+      }
+    } else {
+      const float* wf = static_cast<const float*>(p.dw);
+#pragma unroll
+      for (int i = 0; i < 9; i++) w[i] = *reinterpret_cast<const f32x4*>(wf + i * K + 4 * quad);
+    }
+    if (p.dwb_kind == TFHIP_BCAST_COLUMN) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) dwb[e] = p.dwb[4 * quad + e];
+    } else if (p.dwb_kind == TFHIP_BCAST_SCALAR) {
+      dwb = f32x4{p.dwb[0], p.dwb[0], p.dwb[0], p.dwb[0]};
+    }
+    const Clamp dact = clamp_of(p.dw_act);
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.x, p.x_bytes);
+    const unsigned x_row = (unsigned)(p.W * K * 4);
+    float* const panel_w = panels + (slot * TW) * PITCH + 4 * quad;  // where this lane writes
+    __syncthreads();
+
+    // Input row t of a unit (counted from the top of the padding, ih = t - pt) is filter row kh
+    // of output row (t - kh) / S.  The unit consumes rows t0 .. t_last in turn; rows in the
+    // padding and beyond t_last are read through an offset outside the descriptor (zeros).
+    unsigned col_in[NV];
+    unsigned x_img = 0;
+    int t0 = 0, t_last = -1;
+    auto load_row = [&](int t, f32x4 (&in)[NV]) {
+      const int ih = t - p.pt;
+      const bool row_ok = (unsigned)ih < (unsigned)p.H && t <= t_last;
+      const unsigned at = x_img + (unsigned)ih * x_row;
+#pragma unroll
+      for (int v = 0; v < NV; v++) in[v] = buffer_load_f32x4(rx, row_ok ? at + col_in[v] : OOB_OFFSET);
+    };
+    auto taps = [&](f32x4& acc, const f32x4 (&in)[NV], int j, int kh) {
+#pragma unroll
+      for (int kw = 0; kw < 3; kw++) acc += in[j * S + kw] * w[kh * 3 + kw];
+    };
+    // a finished output row of the strip: bias, activation, into row `rb` of the panel
+    auto emit = [&](float* panel, int rb, const f32x4 (&acc)[TW]) {
+#pragma unroll
+      for (int j = 0; j < TW; j++) {
+        f32x4 v;
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = clamp(acc[j][e] + dwb[e], dact);
+        *reinterpret_cast<f32x4*>(panel + (rb * SW + j) * PITCH) = v;
+      }
+    };
+    f32x4 buf[PD][NV];
+    f32x4 A[TW], B[TW], C[TW];  // output rows in the making, oldest first (stride 2 has A only)
+    int trip = 0, blk = 0;
+    for (int it = 0; it <= total; it++) {
+      if (it < total) {
+        if (blk == 0) {
+          // a new unit: its offsets, the first PD rows, the rows before the first output row
+          const Unit un = unit_of(trip);
+          t0 = un.o0 * S;
+          t_last = un.live ? (un.o0 + un.rows - 1) * S + 2 : t0 - 1;
+          const int iw0 = (un.strip * SW + slot * TW) * S - p.pl;
+#pragma unroll
+          for (int v = 0; v < NV; v++)
+            col_in[v] = (unsigned)(iw0 + v) < (unsigned)p.W ? (unsigned)(((iw0 + v) * K + 4 * quad) * 4)
+                                                            : OOB_OFFSET;
+          x_img = (unsigned)un.n * (unsigned)p.H * x_row;
+#pragma unroll
+          for (int i = 0; i < PD; i++) load_row(t0 + i, buf[i]);
+          if (S == 1) {
+#pragma unroll
+            for (int j = 0; j < TW; j++) {
+              B[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+              taps(B[j], buf[0], j, 0);
+            }
+            load_row(t0 + PD, buf[0]);
+#pragma unroll
+            for (int j = 0; j < TW; j++) {
+              A[j] = B[j];
+              taps(A[j], buf[1 % PD], j, 1);
+              B[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+              taps(B[j], buf[1 % PD], j, 0);
+            }
+            load_row(t0 + 1 + PD, buf[1 % PD]);
+          } else {
+#pragma unroll
+            for (int j = 0; j < TW; j++) {
+              A[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+              taps(A[j], buf[0], j, 0);
+            }
+            load_row(t0 + PD, buf[0]);
+          }
+        }
+        float* const panel = panel_w + (it & 1) * (32 * PITCH);
+        const int i0 = LEAD + blk * RB * S;  // index (from t0) of the first row consumed here
+        // Row i of the unit lives in buffer i % PD; PH = (i0 - LEAD) % PD picks the copy of the
+        // steps whose buffer numbers are compile-time constants.
+        auto steps = [&](auto phase_tag) {
+          constexpr int PH = decltype(phase_tag)::value;
+#pragma unroll
+          for (int rb = 0; rb < RB; rb++) {
+            if (S == 1) {
+              f32x4 (&in)[NV] = buf[(LEAD + PH + rb) % PD];
+#pragma unroll
+              for (int j = 0; j < TW; j++) {
+                C[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                taps(C[j], in, j, 0);
+                taps(B[j], in, j, 1);
+                taps(A[j], in, j, 2);
+              }
+              emit(panel, rb, A);
+#pragma unroll
+              for (int j = 0; j < TW; j++) {
+                A[j] = B[j];
+                B[j] = C[j];
+              }
+              load_row(t0 + i0 + rb + PD, in);
+            } else {
+              f32x4 (&in1)[NV] = buf[(LEAD + PH + 2 * rb) % PD];
+              f32x4 (&in2)[NV] = buf[(LEAD + PH + 2 * rb + 1) % PD];
+#pragma unroll
+              for (int j = 0; j < TW; j++) {
+                taps(A[j], in1, j, 1);
+                taps(A[j], in2, j, 2);
+              }
+              emit(panel, rb, A);
+#pragma unroll
+              for (int j = 0; j < TW; j++) {
+                A[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                taps(A[j], in2, j, 0);
+              }
+              load_row(t0 + i0 + 2 * rb + PD, in1);
+              load_row(t0 + i0 + 2 * rb + 1 + PD, in2);
+            }
+          }
+        };
+        constexpr int STEP = (S * RB) % PD;  // how far a panel moves the phase
+        if (STEP == 0) {
+          steps(std::integral_constant<int, 0>{});
+        } else {
+          static_assert(STEP == 0 || PD % STEP == 0, "the phases repeat");
+          const int phase = (blk * RB * S) % PD;
+          if (PD / (STEP ? STEP : 1) == 2) {
+            if (phase == 0) steps(std::integral_constant<int, 0>{});
+            else steps(std::integral_constant<int, STEP>{});
+          } else {
+            if (phase == 0) steps(std::integral_constant<int, 0>{});
+            else if (phase == STEP) steps(std::integral_constant<int, STEP>{});
+            else if (phase == 2 * STEP) steps(std::integral_constant<int, (2 * STEP) % PD>{});
+            else steps(std::integral_constant<int, (3 * STEP) % PD>{});
+          }
+        }
+        if (++blk == iters) {
+          blk = 0;
+          trip++;
+        }
+      }
+      __syncthreads();  // the panel is complete; the other one has been multiplied
+    }
+  } else {
+    // ---- pointwise wavefronts: panel x filter -> output --------------------------------------
+    float bias_c[NJ];  // pointwise bias of column 32j + l32
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+      bias_c[j] = p.pwb_kind == TFHIP_BCAST_COLUMN ? p.pwb[32 * j + l32]
+                : p.pwb_kind == TFHIP_BCAST_SCALAR ? p.pwb[0] : 0.f;
+    const Clamp pact = clamp_of(p.pw_act);
+    const __amdgpu_buffer_rsrc_t ry = make_rsrc(p.y, p.y_bytes);
+    const unsigned y_row = (unsigned)(p.OW * N * 4);
+    const float* const panel_r = panels + l32 * PITCH + 4 * g;  // where this lane reads its operand
+    __syncthreads();
+
+    int trip = 0, blk = 0;
+    Unit un = unit_of(0);
+    for (int it = 0; it <= total; it++) {
+      if (it > 0) {
+        // the panel filled during the previous step: block `blk` of unit `un`
+        const float* const panel = panel_r + ((it - 1) & 1) * (32 * PITCH);
+        f32x16 acc[NJ];
+        // operands of group q + 1 are read while group q is multiplied; the order is pinned so
+        // that no more than two groups of them are ever live
+        f32x4 a[2], b[2][NJ];
+        auto read_ops = [&](int q, f32x4& ao, f32x4 (&bo)[NJ]) {
+          ao = *reinterpret_cast<const f32x4*>(panel + 8 * q);
+#pragma unroll
+          for (int j = 0; j < NJ; j++)
+            bo[j] = *reinterpret_cast<const f32x4*>(&bl[((q * 2 + g) * N + 32 * j + l32) * 4]);
+        };
+        read_ops(0, a[0], b[0]);
+#pragma unroll
+        for (int q = 0; q < KQ; q++) {
+          if (q + 1 < KQ) read_ops(q + 1, a[(q + 1) & 1], b[(q + 1) & 1]);
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+              // the very first product of a column block starts from the inline zero
+              const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
+                                   0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+              acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q & 1][e], b[q & 1][j][e],
+                                                            q == 0 && e == 0 ? zero : acc[j], 0, 0, 0);
+            }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+
+        // Accumulator register r holds pixel m = 8*(r/4) + 4*(lane/32) + r%4 of the panel,
+        // column l32 of column block j; pixel m is row m / SW, column m % SW of the block.  A
+        // store writes two runs of 32 consecutive floats.
+        const int orow = un.o0 + blk * RB, ocol = un.strip * SW;
+        const unsigned y_blk = (unsigned)((un.n * p.OH + orow) * p.OW + ocol) * (unsigned)(N * 4);
+        const int rows_left = un.rows - blk * RB, cols_left = p.OW - ocol;
+        auto store = [&](auto whole_tag) {
+          constexpr bool whole = decltype(whole_tag)::value;
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int mc = 8 * (r >> 2) + (r & 3);  // + 4 * g
+            int row, col;                            // of the pixel, the lane's part included
+            unsigned at;
+            if (SW >= 8) {
+              row = mc / SW;
+              col = mc % SW + 4 * g;
+              at = y_blk + (unsigned)row * y_row + (unsigned)((mc % SW) * N * 4) +
+                   (unsigned)((4 * g * N + l32) * 4);
+            } else {
+              row = mc / SW + g * (4 / SW);
+              col = mc % SW;
+              at = y_blk + (unsigned)(mc / SW) * y_row + (unsigned)(g * (4 / SW)) * y_row +
+                   (unsigned)((mc % SW) * N * 4) + (unsigned)(l32 * 4);
+            }
+            const bool ok = whole || (row < rows_left && col < cols_left);
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+              const float val = clamp(acc[j][r] + bias_c[j], pact);
+              __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), ry,
+                                                    (int)(ok ? at + (unsigned)(32 * j * 4) : OOB_OFFSET), 0, 0);
+            }
+          }
+        };
+        // (made of the unit's own numbers, so the whole wavefront takes the same branch)
+        if (un.live) {
+          if (rows_left >= RB && cols_left >= SW) store(std::true_type{});
+          else if (rows_left > 0) store(std::false_type{});
+        }
+        if (++blk == iters) {
+          blk = 0;
+          trip++;
+          un = unit_of(trip);
+        }
+      }
+      __syncthreads();  // the next panel is complete; this one may be overwritten
+    }
+  }
+}
+
+template <int KQ, int NJ, int S, int PD, int OCC>
+static int launch_separable(tfhip_ctx* ctx, SepArgs& p) {
+  auto kernel = separable_kernel<KQ, NJ, S, PD, OCC>;
+  constexpr int K = 8 * KQ, N = 32 * NJ;
+  constexpr int SW = 64 / (K / 4) * (S == 1 ? 2 : 1), RB = 32 / SW;
+  const size_t lds = ((size_t)K * N + 8 * 32 * (K + 4)) * sizeof(float);
+  static int per_cu = 0;
+  if (!per_cu) {
+    if (lds > 48 * 1024)
+      (void)hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 512, lds) != hipSuccess || n < 1) {
+      (void)hipGetLastError();
+      n = 1;
+    }
+    per_cu = n;
+  }
+  p.strips = (int)ceil_div(p.OW, SW);
+  // Chunk height: whole panels.  A chunk reads two input rows beyond its own (stride 1), so
+  // chunks are as tall as they can be while every second pair of wavefronts that fits on the
+  // machine still gets a unit.
+  const long long slots = (long long)ctx->num_cus * per_cu * 4;
+  int rh = (int)ceil_div(p.OH, RB) * RB;
+  while (rh > RB && (long long)p.batch * p.strips * ceil_div(p.OH, rh) < slots / 2)
+    rh = (int)ceil_div(ceil_div(rh, 2), RB) * RB;
+  if (const char* e = getenv("TFHIP_SEP_RH")) rh = atoi(e);
+  p.rh = rh;
+  p.chunks = (int)ceil_div(p.OH, rh);
+  p.units = p.batch * p.chunks * p.strips;
+  const long long want = ceil_div(ceil_div(p.units, 8), 4) * 8;
+  const long long resident = (long long)ctx->num_cus * per_cu / 8 * 8;  // a multiple of the XCD count
+  ctx->name_kernel("separable_s%d_k%dxn%d_%s", S, K, N, p.pw_quant ? "u8" : "f32");
+  p.reverse = ctx->take_sweep();
+  tfhip::launch(ctx, kernel, dim3((unsigned)(want < resident || resident < 8 ? want : resident)),
+                dim3(512), lds, p);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace tfhip
+
+using namespace tfhip;
+
+// Ids of the intermediate tensor of the two-kernel form: outside any range a host hands out.
+static int64_t g_scratch_id = INT64_MIN / 2;
+
+extern "C" int tfhip_separable_conv2d(tfhip_ctx* ctx, int64_t x, int64_t dw_filter,
+                                      int64_t pw_filter, int64_t out,
+                                      const tfhip_conv2d_info* dwi, int64_t dw_bias,
+                                      int dw_bias_kind, int dw_act, int64_t pw_bias,
+                                      int pw_bias_kind, int pw_act, const tfhip_qparams* dw_q,
+                                      const tfhip_qparams* pw_q) {
+  if (!ctx || !dwi) return TFHIP_EINVAL;
+  TFHIP_GET(ctx, bx, x);
+  TFHIP_GET(ctx, bdw, dw_filter);
+  TFHIP_GET(ctx, bpw, pw_filter);
+  TFHIP_GET(ctx, bo, out);
+  if (dwi->batch < 0 || dwi->out_h < 0 || dwi->out_w < 0 || dwi->in_c <= 0 || dwi->out_c <= 0 ||
+      dwi->out_c % dwi->in_c != 0)
+    return ctx->fail(TFHIP_EINVAL, "separableConv2d: bad geometry");
+  const int64_t mid_c = dwi->out_c;
+  const int64_t pixels = (int64_t)dwi->batch * dwi->out_h * dwi->out_w;
+  if (bpw->numel % mid_c != 0 || mid_c == 0)
+    return ctx->fail(TFHIP_EINVAL, "separableConv2d: the pointwise filter holds %lld elements, "
+                                   "not a multiple of the %lld depthwise output channels",
+                     (long long)bpw->numel, (long long)mid_c);
+  const int64_t out_c = bpw->numel / mid_c;
+  if (bo->numel != pixels * out_c)
+    return ctx->fail(TFHIP_EINVAL, "separableConv2d: the result holds %lld elements, the geometry "
+                                   "needs %lld", (long long)bo->numel, (long long)(pixels * out_c));
+  for (int act : {dw_act, pw_act})
+    if (act != TFHIP_ACT_LINEAR && act != TFHIP_ACT_RELU && act != TFHIP_ACT_RELU6)
+      return ctx->fail(TFHIP_EINVAL, "separableConv2d: activation %d is not folded here", act);
+  for (int kind : {dw_bias_kind, pw_bias_kind})
+    if (kind != TFHIP_BCAST_NONE && kind != TFHIP_BCAST_SCALAR && kind != TFHIP_BCAST_COLUMN)
+      return ctx->fail(TFHIP_EINVAL, "separableConv2d: bias layout %d is not folded here", kind);
+  if ((bdw->dtype == TFHIP_UINT8Q) != (dw_q != nullptr) || (bpw->dtype == TFHIP_UINT8Q) != (pw_q != nullptr))
+    return ctx->fail(TFHIP_EINVAL, "separableConv2d: qparams must be given exactly for a quantised filter");
+
+  // One kernel when the shapes are the ones it is built for; anything else runs as the two
+  // kernels it stands for, with the intermediate in a pool block.
+  const Buf* bdb = nullptr;
+  const Buf* bpb = nullptr;
+  if (dw_bias_kind != TFHIP_BCAST_NONE && !(bdb = ctx->find(dw_bias))) return TFHIP_ENOENT;
+  if (pw_bias_kind != TFHIP_BCAST_NONE && !(bpb = ctx->find(pw_bias))) return TFHIP_ENOENT;
+  const int K = dwi->in_c, N = (int)out_c, S = dwi->stride_h;
+  const int64_t x_n = (int64_t)dwi->batch * dwi->in_h * dwi->in_w * dwi->in_c;
+  bool one = dwi->filter_h == 3 && dwi->filter_w == 3 && dwi->dilation_h == 1 &&
+             dwi->dilation_w == 1 && dwi->out_c == dwi->in_c && dwi->stride_h == dwi->stride_w &&
+             (S == 1 || S == 2) && dwi->out_w >= 16 && bx->dtype == TFHIP_FLOAT32 &&
+             bo->dtype == TFHIP_FLOAT32 && bx->numel == x_n && bdw->numel == 9 * (int64_t)K &&
+             x_n * 4 < (1ll << 31) && pixels * N * 4 < (1ll << 31) && pixels > 0 &&
+             (!bdb || (bdb->dtype == TFHIP_FLOAT32 &&
+                       bdb->numel == (dw_bias_kind == TFHIP_BCAST_COLUMN ? K : 1))) &&
+             (!bpb || (bpb->dtype == TFHIP_FLOAT32 &&
+                       bpb->numel == (pw_bias_kind == TFHIP_BCAST_COLUMN ? N : 1))) &&
+             (bdw->dtype == TFHIP_FLOAT32 || bdw->dtype == TFHIP_UINT8Q) &&
+             (bpw->dtype == TFHIP_FLOAT32 || bpw->dtype == TFHIP_UINT8Q) && aligned16(bx->ptr) &&
+             aligned16(bo->ptr) &&
+             // enough 32-pixel blocks to give every wavefront of a full machine several
+             pixels >= (int64_t)ctx->num_cus * 8 * 32 * 3;
+  int variant = -1;
+  if (one) {
+    if (K == 32 && N == 64 && S == 1) variant = 0;
+    else if (K == 64 && N == 128 && S == 2) variant = 1;
+  }
+  if (variant >= 0 && !ctx->separable_off) {
+    SepArgs p = {};
+    p.x = static_cast<const float*>(bx->ptr);
+    p.dw = bdw->ptr;
+    p.pw = bpw->ptr;
+    p.y = static_cast<float*>(bo->ptr);
+    p.dwb = bdb ? static_cast<const float*>(bdb->ptr) : nullptr;
+    p.pwb = bpb ? static_cast<const float*>(bpb->ptr) : nullptr;
+    p.batch = dwi->batch;
+    p.H = dwi->in_h;
+    p.W = dwi->in_w;
+    p.OH = dwi->out_h;
+    p.OW = dwi->out_w;
+    p.pt = dwi->pad_top;
+    p.pl = dwi->pad_left;
+    p.dwb_kind = dw_bias_kind;
+    p.pwb_kind = pw_bias_kind;
+    p.dw_act = dw_act;
+    p.pw_act = pw_act;
+    p.dw_quant = dw_q != nullptr;
+    p.pw_quant = pw_q != nullptr;
+    if (dw_q) p.dw_scale = dw_q->scale, p.dw_min = dw_q->min;
+    if (pw_q) p.pw_scale = pw_q->scale, p.pw_min = pw_q->min;
+    p.x_bytes = (unsigned)(x_n * 4);
+    p.y_bytes = (unsigned)(pixels * N * 4);
+    switch (variant) {
+      case 0: {
+        const char* v = getenv("TFHIP_SEP_V");
+        const int vi = v ? atoi(v) : 0;
+        if (vi == 1) return launch_separable<4, 2, 1, 4, 2>(ctx, p);
+        return launch_separable<4, 2, 1, 2, 4>(ctx, p);
+      }
+      case 1: return launch_separable<8, 4, 2, 8, 2>(ctx, p);
+      default: break;
+    }
+  }
+
+  // the two-kernel form
+  const int64_t mid = g_scratch_id++;
+  const int32_t mid_shape[4] = {dwi->batch, dwi->out_h, dwi->out_w, dwi->out_c};
+  int rc = tfhip_register(ctx, mid, mid_shape, 4, TFHIP_FLOAT32);
+  if (rc) return rc;
+  rc = tfhip_depthwise_conv2d(ctx, x, dw_filter, mid, dwi, dw_bias, dw_bias_kind, dw_act, dw_q);
+  if (!rc) {
+    tfhip_conv2d_info pwi = {};
+    pwi.batch = dwi->batch;
+    pwi.in_h = pwi.out_h = dwi->out_h;
+    pwi.in_w = pwi.out_w = dwi->out_w;
+    pwi.in_c = dwi->out_c;
+    pwi.out_c = (int32_t)out_c;
+    pwi.stride_h = pwi.stride_w = pwi.dilation_h = pwi.dilation_w = 1;
+    pwi.filter_h = pwi.filter_w = 1;
+    rc = tfhip_conv2d(ctx, mid, pw_filter, out, &pwi, pw_bias, pw_bias_kind, pw_act, -1,
+                      TFHIP_BCAST_NONE, pw_q);
+  }
+  std::string keep = ctx->err;  // the message of the failing call, not of the clean-up
+  (void)tfhip_dispose(ctx, mid);
+  if (rc) ctx->err = keep;
+  return rc;
+}
+
+// Switches the single-kernel form off (1) or on (0): tests and measurements compare the two
+// forms on the same operands.
+extern "C" int tfhip_separable_single_kernel(tfhip_ctx* ctx, int enable) {
+  if (!ctx) return TFHIP_EINVAL;
+  ctx->separable_off = !enable;
+  return TFHIP_OK;
+}

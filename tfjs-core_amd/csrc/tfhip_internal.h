@@ -69,6 +69,16 @@ struct tfhip_ctx {
     if (ev) free_events.push_back(ev);
   }
   std::unordered_map<void*, hipEvent_t> block_ready;  // pool block -> Buf::ready of its last owner
+  // Blocks whose buffer was disposed while an asynchronous read of it was still copying: they
+  // stay out of the pool until the read's ticket is finished (the copy is complete then), so the
+  // compute stream never waits for the download stream at dispose time.  `done` belongs to the
+  // ticket; `left` is the compute-stream event an upload target leaves behind.
+  struct HeldBlock {
+    void* p;
+    size_t cap;
+    hipEvent_t done, left;
+  };
+  std::vector<HeldBlock> held;
   // Small writes travel through a ring of pinned slots on the compute stream itself.
   static constexpr size_t kSlotBytes = 64 << 10;
   static constexpr int kSlots = 32;
@@ -157,6 +167,7 @@ struct tfhip_ctx {
   // the driver once, at init), and the flag that routes scratch needs there while it runs.
   void* scratch = nullptr;
   bool no_alloc = false;
+  bool separable_off = false;  // tfhip_separable_conv2d always runs its two-kernel form
 
   int fail(int code, const char* fmt, ...);
   // Looks an id up (sets err when missing).  `touch` = the caller queues work on the compute
@@ -166,6 +177,8 @@ struct tfhip_ctx {
   // owner left with it, or nullptr; *recycled whether the block was used before.
   void* alloc(size_t nbytes, size_t* cap, hipEvent_t* ready = nullptr, bool* recycled = nullptr);
   void release(void* p, size_t cap, hipEvent_t ready = nullptr);
+  void park(void* p, size_t cap, hipEvent_t ready);  // release() after the accounting
+  void unhold(hipEvent_t done);                       // held blocks of a finished read -> pool
   void release_buf(tfhip::Buf& b);
   int await_uploads();  // the compute stream waits for every upload still on its way
   void trim();

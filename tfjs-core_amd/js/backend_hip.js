@@ -10,6 +10,7 @@ const path = require('path');
 const util = require('./util');
 const axis_util = require('./axis_util');
 const broadcast_util = require('./broadcast_util');
+const conv_util = require('./conv_util');
 const {DataStorage, KernelBackend} = require('./backend');
 const {Tensor} = require('./tensor');
 const {ENGINE} = require('./engine');
@@ -334,6 +335,36 @@ class MathBackendHIP extends KernelBackend {
     this.napi.depthwiseConv2d(this.ctx, this.h(x), this.h(filter), this.h(out),
                               convInfoArray(convInfo), bk ? this.h(bias) : -1, bk,
                               ACT[activation || 'linear'], this.q(filter));
+    return out;
+  }
+
+  // Extension of the plug-in API (feature-detected by the op wrapper): depthwiseConv2D -> add ->
+  // relu | clip -> conv2d (1x1) -> add -> relu | clip as one call, the block of
+  // depthwise-separable networks (the reference composes it at op level, ops/conv.ts:588-660).
+  // convInfo is that of the depthwise half.  A bias or activation of a kind the kernels do not
+  // fold makes this the two calls.
+  fusedSeparableConv2d(x, depthwiseFilter, pointwiseFilter, convInfo, depthwiseBias,
+                       depthwiseActivation, bias, activation) {
+    const foldable = a => a == null || a === 'linear' || a === 'relu' || a === 'relu6';
+    const midShape = convInfo.outShape;
+    const outShape = midShape.slice(0, 3).concat([pointwiseFilter.shape[3]]);
+    const dk = this.epilogueKind(depthwiseBias, midShape);
+    const pk = this.epilogueKind(bias, outShape);
+    if (dk == null || dk === BCAST.FULL || pk == null || pk === BCAST.FULL ||
+        !foldable(depthwiseActivation) || !foldable(activation)) {
+      const mid = this.fusedDepthwiseConv2D(x, depthwiseFilter, convInfo, depthwiseBias,
+                                            depthwiseActivation);
+      const pwInfo = conv_util.computeConv2DInfo(midShape, pointwiseFilter.shape, 1, 1, 'valid');
+      const r = this.fusedConv2d(mid, pointwiseFilter, pwInfo, bias, activation);
+      mid.dispose();
+      return r;
+    }
+    const out = this.out(outShape);
+    this.napi.separableConv2d(
+        this.ctx, this.h(x), this.h(depthwiseFilter), this.h(pointwiseFilter), this.h(out),
+        convInfoArray(convInfo), dk ? this.h(depthwiseBias) : -1, dk,
+        ACT[depthwiseActivation || 'linear'], pk ? this.h(bias) : -1, pk,
+        ACT[activation || 'linear'], this.q(depthwiseFilter), this.q(pointwiseFilter));
     return out;
   }
 

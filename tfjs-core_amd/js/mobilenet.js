@@ -32,10 +32,10 @@ function forward(tf, w, x) {
                              activation: 'relu6'});
     BLOCKS.forEach((b, i) => {
       const n = i + 1;
-      h = tf.fused.depthwiseConv2d({x: h, filter: w[`dw${n}_w`], strides: b[1], pad: 'same',
-                                    bias: w[`dw${n}_b`], activation: 'relu6'});
-      h = tf.fused.conv2d({x: h, filter: w[`pw${n}_w`], strides: 1, pad: 'same',
-                           bias: w[`pw${n}_b`], activation: 'relu6'});
+      h = tf.fused.separableConv2d({x: h, depthwiseFilter: w[`dw${n}_w`],
+                                    pointwiseFilter: w[`pw${n}_w`], strides: b[1], pad: 'same',
+                                    depthwiseBias: w[`dw${n}_b`], depthwiseActivation: 'relu6',
+                                    bias: w[`pw${n}_b`], activation: 'relu6'});
     });
     h = tf.avgPool(h, [h.shape[1], h.shape[2]], 1, 'valid');
     h = tf.reshape(h, [h.shape[0], h.shape[3]]);

@@ -333,6 +333,47 @@ const depthwiseConv2d = op('depthwiseConv2d', (x, filter, strides, pad, dataForm
 // depthwiseConv2d + add(bias) + relu | clip(0,6).  The plug-in API of the reference has no
 // fused depthwise kernel, so the backend method is feature-detected: backends without it
 // (backend_cpu) run the three reference calls.
+// separableConv2d (ops/conv.ts:588-660: depthwiseConv2d, then a 1x1 conv2d with stride 1 and
+// 'valid' padding) with the add(bias) + relu | clip(0,6) that a folded batch norm leaves after
+// each half: {x, depthwiseFilter, pointwiseFilter, strides, pad, dilations, depthwiseBias,
+// depthwiseActivation, bias, activation}.  One backend call where the backend has the method
+// (feature detection) and folds these biases; otherwise the two fused ops in sequence.
+const fusedSeparableConv2d = op('fusedSeparableConv2d', (config) => {
+  const {$x, x4D, $filter, convInfo, reshapedTo4D} = convPrep(
+      config.x, config.depthwiseFilter, config.strides, config.pad, config.dataFormat,
+      config.dilations, null, 'separableConv2d', true);
+  const $pointwise = convertToTensor(config.pointwiseFilter, 'pointwiseFilter', 'separableConv2d');
+  util.assert($pointwise.rank === 4 && $pointwise.shape[0] === 1 && $pointwise.shape[1] === 1,
+              () => 'Error in separableConv2d: the first two dimensions of pointwise filter ' +
+                  `must be 1, but got ${$pointwise.shape.slice(0, 2)}.`);
+  util.assert($pointwise.shape[2] === convInfo.outChannels,
+              () => 'Error in separableConv2d: the third dimension of pointwise filter must be ' +
+                  `${convInfo.outChannels}, but got ${$pointwise.shape[2]}.`);
+  const conv = b => {
+    if (b == null) return null;
+    let $b = convertToTensor(b, 'bias', 'separableConv2d');
+    [$b] = makeTypesMatch($b, $x);
+    return $b;
+  };
+  const $dBias = conv(config.depthwiseBias), $bias = conv(config.bias);
+  const dAct = config.depthwiseActivation || 'linear', act = config.activation || 'linear';
+  let res;
+  if (typeof ENGINE.backend.fusedSeparableConv2d === 'function' && !ENGINE.isTapeOn()) {
+    res = ENGINE.runKernel(
+        backend => backend.fusedSeparableConv2d(x4D, $filter, $pointwise, convInfo, $dBias, dAct,
+                                                $bias, act),
+        {x: x4D, $filter, $pointwise});
+  } else {
+    // (also while a tape records: the two ops carry the gradient functions)
+    const mid = fusedDepthwiseConv2d({x: x4D, filter: $filter, strides: config.strides,
+                                      pad: config.pad, dataFormat: config.dataFormat,
+                                      dilations: config.dilations, bias: $dBias, activation: dAct});
+    res = fusedConv2d({x: mid, filter: $pointwise, strides: 1, pad: 'valid', bias: $bias,
+                       activation: act});
+  }
+  return lower(res, reshapedTo4D);
+});
+
 const fusedDepthwiseConv2d = op('fusedDepthwiseConv2d', (config) => {
   const activation = config.activation || 'linear';
   const {$x, x4D, $filter, convInfo, reshapedTo4D} = convPrep(
@@ -1585,7 +1626,8 @@ const logSoftmax = op('logSoftmax', (logits, axis) => {
 module.exports = {
   op, tensor, scalar, tensor1d, tensor2d, tensor3d, tensor4d, quantizedTensor, convertToTensor,
   fill, zeros, ones, zerosLike, onesLike, reshape, cast, clone, dequantize, matMul,
-  fused: {matMul: fusedMatMul, conv2d: fusedConv2d, depthwiseConv2d: fusedDepthwiseConv2d},
+  fused: {matMul: fusedMatMul, conv2d: fusedConv2d, depthwiseConv2d: fusedDepthwiseConv2d,
+          separableConv2d: fusedSeparableConv2d},
   conv2d, depthwiseConv2d, separableConv2d, avgPool, maxPool, pool, add, sub, mul, div, maximum,
   minimum, prelu, relu, relu6, exp, log, neg, abs, sigmoid, sqrt, square, tanh, rsqrt,
   clipByValue, sum, max, min, argMax, argMin, logSumExp, softmax, gather, transpose,

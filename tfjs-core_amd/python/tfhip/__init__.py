@@ -15,6 +15,7 @@ class _Fused(object):
     matmul = staticmethod(_ops.fused_matmul)
     conv2d = staticmethod(_ops.fused_conv2d)
     depthwise_conv2d = staticmethod(_ops.fused_depthwise_conv2d)
+    separable_conv2d = staticmethod(_ops.fused_separable_conv2d)
 
 
 fused = _Fused()

@@ -63,6 +63,9 @@ _SIGNATURES = {
                              _INT, _I64, _INT, C.POINTER(QParams)],
     "tfhip_conv2d": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC), _I64, _INT, _INT, _I64, _INT,
                      C.POINTER(QParams)],
+    "tfhip_separable_conv2d": [_PTR, _I64, _I64, _I64, _I64, C.POINTER(Conv2DInfoC), _I64, _INT, _INT,
+                               _I64, _INT, _INT, C.POINTER(QParams), C.POINTER(QParams)],
+    "tfhip_separable_single_kernel": [_PTR, _INT],
     "tfhip_depthwise_conv2d": [_PTR, _I64, _I64, _I64, C.POINTER(Conv2DInfoC), _I64, _INT, _INT,
                                C.POINTER(QParams)],
     "tfhip_pool2d": [_PTR, _I64, _I64, C.POINTER(Conv2DInfoC), _INT],

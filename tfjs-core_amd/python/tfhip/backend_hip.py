@@ -367,6 +367,31 @@ class MathBackendHIP(object):
             self._h(bias) if bk else -1, bk, capi.ACT[activation], self._q(filter)))
         return out
 
+    def fused_separable_conv2d(self, x, depthwise_filter, pointwise_filter, conv_info,
+                               depthwise_bias=None, depthwise_activation=None, bias=None,
+                               activation=None):
+        """Extension of the plug-in API: depthwiseConv2D -> add -> relu|clip -> conv2d (1x1) ->
+        add -> relu|clip as one call (the block of depthwise-separable networks; the reference
+        composes it at op level, ops/conv.ts:588-660).  conv_info is that of the depthwise half.
+        Returns None when the biases / activations are not the foldable kinds, and the op
+        wrapper then issues the separate calls."""
+        acts = (None, "linear", "relu", "relu6")
+        mid_shape = conv_info["outShape"]
+        out_shape = tuple(mid_shape[:3]) + (pointwise_filter.shape[3],)
+        dk = self._epilogue_kind(depthwise_bias, mid_shape)
+        pk = self._epilogue_kind(bias, out_shape)
+        if dk in (None, capi.BCAST_FULL) or pk in (None, capi.BCAST_FULL) or \
+                depthwise_activation not in acts or activation not in acts:
+            return None
+        out = self._out(out_shape)
+        info = _info_c(conv_info)
+        self._ck(self.lib.tfhip_separable_conv2d(
+            self.ctx, self._h(x), self._h(depthwise_filter), self._h(pointwise_filter),
+            self._h(out), C.byref(info), self._h(depthwise_bias) if dk else -1, dk,
+            capi.ACT[depthwise_activation], self._h(bias) if pk else -1, pk, capi.ACT[activation],
+            self._q(depthwise_filter), self._q(pointwise_filter)))
+        return out
+
     def _pool(self, x, conv_info, kind):
         out = self._out(conv_info["outShape"])
         info = _info_c(conv_info)

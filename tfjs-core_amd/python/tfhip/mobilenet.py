@@ -23,11 +23,13 @@ def layer_table(batch=1, size=224):
     cin = 32
     for i, (cout, s) in enumerate(BLOCKS, 1):
         ho = h // s
+        # out_bytes / in_bytes: the activation between the two halves of the block, which a
+        # single-kernel block never writes or reads
         rows.append(dict(name="dw%d" % i, kind="depthwise", C=cin, H=h, HO=ho, stride=s,
-                         macs=batch * ho * ho * cin * 9,
+                         macs=batch * ho * ho * cin * 9, out_bytes=4 * batch * ho * ho * cin,
                          bytes=4 * (batch * h * h * cin + batch * ho * ho * cin + 9 * cin + cin)))
         rows.append(dict(name="pw%d" % i, kind="conv", M=batch * ho * ho, K=cin, N=cout,
-                         macs=batch * ho * ho * cin * cout,
+                         macs=batch * ho * ho * cin * cout, in_bytes=4 * batch * ho * ho * cin,
                          bytes=4 * (batch * ho * ho * (cin + cout) + cin * cout + cout)))
         cin, h = cout, ho
     rows.append(dict(name="avgpool", kind="pool", macs=0,
@@ -89,10 +91,10 @@ def forward(tf, w, x):
     def run():
         h = tf.fused.conv2d(x, w["stem_w"], 2, "same", bias=w["stem_b"], activation="relu6")
         for i, (_, s) in enumerate(BLOCKS, 1):
-            h = tf.fused.depthwise_conv2d(h, w["dw%d_w" % i], s, "same", bias=w["dw%d_b" % i],
+            h = tf.fused.separable_conv2d(h, w["dw%d_w" % i], w["pw%d_w" % i], s, "same",
+                                          depthwise_bias=w["dw%d_b" % i],
+                                          depthwise_activation="relu6", bias=w["pw%d_b" % i],
                                           activation="relu6")
-            h = tf.fused.conv2d(h, w["pw%d_w" % i], 1, "same", bias=w["pw%d_b" % i],
-                                activation="relu6")
         h = tf.avg_pool(h, (h.shape[1], h.shape[2]), 1, "valid")
         h = tf.reshape(h, (h.shape[0], h.shape[3]))
         logits = tf.fused.matmul(h, w["fc_w"], False, False, bias=w["fc_b"], activation="linear")

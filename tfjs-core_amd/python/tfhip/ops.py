@@ -212,6 +212,40 @@ def fused_depthwise_conv2d(x, filt, strides, pad, data_format="NHWC", dilations=
     return ENGINE.tidy(run)
 
 
+def fused_separable_conv2d(x, depthwise_filter, pointwise_filter, strides, pad,
+                           dilations=(1, 1), data_format="NHWC", depthwise_bias=None,
+                           depthwise_activation="linear", bias=None, activation="linear"):
+    """separableConv2d (ops/conv.ts:588-660: depthwiseConv2d, then a 1x1 conv2d with stride 1
+    and 'valid' padding) with the add(bias) + relu|clip(0,6) that a folded batch norm leaves
+    after each half.  One backend call where the backend has it (feature detection); otherwise,
+    and for bias shapes it does not fold, the two fused ops in sequence."""
+    def run():
+        x4, f, ci, lifted = _conv_prep(x, depthwise_filter, strides, pad, data_format, dilations,
+                                       None, "separableConv2d", True)
+        pf = _conv(pointwise_filter, "pointwiseFilter", "separableConv2d")
+        if pf.rank != 4 or pf.shape[0] != 1 or pf.shape[1] != 1:
+            raise ValueError("Error in separableConv2d: the first two dimensions of pointwise "
+                             "filter must be 1, but got %s." % (tuple(pf.shape),))
+        if pf.shape[2] != ci["outChannels"]:
+            raise ValueError("Error in separableConv2d: the third dimension of pointwise filter "
+                             "must be %d, but got %d." % (ci["outChannels"], pf.shape[2]))
+
+        def fwd(be):
+            if hasattr(be, "fused_separable_conv2d"):
+                r = be.fused_separable_conv2d(x4, f, pf, ci, depthwise_bias, depthwise_activation,
+                                              bias, activation)
+                if r is not None:
+                    return r
+            return None
+        r = ENGINE.run_kernel(fwd)
+        if r is None:
+            mid = fused_depthwise_conv2d(x4, f, strides, pad, data_format, dilations, None,
+                                         depthwise_bias, depthwise_activation)
+            r = fused_conv2d(mid, pf, 1, "valid", data_format, 1, None, bias, activation)
+        return _lower(r, lifted)
+    return ENGINE.tidy(run)
+
+
 # ---- pooling (ops/pool.ts:56-203, 266-340) ----
 def _pool_impl(x, filter_size, strides, dilations, pad, rounding, kind):
     def run():
