@@ -648,6 +648,38 @@ def test_js_gradients_through_the_tape(tmp_path, ref):
         c.add("depthwise_" + tag, "gradDepthwise", dict(x=images, filter=filt),
               dict(strides=1, pad="same", wrt=wrt, squared=sq),
               flat(g(title)[0]).reshape(images.shape if wrt == 0 else filt.shape), atol=1e-3)
+    # the fused forms carry the same gradients: depthwise -> add(bias) -> relu | clip(0, 6), chained
+    # by hand from the oracle's backward kernels; then the separable pair on top of them
+    rng2 = np.random.default_rng(54)
+    f2 = lambda *s: rng2.uniform(-1, 1, s).astype(np.float32)
+    xs, fs = f2(2, 6, 6, 4), f2(3, 3, 4, 1) * 0.5
+    bs, dys = f2(4) * 0.3, f2(2, 3, 3, 4)
+    for act, hi in (("relu", np.inf), ("relu6", 6.0), ("linear", None)):
+        pre = ref.depthwise_conv2d(xs * 4, fs * 4, 2, "same") + bs
+        mask = np.ones_like(pre) if hi is None else ((pre > 0) & (pre < hi)).astype(np.float32)
+        dpre = dys * mask
+        wants = (ref.depthwise_der_input(xs.shape, dpre, fs * 4, 2, "same"),
+                 ref.depthwise_der_filter(xs * 4, dpre, fs.shape, 2, "same"),
+                 dpre.astype(np.float64).sum((0, 1, 2)).astype(np.float32))
+        for k, tag in enumerate(("dx", "dw", "db")):
+            c.add("fused_dw_%s_%s" % (act, tag), "gradFusedDepthwise",
+                  dict(x=xs * 4, filter=fs * 4, bias=bs, dy=dys),
+                  dict(strides=2, pad="same", activation=act, wrt=k), wants[k], rtol=1e-3, atol=1e-4)
+    pws, pbs, dy2 = f2(1, 1, 4, 6) * 0.5, f2(6) * 0.2, f2(2, 3, 3, 6)
+    pre = ref.depthwise_conv2d(xs, fs, 2, "same") + bs
+    mid = np.maximum(pre, 0)
+    out = ref.conv2d(mid, pws, 1, "valid") + pbs
+    dout = dy2 * (out > 0)
+    dmid = ref.conv2d_der_input(mid.shape, dout, pws, 1, "valid") * (pre > 0)
+    wants = (ref.depthwise_der_input(xs.shape, dmid, fs, 2, "same"),
+             ref.depthwise_der_filter(xs, dmid, fs.shape, 2, "same"),
+             ref.conv2d_der_filter(mid, dout, pws.shape, 1, "valid"),
+             dmid.astype(np.float64).sum((0, 1, 2)).astype(np.float32),
+             dout.astype(np.float64).sum((0, 1, 2)).astype(np.float32))
+    for k, tag in enumerate(("dx", "dw", "dpw", "db", "dpb")):
+        c.add("fused_sep_" + tag, "gradFusedSeparable",
+              dict(x=xs, filter=fs, pw=pws, bias=bs, pbias=pbs, dy=dy2),
+              dict(strides=2, pad="same", activation="relu", wrt=k), wants[k], rtol=1e-3, atol=1e-4)
     # ops/pool_test.ts
     a = _golden("pool_grad", "gradient x=[5,5,1] f=[3,3] s=2 duplicate max value", "maxPoolBackprop")["arrays"]
     c.add("maxpool_dup", "gradPool", dict(x=flat(a[2]).reshape(a[3]), dy=flat(a[0]).reshape(a[1])),

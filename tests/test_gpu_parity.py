@@ -532,6 +532,53 @@ def test_reductions(hip, ref, rows, cols):
     close(hip.softmax(x), ref.softmax(x), rtol=1e-4, atol=1e-7)
 
 
+def test_reductions_of_few_long_rows_are_cut_into_pieces(hip, ref):
+    """A whole tensor reduced to a scalar (outer = 1), or a handful of long rows: the rows are cut
+    into pieces over the machine and combined by a second launch, with the results (NaN rule, first
+    index of ties, double sums) of the one-wavefront-per-row pass, and at a streaming rate."""
+    tf = hip.tf
+    rng = np.random.default_rng(77)
+    for rows, cols in ((1, 3_000_001), (3, 70_001), (1, 16384), (2, 1_000_000)):
+        x = rng.standard_normal((rows, cols)).astype(np.float32)
+        x[0, [5, cols // 2, cols - 1]] = 9.5           # the maximum three times: first index wins
+        x[-1, [cols - 7, 11]] = -9.5
+        close(hip.sum(x), ref.sum(x), rtol=1e-6, atol=1e-6)
+        assert np.array_equal(hip.max(x), ref.max(x)) and np.array_equal(hip.min(x), ref.min(x))
+        a = hip.argmax(x)
+        assert a.dtype == np.int32 and np.array_equal(a, ref.argmax(x)) and a[0] == 5
+        assert np.array_equal(hip.argmin(x), ref.argmin(x))
+        with tf.tidy():
+            t = tf.tensor(x)
+            info = tf.time(lambda: tf.sum(t, -1))
+            assert [k[0] for k in info["kernelTimes"]] == ["reduce_parts", "reduce_finish"]
+            assert np.array_equal(tf.any(tf.greater(t, tf.tensor(np.float32(9.0))), -1).data_sync(),
+                                  (x > 9).any(-1))
+            assert np.array_equal(tf.all(tf.greater(t, tf.tensor(np.float32(-9.0))), -1).data_sync(),
+                                  (x > -9).all(-1))
+    # NaN: kept from slot 0 only, as in the reference's loop (backend_cpu.ts:658-712)
+    x = rng.standard_normal((2, 200_000)).astype(np.float32)
+    x[0, 0] = np.nan
+    x[1, 150_000] = np.nan
+    assert np.array_equal(hip.max(x), ref.max(x), equal_nan=True)
+    assert np.array_equal(hip.argmax(x), ref.argmax(x)) and np.array_equal(hip.argmin(x), ref.argmin(x))
+    # int32 sums stay exact, products of long rows keep their sign and magnitude
+    xi = rng.integers(-1000, 1000, (1, 1_000_003)).astype(np.int32)
+    p = np.where(rng.random((2, 100_000)) < 0.0005, -1.0001, 1.0).astype(np.float32)
+    with tf.tidy():
+        r = tf.sum(tf.tensor(xi))
+        assert r.dtype == "int32" and int(r.data_sync()) == int(xi.sum())
+        close(tf.prod(tf.tensor(p), -1).data_sync(), np.prod(p.astype(np.float64), -1), rtol=1e-5)
+    # rate: 51.4 M floats (205 MB) summed to one value; one wavefront alone would need ~100 ms
+    with tf.tidy():
+        big = tf.tensor(np.ones((64, 112, 112, 64), np.float32))
+        tf.sum(big).dispose()
+        info = tf.time(lambda: [tf.sum(big) for _ in range(5)])
+        ms = info["kernelMs"] / 5
+        assert float(tf.sum(big).data_sync()) == 64 * 112 * 112 * 64
+        print("sum of 205 MB: %.1f us (%.0f GB/s)" % (ms * 1e3, 205.5e6 / ms * 1e-6), flush=True)
+        assert ms < 0.5
+
+
 def test_argmax_ties_nan_and_windows(hip, ref):
     x = np.zeros((6, 200), np.float32)
     x[0, [5, 70, 130]] = 1          # tie across lanes: first index wins

@@ -9,6 +9,8 @@
 
 namespace tfhip {
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 __device__ __forceinline__ float ld(const void* p, int dt, int64_t i) {
   switch (dt) {
     case TFHIP_FLOAT32: return static_cast<const float*>(p)[i];
@@ -66,6 +68,190 @@ __global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void reduce_rows_kernel(
     if (want_max ? v > best : v < best) {
       best = v;
       idx = j;
+    }
+  }
+  for (int off = WAVE / 2; off > 0; off >>= 1) {
+    const float ob = __shfl_down(best, off, WAVE);
+    const int64_t oi = __shfl_down(idx, off, WAVE);
+    const bool better = want_max ? ob > best : ob < best;
+    if (better || (ob == best && oi < idx)) {
+      best = ob;
+      idx = oi;
+    }
+  }
+  if (lane == 0) {
+    if (op == TFHIP_ARGMAX || op == TFHIP_ARGMIN) out[row] = (OutT)idx;
+    else if (std::is_same<OutT, float>::value) out[row] = (OutT)best;
+    else out[row] = (OutT)(int32_t)best;
+  }
+}
+
+// Few rows, long rows (a whole tensor summed to a scalar, a global norm, a loss): one wavefront
+// per row would leave the machine idle, so every row is cut into `parts` contiguous pieces.  A
+// wavefront reduces one piece exactly as reduce_rows_kernel reduces a row and leaves a partial
+// result: the running sum / product (double), the any/all flag, or the extremum with the index
+// of its first occurrence.  Every piece of a row starts its extremum from the row's element 0,
+// as the single pass does, so NaN survives only from slot 0 here too.
+__global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void reduce_parts_kernel(
+    int op, const void* x, int x_dt, double* pval, long long* pidx, int64_t outer, int64_t inner,
+    int parts, int64_t seg, int vec) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int64_t piece = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+  if (piece >= outer * parts) return;
+  const int64_t row = piece / parts;
+  const int part = (int)(piece - row * parts);
+  const int64_t base = row * inner;
+  const int64_t j0 = part * seg, j1 = min(inner, j0 + seg);
+  // four independent loads per lane and trip keep enough bytes in flight for the HBM rate
+  constexpr int U = 4;
+  if (op == TFHIP_SUM || op == TFHIP_PROD) {
+    const bool sum = op == TFHIP_SUM;
+    double s[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) s[u] = sum ? 0.0 : 1.0;
+    int64_t j = j0 + lane;
+    if (vec) {
+      // float32 rows whose pieces start on 16-byte boundaries: 16 bytes per lane and load
+      const f32x4* xv = reinterpret_cast<const f32x4*>(static_cast<const float*>(x) + base);
+      int64_t q = j0 / 4 + lane;
+      const int64_t q1 = j1 / 4;
+      for (; q + (U - 1) * WAVE < q1; q += U * WAVE) {
+        f32x4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = xv[q + u * WAVE];
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) s[u] = sum ? s[u] + (double)v[u][e] : s[u] * (double)v[u][e];
+      }
+      for (; q < q1; q += WAVE) {
+        const f32x4 v = xv[q];
+#pragma unroll
+        for (int e = 0; e < 4; e++) s[0] = sum ? s[0] + (double)v[e] : s[0] * (double)v[e];
+      }
+      j = q1 * 4 + lane;  // what is left of a row whose length is no multiple of 4
+    }
+    for (; j + (U - 1) * WAVE < j1; j += U * WAVE) {
+      float v[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) v[u] = ld(x, x_dt, base + j + u * WAVE);
+#pragma unroll
+      for (int u = 0; u < U; u++) s[u] = sum ? s[u] + (double)v[u] : s[u] * (double)v[u];
+    }
+    for (; j < j1; j += WAVE) s[0] = sum ? s[0] + (double)ld(x, x_dt, base + j) : s[0] * (double)ld(x, x_dt, base + j);
+    double t = sum ? (s[0] + s[1]) + (s[2] + s[3]) : (s[0] * s[1]) * (s[2] * s[3]);
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const double o = __shfl_down(t, off, WAVE);
+      t = sum ? t + o : t * o;
+    }
+    if (lane == 0) pval[piece] = t;
+    return;
+  }
+  if (op == TFHIP_ALL || op == TFHIP_ANY) {
+    int hit = 0;  // any: a non-zero element; all: a zero element
+    for (int64_t j = j0 + lane; j < j1; j += WAVE) hit |= (ld(x, x_dt, base + j) != 0.f) == (op == TFHIP_ANY);
+    for (int off = WAVE / 2; off > 0; off >>= 1) hit |= __shfl_down(hit, off, WAVE);
+    if (lane == 0) pval[piece] = (double)hit;
+    return;
+  }
+  const bool want_max = op == TFHIP_MAX || op == TFHIP_ARGMAX;
+  float best = ld(x, x_dt, base);
+  int64_t idx = 0;
+  int64_t j = j0 + lane;
+  if (vec) {
+    const f32x4* xv = reinterpret_cast<const f32x4*>(static_cast<const float*>(x) + base);
+    int64_t q = j0 / 4 + lane;
+    const int64_t q1 = j1 / 4;
+    for (; q < q1; q += U * WAVE) {
+      f32x4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) v[u] = q + u * WAVE < q1 ? xv[q + u * WAVE] : f32x4{best, best, best, best};
+      // in ascending index order within the lane, so that of equal values the first is kept
+#pragma unroll
+      for (int u = 0; u < U; u++)
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (want_max ? v[u][e] > best : v[u][e] < best) {
+            best = v[u][e];
+            idx = 4 * (q + u * WAVE) + e;
+          }
+    }
+    j = q1 * 4 + lane;
+  }
+  for (; j + (U - 1) * WAVE < j1; j += U * WAVE) {
+    float v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = ld(x, x_dt, base + j + u * WAVE);
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (want_max ? v[u] > best : v[u] < best) {
+        best = v[u];
+        idx = j + u * WAVE;
+      }
+  }
+  for (; j < j1; j += WAVE) {
+    const float v = ld(x, x_dt, base + j);
+    if (want_max ? v > best : v < best) {
+      best = v;
+      idx = j;
+    }
+  }
+  for (int off = WAVE / 2; off > 0; off >>= 1) {
+    const float ob = __shfl_down(best, off, WAVE);
+    const int64_t oi = __shfl_down(idx, off, WAVE);
+    const bool better = want_max ? ob > best : ob < best;
+    if (better || (ob == best && oi < idx)) {
+      best = ob;
+      idx = oi;
+    }
+  }
+  if (lane == 0) {
+    pval[piece] = (double)best;
+    pidx[piece] = idx;
+  }
+}
+
+// Combines the partial results of every row, one wavefront per row, with the same rules (sums
+// in double; a later piece wins an extremum only when strictly better, equal values keep the
+// lower index), so the result does not depend on how the row was cut.
+template <typename OutT>
+__global__ __launch_bounds__(WAVE* ROWS_PER_BLOCK) void reduce_finish_kernel(
+    int op, const double* pval, const long long* pidx, OutT* out, int64_t outer, int parts) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
+  if (row >= outer) return;
+  const double* pv = pval + row * parts;
+  if (op == TFHIP_SUM || op == TFHIP_PROD) {
+    const bool sum = op == TFHIP_SUM;
+    double s = sum ? 0.0 : 1.0;
+    for (int k = lane; k < parts; k += WAVE) s = sum ? s + pv[k] : s * pv[k];
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+      const double o = __shfl_down(s, off, WAVE);
+      s = sum ? s + o : s * o;
+    }
+    if (lane == 0) {
+      if (std::is_same<OutT, float>::value) out[row] = (OutT)(float)s;
+      else out[row] = (OutT)(int32_t)(uint32_t)(int64_t)s;
+    }
+    return;
+  }
+  if (op == TFHIP_ALL || op == TFHIP_ANY) {
+    int hit = 0;
+    for (int k = lane; k < parts; k += WAVE) hit |= pv[k] != 0.0;
+    for (int off = WAVE / 2; off > 0; off >>= 1) hit |= __shfl_down(hit, off, WAVE);
+    if (lane == 0) out[row] = (OutT)(op == TFHIP_ANY ? hit : !hit);
+    return;
+  }
+  const bool want_max = op == TFHIP_MAX || op == TFHIP_ARGMAX;
+  const long long* pi = pidx + row * parts;
+  float best = (float)pv[0];
+  int64_t idx = pi[0];
+  for (int k = lane; k < parts; k += WAVE) {
+    const float v = (float)pv[k];
+    const int64_t vi = pi[k];
+    if ((want_max ? v > best : v < best) || (v == best && vi < idx)) {
+      best = v;
+      idx = vi;
     }
   }
   for (int off = WAVE / 2; off > 0; off >>= 1) {
@@ -294,7 +480,43 @@ extern "C" int tfhip_reduce(tfhip_ctx* ctx, int op, int64_t x, int64_t out, int6
     return tfhip_fill(ctx, out, 0.0);
   }
   if (ceil_div(outer, ROWS_PER_BLOCK) > 0x7fffffffLL) return ctx->fail(TFHIP_ENOTSUP, "reduce: too many rows");
-  const dim3 grid((unsigned)ceil_div(outer, ROWS_PER_BLOCK)), block(WAVE * ROWS_PER_BLOCK);
+  const dim3 block(WAVE * ROWS_PER_BLOCK);
+  // Fewer rows than the machine has room for wavefronts, and rows long enough to be worth a
+  // second launch: cut every row into pieces, reduce the pieces, then combine them.
+  const int64_t room = (int64_t)ctx->num_cus * 16;
+  if (outer * 2 <= room && inner >= 16384 && !ctx->no_alloc) {
+    const int64_t min_piece = 4096;
+    int64_t parts = std::min<int64_t>(ceil_div(room, outer), ceil_div(inner, min_piece));
+    parts = std::min<int64_t>(parts, 4096);
+    const int64_t seg = ceil_div(ceil_div(inner, parts), WAVE) * WAVE;  // whole trips of a wavefront
+    parts = ceil_div(inner, seg);
+    if (parts > 1) {
+      const int64_t pieces = outer * parts;
+      Temp partial(ctx);
+      if (!partial.get((size_t)pieces * 16)) return TFHIP_EDEVICE;
+      // 16-byte loads: float32, every row and (seg is a multiple of 64) every piece 16-byte aligned
+      const int vec = bx->dtype == TFHIP_FLOAT32 && inner % 4 == 0 &&
+                      (reinterpret_cast<uintptr_t>(bx->ptr) & 15) == 0;
+      double* pval = static_cast<double*>(partial.ptr);
+      long long* pidx = reinterpret_cast<long long*>(pval + pieces);
+      tfhip::launch(ctx, reduce_parts_kernel, dim3((unsigned)ceil_div(pieces, ROWS_PER_BLOCK)), block, 0,
+                    op, bx->ptr, bx->dtype, pval, pidx, outer, inner, (int)parts, seg, vec);
+      TFHIP_LAUNCH_CHECK_NAMED(ctx, "reduce_parts");
+      const dim3 fgrid((unsigned)ceil_div(outer, ROWS_PER_BLOCK));
+      if (bo->dtype == TFHIP_FLOAT32)
+        tfhip::launch(ctx, reduce_finish_kernel<float>, fgrid, block, 0, op, pval, pidx,
+                      (float*)bo->ptr, outer, (int)parts);
+      else if (bo->dtype == TFHIP_BOOL)
+        tfhip::launch(ctx, reduce_finish_kernel<uint8_t>, fgrid, block, 0, op, pval, pidx,
+                      (uint8_t*)bo->ptr, outer, (int)parts);
+      else
+        tfhip::launch(ctx, reduce_finish_kernel<int32_t>, fgrid, block, 0, op, pval, pidx,
+                      (int32_t*)bo->ptr, outer, (int)parts);
+      TFHIP_LAUNCH_CHECK_NAMED(ctx, "reduce_finish");
+      return TFHIP_OK;
+    }
+  }
+  const dim3 grid((unsigned)ceil_div(outer, ROWS_PER_BLOCK));
   if (bo->dtype == TFHIP_FLOAT32)
     tfhip::launch(ctx, reduce_rows_kernel<float>, grid, block, 0, op, bx->ptr,
                        bx->dtype, (float*)bo->ptr, outer, inner);

@@ -94,6 +94,12 @@ function stepOf(x) {
 function fusedDyActivation(dy, y, activation) {
   if (activation == null || activation === 'linear') return dy;
   if (activation === 'relu') return mul(dy, stepOf(y));
+  if (activation === 'relu6') {
+    // clipByValue passes the gradient where its input lies inside [0, 6] (unary_ops.ts:548-555);
+    // from the clipped value that is 0 < y < 6 (the two boundary points aside)
+    const six = fill([], 6, y.dtype);
+    return mul(dy, cast(logicalAnd(greater(y, zeros([], y.dtype)), less(y, six)), 'float32'));
+  }
   throw new Error(`Gradient for activation ${activation} has not been implemented yet.`);
 }
 
@@ -385,17 +391,37 @@ const fusedDepthwiseConv2d = op('fusedDepthwiseConv2d', (config) => {
     [$bias] = makeTypesMatch($bias, $x);
     broadcast_util.assertAndGetBroadcastShape(convInfo.outShape, $bias.shape);
   }
-  const res = ENGINE.runKernel(backend => {
+  const inputs = {x: x4D, $filter};
+  if ($bias != null) inputs.$bias = $bias;
+  const res = ENGINE.runKernel((backend, save) => {
+    let r;
     if (typeof backend.fusedDepthwiseConv2D === 'function') {
-      return backend.fusedDepthwiseConv2D(x4D, $filter, convInfo, $bias, activation);
+      r = backend.fusedDepthwiseConv2D(x4D, $filter, convInfo, $bias, activation);
+    } else {
+      r = backend.depthwiseConv2D(x4D, $filter, convInfo);
+      if ($bias != null) r = backend.add(r, $bias);
+      if (activation === 'relu') r = backend.relu(r);
+      else if (activation === 'relu6') r = backend.clip(r, 0, 6);
+      else if (activation !== 'linear') throw new Error(`Activation ${activation} is not supported after depthwiseConv2d`);
     }
-    let r = backend.depthwiseConv2D(x4D, $filter, convInfo);
-    if ($bias != null) r = backend.add(r, $bias);
-    if (activation === 'relu') r = backend.relu(r);
-    else if (activation === 'relu6') r = backend.clip(r, 0, 6);
-    else if (activation !== 'linear') throw new Error(`Activation ${activation} is not supported after depthwiseConv2d`);
+    save([$filter, x4D, r]);
     return r;
-  }, {x: x4D, $filter});
+  }, inputs, (dy, saved) => {
+    // the gradients of depthwiseConv2d (ops/conv.ts:520-540) behind that of the activation
+    const dil = config.dilations == null ? [1, 1] : config.dilations;
+    util.assert(conv_util.tupleValuesAreOne(dil),
+                () => 'Error in gradient of fused depthwiseConv2d: dilation rates greater than ' +
+                    `1 are not yet supported. Got dilations '${dil}'`);
+    const dyAct = fusedDyActivation(dy, saved[2], activation);
+    const g = {
+      x: () => depthwiseConv2dDerInput(saved[1].shape, dyAct, saved[0], config.strides, config.pad,
+                                       dil, config.dimRoundingMode),
+      $filter: () => depthwiseConv2dDerFilter(saved[1], dyAct, saved[0].shape, config.strides,
+                                              config.pad, dil, config.dimRoundingMode)
+    };
+    if ($bias != null) g.$bias = () => unbroadcast(dyAct, $bias.shape);
+    return g;
+  });
   return lower(res, reshapedTo4D);
 });
 

@@ -226,6 +226,14 @@ const OPS = {
     const y = tf.depthwiseConv2d(x, f, a.strides, a.pad);
     return a.squared ? tf.square(y) : y;
   })([i.x, i.filter])[a.wrt],
+  // fused.depthwiseConv2d / fused.separableConv2d (bias + activation folded in) through the tape
+  gradFusedDepthwise: (i, a) => tf.grads((x, f, b) => tf.fused.depthwiseConv2d(
+      {x, filter: f, strides: a.strides, pad: a.pad, bias: b, activation: a.activation}))(
+      [i.x, i.filter, i.bias], i.dy)[a.wrt],
+  gradFusedSeparable: (i, a) => tf.grads((x, f, pw, db, pb) => tf.fused.separableConv2d(
+      {x, depthwiseFilter: f, pointwiseFilter: pw, strides: a.strides, pad: a.pad, depthwiseBias: db,
+       depthwiseActivation: a.activation, bias: pb, activation: a.activation}))(
+      [i.x, i.filter, i.pw, i.bias, i.pbias], i.dy)[a.wrt],
   gradPool: (i, a) => tf.grad(x => a.kind === 'max' ? tf.maxPool(x, a.filterSize, a.strides, a.pad)
                                                     : tf.avgPool(x, a.filterSize, a.strides, a.pad))(i.x, i.dy),
   // loss = sum((relu(x w1 + b1) w2 - t)^2): d loss / d (w1 | b1 | w2)
