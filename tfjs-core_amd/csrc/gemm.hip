@@ -128,7 +128,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     long long a_base[A_PER];  // row-major: row*lda ; im2col: n*H*W*Cin
     int a_ih0[A_PER], a_iw0[A_PER];
     bool a_ok[A_PER];
+    // FAST loaders whose k offset is the same for every lane (row-major A, every B): the byte
+    // offset of the item inside a tile that lies wholly below K, and inside the one tile that K
+    // cuts (items at or beyond K out of range).  The tile's own offset rides in the scalar
+    // offset of the load, so a k step costs no address arithmetic on the vector ALU, which the
+    // matrix instructions share.
+    unsigned a_voff[A_PER], a_voff_cut[A_PER];
+    unsigned b_voff[B_PER], b_voff_cut[B_PER];
   };
+  constexpr bool A_UNIFORM_K = FAST && AMODE == A_ROWMAJOR;
 
   auto setup = [&](Loader& L, int tile) {
     const int batch = tile / tiles_per_batch;
@@ -173,6 +181,35 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
         }
       }
     }
+    if (FAST) {
+      const int k_cut = p.K / BK * BK;  // first k of the tile that K cuts (if K % BK != 0)
+      if (A_UNIFORM_K) {
+#pragma unroll
+        for (int i = 0; i < A_PER; i++) {
+          const unsigned at = ((unsigned)L.a_base[i] + (unsigned)L.a_kq[i]) * 4u;
+          L.a_voff[i] = L.a_ok[i] ? at : OOB_OFFSET;
+          L.a_voff_cut[i] = L.a_ok[i] && k_cut + L.a_kq[i] < p.K ? at : OOB_OFFSET;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < B_PER; i++) {
+        const int item = tid + i * THREADS;
+        int kk, n;
+        unsigned at;
+        if (BMODE == B_TRANSPOSED) {
+          n = L.bn0 + item / (BK / 4);
+          kk = (item % (BK / 4)) * 4;
+          at = ((unsigned)n * p.ldb + kk) * 4u;
+        } else {
+          kk = item / (BN / 4);
+          n = L.bn0 + (item % (BN / 4)) * 4;
+          at = ((unsigned)kk * p.ldb + n) * (BMODE == B_UINT8 ? 1u : 4u);
+        }
+        const bool ok = item < B_ITEMS && n < p.N;
+        L.b_voff[i] = ok ? at : OOB_OFFSET;
+        L.b_voff_cut[i] = ok && k_cut + kk < p.K ? at : OOB_OFFSET;
+      }
+    }
   };
 
   // FAST: both operands allow aligned 16-byte accesses (K, N, Cin multiples of 4) and span
@@ -180,8 +217,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   // 32-bit offsets — an item that is out of range gets OOB_OFFSET and reads as zero — so the
   // loads of a step are issued back to back and nothing touches their result until the
   // matrix cores are done with the step.
-  __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b;
-  auto load_a = [&](const Loader& L, int k0, f32x4 (&reg)[A_PER]) {
+  __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b, rsrc_a_none, rsrc_b_none;
+  // A tile that starts at k0 lies wholly below K, is cut by K, or lies beyond it (a load issued
+  // ahead of the last step): the same for all lanes, so the choice between the two offset sets
+  // is one select and a tile beyond K reads through the descriptor of length 0.
+  auto load_a = [&](const Loader& L, int k0_, f32x4 (&reg)[A_PER]) {
+    // (k0 is the same for the whole workgroup; saying so keeps the descriptor and the scalar
+    // offset in scalar registers wherever the compiler cannot see it)
+    const int k0 = FAST ? __builtin_amdgcn_readfirstlane(k0_) : k0_;
+    if (A_UNIFORM_K) {
+      const bool cut = k0 + BK > p.K;
+      const __amdgpu_buffer_rsrc_t r = k0 < p.K ? rsrc_a : rsrc_a_none;
+#pragma unroll
+      for (int i = 0; i < A_PER; i++)
+        reg[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                     r, (int)(cut ? L.a_voff_cut[i] : L.a_voff[i]), k0 * 4, 0));
+      return;
+    }
     if (FAST) {
 #pragma unroll
       for (int i = 0; i < A_PER; i++) {
@@ -318,32 +370,24 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   };
 
   // B items: B_ROWMAJOR / B_UINT8: (k, col-quad); B_TRANSPOSED: (col, k-quad)
-  auto load_b = [&](const Loader& L, int k0, f32x4 (&reg)[B_PER]) {
+  auto load_b = [&](const Loader& L, int k0_, f32x4 (&reg)[B_PER]) {
+    const int k0 = FAST ? __builtin_amdgcn_readfirstlane(k0_) : k0_;
     if (FAST) {
+      const bool cut = k0 + BK > p.K;
+      const __amdgpu_buffer_rsrc_t r = k0 < p.K ? rsrc_b : rsrc_b_none;
+      const int soff = BMODE == B_TRANSPOSED ? k0 * 4 : BMODE == B_UINT8 ? k0 * p.ldb : k0 * p.ldb * 4;
 #pragma unroll
       for (int i = 0; i < B_PER; i++) {
-        const int item = tid + i * THREADS;
-        int k, n;
-        unsigned off;
-        if (BMODE == B_TRANSPOSED) {
-          n = L.bn0 + item / (BK / 4);
-          k = k0 + (item % (BK / 4)) * 4;
-          off = (unsigned)n * p.ldb + k;
-        } else {
-          k = k0 + item / (BN / 4);
-          n = L.bn0 + (item % (BN / 4)) * 4;
-          off = (unsigned)k * p.ldb + n;
-        }
-        const bool ok = item < B_ITEMS && k < p.K && n < p.N;
+        const unsigned voff = cut ? L.b_voff_cut[i] : L.b_voff[i];
         if (BMODE == B_UINT8) {
-          const unsigned w =
-              __builtin_amdgcn_raw_buffer_load_b32(rsrc_b, (int)(ok ? off : OOB_OFFSET), 0, 0);
+          // (an item out of range reads 0, which must stay 0 and not become the dequantised minimum)
+          const unsigned w = __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, soff, 0);
           f32x4 v;
 #pragma unroll
           for (int e = 0; e < 4; e++) v[e] = dequant((w >> (8 * e)) & 0xffu, p.qscale, p.qmin);
-          reg[i] = ok ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+          reg[i] = voff != OOB_OFFSET && k0 < p.K ? v : f32x4{0.f, 0.f, 0.f, 0.f};
         } else {
-          reg[i] = buffer_load_f32x4(rsrc_b, ok ? off * 4u : OOB_OFFSET);
+          reg[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, soff, 0));
         }
       }
       return;
@@ -422,6 +466,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   const int n_steps = cur.kt1 - cur.kt0;
   rsrc_a = make_rsrc(L.A, p.a_bytes);
   rsrc_b = make_rsrc(BMODE == B_UINT8 ? (const void*)L.Bq : (const void*)L.Bf, p.b_bytes);
+  rsrc_a_none = make_rsrc(L.A, 0u);
+  rsrc_b_none = make_rsrc(BMODE == B_UINT8 ? (const void*)L.Bq : (const void*)L.Bf, 0u);
 
   // KBLOCKED (matMul): two-level accumulation.  The matrix cores sum 48 consecutive k into
   // `blk` (its first MFMA starts from the inline zero), which is then added to `acc` — the
