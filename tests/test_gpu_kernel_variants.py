@@ -127,7 +127,8 @@ def test_pointwise_conv_tiles(tf, n, h, cin, cout, act, want):
 # -------------------------------------- many rows times a small matrix ----
 @pytest.mark.parametrize("n,h,w_,cin,cout,act,bias,quant,want", [
     (16, 112, 112, 32, 64, "relu6", True, False, "gemm_rowstream_k32xn64_f32"),
-    (1, 449, 449, 32, 64, "prelu", True, False, "gemm_rowstream_k32xn64_f32"),   # odd row count
+    (1, 449, 449, 32, 64, "relu", True, False, "gemm_rowstream_k32xn64_f32"),    # odd row count
+    (1, 449, 449, 32, 64, "prelu", True, False, "gemm_64x64_rowmajor_f32"),      # prelu: the tiled kernel
     (3, 256, 257, 32, 64, "linear", False, False, "gemm_rowstream_k32xn64_f32"),
     (5, 200, 201, 32, 64, "relu", True, True, "gemm_rowstream_k32xn64_u8"),
     (2, 320, 331, 32, 64, "linear", True, True, "gemm_rowstream_k32xn64_u8"),
@@ -169,7 +170,8 @@ def test_rowstream_products(tf, ref, n, h, w_, cin, cout, act, bias, quant, want
 
 
 def test_rowstream_scalar_bias_and_slope(tf):
-    """fused matMul with a scalar bias and a scalar prelu slope through the row-streaming kernel."""
+    """fused matMul with a scalar bias through the row-streaming kernel; with a scalar prelu slope
+    the product goes to the tiled kernel, whose general store path multiplies by the slope."""
     rng = np.random.default_rng(78)
     m = 256 * 8 * 32 * 3 + 11
     a = rng.uniform(-1, 1, (m, 32)).astype(np.float32)
@@ -178,9 +180,13 @@ def test_rowstream_scalar_bias_and_slope(tf):
         got = tf.fused.matmul(tf.tensor(a), tf.tensor(b), bias=tf.tensor(np.float32(0.25)),
                               activation="prelu",
                               prelu_activation_weights=tf.tensor(np.float32(0.1))).data_sync()
+        assert last_kernel(tf).startswith("gemm_64x64_rowmajor_f32"), last_kernel(tf)
+        got_relu = tf.fused.matmul(tf.tensor(a), tf.tensor(b), bias=tf.tensor(np.float32(0.25)),
+                                   activation="relu").data_sync()
         assert last_kernel(tf) == "gemm_rowstream_k32xn64_f32", last_kernel(tf)
     y = a.astype(np.float64) @ b.astype(np.float64) + 0.25
     close(got, np.where(y < 0, np.float64(np.float32(0.1)) * y, y))
+    close(got_relu, np.maximum(y, 0))
 
 
 def test_rowstream_matmul_and_small_fallback(tf):

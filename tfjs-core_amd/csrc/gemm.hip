@@ -658,6 +658,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   const bool full_alpha = p.prelu_kind == TFHIP_BCAST_FULL;
   const bool vec_store = (TN == 2 || TN == 4) && (p.N % TN == 0);
   const ActCfg act = act_cfg(p.act);
+  const Clamp cl = clamp_of(p.act);
+  const bool prelu = p.act == TFHIP_ACT_PRELU;  // takes the FULL path: it alone needs a product
   // FULL: bias or prelu weights with one value per output element (rare) are read here.
   // INTERIOR: the whole tile lies inside the matrix, so no store needs a bounds check.
   // Addresses are a tile base that is the same for the whole wavefront plus a 32-bit offset.
@@ -684,7 +686,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
             if (full_bias && in) bv = p.bias[tile_at + at + j];
             if (full_alpha && in) al = p.prelu[tile_at + at + j];
           }
-          out[j] = activate(res[i][j][r] + bv, act, al);
+          out[j] = FULL ? activate(res[i][j][r] + bv, act, al) : clamp(res[i][j][r] + bv, cl);
         }
         if (vec_store && (INTERIOR || col0 + TN - 1 < p.N)) {
           if (TN == 2) {
@@ -705,7 +707,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     }
   };
   const bool interior = bm0 + BM <= p.M && bn0 + BN <= p.N;
-  if (full_bias || full_alpha) {
+  if (full_bias || full_alpha || prelu) {
     store(std::true_type{}, std::false_type{});
   } else if (!interior) {
     store(std::false_type{}, std::false_type{});
@@ -726,21 +728,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     constexpr int ROWS_PER_PASS = THREADS / QUADS_PER_ROW;
     static_assert(THREADS % QUADS_PER_ROW == 0 && BM % ROWS_PER_PASS == 0, "tile / block shape");
     const int cq = tid % QUADS_PER_ROW, r0 = tid / QUADS_PER_ROW;
-    f32x4 bv = {0.f, 0.f, 0.f, 0.f}, al = {0.f, 0.f, 0.f, 0.f};
+    f32x4 bv = {0.f, 0.f, 0.f, 0.f};
     if (p.bias_kind == TFHIP_BCAST_SCALAR) bv = f32x4{p.bias[0], p.bias[0], p.bias[0], p.bias[0]};
     if (p.bias_kind == TFHIP_BCAST_COLUMN)
 #pragma unroll
       for (int e = 0; e < 4; e++) bv[e] = p.bias[bn0 + 4 * cq + e];
-    if (p.prelu_kind == TFHIP_BCAST_SCALAR) al = f32x4{p.prelu[0], p.prelu[0], p.prelu[0], p.prelu[0]};
-    if (p.prelu_kind == TFHIP_BCAST_COLUMN)
-#pragma unroll
-      for (int e = 0; e < 4; e++) al[e] = p.prelu[bn0 + 4 * cq + e];
 #pragma unroll
     for (int pass = 0; pass < BM / ROWS_PER_PASS; pass++) {
       const int row = r0 + pass * ROWS_PER_PASS;
       f32x4 v = *reinterpret_cast<const f32x4*>(lds + row * LDC_S + 4 * cq);
 #pragma unroll
-      for (int e = 0; e < 4; e++) v[e] = activate(v[e] + bv[e], act, al[e]);
+      for (int e = 0; e < 4; e++) v[e] = clamp(v[e] + bv[e], cl);
       *reinterpret_cast<f32x4*>(Ct + row * p.N + 4 * cq) = v;
     }
   } else {
@@ -983,6 +981,8 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
     const long long out_at = (((long long)n * p.OH + oh) * p.OW) * p.N;  // workgroup-uniform
     float* __restrict__ crow = p.C + out_at;
     const ActCfg act = act_cfg(p.act);
+    const Clamp cl = clamp_of(p.act);
+    const bool prelu = p.act == TFHIP_ACT_PRELU;  // (takes the general path below)
     const float* bias_row = p.bias_kind == TFHIP_BCAST_FULL ? p.bias + out_at : nullptr;
     const float* alpha_row = p.prelu_kind == TFHIP_BCAST_FULL ? p.prelu + out_at : nullptr;
     // the output row as a descriptor: pixels past the row fall out of its range
@@ -1015,7 +1015,7 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
       }
       // accumulator register r holds pixel 8*(r/4) + 4*(lane/32) + r%4 of the strip
       const int px0 = strip * 32 + 4 * g;
-      if (bias_row || alpha_row) {
+      if (bias_row || alpha_row || prelu) {
         const int px0_ = opaque(px0), l32_ = opaque(l32);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -1045,7 +1045,7 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
           const unsigned px_at = (unsigned)((8 * (r >> 2) + (r & 3)) * p.N * 4);
 #pragma unroll
           for (int j = 0; j < TN; j++) {
-            const float v = activate(acc[j][r] + bias_c[j], act, alpha_c[j]);
+            const float v = clamp(acc[j][r] + bias_c[j], cl);
             __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rout,
                                                   (int)(lane_at[j] + px_at), 0, 0);
           }
@@ -1098,17 +1098,15 @@ __global__ __launch_bounds__(256, 2) void gemm_rowstream_kernel(const GemmArgs p
     if (quant) fill(std::true_type{});
     else fill(std::false_type{});
   }
-  float bias_c[NJ], alpha_c[NJ];  // of column 32j + l32
+  float bias_c[NJ];  // of column 32j + l32
 #pragma unroll
   for (int j = 0; j < NJ; j++) {
     const int col = 32 * j + l32;
-    bias_c[j] = alpha_c[j] = 0.f;
+    bias_c[j] = 0.f;
     if (p.bias_kind == TFHIP_BCAST_SCALAR) bias_c[j] = p.bias[0];
     if (p.bias_kind == TFHIP_BCAST_COLUMN) bias_c[j] = p.bias[col];
-    if (p.prelu_kind == TFHIP_BCAST_SCALAR) alpha_c[j] = p.prelu[0];
-    if (p.prelu_kind == TFHIP_BCAST_COLUMN) alpha_c[j] = p.prelu[col];
   }
-  const ActCfg act = act_cfg(p.act);
+  const Clamp cl = clamp_of(p.act);  // (prelu never comes here: the tiled kernel takes it)
   __syncthreads();
 
   // The 32-row blocks are cut into 8 runs, one per XCD (workgroup b runs on XCD b % 8; the grid
@@ -1176,7 +1174,7 @@ __global__ __launch_bounds__(256, 2) void gemm_rowstream_kernel(const GemmArgs p
 #pragma unroll
         for (int j = 0; j < NJ; j++) {
           const int row_c = 8 * (r >> 2) + (r & 3);  // + 4 * g
-          const float v = activate(acc[j][r] + bias_c[j], act, alpha_c[j]);
+          const float v = clamp(acc[j][r] + bias_c[j], cl);
           const unsigned at = whole || row_c + 4 * g < left ? c_at : OOB_OFFSET;
           __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rc, (int)at,
                                                 /*scalar offset=*/(row_c * N + 32 * j) * 4, 0);
@@ -1455,7 +1453,7 @@ static int launch_rowstream_cfg(tfhip_ctx* ctx, const GemmArgs& p, int quant) {
 static int launch_rowstream(tfhip_ctx* ctx, const GemmArgs& p, int batch, int amode, int bmode) {
   if (batch != 1 || amode != A_ROWMAJOR || (bmode != B_ROWMAJOR && bmode != B_UINT8)) return -1;
   if (p.lda != p.K || p.ldb != p.N || !p.a_vec || !p.b_vec) return -1;
-  if (p.bias_kind == TFHIP_BCAST_FULL || p.prelu_kind == TFHIP_BCAST_FULL) return -1;
+  if (p.bias_kind == TFHIP_BCAST_FULL || p.act == TFHIP_ACT_PRELU) return -1;
   // enough 32-row blocks to give every wavefront of a full machine several
   if ((long long)p.M < (long long)ctx->num_cus * 8 * 32 * 3) return -1;
   const int quant = bmode == B_UINT8;

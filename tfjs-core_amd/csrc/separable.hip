@@ -34,23 +34,6 @@
 
 namespace tfhip {
 
-// relu / relu6 / linear as a clamp to [lo, hi] that lets NaN through (no comparison with NaN
-// holds), which is what the reference's Math.max(0, x) and clip do (backend_cpu.ts:1191-1201,
-// :1265-1275): two compares and two selects per value.
-struct Clamp {
-  float lo, hi;
-};
-__device__ __forceinline__ Clamp clamp_of(int act) {
-  Clamp c;
-  c.lo = act == TFHIP_ACT_LINEAR ? -__builtin_inff() : 0.f;
-  c.hi = act == TFHIP_ACT_RELU6 ? 6.f : __builtin_inff();
-  return c;
-}
-__device__ __forceinline__ float clamp(float v, const Clamp& c) {
-  const float r = v < c.lo ? c.lo : v;
-  return r > c.hi ? c.hi : r;
-}
-
 struct SepArgs {
   const float* x;
   const void* dw;    // [3][3][K] float32 or uint8

@@ -54,4 +54,23 @@ __device__ __forceinline__ float activate(float v, const ActCfg& c, float alpha)
   return r > c.hi ? c.hi : r;
 }
 
+// relu / relu6 / linear as a clamp to [lo, hi] that lets NaN through (no comparison with NaN
+// holds), which is what the reference's Math.max(0, x) and clip do (backend_cpu.ts:1191-1201,
+// :1265-1275): two compares and two selects per value, against nine vector instructions of the
+// general form above.  The matrix instructions share their pipe with the vector ALU, so the
+// stores of the dense kernels use this form and leave prelu to their general path.
+struct Clamp {
+  float lo, hi;
+};
+__device__ __forceinline__ Clamp clamp_of(int act) {
+  Clamp c;
+  c.lo = act == TFHIP_ACT_LINEAR ? -__builtin_inff() : 0.f;
+  c.hi = act == TFHIP_ACT_RELU6 ? 6.f : __builtin_inff();
+  return c;
+}
+__device__ __forceinline__ float clamp(float v, const Clamp& c) {
+  const float r = v < c.lo ? c.lo : v;
+  return r > c.hi ? c.hi : r;
+}
+
 }  // namespace tfhip
