@@ -484,7 +484,8 @@ def main():
                           for k, g in groups.items()},
         "layers": [dict(name=r["name"], kernel=r["kernel"], us=round(r["ms"] * 1e3, 2),
                         tflops=round(2e-9 * r["macs"] / r["ms"], 2),
-                        gbs=round(1e-6 * r["bytes"] / r["ms"], 1)) for r in (rows or [])],
+                        gbs=round(1e-6 * r["bytes"] / r["ms"], 1), algorithmic_bytes=r["bytes"],
+                        launches=r["launches"]) for r in (rows or [])],
     }
     if not args.no_ops:
         out["op_configs"] = op_level_configs(tf, np)

@@ -107,11 +107,20 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   constexpr int C_FLOATS = STAGED_STORE ? BM * LDC_S : 0;
   constexpr int LDS_FLOATS = A_FLOATS + B_FLOATS > C_FLOATS ? A_FLOATS + B_FLOATS : C_FLOATS;
   __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
+  // uint8 weights: the 256 values a byte can stand for, each computed once per workgroup exactly
+  // as dequant() does; a weight then costs a bit-field extract and an LDS read instead of four
+  // double-precision instructions on the pipe the matrix instructions need
+  __shared__ float lut[BMODE == B_UINT8 ? 256 : 1];
   float (*As)[BM * LDA_S] = reinterpret_cast<float (*)[BM * LDA_S]>(lds);
   float (*Bs)[BK * LDB_S] = reinterpret_cast<float (*)[BK * LDB_S]>(lds + A_FLOATS);
 
   const int tid = threadIdx.x;
   __builtin_assume(tid >= 0 && tid < THREADS);
+  if (BMODE == B_UINT8 && FAST) {
+    static_assert(THREADS >= 256, "one table entry per thread");
+    if (tid < 256) lut[tid] = dequant((unsigned)tid, p.qscale, p.qmin);
+    __syncthreads();  // (the prologue of the k loop converts weights right away)
+  }
   const int lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int l32 = lane & 31, g = lane >> 5;
@@ -380,12 +389,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       for (int i = 0; i < B_PER; i++) {
         const unsigned voff = cut ? L.b_voff_cut[i] : L.b_voff[i];
         if (BMODE == B_UINT8) {
-          // (an item out of range reads 0, which must stay 0 and not become the dequantised minimum)
+          // The four bytes stay as they are until store_b turns them into floats on their way
+          // into LDS, so nothing waits for this load here.  An item out of range reads 0 and
+          // becomes the (finite) value of byte 0: every A loader zeroes the items at or beyond
+          // K, so such a weight is multiplied by 0, and columns at or beyond N are never stored.
           const unsigned w = __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, soff, 0);
-          f32x4 v;
-#pragma unroll
-          for (int e = 0; e < 4; e++) v[e] = dequant((w >> (8 * e)) & 0xffu, p.qscale, p.qmin);
-          reg[i] = voff != OOB_OFFSET && k0 < p.K ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+          reg[i][0] = __builtin_bit_cast(float, w);
         } else {
           reg[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, soff, 0));
         }
@@ -453,7 +462,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
           for (int e = 0; e < 4; e++) bs[(kq + e) * LDB_S + nn] = reg[i][e];
         } else {
           const int kk = item / (BN / 4), nq = (item % (BN / 4)) * 4;
-          *reinterpret_cast<f32x4*>(&bs[kk * LDB_S + nq]) = reg[i];
+          f32x4 v = reg[i];
+          if (BMODE == B_UINT8 && FAST) {
+            const unsigned w = __builtin_bit_cast(unsigned, reg[i][0]);
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = lut[(w >> (8 * e)) & 0xffu];
+          }
+          *reinterpret_cast<f32x4*>(&bs[kk * LDB_S + nq]) = v;
         }
       }
     }

@@ -51,6 +51,7 @@ struct SepArgs {
   int strips;  // ceil(OW / SW)
   int units;   // batch * chunks * strips
   int reverse;
+  int prio;
 };
 
 template <int KQ, int NJ, int S, int PD, int OCC>
@@ -163,6 +164,9 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.x, p.x_bytes);
     const unsigned x_row = (unsigned)(p.W * K * 4);
     float* const panel_w = panels + (slot * TW) * PITCH + 4 * quad;  // where this lane writes
+    // These wavefronts have little to do per panel and the memory system waits for their loads:
+    // they go first whenever they can issue, ahead of the long matrix chains on the same SIMD.
+    if (p.prio) __builtin_amdgcn_s_setprio(3);
     __syncthreads();
 
     // Input row t of a unit (counted from the top of the padding, ih = t - pt) is filter row kh
@@ -429,6 +433,7 @@ static int launch_separable(tfhip_ctx* ctx, SepArgs& p) {
   const long long resident = (long long)ctx->num_cus * per_cu / 8 * 8;  // a multiple of the XCD count
   ctx->name_kernel("separable_s%d_k%dxn%d_%s", S, K, N, p.pw_quant ? "u8" : "f32");
   p.reverse = ctx->take_sweep();
+  p.prio = getenv("TFHIP_SEP_PRIO") ? atoi(getenv("TFHIP_SEP_PRIO")) : 0;
   tfhip::launch(ctx, kernel, dim3((unsigned)(want < resident || resident < 8 ? want : resident)),
                 dim3(512), lds, p);
   TFHIP_LAUNCH_CHECK(ctx);
