@@ -26,7 +26,6 @@
 //     dword stores of 128-byte runs.
 // Wavefronts of a workgroup share nothing but the filter, so there is no barrier after the set-up;
 // the other wavefronts of the SIMD fill the time one of them waits for memory or the matrix cores.
-#include <cstdlib>
 #include <type_traits>
 
 #include "tfhip_internal.h"
@@ -51,7 +50,6 @@ struct SepArgs {
   int strips;  // ceil(OW / SW)
   int units;   // batch * chunks * strips
   int reverse;
-  int prio;
 };
 
 template <int KQ, int NJ, int S, int PD, int OCC>
@@ -164,9 +162,6 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.x, p.x_bytes);
     const unsigned x_row = (unsigned)(p.W * K * 4);
     float* const panel_w = panels + (slot * TW) * PITCH + 4 * quad;  // where this lane writes
-    // These wavefronts have little to do per panel and the memory system waits for their loads:
-    // they go first whenever they can issue, ahead of the long matrix chains on the same SIMD.
-    if (p.prio) __builtin_amdgcn_s_setprio(3);
     __syncthreads();
 
     // Input row t of a unit (counted from the top of the padding, ih = t - pt) is filter row kh
@@ -425,7 +420,6 @@ static int launch_separable(tfhip_ctx* ctx, SepArgs& p) {
   int rh = (int)ceil_div(p.OH, RB) * RB;
   while (rh > RB && (long long)p.batch * p.strips * ceil_div(p.OH, rh) < slots / 2)
     rh = (int)ceil_div(ceil_div(rh, 2), RB) * RB;
-  if (const char* e = getenv("TFHIP_SEP_RH")) rh = atoi(e);
   p.rh = rh;
   p.chunks = (int)ceil_div(p.OH, rh);
   p.units = p.batch * p.chunks * p.strips;
@@ -433,7 +427,6 @@ static int launch_separable(tfhip_ctx* ctx, SepArgs& p) {
   const long long resident = (long long)ctx->num_cus * per_cu / 8 * 8;  // a multiple of the XCD count
   ctx->name_kernel("separable_s%d_k%dxn%d_%s", S, K, N, p.pw_quant ? "u8" : "f32");
   p.reverse = ctx->take_sweep();
-  p.prio = getenv("TFHIP_SEP_PRIO") ? atoi(getenv("TFHIP_SEP_PRIO")) : 0;
   tfhip::launch(ctx, kernel, dim3((unsigned)(want < resident || resident < 8 ? want : resident)),
                 dim3(512), lds, p);
   TFHIP_LAUNCH_CHECK(ctx);
@@ -535,12 +528,7 @@ extern "C" int tfhip_separable_conv2d(tfhip_ctx* ctx, int64_t x, int64_t dw_filt
     p.x_bytes = (unsigned)(x_n * 4);
     p.y_bytes = (unsigned)(pixels * N * 4);
     switch (variant) {
-      case 0: {
-        const char* v = getenv("TFHIP_SEP_V");
-        const int vi = v ? atoi(v) : 0;
-        if (vi == 1) return launch_separable<4, 2, 1, 4, 2>(ctx, p);
-        return launch_separable<4, 2, 1, 2, 4>(ctx, p);
-      }
+      case 0: return launch_separable<4, 2, 1, 2, 4>(ctx, p);
       case 1: return launch_separable<8, 4, 2, 8, 2>(ctx, p);
       default: break;
     }
