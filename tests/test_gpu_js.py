@@ -1222,3 +1222,15 @@ def test_js_complex_and_spectral(tmp_path):
     results = c.run()
     c.check(results)
     assert results["memory"]["numTensors"] == 0 and results["memory"]["numDeviceBuffers"] == 0
+
+
+def test_js_deferred_epilogues():
+    """conv2d -> add -> relu | clipByValue, matMul -> add -> relu and the depthwise -> 1x1 chain as
+    the reference's graphs spell them: one launch each with the bits of the fused calls, also when
+    inputs are disposed or overwritten before the result is read, intermediates reused, or the
+    result never used (js/test/defer_test.js)."""
+    r = subprocess.run([NODE, os.path.join(JS, "test", "defer_test.js")], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-3000:]
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert out["ok"], out["failures"]

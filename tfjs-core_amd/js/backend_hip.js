@@ -72,6 +72,95 @@ class MathBackendHIP extends KernelBackend {
     this.ctx = this.napi.init(device == null ? ENV.get('HIP_DEVICE') : device);
     this.data = new DataStorage(this, ENGINE);
     this.nextHandle = 1;
+    // Deferred dense ops (see defer()): result dataId -> record, and input dataId -> the records
+    // that still have to read it.
+    this.pending = new Map();
+    this.readersOf = new Map();
+    this.zombies = new Set();  // disposed tensors that a folded record could still have to read
+  }
+
+  // ---- deferred epilogues ------------------------------------------------------------------
+  // The reference's graphs spell a convolution layer as conv2d -> add(bias) -> relu | clipByValue
+  // (three backend calls, three passes over the activation).  conv2d, depthwiseConv2D and
+  // batchMatMul therefore do not launch at once: they leave a record for their result, add() of a
+  // foldable bias and relu() / clip(0, 6) on such a result make a record of their own that carries
+  // the bias / activation, and a 1x1 conv2d of a deferred depthwise result becomes the separable
+  // pair.  A record launches (one kernel, epilogue folded in) when its tensor is first needed:
+  // as an input of any kernel, by read / readSync, or when one of its own inputs is about to be
+  // disposed or overwritten.  A record that was folded into another one and whose tensor is
+  // disposed unused never launches, which is what happens to the two intermediates of the
+  // spelled-out layer.  Every record's inputs are materialised when the record is made, so
+  // records never wait for each other.
+  defer(desc) {
+    this.lazyRegister = true;
+    let out;
+    try {
+      out = this.out(desc.outShape);
+    } finally {
+      this.lazyRegister = false;
+    }
+    const r = Object.assign({}, desc, {out, inputs: desc.inputs.filter(t => t != null)});
+    this.pending.set(out.dataId, r);
+    for (const t of r.inputs) {
+      let readers = this.readersOf.get(t.dataId);
+      if (readers == null) this.readersOf.set(t.dataId, readers = new Set());
+      readers.add(r);
+    }
+    return out;
+  }
+  forget(r) {
+    this.pending.delete(r.out.dataId);
+    for (const t of r.inputs) {
+      const readers = this.readersOf.get(t.dataId);
+      if (readers != null) {
+        readers.delete(r);
+        if (readers.size === 0) {
+          this.readersOf.delete(t.dataId);
+          if (this.zombies.delete(t.dataId)) this.release(t.dataId);
+        }
+      }
+    }
+  }
+  flush(r) {
+    this.forget(r);
+    const rec = this.data.get(r.out.dataId);
+    if (rec.unallocated != null) this.allocate(rec);
+    r.run(r);
+  }
+  materialize(dataId) {
+    const r = this.pending.get(dataId);
+    if (r != null) this.flush(r);
+  }
+  flushReadersOf(dataId) {
+    const readers = this.readersOf.get(dataId);
+    if (readers != null) Array.from(readers).forEach(r => this.flush(r));
+  }
+  // (folded intermediates stay deferred: they run only if someone asks for them)
+  flushAll() {
+    Array.from(this.pending.values()).forEach(r => { if (!r.folded) this.flush(r); });
+  }
+  deferring() { return ENV.get('HIP_DEFER_EPILOGUE') && ENV.get('HIP_FUSE_EPILOGUE'); }
+  // add(t, bias) / relu(t) / clip(t, 0, 6) on a deferred result: a new record that carries them.
+  // (t may be a reshaped alias of the deferred result, e.g. the 2-D view tf.matMul returns of a
+  // batchMatMul: what must agree is the element count and, for a bias, the innermost dimension)
+  foldBias(t, bias) {
+    const p = this.pending.get(t.dataId);
+    if (p == null || p.bias != null || p.act !== 'linear' || bias.dtype !== 'float32' ||
+        t.dtype !== 'float32' || this.pending.has(bias.dataId) || t.rank === 0 ||
+        t.shape[t.rank - 1] !== p.outShape[p.outShape.length - 1] || bias.rank > t.rank) {
+      return null;
+    }
+    const bk = this.epilogueKind(bias, t.shape);
+    if (bk == null || bk === BCAST.NONE || (bk === BCAST.FULL && !p.fullBias)) return null;
+    p.folded = true;
+    return this.defer(Object.assign({}, p, {outShape: t.shape, bias, bk, folded: false,
+                                            inputs: p.inputs.concat([bias])}));
+  }
+  foldActivation(t, act) {
+    const p = this.pending.get(t.dataId);
+    if (p == null || p.act !== 'linear' || t.dtype !== 'float32') return null;
+    p.folded = true;
+    return this.defer(Object.assign({}, p, {outShape: t.shape, act, folded: false}));
   }
 
   // ---- storage (backend.ts:33-44; CPU behaviour backend_cpu.ts:102-129, 199-254) ----
@@ -83,8 +172,15 @@ class MathBackendHIP extends KernelBackend {
     if (code == null) throw new Error(`hip backend: dtype ${dtype} is not supported`);
     const handle = this.nextHandle++;
     const stored = complex ? shape.concat([2]) : shape;
-    this.napi.register(this.ctx, handle, Int32Array.from(stored), code);
-    this.data.set(dataId, {handle, code, size: util.sizeFromShape(stored)});
+    const rec = {handle, code, size: util.sizeFromShape(stored)};
+    // the result of a deferred op gets its device buffer when the op launches, if it ever does
+    if (this.lazyRegister) rec.unallocated = Int32Array.from(stored);
+    else this.napi.register(this.ctx, handle, Int32Array.from(stored), code);
+    this.data.set(dataId, rec);
+  }
+  allocate(rec) {
+    this.napi.register(this.ctx, rec.handle, rec.unallocated, rec.code);
+    rec.unallocated = null;
   }
 
   // Up to 64 KiB the bytes are staged and the call returns at once; a larger array is copied on
@@ -96,7 +192,13 @@ class MathBackendHIP extends KernelBackend {
   // it has been read.
   write(dataId, values) {
     if (values == null) throw new Error('MathBackendHIP.write(): values can not be null');
+    if (this.pending.size !== 0) {
+      this.flushReadersOf(dataId);  // they were promised the old values
+      const p = this.pending.get(dataId);
+      if (p != null) this.forget(p);  // overwritten before anyone looked
+    }
     const rec = this.data.get(dataId);
+    if (rec.unallocated != null) this.allocate(rec);
     let arr = values;
     const want = rec.code === DTYPE.float32 ? Float32Array :
         rec.code === DTYPE.int32 ? Int32Array : Uint8Array;
@@ -117,6 +219,7 @@ class MathBackendHIP extends KernelBackend {
   }
 
   readSync(dataId) {
+    this.materialize(dataId);
     const rec = this.data.get(dataId);
     return this.napi.read(this.ctx, rec.handle, typedArrayFor(rec.code, rec.size));
   }
@@ -128,6 +231,7 @@ class MathBackendHIP extends KernelBackend {
   read(dataId) {
     let rec;
     try {
+      this.materialize(dataId);
       rec = this.data.get(dataId);
       const ctor = rec.code === DTYPE.float32 ? Float32Array :
           rec.code === DTYPE.int32 ? Int32Array : Uint8Array;
@@ -140,8 +244,30 @@ class MathBackendHIP extends KernelBackend {
   }
 
   disposeData(dataId) {
+    if (this.pending.size !== 0) {
+      // An intermediate whose value went into a folded record is never computed for its own sake;
+      // any other deferred result is computed even if nobody reads it, as an eager backend would
+      // (`tf.matMul(a, b).dispose()` in a timing loop measures the product).
+      const p = this.pending.get(dataId);
+      if (p != null) p.folded ? this.forget(p) : this.flush(p);
+      // Deferred ops that still have to read this tensor run now, except folded intermediates:
+      // most of them are about to be disposed unused themselves (the end of a tidy disposes in
+      // creation order, inputs first), so the buffer stays until the last of them is gone.
+      const readers = this.readersOf.get(dataId);
+      if (readers != null) {
+        Array.from(readers).forEach(r => { if (!r.folded) this.flush(r); });
+        if (this.readersOf.has(dataId)) {
+          this.zombies.add(dataId);
+          return;
+        }
+      }
+    }
+    this.release(dataId);
+  }
+  release(dataId) {
     if (this.data.has(dataId)) {
-      this.napi.dispose(this.ctx, this.data.get(dataId).handle);
+      const rec = this.data.get(dataId);
+      if (rec.unallocated == null) this.napi.dispose(this.ctx, rec.handle);
       this.data.delete(dataId);
     }
   }
@@ -160,11 +286,17 @@ class MathBackendHIP extends KernelBackend {
   captureGraph(f) {
     const {ENGINE, getTensorsInContainer} = require('./engine');
     getTensorsInContainer(ENGINE.tidy(f)).forEach(t => t.dispose());
+    this.flushAll();
     this.napi.graphBegin(this.ctx);
     let outputs;
     try {
       outputs = ENGINE.tidy(f);
+      this.flushAll();  // deferred work belongs to the recording
     } catch (e) {
+      this.pending.clear();
+      this.readersOf.clear();
+      this.zombies.forEach(d => this.release(d));
+      this.zombies.clear();
       try {
         this.napi.graphDestroy(this.ctx, this.napi.graphEnd(this.ctx));
       } catch (ignored) {}
@@ -191,10 +323,12 @@ class MathBackendHIP extends KernelBackend {
   // launch: getExtraProfileInfo() returns them as 'name: ms' pairs (the interface asks for a
   // string), kernelTimes as [{name, ms}] in launch order.
   async time(f) {
+    this.flushAll();  // what was deferred before the region is not the region's work
     this.napi.timeBegin(this.ctx);
     let kernelMs;
     try {
       f();
+      this.flushAll();
     } finally {
       kernelMs = this.napi.timeEnd(this.ctx);
     }
@@ -207,11 +341,20 @@ class MathBackendHIP extends KernelBackend {
     };
   }
 
-  sync() { this.napi.sync(this.ctx); }
-  lastKernel() { return this.napi.lastKernel(this.ctx); }
+  sync() {
+    this.flushAll();
+    this.napi.sync(this.ctx);
+  }
+  lastKernel() {
+    this.flushAll();
+    return this.napi.lastKernel(this.ctx);
+  }
   floatPrecision() { return 32; }
 
   dispose() {
+    this.pending.clear();
+    this.readersOf.clear();
+    this.zombies.clear();
     if (this.ctx != null) {
       this.napi.destroy(this.ctx);
       this.ctx = null;
@@ -223,7 +366,10 @@ class MathBackendHIP extends KernelBackend {
   }
 
   // ---- helpers ----
-  h(t) { return this.data.get(t.dataId).handle; }
+  h(t) {
+    if (this.pending.size !== 0) this.materialize(t.dataId);
+    return this.data.get(t.dataId).handle;
+  }
   storageCode(t) { return this.data.get(t.dataId).code; }
   out(shape, dtype) { return Tensor.make(shape, {}, dtype || 'float32', this); }
   q(t) { return t.quantization ? Float64Array.of(t.quantization.scale, t.quantization.min) : null; }
@@ -281,12 +427,24 @@ class MathBackendHIP extends KernelBackend {
       if (bias != null) r = this.add(r, bias);
       return this.mapActivation(r, activation, preluActivationWeights);
     }
+    if (this.deferring() && (activation == null || activation === 'linear')) {
+      // (an add and a relu | clip may follow; see defer())
+      this.h(a);
+      this.h(b);
+      if (bk) this.h(bias);
+      return this.defer({
+        kind: 'matmul', outShape, inputs: [a, b, bk ? bias : null], bias: bk ? bias : null, bk,
+        act: 'linear', fullBias: true,
+        run: r => this.matmulImpl(a, b, batch, m, n, k, transposeA, transposeB, r.bias, r.bk, r.act,
+                                  null, 0, r.out)
+      });
+    }
     return this.matmulImpl(a, b, batch, m, n, k, transposeA, transposeB, bias, bk,
                            activation || 'linear', preluActivationWeights, pk);
   }
 
-  matmulImpl(a, b, batch, m, n, k, tA, tB, bias, bk, activation, prelu, pk) {
-    const out = this.out([batch, m, n]);
+  matmulImpl(a, b, batch, m, n, k, tA, tB, bias, bk, activation, prelu, pk, into) {
+    const out = into || this.out([batch, m, n]);
     this.napi.matmul(this.ctx, this.h(a), this.h(b), this.h(out), batch, m, n, k, tA ? 1 : 0,
                      tB ? 1 : 0, bk ? this.h(bias) : -1, bk, ACT[activation],
                      pk ? this.h(prelu) : -1, pk, this.q(b));
@@ -307,9 +465,44 @@ class MathBackendHIP extends KernelBackend {
       if (bias != null) r = this.add(r, bias);
       return this.mapActivation(r, activation, preluActivationWeights);
     }
+    const act = activation || 'linear';
+    if (this.deferring() && act !== 'prelu') {
+      // A 1x1 convolution of a deferred depthwise result (bias and activation folded or not):
+      // the separable pair, which the library runs as one kernel where it can.
+      const dw = this.pending.get(x.dataId);
+      const foldable = k => k === BCAST.NONE || k === BCAST.SCALAR || k === BCAST.COLUMN;
+      if (dw != null && dw.kind === 'depthwise' && util.arraysEqual(x.shape, dw.outShape) &&
+          convInfo.filterHeight === 1 && convInfo.filterWidth === 1 && convInfo.strideHeight === 1 &&
+          convInfo.strideWidth === 1 && convInfo.padInfo.top === 0 && convInfo.padInfo.left === 0 &&
+          convInfo.padInfo.bottom === 0 && convInfo.padInfo.right === 0 && foldable(dw.bk) &&
+          foldable(bk) && !this.pending.has(filter.dataId)) {
+        if (bk) this.h(bias);
+        dw.folded = true;
+        return this.defer({
+          kind: 'separable', outShape, inputs: dw.inputs.concat([filter, bk ? bias : null]),
+          bias: bk ? bias : null, bk, act, fullBias: false,
+          run: r => this.napi.separableConv2d(
+              this.ctx, this.h(dw.x), this.h(dw.filter), this.h(filter), this.h(r.out),
+              convInfoArray(dw.convInfo), dw.bk ? this.h(dw.bias) : -1, dw.bk, ACT[dw.act],
+              r.bk ? this.h(r.bias) : -1, r.bk, ACT[r.act], this.q(dw.filter), this.q(filter))
+        });
+      }
+      if (act === 'linear') {
+        this.h(x);
+        this.h(filter);
+        if (bk) this.h(bias);
+        return this.defer({
+          kind: 'conv2d', outShape, inputs: [x, filter, bk ? bias : null], bias: bk ? bias : null,
+          bk, act, fullBias: true,
+          run: r => this.napi.conv2d(this.ctx, this.h(x), this.h(filter), this.h(r.out),
+                                     convInfoArray(convInfo), r.bk ? this.h(r.bias) : -1, r.bk,
+                                     ACT[r.act], -1, BCAST.NONE, this.q(filter))
+        });
+      }
+    }
     const out = this.out(outShape);
     this.napi.conv2d(this.ctx, this.h(x), this.h(filter), this.h(out), convInfoArray(convInfo),
-                     bk ? this.h(bias) : -1, bk, ACT[activation || 'linear'],
+                     bk ? this.h(bias) : -1, bk, ACT[act],
                      pk ? this.h(preluActivationWeights) : -1, pk, this.q(filter));
     return out;
   }
@@ -330,6 +523,19 @@ class MathBackendHIP extends KernelBackend {
       let r = this.fusedDepthwiseConv2D(x, filter, convInfo);
       if (bias != null) r = this.add(r, bias);
       return this.mapActivation(r, activation, null);
+    }
+    if (this.deferring()) {
+      // (deferred even with its activation in place: a 1x1 conv2d may make it a separable pair)
+      this.h(x);
+      this.h(filter);
+      if (bk) this.h(bias);
+      return this.defer({
+        kind: 'depthwise', outShape, inputs: [x, filter, bk ? bias : null], x, filter, convInfo,
+        bias: bk ? bias : null, bk, act: activation || 'linear', fullBias: false,
+        run: r => this.napi.depthwiseConv2d(this.ctx, this.h(x), this.h(filter), this.h(r.out),
+                                            convInfoArray(convInfo), r.bk ? this.h(r.bias) : -1,
+                                            r.bk, ACT[r.act], this.q(filter))
+      });
     }
     const out = this.out(outShape);
     this.napi.depthwiseConv2d(this.ctx, this.h(x), this.h(filter), this.h(out),
@@ -419,7 +625,13 @@ class MathBackendHIP extends KernelBackend {
     const dt = util.upcastType(a.dtype, b.dtype);
     return dt === 'bool' ? 'int32' : dt;
   }
-  add(a, b) { return this.binary('add', a, b, this.arithDtype(a, b)); }
+  add(a, b) {
+    if (this.pending.size !== 0) {
+      const folded = this.foldBias(a, b) || this.foldBias(b, a);
+      if (folded != null) return folded;
+    }
+    return this.binary('add', a, b, this.arithDtype(a, b));
+  }
   subtract(a, b) { return this.binary('sub', a, b, this.arithDtype(a, b)); }
   multiply(a, b) { return this.binary('mul', a, b, this.arithDtype(a, b)); }
   realDivide(a, b) { return this.binary('div', a, b, 'float32'); }
@@ -432,8 +644,14 @@ class MathBackendHIP extends KernelBackend {
     this.napi.unary(this.ctx, UNARY[op], this.h(x), this.h(out), p0 || 0, p1 || 0);
     return out;
   }
-  relu(x) { return this.unary('relu', x, x.dtype === 'float32' ? 'float32' : 'int32'); }
-  clip(x, min, max) { return this.unary('clip', x, 'float32', min, max); }
+  relu(x) {
+    const folded = this.pending.size !== 0 ? this.foldActivation(x, 'relu') : null;
+    return folded || this.unary('relu', x, x.dtype === 'float32' ? 'float32' : 'int32');
+  }
+  clip(x, min, max) {
+    const folded = this.pending.size !== 0 && min === 0 && max === 6 ? this.foldActivation(x, 'relu6') : null;
+    return folded || this.unary('clip', x, 'float32', min, max);
+  }
   exp(x) { return this.unary('exp', x); }
   log(x) { return this.unary('log', x); }
   neg(x) { return this.unary('neg', x, x.dtype === 'float32' ? 'float32' : 'int32'); }

@@ -64,5 +64,7 @@ ENV.registerFlag('IS_TEST', () => false);
 ENV.registerFlag('HIP_DEVICE', () => 0);
 // false = run bias / activation as the reference's separate passes instead of the epilogue
 ENV.registerFlag('HIP_FUSE_EPILOGUE', () => true);
+// conv2d / depthwiseConv2D / batchMatMul wait for the add(bias) and relu | clip that may follow
+ENV.registerFlag('HIP_DEFER_EPILOGUE', () => true);
 
 module.exports = {Environment, ENV};
