@@ -103,7 +103,7 @@ def test_conv_smallk_uint8_filter_and_nan(tf, ref):
     (64, 7, 1024, 1024, "relu", "gemm_64x64_rowmajor_f32_tailk"),     # leftover tiles split on K
     (16, 32, 256, 512, "linear", "gemm_128x128_rowmajor_f32"),        # 8 wavefronts of 32x64
     (2, 30, 36, 30, "relu6", None),                                   # N % 4 != 0: guarded store
-    (1, 5, 1024, 24, "linear", None),                                 # few tiles: split along K
+    (1, 5, 4096, 24, "linear", None),                                 # few tiles: split along K
 ])
 def test_pointwise_conv_tiles(tf, n, h, cin, cout, act, want):
     print("pointwise", n, h, cin, cout, act, flush=True)
@@ -208,9 +208,11 @@ def test_rowstream_matmul_and_small_fallback(tf):
 
 @pytest.mark.parametrize("m,k,n,want_prefix", [
     (4096, 784, 1024, "gemm_128x128_rowmajor_f32_kb48"),
-    (256, 512, 256, "gemm_64x64_rowmajor_f32_kb48_splitk"),
-    (64, 1024, 1000, "gemm_64x64_rowmajor_f32_kb48_splitk"),
-    (4096, 1024, 10, "gemm_256x32_rowmajor_f32_kb48"),
+    (256, 512, 256, "gemm_16x16_kwaves_f32"),
+    (64, 1024, 1000, "gemm_16x16_kwaves_f32"),
+    (256, 4096, 256, "gemm_64x64_rowmajor_f32_kb48_splitk"),
+    (4096, 1024, 10, "gemm_16x16_kwaves_f32"),
+    (32768, 1024, 10, "gemm_256x32_rowmajor_f32_kb48"),
 ])
 def test_matmul_tiles_against_float64(tf, m, k, n, want_prefix):
     print("matmul", m, k, n, flush=True)
@@ -222,6 +224,75 @@ def test_matmul_tiles_against_float64(tf, m, k, n, want_prefix):
         kern = last_kernel(tf)
     assert kern.startswith(want_prefix), kern
     close(got, a.astype(np.float64) @ b.astype(np.float64), atol=1e-4)
+
+
+# ------------------------- few output tiles, K cut over the wavefronts of a workgroup ----
+@pytest.mark.parametrize("m,k,n,act,bias_kind,quant", [
+    (256, 512, 256, "linear", None, False),        # benchmark config 1
+    (196, 512, 512, "relu6", "column", False),     # a 14 x 14 pointwise layer of one image
+    (49, 1024, 1024, "relu", "column", True),      # 7 x 7, uint8 weights
+    (1, 1024, 1000, "linear", "column", False),    # a classifier on one image
+    (77, 332, 45, "prelu", "scalar", False),       # ragged rows and columns, K not a multiple of 16
+    (33, 132, 17, "relu", "full", True),           # the last group of k is cut, uint8
+    (500, 2048, 10, "relu6", "column", False),     # the longest contraction it takes
+    (16, 128, 16, "linear", None, False),          # one tile, the shortest contraction
+])
+def test_kwaves_products(tf, ref, m, k, n, act, bias_kind, quant):
+    """Products with few output tiles run as one launch whose workgroups cut K over their 8
+    wavefronts; against a float64 contraction, with every bias shape, prelu and uint8 weights."""
+    print("kwaves", m, k, n, act, bias_kind, quant, flush=True)
+    rng = np.random.default_rng(m * 7 + k * 3 + n)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    if quant:
+        q = rng.integers(0, 256, (k, n)).astype(np.uint8)
+        scale, mn = 0.004, -0.5
+        b = ref.dequantize(q, scale, mn)
+    else:
+        b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    bias = {None: None, "scalar": np.float32(0.3), "column": rng.standard_normal(n).astype(np.float32),
+            "full": rng.standard_normal((m, n)).astype(np.float32)}[bias_kind]
+    alpha = rng.uniform(0.1, 0.5, n).astype(np.float32) if act == "prelu" else None
+    with tf.tidy():
+        bt = tf.quantized_tensor(q, scale, mn) if quant else tf.tensor(b)
+        got = tf.fused.matmul(tf.tensor(a), bt, bias=None if bias is None else tf.tensor(bias),
+                              activation=act,
+                              prelu_activation_weights=None if alpha is None else tf.tensor(alpha)
+                              ).data_sync()
+        assert last_kernel(tf) == ("gemm_16x16_kwaves_u8" if quant else "gemm_16x16_kwaves_f32"), \
+            last_kernel(tf)
+    y = a.astype(np.float64) @ np.asarray(b, np.float64)
+    if bias is not None:
+        y = y + bias
+    y = np.where(y < 0, alpha * y, y) if act == "prelu" else act64(y, act)
+    close(got, y, atol=1e-4)
+    # NaN and infinity stay in their row / column; nothing leaks into the rows and columns that
+    # pad the last tile
+    a2 = a.copy()
+    a2[m // 2, k // 3] = np.nan
+    a2[0, k - 1] = np.inf
+    with tf.tidy():
+        got2 = tf.matmul(tf.tensor(a2), tf.tensor(np.asarray(b, np.float32))).data_sync()
+    bad = ~np.isfinite(got2)
+    rows = sorted(set(np.nonzero(bad.any(axis=1))[0].tolist()))
+    assert rows == sorted({m // 2, 0}), rows
+    assert np.isnan(got2[m // 2]).all()
+
+
+def test_kwaves_hands_over_what_it_does_not_take(tf):
+    """Batched products, transposed operands, long contractions and many tiles stay with the
+    tiled kernels; the same numbers come out of both paths."""
+    rng = np.random.default_rng(5)
+    for (batch, m, k, n, ta, tb) in [(2, 64, 512, 64, False, False), (1, 64, 512, 64, True, False),
+                                     (1, 64, 512, 64, False, True), (1, 64, 4096, 64, False, False),
+                                     (1, 2048, 512, 512, False, False), (1, 64, 126, 64, False, False)]:
+        a = rng.uniform(-1, 1, (batch, k, m) if ta else (batch, m, k)).astype(np.float32)
+        b = rng.uniform(-1, 1, (batch, n, k) if tb else (batch, k, n)).astype(np.float32)
+        with tf.tidy():
+            got = tf.matmul(tf.tensor(a), tf.tensor(b), ta, tb).data_sync()
+            assert "kwaves" not in last_kernel(tf), (batch, m, k, n, ta, tb, last_kernel(tf))
+        a64 = a.astype(np.float64).transpose(0, 2, 1) if ta else a.astype(np.float64)
+        b64 = b.astype(np.float64).transpose(0, 2, 1) if tb else b.astype(np.float64)
+        close(got, a64 @ b64, atol=1e-4)
 
 
 def test_implicit_gemm_3x3_tiles(tf):

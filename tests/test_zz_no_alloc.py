@@ -50,10 +50,11 @@ def _both(tf, a, b, bias=None, act=0, ta=0, tb=0):
 def test_noalloc_matches_matmul_on_calls_in_a_row(tf):
     rng = np.random.default_rng(70)
     seen_split = 0
-    # config 1 of the benchmark is cut along K (too few tiles for 256 CUs); then smaller and
-    # differently shaped products that reuse the same scratch bytes; then one that is not cut
-    for (m, k, n) in [(256, 512, 256), (128, 512, 64), (64, 2048, 64), (32, 300, 20),
-                      (256, 512, 256), (2048, 256, 2048)]:
+    # a product that is cut along K over workgroups (too few tiles for 256 CUs, a contraction
+    # too long for the single-launch kernel of small products); then smaller and differently
+    # shaped ones that reuse the same scratch bytes; then some that need no scratch memory
+    for (m, k, n) in [(128, 4096, 128), (128, 2304, 64), (64, 8192, 64), (32, 300, 20),
+                      (128, 4096, 128), (256, 512, 256), (2048, 256, 2048)]:
         print("noalloc matmul", m, k, n, flush=True)
         a = rng.uniform(-1, 1, (1, m, k)).astype(np.float32)
         b = rng.uniform(-1, 1, (1, k, n)).astype(np.float32)

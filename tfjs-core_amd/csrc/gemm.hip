@@ -1209,6 +1209,106 @@ __global__ __launch_bounds__(256, 2) void gemm_rowstream_kernel(const GemmArgs p
   }
 }
 
+// Small products with a long contraction (a [256, 512] x [512, 256] matMul, the 14 x 14 and
+// 7 x 7 pointwise layers of a single image, a classifier's last layer): too few tiles to fill
+// the machine, and cutting them along K over workgroups costs a second kernel that adds the
+// pieces.  Here the cut is made inside the workgroup: its 8 wavefronts each take an eighth of
+// K for the same 16 x 16 output tile (v_mfma_f32_16x16x4f32), load their operands straight from
+// memory into the registers the matrix instruction reads, and the 8 partial tiles meet in LDS,
+// where they are added in wavefront order (a fixed order: the result does not depend on
+// timing).  One launch, no partial sums in memory, 1 tile per (M / 16) x (N / 16) workgroups.
+// Lane l supplies row / column l % 16 and k = l / 16 of a group of 4; a lane loads 4
+// consecutive k of its row at once, so MFMA e of a group of 16 multiplies k = 16q + 4(l/16) + e.
+template <bool QUANT>
+__global__ __launch_bounds__(512) void gemm_kwaves_kernel(const GemmArgs p, int k_per) {
+  constexpr int WAVES = 8;
+  constexpr int G = 4;  // groups of 16 k per operand set (two sets: 128 k in flight)
+  __shared__ float part[WAVES][4][64];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, kq = lane >> 4;
+  const int m0 = ((int)blockIdx.x / p.tiles_n) * 16, n0 = ((int)blockIdx.x % p.tiles_n) * 16;
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B, p.b_bytes);
+  constexpr int B_EL = QUANT ? 1 : 4;
+  // rows beyond M and columns beyond N read as zeros: their offsets are out of range
+  const unsigned a_at = m0 + l16 < p.M ? (unsigned)(((m0 + l16) * p.lda + 4 * kq) * 4) : OOB_OFFSET;
+  const unsigned b_at = n0 + l16 < p.N ? (unsigned)((4 * kq * p.ldb + n0 + l16) * B_EL) : OOB_OFFSET;
+  const int k_begin = wave * k_per;
+  const int k_end = min(p.K, k_begin + k_per);
+  const int groups = k_end > k_begin ? (k_end - k_begin + 15) >> 4 : 0;
+
+  struct Operands {
+    f32x4 a[G];
+    float b[G][4];
+  };
+  // group q of this wavefront; k at or beyond K (whole groups of 4: K is a multiple of 4) is
+  // turned out of range
+  auto load = [&](int q0, Operands& o) {
+#pragma unroll
+    for (int u = 0; u < G; u++) {
+      if (q0 + u >= groups) break;
+      const int k0 = k_begin + 16 * (q0 + u);
+      const bool in = k0 + 4 * kq < k_end;
+      o.a[u] = buffer_load_f32x4(ra, in ? a_at + (unsigned)k0 * 4 : OOB_OFFSET);
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const unsigned at = in ? b_at + (unsigned)((k0 + e) * p.ldb) * B_EL : OOB_OFFSET;
+        if (QUANT) {
+          const unsigned w = __builtin_amdgcn_raw_buffer_load_b8(rb, (int)at, 0, 0);
+          o.b[u][e] = __builtin_bit_cast(float, w);
+        } else {
+          o.b[u][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb, (int)at, 0, 0));
+        }
+      }
+    }
+  };
+  f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  auto multiply = [&](int q0, const Operands& o) {
+#pragma unroll
+    for (int u = 0; u < G; u++) {
+      if (q0 + u >= groups) break;
+      const int k0 = k_begin + 16 * (q0 + u);
+      const bool in = k0 + 4 * kq < k_end;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        float b = o.b[u][e];
+        // (a byte that was not read is 0, which stands for the weight `min`: drop it)
+        if (QUANT) b = in && n0 + l16 < p.N ? dequant(__builtin_bit_cast(unsigned, b), p.qscale, p.qmin) : 0.f;
+        acc[e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[u][e], b, acc[e & 1], 0, 0, 0);
+      }
+    }
+  };
+  Operands o0, o1;
+  load(0, o0);
+  for (int q0 = 0; q0 < groups; q0 += 2 * G) {
+    load(q0 + G, o1);
+    multiply(q0, o0);
+    load(q0 + 2 * G, o0);
+    multiply(q0 + G, o1);
+  }
+#pragma unroll
+  for (int r = 0; r < 4; r++) part[wave][r][lane] = acc[0][r] + acc[1][r];
+  __syncthreads();
+  if (tid >= 256) return;
+  // accumulator register r of lane l is row 4 * (l / 16) + r, column l % 16 of the tile
+  const int r = tid >> 6;
+  const int row = m0 + 4 * kq + r, col = n0 + l16;
+  float v = part[0][r][lane];
+#pragma unroll
+  for (int w = 1; w < WAVES; w++) v += part[w][r][lane];
+  if (row >= p.M || col >= p.N) return;
+  const long long at = (long long)row * p.N + col;
+  if (p.bias_kind == TFHIP_BCAST_SCALAR) v += p.bias[0];
+  else if (p.bias_kind == TFHIP_BCAST_COLUMN) v += p.bias[col];
+  else if (p.bias_kind == TFHIP_BCAST_FULL) v += p.bias[at];
+  float al = 0.f;
+  if (p.prelu_kind == TFHIP_BCAST_SCALAR) al = p.prelu[0];
+  else if (p.prelu_kind == TFHIP_BCAST_COLUMN) al = p.prelu[col];
+  else if (p.prelu_kind == TFHIP_BCAST_FULL) al = p.prelu[at];
+  p.C[at] = activate(v, act_cfg(p.act), al);
+}
+
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
@@ -1483,6 +1583,38 @@ static int launch_rowstream(tfhip_ctx* ctx, const GemmArgs& p, int batch, int am
   return -1;
 }
 
+// The kernel that cuts K over the wavefronts of a workgroup, for the products it suits;
+// returns -1 for the others.  Measured on MI355X against the tiled kernels (which cut such
+// products along K over workgroups and add the pieces in a second kernel): [256, 512] x
+// [512, 256] 4.0 us against 9.8, [196, 512] x [512, 512] 5.1 against 10.0, [64, 1024] x
+// [1024, 1000] 6.5 against 10.7, [512, 512] x [512, 512] 8.8 against 13.8; it runs at about
+// 3 us + 14.5 us per 2^20 (tiles x K), its operands coming out of L2 without reuse, and meets
+// the tiled kernels there ([1024, 1024] x [1024, 256]: 17.6 against 17.9).  Beyond 256 k per
+// wavefront a workgroup waits for memory more than twice and loses ([128, 4096] x [4096, 128]:
+// 16.6 against 13.8).  With more than 4 tiles per CU the tiled kernels have enough whole tiles.
+static int launch_kwaves(tfhip_ctx* ctx, const GemmArgs& p, int batch, int amode, int bmode,
+                         long long a_bytes, long long b_bytes) {
+  if (batch != 1 || amode != A_ROWMAJOR || (bmode != B_ROWMAJOR && bmode != B_UINT8)) return -1;
+  if (!p.a_vec || p.ldb != p.N || (p.K & 3) || (p.lda & 3)) return -1;
+  if (a_bytes > 0x7fffffffLL || b_bytes > 0x7fffffffLL) return -1;
+  if (p.M < 1 || p.N < 1 || (long long)p.M * p.N > 0x7fffffffLL) return -1;
+  const long long tiles = ceil_div(p.M, 16) * ceil_div(p.N, 16);
+  if (p.K < 128 || p.K > 2048 || tiles > 4 * ctx->num_cus || tiles * p.K > (1LL << 20)) return -1;
+  GemmArgs q = p;
+  q.a_bytes = (unsigned)a_bytes;
+  q.b_bytes = (unsigned)b_bytes;
+  q.tiles_m = (int)ceil_div(p.M, 16);
+  q.tiles_n = (int)ceil_div(p.N, 16);
+  const int k_per = (int)ceil_div(ceil_div(p.K, 8), 16) * 16;
+  ctx->name_kernel("gemm_16x16_kwaves_%s", bmode == B_UINT8 ? "u8" : "f32");
+  if (bmode == B_UINT8)
+    tfhip::launch(ctx, gemm_kwaves_kernel<true>, dim3((unsigned)tiles), dim3(512), 0, q, k_per);
+  else
+    tfhip::launch(ctx, gemm_kwaves_kernel<false>, dim3((unsigned)tiles), dim3(512), 0, q, k_per);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
 static int launch_gemm(tfhip_ctx* ctx, GemmArgs& p, int batch, int amode, int bmode,
                        bool kblocked) {
   {
@@ -1505,6 +1637,10 @@ static int launch_gemm(tfhip_ctx* ctx, GemmArgs& p, int batch, int amode, int bm
   // (an empty contraction has no readable operand bytes: keep it on the guarded path)
   const bool fast = p.a_vec && p.b_vec && p.K > 0 && p.M > 0 && p.N > 0 && a_bytes <= lim &&
                     b_bytes <= lim;
+  {
+    const int rc = launch_kwaves(ctx, p, batch, amode, bmode, a_bytes, b_bytes);
+    if (rc >= 0) return rc;
+  }
   p.a_bytes = fast ? (unsigned)a_bytes : 0;
   p.b_bytes = fast ? (unsigned)b_bytes : 0;
 #define TFHIP_CASE(AM, BM_, KB)                                \
