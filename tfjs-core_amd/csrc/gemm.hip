@@ -817,14 +817,99 @@ __global__ void splitk_finish_kernel(const GemmArgs p, int BM, int BN, int first
 // MFMA operand of 32 output pixels straight out of LDS.  The whole filter lives in
 // registers (k = 8q + 4*(lane/32) + e of MFMA group q, the same summation-order permutation
 // as above).  HBM traffic is the input once (rows shared by neighbouring output rows come out
-// of L2) plus the output once.
-template <int TN, bool QUANT>
-__global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int row_floats,
-                                                          int n_rows) {
-  extern __shared__ __attribute__((aligned(16))) float rows[];  // [KH][row_floats]
+// of L2) plus the output once.  SPLIT (the staged rows of one output row are at most 2048
+// floats): two more wavefronts do the loading, into two LDS buffers of SPLIT_BUF floats.
+constexpr int SPLIT_BUF = 2048 + 16;
+template <int TN, bool QUANT, bool SPLIT>
+__global__ __launch_bounds__(SPLIT ? 384 : 256) void conv_smallk_kernel(const GemmArgs p,
+                                                                       int row_floats, int n_rows) {
+  extern __shared__ __attribute__((aligned(16))) float rows[];  // [KH][row_floats] (+ 1), x 2 if SPLIT
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, g = lane >> 5;
+  const int row_in = p.W * p.Cin;
+  const int stage_n = p.KH * row_floats;
+  // A grid that is a multiple of 8 cuts the output rows into one run per XCD (workgroup b runs
+  // on XCD b % 8): neighbouring output rows, which share input rows, then meet in one L2, and
+  // the kernel that reads the result cuts it the same way.
+  int row_first = blockIdx.x, row_step = gridDim.x, row_end = n_rows;
+  if ((gridDim.x & 7) == 0) {
+    const int xcd = (int)blockIdx.x & 7, per = n_rows >> 3, rem = n_rows & 7;
+    const int run0 = xcd * per + (xcd < rem ? xcd : rem);
+    row_end = run0 + per + (xcd < rem ? 1 : 0);
+    row_first = run0 + ((int)blockIdx.x >> 3);
+    row_step = (int)gridDim.x >> 3;
+  }
+  // (image, output row) of a row of this workgroup, advanced by additions: a division per row
+  // would run on the vector ALU
+  const int step_n = row_step / p.OH, step_oh = row_step - step_n * p.OH;
+  auto advance = [&](int& n, int& oh) {
+    n += step_n;
+    oh += step_oh;
+    if (oh >= p.OH) {
+      oh -= p.OH;
+      n++;
+    }
+  };
+  int n = row_first / p.OH, oh = row_first - n * p.OH;
+
+  // rows this workgroup takes
+  const int count = row_first < row_end ? (row_end - row_first + row_step - 1) / row_step : 0;
+  if constexpr (SPLIT) {
+    // (the zero slots of both buffers, which no loader writes)
+    if (tid == 0) rows[p.KH * row_floats] = rows[SPLIT_BUF + p.KH * row_floats] = 0.f;
+    if (wave >= 4) {
+      const int ptid = tid - 256;
+      // Per lane and staged element, fixed for the lifetime of the workgroup: the byte offset of
+      // (kh, column) relative to the first input row of an output row, or a value that stays out
+      // of range whatever row offset is added (elements past the block, columns in the padding).
+      // The rows above and below the image fall out of the descriptor's range by themselves: a
+      // negative offset wraps to a huge one.  So a staged element costs one add and one load.
+      unsigned ld_const[16];
+#pragma unroll
+      for (int u = 0; u < 16; u++) {
+        const int i = ptid + u * 128;
+        const int kh = i / row_floats;
+        const int e = i - kh * row_floats - p.pl * p.Cin;
+        const bool ok = i < stage_n && (unsigned)e < (unsigned)row_in;
+        ld_const[u] = ok ? (unsigned)((kh * p.dh * row_in + e) * 4) : OOB_OFFSET;
+      }
+      const unsigned img_bytes = (unsigned)(p.H * row_in) * 4u;
+      int ld_n = n, ld_oh = oh;  // the row whose loads are issued next
+      auto stage_load = [&](float (&v)[16]) {
+        const __amdgpu_buffer_rsrc_t rimg = make_rsrc(p.A + (long long)ld_n * p.H * row_in, img_bytes);
+        const unsigned first = (unsigned)((ld_oh * p.sh - p.pt) * row_in * 4);  // may be "negative"
+#pragma unroll
+        for (int u = 0; u < 16; u++)
+          v[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                               rimg, (int)(ld_const[u] + first), 0, 0));
+        advance(ld_n, ld_oh);
+      };
+      auto put = [&](const float (&v)[16], float* rb) {
+#pragma unroll
+        for (int u = 0; u < 16; u++)
+          if (ptid + u * 128 < stage_n) rb[ptid + u * 128] = v[u];
+      };
+      float v0[16], v1[16];
+      if (count > 0) stage_load(v0);
+      if (count > 1) stage_load(v1);
+      if (count > 0) put(v0, rows);
+      if (count > 2) stage_load(v0);
+      __syncthreads();
+      for (int it = 0; it < count; it += 2) {
+        // while row `it` is multiplied out of buffer 0
+        if (it + 1 < count) put(v1, rows + SPLIT_BUF);
+        if (it + 3 < count) stage_load(v1);
+        __syncthreads();
+        if (it + 1 >= count) break;
+        // while row `it + 1` is multiplied out of buffer 1
+        if (it + 2 < count) put(v0, rows);
+        if (it + 4 < count) stage_load(v0);
+        __syncthreads();
+      }
+      return;
+    }
+  }
   // this lane's 16 contraction indices k = 8q + 4g + e: LDS offset of (kh, kw, c), or -1 past
   // K, and row k of the filter.  (kh, kw, c) is counted up with k, which keeps the walk in
   // scalar registers; the filter loads are unconditional (clamped index) so that they are
@@ -876,7 +961,7 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
   // of (kh, kw, c) at its pixel, or a slot behind the staged rows that holds 0 for k past K.
   // Every output row has the same strips, so the first strip's addresses are computed once.
   const int zero_slot = p.KH * row_floats;
-  if (tid == 0) rows[zero_slot] = 0.f;
+  if (!SPLIT && tid == 0) rows[zero_slot] = 0.f;
   // (a copy of a lane constant that the optimiser cannot see through: the address arithmetic of
   // the rarely taken paths below then stays inside them instead of being hoisted out of the row
   // loop into registers that every row pays for)
@@ -904,95 +989,9 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
         addr[q][e] = a_first[q][e] == zero_slot ? zero_slot : a_first[q][e] + shift;
   };
 
-  // Staging plan of this lane: elements i = tid + 256u of the [KH][row_floats] block, as
-  // (kh, offset in the input row); fixed for the lifetime of the workgroup.  A block of up to
-  // 2048 floats is one pass, and then the next output row's loads are issued before the
-  // current row is computed, so that their latency is hidden behind the matrix-core work.
-  const int row_in = p.W * p.Cin;
-  const int stage_n = p.KH * row_floats;
-  // (one pass also needs 32-bit byte offsets inside one image)
-  const bool one_pass = stage_n <= 256 * 8 && (long long)p.H * row_in * 4 < (1LL << 30);
-  // Per lane and staged element, fixed for the lifetime of the workgroup: the byte offset of
-  // (kh, column) relative to the first input row of an output row, or a value that stays out
-  // of range whatever row offset is added (elements past the block, columns in the padding).
-  // The rows above and below the image fall out of the descriptor's range by themselves: a
-  // negative offset wraps to a huge one.  So a staged element costs one add and one load.
-  unsigned ld_const[8];
-#pragma unroll
-  for (int u = 0; u < 8; u++) {
-    const int i = tid + u * 256;
-    const int kh = i / row_floats;
-    const int e = i - kh * row_floats - p.pl * p.Cin;
-    const bool ok = i < stage_n && (unsigned)e < (unsigned)row_in;
-    ld_const[u] = ok ? (unsigned)((kh * p.dh * row_in + e) * 4) : OOB_OFFSET;
-  }
-  const unsigned img_bytes = (unsigned)(p.H * row_in) * 4u;
-  auto stage_load = [&](int n, int oh, float (&v)[8]) {
-    const __amdgpu_buffer_rsrc_t rimg = make_rsrc(p.A + (long long)n * p.H * row_in, img_bytes);
-    const unsigned first = (unsigned)((oh * p.sh - p.pt) * row_in * 4);  // may be "negative"
-#pragma unroll
-    for (int u = 0; u < 8; u++)
-      v[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                           rimg, (int)(ld_const[u] + first), 0, 0));
-  };
-  // A grid that is a multiple of 8 cuts the output rows into one run per XCD (workgroup b runs
-  // on XCD b % 8): neighbouring output rows, which share input rows, then meet in one L2, and
-  // the kernel that reads the result cuts it the same way.
-  int row_first = blockIdx.x, row_step = gridDim.x, row_end = n_rows;
-  if ((gridDim.x & 7) == 0) {
-    const int xcd = (int)blockIdx.x & 7, per = n_rows >> 3, rem = n_rows & 7;
-    const int run0 = xcd * per + (xcd < rem ? xcd : rem);
-    row_end = run0 + per + (xcd < rem ? 1 : 0);
-    row_first = run0 + ((int)blockIdx.x >> 3);
-    row_step = (int)gridDim.x >> 3;
-  }
-  // (image, output row) of the current row and of the next one of this workgroup, advanced by
-  // additions: a division per row would run on the vector ALU
-  const int step_n = row_step / p.OH, step_oh = row_step - step_n * p.OH;
-  auto advance = [&](int& n, int& oh) {
-    n += step_n;
-    oh += step_oh;
-    if (oh >= p.OH) {
-      oh -= p.OH;
-      n++;
-    }
-  };
-  int n = row_first / p.OH, oh = row_first - n * p.OH;
-  int n_next = n, oh_next = oh;
-  advance(n_next, oh_next);
-  float v[8];
-  if (one_pass && row_first < row_end) stage_load(n, oh, v);
-  for (int row = row_first; row < row_end;
-       row += row_step, n = n_next, oh = oh_next, advance(n_next, oh_next)) {
-    __syncthreads();  // the previous row's readers are done
-    if (one_pass) {
-#pragma unroll
-      for (int u = 0; u < 8; u++)
-        if (tid + u * 256 < stage_n) rows[tid + u * 256] = v[u];
-    } else {
-      for (int i0 = opaque(tid); i0 < stage_n; i0 += 256 * 8) {
-        float t[8];
-#pragma unroll
-        for (int u = 0; u < 8; u++) {
-          const int i = i0 + u * 256;
-          const int kh = i / row_floats, r = i - kh * row_floats;
-          const int ih = oh * p.sh - p.pt + kh * p.dh;
-          const int e = r - p.pl * p.Cin;
-          const bool ok = i < stage_n && (unsigned)ih < (unsigned)p.H && (unsigned)e < (unsigned)row_in;
-          const long long at = ok ? ((long long)n * p.H + ih) * row_in + e : 0;
-          const float x = p.A[at];
-          t[u] = ok ? x : 0.f;
-        }
-#pragma unroll
-        for (int u = 0; u < 8; u++) {
-          const int i = i0 + u * 256;
-          if (i < stage_n) rows[i] = t[u];
-        }
-      }
-    }
-    __syncthreads();
-    if (one_pass && row + row_step < row_end) stage_load(n_next, oh_next, v);
-
+  // One output row out of the staged input rows `rb`: each wavefront multiplies strips of 32
+  // pixels and stores them.
+  auto compute_row = [&](int n, int oh, const float* rb) {
     const long long out_at = (((long long)n * p.OH + oh) * p.OW) * p.N;  // workgroup-uniform
     float* __restrict__ crow = p.C + out_at;
     const ActCfg act = act_cfg(p.act);
@@ -1013,7 +1012,7 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
         for (int q = 0; q < 4; q++) {
           float a[4];
 #pragma unroll
-          for (int e = 0; e < 4; e++) a[e] = rows[addr[q][e]];
+          for (int e = 0; e < 4; e++) a[e] = rb[addr[q][e]];
 #pragma unroll
           for (int e = 0; e < 4; e++)
 #pragma unroll
@@ -1066,6 +1065,49 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const GemmArgs p, int 
           }
         }
       }
+    }
+  };
+
+  if constexpr (SPLIT) {
+    // Wavefronts 0..3 multiply and store, wavefronts 4 and 5 only load: a wavefront that does
+    // both finds the acknowledgements of its stores in front of its loads' data (they share one
+    // counter) and waits a trip to memory per row.  The loaders keep two rows in flight and
+    // fill the LDS buffer that is not being read; one barrier per row hands the buffers over.
+    __syncthreads();
+    for (int it = 0; it < count; it += 2) {
+      compute_row(n, oh, rows);
+      advance(n, oh);
+      __syncthreads();
+      if (it + 1 >= count) break;
+      compute_row(n, oh, rows + SPLIT_BUF);
+      advance(n, oh);
+      __syncthreads();
+    }
+  } else {
+    // Input rows of any length, staged in passes by the wavefronts that also multiply.
+    for (int row = row_first; row < row_end; row += row_step, advance(n, oh)) {
+      __syncthreads();  // the previous row's readers are done
+      for (int i0 = opaque(tid); i0 < stage_n; i0 += 256 * 8) {
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const int i = i0 + u * 256;
+          const int kh = i / row_floats, r = i - kh * row_floats;
+          const int ih = oh * p.sh - p.pt + kh * p.dh;
+          const int e = r - p.pl * p.Cin;
+          const bool ok = i < stage_n && (unsigned)ih < (unsigned)p.H && (unsigned)e < (unsigned)row_in;
+          const long long at = ok ? ((long long)n * p.H + ih) * row_in + e : 0;
+          const float x = p.A[at];
+          t[u] = ok ? x : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const int i = i0 + u * 256;
+          if (i < stage_n) rows[i] = t[u];
+        }
+      }
+      __syncthreads();
+      compute_row(n, oh, rows);
     }
   }
 }
@@ -1889,17 +1931,23 @@ extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t o
     const long long span = (long long)(ci->out_w - 1) * ci->stride_w +
                            (long long)(ci->filter_w - 1) * ci->dilation_w + 1;
     const long long row_floats = span * ci->in_c;
-    const long long lds = (row_floats * ci->filter_h + 1) * (long long)sizeof(float);  // + the zero slot
+    const long long stage_n = row_floats * ci->filter_h;
+    // loader wavefronts of their own when a row's input fits their registers (and 32-bit byte
+    // offsets reach every element of an image)
+    const bool split = stage_n <= 2048 && (int64_t)ci->in_h * ci->in_w * ci->in_c * 4 < (1LL << 30);
+    const long long lds = split ? 2LL * SPLIT_BUF * (long long)sizeof(float)
+                                : (stage_n + 1) * (long long)sizeof(float);  // + the zero slot
     if (lds <= 64 * 1024) {
       const int n_rows = ci->batch * ci->out_h;
+      const unsigned threads = split ? 384 : 256;
       // one workgroup per resident slot: each walks its share of the output rows
       auto launch = [&](auto kernel, const char* name) {
         // resident workgroups per CU for this kernel and LDS size, asked once (the query
         // costs microseconds, which a batch-1 step would pay on every call)
-        static std::map<size_t, int> resident;
-        int& per_cu = resident[(size_t)lds];
+        static std::map<std::pair<const void*, size_t>, int> resident;
+        int& per_cu = resident[{reinterpret_cast<const void*>(kernel), (size_t)lds}];
         if (per_cu == 0 &&
-            (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, (size_t)lds) !=
+            (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, (int)threads, (size_t)lds) !=
                  hipSuccess || per_cu < 1)) {
           (void)hipGetLastError();
           per_cu = 1;
@@ -1909,15 +1957,25 @@ extern "C" int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t o
         if (grid >= 64) grid &= ~7u;  // a multiple of the XCD count: one run of rows per XCD
         ctx->name_kernel("%s_%s", name, quant ? "u8" : "f32");
         ctx->sweep = 1;  // this kernel walks the rows forward: its consumer should start at the end
-        tfhip::launch(ctx, kernel, dim3(grid), dim3(256), (size_t)lds, p,
+        tfhip::launch(ctx, kernel, dim3(grid), dim3(threads), (size_t)lds, p,
                            (int)row_floats, n_rows);
       };
       if (p.N <= 32) {
-        if (quant) launch(conv_smallk_kernel<1, true>, "conv_smallk_n32");
-        else launch(conv_smallk_kernel<1, false>, "conv_smallk_n32");
+        if (split) {
+          if (quant) launch(conv_smallk_kernel<1, true, true>, "conv_smallk_n32");
+          else launch(conv_smallk_kernel<1, false, true>, "conv_smallk_n32");
+        } else {
+          if (quant) launch(conv_smallk_kernel<1, true, false>, "conv_smallk_n32_long");
+          else launch(conv_smallk_kernel<1, false, false>, "conv_smallk_n32_long");
+        }
       } else {
-        if (quant) launch(conv_smallk_kernel<2, true>, "conv_smallk_n64");
-        else launch(conv_smallk_kernel<2, false>, "conv_smallk_n64");
+        if (split) {
+          if (quant) launch(conv_smallk_kernel<2, true, true>, "conv_smallk_n64");
+          else launch(conv_smallk_kernel<2, false, true>, "conv_smallk_n64");
+        } else {
+          if (quant) launch(conv_smallk_kernel<2, true, false>, "conv_smallk_n64_long");
+          else launch(conv_smallk_kernel<2, false, false>, "conv_smallk_n64_long");
+        }
       }
       TFHIP_LAUNCH_CHECK(ctx);
       return TFHIP_OK;
