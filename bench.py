@@ -327,6 +327,10 @@ def main():
     ap.add_argument("--loop-pointwise", type=int, default=0, metavar="REPS",
                     help="only launch the 512->512 pointwise layer of the network (pw7: "
                          "[64,14,14,512] x [512,512], bias + relu6) REPS times, for counter runs")
+    ap.add_argument("--loop-depthwise", type=int, default=0, metavar="REPS",
+                    help="only launch the 56 x 56 x 128 stride-1 depthwise layer of the network (dw3: "
+                         "[64,56,56,128], 3x3, bias + relu6) REPS times over four inputs in turn "
+                         "(0.4 GB: every launch reads from HBM), for counter runs")
     ap.add_argument("--calibrate-counters", action="store_true",
                     help="only launch a streaming kernel of known size (relu over 256 MiB: reads "
                          "256 MiB, writes 256 MiB) three times, to scale FETCH_SIZE / WRITE_SIZE")
@@ -362,6 +366,21 @@ def main():
         print(json.dumps({"kernel": be.lib.tfhip_last_kernel(be.ctx).decode(),
                           "launches": args.loop_pointwise,
                           "flops_per_launch": 2.0 * args.batch * 196 * 512 * 512}))
+        return
+
+    if args.loop_depthwise > 0:
+        rng = np.random.default_rng(1)
+        xs = [tf.tensor(rng.uniform(0, 1, (args.batch, 56, 56, 128)).astype(np.float32))
+              for _ in range(4)]
+        wt = tf.tensor((rng.standard_normal((3, 3, 128, 1)) * 0.3).astype(np.float32))
+        bias = tf.tensor(np.zeros(128, np.float32))
+        for i in range(args.loop_depthwise):
+            tf.dispose(tf.fused.depthwise_conv2d(xs[i % 4], wt, 1, "same", bias=bias,
+                                                 activation="relu6"))
+        be.sync()
+        print(json.dumps({"kernel": be.lib.tfhip_last_kernel(be.ctx).decode(),
+                          "launches": args.loop_depthwise,
+                          "bytes_per_launch": 4.0 * (2 * args.batch * 56 * 56 * 128 + 9 * 128 + 128)}))
         return
 
     params = mobilenet.make_params(seed=0)

@@ -99,9 +99,10 @@ def test_conv_smallk_uint8_filter_and_nan(tf, ref):
 # ------------------------------------------------------- GEMM tile shapes ----
 @pytest.mark.parametrize("n,h,cin,cout,act,want", [
     (4, 28, 128, 256, "relu6", "gemm_64x64_rowmajor_f32"),            # staged 16-byte store
-    (64, 7, 512, 1024, "relu6", "gemm_64x128_rowmajor_f32"),          # 8 wavefronts of 32x32
-    (64, 7, 1024, 1024, "relu", "gemm_64x64_rowmajor_f32_tailk"),     # leftover tiles split on K
-    (16, 32, 256, 512, "linear", "gemm_128x128_rowmajor_f32"),        # 8 wavefronts of 32x64
+    (64, 7, 512, 1024, "relu6", "gemm_64x64_rowmajor_f32_tail16"),    # leftover tiles in 16 x 16 pieces
+    (64, 7, 1024, 1024, "relu", "gemm_64x64_rowmajor_f32_tail16"),
+    (64, 14, 512, 512, "relu6", "gemm_64x64_rowmajor_f32_tail16"),    # pw7..pw11 of a batch-64 MobileNet
+    (16, 32, 256, 512, "linear", "gemm_64x64_rowmajor_f32"),
     (2, 30, 36, 30, "relu6", None),                                   # N % 4 != 0: guarded store
     (1, 5, 4096, 24, "linear", None),                                 # few tiles: split along K
 ])
@@ -133,6 +134,8 @@ def test_pointwise_conv_tiles(tf, n, h, cin, cout, act, want):
     (5, 200, 201, 32, 64, "relu", True, True, "gemm_rowstream_k32xn64_u8"),
     (2, 320, 331, 32, 64, "linear", True, True, "gemm_rowstream_k32xn64_u8"),
     (1, 449, 449, 64, 128, "relu6", True, False, "gemm_64x64_rowmajor_f32"),    # stays tiled
+    (64, 14, 14, 512, 512, "relu6", True, True, "gemm_64x64_rowmajor_u8_tail16"),  # uint8 in the 16 x 16 pieces
+    (64, 14, 14, 512, 512, "prelu", True, False, "gemm_64x64_rowmajor_f32_tail16"),
 ])
 def test_rowstream_products(tf, ref, n, h, w_, cin, cout, act, bias, quant, want):
     """Pointwise convolutions with enough pixels for the row-streaming kernel (B resident in
@@ -207,7 +210,9 @@ def test_rowstream_matmul_and_small_fallback(tf):
 
 
 @pytest.mark.parametrize("m,k,n,want_prefix", [
-    (4096, 784, 1024, "gemm_128x128_rowmajor_f32_kb48"),
+    (4096, 784, 1024, "gemm_64x64_rowmajor_f32_kb48"),
+    (4096, 3072, 4096, "gemm_128x128_rowmajor_f32_kb48"),               # 8 wavefronts of 32x64
+    (3137, 1024, 1000, "gemm_64x64_rowmajor_f32_kb48_tail16"),          # ragged rows and columns
     (256, 512, 256, "gemm_16x16_kwaves_f32"),
     (64, 1024, 1000, "gemm_16x16_kwaves_f32"),
     (256, 4096, 256, "gemm_64x64_rowmajor_f32_kb48_splitk"),
@@ -299,18 +304,24 @@ def test_implicit_gemm_3x3_tiles(tf):
     """3x3 convolutions through the im2col loaders at sizes that take the 64x64 and wider
     tiles, against float64 on sampled output positions."""
     rng = np.random.default_rng(9)
-    for (n, h, cin, cout) in ((8, 56, 64, 128), (2, 28, 32, 48), (1, 14, 256, 512)):
+    seen = set()
+    for (n, h, cin, cout) in ((8, 56, 64, 128), (2, 28, 32, 48), (1, 14, 256, 512),
+                              (64, 14, 128, 512)):
         x = rng.uniform(-1, 1, (n, h, h, cin)).astype(np.float32)
         w = (rng.standard_normal((3, 3, cin, cout)) * np.sqrt(2.0 / (9 * cin))).astype(np.float32)
         with tf.tidy():
             got = tf.conv2d(tf.tensor(x), tf.tensor(w), 1, "same").data_sync()
             assert "im2col" in last_kernel(tf)
+            seen.add(last_kernel(tf))
         xp = np.pad(x, ((0, 0), (1, 1), (1, 1), (0, 0))).astype(np.float64)
         w64 = w.astype(np.float64)
         for _ in range(200):
             b, i, j = rng.integers(n), rng.integers(h), rng.integers(h)
             want = np.einsum("abc,abco->o", xp[b, i:i + 3, j:j + 3, :], w64)
             close(got[b, i, j], want)
+    # (the last shape leaves tiles over after whole rounds: they are split along K over
+    # workgroups and finished by a second kernel)
+    assert any(k.endswith("_tailk") for k in seen), seen
 
 
 # ------------------------------------- row lengths that are not multiples of 4 ----

@@ -51,6 +51,9 @@ struct GemmArgs {
   // schedule (see work_item)
   int tiles_m, tiles_n, k_tiles, full_tiles, tail_tiles, splits, kt_per;
   float* partials;  // [tail_tiles * splits][BM * BN] partial tiles when splits > 1
+  // minis > 0: the tail tiles are not split along K over workgroups but cut into `minis` tiles
+  // of 16 x 16 each, one per workgroup, whose wavefronts take mini_k_per of K each (kwaves_tile)
+  int minis, mini_k_per;
   unsigned a_bytes, b_bytes;  // per-batch byte extents of A and B (buffer-load range check)
   int reverse;  // walk the tiles / row blocks of every XCD's run from the end
 };
@@ -86,6 +89,111 @@ __device__ __forceinline__ WorkItem work_item(const GemmArgs& p, int block) {
     if (p.splits > 1) w.slot = h;
   }
   return w;
+}
+
+// Small products with a long contraction (a [256, 512] x [512, 256] matMul, the 14 x 14 and
+// 7 x 7 pointwise layers of a single image, a classifier's last layer): too few tiles to fill
+// the machine, and cutting them along K over workgroups costs a second kernel that adds the
+// pieces.  Here the cut is made inside the workgroup: its WAVES wavefronts each take a share of
+// K for the same 16 x 16 output tile (v_mfma_f32_16x16x4f32), load their operands straight from
+// memory into the registers the matrix instruction reads, and the partial tiles meet in LDS,
+// where they are added in wavefront order (a fixed order: the result does not depend on
+// timing).  One launch, no partial sums in memory.  Lane l supplies row / column l % 16 and
+// k = l / 16 of a group of 4; a lane loads 4 consecutive k of its row at once, so MFMA e of a
+// group of 16 multiplies k = 16q + 4(l/16) + e.  G groups of 16 k make one set of operand
+// registers; two sets are in flight.  `part` is WAVES x 4 x 64 floats of LDS.
+template <int WAVES, int G, bool QUANT>
+__device__ __forceinline__ void kwaves_tile(const GemmArgs& p, int m0, int n0, int k_per,
+                                            float* part, int tid) {
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, kq = lane >> 4;
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B, p.b_bytes);
+  constexpr int B_EL = QUANT ? 1 : 4;
+  // rows beyond M and columns beyond N read as zeros: their offsets are out of range
+  const unsigned a_at = m0 + l16 < p.M ? (unsigned)(((m0 + l16) * p.lda + 4 * kq) * 4) : OOB_OFFSET;
+  const unsigned b_at = n0 + l16 < p.N ? (unsigned)((4 * kq * p.ldb + n0 + l16) * B_EL) : OOB_OFFSET;
+  const int k_begin = wave * k_per;
+  const int k_end = min(p.K, k_begin + k_per);
+  const int groups = k_end > k_begin ? (k_end - k_begin + 15) >> 4 : 0;
+
+  struct Operands {
+    f32x4 a[G];
+    float b[G][4];
+  };
+  // group q of this wavefront; k at or beyond K (whole groups of 4: K is a multiple of 4) is
+  // turned out of range
+  auto load = [&](int q0, Operands& o) {
+#pragma unroll
+    for (int u = 0; u < G; u++) {
+      if (q0 + u >= groups) break;
+      const int k0 = k_begin + 16 * (q0 + u);
+      const bool in = k0 + 4 * kq < k_end;
+      o.a[u] = buffer_load_f32x4(ra, in ? a_at + (unsigned)k0 * 4 : OOB_OFFSET);
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const unsigned at = in ? b_at + (unsigned)((k0 + e) * p.ldb) * B_EL : OOB_OFFSET;
+        if (QUANT) {
+          const unsigned w = __builtin_amdgcn_raw_buffer_load_b8(rb, (int)at, 0, 0);
+          o.b[u][e] = __builtin_bit_cast(float, w);
+        } else {
+          o.b[u][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb, (int)at, 0, 0));
+        }
+      }
+    }
+  };
+  f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  auto multiply = [&](int q0, const Operands& o) {
+#pragma unroll
+    for (int u = 0; u < G; u++) {
+      if (q0 + u >= groups) break;
+      const int k0 = k_begin + 16 * (q0 + u);
+      const bool in = k0 + 4 * kq < k_end;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        float b = o.b[u][e];
+        // (a byte that was not read is 0, which stands for the weight `min`: drop it)
+        if (QUANT) b = in && n0 + l16 < p.N ? dequant(__builtin_bit_cast(unsigned, b), p.qscale, p.qmin) : 0.f;
+        acc[e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[u][e], b, acc[e & 1], 0, 0, 0);
+      }
+    }
+  };
+  Operands o0, o1;
+  load(0, o0);
+  for (int q0 = 0; q0 < groups; q0 += 2 * G) {
+    load(q0 + G, o1);
+    multiply(q0, o0);
+    load(q0 + 2 * G, o0);
+    multiply(q0 + G, o1);
+  }
+#pragma unroll
+  for (int r = 0; r < 4; r++) part[(wave * 4 + r) * 64 + lane] = acc[0][r] + acc[1][r];
+  __syncthreads();
+  if (tid >= 256) return;
+  // accumulator register r of lane l is row 4 * (l / 16) + r, column l % 16 of the tile
+  const int r = tid >> 6;
+  const int row = m0 + 4 * kq + r, col = n0 + l16;
+  float v = part[r * 64 + lane];
+#pragma unroll
+  for (int w = 1; w < WAVES; w++) v += part[(w * 4 + r) * 64 + lane];
+  if (row >= p.M || col >= p.N) return;
+  const long long at = (long long)row * p.N + col;
+  if (p.bias_kind == TFHIP_BCAST_SCALAR) v += p.bias[0];
+  else if (p.bias_kind == TFHIP_BCAST_COLUMN) v += p.bias[col];
+  else if (p.bias_kind == TFHIP_BCAST_FULL) v += p.bias[at];
+  float al = 0.f;
+  if (p.prelu_kind == TFHIP_BCAST_SCALAR) al = p.prelu[0];
+  else if (p.prelu_kind == TFHIP_BCAST_COLUMN) al = p.prelu[col];
+  else if (p.prelu_kind == TFHIP_BCAST_FULL) al = p.prelu[at];
+  p.C[at] = activate(v, act_cfg(p.act), al);
+}
+
+// One 16 x 16 tile per workgroup of 8 wavefronts: (M / 16) x (N / 16) workgroups.
+template <bool QUANT>
+__global__ __launch_bounds__(512) void gemm_kwaves_kernel(const GemmArgs p, int k_per) {
+  __shared__ float part[8 * 4 * 64];
+  kwaves_tile<8, 4, QUANT>(p, ((int)blockIdx.x / p.tiles_n) * 16, ((int)blockIdx.x % p.tiles_n) * 16,
+                           k_per, part, threadIdx.x);
 }
 
 template <int WAVES_M, int WAVES_N, int TM, int TN, int AMODE, int BMODE, bool KBLOCKED, bool FAST>
@@ -474,6 +582,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     }
   };
 
+  if constexpr (FAST && AMODE == A_ROWMAJOR && BMODE != B_TRANSPOSED) {
+    // a 16 x 16 piece of a tail tile (the planner sets minis only for unbatched products)
+    if (p.minis > 0 && (int)blockIdx.x >= p.full_tiles) {
+      const int h = (int)blockIdx.x - p.full_tiles;
+      const int t = p.full_tiles + h / p.minis, mini = h % p.minis;
+      const int m0 = (t / p.tiles_n) * BM + (mini / (BN / 16)) * 16;
+      const int n0 = (t % p.tiles_n) * BN + (mini % (BN / 16)) * 16;
+      if (t >= p.tiles_m * p.tiles_n || m0 >= p.M || n0 >= p.N) return;
+      kwaves_tile<WAVES_M * WAVES_N, 2, BMODE == B_UINT8>(p, m0, n0, p.mini_k_per, lds, tid);
+      return;
+    }
+  }
   Loader L;
   const WorkItem cur = work_item(p, blockIdx.x);
   if (cur.tile < 0) return;
@@ -1251,106 +1371,6 @@ __global__ __launch_bounds__(256, 2) void gemm_rowstream_kernel(const GemmArgs p
   }
 }
 
-// Small products with a long contraction (a [256, 512] x [512, 256] matMul, the 14 x 14 and
-// 7 x 7 pointwise layers of a single image, a classifier's last layer): too few tiles to fill
-// the machine, and cutting them along K over workgroups costs a second kernel that adds the
-// pieces.  Here the cut is made inside the workgroup: its 8 wavefronts each take an eighth of
-// K for the same 16 x 16 output tile (v_mfma_f32_16x16x4f32), load their operands straight from
-// memory into the registers the matrix instruction reads, and the 8 partial tiles meet in LDS,
-// where they are added in wavefront order (a fixed order: the result does not depend on
-// timing).  One launch, no partial sums in memory, 1 tile per (M / 16) x (N / 16) workgroups.
-// Lane l supplies row / column l % 16 and k = l / 16 of a group of 4; a lane loads 4
-// consecutive k of its row at once, so MFMA e of a group of 16 multiplies k = 16q + 4(l/16) + e.
-template <bool QUANT>
-__global__ __launch_bounds__(512) void gemm_kwaves_kernel(const GemmArgs p, int k_per) {
-  constexpr int WAVES = 8;
-  constexpr int G = 4;  // groups of 16 k per operand set (two sets: 128 k in flight)
-  __shared__ float part[WAVES][4][64];
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l16 = lane & 15, kq = lane >> 4;
-  const int m0 = ((int)blockIdx.x / p.tiles_n) * 16, n0 = ((int)blockIdx.x % p.tiles_n) * 16;
-  const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A, p.a_bytes);
-  const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B, p.b_bytes);
-  constexpr int B_EL = QUANT ? 1 : 4;
-  // rows beyond M and columns beyond N read as zeros: their offsets are out of range
-  const unsigned a_at = m0 + l16 < p.M ? (unsigned)(((m0 + l16) * p.lda + 4 * kq) * 4) : OOB_OFFSET;
-  const unsigned b_at = n0 + l16 < p.N ? (unsigned)((4 * kq * p.ldb + n0 + l16) * B_EL) : OOB_OFFSET;
-  const int k_begin = wave * k_per;
-  const int k_end = min(p.K, k_begin + k_per);
-  const int groups = k_end > k_begin ? (k_end - k_begin + 15) >> 4 : 0;
-
-  struct Operands {
-    f32x4 a[G];
-    float b[G][4];
-  };
-  // group q of this wavefront; k at or beyond K (whole groups of 4: K is a multiple of 4) is
-  // turned out of range
-  auto load = [&](int q0, Operands& o) {
-#pragma unroll
-    for (int u = 0; u < G; u++) {
-      if (q0 + u >= groups) break;
-      const int k0 = k_begin + 16 * (q0 + u);
-      const bool in = k0 + 4 * kq < k_end;
-      o.a[u] = buffer_load_f32x4(ra, in ? a_at + (unsigned)k0 * 4 : OOB_OFFSET);
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const unsigned at = in ? b_at + (unsigned)((k0 + e) * p.ldb) * B_EL : OOB_OFFSET;
-        if (QUANT) {
-          const unsigned w = __builtin_amdgcn_raw_buffer_load_b8(rb, (int)at, 0, 0);
-          o.b[u][e] = __builtin_bit_cast(float, w);
-        } else {
-          o.b[u][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rb, (int)at, 0, 0));
-        }
-      }
-    }
-  };
-  f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-  auto multiply = [&](int q0, const Operands& o) {
-#pragma unroll
-    for (int u = 0; u < G; u++) {
-      if (q0 + u >= groups) break;
-      const int k0 = k_begin + 16 * (q0 + u);
-      const bool in = k0 + 4 * kq < k_end;
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        float b = o.b[u][e];
-        // (a byte that was not read is 0, which stands for the weight `min`: drop it)
-        if (QUANT) b = in && n0 + l16 < p.N ? dequant(__builtin_bit_cast(unsigned, b), p.qscale, p.qmin) : 0.f;
-        acc[e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[u][e], b, acc[e & 1], 0, 0, 0);
-      }
-    }
-  };
-  Operands o0, o1;
-  load(0, o0);
-  for (int q0 = 0; q0 < groups; q0 += 2 * G) {
-    load(q0 + G, o1);
-    multiply(q0, o0);
-    load(q0 + 2 * G, o0);
-    multiply(q0 + G, o1);
-  }
-#pragma unroll
-  for (int r = 0; r < 4; r++) part[wave][r][lane] = acc[0][r] + acc[1][r];
-  __syncthreads();
-  if (tid >= 256) return;
-  // accumulator register r of lane l is row 4 * (l / 16) + r, column l % 16 of the tile
-  const int r = tid >> 6;
-  const int row = m0 + 4 * kq + r, col = n0 + l16;
-  float v = part[0][r][lane];
-#pragma unroll
-  for (int w = 1; w < WAVES; w++) v += part[w][r][lane];
-  if (row >= p.M || col >= p.N) return;
-  const long long at = (long long)row * p.N + col;
-  if (p.bias_kind == TFHIP_BCAST_SCALAR) v += p.bias[0];
-  else if (p.bias_kind == TFHIP_BCAST_COLUMN) v += p.bias[col];
-  else if (p.bias_kind == TFHIP_BCAST_FULL) v += p.bias[at];
-  float al = 0.f;
-  if (p.prelu_kind == TFHIP_BCAST_SCALAR) al = p.prelu[0];
-  else if (p.prelu_kind == TFHIP_BCAST_COLUMN) al = p.prelu[col];
-  else if (p.prelu_kind == TFHIP_BCAST_FULL) al = p.prelu[at];
-  p.C[at] = activate(v, act_cfg(p.act), al);
-}
-
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
@@ -1363,6 +1383,7 @@ struct TileCfg {
 // How one tile shape would run a problem: whole tiles, tiles split along K, and a cost.
 struct Plan {
   int grid = 0, full_tiles = 0, tail_tiles = 0, splits = 1, kt_per = 0, tiles_m = 0, tiles_n = 0;
+  int minis = 0;  // > 0: the tail tiles run as this many 16 x 16 pieces each (no split over workgroups)
   double cost = 0;
 };
 
@@ -1401,7 +1422,7 @@ static bool split_tail(Plan& pl, int tail, int want, int k_tiles, bool kblocked)
 }
 
 static Plan make_plan(const GemmArgs& p, int batch, int bm, int bn, int resident, int cus,
-                      double efficiency, bool kblocked) {
+                      double efficiency, bool kblocked, bool minis_ok) {
   Plan pl;
   pl.tiles_m = (int)ceil_div(p.M, bm);
   pl.tiles_n = (int)ceil_div(p.N, bn);
@@ -1436,6 +1457,25 @@ static Plan make_plan(const GemmArgs& p, int batch, int bm, int bn, int resident
       price_plan(sp, bm, bn, cus, efficiency, k_tiles);
       if (sp.cost < pl.cost) pl = sp;
     }
+  }
+  // candidate 4: whole rounds, and the tiles left over cut into pieces of 16 x 16, each a
+  // workgroup whose wavefronts share K among themselves (kwaves_tile: no partial sums in
+  // memory, no second launch).  The pieces are small enough to spread evenly over the CUs; they
+  // run at about a third of the efficiency of a whole tile (operands straight from L2, no
+  // reuse).  Measured on MI355X: [12544, 512] x [512, 512] in 64 x 64 tiles (6.125 per CU)
+  // 52.5 us against 58.3 with a seventh tile on 32 CUs; [3136, 1024] x [1024, 512] 28.4
+  // against 35.0; in 128 x 128 tiles, where more than half a round is left over, 99.7 against 74.6.
+  if (minis_ok && tiles > cus && left > 0) {
+    Plan sp = pl;
+    sp.full_tiles = tiles - left;
+    sp.tail_tiles = left;
+    sp.splits = 1;
+    sp.kt_per = k_tiles;
+    sp.minis = (bm / 16) * (bn / 16);
+    sp.grid = sp.full_tiles + left * sp.minis;
+    const double tile_us = 2.0 * bm * bn * (double)k_tiles * BK / 0.614e6 / efficiency;
+    sp.cost = tile_us * (sp.full_tiles / cus + 3.0 * left / cus) + 1.0;
+    if (sp.cost < pl.cost) pl = sp;
   }
   return pl;
 }
@@ -1496,7 +1536,7 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
   static const char* const b_names[] = {"f32", "f32t", "u8"};
   ctx->name_kernel("gemm_%dx%d_%s_%s%s%s", T::BM, T::BN,
            a_names[AMODE], b_names[BMODE], KBLOCKED ? "_kb48" : "",
-           pl.splits > 1 ? (pl.full_tiles ? "_tailk" : "_splitk") : "");
+           pl.minis ? "_tail16" : pl.splits > 1 ? (pl.full_tiles ? "_tailk" : "_splitk") : "");
   if (!FAST) strncat(ctx->last_kernel, "_unaligned", sizeof ctx->last_kernel - strlen(ctx->last_kernel) - 1);
   p.tiles_m = pl.tiles_m;
   p.tiles_n = pl.tiles_n;
@@ -1505,6 +1545,8 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
   p.splits = pl.splits;
   p.kt_per = pl.kt_per;
   p.k_tiles = (int)ceil_div(p.K, BK);
+  p.minis = pl.minis;
+  p.mini_k_per = (int)ceil_div(ceil_div(p.K, T::WM * T::WN), 16) * 16;
   p.reverse = ctx->take_sweep();
   Temp partials(ctx);
   p.partials = nullptr;
@@ -1538,13 +1580,16 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
   return TFHIP_OK;
 }
 
-// Tile choice: every shape is planned (grid, split along K) and priced, and the cheapest
-// wins; ties go to the larger tile.  Measured on MI355X, at the sizes of a batch-64 MobileNet
-// the 64 x 64 tile (four wavefronts of one 32 x 32 accumulator) is as efficient per flop as
-// the large ones: its small register footprint lets eight workgroups share a CU, and that
-// occupancy hides latency better than a deeper software pipeline in fewer, larger waves;
-// its finer grain also balances the CUs.  The 128 x 128 tile (eight wavefronts of 32 x 64)
-// needs half the LDS traffic per flop and wins on large problems.
+// Tile choice: every shape is planned (grid, split along K, leftover tiles in small pieces) and
+// priced, and the cheapest wins; ties go to the larger tile.  The efficiency per flop of a tile
+// shape is measured on MI355X.  Row-major operands: the 64 x 64 tile (four wavefronts of one
+// 32 x 32 accumulator; seven workgroups share a CU, which hides latency better than a deeper
+// pipeline in fewer, larger wavefronts) beats the 128 x 128 tile by 10 % up to [4096, 1024] x
+// [1024, 1024] (78 against 87 us) and at [12544, 1024] x [1024, 1024] (214 against 238); the
+// large tile, with half the LDS traffic per flop, wins by 9 % at [8192, 4096] x [4096, 4096].
+// Implicit GEMM (the A tile is gathered): 64 x 128 reuses a gathered tile over twice the
+// columns and wins by 9 % over 64 x 64 and 12 % over 128 x 128 (3 x 3 convolutions at 112 x 112
+// x 64 -> 128, 56 x 56 x 128, 28 x 28 x 256, 14 x 14 x 512).
 template <int AMODE, int BMODE, bool KBLOCKED, bool FAST>
 static int launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
   using Big = TileCfg<4, 2, 1, 2>;     // 128 x 128, 8 wavefronts of 32 x 64
@@ -1554,12 +1599,22 @@ static int launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
   using Small = TileCfg<2, 2, 1, 1>;   // 64 x 64, 4 wavefronts of 32 x 32
   constexpr int NCFG = 5;
   const int cus = ctx->num_cus;
+  // (what kwaves_tile needs: unbatched row-major operands it can read with range-checked loads)
+  const bool mk = FAST && AMODE == A_ROWMAJOR && BMODE != B_TRANSPOSED && batch == 1 &&
+                  p.ldb == p.N && (p.K & 3) == 0 && (p.lda & 3) == 0 &&
+                  (long long)p.M * p.N <= 0x7fffffffLL;
   Plan plans[NCFG];
-  plans[0] = make_plan(p, batch, Big::BM, Big::BN, resident_blocks<Big, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 1.00, KBLOCKED);
-  plans[1] = make_plan(p, batch, Mid::BM, Mid::BN, resident_blocks<Mid, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.95, KBLOCKED);
-  plans[2] = make_plan(p, batch, Wide::BM, Wide::BN, resident_blocks<Wide, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 1.00, KBLOCKED);
-  plans[3] = make_plan(p, batch, Thin::BM, Thin::BN, resident_blocks<Thin, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.80, KBLOCKED);
-  plans[4] = make_plan(p, batch, Small::BM, Small::BN, resident_blocks<Small, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.98, KBLOCKED);
+  const bool gathered = AMODE == A_IM2COL || AMODE == A_IM2COL_UP || AMODE == A_IM2COL_T;
+  const bool huge = (double)p.M * p.N * p.K * batch >= 5e10;
+  const double eff_big = gathered ? 0.88 : huge ? 1.00 : 0.88;
+  const double eff_mid = gathered ? 0.93 : 0.90;
+  const double eff_wide = gathered ? 1.00 : 0.97;
+  const double eff_small = gathered ? 0.91 : 0.98;
+  plans[0] = make_plan(p, batch, Big::BM, Big::BN, resident_blocks<Big, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, eff_big, KBLOCKED, mk);
+  plans[1] = make_plan(p, batch, Mid::BM, Mid::BN, resident_blocks<Mid, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, eff_mid, KBLOCKED, mk);
+  plans[2] = make_plan(p, batch, Wide::BM, Wide::BN, resident_blocks<Wide, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, eff_wide, KBLOCKED, mk);
+  plans[3] = make_plan(p, batch, Thin::BM, Thin::BN, resident_blocks<Thin, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, 0.80, KBLOCKED, mk);
+  plans[4] = make_plan(p, batch, Small::BM, Small::BN, resident_blocks<Small, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, eff_small, KBLOCKED, mk);
   // rows and columns beyond M and N are wasted matrix-core work: charge it
   const int bns[NCFG] = {Big::BN, Mid::BN, Wide::BN, Thin::BN, Small::BN};
   const int bms[NCFG] = {Big::BM, Mid::BM, Wide::BM, Thin::BM, Small::BM};
