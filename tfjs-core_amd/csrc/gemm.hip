@@ -188,12 +188,26 @@ __device__ __forceinline__ void kwaves_tile(const GemmArgs& p, int m0, int n0, i
   p.C[at] = activate(v, act_cfg(p.act), al);
 }
 
-// One 16 x 16 tile per workgroup of 8 wavefronts: (M / 16) x (N / 16) workgroups.
+// One 16 x 16 tile per workgroup of 8 wavefronts.  Workgroup b runs on XCD b % 8.  by_columns
+// (at least 8 pairs of tile columns): an XCD takes every eighth pair of tile columns (a pair
+// shares the 128-byte lines of B's rows) with all their tile rows, so that a line of B is
+// fetched into one L2 only; the grid is 8 x (pairs per XCD, rounded up) x 2 x tile rows, and
+// workgroups past the last column leave at once.  Otherwise (few columns: A is the large
+// operand, and a tile row reads its rows of A alone) the tiles are taken in row-major order.
 template <bool QUANT>
-__global__ __launch_bounds__(512) void gemm_kwaves_kernel(const GemmArgs p, int k_per) {
+__global__ __launch_bounds__(512) void gemm_kwaves_kernel(const GemmArgs p, int k_per,
+                                                          int by_columns) {
   __shared__ float part[8 * 4 * 64];
-  kwaves_tile<8, 4, QUANT>(p, ((int)blockIdx.x / p.tiles_n) * 16, ((int)blockIdx.x % p.tiles_n) * 16,
-                           k_per, part, threadIdx.x);
+  int tm = (int)blockIdx.x / p.tiles_n, tn = (int)blockIdx.x % p.tiles_n;
+  if (by_columns) {
+    const int xcd = (int)blockIdx.x & 7, j = (int)blockIdx.x >> 3;
+    const int per_pair = 2 * p.tiles_m;
+    const int pair = xcd + 8 * (j / per_pair), rem = j % per_pair;
+    tn = 2 * pair + (rem & 1);
+    tm = rem >> 1;
+    if (tn >= p.tiles_n) return;
+  }
+  kwaves_tile<8, 4, QUANT>(p, tm * 16, tn * 16, k_per, part, threadIdx.x);
 }
 
 template <int WAVES_M, int WAVES_N, int TM, int TN, int AMODE, int BMODE, bool KBLOCKED, bool FAST>
@@ -585,11 +599,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   if constexpr (FAST && AMODE == A_ROWMAJOR && BMODE != B_TRANSPOSED) {
     // a 16 x 16 piece of a tail tile (the planner sets minis only for unbatched products)
     if (p.minis > 0 && (int)blockIdx.x >= p.full_tiles) {
+      // All pieces of a tail tile go to one XCD (workgroup b runs on XCD b % 8; full_tiles is a
+      // multiple of the CU count), so that the tile's rows of A and columns of B are fetched
+      // into one L2 only; the tail tiles take the XCDs in turn.
       const int h = (int)blockIdx.x - p.full_tiles;
-      const int t = p.full_tiles + h / p.minis, mini = h % p.minis;
+      const int j = h >> 3;
+      const int tt = (h & 7) + 8 * (j / p.minis), mini = j % p.minis;
+      const int t = p.full_tiles + tt;
       const int m0 = (t / p.tiles_n) * BM + (mini / (BN / 16)) * 16;
       const int n0 = (t % p.tiles_n) * BN + (mini % (BN / 16)) * 16;
-      if (t >= p.tiles_m * p.tiles_n || m0 >= p.M || n0 >= p.N) return;
+      if (tt >= p.tail_tiles || m0 >= p.M || n0 >= p.N) return;
       kwaves_tile<WAVES_M * WAVES_N, 2, BMODE == B_UINT8>(p, m0, n0, p.mini_k_per, lds, tid);
       return;
     }
@@ -1472,7 +1491,7 @@ static Plan make_plan(const GemmArgs& p, int batch, int bm, int bn, int resident
     sp.splits = 1;
     sp.kt_per = k_tiles;
     sp.minis = (bm / 16) * (bn / 16);
-    sp.grid = sp.full_tiles + left * sp.minis;
+    sp.grid = sp.full_tiles + (int)ceil_div(left, 8) * 8 * sp.minis;  // (see the kernel's tail branch)
     const double tile_us = 2.0 * bm * bn * (double)k_tiles * BK / 0.614e6 / efficiency;
     sp.cost = tile_us * (sp.full_tiles / cus + 3.0 * left / cus) + 1.0;
     if (sp.cost < pl.cost) pl = sp;
@@ -1703,11 +1722,14 @@ static int launch_kwaves(tfhip_ctx* ctx, const GemmArgs& p, int batch, int amode
   q.tiles_m = (int)ceil_div(p.M, 16);
   q.tiles_n = (int)ceil_div(p.N, 16);
   const int k_per = (int)ceil_div(ceil_div(p.K, 8), 16) * 16;
+  // (see the kernel: pairs of tile columns dealt to the 8 XCDs when there are enough of them)
+  const int by_columns = q.tiles_n >= 16;
+  const long long grid = by_columns ? 8 * ceil_div(ceil_div(q.tiles_n, 2), 8) * 2 * q.tiles_m : tiles;
   ctx->name_kernel("gemm_16x16_kwaves_%s", bmode == B_UINT8 ? "u8" : "f32");
   if (bmode == B_UINT8)
-    tfhip::launch(ctx, gemm_kwaves_kernel<true>, dim3((unsigned)tiles), dim3(512), 0, q, k_per);
+    tfhip::launch(ctx, gemm_kwaves_kernel<true>, dim3((unsigned)grid), dim3(512), 0, q, k_per, by_columns);
   else
-    tfhip::launch(ctx, gemm_kwaves_kernel<false>, dim3((unsigned)tiles), dim3(512), 0, q, k_per);
+    tfhip::launch(ctx, gemm_kwaves_kernel<false>, dim3((unsigned)grid), dim3(512), 0, q, k_per, by_columns);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }
