@@ -1482,8 +1482,8 @@ static Plan make_plan(const GemmArgs& p, int batch, int bm, int bn, int resident
   // memory, no second launch).  The pieces are small enough to spread evenly over the CUs; they
   // run at about a third of the efficiency of a whole tile (operands straight from L2, no
   // reuse).  Measured on MI355X: [12544, 512] x [512, 512] in 64 x 64 tiles (6.125 per CU)
-  // 52.5 us against 58.3 with a seventh tile on 32 CUs; [3136, 1024] x [1024, 512] 28.4
-  // against 35.0; in 128 x 128 tiles, where more than half a round is left over, 99.7 against 74.6.
+  // 53.1 us against 58.8 with a seventh tile on 32 CUs; [3136, 1024] x [1024, 512] 28.4
+  // against 35.0; in 128 x 128 tiles, where more than half a round is left over, 94.0 against 67.1.
   if (minis_ok && tiles > cus && left > 0) {
     Plan sp = pl;
     sp.full_tiles = tiles - left;
@@ -1601,14 +1601,15 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
 
 // Tile choice: every shape is planned (grid, split along K, leftover tiles in small pieces) and
 // priced, and the cheapest wins; ties go to the larger tile.  The efficiency per flop of a tile
-// shape is measured on MI355X.  Row-major operands: the 64 x 64 tile (four wavefronts of one
-// 32 x 32 accumulator; seven workgroups share a CU, which hides latency better than a deeper
-// pipeline in fewer, larger wavefronts) beats the 128 x 128 tile by 10 % up to [4096, 1024] x
-// [1024, 1024] (78 against 87 us) and at [12544, 1024] x [1024, 1024] (214 against 238); the
-// large tile, with half the LDS traffic per flop, wins by 9 % at [8192, 4096] x [4096, 4096].
-// Implicit GEMM (the A tile is gathered): 64 x 128 reuses a gathered tile over twice the
-// columns and wins by 9 % over 64 x 64 and 12 % over 128 x 128 (3 x 3 convolutions at 112 x 112
-// x 64 -> 128, 56 x 56 x 128, 28 x 28 x 256, 14 x 14 x 512).
+// shape is measured on MI355X (every tile forced on every shape, interleaved, clocks warm).
+// Row-major operands: [4096, 1024] x [1024, 1024], where every shape fills whole rounds, takes
+// 77.0 us in 128 x 128 tiles, 80.7 in 128 x 64, 74.0 in 64 x 128 and 73.4 in 64 x 64 (four
+// wavefronts of one 32 x 32 accumulator; seven workgroups share a CU, which hides latency better
+// than a deeper pipeline in fewer, larger wavefronts); at [8192, 4096] x [4096, 4096] the large
+// tile, with half the LDS traffic per flop, wins: 2086 / 2233 / 2219 / 2281 us.
+// Implicit GEMM (the A tile is gathered, so reusing it over more columns pays): a 3 x 3
+// convolution of 112 x 112 x 64 -> 128 takes 514 / 536 / 514 / 561 us, 56 x 56 x 128 -> 128
+// 502 / 520 / 494 / 554.
 template <int AMODE, int BMODE, bool KBLOCKED, bool FAST>
 static int launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
   using Big = TileCfg<4, 2, 1, 2>;     // 128 x 128, 8 wavefronts of 32 x 64
@@ -1625,10 +1626,10 @@ static int launch_mode(tfhip_ctx* ctx, GemmArgs& p, int batch) {
   Plan plans[NCFG];
   const bool gathered = AMODE == A_IM2COL || AMODE == A_IM2COL_UP || AMODE == A_IM2COL_T;
   const bool huge = (double)p.M * p.N * p.K * batch >= 5e10;
-  const double eff_big = gathered ? 0.88 : huge ? 1.00 : 0.88;
-  const double eff_mid = gathered ? 0.93 : 0.90;
-  const double eff_wide = gathered ? 1.00 : 0.97;
-  const double eff_small = gathered ? 0.91 : 0.98;
+  const double eff_big = gathered ? 0.98 : huge ? 1.00 : 0.95;
+  const double eff_mid = gathered ? 0.95 : huge ? 0.93 : 0.91;
+  const double eff_wide = gathered ? 1.00 : huge ? 0.94 : 0.99;
+  const double eff_small = gathered ? 0.92 : huge ? 0.92 : 1.00;
   plans[0] = make_plan(p, batch, Big::BM, Big::BN, resident_blocks<Big, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, eff_big, KBLOCKED, mk);
   plans[1] = make_plan(p, batch, Mid::BM, Mid::BN, resident_blocks<Mid, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, eff_mid, KBLOCKED, mk);
   plans[2] = make_plan(p, batch, Wide::BM, Wide::BN, resident_blocks<Wide, AMODE, BMODE, KBLOCKED, FAST>(ctx), cus, eff_wide, KBLOCKED, mk);
