@@ -50,6 +50,7 @@ struct GemmArgs {
   double qscale, qmin;
   // schedule (see work_item)
   int tiles_m, tiles_n, k_tiles, full_tiles, tail_tiles, splits, kt_per;
+  int tiles_n_shift;  // log2(tiles_n) when that is a power of two, else -1 (a division on the vector ALU)
   float* partials;  // [tail_tiles * splits][BM * BN] partial tiles when splits > 1
   // minis > 0: the tail tiles are not split along K over workgroups but cut into `minis` tiles
   // of 16 x 16 each, one per workgroup, whose wavefronts take mini_k_per of K each (kwaves_tile)
@@ -254,7 +255,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     const float* A;
     const float* Bf;
     const unsigned char* Bq;
-    int bm0, bn0;
+    int bm0, bn0, batch;
     int a_row[A_PER], a_kq[A_PER];
     long long a_base[A_PER];  // row-major: row*lda ; im2col: n*H*W*Cin
     int a_ih0[A_PER], a_iw0[A_PER];
@@ -270,10 +271,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   constexpr bool A_UNIFORM_K = FAST && AMODE == A_ROWMAJOR;
 
   auto setup = [&](Loader& L, int tile) {
-    const int batch = tile / tiles_per_batch;
+    // (integer division runs on the vector ALU, which the matrix instructions share: none for an
+    // unbatched product, a shift for a power-of-two number of tile columns)
+    const int batch = tile < tiles_per_batch ? 0 : tile / tiles_per_batch;
     const int t = tile - batch * tiles_per_batch;
-    L.bm0 = (t / p.tiles_n) * BM;
-    L.bn0 = (t % p.tiles_n) * BN;
+    const int tm = p.tiles_n_shift >= 0 ? t >> p.tiles_n_shift : t / p.tiles_n;
+    L.bm0 = tm * BM;
+    L.bn0 = (t - tm * p.tiles_n) * BN;
+    L.batch = batch;
     L.A = p.A + batch * p.strideA;
     L.Bf = static_cast<const float*>(p.B) + batch * p.strideB;
     L.Bq = static_cast<const unsigned char*>(p.B) + batch * p.strideB;
@@ -781,7 +786,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   // ---- store.  Accumulator register r of a 32x32 tile holds row
   // 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
   const int bm0 = L.bm0, bn0 = L.bn0;
-  const int batch = cur.tile / tiles_per_batch;
+  const int batch = L.batch;
   const int col0 = bn0 + wn * TN * 32 + TN * l32;
   if (cur.slot >= 0) {
     // partial sum of a k range: raw accumulators into the tile-shaped slot
@@ -1559,6 +1564,7 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
   if (!FAST) strncat(ctx->last_kernel, "_unaligned", sizeof ctx->last_kernel - strlen(ctx->last_kernel) - 1);
   p.tiles_m = pl.tiles_m;
   p.tiles_n = pl.tiles_n;
+  p.tiles_n_shift = (pl.tiles_n & (pl.tiles_n - 1)) == 0 ? __builtin_ctz((unsigned)pl.tiles_n) : -1;
   p.full_tiles = pl.full_tiles;
   p.tail_tiles = pl.tail_tiles;
   p.splits = pl.splits;
