@@ -880,7 +880,9 @@ def _separable_oracle(ref, x, dw, pw, stride, dbias, dact, pbias, pact):
 @pytest.mark.parametrize("xs,cout,stride", [
     ((16, 112, 112, 32), 64, 1),    # single kernel: K 32 -> N 64
     ((64, 112, 112, 64), 128, 2),   # single kernel, stride 2 (top/left padding 0)
-    ((64, 56, 56, 128), 128, 1),    # K 128 -> N 128: the filter leaves no room for the panels, two kernels
+    ((64, 56, 56, 128), 128, 1),    # single kernel: K 128 -> N 128, the pointwise filter in registers
+    ((65, 55, 57, 128), 128, 1),    # the same on odd extents
+    ((8, 56, 56, 128), 128, 1),     # too few pixels for it: two kernels
     ((17, 113, 111, 32), 64, 1),    # odd extents: blocks straddle rows and images, last block short
     ((66, 111, 113, 64), 128, 2),   # stride 2 on odd extents (padding 1 on both sides)
     ((2, 20, 20, 32), 64, 1),       # too few pixels for the single kernel: two-kernel form
@@ -917,7 +919,7 @@ def test_separable_conv2d_matches_the_two_op_chain(hip, ref, xs, cout, stride):
         single = len(kernels) == 1 and kernels[0].startswith("separable_")
         pixels = xs[0] * -(-xs[1] // stride) * -(-xs[2] // stride)
         expect_single = pixels >= 256 * 8 * 32 * 3 and \
-            (c, cout, stride) in ((32, 64, 1), (64, 128, 2))
+            (c, cout, stride) in ((32, 64, 1), (64, 128, 2), (128, 128, 1))
         assert single == expect_single, kernels
         want = _separable_oracle(ref, x[pick], dw, pw, stride, db, dact, pb, pact)
         close(got[pick], want)
@@ -931,23 +933,28 @@ def test_separable_conv2d_matches_the_two_op_chain(hip, ref, xs, cout, stride):
             close(got, two, rtol=2e-5, atol=2e-6)
 
 
-def test_separable_conv2d_uint8_filters(hip, ref):
+@pytest.mark.parametrize("xs,cout,name", [
+    ((16, 112, 112, 32), 64, "separable_s1_k32xn64_u8"),
+    ((64, 56, 56, 128), 128, "separable_s1_k128xn128_u8"),
+])
+def test_separable_conv2d_uint8_filters(hip, ref, xs, cout, name):
     """Both filters kept as uint8 in HBM and dequantised inside the single kernel."""
     tf = hip.tf
     from tfhip import mobilenet
-    rng = rng_for("separable-u8")
-    x = rng.uniform(0, 1, (16, 112, 112, 32)).astype(np.float32)
-    params = {"dw_w": (rng.standard_normal((3, 3, 32, 1)) * 0.5).astype(np.float32),
-              "pw_w": (rng.standard_normal((1, 1, 32, 64)) * 0.25).astype(np.float32)}
+    rng = rng_for("separable-u8", xs, cout)
+    c = xs[3]
+    x = rng.uniform(0, 1, xs).astype(np.float32)
+    params = {"dw_w": (rng.standard_normal((3, 3, c, 1)) * 0.5).astype(np.float32),
+              "pw_w": (rng.standard_normal((1, 1, c, cout)) * np.sqrt(2.0 / c)).astype(np.float32)}
     q = mobilenet.quantize_params(params)
     deq = {k: ref.dequantize(*v) for k, v in q.items()}
-    bias = (rng.standard_normal(64) * 0.1).astype(np.float32)
+    bias = (rng.standard_normal(cout) * 0.1).astype(np.float32)
     with tf.tidy():
         out = []
         info = tf.time(lambda: out.append(tf.fused.separable_conv2d(
             tf.tensor(x), tf.quantized_tensor(*q["dw_w"]), tf.quantized_tensor(*q["pw_w"]), 1, "same",
             depthwise_activation="relu6", bias=tf.tensor(bias), activation="relu6")))
         got = out[0].data_sync()
-    assert [k[0] for k in info["kernelTimes"]] == ["separable_s1_k32xn64_u8"]
+    assert [k[0] for k in info["kernelTimes"]] == [name]
     want = _separable_oracle(ref, x[:1], deq["dw_w"], deq["pw_w"], 1, None, "relu6", bias, "relu6")
     close(got[:1], want)

@@ -9,23 +9,28 @@
 // own panel in LDS and multiplies the panel by the pointwise filter on the matrix cores.
 // HBM sees the block's input once and its output once.
 //
-// Shape.  The pointwise filter [K, N] (K = input channels, N = output channels) lies in LDS in
-// operand order for the whole kernel, so this kernel serves the blocks whose filter fits
-// (K * N * 4 <= 64 KiB).  A wavefront works on its own: it takes a strip of SW output columns of
-// one image and walks down a chunk of output rows.
+// Shape.  A workgroup is 8 wavefronts: 4 depthwise wavefronts that only load, and 4 pointwise
+// wavefronts that only store (a wavefront that does both waits for the acknowledgements of its
+// stores whenever it waits for a load: the two share one counter).  Each depthwise wavefront takes
+// a strip of SW output columns of one image and walks down a chunk of output rows; what it
+// produces goes to a panel [32 pixels][K] in LDS, two panels per depthwise wavefront, one barrier
+// per panel: panel i + 1 is filled while panel i is multiplied.
 //   depthwise stage: lanes run along the channels (a lane owns one quad of 4 channels and TW
 //     neighbouring output columns, so a wavefront access is a run of 16-byte pieces).  Every
 //     input row of the strip is fetched once (buffer loads whose offsets fall outside the
 //     descriptor where the padding is; PD rows in flight) and feeds the output rows it belongs
 //     to, which live in rotating accumulators; taps are summed in the order filter row, filter
 //     column, as the reference does.  A finished row gets its bias and activation and goes to
-//     the panel [pixel][k]; RB rows fill the panel's 32 pixels.
+//     the panel; RB rows fill the panel's 32 pixels.
 //   pointwise stage: lane = pixel of the panel (16-byte LDS reads of 4 consecutive k; lanes
-//     0-31 take k = 0..3 and lanes 32-63 k = 4..7 of each group of 8, the operand order the
-//     filter was laid out in), v_mfma_f32_32x32x2f32 into N / 32 accumulators, bias + activation,
-//     dword stores of 128-byte runs.
-// Wavefronts of a workgroup share nothing but the filter, so there is no barrier after the set-up;
-// the other wavefronts of the SIMD fill the time one of them waits for memory or the matrix cores.
+//     0-31 take k = 0..3 and lanes 32-63 k = 4..7 of each group of 8), v_mfma_f32_32x32x2f32,
+//     bias + activation, dword stores of 128-byte runs.  Two forms:
+//     - the pointwise filter [K, N] lies in LDS in operand order (K * N * 4 <= 32 KiB beside the
+//       panels); pointwise wavefront i multiplies the panels of depthwise wavefront i by all N
+//       columns;
+//     - COLS (K = N = 128: the filter would take 64 KiB): pointwise wavefront j keeps the filter's
+//       columns 32j..32j+31 in registers and multiplies the panels of all four depthwise
+//       wavefronts by them; LDS holds panels only.
 #include <type_traits>
 
 #include "tfhip_internal.h"
@@ -52,9 +57,15 @@ struct SepArgs {
   int reverse;
 };
 
-template <int KQ, int NJ, int S, int PD, int OCC>
+template <int KQ, int NJ, int S, int PD, int OCC, bool COLS>
 __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
   constexpr int K = 8 * KQ, N = 32 * NJ;
+  // COLS: the pointwise filter does not fit LDS beside the panels (K = N = 128: 64 KiB).  Then it
+  // lives in registers instead: pointwise wavefront j keeps rows 0..K-1 of columns 32j..32j+31 in
+  // operand order (K / 2 registers) and multiplies every panel of the workgroup by them, so LDS
+  // holds panels only and all four matrix pipes of the CU work on each panel.
+  static_assert(!COLS || NJ == 4, "one pointwise wavefront per block of 32 output columns");
+  constexpr int FILTER_FLOATS = COLS ? 0 : K * N;
   constexpr int QN = K / 4;            // channel quads = lanes side by side along the channels
   constexpr int PX = 64 / QN;          // pixel slots of a wavefront
   constexpr int TW = S == 1 ? 2 : 1;   // output columns of a lane
@@ -74,9 +85,10 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
   const bool producer = wave < 4;
   const int pair = wave & 3;
   const int l32 = lane & 31, g = lane >> 5;
-  float* panels = lds + K * N + pair * (2 * 32 * PITCH);  // the pair's two panels
+  float* const panels0 = lds + FILTER_FLOATS;                // two panels per pair
+  float* panels = panels0 + pair * (2 * 32 * PITCH);         // this pair's
 
-  {
+  if constexpr (!COLS) {
     // the pointwise filter into operand order: an item is 4 consecutive k of one column
     constexpr int PER = (K / 4 * N + 511) / 512;
     auto fill = [&](auto quant_tag) {
@@ -121,9 +133,9 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
     bool live;
     int n, o0, rows, strip;
   };
-  auto unit_of = [&](int trip) {
+  auto unit_of = [&](int trip, int pr) {
     Unit un;
-    const int u = wg_first + trip * stride + pair;
+    const int u = wg_first + trip * stride + pr;
     un.live = u < run1;
     const int unit = p.reverse ? run0 + run1 - 1 - u : u;
     un.strip = unit % p.strips;
@@ -198,7 +210,7 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
       if (it < total) {
         if (blk == 0) {
           // a new unit: its offsets, the first PD rows, the rows before the first output row
-          const Unit un = unit_of(trip);
+          const Unit un = unit_of(trip, pair);
           t0 = un.o0 * S;
           t_last = un.live ? (un.o0 + un.rows - 1) * S + 2 : t0 - 1;
           const int iw0 = (un.strip * SW + slot * TW) * S - p.pl;
@@ -299,6 +311,85 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
       }
       __syncthreads();  // the panel is complete; the other one has been multiplied
     }
+  } else if constexpr (COLS) {
+    // ---- pointwise wavefronts, one per block of 32 output columns: every panel x its columns ----
+    const int cb = pair;
+    float b[KQ][4];  // filter rows k = 8q + 4g + e of column 32 cb + l32
+#pragma unroll
+    for (int q = 0; q < KQ; q++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const int at = (8 * q + 4 * g + e) * N + 32 * cb + l32;
+        b[q][e] = p.pw_quant ? dequant(static_cast<const unsigned char*>(p.pw)[at], p.pw_scale, p.pw_min)
+                             : static_cast<const float*>(p.pw)[at];
+      }
+    const float bias_c = p.pwb_kind == TFHIP_BCAST_COLUMN ? p.pwb[32 * cb + l32]
+                       : p.pwb_kind == TFHIP_BCAST_SCALAR ? p.pwb[0] : 0.f;
+    const Clamp pact = clamp_of(p.pw_act);
+    const __amdgpu_buffer_rsrc_t ry = make_rsrc(p.y, p.y_bytes);
+    const unsigned y_row = (unsigned)(p.OW * N * 4);
+    const float* const panel_r = panels0 + l32 * PITCH + 4 * g;  // this lane's operand in pair 0's first panel
+    __syncthreads();
+
+    int trip = 0, blk = 0;
+    for (int it = 0; it <= total; it++) {
+      if (it > 0) {
+        // the four panels filled during the previous step: block `blk` of the pairs' units
+#pragma nounroll
+        for (int pr = 0; pr < 4; pr++) {
+          const Unit un = unit_of(trip, pr);
+          const int rows_left = un.rows - blk * RB;
+          if (!un.live || rows_left <= 0) continue;  // (the same for the whole wavefront)
+          const float* const panel = panel_r + pr * (2 * 32 * PITCH) + ((it - 1) & 1) * (32 * PITCH);
+          f32x16 acc;
+          f32x4 a[2];
+          a[0] = *reinterpret_cast<const f32x4*>(panel);
+#pragma unroll
+          for (int q = 0; q < KQ; q++) {
+            if (q + 1 < KQ) a[(q + 1) & 1] = *reinterpret_cast<const f32x4*>(panel + 8 * (q + 1));
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
+                                   0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q & 1][e], b[q][e],
+                                                         q == 0 && e == 0 ? zero : acc, 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          // accumulator register r: pixel m = 8*(r/4) + 4*(lane/32) + r%4 of the panel, column l32
+          const int orow = un.o0 + blk * RB, ocol = un.strip * SW;
+          const unsigned y_blk = (unsigned)((un.n * p.OH + orow) * p.OW + ocol) * (unsigned)(N * 4) +
+                                 (unsigned)((32 * cb + l32) * 4);
+          const int cols_left = p.OW - ocol;
+          const bool whole = rows_left >= RB && cols_left >= SW;
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int mc = 8 * (r >> 2) + (r & 3);  // + 4 * g
+            int row, col;
+            unsigned at;
+            if (SW >= 8) {
+              row = mc / SW;
+              col = mc % SW + 4 * g;
+              at = y_blk + (unsigned)row * y_row + (unsigned)((mc % SW + 4 * g) * N * 4);
+            } else {
+              row = mc / SW + g * (4 / SW);
+              col = mc % SW;
+              at = y_blk + (unsigned)row * y_row + (unsigned)(col * N * 4);
+            }
+            const bool ok = whole || (row < rows_left && col < cols_left);
+            const float val = clamp(acc[r] + bias_c, pact);
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), ry,
+                                                  (int)(ok ? at : OOB_OFFSET), 0, 0);
+          }
+        }
+        if (++blk == iters) {
+          blk = 0;
+          trip++;
+        }
+      }
+      __syncthreads();  // the next panels are complete; these may be overwritten
+    }
   } else {
     // ---- pointwise wavefronts: panel x filter -> output --------------------------------------
     float bias_c[NJ];  // pointwise bias of column 32j + l32
@@ -313,7 +404,7 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
     __syncthreads();
 
     int trip = 0, blk = 0;
-    Unit un = unit_of(0);
+    Unit un = unit_of(0, pair);
     for (int it = 0; it <= total; it++) {
       if (it > 0) {
         // the panel filled during the previous step: block `blk` of unit `un`
@@ -387,7 +478,7 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
         if (++blk == iters) {
           blk = 0;
           trip++;
-          un = unit_of(trip);
+          un = unit_of(trip, pair);
         }
       }
       __syncthreads();  // the next panel is complete; this one may be overwritten
@@ -395,12 +486,12 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
   }
 }
 
-template <int KQ, int NJ, int S, int PD, int OCC>
+template <int KQ, int NJ, int S, int PD, int OCC, bool COLS = false>
 static int launch_separable(tfhip_ctx* ctx, SepArgs& p) {
-  auto kernel = separable_kernel<KQ, NJ, S, PD, OCC>;
+  auto kernel = separable_kernel<KQ, NJ, S, PD, OCC, COLS>;
   constexpr int K = 8 * KQ, N = 32 * NJ;
   constexpr int SW = 64 / (K / 4) * (S == 1 ? 2 : 1), RB = 32 / SW;
-  const size_t lds = ((size_t)K * N + 8 * 32 * (K + 4)) * sizeof(float);
+  const size_t lds = ((size_t)(COLS ? 0 : K * N) + 8 * 32 * (K + 4)) * sizeof(float);
   static int per_cu = 0;
   if (!per_cu) {
     if (lds > 48 * 1024)
@@ -501,6 +592,7 @@ extern "C" int tfhip_separable_conv2d(tfhip_ctx* ctx, int64_t x, int64_t dw_filt
   if (one) {
     if (K == 32 && N == 64 && S == 1) variant = 0;
     else if (K == 64 && N == 128 && S == 2) variant = 1;
+    else if (K == 128 && N == 128 && S == 1) variant = 2;
   }
   if (variant >= 0 && !ctx->separable_off) {
     SepArgs p = {};
@@ -530,6 +622,9 @@ extern "C" int tfhip_separable_conv2d(tfhip_ctx* ctx, int64_t x, int64_t dw_filt
     switch (variant) {
       case 0: return launch_separable<4, 2, 1, 2, 4>(ctx, p);
       case 1: return launch_separable<8, 4, 2, 8, 2>(ctx, p);
+      // (measured at [64,56,56,128] -> 128: 4 rows in flight 82 us, 2 rows 85, 8 rows 83; chunks
+      // of 32 / 16 / 8 output rows instead of whole strips 87 / 91 / 89)
+      case 2: return launch_separable<16, 4, 1, 4, 2, true>(ctx, p);
       default: break;
     }
   }
