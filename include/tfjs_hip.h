@@ -207,7 +207,7 @@ int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t out,
  * dw_info is the Conv2DInfo of the depthwise half; pw_filter is [1,1,dw_info.out_c,out_c] and
  * out [batch,out_h,out_w,out_c].  Biases NONE / SCALAR / COLUMN, activations LINEAR / RELU /
  * RELU6; either filter may be TFHIP_UINT8Q with its qparams.  For 3x3 filters, multiplier 1 and
- * (channels, stride) in {(32->64, 1), (64->128, 2)} on large images one kernel computes both
+ * (channels, stride) in {(32->64, 1), (64->128, 2), (128->128, 1)} on large images one kernel computes both
  * halves and the intermediate never reaches HBM; every other shape runs the two kernels with
  * the intermediate in a pool block.  Results are those of the two calls (the single kernel sums
  * the pointwise products in another order: equal within float32 round-off).

@@ -883,6 +883,7 @@ def _separable_oracle(ref, x, dw, pw, stride, dbias, dact, pbias, pact):
     ((64, 56, 56, 128), 128, 1),    # single kernel: K 128 -> N 128, the pointwise filter in registers
     ((65, 55, 57, 128), 128, 1),    # the same on odd extents
     ((8, 56, 56, 128), 128, 1),     # too few pixels for it: two kernels
+    ((33, 55, 57, 128), 256, 2),    # K 128 -> N 256 at stride 2: two kernels
     ((17, 113, 111, 32), 64, 1),    # odd extents: blocks straddle rows and images, last block short
     ((66, 111, 113, 64), 128, 2),   # stride 2 on odd extents (padding 1 on both sides)
     ((2, 20, 20, 32), 64, 1),       # too few pixels for the single kernel: two-kernel form

@@ -64,7 +64,8 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
   // lives in registers instead: pointwise wavefront j keeps rows 0..K-1 of columns 32j..32j+31 in
   // operand order (K / 2 registers) and multiplies every panel of the workgroup by them, so LDS
   // holds panels only and all four matrix pipes of the CU work on each panel.
-  static_assert(!COLS || NJ == 4, "one pointwise wavefront per block of 32 output columns");
+  static_assert(!COLS || NJ % 4 == 0, "every pointwise wavefront takes NJ / 4 blocks of 32 output columns");
+  constexpr int CB = COLS ? NJ / 4 : 1;  // column blocks of a pointwise wavefront (COLS)
   constexpr int FILTER_FLOATS = COLS ? 0 : K * N;
   constexpr int QN = K / 4;            // channel quads = lanes side by side along the channels
   constexpr int PX = 64 / QN;          // pixel slots of a wavefront
@@ -312,19 +313,25 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
       __syncthreads();  // the panel is complete; the other one has been multiplied
     }
   } else if constexpr (COLS) {
-    // ---- pointwise wavefronts, one per block of 32 output columns: every panel x its columns ----
-    const int cb = pair;
-    float b[KQ][4];  // filter rows k = 8q + 4g + e of column 32 cb + l32
+    // ---- pointwise wavefronts, each with CB blocks of 32 output columns: every panel x its columns ----
+    const int col0 = 32 * CB * pair + l32;  // this lane's column in its first block
+    float b[CB][KQ][4];  // filter rows k = 8q + 4g + e of columns col0 + 32 c
 #pragma unroll
-    for (int q = 0; q < KQ; q++)
+    for (int c = 0; c < CB; c++)
 #pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const int at = (8 * q + 4 * g + e) * N + 32 * cb + l32;
-        b[q][e] = p.pw_quant ? dequant(static_cast<const unsigned char*>(p.pw)[at], p.pw_scale, p.pw_min)
-                             : static_cast<const float*>(p.pw)[at];
-      }
-    const float bias_c = p.pwb_kind == TFHIP_BCAST_COLUMN ? p.pwb[32 * cb + l32]
-                       : p.pwb_kind == TFHIP_BCAST_SCALAR ? p.pwb[0] : 0.f;
+      for (int q = 0; q < KQ; q++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int at = (8 * q + 4 * g + e) * N + col0 + 32 * c;
+          b[c][q][e] = p.pw_quant
+                           ? dequant(static_cast<const unsigned char*>(p.pw)[at], p.pw_scale, p.pw_min)
+                           : static_cast<const float*>(p.pw)[at];
+        }
+    float bias_c[CB];
+#pragma unroll
+    for (int c = 0; c < CB; c++)
+      bias_c[c] = p.pwb_kind == TFHIP_BCAST_COLUMN ? p.pwb[col0 + 32 * c]
+                : p.pwb_kind == TFHIP_BCAST_SCALAR ? p.pwb[0] : 0.f;
     const Clamp pact = clamp_of(p.pw_act);
     const __amdgpu_buffer_rsrc_t ry = make_rsrc(p.y, p.y_bytes);
     const unsigned y_row = (unsigned)(p.OW * N * 4);
@@ -341,7 +348,7 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
           const int rows_left = un.rows - blk * RB;
           if (!un.live || rows_left <= 0) continue;  // (the same for the whole wavefront)
           const float* const panel = panel_r + pr * (2 * 32 * PITCH) + ((it - 1) & 1) * (32 * PITCH);
-          f32x16 acc;
+          f32x16 acc[CB];
           f32x4 a[2];
           a[0] = *reinterpret_cast<const f32x4*>(panel);
 #pragma unroll
@@ -349,38 +356,44 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
             if (q + 1 < KQ) a[(q + 1) & 1] = *reinterpret_cast<const f32x4*>(panel + 8 * (q + 1));
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-              const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
-                                   0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q & 1][e], b[q][e],
-                                                         q == 0 && e == 0 ? zero : acc, 0, 0, 0);
-            }
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+              for (int c = 0; c < CB; c++) {
+                const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
+                                     0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                acc[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q & 1][e], b[c][q][e],
+                                                              q == 0 && e == 0 ? zero : acc[c], 0, 0, 0);
+              }
             __builtin_amdgcn_sched_barrier(0);
           }
           // accumulator register r: pixel m = 8*(r/4) + 4*(lane/32) + r%4 of the panel, column l32
           const int orow = un.o0 + blk * RB, ocol = un.strip * SW;
           const unsigned y_blk = (unsigned)((un.n * p.OH + orow) * p.OW + ocol) * (unsigned)(N * 4) +
-                                 (unsigned)((32 * cb + l32) * 4);
+                                 (unsigned)(col0 * 4);
           const int cols_left = p.OW - ocol;
           const bool whole = rows_left >= RB && cols_left >= SW;
 #pragma unroll
           for (int r = 0; r < 16; r++) {
             const int mc = 8 * (r >> 2) + (r & 3);  // + 4 * g
             int row, col;
-            unsigned at;
             if (SW >= 8) {
               row = mc / SW;
               col = mc % SW + 4 * g;
-              at = y_blk + (unsigned)row * y_row + (unsigned)((mc % SW + 4 * g) * N * 4);
-            } else {
-              row = mc / SW + g * (4 / SW);
+            } else if (SW == 4) {
+              row = mc / SW + g;
               col = mc % SW;
-              at = y_blk + (unsigned)row * y_row + (unsigned)(col * N * 4);
+            } else {  // SW == 2: 4 * g pixels further on is 2 rows further down
+              row = mc / SW + 2 * g;
+              col = mc % SW;
             }
+            const unsigned at = y_blk + (unsigned)row * y_row + (unsigned)(col * N * 4);
             const bool ok = whole || (row < rows_left && col < cols_left);
-            const float val = clamp(acc[r] + bias_c, pact);
-            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), ry,
-                                                  (int)(ok ? at : OOB_OFFSET), 0, 0);
+#pragma unroll
+            for (int c = 0; c < CB; c++) {
+              const float val = clamp(acc[c][r] + bias_c[c], pact);
+              __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), ry,
+                                                    (int)(ok ? at + (unsigned)(32 * c * 4) : OOB_OFFSET), 0, 0);
+            }
           }
         }
         if (++blk == iters) {
@@ -585,14 +598,18 @@ extern "C" int tfhip_separable_conv2d(tfhip_ctx* ctx, int64_t x, int64_t dw_filt
                        bpb->numel == (pw_bias_kind == TFHIP_BCAST_COLUMN ? N : 1))) &&
              (bdw->dtype == TFHIP_FLOAT32 || bdw->dtype == TFHIP_UINT8Q) &&
              (bpw->dtype == TFHIP_FLOAT32 || bpw->dtype == TFHIP_UINT8Q) && aligned16(bx->ptr) &&
-             aligned16(bo->ptr) &&
-             // enough 32-pixel blocks to give every wavefront of a full machine several
-             pixels >= (int64_t)ctx->num_cus * 8 * 32 * 3;
+             aligned16(bo->ptr);
   int variant = -1;
   if (one) {
-    if (K == 32 && N == 64 && S == 1) variant = 0;
-    else if (K == 64 && N == 128 && S == 2) variant = 1;
-    else if (K == 128 && N == 128 && S == 1) variant = 2;
+    // enough 32-pixel panels to give every depthwise wavefront of a full machine several
+    const int64_t several = (int64_t)ctx->num_cus * 8 * 32 * 3;
+    if (K == 32 && N == 64 && S == 1 && pixels >= several) variant = 0;
+    else if (K == 64 && N == 128 && S == 2 && pixels >= several) variant = 1;
+    else if (K == 128 && N == 128 && S == 1 && pixels >= several) variant = 2;
+    // (128 -> 256 at stride 2, two column blocks per pointwise wavefront, was built and measured
+    // at [64,56,56,128]: 56 us against 21 + 34 us for the two kernels.  Its 1568 panels are two
+    // rounds of a machine of 1024 depthwise wavefronts, the second three quarters full, and the
+    // first round's loads and the last round's products overlap with nothing.)
   }
   if (variant >= 0 && !ctx->separable_off) {
     SepArgs p = {};
