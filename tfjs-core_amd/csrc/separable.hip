@@ -638,7 +638,9 @@ extern "C" int tfhip_separable_conv2d(tfhip_ctx* ctx, int64_t x, int64_t dw_filt
     p.y_bytes = (unsigned)(pixels * N * 4);
     switch (variant) {
       case 0: return launch_separable<4, 2, 1, 2, 4>(ctx, p);
-      case 1: return launch_separable<8, 4, 2, 8, 2>(ctx, p);
+      // (measured at [64,112,112,64] -> 128, stride 2: the filter in registers, 4 rows in flight and
+      // two workgroups per CU 75.2 us; the filter in LDS, 8 rows in flight, one workgroup 76.8)
+      case 1: return launch_separable<8, 4, 2, 4, 4, true>(ctx, p);
       // (measured at [64,56,56,128] -> 128: 4 rows in flight 82 us, 2 rows 85, 8 rows 83; chunks
       // of 32 / 16 / 8 output rows instead of whole strips 87 / 91 / 89)
       case 2: return launch_separable<16, 4, 1, 4, 2, true>(ctx, p);
