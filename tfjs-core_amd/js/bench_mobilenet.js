@@ -95,7 +95,10 @@ async function main() {
   }
 
   // ---- the network as a graph of the reference's own ops ------------------------------------
-  for (let i = 0; i < Math.min(warmup, 5); i++) step(mobilenet.forwardReference);
+  // (this path runs other JavaScript than the loops above, and V8 compiles a function only after
+  // it has run a few hundred times: warm up until the host is as fast as it will be, or a step
+  // of less than a millisecond is bound by the interpreter instead of the kernels)
+  for (let i = 0; i < Math.max(warmup, 300); i++) step(mobilenet.forwardReference);
   be.sync();
   t0 = now();
   for (let i = 0; i < steps; i++) step(mobilenet.forwardReference);
