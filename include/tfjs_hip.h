@@ -117,6 +117,17 @@ int tfhip_read_finish(tfhip_ctx* ctx, tfhip_pending_read* r, void* host, size_t 
 /* bytes held by live ids / bytes parked in the pool / number of live ids */
 int tfhip_mem_info(tfhip_ctx* ctx, size_t* in_use, size_t* pooled, size_t* num_ids);
 int tfhip_sync(tfhip_ctx* ctx);
+
+/* No counterpart in the reference (its backends queue everything on one context).  A context has
+ * two compute streams; calls that queue work use the selected one (0 after tfhip_init).  Work
+ * queued under one index runs in the order of the calls; work under different indices is not
+ * ordered against each other and may overlap on the device: two independent passes (batch i
+ * under index 0, batch i + 1 under index 1 of a serving loop) then fill each other's idle
+ * phases.  A buffer written under one index must not be used under the other before the host
+ * has waited for it (tfhip_sync, or a read of it); buffers that are only read (weights) may be
+ * shared.  tfhip_read / tfhip_read_begin follow the buffer's own stream, tfhip_sync waits for
+ * both.  Not inside a timed region or a graph capture. */
+int tfhip_select_stream(tfhip_ctx* ctx, int index);
 /* KernelBackend.time (backend.ts:92, backend_cpu.ts:239-244): device time of the work queued
  * between the two calls (two events on the stream).  Regions nest (up to 8 deep), as tf.time()
  * calls may.  BackendTimingInfo.getExtraProfileInfo (backend.ts:27-31) is fed by the per-kernel

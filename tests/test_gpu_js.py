@@ -1234,3 +1234,14 @@ def test_js_deferred_epilogues():
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-3000:]
     out = json.loads(r.stdout.strip().splitlines()[-1])
     assert out["ok"], out["failures"]
+
+
+def test_js_two_compute_streams():
+    """backend.selectStream: passes queued alternately under the two compute streams, with the
+    reference's op spelling (deferred epilogues), page-locked uploads and asynchronous reads, give
+    the bits of the same passes alone (js/test/streams_test.js)."""
+    r = subprocess.run([NODE, os.path.join(JS, "test", "streams_test.js")], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-3000:]
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert out["ok"], out["failures"]

@@ -395,3 +395,104 @@ def test_time_reports_every_kernel_and_nests(tf):
         assert quiet["kernelTimes"] == [] and quiet["kernelMs"] > 0
     finally:
         be.lib.tfhip_time_per_kernel(be.ctx, 1)
+
+
+# ------------------------------------------------------- two compute streams ----
+def _small_net(tf, x, w1, dw, w2):
+    """conv 3x3 -> depthwise 3x3 -> global mean -> matMul: enough kernels, pool blocks and
+    scratch memory (the product is cut along K) to notice a block handed to the wrong stream."""
+    def run():
+        h = tf.fused.conv2d(x, w1, 1, "same", activation="relu6")
+        h = tf.fused.depthwise_conv2d(h, dw, 1, "same", activation="relu6")
+        h = tf.mean(h, [1, 2])
+        return tf.matmul(h, w2)
+    return tf.tidy(run)
+
+
+def test_two_streams_give_the_results_of_one(tf):
+    """Independent passes queued alternately under the two compute streams (select_stream)
+    overlap on the device; every result equals the one the same pass gives alone, the pools give
+    back what they took, and a read follows the stream its tensor was produced on."""
+    be = tf.backend()
+    rng = np.random.default_rng(31)
+    w1 = tf.tensor((rng.standard_normal((3, 3, 16, 64)) * 0.1).astype(np.float32))
+    dw = tf.tensor((rng.standard_normal((3, 3, 64, 1)) * 0.3).astype(np.float32))
+    w2 = tf.tensor((rng.standard_normal((64, 4096)) * 0.1).astype(np.float32))
+    xs = [rng.uniform(0, 1, (8, 48 + 8 * (i % 3), 40, 16)).astype(np.float32) for i in range(6)]
+    want = []
+    for x in xs:                                   # one stream
+        t = tf.tensor(x)
+        y = _small_net(tf, t, w1, dw, w2)
+        want.append(y.data_sync().copy())
+        tf.dispose([t, y])
+    base = tf.memory()
+    for rounds in range(3):
+        outs = []
+        for i, x in enumerate(xs):                 # two streams, nothing awaited in between
+            be.select_stream(i % 2)
+            t = tf.tensor(x)
+            outs.append(_small_net(tf, t, w1, dw, w2))
+            t.dispose()
+        be.select_stream(0)                        # (reads below are issued under index 0)
+        for i, y in enumerate(outs):
+            got = y.data().result() if i % 2 else y.data_sync()
+            assert np.array_equal(got, want[i]), (rounds, i)
+            y.dispose()
+    after = tf.memory()
+    assert after["numTensors"] == base["numTensors"]
+    assert after["numBytesInGPU"] == base["numBytesInGPU"]
+    tf.dispose([w1, dw, w2])
+
+
+def test_select_stream_rejects_what_it_cannot_do(tf):
+    be = tf.backend()
+    with pytest.raises(RuntimeError, match="2 compute streams"):
+        be.select_stream(2)
+    with pytest.raises(RuntimeError, match="2 compute streams"):
+        be.select_stream(-1)
+    a = tf.tensor(np.ones((4, 4), np.float32))
+    with pytest.raises(RuntimeError, match="timed region"):
+        tf.time(lambda: be.select_stream(1))
+    be.select_stream(1)
+    b = tf.relu(a)                                  # produced under index 1 ...
+    be.select_stream(0)
+    assert b.data_sync().tolist() == a.data_sync().tolist()   # ... read under index 0
+    tf.dispose([a, b])                              # ... and disposed under index 0
+
+
+def test_pipelined_uploads_with_two_batches_in_flight(tf):
+    """The serving loop of the benchmark in small: every step uploads its input from page-locked
+    memory, runs under the stream of its parity and is read back asynchronously two steps late.
+    The next upload never has to take the block whose readers are still queued."""
+    be = tf.backend()
+    rng = np.random.default_rng(32)
+    w1 = tf.tensor((rng.standard_normal((3, 3, 16, 64)) * 0.1).astype(np.float32))
+    dw = tf.tensor((rng.standard_normal((3, 3, 64, 1)) * 0.3).astype(np.float32))
+    w2 = tf.tensor((rng.standard_normal((64, 4096)) * 0.1).astype(np.float32))
+    shape = (32, 64, 64, 16)                       # 8 MiB per batch: an upload on the copy stream
+    slots = [tf.pinned_array("float32", shape) for _ in range(3)]
+    want = []
+    for k, s in enumerate(slots):
+        s[...] = rng.uniform(0, 1, shape).astype(np.float32)
+        t = tf.tensor(s)
+        y = _small_net(tf, t, w1, dw, w2)
+        want.append(y.data_sync().copy())
+        tf.dispose([t, y])
+    pending, got = [], []
+    nxt = tf.tensor(slots[0])
+    n = 24
+    for i in range(n):
+        be.select_stream(i % 2)
+        cur = nxt
+        if i + 1 < n:
+            nxt = tf.tensor(slots[(i + 1) % 3])
+        y = _small_net(tf, cur, w1, dw, w2)
+        pending.append(y.data())
+        tf.dispose([cur, y])
+        if len(pending) > 2:
+            got.append(pending.pop(0).result())
+    got += [p.result() for p in pending]
+    be.select_stream(0)
+    for i, g in enumerate(got):
+        assert np.array_equal(g, want[i % 3]), i
+    tf.dispose([w1, dw, w2])

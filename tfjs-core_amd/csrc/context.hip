@@ -117,7 +117,7 @@ bool tfhip_ctx::next_rec(hipEvent_t* start, hipEvent_t* stop) {
   return true;
 }
 
-Buf* tfhip_ctx::find(int64_t id, bool touch) {
+Buf* tfhip_ctx::find(int64_t id, bool touch, bool on_last_stream) {
   auto it = bufs.find(id);
   if (it == bufs.end()) {
     fail(TFHIP_ENOENT, "unknown data id %lld", (long long)id);
@@ -125,8 +125,9 @@ Buf* tfhip_ctx::find(int64_t id, bool touch) {
   }
   Buf& b = it->second;
   if (touch) {
+    if (!on_last_stream) b.sidx = cur;
     if (b.uploaded) {  // the data is still on its way: the compute stream waits for the copy
-      (void)hipStreamWaitEvent(stream, b.uploaded, 0);
+      (void)hipStreamWaitEvent(streams[b.sidx], b.uploaded, 0);
       ev_put(b.uploaded);
       b.uploaded = nullptr;
     }
@@ -171,11 +172,42 @@ void* tfhip_ctx::alloc(size_t nbytes, size_t* cap, hipEvent_t* ready, bool* recy
   const size_t want = tfhip::round_cap(nbytes);
   if (ready) *ready = nullptr;
   if (recycled) *recycled = false;
+  auto& pool = pools[cur];
   auto it = pool.find(want);
   if (it != pool.end() && !it->second.empty()) {
     // most recently freed block first: it is the one most likely still in L2 / MALL
-    void* p = it->second.back();
-    it->second.pop_back();
+    auto& bucket = it->second;
+    if (ready && !block_ready.empty() && !capturing) {
+      // ... unless it left an event behind that has not fired yet (an upload target whose last
+      // readers are still queued: the next upload into it would wait for them).  Then a block
+      // whose event has fired, or a fresh one while the bucket is small, lets the copy start now.
+      auto pending = [&](void* q) {
+        auto ev = block_ready.find(q);
+        return ev != block_ready.end() && hipEventQuery(ev->second) == hipErrorNotReady;
+      };
+      if (pending(bucket.back())) {
+        size_t pick = bucket.size();
+        for (size_t i = bucket.size() - 1; i-- > 0;)
+          if (!pending(bucket[i])) {
+            pick = i;
+            break;
+          }
+        (void)hipGetLastError();  // (hipErrorNotReady is not an error here)
+        if (pick < bucket.size()) {
+          std::swap(bucket[pick], bucket.back());
+        } else if (bucket.size() < 3) {
+          void* fresh = nullptr;
+          if (hipMalloc(&fresh, want) == hipSuccess) {
+            in_use += want;
+            *cap = want;
+            return fresh;
+          }
+          (void)hipGetLastError();
+        }
+      }
+    }
+    void* p = bucket.back();
+    bucket.pop_back();
     pooled -= want;
     in_use += want;
     *cap = want;
@@ -231,17 +263,17 @@ void* tfhip_ctx::alloc(size_t nbytes, size_t* cap, hipEvent_t* ready, bool* recy
   return p;
 }
 
-void tfhip_ctx::release(void* p, size_t cap, hipEvent_t ready) {
+void tfhip_ctx::release(void* p, size_t cap, hipEvent_t ready, int sidx) {
   if (!p) {
     ev_put(ready);
     return;
   }
   in_use -= cap;
   pooled += cap;
-  park(p, cap, ready);
+  park(p, cap, ready, sidx < 0 ? cur : sidx);
 }
 
-void tfhip_ctx::park(void* p, size_t cap, hipEvent_t ready) {
+void tfhip_ctx::park(void* p, size_t cap, hipEvent_t ready, int sidx) {
   if (ready) {
     auto old = block_ready.find(p);
     if (old != block_ready.end()) ev_put(old->second);
@@ -253,13 +285,13 @@ void tfhip_ctx::park(void* p, size_t cap, hipEvent_t ready) {
     graphs[own->second].parked.emplace_back(p, cap);
     return;
   }
-  pool[cap].push_back(p);
+  pools[sidx][cap].push_back(p);
 }
 
 void tfhip_ctx::unhold(hipEvent_t done) {
   for (size_t i = 0; i < held.size();) {
     if (held[i].done == done) {
-      park(held[i].p, held[i].cap, held[i].left);
+      park(held[i].p, held[i].cap, held[i].left, held[i].sidx);
       held[i] = held.back();
       held.pop_back();
     } else {
@@ -273,8 +305,9 @@ void tfhip_ctx::unhold(hipEvent_t done) {
 // through the upload stream leaves an event behind, so that the next upload into it waits for
 // the kernels that read it and for nothing queued later.
 void tfhip_ctx::release_buf(Buf& b) {
+  hipStream_t last = streams[b.sidx];  // the stream whose pool the block goes back to
   if (b.uploaded) {
-    (void)hipStreamWaitEvent(stream, b.uploaded, 0);
+    (void)hipStreamWaitEvent(last, b.uploaded, 0);
     ev_put(b.uploaded);
   }
   hipEvent_t left = nullptr;
@@ -283,7 +316,7 @@ void tfhip_ctx::release_buf(Buf& b) {
     else left = b.ready;  // never touched: the block's history is still what the event says
   }
   if (!left && b.ptr && b.upload_target && !capturing && (left = ev_get())) {
-    if (hipEventRecord(left, stream) != hipSuccess) {
+    if (hipEventRecord(left, last) != hipSuccess) {
       (void)hipGetLastError();
       ev_put(left);
       left = nullptr;
@@ -295,9 +328,9 @@ void tfhip_ctx::release_buf(Buf& b) {
     // every kernel queued after this dispose for the length of a cross-stream round trip.)
     in_use -= b.cap;
     pooled += b.cap;
-    held.push_back({b.ptr, b.cap, b.read_done, left});
+    held.push_back({b.ptr, b.cap, b.read_done, left, b.sidx});
   } else {
-    release(b.ptr, b.cap, left);
+    release(b.ptr, b.cap, left, b.sidx);
   }
   b.ptr = nullptr;
   b.uploaded = b.read_done = b.ready = nullptr;
@@ -305,18 +338,20 @@ void tfhip_ctx::release_buf(Buf& b) {
 
 void tfhip_ctx::trim() {
   // (not while a graph exists: a replay may still read blocks that went back to the pool)
-  if (pool.empty() || capturing || !graphs.empty()) return;
-  (void)hipStreamSynchronize(stream);
-  for (auto& kv : pool)
-    for (void* p : kv.second) {
-      auto ev = block_ready.find(p);
-      if (ev != block_ready.end()) {
-        ev_put(ev->second);
-        block_ready.erase(ev);
+  if ((pools[0].empty() && pools[1].empty()) || capturing || !graphs.empty()) return;
+  for (hipStream_t st : streams) (void)hipStreamSynchronize(st);
+  for (auto& pool : pools) {
+    for (auto& kv : pool)
+      for (void* p : kv.second) {
+        auto ev = block_ready.find(p);
+        if (ev != block_ready.end()) {
+          ev_put(ev->second);
+          block_ready.erase(ev);
+        }
+        (void)hipFree(p);
       }
-      (void)hipFree(p);
-    }
-  pool.clear();
+    pool.clear();
+  }
   pooled = 0;
   for (const HeldBlock& h : held) pooled += h.cap;  // (they wait for their reads, outside the pool)
 }
@@ -343,20 +378,23 @@ int tfhip_init(int device, tfhip_ctx** out) {
   hipDeviceProp_t prop;
   if ((e = hipSetDevice(device)) != hipSuccess ||
       (e = hipGetDeviceProperties(&prop, device)) != hipSuccess ||
-      (e = hipStreamCreate(&ctx->stream)) != hipSuccess ||
+      (e = hipStreamCreate(&ctx->streams[0])) != hipSuccess ||
+      (e = hipStreamCreate(&ctx->streams[1])) != hipSuccess ||
       (e = hipStreamCreateWithFlags(&ctx->upload, hipStreamNonBlocking)) != hipSuccess ||
       (e = hipStreamCreateWithFlags(&ctx->download, hipStreamNonBlocking)) != hipSuccess) {
     g_init_error = std::string("device set-up failed: ") + hipGetErrorString(e);
-    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    for (hipStream_t st : ctx->streams)
+      if (st) (void)hipStreamDestroy(st);
     if (ctx->upload) (void)hipStreamDestroy(ctx->upload);
     if (ctx->download) (void)hipStreamDestroy(ctx->download);
     delete ctx;
     return TFHIP_EDEVICE;
   }
+  ctx->stream = ctx->streams[0];
   if (std::string(prop.gcnArchName).rfind("gfx950", 0) != 0) {
     g_init_error = std::string("libtfjs_hip is built for gfx950 only, device is ") +
                    prop.gcnArchName;
-    (void)hipStreamDestroy(ctx->stream);
+    for (hipStream_t st : ctx->streams) (void)hipStreamDestroy(st);
     (void)hipStreamDestroy(ctx->upload);
     (void)hipStreamDestroy(ctx->download);
     delete ctx;
@@ -365,7 +403,7 @@ int tfhip_init(int device, tfhip_ctx** out) {
   ctx->num_cus = prop.multiProcessorCount;
   if (tfhip::scratch_init(ctx) != TFHIP_OK) {
     g_init_error = ctx->err;
-    (void)hipStreamDestroy(ctx->stream);
+    for (hipStream_t st : ctx->streams) (void)hipStreamDestroy(st);
     (void)hipStreamDestroy(ctx->upload);
     (void)hipStreamDestroy(ctx->download);
     delete ctx;
@@ -380,7 +418,7 @@ void tfhip_destroy(tfhip_ctx* ctx) {
   (void)hipSetDevice(ctx->device);
   (void)hipStreamSynchronize(ctx->upload);
   (void)hipStreamSynchronize(ctx->download);
-  (void)hipStreamSynchronize(ctx->stream);
+  for (hipStream_t st : ctx->streams) (void)hipStreamSynchronize(st);
   // reads that were begun and not finished keep their ticket (tfhip_read_finish with a NULL
   // context frees it); their events are theirs
   for (auto& kv : ctx->bufs) {
@@ -393,8 +431,9 @@ void tfhip_destroy(tfhip_ctx* ctx) {
   for (hipEvent_t ev : ctx->ring_done)
     if (ev) (void)hipEventDestroy(ev);
   if (ctx->ring) (void)hipHostFree(ctx->ring);
-  for (auto& kv : ctx->pool)
-    for (void* p : kv.second) (void)hipFree(p);
+  for (auto& pool : ctx->pools)
+    for (auto& kv : pool)
+      for (void* p : kv.second) (void)hipFree(p);
   for (auto& h : ctx->held) {
     (void)hipFree(h.p);
     if (h.left) (void)hipEventDestroy(h.left);
@@ -411,7 +450,7 @@ void tfhip_destroy(tfhip_ctx* ctx) {
   }
   (void)hipStreamDestroy(ctx->upload);
   (void)hipStreamDestroy(ctx->download);
-  (void)hipStreamDestroy(ctx->stream);
+  for (hipStream_t st : ctx->streams) (void)hipStreamDestroy(st);
   delete ctx;
 }
 
@@ -441,6 +480,7 @@ int tfhip_register(tfhip_ctx* ctx, int64_t id, const int32_t* shape, int rank, i
     b.ptr = ctx->alloc(b.nbytes, &b.cap, &b.ready, &b.recycled);
     if (!b.ptr) return TFHIP_EDEVICE;
   }
+  b.sidx = ctx->cur;  // (the block came out of this stream's pool)
   ctx->bufs.emplace(id, b);
   return TFHIP_OK;
 }
@@ -480,6 +520,8 @@ int tfhip_write(tfhip_ctx* ctx, int64_t id, const void* host, size_t nbytes) {
       return ctx->fail(TFHIP_EDEVICE, "write: could not create an event");
     char* staged = ctx->ring + (size_t)slot * tfhip_ctx::kSlotBytes;
     memcpy(staged, host, nbytes);
+    // (a small write into a buffer that the other compute stream used last is ordered behind
+    // that use only by the caller: work under different stream indices is independent)
     b = ctx->find(id, /*touch=*/true);  // a copy on the compute stream is a use like any kernel
     if (b->read_done) TFHIP_HIP(ctx, hipStreamWaitEvent(ctx->stream, b->read_done, 0));
     TFHIP_HIP(ctx, hipMemcpyAsync(b->ptr, staged, nbytes, hipMemcpyHostToDevice, ctx->stream));
@@ -490,7 +532,7 @@ int tfhip_write(tfhip_ctx* ctx, int64_t id, const void* host, size_t nbytes) {
   if (b->used || (b->recycled && !b->ready)) {
     hipEvent_t fence = ctx->ev_get();
     if (!fence) return ctx->fail(TFHIP_EDEVICE, "write: could not create an event");
-    hipError_t e = hipEventRecord(fence, ctx->stream);
+    hipError_t e = hipEventRecord(fence, ctx->streams[b->sidx]);  // behind the stream that used it last
     if (e == hipSuccess) e = hipStreamWaitEvent(ctx->upload, fence, 0);
     ctx->ev_put(fence);  // the wait has been queued: the event may be recorded again
     if (e != hipSuccess) return ctx->fail(TFHIP_EDEVICE, "write: %s", hipGetErrorString(e));
@@ -521,12 +563,13 @@ int tfhip_write(tfhip_ctx* ctx, int64_t id, const void* host, size_t nbytes) {
 int tfhip_read(tfhip_ctx* ctx, int64_t id, void* host, size_t nbytes) {
   if (!ctx) return TFHIP_EINVAL;
   if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "read: not during a graph capture");
-  TFHIP_GET(ctx, b, id);
+  Buf* b = ctx->find(id, /*touch=*/true, /*on_last_stream=*/true);
+  if (!b) return TFHIP_ENOENT;
   if (nbytes != b->nbytes)
     return ctx->fail(TFHIP_EINVAL, "read: asked %zu bytes of a buffer of %zu", nbytes, b->nbytes);
-  if (nbytes)
-    TFHIP_HIP(ctx, hipMemcpyAsync(host, b->ptr, nbytes, hipMemcpyDeviceToHost, ctx->stream));
-  TFHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  hipStream_t last = ctx->streams[b->sidx];  // the stream that produced (or last used) the buffer
+  if (nbytes) TFHIP_HIP(ctx, hipMemcpyAsync(host, b->ptr, nbytes, hipMemcpyDeviceToHost, last));
+  TFHIP_HIP(ctx, hipStreamSynchronize(last));
   return TFHIP_OK;
 }
 
@@ -535,7 +578,8 @@ int tfhip_read_begin(tfhip_ctx* ctx, int64_t id, tfhip_pending_read** out) {
   if (!ctx || !out) return TFHIP_EINVAL;
   *out = nullptr;
   if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "read: not during a graph capture");
-  TFHIP_GET(ctx, b, id);
+  Buf* b = ctx->find(id, /*touch=*/true, /*on_last_stream=*/true);
+  if (!b) return TFHIP_ENOENT;
   tfhip_pending_read* r = new tfhip_pending_read();
   r->device = ctx->device;
   r->nbytes = b->nbytes;
@@ -545,7 +589,7 @@ int tfhip_read_begin(tfhip_ctx* ctx, int64_t id, tfhip_pending_read** out) {
     r->done = ctx->ev_get();
     hipError_t e = (r->staging && produced && r->done) ? hipSuccess : hipErrorOutOfMemory;
     // the copy runs on the download stream, behind the kernels queued so far and no others
-    if (e == hipSuccess) e = hipEventRecord(produced, ctx->stream);
+    if (e == hipSuccess) e = hipEventRecord(produced, ctx->streams[b->sidx]);
     if (e == hipSuccess) e = hipStreamWaitEvent(ctx->download, produced, 0);
     if (e == hipSuccess)
       e = hipMemcpyAsync(r->staging, b->ptr, b->nbytes, hipMemcpyDeviceToHost, ctx->download);
@@ -655,7 +699,19 @@ int tfhip_sync(tfhip_ctx* ctx) {
   if (!ctx) return TFHIP_EINVAL;
   if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "sync: not during a graph capture");
   TFHIP_HIP(ctx, hipStreamSynchronize(ctx->upload));  // pinned sources are free again after this
-  TFHIP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  for (hipStream_t st : ctx->streams) TFHIP_HIP(ctx, hipStreamSynchronize(st));
+  return TFHIP_OK;
+}
+
+int tfhip_select_stream(tfhip_ctx* ctx, int index) {
+  if (!ctx) return TFHIP_EINVAL;
+  if (index < 0 || index >= tfhip_ctx::kStreams)
+    return ctx->fail(TFHIP_EINVAL, "select_stream: index %d, there are %d compute streams", index,
+                     tfhip_ctx::kStreams);
+  if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "select_stream: not during a graph capture");
+  if (ctx->time_depth) return ctx->fail(TFHIP_EINVAL, "select_stream: not inside a timed region");
+  ctx->cur = index;
+  ctx->stream = ctx->streams[index];
   return TFHIP_OK;
 }
 
@@ -748,16 +804,17 @@ int tfhip_graph_end(tfhip_ctx* ctx, int64_t* graph_id) {
   for (void* p : ctx->capture_blocks) {
     if (ctx->owner.count(p)) continue;
     ctx->owner[p] = id;
-    for (auto& kv : ctx->pool) {
-      auto& v = kv.second;
-      for (size_t i = 0; i < v.size(); i++) {
-        if (v[i] != p) continue;
-        v.erase(v.begin() + i);
-        ctx->pooled -= kv.first;
-        g.parked.emplace_back(p, kv.first);
-        break;
+    for (auto& pool : ctx->pools)
+      for (auto& kv : pool) {
+        auto& v = kv.second;
+        for (size_t i = 0; i < v.size(); i++) {
+          if (v[i] != p) continue;
+          v.erase(v.begin() + i);
+          ctx->pooled -= kv.first;
+          g.parked.emplace_back(p, kv.first);
+          break;
+        }
       }
-    }
   }
   ctx->capture_blocks.clear();
   ctx->graphs.emplace(id, std::move(g));
@@ -783,12 +840,12 @@ int tfhip_graph_destroy(tfhip_ctx* ctx, int64_t graph_id) {
   auto it = ctx->graphs.find(graph_id);
   if (it == ctx->graphs.end()) return TFHIP_OK;
   // queued replays may still run: wait before the blocks can be handed to anyone else
-  (void)hipStreamSynchronize(ctx->stream);
+  for (hipStream_t st : ctx->streams) (void)hipStreamSynchronize(st);
   (void)hipGraphExecDestroy(it->second.exec);
   (void)hipGraphDestroy(it->second.graph);
   for (auto& blk : it->second.parked) {
     ctx->pooled += blk.second;
-    ctx->pool[blk.second].push_back(blk.first);
+    ctx->pools[ctx->cur][blk.second].push_back(blk.first);  // (every stream is idle now)
   }
   for (auto o = ctx->owner.begin(); o != ctx->owner.end();)
     o = o->second == graph_id ? ctx->owner.erase(o) : std::next(o);

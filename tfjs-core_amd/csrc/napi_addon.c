@@ -254,6 +254,15 @@ static napi_value js_sync(napi_env env, napi_callback_info info) {
   return undefined(env);
 }
 
+/* selectStream(ctx, index) */
+static napi_value js_select_stream(napi_env env, napi_callback_info info) {
+  ARGS(2);
+  int index;
+  if (!arg_int(env, argv[1], &index)) return NULL;
+  CHECK(tfhip_select_stream(ctx, index));
+  return undefined(env);
+}
+
 static napi_value js_time_begin(napi_env env, napi_callback_info info) {
   ARGS(1);
   CHECK(tfhip_time_begin(ctx));
@@ -831,7 +840,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
   static const struct { const char* name; napi_callback fn; } fns[] = {
       {"init", js_init}, {"destroy", js_destroy}, {"register", js_register},
       {"write", js_write}, {"read", js_read}, {"dispose", js_dispose},
-      {"memInfo", js_mem_info}, {"sync", js_sync}, {"timeBegin", js_time_begin},
+      {"memInfo", js_mem_info}, {"sync", js_sync}, {"selectStream", js_select_stream}, {"timeBegin", js_time_begin},
       {"timeEnd", js_time_end}, {"timeKernels", js_time_kernels},
       {"timePerKernel", js_time_per_kernel}, {"hostAlloc", js_host_alloc},
       {"readAsync", js_read_async}, {"lastKernel", js_last_kernel}, {"matmul", js_matmul}, {"matmulNoalloc", js_matmul_noalloc},

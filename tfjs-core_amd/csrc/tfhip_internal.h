@@ -35,6 +35,7 @@ struct Buf {
   bool recycled = false;           // the block came out of the pool (its history is unknown)
   bool used = false;               // queued work may have touched the buffer since it was written
   bool upload_target = false;      // written through the upload stream: worth an event on release
+  int sidx = 0;                    // compute stream (tfhip_select_stream) of the last queued use
 };
 
 inline size_t dtype_size(int dtype) {
@@ -77,6 +78,7 @@ struct tfhip_ctx {
     void* p;
     size_t cap;
     hipEvent_t done, left;
+    int sidx;  // the compute stream whose pool the block returns to
   };
   std::vector<HeldBlock> held;
   // Small writes travel through a ring of pinned slots on the compute stream itself.
@@ -87,7 +89,15 @@ struct tfhip_ctx {
   int ring_next = 0;
   std::unordered_map<tfhip_pending_read*, int64_t> reads;  // asynchronous reads not yet finished
   std::unordered_map<int64_t, tfhip::Buf> bufs;
-  std::map<size_t, std::vector<void*>> pool;  // capacity -> free blocks, reused LIFO
+  // Two compute streams (tfhip_select_stream): work queued under one index runs in order, work
+  // under different indices is not ordered against each other, so that two independent passes
+  // (two batches of a serving loop) share the machine.  `stream` is the selected one.  Every
+  // stream has a pool of its own: a block goes back to the pool of the stream that used it last,
+  // where the next owner is ordered behind that use by the stream itself.
+  static constexpr int kStreams = 2;
+  hipStream_t streams[kStreams] = {nullptr, nullptr};
+  int cur = 0;  // index of `stream`
+  std::map<size_t, std::vector<void*>> pools[kStreams];  // capacity -> free blocks, reused LIFO
   size_t in_use = 0, pooled = 0;
   std::string err;
   char last_kernel[96] = "";  // variant chosen by the last dense / image launch
@@ -172,12 +182,15 @@ struct tfhip_ctx {
   int fail(int code, const char* fmt, ...);
   // Looks an id up (sets err when missing).  `touch` = the caller queues work on the compute
   // stream that reads or writes the buffer: a pending upload is waited for first.
-  tfhip::Buf* find(int64_t id, bool touch = true);
+  // touch: the caller queues work that uses the buffer, on the selected compute stream, or (for
+  // host reads of a buffer, which follow its producer) on the stream that used it last.
+  tfhip::Buf* find(int64_t id, bool touch = true, bool on_last_stream = false);
   // nullptr + err on failure (nbytes > 0).  *ready receives the event that the block's last
   // owner left with it, or nullptr; *recycled whether the block was used before.
   void* alloc(size_t nbytes, size_t* cap, hipEvent_t* ready = nullptr, bool* recycled = nullptr);
-  void release(void* p, size_t cap, hipEvent_t ready = nullptr);
-  void park(void* p, size_t cap, hipEvent_t ready);  // release() after the accounting
+  // (sidx: the compute stream that used the block last; -1 = the selected one)
+  void release(void* p, size_t cap, hipEvent_t ready = nullptr, int sidx = -1);
+  void park(void* p, size_t cap, hipEvent_t ready, int sidx);  // release() after the accounting
   void unhold(hipEvent_t done);                       // held blocks of a finished read -> pool
   void release_buf(tfhip::Buf& b);
   int await_uploads();  // the compute stream waits for every upload still on its way

@@ -345,6 +345,14 @@ class MathBackendHIP extends KernelBackend {
     this.flushAll();
     this.napi.sync(this.ctx);
   }
+  // hip extension: the compute stream (0 or 1) that the kernels of the following ops are queued
+  // on.  Two independent passes queued under the two indices may overlap on the device; a tensor
+  // written under one index is not ordered against work under the other (read it, or sync(),
+  // in between).  What was deferred so far is launched under the index it was issued under.
+  selectStream(index) {
+    this.flushAll();
+    this.napi.selectStream(this.ctx, index);
+  }
   lastKernel() {
     this.flushAll();
     return this.napi.lastKernel(this.ctx);

@@ -57,11 +57,15 @@ async function main() {
   const resident = rate(now() - t0);
   resident.host_dispatch_ms_per_step = queued / steps;
   // ---- end to end, pipelined ---------------------------------------------------------------
-  const pipelined = async n => {
+  // `streams` = 2: batch i runs on compute stream i % 2 of the backend, so that two batches are
+  // in flight and each fills the phases in which the other leaves the machine idle (kernel
+  // boundaries, the tails of launches, matrix-bound kernels beside memory-bound ones).
+  const pipelined = async (n, streams) => {
     const pending = [];
     let last = null;
     let next = tf.tensor(slots[0], shape);
     for (let i = 0; i < n; i++) {
+      if (streams > 1) be.selectStream(i % streams);
       const cur = next;
       if (i + 1 < n) next = tf.tensor(slots[(i + 1) % 2], shape);   // overlaps with the step below
       const out = mobilenet.forward(tf, w, cur);
@@ -72,12 +76,33 @@ async function main() {
       if (pending.length > 2) last = await pending.shift();
     }
     while (pending.length) last = await pending.shift();
+    if (streams > 1) be.selectStream(0);
     return last;
   };
-  await pipelined(Math.max(4, warmup));
+  await pipelined(Math.max(4, warmup), 1);
   t0 = now();
-  const lastProbs = await pipelined(steps);
+  const lastProbsOne = await pipelined(steps, 1);
+  const endToEndOne = rate(now() - t0);
+  await pipelined(Math.max(4, warmup), 2);
+  t0 = now();
+  const lastProbs = await pipelined(steps, 2);
   const endToEnd = rate(now() - t0);
+  endToEnd.batches_in_flight = 2;
+  // the input resident, two batches in flight
+  const two = n => {
+    for (let i = 0; i < n; i++) {
+      be.selectStream(i % 2);
+      step(mobilenet.forward);
+    }
+    be.selectStream(0);
+  };
+  two(Math.max(4, warmup));
+  be.sync();
+  t0 = now();
+  two(steps);
+  be.sync();
+  const residentTwo = rate(now() - t0);
+  residentTwo.batches_in_flight = 2;
 
 
   const info = await tf.time(() => { for (let i = 0; i < steps; i++) step(mobilenet.forward); });
@@ -140,6 +165,9 @@ async function main() {
     blockDiff = Math.max(blockDiff, Math.abs(eagerProbs[i] - blockingProbs[i]));
   }
   endToEnd.max_abs_diff_vs_resident = pipeDiff;
+  let oneDiff = 0;
+  for (let i = 0; i < eagerProbs.length; i++) oneDiff = Math.max(oneDiff, Math.abs(eagerProbs[i] - lastProbsOne[i]));
+  endToEndOne.max_abs_diff_vs_resident = oneDiff;
 
   // ---- captured graph ------------------------------------------------------------------------
   const graph = tf.captureGraph(() => mobilenet.forward(tf, w, x).probs);
@@ -158,7 +186,7 @@ async function main() {
   console.log(JSON.stringify({
     batch, steps, warmup, node: process.version, top1_first: top[0],
     tensors: tf.memory().numTensors,
-    end_to_end: endToEnd,
+    end_to_end: endToEnd, end_to_end_one_stream: endToEndOne, resident_two_streams: residentTwo,
     end_to_end_blocking: {images_per_s: batch * nBlocking / (blockingMs / 1e3),
                           ms_per_step: blockingMs / nBlocking, steps: nBlocking,
                           max_abs_diff_vs_resident: blockDiff},

@@ -45,6 +45,7 @@ _SIGNATURES = {
     "tfhip_dispose": [_PTR, _I64],
     "tfhip_mem_info": [_PTR, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "tfhip_sync": [_PTR],
+    "tfhip_select_stream": [_PTR, _INT],
     "tfhip_time_begin": [_PTR],
     "tfhip_time_end": [_PTR, C.POINTER(C.c_float)],
     "tfhip_time_per_kernel": [_PTR, _INT],

@@ -188,6 +188,12 @@ class MathBackendHIP(object):
     def sync(self):
         self._ck(self.lib.tfhip_sync(self.ctx))
 
+    def select_stream(self, index):
+        """Work queued from now on goes to compute stream `index` (0 or 1) of the context (hip
+        extension): two independent passes queued under the two indices may overlap on the device.
+        A tensor written under one index is not ordered against work under the other."""
+        self._ck(self.lib.tfhip_select_stream(self.ctx, int(index)))
+
     def capture_graph(self, f, tidy):
         """Records the kernels that f() queues into a graph that replays with one launch (an
         extension: the reference's backends run every op eagerly).  f runs twice: once eagerly, so
