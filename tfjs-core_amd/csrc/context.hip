@@ -164,6 +164,16 @@ hipEvent_t tfhip_ctx::ev_get() {
   return ev;
 }
 
+namespace tfhip {
+static hipError_t create_streams(hipStream_t* out, int n) {
+  for (int i = 0; i < n; i++) {
+    hipError_t e = hipStreamCreate(&out[i]);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+}  // namespace tfhip
+
 void* tfhip_ctx::alloc(size_t nbytes, size_t* cap, hipEvent_t* ready, bool* recycled) {
   if (no_alloc) {  // a mistake in the library, not in the caller: fail instead of allocating
     fail(TFHIP_EDEVICE, "internal: a no-alloc entry point asked the pool for %zu bytes", nbytes);
@@ -338,7 +348,9 @@ void tfhip_ctx::release_buf(Buf& b) {
 
 void tfhip_ctx::trim() {
   // (not while a graph exists: a replay may still read blocks that went back to the pool)
-  if ((pools[0].empty() && pools[1].empty()) || capturing || !graphs.empty()) return;
+  bool any = false;
+  for (auto& pool : pools) any = any || !pool.empty();
+  if (!any || capturing || !graphs.empty()) return;
   for (hipStream_t st : streams) (void)hipStreamSynchronize(st);
   for (auto& pool : pools) {
     for (auto& kv : pool)
@@ -378,8 +390,7 @@ int tfhip_init(int device, tfhip_ctx** out) {
   hipDeviceProp_t prop;
   if ((e = hipSetDevice(device)) != hipSuccess ||
       (e = hipGetDeviceProperties(&prop, device)) != hipSuccess ||
-      (e = hipStreamCreate(&ctx->streams[0])) != hipSuccess ||
-      (e = hipStreamCreate(&ctx->streams[1])) != hipSuccess ||
+      (e = tfhip::create_streams(ctx->streams, tfhip_ctx::kStreams)) != hipSuccess ||
       (e = hipStreamCreateWithFlags(&ctx->upload, hipStreamNonBlocking)) != hipSuccess ||
       (e = hipStreamCreateWithFlags(&ctx->download, hipStreamNonBlocking)) != hipSuccess) {
     g_init_error = std::string("device set-up failed: ") + hipGetErrorString(e);

@@ -95,7 +95,7 @@ struct tfhip_ctx {
   // stream has a pool of its own: a block goes back to the pool of the stream that used it last,
   // where the next owner is ordered behind that use by the stream itself.
   static constexpr int kStreams = 2;
-  hipStream_t streams[kStreams] = {nullptr, nullptr};
+  hipStream_t streams[kStreams] = {};
   int cur = 0;  // index of `stream`
   std::map<size_t, std::vector<void*>> pools[kStreams];  // capacity -> free blocks, reused LIFO
   size_t in_use = 0, pooled = 0;
