@@ -300,6 +300,32 @@ def test_kwaves_hands_over_what_it_does_not_take(tf):
         close(got, a64 @ b64, atol=1e-4)
 
 
+@pytest.mark.parametrize("m,k,n,act,bias_kind", [
+    (12544, 512, 512, "relu6", "full"),      # bias with one value per output element
+    (12544, 512, 512, "prelu", "scalar"),    # scalar bias, per-column slope
+    (3137, 1024, 1000, "relu", "column"),    # ragged last tile row and column
+])
+def test_leftover_tiles_as_pieces_with_every_epilogue(tf, m, k, n, act, bias_kind):
+    """Products whose tiles leave a remainder after whole rounds of one tile per CU: the leftover
+    tiles run as 16 x 16 pieces in the same launch (_tail16); their epilogue is the general one
+    (every bias layout, prelu), checked against a float64 contraction."""
+    print("tail16", m, k, n, act, bias_kind, flush=True)
+    rng = np.random.default_rng(m + 3 * k + 7 * n)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = (rng.standard_normal((k, n)) * np.sqrt(2.0 / k)).astype(np.float32)
+    bias = {"scalar": np.float32(0.3), "column": rng.standard_normal(n).astype(np.float32),
+            "full": rng.standard_normal((m, n)).astype(np.float32)}[bias_kind]
+    alpha = rng.uniform(0.1, 0.5, n).astype(np.float32) if act == "prelu" else None
+    with tf.tidy():
+        got = tf.fused.matmul(tf.tensor(a), tf.tensor(b), bias=tf.tensor(bias), activation=act,
+                              prelu_activation_weights=None if alpha is None else tf.tensor(alpha)
+                              ).data_sync()
+        assert last_kernel(tf).endswith("_tail16"), last_kernel(tf)
+    y = a.astype(np.float64) @ b.astype(np.float64) + bias
+    y = np.where(y < 0, alpha * y, y) if act == "prelu" else act64(y, act)
+    close(got, y, atol=1e-4)
+
+
 def test_implicit_gemm_3x3_tiles(tf):
     """3x3 convolutions through the im2col loaders at sizes that take the 64x64 and wider
     tiles, against float64 on sampled output positions."""
