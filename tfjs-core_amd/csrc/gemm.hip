@@ -364,10 +364,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     if (A_UNIFORM_K) {
       const bool cut = k0 + BK > p.K;
       const __amdgpu_buffer_rsrc_t r = k0 < p.K ? rsrc_a : rsrc_a_none;
+      // (a branch, the same for the whole workgroup, instead of a select per item: the select
+      // would run on the vector ALU in every k step, the branch is scalar)
+      if (cut) {
 #pragma unroll
-      for (int i = 0; i < A_PER; i++)
-        reg[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                     r, (int)(cut ? L.a_voff_cut[i] : L.a_voff[i]), k0 * 4, 0));
+        for (int i = 0; i < A_PER; i++)
+          reg[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                       r, (int)L.a_voff_cut[i], k0 * 4, 0));
+      } else {
+#pragma unroll
+        for (int i = 0; i < A_PER; i++)
+          reg[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                       r, (int)L.a_voff[i], k0 * 4, 0));
+      }
       return;
     }
     if (FAST) {
@@ -514,7 +523,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       const int soff = BMODE == B_TRANSPOSED ? k0 * 4 : BMODE == B_UINT8 ? k0 * p.ldb : k0 * p.ldb * 4;
 #pragma unroll
       for (int i = 0; i < B_PER; i++) {
-        const unsigned voff = cut ? L.b_voff_cut[i] : L.b_voff[i];
+        // (a row-major B needs no second set: its rows at or beyond K lie beyond the descriptor's
+        // range by themselves, (k * ldb + n) * size >= K * ldb * size >= b_bytes)
+        const unsigned voff = BMODE == B_TRANSPOSED && cut ? L.b_voff_cut[i] : L.b_voff[i];
         if (BMODE == B_UINT8) {
           // The four bytes stay as they are until store_b turns them into floats on their way
           // into LDS, so nothing waits for this load here.  An item out of range reads 0 and
