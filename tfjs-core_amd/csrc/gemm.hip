@@ -357,26 +357,30 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   // A tile that starts at k0 lies wholly below K, is cut by K, or lies beyond it (a load issued
   // ahead of the last step): the same for all lanes, so the choice between the two offset sets
   // is one select and a tile beyond K reads through the descriptor of length 0.
-  auto load_a = [&](const Loader& L, int k0_, f32x4 (&reg)[A_PER]) {
+  auto load_a = [&](Loader& L, int k0_, f32x4 (&reg)[A_PER]) {
     // (k0 is the same for the whole workgroup; saying so keeps the descriptor and the scalar
     // offset in scalar registers wherever the compiler cannot see it)
     const int k0 = FAST ? __builtin_amdgcn_readfirstlane(k0_) : k0_;
     if (A_UNIFORM_K) {
       const bool cut = k0 + BK > p.K;
       const __amdgpu_buffer_rsrc_t r = k0 < p.K ? rsrc_a : rsrc_a_none;
-      // (a branch, the same for the whole workgroup, instead of a select per item: the select
-      // would run on the vector ALU in every k step, the branch is scalar)
+      // (the steps of a workgroup go up in k, so once a tile is cut every later one is cut or
+      // beyond K: the cut set replaces the other for good, under a branch that is the same for
+      // the whole workgroup.  A select per item would run on the vector ALU, which shares its
+      // pipe with the matrix cores, in every k step; the empty asm keeps the compiler from
+      // turning the branch back into that select.)
       if (cut) {
 #pragma unroll
-        for (int i = 0; i < A_PER; i++)
-          reg[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                       r, (int)L.a_voff_cut[i], k0 * 4, 0));
-      } else {
-#pragma unroll
-        for (int i = 0; i < A_PER; i++)
-          reg[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                       r, (int)L.a_voff[i], k0 * 4, 0));
+        for (int i = 0; i < A_PER; i++) {
+          unsigned v = L.a_voff_cut[i];
+          asm volatile("" : "+v"(v));
+          L.a_voff[i] = v;
+        }
       }
+#pragma unroll
+      for (int i = 0; i < A_PER; i++)
+        reg[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                     r, (int)L.a_voff[i], k0 * 4, 0));
       return;
     }
     if (FAST) {
@@ -515,17 +519,26 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   };
 
   // B items: B_ROWMAJOR / B_UINT8: (k, col-quad); B_TRANSPOSED: (col, k-quad)
-  auto load_b = [&](const Loader& L, int k0_, f32x4 (&reg)[B_PER]) {
+  auto load_b = [&](Loader& L, int k0_, f32x4 (&reg)[B_PER]) {
     const int k0 = FAST ? __builtin_amdgcn_readfirstlane(k0_) : k0_;
     if (FAST) {
       const bool cut = k0 + BK > p.K;
       const __amdgpu_buffer_rsrc_t r = k0 < p.K ? rsrc_b : rsrc_b_none;
       const int soff = BMODE == B_TRANSPOSED ? k0 * 4 : BMODE == B_UINT8 ? k0 * p.ldb : k0 * p.ldb * 4;
+      // (a row-major B needs no second set: its rows at or beyond K lie beyond the descriptor's
+      // range by themselves, (k * ldb + n) * size >= K * ldb * size >= b_bytes; a transposed
+      // one switches sets for good like A)
+      if (BMODE == B_TRANSPOSED && cut) {
+#pragma unroll
+        for (int i = 0; i < B_PER; i++) {
+          unsigned v = L.b_voff_cut[i];
+          asm volatile("" : "+v"(v));
+          L.b_voff[i] = v;
+        }
+      }
 #pragma unroll
       for (int i = 0; i < B_PER; i++) {
-        // (a row-major B needs no second set: its rows at or beyond K lie beyond the descriptor's
-        // range by themselves, (k * ldb + n) * size >= K * ldb * size >= b_bytes)
-        const unsigned voff = BMODE == B_TRANSPOSED && cut ? L.b_voff_cut[i] : L.b_voff[i];
+        const unsigned voff = L.b_voff[i];
         if (BMODE == B_UINT8) {
           // The four bytes stay as they are until store_b turns them into floats on their way
           // into LDS, so nothing waits for this load here.  An item out of range reads 0 and
