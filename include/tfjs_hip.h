@@ -123,10 +123,13 @@ int tfhip_sync(tfhip_ctx* ctx);
  * queued under one index runs in the order of the calls; work under different indices is not
  * ordered against each other and may overlap on the device: two independent passes (batch i
  * under index 0, batch i + 1 under index 1 of a serving loop) then fill each other's idle
- * phases.  A buffer written under one index must not be used under the other before the host
- * has waited for it (tfhip_sync, or a read of it); buffers that are only read (weights) may be
- * shared.  tfhip_read / tfhip_read_begin follow the buffer's own stream, tfhip_sync waits for
- * both.  Not inside a timed region or a graph capture. */
+ * phases.  What orders them is the buffers they share: a stream that meets a buffer whose
+ * contents were written under another index waits, once per buffer, for the work queued under that
+ * index so far (an event, no host wait), and a block goes back to the pool behind the work of
+ * every stream that used it.  Buffers that are only read (weights) cost nothing to share.
+ * tfhip_read / tfhip_read_begin follow the buffer's own stream, tfhip_sync waits for both, a
+ * captured graph replays on the stream it was recorded on.  Not inside a timed region or a graph
+ * capture. */
 int tfhip_select_stream(tfhip_ctx* ctx, int index);
 /* KernelBackend.time (backend.ts:92, backend_cpu.ts:239-244): device time of the work queued
  * between the two calls (two events on the stream).  Regions nest (up to 8 deep), as tf.time()
@@ -155,7 +158,7 @@ int tfhip_time_kernel(tfhip_ctx* ctx, int index, const char** name, float* ms);
  *                      hold every block the work needs (run it once before capturing it).
  *   tfhip_graph_end    stops recording and returns a graph id.  The blocks the recorded work
  *                      used stay out of the pool while the graph lives: a replay writes them again.
- *   tfhip_graph_launch queues one replay.  The tensors the recorded work read that were created
+ *   tfhip_graph_launch queues one replay (on the compute stream of the capture).  The tensors the recorded work read that were created
  *                      before the capture (weights, the input) must still exist; new input data is
  *                      written into the same tensor with tfhip_write.  Results appear in the buffers
  *                      of the tensors the recorded work produced.

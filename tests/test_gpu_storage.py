@@ -460,6 +460,60 @@ def test_select_stream_rejects_what_it_cannot_do(tf):
     tf.dispose([a, b])                              # ... and disposed under index 0
 
 
+def test_tensor_handed_from_one_stream_to_the_other(tf):
+    """A tensor produced under one stream index and used under the other right away: the second
+    stream waits for the first one's work (no host wait in between), so the result is the one a
+    single stream gives.  The pool blocks are filled with other values first, so that a kernel
+    that ran ahead of its input would read those."""
+    be = tf.backend()
+    rng = np.random.default_rng(33)
+    n = 3072
+    a = tf.tensor(rng.standard_normal((n, n)).astype(np.float32) * 0.05)
+    w = tf.tensor(rng.standard_normal((n, n)).astype(np.float32) * 0.05)
+    with tf.tidy():
+        want = tf.relu(tf.matmul(tf.matmul(a, w), w)).data_sync().copy()
+    for rounds in range(2):
+        tf.dispose([tf.fill((n, n), -1.0) for _ in range(3)])
+        be.select_stream(0)
+        p = tf.matmul(a, w)                         # a chain of long kernels under index 0 ...
+        q = tf.matmul(p, w)
+        be.select_stream(1)
+        r = tf.relu(q)                              # ... and their result used under index 1
+        be.select_stream(0)
+        got = r.data_sync()
+        assert np.array_equal(got, want), rounds
+        tf.dispose([p, q, r])
+    tf.dispose([a, w])
+
+
+def test_block_used_under_both_streams_returns_behind_both(tf):
+    """A tensor that work under both stream indices reads is disposed and its block taken again
+    at once under the index that used it last: the new owner is ordered behind the other stream's
+    readers too."""
+    be = tf.backend()
+    rng = np.random.default_rng(34)
+    n = 3072
+    a = tf.tensor(rng.standard_normal((n, n)).astype(np.float32) * 0.05)
+    w = tf.tensor(rng.standard_normal((n, n)).astype(np.float32) * 0.05)
+    with tf.tidy():
+        want = tf.matmul(tf.relu(a), w).data_sync().copy()
+    for rounds in range(2):
+        be.select_stream(0)
+        b = tf.relu(a)
+        be.select_stream(1)
+        busy = tf.tidy(lambda: tf.matmul(tf.matmul(a, w), w))   # keeps index 1 busy: b is read late
+        c = tf.matmul(b, w)                         # reads b under index 1
+        be.select_stream(0)
+        d = tf.neg(b)                               # b's last use is under index 0
+        b.dispose()
+        e = tf.fill((n, n), 7.0)                    # takes b's block from the pool of index 0
+        assert np.array_equal(c.data_sync(), want), rounds
+        assert float(e.data_sync().flat[0]) == 7.0
+        tf.dispose([busy, c, d, e])
+    be.select_stream(0)
+    tf.dispose([a, w])
+
+
 def test_pipelined_uploads_with_two_batches_in_flight(tf):
     """The serving loop of the benchmark in small: every step uploads its input from page-locked
     memory, runs under the stream of its parity and is read back asynchronously two steps late.

@@ -125,11 +125,28 @@ Buf* tfhip_ctx::find(int64_t id, bool touch, bool on_last_stream) {
   }
   Buf& b = it->second;
   if (touch) {
-    if (!on_last_stream) b.sidx = cur;
-    if (b.uploaded) {  // the data is still on its way: the compute stream waits for the copy
-      (void)hipStreamWaitEvent(streams[b.sidx], b.uploaded, 0);
+    if (b.uploaded) {  // the data is still on its way: the compute streams wait for the copy
+      all_wait(b.uploaded);
       ev_put(b.uploaded);
       b.uploaded = nullptr;
+      b.wsidx = -1;
+      b.vis = kAllStreams;
+    }
+    if (!on_last_stream) {
+      // Work under different stream indices is ordered through the buffers it shares.  The
+      // first queued work on a buffer is what writes it (tensors are written once); a stream
+      // that meets contents written under another index waits, once, for that stream's work
+      // queued so far.
+      const unsigned char bit = (unsigned char)(1u << cur);
+      if (!b.vis) {
+        b.wsidx = cur;
+        b.vis = bit;
+      } else if (!(b.vis & bit)) {
+        if (b.wsidx >= 0) order(b.wsidx, cur);
+        b.vis |= bit;
+      }
+      b.users |= bit;
+      b.sidx = cur;
     }
     if (b.ready) {  // from here on the block is ordered by the compute stream alone
       ev_put(b.ready);
@@ -143,11 +160,33 @@ Buf* tfhip_ctx::find(int64_t id, bool touch, bool on_last_stream) {
 int tfhip_ctx::await_uploads() {
   for (auto& kv : bufs) {
     if (!kv.second.uploaded) continue;
-    TFHIP_HIP(this, hipStreamWaitEvent(stream, kv.second.uploaded, 0));
+    all_wait(kv.second.uploaded);
     ev_put(kv.second.uploaded);
     kv.second.uploaded = nullptr;
+    kv.second.wsidx = -1;
+    kv.second.vis = kAllStreams;
   }
   return TFHIP_OK;
+}
+
+void tfhip_ctx::all_wait(hipEvent_t uploaded) {
+  for (hipStream_t st : streams)
+    if (hipStreamWaitEvent(st, uploaded, 0) != hipSuccess) (void)hipGetLastError();
+}
+
+void tfhip_ctx::order(int earlier, int later) {
+  if (earlier == later) return;
+  hipEvent_t ev = capturing ? nullptr : ev_get();
+  if (ev && hipEventRecord(ev, streams[earlier]) == hipSuccess &&
+      hipStreamWaitEvent(streams[later], ev, 0) == hipSuccess) {
+    ev_put(ev);  // the wait has been queued: the event may be recorded again
+    return;
+  }
+  // (a stream under capture cannot wait for an event from outside the capture, and without an
+  // event there is nothing to wait for: the host waits instead)
+  (void)hipGetLastError();
+  ev_put(ev);
+  (void)hipStreamSynchronize(streams[earlier]);
 }
 
 hipEvent_t tfhip_ctx::ev_get() {
@@ -316,6 +355,9 @@ void tfhip_ctx::unhold(hipEvent_t done) {
 // the kernels that read it and for nothing queued later.
 void tfhip_ctx::release_buf(Buf& b) {
   hipStream_t last = streams[b.sidx];  // the stream whose pool the block goes back to
+  // (work of the other streams on the block comes before whatever that stream does with it next)
+  for (int s = 0; s < kStreams; s++)
+    if (s != b.sidx && (b.users >> s & 1) && b.ptr) order(s, b.sidx);
   if (b.uploaded) {
     (void)hipStreamWaitEvent(last, b.uploaded, 0);
     ev_put(b.uploaded);
@@ -531,9 +573,12 @@ int tfhip_write(tfhip_ctx* ctx, int64_t id, const void* host, size_t nbytes) {
       return ctx->fail(TFHIP_EDEVICE, "write: could not create an event");
     char* staged = ctx->ring + (size_t)slot * tfhip_ctx::kSlotBytes;
     memcpy(staged, host, nbytes);
-    // (a small write into a buffer that the other compute stream used last is ordered behind
-    // that use only by the caller: work under different stream indices is independent)
     b = ctx->find(id, /*touch=*/true);  // a copy on the compute stream is a use like any kernel
+    // (and a write: behind the other streams' work on the old contents, and theirs to wait for)
+    for (int s = 0; s < tfhip_ctx::kStreams; s++)
+      if (s != ctx->cur && (b->users >> s & 1)) ctx->order(s, ctx->cur);
+    b->wsidx = ctx->cur;
+    b->vis = b->users = (unsigned char)(1u << ctx->cur);
     if (b->read_done) TFHIP_HIP(ctx, hipStreamWaitEvent(ctx->stream, b->read_done, 0));
     TFHIP_HIP(ctx, hipMemcpyAsync(b->ptr, staged, nbytes, hipMemcpyHostToDevice, ctx->stream));
     TFHIP_HIP(ctx, hipEventRecord(ctx->ring_done[slot], ctx->stream));
@@ -543,9 +588,15 @@ int tfhip_write(tfhip_ctx* ctx, int64_t id, const void* host, size_t nbytes) {
   if (b->used || (b->recycled && !b->ready)) {
     hipEvent_t fence = ctx->ev_get();
     if (!fence) return ctx->fail(TFHIP_EDEVICE, "write: could not create an event");
-    hipError_t e = hipEventRecord(fence, ctx->streams[b->sidx]);  // behind the stream that used it last
-    if (e == hipSuccess) e = hipStreamWaitEvent(ctx->upload, fence, 0);
-    ctx->ev_put(fence);  // the wait has been queued: the event may be recorded again
+    // behind every stream with work on the block (the one that got it, when none is known)
+    const unsigned char users = b->users ? b->users : (unsigned char)(1u << b->sidx);
+    hipError_t e = hipSuccess;
+    for (int s = 0; s < tfhip_ctx::kStreams && e == hipSuccess; s++) {
+      if (!(users >> s & 1)) continue;
+      e = hipEventRecord(fence, ctx->streams[s]);
+      if (e == hipSuccess) e = hipStreamWaitEvent(ctx->upload, fence, 0);
+    }
+    ctx->ev_put(fence);  // the waits have been queued: the event may be recorded again
     if (e != hipSuccess) return ctx->fail(TFHIP_EDEVICE, "write: %s", hipGetErrorString(e));
   } else if (b->ready) {
     TFHIP_HIP(ctx, hipStreamWaitEvent(ctx->upload, b->ready, 0));
@@ -556,6 +607,9 @@ int tfhip_write(tfhip_ctx* ctx, int64_t id, const void* host, size_t nbytes) {
   b->used = false;
   b->recycled = false;
   b->upload_target = true;
+  b->users = 0;
+  b->wsidx = -1;
+  b->vis = tfhip_ctx::kAllStreams;  // (with an upload on its way, find() makes every stream wait for it)
   TFHIP_HIP(ctx, hipMemcpyAsync(b->ptr, host, nbytes, hipMemcpyHostToDevice, ctx->upload));
   if (!tfhip::host_is_pinned(host, nbytes)) {
     // the copy reads the caller's pages until it is done, and the caller may change or free
@@ -810,6 +864,7 @@ int tfhip_graph_end(tfhip_ctx* ctx, int64_t* graph_id) {
     return ctx->fail(TFHIP_EDEVICE, "graph capture failed: %s", hipGetErrorString(e));
   }
   const int64_t id = ctx->next_graph++;
+  g.sidx = ctx->cur;
   // Every block the capture handed out now belongs to the graph: those lying free in the pool
   // are taken out of it, the others follow when their tensor lets go of them (release()).
   for (void* p : ctx->capture_blocks) {
@@ -842,7 +897,9 @@ int tfhip_graph_launch(tfhip_ctx* ctx, int64_t graph_id) {
   // through the upload stream has to arrive first
   int rc = ctx->await_uploads();
   if (rc) return rc;
-  TFHIP_HIP(ctx, hipGraphLaunch(it->second.exec, ctx->stream));
+  // (on the stream of the capture, whichever is selected: the tensors the recorded work
+  // produced are booked as written there)
+  TFHIP_HIP(ctx, hipGraphLaunch(it->second.exec, ctx->streams[it->second.sidx]));
   return TFHIP_OK;
 }
 

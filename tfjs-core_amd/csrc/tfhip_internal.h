@@ -36,6 +36,10 @@ struct Buf {
   bool used = false;               // queued work may have touched the buffer since it was written
   bool upload_target = false;      // written through the upload stream: worth an event on release
   int sidx = 0;                    // compute stream (tfhip_select_stream) of the last queued use
+  // Ordering between the compute streams, one bit per stream:
+  int wsidx = -1;                  // the stream whose queued work wrote the contents (-1: a copy did)
+  unsigned char vis = 0;           // streams that are ordered behind that write (0: nothing written yet)
+  unsigned char users = 0;         // streams with queued work on the block since the buffer got it
 };
 
 inline size_t dtype_size(int dtype) {
@@ -90,11 +94,12 @@ struct tfhip_ctx {
   std::unordered_map<tfhip_pending_read*, int64_t> reads;  // asynchronous reads not yet finished
   std::unordered_map<int64_t, tfhip::Buf> bufs;
   // Two compute streams (tfhip_select_stream): work queued under one index runs in order, work
-  // under different indices is not ordered against each other, so that two independent passes
-  // (two batches of a serving loop) share the machine.  `stream` is the selected one.  Every
+  // under different indices is ordered only through the buffers it shares (find()), so that two
+  // independent passes (two batches of a serving loop) share the machine.  `stream` is the selected one.  Every
   // stream has a pool of its own: a block goes back to the pool of the stream that used it last,
   // where the next owner is ordered behind that use by the stream itself.
-  static constexpr int kStreams = 2;
+  static constexpr int kStreams = 2;  // (at most 8: Buf keeps a bit per stream)
+  static constexpr unsigned char kAllStreams = (unsigned char)((1u << kStreams) - 1);
   hipStream_t streams[kStreams] = {};
   int cur = 0;  // index of `stream`
   std::map<size_t, std::vector<void*>> pools[kStreams];  // capacity -> free blocks, reused LIFO
@@ -168,6 +173,7 @@ struct tfhip_ctx {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     std::vector<std::pair<void*, size_t>> parked;  // owned blocks that no tensor holds
+    int sidx = 0;  // the compute stream it was recorded on, and replays on
   };
   bool capturing = false;
   std::vector<void*> capture_blocks;
@@ -195,7 +201,11 @@ struct tfhip_ctx {
   void park(void* p, size_t cap, hipEvent_t ready, int sidx);  // release() after the accounting
   void unhold(hipEvent_t done);                       // held blocks of a finished read -> pool
   void release_buf(tfhip::Buf& b);
-  int await_uploads();  // the compute stream waits for every upload still on its way
+  int await_uploads();  // the compute streams wait for every upload still on its way
+  // Puts compute stream `later` behind everything queued on compute stream `earlier` so far.
+  void order(int earlier, int later);
+  // Every compute stream waits for the copy that `uploaded` stands for.
+  void all_wait(hipEvent_t uploaded);
   void trim();
 };
 

@@ -347,8 +347,9 @@ class MathBackendHIP extends KernelBackend {
   }
   // hip extension: the compute stream (0 or 1) that the kernels of the following ops are queued
   // on.  Two independent passes queued under the two indices may overlap on the device; a tensor
-  // written under one index is not ordered against work under the other (read it, or sync(),
-  // in between).  What was deferred so far is launched under the index it was issued under.
+  // written under one index and used under the other makes that stream wait for the work queued
+  // under the first index so far, and nothing else orders the two.  What was deferred so far is
+  // launched under the index it was issued under.
   selectStream(index) {
     this.flushAll();
     this.napi.selectStream(this.ctx, index);

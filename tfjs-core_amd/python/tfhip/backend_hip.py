@@ -191,7 +191,8 @@ class MathBackendHIP(object):
     def select_stream(self, index):
         """Work queued from now on goes to compute stream `index` (0 or 1) of the context (hip
         extension): two independent passes queued under the two indices may overlap on the device.
-        A tensor written under one index is not ordered against work under the other."""
+        A tensor written under one index and used under the other makes that stream wait for
+        the work queued under the first index so far; nothing else orders the two."""
         self._ck(self.lib.tfhip_select_stream(self.ctx, int(index)))
 
     def capture_graph(self, f, tidy):
