@@ -127,6 +127,9 @@ int tfhip_sync(tfhip_ctx* ctx);
  * contents were written under another index waits, once per buffer, for the work queued under that
  * index so far (an event, no host wait), and a block goes back to the pool behind the work of
  * every stream that used it.  Buffers that are only read (weights) cost nothing to share.
+ * (The contents of a buffer count as written by the first work queued on it, or by tfhip_write:
+ * tensors are written once.  A caller that has a kernel overwrite a live buffer under another
+ * index than the one that wrote it first orders that itself, with tfhip_sync.)
  * tfhip_read / tfhip_read_begin follow the buffer's own stream, tfhip_sync waits for both, a
  * captured graph replays on the stream it was recorded on.  Not inside a timed region or a graph
  * capture. */

@@ -1245,3 +1245,13 @@ def test_js_two_compute_streams():
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-3000:]
     out = json.loads(r.stdout.strip().splitlines()[-1])
     assert out["ok"], out["failures"]
+
+
+def test_js_from_pixels_and_to_pixels():
+    """tf.browser.fromPixels / toPixels: the reference's DOM-free cases (a canvas-like object,
+    PixelData, every toPixels case and error) on the hip backend (js/test/pixels_test.js)."""
+    r = subprocess.run([NODE, os.path.join(JS, "test", "pixels_test.js")], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-3000:]
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert out["ok"], out["failures"]

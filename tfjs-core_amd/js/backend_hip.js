@@ -370,8 +370,38 @@ class MathBackendHIP extends KernelBackend {
     }
   }
 
-  fromPixels() {
-    throw new Error('fromPixels is a browser-only entry point; not available in the hip backend');
+  // KernelBackend.fromPixels (backend.ts:86-90; backend_cpu.ts:130-195): RGBA bytes ->
+  // int32 [height, width, numChannels].  Without a DOM the pixels come as
+  // {data: Uint8Array | Uint8ClampedArray, width, height} (PixelData, ImageData) or from an
+  // object with getContext('2d').getImageData (the canvas of the `canvas` package, which is what
+  // the reference asks for under Node); image and video elements need a browser.
+  fromPixels(pixels, numChannels) {
+    if (pixels == null) throw new Error('pixels passed to tf.browser.fromPixels() can not be null');
+    let vals;
+    if (typeof pixels.getContext === 'function') {
+      vals = pixels.getContext('2d').getImageData(0, 0, pixels.width, pixels.height).data;
+    } else if (pixels.data instanceof Uint8Array || pixels.data instanceof Uint8ClampedArray) {
+      vals = pixels.data;
+    } else {
+      throw new Error(
+          'pixels passed to tf.browser.fromPixels() must be either an HTMLVideoElement, HTMLImageElement, ' +
+          'HTMLCanvasElement, ImageData or {data: Uint32Array, width: number, height: number}, but was ' +
+          (pixels.constructor != null ? pixels.constructor.name : typeof pixels));
+    }
+    const numPixels = pixels.width * pixels.height;
+    if (vals.length < numPixels * 4) {
+      throw new Error(`fromPixels: ${vals.length} bytes are not ${pixels.width} x ${pixels.height} RGBA pixels`);
+    }
+    let values;
+    if (numChannels === 4) {
+      values = new Int32Array(vals.subarray(0, numPixels * 4));
+    } else {
+      values = new Int32Array(numPixels * numChannels);
+      for (let i = 0; i < numPixels; i++) {
+        for (let c = 0; c < numChannels; ++c) values[i * numChannels + c] = vals[i * 4 + c];
+      }
+    }
+    return this.fromHost(values, [pixels.height, pixels.width, numChannels], 'int32');
   }
 
   // ---- helpers ----

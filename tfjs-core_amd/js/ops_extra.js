@@ -756,6 +756,67 @@ async function inTopKAsync(predictions, targets, k) {
   return res;
 }
 const nextFrame = () => new Promise(resolve => setImmediate(resolve));
+// tf.browser (ops/browser.ts:46-56, 75-170): pixels -> int32 tensor and back to RGBA bytes
+const fromPixels = op('fromPixels', (pixels, numChannels) => {
+  if (numChannels == null) numChannels = 3;
+  if (numChannels > 4) throw new Error('Cannot construct Tensor with more than 4 channels from pixels.');
+  return ENGINE.runKernel(backend => backend.fromPixels(pixels, numChannels), {});
+});
+async function toPixels(img, canvas) {
+  let $img = convertToTensor(img, 'img', 'toPixels');
+  if (!(img instanceof Tensor)) {
+    const asInt = cast($img, 'int32');  // a native array is taken to hold int32 values
+    $img.dispose();
+    $img = asInt;
+  }
+  try {
+    if ($img.rank !== 2 && $img.rank !== 3) {
+      throw new Error(`toPixels only supports rank 2 or 3 tensors, got rank ${$img.rank}.`);
+    }
+    const height = $img.shape[0], width = $img.shape[1];
+    const depth = $img.rank === 2 ? 1 : $img.shape[2];
+    if (depth > 4 || depth === 2) {
+      throw new Error(`toPixels only supports depth of size 1, 3 or 4 but got ${depth}`);
+    }
+    if ($img.dtype !== 'float32' && $img.dtype !== 'int32') {
+      throw new Error(`Unsupported type for toPixels: ${$img.dtype}. Please use float32 or int32 tensors.`);
+    }
+    const data = await $img.data();
+    let min = Infinity, max = -Infinity;
+    for (let i = 0; i < data.length; i++) {
+      if (data[i] < min) min = data[i];
+      if (data[i] > max) max = data[i];
+    }
+    const top = $img.dtype === 'float32' ? 1 : 255;
+    if (min < 0 || max > top) {
+      throw new Error(`Tensor values for a ${$img.dtype} Tensor must be in the range [0 - ${top}] but got range [${min} - ${max}].`);
+    }
+    const multiplier = $img.dtype === 'float32' ? 255 : 1;
+    const bytes = new Uint8ClampedArray(width * height * 4);
+    for (let i = 0; i < height * width; ++i) {
+      const j = i * 4;
+      if (depth === 1) {
+        bytes[j] = bytes[j + 1] = bytes[j + 2] = Math.round(data[i] * multiplier);
+        bytes[j + 3] = 255;
+      } else {
+        for (let c = 0; c < 3; c++) bytes[j + c] = Math.round(data[i * depth + c] * multiplier);
+        bytes[j + 3] = depth === 4 ? Math.round(data[i * 4 + 3] * multiplier) : 255;
+      }
+    }
+    if (canvas != null) {
+      canvas.width = width;
+      canvas.height = height;
+      const ctx = canvas.getContext('2d');
+      const imageData = typeof ImageData !== 'undefined' ? new ImageData(bytes, width, height) :
+                                                           ctx.createImageData(width, height);
+      if (imageData.data !== bytes) imageData.data.set(bytes);
+      ctx.putImageData(imageData, 0, 0);
+    }
+    return bytes;
+  } finally {
+    if ($img !== img) $img.dispose();
+  }
+}
 // expectArraysClose of test_util.ts:22-39, 121-138 (absolute epsilon 1e-3 on a 32-bit backend)
 const test_util = {
   expectArraysClose(actual, expected, epsilon) {
@@ -772,6 +833,7 @@ const test_util = {
 
 module.exports = Object.assign({}, strictOps, aliases, {
   TensorBuffer, buffer, print, tensor5d, tensor6d, setdiff1dAsync, inTopKAsync, nextFrame, test_util,
+  browser: {fromPixels, toPixels}, fromPixels, toPixels,
   version_core: '1.2.7-hip',
   signal: {hannWindow, hammingWindow, frame, stft},
   spectral: {fft, ifft, rfft, irfft},
