@@ -377,6 +377,70 @@ def test_matmul_odd_row_lengths(tf, m, k, n, ta, tb):
     close(got, want, atol=1e-4)
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_shapes_against_float64(tf, seed):
+    """Seeded random shapes (sizes on and off every tile, vector and k-block boundary; both
+    transposes; batches; bias + activation; 1x1 and 3x3 convolutions at both strides) against a
+    float64 contraction of the same inputs: whatever variant the planner picks, the result is
+    within tolerance of the exact one, scaled to the largest magnitude of the result (sums of up
+    to 1500 float32 products)."""
+    rng = np.random.default_rng(seed)
+    sizes = [1, 3, 4, 16, 17, 33, 64, 100, 128, 200, 256, 300, 512, 777, 1024, 1500]
+    seen = set()
+    for it in range(240):
+        kind = it % 3
+        if kind == 0:
+            m, n, k = (int(rng.choice(sizes)) for _ in range(3))
+            if rng.random() < 0.3:
+                m *= int(rng.integers(1, 9))
+            b = int(rng.choice([1, 1, 1, 2, 3]))
+            ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+            a_ = rng.standard_normal((b, k, m) if ta else (b, m, k)).astype(np.float32)
+            b_ = rng.standard_normal((b, n, k) if tb else (b, k, n)).astype(np.float32)
+            with tf.tidy():
+                got = tf.matmul(tf.tensor(a_), tf.tensor(b_), ta, tb).data_sync()
+            want = (a_.transpose(0, 2, 1) if ta else a_).astype(np.float64) @ \
+                   (b_.transpose(0, 2, 1) if tb else b_).astype(np.float64)
+            what = ("matmul", b, m, n, k, ta, tb)
+        elif kind == 1:
+            m, n, k = (int(rng.choice([1, 4, 10, 16, 48, 64, 100, 128, 196, 256, 512, 784, 1000, 1024, 3136]))
+                       for _ in range(3))
+            a_ = rng.standard_normal((m, k)).astype(np.float32)
+            b_ = (rng.standard_normal((k, n)) * 0.1).astype(np.float32)
+            bias = rng.standard_normal((n,)).astype(np.float32)
+            act = str(rng.choice(["linear", "relu", "relu6"]))
+            with tf.tidy():
+                got = tf.fused.matmul(tf.tensor(a_), tf.tensor(b_), False, False, bias=tf.tensor(bias),
+                                      activation=act).data_sync()
+            want = act64(a_.astype(np.float64) @ b_.astype(np.float64) + bias, act)
+            what = ("fused matmul", m, n, k, act)
+        else:
+            nb, h, w_ = int(rng.choice([1, 2, 5, 8])), int(rng.choice([1, 7, 14, 15, 28])), int(rng.choice([7, 14, 16, 29]))
+            ci, co = int(rng.choice([3, 4, 8, 20, 32, 64, 128, 256])), int(rng.choice([8, 10, 32, 64, 100, 128, 512]))
+            f, st = int(rng.choice([1, 1, 3])), int(rng.choice([1, 2]))
+            x = rng.standard_normal((nb, h, w_, ci)).astype(np.float32)
+            wt = (rng.standard_normal((f, f, ci, co)) * 0.1).astype(np.float32)
+            bias = rng.standard_normal((co,)).astype(np.float32)
+            with tf.tidy():
+                got = tf.fused.conv2d(tf.tensor(x), tf.tensor(wt), st, "same", bias=tf.tensor(bias),
+                                      activation="relu6").data_sync()
+            oh, ow = -(-h // st), -(-w_ // st)
+            ph, pw = max((oh - 1) * st + f - h, 0), max((ow - 1) * st + f - w_, 0)
+            xp = np.zeros((nb, h + ph, w_ + pw, ci))
+            xp[:, ph // 2:ph // 2 + h, pw // 2:pw // 2 + w_] = x
+            want = np.zeros((nb, oh, ow, co))
+            for kh in range(f):
+                for kw in range(f):
+                    want += xp[:, kh:kh + (oh - 1) * st + 1:st, kw:kw + (ow - 1) * st + 1:st] @ wt[kh, kw].astype(np.float64)
+            want = act64(want + bias, "relu6")
+            what = ("conv2d", nb, h, w_, ci, co, f, st)
+        seen.add(last_kernel(tf))
+        got = np.asarray(got, np.float64).reshape(want.shape)
+        err = np.abs(got - want).max()
+        assert err <= 1e-4 * max(np.abs(want).max(), 1.0), (what, last_kernel(tf), err)
+    assert len(seen) >= 15, seen    # (the cases do spread over the variants)
+
+
 def test_batched_matmul_odd_strides(tf):
     rng = np.random.default_rng(77)
     a = rng.uniform(-1, 1, (3, 9, 7)).astype(np.float32)
