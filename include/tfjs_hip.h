@@ -225,8 +225,10 @@ int tfhip_conv2d(tfhip_ctx* ctx, int64_t x, int64_t filter, int64_t out,
  * out [batch,out_h,out_w,out_c].  Biases NONE / SCALAR / COLUMN, activations LINEAR / RELU /
  * RELU6; either filter may be TFHIP_UINT8Q with its qparams.  For 3x3 filters, multiplier 1 and
  * (channels, stride) in {(32->64, 1), (64->128, 2), (128->128, 1)} on large images one kernel computes both
- * halves and the intermediate never reaches HBM; every other shape runs the two kernels with
- * the intermediate in a pool block.  Results are those of the two calls (the single kernel sums
+ * halves and the intermediate never reaches HBM; so does another for small problems (float32, 3x3,
+ * 32 <= channels <= 1024, at most two tiles of 16 pixels x 64 output columns per CU: the layers of a
+ * network for one or a few images); every other shape runs the two kernels with
+ * the intermediate in a pool block.  Results are those of the two calls (the single kernels may sum
  * the pointwise products in another order: equal within float32 round-off).
  * tfhip_separable_single_kernel(ctx, 0) forces the two-kernel form (1 restores the default). */
 int tfhip_separable_conv2d(tfhip_ctx* ctx, int64_t x, int64_t dw_filter, int64_t pw_filter,

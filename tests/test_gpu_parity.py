@@ -886,7 +886,10 @@ def _separable_oracle(ref, x, dw, pw, stride, dbias, dact, pbias, pact):
     ((33, 55, 57, 128), 256, 2),    # K 128 -> N 256 at stride 2: two kernels
     ((17, 113, 111, 32), 64, 1),    # odd extents: blocks straddle rows and images, last block short
     ((66, 111, 113, 64), 128, 2),   # stride 2 on odd extents (padding 1 on both sides)
-    ((2, 20, 20, 32), 64, 1),       # too few pixels for the single kernel: two-kernel form
+    ((2, 20, 20, 32), 64, 1),       # too few pixels for the panel-walking kernel: the small-problem kernel
+    ((3, 56, 56, 128), 128, 1),     # too many tiles for that one, too few panels for the other: two kernels
+    ((1, 7, 7, 1024), 1024, 1),     # small, but 16 column tiles would each repeat 1024 channels: two kernels
+    ((1, 14, 14, 512), 1024, 2),
     ((1, 9, 9, 12), 20, 2),         # channel counts without a single-kernel variant
 ])
 def test_separable_conv2d_matches_the_two_op_chain(hip, ref, xs, cout, stride):
@@ -919,8 +922,11 @@ def test_separable_conv2d_matches_the_two_op_chain(hip, ref, xs, cout, stride):
         got, kernels = run(dact, pact, db, pb)
         single = len(kernels) == 1 and kernels[0].startswith("separable_")
         pixels = xs[0] * -(-xs[1] // stride) * -(-xs[2] // stride)
-        expect_single = pixels >= 256 * 8 * 32 * 3 and \
-            (c, cout, stride) in ((32, 64, 1), (64, 128, 2), (128, 128, 1))
+        tiles = -(-pixels // 16) * -(-cout // 64)       # the small-problem kernel: 16 pixels x 64 columns
+        small = c >= 32 and c % 4 == 0 and cout % 4 == 0 and tiles <= 512 and \
+            not (tiles < 128 and c * -(-cout // 64) > 4096)
+        expect_single = small or (pixels >= 256 * 8 * 32 * 3 and
+                                  (c, cout, stride) in ((32, 64, 1), (64, 128, 2), (128, 128, 1)))
         assert single == expect_single, kernels
         want = _separable_oracle(ref, x[pick], dw, pw, stride, db, dact, pb, pact)
         close(got[pick], want)
@@ -932,6 +938,64 @@ def test_separable_conv2d_matches_the_two_op_chain(hip, ref, xs, cout, stride):
                 be.lib.tfhip_separable_single_kernel(be.ctx, 1)
             assert len(kernels2) == 2, kernels2
             close(got, two, rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("xs,cout,stride", [
+    ((1, 14, 14, 512), 512, 1),     # the 512 -> 512 blocks of a single image
+    ((1, 28, 28, 256), 256, 1),
+    ((1, 28, 28, 256), 512, 2),
+    ((1, 14, 14, 1024), 256, 1),    # K = 1024: the panel takes 64 KiB of LDS
+    ((2, 14, 14, 512), 512, 1),     # two images
+    ((1, 56, 56, 64), 128, 2),      # K = 64: half of the wavefronts have a share of K
+    ((1, 15, 13, 64), 100, 1),      # columns that end inside a tile, pixels that end inside a tile
+    ((1, 5, 5, 96), 36, 2),
+    ((1, 20, 20, 32), 64, 1),       # K = 32: two wavefronts have a share of K
+    ((3, 9, 11, 200), 72, 1),       # K that the wavefronts share unevenly
+])
+def test_separable_conv2d_small_problems_in_one_kernel(hip, ref, xs, cout, stride):
+    """Small depthwise + pointwise pairs (the layers of a network for one or two images) run as
+    one kernel of 16-pixel x 64-column tiles: against the oracle's chain, and against the backend's
+    own two-kernel form (bit for bit where that form's product shares K among wavefronts in the
+    same way), with every bias layout and activation it folds."""
+    print("separable small", xs, cout, stride, flush=True)
+    tf = hip.tf
+    be = tf.backend()
+    rng = rng_for("separable-small", xs, cout, stride)
+    c = xs[3]
+    x = rng.uniform(0, 1, xs).astype(np.float32)
+    x[0, 0, 0, :3] = np.nan, np.inf, -np.inf if c >= 3 else 0    # (carried like the two kernels carry them)
+    dw = (rng.standard_normal((3, 3, c, 1)) * np.sqrt(2.0 / 9)).astype(np.float32)
+    pw = (rng.standard_normal((1, 1, c, cout)) * np.sqrt(2.0 / c)).astype(np.float32)
+    dbias = (rng.standard_normal(c) * 0.1).astype(np.float32)
+    pbias = (rng.standard_normal(cout) * 0.1).astype(np.float32)
+    out = []
+
+    def run(dact, pact, db, pb, xv):
+        with tf.tidy():
+            t = lambda a: None if a is None else tf.tensor(a)
+            info = tf.time(lambda: out.append(tf.fused.separable_conv2d(
+                t(xv), t(dw), t(pw), stride, "same", depthwise_bias=t(db),
+                depthwise_activation=dact, bias=t(pb), activation=pact)))
+            return out.pop().data_sync(), [k[0] for k in info["kernelTimes"]]
+
+    finite = np.nan_to_num(x, nan=0.5, posinf=0.25, neginf=0.75)
+    for dact, pact, db, pb in (("relu6", "relu6", dbias, pbias), ("linear", "relu", None, pbias),
+                               ("relu", "linear", dbias[:1], pbias[:1]), ("relu6", "linear", dbias, None)):
+        got, kernels = run(dact, pact, db, pb, finite)
+        assert kernels == ["separable_small_s%d_f32" % stride], kernels
+        close(got, _separable_oracle(ref, finite, dw, pw, stride, db, dact, pb, pact))
+        for xv in (finite, x):
+            one, _ = run(dact, pact, db, pb, xv)
+            be.lib.tfhip_separable_single_kernel(be.ctx, 0)
+            try:
+                two, kernels2 = run(dact, pact, db, pb, xv)
+            finally:
+                be.lib.tfhip_separable_single_kernel(be.ctx, 1)
+            assert len(kernels2) == 2, kernels2
+            if kernels2[1] == "gemm_16x16_kwaves_f32":   # K shared by the wavefronts in the same way
+                assert np.array_equal(one, two, equal_nan=True), (dact, pact, kernels2)
+            else:                                        # (short K: the tiled product sums in another order)
+                close(one, two, rtol=2e-5, atol=2e-6)
 
 
 @pytest.mark.parametrize("xs,cout,name", [

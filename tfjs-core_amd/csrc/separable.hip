@@ -539,6 +539,217 @@ static int launch_separable(tfhip_ctx* ctx, SepArgs& p) {
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// The same pair for a small problem (the layers of a network from 28 x 28 pixels down for one or
+// two images): the tiled kernels above need thousands of panels to fill the machine, and as two
+// launches the pair costs two kernels of 4 to 6 us each that are all latency.  Here a workgroup of
+// 8 wavefronts owns a tile of 16 pixels x 64 output columns:
+//   1. all 512 lanes compute the depthwise result of the 16 pixels over all K channels (an item
+//      is one pixel x 4 channels: 9 range-checked 16-byte loads, taps summed in the order filter
+//      row, filter column, bias, activation) into a panel [16][K + 4] in LDS.  The N / 64
+//      workgroups of a pixel tile each do this again: 9 x 16 x K multiply-adds, next to nothing;
+//   2. wavefront w multiplies columns k_per * w .. of the panel by the matching rows of the
+//      pointwise filter, which it reads straight from memory, 16 bytes per lane = the lane's
+//      column in each of the tile's four blocks (block c holds columns n0 + 4 j + c), with
+//      v_mfma_f32_16x16x4f32 into two accumulator chains per block;
+//   3. the 8 partial tiles meet in LDS and are added in wavefront order (fixed, so the result
+//      does not depend on scheduling), then bias, activation and a 16-byte store per lane.
+// K is shared by the wavefronts exactly as the one-launch kernel for small products shares it,
+// so the result has the bits of the two-kernel form.
+struct SepSmallArgs {
+  const float* x;
+  const float* dw;   // [3][3][K]
+  const float* dwb;
+  const float* pw;   // [K][N]
+  const float* pwb;
+  float* y;
+  int H, W, OH, OW, K, N, S, pt, pl;
+  int M;             // batch * OH * OW pixels
+  int tiles_m, tiles_n, k_per, by_columns;
+  int dwb_kind, pwb_kind, dw_act, pw_act;
+  unsigned x_bytes, pw_bytes;
+};
+
+__global__ __launch_bounds__(512) void separable_small_kernel(const SepSmallArgs p) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];  // the panel, then the partial tiles
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15, kq = lane >> 4;
+  const int K = p.K, N = p.N, PITCH = K + 4;
+  // Workgroup b runs on XCD b % 8.  by_columns (at least 8 tile columns): an XCD takes every
+  // eighth tile column with all its pixel tiles, so that a line of the filter enters one L2.
+  int tm = (int)blockIdx.x / p.tiles_n, tn = (int)blockIdx.x % p.tiles_n;
+  if (p.by_columns) {
+    const int xcd = (int)blockIdx.x & 7, j = (int)blockIdx.x >> 3;
+    tn = xcd + 8 * (j / p.tiles_m);
+    tm = j % p.tiles_m;
+    if (tn >= p.tiles_n) return;
+  }
+  const int m0 = tm * 16, n0 = tn * 64;
+
+  // ---- 1. depthwise: 16 pixels x K channels into the panel ----
+  {
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.x, p.x_bytes);
+    const Clamp dact = clamp_of(p.dw_act);
+    const int QN = K >> 2;
+    auto filter_of = [&](int quad, f32x4 (&w)[9], f32x4& b) {
+#pragma unroll
+      for (int t = 0; t < 9; t++) w[t] = *reinterpret_cast<const f32x4*>(p.dw + t * K + 4 * quad);
+      b = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (p.dwb_kind == TFHIP_BCAST_COLUMN) b = *reinterpret_cast<const f32x4*>(p.dwb + 4 * quad);
+      else if (p.dwb_kind == TFHIP_BCAST_SCALAR) b = f32x4{p.dwb[0], p.dwb[0], p.dwb[0], p.dwb[0]};
+    };
+    auto pixel = [&](int px, int quad, const f32x4 (&w)[9], const f32x4& b) {
+      const int m = m0 + px;
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (m < p.M) {
+        const int ow = m % p.OW, r = m / p.OW;
+        const int oh = r % p.OH, n = r / p.OH;
+        const int ih0 = oh * p.S - p.pt, iw0 = ow * p.S - p.pl;
+        f32x4 in[9];
+#pragma unroll
+        for (int t = 0; t < 9; t++) {
+          const int ih = ih0 + t / 3, iw = iw0 + t % 3;
+          const bool ok = (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+          in[t] = buffer_load_f32x4(rx, ok ? (unsigned)((((n * p.H + ih) * p.W + iw) * K + 4 * quad) * 4) : OOB_OFFSET);
+        }
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < 9; t++) acc += in[t] * w[t];
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = clamp(acc[e] + b[e], dact);
+      }
+      *reinterpret_cast<f32x4*>(lds + px * PITCH + 4 * quad) = v;
+    };
+    f32x4 w[9], b;
+    if (512 % QN == 0) {
+      // every item of a lane has the lane's channel quad: its nine filter taps are read once
+      const int quad = tid % QN, step = 512 / QN;
+      filter_of(quad, w, b);
+      for (int px = tid / QN; px < 16; px += step) pixel(px, quad, w, b);
+    } else {
+      for (int item = tid; item < 16 * QN; item += 512) {
+        const int px = item / QN, quad = item - px * QN;
+        filter_of(quad, w, b);
+        pixel(px, quad, w, b);
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- 2. pointwise: this wavefront's share of K ----
+  constexpr int G = 2;
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.pw, p.pw_bytes);
+  const unsigned b_at = n0 + 4 * l16 < N ? (unsigned)((4 * kq * N + n0 + 4 * l16) * 4) : OOB_OFFSET;
+  const float* const a_at = lds + l16 * PITCH + 4 * kq;
+  const int k_begin = wave * p.k_per;
+  const int k_end = min(K, k_begin + p.k_per);
+  const int groups = k_end > k_begin ? (k_end - k_begin + 15) >> 4 : 0;
+  struct Operands {
+    f32x4 a[G];
+    f32x4 b[G][4];  // [e]: row k0 + 4 kq + e of the filter, the lane's column in blocks 0..3
+  };
+  auto load = [&](int q0, Operands& o) {
+#pragma unroll
+    for (int u = 0; u < G; u++) {
+      if (q0 + u >= groups) break;
+      const int k0 = k_begin + 16 * (q0 + u);
+      const bool in = k0 + 4 * kq < k_end;  // (whole groups of 4: K is a multiple of 4)
+      o.a[u] = in ? *reinterpret_cast<const f32x4*>(a_at + k0) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        o.b[u][e] = buffer_load_f32x4(rb, in ? b_at + (unsigned)((k0 + e) * N) * 4 : OOB_OFFSET);
+    }
+  };
+  f32x4 acc[4][2];
+#pragma unroll
+  for (int c = 0; c < 4; c++) acc[c][0] = acc[c][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto multiply = [&](int q0, const Operands& o) {
+#pragma unroll
+    for (int u = 0; u < G; u++) {
+      if (q0 + u >= groups) break;
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+          acc[c][e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(o.a[u][e], o.b[u][e][c], acc[c][e & 1], 0, 0, 0);
+    }
+  };
+  Operands o0, o1;
+  load(0, o0);
+  for (int q0 = 0; q0 < groups; q0 += 2 * G) {
+    load(q0 + G, o1);
+    multiply(q0, o0);
+    load(q0 + 2 * G, o0);
+    multiply(q0 + G, o1);
+  }
+  __syncthreads();  // every wavefront has read its part of the panel: the partial tiles take its place
+
+  // ---- 3. partial tiles, epilogue ----
+#pragma unroll
+  for (int c = 0; c < 4; c++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) lds[((wave * 4 + c) * 4 + r) * 64 + lane] = acc[c][0][r] + acc[c][1][r];
+  __syncthreads();
+  if (tid >= 256) return;
+  // accumulator register r of lane l is pixel 4 * (l / 16) + r, column 4 * (l % 16) + c of block c
+  const int r = tid >> 6;
+  const int row = m0 + 4 * kq + r, col = n0 + 4 * l16;
+  f32x4 v;
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    float s = lds[(c * 4 + r) * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < 8; w++) s += lds[((w * 4 + c) * 4 + r) * 64 + lane];
+    v[c] = s;
+  }
+  if (row >= p.M || col >= N) return;
+  const Clamp pact = clamp_of(p.pw_act);
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    float b = 0.f;
+    if (p.pwb_kind == TFHIP_BCAST_COLUMN) b = p.pwb[col + c];
+    else if (p.pwb_kind == TFHIP_BCAST_SCALAR) b = p.pwb[0];
+    v[c] = clamp(v[c] + b, pact);
+  }
+  *reinterpret_cast<f32x4*>(p.y + (long long)row * N + col) = v;
+}
+
+// Whether and how the small kernel takes the pair; -1 when it does not.
+static int launch_separable_small(tfhip_ctx* ctx, SepSmallArgs& p) {
+  if (p.K < 32 || p.K > 1024 || (p.K & 3) || (p.N & 3)) return -1;
+  const long long tiles = ceil_div(p.M, 16) * ceil_div(p.N, 64);
+  // Where it pays (measured against the two-kernel form, the layers of MobileNet for 1, 2, 4 and 8
+  // images): up to two workgroups per CU: one image 64 -> 128 at 112 x 112 stride 2 6.0 us against
+  // 9.0, 128 -> 128 at 56 x 56 7.3 against 10.9, 256 -> 256 at 28 x 28 6.6 against 11.6, 512 -> 512
+  // at 14 x 14 9.7 against 10.8; four images 512 -> 512 15.8 against 18.5, 1024 -> 1024 at 7 x 7 15.6
+  // against 21.4; with more workgroups the tiled product wins (two images 128 -> 128 at 56 x 56:
+  // 784 workgroups, 12.4 against 11.3).  Every one of the N / 64 workgroups of a pixel tile repeats
+  // the tile's depthwise half, K channels of it: with few pixel tiles and K x N / 64 beyond 4096
+  // that costs more than the second launch (one image 1024 -> 1024 at 7 x 7: 14.2 against 10.9).
+  if (tiles > 2 * ctx->num_cus) return -1;
+  if (tiles < ctx->num_cus / 2 && (long long)p.K * ceil_div(p.N, 64) > 4096) return -1;
+  p.tiles_m = (int)ceil_div(p.M, 16);
+  p.tiles_n = (int)ceil_div(p.N, 64);
+  p.k_per = (int)ceil_div(ceil_div(p.K, 8), 16) * 16;
+  p.by_columns = p.tiles_n >= 8;
+  const long long grid = p.by_columns ? 8 * ceil_div(p.tiles_n, 8) * p.tiles_m : (long long)p.tiles_m * p.tiles_n;
+  const size_t panel = (size_t)16 * (p.K + 4) * sizeof(float), parts = (size_t)8 * 4 * 4 * 64 * sizeof(float);
+  const size_t lds = panel > parts ? panel : parts;
+  static bool large_lds_allowed = false;
+  if (lds > 48 * 1024 && !large_lds_allowed) {
+    if (hipFuncSetAttribute((const void*)separable_small_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)((size_t)16 * (1024 + 4) * sizeof(float))) != hipSuccess) {
+      (void)hipGetLastError();
+      return -1;
+    }
+    large_lds_allowed = true;
+  }
+  ctx->name_kernel("separable_small_s%d_f32", p.S);
+  tfhip::launch(ctx, separable_small_kernel, dim3((unsigned)grid), dim3(512), lds, p);
+  TFHIP_LAUNCH_CHECK(ctx);
+  return TFHIP_OK;
+}
+
 }  // namespace tfhip
 
 using namespace tfhip;
@@ -646,6 +857,46 @@ extern "C" int tfhip_separable_conv2d(tfhip_ctx* ctx, int64_t x, int64_t dw_filt
       case 2: return launch_separable<16, 4, 1, 4, 2, true>(ctx, p);
       default: break;
     }
+  }
+
+  // a small problem: one workgroup per 16 pixels x 64 output columns
+  const bool small = dwi->filter_h == 3 && dwi->filter_w == 3 && dwi->dilation_h == 1 &&
+                     dwi->dilation_w == 1 && dwi->out_c == dwi->in_c && dwi->stride_h == dwi->stride_w &&
+                     (S == 1 || S == 2) && bx->dtype == TFHIP_FLOAT32 && bo->dtype == TFHIP_FLOAT32 &&
+                     bdw->dtype == TFHIP_FLOAT32 && bpw->dtype == TFHIP_FLOAT32 && bx->numel == x_n &&
+                     bdw->numel == 9 * (int64_t)K && x_n * 4 < (1ll << 31) && pixels * N * 4 < (1ll << 31) &&
+                     (int64_t)K * N * 4 < (1ll << 31) && pixels > 0 && pixels < (1ll << 24) &&
+                     (!bdb || (bdb->dtype == TFHIP_FLOAT32 &&
+                               bdb->numel == (dw_bias_kind == TFHIP_BCAST_COLUMN ? K : 1) && aligned16(bdb->ptr))) &&
+                     (!bpb || (bpb->dtype == TFHIP_FLOAT32 &&
+                               bpb->numel == (pw_bias_kind == TFHIP_BCAST_COLUMN ? N : 1))) &&
+                     aligned16(bx->ptr) && aligned16(bdw->ptr) && aligned16(bpw->ptr) && aligned16(bo->ptr);
+  if (small && !ctx->separable_off) {
+    SepSmallArgs q = {};
+    q.x = static_cast<const float*>(bx->ptr);
+    q.dw = static_cast<const float*>(bdw->ptr);
+    q.pw = static_cast<const float*>(bpw->ptr);
+    q.y = static_cast<float*>(bo->ptr);
+    q.dwb = bdb ? static_cast<const float*>(bdb->ptr) : nullptr;
+    q.pwb = bpb ? static_cast<const float*>(bpb->ptr) : nullptr;
+    q.H = dwi->in_h;
+    q.W = dwi->in_w;
+    q.OH = dwi->out_h;
+    q.OW = dwi->out_w;
+    q.K = K;
+    q.N = N;
+    q.S = S;
+    q.pt = dwi->pad_top;
+    q.pl = dwi->pad_left;
+    q.M = (int)pixels;
+    q.dwb_kind = dw_bias_kind;
+    q.pwb_kind = pw_bias_kind;
+    q.dw_act = dw_act;
+    q.pw_act = pw_act;
+    q.x_bytes = (unsigned)(x_n * 4);
+    q.pw_bytes = (unsigned)((int64_t)K * N * 4);
+    const int rc = launch_separable_small(ctx, q);
+    if (rc >= 0) return rc;
   }
 
   // the two-kernel form
