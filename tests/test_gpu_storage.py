@@ -514,6 +514,32 @@ def test_block_used_under_both_streams_returns_behind_both(tf):
     tf.dispose([a, w])
 
 
+def test_graph_captured_under_one_stream_reads_what_the_other_wrote(tf):
+    """A graph recorded under stream index 0 whose kernels read a tensor produced under index 1
+    just before: the producer is waited for before the recording (a captured stream cannot wait
+    for an event from outside), the graph replays on the stream of its capture whichever index is
+    selected, and its result read under either index is the eager one."""
+    be = tf.backend()
+    rng = np.random.default_rng(35)
+    n = 1024
+    a = tf.tensor(rng.standard_normal((n, n)).astype(np.float32) * 0.05)
+    w = tf.tensor(rng.standard_normal((n, n)).astype(np.float32) * 0.05)
+    be.select_stream(1)
+    b = tf.tidy(lambda: tf.matmul(tf.matmul(a, w), w))   # under index 1, still running
+    be.select_stream(0)
+    net = lambda: tf.relu(tf.matmul(b, w))
+    g = tf.capture_graph(net)
+    with tf.tidy():
+        want = net().data_sync().copy()
+    for k in range(3):
+        be.select_stream(k % 2)                            # replays ignore the selected index
+        g.replay()
+        assert np.array_equal(g.outputs.data_sync(), want), k
+    be.select_stream(0)
+    g.dispose()
+    tf.dispose([a, w, b])
+
+
 def test_pipelined_uploads_with_two_batches_in_flight(tf):
     """The serving loop of the benchmark in small: every step uploads its input from page-locked
     memory, runs under the stream of its parity and is read back asynchronously two steps late.

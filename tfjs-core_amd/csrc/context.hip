@@ -354,6 +354,9 @@ void tfhip_ctx::unhold(hipEvent_t done) {
 // through the upload stream leaves an event behind, so that the next upload into it waits for
 // the kernels that read it and for nothing queued later.
 void tfhip_ctx::release_buf(Buf& b) {
+  // (a stream under capture cannot be waited for from outside the capture: a block that it used
+  // too goes back to its pool instead, behind the other streams' work)
+  if (capturing && b.sidx != cur && (b.users >> cur & 1)) b.sidx = cur;
   hipStream_t last = streams[b.sidx];  // the stream whose pool the block goes back to
   // (work of the other streams on the block comes before whatever that stream does with it next)
   for (int s = 0; s < kStreams; s++)
