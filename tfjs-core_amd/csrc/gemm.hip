@@ -526,8 +526,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       const __amdgpu_buffer_rsrc_t r = k0 < p.K ? rsrc_b : rsrc_b_none;
       const int soff = BMODE == B_TRANSPOSED ? k0 * 4 : BMODE == B_UINT8 ? k0 * p.ldb : k0 * p.ldb * 4;
       // (a row-major B needs no second set: its rows at or beyond K lie beyond the descriptor's
-      // range by themselves, (k * ldb + n) * size >= K * ldb * size >= b_bytes; a transposed
-      // one switches sets for good like A)
+      // range by themselves, (k * ldb + n) * size >= K * ldb * size >= b_bytes — gfx950 checks the
+      // sum of the vector and the scalar offset against the range, as a probe with a 64-byte
+      // descriptor shows; a transposed one switches sets for good like A)
       if (BMODE == B_TRANSPOSED && cut) {
 #pragma unroll
         for (int i = 0; i < B_PER; i++) {
@@ -1215,7 +1216,8 @@ __global__ __launch_bounds__(SPLIT ? 384 : 256) void conv_smallk_kernel(const Ge
         }
       } else {
         // one add per store: the lane's base offset (out of range for a column past N) plus
-        // the register's pixel offset, which is the same for all lanes
+        // the register's pixel offset, which is the same for all lanes (that offset as the
+        // store's scalar offset instead was measured: 42.8 us against 33.3)
         unsigned lane_at[TN];
 #pragma unroll
         for (int j = 0; j < TN; j++) {
