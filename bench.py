@@ -331,6 +331,10 @@ def main():
                     help="only launch the 56 x 56 x 128 stride-1 depthwise layer of the network (dw3: "
                          "[64,56,56,128], 3x3, bias + relu6) REPS times over four inputs in turn "
                          "(0.4 GB: every launch reads from HBM), for counter runs")
+    ap.add_argument("--loop-separable", type=int, default=0, metavar="REPS",
+                    help="only launch the third depthwise + pointwise block of the network as one kernel "
+                         "(dw3 + pw3: [64,56,56,128] -> 128, bias + relu6 after each half) REPS times "
+                         "over four inputs in turn, for counter runs")
     ap.add_argument("--calibrate-counters", action="store_true",
                     help="only launch a streaming kernel of known size (relu over 256 MiB: reads "
                          "256 MiB, writes 256 MiB) three times, to scale FETCH_SIZE / WRITE_SIZE")
@@ -381,6 +385,25 @@ def main():
         print(json.dumps({"kernel": be.lib.tfhip_last_kernel(be.ctx).decode(),
                           "launches": args.loop_depthwise,
                           "bytes_per_launch": 4.0 * (2 * args.batch * 56 * 56 * 128 + 9 * 128 + 128)}))
+        return
+
+    if args.loop_separable > 0:
+        rng = np.random.default_rng(1)
+        xs = [tf.tensor(rng.uniform(0, 1, (args.batch, 56, 56, 128)).astype(np.float32))
+              for _ in range(4)]
+        dw = tf.tensor((rng.standard_normal((3, 3, 128, 1)) * 0.3).astype(np.float32))
+        pw = tf.tensor((rng.standard_normal((1, 1, 128, 128)) * 0.1).astype(np.float32))
+        b1, b2 = tf.tensor(np.zeros(128, np.float32)), tf.tensor(np.zeros(128, np.float32))
+        for i in range(args.loop_separable):
+            tf.dispose(tf.fused.separable_conv2d(xs[i % 4], dw, pw, 1, "same", depthwise_bias=b1,
+                                                 depthwise_activation="relu6", bias=b2,
+                                                 activation="relu6"))
+        be.sync()
+        pixels = args.batch * 56 * 56
+        print(json.dumps({"kernel": be.lib.tfhip_last_kernel(be.ctx).decode(),
+                          "launches": args.loop_separable,
+                          "flops_per_launch": 2.0 * pixels * 128 * (128 + 9),
+                          "bytes_per_launch": 4.0 * (2 * pixels * 128 + 9 * 128 + 128 * 128 + 256)}))
         return
 
     params = mobilenet.make_params(seed=0)
