@@ -348,6 +348,19 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
     const Clamp pact = clamp_of(p.pw_act);
     const __amdgpu_buffer_rsrc_t ry = make_rsrc(p.y, p.y_bytes);
     const unsigned y_row = (unsigned)(p.OW * N * 4);
+    // what the lane adds to the address of accumulator register r of a block: its column, and the
+    // 4 pixels that the upper half of the wavefront lies further on (columns, or rows when the
+    // strip is narrower than 8)
+    const unsigned lane_at = (unsigned)(l32 * 4) +
+                             (SW >= 8 ? (unsigned)(4 * g * N * 4) : (unsigned)(g * (4 / SW)) * y_row);
+    // ... and with the register's own pixel (row m / SW, column m % SW of the block): the offset of
+    // accumulator register r from the block's first pixel, the same for every block of the kernel
+    unsigned reg_at[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int mc = 8 * (r >> 2) + (r & 3);
+      reg_at[r] = lane_at + (unsigned)(mc / SW) * y_row + (unsigned)((mc % SW) * N * 4);
+    }
     const float* const panel_r = panels0 + l32 * PITCH + 4 * g;  // this lane's operand in pair 0's first panel
     __syncthreads();
 
@@ -379,33 +392,50 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
               }
             __builtin_amdgcn_sched_barrier(0);
           }
-          // accumulator register r: pixel m = 8*(r/4) + 4*(lane/32) + r%4 of the panel, column l32
+          // accumulator register r: pixel m = 8*(r/4) + 4*(lane/32) + r%4 of the panel, column l32.
+          // The block's own offset is the same for the whole wavefront and rides in the scalar
+          // offset of the stores, what register r and the lane add to it (reg_at, fixed for the
+          // kernel) in the vector offset: a whole block is stored without a vector instruction for
+          // its addresses.
           const int orow = un.o0 + blk * RB, ocol = un.strip * SW;
           const unsigned y_blk = (unsigned)((un.n * p.OH + orow) * p.OW + ocol) * (unsigned)(N * 4) +
-                                 (unsigned)(col0 * 4);
+                                 (unsigned)(32 * CB * pair * 4);
           const int cols_left = p.OW - ocol;
           const bool whole = rows_left >= RB && cols_left >= SW;
+          if (whole) {
+            const int s_blk = __builtin_amdgcn_readfirstlane((int)y_blk);
 #pragma unroll
-          for (int r = 0; r < 16; r++) {
-            const int mc = 8 * (r >> 2) + (r & 3);  // + 4 * g
-            int row, col;
-            if (SW >= 8) {
-              row = mc / SW;
-              col = mc % SW + 4 * g;
-            } else if (SW == 4) {
-              row = mc / SW + g;
-              col = mc % SW;
-            } else {  // SW == 2: 4 * g pixels further on is 2 rows further down
-              row = mc / SW + 2 * g;
-              col = mc % SW;
+            for (int r = 0; r < 16; r++) {
+#pragma unroll
+              for (int c = 0; c < CB; c++) {
+                const float val = clamp(acc[c][r] + bias_c[c], pact);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), ry,
+                                                      (int)(reg_at[r] + (unsigned)(32 * c * 4)), s_blk, 0);
+              }
             }
-            const unsigned at = y_blk + (unsigned)row * y_row + (unsigned)(col * N * 4);
-            const bool ok = whole || (row < rows_left && col < cols_left);
+          } else {
 #pragma unroll
-            for (int c = 0; c < CB; c++) {
-              const float val = clamp(acc[c][r] + bias_c[c], pact);
-              __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), ry,
-                                                    (int)(ok ? at + (unsigned)(32 * c * 4) : OOB_OFFSET), 0, 0);
+            for (int r = 0; r < 16; r++) {
+              const int mc = 8 * (r >> 2) + (r & 3);  // + 4 * g
+              int row, col;
+              if (SW >= 8) {
+                row = mc / SW;
+                col = mc % SW + 4 * g;
+              } else if (SW == 4) {
+                row = mc / SW + g;
+                col = mc % SW;
+              } else {  // SW == 2: 4 * g pixels further on is 2 rows further down
+                row = mc / SW + 2 * g;
+                col = mc % SW;
+              }
+              const unsigned at = y_blk + (unsigned)row * y_row + (unsigned)(col * N * 4) + (unsigned)(l32 * 4);
+              const bool ok = row < rows_left && col < cols_left;
+#pragma unroll
+              for (int c = 0; c < CB; c++) {
+                const float val = clamp(acc[c][r] + bias_c[c], pact);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), ry,
+                                                      (int)(ok ? at + (unsigned)(32 * c * 4) : OOB_OFFSET), 0, 0);
+              }
             }
           }
         }
