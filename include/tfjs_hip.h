@@ -130,9 +130,14 @@ int tfhip_sync(tfhip_ctx* ctx);
  * (The contents of a buffer count as written by the first work queued on it, or by tfhip_write:
  * tensors are written once.  A caller that has a kernel overwrite a live buffer under another
  * index than the one that wrote it first orders that itself, with tfhip_sync.)
- * tfhip_read / tfhip_read_begin follow the buffer's own stream, tfhip_sync waits for both, a
- * captured graph replays on the stream it was recorded on.  Not inside a timed region or a graph
- * capture. */
+ * tfhip_read / tfhip_read_begin follow the buffer's own stream, tfhip_sync waits for both.
+ * A captured graph writes its tensors again on every replay, so replays are ordered as a whole:
+ * a replay runs on the stream it was recorded on, behind everything queued under the other
+ * index so far (new input data copied there by a small tfhip_write, kernels that still read the
+ * previous replay's results) and behind asynchronous reads of its tensors that are still
+ * copying; after it, the tensors the recorded work produced count as written anew on that
+ * stream, so the next consumer under the other index waits for the replay.
+ * Not inside a timed region or a graph capture. */
 int tfhip_select_stream(tfhip_ctx* ctx, int index);
 /* KernelBackend.time (backend.ts:92, backend_cpu.ts:239-244): device time of the work queued
  * between the two calls (two events on the stream).  Regions nest (up to 8 deep), as tf.time()
@@ -204,8 +209,10 @@ int tfhip_matmul(tfhip_ctx* ctx, int64_t a, int64_t b, int64_t out, int batch, i
  * library holds on every GPU it runs on until the process ends.  A product whose partial
  * tiles need more fails with TFHIP_ENOTSUP, as does an operand that is not stored as float32
  * (its converted copy would need a block; b may be TFHIP_UINT8Q).  All calls on one GPU share
- * the array: calls that overlap on one GPU (two contexts, two threads) race on it; calls on
- * one context are ordered by its stream. */
+ * the array: calls that overlap on one GPU (two contexts, two threads) race on it.  Calls on
+ * one context do not: under one stream index they run in order, a call under the other index
+ * (and a replay of a captured graph that recorded such a call) is put behind the array's last
+ * user with an event. */
 int tfhip_matmul_noalloc(tfhip_ctx* ctx, int64_t a, int64_t b, int64_t out, int batch, int m,
                          int n, int k, int transpose_a, int transpose_b, int64_t bias,
                          int bias_kind, int act, int64_t prelu, int prelu_kind,

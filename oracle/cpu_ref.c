@@ -65,15 +65,37 @@ void ref_batch_matmul(const float* a, const float* b, float* out, int batch, int
         }
 }
 
-/* backends/cpu/backend_cpu.ts:1552-1616, channelsLast strides; out-of-bounds taps are
- * skipped (:1586,:1596); `yVals[...] += xVal * w` rounds to float after every MAC. */
-void ref_conv2d(const float* x, const float* w, float* y, const ref_conv2d_info* ci) {
-  const int64_t x_row = (int64_t)ci->in_w * ci->in_c, x_b = x_row * ci->in_h;
-  const int64_t y_row = (int64_t)ci->out_w * ci->out_c, y_b = y_row * ci->out_h;
+/* Element strides of an image tensor in either data format, as backend_cpu.ts:1565-1572 takes
+ * them from x.strides / y.strides: channelsLast [b,h,w,c], channelsFirst [b,c,h,w]. */
+typedef struct img_strides {
+  int64_t b, row, col, ch;
+} img_strides;
+static img_strides strides_of(int h, int w, int c, int channels_first) {
+  img_strides s;
+  s.b = (int64_t)h * w * c;
+  if (channels_first) {
+    s.ch = (int64_t)h * w;
+    s.row = w;
+    s.col = 1;
+  } else {
+    s.row = (int64_t)w * c;
+    s.col = c;
+    s.ch = 1;
+  }
+  return s;
+}
+
+/* backends/cpu/backend_cpu.ts:1552-1616; out-of-bounds taps are skipped (:1586,:1596);
+ * `yVals[...] += xVal * w` rounds to float after every MAC.  The data format only changes the
+ * strides (:1565-1572), not the order of the loops. */
+static void conv2d_strided(const float* x, const float* w, float* y, const ref_conv2d_info* ci,
+                           int channels_first) {
+  const img_strides xs = strides_of(ci->in_h, ci->in_w, ci->in_c, channels_first);
+  const img_strides ys = strides_of(ci->out_h, ci->out_w, ci->out_c, channels_first);
   const int64_t w_s0 = (int64_t)ci->filter_w * ci->in_c * ci->out_c;
   const int64_t w_s1 = (int64_t)ci->in_c * ci->out_c;
   const int oc = ci->out_c;
-  memset(y, 0, sizeof(float) * (size_t)(y_b * ci->batch));
+  memset(y, 0, sizeof(float) * (size_t)(ys.b * ci->batch));
   for (int b = 0; b < ci->batch; ++b)
     for (int yr = 0; yr < ci->out_h; ++yr) {
       const int xr_corner = yr * ci->stride_h - ci->pad_top;
@@ -81,23 +103,30 @@ void ref_conv2d(const float* x, const float* w, float* y, const ref_conv2d_info*
         const int xr = xr_corner + wr * ci->dilation_h;
         if (xr < 0 || xr >= ci->in_h) continue;
         for (int yc = 0; yc < ci->out_w; ++yc) {
-          float* yp = y + b * y_b + yr * y_row + (int64_t)yc * oc;
+          float* yp = y + b * ys.b + yr * ys.row + yc * ys.col;
           const int xc_corner = yc * ci->stride_w - ci->pad_left;
           for (int wc = 0; wc < ci->filter_w; ++wc) {
             const int xc = xc_corner + wc * ci->dilation_w;
             if (xc < 0 || xc >= ci->in_w) continue;
-            const float* xp = x + b * x_b + xr * x_row + (int64_t)xc * ci->in_c;
+            const float* xp = x + b * xs.b + xr * xs.row + xc * xs.col;
             const float* wp = w + wr * w_s0 + wc * w_s1;
             for (int d1 = 0; d1 < ci->in_c; ++d1) {
-              const double xv = (double)xp[d1];
+              const double xv = (double)xp[d1 * xs.ch];
               for (int d2 = 0; d2 < oc; ++d2)
-                yp[d2] = (float)((double)yp[d2] + xv * (double)wp[d2]);
+                yp[d2 * ys.ch] = (float)((double)yp[d2 * ys.ch] + xv * (double)wp[d2]);
               wp += oc;
             }
           }
         }
       }
     }
+}
+void ref_conv2d(const float* x, const float* w, float* y, const ref_conv2d_info* ci) {
+  conv2d_strided(x, w, y, ci, 0);
+}
+/* x [b, in_c, in_h, in_w], y [b, out_c, out_h, out_w]; the filter stays [fh, fw, in_c, out_c]. */
+void ref_conv2d_nchw(const float* x, const float* w, float* y, const ref_conv2d_info* ci) {
+  conv2d_strided(x, w, y, ci, 1);
 }
 
 /* backends/cpu/backend_cpu.ts:1979-2035.  pad_quirk != 0 reproduces :2000 (rows offset by
@@ -180,14 +209,16 @@ void ref_pool2d(const float* x, float* y, const ref_conv2d_info* ci, int kind) {
 
 /* ---- backward kernels --------------------------------------------------------------- */
 
-/* backends/cpu/backend_cpu.ts:1686-1762 (channelsLast).  The loop bounds are JavaScript
- * numbers: yRMax = min(outHeight, (filterHeight + xRCorner) / strideHeight) is fractional and
- * compared with `<`; one double dot product per dx element, stored to float once. */
-void ref_conv2d_der_input(const float* dy, const float* w, float* dx, const ref_conv2d_info* ci) {
+/* backends/cpu/backend_cpu.ts:1686-1762.  The loop bounds are JavaScript numbers: yRMax =
+ * min(outHeight, (filterHeight + xRCorner) / strideHeight) is fractional and compared with `<`;
+ * one double dot product per dx element, stored to float once.  The data format changes the
+ * strides of dx and dy only (:1698-1706). */
+static void conv2d_der_input_strided(const float* dy, const float* w, float* dx,
+                                     const ref_conv2d_info* ci, int channels_first) {
   const int fh = ci->filter_h, fw = ci->filter_w, ic = ci->in_c, oc = ci->out_c;
   const int top_pad = fh - 1 - ci->pad_top, left_pad = fw - 1 - ci->pad_left;
-  const int64_t x_row = (int64_t)ci->in_w * ic, x_b = x_row * ci->in_h;
-  const int64_t y_row = (int64_t)ci->out_w * oc, y_b = y_row * ci->out_h;
+  const img_strides xs = strides_of(ci->in_h, ci->in_w, ic, channels_first);
+  const img_strides ys = strides_of(ci->out_h, ci->out_w, oc, channels_first);
   const int64_t w_s0 = (int64_t)fw * ic * oc, w_s1 = (int64_t)ic * oc, w_s2 = oc;
   for (int b = 0; b < ci->batch; ++b)
     for (int d1 = 0; d1 < ic; ++d1)
@@ -204,22 +235,31 @@ void ref_conv2d_der_input(const float* dy, const float* w, float* dx, const ref_
             const int wr = yr * ci->stride_h - xr_corner;
             for (int yc = (int)yc_min; yc < yc_max; ++yc) {
               const int wc = yc * ci->stride_w - xc_corner;
-              const float* dyp = dy + b * y_b + yr * y_row + (int64_t)yc * oc;
+              const float* dyp = dy + b * ys.b + yr * ys.row + yc * ys.col;
               const float* wp = w + w_s0 * (fh - 1 - wr) + w_s1 * (fw - 1 - wc) + w_s2 * d1;
-              for (int d2 = 0; d2 < oc; ++d2) dot += (double)dyp[d2] * (double)wp[d2];
+              for (int d2 = 0; d2 < oc; ++d2) dot += (double)dyp[d2 * ys.ch] * (double)wp[d2];
             }
           }
-          dx[b * x_b + xr * x_row + (int64_t)xc * ic + d1] = (float)dot;
+          dx[b * xs.b + xr * xs.row + xc * xs.col + d1 * xs.ch] = (float)dot;
         }
       }
 }
+void ref_conv2d_der_input(const float* dy, const float* w, float* dx, const ref_conv2d_info* ci) {
+  conv2d_der_input_strided(dy, w, dx, ci, 0);
+}
+void ref_conv2d_der_input_nchw(const float* dy, const float* w, float* dx,
+                               const ref_conv2d_info* ci) {
+  conv2d_der_input_strided(dy, w, dx, ci, 1);
+}
 
-/* backends/cpu/backend_cpu.ts:1849-1898 (channelsLast): per filter element one double dot
- * product over batch, output rows and columns, stored to float once. */
-void ref_conv2d_der_filter(const float* x, const float* dy, float* dw, const ref_conv2d_info* ci) {
+/* backends/cpu/backend_cpu.ts:1849-1898: per filter element one double dot product over batch,
+ * output rows and columns, stored to float once; channelsFirst reads x and dy through other
+ * strides (:1857-1865). */
+static void conv2d_der_filter_strided(const float* x, const float* dy, float* dw,
+                                      const ref_conv2d_info* ci, int channels_first) {
   const int fh = ci->filter_h, fw = ci->filter_w, ic = ci->in_c, oc = ci->out_c;
-  const int64_t x_row = (int64_t)ci->in_w * ic, x_b = x_row * ci->in_h;
-  const int64_t y_row = (int64_t)ci->out_w * oc, y_b = y_row * ci->out_h;
+  const img_strides xs = strides_of(ci->in_h, ci->in_w, ic, channels_first);
+  const img_strides ys = strides_of(ci->out_h, ci->out_w, oc, channels_first);
   for (int wr = 0; wr < fh; ++wr) {
     const double yr_min = fmax(0.0, ceil((double)(ci->pad_top - wr) / ci->stride_h));
     const double yr_max = fmin((double)ci->out_h, (double)(ci->in_h + ci->pad_top - wr) / ci->stride_h);
@@ -234,14 +274,21 @@ void ref_conv2d_der_filter(const float* x, const float* dy, float* dw, const ref
               const int xr = wr + yr * ci->stride_h - ci->pad_top;
               for (int yc = (int)yc_min; yc < yc_max; ++yc) {
                 const int xc = wc + yc * ci->stride_w - ci->pad_left;
-                dot += (double)x[b * x_b + xr * x_row + (int64_t)xc * ic + d1] *
-                       (double)dy[b * y_b + yr * y_row + (int64_t)yc * oc + d2];
+                dot += (double)x[b * xs.b + xr * xs.row + xc * xs.col + d1 * xs.ch] *
+                       (double)dy[b * ys.b + yr * ys.row + yc * ys.col + d2 * ys.ch];
               }
             }
           dw[(((int64_t)wr * fw + wc) * ic + d1) * oc + d2] = (float)dot;
         }
     }
   }
+}
+void ref_conv2d_der_filter(const float* x, const float* dy, float* dw, const ref_conv2d_info* ci) {
+  conv2d_der_filter_strided(x, dy, dw, ci, 0);
+}
+void ref_conv2d_der_filter_nchw(const float* x, const float* dy, float* dw,
+                                const ref_conv2d_info* ci) {
+  conv2d_der_filter_strided(x, dy, dw, ci, 1);
 }
 
 /* backends/cpu/backend_cpu.ts:2037-2103. */

@@ -86,9 +86,15 @@ def _cond_round(v, mode):  # conv_util.ts:499-517
 
 
 def compute_conv2d_info(in_shape, filter_shape, strides, dilations, pad, rounding_mode=None,
-                        depthwise=False):
-    """computeConv2DInfo (conv_util.ts:123-182) + getPadAndOutInfo (:399-435), NHWC."""
-    batch, in_h, in_w, in_c = in_shape
+                        depthwise=False, data_format="channelsLast"):
+    """computeConv2DInfo (conv_util.ts:123-182) + getPadAndOutInfo (:399-435); data_format
+    'channelsLast' ([b,h,w,c]) or 'channelsFirst' ([b,c,h,w]) as conv_util.ts:131-139."""
+    if data_format == "channelsLast":
+        batch, in_h, in_w, in_c = in_shape
+    elif data_format == "channelsFirst":
+        batch, in_c, in_h, in_w = in_shape
+    else:
+        raise ValueError("Unknown dataFormat %s" % data_format)
     f_h, f_w, _, f_c = filter_shape
     s_h, s_w = _tuple2(strides)
     d_h, d_w = _tuple2(dilations)
@@ -124,7 +130,9 @@ def compute_conv2d_info(in_shape, filter_shape, strides, dilations, pad, roundin
                 filterHeight=f_h, filterWidth=f_w, effectiveFilterHeight=e_h,
                 effectiveFilterWidth=e_w,
                 padInfo=dict(top=top, bottom=bottom, left=left, right=right, type=ptype),
-                inShape=tuple(in_shape), outShape=(batch, out_h, out_w, out_c),
+                dataFormat=data_format, inShape=tuple(in_shape),
+                outShape=((batch, out_c, out_h, out_w) if data_format == "channelsFirst"
+                          else (batch, out_h, out_w, out_c)),
                 filterShape=tuple(filter_shape))
 
 
@@ -204,7 +212,8 @@ def conv2d(x, w, ci):
     x, w = _f32(x), _f32(w)
     y = np.empty(ci["outShape"], np.float32)
     info = _info_c(ci)
-    lib().ref_conv2d(_p(x), _p(w), _p(y), C.byref(info))
+    first = ci.get("dataFormat", "channelsLast") == "channelsFirst"
+    (lib().ref_conv2d_nchw if first else lib().ref_conv2d)(_p(x), _p(w), _p(y), C.byref(info))
     return y
 
 
@@ -246,7 +255,9 @@ def conv2d_der_input(dy, w, ci):
     dy, w = _f32(dy), _f32(w)
     dx = np.empty(ci["inShape"], np.float32)
     info = _info_c(ci)
-    lib().ref_conv2d_der_input(_p(dy), _p(w), _p(dx), C.byref(info))
+    first = ci.get("dataFormat", "channelsLast") == "channelsFirst"
+    (lib().ref_conv2d_der_input_nchw if first else lib().ref_conv2d_der_input)(
+        _p(dy), _p(w), _p(dx), C.byref(info))
     return dx
 
 
@@ -254,7 +265,9 @@ def conv2d_der_filter(x, dy, ci):
     x, dy = _f32(x), _f32(dy)
     dw = np.empty(ci["filterShape"], np.float32)
     info = _info_c(ci)
-    lib().ref_conv2d_der_filter(_p(x), _p(dy), _p(dw), C.byref(info))
+    first = ci.get("dataFormat", "channelsLast") == "channelsFirst"
+    (lib().ref_conv2d_der_filter_nchw if first else lib().ref_conv2d_der_filter)(
+        _p(x), _p(dy), _p(dw), C.byref(info))
     return dw
 
 

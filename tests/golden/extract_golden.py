@@ -104,7 +104,7 @@ CASES = {
 # tf.grads of conv2d and behind conv2dTranspose, the depthwise and pooling backprops).  A
 # describe's beforeEach block is recorded as a case titled "beforeEach".
 GRAD_CASES = {
-    "conv2d_grad": ("tfjs-core/src/ops/conv2d_test.ts", ["conv2d"], r"^gradient(?!.*NCHW)"),
+    "conv2d_grad": ("tfjs-core/src/ops/conv2d_test.ts", ["conv2d"], r"^gradient"),
     "conv2d_transpose": ("tfjs-core/src/ops/conv2d_transpose_test.ts", ["conv2dTranspose"],
                          r"^(input=|gradient)"),
     "depthwise_grad": ("tfjs-core/src/ops/conv2d_depthwise_test.ts",

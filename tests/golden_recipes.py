@@ -221,6 +221,24 @@ def conv2d_known_answers(ops):
 
 
 @recipe
+def conv2d_channels_first(ops):
+    """ops/conv2d_test.ts:109-230: dataFormat 'NCHW' (x [b,c,h,w] or [c,h,w], filter still
+    [fh,fw,in,out], result channels-first)."""
+    for title, xs, ws, pad in (("x=[2,1,2,2] f=[1,1,1,1] s=1 d=1 p=0 NCHW", (2, 1, 2, 2), (1, 1, 1, 1), 0),
+                               ("x=[1,2,2] f=[2,2,1,1] s=1 d=1 p=same NCHW", (1, 2, 2), (2, 2, 1, 1), "same"),
+                               ("x=[2,2,2] f=[2,2,2,1] s=1 d=1 p=same NCHW", (2, 2, 2), (2, 2, 2, 1), "same"),
+                               ("x=[2,1,2,2] f=[2,2,1,1] s=1 d=1 p=same NCHW", (2, 1, 2, 2), (2, 2, 1, 1), "same")):
+        c = golden_case("conv2d", title)
+        a = c["arrays"]
+        assert c["consts"]["dataFormat"] == "NCHW"
+        x, w = f32(a[2], xs), f32(a[3], ws)
+        r = ops.conv2d(_lift(x), w, c["consts"]["stride"], pad, data_format="NCHW")
+        r = r[0] if x.ndim == 3 else r
+        assert list(r.shape) == a[5], title
+        expect_close(r, a[6])
+
+
+@recipe
 def conv2d_dilation_equals_zero_stuffed_filter(ops):
     """ops/conv2d_test.ts:246-279: d=2 on a 2x2 filter == d=1 on the 3x3 zero-stuffed one."""
     c = golden_case("conv2d", "x=[4,4,1] f=[2,2,1,1] s=1 d=2 p=0")["arrays"]
@@ -756,6 +774,21 @@ def conv2d_gradients(ops):
         expect_close(ops.conv2d_der_input(xs, dy, w, 1, 0), a[8])
         want_dw = a[9] if a[9] is not None else [26, 38, 62, 74]   # written as 13 * 2 ... there
         expect_close(ops.conv2d_der_filter(x, dy, (2, 2, 1, 1), 1, 0), want_dw)
+
+
+@recipe
+def conv2d_gradients_channels_first(ops):
+    """ops/conv2d_test.ts:454-508: tf.grads of x.conv2d(filter, 1, 0, 'NCHW')."""
+    for title, xs, dys in (("gradient x=[1,1,3,3] f=[2,2,1,1] s=1 p=0 NCHW", (1, 1, 3, 3), (1, 1, 2, 2)),
+                           ("gradient x=[2,1,3,3] f=[2,2,1,1] s=1 p=0 NCHW", (2, 1, 3, 3), (2, 1, 2, 2))):
+        a = golden_case("conv2d_grad", title)["arrays"]
+        x, dy = f32(a[4], xs), f32(a[5], dys)
+        assert a[6] == list(dys)
+        w = np.ones((2, 2, 1, 1), np.float32)
+        dx = ops.conv2d_der_input(xs, dy, w, 1, 0, data_format="NCHW")
+        assert dx.shape == xs
+        expect_close(dx, a[8])
+        expect_close(ops.conv2d_der_filter(x, dy, (2, 2, 1, 1), 1, 0, data_format="NCHW"), a[9])
 
 
 @recipe

@@ -8,6 +8,9 @@ Both expose the same tf-like calls on numpy arrays:
 import numpy as np
 
 
+_FORMATS = {"NHWC": "channelsLast", "NCHW": "channelsFirst"}   # ops/conv_util.ts:545-554
+
+
 class OracleOps:
     name = "oracle"
 
@@ -23,8 +26,9 @@ class OracleOps:
         return self.r.fused_batch_matmul(a, b, ta, tb, bias, activation, prelu)
 
     def conv2d(self, x, w, strides, pad, dilations=1, bias=None, activation=None, prelu=None,
-               rounding=None):
-        ci = self.r.compute_conv2d_info(x.shape, w.shape, strides, dilations, pad, rounding)
+               rounding=None, data_format="NHWC"):
+        ci = self.r.compute_conv2d_info(x.shape, w.shape, strides, dilations, pad, rounding,
+                                        data_format=_FORMATS[data_format])
         return self.r.fused_conv2d(x, w, ci, bias, activation, prelu)
 
     def depthwise_conv2d(self, x, w, strides, pad, dilations=1, bias=None, activation=None,
@@ -81,12 +85,15 @@ class OracleOps:
 
     # backward kernels; the Conv2DInfo is that of the forward op (ops/conv.ts:354-420,
     # 466-520, ops/pool.ts:333-397), dilation 1 for the convolutions
-    def conv2d_der_input(self, x_shape, dy, w, strides, pad, rounding=None):
-        ci = self.r.compute_conv2d_info(x_shape, w.shape, strides, 1, pad, rounding)
+    def conv2d_der_input(self, x_shape, dy, w, strides, pad, rounding=None, data_format="NHWC"):
+        ci = self.r.compute_conv2d_info(x_shape, w.shape, strides, 1, pad, rounding,
+                                        data_format=_FORMATS[data_format])
         return self.r.conv2d_der_input(dy, w, ci)
 
-    def conv2d_der_filter(self, x, dy, filter_shape, strides, pad, rounding=None):
-        ci = self.r.compute_conv2d_info(x.shape, filter_shape, strides, 1, pad, rounding)
+    def conv2d_der_filter(self, x, dy, filter_shape, strides, pad, rounding=None,
+                          data_format="NHWC"):
+        ci = self.r.compute_conv2d_info(x.shape, filter_shape, strides, 1, pad, rounding,
+                                        data_format=_FORMATS[data_format])
         return self.r.conv2d_der_filter(x, dy, ci)
 
     def depthwise_der_input(self, x_shape, dy, w, strides, pad):
@@ -247,10 +254,10 @@ class HipOps:
             prelu_activation_weights=pr), a, b, bias, prelu)
 
     def conv2d(self, x, w, strides, pad, dilations=1, bias=None, activation=None, prelu=None,
-               rounding=None):
+               rounding=None, data_format="NHWC"):
         tf = self.tf
         if bias is None and activation is None:
-            return self._run(lambda a, b: tf.conv2d(a, b, strides, pad, "NHWC", dilations,
+            return self._run(lambda a, b: tf.conv2d(a, b, strides, pad, data_format, dilations,
                                                     rounding), x, w)
         return self._run(lambda a, b, bi, pr: tf.fused.conv2d(
             a, b, strides, pad, "NHWC", dilations, rounding, bias=bi,
@@ -302,15 +309,16 @@ class HipOps:
     def split(self, x, num_or_sizes, axis=0):
         return self._run_list(lambda a: self.tf.split(a, num_or_sizes, axis), x)
 
-    def conv2d_der_input(self, x_shape, dy, w, strides, pad, rounding=None):
+    def conv2d_der_input(self, x_shape, dy, w, strides, pad, rounding=None, data_format="NHWC"):
         tf = self.tf
-        return self._run(lambda d, f: tf.conv2d_der_input(x_shape, d, f, strides, pad, "NHWC",
-                                                          rounding), dy, w)
+        return self._run(lambda d, f: tf.conv2d_der_input(x_shape, d, f, strides, pad,
+                                                          data_format, rounding), dy, w)
 
-    def conv2d_der_filter(self, x, dy, filter_shape, strides, pad, rounding=None):
+    def conv2d_der_filter(self, x, dy, filter_shape, strides, pad, rounding=None,
+                          data_format="NHWC"):
         tf = self.tf
         return self._run(lambda a, d: tf.conv2d_der_filter(a, d, filter_shape, strides, pad,
-                                                           "NHWC", rounding), x, dy)
+                                                           data_format, rounding), x, dy)
 
     def depthwise_der_input(self, x_shape, dy, w, strides, pad):
         tf = self.tf

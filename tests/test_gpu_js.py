@@ -113,6 +113,13 @@ def test_js_ops_match_oracle(tmp_path, ref):
     c.add("conv", "conv2d", dict(x=x, filter=w), dict(strides=1, pad="same"), ref.conv2d(x, w, 1, "same"))
     c.add("conv_s2", "conv2d", dict(x=x, filter=w), dict(strides=2, pad="same"), ref.conv2d(x, w, 2, "same"))
     c.add("conv_rank3", "conv2d", dict(x=x[0], filter=w), dict(strides=1, pad="valid"), ref.conv2d(x[:1], w, 1, "valid")[0])
+    # dataFormat 'NCHW' (ops/conv.ts:148; the four blocks of ops/conv2d_test.ts:109-230 run with the
+    # other golden recipes)
+    xn = u(2, 8, 11, 9)
+    c.add("conv_nchw", "conv2d", dict(x=xn, filter=w), dict(strides=1, pad="same", dataFormat="NCHW"),
+          ref.conv2d(xn, w, 1, "same", data_format="NCHW"))
+    c.add("conv_nchw_s2_rank3", "conv2d", dict(x=xn[0], filter=w), dict(strides=2, pad="same", dataFormat="NCHW"),
+          ref.conv2d(xn[:1], w, 2, "same", data_format="NCHW")[0])
     for act in ("linear", "relu", "relu6"):
         c.add("fconv_" + act, "fusedConv2d", dict(x=x, filter=w, bias=cb), dict(strides=1, pad="same", activation=act),
               ref.conv2d(x, w, 1, "same", bias=cb, activation=act))
@@ -574,6 +581,14 @@ def test_js_backward_ops_match_oracle(tmp_path, ref):
         c.add("der_filter_" + tag, "conv2dDerFilter", dict(x=x, dy=dy),
               dict(filterShape=list(w.shape), strides=stride, pad=pad),
               ref.conv2d_der_filter(x, dy, w.shape, stride, pad), atol=1e-4)
+    xn = f(2, 8, 9, 11)                              # channels first
+    dyn = f(*ref.conv2d(xn, w, 2, "same", data_format="NCHW").shape)
+    c.add("der_input_nchw", "conv2dDerInput", dict(dy=dyn, filter=w),
+          dict(xShape=list(xn.shape), strides=2, pad="same", dataFormat="NCHW"),
+          ref.conv2d_der_input(xn.shape, dyn, w, 2, "same", data_format="NCHW"), atol=2e-5)
+    c.add("der_filter_nchw", "conv2dDerFilter", dict(x=xn, dy=dyn),
+          dict(filterShape=list(w.shape), strides=2, pad="same", dataFormat="NCHW"),
+          ref.conv2d_der_filter(xn, dyn, w.shape, 2, "same", data_format="NCHW"), atol=1e-4)
     small, wt = f(5, 5, 6), f(4, 4, 3, 6) * 0.3      # rank-3 input: batch of 1 assumed
     c.add("transpose_rank3", "conv2dTranspose", dict(x=small, filter=wt),
           dict(outputShape=[10, 10, 3], strides=2, pad="same"),
@@ -629,6 +644,13 @@ def test_js_gradients_through_the_tape(tmp_path, ref):
           flat(a[8]).reshape(3, 3, 1), atol=1e-3)
     c.add("conv2d_dw", "gradConv2d", dict(x=x, filter=w, dy=dy), dict(strides=1, pad=0, wrt=1),
           flat(a[9]).reshape(2, 2, 1, 1), atol=1e-3)
+    # ops/conv2d_test.ts:482-508: the same through dataFormat 'NCHW'
+    a = _golden("conv2d_grad", "gradient x=[2,1,3,3] f=[2,2,1,1] s=1 p=0 NCHW")["arrays"]
+    x, dy = flat(a[4]).reshape(2, 1, 3, 3), flat(a[5]).reshape(2, 1, 2, 2)
+    c.add("conv2d_nchw_dx", "gradConv2d", dict(x=x, filter=w, dy=dy),
+          dict(strides=1, pad=0, wrt=0, dataFormat="NCHW"), flat(a[8]).reshape(2, 1, 3, 3), atol=1e-3)
+    c.add("conv2d_nchw_dw", "gradConv2d", dict(x=x, filter=w, dy=dy),
+          dict(strides=1, pad=0, wrt=1, dataFormat="NCHW"), flat(a[9]).reshape(2, 2, 1, 1), atol=1e-3)
     # ops/conv2d_transpose_test.ts: stride 2, 'same', two channels
     a = _golden("conv2d_transpose", "gradient input=[1,2,2,2] f=[2,2,2,1] s=[2,2] padding=same")["arrays"]
     x, w = flat(a[6]).reshape(1, 2, 2, 2), flat(a[7]).reshape(2, 2, 2, 2)

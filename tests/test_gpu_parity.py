@@ -131,6 +131,29 @@ def test_conv2d_shapes(hip, ref, xs, fs, stride, pad, dil):
     close(hip.conv2d(x, w, stride, pad, dil), ref.conv2d(x, w, stride, pad, dil))
 
 
+@pytest.mark.parametrize("xs,fs,stride,pad", [
+    ((2, 8, 13, 11), (3, 3, 8, 20), 1, "same"),         # [b, c, h, w]
+    ((1, 3, 16, 18), (3, 3, 3, 32), 2, "same"),         # stem-like, Cin = 3
+    ((3, 64, 7, 7), (1, 1, 64, 48), 1, "valid"),        # pointwise
+])
+def test_conv2d_channels_first(hip, ref, xs, fs, stride, pad):
+    """tf.conv2d(..., 'NCHW') and its two gradients (ops/conv.ts:148, 245, 345;
+    backend_cpu.ts:1565-1572) against the oracle's channels-first loops."""
+    print("conv2d NCHW", xs, fs, stride, pad, flush=True)
+    rng = np.random.default_rng(sum(xs) + sum(fs))
+    x = rng.uniform(0, 1, xs).astype(np.float32)
+    w = (rng.standard_normal(fs) * np.sqrt(2.0 / (fs[0] * fs[1] * fs[2]))).astype(np.float32)
+    want = ref.conv2d(x, w, stride, pad, data_format="NCHW")
+    got = hip.conv2d(x, w, stride, pad, data_format="NCHW")
+    assert got.shape == want.shape and got.shape[1] == fs[3]
+    close(got, want)
+    dy = rng.standard_normal(want.shape).astype(np.float32)
+    close(hip.conv2d_der_input(xs, dy, w, stride, pad, data_format="NCHW"),
+          ref.conv2d_der_input(xs, dy, w, stride, pad, data_format="NCHW"), atol=2e-5)
+    close(hip.conv2d_der_filter(x, dy, fs, stride, pad, data_format="NCHW"),
+          ref.conv2d_der_filter(x, dy, fs, stride, pad, data_format="NCHW"), atol=1e-4)
+
+
 @pytest.mark.parametrize("act", ["linear", "relu", "relu6", "prelu"])
 @pytest.mark.parametrize("bias_kind", ["none", "scalar", "channel", "full", "odd"])
 def test_fused_conv2d_epilogues(hip, ref, act, bias_kind):
@@ -938,6 +961,65 @@ def test_separable_conv2d_matches_the_two_op_chain(hip, ref, xs, cout, stride):
                 be.lib.tfhip_separable_single_kernel(be.ctx, 1)
             assert len(kernels2) == 2, kernels2
             close(got, two, rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("xs,cout,stride,kernel", [
+    ((16, 114, 115, 32), 64, 1, "separable_s1_k32xn64_f32"),
+    ((64, 115, 113, 64), 128, 2, "separable_s2_k64xn128_f32"),
+    ((64, 58, 59, 128), 128, 1, "separable_s1_k128xn128_f32"),
+    ((2, 21, 19, 64), 96, 1, "separable_small_s1_f32"),
+    ((2, 21, 19, 64), 96, 2, "separable_small_s2_f32"),
+])
+@pytest.mark.parametrize("pads", ["valid", (2, 2, 2, 2), (2, 0, 1, 3), (0, 1, 2, 0)])
+def test_separable_conv2d_paddings_other_than_same(hip, ref, xs, cout, stride, kernel, pads):
+    """The single-kernel forms take the depthwise half's padding from the Conv2DInfo like the
+    stand-alone depthwise kernel: 'valid', a numeric pad wider than the filter's reach, and top /
+    left / bottom / right all different (which tf.* cannot ask for, the plug-in interface can).
+    Against the oracle's chain on the same Conv2DInfo and bit for bit against the two-kernel form."""
+    print("separable pads", xs, cout, stride, pads, flush=True)
+    tf = hip.tf
+    be = tf.backend()
+    from tfhip.engine import ENGINE
+    rng = rng_for("separable-pads", xs, cout, stride)
+    c = xs[3]
+    x = rng.uniform(0, 1, xs).astype(np.float32)
+    dw = (rng.standard_normal((3, 3, c, 1)) * np.sqrt(2.0 / 9)).astype(np.float32)
+    pw = (rng.standard_normal((1, 1, c, cout)) * np.sqrt(2.0 / c)).astype(np.float32)
+    dbias = (rng.standard_normal(c) * 0.1).astype(np.float32)
+    pbias = (rng.standard_normal(cout) * 0.1).astype(np.float32)
+
+    def info(shape):
+        if pads == "valid":
+            return ref.r.compute_conv2d_info(shape, dw.shape, stride, 1, "valid", depthwise=True)
+        top, left, bottom, right = pads
+        ci = ref.r.compute_conv2d_info(shape, dw.shape, stride, 1, "valid", depthwise=True)
+        oh = (shape[1] + top + bottom - 3) // stride + 1
+        ow = (shape[2] + left + right - 3) // stride + 1
+        ci.update(outHeight=oh, outWidth=ow, outShape=(shape[0], oh, ow, c),
+                  padInfo=dict(top=top, left=left, bottom=bottom, right=right, type="NUMBER"))
+        return ci
+
+    def run():
+        with tf.tidy():
+            ts = [tf.tensor(a) for a in (x, dw, pw, dbias, pbias)]
+            got = []
+            t = tf.time(lambda: got.append(ENGINE.run_kernel(lambda b: b.fused_separable_conv2d(
+                ts[0], ts[1], ts[2], info(xs), ts[3], "relu6", ts[4], "relu6"))))
+            return got[0].data_sync(), [k[0] for k in t["kernelTimes"]]
+
+    got, kernels = run()
+    assert kernels == [kernel], kernels
+    pick = [0, xs[0] - 1]
+    ci = info((2,) + xs[1:])
+    mid = ref.r.clip(ref.r.add(ref.r.depthwise_conv2d(x[pick], dw, ci, pad_quirk=False), dbias), 0.0, 6.0)
+    close(got[pick], ref.conv2d(mid, pw, 1, "valid", bias=pbias, activation="relu6"))
+    be.lib.tfhip_separable_single_kernel(be.ctx, 0)
+    try:
+        two, kernels2 = run()
+    finally:
+        be.lib.tfhip_separable_single_kernel(be.ctx, 1)
+    assert len(kernels2) == 2, kernels2
+    close(got, two, rtol=2e-5, atol=2e-6)
 
 
 @pytest.mark.parametrize("xs,cout,stride", [

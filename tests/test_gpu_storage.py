@@ -540,6 +540,101 @@ def test_graph_captured_under_one_stream_reads_what_the_other_wrote(tf):
     tf.dispose([a, w, b])
 
 
+def test_graph_replays_are_ordered_against_the_other_stream(tf):
+    """A replayed graph writes its tensors every time, so the rule "tensors are written once"
+    cannot order it.  Recorded under index 0; five replays, each fed by a small write (copied by
+    the selected stream, index 1) and each consumed by kernels under index 1 that are still
+    running when the next replay would overwrite what they read.  No host wait in between."""
+    be = tf.backend()
+    rng = np.random.default_rng(36)
+    n = 2048
+    u = tf.tensor(rng.standard_normal((n, 64)).astype(np.float32) * 0.2)
+    w1 = tf.tensor(rng.standard_normal((64, n)).astype(np.float32) * 0.2)
+    w2 = tf.tensor(rng.standard_normal((n, n)).astype(np.float32) * 0.03)
+    w3 = tf.tensor(rng.standard_normal((n, 64)).astype(np.float32) * 0.03)
+    x = tf.tensor(np.zeros((64, 64), np.float32))            # 16 KiB: written through the ring
+    net = lambda: tf.matmul(tf.relu(tf.matmul(tf.matmul(u, x), w1)), w2)      # [n, n]
+    consume = lambda y: tf.tidy(lambda: tf.matmul(tf.relu(tf.matmul(tf.matmul(y, w2), w2)), w3))
+    inputs = [rng.standard_normal((64, 64)).astype(np.float32) for _ in range(5)]
+    want = []
+    for xi in inputs:
+        be.write(x.data_id, xi)
+        with tf.tidy():
+            want.append(consume(net()).data_sync().copy())
+    g = tf.capture_graph(net)                                 # recorded under index 0
+    pending = []
+    for xi in inputs:
+        be.select_stream(1)
+        be.write(x.data_id, xi)                               # a copy queued on stream 1
+        g.replay()                                            # on stream 0
+        z = consume(g.outputs)                                # on stream 1
+        pending.append(z.data())
+        z.dispose()
+    got = [p.result() for p in pending]
+    # and the other way round: index 0 selected, the consumer runs on the replay's own stream
+    be.select_stream(0)
+    be.write(x.data_id, inputs[0])
+    g.replay()
+    with tf.tidy():
+        got.append(consume(g.outputs).data_sync().copy())
+    # an asynchronous read of the graph's own result, still copying when the next replay comes
+    be.write(x.data_id, inputs[1])
+    g.replay()
+    first = g.outputs.data()
+    be.write(x.data_id, inputs[2])
+    g.replay()
+    second = g.outputs.data_sync().copy()
+    first = first.result()
+    g.dispose()
+    for i, (a, e) in enumerate(zip(got, want + [want[0]])):
+        assert np.array_equal(a, e), i
+    for xi, y in ((inputs[1], first), (inputs[2], second)):
+        be.write(x.data_id, xi)
+        with tf.tidy():
+            assert np.array_equal(net().data_sync(), y)
+    tf.dispose([u, w1, w2, w3, x])
+
+
+def test_block_held_by_a_read_goes_to_the_other_stream_behind_its_last_use(tf):
+    """A tensor is read asynchronously, used again by kernels queued under index 0 and disposed
+    while the copy runs; under index 1 a tensor of the same size then takes that very block (the
+    pool of stream 1 has none of the size) and a kernel overwrites it.  The overwrite has to wait
+    for stream 0's kernels, not only for the copy."""
+    be = tf.backend()
+    rng = np.random.default_rng(37)
+    m, n = 2056, 2048                                         # a capacity no other test leaves behind
+    a = tf.tensor(rng.standard_normal((m, n)).astype(np.float32) * 0.03)
+    w = tf.tensor(rng.standard_normal((n, n)).astype(np.float32) * 0.03)
+
+    def chain(y):
+        def f():
+            tf.matmul(tf.matmul(tf.matmul(w, w), w), w)       # long work queued ahead of y's reader
+            return tf.matmul(y, w)
+        return tf.tidy(f)
+
+    with tf.tidy():
+        y = tf.matmul(a, w)
+        want_y = y.data_sync().copy()
+        want_z = chain(y).data_sync().copy()
+    be.sync()
+    y = tf.matmul(a, w)
+    p = y.data()                                              # copying on the download stream
+    z = chain(y)                                              # long work under index 0 that reads y last
+    pooled0 = tf.memory()["numBytesInGPUPool"]
+    y.dispose()                                               # held: the read is still copying
+    held = tf.memory()["numBytesInGPUPool"] - pooled0
+    be.select_stream(1)
+    t = tf.fill((m, n), 7.0)                                  # stream 1 writes into the block
+    took = pooled0 + held - tf.memory()["numBytesInGPUPool"]
+    tv = t.data_sync()
+    be.select_stream(0)
+    assert np.array_equal(p.result(), want_y)
+    assert np.array_equal(z.data_sync(), want_z)
+    assert np.all(tv == 7.0)
+    assert held >= m * n * 4 and took == held, (held, took)   # the held block was the one handed out
+    tf.dispose([a, w, z, t])
+
+
 def test_pipelined_uploads_with_two_batches_in_flight(tf):
     """The serving loop of the benchmark in small: every step uploads its input from page-locked
     memory, runs under the stream of its parity and is read back asynchronously two steps late.

@@ -25,9 +25,7 @@ def _call(fns, case):
         a += [None] * (6 - len(a))
         return pool(a[0], a[1], a[2], a[3], a[4], a[5])
     a += [None] * (8 - len(a))
-    if a[7] is not None and a[7] != "channelsLast":
-        pytest.skip("channelsFirst is not on the hip path")
-    return conv(a[0], a[1], a[2], a[3], a[4], a[5], bool(a[6]))
+    return conv(a[0], a[1], a[2], a[3], a[4], a[5], bool(a[6]), a[7] or "channelsLast")
 
 
 @pytest.mark.parametrize("impl", ["oracle", "driver"])

@@ -69,6 +69,41 @@ def test_conv2d_vs_float64_brute_force(ops, oracle, shape, fshape, stride, pad, 
     rel_close(ops.conv2d(x, w, stride, pad, dil), want, rel=1e-5, ab=1e-5)
 
 
+@pytest.mark.parametrize("shape,fshape,stride,pad", [
+    ((2, 5, 9, 7), (3, 3, 5, 6), 1, "same"),          # [b, c, h, w] with c, h, w all different
+    ((1, 3, 10, 11), (3, 2, 3, 4), 2, "same"),
+    ((2, 4, 8, 6), (2, 3, 4, 3), (1, 2), "valid"),
+])
+def test_conv2d_channels_first(ops, oracle, shape, fshape, stride, pad):
+    """dataFormat 'NCHW' (backend_cpu.ts:1565-1572 changes strides only): against the float64
+    brute force on the transposed images, and bit for bit against the channels-last routine
+    (the loops and their order are the same); so are the two backward kernels, which are also
+    the adjoints of the channels-first forward pass."""
+    rng = np.random.default_rng(13)
+    x = rng.uniform(0, 1, shape).astype(np.float32)
+    w = rng.standard_normal(fshape).astype(np.float32)
+    to_last, to_first = (0, 2, 3, 1), (0, 3, 1, 2)
+    xl = np.ascontiguousarray(x.transpose(to_last))
+    ci = oracle.compute_conv2d_info(shape, fshape, stride, 1, pad, data_format="channelsFirst")
+    p = ci["padInfo"]
+    assert ci["inChannels"] == shape[1] and ci["outShape"][1] == fshape[3]
+    want = _conv_brute(xl, w, ci["strideHeight"], ci["strideWidth"], 1, 1, p["top"], p["left"],
+                       ci["outHeight"], ci["outWidth"]).transpose(to_first)
+    y = ops.conv2d(x, w, stride, pad, data_format="NCHW")
+    assert y.shape == tuple(ci["outShape"])
+    rel_close(y, want, rel=1e-5, ab=1e-5)
+    assert np.array_equal(y, ops.conv2d(xl, w, stride, pad).transpose(to_first))
+    dy = rng.standard_normal(y.shape).astype(np.float32)
+    dyl = np.ascontiguousarray(dy.transpose(to_last))
+    dx = ops.conv2d_der_input(shape, dy, w, stride, pad, data_format="NCHW")
+    dw = ops.conv2d_der_filter(x, dy, fshape, stride, pad, data_format="NCHW")
+    assert np.array_equal(dx, ops.conv2d_der_input(xl.shape, dyl, w, stride, pad).transpose(to_first))
+    assert np.array_equal(dw, ops.conv2d_der_filter(xl, dyl, fshape, stride, pad))
+    lhs = float((y.astype(np.float64) * dy).sum())
+    assert abs(float((dx.astype(np.float64) * x).sum()) - lhs) < 1e-3 * max(1, abs(lhs))
+    assert abs(float((dw.astype(np.float64) * w).sum()) - lhs) < 1e-3 * max(1, abs(lhs))
+
+
 def test_pointwise_conv_is_matmul(ops):
     rng = np.random.default_rng(4)
     x = rng.uniform(0, 1, (2, 5, 5, 16)).astype(np.float32)

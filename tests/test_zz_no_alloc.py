@@ -96,3 +96,42 @@ def test_noalloc_rejects_what_would_need_memory(tf):
         else:
             assert np.array_equal(r1, r2)
     assert refused >= 1
+
+
+def test_noalloc_under_both_stream_indices_takes_turns_on_the_array(tf):
+    """One scratch array per device, two compute streams per context: products cut along K that
+    are queued under alternating stream indices, without a host wait between them, must not
+    write their partial tiles into the array at the same time."""
+    be = tf.backend()
+    lib, ctx = be.lib, be.ctx
+    rng = np.random.default_rng(72)
+    shapes = [(128, 4096, 128), (64, 8192, 64)]
+    h = lambda t: be.data[t.data_id][0]
+    with tf.tidy():
+        ops, want = [], []
+        for (m, k, n) in shapes:
+            a = tf.tensor(rng.uniform(-1, 1, (1, m, k)).astype(np.float32))
+            b = tf.tensor(rng.uniform(-1, 1, (1, k, n)).astype(np.float32))
+            ref = tf.tensor(np.zeros((1, m, n), np.float32))
+            args = (1, m, n, k, 0, 0, -1, 0, 0, -1, 0, None)
+            be._ck(lib.tfhip_matmul(ctx, h(a), h(b), h(ref), *args))
+            assert "splitk" in lib.tfhip_last_kernel(ctx).decode()
+            want.append(ref.data_sync().copy())
+            ops.append((a, b, args))
+        outs = []
+        for i in range(12):
+            a, b, args = ops[i % 2]
+            be.select_stream(i % 2)
+            out = tf.tensor(np.full((1,) + want[i % 2].shape[1:], np.nan, np.float32))
+            be._ck(lib.tfhip_matmul_noalloc(ctx, h(a), h(b), h(out), *args))
+            outs.append(out)
+        # (and the same product under both indices back to back)
+        for i in range(4):
+            a, b, args = ops[0]
+            be.select_stream(i % 2)
+            out = tf.tensor(np.full(want[0].shape, np.nan, np.float32))
+            be._ck(lib.tfhip_matmul_noalloc(ctx, h(a), h(b), h(out), *args))
+            outs.append(out)
+        be.select_stream(0)
+        for i, out in enumerate(outs):
+            assert np.array_equal(out.data_sync(), want[i % 2 if i < 12 else 0]), i

@@ -12,6 +12,10 @@ static thread_local std::string g_init_error;
 static std::mutex g_host_mu;
 static std::map<uintptr_t, size_t> g_pinned;                  // start -> bytes
 static std::map<size_t, std::vector<void*>> g_staging;        // capacity -> free blocks
+static size_t g_staging_bytes = 0;                            // bytes parked in g_staging
+// Page-locked memory is taken from what the whole machine can pin, so finished reads keep at most
+// this much for the next read; a block that would go beyond it is given back to the driver.
+static constexpr size_t kStagingKeepBytes = size_t(256) << 20;
 
 namespace tfhip {
 static bool host_is_pinned(const void* p, size_t nbytes) {
@@ -37,6 +41,7 @@ static void* staging_get(size_t nbytes, size_t* cap) {
     if (it != g_staging.end() && !it->second.empty()) {
       void* p = it->second.back();
       it->second.pop_back();
+      g_staging_bytes -= *cap;
       return p;
     }
   }
@@ -49,8 +54,16 @@ static void* staging_get(size_t nbytes, size_t* cap) {
 }
 static void staging_put(void* p, size_t cap) {
   if (!p) return;
-  std::lock_guard<std::mutex> lock(g_host_mu);
-  g_staging[cap].push_back(p);
+  {
+    std::lock_guard<std::mutex> lock(g_host_mu);
+    if (g_staging_bytes + cap <= kStagingKeepBytes) {
+      g_staging[cap].push_back(p);
+      g_staging_bytes += cap;
+      return;
+    }
+  }
+  // (the copy that used the block is complete: tfhip_read_finish has waited for it)
+  if (hipHostFree(p) != hipSuccess) (void)hipGetLastError();
 }
 }  // namespace tfhip
 
@@ -272,13 +285,16 @@ void* tfhip_ctx::alloc(size_t nbytes, size_t* cap, hipEvent_t* ready, bool* recy
     }
     return p;
   }
-  for (size_t i = 0; i < held.size(); i++) {
+  // (not while capturing: the wait below is for an event from outside the capture)
+  for (size_t i = 0; i < held.size() && !capturing; i++) {
     if (held[i].cap != want) continue;
-    // no free block of this size, but one whose read is still copying: take it and put the copy
-    // in front of whatever the compute stream does next
+    // no free block of this size, but one whose read is still copying: take it and put the copy,
+    // and whatever its last stream still has queued on it, in front of what the selected stream
+    // does next
     const HeldBlock h = held[i];
     held[i] = held.back();
     held.pop_back();
+    order(h.sidx, cur);
     (void)hipStreamWaitEvent(stream, h.done, 0);
     ev_put(h.left);
     pooled -= want;
@@ -780,6 +796,7 @@ int tfhip_select_stream(tfhip_ctx* ctx, int index) {
   if (ctx->time_depth) return ctx->fail(TFHIP_EINVAL, "select_stream: not inside a timed region");
   ctx->cur = index;
   ctx->stream = ctx->streams[index];
+  ctx->dirty |= (unsigned char)(1u << index);
   return TFHIP_OK;
 }
 
@@ -844,6 +861,7 @@ int tfhip_graph_begin(tfhip_ctx* ctx) {
   if (!ctx) return TFHIP_EINVAL;
   if (ctx->capturing) return ctx->fail(TFHIP_EINVAL, "graph_begin: a capture is already running");
   ctx->capture_blocks.clear();
+  ctx->capture_used_scratch = false;
   // uploads still on their way are waited for before the recording starts: a wait for an
   // event of another stream must not become part of the graph
   int rc = ctx->await_uploads();
@@ -868,6 +886,7 @@ int tfhip_graph_end(tfhip_ctx* ctx, int64_t* graph_id) {
   }
   const int64_t id = ctx->next_graph++;
   g.sidx = ctx->cur;
+  g.uses_scratch = ctx->capture_used_scratch;
   // Every block the capture handed out now belongs to the graph: those lying free in the pool
   // are taken out of it, the others follow when their tensor lets go of them (release()).
   for (void* p : ctx->capture_blocks) {
@@ -900,9 +919,34 @@ int tfhip_graph_launch(tfhip_ctx* ctx, int64_t graph_id) {
   // through the upload stream has to arrive first
   int rc = ctx->await_uploads();
   if (rc) return rc;
-  // (on the stream of the capture, whichever is selected: the tensors the recorded work
-  // produced are booked as written there)
-  TFHIP_HIP(ctx, hipGraphLaunch(it->second.exec, ctx->streams[it->second.sidx]));
+  tfhip_ctx::Graph& g = it->second;
+  // A replay reads its inputs at their addresses and writes its blocks again, every time.  So it
+  // runs behind everything the other compute streams have queued so far (a small write into an
+  // input copied by the other stream, kernels there that still read the previous replay's
+  // results), and behind asynchronous reads still copying out of its blocks ...
+  for (int s = 0; s < tfhip_ctx::kStreams; s++) {
+    if (s == g.sidx || !(ctx->dirty >> s & 1)) continue;
+    ctx->order(s, g.sidx);
+    if (s != ctx->cur) ctx->dirty &= (unsigned char)~(1u << s);
+  }
+  const unsigned char gbit = (unsigned char)(1u << g.sidx);
+  for (auto& kv : ctx->bufs) {
+    Buf& b = kv.second;
+    if (!b.ptr) continue;
+    auto own = ctx->owner.find(b.ptr);
+    if (own == ctx->owner.end() || own->second != graph_id) continue;
+    if (b.read_done) TFHIP_HIP(ctx, hipStreamWaitEvent(ctx->streams[g.sidx], b.read_done, 0));
+    // ... and the tensors on its blocks are booked as written anew on the capture's stream: the
+    // next consumer on another stream waits again, a host read follows this stream.
+    b.wsidx = g.sidx;
+    b.vis = gbit;
+    b.users |= gbit;
+    b.sidx = g.sidx;
+    b.used = true;
+  }
+  if (g.uses_scratch) ctx->scratch_sidx = g.sidx;
+  // (on the stream of the capture, whichever is selected)
+  TFHIP_HIP(ctx, hipGraphLaunch(g.exec, ctx->streams[g.sidx]));
   return TFHIP_OK;
 }
 

@@ -1612,6 +1612,10 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
                          "tfhip_matmul", need, kScratchBytes);
       p.partials = static_cast<float*>(scratch_address(ctx));
       if (!p.partials) return TFHIP_EDEVICE;
+      // one array per device, two compute streams: behind the other stream's last use of it
+      if (ctx->scratch_sidx >= 0 && ctx->scratch_sidx != ctx->cur) ctx->order(ctx->scratch_sidx, ctx->cur);
+      ctx->scratch_sidx = ctx->cur;
+      if (ctx->capturing) ctx->capture_used_scratch = true;
     } else {
       if (!partials.get(need)) return TFHIP_EDEVICE;
       p.partials = static_cast<float*>(partials.ptr);

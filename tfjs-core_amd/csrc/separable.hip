@@ -966,8 +966,9 @@ extern "C" int tfhip_separable_conv2d(tfhip_ctx* ctx, int64_t x, int64_t dw_filt
   return rc;
 }
 
-// Switches the single-kernel form off (1) or on (0): tests and measurements compare the two
-// forms on the same operands.
+// enable = 0 switches the single-kernel forms off (every call then runs its two kernels), any
+// other value switches them on again: tests and measurements compare the two forms on the same
+// operands.
 extern "C" int tfhip_separable_single_kernel(tfhip_ctx* ctx, int enable) {
   if (!ctx) return TFHIP_EINVAL;
   ctx->separable_off = !enable;

@@ -102,6 +102,9 @@ struct tfhip_ctx {
   static constexpr unsigned char kAllStreams = (unsigned char)((1u << kStreams) - 1);
   hipStream_t streams[kStreams] = {};
   int cur = 0;  // index of `stream`
+  // Streams that may hold queued work which a graph replay has not been ordered behind yet (a bit
+  // per stream, set when the stream is selected): a replay waits for these, see tfhip_graph_launch.
+  unsigned char dirty = 1;
   std::map<size_t, std::vector<void*>> pools[kStreams];  // capacity -> free blocks, reused LIFO
   size_t in_use = 0, pooled = 0;
   std::string err;
@@ -174,8 +177,10 @@ struct tfhip_ctx {
     hipGraphExec_t exec = nullptr;
     std::vector<std::pair<void*, size_t>> parked;  // owned blocks that no tensor holds
     int sidx = 0;  // the compute stream it was recorded on, and replays on
+    bool uses_scratch = false;  // a recorded kernel keeps partial tiles in the static scratch array
   };
   bool capturing = false;
+  bool capture_used_scratch = false;
   std::vector<void*> capture_blocks;
   std::unordered_map<void*, int64_t> owner;  // block -> graph that owns it
   std::unordered_map<int64_t, Graph> graphs;
@@ -185,6 +190,7 @@ struct tfhip_ctx {
   // the driver once, at init), and the flag that routes scratch needs there while it runs.
   void* scratch = nullptr;
   bool no_alloc = false;
+  int scratch_sidx = -1;  // the compute stream whose queued work used the scratch array last
   bool separable_off = false;  // tfhip_separable_conv2d always runs its two-kernel form
 
   int fail(int code, const char* fmt, ...);

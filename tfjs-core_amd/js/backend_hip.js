@@ -65,6 +65,12 @@ function convInfoArray(ci) {
   ]);
 }
 
+// The Conv2DInfo of the same convolution on NHWC images.
+function channelsLastInfo(ci) {
+  const last = s => [s[0], s[2], s[3], s[1]];
+  return Object.assign({}, ci, {dataFormat: 'channelsLast', inShape: last(ci.inShape), outShape: last(ci.outShape)});
+}
+
 class MathBackendHIP extends KernelBackend {
   constructor(device) {
     super();
@@ -306,6 +312,7 @@ class MathBackendHIP extends KernelBackend {
     return {
       outputs,
       replay: () => {
+        this.flushAll();  // deferred work that reads the previous replay's results comes first
         this.napi.graphLaunch(this.ctx, id);
         return outputs;
       },
@@ -490,7 +497,14 @@ class MathBackendHIP extends KernelBackend {
     return out;
   }
 
+  // channelsFirst (NCHW; backend_cpu.ts:1565-1572, 1698-1706, 1857-1865 walk the same loops through
+  // other strides): the images are turned to NHWC, which the kernels stream with channel-contiguous
+  // accesses, and the result is turned back.
   conv2d(x, filter, convInfo) {
+    if (convInfo.dataFormat === 'channelsFirst') {
+      const y = this.fusedConv2d(this.transpose(x, [0, 2, 3, 1]), filter, channelsLastInfo(convInfo));
+      return this.transpose(y, [0, 3, 1, 2]);
+    }
     return this.fusedConv2d(x, filter, convInfo);
   }
 
@@ -627,9 +641,18 @@ class MathBackendHIP extends KernelBackend {
     return out;
   }
   conv2dDerInput(dy, filter, convInfo) {
+    if (convInfo.dataFormat === 'channelsFirst') {
+      const ci = channelsLastInfo(convInfo);
+      const dx = this.backward('conv2dDerInput', this.transpose(dy, [0, 2, 3, 1]), filter, ci.inShape, ci);
+      return this.transpose(dx, [0, 3, 1, 2]);
+    }
     return this.backward('conv2dDerInput', dy, filter, convInfo.inShape, convInfo);
   }
   conv2dDerFilter(x, dy, convInfo) {
+    if (convInfo.dataFormat === 'channelsFirst') {
+      return this.backward('conv2dDerFilter', this.transpose(x, [0, 2, 3, 1]), this.transpose(dy, [0, 2, 3, 1]),
+                           convInfo.filterShape, channelsLastInfo(convInfo));
+    }
     return this.backward('conv2dDerFilter', x, dy, convInfo.filterShape, convInfo);
   }
   depthwiseConv2DDerInput(dy, filter, convInfo) {

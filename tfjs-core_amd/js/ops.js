@@ -226,7 +226,8 @@ const fusedMatMul = op('fusedMatMul', (config) => {
 });
 
 // ---- conv2d / depthwiseConv2d -------------------------------------------------------------
-function convPrep(x, filter, strides, pad, dataFormat, dilations, dimRoundingMode, name, depthwise) {
+function convPrep(x, filter, strides, pad, dataFormat, dilations, dimRoundingMode, name, depthwise,
+                  nchwAllowed) {
   const $x = convertToTensor(x, 'x', name);
   const $filter = convertToTensor(filter, 'filter', name);
   let x4D = $x;
@@ -250,10 +251,13 @@ function convPrep(x, filter, strides, pad, dataFormat, dilations, dimRoundingMod
   util.assert(conv_util.eitherStridesOrDilationsAreOne(strides, dilations),
               () => `Error in ${name}: Either strides or dilations must be 1. ` +
                   `Got strides ${strides} and dilations '${dilations}'`);
-  util.assert(dataFormat === 'NHWC',
+  // conv2d takes both formats (ops/conv.ts:148, 184-187); the fused and depthwise ops NHWC only
+  // (ops/fused_ops.ts:332-335)
+  util.assert(dataFormat === 'NHWC' || nchwAllowed === true,
               () => `Error in ${name}: got dataFormat of ${dataFormat} but only NHWC is currently supported.`);
   const convInfo = conv_util.computeConv2DInfo(x4D.shape, $filter.shape, strides, dilations, pad,
-                                               dimRoundingMode, depthwise);
+                                               dimRoundingMode, depthwise,
+                                               conv_util.convertConv2DDataFormat(dataFormat));
   return {$x, x4D, $filter, convInfo, reshapedTo4D};
 }
 
@@ -263,23 +267,25 @@ function lower(res, reshapedTo4D) {
 
 const conv2d = op('conv2d', (x, filter, strides, pad, dataFormat, dilations, dimRoundingMode) => {
   const {x4D, $filter, convInfo, reshapedTo4D} =
-      convPrep(x, filter, strides, pad, dataFormat, dilations, dimRoundingMode, 'conv2d', false);
+      convPrep(x, filter, strides, pad, dataFormat, dilations, dimRoundingMode, 'conv2d', false, true);
   const res = ENGINE.runKernel((backend, save) => {
     save([$filter, x4D]);
     return backend.conv2d(x4D, $filter, convInfo);
-  }, {x: x4D, $filter}, (dy, saved) => conv2dGrads(dy, saved[1], saved[0], strides, pad, dilations));
+  }, {x: x4D, $filter},
+  (dy, saved) => conv2dGrads(dy, saved[1], saved[0], strides, pad, dilations, dataFormat));
   return lower(res, reshapedTo4D);
 });
 
 // ops/conv.ts:236-250
-function conv2dGrads(dy, x4D, filter, strides, pad, dilations) {
+function conv2dGrads(dy, x4D, filter, strides, pad, dilations, dataFormat) {
   if (dilations == null) dilations = [1, 1];
+  if (dataFormat == null) dataFormat = 'NHWC';
   util.assert(conv_util.tupleValuesAreOne(dilations),
               () => 'Error in gradient of conv2D: dilation rates greater than 1 ' +
                   `are not yet supported in gradients. Got dilations '${dilations}'`);
   return {
-    x: () => conv2dDerInput(x4D.shape, dy, filter, strides, pad, 'NHWC'),
-    $filter: () => conv2dDerFilter(x4D, dy, filter.shape, strides, pad, 'NHWC')
+    x: () => conv2dDerInput(x4D.shape, dy, filter, strides, pad, dataFormat),
+    $filter: () => conv2dDerFilter(x4D, dy, filter.shape, strides, pad, dataFormat)
   };
 }
 
@@ -490,19 +496,20 @@ const conv2dDerInput = op('conv2dDerInput', (xShape, dy, filter, strides, pad, d
   util.assert($filter.rank === 4,
               () => `Error in conv2dDerInput: filter must be rank 4, but got rank ${$filter.rank}`);
   if (dataFormat == null) dataFormat = 'NHWC';
-  util.assert(dataFormat === 'NHWC',
-              () => `Error in conv2dDerInput: got dataFormat of ${dataFormat} but only NHWC is currently supported.`);
-  util.assert(xShape4D[3] === $filter.shape[2],
-              () => `Error in conv2dDerInput: depth of input (${xShape4D[3]}) must ` +
+  const inDepth = dataFormat === 'NHWC' ? xShape4D[3] : xShape4D[1];  // ops/conv.ts:274-275
+  const outDepth = dataFormat === 'NHWC' ? dy4D.shape[3] : dy4D.shape[1];
+  util.assert(inDepth === $filter.shape[2],
+              () => `Error in conv2dDerInput: depth of input (${inDepth}) must ` +
                   `match input depth for filter ${$filter.shape[2]}.`);
-  util.assert(dy4D.shape[3] === $filter.shape[3],
-              () => `Error in conv2dDerInput: depth of output (${dy4D.shape[3]}) must ` +
+  util.assert(outDepth === $filter.shape[3],
+              () => `Error in conv2dDerInput: depth of output (${outDepth}) must ` +
                   `match output depth for filter ${$filter.shape[3]}.`);
   if (dimRoundingMode != null) {
     util.assert(util.isInt(pad), () => `Error in conv2dDerInput: pad must be an integer when using, ` +
         `dimRoundingMode ${dimRoundingMode} but got pad ${pad}.`);
   }
-  const convInfo = conv_util.computeConv2DInfo(xShape4D, $filter.shape, strides, 1, pad, dimRoundingMode, false);
+  const convInfo = conv_util.computeConv2DInfo(xShape4D, $filter.shape, strides, 1, pad, dimRoundingMode, false,
+                                               conv_util.convertConv2DDataFormat(dataFormat));
   util.assert(sameShape(convInfo.outShape, dy4D.shape),
               () => `Error in conv2dDerInput: dy has shape ${dy4D.shape}, the convolution of an ` +
                   `input of shape ${xShape4D} gives ${convInfo.outShape}`);
@@ -510,8 +517,8 @@ const conv2dDerInput = op('conv2dDerInput', (xShape, dy, filter, strides, pad, d
     save([$filter, dy4D]);
     return backend.conv2dDerInput(dy4D, $filter, convInfo);
   }, {dy4D, $filter}, (ddx, saved) => ({  // ops/conv.ts:299-311
-    dy4D: () => conv2d(ddx, saved[0], strides, pad, 'NHWC', 1, dimRoundingMode),
-    $filter: () => conv2dDerFilter(ddx, saved[1], saved[0].shape, strides, pad, 'NHWC', dimRoundingMode)
+    dy4D: () => conv2d(ddx, saved[0], strides, pad, dataFormat, 1, dimRoundingMode),
+    $filter: () => conv2dDerFilter(ddx, saved[1], saved[0].shape, strides, pad, dataFormat, dimRoundingMode)
   }));
   return lower(res, reshapedTo4D);
 });
@@ -523,19 +530,20 @@ const conv2dDerFilter = op('conv2dDerFilter', (x, dy, filterShape, strides, pad,
   util.assert(filterShape.length === 4,
               () => `Error in conv2dDerFilter: filterShape must be length 4, but got ${filterShape}.`);
   if (dataFormat == null) dataFormat = 'NHWC';
-  util.assert(dataFormat === 'NHWC',
-              () => `Error in conv2dDerFilter: got dataFormat of ${dataFormat} but only NHWC is currently supported.`);
-  util.assert(x4D.shape[3] === filterShape[2],
-              () => `Error in conv2dDerFilter: depth of input ${x4D.shape[3]}) must ` +
+  const inDepth = dataFormat === 'NHWC' ? x4D.shape[3] : x4D.shape[1];  // ops/conv.ts:367-368
+  const outDepth = dataFormat === 'NHWC' ? dy4D.shape[3] : dy4D.shape[1];
+  util.assert(inDepth === filterShape[2],
+              () => `Error in conv2dDerFilter: depth of input ${inDepth}) must ` +
                   `match input depth in filter (${filterShape[2]}.`);
-  util.assert(dy4D.shape[3] === filterShape[3],
-              () => `Error in conv2dDerFilter: depth of dy (${dy4D.shape[3]}) must ` +
+  util.assert(outDepth === filterShape[3],
+              () => `Error in conv2dDerFilter: depth of dy (${outDepth}) must ` +
                   `match output depth for filter (${filterShape[3]}).`);
   if (dimRoundingMode != null) {
     util.assert(util.isInt(pad), () => `Error in conv2dDerFilter: pad must be an integer when using, ` +
         `dimRoundingMode ${dimRoundingMode} but got pad ${pad}.`);
   }
-  const convInfo = conv_util.computeConv2DInfo(x4D.shape, filterShape, strides, 1, pad, dimRoundingMode, false);
+  const convInfo = conv_util.computeConv2DInfo(x4D.shape, filterShape, strides, 1, pad, dimRoundingMode, false,
+                                               conv_util.convertConv2DDataFormat(dataFormat));
   util.assert(sameShape(convInfo.outShape, dy4D.shape),
               () => `Error in conv2dDerFilter: dy has shape ${dy4D.shape}, the convolution gives ${convInfo.outShape}`);
   return ENGINE.runKernel(backend => backend.conv2dDerFilter(x4D, dy4D, convInfo), {x4D, dy4D});

@@ -30,7 +30,7 @@ const OPS = {
   fusedMatMul: (i, a) => tf.fused.matMul({
     a: i.a, b: i.b, transposeA: a.transposeA, transposeB: a.transposeB, bias: i.bias,
     activation: a.activation, preluActivationWeights: i.prelu}),
-  conv2d: (i, a) => tf.conv2d(i.x, i.filter, a.strides, a.pad, 'NHWC', a.dilations, a.dimRoundingMode),
+  conv2d: (i, a) => tf.conv2d(i.x, i.filter, a.strides, a.pad, a.dataFormat || 'NHWC', a.dilations, a.dimRoundingMode),
   fusedConv2d: (i, a) => tf.fused.conv2d({
     x: i.x, filter: i.filter, strides: a.strides, pad: a.pad, dilations: a.dilations,
     bias: i.bias, activation: a.activation, preluActivationWeights: i.prelu}),
@@ -204,8 +204,8 @@ const OPS = {
   logicalNot: i => tf.logicalNot(i.x),
   batchNorm: (i, a) => tf.batchNorm(i.x, i.mean, i.variance, i.offset, i.scale, a.varianceEpsilon),
   resizeBilinear: (i, a) => tf.resizeBilinear(i.x, a.size, a.alignCorners),
-  conv2dDerInput: (i, a) => tf.conv2dDerInput(a.xShape, i.dy, i.filter, a.strides, a.pad),
-  conv2dDerFilter: (i, a) => tf.conv2dDerFilter(i.x, i.dy, a.filterShape, a.strides, a.pad),
+  conv2dDerInput: (i, a) => tf.conv2dDerInput(a.xShape, i.dy, i.filter, a.strides, a.pad, a.dataFormat),
+  conv2dDerFilter: (i, a) => tf.conv2dDerFilter(i.x, i.dy, a.filterShape, a.strides, a.pad, a.dataFormat),
   conv2dTranspose: (i, a) => tf.conv2dTranspose(i.x, i.filter, a.outputShape, a.strides, a.pad),
   depthwiseConv2dDerInput: (i, a) => tf.depthwiseConv2dDerInput(a.xShape, i.dy, i.filter, a.strides, a.pad),
   depthwiseConv2dDerFilter: (i, a) => tf.depthwiseConv2dDerFilter(i.x, i.dy, a.filterShape, a.strides, a.pad),
@@ -218,7 +218,7 @@ const OPS = {
   splitStack: (i, a) => tf.stack(tf.split(i.x, a.sizes, a.axis).map(t => tf.squeeze(tf.expandDims(t, 0), [0])), a.stackAxis),
   unstackConcat: (i, a) => tf.concat(tf.unstack(i.x, a.axis), a.concatAxis),
   // gradients through the tape (tf.grad / tf.grads); `wrt` picks the argument
-  gradConv2d: (i, a) => tf.grads((x, f) => tf.conv2d(x.clone(), f.clone(), a.strides, a.pad).clone())(
+  gradConv2d: (i, a) => tf.grads((x, f) => tf.conv2d(x.clone(), f.clone(), a.strides, a.pad, a.dataFormat).clone())(
       [i.x, i.filter], i.dy)[a.wrt],
   gradConv2dTranspose: (i, a) => tf.grads((x, f) => tf.conv2dTranspose(x, f, a.outputShape, a.strides, a.pad))(
       [i.x, i.filter], i.dy)[a.wrt],

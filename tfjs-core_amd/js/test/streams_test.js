@@ -79,6 +79,39 @@ async function main() {
   be.selectStream(0);
   check('read across streams', same(t.dataSync(), tf.tidy(() => tf.relu(w2).dataSync())));
   t.dispose();
+
+  // A graph recorded under index 0 and replayed five times; every replay is fed by a small write
+  // while index 1 is selected (the copy is queued on stream 1) and consumed by kernels under
+  // index 1 that still run when the next replay rewrites what they read.  No host wait between.
+  {
+    const n = 1536;
+    const u = tf.tensor(values(n * 64, 20, -0.2, 0.2), [n, 64]);
+    const v1 = tf.tensor(values(64 * n, 21, -0.2, 0.2), [64, n]);
+    const v2 = tf.tensor(values(n * n, 22, -0.03, 0.03), [n, n]);
+    const v3 = tf.tensor(values(n * 64, 23, -0.03, 0.03), [n, 64]);
+    const x = tf.tensor(new Float32Array(64 * 64), [64, 64]);
+    const gnet = () => tf.matMul(tf.relu(tf.matMul(tf.matMul(u, x), v1)), v2);
+    const consume = y => tf.tidy(() => tf.matMul(tf.relu(tf.matMul(tf.matMul(y, v2), v2)), v3));
+    const inputs = [0, 1, 2, 3, 4].map(k => values(64 * 64, 30 + k, -1, 1));
+    const wantG = inputs.map(xi => {
+      be.write(x.dataId, xi);
+      return tf.tidy(() => consume(gnet()).dataSync());
+    });
+    const g = tf.captureGraph(gnet);
+    const reads = [];
+    for (const xi of inputs) {
+      be.selectStream(1);
+      be.write(x.dataId, xi);
+      g.replay();
+      const z = consume(g.outputs);
+      reads.push(z.data());
+      z.dispose();
+    }
+    be.selectStream(0);
+    for (let i = 0; i < reads.length; i++) check('replay ' + i, same(await reads[i], wantG[i]));
+    g.dispose();
+    [u, v1, v2, v3, x].forEach(t => t.dispose());
+  }
   console.log(JSON.stringify({ok: failures.length === 0, failures}));
 }
 main().catch(e => { console.log(JSON.stringify({ok: false, failures: [String(e && e.stack || e)]})); });

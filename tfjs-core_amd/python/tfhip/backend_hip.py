@@ -328,7 +328,22 @@ class MathBackendHIP(object):
             self._h(prelu) if pk else -1, pk, self._q(b)))
         return out
 
+    # channelsFirst (NCHW, backend_cpu.ts:1565-1572, 1698-1706, 1857-1865 walk the same loops
+    # through other strides): the images are turned to NHWC, which the kernels stream with
+    # channel-contiguous accesses, and the result is turned back.
+    _TO_LAST, _TO_FIRST = (0, 2, 3, 1), (0, 3, 1, 2)
+
+    @staticmethod
+    def _channels_last_info(ci):
+        last = lambda s: (s[0], s[2], s[3], s[1])
+        return dict(ci, dataFormat="channelsLast", inShape=last(ci["inShape"]),
+                    outShape=last(ci["outShape"]))
+
     def conv2d(self, x, filter, conv_info):
+        if conv_info.get("dataFormat", "channelsLast") == "channelsFirst":
+            y = self.fused_conv2d(self.transpose(x, self._TO_LAST), filter,
+                                  self._channels_last_info(conv_info), None, None, None)
+            return self.transpose(y, self._TO_FIRST)
         return self.fused_conv2d(x, filter, conv_info, None, None, None)
 
     def fused_conv2d(self, x, filter, conv_info, bias=None, activation=None,
@@ -421,10 +436,19 @@ class MathBackendHIP(object):
         return out
 
     def conv2d_der_input(self, dy, filter, conv_info):
+        if conv_info.get("dataFormat", "channelsLast") == "channelsFirst":
+            ci = self._channels_last_info(conv_info)
+            dx = self._backward(self.lib.tfhip_conv2d_der_input, self.transpose(dy, self._TO_LAST),
+                                filter, ci["inShape"], ci)
+            return self.transpose(dx, self._TO_FIRST)
         return self._backward(self.lib.tfhip_conv2d_der_input, dy, filter, conv_info["inShape"],
                               conv_info)
 
     def conv2d_der_filter(self, x, dy, conv_info):
+        if conv_info.get("dataFormat", "channelsLast") == "channelsFirst":
+            return self._backward(self.lib.tfhip_conv2d_der_filter,
+                                  self.transpose(x, self._TO_LAST), self.transpose(dy, self._TO_LAST),
+                                  conv_info["filterShape"], self._channels_last_info(conv_info))
         return self._backward(self.lib.tfhip_conv2d_der_filter, x, dy, conv_info["filterShape"],
                               conv_info)
 

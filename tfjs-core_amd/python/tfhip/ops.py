@@ -126,7 +126,8 @@ def fused_matmul(a, b, transpose_a=False, transpose_b=False, bias=None, activati
 
 
 # ---- convolutions (ops/conv.ts:145-217, 470-540; ops/fused_ops.ts:276-425) ----
-def _conv_prep(x, filt, strides, pad, data_format, dilations, rounding, name, depthwise=False):
+def _conv_prep(x, filt, strides, pad, data_format, dilations, rounding, name, depthwise=False,
+               nchw_allowed=False):
     x, filt = _conv(x, "x", name), _conv(filt, "filter", name)
     lifted = x.rank == 3
     x4 = reshape(x, (1,) + x.shape) if lifted else x
@@ -137,18 +138,24 @@ def _conv_prep(x, filt, strides, pad, data_format, dilations, rounding, name, de
     if rounding is not None and not (isinstance(pad, (int, float)) and float(pad) == int(pad)):
         raise ValueError("Error in %s: pad must be an integer when using, dimRoundingMode %s but "
                          "got pad %s." % (name, rounding, pad))
-    if x4.shape[3] != filt.shape[2]:
+    if data_format is None:
+        data_format = "NHWC"
+    in_depth = x4.shape[3] if data_format == "NHWC" else x4.shape[1]
+    if in_depth != filt.shape[2]:
         raise ValueError("Error in %s: depth of input (%d) must match input depth for filter %d."
-                         % (name, x4.shape[3], filt.shape[2]))
+                         % (name, in_depth, filt.shape[2]))
     if dilations is None:
         dilations = (1, 1)
     if not su.either_strides_or_dilations_are_one(strides, dilations):
         raise ValueError("Error in %s: Either strides or dilations must be 1. Got strides %s and "
                          "dilations '%s'" % (name, strides, dilations))
-    if data_format != "NHWC":
+    # conv2d takes both formats (ops/conv.ts:148, 184-187); the fused and depthwise ops NHWC only
+    # (ops/fused_ops.ts:332-335)
+    if data_format != "NHWC" and not nchw_allowed:
         raise ValueError("Error in %s: got dataFormat of %s but only NHWC is currently supported."
                          % (name, data_format))
-    ci = su.compute_conv2d_info(x4.shape, filt.shape, strides, dilations, pad, rounding, depthwise)
+    ci = su.compute_conv2d_info(x4.shape, filt.shape, strides, dilations, pad, rounding, depthwise,
+                                su.convert_conv2d_data_format(data_format))
     return x4, filt, ci, lifted
 
 
@@ -159,7 +166,7 @@ def _lower(r, lifted):
 def conv2d(x, filt, strides, pad, data_format="NHWC", dilations=(1, 1), dim_rounding_mode=None):
     def run():
         x4, f, ci, lifted = _conv_prep(x, filt, strides, pad, data_format, dilations,
-                                       dim_rounding_mode, "conv2d")
+                                       dim_rounding_mode, "conv2d", nchw_allowed=True)
         return _lower(ENGINE.run_kernel(lambda be: be.conv2d(x4, f, ci)), lifted)
     return ENGINE.tidy(run)
 
@@ -916,20 +923,19 @@ def conv2d_der_input(x_shape, dy, filt, strides, pad, data_format="NHWC", dim_ro
             raise ValueError("Error in conv2dDerInput: dy must be rank 4, but got rank %d" % dy4.rank)
         if f.rank != 4:
             raise ValueError("Error in conv2dDerInput: filter must be rank 4, but got rank %d" % f.rank)
-        if data_format != "NHWC":
-            raise ValueError("Error in conv2dDerInput: got dataFormat of %s but only NHWC is "
-                             "currently supported." % data_format)
-        if xs4[3] != f.shape[2]:
+        ch = 3 if data_format == "NHWC" else 1   # ops/conv.ts:274-275
+        if xs4[ch] != f.shape[2]:
             raise ValueError("Error in conv2dDerInput: depth of input (%d) must match input depth "
-                             "for filter %d." % (xs4[3], f.shape[2]))
-        if dy4.shape[3] != f.shape[3]:
+                             "for filter %d." % (xs4[ch], f.shape[2]))
+        if dy4.shape[ch] != f.shape[3]:
             raise ValueError("Error in conv2dDerInput: depth of output (%d) must match output depth "
-                             "for filter %d." % (dy4.shape[3], f.shape[3]))
+                             "for filter %d." % (dy4.shape[ch], f.shape[3]))
         if dim_rounding_mode is not None and not (isinstance(pad, (int, float)) and
                                                   float(pad) == int(pad)):
             raise ValueError("Error in conv2dDerInput: pad must be an integer when using, "
                              "dimRoundingMode %s but got pad %s." % (dim_rounding_mode, pad))
-        ci = su.compute_conv2d_info(xs4, f.shape, strides, 1, pad, dim_rounding_mode, False)
+        ci = su.compute_conv2d_info(xs4, f.shape, strides, 1, pad, dim_rounding_mode, False,
+                                    su.convert_conv2d_data_format(data_format))
         if tuple(ci["outShape"]) != tuple(dy4.shape):
             raise ValueError("Error in conv2dDerInput: dy has shape %s, the convolution of an input "
                              "of shape %s gives %s" % (list(dy4.shape), list(xs4),
@@ -952,20 +958,19 @@ def conv2d_der_filter(x, dy, filter_shape, strides, pad, data_format="NHWC", dim
         if len(fs) != 4:
             raise ValueError("Error in conv2dDerFilter: filterShape must be length 4, but got %s."
                              % list(fs))
-        if data_format != "NHWC":
-            raise ValueError("Error in conv2dDerFilter: got dataFormat of %s but only NHWC is "
-                             "currently supported." % data_format)
-        if x4.shape[3] != fs[2]:
+        ch = 3 if data_format == "NHWC" else 1   # ops/conv.ts:367-368
+        if x4.shape[ch] != fs[2]:
             raise ValueError("Error in conv2dDerFilter: depth of input %d) must match input depth "
-                             "in filter (%d." % (x4.shape[3], fs[2]))
-        if dy4.shape[3] != fs[3]:
+                             "in filter (%d." % (x4.shape[ch], fs[2]))
+        if dy4.shape[ch] != fs[3]:
             raise ValueError("Error in conv2dDerFilter: depth of dy (%d) must match output depth "
-                             "for filter (%d)." % (dy4.shape[3], fs[3]))
+                             "for filter (%d)." % (dy4.shape[ch], fs[3]))
         if dim_rounding_mode is not None and not (isinstance(pad, (int, float)) and
                                                   float(pad) == int(pad)):
             raise ValueError("Error in conv2dDerFilter: pad must be an integer when using, "
                              "dimRoundingMode %s but got pad %s." % (dim_rounding_mode, pad))
-        ci = su.compute_conv2d_info(x4.shape, fs, strides, 1, pad, dim_rounding_mode, False)
+        ci = su.compute_conv2d_info(x4.shape, fs, strides, 1, pad, dim_rounding_mode, False,
+                                    su.convert_conv2d_data_format(data_format))
         if tuple(ci["outShape"]) != tuple(dy4.shape):
             raise ValueError("Error in conv2dDerFilter: dy has shape %s, the convolution gives %s"
                              % (list(dy4.shape), list(ci["outShape"])))

@@ -102,6 +102,15 @@ def compute_conv2d_info(in_shape, filter_shape, strides, dilations, pad, roundin
                 filterShape=tuple(filter_shape))
 
 
+def convert_conv2d_data_format(data_format):
+    """convertConv2DDataFormat (ops/conv_util.ts:545-554)."""
+    if data_format == "NHWC":
+        return "channelsLast"
+    if data_format == "NCHW":
+        return "channelsFirst"
+    raise ValueError("Unknown dataFormat %s" % data_format)
+
+
 def compute_pool2d_info(in_shape, filter_size, strides, dilations, pad, rounding_mode=None,
                         data_format="channelsLast"):
     f_h, f_w = _tuple2(filter_size)
