@@ -291,9 +291,11 @@ def write_weight_files(params, directory, shard_bytes=4 << 20):
     return manifest_path
 
 
-def js_host_leg(params, x_host, batch, steps, warmup):
+def js_host_leg(params, x_host, batch, steps, warmup, priming=None, legs=None):
     """The same step driven by the JavaScript host (tf.* graph in Node.js over the N-API
-    addon), as a child process on the same bytes.  None when node is not installed."""
+    addon), as a child process on the same bytes.  None when node is not installed.
+    priming: untimed steps before the warm-up steps (None: the child's default); legs: the
+    measurements to run (None: all of them)."""
     import shutil
     import subprocess
     import tempfile
@@ -305,11 +307,81 @@ def js_host_leg(params, x_host, batch, steps, warmup):
         xb = os.path.join(d, "x.bin")
         mf = write_weight_files(params, d)
         x_host.tofile(xb)
-        r = subprocess.run([node, os.path.join(js, "bench_mobilenet.js"), mf, xb, str(batch),
-                            str(steps), str(warmup)], capture_output=True, text=True, timeout=600)
+        cmd = [node, os.path.join(js, "bench_mobilenet.js"), mf, xb, str(batch), str(steps), str(warmup)]
+        if priming is not None:
+            cmd.append("priming=%d" % priming)
+        if legs is not None:
+            cmd.append("legs=" + ",".join(legs))
+        r = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
     if r.returncode != 0:
         return dict(error=(r.stderr or r.stdout)[-400:])
     return json.loads(r.stdout.strip().splitlines()[-1])
+
+
+def other_configs(tf, mobilenet, params, np):
+    """Short legs for the two other MobileNet configurations of the benchmark definition, through
+    the JavaScript host when node is installed (the Python driver otherwise):
+      batch 1, fp32: one image per step, eager and as a captured graph (a step is 20 launches of a
+        few microseconds, so the host's cost per launch decides);
+      batch 256, uint8 weights dequantised inside the dense kernels: end to end and with the input
+        resident, and the roofline of its dominant kernel from the times inside the running step."""
+    out = {}
+    x1 = np.random.default_rng(2).uniform(0, 1, (1, 224, 224, 3)).astype(np.float32)
+    js = js_host_leg(params, x1, 1, 2000, 100, priming=600, legs=["e2e2", "graph", "latency"])
+    if js is not None and "error" not in js:
+        out["batch1_fp32"] = dict(
+            host="JavaScript (node %s)" % js["node"], steps=js["steps"], warmup=js["warmup"],
+            priming_steps=js["priming_steps"],
+            eager_ms_per_image=round(js["resident"]["ms_per_step"], 4),
+            eager_images_per_s=round(js["resident"]["images_per_s"], 1),
+            host_dispatch_ms_per_image=round(js["resident"]["host_dispatch_ms_per_step"], 4),
+            captured_graph_ms_per_image=round(js["graph_replay"]["ms_per_step"], 4),
+            captured_graph_images_per_s=round(js["graph_replay"]["images_per_s"], 1),
+            end_to_end_ms_per_image=round(js["end_to_end"]["ms_per_step"], 4),
+            latency_ms_one_image=round(js["latency_one_batch"]["ms_median"], 4))
+    else:
+        w = mobilenet.upload(tf, params)
+        x = tf.tensor(x1)
+
+        def step():
+            tf.dispose(list(mobilenet.forward(tf, w, x)))
+        for _ in range(700):
+            step()
+        tf.backend().sync()
+        t0 = time.perf_counter()
+        for _ in range(2000):
+            step()
+        tf.backend().sync()
+        ms = (time.perf_counter() - t0) / 2.0
+        out["batch1_fp32"] = dict(host="python ctypes driver", steps=2000, warmup=700,
+                                  eager_ms_per_image=round(ms, 4), eager_images_per_s=round(1e3 / ms, 1),
+                                  note=(js or {}).get("error", "node is not installed"))
+        tf.dispose([x] + [t for t in w.values() if hasattr(t, "dispose")])
+
+    batch = 256
+    qparams = mobilenet.quantize_params(params)
+    xq = np.random.default_rng(3).random((batch, 224, 224, 3), dtype=np.float32)
+    js = js_host_leg(qparams, xq, batch, 20, 5, priming=60, legs=["e2e2", "kernels"])
+    if js is not None and "error" not in js:
+        leg = dict(host="JavaScript (node %s)" % js["node"], steps=js["steps"], warmup=js["warmup"],
+                   priming_steps=js["priming_steps"],
+                   end_to_end_images_per_s=round(js["end_to_end"]["images_per_s"], 1),
+                   end_to_end_ms_per_step=round(js["end_to_end"]["ms_per_step"], 4),
+                   batches_in_flight=2,
+                   resident_images_per_s=round(js["resident"]["images_per_s"], 1),
+                   resident_ms_per_step=round(js["resident"]["ms_per_step"], 4))
+        kt = [tuple(k) for k in js["kernel_times"]] if js.get("kernel_times") else None
+        rows = rows_of_one_step(kt, mobilenet.layer_table(batch=batch), batch) if kt else None
+        if rows:
+            roof, _ = roofline_of_dominant_kernel(rows)
+            roof.pop("layers", None)
+            leg["roofline"] = roof
+            leg["kernels_per_step"] = len(kt)
+            leg["uint8_kernels"] = sum(1 for k in kt if "_u8" in k[0])
+        out["batch256_uint8"] = leg
+    else:
+        out["batch256_uint8"] = dict(error=(js or {}).get("error", "node is not installed"))
+    return out
 
 
 def main():
@@ -321,6 +393,13 @@ def main():
     ap.add_argument("--quant", action="store_true", help="uint8 weights dequantised in-kernel")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-js", action="store_true", help="skip the Node.js host leg")
+    ap.add_argument("--priming", type=int, default=None, metavar="N",
+                    help="untimed steps before the --warmup steps of every leg (default 300 less "
+                         "--warmup: the device needs a few hundred ms of work to reach its clocks "
+                         "and V8 compiles the host after a few hundred calls); 0 = none.  The line "
+                         "also carries value_without_priming, measured first, whatever N is")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the short legs for batch 1 and batch 256 with uint8 weights")
     ap.add_argument("--no-ops", action="store_true",
                     help="skip the op-level configs (single matMul, MLP layers, conv2d, depthwise)")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
@@ -418,37 +497,7 @@ def main():
     for sl in slots:
         sl[...] = x_host
 
-    # ---- Python driver: input resident in HBM --------------------------------------------------
-    x = tf.tensor(x_host)
-
-    def step():
-        logits, probs = mobilenet.forward(tf, w, x)
-        tf.dispose([logits, probs])
-
-    # Priming, before any warm-up or timed step: the device needs a few hundred ms of work to
-    # reach its clocks (a run with a handful of warm-up steps would time a cold device; the Node
-    # leg does the same and also needs it for V8 to compile the host's functions).  The same
-    # untimed steps in every run, whatever --warmup says; reported as config.priming_steps.
-    priming_steps = max(0, 300 - args.warmup)
-    for _ in range(priming_steps):
-        step()
-    be.sync()
-    for _ in range(args.warmup):
-        step()
-    be.sync()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    be.sync()
-    wall = time.perf_counter() - t0
-    resident = dict(images_per_s=round(args.batch * args.steps / wall, 1),
-                    ms_per_step=round(wall * 1e3 / args.steps, 4))
-    # ---- Python driver: end to end ---------------------------------------------------------------
-    # Every step uploads its batch (page-locked host arrays, upload stream), runs the forward
-    # pass and reads the probabilities back (asynchronous read, awaited two steps late); batch
-    # i+1 uploads while batch i computes.
-    # streams = 2: batch i runs on compute stream i % 2 of the backend, so that two batches are in
-    # flight and each fills the phases in which the other leaves the machine idle.
+    # ---- Python driver: the flags taken at their word (no priming), before anything else ---------
     def pipelined(n, streams):
         pending, last = [], None
         nxt = tf.tensor(slots[0])
@@ -469,6 +518,45 @@ def main():
             be.select_stream(0)
         return last
 
+    if args.warmup > 0:
+        pipelined(args.warmup, 2)
+    t0 = time.perf_counter()
+    pipelined(args.steps, 2)
+    wall = time.perf_counter() - t0
+    py_cold = dict(images_per_s=round(args.batch * args.steps / wall, 1),
+                   ms_per_step=round(wall * 1e3 / args.steps, 4), batches_in_flight=2)
+
+    # ---- Python driver: input resident in HBM --------------------------------------------------
+    x = tf.tensor(x_host)
+
+    def step():
+        logits, probs = mobilenet.forward(tf, w, x)
+        tf.dispose([logits, probs])
+
+    # Priming, before any warm-up or timed step: the device needs a few hundred ms of work to
+    # reach its clocks (a run with a handful of warm-up steps would time a cold device; the Node
+    # leg does the same and also needs it for V8 to compile the host's functions).  The same
+    # untimed steps in every run, whatever --warmup says; reported as config.priming_steps.
+    priming_steps = max(0, 300 - args.warmup) if args.priming is None else max(0, args.priming)
+    for _ in range(priming_steps):
+        step()
+    be.sync()
+    for _ in range(args.warmup):
+        step()
+    be.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    be.sync()
+    wall = time.perf_counter() - t0
+    resident = dict(images_per_s=round(args.batch * args.steps / wall, 1),
+                    ms_per_step=round(wall * 1e3 / args.steps, 4))
+    # ---- Python driver: end to end ---------------------------------------------------------------
+    # Every step uploads its batch (page-locked host arrays, upload stream), runs the forward
+    # pass and reads the probabilities back (asynchronous read, awaited two steps late); batch
+    # i+1 uploads while batch i computes.
+    # streams = 2: batch i runs on compute stream i % 2 of the backend, so that two batches are in
+    # flight and each fills the phases in which the other leaves the machine idle.
     with tf.tidy():
         want_probs = mobilenet.forward(tf, w, x)[1].data_sync()
     py_legs = {}
@@ -483,6 +571,23 @@ def main():
     py_end_to_end = dict(py_legs[2], batches_in_flight=2)
     py_end_to_end_one = py_legs[1]
 
+    # one batch at a time, nothing else in flight: upload from page-locked memory, forward pass,
+    # awaited read of the probabilities
+    def one_batch():
+        t = time.perf_counter()
+        xi = tf.tensor(slots[0])
+        logits, probs = mobilenet.forward(tf, w, xi)
+        probs.data().result()
+        ms = (time.perf_counter() - t) * 1e3
+        tf.dispose([xi, logits, probs])
+        return ms
+    for _ in range(3):
+        one_batch()
+    each = sorted(one_batch() for _ in range(max(5, min(50, args.steps))))
+    py_latency = dict(ms_mean=round(sum(each) / len(each), 4), ms_median=round(each[len(each) // 2], 4),
+                      ms_min=round(each[0], 4), batches=len(each), input="page-locked host array",
+                      batches_in_flight=1)
+
     # the same loop with an event after every launch: the times the kernels take in the step
     info = tf.time(lambda: [step() for _ in range(args.steps)])
     resident["gpu_ms_per_step_events"] = round(info["kernelMs"] / args.steps, 4)
@@ -496,10 +601,13 @@ def main():
     # ---- JavaScript host (the product's host) ----------------------------------------------------
     host = "python ctypes driver over the C ABI"
     end_to_end, resident_input, kernel_times = py_end_to_end, resident, py_kernel_times
-    js = None if args.no_js else js_host_leg(dev_params, x_host, args.batch, args.steps, args.warmup)
+    cold, latency = py_cold, py_latency
+    js = None if args.no_js else js_host_leg(dev_params, x_host, args.batch, args.steps, args.warmup,
+                                             priming=args.priming)
     if js is not None and "error" not in js:
         host = "JavaScript tf.* graph in Node.js %s over the N-API addon" % js["node"]
         end_to_end, resident_input = js["end_to_end"], js["resident"]
+        cold, latency = js["end_to_end_without_priming"], js["latency_one_batch"]
         if js.get("kernel_times"):
             kernel_times = [tuple(k) for k in js["kernel_times"]]
 
@@ -530,6 +638,14 @@ def main():
         "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(end_to_end["ms_per_step"], 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        # the same loop run first thing, with --warmup untimed steps and no priming before it (a
+        # device that has just been woken, the host's functions not yet compiled)
+        "value_without_priming": round(cold["images_per_s"], 1),
+        "ms_per_step_without_priming": round(cold["ms_per_step"], 4),
+        # `value` is a throughput with two batches in flight; this is the time of ONE batch with
+        # nothing else in flight: page-locked upload -> forward pass -> awaited read
+        "latency_ms_one_batch": round(latency["ms_median"], 4),
+        "latency_one_batch": latency,
         "config": {"workload": "MobileNetV1-1.0-224 random-init fp32 NHWC forward + softmax, "
                                "batch %d%s, tf.* graph on the hip backend; every step uploads its "
                                "input batch from host memory and reads the class probabilities "
@@ -546,7 +662,8 @@ def main():
         "end_to_end_one_stream": (js or {}).get("end_to_end_one_stream", py_end_to_end_one)
                                  if js is not None and "error" not in js else py_end_to_end_one,
         "python_driver": {"end_to_end": py_end_to_end, "end_to_end_one_stream": py_end_to_end_one,
-                          "resident_input": resident},
+                          "resident_input": resident, "end_to_end_without_priming": py_cold,
+                          "latency_one_batch": py_latency},
         "js_host": js,
         "dense_tflops": round(sum(2e-9 * r["macs"] for r in dense) / sum(r["ms"] for r in dense), 2)
                         if dense else None,
@@ -560,6 +677,9 @@ def main():
                         gbs=round(1e-6 * r["bytes"] / r["ms"], 1), algorithmic_bytes=r["bytes"],
                         launches=r["launches"]) for r in (rows or [])],
     }
+    if not args.no_configs and args.batch == 64 and not args.quant:
+        tf.dispose([x])
+        out["configs"] = other_configs(tf, mobilenet, params, np)
     if not args.no_ops:
         out["op_configs"] = op_level_configs(tf, np)
         if args.layers:
