@@ -154,16 +154,18 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p) {
 
 // 3x3, stride 1, dilation 1, channel multiplier 1, C % 4 == 0, for large images: one lane =
 // one channel quad of a strip TW outputs wide, walked down `rows` output rows.  Every input
-// row of the strip is fetched once (TW + 2 vectors, the next row already in flight) and
+// row of the strip is fetched once (TW + 2 vectors, the next PF rows already in flight) and
 // feeds the three output rows it belongs to, which live in three rotating accumulator rows;
 // nothing is read twice vertically, and the two halo columns are shared with the
 // neighbouring lane's loads of the same moment.  Each output sums its taps in the order
 // filter row, then filter column, as the patch kernel above and the reference do.
-template <int TW>
+template <int TW, int PF>
 __global__ __launch_bounds__(256) void depthwise3x3_rows_kernel(const DwArgs p, int rows,
                                                                 int chunks, unsigned x_bytes,
                                                                 unsigned y_bytes) {
   constexpr int IW = TW + 2;
+  constexpr int NB = PF + 1;                       // row buffers: PF rows in flight + the one in use
+  constexpr int PERIOD = NB % 3 == 0 ? NB : 3 * NB;  // buffers and accumulator rows take turns
   constexpr unsigned OOB = 0x80000000u;  // beyond any extent below 2 GiB: loads give 0, stores vanish
   const tfhip_conv2d_info& ci = p.ci;
   const int64_t total = (int64_t)ci.batch * chunks * p.tiles_w * p.c4;
@@ -257,31 +259,30 @@ __global__ __launch_bounds__(256) void depthwise3x3_rows_kernel(const DwArgs p, 
       for (int kw = 0; kw < 3; kw++) oldest[j] += in[j + kw] * w[6 + kw];
     }
   };
-  // One step: start the loads of the next input row, feed the current one, store the output
-  // row it completes (input row ih completes output row ih + pad_top - 2).
-  auto step = [&](int ih, const f32x4 (&in)[IW], f32x4 (&next)[IW], f32x4 (&oldest)[TW],
-                  f32x4 (&middle)[TW], f32x4 (&newest)[TW]) {
-    load_row(ih + 1, next);
-    __builtin_amdgcn_sched_barrier(0);  // loads first, and none from a later step
-    feed(in, oldest, middle, newest);
-    store_row(ih + ci.pad_top - 2, oldest);
-    __builtin_amdgcn_sched_barrier(0);
-  };
 
-  f32x4 r0[TW], r1[TW], r2[TW];
+  f32x4 acc[3][TW];
 #pragma unroll
-  for (int j = 0; j < TW; j++) r0[j] = r1[j] = r2[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  f32x4 cur[IW], nxt[IW];
-  load_row(ih_first, cur);
-  // Two row buffers and three accumulator rows take turns: the pattern repeats every 6 rows.
-  // Steps past ih_last load nothing and store nothing.
-  for (int ih = ih_first; ih <= ih_last; ih += 6) {
-    step(ih, cur, nxt, r0, r1, r2);
-    step(ih + 1, nxt, cur, r1, r2, r0);
-    step(ih + 2, cur, nxt, r2, r0, r1);
-    step(ih + 3, nxt, cur, r0, r1, r2);
-    step(ih + 4, cur, nxt, r1, r2, r0);
-    step(ih + 5, nxt, cur, r2, r0, r1);
+  for (int i = 0; i < 3; i++)
+#pragma unroll
+    for (int j = 0; j < TW; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  f32x4 buf[NB][IW];
+#pragma unroll
+  for (int q = 0; q < PF; q++) load_row(ih_first + q, buf[q]);
+  // One step: start the loads of the row PF steps ahead, feed the current row, store the output
+  // row it completes (input row ih completes output row ih + pad_top - 2).  NB row buffers and
+  // three accumulator rows take turns: the pattern repeats every PERIOD rows, and with the loop
+  // unrolled every buffer of a step is known at compile time.  Rows past ih_last load nothing
+  // and store nothing.
+  for (int ih = ih_first; ih <= ih_last; ih += PERIOD) {
+#pragma unroll
+    for (int s = 0; s < PERIOD; s++) {
+
+      load_row(ih + s + PF, buf[(s + PF) % NB]);
+      __builtin_amdgcn_sched_barrier(0);  // loads first, and none from a later step
+      feed(buf[s % NB], acc[s % 3], acc[(s + 1) % 3], acc[(s + 2) % 3]);
+      store_row(ih + s + ci.pad_top - 2, acc[s % 3]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 }
 
@@ -444,14 +445,14 @@ static void launch_dw3x3(tfhip_ctx* ctx, DwArgs& p) {
                      dim3(256), 0, p);
 }
 
-template <int TW>
+template <int TW, int PF>
 static void launch_dw3x3_rows(tfhip_ctx* ctx, DwArgs& p, int rows) {
-  ctx->name_kernel("depthwise3x3_s1_rows_w%d", TW);
+  ctx->name_kernel("depthwise3x3_s1_rows_w%d_ahead%d", TW, PF);
   const int chunks = (int)ceil_div(p.ci.out_h, rows);
   p.tiles_w = (int)ceil_div(p.ci.out_w, TW);
   const int64_t total = (int64_t)p.ci.batch * chunks * p.tiles_w * p.c4;
   p.reverse = ctx->take_sweep();
-  tfhip::launch(ctx, (depthwise3x3_rows_kernel<TW>), dim3((unsigned)ceil_div(total, 256)),
+  tfhip::launch(ctx, (depthwise3x3_rows_kernel<TW, PF>), dim3((unsigned)ceil_div(total, 256)),
                      dim3(256), 0, p, rows, chunks,
                      (unsigned)((int64_t)p.ci.batch * p.ci.in_h * p.ci.in_w * p.ci.in_c * 4),
                      (unsigned)((int64_t)p.ci.batch * p.ci.out_h * p.ci.out_w * p.ci.out_c * 4));
@@ -491,7 +492,11 @@ static int dispatch_depthwise(tfhip_ctx* ctx, DwArgs& p, const tfhip_conv2d_info
       if (waves(rows) < slots / 4) rows = 0;
     }
     if (rows > 0) {
-      launch_dw3x3_rows<2>(ctx, p, rows);
+      // Two input rows in flight per wavefront (measured in a batch-64 MobileNet step against one
+      // row: [64,14,14,512] 10.6 -> 9.4 us, [64,7,7,1024] 7.5 -> 6.8, [64,28,28,256] 25.1 -> 24.6;
+      // three rows in flight, 217 registers: 11.1 / 8.2 / 26.8; strips one output column wide with
+      // one / two / three rows in flight: 10.0 / 10.3 / 11.5 us on the first shape)
+      launch_dw3x3_rows<2, 2>(ctx, p, rows);
     } else if (ci->stride_h == 1) {
       if (ci->out_w >= 112 && ci->in_c >= 128 && ci->out_w % 8 == 0) launch_dw3x3<1, 2, 8>(ctx, p);
       else launch_dw3x3<1, 2, 2>(ctx, p);
