@@ -304,7 +304,10 @@ int tfhip_unary(tfhip_ctx* ctx, int op, int64_t x, int64_t out, float p0, float 
 int tfhip_cast(tfhip_ctx* ctx, int64_t x, int64_t out);
 /* decodeWeights, quantised branch (io/io_utils.ts:122-147): x TFHIP_UINT8Q -> out float32,
  * w = q*scale + min in double, rounded once.  The dense kernels do this while staging
- * their B tile; this entry materialises the float weights for any other consumer. */
+ * their B tile; this entry materialises the float weights for any other consumer.
+ * When x holds two bytes per element of out, they are the 16-bit codes of a 'uint16'
+ * quantisation, low byte first as in the weights file: the bytes of such a shard go to the
+ * device as they are and are expanded here, once, at load time. */
 int tfhip_dequantize(tfhip_ctx* ctx, int64_t x, int64_t out, const tfhip_qparams* q);
 /* fill/zerosLike/onesLike (backend.ts:629-640; backend_cpu.ts:3816-3836). */
 int tfhip_fill(tfhip_ctx* ctx, int64_t out, double value);

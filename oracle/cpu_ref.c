@@ -699,6 +699,10 @@ int ref_transpose(const int32_t* x, const int32_t* shape, int rank, const int32_
 void ref_dequantize_u8(const uint8_t* q, float* out, int64_t n, double scale, double min) {
   for (int64_t i = 0; i < n; i++) out[i] = (float)((double)q[i] * scale + min);
 }
+/* the same branch for quantization.dtype 'uint16' (io/io_utils.ts:131-136) */
+void ref_dequantize_u16(const uint16_t* q, float* out, int64_t n, double scale, double min) {
+  for (int64_t i = 0; i < n; i++) out[i] = (float)((double)q[i] * scale + min);
+}
 
 /* backends/cpu/backend_cpu.ts:1299-1308: Int32Array store of a float = ToInt32 (truncate
  * toward zero, NaN/inf -> 0, wrap modulo 2^32). */

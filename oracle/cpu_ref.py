@@ -577,6 +577,14 @@ def dequantize_u8(q, scale, min_):
     return out
 
 
+def dequantize_u16(q, scale, min_):
+    q = np.ascontiguousarray(q, np.uint16)
+    out = np.empty(q.shape, np.float32)
+    lib().ref_dequantize_u16(_p(q, C.c_uint16), _p(out), C.c_int64(q.size), C.c_double(scale),
+                             C.c_double(min_))
+    return out
+
+
 def to_int(x):
     x = _f32(x)
     out = np.empty(x.shape, np.int32)

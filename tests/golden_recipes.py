@@ -469,6 +469,18 @@ def dequant_uint8_known_answer(ops):
     expect_close(ops.dequantize(q, 0.1, -1.0), a[2], eps=1e-6)
 
 
+@recipe
+def dequant_uint16_known_answer(ops):
+    """io/io_utils_test.ts:496-522: the same codes as 16-bit values."""
+    a = golden_case("dequant", "support quantization uint16 weights")["arrays"]
+    q = np.array(a[1][:3], np.uint16)
+    expect_close(ops.dequantize(q, 0.1, -1.0), a[2], eps=1e-6)
+    # codes beyond one byte, against the double-precision formula rounded once
+    q = np.array([256, 4660, 65535, 32768], np.uint16)
+    want = (q.astype(np.float64) * 0.00731 + -113.25).astype(np.float32)
+    assert np.array_equal(ops.dequantize(q, 0.00731, -113.25), want)
+
+
 # ---- ops/slice_test.ts, strided_slice_test.ts, reverse_test.ts ---------------------------
 @recipe
 def slice_known_answers(ops):

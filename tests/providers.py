@@ -196,7 +196,10 @@ class OracleOps:
     def softmax(self, x): return self.r.softmax(x)
     def gather(self, x, idx, axis): return self.r.gather(x, idx, axis)
     def transpose(self, x, perm): return self.r.transpose(x, perm)
-    def dequantize(self, q, scale, min_): return self.r.dequantize_u8(q, scale, min_)
+    def dequantize(self, q, scale, min_):
+        if np.asarray(q).dtype == np.uint16:
+            return self.r.dequantize_u16(q, scale, min_)
+        return self.r.dequantize_u8(q, scale, min_)
     def to_int(self, x): return self.r.to_int(x)
     def slice(self, x, begin, size): return self.r.slice_(x, begin, size)
 
@@ -411,7 +414,8 @@ class HipOps:
     def dequantize(self, q, scale, min_):
         tf = self.tf
         with tf.tidy():
-            return tf.dequantize(tf.quantized_tensor(q, scale, min_)).data_sync()
+            bits = 16 if np.asarray(q).dtype == np.uint16 else 8
+            return tf.dequantize(tf.quantized_tensor(q, scale, min_), bits).data_sync()
 
     def to_int(self, x): return self._run(lambda t: self.tf.cast(t, "int32"), x)
     def slice(self, x, begin, size): return self._run(lambda t: self.tf.slice(t, begin, size), x)

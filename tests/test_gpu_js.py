@@ -136,6 +136,12 @@ def test_js_ops_match_oracle(tmp_path, ref):
     wd2 = f(3, 3, 8, 2)
     c.add("dw_chmul2", "depthwiseConv2d", dict(x=x, filter=wd2), dict(strides=1, pad="valid"),
           ref.depthwise_conv2d(x, wd2, 1, "valid"))
+    # a uint16-quantised manifest entry goes to the device as bytes and is expanded there
+    q16 = rng.integers(0, 65536, (5, 7, 6)).astype(np.uint16)
+    spec16 = dict(name="w16", shape=list(q16.shape), dtype="float32",
+                  quantization=dict(dtype="uint16", scale=2.7e-5, min=-0.9))
+    c.add("decode_uint16", "decodeWeightsToDevice", dict(bytes=(q16.view(np.uint8).reshape(-1), 0.0, 0.0)),
+          dict(spec=spec16), ref.dequantize(q16, 2.7e-5, -0.9), exact=True)
     q = rng.integers(0, 256, (3, 3, 8, 16)).astype(np.uint8)
     c.add("conv_uint8", "conv2d", dict(x=x, filter=(q, 0.011, -1.4)), dict(strides=1, pad="same"),
           ref.conv2d(x, ref.dequantize(q, 0.011, -1.4), 1, "same"))

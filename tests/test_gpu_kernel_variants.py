@@ -218,6 +218,9 @@ def test_rowstream_matmul_and_small_fallback(tf):
     (256, 4096, 256, "gemm_64x64_rowmajor_f32_kb48_splitk"),
     (4096, 1024, 10, "gemm_16x16_kwaves_f32"),
     (32768, 1024, 10, "gemm_256x32_rowmajor_f32_kb48"),
+    # a right-hand side larger than the left: the tiles are dealt to the XCDs in four column groups
+    (2048, 1024, 4096, "gemm_"),
+    (1100, 520, 2048, "gemm_"),                                         # two groups, ragged rows, K % 16 != 0
 ])
 def test_matmul_tiles_against_float64(tf, m, k, n, want_prefix):
     print("matmul", m, k, n, flush=True)

@@ -656,6 +656,11 @@ def test_uint8_weights_dequantised_in_kernel(hip, ref):
     scale, mn = 0.0137, -1.73
     q = rng.integers(0, 256, (40, 24)).astype(np.uint8)
     assert np.array_equal(hip.dequantize(q, scale, mn), ref.dequantize(q, scale, mn))
+    # 16-bit codes are expanded on the device at load time (io/io_utils.ts:131-136)
+    q16 = rng.integers(0, 65536, (33, 7, 5)).astype(np.uint16)
+    got16 = hip.dequantize(q16, 3.1e-5, -1.02)
+    assert got16.shape == q16.shape
+    assert np.array_equal(got16, ref.dequantize(q16, 3.1e-5, -1.02))
     a = rng.standard_normal((1, 19, 40)).astype(np.float32)
     w = ref.dequantize(q, scale, mn)
     with tf.tidy():

@@ -265,6 +265,21 @@ __global__ void dequantize_kernel(const uint8_t* q, float* out, int64_t n, doubl
   }
 }
 
+// The same for 16-bit codes: two bytes per weight, low byte first (the byte order of a weights
+// file read into a Uint16Array, io/io_utils.ts:131-133).  Read as bytes: a shard places a tensor
+// at any byte offset.
+__global__ void dequantize16_kernel(const uint8_t* q, float* out, int64_t n, double scale,
+                                    double mn) {
+#pragma clang fp contract(off)
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const unsigned code = (unsigned)q[2 * i] | ((unsigned)q[2 * i + 1] << 8);
+    double v = (double)code * scale;
+    v = v + mn;
+    out[i] = (float)v;
+  }
+}
+
 template <typename T>
 __global__ void fill_kernel(T* out, int64_t n, T value) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -417,11 +432,14 @@ extern "C" int tfhip_dequantize(tfhip_ctx* ctx, int64_t x, int64_t out, const tf
   if (!ctx || !q) return TFHIP_EINVAL;
   TFHIP_GET(ctx, bx, x);
   TFHIP_GET(ctx, bo, out);
-  if (bx->dtype != TFHIP_UINT8Q || bo->dtype != TFHIP_FLOAT32 || bx->numel != bo->numel)
-    return ctx->fail(TFHIP_EINVAL, "dequantize: needs a quantised input and a float32 output of equal size");
-  if (bx->numel == 0) return TFHIP_OK;
-  tfhip::launch(ctx, dequantize_kernel, dim3(grid_for(ctx, bx->numel, 256)), dim3(256), 0, (const uint8_t*)bx->ptr, (float*)bo->ptr, bx->numel, q->scale,
-                     q->min);
+  const bool wide = bo->numel > 0 && bx->numel == 2 * bo->numel;  // 16-bit codes
+  if (bx->dtype != TFHIP_UINT8Q || bo->dtype != TFHIP_FLOAT32 || (bx->numel != bo->numel && !wide))
+    return ctx->fail(TFHIP_EINVAL, "dequantize: needs a quantised input of one or two bytes per "
+                                   "element and a float32 output");
+  if (bo->numel == 0) return TFHIP_OK;
+  tfhip::launch(ctx, wide ? dequantize16_kernel : dequantize_kernel,
+                dim3(grid_for(ctx, bo->numel, 256)), dim3(256), 0, (const uint8_t*)bx->ptr,
+                (float*)bo->ptr, bo->numel, q->scale, q->min);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }

@@ -51,6 +51,11 @@ struct GemmArgs {
   // schedule (see work_item)
   int tiles_m, tiles_n, k_tiles, full_tiles, tail_tiles, splits, kt_per;
   int tiles_n_shift;  // log2(tiles_n) when that is a power of two, else -1 (a division on the vector ALU)
+  // col_groups > 1 (unbatched products without a split along K): the tiles are numbered column
+  // group by column group, a group being 1 << cg_shift tile columns of every tile row, so that an
+  // XCD's run of tiles lies inside one group: its L2 then reads 1 / col_groups of B and
+  // col_groups / 8 of A instead of all of B and an eighth of A (see choose_col_groups).
+  int col_groups, cg_shift;
   float* partials;  // [tail_tiles * splits][BM * BN] partial tiles when splits > 1
   // minis > 0: the tail tiles are not split along K over workgroups but cut into `minis` tiles
   // of 16 x 16 each, one per workgroup, whose wavefronts take mini_k_per of K each (kwaves_tile)
@@ -90,6 +95,24 @@ __device__ __forceinline__ WorkItem work_item(const GemmArgs& p, int block) {
     if (p.splits > 1) w.slot = h;
   }
   return w;
+}
+
+// Tile row and tile column of tile t of an unbatched product (t counts row by row, or column
+// group by column group).  t is the same for the whole workgroup.
+__device__ __forceinline__ void tile_row_col(const GemmArgs& p, int t, int& tm, int& tn) {
+  if (p.col_groups > 1) {
+    const int per = p.tiles_m << p.cg_shift;  // tiles of a column group
+    int g = 0;
+    while (t >= per) {  // (at most col_groups - 1 times)
+      t -= per;
+      g++;
+    }
+    tm = t >> p.cg_shift;
+    tn = (g << p.cg_shift) + (t - (tm << p.cg_shift));
+  } else {
+    tm = p.tiles_n_shift >= 0 ? t >> p.tiles_n_shift : t / p.tiles_n;
+    tn = t - tm * p.tiles_n;
+  }
 }
 
 // Small products with a long contraction (a [256, 512] x [512, 256] matMul, the 14 x 14 and
@@ -275,9 +298,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     // unbatched product, a shift for a power-of-two number of tile columns)
     const int batch = tile < tiles_per_batch ? 0 : tile / tiles_per_batch;
     const int t = tile - batch * tiles_per_batch;
-    const int tm = p.tiles_n_shift >= 0 ? t >> p.tiles_n_shift : t / p.tiles_n;
+    int tm, tn;
+    tile_row_col(p, t, tm, tn);
     L.bm0 = tm * BM;
-    L.bn0 = (t - tm * p.tiles_n) * BN;
+    L.bn0 = tn * BN;
     L.batch = batch;
     L.A = p.A + batch * p.strideA;
     L.Bf = static_cast<const float*>(p.B) + batch * p.strideB;
@@ -636,8 +660,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       const int j = h >> 3;
       const int tt = (h & 7) + 8 * (j / p.minis), mini = j % p.minis;
       const int t = p.full_tiles + tt;
-      const int m0 = (t / p.tiles_n) * BM + (mini / (BN / 16)) * 16;
-      const int n0 = (t % p.tiles_n) * BN + (mini % (BN / 16)) * 16;
+      int tm, tn;
+      tile_row_col(p, t, tm, tn);
+      const int m0 = tm * BM + (mini / (BN / 16)) * 16;
+      const int n0 = tn * BN + (mini % (BN / 16)) * 16;
       if (tt >= p.tail_tiles || m0 >= p.M || n0 >= p.N) return;
       kwaves_tile<WAVES_M * WAVES_N, 2, BMODE == B_UINT8>(p, m0, n0, p.mini_k_per, lds, tid);
       return;
@@ -1530,6 +1556,36 @@ static Plan make_plan(const GemmArgs& p, int batch, int bm, int bn, int resident
   return pl;
 }
 
+// How many column groups the tiles of an unbatched row-major product are dealt in.  Workgroup b
+// runs on XCD b % 8 and every XCD has an L2 of its own (4 MiB), so with the tiles numbered row by
+// row an L2 reads an eighth of A and all of B: A + 8 B over the chip.  Numbered in c column groups
+// it reads c / 8 of A and 1 / c of B: c A + (8 / c) B.  A share of B that does not fit half an L2
+// next to the stream of A is fetched more than once (measured: [3136, 1024] x [1024, 1024], B =
+// 4 MiB, fetched 46 to 67 MiB over the chip against the 44 the formula gives), hence the
+// surcharge.  c must divide the tile columns into groups of a power of two, and has to save 15 %
+// to be taken.  Measured (FETCH_SIZE over the chip, every choice forced in turn): the product
+// above 67.6 MiB with c = 1, 48.3 with c = 2 (the formula gives 40.6, and the 16 leftover tiles
+// that run as 16 x 16 pieces add 8), 64.9 with c = 4, durations 51.6 / 52.0 / 52.4 us;
+// [3136, 512] x [512, 1024] 23.2 / 23.4 / 31.7 MiB; [12544, 512] x [512, 512] 36.2 / 57.0 / 105.5.
+static int choose_col_groups(const GemmArgs& p, const Plan& pl, double b_elem_bytes) {
+  if (pl.splits > 1 || pl.tiles_m < 16) return 1;
+  const double a_bytes = 4.0 * p.M * p.K, b_bytes = b_elem_bytes * p.K * p.N;
+  int best = 1;
+  double best_cost = 0;
+  for (int c = 1; c <= 4; c *= 2) {
+    if (pl.tiles_n % c) break;
+    const int w = pl.tiles_n / c;
+    if (w & (w - 1)) break;
+    const double share = b_bytes / c;
+    const double cost = c * a_bytes + (8.0 / c) * b_bytes * (share > 2.0 * (1 << 20) ? 1.5 : 1.0);
+    if (c == 1 || cost < 0.85 * best_cost) {
+      best = c;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
 // Scratch memory of tfhip_matmul_noalloc: a static device array, one copy per GPU, that takes
 // the place of the pool block in which a product cut along K keeps its partial tiles.  Host
 // code reaches it only through the address hipGetSymbolAddress returns for the current
@@ -1591,6 +1647,13 @@ static int launch_cfg(tfhip_ctx* ctx, GemmArgs& p, const Plan& pl) {
   p.tiles_m = pl.tiles_m;
   p.tiles_n = pl.tiles_n;
   p.tiles_n_shift = (pl.tiles_n & (pl.tiles_n - 1)) == 0 ? __builtin_ctz((unsigned)pl.tiles_n) : -1;
+  p.col_groups = 1;
+  p.cg_shift = 0;
+  if (FAST && AMODE == A_ROWMAJOR && BMODE != B_TRANSPOSED && pl.tiles_m * pl.tiles_n == pl.full_tiles + pl.tail_tiles) {
+    // (an unbatched product: the planner counted tiles_m * tiles_n tiles)
+    p.col_groups = choose_col_groups(p, pl, BMODE == B_UINT8 ? 1.0 : 4.0);
+    if (p.col_groups > 1) p.cg_shift = __builtin_ctz((unsigned)(pl.tiles_n / p.col_groups));
+  }
   p.full_tiles = pl.full_tiles;
   p.tail_tiles = pl.tail_tiles;
   p.splits = pl.splits;

@@ -773,7 +773,8 @@ class MathBackendHIP extends KernelBackend {
     return out;
   }
   dequantize(x) {
-    const out = this.out(x.shape, 'float32');
+    const wide = x.quantization != null && x.quantization.bits === 16;  // two bytes per weight
+    const out = this.out(wide ? x.shape.slice(0, -1) : x.shape, 'float32');
     this.napi.dequantize(this.ctx, this.h(x), this.h(out), this.q(x));
     return out;
   }

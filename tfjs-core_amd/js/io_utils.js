@@ -3,7 +3,11 @@
 // (decodeWeights) and io/types.ts:100-107 (quantization: {min, scale, dtype}).
 // decodeWeights() follows the reference: quantised entries are expanded to float32 on the
 // host.  decodeWeightsToDevice() keeps uint8 entries as bytes in HBM and hands back tensors
-// that the dense kernels dequantise on load, so float weights are never materialised.
+// that the dense kernels dequantise on load, so float weights are never materialised.  uint16
+// entries go to the device as bytes too and are expanded there, once, into float32 tensors (the
+// 65 536 values a code can stand for do not fit the table the dense kernels keep in LDS; weights
+// are a per cent of what a batch moves, so their bytes in HBM matter little): the host never
+// holds the float weights either way.
 const DTYPE_VALUE_SIZE_MAP = {float32: 4, int32: 4, uint16: 2, uint8: 1, bool: 1};
 
 function sizeFromShape(shape) {
@@ -69,6 +73,12 @@ function decodeWeightsToDevice(buffer, specs) {
       const piece = sliceOf(buffer, spec, offset);
       offset = piece.next;
       out[spec.name] = ops.quantizedTensor(piece.quantized, spec.shape, q.scale, q.min);
+    } else if (q != null && q.dtype === 'uint16' && spec.dtype === 'float32') {
+      const piece = sliceOf(buffer, spec, offset);
+      offset = piece.next;
+      const codes = ops.quantizedTensor(new Uint8Array(piece.bytes), spec.shape, q.scale, q.min, 16);
+      out[spec.name] = ops.dequantize(codes);
+      codes.dispose();
     } else {
       const one = decodeWeights(buffer.slice(offset), [spec]);
       offset = sliceOf(buffer, spec, offset).next;

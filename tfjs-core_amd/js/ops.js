@@ -55,11 +55,14 @@ const tensor4d = (values, shape, dtype) => tensor(values, shape, dtype);
 
 // A float32 weight tensor kept as uint8 affine-quantised bytes in HBM (io/types.ts:100-107);
 // its consumers dequantise w = q*scale + min while they load it.
-function quantizedTensor(bytes, shape, scale, min) {
+// bits = 16: `bytes` holds the two bytes of every 16-bit code (low byte first, as in the weights
+// file) and the tensor gets a last axis of 2; only dequantize() takes such a tensor.
+function quantizedTensor(bytes, shape, scale, min, bits) {
   util.assert(bytes instanceof Uint8Array, 'quantizedTensor expects a Uint8Array');
+  if (bits === 16) shape = shape.concat([2]);
   util.assert(util.sizeFromShape(shape) === bytes.length, 'quantizedTensor: shape does not match the data');
   const t = new Tensor(shape, 'float32', bytes, null, null, 'uint8q');
-  t.quantization = {scale, min};
+  t.quantization = {scale, min, bits: bits === 16 ? 16 : 8};
   return t;
 }
 

@@ -304,6 +304,18 @@ async function main() {
         entry.dtype = out.logits.dtype;
         entry.probSum = tf.tidy(() => Array.from(tf.sum(out.probs, -1).dataSync()));
         tf.dispose([w, x, out, top]);
+      } else if (c.op === 'decodeWeightsToDevice') {
+        // the bytes of one quantised manifest entry, decoded the way the weights loader does
+        const ab = toArrayBuffer(fs.readFileSync(path.join(dir, c.inputs.bytes.file)));
+        const w = require('../io_utils').decodeWeightsToDevice(ab, [c.attrs.spec])[c.attrs.spec.name];
+        const r = w.quantization != null ? tf.dequantize(w) : w;
+        const vals = r.dataSync();
+        fs.writeFileSync(path.join(dir, c.name + '.out.bin'),
+                         Buffer.from(vals.buffer, vals.byteOffset, vals.byteLength));
+        entry.shape = r.shape;
+        entry.dtype = r.dtype;
+        entry.keptAsBytes = w.quantization != null;
+        tf.dispose([w, r]);
       } else {
         const inputs = {};
         Object.keys(c.inputs).forEach(k => { inputs[k] = load(c.inputs[k]); });

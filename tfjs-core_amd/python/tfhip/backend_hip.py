@@ -579,8 +579,9 @@ class MathBackendHIP(object):
         self._ck(self.lib.tfhip_cast(self.ctx, self._h(x), self._h(out)))
         return out
 
-    def dequantize(self, x):
-        out = self._out(x.shape, "float32")
+    def dequantize(self, x, bits=8):
+        """bits=16: x holds the two bytes of every 16-bit code along a last axis of 2."""
+        out = self._out(x.shape[:-1] if bits == 16 else x.shape, "float32")
         self._ck(self.lib.tfhip_dequantize(self.ctx, self._h(x), self._h(out), self._q(x)))
         return out
 

@@ -40,13 +40,21 @@ def tensor(values, shape=None, dtype=None):
 def quantized_tensor(q, scale, min_, shape=None):
     """A float32 weight tensor kept as uint8 affine-quantised bytes in HBM
     (io/types.ts:100-107); consumers dequantise w = q*scale + min on load."""
-    arr = np.ascontiguousarray(q, np.uint8)
+    if np.asarray(q).dtype == np.uint16:
+        # 16-bit codes: their bytes (low byte first) go to the device, with a last axis of 2; only
+        # dequantize() takes such a tensor, the dense kernels read one byte per weight
+        arr = np.ascontiguousarray(q, "<u2")
+        arr = arr.view(np.uint8).reshape(arr.shape + (2,))
+    else:
+        arr = np.ascontiguousarray(q, np.uint8)
     return Tensor(shape if shape is not None else arr.shape, "float32", None, arr, None,
                   (float(scale), float(min_)))
 
 
-def dequantize(t):
-    return ENGINE.run_kernel(lambda b: b.dequantize(t))
+def dequantize(t, bits=8):
+    """decodeWeights' quantised branch on the device (io/io_utils.ts:122-147); bits=16 for a
+    tensor made from uint16 codes."""
+    return ENGINE.run_kernel(lambda b: b.dequantize(t, bits))
 
 
 def _conv(x, name, op, dtype=None):
