@@ -921,7 +921,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     store(std::true_type{}, std::false_type{});
   } else if (!interior) {
     store(std::false_type{}, std::false_type{});
-  } else if (STAGED_STORE && (p.N & 3) == 0) {
+  } else if (STAGED_STORE && (p.N & 3) == 0 && (long long)BM * p.N * 4 < 0x7fffffffll) {
     // One accumulator column per lane would mean 4-byte stores (two 128-byte runs per
     // instruction).  Pass the tile through LDS instead and store it as 16 bytes per lane,
     // whole 256/512-byte row segments per instruction: a quarter of the store instructions.
@@ -935,6 +935,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
         cs[(i * 32 + 8 * (r >> 2) + (r & 3)) * LDC_S] = res[i][0][r];
     __syncthreads();
     constexpr int QUADS_PER_ROW = BN / 4;
+    // (a tile inside the matrix, its byte offsets below 2 GiB: no store relies on the range
+    // check.  Written through the L2: see STORE_WRITE_THROUGH.)
+    const __amdgpu_buffer_rsrc_t rsrc_ct = make_rsrc(Ct, 0x7fffffffu);
     constexpr int ROWS_PER_PASS = THREADS / QUADS_PER_ROW;
     static_assert(THREADS % QUADS_PER_ROW == 0 && BM % ROWS_PER_PASS == 0, "tile / block shape");
     const int cq = tid % QUADS_PER_ROW, r0 = tid / QUADS_PER_ROW;
@@ -949,7 +952,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       f32x4 v = *reinterpret_cast<const f32x4*>(lds + row * LDC_S + 4 * cq);
 #pragma unroll
       for (int e = 0; e < 4; e++) v[e] = clamp(v[e] + bv[e], cl);
-      *reinterpret_cast<f32x4*>(Ct + row * p.N + 4 * cq) = v;
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc_ct,
+                                             (row * p.N + 4 * cq) * 4, 0, STORE_WRITE_THROUGH);
     }
   } else {
     store(std::false_type{}, std::true_type{});
@@ -1257,7 +1261,7 @@ __global__ __launch_bounds__(SPLIT ? 384 : 256) void conv_smallk_kernel(const Ge
           for (int j = 0; j < TN; j++) {
             const float v = clamp(acc[j][r] + bias_c[j], cl);
             __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rout,
-                                                  (int)(lane_at[j] + px_at), 0, 0);
+                                                  (int)(lane_at[j] + px_at), 0, STORE_WRITE_THROUGH);
           }
         }
       }

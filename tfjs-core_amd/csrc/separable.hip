@@ -410,7 +410,7 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
               for (int c = 0; c < CB; c++) {
                 const float val = clamp(acc[c][r] + bias_c[c], pact);
                 __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), ry,
-                                                      (int)(reg_at[r] + (unsigned)(32 * c * 4)), s_blk, 0);
+                                                      (int)(reg_at[r] + (unsigned)(32 * c * 4)), s_blk, STORE_WRITE_THROUGH);
               }
             }
           } else {
@@ -434,7 +434,7 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
               for (int c = 0; c < CB; c++) {
                 const float val = clamp(acc[c][r] + bias_c[c], pact);
                 __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, val), ry,
-                                                      (int)(ok ? at + (unsigned)(32 * c * 4) : OOB_OFFSET), 0, 0);
+                                                      (int)(ok ? at + (unsigned)(32 * c * 4) : OOB_OFFSET), 0, STORE_WRITE_THROUGH);
               }
             }
           }
