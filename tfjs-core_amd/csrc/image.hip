@@ -63,9 +63,8 @@ struct DwArgs {
 // 3x3, dilation 1, channel multiplier 1, C % 4 == 0, stride S.  One lane = one channel
 // quad of a TH x TW output patch.  Lane order: channel quad fastest, then patch column,
 // patch row, image — neighbours in a wavefront touch neighbouring addresses.
-// WT: the output (below 2 GiB) is written through the L2 (STORE_WRITE_THROUGH).
-template <int S, int TH, int TW, bool WT>
-__global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p, unsigned y_bytes) {
+template <int S, int TH, int TW>
+__global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p) {
   constexpr int IH = (TH - 1) * S + 3, IW = (TW - 1) * S + 3;
   const tfhip_conv2d_info& ci = p.ci;
   const int64_t total = (int64_t)ci.batch * p.tiles_h * p.tiles_w * p.c4;
@@ -137,8 +136,6 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p, unsig
   f32x4 b = {0.f, 0.f, 0.f, 0.f};
   if (p.bias_kind == TFHIP_BCAST_COLUMN) b = *reinterpret_cast<const f32x4*>(p.bias + c);
   else if (p.bias_kind == TFHIP_BCAST_SCALAR) b = f32x4{p.bias[0], p.bias[0], p.bias[0], p.bias[0]};
-  const __amdgpu_buffer_rsrc_t ry =
-      __builtin_amdgcn_make_buffer_rsrc(p.y, (short)0, (int)y_bytes, 0x00020000);
 #pragma unroll
   for (int i = 0; i < TH; i++) {
     const int oh = oh0 + i;
@@ -150,13 +147,7 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p, unsig
       f32x4 v = acc[i][j] + b;
 #pragma unroll
       for (int e = 0; e < 4; e++) v[e] = act_fast(v[e], af);
-      if (WT) {
-        const unsigned at = (unsigned)(((n * ci.out_h + oh) * ci.out_w + ow) * C + c) * 4u;
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), ry, (int)at, 0,
-                                               STORE_WRITE_THROUGH);
-      } else {
-        *reinterpret_cast<f32x4*>(p.y + (((int64_t)n * ci.out_h + oh) * ci.out_w + ow) * C + c) = v;
-      }
+      *reinterpret_cast<f32x4*>(p.y + (((int64_t)n * ci.out_h + oh) * ci.out_w + ow) * C + c) = v;
     }
   }
 }
@@ -168,7 +159,7 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p, unsig
 // nothing is read twice vertically, and the two halo columns are shared with the
 // neighbouring lane's loads of the same moment.  Each output sums its taps in the order
 // filter row, then filter column, as the patch kernel above and the reference do.
-template <int TW, int PF, bool WT>
+template <int TW, int PF>
 __global__ __launch_bounds__(256) void depthwise3x3_rows_kernel(const DwArgs p, int rows,
                                                                 int chunks, unsigned x_bytes,
                                                                 unsigned y_bytes) {
@@ -249,8 +240,7 @@ __global__ __launch_bounds__(256) void depthwise3x3_rows_kernel(const DwArgs p, 
 #pragma unroll
       for (int e = 0; e < 4; e++) v[e] = act_fast(v[e], af);
       __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), ry,
-                                             (int)(row_ok ? at + col_out[j] : OOB), 0,
-                                             WT ? STORE_WRITE_THROUGH : 0);
+                                             (int)(row_ok ? at + col_out[j] : OOB), 0, 0);
     }
   };
   // Input row ih is filter row kh of output row ih + pad_top - kh: `newest` starts with it
@@ -451,24 +441,18 @@ static void launch_dw3x3(tfhip_ctx* ctx, DwArgs& p) {
   p.tiles_w = (int)ceil_div(p.ci.out_w, TW);
   const int64_t total = (int64_t)p.ci.batch * p.tiles_h * p.tiles_w * p.c4;
   p.reverse = ctx->take_sweep();
-  // an output the L2s can hold in full is written through (see launch_dw3x3_rows' caller)
-  const int64_t y_bytes = (int64_t)p.ci.batch * p.ci.out_h * p.ci.out_w * p.ci.out_c * 4;
-  if (y_bytes <= (32ll << 20))
-    tfhip::launch(ctx, (depthwise3x3_kernel<S, TH, TW, true>), dim3((unsigned)ceil_div(total, 256)),
-                       dim3(256), 0, p, (unsigned)y_bytes);
-  else
-    tfhip::launch(ctx, (depthwise3x3_kernel<S, TH, TW, false>), dim3((unsigned)ceil_div(total, 256)),
-                       dim3(256), 0, p, 0u);
+  tfhip::launch(ctx, (depthwise3x3_kernel<S, TH, TW>), dim3((unsigned)ceil_div(total, 256)),
+                     dim3(256), 0, p);
 }
 
-template <int TW, int PF, bool WT>
+template <int TW, int PF>
 static void launch_dw3x3_rows(tfhip_ctx* ctx, DwArgs& p, int rows) {
   ctx->name_kernel("depthwise3x3_s1_rows_w%d_ahead%d", TW, PF);
   const int chunks = (int)ceil_div(p.ci.out_h, rows);
   p.tiles_w = (int)ceil_div(p.ci.out_w, TW);
   const int64_t total = (int64_t)p.ci.batch * chunks * p.tiles_w * p.c4;
   p.reverse = ctx->take_sweep();
-  tfhip::launch(ctx, (depthwise3x3_rows_kernel<TW, PF, WT>), dim3((unsigned)ceil_div(total, 256)),
+  tfhip::launch(ctx, (depthwise3x3_rows_kernel<TW, PF>), dim3((unsigned)ceil_div(total, 256)),
                      dim3(256), 0, p, rows, chunks,
                      (unsigned)((int64_t)p.ci.batch * p.ci.in_h * p.ci.in_w * p.ci.in_c * 4),
                      (unsigned)((int64_t)p.ci.batch * p.ci.out_h * p.ci.out_w * p.ci.out_c * 4));
@@ -512,12 +496,7 @@ static int dispatch_depthwise(tfhip_ctx* ctx, DwArgs& p, const tfhip_conv2d_info
       // row: [64,14,14,512] 10.6 -> 9.4 us, [64,7,7,1024] 7.5 -> 6.8, [64,28,28,256] 25.1 -> 24.6;
       // three rows in flight, 217 registers: 11.1 / 8.2 / 26.8; strips one output column wide with
       // one / two / three rows in flight: 10.0 / 10.3 / 11.5 us on the first shape)
-      // An output that the L2s (4 MiB on each of 8 XCDs) can hold in full would still be there,
-      // dirty, when the kernel ends: written through instead (STORE_WRITE_THROUGH; measured in the
-      // same step: [64,14,14,512] 9.8 -> 9.3 us, [64,7,7,1024] 7.0 -> 6.1, but [64,28,28,256],
-      // 51 MB, 22.8 -> 23.4).
-      if (o_n * 4 <= (32ll << 20)) launch_dw3x3_rows<2, 2, true>(ctx, p, rows);
-      else launch_dw3x3_rows<2, 2, false>(ctx, p, rows);
+      launch_dw3x3_rows<2, 2>(ctx, p, rows);
     } else if (ci->stride_h == 1) {
       if (ci->out_w >= 112 && ci->in_c >= 128 && ci->out_w % 8 == 0) launch_dw3x3<1, 2, 8>(ctx, p);
       else launch_dw3x3<1, 2, 2>(ctx, p);

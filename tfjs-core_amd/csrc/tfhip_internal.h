@@ -28,7 +28,10 @@ namespace tfhip {
 // past that cache too and made those readers slower than it made the writer faster).  Measured
 // inside a batch-64 MobileNet step, the readers' times unchanged: 64 x 64 GEMM tiles
 // [50176,128]x[128,256] 34.1 -> 32.5 us, [12544,512]x[512,512] 52.6 -> 51.6; the 3x3x3 stem
-// 33.9 -> 32.5; the fused 128 -> 128 depthwise + pointwise block 76.9 -> 74.9.
+// 33.9 -> 32.5; the fused 128 -> 128 depthwise + pointwise block 76.9 -> 74.9; the step with
+// the input resident 0.870 -> 0.854 ms.  The depthwise kernels do not use it: their own times
+// fell (14x14x512: 9.8 -> 9.3 us) but the step that uploads its input while the previous batch
+// computes got 8 us longer.
 constexpr int STORE_WRITE_THROUGH = 16;
 
 struct Buf {
