@@ -29,21 +29,20 @@ __device__ __forceinline__ float act_f(float v, int act) {
   }
 }
 
-// The same activations without branches: the kind is unpacked once into values that are
-// the same for every lane.  NaN passes through (it is neither < 0 nor > hi).
+// The same activations as a clamp to [lo, hi] (linear: the whole line): IEEE 754-2019 maximum /
+// minimum, which gfx950 has as v_maximum3_f32 / v_minimum3_f32, return NaN when an operand is NaN,
+// so NaN passes through as it does through the reference's Math.max / Math.min.
 struct ActFlags {
-  bool linear;
-  float hi;
+  float lo, hi;
 };
 __device__ __forceinline__ ActFlags act_flags(int act) {
   ActFlags f;
-  f.linear = act != TFHIP_ACT_RELU && act != TFHIP_ACT_RELU6;
+  f.lo = act == TFHIP_ACT_RELU || act == TFHIP_ACT_RELU6 ? 0.f : -__builtin_inff();
   f.hi = act == TFHIP_ACT_RELU6 ? 6.f : __builtin_inff();
   return f;
 }
 __device__ __forceinline__ float act_fast(float v, const ActFlags& f) {
-  const float r = v < 0.f ? (f.linear ? v : 0.f) : v;
-  return r > f.hi ? f.hi : r;
+  return __builtin_elementwise_minimum(__builtin_elementwise_maximum(v, f.lo), f.hi);
 }
 
 struct DwArgs {

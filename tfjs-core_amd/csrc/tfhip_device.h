@@ -56,8 +56,7 @@ __device__ __forceinline__ float activate(float v, const ActCfg& c, float alpha)
 
 // relu / relu6 / linear as a clamp to [lo, hi] that lets NaN through (no comparison with NaN
 // holds), which is what the reference's Math.max(0, x) and clip do (backend_cpu.ts:1191-1201,
-// :1265-1275): two compares and two selects per value, against nine vector instructions of the
-// general form above.  The matrix instructions share their pipe with the vector ALU, so the
+// :1265-1275): two vector instructions per value, against nine of the general form above.  The matrix instructions share their pipe with the vector ALU, so the
 // stores of the dense kernels use this form and leave prelu to their general path.
 struct Clamp {
   float lo, hi;
@@ -69,10 +68,10 @@ __device__ __forceinline__ Clamp clamp_of(int act) {
   return c;
 }
 __device__ __forceinline__ float clamp(float v, const Clamp& c) {
-  // the median of (v, lo, hi) is the clamped value; NaN (v != v) passes through.  Three vector
-  // instructions instead of the four of two compare-and-select pairs.
-  const float r = __builtin_amdgcn_fmed3f(v, c.lo, c.hi);
-  return v != v ? v : r;
+  // IEEE 754-2019 maximum / minimum return NaN when an operand is NaN, so NaN passes through;
+  // gfx950 has them as v_maximum3_f32 / v_minimum3_f32: two vector instructions per value
+  // (the median of three plus a NaN select took three, two compare-and-select pairs four).
+  return __builtin_elementwise_minimum(__builtin_elementwise_maximum(v, c.lo), c.hi);
 }
 
 }  // namespace tfhip
