@@ -120,14 +120,26 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
   // (workgroup b runs on XCD b % 8; the grid is a multiple of 8): the kernels before and after
   // this one cut their rows the same way, so what an XCD leaves in its L2 is what it reads next.
   // Within its run a workgroup takes four neighbouring units (they share their halo columns),
-  // one per pair of wavefronts, then the four `stride` further on, ...
+  // one per pair of wavefronts, then the four `stride` further on, ...  With the filter in LDS
+  // (EVEN) what is left of the run after the whole trips is dealt evenly, `deal` <= 4
+  // neighbouring units to every workgroup, so that no workgroup (and no CU) gets a whole trip
+  // more than another.  (With the filter in registers the same dealing measured 1.3 us slower on
+  // [64,56,56,128] -> 128, whose units fill whole trips anyway.)
+  constexpr bool EVEN = !COLS;
   const int xcd = (int)blockIdx.x & 7;
   const int per = p.units >> 3, rem = p.units & 7;
   const int run0 = xcd * per + (xcd < rem ? xcd : rem);
   const int run1 = run0 + per + (xcd < rem ? 1 : 0);
-  const int wg_first = run0 + ((int)blockIdx.x >> 3) * 4;
-  const int stride = ((int)gridDim.x >> 3) * 4;
-  const int trips = wg_first < run1 ? (run1 - wg_first + stride - 1) / stride : 0;
+  const int wgs = (int)gridDim.x >> 3, wg = (int)blockIdx.x >> 3;
+  const int stride = wgs * 4;
+  const int wg_first = run0 + wg * 4;
+  const int full = EVEN ? (run1 - run0) / stride : 0;  // trips in which every workgroup has four units
+  const int left = (run1 - run0) - full * stride;      // units of the last, partial trip
+  const int deal = (left + wgs - 1) / wgs;
+  const int mine = min(deal, max(0, left - wg * deal)); // units of this workgroup in that trip
+  const int last_u = run0 + full * stride + wg * deal;
+  const int trips = EVEN ? full + (mine > 0 ? 1 : 0)
+                         : (wg_first < run1 ? (run1 - wg_first + stride - 1) / stride : 0);
   const int iters = (p.rh + RB - 1) / RB;  // panels of a unit
   const int total = trips * iters;
   struct Unit {
@@ -136,8 +148,15 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
   };
   auto unit_of = [&](int trip, int pr) {
     Unit un;
-    const int u = wg_first + trip * stride + pr;
-    un.live = u < run1;
+    int u;
+    if (EVEN) {
+      const bool whole = trip < full;
+      u = (whole ? wg_first + trip * stride : last_u) + pr;
+      un.live = whole || pr < mine;
+    } else {
+      u = wg_first + trip * stride + pr;
+      un.live = u < run1;
+    }
     const int unit = p.reverse ? run0 + run1 - 1 - u : u;
     un.strip = unit % p.strips;
     const int rest = unit / p.strips;
@@ -567,14 +586,50 @@ static int launch_separable(tfhip_ctx* ctx, SepArgs& p) {
   int rh = (int)ceil_div(p.OH, RB) * RB;
   while (rh > RB && (long long)p.batch * p.strips * ceil_div(p.OH, rh) < slots / 2)
     rh = (int)ceil_div(ceil_div(rh, 2), RB) * RB;
+  // Chunk height and grid together: with that height or half of it, and a grid of exactly the
+  // workgroups the units fill or of whole workgroups per CU, which pair leaves the busiest CU the
+  // fewest panels?  A workgroup takes its units four at a time, so a CU's work is (workgroups on
+  // it) x (units of a workgroup) x (panels of a unit); every unit costs a start (its first rows
+  // give no output) and re-reads the rows above and below it.  [64,112,112,32] -> 64: 1792 units
+  // of 14 panels are 448 workgroups, two on 192 CUs and one on 64, 112 panels on the busiest; 3584
+  // units of 7 panels on 512 workgroups are 7 units each, 98 panels on every CU: 76.1 -> 69.5 us
+  // in a batch-64 MobileNet step.  (The 128 -> 128 block, one workgroup per CU, 896 units of 7
+  // panels on 224 of 256 CUs, was measured with its strips cut in two on 256: 75 -> 81 us.)
+  const long long resident = (long long)ctx->num_cus * per_cu / 8 * 8;  // a multiple of the XCD count
+  const int cus = ctx->num_cus;
+  long long grid = 0;
+  double best_cost = 0;
+  int best_rh = rh;
+  const int half = (int)ceil_div(ceil_div(rh, 2), RB) * RB;
+  for (int cand : {rh, half}) {
+    if (cand < RB || (cand == half && half == rh)) continue;
+    const long long units = (long long)p.batch * p.strips * ceil_div(p.OH, cand);
+    const double per_unit = (double)ceil_div(cand, RB) + 0.3;
+    const double halo = 1.0 + (S == 1 ? 2.0 : 0.5) / cand;
+    auto consider = [&](long long g) {
+      // (at least two workgroups on most CUs where that many fit: one alone, two wavefronts per
+      // SIMD, hides too little latency -- [64,112,112,32] -> 64 on 256 workgroups 75.5 us)
+      if (g < 8 || g > resident || g * 8 < (long long)cus * (per_cu < 2 ? per_cu : 2) * 7) return;
+      // (units of the busiest workgroup: dealt evenly, or four per trip with the filter in registers)
+      const double units_wg = COLS ? 4.0 * (double)ceil_div(units, 4 * g) : (double)ceil_div(units, g);
+      const double c = (double)ceil_div(g, cus) * units_wg * per_unit * halo;
+      if (grid == 0 || c < best_cost * 0.999) {
+        grid = g;
+        best_cost = c;
+        best_rh = cand;
+      }
+    };
+    consider(ceil_div(ceil_div(units, 8), 4) * 8);
+    for (int k = 1; k <= per_cu; k++) consider((long long)cus * k / 8 * 8);
+  }
+  if (grid == 0) grid = resident < 8 ? ceil_div(ceil_div((long long)p.batch * p.strips * ceil_div(p.OH, rh), 8), 4) * 8 : resident;
+  rh = best_rh;
   p.rh = rh;
   p.chunks = (int)ceil_div(p.OH, rh);
   p.units = p.batch * p.chunks * p.strips;
-  const long long want = ceil_div(ceil_div(p.units, 8), 4) * 8;
-  const long long resident = (long long)ctx->num_cus * per_cu / 8 * 8;  // a multiple of the XCD count
   ctx->name_kernel("separable_s%d_k%dxn%d_%s", S, K, N, p.pw_quant ? "u8" : "f32");
   p.reverse = ctx->take_sweep();
-  tfhip::launch(ctx, kernel, dim3((unsigned)(want < resident || resident < 8 ? want : resident)),
+  tfhip::launch(ctx, kernel, dim3((unsigned)grid),
                 dim3(512), lds, p);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
