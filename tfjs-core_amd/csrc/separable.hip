@@ -481,8 +481,9 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
     int trip = 0, blk = 0;
     Unit un = unit_of(0, pair);
     for (int it = 0; it <= total; it++) {
-      if (it > 0) {
-        // the panel filled during the previous step: block `blk` of unit `un`
+      // the panel filled during the previous step: block `blk` of unit `un` (a pair without a
+      // unit in this trip has no panel to multiply)
+      if (it > 0 && un.live) {
         const float* const panel = panel_r + ((it - 1) & 1) * (32 * PITCH);
         f32x16 acc[NJ];
         // operands of group q + 1 are read while group q is multiplied; the order is pinned so
@@ -546,15 +547,13 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
           }
         };
         // (made of the unit's own numbers, so the whole wavefront takes the same branch)
-        if (un.live) {
-          if (rows_left >= RB && cols_left >= SW) store(std::true_type{});
-          else if (rows_left > 0) store(std::false_type{});
-        }
-        if (++blk == iters) {
-          blk = 0;
-          trip++;
-          un = unit_of(trip, pair);
-        }
+        if (rows_left >= RB && cols_left >= SW) store(std::true_type{});
+        else if (rows_left > 0) store(std::false_type{});
+      }
+      if (it > 0 && ++blk == iters) {
+        blk = 0;
+        trip++;
+        un = unit_of(trip, pair);
       }
       __syncthreads();  // the next panel is complete; this one may be overwritten
     }
