@@ -591,7 +591,7 @@ static int launch_separable(tfhip_ctx* ctx, SepArgs& p) {
   // it) x (units of a workgroup) x (panels of a unit); every unit costs a start (its first rows
   // give no output) and re-reads the rows above and below it.  [64,112,112,32] -> 64: 1792 units
   // of 14 panels are 448 workgroups, two on 192 CUs and one on 64, 112 panels on the busiest; 3584
-  // units of 7 panels on 512 workgroups are 7 units each, 98 panels on every CU: 76.1 -> 69.5 us
+  // units of 7 panels on 512 workgroups are 7 units each, 98 panels on every CU: 76.4 -> 67.2 us
   // in a batch-64 MobileNet step.  (The 128 -> 128 block, one workgroup per CU, 896 units of 7
   // panels on 224 of 256 CUs, was measured with its strips cut in two on 256: 75 -> 81 us.)
   const long long resident = (long long)ctx->num_cus * per_cu / 8 * 8;  // a multiple of the XCD count
@@ -621,15 +621,16 @@ static int launch_separable(tfhip_ctx* ctx, SepArgs& p) {
     consider(ceil_div(ceil_div(units, 8), 4) * 8);
     for (int k = 1; k <= per_cu; k++) consider((long long)cus * k / 8 * 8);
   }
-  if (grid == 0) grid = resident < 8 ? ceil_div(ceil_div((long long)p.batch * p.strips * ceil_div(p.OH, rh), 8), 4) * 8 : resident;
+  if (grid == 0)  // (a machine of fewer than 8 CUs: one workgroup per four units)
+    grid = resident >= 8 ? resident
+                         : ceil_div(ceil_div((long long)p.batch * p.strips * ceil_div(p.OH, rh), 8), 4) * 8;
   rh = best_rh;
   p.rh = rh;
   p.chunks = (int)ceil_div(p.OH, rh);
   p.units = p.batch * p.chunks * p.strips;
   ctx->name_kernel("separable_s%d_k%dxn%d_%s", S, K, N, p.pw_quant ? "u8" : "f32");
   p.reverse = ctx->take_sweep();
-  tfhip::launch(ctx, kernel, dim3((unsigned)grid),
-                dim3(512), lds, p);
+  tfhip::launch(ctx, kernel, dim3((unsigned)grid), dim3(512), lds, p);
   TFHIP_LAUNCH_CHECK(ctx);
   return TFHIP_OK;
 }
