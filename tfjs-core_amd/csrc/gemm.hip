@@ -1023,6 +1023,7 @@ template <int TN, bool QUANT, bool SPLIT>
 __global__ __launch_bounds__(SPLIT ? 384 : 256) void conv_smallk_kernel(const GemmArgs p,
                                                                        int row_floats, int n_rows) {
   extern __shared__ __attribute__((aligned(16))) float rows[];  // [KH][row_floats] (+ 1), x 2 if SPLIT
+  __builtin_amdgcn_s_setprio(WAVE_PRIORITY_MEMORY_BOUND);
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, g = lane >> 5;

@@ -65,6 +65,7 @@ struct DwArgs {
 template <int S, int TH, int TW>
 __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DwArgs p) {
   constexpr int IH = (TH - 1) * S + 3, IW = (TW - 1) * S + 3;
+  __builtin_amdgcn_s_setprio(WAVE_PRIORITY_MEMORY_BOUND);
   const tfhip_conv2d_info& ci = p.ci;
   const int64_t total = (int64_t)ci.batch * p.tiles_h * p.tiles_w * p.c4;
   // contiguous image regions per XCD: the halo rows two patch rows share are then served
@@ -162,6 +163,7 @@ template <int TW, int PF>
 __global__ __launch_bounds__(256) void depthwise3x3_rows_kernel(const DwArgs p, int rows,
                                                                 int chunks, unsigned x_bytes,
                                                                 unsigned y_bytes) {
+  __builtin_amdgcn_s_setprio(WAVE_PRIORITY_MEMORY_BOUND);
   constexpr int IW = TW + 2;
   constexpr int NB = PF + 1;                       // row buffers: PF rows in flight + the one in use
   constexpr int PERIOD = NB % 3 == 0 ? NB : 3 * NB;  // buffers and accumulator rows take turns

@@ -83,6 +83,7 @@ __global__ __launch_bounds__(512, OCC) void separable_kernel(const SepArgs p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  __builtin_amdgcn_s_setprio(WAVE_PRIORITY_MEMORY_BOUND);
   const bool producer = wave < 4;
   const int pair = wave & 3;
   const int l32 = lane & 31, g = lane >> 5;
