@@ -913,6 +913,7 @@ def _separable_oracle(ref, x, dw, pw, stride, dbias, dact, pbias, pact):
     ((8, 56, 56, 128), 128, 1),     # too few pixels for it: two kernels
     ((33, 55, 57, 128), 256, 2),    # K 128 -> N 256 at stride 2: two kernels
     ((17, 113, 111, 32), 64, 1),    # odd extents: blocks straddle rows and images, last block short
+    ((73, 112, 112, 32), 64, 1),    # units that do not fill whole trips: the rest is dealt evenly, some pairs idle
     ((66, 111, 113, 64), 128, 2),   # stride 2 on odd extents (padding 1 on both sides)
     ((2, 20, 20, 32), 64, 1),       # too few pixels for the panel-walking kernel: the small-problem kernel
     ((3, 56, 56, 128), 128, 1),     # too many tiles for that one, too few panels for the other: two kernels
